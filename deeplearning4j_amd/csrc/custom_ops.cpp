@@ -1,0 +1,637 @@
+// Declarable ops on the decoder path: matmul (+aliases), softmax, layer_norm, dot_product_attention_v2,
+// argmax/argmin, and the glue ops a GPT-2-shaped decode step needs (gather, add, multiply, concat).
+#include "custom_ops.h"
+
+#include <algorithm>
+#include <map>
+#include <mutex>
+
+#include "kernels.h"
+#include "plan.h"
+
+namespace nd4jhip {
+namespace ops {
+
+// ---- hash ----------------------------------------------------------------------------------------------------
+LongType opHash(const std::string& name) {
+  static unsigned long long table[256];
+  static std::once_flag once;
+  std::call_once(once, [] {
+    unsigned long long h = 0x544B2FBACAAF1684ULL;
+    for (int i = 0; i < 256; i++) {
+      for (int j = 0; j < 31; j++) {
+        h = (h >> 7) ^ h;
+        h = (h << 11) ^ h;
+        h = (h >> 10) ^ h;
+      }
+      table[i] = h;
+    }
+  });
+  unsigned long long h = 0xBB40E64DA205B064ULL;
+  const unsigned long long mult = 7664345821815920749ULL;
+  for (char ch : name) {
+    unsigned char uch = (unsigned char)ch;
+    h = (h * mult) ^ table[uch & 0xff];
+    h = (h * mult) ^ table[(uch >> 8) & 0xff];  // an 8-bit value shifted by 8: always entry 0, as in the reference
+  }
+  return (LongType)h;
+}
+
+static hipStream_t stream() { return LaunchContext::defaultContext()->execStream; }
+static LongType iArg(const Context& c, size_t i, LongType def) { return i < c.iArgs.size() ? c.iArgs[i] : def; }
+static double tArg(const Context& c, size_t i, double def) { return i < c.tArgs.size() ? c.tArgs[i] : def; }
+static bool bArg(const Context& c, size_t i, bool def) { return i < c.bArgs.size() ? (bool)c.bArgs[i] : def; }
+static std::vector<LongType> shapeOf(const NDArray* a) {
+  return std::vector<LongType>(shape::shapeOf(a->shapeInfo()), shape::shapeOf(a->shapeInfo()) + a->rankOf());
+}
+static std::string shapeStr(const NDArray* a) {
+  std::string s = "[";
+  for (int i = 0; i < a->rankOf(); i++) s += (i ? "," : "") + std::to_string(a->sizeAt(i));
+  return s + "]";
+}
+
+// ---- matmul ----------------------------------------------------------------------------------------------------
+// generic/blas/matmul.cpp:35-176 of the reference: C = alpha * op(A) op(B) + beta * C; IArgs [transX, transY, transZ],
+// TArgs [alpha, beta]; transZ swaps the inputs and flips both flags.  Transposes are realised through strides
+// (the reference materialises permuted copies, helpers/impl/MmulHelper.cpp:506-526).
+struct MatmulGeometry {
+  NDArray *x, *y;
+  bool transX, transY;
+  LongType M, N, K;
+  LongType aRow, aCol, bRow, bCol;
+  std::vector<LongType> batchShape, xBatch, yBatch;
+  std::vector<LongType> zShape;
+};
+static MatmulGeometry matmulGeometry(Context& c) {
+  MatmulGeometry g;
+  g.x = c.input(0); g.y = c.input(1);
+  g.transX = iArg(c, 0, 0) != 0; g.transY = iArg(c, 1, 0) != 0;
+  const bool transZ = iArg(c, 2, 0) != 0;
+  if (transZ) {
+    std::swap(g.x, g.y);
+    bool t = g.transX; g.transX = !g.transY; g.transY = !t;
+  }
+  NDArray *x = g.x, *y = g.y;
+  int xr = x->rankOf(), yr = y->rankOf();
+  ND4J_REQUIRE(xr > 0 && yr > 0, "MATMUL OP: input arrays must have rank bigger than 0 (should not be scalars), but got instead: x rank = " + std::to_string(xr) + ", y rank = " + std::to_string(yr) + " !");
+  // effective last-two dims and batch dims of x
+  auto split = [](NDArray* a, bool trans, LongType& rows, LongType& cols, LongType& rs, LongType& cs, std::vector<LongType>& bshape, std::vector<LongType>& bstride, bool isX) {
+    int r = a->rankOf();
+    if (r == 1) {
+      if (isX) { rows = 1; cols = a->sizeAt(0); rs = 0; cs = a->strideAt(0); }
+      else { rows = a->sizeAt(0); cols = 1; rs = a->strideAt(0); cs = 0; }
+      return;
+    }
+    int ri = trans ? r - 1 : r - 2, ci = trans ? r - 2 : r - 1;
+    rows = a->sizeAt(ri); cols = a->sizeAt(ci); rs = a->strideAt(ri); cs = a->strideAt(ci);
+    for (int d = 0; d < r - 2; d++) { bshape.push_back(a->sizeAt(d)); bstride.push_back(a->strideAt(d)); }
+  };
+  LongType Ky;
+  std::vector<LongType> xbs, ybs;
+  split(x, g.transX, g.M, g.K, g.aRow, g.aCol, xbs, g.xBatch, true);
+  split(y, g.transY, Ky, g.N, g.bRow, g.bCol, ybs, g.yBatch, false);
+  if (xr == 1 && yr == 1) {
+    ND4J_REQUIRE(g.K == Ky, "MATMUL OP: since input arrays are vectors they must have the same length, but got x length = " + std::to_string(g.K) + ", y length = " + std::to_string(Ky) + " !");
+    g.zShape = {};
+  } else if (xr == 1 && yr == 2) {
+    ND4J_REQUIRE(g.K == Ky, "MATMUL OP: input arrays have inconsistent shapes for vector-matrix product: x " + shapeStr(x) + ", y " + shapeStr(y) + " !");
+    g.zShape = {g.N};
+  } else if (xr == 2 && yr == 1) {
+    ND4J_REQUIRE(g.K == Ky, "MATMUL OP: input arrays have inconsistent shapes for matrix-vector product: x " + shapeStr(x) + ", y " + shapeStr(y) + " !");
+    g.zShape = {g.M};
+  } else {
+    // leading singleton dims of the higher-rank operand are squeezed against a rank-2 partner (matmul.cpp:80-118)
+    auto allOnes = [](const std::vector<LongType>& v) { return std::all_of(v.begin(), v.end(), [](LongType s) { return s == 1; }); };
+    if (xr != yr) {
+      ND4J_REQUIRE((xr > yr && yr == 2 && allOnes(xbs)) || (yr > xr && xr == 2 && allOnes(ybs)),
+                   "MATMUL OP: input and output arrays must have the same rank, but got instead: x rank = " + std::to_string(xr) + ", y rank = " + std::to_string(yr) + " !");
+      g.zShape = xr > yr ? xbs : ybs;
+      g.batchShape.clear(); g.xBatch.clear(); g.yBatch.clear();
+    } else {
+      for (size_t d = 0; d < xbs.size(); d++)
+        ND4J_REQUIRE(xbs[d] == ybs[d], "MATMUL OP: input/output arrays have inconsistent shapes for matrix product: x " + shapeStr(x) + ", y " + shapeStr(y) + " !");
+      g.batchShape = xbs;
+      g.zShape = xbs;
+    }
+    ND4J_REQUIRE(g.K == Ky, "MATMUL OP: input/output arrays have inconsistent shapes for matrix product: x " + shapeStr(x) + ", y " + shapeStr(y) + " !");
+    g.zShape.push_back(g.M); g.zShape.push_back(g.N);
+  }
+  return g;
+}
+
+static std::vector<std::vector<LongType>> matmulShapeFn(Context& c) {
+  MatmulGeometry g = matmulGeometry(c);
+  // order 'c' iff both inputs are 'c'; dtype = the higher of the two codes (matmul.cpp:189-219)
+  char order = g.x->ordering() == 'c' && g.y->ordering() == 'c' ? 'c' : 'f';
+  DataType dt = g.x->dataType() > g.y->dataType() ? g.x->dataType() : g.y->dataType();
+  if (g.x->isEmpty() || g.y->isEmpty()) return {makeShapeInfo(g.x->dataType(), order, g.zShape, nullptr, ARRAY_EMPTY)};
+  return {makeShapeInfo(dt, order, g.zShape)};
+}
+
+static void matmulExec(Context& c) {
+  ND4J_REQUIRE(c.width() >= 2, "MATMUL OP: two input arrays are required");
+  NDArray* z = c.output(0);
+  if (c.input(0)->isEmpty() || c.input(1)->isEmpty()) return;
+  MatmulGeometry g = matmulGeometry(c);
+  ND4J_REQUIRE(z->lengthOf() == [&] { LongType n = 1; for (auto s : g.zShape) n *= s; return n; }(),
+               "NDArrayFactory::matmul static method: input shape of output array is wrong, actual is " + shapeStr(z) + " !");
+  // z must carry the expected shape up to unit dims
+  {
+    std::vector<LongType> a, b;
+    for (auto s : g.zShape) if (s != 1) a.push_back(s);
+    for (int d = 0; d < z->rankOf(); d++) if (z->sizeAt(d) != 1) b.push_back(z->sizeAt(d));
+    ND4J_REQUIRE(a == b, "NDArrayFactory::matmul static method: input shape of output array is wrong, actual is " + shapeStr(z) + " !");
+  }
+  if (z->isEmpty()) return;
+  DataType dt = z->dataType();
+  ND4J_REQUIRE(g.x->dataType() == dt && g.y->dataType() == dt, "MATMUL OP: nd4j-hip requires x, y and z to share one data type");
+  ND4J_REQUIRE(isFloatType(dt), "MATMUL OP: integer types are not implemented in nd4j-hip");
+  GemmDesc d;
+  d.M = g.M; d.N = g.N; d.K = g.K;
+  d.aRow = g.aRow; d.aCol = g.aCol; d.bRow = g.bRow; d.bCol = g.bCol;
+  d.alpha = (float)tArg(c, 0, 1.0); d.beta = (float)tArg(c, 1, 0.0);
+  // strides of z's matrix dims: the non-unit dims of z in order, lined up with [batch.., M, N]
+  std::vector<LongType> zs;   // stride per entry of zShape
+  {
+    int zd = 0;
+    for (size_t i = 0; i < g.zShape.size(); i++) {
+      if (g.zShape[i] == 1) { zs.push_back(0); continue; }
+      while (zd < z->rankOf() && z->sizeAt(zd) == 1) zd++;
+      zs.push_back(z->strideAt(zd++));
+    }
+  }
+  const int xr = g.x->rankOf(), yr = g.y->rankOf();
+  if (xr == 1 && yr == 1) { d.cRow = 0; d.cCol = 0; }
+  else if (xr == 1) { d.cRow = 0; d.cCol = zs.empty() ? 0 : zs.back(); }
+  else if (yr == 1) { d.cRow = zs.empty() ? 0 : zs.back(); d.cCol = 0; }
+  else { d.cRow = zs[zs.size() - 2]; d.cCol = zs[zs.size() - 1]; }
+  // batch dims: collapse jointly; what does not collapse into one dim is looped on the host
+  std::vector<LongType> bshape = g.batchShape, xb = g.xBatch, yb = g.yBatch, zb;
+  for (size_t i = 0; i < bshape.size(); i++) zb.push_back(zs[i]);
+  int br = 0;
+  if (!bshape.empty()) {
+    LongType* ptr[3] = {xb.data(), yb.data(), zb.data()};
+    br = collapseDims((int)bshape.size(), bshape.data(), ptr, 3);
+    bshape.resize(br); xb.resize(br); yb.resize(br); zb.resize(br);
+    if (br == 1 && bshape[0] == 1) br = 0;
+  }
+  prepareSpecialUse({z}, {g.x, g.y});
+  const size_t es = sizeOf(dt);
+  const char* A = (const char*)g.x->specialBuffer();
+  const char* B = (const char*)g.y->specialBuffer();
+  char* C = (char*)z->specialBuffer();
+  if (br == 0) {
+    d.batch = 1;
+    launchGemm(stream(), dt, A, B, C, d);
+  } else {
+    d.batch = bshape[br - 1]; d.aBatch = xb[br - 1]; d.bBatch = yb[br - 1]; d.cBatch = zb[br - 1];
+    LongType outer = 1;
+    for (int i = 0; i < br - 1; i++) outer *= bshape[i];
+    for (LongType o = 0; o < outer; o++) {
+      LongType idx = o, ao = 0, bo = 0, co = 0;
+      for (int i = br - 2; i >= 0; i--) { LongType q = idx % bshape[i]; idx /= bshape[i]; ao += q * xb[i]; bo += q * yb[i]; co += q * zb[i]; }
+      launchGemm(stream(), dt, A + ao * es, B + bo * es, C + co * es, d);
+    }
+  }
+  registerSpecialUse({z}, {g.x, g.y});
+}
+
+// ---- softmax -----------------------------------------------------------------------------------------------------
+// generic/nn/softmax.cpp:37-52 -> helpers/cpu/softmax.cpp:252-353
+static bool sameShapeStrict(const NDArray* a, const NDArray* b) {
+  if (a->rankOf() != b->rankOf()) return false;
+  for (int d = 0; d < a->rankOf(); d++) if (a->sizeAt(d) != b->sizeAt(d) || a->strideAt(d) != b->strideAt(d)) return false;
+  return true;
+}
+static bool isVector(const NDArray* a) {
+  if (a->rankOf() == 1) return true;
+  if (a->rankOf() == 2) return (a->sizeAt(0) == 1 || a->sizeAt(1) == 1) && a->lengthOf() > 1;
+  return false;
+}
+static void fillValue(NDArray* z, double v) {
+  EwPlan p = buildEwPlan({z->shapeInfo(), z->shapeInfo()});
+  launchScalarOp(stream(), P_COPY, z->dataType(), z->specialBuffer(), v, z->specialBuffer(), p);
+}
+static void softmaxExec(Context& c) {
+  NDArray* x = c.input(0);
+  NDArray* z = c.output(0);
+  const int rank = x->rankOf();
+  int dim = (int)iArg(c, 0, rank - 1);
+  ND4J_REQUIRE(dim < rank, "SOFTMAX OP: the value of input integer parameter (dimension) must be less than input array rank " + std::to_string(rank) + ", but got dimension = " + std::to_string(dim) + " instead !");
+  if (dim < 0) dim += rank;
+  ND4J_REQUIRE(rank == 0 || dim >= 0, "SOFTMAX OP: dimension out of range");
+  ND4J_REQUIRE(x->dataType() == z->dataType() && isFloatType(x->dataType()), "SOFTMAX OP: input and output must share a floating point type");
+  ND4J_REQUIRE(x->lengthOf() == z->lengthOf(), "SOFTMAX OP: input and output lengths differ");
+  if (x->isEmpty()) return;
+  prepareSpecialUse({z}, {x});
+  bool clamp = sameShapeStrict(x, z);
+  if (isVector(x)) {
+    if (rank != 1 && x->sizeAt(dim) == 1) {  // softmax.cpp:255-259: a vector reduced along its unit axis is all ones
+      fillValue(z, 1.0);
+      registerSpecialUse({z}, {x});
+      return;
+    }
+    // the vector path ignores `dim` and normalises the whole vector, always with the clamp semantics
+    clamp = true;
+    if (rank == 2) dim = x->sizeAt(0) == 1 ? 1 : 0;
+  }
+  if (rank == 0) { fillValue(z, 1.0); registerSpecialUse({z}, {x}); return; }
+  RowPlan p = buildRowPlan(x->shapeInfo(), z->shapeInfo(), dim);
+  launchSoftmax(stream(), x->dataType(), x->specialBuffer(), z->specialBuffer(), p, clamp);
+  registerSpecialUse({z}, {x});
+}
+static std::vector<std::vector<LongType>> sameAsInputShapeFn(Context& c) {
+  NDArray* x = c.input(0);
+  return {makeShapeInfo(x->dataType(), x->ordering(), shapeOf(x))};
+}
+
+// ---- layer_norm ------------------------------------------------------------------------------------------------------
+// generic/nn/layer_norm.cpp:35-79: standardize over IArgs axes, then * gain (+ bias) along dim 1 (BArg0 true or
+// absent) or the last dim (BArg0 false); eps 1e-5 inside the sqrt (generic/transforms/standardize.cpp:34-78)
+static void layerNormImpl(Context& c, NDArray* x, NDArray* gain, NDArray* bias, NDArray* z, const std::vector<LongType>& axesIn, bool channelsFirst, const char* opName) {
+  const int rank = x->rankOf();
+  ND4J_REQUIRE(!axesIn.empty(), "STANDARDIZE OP: axis has to be non-empty");
+  auto axes = normalizeDims(rank, axesIn.data(), (LongType)axesIn.size(), opName);
+  ND4J_REQUIRE(x->dataType() == z->dataType() && isFloatType(x->dataType()), std::string(opName) + ": input and output must share a floating point type");
+  ND4J_REQUIRE(sameShapeStrict(x, z) || shapeOf(x) == shapeOf(z), std::string(opName) + ": input and output shapes differ");
+  int dimC = -1;
+  if (gain) {
+    dimC = channelsFirst ? 1 : rank - 1;
+    ND4J_REQUIRE(dimC < rank, std::string(opName) + ": input rank too small for the channel axis");
+    ND4J_REQUIRE(gain->rankOf() == 1 && gain->sizeAt(0) == x->sizeAt(dimC),
+                 "LAYER_NORM OP: wrong shape of gain array, expected is {" + std::to_string(x->sizeAt(dimC)) + "}, but got " + shapeStr(gain) + " instead !");
+    if (bias) ND4J_REQUIRE(bias->rankOf() == 1 && bias->sizeAt(0) == x->sizeAt(dimC),
+                           "LAYER_NORM OP: wrong shape of bias array, expected is {" + std::to_string(x->sizeAt(dimC)) + "}, but got " + shapeStr(bias) + " instead !");
+    ND4J_REQUIRE(gain->dataType() == x->dataType() && (!bias || bias->dataType() == x->dataType()), "LAYER_NORM OP: nd4j-hip requires gain and bias to carry the input's data type");
+  }
+  if (x->isEmpty()) return;
+  std::vector<NDArray*> reads = {x};
+  if (gain) reads.push_back(gain);
+  if (bias) reads.push_back(bias);
+  prepareSpecialUse(std::vector<NDArray*>{z}, reads);
+  const float eps = 1e-5f;
+  const bool lastAxisOnly = axes.size() == 1 && axes[0] == rank - 1 && dimC == rank - 1 && gain && gain->strideAt(0) == 1 && (!bias || bias->strideAt(0) == 1);
+  if (lastAxisOnly && x->sizeAt(rank - 1) <= 8192) {
+    RowPlan p = buildRowPlan(x->shapeInfo(), z->shapeInfo(), rank - 1);
+    launchLayerNormRows(stream(), x->dataType(), x->specialBuffer(), gain->specialBuffer(), bias ? bias->specialBuffer() : nullptr, z->specialBuffer(), p, eps);
+  } else {
+    ND4J_REQUIRE(gain != nullptr, "STANDARDIZE OP: the stand-alone op is reached through layer_norm in nd4j-hip");
+    ND4J_REQUIRE(gain->strideAt(0) == 1 && (!bias || bias->strideAt(0) == 1), "LAYER_NORM OP: gain/bias must be dense");
+    LnGenericPlan p;
+    std::vector<bool> red(rank, false);
+    for (auto a : axes) red[a] = true;
+    std::vector<LongType> os, oxs, ozs, is, ixs, izs;
+    for (int d = 0; d < rank; d++) {
+      if (red[d]) { if (d == dimC) { p.channelInInner = 1; p.channelPos = (int)is.size(); } is.push_back(x->sizeAt(d)); ixs.push_back(x->strideAt(d)); izs.push_back(z->strideAt(d)); }
+      else { if (d == dimC) { p.channelInInner = 0; p.channelPos = (int)os.size(); } os.push_back(x->sizeAt(d)); oxs.push_back(x->strideAt(d)); ozs.push_back(z->strideAt(d)); }
+    }
+    p.outerLen = 1; for (auto s : os) p.outerLen *= s;
+    p.innerLen = 1; for (auto s : is) p.innerLen *= s;
+    p.outerX = toDevShape(os, oxs); p.outerZ = toDevShape(os, ozs);
+    p.innerX = toDevShape(is, ixs); p.innerZ = toDevShape(is, izs);
+    launchLayerNormGeneric(stream(), x->dataType(), x->specialBuffer(), gain->specialBuffer(), bias ? bias->specialBuffer() : nullptr, z->specialBuffer(), p, eps);
+  }
+  registerSpecialUse(std::vector<NDArray*>{z}, reads);
+}
+static void layerNormExec(Context& c) {
+  ND4J_REQUIRE(c.width() >= 2, "LAYER_NORM OP: input and gain arrays are required");
+  NDArray* bias = c.width() > 2 ? c.input(2) : nullptr;
+  layerNormImpl(c, c.input(0), c.input(1), bias, c.output(0), c.iArgs, bArg(c, 0, true), "LAYER_NORM OP");
+}
+
+// ---- dot_product_attention_v2 ---------------------------------------------------------------------------------------------
+// generic/nn/dot_product_attention_v2.cpp:35-125 -> helpers/impl/AttentionHelper.cpp:411-469.
+// Inputs (queries, values, keys?); TArgs [scale, dropout]; BArgs [useCausalMask, training];
+// outputs [out, weights?, logits?].  logits = clip(scale * q k^T, +-1e4) (scale applied unless 0 or 1),
+// masked (j > i) logits get 65504 (bf16) / 1e9 (other types) subtracted, weights = softmax(logits),
+// out = weights v.  With only `out` supplied the fused kernel runs and nothing of size Tq x Tv is written.
+struct AttnViews { NDArray q, k, v, out, w, l; };
+static NDArray as3d(const NDArray* a) {
+  NDArray r = *a;
+  const int rank = a->rankOf();
+  std::vector<LongType> shp, st;
+  if (rank == 2) { shp = {1, a->sizeAt(0), a->sizeAt(1)}; st = {a->sizeAt(0) * a->strideAt(0), a->strideAt(0), a->strideAt(1)}; }
+  else if (rank == 3) return r;
+  else {
+    // rank > 3: fold the leading dims into one batch dim when their strides nest
+    std::vector<LongType> bs, bst;
+    for (int d = 0; d < rank - 2; d++) { bs.push_back(a->sizeAt(d)); bst.push_back(a->strideAt(d)); }
+    LongType* ptr[1] = {bst.data()};
+    int nr = collapseDims((int)bs.size(), bs.data(), ptr, 1);
+    ND4J_REQUIRE(nr == 1, "dot_product_attention_v2: leading dims of a rank-" + std::to_string(rank) + " input do not fold into one batch dim");
+    shp = {bs[0], a->sizeAt(rank - 2), a->sizeAt(rank - 1)}; st = {bst[0], a->strideAt(rank - 2), a->strideAt(rank - 1)};
+  }
+  r.si = makeShapeInfo(a->dataType(), 'c', shp, st.data());
+  return r;
+}
+static void attentionExec(Context& c) {
+  ND4J_REQUIRE(c.width() >= 2, "dot_product_attention_v2: queries and values are required");
+  NDArray* q0 = c.input(0); NDArray* v0 = c.input(1); NDArray* k0 = c.width() > 2 ? c.input(2) : v0;
+  ND4J_REQUIRE(q0->rankOf() == v0->rankOf(), "Queries and values must be same ranks!");
+  for (int i = 3; i < c.width(); i++)
+    ND4J_REQUIRE(c.inputs[i] == nullptr || c.inputs[i]->isEmpty(), "dot_product_attention_v2: query/value masks are not implemented in nd4j-hip");
+  const double dropout = tArg(c, 1, 0.0);
+  const double scale = tArg(c, 0, 1.0);
+  const bool causal = bArg(c, 0, false), training = bArg(c, 1, false);
+  ND4J_REQUIRE(!(training && dropout > 0.0), "dot_product_attention_v2: dropout is not implemented in nd4j-hip");
+  NDArray q = as3d(q0), v = as3d(v0), k = as3d(k0), out = as3d(c.output(0));
+  const bool wantW = c.outputs.size() > 1 && c.outputs[1] != nullptr, wantL = c.outputs.size() > 2 && c.outputs[2] != nullptr;
+  DataType dt = q.dataType();
+  ND4J_REQUIRE(isFloatType(dt) && dt != DOUBLE, "dot_product_attention_v2: nd4j-hip implements FLOAT, HALF and BFLOAT16");
+  ND4J_REQUIRE(k.dataType() == dt && v.dataType() == dt && out.dataType() == dt, "dot_product_attention_v2: all arrays must share one data type");
+  AttnDesc d;
+  d.B = q.sizeAt(0); d.Tq = q.sizeAt(1); d.D = q.sizeAt(2); d.Tv = v.sizeAt(1); d.Dv = v.sizeAt(2);
+  ND4J_REQUIRE(k.sizeAt(0) == d.B && v.sizeAt(0) == d.B, "dot_product_attention_v2: batch sizes differ");
+  ND4J_REQUIRE(k.sizeAt(1) == d.Tv && k.sizeAt(2) == d.D, "dot_product_attention_v2: keys must be [batch, Tv, dim], got " + shapeStr(&k));
+  ND4J_REQUIRE(out.sizeAt(0) == d.B && out.sizeAt(1) == d.Tq && out.sizeAt(2) == d.Dv, "dot_product_attention_v2: output must be [batch, Tq, dimV], got " + shapeStr(&out));
+  d.scale = (float)scale; d.applyScale = scale != 0.0 && scale != 1.0; d.causal = causal;
+  d.maskValue = dt == BFLOAT16 ? 65504.0f : 1.0e9f;
+  std::vector<NDArray*> reads = {q0, v0, k0};
+  std::vector<NDArray*> writes = {c.output(0)};
+  if (wantW) writes.push_back(c.outputs[1]);
+  if (wantL) writes.push_back(c.outputs[2]);
+  if (d.B * d.Tq == 0) return;
+  prepareSpecialUse(writes, reads);
+  const bool unitInner = q.strideAt(2) == 1 && k.strideAt(2) == 1 && v.strideAt(2) == 1 && out.strideAt(2) == 1;
+  if (!wantW && !wantL && unitInner && attentionFusedSupported(dt, d)) {
+    d.qB = q.strideAt(0); d.qT = q.strideAt(1); d.kB = k.strideAt(0); d.kT = k.strideAt(1);
+    d.vB = v.strideAt(0); d.vT = v.strideAt(1); d.oB = out.strideAt(0); d.oT = out.strideAt(1);
+    launchAttentionFused(stream(), dt, q.specialBuffer(), k.specialBuffer(), v.specialBuffer(), out.specialBuffer(), d);
+  } else {
+    // composition: logits = q k^T -> fix-up (scale, clip, mask) -> softmax -> out = weights v
+    NDArray logits, weights;
+    std::shared_ptr<DataBuffer> tmpL, tmpW;
+    auto dense = [&](std::shared_ptr<DataBuffer>& hold) {
+      NDArray t;
+      hold = std::make_shared<DataBuffer>((void*)nullptr, (void*)nullptr, (size_t)(d.B * d.Tq * d.Tv) * sizeOf(dt), dt);
+      hold->allocateSpecial();
+      t.buf = hold;
+      t.si = makeShapeInfo(dt, 'c', {d.B, d.Tq, d.Tv});
+      return t;
+    };
+    if (wantL) { logits = as3d(c.outputs[2]); ND4J_REQUIRE(logits.sizeAt(0) == d.B && logits.sizeAt(1) == d.Tq && logits.sizeAt(2) == d.Tv && logits.dataType() == dt, "dot_product_attention_v2: logits output must be [batch, Tq, Tv]"); }
+    else logits = dense(tmpL);
+    if (wantW) { weights = as3d(c.outputs[1]); ND4J_REQUIRE(weights.sizeAt(0) == d.B && weights.sizeAt(1) == d.Tq && weights.sizeAt(2) == d.Tv && weights.dataType() == dt, "dot_product_attention_v2: weights output must be [batch, Tq, Tv]"); }
+    else weights = dense(tmpW);
+    ND4J_REQUIRE(logits.strideAt(2) == 1 && logits.strideAt(1) == d.Tv && logits.strideAt(0) == d.Tq * d.Tv, "dot_product_attention_v2: logits output must be dense row-major");
+    GemmDesc g1;
+    g1.M = d.Tq; g1.N = d.Tv; g1.K = d.D; g1.batch = d.B;
+    g1.aRow = q.strideAt(1); g1.aCol = q.strideAt(2); g1.aBatch = q.strideAt(0);
+    g1.bRow = k.strideAt(2); g1.bCol = k.strideAt(1); g1.bBatch = k.strideAt(0);   // k^T
+    g1.cRow = logits.strideAt(1); g1.cCol = logits.strideAt(2); g1.cBatch = logits.strideAt(0);
+    launchGemm(stream(), dt, q.specialBuffer(), k.specialBuffer(), logits.specialBuffer(), g1);
+    launchAttentionLogitsFixup(stream(), dt, logits.specialBuffer(), d);
+    RowPlan rp = buildRowPlan(logits.shapeInfo(), weights.shapeInfo(), 2);
+    launchSoftmax(stream(), dt, logits.specialBuffer(), weights.specialBuffer(), rp, true);
+    GemmDesc g2;
+    g2.M = d.Tq; g2.N = d.Dv; g2.K = d.Tv; g2.batch = d.B;
+    g2.aRow = weights.strideAt(1); g2.aCol = weights.strideAt(2); g2.aBatch = weights.strideAt(0);
+    g2.bRow = v.strideAt(1); g2.bCol = v.strideAt(2); g2.bBatch = v.strideAt(0);
+    g2.cRow = out.strideAt(1); g2.cCol = out.strideAt(2); g2.cBatch = out.strideAt(0);
+    launchGemm(stream(), dt, weights.specialBuffer(), v.specialBuffer(), out.specialBuffer(), g2);
+    if (tmpL || tmpW) HIP_CHECK(hipStreamSynchronize(stream()));  // temporaries are released on return
+  }
+  registerSpecialUse(writes, reads);
+}
+static std::vector<std::vector<LongType>> attentionShapeFn(Context& c) {
+  // The reference's shape function (dot_product_attention_v2.cpp:132-183) reports [batch, Tq, dim] for the weights
+  // and logits of rank-3 inputs, which cannot hold what doAttention writes; this one reports [batch, Tq, Tv].
+  NDArray* q = c.input(0); NDArray* v = c.input(1);
+  DataType dt = q->dataType();
+  std::vector<LongType> qs = shapeOf(q), vs = shapeOf(v);
+  ND4J_REQUIRE(qs.size() >= 2 && qs.size() == vs.size(), "Queries and values must be same ranks!");
+  std::vector<LongType> o(qs.begin(), qs.end() - 1), w(qs.begin(), qs.end() - 1);
+  o.push_back(vs.back());
+  w.push_back(vs[vs.size() - 2]);
+  return {makeShapeInfo(dt, 'c', o), makeShapeInfo(dt, 'c', w), makeShapeInfo(dt, 'c', w)};
+}
+
+// ---- argmax / argmin ---------------------------------------------------------------------------------------------------------
+// generic/reduce/argmax.cpp:38-103: dims from IArgs or from input 1; BArg0 keepDims; DArg0 output dtype (INT64)
+static std::vector<LongType> argDims(Context& c) {
+  std::vector<LongType> dims = c.iArgs;
+  if (c.width() > 1 && dims.empty()) {
+    NDArray* ax = c.input(1);
+    ax->buf->syncToPrimary();
+    for (LongType i = 0; i < ax->lengthOf(); i++) {
+      if (ax->dataType() == INT64) dims.push_back(ax->hostAs<LongType>()[i * (ax->rankOf() ? ax->strideAt(ax->rankOf() - 1) : 1)]);
+      else if (ax->dataType() == INT32) dims.push_back(ax->hostAs<int>()[i * (ax->rankOf() ? ax->strideAt(ax->rankOf() - 1) : 1)]);
+      else ND4J_THROW("ArgMax: axis array must be INT32 or INT64");
+    }
+  }
+  return dims;
+}
+static void argExec(Context& c, int opNum, const char* name) {
+  NDArray* x = c.input(0);
+  NDArray* z = c.output(0);
+  if (z->isEmpty() || z->lengthOf() < 1) return;
+  auto raw = argDims(c);
+  for (auto d : raw) if (d != 2147483647LL) ND4J_REQUIRE((d < 0 ? d + x->rankOf() : d) < x->rankOf() && (d < 0 ? d + x->rankOf() : d) >= 0, std::string(name) + ": axis can't be above rank");
+  auto dims = normalizeDims(x->rankOf(), raw.data(), (LongType)raw.size(), name);
+  runIndexReduce(name, opNum, x, z, dims);
+}
+static std::vector<std::vector<LongType>> argShapeFn(Context& c) {
+  NDArray* x = c.input(0);
+  DataType dt = c.dArgs.empty() ? INT64 : c.dArgs[0];
+  if (x->rankOf() == 0) return {scalarShapeInfo(INT64)};
+  auto raw = argDims(c);
+  const bool keepDims = bArg(c, 0, false);
+  auto dims = normalizeDims(x->rankOf(), raw.data(), (LongType)raw.size(), "ArgMax");
+  if (dims.empty()) return {scalarShapeInfo(dt)};
+  std::vector<LongType> out;
+  for (int d = 0; d < x->rankOf(); d++) {
+    bool red = std::find(dims.begin(), dims.end(), (LongType)d) != dims.end();
+    if (red) { ND4J_REQUIRE(x->sizeAt(d) != 0, "ArgMax: you can't reduce along axis with 0 in shape"); if (keepDims) out.push_back(1); }
+    else out.push_back(x->sizeAt(d));
+  }
+  return {makeShapeInfo(dt, 'c', out)};
+}
+
+// ---- glue ops for the decode step ----------------------------------------------------------------------------------------------
+// gather (generic/transforms/gather.cpp:34): rows of a dense 2-D table picked by an index array, axis 0
+static void gatherExec(Context& c) {
+  NDArray* table = c.input(0);
+  ND4J_REQUIRE(c.width() > 1, "GATHER OP: nd4j-hip takes the indices as the second input array");
+  NDArray* idx = c.input(1);
+  NDArray* z = c.output(0);
+  const LongType axis = iArg(c, 0, 0);
+  ND4J_REQUIRE(axis == 0 && table->rankOf() == 2 && table->strideAt(1) == 1 && table->strideAt(0) == table->sizeAt(1),
+               "GATHER OP: nd4j-hip implements axis 0 of a dense rank-2 input");
+  ND4J_REQUIRE(z->dataType() == table->dataType(), "GATHER OP: output must carry the input's data type");
+  ND4J_REQUIRE(z->lengthOf() == idx->lengthOf() * table->sizeAt(1), "GATHER OP: wrong output length");
+  EwPlan pz = buildEwPlan({z->shapeInfo(), z->shapeInfo()});
+  EwPlan pi = buildEwPlan({idx->shapeInfo(), idx->shapeInfo()});
+  ND4J_REQUIRE(pz.contiguous && pi.contiguous, "GATHER OP: indices and output must be dense");
+  if (z->isEmpty() || z->lengthOf() == 0) return;
+  prepareSpecialUse({z}, {table, idx});
+  launchGatherRows(stream(), table->dataType(), idx->dataType(), table->specialBuffer(), idx->specialBuffer(), z->specialBuffer(), idx->lengthOf(), table->sizeAt(1), table->sizeAt(0));
+  registerSpecialUse({z}, {table, idx});
+}
+static std::vector<std::vector<LongType>> gatherShapeFn(Context& c) {
+  NDArray* table = c.input(0); NDArray* idx = c.input(1);
+  std::vector<LongType> out = shapeOf(idx);
+  for (int d = 1; d < table->rankOf(); d++) out.push_back(table->sizeAt(d));
+  return {makeShapeInfo(table->dataType(), 'c', out)};
+}
+
+// broadcastable add / multiply / subtract / divide (generic/broadcastable/*.cpp, generic/helpers/BroadcastHelper.h:43-66):
+// numpy-style broadcasting of y against x realised with zero strides
+static std::vector<LongType> broadcastShape(const NDArray* x, const NDArray* y) {
+  int r = std::max(x->rankOf(), y->rankOf());
+  std::vector<LongType> out(r);
+  for (int i = 0; i < r; i++) {
+    int xd = i - (r - x->rankOf()), yd = i - (r - y->rankOf());
+    LongType xs = xd >= 0 ? x->sizeAt(xd) : 1, ys = yd >= 0 ? y->sizeAt(yd) : 1;
+    ND4J_REQUIRE(xs == ys || xs == 1 || ys == 1, "broadcastable op: shapes " + shapeStr(x) + " and " + shapeStr(y) + " do not broadcast");
+    out[i] = xs == 1 ? ys : xs;
+  }
+  return out;
+}
+static std::vector<LongType> broadcastStrides(const NDArray* a, const std::vector<LongType>& out) {
+  int r = (int)out.size();
+  std::vector<LongType> st(r, 0);
+  for (int i = 0; i < r; i++) {
+    int ad = i - (r - a->rankOf());
+    if (ad >= 0 && a->sizeAt(ad) != 1) st[i] = a->strideAt(ad);
+  }
+  return st;
+}
+static void broadcastableExec(Context& c, PairwiseKind k, const char* name) {
+  ND4J_REQUIRE(c.width() >= 2, std::string(name) + ": two inputs are required");
+  NDArray* x = c.input(0); NDArray* y = c.input(1); NDArray* z = c.output(0);
+  ND4J_REQUIRE(x->dataType() == z->dataType() && y->dataType() == z->dataType() && isFloatType(z->dataType()), std::string(name) + ": nd4j-hip implements same-type float arrays only");
+  if (x->isEmpty() || y->isEmpty() || z->isEmpty()) return;
+  auto out = broadcastShape(x, y);
+  ND4J_REQUIRE(out == shapeOf(z), std::string(name) + ": output shape " + shapeStr(z) + " does not match the broadcast shape");
+  auto xs = broadcastStrides(x, out), ys = broadcastStrides(y, out);
+  auto xsi = makeShapeInfo(x->dataType(), 'c', out, xs.data()), ysi = makeShapeInfo(y->dataType(), 'c', out, ys.data());
+  EwPlan p = buildEwPlan({z->shapeInfo(), xsi.data(), ysi.data()});
+  prepareSpecialUse({z}, {x, y});
+  launchPairwise(stream(), k, x->dataType(), y->dataType(), z->dataType(), x->specialBuffer(), y->specialBuffer(), z->specialBuffer(), p);
+  registerSpecialUse({z}, {x, y});
+}
+static std::vector<std::vector<LongType>> broadcastableShapeFn(Context& c) {
+  NDArray* x = c.input(0); NDArray* y = c.input(1);
+  return {makeShapeInfo(x->dataType(), x->ordering(), broadcastShape(x, y))};
+}
+
+// concat (generic/transforms/concat.cpp:34): inputs joined along IArg0 (or the last input when BArg0 is set)
+static void concatExec(Context& c) {
+  int n = c.width();
+  ND4J_REQUIRE(n >= 1, "CONCAT OP: at least one input is required");
+  LongType axis;
+  if (bArg(c, 0, false)) {
+    NDArray* ax = c.input(n - 1);
+    ax->buf->syncToPrimary();
+    axis = ax->dataType() == INT64 ? ax->hostAs<LongType>()[0] : ax->hostAs<int>()[0];
+    n--;
+  } else axis = iArg(c, 0, 0);
+  NDArray* z = c.output(0);
+  const int rank = z->rankOf();
+  if (axis < 0) axis += rank;
+  ND4J_REQUIRE(axis >= 0 && axis < rank, "CONCAT OP: axis out of range");
+  std::vector<NDArray*> reads;
+  LongType total = 0;
+  for (int i = 0; i < n; i++) {
+    NDArray* a = c.input(i);
+    if (a->isEmpty()) continue;
+    ND4J_REQUIRE(a->rankOf() == rank && a->dataType() == z->dataType(), "CONCAT OP: inputs must share rank and data type with the output");
+    for (int d = 0; d < rank; d++) if (d != axis) ND4J_REQUIRE(a->sizeAt(d) == z->sizeAt(d), "CONCAT OP: input shapes differ outside the concat axis");
+    total += a->sizeAt((int)axis);
+    reads.push_back(a);
+  }
+  ND4J_REQUIRE(total == z->sizeAt((int)axis), "CONCAT OP: output extent along the axis does not match the inputs");
+  prepareSpecialUse(std::vector<NDArray*>{z}, reads);
+  LongType at = 0;
+  for (NDArray* a : reads) {
+    // view of z covering this input's slot
+    std::vector<LongType> shp = shapeOf(a), st(rank);
+    for (int d = 0; d < rank; d++) st[d] = z->strideAt(d);
+    auto vsi = makeShapeInfo(z->dataType(), 'c', shp, st.data());
+    EwPlan p = buildEwPlan({vsi.data(), a->shapeInfo()});
+    char* dst = (char*)z->specialBuffer() + (size_t)(at * z->strideAt((int)axis)) * sizeOf(z->dataType());
+    launchUnary(stream(), U_IDENTITY, a->dataType(), z->dataType(), a->specialBuffer(), dst, p);
+    at += a->sizeAt((int)axis);
+  }
+  registerSpecialUse(std::vector<NDArray*>{z}, reads);
+}
+static std::vector<std::vector<LongType>> concatShapeFn(Context& c) {
+  int n = c.width();
+  LongType axis = iArg(c, 0, 0);
+  if (bArg(c, 0, false)) { NDArray* ax = c.input(n - 1); ax->buf->syncToPrimary(); axis = ax->dataType() == INT64 ? ax->hostAs<LongType>()[0] : ax->hostAs<int>()[0]; n--; }
+  NDArray* first = c.input(0);
+  std::vector<LongType> out = shapeOf(first);
+  if (axis < 0) axis += first->rankOf();
+  ND4J_REQUIRE(axis >= 0 && axis < first->rankOf(), "CONCAT OP: axis out of range");
+  out[axis] = 0;
+  for (int i = 0; i < n; i++) if (!c.input(i)->isEmpty()) out[axis] += c.input(i)->sizeAt((int)axis);
+  return {makeShapeInfo(first->dataType(), 'c', out)};
+}
+
+// ---- registry ---------------------------------------------------------------------------------------------------------------
+static std::map<LongType, OpDescriptor>& byHash() {
+  static std::map<LongType, OpDescriptor> m;
+  return m;
+}
+static std::map<std::string, LongType>& byName() {
+  static std::map<std::string, LongType> m;
+  return m;
+}
+static void reg(const std::string& name, int nIn, int nOut, bool inplace, int nT, int nI, std::function<void(Context&)> exec,
+                std::function<std::vector<std::vector<LongType>>(Context&)> shapeFn) {
+  OpDescriptor d{name, opHash(name), nIn, nOut, inplace, nT, nI, std::move(exec), std::move(shapeFn)};
+  byName()[name] = d.hash;
+  byHash()[d.hash] = std::move(d);
+}
+static void ensureRegistered() {
+  static std::once_flag once;
+  std::call_once(once, [] {
+    // arities as declared by the reference's *_OP_IMPL macros
+    for (const char* alias : {"matmul", "mMul", "mmul", "gemm", "gemv", "dot"}) reg(alias, 2, 1, false, 0, -2, matmulExec, matmulShapeFn);
+    reg("softmax", 1, 1, true, 0, 0, softmaxExec, sameAsInputShapeFn);
+    reg("layer_norm", 2, 1, false, 0, -1, layerNormExec, sameAsInputShapeFn);
+    reg("dot_product_attention_v2", -2, -1, false, -2, -2, attentionExec, attentionShapeFn);
+    reg("argmax", 1, 1, false, 0, -2, [](Context& c) { argExec(c, 0, "ArgMax"); }, argShapeFn);
+    reg("argmin", 1, 1, false, 0, -2, [](Context& c) { argExec(c, 1, "ArgMin"); }, argShapeFn);
+    reg("gather", 1, 1, false, 0, -2, gatherExec, gatherShapeFn);
+    reg("concat", -1, 1, false, 0, 0, concatExec, concatShapeFn);
+    reg("add", 2, 1, true, 0, 0, [](Context& c) { broadcastableExec(c, P_ADD, "ADD OP"); }, broadcastableShapeFn);
+    reg("subtract", 2, 1, true, 0, 0, [](Context& c) { broadcastableExec(c, P_SUB, "SUBTRACT OP"); }, broadcastableShapeFn);
+    reg("multiply", 2, 1, true, 0, 0, [](Context& c) { broadcastableExec(c, P_MUL, "MULTIPLY OP"); }, broadcastableShapeFn);
+    reg("divide", 2, 1, true, 0, 0, [](Context& c) { broadcastableExec(c, P_DIV, "DIVIDE OP"); }, broadcastableShapeFn);
+  });
+}
+const OpDescriptor* findOp(LongType hash) {
+  ensureRegistered();
+  auto it = byHash().find(hash);
+  return it == byHash().end() ? nullptr : &it->second;
+}
+const OpDescriptor* findOpByName(const std::string& name) {
+  ensureRegistered();
+  auto it = byName().find(name);
+  return it == byName().end() ? nullptr : findOp(it->second);
+}
+const char* allCustomOps() {
+  ensureRegistered();
+  static std::string list;
+  static std::once_flag once;
+  std::call_once(once, [] {
+    for (auto& kv : byName()) {
+      const OpDescriptor& d = byHash()[kv.second];
+      list += d.name + ":" + std::to_string(d.hash) + ":" + std::to_string(d.nIn) + ":" + std::to_string(d.nOut) + ":" +
+              std::to_string((int)d.inplace) + ":" + std::to_string(d.nT) + ":" + std::to_string(d.nI) + ":;";
+    }
+  });
+  return list.c_str();
+}
+
+void executeOp(const OpDescriptor& op, Context& ctx) {
+  // DeclarableOp::execute validations (ops/declarable/impl/DeclarableOp.cpp:866-919): arity and null checks
+  if (op.nIn > 0) ND4J_REQUIRE(ctx.width() >= op.nIn, "Op [" + op.name + "] expects at least " + std::to_string(op.nIn) + " input arrays, got " + std::to_string(ctx.width()));
+  for (int i = 0; i < ctx.width(); i++) ND4J_REQUIRE(ctx.inputs[i] != nullptr, "Op [" + op.name + "]: input array " + std::to_string(i) + " is null");
+  ND4J_REQUIRE(!ctx.outputs.empty() && ctx.outputs[0] != nullptr, "Op [" + op.name + "]: output array 0 is missing (outputs must be supplied; use calculateOutputShapes2 to size them)");
+  op.exec(ctx);
+}
+
+}  // namespace ops
+}  // namespace nd4jhip

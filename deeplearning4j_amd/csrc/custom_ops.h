@@ -1,0 +1,33 @@
+// Registry of declarable ("custom") ops reached through execCustomOp2 / calculateOutputShapes2.
+#pragma once
+#include <functional>
+#include <string>
+#include <vector>
+
+#include "runtime.h"
+
+namespace nd4jhip {
+namespace ops {
+
+struct OpDescriptor {
+  std::string name;
+  LongType hash;
+  int nIn, nOut;      // declared arities as the reference registers them (negative = variable)
+  bool inplace;
+  int nT, nI;
+  std::function<void(Context&)> exec;
+  std::function<std::vector<std::vector<LongType>>(Context&)> shapeFn;
+};
+
+LongType opHash(const std::string& name);  // helpers/impl/helper_hash.cpp:33-70 of the reference
+const OpDescriptor* findOp(LongType hash);
+const OpDescriptor* findOpByName(const std::string& name);
+const char* allCustomOps();                // "name:hash:nIn:nOut:inplace:nT:nI:;" per op (OpRegistrator.cpp:106-125)
+void executeOp(const OpDescriptor& op, Context& ctx);
+
+}  // namespace ops
+
+// shared with the legacy facade
+void runIndexReduce(const char* fn, int opNum, NDArray* x, NDArray* z, const std::vector<LongType>& dims);
+
+}  // namespace nd4jhip

@@ -1,0 +1,124 @@
+// Host-callable launchers of the HIP kernels.  Callers (the facade) validate dtypes and shapes and
+// build the plans; launchers only pick a kernel variant and a grid.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "types.h"
+
+namespace nd4jhip {
+
+// ---- elementwise ---------------------------------------------------------------------------------
+enum UnaryKind : int {
+  // TransformStrict (loops/legacy_ops.h:54-64 of the reference)
+  U_COS, U_EXP, U_LOG, U_SIGMOID, U_SIN, U_SOFTPLUS, U_TANH, U_SWISH, U_ERF, U_GELU, U_PRECISE_GELU,
+  // TransformFloat (legacy_ops.h:67)
+  U_SQRT, U_RSQRT,
+  // TransformSame (legacy_ops.h:40-44) and TransformAny Assign (legacy_ops.h:46)
+  U_ABS, U_NEG, U_SQUARE, U_RECIPROCAL, U_IDENTITY, U_ONE_MINUS, U_CUBE,
+  U_COUNT
+};
+enum PairwiseKind : int {
+  P_ADD, P_COPY, P_DIV, P_MUL, P_RSUB, P_SUB, P_MAX, P_MIN, P_RDIV, P_SQSUB, P_COUNT
+};
+
+// Joint iteration plan of up to three operands of equal length.
+struct EwPlan {
+  int nOperands = 0;       // operand 0 is the output
+  LongType length = 0;
+  bool sameShape = true;   // false: every operand is walked through its own shape (own[])
+  bool contiguous = false; // collapsed rank 1 and unit strides everywhere
+  bool index32 = true;     // length and every reachable offset fit 31 bits
+  int rank = 0;            // collapsed common shape
+  LongType shape[MAX_DEV_RANK];
+  LongType stride[3][MAX_DEV_RANK];
+  DevShape own[3];
+};
+
+void launchUnary(hipStream_t s, UnaryKind k, DataType xdt, DataType zdt, const void* x, void* z, const EwPlan& p);
+void launchPairwise(hipStream_t s, PairwiseKind k, DataType xdt, DataType ydt, DataType zdt, const void* x,
+                    const void* y, void* z, const EwPlan& p);
+// z[outer.., c] = x[outer.., c] (op) v[c]: broadcast of a vector along the last axis of a dense array
+void launchRowBroadcast(hipStream_t s, PairwiseKind k, DataType dt, const void* x, const void* v, void* z,
+                        LongType rows, LongType cols);
+// z = x (op) scalar
+void launchScalarOp(hipStream_t s, PairwiseKind k, DataType dt, const void* x, double scalar, void* z, const EwPlan& p);
+
+// ---- reductions ----------------------------------------------------------------------------------
+enum ReduceKind : int {
+  R_SUM, R_MAX, R_MIN, R_PROD, R_ASUM, R_AMAX, R_AMIN,        // ReduceSame 0..6
+  R_MEAN, R_AMEAN, R_NORM1, R_NORM2, R_NORMMAX, R_SQNORM,     // ReduceFloat 0,1,2,3,4,7
+  R_COUNT
+};
+enum IndexKind : int { I_MAX, I_MIN, I_AMAX, I_AMIN, I_COUNT };
+
+// outer = kept dims (one output element each), inner = reduced dims
+struct ReducePlan {
+  DevShape outer;        // strides into x
+  DevShape inner;        // strides into x
+  DevShape zOuter;       // same shape as outer, strides into z
+  LongType outerLen = 1, innerLen = 1;
+  bool index32 = true;
+  bool zLinear = false;  // write z[o] instead of walking zOuter (index reduce)
+};
+
+void launchReduce(hipStream_t s, ReduceKind k, DataType xdt, DataType zdt, const void* x, void* z, const ReducePlan& p,
+                  void* scratch, size_t scratchBytes);
+void launchIndexReduce(hipStream_t s, IndexKind k, DataType xdt, DataType zdt, const void* x, void* z,
+                       const ReducePlan& p, void* scratch, size_t scratchBytes);
+
+// ---- row ops ---------------------------------------------------------------------------------------
+struct RowPlan {
+  DevShape outerX;     // row start offsets of the input
+  DevShape outerZ;     // row start offsets of the output
+  LongType rows = 1, rowLen = 1;
+  LongType xInner = 1, zInner = 1;  // element stride along the row
+  bool index32 = true;
+};
+// clampMode: true = the reference's same-shape branch (finite max, +-88 clamp, sum floor 1e-6)
+void launchSoftmax(hipStream_t s, DataType dt, const void* x, void* z, const RowPlan& p, bool clampMode);
+void launchLayerNormRows(hipStream_t s, DataType dt, const void* x, const void* gain, const void* bias, void* z,
+                         const RowPlan& p, float eps);
+// generic layer norm over arbitrary axes: one block per statistics group
+struct LnGenericPlan {
+  DevShape outerX, innerX, outerZ, innerZ;
+  LongType outerLen = 1, innerLen = 1;
+  int channelInInner = 1;   // does the gain/bias axis belong to the reduced set
+  int channelPos = 0;       // its position inside that set
+};
+void launchLayerNormGeneric(hipStream_t s, DataType dt, const void* x, const void* gain, const void* bias, void* z,
+                            const LnGenericPlan& p, float eps);
+
+// ---- GEMM ------------------------------------------------------------------------------------------
+struct GemmDesc {
+  LongType M = 0, N = 0, K = 0, batch = 1;
+  LongType aRow = 0, aCol = 0;   // element strides of op(A)[m][k]
+  LongType bRow = 0, bCol = 0;   // element strides of op(B)[k][n]
+  LongType cRow = 0, cCol = 0;
+  LongType aBatch = 0, bBatch = 0, cBatch = 0;
+  float alpha = 1.f, beta = 0.f;
+};
+void launchGemm(hipStream_t s, DataType dt, const void* A, const void* B, void* C, const GemmDesc& d);
+
+// ---- attention -------------------------------------------------------------------------------------
+struct AttnDesc {
+  LongType B = 0, Tq = 0, Tv = 0, D = 0, Dv = 0;
+  LongType qB = 0, qT = 0, kB = 0, kT = 0, vB = 0, vT = 0, oB = 0, oT = 0;  // innermost stride is 1
+  float scale = 1.f;
+  bool applyScale = false;
+  bool causal = false;
+  float maskValue = 1e9f;
+};
+// fused path (no logits/weights written)
+bool attentionFusedSupported(DataType dt, const AttnDesc& d);
+void launchAttentionFused(hipStream_t s, DataType dt, const void* q, const void* k, const void* v, void* out,
+                          const AttnDesc& d);
+// logits[b,i,j] = clip(scale * logits, +-1e4) - mask  (in place, row-major [B,Tq,Tv])
+void launchAttentionLogitsFixup(hipStream_t s, DataType dt, void* logits, const AttnDesc& d);
+
+// ---- misc ------------------------------------------------------------------------------------------
+// z[i, :] = table[idx[i], :]
+void launchGatherRows(hipStream_t s, DataType dt, DataType idxDt, const void* table, const void* idx, void* z,
+                      LongType nIdx, LongType rowLen, LongType tableRows);
+void launchFill(hipStream_t s, void* p, int byteValue, size_t bytes);
+
+}  // namespace nd4jhip

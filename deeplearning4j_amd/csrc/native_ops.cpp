@@ -1,0 +1,842 @@
+// The C-ABI facade: handle types, buffers, descriptors, device utilities and the legacy exec* loops.
+// Every function catches exceptions and records them in the error slot, the way the reference's
+// facade does (libnd4j/include/legacy/cpu/NativeOps.cpp:1118-1121).
+#include "../../include/nd4jhip/NativeOps.h"
+
+#include <cstring>
+
+#include "custom_ops.h"
+#include "kernels.h"
+#include "plan.h"
+#include "runtime.h"
+
+using namespace nd4jhip;
+
+struct Nd4jHipDataBuffer : public InteropDataBuffer {};
+struct Nd4jHipNDArray : public NDArray {};
+struct Nd4jHipContext : public Context {};
+struct Nd4jHipShapeList : public ShapeList {};
+struct Nd4jHipTadPack : public TadPack {};
+struct Nd4jHipConstantShapeBuffer : public ConstantShapeBuffer {};
+struct Nd4jHipLaunchContext : public LaunchContext {};
+
+#define GUARD_BEGIN try {
+#define GUARD_END(ret)                         \
+  }                                            \
+  catch (std::exception & e) {                 \
+    errorRef().set(1, e.what());               \
+    return ret;                                \
+  }                                            \
+  catch (...) {                                \
+    errorRef().set(1, "unknown native error"); \
+    return ret;                                \
+  }
+#define GUARD_END_VOID GUARD_END()
+
+static NDArray* arr(OpaqueNDArray a, const char* fn, const char* name) {
+  if (a == nullptr) ND4J_THROW(std::string(fn) + ": " + name + " is null");
+  return static_cast<NDArray*>(a);
+}
+static hipStream_t execStream() { return LaunchContext::defaultContext()->execStream; }
+
+extern "C" {
+
+// ---- library / device ------------------------------------------------------------------------------
+void initializeDevicesAndFunctions(void) {
+  GUARD_BEGIN
+  LaunchContext::defaultContext();
+  GUARD_END_VOID
+}
+void initializeShapeCache(void) {}
+void initializeTadCache(void) {}
+int getAvailableDevices(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) { (void)hipGetLastError(); return 0; }
+  return n;
+}
+int setDevice(int deviceId) {
+  GUARD_BEGIN
+  HIP_CHECK(hipSetDevice(deviceId));
+  return 1;
+  GUARD_END(0)
+}
+int getDevice(void) {
+  int d = 0;
+  if (hipGetDevice(&d) != hipSuccess) { (void)hipGetLastError(); return 0; }
+  return d;
+}
+const char* getDeviceName(int device) {
+  static thread_local char name[256];
+  hipDeviceProp_t p;
+  if (hipGetDeviceProperties(&p, device) != hipSuccess) { (void)hipGetLastError(); return "unknown"; }
+  snprintf(name, sizeof(name), "%s (%s)", p.name, p.gcnArchName);
+  return name;
+}
+int getDeviceMajor(int device) {
+  hipDeviceProp_t p;
+  if (hipGetDeviceProperties(&p, device) != hipSuccess) { (void)hipGetLastError(); return 0; }
+  return p.major;
+}
+int getDeviceMinor(int device) {
+  hipDeviceProp_t p;
+  if (hipGetDeviceProperties(&p, device) != hipSuccess) { (void)hipGetLastError(); return 0; }
+  return p.minor;
+}
+Nd4jLong getDeviceFreeMemory(int device) {
+  GUARD_BEGIN
+  int cur = 0;
+  HIP_CHECK(hipGetDevice(&cur));
+  if (device >= 0 && device != cur) HIP_CHECK(hipSetDevice(device));
+  size_t f = 0, t = 0;
+  HIP_CHECK(hipMemGetInfo(&f, &t));
+  if (device >= 0 && device != cur) HIP_CHECK(hipSetDevice(cur));
+  return (Nd4jLong)f;
+  GUARD_END(0)
+}
+Nd4jLong getDeviceFreeMemoryDefault(void) { return getDeviceFreeMemory(-1); }
+Nd4jLong getDeviceTotalMemory(int device) {
+  hipDeviceProp_t p;
+  if (hipGetDeviceProperties(&p, device) != hipSuccess) { (void)hipGetLastError(); return 0; }
+  return (Nd4jLong)p.totalGlobalMem;
+}
+void enableDebugMode(bool e) { Environment::get().debug = e; }
+void enableVerboseMode(bool e) { Environment::get().verbose = e; }
+void setOmpNumThreads(int) {}
+int ompGetMaxThreads(void) { return 1; }
+void setElementThreshold(int) {}
+void setTADThreshold(int) {}
+int lastErrorCode(void) {
+  std::lock_guard<std::mutex> g(errorRef().lock);
+  return errorRef().code;
+}
+const char* lastErrorMessage(void) {
+  // fetching the message consumes the error: the code goes back to 0 (execution/impl/ErrorReference.cpp:28-34)
+  static thread_local std::string copy;
+  std::lock_guard<std::mutex> g(errorRef().lock);
+  copy = errorRef().message;
+  errorRef().code = 0;
+  return copy.c_str();
+}
+
+Nd4jPointer mallocHost(Nd4jLong memorySize, int) {
+  GUARD_BEGIN
+  void* p = nullptr;
+  HIP_CHECK(hipHostMalloc(&p, (size_t)memorySize + 8, hipHostMallocDefault));
+  return p;
+  GUARD_END(nullptr)
+}
+Nd4jPointer mallocDevice(Nd4jLong memorySize, int, int) {
+  GUARD_BEGIN
+  void* p = nullptr;
+  HIP_CHECK(hipMalloc(&p, (size_t)memorySize + 8));
+  return p;
+  GUARD_END(nullptr)
+}
+int freeHost(Nd4jPointer pointer) {
+  GUARD_BEGIN
+  HIP_CHECK(hipHostFree(pointer));
+  return 1;
+  GUARD_END(0)
+}
+int freeDevice(Nd4jPointer pointer, int) {
+  GUARD_BEGIN
+  HIP_CHECK(hipFree(pointer));
+  return 1;
+  GUARD_END(0)
+}
+Nd4jPointer createStream(void) {
+  GUARD_BEGIN
+  auto* s = new hipStream_t;
+  HIP_CHECK(hipStreamCreateWithFlags(s, hipStreamNonBlocking));
+  return s;
+  GUARD_END(nullptr)
+}
+Nd4jPointer createEvent(void) {
+  GUARD_BEGIN
+  hipEvent_t e;
+  HIP_CHECK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+  return (Nd4jPointer)e;
+  GUARD_END(nullptr)
+}
+Nd4jPointer nd4jhipCreateTimingEvent(void) {
+  GUARD_BEGIN
+  hipEvent_t e;
+  HIP_CHECK(hipEventCreate(&e));
+  return (Nd4jPointer)e;
+  GUARD_END(nullptr)
+}
+float nd4jhipEventElapsedMs(Nd4jPointer a, Nd4jPointer b) {
+  GUARD_BEGIN
+  float ms = 0;
+  HIP_CHECK(hipEventElapsedTime(&ms, (hipEvent_t)a, (hipEvent_t)b));
+  return ms;
+  GUARD_END(-1.f)
+}
+static hipStream_t streamOf(Nd4jPointer p) { return p ? *reinterpret_cast<hipStream_t*>(p) : execStream(); }
+int registerEvent(Nd4jPointer event, Nd4jPointer stream) {
+  GUARD_BEGIN
+  HIP_CHECK(hipEventRecord((hipEvent_t)event, streamOf(stream)));
+  return 1;
+  GUARD_END(0)
+}
+int destroyEvent(Nd4jPointer event) {
+  GUARD_BEGIN
+  HIP_CHECK(hipEventDestroy((hipEvent_t)event));
+  return 1;
+  GUARD_END(0)
+}
+int streamSynchronize(Nd4jPointer stream) {
+  GUARD_BEGIN
+  HIP_CHECK(hipStreamSynchronize(streamOf(stream)));
+  return 1;
+  GUARD_END(0)
+}
+int eventSynchronize(Nd4jPointer event) {
+  GUARD_BEGIN
+  HIP_CHECK(hipEventSynchronize((hipEvent_t)event));
+  return 1;
+  GUARD_END(0)
+}
+static hipMemcpyKind kindOf(int flags) {
+  switch (flags) {
+    case 0: return hipMemcpyHostToHost;
+    case 1: return hipMemcpyHostToDevice;
+    case 2: return hipMemcpyDeviceToHost;
+    case 3: return hipMemcpyDeviceToDevice;
+    default: ND4J_THROW("UNDEFINED MEMCPY");
+  }
+}
+int memcpySync(Nd4jPointer dst, Nd4jPointer src, Nd4jLong size, int flags, Nd4jPointer) {
+  GUARD_BEGIN
+  HIP_CHECK(hipMemcpy(dst, src, (size_t)size, kindOf(flags)));
+  return 1;
+  GUARD_END(0)
+}
+int memcpyAsync(Nd4jPointer dst, Nd4jPointer src, Nd4jLong size, int flags, Nd4jPointer reserved) {
+  GUARD_BEGIN
+  HIP_CHECK(hipMemcpyAsync(dst, src, (size_t)size, kindOf(flags), streamOf(reserved)));
+  return 1;
+  GUARD_END(0)
+}
+int memsetSync(Nd4jPointer dst, int value, Nd4jLong size, int, Nd4jPointer) {
+  GUARD_BEGIN
+  HIP_CHECK(hipMemset(dst, value, (size_t)size));
+  return 1;
+  GUARD_END(0)
+}
+int memsetAsync(Nd4jPointer dst, int value, Nd4jLong size, int, Nd4jPointer reserved) {
+  GUARD_BEGIN
+  // a fill kernel rather than a memset node, so that callers may capture this call into a graph
+  launchFill(streamOf(reserved), dst, value, (size_t)size);
+  return 1;
+  GUARD_END(0)
+}
+
+OpaqueLaunchContext defaultLaunchContext(void) {
+  GUARD_BEGIN
+  return static_cast<OpaqueLaunchContext>(LaunchContext::defaultContext());
+  GUARD_END(nullptr)
+}
+Nd4jPointer lcScalarPointer(OpaqueLaunchContext lc) { return lc ? lc->scalarBuffer : nullptr; }
+Nd4jPointer lcReductionPointer(OpaqueLaunchContext lc) { return lc ? lc->reductionBuffer : nullptr; }
+Nd4jPointer lcAllocationPointer(OpaqueLaunchContext lc) { return lc ? lc->allocationBuffer : nullptr; }
+Nd4jPointer lcExecutionStream(OpaqueLaunchContext lc) { return lc ? &lc->execStream : nullptr; }
+Nd4jPointer lcCopyStream(OpaqueLaunchContext lc) { return lc ? &lc->copyStream : nullptr; }
+Nd4jPointer lcBlasHandle(OpaqueLaunchContext) { return nullptr; }
+
+// ---- data buffers -----------------------------------------------------------------------------------
+OpaqueDataBuffer* allocateDataBuffer(Nd4jLong elements, int dataType, bool allocateBoth) {
+  GUARD_BEGIN
+  DataType dt = (DataType)dataType;
+  ND4J_REQUIRE(sizeOf(dt) > 0, "allocateDataBuffer: unsupported data type " + std::to_string(dataType));
+  ND4J_REQUIRE(elements >= 0, "allocateDataBuffer: negative length");
+  // zero elements still owns one element, as in the reference (NativeOpsHelpers_DataBuffers.cpp allocateDataBuffer)
+  size_t bytes = (size_t)(elements == 0 ? 1 : elements) * sizeOf(dt);
+  auto* h = new Nd4jHipDataBuffer();
+  h->db = std::make_shared<DataBuffer>(bytes, dt, allocateBoth);
+  return h;
+  GUARD_END(nullptr)
+}
+OpaqueDataBuffer* dbAllocateDataBuffer(Nd4jLong elements, int dataType, bool allocateBoth) {
+  return allocateDataBuffer(elements, dataType, allocateBoth);
+}
+OpaqueDataBuffer* dbCreateExternalDataBuffer(Nd4jLong elements, int dataType, Nd4jPointer primary, Nd4jPointer special) {
+  GUARD_BEGIN
+  DataType dt = (DataType)dataType;
+  ND4J_REQUIRE(sizeOf(dt) > 0, "dbCreateExternalDataBuffer: unsupported data type");
+  auto* h = new Nd4jHipDataBuffer();
+  h->db = std::make_shared<DataBuffer>(primary, special, (size_t)elements * sizeOf(dt), dt);
+  return h;
+  GUARD_END(nullptr)
+}
+OpaqueDataBuffer* dbCreateView(OpaqueDataBuffer* dataBuffer, Nd4jLong length) {
+  GUARD_BEGIN
+  ND4J_REQUIRE(dataBuffer && dataBuffer->db, "dbCreateView: buffer is null");
+  auto* h = new Nd4jHipDataBuffer();
+  h->db = dataBuffer->db;
+  h->offsetBytes = dataBuffer->offsetBytes;
+  (void)length;
+  return h;
+  GUARD_END(nullptr)
+}
+Nd4jPointer dbPrimaryBuffer(OpaqueDataBuffer* b) { return b ? b->primary() : nullptr; }
+Nd4jPointer dbSpecialBuffer(OpaqueDataBuffer* b) { return b ? b->special() : nullptr; }
+Nd4jLong dbBufferLength(OpaqueDataBuffer* b) { return b && b->db ? b->db->numElements() : 0; }
+void dbSetPrimaryBuffer(OpaqueDataBuffer* b, Nd4jPointer p, Nd4jLong numBytes) {
+  GUARD_BEGIN
+  ND4J_REQUIRE(b && b->db, "dbSetPrimaryBuffer: buffer is null");
+  if (b->db->ownsPrimary && b->db->primary) free(b->db->primary);
+  b->db->primary = p; b->db->ownsPrimary = false; b->db->lenBytes = (size_t)numBytes;
+  b->db->tickWritePrimary();
+  GUARD_END_VOID
+}
+void dbSetSpecialBuffer(OpaqueDataBuffer* b, Nd4jPointer p, Nd4jLong numBytes) {
+  GUARD_BEGIN
+  ND4J_REQUIRE(b && b->db, "dbSetSpecialBuffer: buffer is null");
+  if (b->db->ownsSpecial && b->db->special) HIP_CHECK(hipFree(b->db->special));
+  b->db->special = p; b->db->ownsSpecial = false; b->db->lenBytes = (size_t)numBytes;
+  b->db->tickWriteSpecial();
+  GUARD_END_VOID
+}
+void dbAllocatePrimaryBuffer(OpaqueDataBuffer* b) {
+  GUARD_BEGIN
+  ND4J_REQUIRE(b && b->db, "dbAllocatePrimaryBuffer: buffer is null");
+  b->db->allocatePrimary();
+  GUARD_END_VOID
+}
+void dbAllocateSpecialBuffer(OpaqueDataBuffer* b) {
+  GUARD_BEGIN
+  ND4J_REQUIRE(b && b->db, "dbAllocateSpecialBuffer: buffer is null");
+  b->db->allocateSpecial();
+  GUARD_END_VOID
+}
+void dbExpandBuffer(OpaqueDataBuffer* b, Nd4jLong elements) {
+  GUARD_BEGIN
+  ND4J_REQUIRE(b && b->db, "dbExpandBuffer: buffer is null");
+  b->db->expand((size_t)elements * sizeOf(b->db->dtype));
+  GUARD_END_VOID
+}
+void dbExpand(OpaqueDataBuffer* b, Nd4jLong elements) { dbExpandBuffer(b, elements); }
+int dbUseCount(OpaqueDataBuffer* b) { return b && b->db ? (int)b->db.use_count() : 0; }
+void dbSyncToSpecial(OpaqueDataBuffer* b) {
+  GUARD_BEGIN
+  ND4J_REQUIRE(b && b->db, "dbSyncToSpecial: buffer is null");
+  b->db->syncToSpecial();
+  GUARD_END_VOID
+}
+void dbSyncToPrimary(OpaqueDataBuffer* b) {
+  GUARD_BEGIN
+  ND4J_REQUIRE(b && b->db, "dbSyncToPrimary: buffer is null");
+  b->db->syncToPrimary();
+  GUARD_END_VOID
+}
+void dbTickHostRead(OpaqueDataBuffer* b) { if (b && b->db) b->db->tickReadPrimary(); }
+void dbTickHostWrite(OpaqueDataBuffer* b) { if (b && b->db) b->db->tickWritePrimary(); }
+void dbTickDeviceRead(OpaqueDataBuffer* b) { if (b && b->db) b->db->tickReadSpecial(); }
+void dbTickDeviceWrite(OpaqueDataBuffer* b) { if (b && b->db) b->db->tickWriteSpecial(); }
+void dbClose(OpaqueDataBuffer* b) {
+  GUARD_BEGIN
+  if (b && b->db) b->db->close();
+  GUARD_END_VOID
+}
+int dbDeviceId(OpaqueDataBuffer* b) { return b && b->db ? b->db->deviceId : 0; }
+void dbSetDeviceId(OpaqueDataBuffer* b, int deviceId) { if (b && b->db) b->db->deviceId = deviceId; }
+int dbLocality(OpaqueDataBuffer* b) {
+  if (!b || !b->db) return 0;
+  bool p = b->db->isPrimaryActual(), s = b->db->isSpecialActual();
+  if (p && !s) return -1;
+  if (s && !p) return 1;
+  return 0;
+}
+void deleteDataBuffer(OpaqueDataBuffer* b) { delete b; }
+
+// ---- shape descriptors --------------------------------------------------------------------------------
+OpaqueConstantShapeBuffer shapeBufferEx(int rank, Nd4jLong* shp, Nd4jLong* strides, int dtype, char order, Nd4jLong ews, Nd4jLong extras) {
+  GUARD_BEGIN
+  ND4J_REQUIRE(rank >= 0 && rank <= MAX_RANK, "shapeBuffer: rank out of range");
+  ND4J_REQUIRE(rank == 0 || shp != nullptr, "shapeBuffer: shape is null");
+  std::vector<LongType> s(shp, shp + rank);
+  auto si = makeShapeInfo((DataType)dtype, order, s, strides, extras);
+  (void)ews;  // recomputed from the strides
+  return static_cast<OpaqueConstantShapeBuffer>(cachedShapeBuffer(si.data()));
+  GUARD_END(nullptr)
+}
+OpaqueConstantShapeBuffer shapeBuffer(int rank, Nd4jLong* shp, Nd4jLong* strides, int dtype, char order, Nd4jLong ews, bool empty) {
+  return shapeBufferEx(rank, shp, strides, dtype, order, ews, empty ? ARRAY_EMPTY : 0);
+}
+OpaqueConstantShapeBuffer cacheAndStoreShapeBuffer(Nd4jLong* shapeInfo) {
+  GUARD_BEGIN
+  return static_cast<OpaqueConstantShapeBuffer>(cachedShapeBuffer(shapeInfo));
+  GUARD_END(nullptr)
+}
+Nd4jPointer getConstantShapeBufferPrimary(OpaqueConstantShapeBuffer b) { return b ? (Nd4jPointer)b->primary() : nullptr; }
+Nd4jPointer getConstantShapeBufferSpecial(OpaqueConstantShapeBuffer b) {
+  GUARD_BEGIN
+  return b ? (Nd4jPointer)b->special() : nullptr;
+  GUARD_END(nullptr)
+}
+void deleteConstantShapeBuffer(OpaqueConstantShapeBuffer*) {}
+
+// ---- array handles ------------------------------------------------------------------------------------
+OpaqueNDArray createOpaqueNDArray(OpaqueDataBuffer* shapeInfo, OpaqueDataBuffer* buffer, OpaqueDataBuffer* specialBuffer, Nd4jLong offset) {
+  GUARD_BEGIN
+  ND4J_REQUIRE(shapeInfo != nullptr, "createOpaqueNDArray: Shape info was null!");
+  const LongType* si = reinterpret_cast<const LongType*>(shapeInfo->primary());
+  ND4J_REQUIRE(si != nullptr, "createOpaqueNDArray: shapeInfo->primary() returned nullptr - shape buffer is invalid!");
+  const int rank = shape::rank(si);
+  ND4J_REQUIRE(rank >= 0 && rank <= MAX_RANK, "createOpaqueNDArray: rank out of range");
+  if (shape::isEmpty(si) && buffer != nullptr) ND4J_THROW("createOpaqueNDArray: Shape info was empty but buffer was not null!");
+  if (!shape::isEmpty(si) && buffer == nullptr) ND4J_THROW("createOpaqueNDArray: Shape info was not empty but buffer was null!");
+  ND4J_REQUIRE(shape::dataType(si) != UNKNOWN, "createOpaqueNDArray: descriptor carries no known data type");
+  (void)specialBuffer;  // the device side lives in the same buffer object
+  auto* a = new Nd4jHipNDArray();
+  a->si.assign(si, si + shape::shapeInfoLength(rank));
+  a->offset = offset;
+  if (buffer) {
+    a->buf = buffer->db;
+    a->bufOffsetBytes = buffer->offsetBytes;
+    // bounds: the furthest element of the view must lie inside the buffer
+    LongType maxOff = offset;
+    for (int d = 0; d < rank; d++) {
+      LongType st = shape::strideOf(si)[d];
+      if (shape::shapeOf(si)[d] > 0 && st > 0) maxOff += (shape::shapeOf(si)[d] - 1) * st;
+    }
+    ND4J_REQUIRE(offset >= 0, "createOpaqueNDArray: negative offset");
+    ND4J_REQUIRE((size_t)(maxOff + 1) * sizeOf(a->dataType()) + a->bufOffsetBytes <= a->buf->lenBytes,
+                 "createOpaqueNDArray: shape/strides/offset reach beyond the end of the data buffer");
+  }
+  return a;
+  GUARD_END(nullptr)
+}
+void deleteNDArray(OpaqueNDArray array) { delete array; }
+Nd4jLong getOpaqueNDArrayOffset(OpaqueNDArray a) { return a ? a->offset : 0; }
+const Nd4jLong* getOpaqueNDArrayShapeInfo(OpaqueNDArray a) { return a ? a->shapeInfo() : nullptr; }
+void* getOpaqueNDArrayBuffer(OpaqueNDArray a) { return a ? a->buffer() : nullptr; }
+void* getOpaqueNDArraySpecialBuffer(OpaqueNDArray a) { return a ? a->specialBuffer() : nullptr; }
+Nd4jLong getOpaqueNDArrayLength(OpaqueNDArray a) { return a && a->buf ? a->buf->numElements() : 0; }
+Nd4jLong getOpaqueNDArrayShapeInfoLength(OpaqueNDArray a) { return a ? shape::shapeInfoLength(a->rankOf()) : 0; }
+
+// ---- TAD packs -------------------------------------------------------------------------------------------
+OpaqueTadPack* tadOnlyShapeInfo(OpaqueDataBuffer* hXShapeInfo, Nd4jLong* dimension, Nd4jLong dimensionLength) {
+  GUARD_BEGIN
+  ND4J_REQUIRE(hXShapeInfo && hXShapeInfo->primary(), "tadOnlyShapeInfo: shape info is null");
+  return static_cast<OpaqueTadPack*>(tadForDimensions(reinterpret_cast<const LongType*>(hXShapeInfo->primary()), dimension, (int)dimensionLength));
+  GUARD_END(nullptr)
+}
+const Nd4jLong* getPrimaryShapeInfo(OpaqueTadPack* p) { return p ? p->tadShape->primary() : nullptr; }
+const Nd4jLong* getPrimaryOffsets(OpaqueTadPack* p) { return p ? p->offsets.data() : nullptr; }
+const Nd4jLong* getSpecialShapeInfo(OpaqueTadPack* p) {
+  GUARD_BEGIN
+  return p ? p->tadShape->special() : nullptr;
+  GUARD_END(nullptr)
+}
+const Nd4jLong* getSpecialOffsets(OpaqueTadPack* p) {
+  GUARD_BEGIN
+  return p ? p->specialOffsets() : nullptr;
+  GUARD_END(nullptr)
+}
+Nd4jLong getNumberOfTads(OpaqueTadPack* p) { return p ? p->numTads : 0; }
+int getShapeInfoLength(OpaqueTadPack* p) { return p ? shape::shapeInfoLength(shape::rank(p->tadShape->primary())) : 0; }
+void deleteTadPack(OpaqueTadPack*) {}
+
+// ---- legacy loops --------------------------------------------------------------------------------------------
+static void runUnary(const char* fn, UnaryKind k, NDArray* x, NDArray* z) {
+  if (x->isEmpty() || z->isEmpty()) return;
+  EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo()});
+  prepareSpecialUse({z}, {x});
+  launchUnary(execStream(), k, x->dataType(), z->dataType(), x->specialBuffer(), z->specialBuffer(), p);
+  registerSpecialUse({z}, {x});
+}
+
+void execTransformStrict(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
+  GUARD_BEGIN
+  NDArray* x = arr(xa, "execTransformStrict", "x"); NDArray* z = arr(za, "execTransformStrict", "z");
+  // X -> X over float types only (NativeOpExecutioner_transform.cpp:115-131)
+  ND4J_REQUIRE(x->dataType() == z->dataType() && isFloatType(x->dataType()),
+               std::string("NativeOpExecutioner::execTransformStrict requires X & Z to have same floating point type, got ") + dtypeName(x->dataType()) + " and " + dtypeName(z->dataType()));
+  UnaryKind k;
+  switch (opNum) {  // loops/legacy_ops.h:54-64
+    case 22: k = U_COS; break; case 23: k = U_EXP; break; case 24: k = U_LOG; break; case 26: k = U_SIGMOID; break;
+    case 27: k = U_SIN; break; case 28: k = U_SOFTPLUS; break; case 29: k = U_TANH; break; case 43: k = U_SWISH; break;
+    case 45: k = U_ERF; break; case 53: k = U_GELU; break; case 55: k = U_PRECISE_GELU; break;
+    default: ND4J_THROW("execTransformStrict: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
+  }
+  runUnary("execTransformStrict", k, x, z);
+  GUARD_END_VOID
+}
+void execTransformFloat(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
+  GUARD_BEGIN
+  NDArray* x = arr(xa, "execTransformFloat", "x"); NDArray* z = arr(za, "execTransformFloat", "z");
+  ND4J_REQUIRE(isFloatType(z->dataType()), "NativeOpExecutioner::execTransformFloat requires Z to have floating point type");
+  ND4J_REQUIRE(isFloatType(x->dataType()), "execTransformFloat: non-float inputs are not implemented in nd4j-hip");
+  UnaryKind k;
+  switch (opNum) {  // loops/legacy_ops.h:67
+    case 1: k = U_SQRT; break; case 3: k = U_RSQRT; break;
+    default: ND4J_THROW("execTransformFloat: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
+  }
+  runUnary("execTransformFloat", k, x, z);
+  GUARD_END_VOID
+}
+void execTransformSame(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
+  GUARD_BEGIN
+  NDArray* x = arr(xa, "execTransformSame", "x"); NDArray* z = arr(za, "execTransformSame", "z");
+  ND4J_REQUIRE(x->dataType() == z->dataType(), "NativeOpExecutioner::execTransformSame requires X & Z to have same type");
+  ND4J_REQUIRE(isFloatType(x->dataType()), "execTransformSame: non-float types are not implemented in nd4j-hip");
+  UnaryKind k;
+  switch (opNum) {  // loops/legacy_ops.h:40-44
+    case 0: k = U_ABS; break; case 3: k = U_NEG; break; case 6: k = U_CUBE; break; case 7: k = U_ONE_MINUS; break;
+    case 11: k = U_RECIPROCAL; break; case 12: k = U_SQUARE; break; case 15: case 21: k = U_IDENTITY; break;
+    default: ND4J_THROW("execTransformSame: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
+  }
+  runUnary("execTransformSame", k, x, z);
+  GUARD_END_VOID
+}
+void execTransformAny(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
+  GUARD_BEGIN
+  NDArray* x = arr(xa, "execTransformAny", "x"); NDArray* z = arr(za, "execTransformAny", "z");
+  ND4J_REQUIRE(opNum == 0, "execTransformAny: only Assign (opNum 0) exists (loops/legacy_ops.h:46)");
+  runUnary("execTransformAny", U_IDENTITY, x, z);
+  GUARD_END_VOID
+}
+
+static PairwiseKind pairwiseKind(int opNum) {
+  switch (opNum) {  // loops/legacy_ops.h:121-129
+    case 0: return P_ADD; case 1: return P_COPY; case 2: return P_DIV; case 3: return P_MUL; case 5: return P_RSUB;
+    case 6: return P_SUB; case 7: return P_MAX; case 8: return P_MIN; case 11: return P_RDIV; case 20: return P_SQSUB;
+    default: ND4J_THROW("execPairwiseTransform: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
+  }
+}
+void execPairwiseTransform(Nd4jPointer*, int opNum, OpaqueNDArray xa, OpaqueNDArray ya, OpaqueNDArray za, void*) {
+  GUARD_BEGIN
+  NDArray* x = arr(xa, "execPairwiseTransform", "x"); NDArray* y = arr(ya, "execPairwiseTransform", "y");
+  NDArray* z = arr(za, "execPairwiseTransform", "z");
+  // NativeOpExecutioner_pairwise_floats.cpp:34-57
+  ND4J_REQUIRE(x->dataType() == z->dataType() || y->dataType() == z->dataType(),
+               std::string("NativeOpExecutioner::execPairwiseTransform requires X or Y to have the same type as Z, got ") + dtypeName(x->dataType()) + ", " + dtypeName(y->dataType()) + " -> " + dtypeName(z->dataType()));
+  ND4J_REQUIRE(isFloatType(z->dataType()) && isFloatType(x->dataType()) && isFloatType(y->dataType()),
+               "execPairwiseTransform: non-float types are not implemented in nd4j-hip");
+  PairwiseKind k = pairwiseKind(opNum);
+  if (z->isEmpty()) return;
+  EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo(), y->shapeInfo()});
+  prepareSpecialUse({z}, {x, y});
+  // each view's offset is applied once here (specialBuffer()); the reference's CPU facade adds x->offset()
+  // a second time for views (legacy/cpu/NativeOps.cpp:1245-1257)
+  launchPairwise(execStream(), k, x->dataType(), y->dataType(), z->dataType(), x->specialBuffer(), y->specialBuffer(), z->specialBuffer(), p);
+  registerSpecialUse({z}, {x, y});
+  GUARD_END_VOID
+}
+
+static double hostScalar(NDArray* s) {
+  ND4J_REQUIRE(s->lengthOf() >= 1 && s->buf, "scalar operand is empty");
+  s->buf->syncToPrimary();
+  const void* p = s->buffer();
+  switch (s->dataType()) {
+    case FLOAT32: return *(const float*)p;
+    case DOUBLE: return *(const double*)p;
+    case INT32: return *(const int*)p;
+    case INT64: return (double)*(const LongType*)p;
+    case HALF: { unsigned short h = *(const unsigned short*)p; unsigned sign = (h & 0x8000u) << 16, e = (h >> 10) & 31, m = h & 1023; float f; unsigned u;
+      if (e == 0) { f = (float)m / 16777216.0f; if (sign) f = -f; return f; }
+      if (e == 31) u = sign | 0x7f800000u | (m << 13); else u = sign | ((e + 112) << 23) | (m << 13);
+      memcpy(&f, &u, 4); return f; }
+    case BFLOAT16: { unsigned u = ((unsigned)*(const unsigned short*)p) << 16; float f; memcpy(&f, &u, 4); return f; }
+    default: ND4J_THROW("scalar operand has an unsupported data type");
+  }
+}
+void execScalar(Nd4jPointer*, int opNum, OpaqueNDArray xa, OpaqueNDArray za, OpaqueNDArray sa, void*) {
+  GUARD_BEGIN
+  NDArray* x = arr(xa, "execScalar", "x"); NDArray* z = arr(za, "execScalar", "z"); NDArray* s = arr(sa, "execScalar", "scalar");
+  ND4J_REQUIRE(x->dataType() == z->dataType() && isFloatType(x->dataType()), "execScalar: nd4j-hip implements same-type float arrays only");
+  PairwiseKind k;
+  switch (opNum) {  // loops/legacy_ops.h:78-86
+    case 0: k = P_ADD; break; case 1: k = P_SUB; break; case 2: k = P_MUL; break; case 3: k = P_DIV; break;
+    case 4: k = P_RDIV; break; case 5: k = P_RSUB; break; case 6: k = P_MAX; break; case 13: k = P_MIN; break; case 14: k = P_COPY; break;
+    default: ND4J_THROW("execScalar: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
+  }
+  if (z->isEmpty()) return;
+  double sc = hostScalar(s);
+  EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo()});
+  ND4J_REQUIRE(p.sameShape, "execScalar: x and z must share a shape");
+  prepareSpecialUse({z}, {x});
+  launchScalarOp(execStream(), k, x->dataType(), x->specialBuffer(), sc, z->specialBuffer(), p);
+  registerSpecialUse({z}, {x});
+  GUARD_END_VOID
+}
+
+static std::vector<LongType> hostDims(NDArray* dimension, int rank, const char* fn) {
+  if (!dimension || dimension->isEmpty() || dimension->lengthOf() == 0) return {};
+  ND4J_REQUIRE(dimension->buf, std::string(fn) + ": dimension array has no buffer");
+  dimension->buf->syncToPrimary();
+  std::vector<LongType> raw(dimension->lengthOf());
+  for (LongType i = 0; i < (LongType)raw.size(); i++) {
+    LongType off = 0, idx = i;
+    for (int d = dimension->rankOf() - 1; d >= 0; d--) { off += (idx % dimension->sizeAt(d)) * dimension->strideAt(d); idx /= dimension->sizeAt(d); }
+    if (dimension->dataType() == INT64) raw[i] = dimension->hostAs<LongType>()[off];
+    else if (dimension->dataType() == INT32) raw[i] = dimension->hostAs<int>()[off];
+    else ND4J_THROW(std::string(fn) + ": dimension array must be INT32 or INT64");
+  }
+  return normalizeDims(rank, raw.data(), (LongType)raw.size(), fn);
+}
+
+// y is a smaller array whose dims line up with `dimension` of x (loops/cpu/broadcasting.hpp); realised as a
+// pairwise walk in which y's stride is 0 along every other dim
+void execBroadcast(Nd4jPointer*, int opNum, OpaqueNDArray xa, OpaqueNDArray ya, OpaqueNDArray za, void*, OpaqueNDArray da) {
+  GUARD_BEGIN
+  NDArray* x = arr(xa, "execBroadcast", "x"); NDArray* y = arr(ya, "execBroadcast", "y"); NDArray* z = arr(za, "execBroadcast", "z");
+  NDArray* dim = arr(da, "execBroadcast", "dimension");
+  ND4J_REQUIRE(x->dataType() == z->dataType() && y->dataType() == z->dataType() && isFloatType(z->dataType()),
+               "execBroadcast: nd4j-hip implements same-type float arrays only");
+  PairwiseKind k;
+  switch (opNum) {  // loops/legacy_ops.h:34-39
+    case 0: k = P_ADD; break; case 1: k = P_SUB; break; case 2: k = P_MUL; break; case 3: k = P_DIV; break;
+    case 4: k = P_RDIV; break; case 5: k = P_RSUB; break; case 6: k = P_COPY; break;
+    case 13: k = P_MIN; break; case 14: k = P_MAX; break; case 17: k = P_SQSUB; break;
+    default: ND4J_THROW("execBroadcast: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
+  }
+  if (z->isEmpty()) return;
+  auto dims = hostDims(dim, x->rankOf(), "execBroadcast");
+  // squeeze y's unit dims, then its remaining dims must match x along `dims`
+  std::vector<LongType> yshape, ystride;
+  for (int d = 0; d < y->rankOf(); d++) if (y->sizeAt(d) != 1) { yshape.push_back(y->sizeAt(d)); ystride.push_back(y->strideAt(d)); }
+  std::vector<LongType> bstride(x->rankOf(), 0);
+  size_t q = 0;
+  for (auto d : dims) {
+    if (x->sizeAt((int)d) == 1) continue;
+    ND4J_REQUIRE(q < yshape.size() && yshape[q] == x->sizeAt((int)d), "execBroadcast: y's shape does not match x along the broadcast dimensions");
+    bstride[d] = ystride[q++];
+  }
+  ND4J_REQUIRE(q == yshape.size(), "execBroadcast: y has more non-unit dims than broadcast dimensions");
+  std::vector<LongType> xshape(x->rankOf());
+  for (int d = 0; d < x->rankOf(); d++) xshape[d] = x->sizeAt(d);
+  auto ysi = makeShapeInfo(y->dataType(), 'c', xshape, bstride.data());
+  EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo(), ysi.data()});
+  prepareSpecialUse({z}, {x, y});
+  launchPairwise(execStream(), k, x->dataType(), y->dataType(), z->dataType(), x->specialBuffer(), y->specialBuffer(), z->specialBuffer(), p);
+  registerSpecialUse({z}, {x, y});
+  GUARD_END_VOID
+}
+
+static void runReduce(const char* fn, ReduceKind k, NDArray* x, NDArray* z, const std::vector<LongType>& dims) {
+  ND4J_REQUIRE(isFloatType(x->dataType()), std::string(fn) + ": non-float inputs are not implemented in nd4j-hip");
+  ND4J_REQUIRE(x->dataType() == z->dataType(), std::string(fn) + ": nd4j-hip requires Z to have X's type, got " + dtypeName(x->dataType()) + " -> " + dtypeName(z->dataType()));
+  ND4J_REQUIRE(!x->isEmpty(), std::string(fn) + ": reductions of empty arrays are not implemented in nd4j-hip");
+  if (z->isEmpty()) return;
+  std::vector<LongType> d = dims;
+  if (z->lengthOf() == 1 && x->lengthOf() != 1) {
+    // a single output means "reduce everything" unless the kept dims are all of extent 1
+    bool keptAllUnit = true;
+    std::vector<bool> red(x->rankOf(), false);
+    for (auto v : d) red[v] = true;
+    for (int i = 0; i < x->rankOf(); i++) if (!red[i] && x->sizeAt(i) != 1) keptAllUnit = false;
+    if (!keptAllUnit) d.clear();
+  }
+  ReducePlan p = buildReducePlan(x->shapeInfo(), z->shapeInfo(), d, false);
+  auto lc = LaunchContext::defaultContext();
+  prepareSpecialUse({z}, {x});
+  launchReduce(lc->execStream, k, x->dataType(), z->dataType(), x->specialBuffer(), z->specialBuffer(), p, lc->reductionBuffer, LaunchContext::REDUCTION_BYTES);
+  registerSpecialUse({z}, {x});
+}
+static ReduceKind reduceSameKind(int opNum) {
+  switch (opNum) {  // loops/legacy_ops.h:100-101
+    case 0: return R_SUM; case 1: return R_MAX; case 2: return R_MIN; case 3: return R_PROD; case 4: return R_ASUM;
+    case 5: return R_AMAX; case 6: return R_AMIN;
+    default: ND4J_THROW("execReduceSame: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
+  }
+}
+static ReduceKind reduceFloatKind(int opNum) {
+  switch (opNum) {  // loops/legacy_ops.h:103-105
+    case 0: return R_MEAN; case 1: return R_AMEAN; case 2: return R_NORM1; case 3: return R_NORM2; case 4: return R_NORMMAX;
+    case 5: return R_NORM2;  // NormFrobenius = sqrt(sum |x|^2)
+    case 7: return R_SQNORM;
+    default: ND4J_THROW("execReduceFloat: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
+  }
+}
+void execReduceSame(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
+  GUARD_BEGIN
+  if (xa == nullptr || za == nullptr) ND4J_THROW("execReduceSame: null pointer in input parameters");
+  runReduce("execReduceSame", reduceSameKind(opNum), xa, za, {});
+  GUARD_END_VOID
+}
+void execReduceSame2(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
+  GUARD_BEGIN
+  if (xa == nullptr || za == nullptr || da == nullptr) ND4J_THROW("execReduceSame2: null pointer in input parameters");
+  runReduce("execReduceSame2", reduceSameKind(opNum), xa, za, hostDims(da, xa->rankOf(), "execReduceSame2"));
+  GUARD_END_VOID
+}
+void execReduceFloat(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
+  GUARD_BEGIN
+  if (xa == nullptr || za == nullptr) ND4J_THROW("execReduceFloat: null pointer in input parameters");
+  runReduce("execReduceFloat", reduceFloatKind(opNum), xa, za, {});
+  GUARD_END_VOID
+}
+void execReduceFloat2(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
+  GUARD_BEGIN
+  if (xa == nullptr || za == nullptr || da == nullptr) ND4J_THROW("execReduceFloat2: null pointer in input parameters");
+  runReduce("execReduceFloat2", reduceFloatKind(opNum), xa, za, hostDims(da, xa->rankOf(), "execReduceFloat2"));
+  GUARD_END_VOID
+}
+
+static IndexKind indexKind(int opNum) {
+  switch (opNum) {  // loops/legacy_ops.h:131-132
+    case 0: return I_MAX; case 1: return I_MIN; case 2: return I_AMAX; case 3: return I_AMIN;
+    default: ND4J_THROW("execIndexReduce: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
+  }
+}
+}  // extern "C"
+namespace nd4jhip {
+void runIndexReduce(const char* fn, int opNum, NDArray* x, NDArray* z, const std::vector<LongType>& dims) {
+  ND4J_REQUIRE(isFloatType(x->dataType()), std::string(fn) + ": non-float inputs are not implemented in nd4j-hip");
+  ND4J_REQUIRE(z->dataType() == INT64 || z->dataType() == INT32,
+               std::string("NativeOpExecutioner::") + fn + " requires Z operand to have INT32/INT64 type, got " + dtypeName(z->dataType()));
+  ND4J_REQUIRE(!x->isEmpty(), std::string(fn) + ": index reductions of empty arrays are not implemented in nd4j-hip");
+  if (z->isEmpty()) return;
+  IndexKind k = indexKind(opNum);
+  std::vector<LongType> d = dims;
+  if (z->lengthOf() == 1 && (int)d.size() < x->rankOf()) {
+    bool keptAllUnit = true;
+    std::vector<bool> red(x->rankOf(), false);
+    for (auto v : d) red[v] = true;
+    for (int i = 0; i < x->rankOf(); i++) if (!red[i] && x->sizeAt(i) != 1) keptAllUnit = false;
+    if (!keptAllUnit) d.clear();
+  }
+  // z is addressed linearly, z[i] for the i-th sub-array (helpers/cpu/loops/IndexReductionLoops.hpp:61-75);
+  // with a dense z that is also what walking its shape gives
+  ReducePlan p = buildReducePlan(x->shapeInfo(), z->shapeInfo(), d, false);
+  auto lc = LaunchContext::defaultContext();
+  prepareSpecialUse({z}, {x});
+  launchIndexReduce(lc->execStream, k, x->dataType(), z->dataType(), x->specialBuffer(), z->specialBuffer(), p, lc->reductionBuffer, LaunchContext::REDUCTION_BYTES);
+  registerSpecialUse({z}, {x});
+}
+}  // namespace nd4jhip
+extern "C" {
+void execIndexReduce(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
+  GUARD_BEGIN
+  NDArray* x = arr(xa, "execIndexReduce", "x"); NDArray* z = arr(za, "execIndexReduce", "z"); NDArray* d = arr(da, "execIndexReduce", "dimension");
+  runIndexReduce("execIndexReduce", opNum, x, z, hostDims(d, x->rankOf(), "execIndexReduce"));
+  GUARD_END_VOID
+}
+void execIndexReduceScalar(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
+  GUARD_BEGIN
+  NDArray* x = arr(xa, "execIndexReduceScalar", "x"); NDArray* z = arr(za, "execIndexReduceScalar", "z");
+  runIndexReduce("execIndexReduceScalar", opNum, x, z, {});
+  GUARD_END_VOID
+}
+
+// ---- op context ---------------------------------------------------------------------------------------------
+OpaqueContext* createGraphContext(int nodeId) {
+  auto* c = new Nd4jHipContext();
+  c->nodeId = nodeId;
+  return c;
+}
+void deleteGraphContext(OpaqueContext* ptr) { delete ptr; }
+void markGraphContextInplace(OpaqueContext* ptr, bool v) { if (ptr) ptr->inplace = v; }
+static void setAt(std::vector<NDArray*>& v, int index, NDArray* a) {
+  if (index < 0) ND4J_THROW("graph context: negative array index");
+  if ((int)v.size() <= index) v.resize(index + 1, nullptr);
+  v[index] = a;
+}
+void setGraphContextInputArray(OpaqueContext* ptr, int index, OpaqueNDArray a) {
+  GUARD_BEGIN
+  if (a == nullptr) ND4J_THROW("setGraphContextInputArray: Input arrays were null!");
+  ND4J_REQUIRE(ptr != nullptr, "setGraphContextInputArray: Context was null!");
+  setAt(ptr->inputs, index, a);
+  GUARD_END_VOID
+}
+void setGraphContextOutputArray(OpaqueContext* ptr, int index, OpaqueNDArray a) {
+  GUARD_BEGIN
+  if (a == nullptr) ND4J_THROW("setGraphContextOutputArray: Input arrays were null!");
+  ND4J_REQUIRE(ptr != nullptr, "setGraphContextOutputArray: Context was null!");
+  setAt(ptr->outputs, index, a);
+  GUARD_END_VOID
+}
+void setGraphContextInputArraysArr(OpaqueContext* ptr, int n, OpaqueNDArrayArr a) {
+  GUARD_BEGIN
+  if (a == nullptr) ND4J_THROW("setGraphContextInputArraysArr: Input arrays were null!");
+  if (ptr == nullptr) ND4J_THROW("setGraphContextInputArraysArr: Context was null!");
+  for (int i = 0; i < n; i++) {
+    if (a[i] == nullptr) ND4J_THROW("setGraphContextInputArraysArr: Input array at index " + std::to_string(i) + " was null!");
+    setAt(ptr->inputs, i, a[i]);
+  }
+  GUARD_END_VOID
+}
+void setGraphContextOutputArraysArr(OpaqueContext* ptr, int n, OpaqueNDArrayArr a) {
+  GUARD_BEGIN
+  if (a == nullptr) ND4J_THROW("setGraphContextOutputArraysArr: Output arrays were null!");
+  if (ptr == nullptr) ND4J_THROW("setGraphContextOutputArraysArr: Context was null!");
+  for (int i = 0; i < n; i++) {
+    if (a[i] == nullptr) ND4J_THROW("setGraphContextOutputArraysArr: Output array at index " + std::to_string(i) + " was null!");
+    setAt(ptr->outputs, i, a[i]);
+  }
+  GUARD_END_VOID
+}
+void setGraphContextTArguments(OpaqueContext* ptr, double* a, int n) { if (ptr) ptr->tArgs.assign(a, a + (n > 0 ? n : 0)); }
+void setGraphContextIArguments(OpaqueContext* ptr, Nd4jLong* a, int n) { if (ptr) ptr->iArgs.assign(a, a + (n > 0 ? n : 0)); }
+void setGraphContextBArguments(OpaqueContext* ptr, bool* a, int n) { if (ptr) ptr->bArgs.assign(a, a + (n > 0 ? n : 0)); }
+void setGraphContextDArguments(OpaqueContext* ptr, int* a, int n) {
+  if (!ptr) return;
+  ptr->dArgs.clear();
+  for (int i = 0; i < n; i++) ptr->dArgs.push_back((DataType)a[i]);
+}
+void ctxAllowHelpers(OpaqueContext* ptr, bool v) { if (ptr) ptr->helpersAllowed = v; }
+void ctxShapeFunctionOverride(OpaqueContext* ptr, bool v) { if (ptr) ptr->shapeFunctionOverride = v; }
+void ctxSetExecutionMode(OpaqueContext* ptr, int m) { if (ptr) ptr->execMode = m; }
+void ctxPurge(OpaqueContext* ptr) {
+  if (!ptr) return;
+  ptr->inputs.clear(); ptr->outputs.clear(); ptr->tArgs.clear(); ptr->iArgs.clear(); ptr->bArgs.clear(); ptr->dArgs.clear();
+}
+OpaqueNDArray getInputArrayNative(OpaqueContext* ptr, int idx) {
+  if (!ptr || idx < 0 || idx >= (int)ptr->inputs.size()) return nullptr;
+  return static_cast<OpaqueNDArray>(ptr->inputs[idx]);
+}
+OpaqueNDArray getOutputArrayNative(OpaqueContext* ptr, int idx) {
+  if (!ptr || idx < 0 || idx >= (int)ptr->outputs.size()) return nullptr;
+  return static_cast<OpaqueNDArray>(ptr->outputs[idx]);
+}
+Nd4jLong numInputsNative(OpaqueContext* ptr) { return ptr ? (Nd4jLong)ptr->inputs.size() : 0; }
+Nd4jLong numOutputsNative(OpaqueContext* ptr) { return ptr ? (Nd4jLong)ptr->outputs.size() : 0; }
+Nd4jLong numTArgumentsNative(OpaqueContext* ptr) { return ptr ? (Nd4jLong)ptr->tArgs.size() : 0; }
+Nd4jLong numIArgumentsNative(OpaqueContext* ptr) { return ptr ? (Nd4jLong)ptr->iArgs.size() : 0; }
+Nd4jLong numBNative(OpaqueContext* ptr) { return ptr ? (Nd4jLong)ptr->bArgs.size() : 0; }
+Nd4jLong numDNative(OpaqueContext* ptr) { return ptr ? (Nd4jLong)ptr->dArgs.size() : 0; }
+double tArgumentNative(OpaqueContext* ptr, int idx) { return ptr && idx >= 0 && idx < (int)ptr->tArgs.size() ? ptr->tArgs[idx] : 0.0; }
+Nd4jLong iArgumentAtNative(OpaqueContext* ptr, int idx) { return ptr && idx >= 0 && idx < (int)ptr->iArgs.size() ? ptr->iArgs[idx] : 0; }
+bool bArgAtNative(OpaqueContext* ptr, int idx) { return ptr && idx >= 0 && idx < (int)ptr->bArgs.size() ? (bool)ptr->bArgs[idx] : false; }
+Nd4jLong dataTypeNativeAt(OpaqueContext* ptr, int idx) { return ptr && idx >= 0 && idx < (int)ptr->dArgs.size() ? (Nd4jLong)ptr->dArgs[idx] : 0; }
+
+// ---- declarable ops --------------------------------------------------------------------------------------------
+const char* getAllCustomOps(void) { return ops::allCustomOps(); }
+Nd4jLong nd4jhipOpHash(const char* name) { return name ? ops::opHash(name) : 0; }
+
+Nd4jStatus execCustomOp2(Nd4jPointer*, Nd4jLong hash, OpaqueContext* ctx) {
+  GUARD_BEGIN
+  ND4J_REQUIRE(ctx != nullptr, "execCustomOp2: context is null");
+  const ops::OpDescriptor* op = ops::findOp(hash);
+  if (!op) ND4J_THROW("execCustomOp2: unknown op hash " + std::to_string(hash) + " (op is not implemented in nd4j-hip)");
+  ops::executeOp(*op, *ctx);
+  if (Environment::get().syncAfterCustomOp) HIP_CHECK(hipStreamSynchronize(execStream()));
+  return 0;
+  GUARD_END(1)
+}
+OpaqueShapeList* calculateOutputShapes2(Nd4jPointer*, Nd4jLong hash, OpaqueContext* ctx) {
+  GUARD_BEGIN
+  ND4J_REQUIRE(ctx != nullptr, "calculateOutputShapes2: context is null");
+  const ops::OpDescriptor* op = ops::findOp(hash);
+  if (!op) ND4J_THROW("calculateOutputShapes2: unknown op hash " + std::to_string(hash));
+  auto* list = new Nd4jHipShapeList();
+  try {
+    for (auto& si : op->shapeFn(*ctx)) list->shapes.push_back(cachedShapeBuffer(si.data()));
+  } catch (...) { delete list; throw; }
+  return list;
+  GUARD_END(nullptr)
+}
+Nd4jLong getShapeListSize(OpaqueShapeList* list) { return list ? (Nd4jLong)list->shapes.size() : 0; }
+const Nd4jLong* getShape(OpaqueShapeList* list, Nd4jLong i) {
+  if (!list || i < 0 || i >= (Nd4jLong)list->shapes.size()) return nullptr;
+  return list->shapes[i]->primary();
+}
+void deleteShapeList(Nd4jPointer shapeList) { delete static_cast<Nd4jHipShapeList*>(shapeList); }
+
+void nd4jhipSetSyncAfterCustomOp(int enable) { Environment::get().syncAfterCustomOp = enable != 0; }
+const char* nd4jhipBuildInfo(void) { return "nd4j-hip gfx950 (hand-written HIP kernels; no CPU fallback)"; }
+
+}  // extern "C"

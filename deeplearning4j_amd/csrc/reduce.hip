@@ -1,0 +1,457 @@
+// Reductions along dimensions and full reductions (value and index flavours).
+//
+// Layout: the host splits x's dims into `outer` (kept, one output each) and `inner` (reduced).
+//   coop kernel   - TPR (64 or 256) threads share one output; the inner run is read with 16-byte loads
+//                   when it is unit-stride, otherwise element-wise through the inner strides.  Long inner
+//                   runs with few outputs are cut into `splits` segments whose partials go through the
+//                   launch context's reduction scratch and a small second kernel (deterministic order).
+//   flat kernel   - one thread per output walking the inner dims; used when there are many outputs and
+//                   the inner run is strided, so that neighbouring threads read neighbouring addresses.
+// All of these are HBM-bound: algorithmic bytes = sizeof(T) per input element + one output per row.
+//
+// Value semantics follow the reference's reduce functors (libnd4j/include/ops/ops.h:2363-2378,1170-1298):
+// accumulate in float for fp16/bf16/fp32 and in double for fp64, post-process (mean: / n, norm2: sqrt).
+// The reference accumulates each output sequentially; a tree changes the rounding order only.
+// Index semantics (ops/op_macros_index_reduce.h:33-69): strict comparison from {start, 0}, so the first
+// extreme wins, NaN is never selected and an all -inf row gives 0.  Here: NaN is mapped to the start
+// value on load and ties resolve to the lowest index, which yields the same integer.
+#include "device.h"
+#include "kernels.h"
+#include "runtime.h"
+
+namespace nd4jhip {
+
+enum PreKind { PRE_ID = 0, PRE_ABS = 1, PRE_SQ = 2 };
+enum PostKind { POST_ID = 0, POST_DIV_N = 1, POST_SQRT = 2 };
+
+template <typename Op, typename A> struct Identity;
+template <typename A> struct Identity<SumOp, A> { static __device__ __forceinline__ A v() { return (A)0; } };
+template <typename A> struct Identity<ProdOp, A> { static __device__ __forceinline__ A v() { return (A)1; } };
+template <typename A> struct Identity<MaxOp, A> { static __device__ __forceinline__ A v() { return -(A)INFINITY; } };
+template <typename A> struct Identity<MinOp, A> { static __device__ __forceinline__ A v() { return (A)INFINITY; } };
+
+template <int PRE, typename A>
+__device__ __forceinline__ A pre(A x) {
+  if (PRE == PRE_ABS) return x < 0 ? -x : x;
+  if (PRE == PRE_SQ) return x * x;
+  return x;
+}
+template <typename A>
+__device__ __forceinline__ A post(A s, int kind, LongType n) {
+  if (kind == POST_DIV_N) return s / (A)n;
+  if (kind == POST_SQRT) return sizeof(A) == 8 ? (A)sqrt((double)s) : (A)sqrtf((float)s);
+  return s;
+}
+
+struct CoopArgs {
+  DevShape outer, inner, zOuter;
+  LongType outerLen, innerLen;
+  LongType segLen;   // elements of the inner run handled by one block (== innerLen when splits == 1)
+  int splits;
+  int zLinear;
+  int postKind;
+};
+
+// ---- value reduce, cooperative -------------------------------------------------------------------------
+template <typename Op, int PRE, typename T, int TPR>
+__global__ __launch_bounds__(256) void reduce_coop(CoopArgs a, const T* __restrict__ x, T* __restrict__ z,
+                                                   typename Conv<T>::acc* __restrict__ partials, int vectorOk) {
+  using A = typename Conv<T>::acc;
+  constexpr int V = 16 / sizeof(T);
+  constexpr int ROWS = 256 / TPR;
+  __shared__ A lds[4];
+  const int t = threadIdx.x % TPR;
+  const LongType unit = (LongType)blockIdx.x * ROWS + threadIdx.x / TPR;  // (row, split) pair
+  const LongType row = unit / a.splits;
+  const int split = (int)(unit - row * a.splits);
+  A acc = Identity<Op, A>::v();
+  const bool live = row < a.outerLen;
+  if (live) {
+    const LongType base = walk<LongType>(a.outer, row);
+    const LongType j0 = (LongType)split * a.segLen;
+    LongType j1 = j0 + a.segLen;
+    if (j1 > a.innerLen) j1 = a.innerLen;
+    if (a.inner.rank == 1 && a.inner.stride[0] == 1) {
+      const T* p = x + base;
+      LongType j = j0;
+      if (vectorOk) {
+        using VT = Vec<T, V>;
+        const LongType nv = (j1 - j0) / V;
+        const VT* pv = reinterpret_cast<const VT*>(p + j0);
+        LongType i = t;
+        for (; i + 3 * TPR < nv; i += 4 * TPR) {
+          VT v0 = pv[i], v1 = pv[i + TPR], v2 = pv[i + 2 * TPR], v3 = pv[i + 3 * TPR];
+#pragma unroll
+          for (int e = 0; e < V; e++) {
+            acc = Op::apply(acc, pre<PRE, A>((A)to_float(v0.v[e])));
+            acc = Op::apply(acc, pre<PRE, A>((A)to_float(v1.v[e])));
+            acc = Op::apply(acc, pre<PRE, A>((A)to_float(v2.v[e])));
+            acc = Op::apply(acc, pre<PRE, A>((A)to_float(v3.v[e])));
+          }
+        }
+        for (; i < nv; i += TPR) {
+          VT v0 = pv[i];
+#pragma unroll
+          for (int e = 0; e < V; e++) acc = Op::apply(acc, pre<PRE, A>((A)to_float(v0.v[e])));
+        }
+        j = j0 + nv * V;
+      }
+      for (LongType q = j + t; q < j1; q += TPR) acc = Op::apply(acc, pre<PRE, A>((A)to_float(p[q])));
+    } else if (a.inner.rank == 1) {
+      const LongType st = a.inner.stride[0];
+      for (LongType q = j0 + t; q < j1; q += TPR) acc = Op::apply(acc, pre<PRE, A>((A)to_float(x[base + q * st])));
+    } else {
+      for (LongType q = j0 + t; q < j1; q += TPR)
+        acc = Op::apply(acc, pre<PRE, A>((A)to_float(x[base + walk<LongType>(a.inner, q)])));
+    }
+  }
+  if (TPR == 64) acc = wave_allreduce<Op>(acc);
+  else acc = block_allreduce<Op, 4, A>(acc, lds);
+  if (live && t == 0) {
+    if (a.splits == 1) {
+      const LongType zo = a.zLinear ? row : walk<LongType>(a.zOuter, row);
+      z[zo] = Conv<T>::from(post<A>(acc, a.postKind, a.innerLen));
+    } else {
+      partials[unit] = acc;
+    }
+  }
+}
+
+template <typename Op, typename T>
+__global__ __launch_bounds__(256) void reduce_finish(CoopArgs a, const typename Conv<T>::acc* __restrict__ partials,
+                                                     T* __restrict__ z) {
+  using A = typename Conv<T>::acc;
+  const LongType row = (LongType)blockIdx.x * 256 + threadIdx.x;
+  if (row >= a.outerLen) return;
+  A acc = Identity<Op, A>::v();
+  for (int s = 0; s < a.splits; s++) acc = Op::apply(acc, partials[row * a.splits + s]);
+  const LongType zo = a.zLinear ? row : walk<LongType>(a.zOuter, row);
+  z[zo] = Conv<T>::from(post<A>(acc, a.postKind, a.innerLen));
+}
+
+// ---- value reduce, one thread per output -----------------------------------------------------------------
+template <typename Op, int PRE, typename T>
+__global__ __launch_bounds__(256) void reduce_flat(CoopArgs a, const T* __restrict__ x, T* __restrict__ z) {
+  using A = typename Conv<T>::acc;
+  const LongType row = (LongType)blockIdx.x * 256 + threadIdx.x;
+  if (row >= a.outerLen) return;
+  const LongType base = walk<LongType>(a.outer, row);
+  A acc = Identity<Op, A>::v();
+  if (a.inner.rank == 1) {
+    const LongType st = a.inner.stride[0];
+    for (LongType q = 0; q < a.innerLen; q++) acc = Op::apply(acc, pre<PRE, A>((A)to_float(x[base + q * st])));
+  } else {
+    for (LongType q = 0; q < a.innerLen; q++)
+      acc = Op::apply(acc, pre<PRE, A>((A)to_float(x[base + walk<LongType>(a.inner, q)])));
+  }
+  const LongType zo = a.zLinear ? row : walk<LongType>(a.zOuter, row);
+  z[zo] = Conv<T>::from(post<A>(acc, a.postKind, a.innerLen));
+}
+
+// ---- planning shared by value and index flavours -----------------------------------------------------------
+struct LaunchShape {
+  int tpr;
+  int splits;
+  LongType segLen;
+  bool flat;
+  int vectorOk;
+};
+
+static LaunchShape shapeLaunch(const ReducePlan& p, size_t elemSize, const void* x, size_t partialSize, size_t scratchBytes) {
+  LaunchShape s;
+  const bool unitInner = p.inner.rank == 1 && p.inner.stride[0] == 1;
+  s.flat = !unitInner && p.outerLen >= 4096;
+  s.tpr = p.innerLen >= 2048 ? 256 : 64;
+  s.splits = 1;
+  s.segLen = p.innerLen;
+  // few outputs and a long run: cut the run so that the whole chip participates
+  const LongType targetBlocks = 1024;
+  const LongType rowsPerBlock = 256 / s.tpr;
+  const LongType blocksNow = (p.outerLen + rowsPerBlock - 1) / rowsPerBlock;
+  if (!s.flat && blocksNow < targetBlocks && p.innerLen >= 16384) {
+    LongType want = targetBlocks / (blocksNow > 0 ? blocksNow : 1);
+    LongType maxBySeg = p.innerLen / 8192;   // keep >= 8192 elements per segment
+    if (want > maxBySeg) want = maxBySeg;
+    LongType maxByScratch = (LongType)(scratchBytes / partialSize) / (p.outerLen > 0 ? p.outerLen : 1);
+    if (want > maxByScratch) want = maxByScratch;
+    if (want > 1) {
+      s.tpr = 256;
+      const LongType V = 16 / (LongType)elemSize;
+      LongType seg = (p.innerLen + want - 1) / want;
+      seg = (seg + 255) / 256 * 256;   // keeps segments vector-aligned
+      (void)V;
+      s.segLen = seg;
+      s.splits = (int)((p.innerLen + seg - 1) / seg);
+    }
+  }
+  // vector loads need 16-byte aligned row starts
+  const LongType V = 16 / (LongType)elemSize;
+  bool ok = unitInner && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+  for (int d = 0; d < p.outer.rank && ok; d++) if (p.outer.shape[d] > 1 && p.outer.stride[d] % V != 0) ok = false;
+  if (s.splits > 1 && s.segLen % V != 0) ok = false;
+  s.vectorOk = ok ? 1 : 0;
+  return s;
+}
+
+static CoopArgs makeArgs(const ReducePlan& p, const LaunchShape& s, int postKind) {
+  CoopArgs a;
+  a.outer = p.outer; a.inner = p.inner; a.zOuter = p.zOuter;
+  a.outerLen = p.outerLen; a.innerLen = p.innerLen;
+  a.segLen = s.segLen; a.splits = s.splits; a.zLinear = p.zLinear ? 1 : 0; a.postKind = postKind;
+  return a;
+}
+
+template <typename Op, int PRE, typename T>
+static void reduceTyped(hipStream_t st, const void* x, void* z, const ReducePlan& p, int postKind, void* scratch,
+                        size_t scratchBytes) {
+  using A = typename Conv<T>::acc;
+  LaunchShape s = shapeLaunch(p, sizeof(T), x, sizeof(A), scratchBytes);
+  CoopArgs a = makeArgs(p, s, postKind);
+  if (s.flat) {
+    hipLaunchKernelGGL((reduce_flat<Op, PRE, T>), dim3((unsigned)((p.outerLen + 255) / 256)), dim3(256), 0, st, a, (const T*)x, (T*)z);
+    return;
+  }
+  const LongType units = p.outerLen * s.splits;
+  if (s.tpr == 64) {
+    hipLaunchKernelGGL((reduce_coop<Op, PRE, T, 64>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, st, a, (const T*)x, (T*)z, (A*)scratch, s.vectorOk);
+  } else {
+    hipLaunchKernelGGL((reduce_coop<Op, PRE, T, 256>), dim3((unsigned)units), dim3(256), 0, st, a, (const T*)x, (T*)z, (A*)scratch, s.vectorOk);
+  }
+  if (s.splits > 1)
+    hipLaunchKernelGGL((reduce_finish<Op, T>), dim3((unsigned)((p.outerLen + 255) / 256)), dim3(256), 0, st, a, (const A*)scratch, (T*)z);
+}
+
+template <typename Op, int PRE>
+static void reduceDtype(hipStream_t st, DataType dt, const void* x, void* z, const ReducePlan& p, int postKind,
+                        void* scratch, size_t scratchBytes) {
+  switch (dt) {
+    case FLOAT32: return reduceTyped<Op, PRE, float>(st, x, z, p, postKind, scratch, scratchBytes);
+    case DOUBLE: return reduceTyped<Op, PRE, double>(st, x, z, p, postKind, scratch, scratchBytes);
+    case HALF: return reduceTyped<Op, PRE, f16_t>(st, x, z, p, postKind, scratch, scratchBytes);
+    case BFLOAT16: return reduceTyped<Op, PRE, bf16_t>(st, x, z, p, postKind, scratch, scratchBytes);
+    default: ND4J_THROW("reduce: unsupported dtype");
+  }
+}
+
+void launchReduce(hipStream_t st, ReduceKind k, DataType xdt, DataType zdt, const void* x, void* z, const ReducePlan& p,
+                  void* scratch, size_t scratchBytes) {
+  ND4J_REQUIRE(xdt == zdt, "reduce: output dtype must equal input dtype on this backend");
+  ND4J_REQUIRE(p.outerLen < (1LL << 31) * 4, "reduce: too many outputs");
+  if (p.outerLen == 0) return;
+  switch (k) {
+    case R_SUM: reduceDtype<SumOp, PRE_ID>(st, xdt, x, z, p, POST_ID, scratch, scratchBytes); break;
+    case R_MAX: reduceDtype<MaxOp, PRE_ID>(st, xdt, x, z, p, POST_ID, scratch, scratchBytes); break;
+    case R_MIN: reduceDtype<MinOp, PRE_ID>(st, xdt, x, z, p, POST_ID, scratch, scratchBytes); break;
+    case R_PROD: reduceDtype<ProdOp, PRE_ID>(st, xdt, x, z, p, POST_ID, scratch, scratchBytes); break;
+    case R_ASUM: reduceDtype<SumOp, PRE_ABS>(st, xdt, x, z, p, POST_ID, scratch, scratchBytes); break;
+    case R_AMAX: reduceDtype<MaxOp, PRE_ABS>(st, xdt, x, z, p, POST_ID, scratch, scratchBytes); break;
+    case R_AMIN: reduceDtype<MinOp, PRE_ABS>(st, xdt, x, z, p, POST_ID, scratch, scratchBytes); break;
+    case R_MEAN: reduceDtype<SumOp, PRE_ID>(st, xdt, x, z, p, POST_DIV_N, scratch, scratchBytes); break;
+    case R_AMEAN: reduceDtype<SumOp, PRE_ABS>(st, xdt, x, z, p, POST_DIV_N, scratch, scratchBytes); break;
+    case R_NORM1: reduceDtype<SumOp, PRE_ABS>(st, xdt, x, z, p, POST_ID, scratch, scratchBytes); break;
+    case R_NORM2: reduceDtype<SumOp, PRE_SQ>(st, xdt, x, z, p, POST_SQRT, scratch, scratchBytes); break;
+    case R_NORMMAX: reduceDtype<MaxOp, PRE_ABS>(st, xdt, x, z, p, POST_ID, scratch, scratchBytes); break;
+    case R_SQNORM: reduceDtype<SumOp, PRE_SQ>(st, xdt, x, z, p, POST_ID, scratch, scratchBytes); break;
+    default: ND4J_THROW("reduce: unknown op kind");
+  }
+  HIP_CHECK(hipGetLastError());
+}
+
+// ---- index reduce ------------------------------------------------------------------------------------------
+template <typename A> struct IdxVal { A v; int i; };
+
+// IK: 0 max, 1 min, 2 abs-max, 3 abs-min
+template <int IK, typename A>
+__device__ __forceinline__ A idxStart() {
+  if (IK == I_MAX) return -(A)INFINITY;
+  if (IK == I_AMAX) return (A)0;
+  return (A)INFINITY;
+}
+template <int IK, typename A>
+__device__ __forceinline__ A idxPre(A x) {
+  if (IK == I_AMAX || IK == I_AMIN) x = x < 0 ? -x : x;
+  // NaN can never win a strict comparison in the reference's scan: park it on the start value
+  if (x != x) x = idxStart<IK, A>();
+  return x;
+}
+// true if candidate (bv, bi) beats (av, ai); ties go to the lower index
+template <int IK, typename A>
+__device__ __forceinline__ bool idxBetter(A av, int ai, A bv, int bi) {
+  if (IK == I_MAX || IK == I_AMAX) return bv > av || (bv == av && bi < ai);
+  return bv < av || (bv == av && bi < ai);
+}
+template <int IK, typename A>
+__device__ __forceinline__ void idxMerge(A& av, int& ai, A bv, int bi) {
+  if (idxBetter<IK, A>(av, ai, bv, bi)) { av = bv; ai = bi; }
+}
+template <int IK>
+__device__ __forceinline__ void wave_idx_allreduce(float& v, int& i) {
+  idxMerge<IK, float>(v, i, dpp_f<0xB1>(v), dpp_i<0xB1>(i));
+  idxMerge<IK, float>(v, i, dpp_f<0x4E>(v), dpp_i<0x4E>(i));
+  idxMerge<IK, float>(v, i, dpp_f<0x141>(v), dpp_i<0x141>(i));
+  idxMerge<IK, float>(v, i, dpp_f<0x140>(v), dpp_i<0x140>(i));
+  idxMerge<IK, float>(v, i, __shfl_xor(v, 16, WAVE), __shfl_xor(i, 16, WAVE));
+  idxMerge<IK, float>(v, i, __shfl_xor(v, 32, WAVE), __shfl_xor(i, 32, WAVE));
+}
+template <int IK>
+__device__ __forceinline__ void wave_idx_allreduce(double& v, int& i) {
+#pragma unroll
+  for (int m = 1; m < WAVE; m <<= 1) idxMerge<IK, double>(v, i, __shfl_xor(v, m, WAVE), __shfl_xor(i, m, WAVE));
+}
+
+template <typename ZT>
+__device__ __forceinline__ void storeIndex(ZT* z, LongType off, int idx) { z[off] = (ZT)idx; }
+
+template <int IK, typename T, int TPR, typename ZT>
+__global__ __launch_bounds__(256) void index_coop(CoopArgs a, const T* __restrict__ x, ZT* __restrict__ z,
+                                                  IdxVal<typename Conv<T>::acc>* __restrict__ partials, int vectorOk) {
+  using A = typename Conv<T>::acc;
+  constexpr int V = 16 / sizeof(T);
+  constexpr int ROWS = 256 / TPR;
+  __shared__ A ldsV[4];
+  __shared__ int ldsI[4];
+  const int t = threadIdx.x % TPR;
+  const LongType unit = (LongType)blockIdx.x * ROWS + threadIdx.x / TPR;
+  const LongType row = unit / a.splits;
+  const int split = (int)(unit - row * a.splits);
+  A bv = idxStart<IK, A>();
+  int bi = 0x7fffffff;   // "no element seen": loses every tie
+  const bool live = row < a.outerLen;
+  if (live) {
+    const LongType base = walk<LongType>(a.outer, row);
+    const LongType j0 = (LongType)split * a.segLen;
+    LongType j1 = j0 + a.segLen;
+    if (j1 > a.innerLen) j1 = a.innerLen;
+    if (a.inner.rank == 1 && a.inner.stride[0] == 1) {
+      const T* p = x + base;
+      LongType j = j0;
+      if (vectorOk) {
+        using VT = Vec<T, V>;
+        const LongType nv = (j1 - j0) / V;
+        const VT* pv = reinterpret_cast<const VT*>(p + j0);
+        LongType i = t;
+        for (; i + 3 * TPR < nv; i += 4 * TPR) {
+          VT v0 = pv[i], v1 = pv[i + TPR], v2 = pv[i + 2 * TPR], v3 = pv[i + 3 * TPR];
+          // ascending index order inside a thread: a strict comparison keeps the first extreme
+#pragma unroll
+          for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v0.v[e])); int ci = (int)(j0 + i * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
+#pragma unroll
+          for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v1.v[e])); int ci = (int)(j0 + (i + TPR) * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
+#pragma unroll
+          for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v2.v[e])); int ci = (int)(j0 + (i + 2 * TPR) * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
+#pragma unroll
+          for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v3.v[e])); int ci = (int)(j0 + (i + 3 * TPR) * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
+        }
+        for (; i < nv; i += TPR) {
+          VT v0 = pv[i];
+#pragma unroll
+          for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v0.v[e])); int ci = (int)(j0 + i * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
+        }
+        j = j0 + nv * V;
+      }
+      for (LongType q = j + t; q < j1; q += TPR) { A c = idxPre<IK, A>((A)to_float(p[q])); if (idxBetter<IK, A>(bv, bi, c, (int)q)) { bv = c; bi = (int)q; } }
+    } else if (a.inner.rank == 1) {
+      const LongType st = a.inner.stride[0];
+      for (LongType q = j0 + t; q < j1; q += TPR) { A c = idxPre<IK, A>((A)to_float(x[base + q * st])); if (idxBetter<IK, A>(bv, bi, c, (int)q)) { bv = c; bi = (int)q; } }
+    } else {
+      for (LongType q = j0 + t; q < j1; q += TPR) { A c = idxPre<IK, A>((A)to_float(x[base + walk<LongType>(a.inner, q)])); if (idxBetter<IK, A>(bv, bi, c, (int)q)) { bv = c; bi = (int)q; } }
+    }
+  }
+  wave_idx_allreduce<IK>(bv, bi);
+  if (TPR == 256) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    if (lane == 0) { ldsV[w] = bv; ldsI[w] = bi; }
+    __syncthreads();
+    bv = ldsV[0]; bi = ldsI[0];
+#pragma unroll
+    for (int q = 1; q < 4; q++) idxMerge<IK, A>(bv, bi, ldsV[q], ldsI[q]);
+  }
+  if (live && t == 0) {
+    if (a.splits == 1) {
+      const LongType zo = a.zLinear ? row : walk<LongType>(a.zOuter, row);
+      storeIndex<ZT>(z, zo, bi == 0x7fffffff ? 0 : bi);
+    } else {
+      partials[unit].v = bv; partials[unit].i = bi;
+    }
+  }
+}
+
+template <int IK, typename T, typename ZT>
+__global__ __launch_bounds__(256) void index_finish(CoopArgs a, const IdxVal<typename Conv<T>::acc>* __restrict__ partials,
+                                                    ZT* __restrict__ z) {
+  using A = typename Conv<T>::acc;
+  const LongType row = (LongType)blockIdx.x * 256 + threadIdx.x;
+  if (row >= a.outerLen) return;
+  A bv = idxStart<IK, A>();
+  int bi = 0x7fffffff;
+  for (int s = 0; s < a.splits; s++) idxMerge<IK, A>(bv, bi, partials[row * a.splits + s].v, partials[row * a.splits + s].i);
+  const LongType zo = a.zLinear ? row : walk<LongType>(a.zOuter, row);
+  storeIndex<ZT>(z, zo, bi == 0x7fffffff ? 0 : bi);
+}
+
+template <int IK, typename T, typename ZT>
+__global__ __launch_bounds__(256) void index_flat(CoopArgs a, const T* __restrict__ x, ZT* __restrict__ z) {
+  using A = typename Conv<T>::acc;
+  const LongType row = (LongType)blockIdx.x * 256 + threadIdx.x;
+  if (row >= a.outerLen) return;
+  const LongType base = walk<LongType>(a.outer, row);
+  A bv = idxStart<IK, A>();
+  int bi = 0;
+  for (LongType q = 0; q < a.innerLen; q++) {
+    const LongType off = a.inner.rank == 1 ? q * a.inner.stride[0] : walk<LongType>(a.inner, q);
+    A c = idxPre<IK, A>((A)to_float(x[base + off]));
+    const bool better = (IK == I_MAX || IK == I_AMAX) ? c > bv : c < bv;
+    if (better) { bv = c; bi = (int)q; }
+  }
+  const LongType zo = a.zLinear ? row : walk<LongType>(a.zOuter, row);
+  storeIndex<ZT>(z, zo, bi);
+}
+
+template <int IK, typename T, typename ZT>
+static void indexTyped(hipStream_t st, const void* x, void* z, const ReducePlan& p, void* scratch, size_t scratchBytes) {
+  using A = typename Conv<T>::acc;
+  LaunchShape s = shapeLaunch(p, sizeof(T), x, sizeof(IdxVal<A>), scratchBytes);
+  CoopArgs a = makeArgs(p, s, POST_ID);
+  if (s.flat) {
+    hipLaunchKernelGGL((index_flat<IK, T, ZT>), dim3((unsigned)((p.outerLen + 255) / 256)), dim3(256), 0, st, a, (const T*)x, (ZT*)z);
+    return;
+  }
+  const LongType units = p.outerLen * s.splits;
+  if (s.tpr == 64)
+    hipLaunchKernelGGL((index_coop<IK, T, 64, ZT>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, st, a, (const T*)x, (ZT*)z, (IdxVal<A>*)scratch, s.vectorOk);
+  else
+    hipLaunchKernelGGL((index_coop<IK, T, 256, ZT>), dim3((unsigned)units), dim3(256), 0, st, a, (const T*)x, (ZT*)z, (IdxVal<A>*)scratch, s.vectorOk);
+  if (s.splits > 1)
+    hipLaunchKernelGGL((index_finish<IK, T, ZT>), dim3((unsigned)((p.outerLen + 255) / 256)), dim3(256), 0, st, a, (const IdxVal<A>*)scratch, (ZT*)z);
+}
+template <int IK, typename ZT>
+static void indexDtype(hipStream_t st, DataType dt, const void* x, void* z, const ReducePlan& p, void* scratch, size_t scratchBytes) {
+  switch (dt) {
+    case FLOAT32: return indexTyped<IK, float, ZT>(st, x, z, p, scratch, scratchBytes);
+    case DOUBLE: return indexTyped<IK, double, ZT>(st, x, z, p, scratch, scratchBytes);
+    case HALF: return indexTyped<IK, f16_t, ZT>(st, x, z, p, scratch, scratchBytes);
+    case BFLOAT16: return indexTyped<IK, bf16_t, ZT>(st, x, z, p, scratch, scratchBytes);
+    default: ND4J_THROW("index reduce: unsupported input dtype");
+  }
+}
+template <int IK>
+static void indexKind(hipStream_t st, DataType xdt, DataType zdt, const void* x, void* z, const ReducePlan& p, void* scratch, size_t scratchBytes) {
+  if (zdt == INT64) return indexDtype<IK, LongType>(st, xdt, x, z, p, scratch, scratchBytes);
+  if (zdt == INT32) return indexDtype<IK, int>(st, xdt, x, z, p, scratch, scratchBytes);
+  ND4J_THROW("index reduce: output must be INT32 or INT64");
+}
+void launchIndexReduce(hipStream_t st, IndexKind k, DataType xdt, DataType zdt, const void* x, void* z,
+                       const ReducePlan& p, void* scratch, size_t scratchBytes) {
+  ND4J_REQUIRE(p.innerLen < 0x7fffffffLL, "index reduce: sub-array longer than 2^31-1 elements");
+  if (p.outerLen == 0) return;
+  switch (k) {
+    case I_MAX: indexKind<I_MAX>(st, xdt, zdt, x, z, p, scratch, scratchBytes); break;
+    case I_MIN: indexKind<I_MIN>(st, xdt, zdt, x, z, p, scratch, scratchBytes); break;
+    case I_AMAX: indexKind<I_AMAX>(st, xdt, zdt, x, z, p, scratch, scratchBytes); break;
+    case I_AMIN: indexKind<I_AMIN>(st, xdt, zdt, x, z, p, scratch, scratchBytes); break;
+    default: ND4J_THROW("index reduce: unknown op kind");
+  }
+  HIP_CHECK(hipGetLastError());
+}
+
+}  // namespace nd4jhip

@@ -1,0 +1,390 @@
+// Row kernels: softmax and layer_norm.
+//
+// softmax (reference: libnd4j/include/ops/declarable/helpers/cpu/softmax.cpp:252-353)
+//   One wave (rows up to 64*NV*VEC elements) or one 256-thread block owns a row and keeps it in
+//   registers: one read of x, one write of z => algorithmic bytes 2*sizeof(T) per element, HBM-bound.
+//   Rows sit at offsets given by the outer dims of input and output separately, so a permuted input
+//   view with a contiguous last axis runs at the same speed as a dense one.
+//   clamp mode reproduces the reference's same-shape branch: max over finite values (0 if none),
+//   inf/nan mapped to max+-88, diff clamped to +-88, sum floored at 1e-6.  Plain mode is the fallback
+//   branch (max, sub, exp, sum, div).  All arithmetic in float (double for fp64 arrays).
+//
+// layer_norm (reference: generic/nn/layer_norm.cpp:35-79 = standardize (generic/transforms/
+//   standardize.cpp:34-78) * gain + bias): one fused pass instead of the reference's eight:
+//   mean, population variance, y = (x - mean) / sqrt(var + 1e-5) * gain + bias.
+#include "device.h"
+#include "kernels.h"
+#include "runtime.h"
+
+namespace nd4jhip {
+
+struct RowArgs {
+  DevShape outerX, outerZ;
+  LongType rows, rowLen, xInner, zInner;
+};
+
+template <typename A> __device__ __forceinline__ A r_exp(A x);
+template <> __device__ __forceinline__ float r_exp<float>(float x) { return expf(x); }
+template <> __device__ __forceinline__ double r_exp<double>(double x) { return exp(x); }
+template <typename A> __device__ __forceinline__ bool r_finite(A x) { return x == x && x != (A)INFINITY && x != -(A)INFINITY; }
+template <typename A> __device__ __forceinline__ A r_tmax();
+template <> __device__ __forceinline__ float r_tmax<float>() { return 3.4028234663852886e38f; }
+template <> __device__ __forceinline__ double r_tmax<double>() { return 1.7976931348623157e308; }
+
+template <typename Op, int TPR, typename A>
+__device__ __forceinline__ A row_allreduce(A v, A* lds) {
+  if (TPR == 64) return wave_allreduce<Op>(v);
+  return block_allreduce<Op, 4, A>(v, lds);
+}
+
+// softmax transform of one cached value given the row max
+template <typename A>
+__device__ __forceinline__ A softmax_term(A v, A mx, int clamp) {
+  if (clamp) {
+    if (!r_finite(v)) v = (v > 0 || v != v) ? (A)88 + mx : (A)-88 + mx;
+    A d = v - mx;
+    d = d > (A)88 ? (A)88 : d;
+    d = d < (A)-88 ? (A)-88 : d;
+    return r_exp<A>(d);
+  }
+  return r_exp<A>(v - mx);
+}
+
+// VEC == 1: element loads through xInner/zInner strides; VEC > 1: 16-byte loads, unit strides
+template <typename T, int TPR, int NV, int VEC>
+__global__ __launch_bounds__(256) void softmax_rows(RowArgs a, const T* __restrict__ x, T* __restrict__ z, int clamp) {
+  using A = typename Conv<T>::acc;
+  using VT = Vec<T, VEC>;
+  constexpr int ROWS = 256 / TPR;
+  __shared__ A lds[4];
+  const int t = threadIdx.x % TPR;
+  LongType row = (LongType)blockIdx.x * ROWS + threadIdx.x / TPR;
+  const bool live = row < a.rows;
+  if (!live) row = a.rows - 1;  // keep the wave convergent for the block-wide reductions
+  const LongType xb = walk<LongType>(a.outerX, row), zb = walk<LongType>(a.outerZ, row);
+  const LongType L = a.rowLen;
+  A vals[NV * VEC];
+  const A NEG = -r_tmax<A>();
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const LongType e0 = ((LongType)t + (LongType)i * TPR) * VEC;
+    if (VEC > 1) {
+      if (e0 < L) {
+        VT v = *reinterpret_cast<const VT*>(x + xb + e0);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) vals[i * VEC + e] = (A)to_float(v.v[e]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) vals[i * VEC + e] = NEG;
+      }
+    } else {
+      vals[i] = e0 < L ? (A)to_float(x[xb + e0 * a.xInner]) : NEG;
+    }
+  }
+  A mx = NEG;
+#pragma unroll
+  for (int i = 0; i < NV * VEC; i++) {
+    A v = vals[i];
+    if (clamp) { if (r_finite(v)) mx = v > mx ? v : mx; }
+    else mx = v > mx ? v : mx;
+  }
+  mx = row_allreduce<MaxOp, TPR, A>(mx, lds);
+  if (clamp && mx == NEG) mx = (A)0;
+  A sum = (A)0;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const LongType e0 = ((LongType)t + (LongType)i * TPR) * VEC;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+      if (e0 + e < L) { A r = softmax_term<A>(vals[i * VEC + e], mx, clamp); vals[i * VEC + e] = r; sum += r; }
+    }
+  }
+  sum = row_allreduce<SumOp, TPR, A>(sum, lds);
+  if (clamp) sum = sum > (A)1e-6f ? sum : (A)1e-6f;
+  if (!live) return;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const LongType e0 = ((LongType)t + (LongType)i * TPR) * VEC;
+    if (e0 >= L) continue;
+    if (VEC > 1) {
+      VT o;
+#pragma unroll
+      for (int e = 0; e < VEC; e++) o.v[e] = Conv<T>::from(vals[i * VEC + e] / sum);
+      *reinterpret_cast<VT*>(z + zb + e0) = o;
+    } else {
+      z[zb + e0 * a.zInner] = Conv<T>::from(vals[i] / sum);
+    }
+  }
+}
+
+// rows longer than the register budget: three passes over global memory, one block per row
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_long(RowArgs a, const T* __restrict__ x, T* __restrict__ z, int clamp) {
+  using A = typename Conv<T>::acc;
+  __shared__ A lds[4];
+  const LongType row = blockIdx.x;
+  const LongType xb = walk<LongType>(a.outerX, row), zb = walk<LongType>(a.outerZ, row);
+  const A NEG = -r_tmax<A>();
+  A mx = NEG;
+  for (LongType j = threadIdx.x; j < a.rowLen; j += 256) {
+    A v = (A)to_float(x[xb + j * a.xInner]);
+    if (clamp) { if (r_finite(v)) mx = v > mx ? v : mx; }
+    else mx = v > mx ? v : mx;
+  }
+  mx = block_allreduce<MaxOp, 4, A>(mx, lds);
+  if (clamp && mx == NEG) mx = (A)0;
+  A sum = (A)0;
+  for (LongType j = threadIdx.x; j < a.rowLen; j += 256) sum += softmax_term<A>((A)to_float(x[xb + j * a.xInner]), mx, clamp);
+  sum = block_allreduce<SumOp, 4, A>(sum, lds);
+  if (clamp) sum = sum > (A)1e-6f ? sum : (A)1e-6f;
+  for (LongType j = threadIdx.x; j < a.rowLen; j += 256)
+    z[zb + j * a.zInner] = Conv<T>::from(softmax_term<A>((A)to_float(x[xb + j * a.xInner]), mx, clamp) / sum);
+}
+
+// many short strided rows (softmax over a non-last axis): one thread per row, neighbouring threads
+// own neighbouring rows so that accesses coalesce across the wave
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_flat(RowArgs a, const T* __restrict__ x, T* __restrict__ z, int clamp) {
+  using A = typename Conv<T>::acc;
+  const LongType row = (LongType)blockIdx.x * 256 + threadIdx.x;
+  if (row >= a.rows) return;
+  const LongType xb = walk<LongType>(a.outerX, row), zb = walk<LongType>(a.outerZ, row);
+  const A NEG = -r_tmax<A>();
+  A mx = NEG;
+  for (LongType j = 0; j < a.rowLen; j++) {
+    A v = (A)to_float(x[xb + j * a.xInner]);
+    if (clamp) { if (r_finite(v)) mx = v > mx ? v : mx; }
+    else mx = v > mx ? v : mx;
+  }
+  if (clamp && mx == NEG) mx = (A)0;
+  A sum = (A)0;
+  for (LongType j = 0; j < a.rowLen; j++) sum += softmax_term<A>((A)to_float(x[xb + j * a.xInner]), mx, clamp);
+  if (clamp) sum = sum > (A)1e-6f ? sum : (A)1e-6f;
+  for (LongType j = 0; j < a.rowLen; j++)
+    z[zb + j * a.zInner] = Conv<T>::from(softmax_term<A>((A)to_float(x[xb + j * a.xInner]), mx, clamp) / sum);
+}
+
+static RowArgs rowArgs(const RowPlan& p) {
+  RowArgs a;
+  a.outerX = p.outerX; a.outerZ = p.outerZ; a.rows = p.rows; a.rowLen = p.rowLen; a.xInner = p.xInner; a.zInner = p.zInner;
+  return a;
+}
+static bool rowsVectorOk(const RowPlan& p, const void* x, const void* z, int V) {
+  if (p.xInner != 1 || p.zInner != 1 || p.rowLen % V != 0) return false;
+  if ((reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(z) & 15)) return false;
+  for (int d = 0; d < p.outerX.rank; d++) {
+    if (p.outerX.shape[d] > 1 && (p.outerX.stride[d] % V != 0 || p.outerZ.stride[d] % V != 0)) return false;
+  }
+  return true;
+}
+
+template <typename T>
+static void softmaxTyped(hipStream_t s, const void* x, void* z, const RowPlan& p, int clamp) {
+  constexpr int V = 16 / sizeof(T);
+  RowArgs a = rowArgs(p);
+  const T* xt = (const T*)x;
+  T* zt = (T*)z;
+  const LongType L = p.rowLen;
+  if (p.xInner != 1 && p.rows >= 4096 && L <= 4096) {
+    hipLaunchKernelGGL((softmax_flat<T>), dim3((unsigned)((p.rows + 255) / 256)), dim3(256), 0, s, a, xt, zt, clamp);
+    return;
+  }
+  const unsigned gw = (unsigned)((p.rows + 3) / 4), gb = (unsigned)p.rows;
+  if (rowsVectorOk(p, x, z, V)) {
+    const LongType perWave = 64 * V, perBlock = 256 * V;
+#define SM(TPR, NV, GRID) hipLaunchKernelGGL((softmax_rows<T, TPR, NV, V>), dim3(GRID), dim3(256), 0, s, a, xt, zt, clamp)
+    if (L <= perWave) { SM(64, 1, gw); return; }
+    if (L <= 2 * perWave) { SM(64, 2, gw); return; }
+    if (L <= 4 * perWave) { SM(64, 4, gw); return; }
+    if (L <= 4 * perBlock && p.rows < 2048) { SM(256, 4, gb); return; }   // few rows: spread each over a block
+    if (L <= 8 * perWave) { SM(64, 8, gw); return; }
+    if (L <= 4 * perBlock) { SM(256, 4, gb); return; }
+    if (L <= 8 * perBlock) { SM(256, 8, gb); return; }
+#undef SM
+  } else {
+    if (L <= 64 * 16) { hipLaunchKernelGGL((softmax_rows<T, 64, 16, 1>), dim3(gw), dim3(256), 0, s, a, xt, zt, clamp); return; }
+    if (L <= 256 * 32) { hipLaunchKernelGGL((softmax_rows<T, 256, 32, 1>), dim3(gb), dim3(256), 0, s, a, xt, zt, clamp); return; }
+  }
+  hipLaunchKernelGGL((softmax_long<T>), dim3(gb), dim3(256), 0, s, a, xt, zt, clamp);
+}
+
+void launchSoftmax(hipStream_t s, DataType dt, const void* x, void* z, const RowPlan& p, bool clampMode) {
+  if (p.rows == 0 || p.rowLen == 0) return;
+  ND4J_REQUIRE(p.rows < (1LL << 31), "softmax: too many rows");
+  switch (dt) {
+    case FLOAT32: softmaxTyped<float>(s, x, z, p, clampMode); break;
+    case DOUBLE: softmaxTyped<double>(s, x, z, p, clampMode); break;
+    case HALF: softmaxTyped<f16_t>(s, x, z, p, clampMode); break;
+    case BFLOAT16: softmaxTyped<bf16_t>(s, x, z, p, clampMode); break;
+    default: ND4J_THROW("softmax: unsupported dtype");
+  }
+  HIP_CHECK(hipGetLastError());
+}
+
+// ---- layer_norm -------------------------------------------------------------------------------------------
+template <typename A> __device__ __forceinline__ A r_sqrt(A x);
+template <> __device__ __forceinline__ float r_sqrt<float>(float x) { return sqrtf(x); }
+template <> __device__ __forceinline__ double r_sqrt<double>(double x) { return sqrt(x); }
+
+template <typename T, int TPR, int NV, int VEC>
+__global__ __launch_bounds__(256) void layernorm_rows(RowArgs a, const T* __restrict__ x, const T* __restrict__ gain,
+                                                      const T* __restrict__ bias, T* __restrict__ z, float eps) {
+  using A = typename Conv<T>::acc;
+  using VT = Vec<T, VEC>;
+  constexpr int ROWS = 256 / TPR;
+  __shared__ A lds[4];
+  const int t = threadIdx.x % TPR;
+  LongType row = (LongType)blockIdx.x * ROWS + threadIdx.x / TPR;
+  const bool live = row < a.rows;
+  if (!live) row = a.rows - 1;
+  const LongType xb = walk<LongType>(a.outerX, row), zb = walk<LongType>(a.outerZ, row);
+  const LongType L = a.rowLen;
+  A vals[NV * VEC];
+  A sum = (A)0;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const LongType e0 = ((LongType)t + (LongType)i * TPR) * VEC;
+    if (VEC > 1) {
+      if (e0 < L) {
+        VT v = *reinterpret_cast<const VT*>(x + xb + e0);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) { vals[i * VEC + e] = (A)to_float(v.v[e]); sum += vals[i * VEC + e]; }
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) vals[i * VEC + e] = (A)0;
+      }
+    } else {
+      vals[i] = e0 < L ? (A)to_float(x[xb + e0 * a.xInner]) : (A)0;
+      sum += vals[i];
+    }
+  }
+  sum = row_allreduce<SumOp, TPR, A>(sum, lds);
+  const A mean = sum / (A)L;
+  A sq = (A)0;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const LongType e0 = ((LongType)t + (LongType)i * TPR) * VEC;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) if (e0 + e < L) { A d = vals[i * VEC + e] - mean; sq += d * d; }
+  }
+  sq = row_allreduce<SumOp, TPR, A>(sq, lds);
+  const A var = L > 1 ? sq / (A)L : (A)0;
+  const A sd = r_sqrt<A>(var + (A)eps);
+  if (!live) return;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const LongType e0 = ((LongType)t + (LongType)i * TPR) * VEC;
+    if (e0 >= L) continue;
+    if (VEC > 1) {
+      VT g = *reinterpret_cast<const VT*>(gain + e0), b, o;
+      if (bias) b = *reinterpret_cast<const VT*>(bias + e0);
+#pragma unroll
+      for (int e = 0; e < VEC; e++) {
+        A y = (vals[i * VEC + e] - mean) / sd * (A)to_float(g.v[e]);
+        if (bias) y += (A)to_float(b.v[e]);
+        o.v[e] = Conv<T>::from(y);
+      }
+      *reinterpret_cast<VT*>(z + zb + e0) = o;
+    } else {
+      A y = (vals[i] - mean) / sd * (A)to_float(gain[e0]);
+      if (bias) y += (A)to_float(bias[e0]);
+      z[zb + e0 * a.zInner] = Conv<T>::from(y);
+    }
+  }
+}
+
+template <typename T>
+static void layerNormTyped(hipStream_t s, const void* x, const void* gain, const void* bias, void* z, const RowPlan& p, float eps) {
+  constexpr int V = 16 / sizeof(T);
+  RowArgs a = rowArgs(p);
+  const T* xt = (const T*)x; const T* gt = (const T*)gain; const T* bt = (const T*)bias; T* zt = (T*)z;
+  const LongType L = p.rowLen;
+  const unsigned gw = (unsigned)((p.rows + 3) / 4), gb = (unsigned)p.rows;
+  bool vec = rowsVectorOk(p, x, z, V) && (reinterpret_cast<uintptr_t>(gain) & 15) == 0 && (!bias || (reinterpret_cast<uintptr_t>(bias) & 15) == 0);
+  if (vec) {
+    const LongType perWave = 64 * V, perBlock = 256 * V;
+#define LN(TPR, NV, GRID) hipLaunchKernelGGL((layernorm_rows<T, TPR, NV, V>), dim3(GRID), dim3(256), 0, s, a, xt, gt, bt, zt, eps)
+    if (L <= perWave) { LN(64, 1, gw); return; }
+    if (L <= 2 * perWave) { LN(64, 2, gw); return; }
+    if (L <= 4 * perWave) { LN(64, 4, gw); return; }
+    if (L <= 8 * perWave) { LN(64, 8, gw); return; }
+    if (L <= 4 * perBlock) { LN(256, 4, gb); return; }
+    if (L <= 8 * perBlock) { LN(256, 8, gb); return; }
+#undef LN
+  }
+  if (L <= 64 * 16) { hipLaunchKernelGGL((layernorm_rows<T, 64, 16, 1>), dim3(gw), dim3(256), 0, s, a, xt, gt, bt, zt, eps); return; }
+  if (L <= 256 * 32) { hipLaunchKernelGGL((layernorm_rows<T, 256, 32, 1>), dim3(gb), dim3(256), 0, s, a, xt, gt, bt, zt, eps); return; }
+  ND4J_THROW("layer_norm: rows longer than 8192 elements take the generic path");
+}
+
+void launchLayerNormRows(hipStream_t s, DataType dt, const void* x, const void* gain, const void* bias, void* z,
+                         const RowPlan& p, float eps) {
+  if (p.rows == 0 || p.rowLen == 0) return;
+  switch (dt) {
+    case FLOAT32: layerNormTyped<float>(s, x, gain, bias, z, p, eps); break;
+    case DOUBLE: layerNormTyped<double>(s, x, gain, bias, z, p, eps); break;
+    case HALF: layerNormTyped<f16_t>(s, x, gain, bias, z, p, eps); break;
+    case BFLOAT16: layerNormTyped<bf16_t>(s, x, gain, bias, z, p, eps); break;
+    default: ND4J_THROW("layer_norm: unsupported dtype");
+  }
+  HIP_CHECK(hipGetLastError());
+}
+
+// generic axes: one block per statistics group, elements reached through the inner walk; gain/bias are
+// indexed by the coordinate along the channel axis
+struct LnArgs {
+  DevShape outerX, innerX, outerZ, innerZ;
+  LongType outerLen, innerLen;
+  int channelInInner, channelPos;
+};
+__device__ __forceinline__ LongType coordAt(const DevShape& s, LongType idx, int pos) {
+  for (int d = s.rank - 1; d >= 0; d--) {
+    LongType q = idx / s.shape[d], c = idx - q * s.shape[d];
+    if (d == pos) return c;
+    idx = q;
+  }
+  return 0;
+}
+template <typename T>
+__global__ __launch_bounds__(256) void layernorm_generic(LnArgs a, const T* __restrict__ x, const T* __restrict__ gain,
+                                                         const T* __restrict__ bias, T* __restrict__ z, float eps) {
+  using A = typename Conv<T>::acc;
+  __shared__ A lds[4];
+  const LongType o = blockIdx.x;
+  const LongType xb = walk<LongType>(a.outerX, o), zb = walk<LongType>(a.outerZ, o);
+  A sum = (A)0;
+  for (LongType j = threadIdx.x; j < a.innerLen; j += 256) sum += (A)to_float(x[xb + walk<LongType>(a.innerX, j)]);
+  sum = block_allreduce<SumOp, 4, A>(sum, lds);
+  const A mean = sum / (A)a.innerLen;
+  A sq = (A)0;
+  for (LongType j = threadIdx.x; j < a.innerLen; j += 256) { A d = (A)to_float(x[xb + walk<LongType>(a.innerX, j)]) - mean; sq += d * d; }
+  sq = block_allreduce<SumOp, 4, A>(sq, lds);
+  const A var = a.innerLen > 1 ? sq / (A)a.innerLen : (A)0;
+  const A sd = r_sqrt<A>(var + (A)eps);
+  const LongType cOuter = a.channelInInner ? 0 : coordAt(a.outerX, o, a.channelPos);
+  for (LongType j = threadIdx.x; j < a.innerLen; j += 256) {
+    const LongType c = a.channelInInner ? coordAt(a.innerX, j, a.channelPos) : cOuter;
+    A y = ((A)to_float(x[xb + walk<LongType>(a.innerX, j)]) - mean) / sd * (A)to_float(gain[c]);
+    if (bias) y += (A)to_float(bias[c]);
+    z[zb + walk<LongType>(a.innerZ, j)] = Conv<T>::from(y);
+  }
+}
+void launchLayerNormGeneric(hipStream_t s, DataType dt, const void* x, const void* gain, const void* bias, void* z,
+                            const LnGenericPlan& p, float eps) {
+  if (p.outerLen == 0 || p.innerLen == 0) return;
+  ND4J_REQUIRE(p.outerLen < (1LL << 31), "layer_norm: too many groups");
+  LnArgs a;
+  a.outerX = p.outerX; a.innerX = p.innerX; a.outerZ = p.outerZ; a.innerZ = p.innerZ;
+  a.outerLen = p.outerLen; a.innerLen = p.innerLen; a.channelInInner = p.channelInInner; a.channelPos = p.channelPos;
+  dim3 g((unsigned)p.outerLen), b(256);
+  switch (dt) {
+    case FLOAT32: hipLaunchKernelGGL((layernorm_generic<float>), g, b, 0, s, a, (const float*)x, (const float*)gain, (const float*)bias, (float*)z, eps); break;
+    case DOUBLE: hipLaunchKernelGGL((layernorm_generic<double>), g, b, 0, s, a, (const double*)x, (const double*)gain, (const double*)bias, (double*)z, eps); break;
+    case HALF: hipLaunchKernelGGL((layernorm_generic<f16_t>), g, b, 0, s, a, (const f16_t*)x, (const f16_t*)gain, (const f16_t*)bias, (f16_t*)z, eps); break;
+    case BFLOAT16: hipLaunchKernelGGL((layernorm_generic<bf16_t>), g, b, 0, s, a, (const bf16_t*)x, (const bf16_t*)gain, (const bf16_t*)bias, (bf16_t*)z, eps); break;
+    default: ND4J_THROW("layer_norm: unsupported dtype");
+  }
+  HIP_CHECK(hipGetLastError());
+}
+
+}  // namespace nd4jhip

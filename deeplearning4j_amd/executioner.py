@@ -1,0 +1,251 @@
+"""Host-side op executioner: the stand-in for the Java `NativeOpExecutioner` / `CudaExecutioner`.
+
+Follows the call protocol of
+nd4j/nd4j-backends/nd4j-backend-impls/nd4j-cpu-backend-common/src/main/java/org/nd4j/linalg/cpu/nativecpu/ops/NativeOpExecutioner.java:
+  * legacy ops: allocate z when it is not given (:676), pass array handles, poll lastErrorCode() after
+    the call (:194, :440, :715);
+  * index accumulations produce INT64 (:157); reduce "same" keeps the input type, reduce "float" of a
+    float input keeps it too (:304-305);
+  * custom ops: build an OpContext, ask calculateOutputShapes2 for the output shapes when outputs are
+    not supplied, push arrays and T/I/B/D arguments, call execCustomOp2 and turn a non-zero status into
+    an exception carrying lastErrorMessage() (:1001-1091).
+"""
+import ctypes
+
+import numpy as np
+
+from . import nativeops as N
+from .ndarray import BOOL, DOUBLE, FLOAT32, HALF, BFLOAT16, INT32, INT64, NDArray  # noqa: F401
+
+
+# opNum tables: libnd4j/include/loops/legacy_ops.h
+class Pairwise:
+    Add, CopyPws, Divide, Multiply, ReverseSubtract, Subtract, MaxPairwise, MinPairwise = 0, 1, 2, 3, 5, 6, 7, 8
+    ReverseDivide, SquaredSubtract = 11, 20
+
+
+class TransformStrict:
+    Cosine, Exp, Log, Sigmoid, Sin, SoftPlus, Tanh, Swish, Erf, GELU, PreciseGELU = 22, 23, 24, 26, 27, 28, 29, 43, 45, 53, 55
+
+
+class TransformFloat:
+    Sqrt, RSqrt = 1, 3
+
+
+class TransformSame:
+    Abs, Neg, Cube, OneMinus, Reciprocal, Square, Identity, Copy = 0, 3, 6, 7, 11, 12, 15, 21
+
+
+class ReduceSame:
+    Sum, Max, Min, Prod, ASum, AMax, AMin = 0, 1, 2, 3, 4, 5, 6
+
+
+class ReduceFloat:
+    Mean, AMean, Norm1, Norm2, NormMax, NormFrobenius, SquaredNorm = 0, 1, 2, 3, 4, 5, 7
+
+
+class IndexReduce:
+    IndexMax, IndexMin, IndexAbsoluteMax, IndexAbsoluteMin = 0, 1, 2, 3
+
+
+class Scalar:
+    Add, Subtract, Multiply, Divide, ReverseDivide, ReverseSubtract, MaxPairwise, MinPairwise, CopyPws = 0, 1, 2, 3, 4, 5, 6, 13, 14
+
+
+class Broadcast:
+    Add, Subtract, Multiply, Divide, ReverseDivide, ReverseSubtract, CopyPws = 0, 1, 2, 3, 4, 5, 6
+
+
+def _reduced_shape(shape, dims, keep_dims):
+    if dims is None or len(dims) == 0:
+        return [1] * len(shape) if keep_dims else []
+    r = len(shape)
+    dims = sorted(d + r if d < 0 else d for d in dims)
+    out = []
+    for i, s in enumerate(shape):
+        if i in dims:
+            if keep_dims:
+                out.append(1)
+        else:
+            out.append(s)
+    return out
+
+
+def _dims_array(dims):
+    return NDArray.from_numpy(np.asarray(dims, dtype=np.int64))
+
+
+class OpContext:
+    """graph::Context wrapper (the Java side's CpuOpContext / CudaOpContext)."""
+
+    def __init__(self):
+        self.ptr = N.load().createGraphContext(1)
+        self._keep = []
+
+    def set_inputs(self, arrays):
+        L = N.load()
+        arr = (ctypes.c_void_p * len(arrays))(*[a.handle for a in arrays])
+        L.setGraphContextInputArraysArr(self.ptr, len(arrays), arr)
+        N.check("setGraphContextInputArraysArr")
+        self._keep.append(list(arrays))
+
+    def set_outputs(self, arrays):
+        L = N.load()
+        for i, a in enumerate(arrays):
+            if a is not None:
+                L.setGraphContextOutputArray(self.ptr, i, a.handle)
+        N.check("setGraphContextOutputArray")
+        self._keep.append(list(arrays))
+
+    def set_args(self, t_args=(), i_args=(), b_args=(), d_args=()):
+        L = N.load()
+        if len(t_args):
+            L.setGraphContextTArguments(self.ptr, (ctypes.c_double * len(t_args))(*[float(t) for t in t_args]), len(t_args))
+        if len(i_args):
+            L.setGraphContextIArguments(self.ptr, (ctypes.c_longlong * len(i_args))(*[int(i) for i in i_args]), len(i_args))
+        if len(b_args):
+            L.setGraphContextBArguments(self.ptr, (ctypes.c_bool * len(b_args))(*[bool(b) for b in b_args]), len(b_args))
+        if len(d_args):
+            L.setGraphContextDArguments(self.ptr, (ctypes.c_int * len(d_args))(*[int(d) for d in d_args]), len(d_args))
+
+    def close(self):
+        if self.ptr:
+            N.load().deleteGraphContext(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Executioner:
+    def __init__(self):
+        self.L = N.load()
+        self.L.initializeDevicesAndFunctions()
+        N.check("initializeDevicesAndFunctions")
+        self._hashes = {}
+        for item in self.L.getAllCustomOps().decode().split(";"):
+            if item:
+                parts = item.split(":")
+                self._hashes[parts[0]] = int(parts[1])
+
+    # ---- legacy ops ----
+    def exec_transform_strict(self, op_num, x, z=None):
+        z = z if z is not None else NDArray.empty(x.shape, x.dtype)
+        self.L.execTransformStrict(None, op_num, x.handle, None, z.handle)
+        N.check("execTransformStrict")
+        return z
+
+    def exec_transform_float(self, op_num, x, z=None):
+        z = z if z is not None else NDArray.empty(x.shape, x.dtype)
+        self.L.execTransformFloat(None, op_num, x.handle, None, z.handle)
+        N.check("execTransformFloat")
+        return z
+
+    def exec_transform_same(self, op_num, x, z=None):
+        z = z if z is not None else NDArray.empty(x.shape, x.dtype)
+        self.L.execTransformSame(None, op_num, x.handle, None, z.handle)
+        N.check("execTransformSame")
+        return z
+
+    def exec_assign(self, x, z):
+        self.L.execTransformAny(None, 0, x.handle, None, z.handle)
+        N.check("execTransformAny")
+        return z
+
+    def exec_pairwise(self, op_num, x, y, z=None):
+        z = z if z is not None else NDArray.empty(x.shape, x.dtype)
+        self.L.execPairwiseTransform(None, op_num, x.handle, y.handle, z.handle, None)
+        N.check("execPairwiseTransform")
+        return z
+
+    def exec_scalar(self, op_num, x, scalar, z=None):
+        z = z if z is not None else NDArray.empty(x.shape, x.dtype)
+        s = scalar if isinstance(scalar, NDArray) else NDArray.scalar(scalar, x.dtype)
+        self.L.execScalar(None, op_num, x.handle, z.handle, s.handle, None)
+        N.check("execScalar")
+        return z
+
+    def exec_broadcast(self, op_num, x, y, dims, z=None):
+        z = z if z is not None else NDArray.empty(x.shape, x.dtype)
+        d = _dims_array(dims)
+        self.L.execBroadcast(None, op_num, x.handle, y.handle, z.handle, None, d.handle)
+        N.check("execBroadcast")
+        return z
+
+    def _reduce(self, scalar_fn, dim_fn, name, op_num, x, dims, keep_dims, z, zdtype):
+        if z is None:
+            z = NDArray.empty(_reduced_shape(x.shape, dims, keep_dims), zdtype)
+        if dims is None or len(dims) == 0:
+            scalar_fn(None, op_num, x.handle, None, z.handle)
+        else:
+            d = _dims_array(dims)
+            dim_fn(None, op_num, x.handle, None, z.handle, d.handle)
+        N.check(name)
+        return z
+
+    def exec_reduce_same(self, op_num, x, dims=None, keep_dims=False, z=None):
+        return self._reduce(self.L.execReduceSame, self.L.execReduceSame2, "execReduceSame", op_num, x, dims, keep_dims, z, x.dtype)
+
+    def exec_reduce_float(self, op_num, x, dims=None, keep_dims=False, z=None):
+        return self._reduce(self.L.execReduceFloat, self.L.execReduceFloat2, "execReduceFloat", op_num, x, dims, keep_dims, z, x.dtype)
+
+    def exec_index_reduce(self, op_num, x, dims=None, keep_dims=False, z=None):
+        return self._reduce(self.L.execIndexReduceScalar, self.L.execIndexReduce, "execIndexReduce", op_num, x, dims, keep_dims, z, INT64)
+
+    # ---- custom ops ----
+    def op_hash(self, name):
+        if name not in self._hashes:
+            raise N.NativeOpsError("custom op '%s' is not registered in nd4j-hip" % name)
+        return self._hashes[name]
+
+    def calculate_output_shapes(self, name, inputs, t_args=(), i_args=(), b_args=(), d_args=()):
+        ctx = OpContext()
+        try:
+            ctx.set_inputs(inputs)
+            ctx.set_args(t_args, i_args, b_args, d_args)
+            sl = self.L.calculateOutputShapes2(None, self.op_hash(name), ctx.ptr)
+            N.check("calculateOutputShapes2")
+            out = []
+            for i in range(self.L.getShapeListSize(sl)):
+                p = self.L.getShape(sl, i)
+                rank = p[0]
+                n = 6 if rank == 0 else 2 * rank + 4
+                out.append(np.array([p[j] for j in range(n)], dtype=np.int64))
+            self.L.deleteShapeList(sl)
+            return out
+        finally:
+            ctx.close()
+
+    def exec_custom(self, name, inputs, outputs=None, t_args=(), i_args=(), b_args=(), d_args=(), n_outputs=None):
+        """Returns the list of output arrays.  `outputs=None` sizes them with calculateOutputShapes2;
+        `n_outputs` limits how many of the reported outputs are materialised."""
+        from .ndarray import DT_FLAG
+        if outputs is None:
+            shapes = self.calculate_output_shapes(name, inputs, t_args, i_args, b_args, d_args)
+            if n_outputs is not None:
+                shapes = shapes[:n_outputs]
+            outputs = []
+            for si in shapes:
+                rank = int(si[0])
+                extra = int(si[3] if rank == 0 else si[2 * rank + 1])
+                dt = [k for k, v in DT_FLAG.items() if extra & v][0]
+                order = chr(int(si[-1]))
+                outputs.append(NDArray.empty([int(s) for s in si[1:1 + rank]], dt, order))
+        ctx = OpContext()
+        try:
+            ctx.set_inputs(inputs)
+            ctx.set_outputs(outputs)
+            ctx.set_args(t_args, i_args, b_args, d_args)
+            status = self.L.execCustomOp2(None, self.op_hash(name), ctx.ptr)
+            if status != 0:
+                raise N.NativeOpsError("Op [%s] execution failed: %s" % (name, self.L.lastErrorMessage().decode(errors="replace")))
+        finally:
+            ctx.close()
+        return outputs
+
+    def synchronize(self):
+        self.L.streamSynchronize(None)
+        N.check("streamSynchronize")

@@ -1,0 +1,226 @@
+/*
+ * nd4j-hip: C ABI of the MI355X (gfx950) op backend.
+ *
+ * Every entry point below replaces the function of the same name in the reference's
+ * libnd4j/include/legacy/NativeOps.h (cited as "ref :line" on each declaration).  The reference
+ * exports these with C++ linkage and lets JavaCPP parse the C++ header; here they are `extern "C"`
+ * with opaque handle types so that any FFI (JavaCPP, JNI, ctypes) can bind them.  Two consequences:
+ *   - the reference's C++ overloads get distinct names here (getOpaqueNDArrayShapeInfoLength,
+ *     lc*FromHandle); everything else keeps its name, argument order and meaning;
+ *   - handles are plain pointers: OpaqueNDArray = array handle created by createOpaqueNDArray,
+ *     OpaqueDataBuffer = host+device buffer pair, OpaqueContext = per-op argument bag.
+ *
+ * Error convention (ref legacy/cpu/NativeOps.cpp:1118-1121): exec* functions return void; a failure
+ * stores {code, message} in a process-wide slot which the caller polls with lastErrorCode() /
+ * lastErrorMessage().  execCustomOp2 additionally returns a status (0 = OK).  The slot keeps the last
+ * failure until lastErrorMessage() is fetched, which resets the code to 0 (ref
+ * execution/impl/ErrorReference.cpp:28-34); successful calls do not touch it.
+ *
+ * Device model: this library has no CPU execution path.  All compute entry points run HIP kernels on
+ * the current device and fail with an error if no device is present.  Arrays carry a host ("primary")
+ * and a device ("special") buffer; exec* synchronises host->device lazily by the buffers' read/write
+ * stamps (ref array/cuda/DataBuffer.cu:597-606) and marks outputs as written on the device.
+ * Legacy exec* calls are asynchronous on the execution stream; execCustomOp2 synchronises before it
+ * returns (ref legacy/cuda/NativeOps.cu:118).
+ */
+#ifndef ND4JHIP_NATIVEOPS_H
+#define ND4JHIP_NATIVEOPS_H
+
+#include <stdbool.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ND4JHIP_EXPORT __attribute__((visibility("default")))
+
+typedef long long Nd4jLong;  /* sd::LongType */
+typedef void* Nd4jPointer;   /* sd::Pointer */
+typedef int Nd4jStatus;      /* sd::Status: 0 = OK, non-zero = failure (ref system/common.h:184-187) */
+
+typedef struct Nd4jHipDataBuffer OpaqueDataBuffer;            /* ref :57  sd::InteropDataBuffer */
+typedef struct Nd4jHipNDArray* OpaqueNDArray;                 /* ref :61  sd::NDArray* */
+typedef OpaqueNDArray* OpaqueNDArrayArr;                      /* ref :62 */
+typedef struct Nd4jHipContext OpaqueContext;                  /* ref :60  sd::graph::Context */
+typedef struct Nd4jHipShapeList OpaqueShapeList;              /* ref :59 */
+typedef struct Nd4jHipTadPack OpaqueTadPack;                  /* ref :68 */
+typedef struct Nd4jHipConstantShapeBuffer* OpaqueConstantShapeBuffer; /* ref :71 */
+typedef struct Nd4jHipLaunchContext* OpaqueLaunchContext;     /* ref :63 */
+
+/* dtype codes (ref array/DataType.h:26-50) */
+enum Nd4jDataType {
+  ND4J_BOOL = 1, ND4J_HALF = 3, ND4J_FLOAT32 = 5, ND4J_DOUBLE = 6, ND4J_INT8 = 7, ND4J_INT16 = 8, ND4J_INT32 = 9,
+  ND4J_INT64 = 10, ND4J_UINT8 = 11, ND4J_UINT16 = 12, ND4J_UINT32 = 13, ND4J_UINT64 = 14, ND4J_BFLOAT16 = 17
+};
+
+/* ---- library / device -------------------------------------------------------------------------- */
+ND4JHIP_EXPORT void initializeDevicesAndFunctions(void);                               /* ref :225 */
+ND4JHIP_EXPORT void initializeShapeCache(void);                                        /* ref :238 */
+ND4JHIP_EXPORT void initializeTadCache(void);                                          /* ref :252 */
+ND4JHIP_EXPORT int getAvailableDevices(void);                                          /* ref :273 */
+ND4JHIP_EXPORT int setDevice(int deviceId);                                            /* ref :262 */
+ND4JHIP_EXPORT int getDevice(void);                                                    /* ref :318 */
+ND4JHIP_EXPORT const char* getDeviceName(int device);                                  /* ref :164 */
+ND4JHIP_EXPORT int getDeviceMajor(int device);                                         /* ref :311 */
+ND4JHIP_EXPORT int getDeviceMinor(int device);                                         /* ref :312 */
+ND4JHIP_EXPORT Nd4jLong getDeviceFreeMemory(int device);                               /* ref :264 */
+ND4JHIP_EXPORT Nd4jLong getDeviceFreeMemoryDefault(void);                              /* ref :263 */
+ND4JHIP_EXPORT Nd4jLong getDeviceTotalMemory(int device);                              /* ref :265 */
+ND4JHIP_EXPORT void enableDebugMode(bool reallyEnable);                                /* ref :274 */
+ND4JHIP_EXPORT void enableVerboseMode(bool reallyEnable);                              /* ref :310 */
+ND4JHIP_EXPORT void setOmpNumThreads(int threads);                                     /* ref :278 (host threads are not used; kept as a no-op) */
+ND4JHIP_EXPORT int ompGetMaxThreads(void);                                             /* ref :276 */
+ND4JHIP_EXPORT void setElementThreshold(int num);                                      /* ref :319 (no-op) */
+ND4JHIP_EXPORT void setTADThreshold(int num);                                          /* ref :320 (no-op) */
+ND4JHIP_EXPORT int lastErrorCode(void);                                                /* ref :553 */
+ND4JHIP_EXPORT const char* lastErrorMessage(void);                                     /* ref :552 */
+
+/* memory, streams, events.  Streams travel as pointer-to-handle (hipStream_t*), events as the handle
+ * itself, exactly as the reference's device backend does (ref legacy/cuda/NativeOps.cu:1235-1260). */
+ND4JHIP_EXPORT Nd4jPointer mallocHost(Nd4jLong memorySize, int flags);                 /* ref :254 (pinned) */
+ND4JHIP_EXPORT Nd4jPointer mallocDevice(Nd4jLong memorySize, int deviceId, int flags); /* ref :255 */
+ND4JHIP_EXPORT int freeHost(Nd4jPointer pointer);                                      /* ref :256 */
+ND4JHIP_EXPORT int freeDevice(Nd4jPointer pointer, int deviceId);                      /* ref :257 */
+ND4JHIP_EXPORT Nd4jPointer createStream(void);                                         /* ref :259 */
+ND4JHIP_EXPORT Nd4jPointer createEvent(void);                                          /* ref :260 */
+ND4JHIP_EXPORT int registerEvent(Nd4jPointer event, Nd4jPointer stream);               /* ref :261 */
+ND4JHIP_EXPORT int destroyEvent(Nd4jPointer event);                                    /* ref :270 */
+ND4JHIP_EXPORT int streamSynchronize(Nd4jPointer stream);                              /* ref :271 */
+ND4JHIP_EXPORT int eventSynchronize(Nd4jPointer event);                                /* ref :272 */
+/* flags: 0 host->host, 1 host->device, 2 device->host, 3 device->device; `reserved` = stream (async) */
+ND4JHIP_EXPORT int memcpySync(Nd4jPointer dst, Nd4jPointer src, Nd4jLong size, int flags, Nd4jPointer reserved);  /* ref :266 */
+ND4JHIP_EXPORT int memcpyAsync(Nd4jPointer dst, Nd4jPointer src, Nd4jLong size, int flags, Nd4jPointer reserved); /* ref :267 */
+ND4JHIP_EXPORT int memsetSync(Nd4jPointer dst, int value, Nd4jLong size, int flags, Nd4jPointer reserved);        /* ref :268 */
+ND4JHIP_EXPORT int memsetAsync(Nd4jPointer dst, int value, Nd4jLong size, int flags, Nd4jPointer reserved);       /* ref :269 */
+
+/* launch context (ref :451-457,500-512) */
+ND4JHIP_EXPORT OpaqueLaunchContext defaultLaunchContext(void);                         /* ref :500 */
+ND4JHIP_EXPORT Nd4jPointer lcScalarPointer(OpaqueLaunchContext lc);                    /* ref :451 */
+ND4JHIP_EXPORT Nd4jPointer lcReductionPointer(OpaqueLaunchContext lc);                 /* ref :452 */
+ND4JHIP_EXPORT Nd4jPointer lcAllocationPointer(OpaqueLaunchContext lc);                /* ref :453 */
+ND4JHIP_EXPORT Nd4jPointer lcExecutionStream(OpaqueLaunchContext lc);                  /* ref :454 */
+ND4JHIP_EXPORT Nd4jPointer lcCopyStream(OpaqueLaunchContext lc);                       /* ref :455 */
+ND4JHIP_EXPORT Nd4jPointer lcBlasHandle(OpaqueLaunchContext lc);                       /* ref :456 (no vendor BLAS is used: returns NULL) */
+
+/* ---- data buffers (ref :466-488) ------------------------------------------------------------------- */
+ND4JHIP_EXPORT OpaqueDataBuffer* dbAllocateDataBuffer(Nd4jLong elements, int dataType, bool allocateBoth);        /* ref :487 */
+ND4JHIP_EXPORT OpaqueDataBuffer* allocateDataBuffer(Nd4jLong elements, int dataType, bool allocateBoth);          /* ref :496 */
+ND4JHIP_EXPORT OpaqueDataBuffer* dbCreateExternalDataBuffer(Nd4jLong elements, int dataType, Nd4jPointer primary, Nd4jPointer special); /* ref :488 */
+ND4JHIP_EXPORT OpaqueDataBuffer* dbCreateView(OpaqueDataBuffer* dataBuffer, Nd4jLong length);                     /* ref :486 */
+ND4JHIP_EXPORT Nd4jPointer dbPrimaryBuffer(OpaqueDataBuffer* dataBuffer);              /* ref :466 */
+ND4JHIP_EXPORT Nd4jPointer dbSpecialBuffer(OpaqueDataBuffer* dataBuffer);              /* ref :467 */
+ND4JHIP_EXPORT Nd4jLong dbBufferLength(OpaqueDataBuffer* dataBuffer);                  /* ref :181 */
+ND4JHIP_EXPORT void dbSetPrimaryBuffer(OpaqueDataBuffer* dataBuffer, Nd4jPointer primaryBuffer, Nd4jLong numBytes); /* ref :469 */
+ND4JHIP_EXPORT void dbSetSpecialBuffer(OpaqueDataBuffer* dataBuffer, Nd4jPointer specialBuffer, Nd4jLong numBytes); /* ref :470 */
+ND4JHIP_EXPORT void dbAllocatePrimaryBuffer(OpaqueDataBuffer* dataBuffer);             /* ref :471 */
+ND4JHIP_EXPORT void dbAllocateSpecialBuffer(OpaqueDataBuffer* dataBuffer);             /* ref :472 */
+ND4JHIP_EXPORT void dbExpandBuffer(OpaqueDataBuffer* dataBuffer, Nd4jLong elements);   /* ref :473 */
+ND4JHIP_EXPORT void dbExpand(OpaqueDataBuffer* dataBuffer, Nd4jLong elements);         /* ref :481 */
+ND4JHIP_EXPORT int dbUseCount(OpaqueDataBuffer* dataBuffer);                           /* ref :474 */
+ND4JHIP_EXPORT void dbSyncToSpecial(OpaqueDataBuffer* dataBuffer);                     /* ref :475 */
+ND4JHIP_EXPORT void dbSyncToPrimary(OpaqueDataBuffer* dataBuffer);                     /* ref :476 */
+ND4JHIP_EXPORT void dbTickHostRead(OpaqueDataBuffer* dataBuffer);                      /* ref :477 */
+ND4JHIP_EXPORT void dbTickHostWrite(OpaqueDataBuffer* dataBuffer);                     /* ref :478 */
+ND4JHIP_EXPORT void dbTickDeviceRead(OpaqueDataBuffer* dataBuffer);                    /* ref :479 */
+ND4JHIP_EXPORT void dbTickDeviceWrite(OpaqueDataBuffer* dataBuffer);                   /* ref :480 */
+ND4JHIP_EXPORT void dbClose(OpaqueDataBuffer* dataBuffer);                             /* ref :482 */
+ND4JHIP_EXPORT int dbDeviceId(OpaqueDataBuffer* dataBuffer);                           /* ref :483 */
+ND4JHIP_EXPORT void dbSetDeviceId(OpaqueDataBuffer* dataBuffer, int deviceId);         /* ref :484 */
+ND4JHIP_EXPORT int dbLocality(OpaqueDataBuffer* dataBuffer);                           /* ref :485: -1 host current, 1 device current, 0 both */
+ND4JHIP_EXPORT void deleteDataBuffer(OpaqueDataBuffer* dataBuffer);                    /* ref :468 */
+
+/* ---- shape descriptors (ref :490-495, :395-404) ------------------------------------------------------ */
+ND4JHIP_EXPORT OpaqueConstantShapeBuffer shapeBuffer(int rank, Nd4jLong* shape, Nd4jLong* strides, int dtype, char order, Nd4jLong ews, bool empty); /* ref :491 */
+ND4JHIP_EXPORT OpaqueConstantShapeBuffer shapeBufferEx(int rank, Nd4jLong* shape, Nd4jLong* strides, int dtype, char order, Nd4jLong ews, Nd4jLong extras); /* ref :493 */
+ND4JHIP_EXPORT OpaqueConstantShapeBuffer cacheAndStoreShapeBuffer(Nd4jLong* shapeInfo);                           /* ref :490 */
+ND4JHIP_EXPORT Nd4jPointer getConstantShapeBufferPrimary(OpaqueConstantShapeBuffer dbf);                          /* ref :403 */
+ND4JHIP_EXPORT Nd4jPointer getConstantShapeBufferSpecial(OpaqueConstantShapeBuffer dbf);                          /* ref :404 */
+ND4JHIP_EXPORT void deleteConstantShapeBuffer(OpaqueConstantShapeBuffer* ptr);                                    /* ref :395 (cache-owned: no-op) */
+
+/* ---- array handles (ref :111-125, :336-342) ------------------------------------------------------------ */
+ND4JHIP_EXPORT OpaqueNDArray createOpaqueNDArray(OpaqueDataBuffer* shapeInfo, OpaqueDataBuffer* buffer, OpaqueDataBuffer* specialBuffer, Nd4jLong offset); /* ref :122 */
+ND4JHIP_EXPORT void deleteNDArray(OpaqueNDArray array);                                /* ref :111 */
+ND4JHIP_EXPORT Nd4jLong getOpaqueNDArrayOffset(OpaqueNDArray array);                   /* ref :113 */
+ND4JHIP_EXPORT const Nd4jLong* getOpaqueNDArrayShapeInfo(OpaqueNDArray array);         /* ref :116 */
+ND4JHIP_EXPORT void* getOpaqueNDArrayBuffer(OpaqueNDArray array);                      /* ref :118 */
+ND4JHIP_EXPORT void* getOpaqueNDArraySpecialBuffer(OpaqueNDArray array);               /* ref :120 */
+ND4JHIP_EXPORT Nd4jLong getOpaqueNDArrayLength(OpaqueNDArray array);                   /* ref :342 */
+ND4JHIP_EXPORT Nd4jLong getOpaqueNDArrayShapeInfoLength(OpaqueNDArray array);          /* ref :341 getShapeInfoLength(OpaqueNDArray) */
+
+/* ---- TAD packs (ref :142-159, :397) ---------------------------------------------------------------------- */
+ND4JHIP_EXPORT OpaqueTadPack* tadOnlyShapeInfo(OpaqueDataBuffer* hXShapeInfo, Nd4jLong* dimension, Nd4jLong dimensionLength); /* ref :159 */
+ND4JHIP_EXPORT const Nd4jLong* getPrimaryShapeInfo(OpaqueTadPack* pack);               /* ref :142 */
+ND4JHIP_EXPORT const Nd4jLong* getPrimaryOffsets(OpaqueTadPack* pack);                 /* ref :143 */
+ND4JHIP_EXPORT const Nd4jLong* getSpecialShapeInfo(OpaqueTadPack* pack);               /* ref :144 */
+ND4JHIP_EXPORT const Nd4jLong* getSpecialOffsets(OpaqueTadPack* pack);                 /* ref :145 */
+ND4JHIP_EXPORT Nd4jLong getNumberOfTads(OpaqueTadPack* pack);                          /* ref :146 */
+ND4JHIP_EXPORT int getShapeInfoLength(OpaqueTadPack* pack);                            /* ref :147 */
+ND4JHIP_EXPORT void deleteTadPack(OpaqueTadPack* ptr);                                 /* ref :397 (cache-owned: no-op) */
+
+/* ---- legacy loops ------------------------------------------------------------------------------------------ */
+ND4JHIP_EXPORT void execPairwiseTransform(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, OpaqueNDArray y, OpaqueNDArray z, void* extraParams); /* ref :195 */
+ND4JHIP_EXPORT void execTransformStrict(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z); /* ref :220 */
+ND4JHIP_EXPORT void execTransformFloat(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z);  /* ref :221 */
+ND4JHIP_EXPORT void execTransformSame(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z);   /* ref :217 */
+ND4JHIP_EXPORT void execTransformAny(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z);    /* ref :219 */
+ND4JHIP_EXPORT void execReduceFloat(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z);     /* ref :207 */
+ND4JHIP_EXPORT void execReduceFloat2(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z, OpaqueNDArray dimension); /* ref :215 */
+ND4JHIP_EXPORT void execReduceSame(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z);      /* ref :321 */
+ND4JHIP_EXPORT void execReduceSame2(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z, OpaqueNDArray dimension);  /* ref :323 */
+ND4JHIP_EXPORT void execIndexReduce(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z, OpaqueNDArray dimension);  /* ref :214 */
+ND4JHIP_EXPORT void execIndexReduceScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z); /* ref :216 */
+ND4JHIP_EXPORT void execScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, OpaqueNDArray z, OpaqueNDArray scalar, void* extraParams); /* ref :204 */
+ND4JHIP_EXPORT void execBroadcast(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, OpaqueNDArray y, OpaqueNDArray z, void* extraParams, OpaqueNDArray dimension); /* ref :206 */
+
+/* ---- op context + declarable ops ---------------------------------------------------------------------------- */
+ND4JHIP_EXPORT const char* getAllCustomOps(void);                                      /* ref :76 */
+ND4JHIP_EXPORT OpaqueContext* createGraphContext(int nodeId);                          /* ref :79 */
+ND4JHIP_EXPORT void deleteGraphContext(OpaqueContext* ptr);                            /* ref :437 */
+ND4JHIP_EXPORT void markGraphContextInplace(OpaqueContext* ptr, bool reallyInplace);   /* ref :416 */
+ND4JHIP_EXPORT void setGraphContextInputArray(OpaqueContext* ptr, int index, OpaqueNDArray arr);   /* ref :430 */
+ND4JHIP_EXPORT void setGraphContextOutputArray(OpaqueContext* ptr, int index, OpaqueNDArray arr);  /* ref :429 */
+ND4JHIP_EXPORT void setGraphContextInputArraysArr(OpaqueContext* ptr, int numArrays, OpaqueNDArrayArr arr);  /* ref :432 */
+ND4JHIP_EXPORT void setGraphContextOutputArraysArr(OpaqueContext* ptr, int numArrays, OpaqueNDArrayArr arr); /* ref :431 */
+ND4JHIP_EXPORT void setGraphContextTArguments(OpaqueContext* ptr, double* arguments, int numberOfArguments);   /* ref :433 */
+ND4JHIP_EXPORT void setGraphContextIArguments(OpaqueContext* ptr, Nd4jLong* arguments, int numberOfArguments); /* ref :434 */
+ND4JHIP_EXPORT void setGraphContextBArguments(OpaqueContext* ptr, bool* arguments, int numberOfArguments);     /* ref :435 */
+ND4JHIP_EXPORT void setGraphContextDArguments(OpaqueContext* ptr, int* arguments, int numberOfArguments);      /* ref :436 */
+ND4JHIP_EXPORT void ctxAllowHelpers(OpaqueContext* ptr, bool reallyAllow);             /* ref :464 */
+ND4JHIP_EXPORT void ctxShapeFunctionOverride(OpaqueContext* ptr, bool reallyOverride); /* ref :458 */
+ND4JHIP_EXPORT void ctxSetExecutionMode(OpaqueContext* ptr, int execMode);             /* ref :465 */
+ND4JHIP_EXPORT void ctxPurge(OpaqueContext* ptr);                                      /* ref :459 */
+ND4JHIP_EXPORT OpaqueNDArray getInputArrayNative(OpaqueContext* ptr, int idx);         /* ref :418 */
+ND4JHIP_EXPORT OpaqueNDArray getOutputArrayNative(OpaqueContext* ptr, int idx);        /* ref :417 */
+ND4JHIP_EXPORT Nd4jLong numInputsNative(OpaqueContext* ptr);                           /* ref :425 */
+ND4JHIP_EXPORT Nd4jLong numOutputsNative(OpaqueContext* ptr);                          /* ref :424 */
+ND4JHIP_EXPORT Nd4jLong numTArgumentsNative(OpaqueContext* ptr);                       /* ref :427 */
+ND4JHIP_EXPORT Nd4jLong numIArgumentsNative(OpaqueContext* ptr);                       /* ref :428 */
+ND4JHIP_EXPORT Nd4jLong numBNative(OpaqueContext* ptr);                                /* ref :423 */
+ND4JHIP_EXPORT Nd4jLong numDNative(OpaqueContext* ptr);                                /* ref :422 */
+ND4JHIP_EXPORT double tArgumentNative(OpaqueContext* ptr, int idx);                    /* ref :426 */
+ND4JHIP_EXPORT Nd4jLong iArgumentAtNative(OpaqueContext* ptr, int idx);                /* ref :421 */
+ND4JHIP_EXPORT bool bArgAtNative(OpaqueContext* ptr, int idx);                         /* ref :420 */
+ND4JHIP_EXPORT Nd4jLong dataTypeNativeAt(OpaqueContext* ptr, int idx);                 /* ref :419 */
+ND4JHIP_EXPORT Nd4jStatus execCustomOp2(Nd4jPointer* extraPointers, Nd4jLong hash, OpaqueContext* opContext);  /* ref :370 */
+ND4JHIP_EXPORT OpaqueShapeList* calculateOutputShapes2(Nd4jPointer* extraPointers, Nd4jLong hash, OpaqueContext* context); /* ref :175 */
+ND4JHIP_EXPORT Nd4jLong getShapeListSize(OpaqueShapeList* list);                       /* ref :177 */
+ND4JHIP_EXPORT const Nd4jLong* getShape(OpaqueShapeList* list, Nd4jLong i);            /* ref :174 */
+ND4JHIP_EXPORT void deleteShapeList(Nd4jPointer shapeList);                            /* ref :386 */
+
+/* ---- additions without a counterpart in the reference ------------------------------------------------------- */
+/* 64-bit hash of an op name, the key execCustomOp2 takes (ref helpers/impl/helper_hash.cpp:33-70 computes it
+ * inside the library only; callers normally parse it out of getAllCustomOps()). */
+ND4JHIP_EXPORT Nd4jLong nd4jhipOpHash(const char* opName);
+/* Events that record time, for benchmarks: createEvent() above disables timing like the reference does. */
+ND4JHIP_EXPORT Nd4jPointer nd4jhipCreateTimingEvent(void);
+ND4JHIP_EXPORT float nd4jhipEventElapsedMs(Nd4jPointer startEvent, Nd4jPointer stopEvent);
+/* 1: execCustomOp2 synchronises the stream before returning (default, reference behaviour); 0: the caller
+ * synchronises itself (streamSynchronize / dbSyncToPrimary) -- used by tight decode loops. */
+ND4JHIP_EXPORT void nd4jhipSetSyncAfterCustomOp(int enable);
+ND4JHIP_EXPORT const char* nd4jhipBuildInfo(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ND4JHIP_NATIVEOPS_H */

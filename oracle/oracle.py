@@ -1,0 +1,229 @@
+"""ctypes binding of the CPU oracle (libnd4j_oracle.so) -- test infrastructure only.
+
+Arrays cross the boundary as numpy arrays plus a shapeInfo descriptor built from the numpy
+view itself (shape, element strides, dtype, order), so strided/permuted numpy views exercise
+the same shapeInfo walk the reference performs.  bf16 arrays are numpy uint16 arrays tagged
+with dtype code BFLOAT16; fp16 uses numpy float16.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libnd4j_oracle.so")
+
+BOOL, HALF, FLOAT32, DOUBLE, INT32, INT64, BFLOAT16 = 1, 3, 5, 6, 9, 10, 17
+_NP2DT = {np.dtype(np.float16): HALF, np.dtype(np.float32): FLOAT32, np.dtype(np.float64): DOUBLE,
+          np.dtype(np.int32): INT32, np.dtype(np.int64): INT64, np.dtype(np.bool_): BOOL}
+DT_FLAG = {HALF: 4096, BFLOAT16: 2048, FLOAT32: 8192, DOUBLE: 16384, INT32: 131072, INT64: 262144, BOOL: 524288}
+DT_NP = {HALF: np.float16, BFLOAT16: np.uint16, FLOAT32: np.float32, DOUBLE: np.float64, INT32: np.int32,
+         INT64: np.int64, BOOL: np.bool_}
+
+
+def build(force=False):
+    """Compile the oracle with the Makefile next to this file."""
+    if force or not os.path.exists(LIB_PATH):
+        subprocess.check_call(["make", "-C", HERE, "-B" if force else "-s", "libnd4j_oracle.so"])
+    return LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        L = ctypes.CDLL(LIB_PATH)
+        vp, i64p, i32, i64, dbl = ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64), ctypes.c_int, ctypes.c_int64, ctypes.c_double
+        L.orc_hash.restype = i64
+        L.orc_hash.argtypes = [ctypes.c_char_p]
+        L.orc_offset.restype = i64
+        L.orc_offset.argtypes = [i64p, i64]
+        L.orc_length.restype = i64
+        L.orc_length.argtypes = [i64p]
+        L.orc_tad.restype = i64
+        L.orc_tad.argtypes = [i64p, i64p, i32, i64p, i64p]
+        L.orc_f32_to_bf16.restype = ctypes.c_uint16
+        L.orc_f32_to_bf16.argtypes = [ctypes.c_float]
+        L.orc_f32_to_f16.restype = ctypes.c_uint16
+        L.orc_f32_to_f16.argtypes = [ctypes.c_float]
+        L.orc_f16_to_f32.restype = ctypes.c_float
+        L.orc_f16_to_f32.argtypes = [ctypes.c_uint16]
+        L.orc_pairwise.argtypes = [i32, vp, i64p, vp, i64p, vp, i64p]
+        L.orc_transform_strict.argtypes = [i32, vp, i64p, vp, i64p]
+        L.orc_transform_float.argtypes = [i32, vp, i64p, vp, i64p]
+        for f in (L.orc_reduce_same, L.orc_reduce_float, L.orc_index_reduce):
+            f.argtypes = [i32, vp, i64p, vp, i64p, i64p, i32]
+        L.orc_softmax.argtypes = [vp, i64p, vp, i64p, i32, i32]
+        L.orc_layer_norm.argtypes = [vp, i64p, vp, i64p, vp, i64p, vp, i64p, i64p, i32, i32]
+        L.orc_matmul.argtypes = [vp, i64p, vp, i64p, vp, i64p, i32, i32, i32, dbl, dbl, i32]
+        L.orc_attention_v2.argtypes = [vp, i64p, vp, i64p, vp, i64p, vp, i64p, vp, i64p, vp, i64p, dbl, i32]
+        L.orc_add_row_vector.argtypes = [vp, i64p, vp, i64p, vp, i64p]
+        L.orc_set_threads.argtypes = [i32]
+        L.orc_get_threads.restype = i32
+        _lib = L
+    return _lib
+
+
+def f32_to_bf16(a):
+    """RNE float32 -> bf16 bit patterns (uint16), NaN -> 0x7FC0 (types/bfloat16.h:186-213)."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    u = a.view(np.uint32).astype(np.uint64)
+    lsb = (u >> 16) & 1
+    r = ((u + 0x7FFF + lsb) >> 16).astype(np.uint16)
+    r[np.isnan(a)] = 0x7FC0
+    return r
+
+
+def bf16_to_f32(h):
+    return (np.asarray(h, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def shape_info(a, dtype=None, order=None):
+    """Reference descriptor int64[2*rank+4] for a numpy view (helpers/shape.h:76-104)."""
+    dt = dtype if dtype is not None else _NP2DT[a.dtype]
+    r = a.ndim
+    if r == 0:
+        return np.array([0, 0, 1, DT_FLAG[dt], 1, 99], dtype=np.int64)
+    strides = [s // a.itemsize for s in a.strides]
+    if order is None:
+        order = 'c' if a.flags['C_CONTIGUOUS'] or not a.flags['F_CONTIGUOUS'] else 'f'
+    dense = a.flags['C_CONTIGUOUS'] or a.flags['F_CONTIGUOUS']
+    return np.array([r, *a.shape, *strides, DT_FLAG[dt], 1 if dense else 0, ord(order)], dtype=np.int64)
+
+
+def _p(a):
+    return ctypes.c_void_p(a.ctypes.data) if a is not None else None
+
+
+def _s(si):
+    return si.ctypes.data_as(ctypes.POINTER(ctypes.c_int64)) if si is not None else None
+
+
+class Arr:
+    """numpy view + dtype code (bf16 lives in uint16 storage)."""
+
+    def __init__(self, a, dtype=None):
+        self.a = a
+        self.dt = dtype if dtype is not None else _NP2DT[a.dtype]
+        self.si = shape_info(a, self.dt)
+
+
+def _arr(a):
+    return a if isinstance(a, Arr) else Arr(a)
+
+
+def _check(rc, what):
+    if rc != 0:
+        raise ValueError("oracle %s: unsupported arguments (code %d)" % (what, rc))
+
+
+def _dims(dims):
+    d = np.asarray([] if dims is None else dims, dtype=np.int64).reshape(-1)
+    return d, len(d)
+
+
+def hash_name(name):
+    return lib().orc_hash(name.encode())
+
+
+def offset(si, i):
+    return lib().orc_offset(_s(si), i)
+
+
+def tad(a, dims):
+    a = _arr(a)
+    d, n = _dims(dims)
+    tsi = np.zeros(2 * max(a.a.ndim, 1) + 4, dtype=np.int64)
+    cnt = lib().orc_tad(_s(a.si), _s(d), n, _s(tsi), None)
+    offs = np.zeros(max(cnt, 1), dtype=np.int64)
+    lib().orc_tad(_s(a.si), _s(d), n, _s(tsi), _s(offs))
+    rank = int(tsi[0])
+    return tsi[: (6 if rank == 0 else 2 * rank + 4)], offs[:cnt]
+
+
+def pairwise(op, x, y, z):
+    x, y, z = _arr(x), _arr(y), _arr(z)
+    _check(lib().orc_pairwise(op, _p(x.a), _s(x.si), _p(y.a), _s(y.si), _p(z.a), _s(z.si)), "pairwise")
+    return z.a
+
+
+def transform_strict(op, x, z):
+    x, z = _arr(x), _arr(z)
+    _check(lib().orc_transform_strict(op, _p(x.a), _s(x.si), _p(z.a), _s(z.si)), "transform_strict")
+    return z.a
+
+
+def transform_float(op, x, z):
+    x, z = _arr(x), _arr(z)
+    _check(lib().orc_transform_float(op, _p(x.a), _s(x.si), _p(z.a), _s(z.si)), "transform_float")
+    return z.a
+
+
+def _reduce(fn, name, op, x, z, dims):
+    x, z = _arr(x), _arr(z)
+    d, n = _dims(dims)
+    _check(fn(op, _p(x.a), _s(x.si), _p(z.a), _s(z.si), _s(d), n), name)
+    return z.a
+
+
+def reduce_same(op, x, z, dims=None):
+    return _reduce(lib().orc_reduce_same, "reduce_same", op, x, z, dims)
+
+
+def reduce_float(op, x, z, dims=None):
+    return _reduce(lib().orc_reduce_float, "reduce_float", op, x, z, dims)
+
+
+def index_reduce(op, x, z, dims=None):
+    return _reduce(lib().orc_index_reduce, "index_reduce", op, x, z, dims)
+
+
+def softmax(x, z, dim=-1, literal_half=False):
+    x, z = _arr(x), _arr(z)
+    _check(lib().orc_softmax(_p(x.a), _s(x.si), _p(z.a), _s(z.si), dim, int(literal_half)), "softmax")
+    return z.a
+
+
+def layer_norm(x, gain, bias, z, axes, channels_first=True):
+    x, gain, z = _arr(x), _arr(gain), _arr(z)
+    bias = _arr(bias) if bias is not None else None
+    d, n = _dims(axes)
+    _check(lib().orc_layer_norm(_p(x.a), _s(x.si), _p(gain.a), _s(gain.si), _p(bias.a) if bias else None,
+                                _s(bias.si) if bias else None, _p(z.a), _s(z.si), _s(d), n, int(channels_first)),
+           "layer_norm")
+    return z.a
+
+
+def matmul(x, y, z, trans_x=False, trans_y=False, trans_z=False, alpha=1.0, beta=0.0, accumulate=1):
+    x, y, z = _arr(x), _arr(y), _arr(z)
+    _check(lib().orc_matmul(_p(x.a), _s(x.si), _p(y.a), _s(y.si), _p(z.a), _s(z.si), int(trans_x), int(trans_y),
+                            int(trans_z), alpha, beta, accumulate), "matmul")
+    return z.a
+
+
+def attention_v2(q, v, k, out, weights=None, logits=None, scale=1.0, causal=False):
+    q, v, k, out = _arr(q), _arr(v), _arr(k), _arr(out)
+    w = _arr(weights) if weights is not None else None
+    lg = _arr(logits) if logits is not None else None
+    _check(lib().orc_attention_v2(_p(q.a), _s(q.si), _p(v.a), _s(v.si), _p(k.a), _s(k.si), _p(out.a), _s(out.si),
+                                  _p(w.a) if w else None, _s(w.si) if w else None, _p(lg.a) if lg else None,
+                                  _s(lg.si) if lg else None, scale, int(causal)), "attention_v2")
+    return out.a
+
+
+def add_row_vector(x, row, z):
+    x, row, z = _arr(x), _arr(row), _arr(z)
+    _check(lib().orc_add_row_vector(_p(x.a), _s(x.si), _p(row.a), _s(row.si), _p(z.a), _s(z.si)), "add_row_vector")
+    return z.a
+
+
+def set_threads(n):
+    lib().orc_set_threads(n)
+
+
+def get_threads():
+    return lib().orc_get_threads()

@@ -1,0 +1,133 @@
+"""CPU tests of the C-ABI library: it loads, exports every declared entry point, and its host-side logic
+(op hash, registry listing, descriptor cache, TAD packs, error slot) behaves like the reference's.
+No compute entry point is called here."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from deeplearning4j_amd import nativeops as N
+
+
+def test_library_exports_every_declared_symbol():
+    L = N.load()
+    names = N.declared_symbols()
+    assert len(names) > 120
+    missing = [n for n in names if not hasattr(L, n)]
+    assert not missing, missing
+    untyped = [n for n in names if n not in N._SIGS and n not in ("setOmpNumThreads", "ompGetMaxThreads", "setElementThreshold", "setTADThreshold",
+                                                                 "initializeShapeCache", "initializeTadCache", "deleteConstantShapeBuffer", "deleteTadPack")]
+    assert not untyped, untyped
+
+
+def test_op_hash_reference_vectors():
+    # libnd4j/tests_cpu/layers_tests/HashUtilsTests.cpp:28-41
+    L = N.load()
+    assert L.nd4jhipOpHash(b"Conv2D") == -1637140380760460323
+    assert L.nd4jhipOpHash(b"switch") == -1988317239813741487
+
+
+def test_registry_listing_format(oracle):
+    L = N.load()
+    items = [i for i in L.getAllCustomOps().decode().split(";") if i]
+    names = {}
+    for it in items:
+        parts = it.split(":")
+        assert len(parts) == 8 and parts[7] == ""       # name:hash:nIn:nOut:inplace:nT:nI:
+        names[parts[0]] = int(parts[1])
+        assert int(parts[1]) == oracle.hash_name(parts[0])
+    for op in ("matmul", "mmul", "mMul", "gemm", "softmax", "layer_norm", "dot_product_attention_v2", "argmax", "argmin"):
+        assert op in names
+
+
+def _si(L, shape, strides, dtype=5, order=b"c"):
+    sh = (ctypes.c_longlong * max(len(shape), 1))(*shape)
+    st = (ctypes.c_longlong * max(len(strides), 1))(*strides) if strides is not None else None
+    buf = L.shapeBuffer(len(shape), sh, st, dtype, order, 1, False)
+    p = ctypes.cast(L.getConstantShapeBufferPrimary(buf), ctypes.POINTER(ctypes.c_longlong))
+    n = 6 if len(shape) == 0 else 2 * len(shape) + 4
+    return buf, [p[i] for i in range(n)]
+
+
+def test_shape_buffer_layout():
+    L = N.load()
+    # config-1 descriptor: [2, 8192, 4096, 4096, 1, 8192, 1, 99]
+    _, si = _si(L, [8192, 4096], None)
+    assert si == [2, 8192, 4096, 4096, 1, 8192, 1, 99]
+    _, si = _si(L, [3, 4], None, 17, b"f")
+    assert si == [2, 3, 4, 1, 3, 2048, 1, 102]
+    _, si = _si(L, [], None, 10)
+    assert si == [0, 0, 1, 262144, 1, 99]
+    b1, si = _si(L, [2, 3], [1, 2], 6)
+    assert si == [2, 2, 3, 1, 2, 16384, 0, 99]
+    b2, _ = _si(L, [2, 3], [1, 2], 6)
+    assert b1 == b2                                      # cached: same descriptor, same buffer
+
+
+def test_tad_pack_matches_oracle(oracle):
+    L = N.load()
+    from deeplearning4j_amd.ndarray import DataBuffer, INT64, make_shape_info
+    for shape, dims in [((5, 5), [1]), ((2, 3, 4), [0, 2]), ((2, 3, 4, 5), [1, 3]), ((3, 4), [0, 1])]:
+        a = np.zeros(shape, np.float32)
+        si = make_shape_info(shape, [s // 4 for s in a.strides], 5)
+        buf = DataBuffer(len(si), INT64, allocate_both=False)
+        buf.host_view()[: len(si)] = si
+        d = (ctypes.c_longlong * len(dims))(*dims)
+        pack = L.tadOnlyShapeInfo(buf.ptr, d, len(dims))
+        N.check("tadOnlyShapeInfo")
+        n = L.getNumberOfTads(pack)
+        tsi_want, offs_want = oracle.tad(a, dims)
+        assert n == len(offs_want)
+        offs = L.getPrimaryOffsets(pack)
+        assert [offs[i] for i in range(n)] == list(offs_want)
+        tsi = L.getPrimaryShapeInfo(pack)
+        ln = L.getShapeInfoLength(pack)
+        assert ln == len(tsi_want)
+        got = [tsi[i] for i in range(ln)]
+        rank = got[0]
+        assert got[:1 + 2 * rank] == list(tsi_want[:1 + 2 * rank])
+
+
+def test_error_slot_semantics():
+    # a failure parks {code, message}; fetching the message consumes the code (execution/impl/ErrorReference.cpp:28-34)
+    L = N.load()
+    L.lastErrorMessage()
+    assert L.lastErrorCode() == 0
+    assert L.createOpaqueNDArray(None, None, None, 0) is None
+    assert L.lastErrorCode() == 1
+    assert L.lastErrorCode() == 1
+    assert b"Shape info was null" in L.lastErrorMessage()
+    assert L.lastErrorCode() == 0
+    # unknown op hash -> non-zero status + message
+    ctx = L.createGraphContext(1)
+    assert L.execCustomOp2(None, 12345, ctx) != 0
+    assert b"unknown op hash" in L.lastErrorMessage()
+    L.deleteGraphContext(ctx)
+    # null operands on a legacy loop
+    L.execReduceFloat(None, 0, None, None, None)
+    assert L.lastErrorCode() == 1
+    assert b"null pointer" in L.lastErrorMessage()
+
+
+def test_context_argument_round_trip():
+    L = N.load()
+    ctx = L.createGraphContext(7)
+    L.setGraphContextTArguments(ctx, (ctypes.c_double * 2)(0.125, 0.0), 2)
+    L.setGraphContextIArguments(ctx, (ctypes.c_longlong * 3)(0, 1, -1), 3)
+    L.setGraphContextBArguments(ctx, (ctypes.c_bool * 2)(True, False), 2)
+    L.setGraphContextDArguments(ctx, (ctypes.c_int * 1)(10), 1)
+    assert (L.numTArgumentsNative(ctx), L.numIArgumentsNative(ctx), L.numBNative(ctx), L.numDNative(ctx)) == (2, 3, 2, 1)
+    assert L.tArgumentNative(ctx, 0) == 0.125 and L.iArgumentAtNative(ctx, 2) == -1 and L.bArgAtNative(ctx, 0) and L.dataTypeNativeAt(ctx, 0) == 10
+    assert L.numInputsNative(ctx) == 0 and L.getInputArrayNative(ctx, 0) is None
+    L.ctxPurge(ctx)
+    assert L.numIArgumentsNative(ctx) == 0
+    L.deleteGraphContext(ctx)
+
+
+def test_compute_without_gpu_fails_loudly():
+    L = N.load()
+    if L.getAvailableDevices() > 0:
+        pytest.skip("a GPU is present")
+    L.initializeDevicesAndFunctions()
+    assert L.lastErrorCode() != 0
+    assert b"no CPU fallback" in L.lastErrorMessage()

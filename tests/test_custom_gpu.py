@@ -1,0 +1,307 @@
+"""GPU parity tests of the declarable ops (matmul, softmax, layer_norm, dot_product_attention_v2, argmax and the
+decoder glue ops), driven through OpContext + execCustomOp2 exactly as the Java executioner drives them.
+
+Gates (north star): fp32 softmax / layer_norm |a-b| <= 1e-6 + 1e-5 |b|; fp32 mmul / attention <= 1e-4;
+fp16 / bf16 <= 1e-2 against the fp32-accumulated oracle on the rounded inputs; argmax bit-exact.
+"""
+import math
+
+import numpy as np
+import pytest
+
+from conftest import assert_close, materialize
+from deeplearning4j_amd.ndarray import BFLOAT16, DOUBLE, FLOAT32, HALF, INT32, INT64, NDArray, bf16_bits_to_f32, f32_to_bf16_bits
+from deeplearning4j_amd.nativeops import NativeOpsError
+
+pytestmark = pytest.mark.gpu
+
+
+def _pair(oracle, a, dtype):
+    if dtype == BFLOAT16:
+        bits = f32_to_bf16_bits(np.asarray(a, np.float32))
+        return oracle.Arr(bits, oracle.BFLOAT16), NDArray.from_numpy(bits, BFLOAT16)
+    npdt = {HALF: np.float16, FLOAT32: np.float32, DOUBLE: np.float64}[dtype]
+    h = np.asarray(a).astype(npdt)
+    return oracle.Arr(h), NDArray.from_numpy(h)
+
+
+def _ozeros(oracle, shape, dtype):
+    npdt = {HALF: np.float16, FLOAT32: np.float32, DOUBLE: np.float64, BFLOAT16: np.uint16}[dtype]
+    return oracle.Arr(np.zeros(shape, npdt), dtype)
+
+
+def _f(oa):
+    return bf16_bits_to_f32(oa.a).astype(np.float64) if oa.dt == 17 else oa.a.astype(np.float64)
+
+
+def _nd(spec, dtype=None):
+    a = materialize(spec)
+    return NDArray.from_numpy(np.ascontiguousarray(a) if spec["order"] != "f" else a, dtype, order=spec["order"] if a.ndim > 1 else "c")
+
+
+# ---- the reference's own known-answer vectors ----------------------------------------------------------------------
+def test_golden_matmul(ex, golden):
+    cases = [c for c in golden if c["op"] == "matmul"]
+    assert len(cases) >= 35
+    for c in cases:
+        x, y = _nd(c["inputs"][0]), _nd(c["inputs"][1])
+        exp = materialize(c["expected"])
+        outs = [_nd(c["initial_output"])] if "initial_output" in c else None
+        z = ex.exec_custom("matmul", [x, y], outs, t_args=c["targs"], i_args=c["iargs"])[0]
+        assert tuple(z.shape) == tuple(exp.shape), c["name"]
+        if outs is None:
+            # shape function: 'c' only when both inputs are 'c' (generic/blas/matmul.cpp:189-219)
+            assert z.order == ("c" if x.order == "c" and y.order == "c" else "f"), c["name"]
+        assert_close(z.to_numpy(), exp, 1e-6, 1e-9, c["name"])
+
+
+def test_golden_softmax(ex, golden):
+    cases = [c for c in golden if c["op"] == "softmax"]
+    assert len(cases) == 12
+    for c in cases:
+        x = _nd(c["inputs"][0])
+        z = ex.exec_custom("softmax", [x], i_args=c["iargs"])[0]
+        assert_close(z.to_numpy(), materialize(c["expected"]), 1e-4, 1e-5, c["name"])
+
+
+def test_golden_argmax(ex, golden):
+    cases = [c for c in golden if c["op"] == "argmax"]
+    for c in cases:
+        x = _nd(c["inputs"][0])
+        ins = [x]
+        if len(c["inputs"]) > 1:   # axis array: the Java side passes integer axes
+            ins.append(NDArray.from_numpy(materialize(c["inputs"][1]).astype(np.int64).ravel()))
+        z = ex.exec_custom("argmax", ins, i_args=c["iargs"])[0]
+        exp = materialize(c["expected"]).astype(np.int64)
+        assert z.dtype == INT64 and np.array_equal(z.to_numpy(), exp), c["name"]
+
+
+# ---- matmul ----------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype,tol", [(FLOAT32, 1e-4), (HALF, 1e-2), (BFLOAT16, 1e-2), (DOUBLE, 1e-10)])
+@pytest.mark.parametrize("M,N,K", [(64, 64, 64), (256, 256, 256), (130, 70, 50), (1, 768, 2304), (32, 768, 3072), (257, 129, 1024), (512, 384, 72)])
+def test_matmul_vs_oracle(ex, oracle, dtype, tol, M, N, K):
+    rng = np.random.default_rng(M + N + K)
+    a = rng.normal(0, 1 / math.sqrt(K), (M, K))
+    b = rng.normal(0, 1 / math.sqrt(K), (K, N))
+    oa, da = _pair(oracle, a, dtype)
+    ob, db = _pair(oracle, b, dtype)
+    oz = _ozeros(oracle, (M, N), dtype)
+    oracle.matmul(oa, ob, oz, accumulate=2 if dtype == DOUBLE else 1)
+    z = ex.exec_custom("matmul", [da, db])[0]
+    got = z.to_float() if dtype != DOUBLE else z.to_numpy()
+    assert_close(got, _f(oz), tol, tol, "matmul %dx%dx%d dtype %d" % (M, N, K, dtype))
+    # transposeB variant: same numbers from B stored as [N, K]
+    obt, dbt = _pair(oracle, b.T.copy(), dtype)
+    zt = ex.exec_custom("matmul", [da, dbt], i_args=[0, 1])[0]
+    gt = zt.to_float() if dtype != DOUBLE else zt.to_numpy()
+    assert_close(gt, _f(oz), tol, tol, "matmul transposeB")
+    # transposeA
+    oat, dat = _pair(oracle, a.T.copy(), dtype)
+    za = ex.exec_custom("matmul", [dat, db], i_args=[1, 0])[0]
+    ga = za.to_float() if dtype != DOUBLE else za.to_numpy()
+    assert_close(ga, _f(oz), tol, tol, "matmul transposeA")
+
+
+@pytest.mark.parametrize("dtype,tol", [(FLOAT32, 1e-4), (BFLOAT16, 1e-2)])
+def test_matmul_batched_alpha_beta_views(ex, oracle, dtype, tol):
+    rng = np.random.default_rng(21)
+    a = rng.normal(0, 0.2, (3, 2, 40, 24))
+    b = rng.normal(0, 0.2, (3, 2, 24, 56))
+    c0 = rng.normal(0, 1, (3, 2, 40, 56))
+    oa, da = _pair(oracle, a, dtype)
+    ob, db = _pair(oracle, b, dtype)
+    oc, dc = _pair(oracle, c0, dtype)
+    oracle.matmul(oa, ob, oc, alpha=0.5, beta=2.0, accumulate=1)
+    ex.exec_custom("matmul", [da, db], [dc], t_args=[0.5, 2.0])
+    assert_close(dc.to_float(), _f(oc), tol, tol, "batched alpha/beta")
+    # permuted (strided) operands: x^T through a view instead of the transpose flag
+    z = ex.exec_custom("matmul", [da.permute(0, 1, 3, 2), db], i_args=[1, 0])[0]
+    oz = _ozeros(oracle, (3, 2, 40, 56), dtype)
+    oracle.matmul(oa, ob, oz, accumulate=1)
+    assert_close(z.to_float(), _f(oz), tol, tol, "permuted view + transX")
+
+
+def test_matmul_shape_and_type_errors(ex):
+    x = NDArray.from_numpy(np.zeros((3, 4), np.float32))
+    y = NDArray.from_numpy(np.zeros((5, 3), np.float32))
+    with pytest.raises(NativeOpsError, match="inconsistent shapes"):
+        ex.exec_custom("matmul", [x, y])
+    with pytest.raises(NativeOpsError, match="share one data type"):
+        ex.exec_custom("matmul", [x, NDArray.from_numpy(np.zeros((4, 2), np.float64))], [NDArray.empty((3, 2), FLOAT32)])
+    with pytest.raises(NativeOpsError, match="output array is wrong"):
+        ex.exec_custom("matmul", [x, NDArray.from_numpy(np.zeros((4, 2), np.float32))], [NDArray.empty((3, 3), FLOAT32)])
+    with pytest.raises(NativeOpsError, match="not registered"):
+        ex.exec_custom("conv2d", [x])
+
+
+def test_mmul_full_size_properties(ex):
+    """4096^3 bf16 (BASELINE config 2): the oracle checks a sample of output elements in fp64; linearity and
+    the transposeB identity hold for the whole result."""
+    rng = np.random.default_rng(2002)
+    n = 4096
+    a = f32_to_bf16_bits(rng.normal(0, 1 / 64, (n, n)).astype(np.float32))
+    b = f32_to_bf16_bits(rng.normal(0, 1 / 64, (n, n)).astype(np.float32))
+    A, B = NDArray.from_numpy(a, BFLOAT16), NDArray.from_numpy(b, BFLOAT16)
+    z = ex.exec_custom("matmul", [A, B])[0].to_float()
+    af, bf = bf16_bits_to_f32(a).astype(np.float64), bf16_bits_to_f32(b).astype(np.float64)
+    rows = rng.choice(n, 16, replace=False)
+    cols = rng.choice(n, 16, replace=False)
+    want = af[rows] @ bf[:, cols]
+    assert_close(z[np.ix_(rows, cols)], want, 1e-2, 1e-2, "sampled elements")
+    Bt = NDArray.from_numpy(np.ascontiguousarray(b.T), BFLOAT16)
+    zt = ex.exec_custom("matmul", [A, Bt], i_args=[0, 1])[0].to_float()
+    assert_close(zt, z, 1e-2, 1e-2, "transposeB agrees with plain B")
+
+
+# ---- softmax ---------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype,rtol,atol", [(FLOAT32, 1e-5, 1e-6), (BFLOAT16, 1e-2, 1e-4), (HALF, 1e-2, 1e-4), (DOUBLE, 1e-12, 1e-14)])
+@pytest.mark.parametrize("shape,dim", [((4, 3, 8, 1024), 3), ((17, 33), 1), ((17, 33), 0), ((5, 6, 7), 1), ((3, 5000), 1), ((2, 20000), 1), ((6, 1000), -1)])
+def test_softmax_vs_oracle(ex, oracle, dtype, rtol, atol, shape, dim):
+    rng = np.random.default_rng(abs(dim) + len(shape) + shape[-1])
+    a = rng.normal(0, 2, shape)
+    ox, dx = _pair(oracle, a, dtype)
+    oz = _ozeros(oracle, shape, dtype)
+    oracle.softmax(ox, oz, dim)
+    z = ex.exec_custom("softmax", [dx], i_args=[dim])[0]
+    got = z.to_float() if dtype != DOUBLE else z.to_numpy()
+    assert_close(got, _f(oz), rtol, atol, "softmax %s dim %d dtype %d" % (shape, dim, dtype))
+    assert_close(got.astype(np.float64).sum(dim), np.ones(np.delete(np.array(shape), dim)), 2e-2 if dtype in (HALF, BFLOAT16) else 1e-5, 0, "rows sum to one")
+
+
+@pytest.mark.parametrize("dtype,rtol,atol", [(FLOAT32, 1e-5, 1e-6), (BFLOAT16, 1e-2, 1e-4)])
+def test_softmax_permuted_view(ex, oracle, dtype, rtol, atol):
+    # BASELINE config 3 layout at reduced batch: buffer [B, T, H, T] viewed through permute(0, 2, 1, 3), dense output
+    rng = np.random.default_rng(3003)
+    B, H, T = 2, 12, 256
+    a = rng.normal(0, 2, (B, T, H, T))
+    ox, dx = _pair(oracle, a, dtype)
+    oxv = oracle.Arr(ox.a.transpose(0, 2, 1, 3), ox.dt)
+    oz = _ozeros(oracle, (B, H, T, T), dtype)
+    oracle.softmax(oxv, oz, 3)
+    z = ex.exec_custom("softmax", [dx.permute(0, 2, 1, 3)], [NDArray.empty((B, H, T, T), dtype)], i_args=[3])[0]
+    assert_close(z.to_float(), _f(oz), rtol, atol, "softmax on a permuted view")
+
+
+def test_softmax_edge_semantics(ex, oracle):
+    inf, nan = np.inf, np.nan
+    rows = np.array([[0, inf, 1, -inf], [nan, 0, 0, 0], [-inf, -inf, -inf, -inf], [1e4, -1e4, 0, 5], [3, 3, 3, 3]], np.float32)
+    rows = np.repeat(rows, 2, axis=0)
+    want = oracle.softmax(rows, np.zeros_like(rows), 1)
+    got = ex.exec_custom("softmax", [NDArray.from_numpy(rows)], i_args=[1])[0].to_numpy()
+    assert_close(got, want, 1e-5, 1e-30, "inf/nan/clamp rows")
+    # vector along its unit axis is all ones; rank-1 ignores the axis argument
+    v = NDArray.from_numpy(np.array([[-1, 1, -2, 2, 3]], np.float32))
+    assert np.array_equal(ex.exec_custom("softmax", [v], i_args=[0])[0].to_numpy(), np.ones((1, 5), np.float32))
+    with pytest.raises(NativeOpsError, match="must be less than input array rank"):
+        ex.exec_custom("softmax", [v], i_args=[2])
+
+
+# ---- layer_norm ------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype,rtol,atol", [(FLOAT32, 1e-5, 1e-5), (BFLOAT16, 1e-2, 1e-2), (HALF, 1e-2, 1e-2)])
+@pytest.mark.parametrize("shape", [(4, 64, 768), (3, 5, 100), (7, 2048), (2, 3, 5000)])
+def test_layer_norm_last_axis(ex, oracle, dtype, rtol, atol, shape):
+    rng = np.random.default_rng(shape[-1])
+    C = shape[-1]
+    ox, dx = _pair(oracle, rng.normal(0, 1, shape), dtype)
+    og, dg = _pair(oracle, rng.normal(1, 0.02, C), dtype)
+    ob, db = _pair(oracle, rng.normal(0, 0.02, C), dtype)
+    oz = _ozeros(oracle, shape, dtype)
+    axes = [len(shape) - 1]
+    oracle.layer_norm(ox, og, ob, oz, axes, channels_first=False)
+    z = ex.exec_custom("layer_norm", [dx, dg, db], i_args=axes, b_args=[False])[0]
+    assert_close(z.to_float(), _f(oz), rtol, atol, "layer_norm %s" % (shape,))
+    oz2 = _ozeros(oracle, shape, dtype)
+    oracle.layer_norm(ox, og, None, oz2, axes, channels_first=False)
+    z2 = ex.exec_custom("layer_norm", [dx, dg], i_args=axes, b_args=[False])[0]
+    assert_close(z2.to_float(), _f(oz2), rtol, atol, "layer_norm without bias")
+
+
+def test_layer_norm_channels_first_and_views(ex, oracle):
+    rng = np.random.default_rng(31)
+    x = rng.normal(0, 1, (3, 5, 4, 6)).astype(np.float32)
+    g = rng.normal(1, 0.1, 5).astype(np.float32)
+    b = rng.normal(0, 0.1, 5).astype(np.float32)
+    want = oracle.layer_norm(x, g, b, np.zeros_like(x), [1, 2, 3], channels_first=True)
+    z = ex.exec_custom("layer_norm", [NDArray.from_numpy(x), NDArray.from_numpy(g), NDArray.from_numpy(b)], i_args=[1, 2, 3])[0]   # BArg absent = channels first
+    assert_close(z.to_numpy(), want, 1e-5, 1e-5, "NCHW over dims 1..3")
+    x64 = x.astype(np.float64)
+    closed = (x64 - x64.mean((1, 2, 3), keepdims=True)) / np.sqrt(x64.var((1, 2, 3), keepdims=True) + 1e-5) * g[None, :, None, None] + b[None, :, None, None]
+    assert_close(z.to_numpy(), closed, 1e-5, 1e-5, "NCHW closed form")
+    # strided rows: a sliced view along the row axis keeps unit stride inside rows
+    X = NDArray.from_numpy(rng.normal(0, 1, (16, 10, 64)).astype(np.float32))
+    g2 = rng.normal(1, 0.1, 64).astype(np.float32)
+    xv = X.slice(1, 2, 9)
+    want2 = oracle.layer_norm(X.to_numpy()[:, 2:9], g2, None, np.zeros((16, 7, 64), np.float32), [2], channels_first=False)
+    z2 = ex.exec_custom("layer_norm", [xv, NDArray.from_numpy(g2)], [NDArray.empty((16, 7, 64), FLOAT32)], i_args=[2], b_args=[False])[0]
+    assert_close(z2.to_numpy(), want2, 1e-5, 1e-5, "sliced view")
+    with pytest.raises(NativeOpsError, match="wrong shape of gain"):
+        ex.exec_custom("layer_norm", [X, NDArray.from_numpy(np.ones(7, np.float32))], i_args=[2], b_args=[False])
+
+
+# ---- attention -------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype,tol", [(FLOAT32, 1e-4), (HALF, 1e-2), (BFLOAT16, 1e-2)])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("B,Tq,Tv,D", [(3, 64, 64, 64), (2, 100, 100, 64), (2, 128, 256, 64), (1, 37, 91, 32)])
+def test_attention_vs_oracle(ex, oracle, dtype, tol, causal, B, Tq, Tv, D):
+    if causal and Tq != Tv:
+        pytest.skip("causal mask is exercised on square score matrices")
+    rng = np.random.default_rng(B * Tq + D)
+    oq, dq = _pair(oracle, rng.normal(0, 1, (B, Tq, D)), dtype)
+    ok, dk = _pair(oracle, rng.normal(0, 1, (B, Tv, D)), dtype)
+    ov, dv = _pair(oracle, rng.normal(0, 1, (B, Tv, D)), dtype)
+    oo, ow, ol = _ozeros(oracle, (B, Tq, D), dtype), _ozeros(oracle, (B, Tq, Tv), dtype), _ozeros(oracle, (B, Tq, Tv), dtype)
+    scale = 1 / math.sqrt(D)
+    oracle.attention_v2(oq, ov, ok, oo, ow, ol, scale=scale, causal=causal)
+    # all three outputs (composition path)
+    out, w, lg = ex.exec_custom("dot_product_attention_v2", [dq, dv, dk], t_args=[scale, 0.0], b_args=[causal, False])
+    assert_close(out.to_float(), _f(oo), tol, tol, "out")
+    assert_close(w.to_float(), _f(ow), tol, tol * 1e-2, "weights")
+    keep = np.tril(np.ones((Tq, Tv), bool)) if causal else np.ones((Tq, Tv), bool)
+    assert_close(lg.to_float()[:, keep], _f(ol)[:, keep], tol, tol, "logits")
+    # output only (fused path where available): same numbers
+    out1 = ex.exec_custom("dot_product_attention_v2", [dq, dv, dk], [NDArray.empty((B, Tq, D), dtype)], t_args=[scale, 0.0], b_args=[causal, False])[0]
+    assert_close(out1.to_float(), _f(oo), tol, tol, "out-only call")
+
+
+def test_attention_rank4_and_default_keys(ex, oracle):
+    rng = np.random.default_rng(41)
+    B, H, T, D = 2, 3, 48, 64
+    q = rng.normal(0, 1, (B, H, T, D)).astype(np.float32)
+    v = rng.normal(0, 1, (B, H, T, D)).astype(np.float32)
+    oo = np.zeros((B * H, T, D), np.float32)
+    oracle.attention_v2(q.reshape(B * H, T, D), v.reshape(B * H, T, D), v.reshape(B * H, T, D), oo, scale=0.125, causal=True)
+    out = ex.exec_custom("dot_product_attention_v2", [NDArray.from_numpy(q), NDArray.from_numpy(v)], [NDArray.empty((B, H, T, D), FLOAT32)],
+                         t_args=[0.125], b_args=[True])[0]
+    assert_close(out.to_numpy().reshape(B * H, T, D), oo, 1e-4, 1e-4, "rank 4, keys = values")
+
+
+# ---- argmax + glue ops -----------------------------------------------------------------------------------------------
+def test_argmax_logits_shape(ex, oracle):
+    rng = np.random.default_rng(51)
+    x = rng.normal(0, 1, (32, 50257)).astype(np.float32)
+    x[3, [100, 40000]] = 9.0    # tie: the lower index wins
+    z = ex.exec_custom("argmax", [NDArray.from_numpy(x)], i_args=[-1])[0]
+    assert z.dtype == INT64 and z.shape == (32,)
+    assert np.array_equal(z.to_numpy(), oracle.index_reduce(0, x, np.zeros(32, np.int64), [1]))
+    assert z.to_numpy()[3] == 100
+    zk = ex.exec_custom("argmax", [NDArray.from_numpy(x)], i_args=[1], b_args=[True], d_args=[INT32])[0]
+    assert zk.shape == (32, 1) and zk.dtype == INT32
+    zmin = ex.exec_custom("argmin", [NDArray.from_numpy(x)], i_args=[1])[0]
+    assert np.array_equal(zmin.to_numpy(), np.argmin(x, 1))
+
+
+def test_gather_add_concat(ex, oracle):
+    rng = np.random.default_rng(61)
+    table = rng.normal(0, 1, (1000, 96)).astype(np.float32)
+    idx = rng.integers(0, 1000, (4, 7)).astype(np.int64)
+    g = ex.exec_custom("gather", [NDArray.from_numpy(table), NDArray.from_numpy(idx)], i_args=[0])[0]
+    assert g.shape == (4, 7, 96) and np.array_equal(g.to_numpy(), table[idx])
+    bias = rng.normal(0, 1, 96).astype(np.float32)
+    s = ex.exec_custom("add", [g, NDArray.from_numpy(bias)])[0]
+    assert np.array_equal(s.to_numpy(), table[idx] + bias)
+    m = ex.exec_custom("multiply", [g, NDArray.from_numpy(rng.normal(0, 1, (4, 1, 96)).astype(np.float32))])[0]
+    assert m.shape == (4, 7, 96)
+    a = rng.normal(0, 1, (2, 5, 8)).astype(np.float32)
+    b = rng.normal(0, 1, (2, 3, 8)).astype(np.float32)
+    c = ex.exec_custom("concat", [NDArray.from_numpy(a), NDArray.from_numpy(b)], i_args=[1])[0]
+    assert np.array_equal(c.to_numpy(), np.concatenate([a, b], 1))
