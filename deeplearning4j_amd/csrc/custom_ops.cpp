@@ -175,7 +175,10 @@ static void matmulExec(Context& c) {
     bshape.resize(br); xb.resize(br); yb.resize(br); zb.resize(br);
     if (br == 1 && bshape[0] == 1) br = 0;
   }
-  prepareSpecialUse({z}, {g.x, g.y});
+  // with beta != 0 the output is read as well: its current contents must be on the device
+  std::vector<NDArray*> reads = {g.x, g.y};
+  if (d.beta != 0.f) reads.push_back(z);
+  prepareSpecialUse(std::vector<NDArray*>{z}, reads);
   const size_t es = sizeOf(dt);
   const char* A = (const char*)g.x->specialBuffer();
   const char* B = (const char*)g.y->specialBuffer();
@@ -193,7 +196,7 @@ static void matmulExec(Context& c) {
       launchGemm(stream(), dt, A + ao * es, B + bo * es, C + co * es, d);
     }
   }
-  registerSpecialUse({z}, {g.x, g.y});
+  registerSpecialUse(std::vector<NDArray*>{z}, reads);
 }
 
 // ---- softmax -----------------------------------------------------------------------------------------------------

@@ -1,10 +1,19 @@
 // GEMM kernels: C = alpha * op(A) op(B) + beta * C, batched through blockIdx.z.
 //
-//   gemm_simple - any float dtype, any strides: 32x32 output tile per block staged through LDS, fp32
-//                 (fp64 for DOUBLE) accumulation.  Correctness path for small, odd-shaped or oddly strided
-//                 problems.
-// The MFMA kernels for fp16/bf16/fp32 live further down and take over whenever their alignment
-// requirements hold.
+//   gemm_mfma16  fp16 / bf16 inputs, fp32 accumulation on the matrix cores (v_mfma_f32_32x32x16_{f16,bf16}).
+//                Block tile BM x BN x 64, double-buffered through LDS.  Both operand tiles sit in LDS as
+//                [k/8][row][8 k-values] (16 bytes per (k-group,row), one padding slot per k-group), which is
+//                exactly what one MFMA lane consumes, so fragment reads are conflict-free ds_read_b128.
+//                An operand whose K axis is contiguous in memory is copied 16 bytes at a time; an operand
+//                whose M/N axis is contiguous (plain row-major B, column-major A) is loaded as 8x8 blocks and
+//                transposed in registers with byte permutes on the way into LDS -- no transposed copy of
+//                the matrix is ever materialised.  Workgroup ids are re-mapped so that the 32 CUs of one XCD
+//                work on neighbouring tiles and share operand panels in that XCD's L2.
+//                Bound: MFMA (2*M*N*K flop against the dtype's dense peak).
+//   gemm_mfma32  fp32 on v_mfma_f32_32x32x2f32, tile BM x BN x 16, LDS layout [k][row].
+//   gemv_*       M == 1 or N == 1: HBM-bound streaming of the matrix operand.
+//   gemm_simple  any float dtype, any strides (also fp64): 32x32 tile per block through LDS.  Correctness
+//                path for small, odd-shaped or oddly strided problems.
 #include "device.h"
 #include "kernels.h"
 #include "runtime.h"
@@ -18,6 +27,12 @@ struct GemmArgs {
   float alpha, beta;
 };
 
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+// ---- fallback --------------------------------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void gemm_simple(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C) {
   using Acc = typename Conv<T>::acc;
@@ -30,7 +45,6 @@ __global__ __launch_bounds__(256) void gemm_simple(GemmArgs g, const T* __restri
   const LongType m0 = (LongType)blockIdx.y * TS, n0 = (LongType)blockIdx.x * TS;
   Acc acc[2][2] = {{0, 0}, {0, 0}};
   for (LongType k0 = 0; k0 < g.K; k0 += KS) {
-    // 512 elements per operand tile, 256 threads: two each
     for (int e = threadIdx.x; e < KS * TS; e += 256) {
       const int kk = e / TS, mm = e % TS;
       const LongType k = k0 + kk;
@@ -59,6 +73,465 @@ __global__ __launch_bounds__(256) void gemm_simple(GemmArgs g, const T* __restri
     }
 }
 
+// ---- tile scheduling ---------------------------------------------------------------------------------------------
+// Hardware hands consecutive workgroup ids to the 8 XCDs round-robin.  Give every XCD a contiguous range of
+// tiles instead, and walk that range in groups of GROUP_M tile-rows so that concurrently running workgroups
+// of one XCD share A and B panels in its L2.
+__device__ __forceinline__ void tileOf(unsigned bid, unsigned nb, unsigned tilesM, unsigned tilesN, unsigned& tm, unsigned& tn) {
+  constexpr unsigned XCDS = 8, GROUP_M = 4;
+  unsigned tile = bid;
+  if (nb >= XCDS * 4) {
+    const unsigned xcd = bid % XCDS, q = bid / XCDS;
+    const unsigned per = nb / XCDS, rem = nb % XCDS;
+    tile = xcd * per + (xcd < rem ? xcd : rem) + q;
+  }
+  const unsigned perGroup = GROUP_M * tilesN;
+  const unsigned group = tile / perGroup, inGroup = tile % perGroup;
+  const unsigned firstM = group * GROUP_M;
+  const unsigned gsz = tilesM - firstM < GROUP_M ? tilesM - firstM : GROUP_M;
+  tm = firstM + inGroup % gsz;
+  tn = inGroup / gsz;
+}
+
+// ---- 16-bit MFMA kernel ----------------------------------------------------------------------------------------------
+template <typename T> struct Mfma16;
+template <> struct Mfma16<f16_t> {
+  static __device__ __forceinline__ f32x16 mma(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mfma16<bf16_t> {
+  static __device__ __forceinline__ f32x16 mma(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+
+// transpose an 8x8 block of 16-bit values held as 8 row vectors; out[c] collects element c of every row
+__device__ __forceinline__ void transpose8x8(const u32x4 (&r)[8], u32x4 (&out)[8]) {
+#pragma unroll
+  for (int c = 0; c < 8; c++) {
+    const unsigned sel = (c & 1) ? 0x07060302u : 0x05040100u;
+#pragma unroll
+    for (int d = 0; d < 4; d++) out[c][d] = __builtin_amdgcn_perm(r[2 * d + 1][c / 2], r[2 * d][c / 2], sel);
+  }
+}
+
+// Loader for one operand tile of `ROWS` rows (M or N index) x 64 k.
+//   KC = true : memory is [row][k] with unit k stride; ld = row pitch
+//   KC = false: memory is [k][row] with unit row stride; ld = k pitch
+template <int ROWS, int NT, bool KC>
+struct TileLoader {
+  static constexpr int VECS = KC ? (ROWS * 8 + NT - 1) / NT : 0;        // 16-byte vectors per thread
+  static constexpr int BLKS = KC ? 0 : (ROWS + NT - 1) / NT;            // 8x8 blocks per thread
+  static constexpr int NREG = KC ? VECS : BLKS * 8;
+  u32x4 reg[NREG > 0 ? NREG : 1];
+
+  template <typename T>
+  __device__ __forceinline__ void load(const T* __restrict__ base, LongType ld, LongType row0, LongType rowLimit, LongType k0, LongType K, int t) {
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    if (KC) {
+#pragma unroll
+      for (int i = 0; i < VECS; i++) {
+        const int v = t + i * NT;
+        if (VECS * NT != ROWS * 8 && v >= ROWS * 8) break;
+        const int kg = v & 7, row = v >> 3;
+        LongType r = row0 + row;
+        r = r < rowLimit ? r : rowLimit - 1;
+        const LongType k = k0 + kg * 8;
+        reg[i] = k < K ? *reinterpret_cast<const u32x4*>(base + r * ld + k) : zero;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < BLKS; i++) {
+        const int b = t + i * NT;
+        if (BLKS * NT != ROWS && b >= ROWS) break;
+        const int rb = b % (ROWS / 8), kg = b / (ROWS / 8);
+        LongType r = row0 + rb * 8;
+        r = r + 8 <= rowLimit ? r : rowLimit - 8;
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+          const LongType k = k0 + kg * 8 + q;
+          reg[i * 8 + q] = k < K ? *reinterpret_cast<const u32x4*>(base + k * ld + r) : zero;
+        }
+      }
+    }
+  }
+  // lds: [8 k-groups][ROWS + 1] slots of 16 bytes
+  __device__ __forceinline__ void store(u32x4* __restrict__ lds, LongType row0, LongType rowLimit, int t) {
+    if (KC) {
+#pragma unroll
+      for (int i = 0; i < VECS; i++) {
+        const int v = t + i * NT;
+        if (VECS * NT != ROWS * 8 && v >= ROWS * 8) break;
+        const int kg = v & 7, row = v >> 3;
+        lds[kg * (ROWS + 1) + row] = reg[i];
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < BLKS; i++) {
+        const int b = t + i * NT;
+        if (BLKS * NT != ROWS && b >= ROWS) break;
+        const int rb = b % (ROWS / 8), kg = b / (ROWS / 8);
+        u32x4 rows[8], cols[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) rows[q] = reg[i * 8 + q];
+        transpose8x8(rows, cols);
+        // a block clamped at the edge (row0 + rb*8 + 8 > rowLimit) was loaded from rowLimit-8: it is stored at
+        // its nominal slot; its values belong to rows that the epilogue never writes
+#pragma unroll
+        for (int c = 0; c < 8; c++) lds[kg * (ROWS + 1) + rb * 8 + c] = cols[c];
+      }
+    }
+  }
+};
+
+template <typename T, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
+                                                             unsigned tilesM, unsigned tilesN) {
+  constexpr int BK = 64, NT = WM * WN * 64;
+  constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
+  constexpr int SLOTS_A = 8 * (BM + 1), SLOTS_B = 8 * (BN + 1), STAGE = SLOTS_A + SLOTS_B;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  u32x4* smem = reinterpret_cast<u32x4*>(smem_raw);
+
+  unsigned tm, tn;
+  tileOf(blockIdx.x, gridDim.x, tilesM, tilesN, tm, tn);
+  const LongType m0 = (LongType)tm * BM, n0 = (LongType)tn * BN;
+  const LongType bz = blockIdx.z;
+  A += bz * g.aBatch; B += bz * g.bBatch; C += bz * g.cBatch;
+  const LongType lda = A_KC ? g.aRow : g.aCol, ldb = B_KC ? g.bCol : g.bRow;
+
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+  TileLoader<BM, NT, A_KC> la;
+  TileLoader<BN, NT, B_KC> lb;
+  const LongType KT = (g.K + BK - 1) / BK;
+
+  la.load(A, lda, m0, g.M, 0, g.K, t);
+  lb.load(B, ldb, n0, g.N, 0, g.K, t);
+  la.store(smem, m0, g.M, t);
+  lb.store(smem + SLOTS_A, n0, g.N, t);
+  __syncthreads();
+
+  for (LongType kt = 0; kt < KT; kt++) {
+    const int cur = (int)(kt & 1);
+    if (kt + 1 < KT) {
+      la.load(A, lda, m0, g.M, (kt + 1) * BK, g.K, t);
+      lb.load(B, ldb, n0, g.N, (kt + 1) * BK, g.K, t);
+    }
+    const u32x4* sA = smem + cur * STAGE;
+    const u32x4* sB = sA + SLOTS_A;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ks++) {
+      const int kg = ks * 2 + (lane >> 5);
+      u32x4 fa[TM], fb[TN];
+#pragma unroll
+      for (int i = 0; i < TM; i++) fa[i] = sA[kg * (BM + 1) + wm * WTM + i * 32 + (lane & 31)];
+#pragma unroll
+      for (int j = 0; j < TN; j++) fb[j] = sB[kg * (BN + 1) + wn * WTN + j * 32 + (lane & 31)];
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = Mfma16<T>::mma(fa[i], fb[j], acc[i][j]);
+    }
+    if (kt + 1 < KT) {
+      u32x4* dst = smem + (cur ^ 1) * STAGE;
+      la.store(dst, m0, g.M, t);
+      lb.store(dst + SLOTS_A, n0, g.N, t);
+    }
+    __syncthreads();
+  }
+
+  // epilogue: lane owns column (lane % 32); register r of a 32x32 tile is row 8*(r/4) + 4*(lane/32) + r%4
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const LongType col = n0 + wn * WTN + j * 32 + (lane & 31);
+      if (col >= g.N) continue;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const LongType row = m0 + wm * WTM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r & 3);
+        if (row < g.M) {
+          const LongType off = row * g.cRow + col * g.cCol;
+          float v = g.alpha * acc[i][j][r];
+          if (g.beta != 0.f) v += g.beta * to_float(C[off]);
+          C[off] = Conv<T>::from(v);
+        }
+      }
+    }
+}
+
+template <typename T, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC>
+static void launchMfma16Cfg(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C, LongType batch) {
+  constexpr int NT = WM * WN * 64;
+  constexpr size_t LDS = (size_t)2 * (8 * (BM + 1) + 8 * (BN + 1)) * 16;
+  auto kern = gemm_mfma16<T, BM, BN, WM, WN, A_KC, B_KC>;
+  static bool attrSet = false;
+  if (!attrSet) {
+    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS));
+    attrSet = true;
+  }
+  const unsigned tilesM = (unsigned)((g.M + BM - 1) / BM), tilesN = (unsigned)((g.N + BN - 1) / BN);
+  hipLaunchKernelGGL(kern, dim3(tilesM * tilesN, 1, (unsigned)batch), dim3(NT), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tilesM, tilesN);
+}
+
+template <typename T, bool A_KC, bool B_KC>
+static void launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C, LongType batch) {
+  const LongType tiles256 = ((g.M + 255) / 256) * ((g.N + 255) / 256) * batch;
+  const LongType tiles128 = ((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
+  if (g.M <= 32) return launchMfma16Cfg<T, 32, 128, 1, 4, A_KC, B_KC>(s, g, A, B, C, batch);
+  if (g.M <= 64 || g.N <= 64 || tiles128 < 192) return launchMfma16Cfg<T, 64, 64, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
+  if (tiles256 < 192) return launchMfma16Cfg<T, 128, 128, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
+  return launchMfma16Cfg<T, 256, 256, 2, 4, A_KC, B_KC>(s, g, A, B, C, batch);
+}
+
+// ---- fp32 MFMA kernel ------------------------------------------------------------------------------------------------
+// tile BM x BN x 16; LDS holds [k][row + pad] floats; one MFMA 32x32x2 consumes k = 2*s + lane/32, row = lane%32
+template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32(GemmArgs g, const float* __restrict__ A, const float* __restrict__ B,
+                                                             float* __restrict__ C, unsigned tilesM, unsigned tilesN) {
+  constexpr int BK = 16, NT = WM * WN * 64, PA = BM + 4, PB = BN + 4;
+  constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
+  constexpr int VA = BM * BK / 4 / NT, VB = BN * BK / 4 / NT;   // float4 per thread
+  __shared__ __attribute__((aligned(16))) float sA[2][BK * PA];
+  __shared__ __attribute__((aligned(16))) float sB[2][BK * PB];
+  unsigned tm, tn;
+  tileOf(blockIdx.x, gridDim.x, tilesM, tilesN, tm, tn);
+  const LongType m0 = (LongType)tm * BM, n0 = (LongType)tn * BN;
+  const LongType bz = blockIdx.z;
+  A += bz * g.aBatch; B += bz * g.bBatch; C += bz * g.cBatch;
+  const LongType lda = A_KC ? g.aRow : g.aCol, ldb = B_KC ? g.bCol : g.bRow;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wm = wave / WN, wn = wave % WN;
+  typedef __attribute__((ext_vector_type(4))) float f32x4;
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+  f32x4 ra[VA], rb[VB];
+  const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+
+  auto loadA = [&](LongType k0) {
+#pragma unroll
+    for (int i = 0; i < VA; i++) {
+      const int v = t + i * NT;
+      if (A_KC) {
+        const int kq = v & 3, row = v >> 2;
+        LongType r = m0 + row; r = r < g.M ? r : g.M - 1;
+        const LongType k = k0 + kq * 4;
+        ra[i] = k < g.K ? *reinterpret_cast<const f32x4*>(A + r * lda + k) : zero;
+      } else {
+        const int rq = v % (BM / 4), kk = v / (BM / 4);
+        LongType r = m0 + rq * 4; r = r + 4 <= g.M ? r : g.M - 4;
+        const LongType k = k0 + kk;
+        ra[i] = k < g.K ? *reinterpret_cast<const f32x4*>(A + k * lda + r) : zero;
+      }
+    }
+  };
+  auto loadB = [&](LongType k0) {
+#pragma unroll
+    for (int i = 0; i < VB; i++) {
+      const int v = t + i * NT;
+      if (B_KC) {
+        const int kq = v & 3, row = v >> 2;
+        LongType r = n0 + row; r = r < g.N ? r : g.N - 1;
+        const LongType k = k0 + kq * 4;
+        rb[i] = k < g.K ? *reinterpret_cast<const f32x4*>(B + r * ldb + k) : zero;
+      } else {
+        const int rq = v % (BN / 4), kk = v / (BN / 4);
+        LongType r = n0 + rq * 4; r = r + 4 <= g.N ? r : g.N - 4;
+        const LongType k = k0 + kk;
+        rb[i] = k < g.K ? *reinterpret_cast<const f32x4*>(B + k * ldb + r) : zero;
+      }
+    }
+  };
+  auto storeA = [&](int stage) {
+#pragma unroll
+    for (int i = 0; i < VA; i++) {
+      const int v = t + i * NT;
+      if (A_KC) {
+        const int kq = v & 3, row = v >> 2;
+#pragma unroll
+        for (int q = 0; q < 4; q++) sA[stage][(kq * 4 + q) * PA + row] = ra[i][q];
+      } else {
+        const int rq = v % (BM / 4), kk = v / (BM / 4);
+        *reinterpret_cast<f32x4*>(&sA[stage][kk * PA + rq * 4]) = ra[i];
+      }
+    }
+  };
+  auto storeB = [&](int stage) {
+#pragma unroll
+    for (int i = 0; i < VB; i++) {
+      const int v = t + i * NT;
+      if (B_KC) {
+        const int kq = v & 3, row = v >> 2;
+#pragma unroll
+        for (int q = 0; q < 4; q++) sB[stage][(kq * 4 + q) * PB + row] = rb[i][q];
+      } else {
+        const int rq = v % (BN / 4), kk = v / (BN / 4);
+        *reinterpret_cast<f32x4*>(&sB[stage][kk * PB + rq * 4]) = rb[i];
+      }
+    }
+  };
+
+  const LongType KT = (g.K + BK - 1) / BK;
+  loadA(0); loadB(0); storeA(0); storeB(0);
+  __syncthreads();
+  for (LongType kt = 0; kt < KT; kt++) {
+    const int cur = (int)(kt & 1);
+    if (kt + 1 < KT) { loadA((kt + 1) * BK); loadB((kt + 1) * BK); }
+#pragma unroll
+    for (int ks = 0; ks < BK / 2; ks++) {
+      const int k = ks * 2 + (lane >> 5);
+      float fa[TM], fb[TN];
+#pragma unroll
+      for (int i = 0; i < TM; i++) fa[i] = sA[cur][k * PA + wm * WTM + i * 32 + (lane & 31)];
+#pragma unroll
+      for (int j = 0; j < TN; j++) fb[j] = sB[cur][k * PB + wn * WTN + j * 32 + (lane & 31)];
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < KT) { storeA(cur ^ 1); storeB(cur ^ 1); }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const LongType col = n0 + wn * WTN + j * 32 + (lane & 31);
+      if (col >= g.N) continue;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const LongType row = m0 + wm * WTM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r & 3);
+        if (row < g.M) {
+          const LongType off = row * g.cRow + col * g.cCol;
+          float v = g.alpha * acc[i][j][r];
+          if (g.beta != 0.f) v += g.beta * C[off];
+          C[off] = v;
+        }
+      }
+    }
+}
+
+template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC>
+static void launchMfma32Cfg(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C, LongType batch) {
+  const unsigned tilesM = (unsigned)((g.M + BM - 1) / BM), tilesN = (unsigned)((g.N + BN - 1) / BN);
+  hipLaunchKernelGGL((gemm_mfma32<BM, BN, WM, WN, A_KC, B_KC>), dim3(tilesM * tilesN, 1, (unsigned)batch), dim3(WM * WN * 64), 0, s, g,
+                     (const float*)A, (const float*)B, (float*)C, tilesM, tilesN);
+}
+template <bool A_KC, bool B_KC>
+static void launchMfma32(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C, LongType batch) {
+  const LongType tiles128 = ((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
+  if (g.M <= 64 || g.N <= 64 || tiles128 < 192) return launchMfma32Cfg<64, 64, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
+  return launchMfma32Cfg<128, 128, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
+}
+
+// ---- GEMV: one skinny operand, the matrix is streamed once ----------------------------------------------------------
+// y[n] = alpha * sum_k x[k] * W[n][k] (+ beta y): W rows contiguous in k.  One wave per output row.
+template <typename T>
+__global__ __launch_bounds__(256) void gemv_rowdot(const T* __restrict__ W, LongType ldw, const T* __restrict__ x, LongType xs, T* __restrict__ y,
+                                                   LongType ys, LongType N, LongType K, float alpha, float beta) {
+  using A = typename Conv<T>::acc;
+  constexpr int V = 16 / sizeof(T);
+  using VT = Vec<T, V>;
+  const int lane = threadIdx.x & 63;
+  const LongType n = (LongType)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (n >= N) return;
+  const T* w = W + n * ldw;
+  A acc = 0;
+  const bool vec = xs == 1 && K % V == 0 && ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(x)) & 15) == 0;
+  if (vec) {
+    const VT* wv = reinterpret_cast<const VT*>(w);
+    const VT* xv = reinterpret_cast<const VT*>(x);
+    for (LongType i = lane; i < K / V; i += 64) {
+      VT a = wv[i], b = xv[i];
+#pragma unroll
+      for (int e = 0; e < V; e++) acc += (A)to_float(a.v[e]) * (A)to_float(b.v[e]);
+    }
+  } else {
+    for (LongType k = lane; k < K; k += 64) acc += (A)to_float(w[k]) * (A)to_float(x[k * xs]);
+  }
+  acc = wave_allreduce<SumOp>(acc);
+  if (lane == 0) {
+    A v = (A)alpha * acc;
+    if (beta != 0.f) v += (A)beta * (A)to_float(y[n * ys]);
+    y[n * ys] = Conv<T>::from(v);
+  }
+}
+// y[n] = alpha * sum_k x[k] * W[k][n]: W rows contiguous in n.  A thread owns V consecutive outputs of one k-slice;
+// slices are combined through LDS (block = 64 column groups x 4 k-slices).
+template <typename T>
+__global__ __launch_bounds__(256) void gemv_colsum(const T* __restrict__ W, LongType ldw, const T* __restrict__ x, LongType xs, T* __restrict__ y,
+                                                   LongType ys, LongType N, LongType K, float alpha, float beta) {
+  using A = typename Conv<T>::acc;
+  constexpr int V = 16 / sizeof(T);
+  using VT = Vec<T, V>;
+  __shared__ A part[4][64 * V];
+  const int cg = threadIdx.x & 63, slice = threadIdx.x >> 6;
+  const LongType n0 = ((LongType)blockIdx.x * 64 + cg) * V;
+  A acc[V];
+#pragma unroll
+  for (int e = 0; e < V; e++) acc[e] = 0;
+  if (n0 < N) {
+    const bool vec = N % V == 0 && ldw % V == 0 && (reinterpret_cast<uintptr_t>(W) & 15) == 0;
+    for (LongType k = slice; k < K; k += 4) {
+      const A xv = (A)to_float(x[k * xs]);
+      if (vec) {
+        VT w = *reinterpret_cast<const VT*>(W + k * ldw + n0);
+#pragma unroll
+        for (int e = 0; e < V; e++) acc[e] += xv * (A)to_float(w.v[e]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < V; e++) if (n0 + e < N) acc[e] += xv * (A)to_float(W[k * ldw + n0 + e]);
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < V; e++) part[slice][cg * V + e] = acc[e];
+  __syncthreads();
+  if (slice == 0 && n0 < N) {
+#pragma unroll
+    for (int e = 0; e < V; e++) {
+      if (n0 + e >= N) break;
+      A v = (A)alpha * (part[0][cg * V + e] + part[1][cg * V + e] + part[2][cg * V + e] + part[3][cg * V + e]);
+      if (beta != 0.f) v += (A)beta * (A)to_float(y[(n0 + e) * ys]);
+      y[(n0 + e) * ys] = Conv<T>::from(v);
+    }
+  }
+}
+
+template <typename T>
+static bool tryGemv(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
+  if (d.batch != 1) return false;
+  constexpr int V = 16 / sizeof(T);
+  if (d.M == 1 && d.N > 1) {
+    // y[n] = sum_k a[k] * op(B)[k][n]
+    if (d.bRow == 1) { hipLaunchKernelGGL((gemv_rowdot<T>), dim3((unsigned)((d.N + 3) / 4)), dim3(256), 0, s, (const T*)B, d.bCol, (const T*)A, d.aCol, (T*)C, d.cCol, d.N, d.K, d.alpha, d.beta); return true; }
+    if (d.bCol == 1) { hipLaunchKernelGGL((gemv_colsum<T>), dim3((unsigned)((d.N + 64 * V - 1) / (64 * V))), dim3(256), 0, s, (const T*)B, d.bRow, (const T*)A, d.aCol, (T*)C, d.cCol, d.N, d.K, d.alpha, d.beta); return true; }
+  }
+  if (d.N == 1 && d.M > 1) {
+    // y[m] = sum_k op(A)[m][k] * b[k]
+    if (d.aCol == 1) { hipLaunchKernelGGL((gemv_rowdot<T>), dim3((unsigned)((d.M + 3) / 4)), dim3(256), 0, s, (const T*)A, d.aRow, (const T*)B, d.bRow, (T*)C, d.cRow, d.M, d.K, d.alpha, d.beta); return true; }
+    if (d.aRow == 1) { hipLaunchKernelGGL((gemv_colsum<T>), dim3((unsigned)((d.M + 64 * V - 1) / (64 * V))), dim3(256), 0, s, (const T*)A, d.aCol, (const T*)B, d.bRow, (T*)C, d.cRow, d.M, d.K, d.alpha, d.beta); return true; }
+  }
+  return false;
+}
+
+// ---- dispatch ---------------------------------------------------------------------------------------------------------
 static GemmArgs toArgs(const GemmDesc& d) {
   GemmArgs g;
   g.M = d.M; g.N = d.N; g.K = d.K;
@@ -75,14 +548,56 @@ static void launchSimple(hipStream_t s, const void* A, const void* B, void* C, c
   hipLaunchKernelGGL((gemm_simple<T>), grid, dim3(256), 0, s, g, (const T*)A, (const T*)B, (T*)C);
 }
 
+// can the MFMA kernels take this problem: 16-byte aligned vectors along each operand's contiguous axis
+static bool mfmaEligible(const GemmDesc& d, const void* A, const void* B, size_t es, bool& aKC, bool& bKC) {
+  const LongType V = 16 / (LongType)es;
+  if (d.M < 1 || d.N < 1 || d.K < 1) return false;
+  if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) return false;
+  if (d.batch > 1 && (d.aBatch % V || d.bBatch % V)) return false;
+  if (d.aCol == 1 && d.K % V == 0 && d.aRow % V == 0) aKC = true;
+  else if (d.aRow == 1 && d.M % V == 0 && d.M >= V && d.aCol % V == 0) aKC = false;
+  else return false;
+  if (d.bRow == 1 && d.K % V == 0 && d.bCol % V == 0) bKC = true;
+  else if (d.bCol == 1 && d.N % V == 0 && d.N >= V && d.bRow % V == 0) bKC = false;
+  else return false;
+  if (d.aRow < 0 || d.aCol < 0 || d.bRow < 0 || d.bCol < 0) return false;
+  return true;
+}
+
+template <typename T>
+static void dispatch16(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
+  if (tryGemv<T>(s, d, A, B, C)) return;
+  bool aKC = false, bKC = false;
+  if (d.M * d.N >= 1024 && d.K >= 32 && mfmaEligible(d, A, B, sizeof(T), aKC, bKC)) {
+    GemmArgs g = toArgs(d);
+    if (aKC && bKC) return launchMfma16<T, true, true>(s, g, A, B, C, d.batch);
+    if (aKC && !bKC) return launchMfma16<T, true, false>(s, g, A, B, C, d.batch);
+    if (!aKC && bKC) return launchMfma16<T, false, true>(s, g, A, B, C, d.batch);
+    return launchMfma16<T, false, false>(s, g, A, B, C, d.batch);
+  }
+  launchSimple<T>(s, A, B, C, d);
+}
+static void dispatch32(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
+  if (tryGemv<float>(s, d, A, B, C)) return;
+  bool aKC = false, bKC = false;
+  if (d.M * d.N >= 1024 && d.K >= 16 && mfmaEligible(d, A, B, 4, aKC, bKC)) {
+    GemmArgs g = toArgs(d);
+    if (aKC && bKC) return launchMfma32<true, true>(s, g, A, B, C, d.batch);
+    if (aKC && !bKC) return launchMfma32<true, false>(s, g, A, B, C, d.batch);
+    if (!aKC && bKC) return launchMfma32<false, true>(s, g, A, B, C, d.batch);
+    return launchMfma32<false, false>(s, g, A, B, C, d.batch);
+  }
+  launchSimple<float>(s, A, B, C, d);
+}
+
 void launchGemm(hipStream_t s, DataType dt, const void* A, const void* B, void* C, const GemmDesc& d) {
   if (d.M == 0 || d.N == 0 || d.batch == 0) return;
-  ND4J_REQUIRE(d.batch < 65536 && (d.M + 31) / 32 < 65536, "matmul: problem too large for the fallback grid");
+  ND4J_REQUIRE(d.batch < 65536 && (d.M + 31) / 32 < 65536 && (d.N + 31) / 32 < (1LL << 31), "matmul: problem too large for the launch grid");
   switch (dt) {
-    case FLOAT32: launchSimple<float>(s, A, B, C, d); break;
+    case FLOAT32: dispatch32(s, d, A, B, C); break;
     case DOUBLE: launchSimple<double>(s, A, B, C, d); break;
-    case HALF: launchSimple<f16_t>(s, A, B, C, d); break;
-    case BFLOAT16: launchSimple<bf16_t>(s, A, B, C, d); break;
+    case HALF: dispatch16<f16_t>(s, d, A, B, C); break;
+    case BFLOAT16: dispatch16<bf16_t>(s, d, A, B, C); break;
     default: ND4J_THROW("matmul: unsupported dtype");
   }
   HIP_CHECK(hipGetLastError());

@@ -43,6 +43,8 @@ def materialize(spec):
     else:
         a = np.array(spec["logical"], dtype=np.float64).reshape(shape)
     a = a.astype(dt)
+    if a.ndim == 0:
+        return a
     return np.asfortranarray(a) if spec["order"] == "f" and a.ndim > 1 else np.ascontiguousarray(a)
 
 
