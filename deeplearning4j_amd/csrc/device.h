@@ -26,12 +26,14 @@ template <> struct Conv<float> { using acc = float; static __device__ __forceinl
 template <> struct Conv<double> { using acc = double; static __device__ __forceinline__ double from(double v) { return v; } };
 template <> struct Conv<bf16_t> {
   using acc = float;
+  // gfx950 converts in hardware (v_cvt_pk_bf16_f32, round-to-nearest-even); a NaN stays a quiet NaN but
+  // its payload is the hardware's, not necessarily the reference's 0x7FC0
   static __device__ __forceinline__ bf16_t from(float f) {
-    unsigned u = __float_as_uint(f);
+    // the empty asm pins the value in a register: it keeps the compiler from folding a preceding negation
+    // into the conversion's source modifier, a pattern this compiler version fails to select
+    asm("" : "+v"(f));
     bf16_t r;
-    if ((u & 0x7fffffffu) > 0x7f800000u) { r.bits = 0x7FC0; return r; }
-    u += 0x7fffu + ((u >> 16) & 1u);
-    r.bits = (unsigned short)(u >> 16);
+    r.bits = __builtin_bit_cast(unsigned short, (__bf16)f);
     return r;
   }
 };
@@ -42,6 +44,85 @@ template <> struct Conv<f16_t> {
 
 // 16-byte (or narrower) vector of storage elements
 template <typename T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };
+
+// 16-byte register images per storage type, with conversion to and from the accumulation type.  Memory
+// instructions (also the non-temporal ones) work on these vector types directly.
+typedef __attribute__((ext_vector_type(4))) float raw_f32x4;
+typedef __attribute__((ext_vector_type(2))) double raw_f64x2;
+typedef __attribute__((ext_vector_type(4))) unsigned raw_u32x4;
+template <typename T> struct RawIO;
+template <> struct RawIO<float> {
+  using raw = raw_f32x4;
+  static constexpr int N = 4;
+  static __device__ __forceinline__ void unpack(raw r, float* out) {
+#pragma unroll
+    for (int e = 0; e < 4; e++) out[e] = r[e];
+  }
+  static __device__ __forceinline__ raw pack(const float* in) { raw r = {in[0], in[1], in[2], in[3]}; return r; }
+};
+template <> struct RawIO<double> {
+  using raw = raw_f64x2;
+  static constexpr int N = 2;
+  static __device__ __forceinline__ void unpack(raw r, double* out) { out[0] = r[0]; out[1] = r[1]; }
+  static __device__ __forceinline__ raw pack(const double* in) { raw r = {in[0], in[1]}; return r; }
+};
+template <> struct RawIO<bf16_t> {
+  using raw = raw_u32x4;
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void unpack(raw r, float* out) {
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+      out[2 * p] = __uint_as_float(r[p] << 16);
+      out[2 * p + 1] = __uint_as_float(r[p] & 0xffff0000u);
+    }
+  }
+  static __device__ __forceinline__ raw pack(const float* in) {
+    raw r;
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+      const unsigned lo = Conv<bf16_t>::from(in[2 * p]).bits, hi = Conv<bf16_t>::from(in[2 * p + 1]).bits;
+      r[p] = lo | (hi << 16);
+    }
+    return r;
+  }
+};
+template <> struct RawIO<f16_t> {
+  using raw = raw_u32x4;
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void unpack(raw r, float* out) {
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+      out[2 * p] = __half2float(__ushort_as_half((unsigned short)(r[p] & 0xffffu)));
+      out[2 * p + 1] = __half2float(__ushort_as_half((unsigned short)(r[p] >> 16)));
+    }
+  }
+  static __device__ __forceinline__ raw pack(const float* in) {
+    raw r;
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+      const unsigned lo = Conv<f16_t>::from(in[2 * p]).bits, hi = Conv<f16_t>::from(in[2 * p + 1]).bits;
+      r[p] = lo | (hi << 16);
+    }
+    return r;
+  }
+};
+
+// ---- fast math for the fused row/activation kernels ---------------------------------------------------
+// 1/x from the hardware reciprocal (1 ulp) instead of the 11-instruction IEEE division sequence
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ double fast_rcp(double x) { return 1.0 / x; }
+// e^x through v_exp_f32 with the rounding error of x*log2(e) folded back in (about 2 ulp over the whole
+// range, 6 instructions); no special handling beyond what v_exp_f32 does for overflow/underflow
+__device__ __forceinline__ float fast_exp(float x) {
+  const float L2E = 1.44269502162933349609375f, L2E_LO = 1.925963033500011e-08f, LN2 = 0.693147182464599609375f;
+  float t = x * L2E;
+  float lo = __builtin_fmaf(x, L2E, -t);
+  lo = __builtin_fmaf(x, L2E_LO, lo);
+  lo = __builtin_fabsf(t) == INFINITY ? 0.f : lo;   // keeps e^(+-inf) = inf / 0 instead of NaN
+  float r = __builtin_amdgcn_exp2f(t);
+  return __builtin_fmaf(r, lo * LN2, r);
+}
+__device__ __forceinline__ double fast_exp(double x) { return exp(x); }
 
 // ---- wave reductions ---------------------------------------------------------------------------------
 // Butterfly over a row of 16 lanes with DPP (quad_perm 1,0,3,2 / 2,3,0,1 / row_half_mirror / row_mirror),

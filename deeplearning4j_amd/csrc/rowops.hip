@@ -37,17 +37,33 @@ __device__ __forceinline__ A row_allreduce(A v, A* lds) {
   return block_allreduce<Op, 4, A>(v, lds);
 }
 
-// softmax transform of one cached value given the row max
-template <typename A>
-__device__ __forceinline__ A softmax_term(A v, A mx, int clamp) {
+// softmax numerator of one value given the row max.  Clamp mode: finite x gives exp(max(x - max, -88)) (the
+// upper clamp can only bind for +inf/NaN, which the reference maps to max + 88); plain mode: exp(x - max).
+// The exponential is v_exp_f32 on d*log2(e): its error relative to the row's largest term is below 3e-8.
+__device__ __forceinline__ float softmax_term(float v, float mx, int clamp) {
+  const float L2E = 1.44269502162933349609375f;
+  float d = v - mx;
   if (clamp) {
-    if (!r_finite(v)) v = (v > 0 || v != v) ? (A)88 + mx : (A)-88 + mx;
-    A d = v - mx;
-    d = d > (A)88 ? (A)88 : d;
-    d = d < (A)-88 ? (A)-88 : d;
-    return r_exp<A>(d);
+    d = __builtin_fmaxf(d, -88.f);                      // -inf and finite underflow; a NaN operand is dropped
+    d = (v <= 3.4028234663852886e38f) ? d : 88.f;       // +inf and NaN take the upper clamp
   }
-  return r_exp<A>(v - mx);
+  return __builtin_amdgcn_exp2f(d * L2E);
+}
+__device__ __forceinline__ double softmax_term(double v, double mx, int clamp) {
+  if (clamp) {
+    if (!r_finite(v)) v = (v > 0 || v != v) ? 88.0 + mx : -88.0 + mx;
+    double d = v - mx;
+    d = d > 88.0 ? 88.0 : d;
+    d = d < -88.0 ? -88.0 : d;
+    return exp(d);
+  }
+  return exp(v - mx);
+}
+// max over the finite values only (clamp mode) folded into one compare + select
+template <typename A>
+__device__ __forceinline__ A softmax_maxstep(A mx, A v, int clamp) {
+  if (clamp) v = (v < 0 ? -v : v) <= r_tmax<A>() ? v : -r_tmax<A>();
+  return v > mx ? v : mx;
 }
 
 // VEC == 1: element loads through xInner/zInner strides; VEC > 1: 16-byte loads, unit strides
@@ -70,9 +86,7 @@ __global__ __launch_bounds__(256) void softmax_rows(RowArgs a, const T* __restri
     const LongType e0 = ((LongType)t + (LongType)i * TPR) * VEC;
     if (VEC > 1) {
       if (e0 < L) {
-        VT v = *reinterpret_cast<const VT*>(x + xb + e0);
-#pragma unroll
-        for (int e = 0; e < VEC; e++) vals[i * VEC + e] = (A)to_float(v.v[e]);
+        RawIO<T>::unpack(*reinterpret_cast<const typename RawIO<T>::raw*>(x + xb + e0), &vals[i * VEC]);
       } else {
 #pragma unroll
         for (int e = 0; e < VEC; e++) vals[i * VEC + e] = NEG;
@@ -84,9 +98,7 @@ __global__ __launch_bounds__(256) void softmax_rows(RowArgs a, const T* __restri
   A mx = NEG;
 #pragma unroll
   for (int i = 0; i < NV * VEC; i++) {
-    A v = vals[i];
-    if (clamp) { if (r_finite(v)) mx = v > mx ? v : mx; }
-    else mx = v > mx ? v : mx;
+    mx = softmax_maxstep<A>(mx, vals[i], clamp);
   }
   mx = row_allreduce<MaxOp, TPR, A>(mx, lds);
   if (clamp && mx == NEG) mx = (A)0;
@@ -96,23 +108,23 @@ __global__ __launch_bounds__(256) void softmax_rows(RowArgs a, const T* __restri
     const LongType e0 = ((LongType)t + (LongType)i * TPR) * VEC;
 #pragma unroll
     for (int e = 0; e < VEC; e++) {
-      if (e0 + e < L) { A r = softmax_term<A>(vals[i * VEC + e], mx, clamp); vals[i * VEC + e] = r; sum += r; }
+      if (e0 + e < L) { A r = softmax_term(vals[i * VEC + e], mx, clamp); vals[i * VEC + e] = r; sum += r; }
     }
   }
   sum = row_allreduce<SumOp, TPR, A>(sum, lds);
   if (clamp) sum = sum > (A)1e-6f ? sum : (A)1e-6f;
   if (!live) return;
+  const A inv = (A)1 / sum;   // one division per row; every element is scaled by the reciprocal
 #pragma unroll
   for (int i = 0; i < NV; i++) {
     const LongType e0 = ((LongType)t + (LongType)i * TPR) * VEC;
     if (e0 >= L) continue;
     if (VEC > 1) {
-      VT o;
 #pragma unroll
-      for (int e = 0; e < VEC; e++) o.v[e] = Conv<T>::from(vals[i * VEC + e] / sum);
-      *reinterpret_cast<VT*>(z + zb + e0) = o;
+      for (int e = 0; e < VEC; e++) vals[i * VEC + e] *= inv;
+      *reinterpret_cast<typename RawIO<T>::raw*>(z + zb + e0) = RawIO<T>::pack(&vals[i * VEC]);
     } else {
-      z[zb + e0 * a.zInner] = Conv<T>::from(vals[i] / sum);
+      z[zb + e0 * a.zInner] = Conv<T>::from(vals[i] * inv);
     }
   }
 }
@@ -127,18 +139,16 @@ __global__ __launch_bounds__(256) void softmax_long(RowArgs a, const T* __restri
   const A NEG = -r_tmax<A>();
   A mx = NEG;
   for (LongType j = threadIdx.x; j < a.rowLen; j += 256) {
-    A v = (A)to_float(x[xb + j * a.xInner]);
-    if (clamp) { if (r_finite(v)) mx = v > mx ? v : mx; }
-    else mx = v > mx ? v : mx;
+    mx = softmax_maxstep<A>(mx, (A)to_float(x[xb + j * a.xInner]), clamp);
   }
   mx = block_allreduce<MaxOp, 4, A>(mx, lds);
   if (clamp && mx == NEG) mx = (A)0;
   A sum = (A)0;
-  for (LongType j = threadIdx.x; j < a.rowLen; j += 256) sum += softmax_term<A>((A)to_float(x[xb + j * a.xInner]), mx, clamp);
+  for (LongType j = threadIdx.x; j < a.rowLen; j += 256) sum += softmax_term((A)to_float(x[xb + j * a.xInner]), mx, clamp);
   sum = block_allreduce<SumOp, 4, A>(sum, lds);
   if (clamp) sum = sum > (A)1e-6f ? sum : (A)1e-6f;
   for (LongType j = threadIdx.x; j < a.rowLen; j += 256)
-    z[zb + j * a.zInner] = Conv<T>::from(softmax_term<A>((A)to_float(x[xb + j * a.xInner]), mx, clamp) / sum);
+    z[zb + j * a.zInner] = Conv<T>::from(softmax_term((A)to_float(x[xb + j * a.xInner]), mx, clamp) / sum);
 }
 
 // many short strided rows (softmax over a non-last axis): one thread per row, neighbouring threads
@@ -152,16 +162,14 @@ __global__ __launch_bounds__(256) void softmax_flat(RowArgs a, const T* __restri
   const A NEG = -r_tmax<A>();
   A mx = NEG;
   for (LongType j = 0; j < a.rowLen; j++) {
-    A v = (A)to_float(x[xb + j * a.xInner]);
-    if (clamp) { if (r_finite(v)) mx = v > mx ? v : mx; }
-    else mx = v > mx ? v : mx;
+    mx = softmax_maxstep<A>(mx, (A)to_float(x[xb + j * a.xInner]), clamp);
   }
   if (clamp && mx == NEG) mx = (A)0;
   A sum = (A)0;
-  for (LongType j = 0; j < a.rowLen; j++) sum += softmax_term<A>((A)to_float(x[xb + j * a.xInner]), mx, clamp);
+  for (LongType j = 0; j < a.rowLen; j++) sum += softmax_term((A)to_float(x[xb + j * a.xInner]), mx, clamp);
   if (clamp) sum = sum > (A)1e-6f ? sum : (A)1e-6f;
   for (LongType j = 0; j < a.rowLen; j++)
-    z[zb + j * a.zInner] = Conv<T>::from(softmax_term<A>((A)to_float(x[xb + j * a.xInner]), mx, clamp) / sum);
+    z[zb + j * a.zInner] = Conv<T>::from(softmax_term((A)to_float(x[xb + j * a.xInner]), mx, clamp) / sum);
 }
 
 static RowArgs rowArgs(const RowPlan& p) {
@@ -246,9 +254,9 @@ __global__ __launch_bounds__(256) void layernorm_rows(RowArgs a, const T* __rest
     const LongType e0 = ((LongType)t + (LongType)i * TPR) * VEC;
     if (VEC > 1) {
       if (e0 < L) {
-        VT v = *reinterpret_cast<const VT*>(x + xb + e0);
+        RawIO<T>::unpack(*reinterpret_cast<const typename RawIO<T>::raw*>(x + xb + e0), &vals[i * VEC]);
 #pragma unroll
-        for (int e = 0; e < VEC; e++) { vals[i * VEC + e] = (A)to_float(v.v[e]); sum += vals[i * VEC + e]; }
+        for (int e = 0; e < VEC; e++) sum += vals[i * VEC + e];
       } else {
 #pragma unroll
         for (int e = 0; e < VEC; e++) vals[i * VEC + e] = (A)0;
@@ -269,24 +277,25 @@ __global__ __launch_bounds__(256) void layernorm_rows(RowArgs a, const T* __rest
   }
   sq = row_allreduce<SumOp, TPR, A>(sq, lds);
   const A var = L > 1 ? sq / (A)L : (A)0;
-  const A sd = r_sqrt<A>(var + (A)eps);
+  const A rstd = (A)1 / r_sqrt<A>(var + (A)eps);   // one division per row
   if (!live) return;
 #pragma unroll
   for (int i = 0; i < NV; i++) {
     const LongType e0 = ((LongType)t + (LongType)i * TPR) * VEC;
     if (e0 >= L) continue;
     if (VEC > 1) {
-      VT g = *reinterpret_cast<const VT*>(gain + e0), b, o;
-      if (bias) b = *reinterpret_cast<const VT*>(bias + e0);
+      A g[VEC], b[VEC];
+      RawIO<T>::unpack(*reinterpret_cast<const typename RawIO<T>::raw*>(gain + e0), g);
+      if (bias) RawIO<T>::unpack(*reinterpret_cast<const typename RawIO<T>::raw*>(bias + e0), b);
 #pragma unroll
       for (int e = 0; e < VEC; e++) {
-        A y = (vals[i * VEC + e] - mean) / sd * (A)to_float(g.v[e]);
-        if (bias) y += (A)to_float(b.v[e]);
-        o.v[e] = Conv<T>::from(y);
+        A y = (vals[i * VEC + e] - mean) * rstd * g[e];
+        if (bias) y += b[e];
+        vals[i * VEC + e] = y;
       }
-      *reinterpret_cast<VT*>(z + zb + e0) = o;
+      *reinterpret_cast<typename RawIO<T>::raw*>(z + zb + e0) = RawIO<T>::pack(&vals[i * VEC]);
     } else {
-      A y = (vals[i] - mean) / sd * (A)to_float(gain[e0]);
+      A y = (vals[i] - mean) * rstd * (A)to_float(gain[e0]);
       if (bias) y += (A)to_float(bias[e0]);
       z[zb + e0 * a.zInner] = Conv<T>::from(y);
     }

@@ -71,8 +71,17 @@ def _reduced_shape(shape, dims, keep_dims):
     return out
 
 
+_DIMS_CACHE = {}
+
+
 def _dims_array(dims):
-    return NDArray.from_numpy(np.asarray(dims, dtype=np.int64))
+    """INT64 host array holding the dimensions (cached: the same few tuples recur on every call)."""
+    key = tuple(int(d) for d in dims)
+    arr = _DIMS_CACHE.get(key)
+    if arr is None:
+        arr = NDArray.from_numpy(np.asarray(key, dtype=np.int64))
+        _DIMS_CACHE[key] = arr
+    return arr
 
 
 class OpContext:
@@ -245,6 +254,22 @@ class Executioner:
         finally:
             ctx.close()
         return outputs
+
+    def bind_custom(self, name, inputs, outputs, t_args=(), i_args=(), b_args=(), d_args=()):
+        """Build the OpContext once and return a zero-argument callable that runs execCustomOp2 on it.
+        For loops that execute the same op on the same arrays many times (benchmarks, decode steps)."""
+        ctx = OpContext()
+        ctx.set_inputs(inputs)
+        ctx.set_outputs(outputs)
+        ctx.set_args(t_args, i_args, b_args, d_args)
+        h = self.op_hash(name)
+        run = self.L.execCustomOp2
+
+        def call():
+            if run(None, h, ctx.ptr) != 0:
+                raise N.NativeOpsError("Op [%s] execution failed: %s" % (name, self.L.lastErrorMessage().decode(errors="replace")))
+        call.ctx = ctx
+        return call
 
     def synchronize(self):
         self.L.streamSynchronize(None)
