@@ -1,9 +1,25 @@
-// Attention kernels for dot_product_attention_v2.
+// Attention kernels for dot_product_attention_v2
+// (reference: libnd4j/include/helpers/impl/AttentionHelper.cpp:340-352 logits, :70-79 mask, :189-241 scores).
 //
-//   logits fix-up - in-place pass over dense [B, Tq, Tv] logits: optional scale, clip to +-1e4, and the
-//                   causal mask penalty (reference: helpers/impl/AttentionHelper.cpp:340-352, :189-241).
+//   attn_fused    - out = softmax(mask(clip(scale * q k^T))) v without materialising anything of size Tq x Tv.
+//                   One block = 128 queries of one batch entry (4 waves x 32 queries), looping over 64-key tiles
+//                   of K and V staged in LDS.  The score tile is computed TRANSPOSED, S^T = K Q^T, so that an MFMA
+//                   lane owns one query column: the softmax statistics (running max / running sum) and the
+//                   rescaling of the output accumulator O^T = V^T P^T are then per-lane scalars, and the row
+//                   reductions run over a lane's own registers plus one exchange with the other half-wave.
+//                   P^T feeds the second MFMA straight from the score accumulators (the MFMA k-slots are
+//                   assigned to keys in exactly the order the accumulator registers hold them, and V^T is read
+//                   from LDS in that same order), so the probabilities never leave registers.
+//                   Logits are rounded through the storage type before the softmax, as the reference's
+//                   op-by-op composition stores them in an array of that type.  Masked (key > query) and
+//                   out-of-range keys contribute exactly zero; the reference's clamped softmax gives them
+//                   e^-88 / sum, below 1e-36.
+//                   Bound: MFMA for the contractions, in practice the per-score VALU work (exp, max, convert).
+//   logits fix-up - in-place pass over dense [B, Tq, Tv] logits for the composition path that writes the
+//                   logits / weights outputs: optional scale, clip to +-1e4, causal penalty.
 #include "device.h"
 #include "kernels.h"
+#include "mfma_tile.h"
 #include "runtime.h"
 
 namespace nd4jhip {
@@ -27,9 +43,6 @@ __global__ __launch_bounds__(256) void logits_fixup(T* __restrict__ l, LongType 
 void launchAttentionLogitsFixup(hipStream_t s, DataType dt, void* logits, const AttnDesc& d) {
   const LongType total = d.B * d.Tq * d.Tv;
   if (total == 0) return;
-  if (!d.applyScale && !d.causal) {
-    // clip only; still needed because values beyond +-1e4 must be clamped
-  }
   LongType blocks = (total + 255) / 256;
   if (blocks > 256 * 16) blocks = 256 * 16;
   dim3 g((unsigned)blocks), b(256);
@@ -42,9 +55,205 @@ void launchAttentionLogitsFixup(hipStream_t s, DataType dt, void* logits, const 
   HIP_CHECK(hipGetLastError());
 }
 
-bool attentionFusedSupported(DataType, const AttnDesc&) { return false; }
-void launchAttentionFused(hipStream_t, DataType, const void*, const void*, const void*, void*, const AttnDesc&) {
-  ND4J_THROW("attention: fused kernel is not available in this build");
+// ---- fused kernel ------------------------------------------------------------------------------------------------
+struct FusedArgs {
+  LongType Tq, Tv;
+  LongType qB, qT, kB, kT, vB, vT, oB, oT;
+  float scale;
+  int applyScale, causal;
+  int qTiles;
+};
+
+template <typename T> __device__ __forceinline__ float round_storage(float v) { return to_float(Conv<T>::from(v)); }
+template <typename T> __device__ __forceinline__ unsigned pack2(float a, float b) {
+  return (unsigned)Conv<T>::from(a).bits | ((unsigned)Conv<T>::from(b).bits << 16);
+}
+
+template <typename T, int D>
+__global__ __launch_bounds__(256) void attn_fused(FusedArgs a, const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
+                                                  T* __restrict__ O) {
+  constexpr int BQ = 128, BKV = 64, NT = 256;
+  constexpr int DG = D / 8;                      // 16-byte groups along d
+  constexpr int KSLOTS = DG * (BKV + 1);         // K tile: [d/8][key][8 d]
+  constexpr int VSLOTS = (BKV / 8) * (D + 1);    // V tile: [key/8][dv][8 keys]
+  constexpr int DT = D / 32;                     // dv tiles of the output accumulator
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  u32x4* smem = reinterpret_cast<u32x4*>(smem_raw);   // two stages of (K tile, V tile)
+
+  // heavy (late) query tiles first under the causal mask
+  const int qt = a.qTiles - 1 - (int)(blockIdx.x % a.qTiles);
+  const LongType b = blockIdx.x / a.qTiles;
+  const LongType q0 = (LongType)qt * BQ;
+  Q += b * a.qB; K += b * a.kB; V += b * a.vB; O += b * a.oB;
+
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, h = lane >> 5;
+  const LongType query = q0 + wave * 32 + (lane & 31);
+  const LongType qrow = query < a.Tq ? query : a.Tq - 1;
+
+  // Q^T fragments: lane (query, h) holds d = 16*ks + 8*h .. +7 for every k-step
+  u32x4 qf[D / 16];
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ks++) qf[ks] = *reinterpret_cast<const u32x4*>(Q + qrow * a.qT + ks * 16 + h * 8);
+
+  f32x16 o[DT];
+#pragma unroll
+  for (int i = 0; i < DT; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) o[i][r] = 0.f;
+  float m = -1.0e30f, l = 0.f;
+  const float L2E = 1.44269502162933349609375f;
+
+  LongType kvEnd = a.Tv;
+  if (a.causal) { const LongType lim = q0 + BQ; kvEnd = lim < kvEnd ? lim : kvEnd; }
+  const LongType nTiles = (kvEnd + BKV - 1) / BKV;
+
+  // the loader moves 64 k-values per pass: the K tile (D values of d per key) takes D/64 of them
+  TileLoader<BKV, NT, true> lk[D / 64];   // rows = keys, contiguous along d
+  TileLoader<D, NT, false> lv;            // rows = dv (contiguous in memory), "k" = keys
+  auto loadKV = [&](LongType kv0) {
+#pragma unroll
+    for (int part = 0; part < D / 64; part++) lk[part].load(K + part * 64, a.kT, kv0, a.Tv, 0, 64, t);
+    lv.load(V, a.vT, 0, D, kv0, a.Tv, t);
+  };
+  auto storeKV = [&](u32x4* dst) {
+#pragma unroll
+    for (int part = 0; part < D / 64; part++) lk[part].store(dst + part * 8 * (BKV + 1), 0, a.Tv, t);
+    lv.store(dst + KSLOTS, 0, D, t);
+  };
+
+  if (nTiles > 0) {
+    loadKV(0);
+    storeKV(smem);
+  }
+  __syncthreads();
+
+  for (LongType it = 0; it < nTiles; it++) {
+    const int cur = (int)(it & 1);
+    const LongType kv0 = it * BKV;
+    const u32x4* sK = smem + cur * (KSLOTS + VSLOTS);
+    const u32x4* sV = sK + KSLOTS;
+    const bool more = it + 1 < nTiles;
+    if (more) loadKV(kv0 + BKV);   // in flight while this tile is computed
+
+    // S^T = K Q^T : two 32-key tiles, D/16 k-steps
+    f32x16 s[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; kt++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) s[kt][r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ks++) {
+        const u32x4 kf = sK[(ks * 2 + h) * (BKV + 1) + kt * 32 + (lane & 31)];
+        s[kt] = Mfma16<T>::mma(kf, qf[ks], s[kt]);
+      }
+    }
+    // scores of this lane's query: register r of tile kt is key kv0 + 32*kt + 8*(r/4) + 4*h + r%4
+    float tmax = -1.0e30f;
+#pragma unroll
+    for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        float v = s[kt][r];
+        if (a.applyScale) v *= a.scale;
+        v = __builtin_fminf(__builtin_fmaxf(v, -1.0e4f), 1.0e4f);
+        v = round_storage<T>(v);
+        const LongType key = kv0 + kt * 32 + 8 * (r / 4) + 4 * h + (r & 3);
+        const bool masked = key >= a.Tv || (a.causal && key > query);
+        v = masked ? -1.0e30f : v;
+        s[kt][r] = v;
+        tmax = __builtin_fmaxf(tmax, v);
+      }
+    tmax = __builtin_fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+    const float mNew = __builtin_fmaxf(m, tmax);
+    const float alpha = __builtin_amdgcn_exp2f((m - mNew) * L2E);
+    m = mNew;
+    float psum = 0.f;
+    u32x4 pf[4];   // P^T operand of k-step ks: registers 8*(ks%2) .. +7 of tile ks/2
+#pragma unroll
+    for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) {
+        // a fully masked history keeps m at the floor; masked entries are forced to zero explicitly
+        float p0 = s[kt][r] <= -1.0e29f ? 0.f : __builtin_amdgcn_exp2f((s[kt][r] - mNew) * L2E);
+        float p1 = s[kt][r + 1] <= -1.0e29f ? 0.f : __builtin_amdgcn_exp2f((s[kt][r + 1] - mNew) * L2E);
+        psum += p0 + p1;
+        pf[kt * 2 + r / 8][(r % 8) / 2] = pack2<T>(p0, p1);
+      }
+    l = l * alpha + psum;
+#pragma unroll
+    for (int i = 0; i < DT; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) o[i][r] *= alpha;
+
+    // O^T += V^T P^T : k-slot e of k-step ks on half h is key 16*ks + 8*(e/4) + 4*h + e%4 (the accumulator order)
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+#pragma unroll
+      for (int i = 0; i < DT; i++) {
+        const int dv = i * 32 + (lane & 31);
+        const u32x2* g0 = reinterpret_cast<const u32x2*>(&sV[(2 * ks) * (D + 1) + dv]);
+        const u32x2* g1 = reinterpret_cast<const u32x2*>(&sV[(2 * ks + 1) * (D + 1) + dv]);
+        const u32x2 lo = g0[h], hi = g1[h];
+        const u32x4 vf = {lo[0], lo[1], hi[0], hi[1]};
+        o[i] = Mfma16<T>::mma(vf, pf[ks], o[i]);
+      }
+    }
+    if (more) storeKV(smem + (cur ^ 1) * (KSLOTS + VSLOTS));
+    __syncthreads();
+  }
+
+  // normalise and write O: register r of dv-tile i is dv = 32*i + 8*(r/4) + 4*h + r%4
+  l += __shfl_xor(l, 32, WAVE);
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  if (query < a.Tq) {
+    T* orow = O + query * a.oT;
+#pragma unroll
+    for (int i = 0; i < DT; i++)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; r4++) {
+        const int dv = i * 32 + 8 * r4 + 4 * h;
+        u32x2 w;
+        w[0] = pack2<T>(o[i][4 * r4] * inv, o[i][4 * r4 + 1] * inv);
+        w[1] = pack2<T>(o[i][4 * r4 + 2] * inv, o[i][4 * r4 + 3] * inv);
+        *reinterpret_cast<u32x2*>(orow + dv) = w;
+      }
+  }
+}
+
+bool attentionFusedSupported(DataType dt, const AttnDesc& d) {
+  if (dt != HALF && dt != BFLOAT16) return false;
+  if (d.D != d.Dv || (d.D != 64 && d.D != 128)) return false;
+  if (d.Tq < 1 || d.Tv < 8 || d.Tv % 8 != 0) return false;           // 8x8 blocks of V must not straddle the end
+  // 16-byte aligned rows
+  for (LongType st : {d.qB, d.qT, d.kB, d.kT, d.vB, d.vT}) if (st % 8 != 0) return false;
+  if (d.oB % 4 != 0 || d.oT % 4 != 0) return false;
+  return true;
+}
+
+template <typename T, int D>
+static void launchFusedTyped(hipStream_t s, const void* q, const void* k, const void* v, void* out, const AttnDesc& d) {
+  FusedArgs a;
+  a.Tq = d.Tq; a.Tv = d.Tv;
+  a.qB = d.qB; a.qT = d.qT; a.kB = d.kB; a.kT = d.kT; a.vB = d.vB; a.vT = d.vT; a.oB = d.oB; a.oT = d.oT;
+  a.scale = d.scale; a.applyScale = d.applyScale ? 1 : 0; a.causal = d.causal ? 1 : 0;
+  a.qTiles = (int)((d.Tq + 127) / 128);
+  constexpr size_t LDS = (size_t)2 * ((D / 8) * (64 + 1) + (64 / 8) * (D + 1)) * 16;
+  auto kern = attn_fused<T, D>;
+  static bool attrSet = false;
+  if (!attrSet) {
+    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS));
+    attrSet = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)(a.qTiles * d.B)), dim3(256), LDS, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
+}
+
+void launchAttentionFused(hipStream_t s, DataType dt, const void* q, const void* k, const void* v, void* out, const AttnDesc& d) {
+  ND4J_REQUIRE(attentionFusedSupported(dt, d), "attention: fused kernel does not take this problem");
+  ND4J_REQUIRE((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) == 0 && ((uintptr_t)out & 7) == 0, "attention: operands must be 16-byte aligned");
+  ND4J_REQUIRE(((d.Tq + 127) / 128) * d.B < (1LL << 31), "attention: too many query tiles");
+  if (dt == HALF) { if (d.D == 64) launchFusedTyped<f16_t, 64>(s, q, k, v, out, d); else launchFusedTyped<f16_t, 128>(s, q, k, v, out, d); }
+  else { if (d.D == 64) launchFusedTyped<bf16_t, 64>(s, q, k, v, out, d); else launchFusedTyped<bf16_t, 128>(s, q, k, v, out, d); }
+  HIP_CHECK(hipGetLastError());
 }
 
 }  // namespace nd4jhip

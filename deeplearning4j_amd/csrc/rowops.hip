@@ -68,7 +68,7 @@ __device__ __forceinline__ A softmax_maxstep(A mx, A v, int clamp) {
 
 // VEC == 1: element loads through xInner/zInner strides; VEC > 1: 16-byte loads, unit strides
 template <typename T, int TPR, int NV, int VEC>
-__global__ __launch_bounds__(256) void softmax_rows(RowArgs a, const T* __restrict__ x, T* __restrict__ z, int clamp) {
+__global__ __launch_bounds__(256) void softmax_rows(RowArgs a, const T* __restrict__ x, T* __restrict__ z, int clamp, int nt) {
   using A = typename Conv<T>::acc;
   using VT = Vec<T, VEC>;
   constexpr int ROWS = 256 / TPR;
@@ -86,7 +86,8 @@ __global__ __launch_bounds__(256) void softmax_rows(RowArgs a, const T* __restri
     const LongType e0 = ((LongType)t + (LongType)i * TPR) * VEC;
     if (VEC > 1) {
       if (e0 < L) {
-        RawIO<T>::unpack(*reinterpret_cast<const typename RawIO<T>::raw*>(x + xb + e0), &vals[i * VEC]);
+        const typename RawIO<T>::raw* src = reinterpret_cast<const typename RawIO<T>::raw*>(x + xb + e0);
+        RawIO<T>::unpack(nt ? __builtin_nontemporal_load(src) : *src, &vals[i * VEC]);
       } else {
 #pragma unroll
         for (int e = 0; e < VEC; e++) vals[i * VEC + e] = NEG;
@@ -122,7 +123,9 @@ __global__ __launch_bounds__(256) void softmax_rows(RowArgs a, const T* __restri
     if (VEC > 1) {
 #pragma unroll
       for (int e = 0; e < VEC; e++) vals[i * VEC + e] *= inv;
-      *reinterpret_cast<typename RawIO<T>::raw*>(z + zb + e0) = RawIO<T>::pack(&vals[i * VEC]);
+      typename RawIO<T>::raw* dst = reinterpret_cast<typename RawIO<T>::raw*>(z + zb + e0);
+      if (nt) __builtin_nontemporal_store(RawIO<T>::pack(&vals[i * VEC]), dst);
+      else *dst = RawIO<T>::pack(&vals[i * VEC]);
     } else {
       z[zb + e0 * a.zInner] = Conv<T>::from(vals[i] * inv);
     }
@@ -200,7 +203,9 @@ static void softmaxTyped(hipStream_t s, const void* x, void* z, const RowPlan& p
   const unsigned gw = (unsigned)((p.rows + 3) / 4), gb = (unsigned)p.rows;
   if (rowsVectorOk(p, x, z, V)) {
     const LongType perWave = 64 * V, perBlock = 256 * V;
-#define SM(TPR, NV, GRID) hipLaunchKernelGGL((softmax_rows<T, TPR, NV, V>), dim3(GRID), dim3(256), 0, s, a, xt, zt, clamp)
+    // rows streamed once and larger than the last-level cache: non-temporal accesses
+    const int nt = (size_t)p.rows * (size_t)L * sizeof(T) * 2 > ((size_t)288 << 20) ? 1 : 0;
+#define SM(TPR, NV, GRID) hipLaunchKernelGGL((softmax_rows<T, TPR, NV, V>), dim3(GRID), dim3(256), 0, s, a, xt, zt, clamp, nt)
     if (L <= perWave) { SM(64, 1, gw); return; }
     if (L <= 2 * perWave) { SM(64, 2, gw); return; }
     if (L <= 4 * perWave) { SM(64, 4, gw); return; }
@@ -210,8 +215,8 @@ static void softmaxTyped(hipStream_t s, const void* x, void* z, const RowPlan& p
     if (L <= 8 * perBlock) { SM(256, 8, gb); return; }
 #undef SM
   } else {
-    if (L <= 64 * 16) { hipLaunchKernelGGL((softmax_rows<T, 64, 16, 1>), dim3(gw), dim3(256), 0, s, a, xt, zt, clamp); return; }
-    if (L <= 256 * 32) { hipLaunchKernelGGL((softmax_rows<T, 256, 32, 1>), dim3(gb), dim3(256), 0, s, a, xt, zt, clamp); return; }
+    if (L <= 64 * 16) { hipLaunchKernelGGL((softmax_rows<T, 64, 16, 1>), dim3(gw), dim3(256), 0, s, a, xt, zt, clamp, 0); return; }
+    if (L <= 256 * 32) { hipLaunchKernelGGL((softmax_rows<T, 256, 32, 1>), dim3(gb), dim3(256), 0, s, a, xt, zt, clamp, 0); return; }
   }
   hipLaunchKernelGGL((softmax_long<T>), dim3(gb), dim3(256), 0, s, a, xt, zt, clamp);
 }
