@@ -74,8 +74,10 @@ __global__ __launch_bounds__(256) void attn_fused(FusedArgs a, const T* __restri
                                                   T* __restrict__ O) {
   constexpr int BQ = 128, BKV = 64, NT = 256;
   constexpr int DG = D / 8;                      // 16-byte groups along d
-  constexpr int KSLOTS = DG * (BKV + 1);         // K tile: [d/8][key][8 d]
-  constexpr int VSLOTS = (BKV / 8) * (D + 1);    // V tile: [key/8][dv][8 keys]
+  using LayK = TileLayout<BKV, true>;            // K tile: [d/8][key][8 d], one 64-wide pass per 64 values of d
+  using LayV = TileLayout<D, false>;             // V tile: [key/8][dv (permuted)][8 keys]
+  constexpr int KSLOTS = (D / 64) * LayK::SLOTS;
+  constexpr int VSLOTS = LayV::SLOTS;
   constexpr int DT = D / 32;                     // dv tiles of the output accumulator
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   u32x4* smem = reinterpret_cast<u32x4*>(smem_raw);   // two stages of (K tile, V tile)
@@ -117,8 +119,8 @@ __global__ __launch_bounds__(256) void attn_fused(FusedArgs a, const T* __restri
   };
   auto storeKV = [&](u32x4* dst) {
 #pragma unroll
-    for (int part = 0; part < D / 64; part++) lk[part].store(dst + part * 8 * (BKV + 1), 0, a.Tv, t);
-    lv.store(dst + KSLOTS, 0, D, t);
+    for (int part = 0; part < D / 64; part++) lk[part].store(dst + part * LayK::SLOTS, t);
+    lv.store(dst + KSLOTS, t);
   };
 
   if (nTiles > 0) {
@@ -143,7 +145,7 @@ __global__ __launch_bounds__(256) void attn_fused(FusedArgs a, const T* __restri
       for (int r = 0; r < 16; r++) s[kt][r] = 0.f;
 #pragma unroll
       for (int ks = 0; ks < D / 16; ks++) {
-        const u32x4 kf = sK[(ks * 2 + h) * (BKV + 1) + kt * 32 + (lane & 31)];
+        const u32x4 kf = sK[LayK::slot(ks * 2 + h, kt * 32 + (lane & 31))];   // parts of 8 k-groups follow each other
         s[kt] = Mfma16<T>::mma(kf, qf[ks], s[kt]);
       }
     }
@@ -191,8 +193,8 @@ __global__ __launch_bounds__(256) void attn_fused(FusedArgs a, const T* __restri
 #pragma unroll
       for (int i = 0; i < DT; i++) {
         const int dv = i * 32 + (lane & 31);
-        const u32x2* g0 = reinterpret_cast<const u32x2*>(&sV[(2 * ks) * (D + 1) + dv]);
-        const u32x2* g1 = reinterpret_cast<const u32x2*>(&sV[(2 * ks + 1) * (D + 1) + dv]);
+        const u32x2* g0 = reinterpret_cast<const u32x2*>(&sV[LayV::slot(2 * ks, dv)]);
+        const u32x2* g1 = reinterpret_cast<const u32x2*>(&sV[LayV::slot(2 * ks + 1, dv)]);
         const u32x2 lo = g0[h], hi = g1[h];
         const u32x4 vf = {lo[0], lo[1], hi[0], hi[1]};
         o[i] = Mfma16<T>::mma(vf, pf[ks], o[i]);
@@ -237,7 +239,7 @@ static void launchFusedTyped(hipStream_t s, const void* q, const void* k, const 
   a.qB = d.qB; a.qT = d.qT; a.kB = d.kB; a.kT = d.kT; a.vB = d.vB; a.vT = d.vT; a.oB = d.oB; a.oT = d.oT;
   a.scale = d.scale; a.applyScale = d.applyScale ? 1 : 0; a.causal = d.causal ? 1 : 0;
   a.qTiles = (int)((d.Tq + 127) / 128);
-  constexpr size_t LDS = (size_t)2 * ((D / 8) * (64 + 1) + (64 / 8) * (D + 1)) * 16;
+  constexpr size_t LDS = (size_t)2 * ((D / 64) * TileLayout<64, true>::SLOTS + TileLayout<D, false>::SLOTS) * 16;
   auto kern = attn_fused<T, D>;
   static bool attrSet = false;
   if (!attrSet) {

@@ -14,6 +14,8 @@
 //   gemv_*       M == 1 or N == 1: HBM-bound streaming of the matrix operand.
 //   gemm_simple  any float dtype, any strides (also fp64): 32x32 tile per block through LDS.  Correctness
 //                path for small, odd-shaped or oddly strided problems.
+#include <cstdlib>
+
 #include "device.h"
 #include "kernels.h"
 #include "mfma_tile.h"
@@ -96,7 +98,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16(GemmArgs g, const T*
                                                              unsigned tilesM, unsigned tilesN) {
   constexpr int BK = 64, NT = WM * WN * 64;
   constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
-  constexpr int SLOTS_A = 8 * (BM + 1), SLOTS_B = 8 * (BN + 1), STAGE = SLOTS_A + SLOTS_B;
+  using LayA = TileLayout<BM, A_KC>;
+  using LayB = TileLayout<BN, B_KC>;
+  constexpr int SLOTS_A = LayA::SLOTS, SLOTS_B = LayB::SLOTS, STAGE = SLOTS_A + SLOTS_B;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   u32x4* smem = reinterpret_cast<u32x4*>(smem_raw);
 
@@ -124,8 +128,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16(GemmArgs g, const T*
 
   la.load(A, lda, m0, g.M, 0, g.K, t);
   lb.load(B, ldb, n0, g.N, 0, g.K, t);
-  la.store(smem, m0, g.M, t);
-  lb.store(smem + SLOTS_A, n0, g.N, t);
+  la.store(smem, t);
+  lb.store(smem + SLOTS_A, t);
   __syncthreads();
 
   for (LongType kt = 0; kt < KT; kt++) {
@@ -141,9 +145,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16(GemmArgs g, const T*
       const int kg = ks * 2 + (lane >> 5);
       u32x4 fa[TM], fb[TN];
 #pragma unroll
-      for (int i = 0; i < TM; i++) fa[i] = sA[kg * (BM + 1) + wm * WTM + i * 32 + (lane & 31)];
+      for (int i = 0; i < TM; i++) fa[i] = sA[LayA::slot(kg, wm * WTM + i * 32 + (lane & 31))];
 #pragma unroll
-      for (int j = 0; j < TN; j++) fb[j] = sB[kg * (BN + 1) + wn * WTN + j * 32 + (lane & 31)];
+      for (int j = 0; j < TN; j++) fb[j] = sB[LayB::slot(kg, wn * WTN + j * 32 + (lane & 31))];
 #pragma unroll
       for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -151,8 +155,108 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16(GemmArgs g, const T*
     }
     if (kt + 1 < KT) {
       u32x4* dst = smem + (cur ^ 1) * STAGE;
-      la.store(dst, m0, g.M, t);
-      lb.store(dst + SLOTS_A, n0, g.N, t);
+      la.store(dst, t);
+      lb.store(dst + SLOTS_A, t);
+    }
+    __syncthreads();
+  }
+
+  // epilogue: lane owns column (lane % 32); register r of a 32x32 tile is row 8*(r/4) + 4*(lane/32) + r%4
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const LongType col = n0 + wn * WTN + j * 32 + (lane & 31);
+      if (col >= g.N) continue;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const LongType row = m0 + wm * WTM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r & 3);
+        if (row < g.M) {
+          const LongType off = row * g.cRow + col * g.cCol;
+          float v = g.alpha * acc[i][j][r];
+          if (g.beta != 0.f) v += g.beta * to_float(C[off]);
+          C[off] = Conv<T>::from(v);
+        }
+      }
+    }
+}
+
+template <typename T, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16p(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
+                                                             unsigned tilesM, unsigned tilesN) {
+  constexpr int BK = 64, NT = WM * WN * 64;
+  constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
+  using LayA = TileLayout<BM, A_KC>;
+  using LayB = TileLayout<BN, B_KC>;
+  constexpr int SLOTS_A = LayA::SLOTS, SLOTS_B = LayB::SLOTS, STAGE = SLOTS_A + SLOTS_B;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  u32x4* smem = reinterpret_cast<u32x4*>(smem_raw);
+
+  unsigned tm, tn;
+  tileOf(blockIdx.x, gridDim.x, tilesM, tilesN, tm, tn);
+  const LongType m0 = (LongType)tm * BM, n0 = (LongType)tn * BN;
+  const LongType bz = blockIdx.z;
+  A += bz * g.aBatch; B += bz * g.bBatch; C += bz * g.cBatch;
+  const LongType lda = A_KC ? g.aRow : g.aCol, ldb = B_KC ? g.bCol : g.bRow;
+
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+  TileLoader<BM, NT, A_KC> la;
+  TileLoader<BN, NT, B_KC> lb;
+  const LongType KT = (g.K + BK - 1) / BK;
+
+  la.load(A, lda, m0, g.M, 0, g.K, t);
+  lb.load(B, ldb, n0, g.N, 0, g.K, t);
+  la.store(smem, t);
+  lb.store(smem + SLOTS_A, t);
+  __syncthreads();
+
+  for (LongType kt = 0; kt < KT; kt++) {
+    const int cur = (int)(kt & 1);
+    if (kt + 1 < KT) {
+      la.load(A, lda, m0, g.M, (kt + 1) * BK, g.K, t);
+      lb.load(B, ldb, n0, g.N, (kt + 1) * BK, g.K, t);
+    }
+    const u32x4* sA = smem + cur * STAGE;
+    const u32x4* sB = sA + SLOTS_A;
+    // software pipeline over the four k-steps: fragments of step ks+1 are read while the MFMAs of step ks
+    // run; the next tile's registers are written to the other LDS stage in the shadow of step 2
+    u32x4 fa[2][TM], fb[2][TN];
+    auto readFrag = [&](int ks, int buf) {
+      const int kg = ks * 2 + (lane >> 5);
+#pragma unroll
+      for (int i = 0; i < TM; i++) fa[buf][i] = sA[LayA::slot(kg, wm * WTM + i * 32 + (lane & 31))];
+#pragma unroll
+      for (int j = 0; j < TN; j++) fb[buf][j] = sB[LayB::slot(kg, wn * WTN + j * 32 + (lane & 31))];
+    };
+    readFrag(0, 0);
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ks++) {
+      if (ks + 1 < BK / 16) readFrag(ks + 1, (ks + 1) & 1);
+      if (ks == 2 && kt + 1 < KT) {
+        u32x4* dst = smem + (cur ^ 1) * STAGE;
+        la.store(dst, t);
+        lb.store(dst + SLOTS_A, t);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = Mfma16<T>::mma(fa[ks & 1][i], fb[ks & 1][j], acc[i][j]);
+      // interleave: one LDS read issued per pair of MFMAs
+#pragma unroll
+      for (int q = 0; q < (TM + TN); q++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, (TM * TN) / (TM + TN) > 0 ? (TM * TN) / (TM + TN) : 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
     }
     __syncthreads();
   }
@@ -180,8 +284,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16(GemmArgs g, const T*
 template <typename T, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC>
 static void launchMfma16Cfg(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C, LongType batch) {
   constexpr int NT = WM * WN * 64;
-  constexpr size_t LDS = (size_t)2 * (8 * (BM + 1) + 8 * (BN + 1)) * 16;
-  auto kern = gemm_mfma16<T, BM, BN, WM, WN, A_KC, B_KC>;
+  constexpr size_t LDS = (size_t)2 * (TileLayout<BM, A_KC>::SLOTS + TileLayout<BN, B_KC>::SLOTS) * 16;
+  static const bool pipelined = getenv("ND4JHIP_GEMM_PIPE") ? atoi(getenv("ND4JHIP_GEMM_PIPE")) != 0 : true;
+  auto kern = pipelined ? gemm_mfma16p<T, BM, BN, WM, WN, A_KC, B_KC> : gemm_mfma16<T, BM, BN, WM, WN, A_KC, B_KC>;
   static bool attrSet = false;
   if (!attrSet) {
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS));
@@ -198,6 +303,10 @@ static void launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const 
   if (g.M <= 32) return launchMfma16Cfg<T, 32, 128, 1, 4, A_KC, B_KC>(s, g, A, B, C, batch);
   if (g.M <= 64 || g.N <= 64 || tiles128 < 192) return launchMfma16Cfg<T, 64, 64, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
   if (tiles256 < 192) return launchMfma16Cfg<T, 128, 128, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
+  static const int cfg = getenv("ND4JHIP_GEMM_CFG") ? atoi(getenv("ND4JHIP_GEMM_CFG")) : 0;
+  if (cfg == 1) return launchMfma16Cfg<T, 256, 256, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
+  if (cfg == 2) return launchMfma16Cfg<T, 128, 256, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
+  if (cfg == 3) return launchMfma16Cfg<T, 128, 128, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
   return launchMfma16Cfg<T, 256, 256, 2, 4, A_KC, B_KC>(s, g, A, B, C, batch);
 }
 

@@ -33,70 +33,75 @@ __device__ __forceinline__ void transpose8x8(const u32x4 (&r)[8], u32x4 (&out)[8
   }
 }
 
-// Loader for one operand tile of `ROWS` rows (M or N index) x 64 k.
-//   KC = true : memory is [row][k] with unit k stride; ld = row pitch
-//   KC = false: memory is [k][row] with unit row stride; ld = k pitch
+// Loader for one operand tile of `ROWS` rows (M or N index) x 64 k, and the LDS layout it fills.
+//   KC = true : memory is [row][k] with unit k stride; ld = row pitch.  16-byte vectors (8 k of one row) are
+//               copied as they are.  LDS slot of (k-group kg, row r): kg * (ROWS + 1) + r.
+//   KC = false: memory is [k][row] with unit row stride; ld = k pitch.  A thread loads a 4 (k) x 8 (rows) block,
+//               transposes it in registers and writes eight 8-byte half-slots.  Rows are permuted inside a
+//               k-group, slot = kg * (ROWS + 8) + (r % 8) * (ROWS / 8 + 1) + r / 8, so that the writes of one
+//               instruction (fixed r % 8, neighbouring lanes = neighbouring r / 8) land in consecutive slots and
+//               the fragment reads (32 consecutive rows) stay spread over the banks.
+template <int ROWS, bool KC>
+struct TileLayout {
+  static constexpr int GROUP = KC ? ROWS + 1 : ROWS + 8;   // slots per k-group
+  static constexpr int SLOTS = 8 * GROUP;                  // slots per 64-k tile
+  static __device__ __forceinline__ int slot(int kg, int r) {
+    return KC ? kg * GROUP + r : kg * GROUP + (r & 7) * (ROWS / 8 + 1) + (r >> 3);
+  }
+};
+
 template <int ROWS, int NT, bool KC>
 struct TileLoader {
-  static constexpr int VECS = KC ? (ROWS * 8 + NT - 1) / NT : 0;        // 16-byte vectors per thread
-  static constexpr int BLKS = KC ? 0 : (ROWS + NT - 1) / NT;            // 8x8 blocks per thread
-  static constexpr int NREG = KC ? VECS : BLKS * 8;
-  u32x4 reg[NREG > 0 ? NREG : 1];
+  using Layout = TileLayout<ROWS, KC>;
+  static constexpr int UNITS = KC ? ROWS * 8 : ROWS * 2;                 // vectors / 4x8 blocks per tile
+  static constexpr int PER = (UNITS + NT - 1) / NT;                      // per thread
+  static constexpr int NREG = KC ? PER : PER * 4;
+  u32x4 reg[NREG];
 
   template <typename T>
   __device__ __forceinline__ void load(const T* __restrict__ base, LongType ld, LongType row0, LongType rowLimit, LongType k0, LongType K, int t) {
     const u32x4 zero = {0u, 0u, 0u, 0u};
-    if (KC) {
 #pragma unroll
-      for (int i = 0; i < VECS; i++) {
-        const int v = t + i * NT;
-        if (VECS * NT != ROWS * 8 && v >= ROWS * 8) break;
-        const int kg = v & 7, row = v >> 3;
+    for (int i = 0; i < PER; i++) {
+      const int u = t + i * NT;
+      if (PER * NT != UNITS && u >= UNITS) break;
+      if (KC) {
+        const int kg = u & 7, row = u >> 3;
         LongType r = row0 + row;
         r = r < rowLimit ? r : rowLimit - 1;
         const LongType k = k0 + kg * 8;
         reg[i] = k < K ? *reinterpret_cast<const u32x4*>(base + r * ld + k) : zero;
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < BLKS; i++) {
-        const int b = t + i * NT;
-        if (BLKS * NT != ROWS && b >= ROWS) break;
-        const int rb = b % (ROWS / 8), kg = b / (ROWS / 8);
+      } else {
+        const int rb = u % (ROWS / 8), kq = u / (ROWS / 8);   // 8-row block, 4-k quad (16 per tile)
         LongType r = row0 + rb * 8;
         r = r + 8 <= rowLimit ? r : rowLimit - 8;
 #pragma unroll
-        for (int q = 0; q < 8; q++) {
-          const LongType k = k0 + kg * 8 + q;
-          reg[i * 8 + q] = k < K ? *reinterpret_cast<const u32x4*>(base + k * ld + r) : zero;
+        for (int q = 0; q < 4; q++) {
+          const LongType k = k0 + kq * 4 + q;
+          reg[i * 4 + q] = k < K ? *reinterpret_cast<const u32x4*>(base + k * ld + r) : zero;
         }
       }
     }
   }
-  // lds: [8 k-groups][ROWS + 1] slots of 16 bytes
-  __device__ __forceinline__ void store(u32x4* __restrict__ lds, LongType row0, LongType rowLimit, int t) {
-    if (KC) {
+  __device__ __forceinline__ void store(u32x4* __restrict__ lds, int t) {
 #pragma unroll
-      for (int i = 0; i < VECS; i++) {
-        const int v = t + i * NT;
-        if (VECS * NT != ROWS * 8 && v >= ROWS * 8) break;
-        const int kg = v & 7, row = v >> 3;
-        lds[kg * (ROWS + 1) + row] = reg[i];
-      }
-    } else {
+    for (int i = 0; i < PER; i++) {
+      const int u = t + i * NT;
+      if (PER * NT != UNITS && u >= UNITS) break;
+      if (KC) {
+        lds[Layout::slot(u & 7, u >> 3)] = reg[i];
+      } else {
+        const int rb = u % (ROWS / 8), kq = u / (ROWS / 8);
+        // column c of the 4x8 block: k = kq*4 .. +3 of row rb*8 + c -> half (kq & 1) of slot (kq / 2, row).
+        // A block clamped at the tile edge holds values of rows that the epilogue never writes.
 #pragma unroll
-      for (int i = 0; i < BLKS; i++) {
-        const int b = t + i * NT;
-        if (BLKS * NT != ROWS && b >= ROWS) break;
-        const int rb = b % (ROWS / 8), kg = b / (ROWS / 8);
-        u32x4 rows[8], cols[8];
-#pragma unroll
-        for (int q = 0; q < 8; q++) rows[q] = reg[i * 8 + q];
-        transpose8x8(rows, cols);
-        // a block clamped at the edge (row0 + rb*8 + 8 > rowLimit) was loaded from rowLimit-8: it is stored at
-        // its nominal slot; its values belong to rows that the epilogue never writes
-#pragma unroll
-        for (int c = 0; c < 8; c++) lds[kg * (ROWS + 1) + rb * 8 + c] = cols[c];
+        for (int c = 0; c < 8; c++) {
+          const unsigned sel = (c & 1) ? 0x07060302u : 0x05040100u;
+          u32x2 w;
+          w[0] = __builtin_amdgcn_perm(reg[i * 4 + 1][c / 2], reg[i * 4 + 0][c / 2], sel);
+          w[1] = __builtin_amdgcn_perm(reg[i * 4 + 3][c / 2], reg[i * 4 + 2][c / 2], sel);
+          reinterpret_cast<u32x2*>(&lds[Layout::slot(kq >> 1, rb * 8 + c)])[kq & 1] = w;
+        }
       }
     }
   }
