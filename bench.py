@@ -68,7 +68,7 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this backend is built and measured on one GPU; --gpus %d is not supported (no collectives are part of the op path)" % args.gpus)
 
-    from deeplearning4j_amd.executioner import Executioner, IndexReduce, Pairwise, ReduceSame, TransformStrict
+    from deeplearning4j_amd.executioner import Executioner, IndexReduce, Pairwise, ReduceSame, TransformSame, TransformStrict
     from deeplearning4j_amd.ndarray import BFLOAT16, FLOAT32, HALF, NDArray, f32_to_bf16_bits
 
     ex = Executioner()
@@ -135,6 +135,7 @@ def main():
         ex.exec_pairwise(Pairwise.Add, X, Y, S)
         ex.exec_transform_strict(TransformStrict.Tanh, S, T)
         for name, fn, nbytes in [
+            ("copy fp32 [8192,4096] (transform_same Copy; calibrates HBM counters)", lambda: ex.exec_transform_same(TransformSame.Copy, X, S), 2 * 4 * ne),
             ("pairwise_add fp32 [8192,4096]", lambda: ex.exec_pairwise(Pairwise.Add, X, Y, S), 3 * 4 * ne),
             ("transform_tanh fp32 [8192,4096]", lambda: ex.exec_transform_strict(TransformStrict.Tanh, S, T), 2 * 4 * ne),
             ("reduce_sum dim1 fp32 [8192,4096]", lambda: ex.exec_reduce_same(ReduceSame.Sum, T, [1], z=R), 4 * ne + 4 * shp[0]),
