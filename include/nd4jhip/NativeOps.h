@@ -5,8 +5,10 @@
  * libnd4j/include/legacy/NativeOps.h (cited as "ref :line" on each declaration).  The reference
  * exports these with C++ linkage and lets JavaCPP parse the C++ header; here they are `extern "C"`
  * with opaque handle types so that any FFI (JavaCPP, JNI, ctypes) can bind them.  Two consequences:
- *   - the reference's C++ overloads get distinct names here (getOpaqueNDArrayShapeInfoLength,
- *     lc*FromHandle); everything else keeps its name, argument order and meaning;
+ *   - the reference's C++ overload getShapeInfoLength(OpaqueNDArray) gets the distinct name
+ *     getOpaqueNDArrayShapeInfoLength, and of the two lc* overload sets (by value :451-457, by pointer
+ *     :500-512) only the by-value one is exported; everything else keeps its name, argument order and
+ *     meaning;
  *   - handles are plain pointers: OpaqueNDArray = array handle created by createOpaqueNDArray,
  *     OpaqueDataBuffer = host+device buffer pair, OpaqueContext = per-op argument bag.
  *
@@ -105,7 +107,7 @@ ND4JHIP_EXPORT Nd4jPointer lcBlasHandle(OpaqueLaunchContext lc);                
 
 /* ---- data buffers (ref :466-488) ------------------------------------------------------------------- */
 ND4JHIP_EXPORT OpaqueDataBuffer* dbAllocateDataBuffer(Nd4jLong elements, int dataType, bool allocateBoth);        /* ref :487 */
-ND4JHIP_EXPORT OpaqueDataBuffer* allocateDataBuffer(Nd4jLong elements, int dataType, bool allocateBoth);          /* ref :496 */
+ND4JHIP_EXPORT OpaqueDataBuffer* allocateDataBuffer(Nd4jLong elements, int dataType, bool allocateBoth);          /* ref :497 */
 ND4JHIP_EXPORT OpaqueDataBuffer* dbCreateExternalDataBuffer(Nd4jLong elements, int dataType, Nd4jPointer primary, Nd4jPointer special); /* ref :488 */
 ND4JHIP_EXPORT OpaqueDataBuffer* dbCreateView(OpaqueDataBuffer* dataBuffer, Nd4jLong length);                     /* ref :486 */
 ND4JHIP_EXPORT Nd4jPointer dbPrimaryBuffer(OpaqueDataBuffer* dataBuffer);              /* ref :466 */
@@ -203,7 +205,7 @@ ND4JHIP_EXPORT Nd4jLong iArgumentAtNative(OpaqueContext* ptr, int idx);         
 ND4JHIP_EXPORT bool bArgAtNative(OpaqueContext* ptr, int idx);                         /* ref :420 */
 ND4JHIP_EXPORT Nd4jLong dataTypeNativeAt(OpaqueContext* ptr, int idx);                 /* ref :419 */
 ND4JHIP_EXPORT Nd4jStatus execCustomOp2(Nd4jPointer* extraPointers, Nd4jLong hash, OpaqueContext* opContext);  /* ref :370 */
-ND4JHIP_EXPORT OpaqueShapeList* calculateOutputShapes2(Nd4jPointer* extraPointers, Nd4jLong hash, OpaqueContext* context); /* ref :175 */
+ND4JHIP_EXPORT OpaqueShapeList* calculateOutputShapes2(Nd4jPointer* extraPointers, Nd4jLong hash, OpaqueContext* context); /* ref :176 */
 ND4JHIP_EXPORT Nd4jLong getShapeListSize(OpaqueShapeList* list);                       /* ref :177 */
 ND4JHIP_EXPORT const Nd4jLong* getShape(OpaqueShapeList* list, Nd4jLong i);            /* ref :174 */
 ND4JHIP_EXPORT void deleteShapeList(Nd4jPointer shapeList);                            /* ref :386 */
