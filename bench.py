@@ -211,6 +211,54 @@ def main():
             ops.append({"op": "dot_product_attention_v2 %s causal [96,1024,64] (output only)" % dtn, "ms": round(e, 4), "wall_ms": round(w, 4),
                         "roofline": mfma_entry(4.0 * 96 * 1024 * 1024 * 64, e, dtn)})
             del Q, K_, V, O_
+        # config 5: GPT-2-small-shaped greedy decode, bf16, prefill 512 then 128 steps with a key/value cache
+        from deeplearning4j_amd.decoder import Decoder, DecoderConfig, init_weights
+        cfg = DecoderConfig.gpt2_small()
+        weights = init_weights(cfg, 5005)
+        n_param_bytes = 2 * (cfg.n_layer * (cfg.d_model * 3 * cfg.d_model + cfg.d_model * cfg.d_model + 2 * cfg.d_model * cfg.d_ff) + cfg.vocab * cfg.d_model)
+        prefill, n_new = 512, 128
+        for batch in (1, 32):
+            ids = np.random.default_rng(5005).integers(0, cfg.vocab, (batch, prefill))
+            dec = Decoder(cfg, weights, BFLOAT16, batch=batch, executioner=ex)
+            dec.generate(ids[:, :prefill], 4)      # builds and warms the prefill program and the first decode programs
+            for _ in range(2):                     # second pass replays fully built programs
+                dec.reset()
+                L.streamSynchronize(None)
+                t0 = time.perf_counter()
+                dec.forward(ids)
+                L.streamSynchronize(None)
+                t1 = time.perf_counter()
+                for _ in range(n_new - 1):
+                    dec.forward(None)
+                L.streamSynchronize(None)
+                t2 = time.perf_counter()
+            step_ms = (t2 - t1) * 1e3 / (n_new - 1)
+            kv_bytes = cfg.n_layer * 2 * (prefill + n_new / 2) * cfg.d_model * 2 * batch
+            ops.append({"op": "gpt2-small decode bf16 batch %d (prefill %d, %d greedy steps, KV cache)" % (batch, prefill, n_new),
+                        "ms": round(step_ms, 4), "wall_ms": round(step_ms, 4), "tokens_per_s": round(batch * 1e3 / step_ms, 1),
+                        "prefill_ms": round((t1 - t0) * 1e3, 3), "prefill_tokens_per_s": round(batch * prefill / (t1 - t0), 1),
+                        "roofline": hbm_entry(n_param_bytes + kv_bytes, step_ms)})
+            del dec
+        if not args.skip_cpu:
+            # CPU side of config 5 (part of the cpu-baseline leg): the oracle's composition of the same ops, fp32, batch 1,
+            # on a bounded sample (prompt of 32 tokens, 8 greedy steps); its ids are also compared with the HIP fp32 run
+            from oracle import oracle as O
+            from oracle.decoder_oracle import OracleDecoder
+            ids = np.random.default_rng(5005).integers(0, cfg.vocab, (1, 32))
+            cpu = OracleDecoder(cfg, weights, O.FLOAT32, batch=1)
+            nxt = cpu.forward(ids)
+            cpu_ids = [nxt]
+            t0 = time.perf_counter()
+            for _ in range(7):
+                nxt = cpu.forward(nxt.reshape(1, 1))
+                cpu_ids.append(nxt)
+            cpu_step = (time.perf_counter() - t0) / 7
+            dec = Decoder(cfg, weights, FLOAT32, batch=1, executioner=ex)
+            gpu_ids = dec.generate(ids, 8)
+            ops[-2]["cpu_tokens_per_s"] = round(1.0 / cpu_step, 2)
+            ops[-2]["cpu_sample"] = "oracle decoder fp32, batch 1, 7 decode steps after a 32-token prompt, %d threads" % O.get_threads()
+            ops[-2]["fp32_ids_match_cpu"] = bool((gpu_ids == np.stack(cpu_ids, 1)).all())
+            del dec, cpu
         result["ops"] = ops
     print(json.dumps(result))
 

@@ -59,6 +59,7 @@ void launchAttentionLogitsFixup(hipStream_t s, DataType dt, void* logits, const 
 struct FusedArgs {
   LongType Tq, Tv;
   LongType qB, qT, kB, kT, vB, vT, oB, oT;
+  LongType H, qB2, kB2, vB2, oB2;     // second batch level (H = 0: none)
   float scale;
   int applyScale, causal;
   int qTiles;
@@ -86,7 +87,12 @@ __global__ __launch_bounds__(256) void attn_fused(FusedArgs a, const T* __restri
   const int qt = a.qTiles - 1 - (int)(blockIdx.x % a.qTiles);
   const LongType b = blockIdx.x / a.qTiles;
   const LongType q0 = (LongType)qt * BQ;
-  Q += b * a.qB; K += b * a.kB; V += b * a.vB; O += b * a.oB;
+  if (a.H > 0) {
+    const LongType hi = b / a.H, lo = b - hi * a.H;
+    Q += hi * a.qB2 + lo * a.qB; K += hi * a.kB2 + lo * a.kB; V += hi * a.vB2 + lo * a.vB; O += hi * a.oB2 + lo * a.oB;
+  } else {
+    Q += b * a.qB; K += b * a.kB; V += b * a.vB; O += b * a.oB;
+  }
 
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, h = lane >> 5;
   const LongType query = q0 + wave * 32 + (lane & 31);
@@ -222,13 +228,150 @@ __global__ __launch_bounds__(256) void attn_fused(FusedArgs a, const T* __restri
   }
 }
 
+// ---- decode kernel -------------------------------------------------------------------------------------------------
+// A handful of query rows against a long key/value history (Tq <= 8, no causal mask): the work is streaming K and V
+// once, so it runs on the vector ALU with 16-byte loads.  One block per (batch entry, query); a key row is covered by
+// D/8 neighbouring lanes (8 values of d each), so a wave reads 64 / (D/8) whole rows per load instruction.  The dot
+// product is finished with a butterfly over those lanes, which leaves the score in every lane of the key's group --
+// exactly where the P V accumulation needs it.  Each lane group keeps its own running (max, sum, o[8]) state;
+// states are merged across groups (shuffles), across waves (LDS) and normalised once.  Logits go through the same
+// scale / clip / storage-type rounding as in the tile kernel above; probabilities stay in fp32.
+template <typename T, int D, int NW>
+__global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
+                                                       T* __restrict__ O) {
+  constexpr int CH = D / 8;          // lanes per key row
+  constexpr int KPS = 64 / CH;       // key rows per load instruction
+  constexpr int U = 4;               // load instructions in flight per operand
+  __shared__ float sm[NW][D + 2];
+  const LongType b = blockIdx.x, qi = blockIdx.y;
+  if (a.H > 0) {
+    const LongType hi = b / a.H, lo = b - hi * a.H;
+    Q += hi * a.qB2 + lo * a.qB; K += hi * a.kB2 + lo * a.kB; V += hi * a.vB2 + lo * a.vB; O += hi * a.oB2 + lo * a.oB;
+  } else {
+    Q += b * a.qB; K += b * a.kB; V += b * a.vB; O += b * a.oB;
+  }
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int g = lane / CH, c = lane % CH;
+  float q[8];
+  RawIO<T>::unpack(*reinterpret_cast<const typename RawIO<T>::raw*>(Q + qi * a.qT + c * 8), q);
+  const float L2E = 1.44269502162933349609375f;
+  float m = -1.0e30f, l = 0.f, o[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) o[e] = 0.f;
+
+  for (LongType k0 = (LongType)wave * (KPS * U); k0 < a.Tv; k0 += (LongType)NW * (KPS * U)) {
+    typename RawIO<T>::raw kr[U], vr[U];
+    bool valid[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      LongType key = k0 + u * KPS + g;
+      valid[u] = key < a.Tv;
+      key = valid[u] ? key : a.Tv - 1;
+      kr[u] = *reinterpret_cast<const typename RawIO<T>::raw*>(K + key * a.kT + c * 8);
+      vr[u] = *reinterpret_cast<const typename RawIO<T>::raw*>(V + key * a.vT + c * 8);
+    }
+    float sc[U], tmax = m;
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      float kf[8];
+      RawIO<T>::unpack(kr[u], kf);
+      float d = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e++) d = __builtin_fmaf(q[e], kf[e], d);
+#pragma unroll
+      for (int sh = 1; sh < CH; sh <<= 1) d += __shfl_xor(d, sh, WAVE);
+      if (a.applyScale) d *= a.scale;
+      d = __builtin_fminf(__builtin_fmaxf(d, -1.0e4f), 1.0e4f);
+      d = round_storage<T>(d);
+      sc[u] = valid[u] ? d : -1.0e30f;
+      tmax = __builtin_fmaxf(tmax, sc[u]);
+    }
+    const float alpha = __builtin_amdgcn_exp2f((m - tmax) * L2E);
+    m = tmax;
+    l *= alpha;
+#pragma unroll
+    for (int e = 0; e < 8; e++) o[e] *= alpha;
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const float p = valid[u] ? __builtin_amdgcn_exp2f((sc[u] - m) * L2E) : 0.f;
+      float vf[8];
+      RawIO<T>::unpack(vr[u], vf);
+      l += p;
+#pragma unroll
+      for (int e = 0; e < 8; e++) o[e] = __builtin_fmaf(p, vf[e], o[e]);
+    }
+  }
+  // merge the lane groups of the wave (lanes with equal c): bring every state to the common maximum, then add
+  float mAll = m;
+#pragma unroll
+  for (int sh = CH; sh < 64; sh <<= 1) mAll = __builtin_fmaxf(mAll, __shfl_xor(mAll, sh, WAVE));
+  const float f = __builtin_amdgcn_exp2f((m - mAll) * L2E);
+  l *= f;
+#pragma unroll
+  for (int e = 0; e < 8; e++) o[e] *= f;
+#pragma unroll
+  for (int sh = CH; sh < 64; sh <<= 1) {
+    l += __shfl_xor(l, sh, WAVE);
+#pragma unroll
+    for (int e = 0; e < 8; e++) o[e] += __shfl_xor(o[e], sh, WAVE);
+  }
+  if (g == 0) {
+#pragma unroll
+    for (int e = 0; e < 8; e++) sm[wave][c * 8 + e] = o[e];
+    if (c == 0) { sm[wave][D] = mAll; sm[wave][D + 1] = l; }
+  }
+  __syncthreads();
+  if (t < D) {
+    float mm = -1.0e30f;
+#pragma unroll
+    for (int w = 0; w < NW; w++) mm = __builtin_fmaxf(mm, sm[w][D]);
+    float lt = 0.f, ot = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; w++) {
+      const float fw = __builtin_amdgcn_exp2f((sm[w][D] - mm) * L2E);
+      lt = __builtin_fmaf(sm[w][D + 1], fw, lt);
+      ot = __builtin_fmaf(sm[w][t], fw, ot);
+    }
+    O[qi * a.oT + t] = Conv<T>::from(lt > 0.f ? ot / lt : 0.f);
+  }
+}
+
+bool attentionDecodeSupported(DataType dt, const AttnDesc& d) {
+  if (dt != HALF && dt != BFLOAT16) return false;
+  if (d.D != d.Dv || (d.D != 64 && d.D != 128)) return false;
+  if (d.causal || d.Tq < 1 || d.Tq > 8 || d.Tv < 1) return false;
+  for (LongType st : {d.qB, d.qT, d.kB, d.kT, d.vB, d.vT, d.qB2, d.kB2, d.vB2}) if (st % 8 != 0) return false;
+  return d.B < (1LL << 31);
+}
+
+template <typename T, int D>
+static void launchDecodeTyped(hipStream_t s, const void* q, const void* k, const void* v, void* out, const AttnDesc& d) {
+  FusedArgs a;
+  a.Tq = d.Tq; a.Tv = d.Tv;
+  a.qB = d.qB; a.qT = d.qT; a.kB = d.kB; a.kT = d.kT; a.vB = d.vB; a.vT = d.vT; a.oB = d.oB; a.oT = d.oT;
+  a.H = d.H; a.qB2 = d.qB2; a.kB2 = d.kB2; a.vB2 = d.vB2; a.oB2 = d.oB2;
+  a.scale = d.scale; a.applyScale = d.applyScale ? 1 : 0; a.causal = 0; a.qTiles = 1;
+  const dim3 grid((unsigned)d.B, (unsigned)d.Tq);
+  // few (batch, head) rows: more waves per row, so that the history is still spread over many loads in flight
+  if (d.B * d.Tq < 128) hipLaunchKernelGGL((attn_decode<T, D, 16>), grid, dim3(1024), 0, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
+  else hipLaunchKernelGGL((attn_decode<T, D, 4>), grid, dim3(256), 0, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
+}
+
+void launchAttentionDecode(hipStream_t s, DataType dt, const void* q, const void* k, const void* v, void* out, const AttnDesc& d) {
+  ND4J_REQUIRE(attentionDecodeSupported(dt, d), "attention: decode kernel does not take this problem");
+  ND4J_REQUIRE((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) == 0, "attention: operands must be 16-byte aligned");
+  if (dt == HALF) { if (d.D == 64) launchDecodeTyped<f16_t, 64>(s, q, k, v, out, d); else launchDecodeTyped<f16_t, 128>(s, q, k, v, out, d); }
+  else { if (d.D == 64) launchDecodeTyped<bf16_t, 64>(s, q, k, v, out, d); else launchDecodeTyped<bf16_t, 128>(s, q, k, v, out, d); }
+  HIP_CHECK(hipGetLastError());
+}
+
 bool attentionFusedSupported(DataType dt, const AttnDesc& d) {
   if (dt != HALF && dt != BFLOAT16) return false;
   if (d.D != d.Dv || (d.D != 64 && d.D != 128)) return false;
-  if (d.Tq < 1 || d.Tv < 8 || d.Tv % 8 != 0) return false;           // 8x8 blocks of V must not straddle the end
+  if (d.Tq < 1 || d.Tv < 1) return false;
   // 16-byte aligned rows
-  for (LongType st : {d.qB, d.qT, d.kB, d.kT, d.vB, d.vT}) if (st % 8 != 0) return false;
-  if (d.oB % 4 != 0 || d.oT % 4 != 0) return false;
+  for (LongType st : {d.qB, d.qT, d.kB, d.kT, d.vB, d.vT, d.qB2, d.kB2, d.vB2}) if (st % 8 != 0) return false;
+  if (d.oB % 4 != 0 || d.oT % 4 != 0 || d.oB2 % 4 != 0) return false;
   return true;
 }
 
@@ -237,6 +380,7 @@ static void launchFusedTyped(hipStream_t s, const void* q, const void* k, const 
   FusedArgs a;
   a.Tq = d.Tq; a.Tv = d.Tv;
   a.qB = d.qB; a.qT = d.qT; a.kB = d.kB; a.kT = d.kT; a.vB = d.vB; a.vT = d.vT; a.oB = d.oB; a.oT = d.oT;
+  a.H = d.H; a.qB2 = d.qB2; a.kB2 = d.kB2; a.vB2 = d.vB2; a.oB2 = d.oB2;
   a.scale = d.scale; a.applyScale = d.applyScale ? 1 : 0; a.causal = d.causal ? 1 : 0;
   a.qTiles = (int)((d.Tq + 127) / 128);
   constexpr size_t LDS = (size_t)2 * ((D / 64) * TileLayout<64, true>::SLOTS + TileLayout<D, false>::SLOTS) * 16;

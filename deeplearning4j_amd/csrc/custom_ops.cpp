@@ -188,11 +188,17 @@ static void matmulExec(Context& c) {
     launchGemm(stream(), dt, A, B, C, d);
   } else {
     d.batch = bshape[br - 1]; d.aBatch = xb[br - 1]; d.bBatch = yb[br - 1]; d.cBatch = zb[br - 1];
+    int inKernel = 1;   // batch dims resolved inside the kernel; the rest is looped here
+    if (br >= 2 && bshape[br - 2] * bshape[br - 1] < 65536) {
+      d.batchInner = bshape[br - 1]; d.batch = bshape[br - 2] * bshape[br - 1];
+      d.aBatch2 = xb[br - 2]; d.bBatch2 = yb[br - 2]; d.cBatch2 = zb[br - 2];
+      inKernel = 2;
+    }
     LongType outer = 1;
-    for (int i = 0; i < br - 1; i++) outer *= bshape[i];
+    for (int i = 0; i < br - inKernel; i++) outer *= bshape[i];
     for (LongType o = 0; o < outer; o++) {
       LongType idx = o, ao = 0, bo = 0, co = 0;
-      for (int i = br - 2; i >= 0; i--) { LongType q = idx % bshape[i]; idx /= bshape[i]; ao += q * xb[i]; bo += q * yb[i]; co += q * zb[i]; }
+      for (int i = br - inKernel - 1; i >= 0; i--) { LongType q = idx % bshape[i]; idx /= bshape[i]; ao += q * xb[i]; bo += q * yb[i]; co += q * zb[i]; }
       launchGemm(stream(), dt, A + ao * es, B + bo * es, C + co * es, d);
     }
   }
@@ -308,28 +314,38 @@ static void layerNormExec(Context& c) {
 // outputs [out, weights?, logits?].  logits = clip(scale * q k^T, +-1e4) (scale applied unless 0 or 1),
 // masked (j > i) logits get 65504 (bf16) / 1e9 (other types) subtracted, weights = softmax(logits),
 // out = weights v.  With only `out` supplied the fused kernel runs and nothing of size Tq x Tv is written.
-struct AttnViews { NDArray q, k, v, out, w, l; };
-static NDArray as3d(const NDArray* a) {
-  NDArray r = *a;
+// An operand seen as [outer, H, T, D]: rank 2 has no batch, rank 3 one batch level (H = 0), rank >= 4 two levels
+// (the last leading dim is the inner level; the dims before it must fold into one).  The two-level form is what a
+// [batch, heads, T, D] view of a token-major [batch, T, heads * D] buffer needs: its batch dims do not nest.
+struct BatchedView {
+  LongType B = 1, H = 0, T = 0, D = 0;     // B counts all batch entries
+  LongType sB = 0, sB2 = 0, sT = 0, sD = 0;
+};
+static BatchedView batchedView(const NDArray* a, const char* what) {
+  BatchedView r;
   const int rank = a->rankOf();
-  std::vector<LongType> shp, st;
-  if (rank == 2) { shp = {1, a->sizeAt(0), a->sizeAt(1)}; st = {a->sizeAt(0) * a->strideAt(0), a->strideAt(0), a->strideAt(1)}; }
-  else if (rank == 3) return r;
-  else {
-    // rank > 3: fold the leading dims into one batch dim when their strides nest
-    std::vector<LongType> bs, bst;
-    for (int d = 0; d < rank - 2; d++) { bs.push_back(a->sizeAt(d)); bst.push_back(a->strideAt(d)); }
-    LongType* ptr[1] = {bst.data()};
-    int nr = collapseDims((int)bs.size(), bs.data(), ptr, 1);
-    ND4J_REQUIRE(nr == 1, "dot_product_attention_v2: leading dims of a rank-" + std::to_string(rank) + " input do not fold into one batch dim");
-    shp = {bs[0], a->sizeAt(rank - 2), a->sizeAt(rank - 1)}; st = {bst[0], a->strideAt(rank - 2), a->strideAt(rank - 1)};
-  }
-  r.si = makeShapeInfo(a->dataType(), 'c', shp, st.data());
+  ND4J_REQUIRE(rank >= 2, std::string("dot_product_attention_v2: ") + what + " must have rank >= 2");
+  r.T = a->sizeAt(rank - 2); r.D = a->sizeAt(rank - 1); r.sT = a->strideAt(rank - 2); r.sD = a->strideAt(rank - 1);
+  if (rank == 2) { r.B = 1; return r; }
+  if (rank == 3) { r.B = a->sizeAt(0); r.sB = a->strideAt(0); return r; }
+  std::vector<LongType> bs, bst;
+  for (int d = 0; d < rank - 3; d++) { bs.push_back(a->sizeAt(d)); bst.push_back(a->strideAt(d)); }
+  LongType* ptr[1] = {bst.data()};
+  const int nr = collapseDims((int)bs.size(), bs.data(), ptr, 1);
+  ND4J_REQUIRE(nr == 1, std::string("dot_product_attention_v2: leading dims of ") + what + " (rank " + std::to_string(rank) + ") do not fold into [batch, heads]");
+  r.H = a->sizeAt(rank - 3); r.sB = a->strideAt(rank - 3);
+  r.B = bs[0] * r.H; r.sB2 = bs[0] > 1 ? bst[0] : 0;   // a unit outer dim never moves
   return r;
+}
+static bool denseRows(const BatchedView& v) {   // row-major [B, T, D] without gaps
+  if (v.sD != 1 || v.sT != v.D) return false;
+  if (v.H > 0) return v.sB == v.T * v.D && v.sB2 == v.H * v.T * v.D;
+  return v.B == 1 || v.sB == v.T * v.D;
 }
 static void attentionExec(Context& c) {
   ND4J_REQUIRE(c.width() >= 2, "dot_product_attention_v2: queries and values are required");
   NDArray* q0 = c.input(0); NDArray* v0 = c.input(1); NDArray* k0 = c.width() > 2 ? c.input(2) : v0;
+  NDArray* o0 = c.output(0);
   ND4J_REQUIRE(q0->rankOf() == v0->rankOf(), "Queries and values must be same ranks!");
   for (int i = 3; i < c.width(); i++)
     ND4J_REQUIRE(c.inputs[i] == nullptr || c.inputs[i]->isEmpty(), "dot_product_attention_v2: query/value masks are not implemented in nd4j-hip");
@@ -337,61 +353,64 @@ static void attentionExec(Context& c) {
   const double scale = tArg(c, 0, 1.0);
   const bool causal = bArg(c, 0, false), training = bArg(c, 1, false);
   ND4J_REQUIRE(!(training && dropout > 0.0), "dot_product_attention_v2: dropout is not implemented in nd4j-hip");
-  NDArray q = as3d(q0), v = as3d(v0), k = as3d(k0), out = as3d(c.output(0));
+  const BatchedView q = batchedView(q0, "queries"), v = batchedView(v0, "values"), k = batchedView(k0, "keys"), out = batchedView(o0, "output");
   const bool wantW = c.outputs.size() > 1 && c.outputs[1] != nullptr, wantL = c.outputs.size() > 2 && c.outputs[2] != nullptr;
-  DataType dt = q.dataType();
+  DataType dt = q0->dataType();
   ND4J_REQUIRE(isFloatType(dt) && dt != DOUBLE, "dot_product_attention_v2: nd4j-hip implements FLOAT, HALF and BFLOAT16");
-  ND4J_REQUIRE(k.dataType() == dt && v.dataType() == dt && out.dataType() == dt, "dot_product_attention_v2: all arrays must share one data type");
+  ND4J_REQUIRE(k0->dataType() == dt && v0->dataType() == dt && o0->dataType() == dt, "dot_product_attention_v2: all arrays must share one data type");
   AttnDesc d;
-  d.B = q.sizeAt(0); d.Tq = q.sizeAt(1); d.D = q.sizeAt(2); d.Tv = v.sizeAt(1); d.Dv = v.sizeAt(2);
-  ND4J_REQUIRE(k.sizeAt(0) == d.B && v.sizeAt(0) == d.B, "dot_product_attention_v2: batch sizes differ");
-  ND4J_REQUIRE(k.sizeAt(1) == d.Tv && k.sizeAt(2) == d.D, "dot_product_attention_v2: keys must be [batch, Tv, dim], got " + shapeStr(&k));
-  ND4J_REQUIRE(out.sizeAt(0) == d.B && out.sizeAt(1) == d.Tq && out.sizeAt(2) == d.Dv, "dot_product_attention_v2: output must be [batch, Tq, dimV], got " + shapeStr(&out));
+  d.B = q.B; d.H = q.H; d.Tq = q.T; d.D = q.D; d.Tv = v.T; d.Dv = v.D;
+  ND4J_REQUIRE(k.B == d.B && v.B == d.B && k.H == d.H && v.H == d.H, "dot_product_attention_v2: batch sizes differ");
+  ND4J_REQUIRE(k.T == d.Tv && k.D == d.D, "dot_product_attention_v2: keys must be [batch, Tv, dim], got " + shapeStr(k0));
+  ND4J_REQUIRE(out.B == d.B && out.H == d.H && out.T == d.Tq && out.D == d.Dv, "dot_product_attention_v2: output must be [batch, Tq, dimV], got " + shapeStr(o0));
   d.scale = (float)scale; d.applyScale = scale != 0.0 && scale != 1.0; d.causal = causal;
   d.maskValue = dt == BFLOAT16 ? 65504.0f : 1.0e9f;
   std::vector<NDArray*> reads = {q0, v0, k0};
-  std::vector<NDArray*> writes = {c.output(0)};
+  std::vector<NDArray*> writes = {o0};
   if (wantW) writes.push_back(c.outputs[1]);
   if (wantL) writes.push_back(c.outputs[2]);
   if (d.B * d.Tq == 0) return;
   prepareSpecialUse(writes, reads);
-  const bool unitInner = q.strideAt(2) == 1 && k.strideAt(2) == 1 && v.strideAt(2) == 1 && out.strideAt(2) == 1;
-  if (!wantW && !wantL && unitInner && attentionFusedSupported(dt, d)) {
-    d.qB = q.strideAt(0); d.qT = q.strideAt(1); d.kB = k.strideAt(0); d.kT = k.strideAt(1);
-    d.vB = v.strideAt(0); d.vT = v.strideAt(1); d.oB = out.strideAt(0); d.oT = out.strideAt(1);
-    launchAttentionFused(stream(), dt, q.specialBuffer(), k.specialBuffer(), v.specialBuffer(), out.specialBuffer(), d);
+  d.qB = q.sB; d.qT = q.sT; d.kB = k.sB; d.kT = k.sT; d.vB = v.sB; d.vT = v.sT; d.oB = out.sB; d.oT = out.sT;
+  d.qB2 = q.sB2; d.kB2 = k.sB2; d.vB2 = v.sB2; d.oB2 = out.sB2;
+  const bool unitInner = q.sD == 1 && k.sD == 1 && v.sD == 1 && out.sD == 1;
+  if (!wantW && !wantL && unitInner && attentionDecodeSupported(dt, d)) {
+    launchAttentionDecode(stream(), dt, q0->specialBuffer(), k0->specialBuffer(), v0->specialBuffer(), o0->specialBuffer(), d);
+  } else if (!wantW && !wantL && unitInner && attentionFusedSupported(dt, d)) {
+    launchAttentionFused(stream(), dt, q0->specialBuffer(), k0->specialBuffer(), v0->specialBuffer(), o0->specialBuffer(), d);
   } else {
     // composition: logits = q k^T -> fix-up (scale, clip, mask) -> softmax -> out = weights v
-    NDArray logits, weights;
+    const LongType lw = d.Tq * d.Tv;
     std::shared_ptr<DataBuffer> tmpL, tmpW;
-    auto dense = [&](std::shared_ptr<DataBuffer>& hold) {
-      NDArray t;
-      hold = std::make_shared<DataBuffer>((void*)nullptr, (void*)nullptr, (size_t)(d.B * d.Tq * d.Tv) * sizeOf(dt), dt);
+    auto scratch = [&](std::shared_ptr<DataBuffer>& hold) {
+      hold = std::make_shared<DataBuffer>((void*)nullptr, (void*)nullptr, (size_t)(d.B * lw) * sizeOf(dt), dt);
       hold->allocateSpecial();
-      t.buf = hold;
-      t.si = makeShapeInfo(dt, 'c', {d.B, d.Tq, d.Tv});
-      return t;
+      return hold->special;
     };
-    if (wantL) { logits = as3d(c.outputs[2]); ND4J_REQUIRE(logits.sizeAt(0) == d.B && logits.sizeAt(1) == d.Tq && logits.sizeAt(2) == d.Tv && logits.dataType() == dt, "dot_product_attention_v2: logits output must be [batch, Tq, Tv]"); }
-    else logits = dense(tmpL);
-    if (wantW) { weights = as3d(c.outputs[1]); ND4J_REQUIRE(weights.sizeAt(0) == d.B && weights.sizeAt(1) == d.Tq && weights.sizeAt(2) == d.Tv && weights.dataType() == dt, "dot_product_attention_v2: weights output must be [batch, Tq, Tv]"); }
-    else weights = dense(tmpW);
-    ND4J_REQUIRE(logits.strideAt(2) == 1 && logits.strideAt(1) == d.Tv && logits.strideAt(0) == d.Tq * d.Tv, "dot_product_attention_v2: logits output must be dense row-major");
+    auto denseOutput = [&](NDArray* a, const char* what) {
+      const BatchedView b = batchedView(a, what);
+      ND4J_REQUIRE(b.B == d.B && b.T == d.Tq && b.D == d.Tv && a->dataType() == dt && denseRows(b),
+                   std::string("dot_product_attention_v2: ") + what + " output must be a dense row-major [batch, Tq, Tv] array");
+      return a->specialBuffer();
+    };
+    void* logits = wantL ? denseOutput(c.outputs[2], "logits") : scratch(tmpL);
+    void* weights = wantW ? denseOutput(c.outputs[1], "weights") : scratch(tmpW);
     GemmDesc g1;
-    g1.M = d.Tq; g1.N = d.Tv; g1.K = d.D; g1.batch = d.B;
-    g1.aRow = q.strideAt(1); g1.aCol = q.strideAt(2); g1.aBatch = q.strideAt(0);
-    g1.bRow = k.strideAt(2); g1.bCol = k.strideAt(1); g1.bBatch = k.strideAt(0);   // k^T
-    g1.cRow = logits.strideAt(1); g1.cCol = logits.strideAt(2); g1.cBatch = logits.strideAt(0);
-    launchGemm(stream(), dt, q.specialBuffer(), k.specialBuffer(), logits.specialBuffer(), g1);
-    launchAttentionLogitsFixup(stream(), dt, logits.specialBuffer(), d);
-    RowPlan rp = buildRowPlan(logits.shapeInfo(), weights.shapeInfo(), 2);
-    launchSoftmax(stream(), dt, logits.specialBuffer(), weights.specialBuffer(), rp, true);
+    g1.M = d.Tq; g1.N = d.Tv; g1.K = d.D; g1.batch = d.B; g1.batchInner = d.H;
+    g1.aRow = q.sT; g1.aCol = q.sD; g1.aBatch = q.sB; g1.aBatch2 = q.sB2;
+    g1.bRow = k.sD; g1.bCol = k.sT; g1.bBatch = k.sB; g1.bBatch2 = k.sB2;   // k^T
+    g1.cRow = d.Tv; g1.cCol = 1; g1.cBatch = lw; g1.cBatch2 = d.H * lw;
+    launchGemm(stream(), dt, q0->specialBuffer(), k0->specialBuffer(), logits, g1);
+    launchAttentionLogitsFixup(stream(), dt, logits, d);
+    auto si3 = makeShapeInfo(dt, 'c', {d.B, d.Tq, d.Tv});
+    RowPlan rp = buildRowPlan(si3.data(), si3.data(), 2);
+    launchSoftmax(stream(), dt, logits, weights, rp, true);
     GemmDesc g2;
-    g2.M = d.Tq; g2.N = d.Dv; g2.K = d.Tv; g2.batch = d.B;
-    g2.aRow = weights.strideAt(1); g2.aCol = weights.strideAt(2); g2.aBatch = weights.strideAt(0);
-    g2.bRow = v.strideAt(1); g2.bCol = v.strideAt(2); g2.bBatch = v.strideAt(0);
-    g2.cRow = out.strideAt(1); g2.cCol = out.strideAt(2); g2.cBatch = out.strideAt(0);
-    launchGemm(stream(), dt, weights.specialBuffer(), v.specialBuffer(), out.specialBuffer(), g2);
+    g2.M = d.Tq; g2.N = d.Dv; g2.K = d.Tv; g2.batch = d.B; g2.batchInner = d.H;
+    g2.aRow = d.Tv; g2.aCol = 1; g2.aBatch = lw; g2.aBatch2 = d.H * lw;
+    g2.bRow = v.sT; g2.bCol = v.sD; g2.bBatch = v.sB; g2.bBatch2 = v.sB2;
+    g2.cRow = out.sT; g2.cCol = out.sD; g2.cBatch = out.sB; g2.cBatch2 = out.sB2;
+    launchGemm(stream(), dt, weights, v0->specialBuffer(), o0->specialBuffer(), g2);
     if (tmpL || tmpW) HIP_CHECK(hipStreamSynchronize(stream()));  // temporaries are released on return
   }
   registerSpecialUse(writes, reads);

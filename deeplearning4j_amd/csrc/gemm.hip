@@ -27,9 +27,26 @@ struct GemmArgs {
   LongType M, N, K;
   LongType aRow, aCol, bRow, bCol, cRow, cCol;
   LongType aBatch, bBatch, cBatch;
+  LongType batchInner;                 // > 0: batch index = outer * batchInner + inner, outer strides below
+  LongType aBatch2, bBatch2, cBatch2;
   float alpha, beta;
+  // split-K (16-bit MFMA kernel): blockIdx.y owns ktPerSplit K-tiles and parks its partial tile in `partial`;
+  // splitk_finish adds the partials up in split order and writes C
+  int splits;
+  LongType ktPerSplit;
+  float* partial;
 };
+typedef __attribute__((ext_vector_type(4))) float f32x4v;
 
+// operand offsets of batch entry bz (one or two batch levels)
+__device__ __forceinline__ void batchOffsets(const GemmArgs& g, LongType bz, LongType& oa, LongType& ob, LongType& oc) {
+  if (g.batchInner > 0) {
+    const LongType hi = bz / g.batchInner, lo = bz - hi * g.batchInner;
+    oa = hi * g.aBatch2 + lo * g.aBatch; ob = hi * g.bBatch2 + lo * g.bBatch; oc = hi * g.cBatch2 + lo * g.cBatch;
+  } else {
+    oa = bz * g.aBatch; ob = bz * g.bBatch; oc = bz * g.cBatch;
+  }
+}
 
 // ---- fallback --------------------------------------------------------------------------------------------------
 template <typename T>
@@ -39,7 +56,7 @@ __global__ __launch_bounds__(256) void gemm_simple(GemmArgs g, const T* __restri
   __shared__ Acc sa[KS][TS + 1];
   __shared__ Acc sb[KS][TS + 1];
   const LongType bz = blockIdx.z;
-  A += bz * g.aBatch; B += bz * g.bBatch; C += bz * g.cBatch;
+  { LongType oa, ob, oc; batchOffsets(g, bz, oa, ob, oc); A += oa; B += ob; C += oc; }
   const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;  // each thread: 2x2 outputs
   const LongType m0 = (LongType)blockIdx.y * TS, n0 = (LongType)blockIdx.x * TS;
   Acc acc[2][2] = {{0, 0}, {0, 0}};
@@ -108,7 +125,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16(GemmArgs g, const T*
   tileOf(blockIdx.x, gridDim.x, tilesM, tilesN, tm, tn);
   const LongType m0 = (LongType)tm * BM, n0 = (LongType)tn * BN;
   const LongType bz = blockIdx.z;
-  A += bz * g.aBatch; B += bz * g.bBatch; C += bz * g.cBatch;
+  { LongType oa, ob, oc; batchOffsets(g, bz, oa, ob, oc); A += oa; B += ob; C += oc; }
   const LongType lda = A_KC ? g.aRow : g.aCol, ldb = B_KC ? g.bCol : g.bRow;
 
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
@@ -124,16 +141,20 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16(GemmArgs g, const T*
 
   TileLoader<BM, NT, A_KC> la;
   TileLoader<BN, NT, B_KC> lb;
-  const LongType KT = (g.K + BK - 1) / BK;
+  LongType kt0 = 0, KT = (g.K + BK - 1) / BK;
+  if (g.splits > 1) {
+    kt0 = (LongType)blockIdx.y * g.ktPerSplit;
+    KT = kt0 + g.ktPerSplit < KT ? kt0 + g.ktPerSplit : KT;
+  }
 
-  la.load(A, lda, m0, g.M, 0, g.K, t);
-  lb.load(B, ldb, n0, g.N, 0, g.K, t);
+  la.load(A, lda, m0, g.M, kt0 * BK, g.K, t);
+  lb.load(B, ldb, n0, g.N, kt0 * BK, g.K, t);
   la.store(smem, t);
   lb.store(smem + SLOTS_A, t);
   __syncthreads();
 
-  for (LongType kt = 0; kt < KT; kt++) {
-    const int cur = (int)(kt & 1);
+  for (LongType kt = kt0; kt < KT; kt++) {
+    const int cur = (int)((kt - kt0) & 1);
     if (kt + 1 < KT) {
       la.load(A, lda, m0, g.M, (kt + 1) * BK, g.K, t);
       lb.load(B, ldb, n0, g.N, (kt + 1) * BK, g.K, t);
@@ -161,7 +182,28 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16(GemmArgs g, const T*
     __syncthreads();
   }
 
-  // epilogue: lane owns column (lane % 32); register r of a 32x32 tile is row 8*(r/4) + 4*(lane/32) + r%4
+  // lane owns column (lane % 32); register r of a 32x32 tile is row 8*(r/4) + 4*(lane/32) + r%4
+  if (g.splits > 1) {
+    // split-K: park this block's partial tile for splitk_finish.  Layout of one partial tile:
+    // [q-group (i, j, r / 4)][thread][4 floats] -- 16-byte accesses, coalesced over the block.  A q-group holds 4
+    // consecutive rows of one column; groups whose rows all lie beyond M are skipped.
+    constexpr int Q = TM * TN * 4;
+    const LongType tileLinear = (bz * tilesM + tm) * tilesN + tn;
+    f32x4v* const mine = reinterpret_cast<f32x4v*>(g.partial) + (tileLinear * g.splits + blockIdx.y) * (LongType)(Q * NT);
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const int idx = (i * TN + j) * 4 + q;
+          if (m0 + wm * WTM + i * 32 + 8 * q + 4 * (lane >> 5) < g.M && n0 + wn * WTN + j * 32 + (lane & 31) < g.N) {
+            const f32x4v v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+            mine[idx * NT + t] = v;
+          }
+        }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -181,6 +223,44 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16(GemmArgs g, const T*
     }
 }
 
+// Second half of a split-K product: one block per (output tile, q-group), same thread -> element mapping as
+// gemm_mfma16; adds the partial tiles in split order (deterministic), applies alpha / beta and writes C.
+template <typename T, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM * WN * 64) void splitk_finish(GemmArgs g, T* __restrict__ C, unsigned tilesM, unsigned tilesN) {
+  constexpr int NT = WM * WN * 64;
+  constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32, Q = TM * TN * 4;
+  const unsigned tm = blockIdx.x / tilesN, tn = blockIdx.x % tilesN;
+  const LongType m0 = (LongType)tm * BM, n0 = (LongType)tn * BN, bz = blockIdx.z;
+  { LongType oa, ob, oc; batchOffsets(g, bz, oa, ob, oc); C += oc; }
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  const int idx = blockIdx.y, q = idx & 3, j = (idx >> 2) % TN, i = (idx >> 2) / TN;
+  const LongType tileLinear = (bz * tilesM + tm) * tilesN + tn;
+  const LongType col = n0 + wn * WTN + j * 32 + (lane & 31);
+  const LongType row0 = m0 + wm * WTM + i * 32 + 8 * q + 4 * (lane >> 5);
+  if (col >= g.N || row0 >= g.M) return;
+  const f32x4v* src = reinterpret_cast<const f32x4v*>(g.partial) + tileLinear * g.splits * (LongType)(Q * NT) + idx * NT + t;
+  f32x4v tot = {0.f, 0.f, 0.f, 0.f};
+  for (int sp0 = 0; sp0 < g.splits; sp0 += 8) {
+    f32x4v v[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      v[u] = f32x4v{0.f, 0.f, 0.f, 0.f};
+      if (sp0 + u < g.splits) v[u] = src[(LongType)(sp0 + u) * (Q * NT)];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; u++) tot += v[u];
+  }
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    if (row0 + e >= g.M) break;
+    const LongType off = (row0 + e) * g.cRow + col * g.cCol;
+    float v = g.alpha * tot[e];
+    if (g.beta != 0.f) v += g.beta * to_float(C[off]);
+    C[off] = Conv<T>::from(v);
+  }
+}
+
 template <typename T, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16p(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
                                                              unsigned tilesM, unsigned tilesN) {
@@ -196,7 +276,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16p(GemmArgs g, const T
   tileOf(blockIdx.x, gridDim.x, tilesM, tilesN, tm, tn);
   const LongType m0 = (LongType)tm * BM, n0 = (LongType)tn * BN;
   const LongType bz = blockIdx.z;
-  A += bz * g.aBatch; B += bz * g.bBatch; C += bz * g.cBatch;
+  { LongType oa, ob, oc; batchOffsets(g, bz, oa, ob, oc); A += oa; B += ob; C += oc; }
   const LongType lda = A_KC ? g.aRow : g.aCol, ldb = B_KC ? g.bCol : g.bRow;
 
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
@@ -281,27 +361,57 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16p(GemmArgs g, const T
     }
 }
 
+// How many K-splits a launch of BM x BN tiles gets: enough to put about two blocks on every CU when the tiles alone
+// cannot, bounded by the K-tiles there are and the partial-tile scratch.
+template <int BM, int BN>
+static int chooseSplits(const GemmArgs& g, LongType batch, LongType& ktPerSplit) {
+  const LongType tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN) * batch, KT = (g.K + 63) / 64;
+  ktPerSplit = KT;
+  if (tiles >= 192 || KT < 2) return 1;
+  LongType want = (512 + tiles - 1) / tiles;
+  want = want < KT ? want : KT;
+  want = want < 16 ? want : 16;          // one finishing block reads every partial of its tile
+  const LongType cap = (LongType)(LaunchContext::ALLOCATION_BYTES / sizeof(float)) / (tiles * BM * BN);
+  want = want < cap ? want : cap;
+  if (want < 2) return 1;
+  ktPerSplit = (KT + want - 1) / want;
+  return (int)((KT + ktPerSplit - 1) / ktPerSplit);
+}
+
 template <typename T, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC>
-static void launchMfma16Cfg(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C, LongType batch) {
+static void launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void* B, void* C, LongType batch, bool allowSplit = false) {
   constexpr int NT = WM * WN * 64;
   constexpr size_t LDS = (size_t)2 * (TileLayout<BM, A_KC>::SLOTS + TileLayout<BN, B_KC>::SLOTS) * 16;
   static const bool pipelined = getenv("ND4JHIP_GEMM_PIPE") ? atoi(getenv("ND4JHIP_GEMM_PIPE")) != 0 : true;
-  auto kern = pipelined ? gemm_mfma16p<T, BM, BN, WM, WN, A_KC, B_KC> : gemm_mfma16<T, BM, BN, WM, WN, A_KC, B_KC>;
-  static bool attrSet = false;
-  if (!attrSet) {
+  int splits = 1;
+  if (allowSplit) {
+    LongType per = 0;
+    splits = chooseSplits<BM, BN>(g, batch, per);
+    if (splits > 1) {
+      LaunchContext* lc = LaunchContext::defaultContext();
+      g.splits = splits; g.ktPerSplit = per;
+      g.partial = static_cast<float*>(lc->allocationBuffer);
+    }
+  }
+  const bool usePipe = pipelined && splits == 1;   // the split-K epilogue lives in the plain kernel
+  auto kern = usePipe ? gemm_mfma16p<T, BM, BN, WM, WN, A_KC, B_KC> : gemm_mfma16<T, BM, BN, WM, WN, A_KC, B_KC>;
+  static bool attrSet[2] = {false, false};
+  if (!attrSet[usePipe]) {
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS));
-    attrSet = true;
+    attrSet[usePipe] = true;
   }
   const unsigned tilesM = (unsigned)((g.M + BM - 1) / BM), tilesN = (unsigned)((g.N + BN - 1) / BN);
-  hipLaunchKernelGGL(kern, dim3(tilesM * tilesN, 1, (unsigned)batch), dim3(NT), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tilesM, tilesN);
+  hipLaunchKernelGGL(kern, dim3(tilesM * tilesN, (unsigned)splits, (unsigned)batch), dim3(NT), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tilesM, tilesN);
+  if (splits > 1)
+    hipLaunchKernelGGL((splitk_finish<T, BM, BN, WM, WN>), dim3(tilesM * tilesN, (BM / WM / 32) * (BN / WN / 32) * 4, (unsigned)batch), dim3(NT), 0, s, g, (T*)C, tilesM, tilesN);
 }
 
 template <typename T, bool A_KC, bool B_KC>
 static void launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C, LongType batch) {
   const LongType tiles256 = ((g.M + 255) / 256) * ((g.N + 255) / 256) * batch;
   const LongType tiles128 = ((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
-  if (g.M <= 32) return launchMfma16Cfg<T, 32, 128, 1, 4, A_KC, B_KC>(s, g, A, B, C, batch);
-  if (g.M <= 64 || g.N <= 64 || tiles128 < 192) return launchMfma16Cfg<T, 64, 64, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
+  if (g.M <= 32) return launchMfma16Cfg<T, 32, 128, 1, 4, A_KC, B_KC>(s, g, A, B, C, batch, true);
+  if (g.M <= 64 || g.N <= 64 || tiles128 < 192) return launchMfma16Cfg<T, 64, 64, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch, true);
   if (tiles256 < 192) return launchMfma16Cfg<T, 128, 128, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
   static const int cfg = getenv("ND4JHIP_GEMM_CFG") ? atoi(getenv("ND4JHIP_GEMM_CFG")) : 0;
   if (cfg == 1) return launchMfma16Cfg<T, 256, 256, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
@@ -324,7 +434,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32(GemmArgs g, const fl
   tileOf(blockIdx.x, gridDim.x, tilesM, tilesN, tm, tn);
   const LongType m0 = (LongType)tm * BM, n0 = (LongType)tn * BN;
   const LongType bz = blockIdx.z;
-  A += bz * g.aBatch; B += bz * g.bBatch; C += bz * g.cBatch;
+  { LongType oa, ob, oc; batchOffsets(g, bz, oa, ob, oc); A += oa; B += ob; C += oc; }
   const LongType lda = A_KC ? g.aRow : g.aCol, ldb = B_KC ? g.bCol : g.bRow;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wm = wave / WN, wn = wave % WN;
   typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -552,7 +662,9 @@ static GemmArgs toArgs(const GemmDesc& d) {
   g.M = d.M; g.N = d.N; g.K = d.K;
   g.aRow = d.aRow; g.aCol = d.aCol; g.bRow = d.bRow; g.bCol = d.bCol; g.cRow = d.cRow; g.cCol = d.cCol;
   g.aBatch = d.aBatch; g.bBatch = d.bBatch; g.cBatch = d.cBatch;
+  g.batchInner = d.batchInner; g.aBatch2 = d.aBatch2; g.bBatch2 = d.bBatch2; g.cBatch2 = d.cBatch2;
   g.alpha = d.alpha; g.beta = d.beta;
+  g.splits = 1; g.ktPerSplit = 0; g.partial = nullptr;
   return g;
 }
 
@@ -569,6 +681,7 @@ static bool mfmaEligible(const GemmDesc& d, const void* A, const void* B, size_t
   if (d.M < 1 || d.N < 1 || d.K < 1) return false;
   if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) return false;
   if (d.batch > 1 && (d.aBatch % V || d.bBatch % V)) return false;
+  if (d.batchInner > 0 && (d.aBatch2 % V || d.bBatch2 % V)) return false;
   if (d.aCol == 1 && d.K % V == 0 && d.aRow % V == 0) aKC = true;
   else if (d.aRow == 1 && d.M % V == 0 && d.M >= V && d.aCol % V == 0) aKC = false;
   else return false;
@@ -581,9 +694,13 @@ static bool mfmaEligible(const GemmDesc& d, const void* A, const void* B, size_t
 
 template <typename T>
 static void dispatch16(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
-  if (tryGemv<T>(s, d, A, B, C)) return;
   bool aKC = false, bKC = false;
-  if (d.M * d.N >= 1024 && d.K >= 32 && mfmaEligible(d, A, B, sizeof(T), aKC, bKC)) {
+  const bool eligible = (d.M * d.N >= 1024 || (d.M == 1 && d.N >= 64)) && d.K >= 32 && mfmaEligible(d, A, B, sizeof(T), aKC, bKC);
+  // x[1, K] times row-major W[K, N]: the split-K tile kernel streams W with far more loads in flight than the
+  // column-sum GEMV (the unused 31 rows of the MFMA tile cost nothing here)
+  const bool rowTimesRowMajor = d.M == 1 && eligible && aKC && !bKC && d.batch == 1;
+  if (!rowTimesRowMajor && tryGemv<T>(s, d, A, B, C)) return;
+  if (eligible) {
     GemmArgs g = toArgs(d);
     if (aKC && bKC) return launchMfma16<T, true, true>(s, g, A, B, C, d.batch);
     if (aKC && !bKC) return launchMfma16<T, true, false>(s, g, A, B, C, d.batch);

@@ -95,14 +95,20 @@ struct GemmDesc {
   LongType bRow = 0, bCol = 0;   // element strides of op(B)[k][n]
   LongType cRow = 0, cCol = 0;
   LongType aBatch = 0, bBatch = 0, cBatch = 0;
+  // optional second batch level: entry i of `batch` = (i / batchInner, i % batchInner), the outer index moving
+  // by the *Batch2 strides (batchInner = 0: one level)
+  LongType batchInner = 0, aBatch2 = 0, bBatch2 = 0, cBatch2 = 0;
   float alpha = 1.f, beta = 0.f;
 };
 void launchGemm(hipStream_t s, DataType dt, const void* A, const void* B, void* C, const GemmDesc& d);
 
 // ---- attention -------------------------------------------------------------------------------------
 struct AttnDesc {
-  LongType B = 0, Tq = 0, Tv = 0, D = 0, Dv = 0;
+  LongType B = 0, Tq = 0, Tv = 0, D = 0, Dv = 0;   // B counts all batch entries (outer x H)
   LongType qB = 0, qT = 0, kB = 0, kT = 0, vB = 0, vT = 0, oB = 0, oT = 0;  // innermost stride is 1
+  // optional second batch level (e.g. [batch, heads, T, D] views of token-major buffers): entry i of B is
+  // (i / H, i % H); *B strides move the inner (head) index, *B2 the outer one.  H = 0: one level.
+  LongType H = 0, qB2 = 0, kB2 = 0, vB2 = 0, oB2 = 0;
   float scale = 1.f;
   bool applyScale = false;
   bool causal = false;
@@ -112,6 +118,10 @@ struct AttnDesc {
 bool attentionFusedSupported(DataType dt, const AttnDesc& d);
 void launchAttentionFused(hipStream_t s, DataType dt, const void* q, const void* k, const void* v, void* out,
                           const AttnDesc& d);
+// a few query rows against a long history, no causal mask (decode steps with a key/value cache)
+bool attentionDecodeSupported(DataType dt, const AttnDesc& d);
+void launchAttentionDecode(hipStream_t s, DataType dt, const void* q, const void* k, const void* v, void* out,
+                           const AttnDesc& d);
 // logits[b,i,j] = clip(scale * logits, +-1e4) - mask  (in place, row-major [B,Tq,Tv])
 void launchAttentionLogitsFixup(hipStream_t s, DataType dt, void* logits, const AttnDesc& d);
 

@@ -102,6 +102,33 @@ def test_matmul_vs_oracle(ex, oracle, dtype, tol, M, N, K):
     assert_close(ga, _f(oz), tol, tol, "matmul transposeA")
 
 
+@pytest.mark.parametrize("dtype", [HALF, BFLOAT16])
+@pytest.mark.parametrize("M,N,K", [(1, 2304, 768), (5, 768, 3072), (32, 3072, 768), (48, 200, 1024), (64, 64, 4096)])
+def test_matmul_small_m_split_k(ex, oracle, dtype, M, N, K):
+    """Skinny products take the split-K path (partial tiles + arrival tickets); run it repeatedly, so that tickets left
+    over by one launch would show in the next, and with alpha/beta so the last-arriving block's epilogue is covered."""
+    rng = np.random.default_rng(M * 7 + N + K)
+    a = rng.normal(0, 1 / math.sqrt(K), (M, K))
+    b = rng.normal(0, 1 / math.sqrt(K), (K, N))
+    c0 = rng.normal(0, 1, (M, N))
+    oa, da = _pair(oracle, a, dtype)
+    ob, db = _pair(oracle, b, dtype)
+    oz, dz = _pair(oracle, c0, dtype)
+    oracle.matmul(oa, ob, oz, alpha=0.5, beta=2.0, accumulate=1)
+    for rep in range(3):
+        _, dz = _pair(oracle, c0, dtype)
+        ex.exec_custom("matmul", [da, db], [dz], t_args=[0.5, 2.0])
+        assert_close(dz.to_float(), _f(oz), 1e-2, 1e-2, "split-K repeat %d" % rep)
+    # many launches back to back on one output, read once
+    outs = [NDArray.empty((M, N), dtype) for _ in range(8)]
+    for o in outs:
+        ex.exec_custom("matmul", [da, db], [o])
+    oz1 = _ozeros(oracle, (M, N), dtype)
+    oracle.matmul(oa, ob, oz1, accumulate=1)
+    for o in outs:
+        assert_close(o.to_float(), _f(oz1), 1e-2, 1e-2, "split-K back to back")
+
+
 @pytest.mark.parametrize("dtype,tol", [(FLOAT32, 1e-4), (BFLOAT16, 1e-2)])
 def test_matmul_batched_alpha_beta_views(ex, oracle, dtype, tol):
     rng = np.random.default_rng(21)
@@ -273,6 +300,56 @@ def test_attention_rank4_and_default_keys(ex, oracle):
     out = ex.exec_custom("dot_product_attention_v2", [NDArray.from_numpy(q), NDArray.from_numpy(v)], [NDArray.empty((B, H, T, D), FLOAT32)],
                          t_args=[0.125], b_args=[True])[0]
     assert_close(out.to_numpy().reshape(B * H, T, D), oo, 1e-4, 1e-4, "rank 4, keys = values")
+
+
+@pytest.mark.parametrize("dtype,tol", [(FLOAT32, 1e-4), (BFLOAT16, 1e-2), (HALF, 1e-2)])
+@pytest.mark.parametrize("Tq,Tv,causal", [(40, 40, True), (1, 37, False), (5, 131, False)])
+def test_attention_token_major_head_views(ex, oracle, dtype, tol, Tq, Tv, causal):
+    """[batch, heads, T, 64] views of token-major buffers: the batch dims do not nest, key counts are ragged, the
+    output is written through a strided view (the layout of a decoder's fused qkv buffer and its key/value cache)."""
+    rng = np.random.default_rng(Tq * 1000 + Tv)
+    B, H, D, M = 2, 3, 64, 160
+    d = H * D
+    qkv = rng.normal(0, 1, (B, Tq, 3 * d)).astype(np.float32)
+    kc = rng.normal(0, 1, (B, M, d)).astype(np.float32)
+    vc = rng.normal(0, 1, (B, M, d)).astype(np.float32)
+    oqkv, dqkv = _pair(oracle, qkv, dtype)
+    okc, dkc = _pair(oracle, kc, dtype)
+    ovc, dvc = _pair(oracle, vc, dtype)
+    want = _ozeros(oracle, (B, Tq, H, D), dtype)
+    for b in range(B):
+        q3 = oqkv.a[b].reshape(Tq, 3, H, D)[:, 0].transpose(1, 0, 2)
+        k3 = okc.a[b, :Tv].reshape(Tv, H, D).transpose(1, 0, 2)
+        v3 = ovc.a[b, :Tv].reshape(Tv, H, D).transpose(1, 0, 2)
+        oracle.attention_v2(oracle.Arr(q3, oqkv.dt), oracle.Arr(v3, oqkv.dt), oracle.Arr(k3, oqkv.dt),
+                            oracle.Arr(want.a[b].transpose(1, 0, 2), oqkv.dt), scale=0.125, causal=causal)
+    q4 = dqkv.view((B, H, Tq, D), (Tq * 3 * d, D, 3 * d, 1), 0)
+    k4 = dkc.view((B, H, Tv, D), (M * d, D, d, 1), 0)
+    v4 = dvc.view((B, H, Tv, D), (M * d, D, d, 1), 0)
+    att = NDArray.empty((B, Tq, d), dtype)
+    o4 = att.view((B, H, Tq, D), (Tq * d, D, d, 1), 0)
+    ex.exec_custom("dot_product_attention_v2", [q4, v4, k4], [o4], t_args=[0.125, 0.0], b_args=[causal, False])
+    assert_close(att.to_float().reshape(B, Tq, H, D), _f(want), tol, tol, "token-major heads")
+
+
+@pytest.mark.parametrize("dtype,tol", [(FLOAT32, 1e-4), (BFLOAT16, 1e-2)])
+def test_matmul_batch_dims_that_do_not_nest(ex, oracle, dtype, tol):
+    """x is a [B, H, T, D] view of a token-major buffer (strides of B and H do not fold), y is dense [B, H, D, N]."""
+    rng = np.random.default_rng(73)
+    B, H, T, D, Nn = 3, 4, 40, 64, 48
+    xa = rng.normal(0, 1, (B, T, H * D)).astype(np.float32)
+    ya = rng.normal(0, 0.2, (B, H, D, Nn)).astype(np.float32)
+    ox, dx = _pair(oracle, xa, dtype)
+    oy, dy = _pair(oracle, ya, dtype)
+    want = _ozeros(oracle, (B, H, T, Nn), dtype)
+    for b in range(B):
+        for h in range(H):
+            x2 = ox.a[b].reshape(T, H, D)[:, h]
+            oracle.matmul(oracle.Arr(x2, ox.dt), oracle.Arr(oy.a[b, h], ox.dt), oracle.Arr(want.a[b, h], ox.dt))
+    x4 = dx.view((B, H, T, D), (T * H * D, D, H * D, 1), 0)
+    z = ex.exec_custom("matmul", [x4, dy])[0]
+    assert z.shape == (B, H, T, Nn)
+    assert_close(z.to_float(), _f(want), tol, tol, "two batch levels")
 
 
 # ---- argmax + glue ops -----------------------------------------------------------------------------------------------
