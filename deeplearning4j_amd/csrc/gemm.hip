@@ -361,6 +361,165 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16p(GemmArgs g, const T
     }
 }
 
+// Steady-state kernel for problems made of whole tiles (M % BM == 0, N % BN == 0, K % 64 == 0): no bounds handling,
+// so the K loop is one basic block and the instruction order below is the order the hardware sees.  A wave issues
+// in order, and an MFMA 32x32x16 keeps the matrix pipe busy for 32 cycles: every LDS / global instruction is placed
+// between two MFMAs, so that its issue and its latency sit in the shadow of matrix work.
+//   k-steps 0..2: fragments of the following step <- LDS                                    | 8 MFMAs each
+//   k-step 3    : registers holding K-tile kt+1 -> other LDS stage                           | 4 MFMAs
+//                 barrier; fragments of step 0 of tile kt+1 <- LDS; global loads of tile kt+2 | 4 MFMAs
+// Global loads therefore stay in flight for a whole K-tile (about 2000 cycles) before they are needed.
+template <typename T, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16f(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
+                                                             unsigned tilesM, unsigned tilesN) {
+  constexpr int BK = 64, NT = WM * WN * 64;
+  constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32, NF = TM + TN, NM = TM * TN;
+  using LayA = TileLayout<BM, A_KC>;
+  using LayB = TileLayout<BN, B_KC>;
+  constexpr int SLOTS_A = LayA::SLOTS, SLOTS_B = LayB::SLOTS, STAGE = SLOTS_A + SLOTS_B;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  u32x4* smem = reinterpret_cast<u32x4*>(smem_raw);
+
+  unsigned tm, tn;
+  tileOf(blockIdx.x, gridDim.x, tilesM, tilesN, tm, tn);
+  const LongType m0 = (LongType)tm * BM, n0 = (LongType)tn * BN;
+  const LongType bz = blockIdx.z;
+  { LongType oa, ob, oc; batchOffsets(g, bz, oa, ob, oc); A += oa; B += ob; C += oc; }
+  const LongType lda = A_KC ? g.aRow : g.aCol, ldb = B_KC ? g.bCol : g.bRow;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+  TileLoader<BM, NT, A_KC> la;
+  TileLoader<BN, NT, B_KC> lb;
+  const LongType KT = g.K / BK;
+  u32x4 fa[2][TM], fb[2][TN];
+  // lane's fragment slots inside a stage, per k-step parity of (lane >> 5)
+  int offA[TM], offB[TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++) offA[i] = LayA::slot(lane >> 5, wm * WTM + i * 32 + (lane & 31));
+#pragma unroll
+  for (int j = 0; j < TN; j++) offB[j] = SLOTS_A + LayB::slot(lane >> 5, wn * WTN + j * 32 + (lane & 31));
+  auto readFrag = [&](const u32x4* stage, int ks, int buf) {
+#pragma unroll
+    for (int i = 0; i < TM; i++) fa[buf][i] = stage[offA[i] + ks * 2 * LayA::GROUP];
+#pragma unroll
+    for (int j = 0; j < TN; j++) fb[buf][j] = stage[offB[j] + ks * 2 * LayB::GROUP];
+  };
+  auto mfmas = [&](int buf, int from, int to) {
+#pragma unroll
+    for (int idx = from; idx < to; idx++) {
+      const int i = idx / TN, j = idx % TN;
+      acc[i][j] = Mfma16<T>::mma(fa[buf][i], fb[buf][j], acc[i][j]);
+    }
+  };
+
+  la.loadFull(A, lda, m0, 0, t);
+  lb.loadFull(B, ldb, n0, 0, t);
+  la.store(smem, t);
+  lb.store(smem + SLOTS_A, t);
+  la.loadFull(A, lda, m0, BK, t);        // K-tile 1 waits in registers (K >= 2 tiles)
+  lb.loadFull(B, ldb, n0, BK, t);
+  __syncthreads();
+  readFrag(smem, 0, 0);
+
+  for (LongType kt = 0; kt + 1 < KT; kt++) {
+    const u32x4* cur = smem + (kt & 1) * STAGE;
+    u32x4* nxt = smem + ((kt + 1) & 1) * STAGE;
+    const LongType kAhead = (kt + 2 < KT ? kt + 2 : KT - 1) * BK;   // the last round fetches a tile nobody uses
+    // k-step 0
+    readFrag(cur, 1, 1);
+    mfmas(0, 0, NM);
+#pragma unroll
+    for (int q = 0; q < NM; q++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // k-step 1
+    readFrag(cur, 2, 0);
+    mfmas(1, 0, NM);
+#pragma unroll
+    for (int q = 0; q < NM; q++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // k-step 2
+    readFrag(cur, 3, 1);
+    mfmas(0, 0, NM);
+#pragma unroll
+    for (int q = 0; q < NM; q++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // k-step 3, first half: the registers (K-tile kt + 1, in flight for a whole tile) go to the other stage
+    la.store(nxt, t);
+    lb.store(nxt + SLOTS_A, t);
+    mfmas(1, 0, NM / 2);
+#pragma unroll
+    for (int q = 0; q < NM / 2; q++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);   // the transposing store's permutes
+      __builtin_amdgcn_sched_group_barrier(0x200, 4, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    // second half: first fragments of the next tile, global loads of the tile after it
+    readFrag(nxt, 0, 0);
+    la.loadFull(A, lda, m0, kAhead, t);
+    lb.loadFull(B, ldb, n0, kAhead, t);
+    mfmas(1, NM / 2, NM);
+#pragma unroll
+    for (int q = 0; q < NM / 2; q++) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  {
+    // last K-tile: nothing left to fetch
+    const u32x4* cur = smem + ((KT - 1) & 1) * STAGE;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ks++) {
+      if (ks + 1 < BK / 16) readFrag(cur, ks + 1, (ks + 1) & 1);
+      mfmas(ks & 1, 0, NM);
+#pragma unroll
+      for (int q = 0; q < NM; q++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+  // epilogue: lane owns column (lane % 32); register r of a 32x32 tile is row 8*(r/4) + 4*(lane/32) + r%4
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const LongType col = n0 + wn * WTN + j * 32 + (lane & 31);
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const LongType row = m0 + wm * WTM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r & 3);
+        const LongType off = row * g.cRow + col * g.cCol;
+        float v = g.alpha * acc[i][j][r];
+        if (g.beta != 0.f) v += g.beta * to_float(C[off]);
+        C[off] = Conv<T>::from(v);
+      }
+    }
+}
+
 // How many K-splits a launch of BM x BN tiles gets: enough to put about two blocks on every CU when the tiles alone
 // cannot, bounded by the K-tiles there are and the partial-tile scratch.
 template <int BM, int BN>
@@ -394,11 +553,16 @@ static void launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
     }
   }
   const bool usePipe = pipelined && splits == 1;   // the split-K epilogue lives in the plain kernel
-  auto kern = usePipe ? gemm_mfma16p<T, BM, BN, WM, WN, A_KC, B_KC> : gemm_mfma16<T, BM, BN, WM, WN, A_KC, B_KC>;
-  static bool attrSet[2] = {false, false};
-  if (!attrSet[usePipe]) {
+  // whole tiles only: the kernel without bounds handling (its K loop needs two K-tiles at least)
+  static const bool fullAllowed = getenv("ND4JHIP_GEMM_FULL") ? atoi(getenv("ND4JHIP_GEMM_FULL")) != 0 : true;
+  const bool useFull = usePipe && fullAllowed && BM * BN >= 128 * 128 && g.M % BM == 0 && g.N % BN == 0 && g.K % 64 == 0 && g.K >= 128;
+  auto kern = useFull ? gemm_mfma16f<T, BM, BN, WM, WN, A_KC, B_KC>
+                      : usePipe ? gemm_mfma16p<T, BM, BN, WM, WN, A_KC, B_KC> : gemm_mfma16<T, BM, BN, WM, WN, A_KC, B_KC>;
+  const int which = useFull ? 2 : usePipe ? 1 : 0;
+  static bool attrSet[3] = {false, false, false};
+  if (!attrSet[which]) {
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS));
-    attrSet[usePipe] = true;
+    attrSet[which] = true;
   }
   const unsigned tilesM = (unsigned)((g.M + BM - 1) / BM), tilesN = (unsigned)((g.N + BN - 1) / BN);
   hipLaunchKernelGGL(kern, dim3(tilesM * tilesN, (unsigned)splits, (unsigned)batch), dim3(NT), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tilesM, tilesN);

@@ -37,16 +37,17 @@ __device__ __forceinline__ void transpose8x8(const u32x4 (&r)[8], u32x4 (&out)[8
 //   KC = true : memory is [row][k] with unit k stride; ld = row pitch.  16-byte vectors (8 k of one row) are
 //               copied as they are.  LDS slot of (k-group kg, row r): kg * (ROWS + 1) + r.
 //   KC = false: memory is [k][row] with unit row stride; ld = k pitch.  A thread loads a 4 (k) x 8 (rows) block,
-//               transposes it in registers and writes eight 8-byte half-slots.  Rows are permuted inside a
-//               k-group, slot = kg * (ROWS + 8) + (r % 8) * (ROWS / 8 + 1) + r / 8, so that the writes of one
-//               instruction (fixed r % 8, neighbouring lanes = neighbouring r / 8) land in consecutive slots and
-//               the fragment reads (32 consecutive rows) stay spread over the banks.
+//               transposes it in registers and writes eight 8-byte half-slots; neighbouring lanes hold the two
+//               k-quads of one k-group, so a lane pair fills whole slots.  Rows are swizzled inside aligned groups
+//               of 16, slot = kg * GROUP + (r ^ ((r >> 4) & 7)): the fragment reads (16 consecutive rows per
+//               LDS pass) still cover 16 consecutive slots, and the writes of one instruction (fixed r % 8, lane
+//               pairs = consecutive r / 8) land in 16 different slots modulo 16 -- both free of bank conflicts.
 template <int ROWS, bool KC>
 struct TileLayout {
   static constexpr int GROUP = KC ? ROWS + 1 : ROWS + 8;   // slots per k-group
   static constexpr int SLOTS = 8 * GROUP;                  // slots per 64-k tile
   static __device__ __forceinline__ int slot(int kg, int r) {
-    return KC ? kg * GROUP + r : kg * GROUP + (r & 7) * (ROWS / 8 + 1) + (r >> 3);
+    return KC ? kg * GROUP + r : kg * GROUP + (r ^ ((r >> 4) & 7));
   }
 };
 
@@ -72,7 +73,7 @@ struct TileLoader {
         const LongType k = k0 + kg * 8;
         reg[i] = k < K ? *reinterpret_cast<const u32x4*>(base + r * ld + k) : zero;
       } else {
-        const int rb = u % (ROWS / 8), kq = u / (ROWS / 8);   // 8-row block, 4-k quad (16 per tile)
+        const int rb = (u >> 1) % (ROWS / 8), kq = (u / (ROWS / 4)) * 2 + (u & 1);   // 8-row block, 4-k quad (16 per tile)
         LongType r = row0 + rb * 8;
         r = r + 8 <= rowLimit ? r : rowLimit - 8;
 #pragma unroll
@@ -80,6 +81,22 @@ struct TileLoader {
           const LongType k = k0 + kq * 4 + q;
           reg[i * 4 + q] = k < K ? *reinterpret_cast<const u32x4*>(base + k * ld + r) : zero;
         }
+      }
+    }
+  }
+  // same as load() for a tile that lies wholly inside the operand: no clamping, no predicates
+  template <typename T>
+  __device__ __forceinline__ void loadFull(const T* __restrict__ base, LongType ld, LongType row0, LongType k0, int t) {
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      const int u = t + i * NT;
+      if (PER * NT != UNITS && u >= UNITS) break;
+      if (KC) {
+        reg[i] = *reinterpret_cast<const u32x4*>(base + (row0 + (u >> 3)) * ld + k0 + (u & 7) * 8);
+      } else {
+        const int rb = (u >> 1) % (ROWS / 8), kq = (u / (ROWS / 4)) * 2 + (u & 1);
+#pragma unroll
+        for (int q = 0; q < 4; q++) reg[i * 4 + q] = *reinterpret_cast<const u32x4*>(base + (k0 + kq * 4 + q) * ld + row0 + rb * 8);
       }
     }
   }
@@ -91,7 +108,7 @@ struct TileLoader {
       if (KC) {
         lds[Layout::slot(u & 7, u >> 3)] = reg[i];
       } else {
-        const int rb = u % (ROWS / 8), kq = u / (ROWS / 8);
+        const int rb = (u >> 1) % (ROWS / 8), kq = (u / (ROWS / 4)) * 2 + (u & 1);
         // column c of the 4x8 block: k = kq*4 .. +3 of row rb*8 + c -> half (kq & 1) of slot (kq / 2, row).
         // A block clamped at the tile edge holds values of rows that the epilogue never writes.
 #pragma unroll
