@@ -96,20 +96,45 @@ __global__ __launch_bounds__(256) void softmax_rows(RowArgs a, const T* __restri
       vals[i] = e0 < L ? (A)to_float(x[xb + e0 * a.xInner]) : NEG;
     }
   }
-  A mx = NEG;
+  A mx = NEG, sum = (A)0;
+  // Rows of finite numbers (all of them, in practice) need neither the finite-only maximum nor the +-88 clamps:
+  // below -88 the clamp would put e^-88 = 6e-39 where this path puts a smaller number or 0, far below what the
+  // output type or the sum can resolve.  0 * v is NaN exactly for v = +-inf or NaN, which makes a one-instruction
+  // probe; padding slots hold -FLT_MAX and contribute exp2(-inf) = 0 without a bounds test.
+  bool fast = false;
+  if (TPR == 64 && sizeof(A) == 4) {
+    A probe = (A)0;
 #pragma unroll
-  for (int i = 0; i < NV * VEC; i++) {
-    mx = softmax_maxstep<A>(mx, vals[i], clamp);
+    for (int i = 0; i < NV * VEC; i++) {
+      probe = __builtin_fmaf((float)vals[i], 0.f, (float)probe);
+      mx = vals[i] > mx ? vals[i] : mx;
+    }
+    fast = __builtin_amdgcn_ballot_w64(probe != probe) == 0;
   }
-  mx = row_allreduce<MaxOp, TPR, A>(mx, lds);
-  if (clamp && mx == NEG) mx = (A)0;
-  A sum = (A)0;
+  if (fast) {
+    mx = row_allreduce<MaxOp, TPR, A>(mx, lds);
+    const float L2E = 1.44269502162933349609375f;
 #pragma unroll
-  for (int i = 0; i < NV; i++) {
-    const LongType e0 = ((LongType)t + (LongType)i * TPR) * VEC;
+    for (int i = 0; i < NV * VEC; i++) {
+      const A r = (A)__builtin_amdgcn_exp2f(((float)vals[i] - (float)mx) * L2E);
+      vals[i] = r;
+      sum += r;
+    }
+  } else {
+    mx = NEG;
 #pragma unroll
-    for (int e = 0; e < VEC; e++) {
-      if (e0 + e < L) { A r = softmax_term(vals[i * VEC + e], mx, clamp); vals[i * VEC + e] = r; sum += r; }
+    for (int i = 0; i < NV * VEC; i++) {
+      mx = softmax_maxstep<A>(mx, vals[i], clamp);
+    }
+    mx = row_allreduce<MaxOp, TPR, A>(mx, lds);
+    if (clamp && mx == NEG) mx = (A)0;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      const LongType e0 = ((LongType)t + (LongType)i * TPR) * VEC;
+#pragma unroll
+      for (int e = 0; e < VEC; e++) {
+        if (e0 + e < L) { A r = softmax_term(vals[i * VEC + e], mx, clamp); vals[i * VEC + e] = r; sum += r; }
+      }
     }
   }
   sum = row_allreduce<SumOp, TPR, A>(sum, lds);
@@ -307,6 +332,73 @@ __global__ __launch_bounds__(256) void layernorm_rows(RowArgs a, const T* __rest
   }
 }
 
+// One wave per row for rows at a constant pitch (the usual case: a dense or row-strided matrix), vector path only.
+// No shape walk and no predicated loads: every lane issues its x / gain / bias vectors at once (lanes past the row's
+// end re-read the last vector and are masked out of the sums), so the three latencies overlap instead of queueing.
+template <typename T, int NV, bool HAS_BIAS>
+__global__ __launch_bounds__(256) void layernorm_linear(const T* __restrict__ x, const T* __restrict__ gain, const T* __restrict__ bias,
+                                                        T* __restrict__ z, LongType rows, int L, LongType xPitch, LongType zPitch, float eps) {
+  using A = typename Conv<T>::acc;
+  using Raw = typename RawIO<T>::raw;
+  constexpr int VEC = RawIO<T>::N;
+  const int t = threadIdx.x & 63;
+  const LongType row = (LongType)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const T* xr = x + row * xPitch;
+  int e0[NV];
+  A keep[NV];
+  Raw xv[NV], gv[NV], bv[NV];
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const int e = (t + i * 64) * VEC;
+    keep[i] = e < L ? (A)1 : (A)0;
+    e0[i] = e < L ? e : L - VEC;
+    xv[i] = *reinterpret_cast<const Raw*>(xr + e0[i]);
+  }
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    gv[i] = *reinterpret_cast<const Raw*>(gain + e0[i]);
+    if (HAS_BIAS) bv[i] = *reinterpret_cast<const Raw*>(bias + e0[i]);
+  }
+  A vals[NV * VEC];
+  A sum = (A)0;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    RawIO<T>::unpack(xv[i], &vals[i * VEC]);
+    A part = (A)0;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) part += vals[i * VEC + e];
+    sum += part * keep[i];
+  }
+  sum = wave_allreduce<SumOp>(sum);
+  const A mean = sum / (A)L;
+  A sq = (A)0;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    A part = (A)0;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) { const A d = vals[i * VEC + e] - mean; vals[i * VEC + e] = d; part += d * d; }
+    sq += part * keep[i];
+  }
+  sq = wave_allreduce<SumOp>(sq);
+  const A var = L > 1 ? sq / (A)L : (A)0;
+  const A rstd = (A)1 / r_sqrt<A>(var + (A)eps);
+  T* zr = z + row * zPitch;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    A g[VEC], b[VEC];
+    RawIO<T>::unpack(gv[i], g);
+    if (HAS_BIAS) RawIO<T>::unpack(bv[i], b);
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+      A y = vals[i * VEC + e] * rstd * g[e];
+      if (HAS_BIAS) y += b[e];
+      vals[i * VEC + e] = y;
+    }
+    if (keep[i] != (A)0) *reinterpret_cast<Raw*>(zr + e0[i]) = RawIO<T>::pack(&vals[i * VEC]);
+  }
+}
+
 template <typename T>
 static void layerNormTyped(hipStream_t s, const void* x, const void* gain, const void* bias, void* z, const RowPlan& p, float eps) {
   constexpr int V = 16 / sizeof(T);
@@ -318,6 +410,17 @@ static void layerNormTyped(hipStream_t s, const void* x, const void* gain, const
   if (vec) {
     const LongType perWave = 64 * V, perBlock = 256 * V;
 #define LN(TPR, NV, GRID) hipLaunchKernelGGL((layernorm_rows<T, TPR, NV, V>), dim3(GRID), dim3(256), 0, s, a, xt, gt, bt, zt, eps)
+    // rows at a constant pitch that fit one wave
+    const bool linear = p.outerX.rank <= 1 && p.outerZ.rank <= 1 && L < (1 << 30);
+    if (linear && L <= 4 * perWave) {
+      const LongType xp = p.outerX.rank ? p.outerX.stride[0] : 0, zp = p.outerZ.rank ? p.outerZ.stride[0] : 0;
+#define LNL(NV) do { if (bt) hipLaunchKernelGGL((layernorm_linear<T, NV, true>), dim3(gw), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); \
+                     else hipLaunchKernelGGL((layernorm_linear<T, NV, false>), dim3(gw), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); } while (0)
+      if (L <= perWave) { LNL(1); return; }
+      if (L <= 2 * perWave) { LNL(2); return; }
+      LNL(4); return;
+#undef LNL
+    }
     if (L <= perWave) { LN(64, 1, gw); return; }
     if (L <= 2 * perWave) { LN(64, 2, gw); return; }
     if (L <= 4 * perWave) { LN(64, 4, gw); return; }
