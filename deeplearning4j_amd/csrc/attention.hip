@@ -62,16 +62,36 @@ struct FusedArgs {
   LongType H, qB2, kB2, vB2, oB2;     // second batch level (H = 0: none)
   float scale;
   int applyScale, causal;
-  int qTiles;
+  int qTiles, perBatch;
 };
 
 template <typename T> __device__ __forceinline__ float round_storage(float v) { return to_float(Conv<T>::from(v)); }
+// two floats -> one register of two storage values (first in the low half), with one packed conversion for bf16
+typedef __attribute__((ext_vector_type(2))) float f32x2a;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2a;
+template <typename T> __device__ __forceinline__ unsigned pack_pair(float a, float b);
+template <> __device__ __forceinline__ unsigned pack_pair<bf16_t>(float a, float b) {
+  asm("" : "+v"(a), "+v"(b));   // keeps source modifiers out of the packed conversion (see Conv<bf16_t>::from)
+  const f32x2a v = {a, b};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2a));
+}
+template <> __device__ __forceinline__ unsigned pack_pair<f16_t>(float a, float b) {
+  return (unsigned)Conv<f16_t>::from(a).bits | ((unsigned)Conv<f16_t>::from(b).bits << 16);
+}
+// round two values through the storage type in place
+template <typename T> __device__ __forceinline__ void round_pair(float& a, float& b);
+template <> __device__ __forceinline__ void round_pair<bf16_t>(float& a, float& b) {
+  const unsigned p = pack_pair<bf16_t>(a, b);
+  a = __uint_as_float(p << 16);
+  b = __uint_as_float(p & 0xffff0000u);
+}
+template <> __device__ __forceinline__ void round_pair<f16_t>(float& a, float& b) { a = round_storage<f16_t>(a); b = round_storage<f16_t>(b); }
 template <typename T> __device__ __forceinline__ unsigned pack2(float a, float b) {
   return (unsigned)Conv<T>::from(a).bits | ((unsigned)Conv<T>::from(b).bits << 16);
 }
 
 template <typename T, int D>
-__global__ __launch_bounds__(256) void attn_fused(FusedArgs a, const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
+__global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
                                                   T* __restrict__ O) {
   constexpr int BQ = 128, BKV = 64, NT = 256;
   constexpr int DG = D / 8;                      // 16-byte groups along d
@@ -83,18 +103,32 @@ __global__ __launch_bounds__(256) void attn_fused(FusedArgs a, const T* __restri
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   u32x4* smem = reinterpret_cast<u32x4*>(smem_raw);   // two stages of (K tile, V tile)
 
-  // heavy (late) query tiles first under the causal mask
-  const int qt = a.qTiles - 1 - (int)(blockIdx.x % a.qTiles);
-  const LongType b = blockIdx.x / a.qTiles;
-  const LongType q0 = (LongType)qt * BQ;
+  // Consecutive block ids go to different XCDs (8 of them, round-robin).  Give every XCD a contiguous run of the
+  // (batch entry, query tile) sequence instead: the query tiles of one batch entry then share that XCD's L2 copy of
+  // K and V, and under the causal mask every XCD gets the same mix of heavy (late) and light (early) query tiles,
+  // heavy first.
+  unsigned item;
+  {
+    const unsigned total = gridDim.x, xcd = blockIdx.x & 7u, idx = blockIdx.x >> 3, per = total >> 3, rem = total & 7u;
+    item = xcd * per + (xcd < rem ? xcd : rem) + idx;
+  }
+  // under the causal mask a block takes a heavy query tile and then its light mirror image, so that every block
+  // carries the same number of key tiles (a.perBatch = ceil(qTiles / 2) work slots per batch entry, else qTiles)
+  const int slot = (int)(item % a.perBatch);
+  const LongType b = item / a.perBatch;
   if (a.H > 0) {
     const LongType hi = b / a.H, lo = b - hi * a.H;
     Q += hi * a.qB2 + lo * a.qB; K += hi * a.kB2 + lo * a.kB; V += hi * a.vB2 + lo * a.vB; O += hi * a.oB2 + lo * a.oB;
   } else {
     Q += b * a.qB; K += b * a.kB; V += b * a.vB; O += b * a.oB;
   }
-
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, h = lane >> 5;
+  const float L2E = 1.44269502162933349609375f;
+  const bool paired = a.perBatch != a.qTiles;
+  for (int pass = 0; pass < (paired ? 2 : 1); pass++) {
+  const int qt = pass == 0 ? a.qTiles - 1 - slot : slot;
+  if (pass == 1 && qt >= a.qTiles - 1 - slot) break;   // odd count: the middle tile has no mirror image
+  const LongType q0 = (LongType)qt * BQ;
   const LongType query = q0 + wave * 32 + (lane & 31);
   const LongType qrow = query < a.Tq ? query : a.Tq - 1;
 
@@ -109,7 +143,6 @@ __global__ __launch_bounds__(256) void attn_fused(FusedArgs a, const T* __restri
 #pragma unroll
     for (int r = 0; r < 16; r++) o[i][r] = 0.f;
   float m = -1.0e30f, l = 0.f;
-  const float L2E = 1.44269502162933349609375f;
 
   LongType kvEnd = a.Tv;
   if (a.causal) { const LongType lim = q0 + BQ; kvEnd = lim < kvEnd ? lim : kvEnd; }
@@ -155,43 +188,61 @@ __global__ __launch_bounds__(256) void attn_fused(FusedArgs a, const T* __restri
         s[kt] = Mfma16<T>::mma(kf, qf[ks], s[kt]);
       }
     }
-    // scores of this lane's query: register r of tile kt is key kv0 + 32*kt + 8*(r/4) + 4*h + r%4
-    float tmax = -1.0e30f;
+    // scores of this lane's query: register r of tile kt is key kv0 + 32*kt + 8*(r/4) + 4*h + r%4.
+    // scale, clip to +-1e4, round through the storage type (two scores per conversion)
+    float tmax = m;
 #pragma unroll
     for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        float v = s[kt][r];
-        if (a.applyScale) v *= a.scale;
-        v = __builtin_fminf(__builtin_fmaxf(v, -1.0e4f), 1.0e4f);
-        v = round_storage<T>(v);
-        const LongType key = kv0 + kt * 32 + 8 * (r / 4) + 4 * h + (r & 3);
-        const bool masked = key >= a.Tv || (a.causal && key > query);
-        v = masked ? -1.0e30f : v;
-        s[kt][r] = v;
-        tmax = __builtin_fmaxf(tmax, v);
+      for (int r = 0; r < 16; r += 2) {
+        float v0 = s[kt][r], v1 = s[kt][r + 1];
+        if (a.applyScale) { v0 *= a.scale; v1 *= a.scale; }
+        v0 = __builtin_amdgcn_fmed3f(v0, -1.0e4f, 1.0e4f);
+        v1 = __builtin_amdgcn_fmed3f(v1, -1.0e4f, 1.0e4f);
+        round_pair<T>(v0, v1);
+        s[kt][r] = v0; s[kt][r + 1] = v1;
       }
+    // only tiles that touch the diagonal or the end of the keys carry masked entries (wave-uniform test)
+    const int qFirst = (int)q0 + wave * 32;
+    if ((a.causal && (int)kv0 + BKV - 1 > qFirst) || kv0 + BKV > a.Tv) {
+      const int lastKey = a.causal ? ((int)query < (int)a.Tv - 1 ? (int)query : (int)a.Tv - 1) : (int)a.Tv - 1;
+#pragma unroll
+      for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int key = (int)kv0 + kt * 32 + 8 * (r / 4) + 4 * h + (r & 3);
+          s[kt][r] = key > lastKey ? -1.0e30f : s[kt][r];
+        }
+    }
+#pragma unroll
+    for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) tmax = __builtin_fmaxf(tmax, s[kt][r]);
     tmax = __builtin_fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
-    const float mNew = __builtin_fmaxf(m, tmax);
-    const float alpha = __builtin_amdgcn_exp2f((m - mNew) * L2E);
-    m = mNew;
+    // every query has seen key 0 by now, so the running maximum is a real score and masked entries (-1e30)
+    // underflow to exactly 0 in the exponential
+    const float mL = tmax * L2E;
+    const float alpha = __builtin_amdgcn_exp2f(m * L2E - mL);
+    m = tmax;
     float psum = 0.f;
     u32x4 pf[4];   // P^T operand of k-step ks: registers 8*(ks%2) .. +7 of tile ks/2
 #pragma unroll
     for (int kt = 0; kt < 2; kt++)
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
-        // a fully masked history keeps m at the floor; masked entries are forced to zero explicitly
-        float p0 = s[kt][r] <= -1.0e29f ? 0.f : __builtin_amdgcn_exp2f((s[kt][r] - mNew) * L2E);
-        float p1 = s[kt][r + 1] <= -1.0e29f ? 0.f : __builtin_amdgcn_exp2f((s[kt][r + 1] - mNew) * L2E);
+        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][r], L2E, -mL));
+        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][r + 1], L2E, -mL));
         psum += p0 + p1;
-        pf[kt * 2 + r / 8][(r % 8) / 2] = pack2<T>(p0, p1);
+        pf[kt * 2 + r / 8][(r % 8) / 2] = pack_pair<T>(p0, p1);
       }
     l = l * alpha + psum;
+    // the accumulator only needs rescaling when some query's maximum moved
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
 #pragma unroll
-    for (int i = 0; i < DT; i++)
+      for (int i = 0; i < DT; i++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) o[i][r] *= alpha;
+        for (int r = 0; r < 16; r++) o[i][r] *= alpha;
+    }
 
     // O^T += V^T P^T : k-slot e of k-step ks on half h is key 16*ks + 8*(e/4) + 4*h + e%4 (the accumulator order)
 #pragma unroll
@@ -226,6 +277,7 @@ __global__ __launch_bounds__(256) void attn_fused(FusedArgs a, const T* __restri
         *reinterpret_cast<u32x2*>(orow + dv) = w;
       }
   }
+  }   // pass
 }
 
 // ---- decode kernel -------------------------------------------------------------------------------------------------
@@ -350,7 +402,7 @@ static void launchDecodeTyped(hipStream_t s, const void* q, const void* k, const
   a.Tq = d.Tq; a.Tv = d.Tv;
   a.qB = d.qB; a.qT = d.qT; a.kB = d.kB; a.kT = d.kT; a.vB = d.vB; a.vT = d.vT; a.oB = d.oB; a.oT = d.oT;
   a.H = d.H; a.qB2 = d.qB2; a.kB2 = d.kB2; a.vB2 = d.vB2; a.oB2 = d.oB2;
-  a.scale = d.scale; a.applyScale = d.applyScale ? 1 : 0; a.causal = 0; a.qTiles = 1;
+  a.scale = d.scale; a.applyScale = d.applyScale ? 1 : 0; a.causal = 0; a.qTiles = 1; a.perBatch = 1;
   const dim3 grid((unsigned)d.B, (unsigned)d.Tq);
   // few (batch, head) rows: more waves per row, so that the history is still spread over many loads in flight
   if (d.B * d.Tq < 128) hipLaunchKernelGGL((attn_decode<T, D, 16>), grid, dim3(1024), 0, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
@@ -383,6 +435,7 @@ static void launchFusedTyped(hipStream_t s, const void* q, const void* k, const 
   a.H = d.H; a.qB2 = d.qB2; a.kB2 = d.kB2; a.vB2 = d.vB2; a.oB2 = d.oB2;
   a.scale = d.scale; a.applyScale = d.applyScale ? 1 : 0; a.causal = d.causal ? 1 : 0;
   a.qTiles = (int)((d.Tq + 127) / 128);
+  a.perBatch = d.causal ? (a.qTiles + 1) / 2 : a.qTiles;
   constexpr size_t LDS = (size_t)2 * ((D / 64) * TileLayout<64, true>::SLOTS + TileLayout<D, false>::SLOTS) * 16;
   auto kern = attn_fused<T, D>;
   static bool attrSet = false;
@@ -390,7 +443,7 @@ static void launchFusedTyped(hipStream_t s, const void* q, const void* k, const 
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS));
     attrSet = true;
   }
-  hipLaunchKernelGGL(kern, dim3((unsigned)(a.qTiles * d.B)), dim3(256), LDS, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(a.perBatch * d.B)), dim3(256), LDS, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
 }
 
 void launchAttentionFused(hipStream_t s, DataType dt, const void* q, const void* k, const void* v, void* out, const AttnDesc& d) {
