@@ -27,6 +27,25 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_PEAK = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}   # dense TFLOP/s
 
+# HBM-side bytes per launch of the kernel behind each line, measured once with `rocprofv3 --pmc FETCH_SIZE` and
+# `--pmc WRITE_SIZE` (separate runs of this script) and scaled by what the same counters read for the plain copy
+# kernel; the summary of those runs sits under profiles/.  Static figures: they are not re-measured here.
+TRAFFIC_MB = {
+    "mmul bf16 4096": 235.1, "mmul f16 4096": 235.1, "mmul f32 4096^3": 845.1, "mmul f32 4096^3 transposeB": 947.7,
+    "mmul f32 1024": 29.4, "mmul f16 1024": 14.8, "mmul bf16 1024": 14.8,
+    "copy fp32": 268.4, "pairwise_add fp32": 402.6, "transform_tanh fp32": 268.4, "reduce_sum": 134.6, "argmax dim1": 134.6,
+    "layer_norm fp32": 100.8, "gelu fp32": 100.7, "softmax fp32": 1610.6, "layer_norm bf16": 50.4, "gelu bf16": 50.4,
+    "softmax bf16": 805.3, "dot_product_attention_v2": 53.5,
+}
+
+
+def traffic_of(label):
+    best = None
+    for k, v in TRAFFIC_MB.items():
+        if label.startswith(k) and (best is None or len(k) > len(best[0])):
+            best = (k, v)
+    return None if best is None else int(best[1] * 1e6)
+
 
 def timed(ex, L, fn, steps, warmup):
     """Run fn() warmup + steps times; returns (wall ms per step, event ms per step on the execution stream)."""
@@ -47,14 +66,16 @@ def timed(ex, L, fn, steps, warmup):
     return (t1 - t0) * 1e3 / steps, ev / steps
 
 
-def hbm_entry(bytes_per_launch, ev_ms):
+def hbm_entry(bytes_per_launch, ev_ms, label=""):
     ach = bytes_per_launch / (ev_ms * 1e-3) / 1e9
-    return {"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None}
+    return {"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
+            "traffic": traffic_of(label)}
 
 
-def mfma_entry(flops, ev_ms, dtype):
+def mfma_entry(flops, ev_ms, dtype, label=""):
     ach = flops / (ev_ms * 1e-3) / 1e12
-    return {"bound": "mfma", "achieved": round(ach, 2), "peak": MFMA_PEAK[dtype], "unit": "TFLOP/s", "frac": round(ach / MFMA_PEAK[dtype], 4), "traffic": None}
+    return {"bound": "mfma", "achieved": round(ach, 2), "peak": MFMA_PEAK[dtype], "unit": "TFLOP/s", "frac": round(ach / MFMA_PEAK[dtype], 4),
+            "traffic": traffic_of(label)}
 
 
 def main():
@@ -62,8 +83,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--skip-ops", action="store_true", help="only the headline workload")
+    ap.add_argument("--skip-ops", action="store_true", help="leave out the per-op lines of BASELINE configs 1-4")
     ap.add_argument("--skip-cpu", action="store_true", help="leave out the cpu_baseline leg")
+    ap.add_argument("--skip-decode", action="store_true", help="leave out the GPT-2-shaped decode (tens of thousands of launches)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend is built and measured on one GPU; --gpus %d is not supported (no collectives are part of the op path)" % args.gpus)
@@ -93,7 +115,7 @@ def main():
         "steps": steps, "warmup": warmup, "ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "mmul bf16 A[4096,4096] x B[4096,4096] (BASELINE config 2), N(0,1/sqrt(K)) seed 2002, via execCustomOp2(matmul)"},
-        "roofline": mfma_entry(flops, ev_ms, "bf16"),
+        "roofline": mfma_entry(flops, ev_ms, "bf16", "mmul bf16 4096"),
     }
 
     # ---- cpu baseline: the oracle's usualGemm restatement on a bounded sample ------------------------------------
@@ -142,7 +164,7 @@ def main():
             ("argmax dim1 fp32 [8192,4096]", lambda: ex.exec_index_reduce(IndexReduce.IndexMax, T, [1], z=AM), 4 * ne + 8 * shp[0]),
         ]:
             w, e = timed(ex, L, fn, steps, warmup)
-            ops.append({"op": name, "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": hbm_entry(nbytes, e)})
+            ops.append({"op": name, "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": hbm_entry(nbytes, e, name)})
         del X, Y, S, T, R, AM
         # config 3: row ops on [16, 1024, 768] and softmax on [16, 12, 1024, 1024]
         rng = np.random.default_rng(3003)
@@ -156,9 +178,9 @@ def main():
             for arr in (Xr, G, Bv):
                 arr.sync_to_device()
             w, e = timed(ex, L, ex.bind_custom("layer_norm", [Xr, G, Bv], [Zr], i_args=[2], b_args=[False]), steps, warmup)
-            ops.append({"op": "layer_norm %s [16,1024,768]" % dtn, "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": hbm_entry(2 * es * nx + 2 * es * 768, e)})
+            ops.append({"op": "layer_norm %s [16,1024,768]" % dtn, "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": hbm_entry(2 * es * nx + 2 * es * 768, e, "layer_norm %s" % dtn)})
             w, e = timed(ex, L, lambda: ex.exec_transform_strict(TransformStrict.GELU, Zr, Zg), steps, warmup)
-            ops.append({"op": "gelu %s [16,1024,768]" % dtn, "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": hbm_entry(2 * es * nx, e)})
+            ops.append({"op": "gelu %s [16,1024,768]" % dtn, "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": hbm_entry(2 * es * nx, e, "gelu %s" % dtn)})
             del Xr, Zr, Zg
             ls = (16, 12, 1024, 1024)
             nl = 16 * 12 * 1024 * 1024
@@ -170,10 +192,10 @@ def main():
             Zs = NDArray.empty(ls, dt)
             dense = Lg.reshape(16, 12, 1024, 1024)
             w, e = timed(ex, L, ex.bind_custom("softmax", [dense], [Zs], i_args=[3]), steps, warmup)
-            ops.append({"op": "softmax %s [16,12,1024,1024]" % dtn, "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": hbm_entry(2 * es * nl, e)})
+            ops.append({"op": "softmax %s [16,12,1024,1024]" % dtn, "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": hbm_entry(2 * es * nl, e, "softmax %s" % dtn)})
             view = Lg.permute(0, 2, 1, 3)
             w, e = timed(ex, L, ex.bind_custom("softmax", [view], [Zs], i_args=[3]), steps, warmup)
-            ops.append({"op": "softmax %s permuted[0,2,1,3] view" % dtn, "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": hbm_entry(2 * es * nl, e)})
+            ops.append({"op": "softmax %s permuted[0,2,1,3] view" % dtn, "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": hbm_entry(2 * es * nl, e, "softmax %s" % dtn)})
             del Lg, Zs, dense, view
         # config 2, the remaining sizes/dtypes
         for dt, dtn, peak in [(FLOAT32, "f32", "f32"), (HALF, "f16", "f16"), (BFLOAT16, "bf16", "bf16")]:
@@ -192,7 +214,7 @@ def main():
                     ia = [0, 1] if transb else []
                     w, e = timed(ex, L, ex.bind_custom("matmul", [Am, Bm], [Zm], i_args=ia), steps, warmup)
                     ops.append({"op": "mmul %s %d^3%s" % (dtn, m, " transposeB" if transb else ""), "ms": round(e, 4), "wall_ms": round(w, 4),
-                                "roofline": mfma_entry(2.0 * m * m * m, e, peak)})
+                                "roofline": mfma_entry(2.0 * m * m * m, e, peak, "mmul %s %d^3%s" % (dtn, m, " transposeB" if transb else ""))})
                     del Am, Bm, Zm
         # config 4: attention prefill, causal
         for dt, dtn in [(HALF, "f16"), (BFLOAT16, "bf16")]:
@@ -209,8 +231,12 @@ def main():
             w, e = timed(ex, L, ex.bind_custom("dot_product_attention_v2", [Q, V, K_], [O_], t_args=[0.125, 0.0], b_args=[True, False]),
                          max(steps // 5, 3), max(warmup // 5, 1))
             ops.append({"op": "dot_product_attention_v2 %s causal [96,1024,64] (output only)" % dtn, "ms": round(e, 4), "wall_ms": round(w, 4),
-                        "roofline": mfma_entry(4.0 * 96 * 1024 * 1024 * 64, e, dtn)})
+                        "roofline": mfma_entry(4.0 * 96 * 1024 * 1024 * 64, e, dtn, "dot_product_attention_v2"),
+                        "note": "achieved counts the dense 4*B*T*T*D flops; the causal mask makes about half of them useful"})
             del Q, K_, V, O_
+        result["ops"] = ops
+    if not args.skip_decode:
+        ops = result.setdefault("ops", [])
         # config 5: GPT-2-small-shaped greedy decode, bf16, prefill 512 then 128 steps with a key/value cache
         from deeplearning4j_amd.decoder import Decoder, DecoderConfig, init_weights
         cfg = DecoderConfig.gpt2_small()

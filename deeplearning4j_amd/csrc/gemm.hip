@@ -541,7 +541,6 @@ template <typename T, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC>
 static void launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void* B, void* C, LongType batch, bool allowSplit = false) {
   constexpr int NT = WM * WN * 64;
   constexpr size_t LDS = (size_t)2 * (TileLayout<BM, A_KC>::SLOTS + TileLayout<BN, B_KC>::SLOTS) * 16;
-  static const bool pipelined = getenv("ND4JHIP_GEMM_PIPE") ? atoi(getenv("ND4JHIP_GEMM_PIPE")) != 0 : true;
   int splits = 1;
   if (allowSplit) {
     LongType per = 0;
@@ -552,10 +551,9 @@ static void launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
       g.partial = static_cast<float*>(lc->allocationBuffer);
     }
   }
-  const bool usePipe = pipelined && splits == 1;   // the split-K epilogue lives in the plain kernel
+  const bool usePipe = splits == 1;   // the split-K epilogue lives in the plain kernel
   // whole tiles only: the kernel without bounds handling (its K loop needs two K-tiles at least)
-  static const bool fullAllowed = getenv("ND4JHIP_GEMM_FULL") ? atoi(getenv("ND4JHIP_GEMM_FULL")) != 0 : true;
-  const bool useFull = usePipe && fullAllowed && BM * BN >= 128 * 128 && g.M % BM == 0 && g.N % BN == 0 && g.K % 64 == 0 && g.K >= 128;
+  const bool useFull = usePipe && BM * BN >= 128 * 128 && g.M % BM == 0 && g.N % BN == 0 && g.K % 64 == 0 && g.K >= 128;
   auto kern = useFull ? gemm_mfma16f<T, BM, BN, WM, WN, A_KC, B_KC>
                       : usePipe ? gemm_mfma16p<T, BM, BN, WM, WN, A_KC, B_KC> : gemm_mfma16<T, BM, BN, WM, WN, A_KC, B_KC>;
   const int which = useFull ? 2 : usePipe ? 1 : 0;
@@ -577,10 +575,6 @@ static void launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const 
   if (g.M <= 32) return launchMfma16Cfg<T, 32, 128, 1, 4, A_KC, B_KC>(s, g, A, B, C, batch, true);
   if (g.M <= 64 || g.N <= 64 || tiles128 < 192) return launchMfma16Cfg<T, 64, 64, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch, true);
   if (tiles256 < 192) return launchMfma16Cfg<T, 128, 128, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
-  static const int cfg = getenv("ND4JHIP_GEMM_CFG") ? atoi(getenv("ND4JHIP_GEMM_CFG")) : 0;
-  if (cfg == 1) return launchMfma16Cfg<T, 256, 256, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
-  if (cfg == 2) return launchMfma16Cfg<T, 128, 256, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
-  if (cfg == 3) return launchMfma16Cfg<T, 128, 128, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
   return launchMfma16Cfg<T, 256, 256, 2, 4, A_KC, B_KC>(s, g, A, B, C, batch);
 }
 
