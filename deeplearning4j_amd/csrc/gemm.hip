@@ -17,6 +17,8 @@
 #include <cstdlib>
 
 #include "device.h"
+#include <type_traits>
+
 #include "kernels.h"
 #include "mfma_tile.h"
 #include "runtime.h"
@@ -520,6 +522,209 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16f(GemmArgs g, const T
     }
 }
 
+// Whole-tile kernel whose global loads write LDS directly (global_load_lds_dwordx4): no staging registers, no LDS
+// write instructions, and the data of K-tile kt+2 travels while tile kt is multiplied.  A wave-wide load deposits
+// its 64 x 16 bytes contiguously in lane order, so the LDS layouts are chosen per lane on the global side:
+//   k-contiguous operand (A, transposed B): a 1 KiB chunk holds 16 rows x 4 k-groups (8 k each); slot 4j + c of the
+//     chunk holds row j, k-group (c + j/4) % 4.  Four neighbouring lanes fetch 64 contiguous bytes of a row, and the
+//     16 rows a fragment read touches per LDS pass fall into 16 different 16-byte bank groups.
+//   row-major B ([k][n], n contiguous): a 1 KiB chunk holds two k-rows of 256 n; the 16-byte column group c of row k
+//     sits at position c ^ 4 (k % 4).  Fragments come out of LDS through the transposing read ds_read_b64_tr_b16:
+//     in a group of 16 lanes, lane R hands in the address of B[k0 + R/4][n0 + 4 (R%4) ..+3] and lane i receives
+//     B[k0 .. k0+3][n0 + i] -- 16 columns x 4 k per read, two reads per MFMA operand.
+// Two LDS stages of 64 KiB.  Per K-tile: k-steps 0..2 prefetch the next step's fragments; k-step 3 runs half of its
+// MFMAs, waits for the direct loads of tile kt+1, meets the barrier, then reads the first fragments of tile kt+1 and
+// issues the direct loads of tile kt+2 into the stage that was just drained.
+template <typename T, bool B_KC>
+__global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
+                                                    unsigned tilesM, unsigned tilesN) {
+  constexpr int BM = 256, BN = 256, BK = 64, WN = 4, WTM = 128, WTN = 64, TM = 4, TN = 2, NM = TM * TN;
+  constexpr int SLOTS_OP = 256 * 8;              // 16-byte slots of one operand tile (32 KiB)
+  constexpr int STAGE = 2 * SLOTS_OP;
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  typedef const __attribute__((address_space(1))) void* glb_ptr;
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  u32x4* smem = reinterpret_cast<u32x4*>(smem_raw);
+
+  unsigned tm, tn;
+  tileOf(blockIdx.x, gridDim.x, tilesM, tilesN, tm, tn);
+  const LongType m0 = (LongType)tm * BM, n0 = (LongType)tn * BN;
+  const LongType bz = blockIdx.z;
+  { LongType oa, ob, oc; batchOffsets(g, bz, oa, ob, oc); A += oa; B += ob; C += oc; }
+  const LongType lda = g.aRow, ldb = B_KC ? g.bCol : g.bRow;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, h = lane >> 5;
+  const int wm = wave / WN, wn = wave % WN;
+
+  // ---- global side: this wave's four chunks of each operand ------------------------------------------------------
+  // k-contiguous operand, chunk id cw = wave * 4 + i: rows (cw / 2) * 16 .. +15, k-groups (cw % 2) * 4 .. +3
+  const int lj = lane >> 2, lc = lane & 3, lkg = (lc + (lj >> 2)) & 3;
+  const T* aSrc[4];
+  const T* bSrc[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int cw = wave * 4 + i;
+    aSrc[i] = A + (m0 + (cw >> 1) * 16 + lj) * lda + ((cw & 1) * 4 + lkg) * 8;
+    if (B_KC) {
+      bSrc[i] = B + (n0 + (cw >> 1) * 16 + lj) * ldb + ((cw & 1) * 4 + lkg) * 8;
+    } else {
+      const int kr = 2 * cw + (lane >> 5), q = lane & 31, c = q ^ (4 * (kr & 3));
+      bSrc[i] = B + (LongType)kr * ldb + n0 + 8 * c;
+    }
+  }
+  const LongType aStep = BK, bStep = B_KC ? (LongType)BK : (LongType)BK * ldb;
+  auto issueLoads = [&](u32x4* stage, int from, int to) {
+#pragma unroll
+    for (int i = from; i < to; i++) {
+      if (i < 4) {
+        __builtin_amdgcn_global_load_lds((glb_ptr)aSrc[i], (lds_ptr)(stage + (wave * 4 + i) * 64), 16, 0, 0);
+        aSrc[i] += aStep;
+      } else {
+        __builtin_amdgcn_global_load_lds((glb_ptr)bSrc[i - 4], (lds_ptr)(stage + SLOTS_OP + (wave * 4 + i - 4) * 64), 16, 0, 0);
+        bSrc[i - 4] += bStep;
+      }
+    }
+  };
+
+  // ---- LDS side: fragment addresses ---------------------------------------------------------------------------------
+  // k-contiguous layout: row r, k-group kg = 2 ks + h -> chunk (r / 16) * 2 + ks / 2, slot 4 j + ((kg % 4 - j / 4) & 3)
+  int offA[TM][2], offB[TN][2];
+#pragma unroll
+  for (int i = 0; i < TM; i++) {
+    const int r = wm * WTM + i * 32 + (lane & 31), j = r & 15;
+#pragma unroll
+    for (int par = 0; par < 2; par++) offA[i][par] = (r >> 4) * 128 + 4 * j + ((2 * par + h - (j >> 2)) & 3);
+  }
+  int trB[TN];   // byte offsets of the transposing reads (row-major B)
+#pragma unroll
+  for (int jt = 0; jt < TN; jt++) {
+    if (B_KC) {
+      const int r = wn * WTN + jt * 32 + (lane & 31), j = r & 15;
+#pragma unroll
+      for (int par = 0; par < 2; par++) offB[jt][par] = SLOTS_OP + (r >> 4) * 128 + 4 * j + ((2 * par + h - (j >> 2)) & 3);
+      trB[jt] = 0;
+    } else {
+      const int grp = lane >> 4, i16 = lane & 15;
+      const int n4 = wn * WTN + jt * 32 + 16 * (grp & 1) + 4 * (i16 & 3);
+      const int k = 8 * (grp >> 1) + (i16 >> 2);                       // + 16 ks + 4 rd
+      const int phys = (n4 >> 3) ^ (4 * ((i16 >> 2) & 3));
+      trB[jt] = SLOTS_OP * 16 + k * 512 + phys * 16 + ((n4 >> 2) & 1) * 8;
+      offB[jt][0] = offB[jt][1] = 0;
+    }
+  }
+  u32x4 fa[2][TM], fb[2][TN];
+  auto readFrag = [&](const u32x4* stage, int ks, int buf) {
+#pragma unroll
+    for (int i = 0; i < TM; i++) fa[buf][i] = stage[offA[i][ks & 1] + (ks >> 1) * 64];
+#pragma unroll
+    for (int jt = 0; jt < TN; jt++) {
+      if (B_KC) {
+        fb[buf][jt] = stage[offB[jt][ks & 1] + (ks >> 1) * 64];
+      } else {
+        const __attribute__((address_space(3))) unsigned char* base =
+            (const __attribute__((address_space(3))) unsigned char*)(lds_ptr)stage + trB[jt] + ks * 8192;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)base);
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(base + 2048));
+        const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+        fb[buf][jt] = u32x4{l2[0], l2[1], h2[0], h2[1]};
+      }
+    }
+  };
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+  auto mfmas = [&](int buf, int from, int to) {
+#pragma unroll
+    for (int idx = from; idx < to; idx++) {
+      const int i = idx / TN, j = idx % TN;
+      acc[i][j] = Mfma16<T>::mma(fa[buf][i], fb[buf][j], acc[i][j]);
+    }
+  };
+
+  const LongType KT = g.K / BK;
+  issueLoads(smem, 0, 8);            // tile 0 -> stage 0
+  issueLoads(smem + STAGE, 0, 8);    // tile 1 -> stage 1 (K >= 2 tiles)
+  asm volatile("s_waitcnt vmcnt(8)" ::: "memory");   // tile 0 has landed (loads complete in order)
+  __syncthreads();
+  readFrag(smem, 0, 0);
+
+  // one K-tile round; LOADS: the direct loads of tile kt + 2 are issued in this round (second half of k-step 3) and
+  // the first half of them in the NEXT round's k-step 0 -- spread out, each between two MFMAs
+  auto round = [&](LongType kt, auto loadsNow, auto loadsLate) {
+    u32x4* cur = smem + (kt & 1) * STAGE;
+    u32x4* nxt = smem + ((kt + 1) & 1) * STAGE;
+#pragma unroll
+    for (int ks = 0; ks < 3; ks++) {
+      readFrag(cur, ks + 1, (ks + 1) & 1);
+      if (ks == 0 && decltype(loadsLate)::value) issueLoads(nxt, 4, 8);   // second half of tile kt + 1 (B operand)
+      mfmas(ks & 1, 0, NM);
+#pragma unroll
+      for (int q = 0; q < NM; q++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, B_KC ? 1 : 2, 0);
+        if (ks == 0 && decltype(loadsLate)::value && (q & 1)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // k-step 3: half of the MFMAs, then tile kt + 1 must be in LDS for everybody
+    mfmas(1, 0, NM / 2);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    readFrag(nxt, 0, 0);
+    if (decltype(loadsNow)::value) issueLoads(cur, 0, 4);   // first half of tile kt + 2 (A operand) into the drained stage
+    mfmas(1, NM / 2, NM);
+#pragma unroll
+    for (int q = 0; q < NM / 2; q++) {
+      __builtin_amdgcn_sched_group_barrier(0x100, B_KC ? 2 : 3, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (decltype(loadsNow)::value) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  using Yes = std::true_type;
+  using No = std::false_type;
+  // round kt consumes tile kt; tile kt + 1 is complete in LDS by its barrier.  Tile 1 was issued whole in the prologue.
+  if (KT >= 3) {
+    round(0, Yes{}, No{});
+    for (LongType kt = 1; kt + 2 < KT; kt++) round(kt, Yes{}, Yes{});
+    round(KT - 2, No{}, Yes{});
+  } else {
+    round(0, No{}, No{});
+  }
+  {
+    const u32x4* cur = smem + ((KT - 1) & 1) * STAGE;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ks++) {
+      if (ks + 1 < BK / 16) readFrag(cur, ks + 1, (ks + 1) & 1);
+      mfmas(ks & 1, 0, NM);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+  // epilogue: lane owns column (lane % 32); register r of a 32x32 tile is row 8*(r/4) + 4*(lane/32) + r%4
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const LongType col = n0 + wn * WTN + j * 32 + (lane & 31);
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const LongType row = m0 + wm * WTM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r & 3);
+        const LongType off = row * g.cRow + col * g.cCol;
+        float v = g.alpha * acc[i][j][r];
+        if (g.beta != 0.f) v += g.beta * to_float(C[off]);
+        C[off] = Conv<T>::from(v);
+      }
+    }
+}
+
 // How many K-splits a launch of BM x BN tiles gets: enough to put about two blocks on every CU when the tiles alone
 // cannot, bounded by the K-tiles there are and the partial-tile scratch.
 template <int BM, int BN>
@@ -575,6 +780,19 @@ static void launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const 
   if (g.M <= 32) return launchMfma16Cfg<T, 32, 128, 1, 4, A_KC, B_KC>(s, g, A, B, C, batch, true);
   if (g.M <= 64 || g.N <= 64 || tiles128 < 192) return launchMfma16Cfg<T, 64, 64, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch, true);
   if (tiles256 < 192) return launchMfma16Cfg<T, 128, 128, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
+  static const bool direct = getenv("ND4JHIP_GEMM_DIRECT") ? atoi(getenv("ND4JHIP_GEMM_DIRECT")) != 0 : true;
+  if (direct && A_KC && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 64 == 0 && g.K >= 128) {
+    constexpr size_t LDS = 2 * 2 * 256 * 8 * 16;
+    auto kern = gemm_mfma16d<T, B_KC>;
+    static bool attrSet = false;
+    if (!attrSet) {
+      HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS));
+      attrSet = true;
+    }
+    const unsigned tM = (unsigned)(g.M / 256), tN = (unsigned)(g.N / 256);
+    hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(512), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
+    return;
+  }
   return launchMfma16Cfg<T, 256, 256, 2, 4, A_KC, B_KC>(s, g, A, B, C, batch);
 }
 
