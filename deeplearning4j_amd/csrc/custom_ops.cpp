@@ -205,6 +205,86 @@ static void matmulExec(Context& c) {
   registerSpecialUse(std::vector<NDArray*>{z}, reads);
 }
 
+// ---- xw_plus_b ---------------------------------------------------------------------------------------------------
+// generic/nn/xw_plus_b.cpp:36-160: z = x w + b with b a row vector over the output features.  IArgs (each "== 1"):
+// [transpose x, transpose w, transpose z]; x of rank > 2 is flattened to [prod(leading dims), last] (the reference
+// reshapes it 'c', so it must be dense here).  The reference runs mmul and then addiRowVector; here the bias row is
+// added in the product's epilogue (one rounding instead of two for 16-bit types).
+struct XwGeometry {
+  LongType M, N, K;
+  LongType aRow, aCol, bRow, bCol, cRow, cCol;
+  std::vector<LongType> zShape;
+};
+static bool denseC(const NDArray* a) {
+  LongType expect = 1;
+  for (int d = a->rankOf() - 1; d >= 0; d--) {
+    if (a->sizeAt(d) != 1 && a->strideAt(d) != expect) return false;
+    expect *= a->sizeAt(d);
+  }
+  return true;
+}
+static XwGeometry xwGeometry(Context& c, bool needOutput) {
+  ND4J_REQUIRE(c.width() >= 3, "xw_plus_b: x, weights and bias are required");
+  NDArray* x = c.input(0); NDArray* w = c.input(1); NDArray* b = c.input(2);
+  const bool aT = iArg(c, 0, 0) == 1, bT = iArg(c, 1, 0) == 1, cT = iArg(c, 2, 0) == 1;
+  XwGeometry g;
+  std::vector<LongType> lead;
+  ND4J_REQUIRE(x->rankOf() >= 2, "xw_plus_b: After reshaping, input x array should have rank equal 2, but got instead " + std::to_string(x->rankOf()) + "!");
+  ND4J_REQUIRE(w->rankOf() == 2, "xw_plus_b: Input weights array should have rank equal 2, but got instead " + std::to_string(w->rankOf()) + "!");
+  if (x->rankOf() > 2) {
+    ND4J_REQUIRE(denseC(x), "xw_plus_b: nd4j-hip needs a dense c-order x of rank > 2 (it is flattened to two dims)");
+    LongType m = 1;
+    for (int d = 0; d < x->rankOf() - 1; d++) { m *= x->sizeAt(d); lead.push_back(x->sizeAt(d)); }
+    g.M = m; g.K = x->sizeAt(x->rankOf() - 1); g.aRow = g.K; g.aCol = 1;
+  } else {
+    g.M = x->sizeAt(0); g.K = x->sizeAt(1); g.aRow = x->strideAt(0); g.aCol = x->strideAt(1);
+    lead = {g.M};
+  }
+  if (aT) { std::swap(g.M, g.K); std::swap(g.aRow, g.aCol); lead = {g.M}; }
+  LongType Kw = w->sizeAt(0);
+  g.N = w->sizeAt(1); g.bRow = w->strideAt(0); g.bCol = w->strideAt(1);
+  if (bT) { std::swap(Kw, g.N); std::swap(g.bRow, g.bCol); }
+  ND4J_REQUIRE(Kw == g.K, "xw_plus_b: input arrays have inconsistent shapes for matrix product: x " + shapeStr(x) + ", weights " + shapeStr(w) + " !");
+  ND4J_REQUIRE(b->lengthOf() == g.N, "xw_plus_b: Input bias vector should be 1D and have proper dimension 1x" + std::to_string(g.N) + ". But got length " + std::to_string(b->lengthOf()) + " instead !");
+  g.zShape = lead; g.zShape.push_back(g.N);
+  if (cT) { ND4J_REQUIRE(g.zShape.size() == 2, "xw_plus_b: a transposed output needs a rank-2 product"); std::swap(g.zShape[0], g.zShape[1]); }
+  if (needOutput) {
+    NDArray* z = c.output(0);
+    ND4J_REQUIRE(shapeOf(z) == g.zShape, "xw_plus_b: output array has shape " + shapeStr(z) + ", expected the product's shape");
+    if (z->rankOf() > 2) {
+      ND4J_REQUIRE(denseC(z), "xw_plus_b: nd4j-hip needs a dense c-order output of rank > 2");
+      g.cRow = g.N; g.cCol = 1;
+    } else {
+      g.cRow = z->strideAt(0); g.cCol = z->strideAt(1);
+      if (cT) std::swap(g.cRow, g.cCol);
+    }
+  }
+  return g;
+}
+static void xwPlusBExec(Context& c) {
+  ND4J_REQUIRE(c.width() >= 3, "xw_plus_b: x, weights and bias are required");
+  NDArray* x = c.input(0); NDArray* w = c.input(1); NDArray* b = c.input(2); NDArray* z = c.output(0);
+  if (x->isEmpty() || w->isEmpty() || b->isEmpty()) return;
+  XwGeometry g = xwGeometry(c, true);
+  const DataType dt = z->dataType();
+  ND4J_REQUIRE(x->dataType() == dt && w->dataType() == dt && b->dataType() == dt && isFloatType(dt), "xw_plus_b: nd4j-hip requires one floating point type for x, weights, bias and output");
+  // the bias row is read as a dense vector
+  LongType bstride = 1;
+  for (int d = 0; d < b->rankOf(); d++) if (b->sizeAt(d) != 1) bstride = b->strideAt(d);
+  ND4J_REQUIRE(bstride == 1 || g.N == 1, "xw_plus_b: nd4j-hip needs a contiguous bias vector");
+  GemmDesc d;
+  d.M = g.M; d.N = g.N; d.K = g.K;
+  d.aRow = g.aRow; d.aCol = g.aCol; d.bRow = g.bRow; d.bCol = g.bCol; d.cRow = g.cRow; d.cCol = g.cCol;
+  prepareSpecialUse({z}, {x, w, b});
+  d.bias = b->specialBuffer();
+  launchGemm(stream(), dt, x->specialBuffer(), w->specialBuffer(), z->specialBuffer(), d);
+  registerSpecialUse({z}, {x, w, b});
+}
+static std::vector<std::vector<LongType>> xwPlusBShapeFn(Context& c) {
+  XwGeometry g = xwGeometry(c, false);
+  return {makeShapeInfo(c.input(0)->dataType(), 'c', g.zShape)};
+}
+
 // ---- softmax -----------------------------------------------------------------------------------------------------
 // generic/nn/softmax.cpp:37-52 -> helpers/cpu/softmax.cpp:252-353
 static bool sameShapeStrict(const NDArray* a, const NDArray* b) {
@@ -610,6 +690,7 @@ static void ensureRegistered() {
   std::call_once(once, [] {
     // arities as declared by the reference's *_OP_IMPL macros
     for (const char* alias : {"matmul", "mMul", "mmul", "gemm", "gemv", "dot"}) reg(alias, 2, 1, false, 0, -2, matmulExec, matmulShapeFn);
+    reg("xw_plus_b", 3, 1, false, 0, 0, xwPlusBExec, xwPlusBShapeFn);
     reg("softmax", 1, 1, true, 0, 0, softmaxExec, sameAsInputShapeFn);
     reg("layer_norm", 2, 1, false, 0, -1, layerNormExec, sameAsInputShapeFn);
     reg("dot_product_attention_v2", -2, -1, false, -2, -2, attentionExec, attentionShapeFn);

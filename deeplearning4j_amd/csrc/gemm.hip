@@ -37,6 +37,7 @@ struct GemmArgs {
   int splits;
   LongType ktPerSplit;
   float* partial;
+  const void* bias;   // optional [N] row added to every output row (xw_plus_b), same type as C
 };
 typedef __attribute__((ext_vector_type(4))) float f32x4v;
 
@@ -86,6 +87,7 @@ __global__ __launch_bounds__(256) void gemm_simple(GemmArgs g, const T* __restri
         const LongType off = m * g.cRow + n * g.cCol;
         Acc v = (Acc)g.alpha * acc[i][j];
         if (g.beta != 0.f) v += (Acc)g.beta * (Acc)to_float(C[off]);
+        if (g.bias) v += (Acc)to_float(static_cast<const T*>(g.bias)[n]);
         C[off] = Conv<T>::from(v);
       }
     }
@@ -219,6 +221,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16(GemmArgs g, const T*
           const LongType off = row * g.cRow + col * g.cCol;
           float v = g.alpha * acc[i][j][r];
           if (g.beta != 0.f) v += g.beta * to_float(C[off]);
+          if (g.bias) v += to_float(static_cast<const T*>(g.bias)[col]);
           C[off] = Conv<T>::from(v);
         }
       }
@@ -259,6 +262,7 @@ __global__ __launch_bounds__(WM * WN * 64) void splitk_finish(GemmArgs g, T* __r
     const LongType off = (row0 + e) * g.cRow + col * g.cCol;
     float v = g.alpha * tot[e];
     if (g.beta != 0.f) v += g.beta * to_float(C[off]);
+    if (g.bias) v += to_float(static_cast<const T*>(g.bias)[col]);
     C[off] = Conv<T>::from(v);
   }
 }
@@ -357,6 +361,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16p(GemmArgs g, const T
           const LongType off = row * g.cRow + col * g.cCol;
           float v = g.alpha * acc[i][j][r];
           if (g.beta != 0.f) v += g.beta * to_float(C[off]);
+          if (g.bias) v += to_float(static_cast<const T*>(g.bias)[col]);
           C[off] = Conv<T>::from(v);
         }
       }
@@ -517,6 +522,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16f(GemmArgs g, const T
         const LongType off = row * g.cRow + col * g.cCol;
         float v = g.alpha * acc[i][j][r];
         if (g.beta != 0.f) v += g.beta * to_float(C[off]);
+        if (g.bias) v += to_float(static_cast<const T*>(g.bias)[col]);
         C[off] = Conv<T>::from(v);
       }
     }
@@ -720,6 +726,7 @@ __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restr
         const LongType off = row * g.cRow + col * g.cCol;
         float v = g.alpha * acc[i][j][r];
         if (g.beta != 0.f) v += g.beta * to_float(C[off]);
+        if (g.bias) v += to_float(static_cast<const T*>(g.bias)[col]);
         C[off] = Conv<T>::from(v);
       }
     }
@@ -922,6 +929,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32(GemmArgs g, const fl
           const LongType off = row * g.cRow + col * g.cCol;
           float v = g.alpha * acc[i][j][r];
           if (g.beta != 0.f) v += g.beta * C[off];
+          if (g.bias) v += static_cast<const float*>(g.bias)[col];
           C[off] = v;
         }
       }
@@ -945,7 +953,7 @@ static void launchMfma32(hipStream_t s, const GemmArgs& g, const void* A, const 
 // y[n] = alpha * sum_k x[k] * W[n][k] (+ beta y): W rows contiguous in k.  One wave per output row.
 template <typename T>
 __global__ __launch_bounds__(256) void gemv_rowdot(const T* __restrict__ W, LongType ldw, const T* __restrict__ x, LongType xs, T* __restrict__ y,
-                                                   LongType ys, LongType N, LongType K, float alpha, float beta) {
+                                                   LongType ys, LongType N, LongType K, float alpha, float beta, const T* __restrict__ bias) {
   using A = typename Conv<T>::acc;
   constexpr int V = 16 / sizeof(T);
   using VT = Vec<T, V>;
@@ -970,6 +978,7 @@ __global__ __launch_bounds__(256) void gemv_rowdot(const T* __restrict__ W, Long
   if (lane == 0) {
     A v = (A)alpha * acc;
     if (beta != 0.f) v += (A)beta * (A)to_float(y[n * ys]);
+    if (bias) v += (A)to_float(bias[n]);
     y[n * ys] = Conv<T>::from(v);
   }
 }
@@ -977,7 +986,7 @@ __global__ __launch_bounds__(256) void gemv_rowdot(const T* __restrict__ W, Long
 // slices are combined through LDS (block = 64 column groups x 4 k-slices).
 template <typename T>
 __global__ __launch_bounds__(256) void gemv_colsum(const T* __restrict__ W, LongType ldw, const T* __restrict__ x, LongType xs, T* __restrict__ y,
-                                                   LongType ys, LongType N, LongType K, float alpha, float beta) {
+                                                   LongType ys, LongType N, LongType K, float alpha, float beta, const T* __restrict__ bias) {
   using A = typename Conv<T>::acc;
   constexpr int V = 16 / sizeof(T);
   using VT = Vec<T, V>;
@@ -1010,6 +1019,7 @@ __global__ __launch_bounds__(256) void gemv_colsum(const T* __restrict__ W, Long
       if (n0 + e >= N) break;
       A v = (A)alpha * (part[0][cg * V + e] + part[1][cg * V + e] + part[2][cg * V + e] + part[3][cg * V + e]);
       if (beta != 0.f) v += (A)beta * (A)to_float(y[(n0 + e) * ys]);
+      if (bias) v += (A)to_float(bias[n0 + e]);
       y[(n0 + e) * ys] = Conv<T>::from(v);
     }
   }
@@ -1021,13 +1031,13 @@ static bool tryGemv(hipStream_t s, const GemmDesc& d, const void* A, const void*
   constexpr int V = 16 / sizeof(T);
   if (d.M == 1 && d.N > 1) {
     // y[n] = sum_k a[k] * op(B)[k][n]
-    if (d.bRow == 1) { hipLaunchKernelGGL((gemv_rowdot<T>), dim3((unsigned)((d.N + 3) / 4)), dim3(256), 0, s, (const T*)B, d.bCol, (const T*)A, d.aCol, (T*)C, d.cCol, d.N, d.K, d.alpha, d.beta); return true; }
-    if (d.bCol == 1) { hipLaunchKernelGGL((gemv_colsum<T>), dim3((unsigned)((d.N + 64 * V - 1) / (64 * V))), dim3(256), 0, s, (const T*)B, d.bRow, (const T*)A, d.aCol, (T*)C, d.cCol, d.N, d.K, d.alpha, d.beta); return true; }
+    if (d.bRow == 1) { hipLaunchKernelGGL((gemv_rowdot<T>), dim3((unsigned)((d.N + 3) / 4)), dim3(256), 0, s, (const T*)B, d.bCol, (const T*)A, d.aCol, (T*)C, d.cCol, d.N, d.K, d.alpha, d.beta, (const T*)d.bias); return true; }
+    if (d.bCol == 1) { hipLaunchKernelGGL((gemv_colsum<T>), dim3((unsigned)((d.N + 64 * V - 1) / (64 * V))), dim3(256), 0, s, (const T*)B, d.bRow, (const T*)A, d.aCol, (T*)C, d.cCol, d.N, d.K, d.alpha, d.beta, (const T*)d.bias); return true; }
   }
-  if (d.N == 1 && d.M > 1) {
+  if (d.N == 1 && d.M > 1 && !d.bias) {
     // y[m] = sum_k op(A)[m][k] * b[k]
-    if (d.aCol == 1) { hipLaunchKernelGGL((gemv_rowdot<T>), dim3((unsigned)((d.M + 3) / 4)), dim3(256), 0, s, (const T*)A, d.aRow, (const T*)B, d.bRow, (T*)C, d.cRow, d.M, d.K, d.alpha, d.beta); return true; }
-    if (d.aRow == 1) { hipLaunchKernelGGL((gemv_colsum<T>), dim3((unsigned)((d.M + 64 * V - 1) / (64 * V))), dim3(256), 0, s, (const T*)A, d.aCol, (const T*)B, d.bRow, (T*)C, d.cRow, d.M, d.K, d.alpha, d.beta); return true; }
+    if (d.aCol == 1) { hipLaunchKernelGGL((gemv_rowdot<T>), dim3((unsigned)((d.M + 3) / 4)), dim3(256), 0, s, (const T*)A, d.aRow, (const T*)B, d.bRow, (T*)C, d.cRow, d.M, d.K, d.alpha, d.beta, (const T*)nullptr); return true; }
+    if (d.aRow == 1) { hipLaunchKernelGGL((gemv_colsum<T>), dim3((unsigned)((d.M + 64 * V - 1) / (64 * V))), dim3(256), 0, s, (const T*)A, d.aCol, (const T*)B, d.bRow, (T*)C, d.cRow, d.M, d.K, d.alpha, d.beta, (const T*)nullptr); return true; }
   }
   return false;
 }
@@ -1040,7 +1050,7 @@ static GemmArgs toArgs(const GemmDesc& d) {
   g.aBatch = d.aBatch; g.bBatch = d.bBatch; g.cBatch = d.cBatch;
   g.batchInner = d.batchInner; g.aBatch2 = d.aBatch2; g.bBatch2 = d.bBatch2; g.cBatch2 = d.cBatch2;
   g.alpha = d.alpha; g.beta = d.beta;
-  g.splits = 1; g.ktPerSplit = 0; g.partial = nullptr;
+  g.splits = 1; g.ktPerSplit = 0; g.partial = nullptr; g.bias = d.bias;
   return g;
 }
 

@@ -99,6 +99,7 @@ struct GemmDesc {
   // by the *Batch2 strides (batchInner = 0: one level)
   LongType batchInner = 0, aBatch2 = 0, bBatch2 = 0, cBatch2 = 0;
   float alpha = 1.f, beta = 0.f;
+  const void* bias = nullptr;   // optional dense [N] row (type of C) added to every output row
 };
 void launchGemm(hipStream_t s, DataType dt, const void* A, const void* B, void* C, const GemmDesc& d);
 

@@ -3,9 +3,10 @@
 Stands in for what a SameDiff inference session does with such a graph in the reference
 (nd4j-api .../autodiff/samediff/internal/InferenceSession.java: one native call per graph node): every step below is
 one reference op executed through `execCustomOp2` or a legacy `exec*` entry point -- `gather` (token and position
-embeddings), `layer_norm`, `matmul`, broadcastable `add`, transform-strict GELU (opNum 53), transform-any Assign (the
-write into the key/value cache), `dot_product_attention_v2`, pairwise Add (residuals), `argmax`.  Nothing is fused on
-the Python side and no array leaves the device between ops.
+embeddings), broadcastable `add`, `layer_norm`, `xw_plus_b` (the linear layers), transform-strict GELU (opNum 53),
+transform-any Assign (the write into the key/value cache), `dot_product_attention_v2`, pairwise Add (residuals),
+`matmul` (tied output embedding), `argmax`.  Nothing is fused on the Python side and no array leaves the device
+between ops.
 
 Memory layout (all activations token-major, so the head split needs no copy):
   x, attention output ... [B, T, d_model]
@@ -137,8 +138,7 @@ class Decoder:
         for li, w in enumerate(self.layers):
             kc, vc = self.kcache[li], self.vcache[li]
             ops.append(self._custom("layer_norm", [x2, w["ln1_g"], w["ln1_b"]], [ln2], i_args=[1], b_args=[False]))
-            ops.append(self._custom("matmul", [ln2, w["w_qkv"]], [qkv2]))
-            ops.append(self._custom("add", [qkv2, w["b_qkv"]], [qkv2]))
+            ops.append(self._custom("xw_plus_b", [ln2, w["w_qkv"], w["b_qkv"]], [qkv2]))
             # append this chunk's keys / values to the cache
             ops.append(self._assign(knew, kc.view((B, T, d), (M * d, d, 1), past * d)))
             ops.append(self._assign(vnew, vc.view((B, T, d), (M * d, d, 1), past * d)))
@@ -146,15 +146,12 @@ class Decoder:
             v4 = vc.view((B, H, total, Dh), (M * d, Dh, d, 1), 0)
             # a chunk that starts at position 0 attends causally; a single new token sees the whole cache
             ops.append(self._custom("dot_product_attention_v2", [q4, v4, k4], [o4], t_args=[scale, 0.0], b_args=[past == 0 and T > 1, False]))
-            ops.append(self._custom("matmul", [att2, w["w_o"]], [proj2]))
-            ops.append(self._custom("add", [proj2, w["b_o"]], [proj2]))
+            ops.append(self._custom("xw_plus_b", [att2, w["w_o"], w["b_o"]], [proj2]))
             ops.append(self._pairwise_add(x2, proj2, x2))
             ops.append(self._custom("layer_norm", [x2, w["ln2_g"], w["ln2_b"]], [ln2], i_args=[1], b_args=[False]))
-            ops.append(self._custom("matmul", [ln2, w["w_fc"]], [h2]))
-            ops.append(self._custom("add", [h2, w["b_fc"]], [h2]))
+            ops.append(self._custom("xw_plus_b", [ln2, w["w_fc"], w["b_fc"]], [h2]))
             ops.append(self._gelu(h2, g2))
-            ops.append(self._custom("matmul", [g2, w["w_proj"]], [proj2]))
-            ops.append(self._custom("add", [proj2, w["b_proj"]], [proj2]))
+            ops.append(self._custom("xw_plus_b", [g2, w["w_proj"], w["b_proj"]], [proj2]))
             ops.append(self._pairwise_add(x2, proj2, x2))
         # final layer norm on the last position only, tied output projection, greedy pick
         xlast = a["x"].view((B, d), (T * d, 1), (T - 1) * d)

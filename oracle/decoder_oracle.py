@@ -1,7 +1,8 @@
 """CPU composition of the GPT-2-shaped decode step out of the oracle's ops -- test infrastructure only.
 
-Mirrors deeplearning4j_amd/decoder.py op for op (gather, add, layer_norm, matmul, bias add, GELU opNum 53,
-dot_product_attention_v2, argmax), each executed by the CPU restatement in nd4j_oracle.c, so that greedy token ids
+Mirrors deeplearning4j_amd/decoder.py op for op (gather, add, layer_norm, xw_plus_b = mmul followed by the bias row
+as in generic/nn/xw_plus_b.cpp:117-133, GELU opNum 53, dot_product_attention_v2, argmax), each executed by the CPU
+restatement in nd4j_oracle.c, so that greedy token ids
 and logits of the HIP path can be compared on the same seeded weights.  Arrays are numpy: float32, or uint16 bit
 patterns for bf16.
 """

@@ -180,6 +180,46 @@ def test_mmul_full_size_properties(ex):
     assert_close(zt, z, 1e-2, 1e-2, "transposeB agrees with plain B")
 
 
+@pytest.mark.parametrize("dtype,tol", [(FLOAT32, 1e-4), (HALF, 1e-2), (BFLOAT16, 1e-2)])
+@pytest.mark.parametrize("M,K,N", [(1, 768, 2304), (32, 3072, 768), (300, 256, 512), (7, 40, 24), (512, 512, 512)])
+def test_xw_plus_b_vs_oracle(ex, oracle, dtype, tol, M, K, N):
+    """z = x w + b; the oracle runs the reference's own two steps (mmul, then the bias row added to every row)."""
+    rng = np.random.default_rng(M + K + N)
+    x = rng.normal(0, 1 / math.sqrt(K), (M, K))
+    w = rng.normal(0, 1, (K, N))
+    b = rng.normal(0, 1, (N,))
+    ox, dx = _pair(oracle, x, dtype)
+    ow, dw = _pair(oracle, w, dtype)
+    ob, db = _pair(oracle, b, dtype)
+    oz = _ozeros(oracle, (M, N), dtype)
+    oracle.matmul(ox, ow, oz, accumulate=1)
+    oracle.add_row_vector(oz, ob, oz)
+    z = ex.exec_custom("xw_plus_b", [dx, dw, db])[0]
+    assert z.shape == (M, N)
+    assert_close(z.to_float(), _f(oz), tol, tol, "xw_plus_b")
+    # weights stored [N, K] (transpose flag 1) and a rank-3 x
+    owt, dwt = _pair(oracle, w.T.copy(), dtype)
+    zt = ex.exec_custom("xw_plus_b", [dx, dwt, db], i_args=[0, 1])[0]
+    assert_close(zt.to_float(), _f(oz), tol, tol, "xw_plus_b, transposed weights")
+    if M % 4 == 0:
+        x3 = NDArray.from_numpy(np.asarray(ox.a).reshape(4, M // 4, K), dtype)
+        z3 = ex.exec_custom("xw_plus_b", [x3, dw, db])[0]
+        assert z3.shape == (4, M // 4, N)
+        assert_close(z3.to_float().reshape(M, N), _f(oz), tol, tol, "xw_plus_b, rank-3 x")
+
+
+def test_xw_plus_b_errors(ex):
+    x = NDArray.from_numpy(np.ones((4, 8), np.float32))
+    w = NDArray.from_numpy(np.ones((9, 5), np.float32))
+    b = NDArray.from_numpy(np.ones((5,), np.float32))
+    with pytest.raises(NativeOpsError, match="inconsistent shapes"):
+        ex.exec_custom("xw_plus_b", [x, w, b])
+    w2 = NDArray.from_numpy(np.ones((8, 5), np.float32))
+    b2 = NDArray.from_numpy(np.ones((6,), np.float32))
+    with pytest.raises(NativeOpsError, match="bias"):
+        ex.exec_custom("xw_plus_b", [x, w2, b2])
+
+
 # ---- softmax ---------------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype,rtol,atol", [(FLOAT32, 1e-5, 1e-6), (BFLOAT16, 1e-2, 1e-4), (HALF, 1e-2, 1e-4), (DOUBLE, 1e-12, 1e-14)])
 @pytest.mark.parametrize("shape,dim", [((4, 3, 8, 1024), 3), ((17, 33), 1), ((17, 33), 0), ((5, 6, 7), 1), ((3, 5000), 1), ((2, 20000), 1), ((6, 1000), -1)])
