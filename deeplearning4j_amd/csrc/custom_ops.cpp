@@ -508,6 +508,63 @@ static std::vector<std::vector<LongType>> attentionShapeFn(Context& c) {
   return {makeShapeInfo(dt, 'c', o), makeShapeInfo(dt, 'c', w), makeShapeInfo(dt, 'c', w)};
 }
 
+// ---- top_k -----------------------------------------------------------------------------------------------------------------
+// generic/parity_ops/top_k.cpp:31-57: k from IArg0 or from a second input; BArg0 = sort by value (default true, else the
+// picks come in index order); outputs [values (input type), indices (INT64 by the shape function)] with the last
+// dim replaced by k.  For k = 1 the first maximum wins, as in the reference.  For k > 1 the reference's insertion
+// loop (helpers/cpu/top_k.cpp:62-99) never admits a value that is already in its candidate set and recovers
+// positions by value afterwards, so rows with repeated values among the winners give it fewer distinct picks or one
+// position twice; this implementation returns the k largest elements with ties resolved to the lower index, which
+// is the same result whenever the winners are pairwise different.
+static int topKCount(Context& c) {
+  if (c.width() > 1) {
+    NDArray* ka = c.input(1);
+    ka->buf->syncToPrimary();
+    ND4J_REQUIRE(ka->lengthOf() >= 1, "top_k: k array is empty");
+    if (ka->dataType() == INT64) return (int)ka->hostAs<LongType>()[0];
+    if (ka->dataType() == INT32) return ka->hostAs<int>()[0];
+    ND4J_THROW("top_k: k array must be INT32 or INT64");
+  }
+  return (int)iArg(c, 0, 1);
+}
+static std::vector<LongType> widened(const NDArray* z, LongType n) {
+  // z's descriptor with the last extent set to n: lets the row planner pair it with x
+  std::vector<LongType> shp = shapeOf(z), st;
+  for (int d = 0; d < z->rankOf(); d++) st.push_back(z->strideAt(d));
+  shp.back() = n;
+  return makeShapeInfo(z->dataType(), 'c', shp, st.data());
+}
+static void topKExec(Context& c) {
+  NDArray* x = c.input(0);
+  ND4J_REQUIRE(c.outputs.size() >= 2 && c.outputs[0] && c.outputs[1], "top_k: values and indices outputs are required");
+  NDArray* v = c.output(0); NDArray* idx = c.outputs[1];
+  const int k = topKCount(c);
+  const bool needSort = bArg(c, 0, true);
+  ND4J_REQUIRE(x->rankOf() >= 1, "top_k: input must have rank >= 1");
+  const LongType n = x->sizeAt(x->rankOf() - 1);
+  ND4J_REQUIRE(k <= n, "top_k: k should not be greater than last dimension");
+  ND4J_REQUIRE(k > 0, "top_k: k should be positive, but " + std::to_string(k) + " given.");
+  std::vector<LongType> want = shapeOf(x);
+  want.back() = k;
+  ND4J_REQUIRE(shapeOf(v) == want && shapeOf(idx) == want, "top_k: outputs must have the input's shape with the last dim replaced by k");
+  ND4J_REQUIRE(v->dataType() == x->dataType(), "top_k: values must carry the input's data type");
+  if (x->isEmpty()) return;
+  auto vsi = widened(v, n), isi = widened(idx, n);
+  RowPlan pv = buildRowPlan(x->shapeInfo(), vsi.data(), x->rankOf() - 1), pi = buildRowPlan(x->shapeInfo(), isi.data(), x->rankOf() - 1);
+  prepareSpecialUse({v, idx}, {x});
+  launchTopK(stream(), x->dataType(), idx->dataType(), x->specialBuffer(), v->specialBuffer(), idx->specialBuffer(), pv, pi, k, needSort);
+  registerSpecialUse({v, idx}, {x});
+}
+static std::vector<std::vector<LongType>> topKShapeFn(Context& c) {
+  NDArray* x = c.input(0);
+  const int k = topKCount(c);
+  ND4J_REQUIRE(k > 0, "top_k: k should be positive, but " + std::to_string(k) + " given.");
+  std::vector<LongType> shp = shapeOf(x);
+  ND4J_REQUIRE(!shp.empty(), "top_k: input must have rank >= 1");
+  shp.back() = k;
+  return {makeShapeInfo(x->dataType(), x->ordering(), shp), makeShapeInfo(INT64, x->ordering(), shp)};
+}
+
 // ---- argmax / argmin ---------------------------------------------------------------------------------------------------------
 // generic/reduce/argmax.cpp:38-103: dims from IArgs or from input 1; BArg0 keepDims; DArg0 output dtype (INT64)
 static std::vector<LongType> argDims(Context& c) {
@@ -692,6 +749,7 @@ static void ensureRegistered() {
     for (const char* alias : {"matmul", "mMul", "mmul", "gemm", "gemv", "dot"}) reg(alias, 2, 1, false, 0, -2, matmulExec, matmulShapeFn);
     reg("xw_plus_b", 3, 1, false, 0, 0, xwPlusBExec, xwPlusBShapeFn);
     reg("softmax", 1, 1, true, 0, 0, softmaxExec, sameAsInputShapeFn);
+    reg("top_k", 1, 2, false, 0, -1, topKExec, topKShapeFn);
     reg("layer_norm", 2, 1, false, 0, -1, layerNormExec, sameAsInputShapeFn);
     reg("dot_product_attention_v2", -2, -1, false, -2, -2, attentionExec, attentionShapeFn);
     reg("argmax", 1, 1, false, 0, -2, [](Context& c) { argExec(c, 0, "ArgMax"); }, argShapeFn);

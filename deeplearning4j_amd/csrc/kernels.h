@@ -78,6 +78,10 @@ struct RowPlan {
 void launchSoftmax(hipStream_t s, DataType dt, const void* x, void* z, const RowPlan& p, bool clampMode);
 void launchLayerNormRows(hipStream_t s, DataType dt, const void* x, const void* gain, const void* bias, void* z,
                          const RowPlan& p, float eps);
+// k largest elements of every row (last axis) with their positions; pv / pi are the row plans (x, values) and
+// (x, indices); sorted: descending values, else ascending positions
+void launchTopK(hipStream_t s, DataType xdt, DataType idt, const void* x, void* values, void* indices, const RowPlan& pv,
+                const RowPlan& pi, int k, bool sorted);
 // generic layer norm over arbitrary axes: one block per statistics group
 struct LnGenericPlan {
   DevShape outerX, innerX, outerZ, innerZ;

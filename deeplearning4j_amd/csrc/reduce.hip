@@ -454,4 +454,105 @@ void launchIndexReduce(hipStream_t st, IndexKind k, DataType xdt, DataType zdt, 
   HIP_CHECK(hipGetLastError());
 }
 
+
+// ---- top-k along the last axis -------------------------------------------------------------------------------
+// generic/parity_ops/top_k.cpp:31-57 -> helpers/cpu/top_k.cpp:34-125.  One block per row, k rounds of selection:
+// round j picks the largest element that comes after the previous pick in the total order "greater value first,
+// lower index first", so values come out in descending order and equal values in index order; NaN sorts below
+// every number.  With sorted = false the k picks are put in index order afterwards.
+struct TopKArgs {
+  DevShape outerX, outerV, outerI;
+  LongType rows, rowLen, xInner, vInner, iInner;
+  int k, sorted;
+};
+template <typename A> struct Pick { A v; int i; };
+template <typename A>
+__device__ __forceinline__ bool pickBefore(A av, int ai, A bv, int bi) { return av > bv || (av == bv && ai < bi); }
+template <typename T, typename ZT>
+__global__ __launch_bounds__(256) void topk_rows(TopKArgs a, const T* __restrict__ x, T* __restrict__ v, ZT* __restrict__ idx) {
+  using A = typename Conv<T>::acc;
+  __shared__ A wv[4];
+  __shared__ int wi[4];
+  extern __shared__ __attribute__((aligned(8))) unsigned char picked_raw[];   // k picks when an index sort follows
+  int* pickedIdx = reinterpret_cast<int*>(picked_raw);
+  const LongType row = blockIdx.x;
+  const LongType xb = walk<LongType>(a.outerX, row), vb = walk<LongType>(a.outerV, row), ib = walk<LongType>(a.outerI, row);
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const A LOWEST = -(A)INFINITY;
+  A pv = (A)INFINITY;
+  int pi = -1;
+  for (int j = 0; j < a.k; j++) {
+    A bv = LOWEST;
+    int bi = 0x7fffffff;
+    for (LongType e = t; e < a.rowLen; e += 256) {
+      A c = (A)to_float(x[xb + e * a.xInner]);
+      c = c == c ? c : LOWEST;                                    // NaN below everything
+      const bool after = pickBefore<A>(pv, pi, c, (int)e);       // strictly after the previous pick
+      if (after && pickBefore<A>(c, (int)e, bv, bi)) { bv = c; bi = (int)e; }
+    }
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) {
+      const A ov = __shfl_xor(bv, m, WAVE);
+      const int oi = __shfl_xor(bi, m, WAVE);
+      if (pickBefore<A>(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+    }
+    __syncthreads();
+    if (lane == 0) { wv[wave] = bv; wi[wave] = bi; }
+    __syncthreads();
+    bv = wv[0]; bi = wi[0];
+#pragma unroll
+    for (int w = 1; w < 4; w++) if (pickBefore<A>(wv[w], wi[w], bv, bi)) { bv = wv[w]; bi = wi[w]; }
+    pv = bv; pi = bi;
+    if (a.sorted) {
+      if (t == 0) {
+        if (v) v[vb + j * a.vInner] = x[xb + (LongType)bi * a.xInner];
+        if (idx) idx[ib + j * a.iInner] = (ZT)bi;
+      }
+    } else if (t == 0) {
+      pickedIdx[j] = bi;
+    }
+  }
+  if (!a.sorted) {
+    __syncthreads();
+    if (t == 0) {
+      for (int j = 1; j < a.k; j++) {           // insertion sort by index (k is small)
+        const int cur = pickedIdx[j];
+        int q = j - 1;
+        while (q >= 0 && pickedIdx[q] > cur) { pickedIdx[q + 1] = pickedIdx[q]; q--; }
+        pickedIdx[q + 1] = cur;
+      }
+      for (int j = 0; j < a.k; j++) {
+        if (v) v[vb + j * a.vInner] = x[xb + (LongType)pickedIdx[j] * a.xInner];
+        if (idx) idx[ib + j * a.iInner] = (ZT)pickedIdx[j];
+      }
+    }
+  }
+}
+
+template <typename T>
+static void topkTyped(hipStream_t st, const TopKArgs& a, DataType idt, const void* x, void* v, void* idx) {
+  const size_t lds = a.sorted ? 0 : (size_t)a.k * sizeof(int);
+  if (idt == INT64) hipLaunchKernelGGL((topk_rows<T, LongType>), dim3((unsigned)a.rows), dim3(256), lds, st, a, (const T*)x, (T*)v, (LongType*)idx);
+  else if (idt == INT32) hipLaunchKernelGGL((topk_rows<T, int>), dim3((unsigned)a.rows), dim3(256), lds, st, a, (const T*)x, (T*)v, (int*)idx);
+  else ND4J_THROW("top_k: indices must be INT32 or INT64");
+}
+void launchTopK(hipStream_t st, DataType xdt, DataType idt, const void* x, void* values, void* indices, const RowPlan& pv,
+                const RowPlan& pi, int k, bool sorted) {
+  if (pv.rows == 0 || k == 0) return;
+  ND4J_REQUIRE(pv.rowLen < 0x7fffffffLL && pv.rows < 0x7fffffffLL, "top_k: array too large");
+  ND4J_REQUIRE(k <= 4096, "top_k: nd4j-hip selects at most 4096 elements per row");
+  TopKArgs a;
+  a.outerX = pv.outerX; a.outerV = pv.outerZ; a.outerI = pi.outerZ;
+  a.rows = pv.rows; a.rowLen = pv.rowLen; a.xInner = pv.xInner; a.vInner = pv.zInner; a.iInner = pi.zInner;
+  a.k = k; a.sorted = sorted ? 1 : 0;
+  switch (xdt) {
+    case FLOAT32: topkTyped<float>(st, a, idt, x, values, indices); break;
+    case DOUBLE: topkTyped<double>(st, a, idt, x, values, indices); break;
+    case HALF: topkTyped<f16_t>(st, a, idt, x, values, indices); break;
+    case BFLOAT16: topkTyped<bf16_t>(st, a, idt, x, values, indices); break;
+    default: ND4J_THROW("top_k: nd4j-hip implements floating point inputs");
+  }
+  HIP_CHECK(hipGetLastError());
+}
+
 }  // namespace nd4jhip

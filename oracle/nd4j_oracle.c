@@ -608,6 +608,77 @@ int orc_index_reduce(int opNum, const void *x, const int64_t *xsi, void *z, cons
 }
 
 /* ---------------------------------------------------------------------------------------------
+ * top_k                                        ops/declarable/generic/parity_ops/top_k.cpp:31-57
+ *   -> ops/declarable/helpers/cpu/top_k.cpp:34-125, restated literally, quirks included:
+ *   k == 1: first maximum (strict <).  k > 1: the first k elements seed the candidate set; a later
+ *   element enters only if it exceeds the current minimum AND equals no candidate (std::binary_search
+ *   over the sorted copy), replacing the first candidate equal to that minimum.  needSort: values
+ *   descending, and every position is re-derived as the LAST j with x[j] == value (so equal values
+ *   share one position); else the candidates are ordered by their recorded positions (std::map).
+ *   Values are compared as doubles (exact for every supported storage type).
+ * ------------------------------------------------------------------------------------------- */
+static int cmp_asc(const void *a, const void *b) { double x = *(const double *)a, y = *(const double *)b; return (x > y) - (x < y); }
+int orc_top_k(const void *x, const int64_t *xsi, void *values, const int64_t *vsi, void *indices, const int64_t *isi,
+              int64_t k, int needSort) {
+  int r = si_rank(xsi), dt = orc_dtype(xsi), idt = orc_dtype(isi);
+  if (r < 1) return 3;
+  int64_t width = si_shape(xsi)[r - 1];
+  if (k < 1 || k > width) return 3;
+  if (idt != ORC_INT64 && idt != ORC_INT32) return 2;
+  int64_t rows = orc_length(xsi) / width;
+  const int64_t *xs = si_stride(xsi), *vs = si_stride(vsi), *is = si_stride(isi);
+  double *top = (double *)malloc(sizeof(double) * (size_t)k), *sorted = (double *)malloc(sizeof(double) * (size_t)k);
+  int64_t *tix = (int64_t *)malloc(sizeof(int64_t) * (size_t)k);
+  for (int64_t e = 0; e < rows; e++) {
+    int64_t xb = walk(r - 1, si_shape(xsi), xs, e), vb = walk(r - 1, si_shape(vsi), vs, e), ib = walk(r - 1, si_shape(isi), is, e);
+#define XV(j) ld(x, dt, xb + (j) * xs[r - 1])
+    if (k == 1) {
+      int64_t maxPos = 0;
+      double maxVal = XV(0);
+      for (int64_t pos = 1; pos < width; pos++) if (maxVal < XV(pos)) { maxPos = pos; maxVal = XV(pos); }
+      top[0] = maxVal; tix[0] = maxPos;
+    } else {
+      for (int64_t pos = 0; pos < k; pos++) { tix[pos] = pos; top[pos] = XV(pos); sorted[pos] = top[pos]; }
+      qsort(sorted, (size_t)k, sizeof(double), cmp_asc);
+      for (int64_t i = k; i < width; i++) {
+        double val = XV(i), minTop = sorted[0];
+        if (minTop < val) {
+          int exists = 0;
+          { int64_t lo = 0, hi = k; while (lo < hi) { int64_t mid = (lo + hi) / 2; if (sorted[mid] < val) lo = mid + 1; else hi = mid; }
+            exists = lo < k && !(val < sorted[lo]); }
+          if (!exists) {
+            int64_t pos = 0;
+            while (pos < k && top[pos] != sorted[0]) pos++;
+            if (pos < k) { top[pos] = val; tix[pos] = i; }   /* std::find returning end() would write past the array */
+            sorted[0] = val;
+            qsort(sorted, (size_t)k, sizeof(double), cmp_asc);
+          }
+        }
+      }
+      if (needSort) {
+        qsort(top, (size_t)k, sizeof(double), cmp_asc);
+        for (int64_t a = 0, b = k - 1; a < b; a++, b--) { double tmp = top[a]; top[a] = top[b]; top[b] = tmp; }   /* descending */
+        for (int64_t j = 0; j < width; j++) for (int64_t pos = 0; pos < k; pos++) if (top[pos] == XV(j)) tix[pos] = j;
+      } else {
+        /* std::map<index, value>: ascending positions, a repeated position keeps its last value */
+        for (int64_t a = 1; a < k; a++) {
+          int64_t ci = tix[a]; double cv = top[a]; int64_t b = a - 1;
+          while (b >= 0 && tix[b] > ci) { tix[b + 1] = tix[b]; top[b + 1] = top[b]; b--; }
+          tix[b + 1] = ci; top[b + 1] = cv;
+        }
+      }
+    }
+#undef XV
+    for (int64_t pos = 0; pos < k; pos++) {
+      if (values) st(values, dt, vb + pos * vs[r - 1], top[pos]);
+      if (indices) { if (idt == ORC_INT64) ((int64_t *)indices)[ib + pos * is[r - 1]] = tix[pos]; else ((int32_t *)indices)[ib + pos * is[r - 1]] = (int32_t)tix[pos]; }
+    }
+  }
+  free(top); free(sorted); free(tix);
+  return 0;
+}
+
+/* ---------------------------------------------------------------------------------------------
  * softmax                                     ops/declarable/generic/nn/softmax.cpp:37-52
  *   -> ops/declarable/helpers/cpu/softmax.cpp:36-107 (vector), :252-353 (TAD loop / fallback)
  * same-shape-strict branch: max over finite values only (0 if none), inf/nan inputs mapped to

@@ -28,6 +28,9 @@
  *   reduce same/float ................. NativeOpsTests.cpp:209-238, fp64 bounds
  *   index reduce / argmax ............. NativeOpsTests.cpp:84-117, LegacyOpsTests.cpp:279-310,
  *                                       DeclarableOpsTests1.cpp:2197-2300, brute force
+ *   top_k ............................. DeclarableOpsTests5.cpp:1074-1245 (Test_TopK_0..5), brute force
+ *                                       on tie-free rows; behaviour on repeated values: source only
+ *   xw_plus_b ......................... composition of matmul and the bias row (xw_plus_b.cpp:117-133)
  *   matmul ............................ DeclarableOpsTests14.cpp:601-1260, DeclarableOpsTests19.cpp:52-140
  *   softmax ........................... DeclarableOpsTests1.cpp:2523-2740; inf/nan clamp
  *                                       semantics: parity unpinned (source only)
@@ -79,6 +82,8 @@ int orc_index_reduce(int opNum, const void *x, const int64_t *xsi, void *z, cons
                      int ndims);
 
 /* declarable ops */
+int orc_top_k(const void *x, const int64_t *xsi, void *values, const int64_t *vsi, void *indices, const int64_t *isi,
+              int64_t k, int needSort);
 int orc_softmax(const void *x, const int64_t *xsi, void *z, const int64_t *zsi, int dim, int literal_half);
 int orc_layer_norm(const void *x, const int64_t *xsi, const void *gain, const int64_t *gsi, const void *bias,
                    const int64_t *bsi, void *z, const int64_t *zsi, const int64_t *axes, int naxes, int channelsFirst);

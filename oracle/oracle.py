@@ -58,6 +58,7 @@ def lib():
         for f in (L.orc_reduce_same, L.orc_reduce_float, L.orc_index_reduce):
             f.argtypes = [i32, vp, i64p, vp, i64p, i64p, i32]
         L.orc_softmax.argtypes = [vp, i64p, vp, i64p, i32, i32]
+        L.orc_top_k.argtypes = [vp, i64p, vp, i64p, vp, i64p, i64, i32]
         L.orc_layer_norm.argtypes = [vp, i64p, vp, i64p, vp, i64p, vp, i64p, i64p, i32, i32]
         L.orc_matmul.argtypes = [vp, i64p, vp, i64p, vp, i64p, i32, i32, i32, dbl, dbl, i32]
         L.orc_attention_v2.argtypes = [vp, i64p, vp, i64p, vp, i64p, vp, i64p, vp, i64p, vp, i64p, dbl, i32]
@@ -180,6 +181,12 @@ def reduce_float(op, x, z, dims=None):
 
 def index_reduce(op, x, z, dims=None):
     return _reduce(lib().orc_index_reduce, "index_reduce", op, x, z, dims)
+
+
+def top_k(x, values, indices, k, need_sort=True):
+    x, values, indices = _arr(x), _arr(values), _arr(indices)
+    _check(lib().orc_top_k(_p(x.a), _s(x.si), _p(values.a), _s(values.si), _p(indices.a), _s(indices.si), int(k), int(need_sort)), "top_k")
+    return values.a, indices.a
 
 
 def softmax(x, z, dim=-1, literal_half=False):

@@ -422,3 +422,71 @@ def test_gather_add_concat(ex, oracle):
     b = rng.normal(0, 1, (2, 3, 8)).astype(np.float32)
     c = ex.exec_custom("concat", [NDArray.from_numpy(a), NDArray.from_numpy(b)], i_args=[1])[0]
     assert np.array_equal(c.to_numpy(), np.concatenate([a, b], 1))
+
+
+# ---- top_k ---------------------------------------------------------------------------------------------------------------
+def _topk_cases():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "top_k_vectors.json")) as f:
+        return json.load(f)["cases"]
+
+
+@pytest.mark.parametrize("case", _topk_cases(), ids=lambda c: c["name"])
+def test_golden_top_k(ex, case):
+    order = case["order"]
+    x = np.array(case["x"], np.float64).reshape(case["shape"], order=order.upper())
+    dx = NDArray.from_numpy(x, DOUBLE, order=order)
+    v, i = ex.exec_custom("top_k", [dx], i_args=[case["k"]], b_args=[case["sort"]])
+    assert v.shape == tuple(case["zshape"]) and i.shape == tuple(case["zshape"]) and i.dtype == INT64
+    assert np.array_equal(v.to_numpy(), np.array(case["v"], np.float64).reshape(case["zshape"], order=order.upper()))
+    assert np.array_equal(i.to_numpy(), np.array(case["i"], np.int64).reshape(case["zshape"], order=order.upper()))
+
+
+@pytest.mark.parametrize("shape,k", [((32, 50257), 40), ((3, 5, 129), 5), ((7, 64), 64), ((2, 4097), 1)])
+@pytest.mark.parametrize("sort", [True, False])
+def test_top_k_vs_oracle_distinct_values(ex, oracle, shape, k, sort):
+    """Indices are bit-exact against the reference's algorithm wherever a row's values are pairwise different."""
+    rng = np.random.default_rng(k + shape[-1])
+    n = shape[-1]
+    rows = int(np.prod(shape[:-1]))
+    # every row a shuffled ramp: pairwise distinct floats (random normal draws of this length repeat values)
+    x = np.stack([rng.permutation(n) for _ in range(rows)]).astype(np.float32).reshape(shape) * np.float32(0.25) - np.float32(100)
+    ov = np.zeros(shape[:-1] + (k,), np.float32)
+    oi = np.zeros(shape[:-1] + (k,), np.int64)
+    oracle.top_k(x, ov, oi, k, sort)
+    v, i = ex.exec_custom("top_k", [NDArray.from_numpy(x)], i_args=[k], b_args=[sort])
+    assert np.array_equal(i.to_numpy(), oi)
+    assert np.array_equal(v.to_numpy(), ov)
+
+
+def test_top_k_types_views_ties_and_errors(ex, oracle):
+    rng = np.random.default_rng(3)
+    # bf16 values, int32 indices, k from a second input, permuted input view
+    vals = rng.permutation(240).astype(np.float32).reshape(6, 40) - 100.0      # exact in bf16, pairwise distinct
+    dx = NDArray.from_numpy(np.ascontiguousarray(vals.T), BFLOAT16).permute(1, 0)   # [6, 40] view with strides [1, 6]
+    ox = oracle.Arr(f32_to_bf16_bits(vals), oracle.BFLOAT16)
+    ov, oi = oracle.Arr(np.zeros((6, 4), np.uint16), oracle.BFLOAT16), np.zeros((6, 4), np.int64)
+    oracle.top_k(ox, ov, oi, 4, True)
+    kk = NDArray.from_numpy(np.array([4], np.int32))
+    v, i = ex.exec_custom("top_k", [dx, kk], [NDArray.empty((6, 4), BFLOAT16), NDArray.empty((6, 4), INT32)])
+    assert np.array_equal(i.to_numpy(), oi.astype(np.int32))
+    assert np.array_equal(v.to_numpy(), ov.a)
+    # k = 1: the first maximum wins, as in the reference
+    t = np.array([[1, 9, 3, 9, 2], [5, 5, 5, 5, 5]], np.float32)
+    ov1, oi1 = np.zeros((2, 1), np.float32), np.zeros((2, 1), np.int64)
+    oracle.top_k(t, ov1, oi1, 1, True)
+    v1, i1 = ex.exec_custom("top_k", [NDArray.from_numpy(t)], i_args=[1])
+    assert np.array_equal(i1.to_numpy(), oi1) and list(i1.to_numpy().ravel()) == [1, 0]
+    # k > 1 with repeated values: the k largest elements, ties to the lower index (the reference's loop differs here)
+    v2, i2 = ex.exec_custom("top_k", [NDArray.from_numpy(t)], i_args=[3])
+    assert np.array_equal(i2.to_numpy(), np.array([[1, 3, 2], [0, 1, 2]]))
+    assert np.array_equal(v2.to_numpy(), np.array([[9, 9, 3], [5, 5, 5]], np.float32))
+    # NaN sorts below every number
+    tn = np.array([[np.nan, 2, 7, np.nan, 4]], np.float32)
+    _, i3 = ex.exec_custom("top_k", [NDArray.from_numpy(tn)], i_args=[3])
+    assert list(i3.to_numpy().ravel()) == [2, 4, 1]
+    with pytest.raises(NativeOpsError, match="k should not be greater than last dimension"):
+        ex.exec_custom("top_k", [NDArray.from_numpy(t)], [NDArray.empty((2, 6), FLOAT32), NDArray.empty((2, 6), INT64)], i_args=[6])
+    with pytest.raises(NativeOpsError, match="k should be positive"):
+        ex.exec_custom("top_k", [NDArray.from_numpy(t)], i_args=[0])

@@ -359,3 +359,37 @@ def test_attention_is_matmul_softmax_matmul(oracle):
     assert_close(w, p, 1e-5, 1e-7, "causal weights")
     assert_close(out, p @ v.astype(np.float64), 1e-5, 1e-6, "causal out")
     assert (w[:, 0, 1:] < 1e-30).all() and w[:, 0, 0] == pytest.approx(1.0)
+
+
+# ---- top_k --------------------------------------------------------------------------------------------------------------
+def _topk_cases():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "top_k_vectors.json")) as f:
+        return json.load(f)["cases"]
+
+
+@pytest.mark.parametrize("case", _topk_cases(), ids=lambda c: c["name"])
+def test_golden_top_k(oracle, case):
+    """Known answers of the reference's own top_k tests ('f'-ordered buffers are laid out as the reference lays them out)."""
+    order = case["order"].upper()
+    x = np.array(case["x"], np.float64).reshape(case["shape"], order=order)
+    v = np.zeros(case["zshape"], np.float64, order=order)
+    i = np.zeros(case["zshape"], np.int64, order=order)
+    oracle.top_k(x, v, i, case["k"], case["sort"])
+    assert np.array_equal(v, np.array(case["v"], np.float64).reshape(case["zshape"], order=order))
+    assert np.array_equal(i, np.array(case["i"], np.int64).reshape(case["zshape"], order=order))
+
+
+def test_top_k_brute_force_on_distinct_values(oracle):
+    rng = np.random.default_rng(7)
+    for shape, k in [((5, 17), 3), ((2, 3, 40), 7), ((1, 1000), 40), ((4, 9), 9)]:
+        x = rng.permutation(int(np.prod(shape))).astype(np.float32).reshape(shape)   # pairwise distinct
+        v = np.zeros(shape[:-1] + (k,), np.float32)
+        i = np.zeros(shape[:-1] + (k,), np.int64)
+        oracle.top_k(x, v, i, k, True)
+        want_i = np.argsort(-x, axis=-1, kind="stable")[..., :k]
+        assert np.array_equal(i, want_i)
+        assert np.array_equal(v, np.take_along_axis(x, want_i, -1))
+        oracle.top_k(x, v, i, k, False)
+        assert np.array_equal(i, np.sort(want_i, axis=-1))
