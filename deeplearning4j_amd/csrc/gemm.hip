@@ -531,9 +531,10 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16f(GemmArgs g, const T
 // Whole-tile kernel whose global loads write LDS directly (global_load_lds_dwordx4): no staging registers, no LDS
 // write instructions, and the data of K-tile kt+2 travels while tile kt is multiplied.  A wave-wide load deposits
 // its 64 x 16 bytes contiguously in lane order, so the LDS layouts are chosen per lane on the global side:
-//   k-contiguous operand (A, transposed B): a 1 KiB chunk holds 16 rows x 4 k-groups (8 k each); slot 4j + c of the
-//     chunk holds row j, k-group (c + j/4) % 4.  Four neighbouring lanes fetch 64 contiguous bytes of a row, and the
-//     16 rows a fragment read touches per LDS pass fall into 16 different 16-byte bank groups.
+//   k-contiguous operand (A, transposed B): a 1 KiB chunk holds 8 rows x 8 k-groups (8 k each), i.e. the whole
+//     128-byte line of each row; slot 8j + p of chunk q holds row j, k-group (p - 4 (q%2) - j/2) % 8.  Eight
+//     neighbouring lanes fetch one full line, and the 16 rows a fragment read touches per LDS pass fall into 16
+//     different 16-byte bank groups.
 //   row-major B ([k][n], n contiguous): a 1 KiB chunk holds two k-rows of 256 n; the 16-byte column group c of row k
 //     sits at position c ^ 4 (k % 4).  Fragments come out of LDS through the transposing read ds_read_b64_tr_b16:
 //     in a group of 16 lanes, lane R hands in the address of B[k0 + R/4][n0 + 4 (R%4) ..+3] and lane i receives
@@ -563,16 +564,17 @@ __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restr
   const int wm = wave / WN, wn = wave % WN;
 
   // ---- global side: this wave's four chunks of each operand ------------------------------------------------------
-  // k-contiguous operand, chunk id cw = wave * 4 + i: rows (cw / 2) * 16 .. +15, k-groups (cw % 2) * 4 .. +3
-  const int lj = lane >> 2, lc = lane & 3, lkg = (lc + (lj >> 2)) & 3;
+  // k-contiguous operand, chunk id cw = wave * 4 + i: rows cw * 8 .. +7, all 8 k-groups (a whole 128-byte line per row)
+  const int lj = lane >> 3, lp = lane & 7;
   const T* aSrc[4];
   const T* bSrc[4];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     const int cw = wave * 4 + i;
-    aSrc[i] = A + (m0 + (cw >> 1) * 16 + lj) * lda + ((cw & 1) * 4 + lkg) * 8;
+    const int lkg = (lp - 4 * (cw & 1) - (lj >> 1)) & 7;
+    aSrc[i] = A + (m0 + cw * 8 + lj) * lda + lkg * 8;
     if (B_KC) {
-      bSrc[i] = B + (n0 + (cw >> 1) * 16 + lj) * ldb + ((cw & 1) * 4 + lkg) * 8;
+      bSrc[i] = B + (n0 + cw * 8 + lj) * ldb + lkg * 8;
     } else {
       const int kr = 2 * cw + (lane >> 5), q = lane & 31, c = q ^ (4 * (kr & 3));
       bSrc[i] = B + (LongType)kr * ldb + n0 + 8 * c;
@@ -593,21 +595,22 @@ __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restr
   };
 
   // ---- LDS side: fragment addresses ---------------------------------------------------------------------------------
-  // k-contiguous layout: row r, k-group kg = 2 ks + h -> chunk (r / 16) * 2 + ks / 2, slot 4 j + ((kg % 4 - j / 4) & 3)
-  int offA[TM][2], offB[TN][2];
+  // k-contiguous layout: row r, k-group kg = 2 ks + h -> chunk r / 8, slot 8 (r % 8) + ((kg + 4 (r / 8 % 2) + r % 8 / 2) & 7)
+  int offA[TM][4], offB[TN][4];
 #pragma unroll
   for (int i = 0; i < TM; i++) {
-    const int r = wm * WTM + i * 32 + (lane & 31), j = r & 15;
+    const int r = wm * WTM + i * 32 + (lane & 31);
 #pragma unroll
-    for (int par = 0; par < 2; par++) offA[i][par] = (r >> 4) * 128 + 4 * j + ((2 * par + h - (j >> 2)) & 3);
+    for (int ks = 0; ks < 4; ks++) offA[i][ks] = (r >> 3) * 64 + 8 * (r & 7) + ((2 * ks + h + 4 * ((r >> 3) & 1) + ((r & 7) >> 1)) & 7);
   }
   int trB[TN];   // byte offsets of the transposing reads (row-major B)
 #pragma unroll
   for (int jt = 0; jt < TN; jt++) {
     if (B_KC) {
-      const int r = wn * WTN + jt * 32 + (lane & 31), j = r & 15;
+      const int r = wn * WTN + jt * 32 + (lane & 31);
 #pragma unroll
-      for (int par = 0; par < 2; par++) offB[jt][par] = SLOTS_OP + (r >> 4) * 128 + 4 * j + ((2 * par + h - (j >> 2)) & 3);
+      for (int ks = 0; ks < 4; ks++)
+        offB[jt][ks] = SLOTS_OP + (r >> 3) * 64 + 8 * (r & 7) + ((2 * ks + h + 4 * ((r >> 3) & 1) + ((r & 7) >> 1)) & 7);
       trB[jt] = 0;
     } else {
       const int grp = lane >> 4, i16 = lane & 15;
@@ -615,17 +618,17 @@ __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restr
       const int k = 8 * (grp >> 1) + (i16 >> 2);                       // + 16 ks + 4 rd
       const int phys = (n4 >> 3) ^ (4 * ((i16 >> 2) & 3));
       trB[jt] = SLOTS_OP * 16 + k * 512 + phys * 16 + ((n4 >> 2) & 1) * 8;
-      offB[jt][0] = offB[jt][1] = 0;
+      offB[jt][0] = offB[jt][1] = offB[jt][2] = offB[jt][3] = 0;
     }
   }
   u32x4 fa[2][TM], fb[2][TN];
   auto readFrag = [&](const u32x4* stage, int ks, int buf) {
 #pragma unroll
-    for (int i = 0; i < TM; i++) fa[buf][i] = stage[offA[i][ks & 1] + (ks >> 1) * 64];
+    for (int i = 0; i < TM; i++) fa[buf][i] = stage[offA[i][ks]];
 #pragma unroll
     for (int jt = 0; jt < TN; jt++) {
       if (B_KC) {
-        fb[buf][jt] = stage[offB[jt][ks & 1] + (ks >> 1) * 64];
+        fb[buf][jt] = stage[offB[jt][ks]];
       } else {
         const __attribute__((address_space(3))) unsigned char* base =
             (const __attribute__((address_space(3))) unsigned char*)(lds_ptr)stage + trB[jt] + ks * 8192;
