@@ -560,7 +560,7 @@ __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restr
   const LongType bz = blockIdx.z;
   { LongType oa, ob, oc; batchOffsets(g, bz, oa, ob, oc); A += oa; B += ob; C += oc; }
   const LongType lda = g.aRow, ldb = B_KC ? g.bCol : g.bRow;
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, h = lane >> 5;
+  const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6), h = lane >> 5;
   const int wm = wave / WN, wn = wave % WN;
 
   // ---- global side: this wave's four chunks of each operand ------------------------------------------------------
