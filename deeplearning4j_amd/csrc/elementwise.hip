@@ -103,6 +103,176 @@ PAIRWISE(P_MIN, a < b ? a : b);      // ops.h:110-115
 PAIRWISE(P_RDIV, b / a);             // ops.h:64
 PAIRWISE(P_SQSUB, (a - b) * (a - b)); // ops.h:174
 
+// ---- the long tail of the op tables: op picked at run time inside one kernel per dtype ------------------------
+// Formulas restate ops/ops.h and math/templatemath.h of the reference (line numbers beside each case).  A = float
+// for the half/bfloat16/float flavours, double for double.
+template <typename A> struct Tm;
+template <> struct Tm<float> {
+  static __device__ __forceinline__ float exp_(float x) { return expf(x); }
+  static __device__ __forceinline__ float log_(float x) { return logf(x); }
+  static __device__ __forceinline__ float cosh_(float x) { return coshf(x); }
+  static __device__ __forceinline__ float sinh_(float x) { return sinhf(x); }
+  static __device__ __forceinline__ float tan_(float x) { return tanf(x); }
+  static __device__ __forceinline__ float acos_(float x) { return acosf(x); }
+  static __device__ __forceinline__ float asin_(float x) { return asinf(x); }
+  static __device__ __forceinline__ float atan_(float x) { return atanf(x); }
+  static __device__ __forceinline__ float acosh_(float x) { return acoshf(x); }
+  static __device__ __forceinline__ float asinh_(float x) { return asinhf(x); }
+  static __device__ __forceinline__ float atanh_(float x) { return atanhf(x); }
+  static __device__ __forceinline__ float erfc_(float x) { return erfcf(x); }
+  static __device__ __forceinline__ float rint_(float x) { return rintf(x); }
+  static __device__ __forceinline__ float round_(float x) { return roundf(x); }
+  static __device__ __forceinline__ float ceil_(float x) { return ceilf(x); }
+  static __device__ __forceinline__ float floor_(float x) { return floorf(x); }
+  static __device__ __forceinline__ float pow_(float a, float b) { return powf(a, b); }
+  static __device__ __forceinline__ float fmod_(float a, float b) { return fmodf(a, b); }
+  static __device__ __forceinline__ float remainder_(float a, float b) { return remainderf(a, b); }
+  static __device__ __forceinline__ float atan2_(float a, float b) { return atan2f(a, b); }
+};
+template <> struct Tm<double> {
+  static __device__ __forceinline__ double exp_(double x) { return exp(x); }
+  static __device__ __forceinline__ double log_(double x) { return log(x); }
+  static __device__ __forceinline__ double cosh_(double x) { return cosh(x); }
+  static __device__ __forceinline__ double sinh_(double x) { return sinh(x); }
+  static __device__ __forceinline__ double tan_(double x) { return tan(x); }
+  static __device__ __forceinline__ double acos_(double x) { return acos(x); }
+  static __device__ __forceinline__ double asin_(double x) { return asin(x); }
+  static __device__ __forceinline__ double atan_(double x) { return atan(x); }
+  static __device__ __forceinline__ double acosh_(double x) { return acosh(x); }
+  static __device__ __forceinline__ double asinh_(double x) { return asinh(x); }
+  static __device__ __forceinline__ double atanh_(double x) { return atanh(x); }
+  static __device__ __forceinline__ double erfc_(double x) { return erfc(x); }
+  static __device__ __forceinline__ double rint_(double x) { return rint(x); }
+  static __device__ __forceinline__ double round_(double x) { return round(x); }
+  static __device__ __forceinline__ double ceil_(double x) { return ceil(x); }
+  static __device__ __forceinline__ double floor_(double x) { return floor(x); }
+  static __device__ __forceinline__ double pow_(double a, double b) { return pow(a, b); }
+  static __device__ __forceinline__ double fmod_(double a, double b) { return fmod(a, b); }
+  static __device__ __forceinline__ double remainder_(double a, double b) { return remainder(a, b); }
+  static __device__ __forceinline__ double atan2_(double a, double b) { return atan2(a, b); }
+};
+// 1 / (1 + e^-x) with the library exponential: derivatives subtract it from one, so it keeps full precision
+template <typename A> __device__ __forceinline__ A exact_sigmoid(A x) { return (A)1 / ((A)1 + Tm<A>::exp_(-x)); }
+template <typename A> __device__ __forceinline__ A sgn_(A x) { return x < (A)0 ? (A)-1 : x > (A)0 ? (A)1 : (A)0; }   // templatemath.h:359-362
+
+template <typename A>
+__device__ __forceinline__ A unary_tail(int k, A x) {
+  using M = Tm<A>;
+  const A one = (A)1;
+  switch (k) {
+    case U_TANH_D: { A t = d_tanh(x); return one - t * t; }                                   // templatemath.h:335-339
+    case U_SIGMOID_D: { A s = exact_sigmoid(x); return s * (one - s); }                       // templatemath.h:343-347
+    case U_SOFTSIGN_D: { A y = one + d_abs(x); return one / (y * y); }                        // templatemath.h:351-355
+    case U_TAN_D: { A c = d_cos(x); return one / (c * c); }                                   // ops.h:169
+    case U_SELU_D: return x > (A)0 ? (A)1.0507009873554804934193349852946                     // ops.h:966-970
+                                   : (A)1.6732632423543772848170429916717 * (A)1.0507009873554804934193349852946 * M::exp_(x);
+    case U_RATIONAL_TANH_D: {                                                                 // ops.h:1076-1086
+      A dis = ((A)2 / (A)3) * x, d2 = dis * dis;
+      A a = one + d_abs(dis) + d2 + (A)1.41645f * d2 * d2;
+      A t = (one + sgn_(dis) * ((A)2 * dis + (A)4 * (A)1.41645f * d2 * dis)) / (a * a);
+      return (A)1.7159f * ((A)2 / (A)3) * t;
+    }
+    case U_RECTIFIED_TANH_D: { if (!(x > (A)0)) return (A)0; A t = d_tanh(x); return one - t * t; }   // ops.h:72-75
+    case U_SWISH_D: { A ex = M::exp_(x), d = ex + one; return (ex * (x + ex + one)) / (d * d); }      // ops.h:993-996
+    case U_ACOSH_D: return one / (d_sqrt(x - one) * d_sqrt(x + one));                          // ops.h:159-160
+    case U_ASINH_D: return one / d_sqrt(x * x + one);                                          // ops.h:155-156
+    case U_SINH_D: return M::cosh_(x);                                                         // ops.h:1048
+    case U_LOG_SIGMOID_D: return one / (M::exp_(x) + one);                                     // ops.h:1042-1045
+    case U_SPECIAL_D: return x * (one - x);                                                    // ops.h:1167
+    case U_CUBE_D: return (A)3 * x * x;                                                        // ops.h:1166
+    case U_ACOS: return M::acos_(x);                                                           // ops.h:364
+    case U_ASIN: return M::asin_(x);                                                           // ops.h:363
+    case U_ATAN: return M::atan_(x);                                                           // ops.h:365
+    case U_HARD_TANH: return x < (A)-1 ? (A)-1 : x > one ? one : x;                            // ops.h:67-70
+    case U_SOFTSIGN: return x / (one + d_abs(x));                                              // templatemath.h:302-306
+    case U_HARD_SIGMOID: { A v = (A)0.2f * x + (A)0.5f; v = v > (A)0 ? v : (A)0; return v < one ? v : one; }   // ops.h:973-976
+    case U_RATIONAL_TANH: {                                                                    // ops.h:1065-1074
+      A dis = ((A)2 / (A)3) * x, d2 = dis * dis;
+      A t = sgn_(dis) * (one - one / (one + d_abs(dis) + d2 + (A)1.41645f * d2 * d2));
+      return (A)1.7159f * t;
+    }
+    case U_RECTIFIED_TANH: { A t = d_tanh(x); return t > (A)0 ? t : (A)0; }                    // ops.h:1093-1095
+    case U_SINH: return M::sinh_(x);                                                           // ops.h:369
+    case U_COSH: return M::cosh_(x);                                                           // ops.h:370
+    case U_TAN: return M::tan_(x);                                                             // ops.h:371
+    case U_SELU: return x > (A)0 ? (A)1.0507009873554804934193349852946 * x                    // ops.h:978-982
+                                 : (A)1.0507009873554804934193349852946 *
+                                       ((A)1.6732632423543772848170429916717 * M::exp_(x) - (A)1.6732632423543772848170429916717);
+    case U_LOG1P: return M::log_(one + x);                                                     // ops.h:375
+    case U_ACOSH: return M::acosh_(x);                                                         // ops.h:368
+    case U_ASINH: return M::asinh_(x);                                                         // ops.h:367
+    case U_RINT: return M::rint_(x);                                                           // ops.h:360
+    case U_LOG_SIGMOID: return M::log_(exact_sigmoid(x));                                      // ops.h:1038-1040
+    case U_ERFC: return M::erfc_(x);                                                           // ops.h:362
+    case U_EXPM1: return M::exp_(x) - one;                                                     // ops.h:378
+    case U_ATANH: return M::atanh_(x);                                                         // ops.h:366
+    case U_GELU_D: {                                                                           // ops.h:1020-1025
+      A x17 = (A)1.702f * x, ep = M::exp_(x17), o = one + ep;
+      return (ep * (o + x17)) / (o * o);
+    }
+    case U_PRECISE_GELU_D: {                                                                   // ops.h:1027-1036
+      A x79 = (A)0.797885 * x, t1 = (A)0.0356774 * x, x03 = t1 * t1 * t1;
+      A x39 = (A)0.398942 * x, t2 = (A)0.0535161 * x, x05 = t2 * t2 * t2;
+      A scz = one / M::cosh_(x79 + x03);
+      return (A)0.5 + (x39 + x05) * (scz * scz) + (A)0.5 * d_tanh(x79 + x03);
+    }
+    case U_MISH: return x * d_tanh(M::log_(one + M::exp_(x)));                                 // ops.h:999-1001
+    case U_MISH_D: {                                                                           // ops.h:1003-1008
+      A ex = M::exp_(x), e2x = ex * ex, e3x = ex * ex * ex, d = (A)2 * ex + e2x + (A)2;
+      return (ex * ((A)4 * (x + one) + (A)4 * e2x + e3x + ex * ((A)4 * x + (A)6))) / (d * d);
+    }
+    case U_ONES: return one;                                                                   // ops.h:481
+    case U_ROUND: return M::round_(x);                                                         // ops.h:359
+    case U_TIMES_ONE_MINUS: return x * (one - x);                                              // ops.h:1165
+    case U_CEIL: return M::ceil_(x);                                                           // ops.h:193
+    case U_FLOOR: return M::floor_(x);                                                         // ops.h:196
+    default: return x;
+  }
+}
+
+// a = element of x, b = element of y or the scalar
+template <typename A>
+__device__ __forceinline__ A binary_tail(int k, A a, A b) {
+  using M = Tm<A>;
+  switch (k) {
+    case P_POW: return M::pow_(a, b);                                                          // ops.h:165
+    case P_REMAINDER: return M::remainder_(a, b);                                              // ops.h:228
+    case P_FMOD: return M::fmod_(a, b);                                                        // ops.h:229
+    case P_ATAN2: return M::atan2_(a, b);                                                      // ops.h:79, templatemath.h:321-324
+    case P_TRUNCATE_DIV: { int ib = (int)b; return ib == 0 ? (A)0 : (A)((int)a / ib); }        // ops.h:240-245 (a zero divisor traps there)
+    case P_FLOOR_DIV: return (A)floor((double)a / (double)b);                                  // op_macros_special.h:87-93
+    case P_FLOOR_MOD: {                                                                        // ops.h:260-267
+      A m = M::fmod_(a, b);
+      return ((a < (A)0) == (b < (A)0)) ? m : M::fmod_(m + b, b);
+    }
+    case P_REVERSE_MOD: { int ia = (int)a; return ia == 0 ? (A)0 : (A)((int)b % ia); }         // ops.h:1747-1752
+    case P_SAFE_DIVIDE: case P_DIVIDE_NO_NAN: return b == (A)0 ? (A)0 : a / b;                 // ops.h:232-233
+    case P_MOD: return a - M::floor_(a / b) * b;                                               // ops.h:1708-1715
+    case P_LOGICAL_OR: return (A)((int)a | (int)b);                                            // ops.h:2423-2428
+    case P_LOGICAL_XOR: return (A)(((int)a | (int)b) & ~((int)a & (int)b));                    // ops.h:2407-2412
+    case P_LOGICAL_NOT: return (A)(!((int)a && (int)b));                                       // ops.h:2399-2404
+    case P_LOGICAL_AND: return (A)((int)a & (int)b);                                           // ops.h:2415-2420
+    case P_AMAX: return d_abs(a) > d_abs(b) ? a : b;                                           // ops.h:89-94
+    case P_AMIN: return d_abs(a) < d_abs(b) ? a : b;                                           // ops.h:96-101
+    case P_TRUNCATE_MOD: { int ib = (int)b; return ib == 0 ? (A)0 : (A)((int)a % ib); }        // ops.h:247-252
+    case P_REPLACE_NANS: return a != a ? b : a;                                                // ops.h:582-587
+    case P_ELU: return a >= (A)0 ? a : b * (M::exp_(a) - (A)1);                                // templatemath.h:233-240
+    case P_ELU_D: return a >= (A)0 ? (A)1 : b * M::exp_(a);                                    // templatemath.h:255-262
+    case P_LEAKY_RELU: return a < (A)0 ? b * a : a;                                            // ops.h:1127-1131
+    case P_LEAKY_RELU_D: return a >= (A)0 ? (A)1 : b;                                          // ops.h:1133-1138
+    case P_LOG_X: return M::log_(a) / M::log_(b);                                              // ops.h:144-149
+    case P_RELU: return a < b ? b : a;                                                         // ops.h:1108-1112
+    case P_RELU6: { A r = a < b ? b : a; return r < (A)6 ? r : (A)6; }                         // ops.h:1122-1125
+    case P_RELU_D: return a > b ? (A)1 : (A)0;                                                 // ops.h:1115-1119
+    case P_STEP: return a > b ? (A)1 : (A)0;                                                   // ops.h:347-350
+    case P_LSTM_CLIP: return a > b ? b : a < -b ? -b : a;                                      // ops.h:337-345
+    case P_SQ_RSUB: { A d = b - a; return d * d; }                                             // op_macros_special.h:820-827
+    case P_REVERSE_POW: return M::pow_(b, a);                                                  // ops.h:166
+    case P_SXE_LOGITS_SMOOTHER: return a * ((A)1 - b) + (A)0.5f * b;                           // ops.h:352-355
+    default: return a;
+  }
+}
+
 // ---- contiguous kernels ------------------------------------------------------------------------------
 // One 16-byte vector per operand and thread, grid = one thread per vector: measured on MI355X this beats
 // grid-stride loops with several vectors in flight.  NT = non-temporal loads/stores, chosen by the host when
@@ -258,6 +428,49 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_generic(DevShape sz, DevShape sx,
   }
 }
 
+// Tail ops: the same access patterns with the op code as a kernel argument (uniform branch per element).
+template <typename T, int NIN>
+__global__ __launch_bounds__(EW_BLOCK) void tail_contig(int k, const T* __restrict__ x, const T* __restrict__ y,
+                                                        T* __restrict__ z, LongType n) {
+  constexpr int V = 16 / sizeof(T);
+  using IO = RawIO<T>;
+  using RT = typename IO::raw;
+  using A = typename Conv<T>::acc;
+  const LongType nvec = n / V;
+  const LongType i = (LongType)blockIdx.x * EW_BLOCK + threadIdx.x;
+  if (i < nvec) {
+    A a[V], b[V];
+    IO::unpack(*(reinterpret_cast<const RT*>(x) + i), a);
+    if (NIN > 1) IO::unpack(*(reinterpret_cast<const RT*>(y) + i), b);
+#pragma unroll
+    for (int e = 0; e < V; e++) a[e] = NIN > 1 ? binary_tail<A>(k, a[e], b[e]) : unary_tail<A>(k, a[e]);
+    *(reinterpret_cast<RT*>(z) + i) = IO::pack(a);
+  }
+  const LongType tail = nvec * V + i;
+  if (tail < n) {
+    A a = (A)to_float(x[tail]);
+    z[tail] = Conv<T>::from(NIN > 1 ? binary_tail<A>(k, a, (A)to_float(y[tail])) : unary_tail<A>(k, a));
+  }
+}
+// any strides, any float dtypes; hasScalar: the second operand is `scalar`
+template <int NIN>
+__global__ __launch_bounds__(EW_BLOCK) void tail_generic(int k, DevShape sz, DevShape sx, DevShape sy, int zdt, int xdt, int ydt,
+                                                         void* z, const void* x, const void* y, LongType n, double scalar,
+                                                         int hasScalar) {
+  const LongType step = (LongType)gridDim.x * EW_BLOCK;
+  for (LongType i = (LongType)blockIdx.x * EW_BLOCK + threadIdx.x; i < n; i += step) {
+    LongType oz = walk<LongType>(sz, i), ox = walk<LongType>(sx, i);
+    double a = load_any(x, xdt, ox), b = scalar;
+    if (NIN > 1 && !hasScalar) b = load_any(y, ydt, walk<LongType>(sy, i));
+    if (zdt == DOUBLE) {
+      store_any(z, zdt, oz, NIN > 1 ? binary_tail<double>(k, a, b) : unary_tail<double>(k, a));
+    } else {
+      float fa = round_as((float)a, zdt), fb = round_as((float)b, zdt);
+      store_any(z, zdt, oz, NIN > 1 ? binary_tail<float>(k, fa, fb) : unary_tail<float>(k, fa));
+    }
+  }
+}
+
 // ---- launch helpers ------------------------------------------------------------------------------------
 static int gridFor(LongType work, int perBlock) {
   LongType blocks = (work + perBlock - 1) / perBlock;
@@ -324,8 +537,32 @@ static void unaryKind(hipStream_t s, DataType xdt, DataType zdt, const void* x, 
   hipLaunchKernelGGL((ew_generic<UnaryAs2<K>, 1>), dim3(gridFor(p.length, EW_BLOCK)), dim3(EW_BLOCK), 0, s, p.own[0], p.own[1], p.own[1], (int)zdt, (int)xdt, (int)xdt, z, x, x, p.length);
 }
 
+template <typename T, int NIN>
+static void tailContigTyped(hipStream_t s, int k, const void* x, const void* y, void* z, LongType n) {
+  constexpr int V = 16 / sizeof(T);
+  const unsigned grid = (unsigned)((n / V + EW_BLOCK) / EW_BLOCK);
+  hipLaunchKernelGGL((tail_contig<T, NIN>), dim3(grid), dim3(EW_BLOCK), 0, s, k, (const T*)x, (const T*)y, (T*)z, n);
+}
+template <int NIN>
+static bool tailContig(hipStream_t s, int k, DataType dt, const void* x, const void* y, void* z, LongType n) {
+  switch (dt) {
+    case FLOAT32: tailContigTyped<float, NIN>(s, k, x, y, z, n); return true;
+    case DOUBLE: tailContigTyped<double, NIN>(s, k, x, y, z, n); return true;
+    case HALF: tailContigTyped<f16_t, NIN>(s, k, x, y, z, n); return true;
+    case BFLOAT16: tailContigTyped<bf16_t, NIN>(s, k, x, y, z, n); return true;
+    default: return false;
+  }
+}
+
 void launchUnary(hipStream_t s, UnaryKind k, DataType xdt, DataType zdt, const void* x, void* z, const EwPlan& p) {
   if (p.length == 0) return;
+  if (k >= U_TAIL_FIRST && k < U_TAIL_END) {
+    if (!(p.sameShape && xdt == zdt && p.contiguous && aligned16(x) && aligned16(z) && tailContig<1>(s, k, xdt, x, x, z, p.length)))
+      hipLaunchKernelGGL((tail_generic<1>), dim3(gridFor(p.length, EW_BLOCK)), dim3(EW_BLOCK), 0, s, (int)k, p.own[0], p.own[1], p.own[1],
+                         (int)zdt, (int)xdt, (int)xdt, z, x, x, p.length, 0.0, 0);
+    HIP_CHECK(hipGetLastError());
+    return;
+  }
   switch (k) {
 #define CASE(K) case K: unaryKind<K>(s, xdt, zdt, x, z, p); break;
     CASE(U_COS) CASE(U_EXP) CASE(U_LOG) CASE(U_SIGMOID) CASE(U_SIN) CASE(U_SOFTPLUS) CASE(U_TANH) CASE(U_SWISH)
@@ -367,6 +604,14 @@ static void pairwiseKind(hipStream_t s, DataType xdt, DataType ydt, DataType zdt
 void launchPairwise(hipStream_t s, PairwiseKind k, DataType xdt, DataType ydt, DataType zdt, const void* x,
                     const void* y, void* z, const EwPlan& p) {
   if (p.length == 0) return;
+  if (k >= P_TAIL_FIRST && k < P_TAIL_END) {
+    if (!(p.sameShape && xdt == zdt && ydt == zdt && p.contiguous && aligned16(x) && aligned16(y) && aligned16(z) &&
+          tailContig<2>(s, k, zdt, x, y, z, p.length)))
+      hipLaunchKernelGGL((tail_generic<2>), dim3(gridFor(p.length, EW_BLOCK)), dim3(EW_BLOCK), 0, s, (int)k, p.own[0], p.own[1], p.own[2],
+                         (int)zdt, (int)xdt, (int)ydt, z, x, y, p.length, 0.0, 0);
+    HIP_CHECK(hipGetLastError());
+    return;
+  }
   switch (k) {
 #define CASE(K) case K: pairwiseKind<K>(s, xdt, ydt, zdt, x, y, z, p); break;
     CASE(P_ADD) CASE(P_COPY) CASE(P_DIV) CASE(P_MUL) CASE(P_RSUB) CASE(P_SUB) CASE(P_MAX) CASE(P_MIN) CASE(P_RDIV)
@@ -475,6 +720,13 @@ static void scalarKind(hipStream_t s, DataType dt, const void* x, double sc, voi
 void launchScalarOp(hipStream_t s, PairwiseKind k, DataType dt, const void* x, double scalar, void* z, const EwPlan& p) {
   if (p.length == 0) return;
   ND4J_REQUIRE(p.sameShape && p.rank >= 1, "scalar op: operands must share a shape");
+  if (k >= P_TAIL_FIRST && k < P_TAIL_END) {
+    // the scalar takes the array's storage type first, as the reference holds it in an array of that type
+    hipLaunchKernelGGL((tail_generic<2>), dim3(gridFor(p.length, EW_BLOCK)), dim3(EW_BLOCK), 0, s, (int)k,
+                       p.own[0], p.own[1], p.own[1], (int)dt, (int)dt, (int)dt, z, x, x, p.length, scalar, 1);
+    HIP_CHECK(hipGetLastError());
+    return;
+  }
   switch (k) {
     case P_ADD: scalarKind<P_ADD>(s, dt, x, scalar, z, p); break;
     case P_SUB: scalarKind<P_SUB>(s, dt, x, scalar, z, p); break;

@@ -15,10 +15,29 @@ enum UnaryKind : int {
   U_SQRT, U_RSQRT,
   // TransformSame (legacy_ops.h:40-44) and TransformAny Assign (legacy_ops.h:46)
   U_ABS, U_NEG, U_SQUARE, U_RECIPROCAL, U_IDENTITY, U_ONE_MINUS, U_CUBE,
-  U_COUNT
+  U_COUNT,
+  // The rest of the transform tables: one kernel per dtype with the op chosen at run time (U_TAIL_FIRST ..).
+  // TransformStrict
+  U_TAIL_FIRST = 64,
+  U_TANH_D = U_TAIL_FIRST, U_SIGMOID_D, U_SOFTSIGN_D, U_TAN_D, U_SELU_D, U_RATIONAL_TANH_D, U_RECTIFIED_TANH_D, U_SWISH_D,
+  U_ACOSH_D, U_ASINH_D, U_SINH_D, U_LOG_SIGMOID_D, U_SPECIAL_D, U_CUBE_D, U_ACOS, U_ASIN, U_ATAN, U_HARD_TANH,
+  U_SOFTSIGN, U_HARD_SIGMOID, U_RATIONAL_TANH, U_RECTIFIED_TANH, U_SINH, U_COSH, U_TAN, U_SELU, U_LOG1P, U_ACOSH,
+  U_ASINH, U_RINT, U_LOG_SIGMOID, U_ERFC, U_EXPM1, U_ATANH, U_GELU_D, U_PRECISE_GELU_D, U_MISH, U_MISH_D,
+  // TransformSame
+  U_ONES, U_ROUND, U_TIMES_ONE_MINUS, U_CEIL, U_FLOOR,
+  U_TAIL_END
 };
 enum PairwiseKind : int {
-  P_ADD, P_COPY, P_DIV, P_MUL, P_RSUB, P_SUB, P_MAX, P_MIN, P_RDIV, P_SQSUB, P_COUNT
+  P_ADD, P_COPY, P_DIV, P_MUL, P_RSUB, P_SUB, P_MAX, P_MIN, P_RDIV, P_SQSUB, P_COUNT,
+  // The rest of the pairwise / scalar / broadcast tables, op chosen at run time (P_TAIL_FIRST ..)
+  P_TAIL_FIRST = 64,
+  P_POW = P_TAIL_FIRST, P_REMAINDER, P_FMOD, P_ATAN2, P_TRUNCATE_DIV, P_FLOOR_DIV, P_FLOOR_MOD, P_REVERSE_MOD,
+  P_SAFE_DIVIDE, P_MOD, P_LOGICAL_OR, P_LOGICAL_XOR, P_LOGICAL_NOT, P_LOGICAL_AND, P_AMAX, P_AMIN, P_TRUNCATE_MOD,
+  P_REPLACE_NANS, P_DIVIDE_NO_NAN,
+  // scalar table only
+  P_ELU, P_ELU_D, P_LEAKY_RELU, P_LEAKY_RELU_D, P_LOG_X, P_RELU, P_RELU6, P_RELU_D, P_STEP, P_LSTM_CLIP,
+  P_SQ_RSUB, P_REVERSE_POW, P_SXE_LOGITS_SMOOTHER,
+  P_TAIL_END
 };
 
 // Joint iteration plan of up to three operands of equal length.
@@ -47,6 +66,7 @@ void launchScalarOp(hipStream_t s, PairwiseKind k, DataType dt, const void* x, d
 enum ReduceKind : int {
   R_SUM, R_MAX, R_MIN, R_PROD, R_ASUM, R_AMAX, R_AMIN,        // ReduceSame 0..6
   R_MEAN, R_AMEAN, R_NORM1, R_NORM2, R_NORMMAX, R_SQNORM,     // ReduceFloat 0,1,2,3,4,7
+  R_ENTROPY, R_LOG_ENTROPY, R_SHANNON_ENTROPY,               // ReduceFloat 8,9,10
   R_COUNT
 };
 enum IndexKind : int { I_MAX, I_MIN, I_AMAX, I_AMIN, I_COUNT };

@@ -459,6 +459,19 @@ void execTransformStrict(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, Opaqu
     case 22: k = U_COS; break; case 23: k = U_EXP; break; case 24: k = U_LOG; break; case 26: k = U_SIGMOID; break;
     case 27: k = U_SIN; break; case 28: k = U_SOFTPLUS; break; case 29: k = U_TANH; break; case 43: k = U_SWISH; break;
     case 45: k = U_ERF; break; case 53: k = U_GELU; break; case 55: k = U_PRECISE_GELU; break;
+    case 4: k = U_TANH_D; break; case 6: k = U_SIGMOID_D; break; case 7: k = U_SOFTSIGN_D; break; case 8: k = U_TAN_D; break;
+    case 9: k = U_SELU_D; break; case 11: k = U_RATIONAL_TANH_D; break; case 12: k = U_RECTIFIED_TANH_D; break;
+    case 13: k = U_SWISH_D; break; case 14: k = U_ACOSH_D; break; case 15: k = U_ASINH_D; break; case 16: k = U_SINH_D; break;
+    case 17: k = U_LOG_SIGMOID_D; break; case 18: k = U_SPECIAL_D; break; case 21: k = U_CUBE_D; break;
+    case 30: k = U_ACOS; break; case 31: k = U_ASIN; break; case 32: k = U_ATAN; break; case 33: k = U_HARD_TANH; break;
+    case 34: k = U_SOFTSIGN; break; case 36: k = U_HARD_SIGMOID; break; case 37: k = U_RATIONAL_TANH; break;
+    case 38: k = U_RECTIFIED_TANH; break; case 39: k = U_SINH; break; case 40: k = U_COSH; break; case 41: k = U_TAN; break;
+    case 42: k = U_SELU; break; case 44: k = U_LOG1P; break; case 46: k = U_ACOSH; break; case 47: k = U_ASINH; break;
+    case 48: k = U_RINT; break; case 49: k = U_LOG_SIGMOID; break; case 50: k = U_ERFC; break; case 51: k = U_EXPM1; break;
+    case 52: k = U_ATANH; break; case 54: k = U_GELU_D; break; case 56: k = U_PRECISE_GELU_D; break; case 57: k = U_MISH; break;
+    case 58: k = U_MISH_D; break;
+    // 2 ScaledTanh, 3 Affine, 19 Stabilize, 25 SetRange read extra parameters; 5 HardTanhDerivative, 10 HardSigmoidDerivative and
+    // 20 StabilizeFP16 are not restated (their reference macros return the input unchanged / a platform constant)
     default: ND4J_THROW("execTransformStrict: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
   runUnary("execTransformStrict", k, x, z);
@@ -486,6 +499,10 @@ void execTransformSame(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueN
   switch (opNum) {  // loops/legacy_ops.h:40-44
     case 0: k = U_ABS; break; case 3: k = U_NEG; break; case 6: k = U_CUBE; break; case 7: k = U_ONE_MINUS; break;
     case 11: k = U_RECIPROCAL; break; case 12: k = U_SQUARE; break; case 15: case 21: k = U_IDENTITY; break;
+    case 2: k = U_ONES; break; case 4: k = U_ROUND; break; case 5: k = U_TIMES_ONE_MINUS; break; case 17: k = U_CEIL; break;
+    case 18: k = U_FLOOR; break;
+    // 13 CompareAndSetTransform and 19 ClipByValue read extra parameters; 1 Sign is not restated (the reference macro
+    // yields +1 for every non-zero input and -1 for zero)
     default: ND4J_THROW("execTransformSame: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
   runUnary("execTransformSame", k, x, z);
@@ -503,6 +520,13 @@ static PairwiseKind pairwiseKind(int opNum) {
   switch (opNum) {  // loops/legacy_ops.h:121-129
     case 0: return P_ADD; case 1: return P_COPY; case 2: return P_DIV; case 3: return P_MUL; case 5: return P_RSUB;
     case 6: return P_SUB; case 7: return P_MAX; case 8: return P_MIN; case 11: return P_RDIV; case 20: return P_SQSUB;
+    case 4: return P_POW; case 9: return P_COPY; case 14: return P_REMAINDER; case 15: return P_FMOD; case 16: return P_ATAN2;
+    case 17: return P_TRUNCATE_DIV; case 18: return P_FLOOR_DIV; case 19: return P_FLOOR_MOD; case 21: return P_REVERSE_MOD;
+    case 22: return P_SAFE_DIVIDE; case 23: return P_MOD; case 27: return P_LOGICAL_OR; case 28: return P_LOGICAL_XOR;
+    case 29: return P_LOGICAL_NOT; case 30: return P_LOGICAL_AND; case 34: return P_AMAX; case 35: return P_AMIN;
+    case 36: return P_TRUNCATE_MOD; case 37: return P_REPLACE_NANS; case 38: return P_DIVIDE_NO_NAN;
+    // 10 Axpy, 12/13 CompareAnd*, 24-26 relative errors, 31 PowDerivative read extra parameters; 32/33 LogPoissonLoss and
+    // 39/40 IGamma* are not implemented
     default: ND4J_THROW("execPairwiseTransform: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
 }
@@ -551,6 +575,17 @@ void execScalar(Nd4jPointer*, int opNum, OpaqueNDArray xa, OpaqueNDArray za, Opa
   switch (opNum) {  // loops/legacy_ops.h:78-86
     case 0: k = P_ADD; break; case 1: k = P_SUB; break; case 2: k = P_MUL; break; case 3: k = P_DIV; break;
     case 4: k = P_RDIV; break; case 5: k = P_RSUB; break; case 6: k = P_MAX; break; case 13: k = P_MIN; break; case 14: k = P_COPY; break;
+    case 7: k = P_ELU; break; case 8: k = P_ELU_D; break; case 15: k = P_MOD; break; case 16: k = P_REVERSE_MOD; break;
+    case 17: k = P_REMAINDER; break; case 18: k = P_FMOD; break; case 19: k = P_TRUNCATE_DIV; break; case 20: k = P_FLOOR_DIV; break;
+    case 21: k = P_FLOOR_MOD; break; case 22: case 44: k = P_SQ_RSUB; break;   // (x - s)^2 == (s - x)^2
+    case 23: k = P_SAFE_DIVIDE; break; case 24: k = P_AMAX; break; case 25: k = P_AMIN; break; case 26: k = P_ATAN2; break;
+    case 27: k = P_LOGICAL_OR; break; case 28: k = P_LOGICAL_XOR; break; case 29: k = P_LOGICAL_NOT; break;
+    case 30: k = P_LOGICAL_AND; break; case 31: k = P_POW; break; case 34: k = P_SXE_LOGITS_SMOOTHER; break;
+    case 35: k = P_LEAKY_RELU; break; case 36: k = P_LEAKY_RELU_D; break; case 37: k = P_REPLACE_NANS; break;
+    case 38: k = P_LOG_X; break; case 39: k = P_RELU; break; case 40: k = P_RELU6; break; case 41: k = P_STEP; break;
+    case 42: k = P_LSTM_CLIP; break; case 43: k = P_TRUNCATE_MOD; break; case 45: k = P_REVERSE_POW; break;
+    case 46: k = P_DIVIDE_NO_NAN; break; case 49: k = P_RELU_D; break;
+    // 32 PowDerivative, 33 CompareAndSet read extra parameters; 47/48 IGamma* are not implemented
     default: ND4J_THROW("execScalar: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
   if (z->isEmpty()) return;
@@ -591,6 +626,11 @@ void execBroadcast(Nd4jPointer*, int opNum, OpaqueNDArray xa, OpaqueNDArray ya, 
     case 0: k = P_ADD; break; case 1: k = P_SUB; break; case 2: k = P_MUL; break; case 3: k = P_DIV; break;
     case 4: k = P_RDIV; break; case 5: k = P_RSUB; break; case 6: k = P_COPY; break;
     case 13: k = P_MIN; break; case 14: k = P_MAX; break; case 17: k = P_SQSUB; break;
+    case 7: k = P_POW; break; case 15: k = P_AMIN; break; case 16: k = P_AMAX; break; case 18: k = P_FLOOR_MOD; break;
+    case 19: k = P_FLOOR_DIV; break; case 20: k = P_REVERSE_MOD; break; case 21: k = P_SAFE_DIVIDE; break; case 22: k = P_MOD; break;
+    case 23: k = P_TRUNCATE_DIV; break; case 26: k = P_ATAN2; break; case 27: k = P_LOGICAL_OR; break; case 28: k = P_LOGICAL_XOR; break;
+    case 29: k = P_LOGICAL_NOT; break; case 30: k = P_LOGICAL_AND; break; case 31: k = P_DIVIDE_NO_NAN; break;
+    // 32/33 IGamma* and 34 PowDerivative are not implemented
     default: ND4J_THROW("execBroadcast: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
   if (z->isEmpty()) return;
@@ -648,6 +688,8 @@ static ReduceKind reduceFloatKind(int opNum) {
     case 0: return R_MEAN; case 1: return R_AMEAN; case 2: return R_NORM1; case 3: return R_NORM2; case 4: return R_NORMMAX;
     case 5: return R_NORM2;  // NormFrobenius = sqrt(sum |x|^2)
     case 7: return R_SQNORM;
+    case 8: return R_ENTROPY; case 9: return R_LOG_ENTROPY; case 10: return R_SHANNON_ENTROPY;
+    // 6 NormP reads its exponent from the extra parameters
     default: ND4J_THROW("execReduceFloat: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
 }

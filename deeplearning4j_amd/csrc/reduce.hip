@@ -21,8 +21,8 @@
 
 namespace nd4jhip {
 
-enum PreKind { PRE_ID = 0, PRE_ABS = 1, PRE_SQ = 2 };
-enum PostKind { POST_ID = 0, POST_DIV_N = 1, POST_SQRT = 2 };
+enum PreKind { PRE_ID = 0, PRE_ABS = 1, PRE_SQ = 2, PRE_XLOGX = 3, PRE_XLOG2X = 4 };
+enum PostKind { POST_ID = 0, POST_DIV_N = 1, POST_SQRT = 2, POST_NEG = 3, POST_LOG_NEG = 4 };
 
 template <typename Op, typename A> struct Identity;
 template <typename A> struct Identity<SumOp, A> { static __device__ __forceinline__ A v() { return (A)0; } };
@@ -34,12 +34,16 @@ template <int PRE, typename A>
 __device__ __forceinline__ A pre(A x) {
   if (PRE == PRE_ABS) return x < 0 ? -x : x;
   if (PRE == PRE_SQ) return x * x;
+  if (PRE == PRE_XLOGX) return x * (sizeof(A) == 8 ? (A)log((double)x) : (A)logf((float)x));      // ops.h:2147-2153
+  if (PRE == PRE_XLOG2X) return x * (sizeof(A) == 8 ? (A)log2((double)x) : (A)log2f((float)x));   // ops.h:1956-1963
   return x;
 }
 template <typename A>
 __device__ __forceinline__ A post(A s, int kind, LongType n) {
   if (kind == POST_DIV_N) return s / (A)n;
   if (kind == POST_SQRT) return sizeof(A) == 8 ? (A)sqrt((double)s) : (A)sqrtf((float)s);
+  if (kind == POST_NEG) return -s;
+  if (kind == POST_LOG_NEG) return sizeof(A) == 8 ? (A)log((double)-s) : (A)logf((float)-s);      // ops.h:1966-1973
   return s;
 }
 
@@ -252,6 +256,9 @@ void launchReduce(hipStream_t st, ReduceKind k, DataType xdt, DataType zdt, cons
     case R_NORM2: reduceDtype<SumOp, PRE_SQ>(st, xdt, x, z, p, POST_SQRT, scratch, scratchBytes); break;
     case R_NORMMAX: reduceDtype<MaxOp, PRE_ABS>(st, xdt, x, z, p, POST_ID, scratch, scratchBytes); break;
     case R_SQNORM: reduceDtype<SumOp, PRE_SQ>(st, xdt, x, z, p, POST_ID, scratch, scratchBytes); break;
+    case R_ENTROPY: reduceDtype<SumOp, PRE_XLOGX>(st, xdt, x, z, p, POST_NEG, scratch, scratchBytes); break;
+    case R_LOG_ENTROPY: reduceDtype<SumOp, PRE_XLOGX>(st, xdt, x, z, p, POST_LOG_NEG, scratch, scratchBytes); break;
+    case R_SHANNON_ENTROPY: reduceDtype<SumOp, PRE_XLOG2X>(st, xdt, x, z, p, POST_NEG, scratch, scratchBytes); break;
     default: ND4J_THROW("reduce: unknown op kind");
   }
   HIP_CHECK(hipGetLastError());

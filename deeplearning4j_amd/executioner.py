@@ -20,12 +20,19 @@ from .ndarray import BOOL, DOUBLE, FLOAT32, HALF, BFLOAT16, INT32, INT64, NDArra
 
 # opNum tables: libnd4j/include/loops/legacy_ops.h
 class Pairwise:
-    Add, CopyPws, Divide, Multiply, ReverseSubtract, Subtract, MaxPairwise, MinPairwise = 0, 1, 2, 3, 5, 6, 7, 8
-    ReverseDivide, SquaredSubtract = 11, 20
+    Add, CopyPws, Divide, Multiply, Pow, ReverseSubtract, Subtract, MaxPairwise, MinPairwise, Copy2 = 0, 1, 2, 3, 4, 5, 6, 7, 8, 9
+    ReverseDivide, Remainder, FMod, Atan2, TruncateDiv, FloorDiv, FloorMod, SquaredSubtract = 11, 14, 15, 16, 17, 18, 19, 20
+    ReverseMod, SafeDivide, Mod, LogicalOr, LogicalXor, LogicalNot, LogicalAnd = 21, 22, 23, 27, 28, 29, 30
+    AMaxPairwise, AMinPairwise, TruncateMod, ReplaceNans, DivideNoNan = 34, 35, 36, 37, 38
 
 
 class TransformStrict:
     Cosine, Exp, Log, Sigmoid, Sin, SoftPlus, Tanh, Swish, Erf, GELU, PreciseGELU = 22, 23, 24, 26, 27, 28, 29, 43, 45, 53, 55
+    TanhDerivative, SigmoidDerivative, SoftSignDerivative, TanDerivative, SELUDerivative = 4, 6, 7, 8, 9
+    RationalTanhDerivative, RectifiedTanhDerivative, SwishDerivative, ACoshDerivative, ASinhDerivative = 11, 12, 13, 14, 15
+    SinhDerivative, LogSigmoidDerivative, SpecialDerivative, CubeDerivative = 16, 17, 18, 21
+    ACos, ASin, ATan, HardTanh, SoftSign, HardSigmoid, RationalTanh, RectifiedTanh, Sinh, Cosh, Tan, SELU = 30, 31, 32, 33, 34, 36, 37, 38, 39, 40, 41, 42
+    Log1p, ACosh, ASinh, Rint, LogSigmoid, Erfc, Expm1, ATanh, GELUDerivative, PreciseGELUDerivative, Mish, MishDerivative = 44, 46, 47, 48, 49, 50, 51, 52, 54, 56, 57, 58
 
 
 class TransformFloat:
@@ -33,7 +40,7 @@ class TransformFloat:
 
 
 class TransformSame:
-    Abs, Neg, Cube, OneMinus, Reciprocal, Square, Identity, Copy = 0, 3, 6, 7, 11, 12, 15, 21
+    Abs, Ones, Neg, Round, TimesOneMinus, Cube, OneMinus, Reciprocal, Square, Identity, Ceiling, Floor, Copy = 0, 2, 3, 4, 5, 6, 7, 11, 12, 15, 17, 18, 21
 
 
 class ReduceSame:
@@ -41,7 +48,7 @@ class ReduceSame:
 
 
 class ReduceFloat:
-    Mean, AMean, Norm1, Norm2, NormMax, NormFrobenius, SquaredNorm = 0, 1, 2, 3, 4, 5, 7
+    Mean, AMean, Norm1, Norm2, NormMax, NormFrobenius, SquaredNorm, Entropy, LogEntropy, ShannonEntropy = 0, 1, 2, 3, 4, 5, 7, 8, 9, 10
 
 
 class IndexReduce:
@@ -49,11 +56,17 @@ class IndexReduce:
 
 
 class Scalar:
-    Add, Subtract, Multiply, Divide, ReverseDivide, ReverseSubtract, MaxPairwise, MinPairwise, CopyPws = 0, 1, 2, 3, 4, 5, 6, 13, 14
+    Add, Subtract, Multiply, Divide, ReverseDivide, ReverseSubtract, MaxPairwise, ELU, ELUDerivative = 0, 1, 2, 3, 4, 5, 6, 7, 8
+    MinPairwise, CopyPws, Mod, ReverseMod, Remainder, FMod, TruncateDiv, FloorDiv, FloorMod, SquaredSubtract = 13, 14, 15, 16, 17, 18, 19, 20, 21, 22
+    SafeDivide, AMaxPairwise, AMinPairwise, Atan2, LogicalOr, LogicalXor, LogicalNot, LogicalAnd, Pow = 23, 24, 25, 26, 27, 28, 29, 30, 31
+    SXELogitsSmoother, LeakyRELU, LeakyRELUDerivative, ReplaceNans, LogX, RELU, RELU6, Step, LstmClip = 34, 35, 36, 37, 38, 39, 40, 41, 42
+    TruncateMod, SquaredReverseSubtract, ReversePow, DivideNoNan, RELUDerivative = 43, 44, 45, 46, 49
 
 
 class Broadcast:
-    Add, Subtract, Multiply, Divide, ReverseDivide, ReverseSubtract, CopyPws = 0, 1, 2, 3, 4, 5, 6
+    Add, Subtract, Multiply, Divide, ReverseDivide, ReverseSubtract, CopyPws, Pow = 0, 1, 2, 3, 4, 5, 6, 7
+    MinPairwise, MaxPairwise, AMinPairwise, AMaxPairwise, SquaredSubtract, FloorMod, FloorDiv, ReverseMod = 13, 14, 15, 16, 17, 18, 19, 20
+    SafeDivide, Mod, TruncateDiv, Atan2, LogicalOr, LogicalXor, LogicalNot, LogicalAnd, DivideNoNan = 21, 22, 23, 26, 27, 28, 29, 30, 31
 
 
 def _reduced_shape(shape, dims, keep_dims):

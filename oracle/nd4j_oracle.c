@@ -299,6 +299,81 @@ static inline double ref_tanhd(double x) {
 static inline float ref_sigmoidf(float x) { return 1.0f / (1.0f + expf(-x)); }   /* templatemath.h:225-229 */
 static inline double ref_sigmoidd(double x) { return 1.0 / (1.0 + exp(-x)); }
 
+/* The rest of the TransformStrict table (loops/legacy_ops.h:54-64), restated from ops/ops.h and
+ * math/templatemath.h (lines beside each case).  One body, expanded for float (libm *f functions, as the
+ * reference's float path uses) and for double.  Not restated: 2 ScaledTanh, 3 Affine, 19 Stabilize, 25 SetRange
+ * (extra parameters), 5 HardTanhDerivative, 10 HardSigmoidDerivative (their macros return the input), 20. */
+#define SELU_A 1.6732632423543772848170429916717
+#define SELU_L 1.0507009873554804934193349852946
+#define STRICT_TAIL(T, M, TANH, SIGM)                                                                         \
+  switch (op) {                                                                                               \
+    case 4: { T t = TANH(x); *out = (T)1 - t * t; return 0; }                 /* templatemath.h:335-339 */   \
+    case 6: { T g = SIGM(x); *out = g * ((T)1 - g); return 0; }               /* templatemath.h:343-347 */   \
+    case 7: { T y = (T)1 + M(fabs)(x); *out = (T)1 / (y * y); return 0; }     /* templatemath.h:351-355 */   \
+    case 8: *out = (T)1 / M(pow)(M(cos)(x), (T)2); return 0;                  /* ops.h:169 */                \
+    case 9: *out = x > (T)0 ? (T)SELU_L : (T)SELU_A * (T)SELU_L * M(exp)(x); return 0;  /* ops.h:966-970 */  \
+    case 11: {                                                                /* ops.h:1076-1086 */          \
+      T dis = ((T)2 / (T)3) * x;                                                                              \
+      T a = (T)1 + M(fabs)(dis) + M(pow)(dis, (T)2) + (T)1.41645f * M(pow)(dis, (T)4);                        \
+      T sg = dis < 0 ? (T)-1 : dis > 0 ? (T)1 : (T)0;                                                         \
+      T td = ((T)1 + sg * ((T)2 * dis + (T)4 * (T)1.41645f * M(pow)(dis, (T)3))) / (a * a);                   \
+      *out = (T)1.7159f * ((T)2 / (T)3) * td; return 0;                                                       \
+    }                                                                                                         \
+    case 12: { if (x > (T)0) { T t = TANH(x); *out = (T)1 - t * t; } else *out = 0; return 0; }  /* ops.h:72-75 */ \
+    case 13: { T ex = M(pow)((T)M_E, x); *out = (ex * (x + ex + (T)1)) / M(pow)(ex + (T)1, (T)2); return 0; } /* ops.h:993-996 */ \
+    case 14: *out = (T)1 / (M(sqrt)(x - (T)1) * M(sqrt)(x + (T)1)); return 0;  /* ops.h:159-160 */           \
+    case 15: *out = (T)1 / M(sqrt)(M(pow)(x, (T)2) + (T)1); return 0;          /* ops.h:155-156 */           \
+    case 16: *out = M(cosh)(x); return 0;                                      /* ops.h:1048 */              \
+    case 17: *out = (T)1 / (M(exp)(x) + (T)1); return 0;                       /* ops.h:1042-1045 */         \
+    case 18: *out = x * ((T)1 - x); return 0;                                  /* ops.h:1167 */              \
+    case 21: *out = (T)3 * x * x; return 0;                                    /* ops.h:1166 */              \
+    case 30: *out = M(acos)(x); return 0;                                      /* ops.h:363-365 */           \
+    case 31: *out = M(asin)(x); return 0;                                                                     \
+    case 32: *out = M(atan)(x); return 0;                                                                     \
+    case 33: *out = x < (T)-1 ? (T)-1 : x > (T)1 ? (T)1 : x; return 0;         /* ops.h:67-70 */             \
+    case 34: *out = x / ((T)1 + M(fabs)(x)); return 0;                         /* templatemath.h:302-306 */  \
+    case 36: { T v = (T)0.2f * x + (T)0.5f; v = v > 0 ? v : 0; *out = v < 1 ? v : 1; return 0; } /* ops.h:973-976 */ \
+    case 37: {                                                                 /* ops.h:1065-1074 */         \
+      T dis = ((T)2 / (T)3) * x;                                                                              \
+      T sg = dis < 0 ? (T)-1 : dis > 0 ? (T)1 : (T)0;                                                         \
+      T th = sg * ((T)1 - ((T)1 / ((T)1 + M(fabs)(dis) + M(pow)(dis, (T)2) + (T)1.41645f * M(pow)(dis, (T)4)))); \
+      *out = (T)1.7159f * th; return 0;                                                                       \
+    }                                                                                                         \
+    case 38: { T t = TANH(x); *out = t > 0 ? t : 0; return 0; }                /* ops.h:1093-1095 */         \
+    case 39: *out = M(sinh)(x); return 0;                                      /* ops.h:369-371 */           \
+    case 40: *out = M(cosh)(x); return 0;                                                                     \
+    case 41: *out = M(tan)(x); return 0;                                                                      \
+    case 42: *out = x > (T)0 ? (T)SELU_L * x : (T)SELU_L * ((T)SELU_A * M(exp)(x) - (T)SELU_A); return 0; /* ops.h:978-982 */ \
+    case 44: *out = M(log)(1 + x); return 0;                                   /* ops.h:375 */               \
+    case 46: *out = M(acosh)(x); return 0;                                     /* ops.h:366-368 */           \
+    case 47: *out = M(asinh)(x); return 0;                                                                    \
+    case 48: *out = M(rint)(x); return 0;                                      /* ops.h:360 */               \
+    case 49: *out = M(log)(SIGM(x)); return 0;                                 /* ops.h:1038-1040 */         \
+    case 50: *out = M(erfc)(x); return 0;                                      /* ops.h:362 */               \
+    case 51: *out = M(exp)(x) - (T)1; return 0;                                /* ops.h:378 */               \
+    case 52: *out = M(atanh)(x); return 0;                                                                    \
+    case 54: {                                                                 /* ops.h:1020-1025 */         \
+      T x17 = (T)1.702f * x, ep = M(exp)(x17), o = (T)1 + ep;                                                 \
+      *out = (ep * (o + x17)) / (o * o); return 0;                                                            \
+    }                                                                                                         \
+    case 56: {                                                                 /* ops.h:1027-1036 */         \
+      T x79 = (T)0.797885 * x, t1 = (T)0.0356774 * x, x03 = t1 * t1 * t1;                                     \
+      T x39 = (T)0.398942 * x, t2 = (T)0.0535161 * x, x05 = t2 * t2 * t2;                                     \
+      T scz = (T)1 / M(cosh)(x79 + x03);                                                                      \
+      *out = (T)0.5 + (x39 + x05) * (scz * scz) + (T)0.5 * TANH(x79 + x03); return 0;                         \
+    }                                                                                                         \
+    case 57: *out = x * TANH(M(log)((T)1 + M(exp)(x))); return 0;              /* ops.h:999-1001 */          \
+    case 58: {                                                                 /* ops.h:1003-1008 */         \
+      T ex = M(exp)(x), e2x = ex * ex, e3x = ex * ex * ex;                                                    \
+      *out = (ex * (4 * (x + 1) + 4 * e2x + e3x + ex * (4 * x + 6))) / M(pow)(2 * ex + e2x + 2, (T)2); return 0; \
+    }                                                                                                         \
+    default: return 1;                                                                                        \
+  }
+#define MF(fn) fn##f
+#define MD(fn) fn
+static int strict_tail_f(int op, float x, float *out) { STRICT_TAIL(float, MF, ref_tanhf, ref_sigmoidf) }
+static int strict_tail_d(int op, double x, double *out) { STRICT_TAIL(double, MD, ref_tanhd, ref_sigmoidd) }
+
 /* TransformStrict opNums                      loops/legacy_ops.h:54-64; functors ops/ops.h:192-200,988-1019 */
 static int strict_f(int op, float x, float *out) {
   switch (op) {
@@ -318,7 +393,7 @@ static int strict_f(int op, float x, float *out) {
       *out = (x / 2.0f) * (1.0f + ref_tanhf(sp * xp));
       return 0;
     }
-    default: return 1;
+    default: return strict_tail_f(op, x, out);
   }
 }
 static int strict_d(int op, double x, double *out) {
@@ -339,7 +414,7 @@ static int strict_d(int op, double x, double *out) {
       *out = (x / 2.0) * (1.0 + ref_tanhd(sp * xp));
       return 0;
     }
-    default: return 1;
+    default: return strict_tail_d(op, x, out);
   }
 }
 
@@ -391,6 +466,60 @@ int orc_transform_float(int opNum, const void *x, const int64_t *xsi, void *z, c
   return 0;
 }
 
+/* TransformSame: loops/legacy_ops.h:40-44; functors ops/ops.h:192-207,359,481,1165.  Not restated: 1 Sign (its
+ * macro yields +1 for every non-zero input), 13 CompareAndSetTransform and 19 ClipByValue (extra parameters). */
+static int same_d(int op, double x, double *out) {
+  switch (op) {
+    case 0: *out = fabs(x); return 0;
+    case 2: *out = 1.0; return 0;
+    case 3: *out = -x; return 0;
+    case 4: *out = round(x); return 0;           /* p_round = round(): halves away from zero */
+    case 5: *out = x * (1.0 - x); return 0;
+    case 6: *out = x * x * x; return 0;
+    case 7: *out = 1.0 - x; return 0;
+    case 11: *out = 1.0 / x; return 0;
+    case 12: *out = x * x; return 0;
+    case 15: case 21: *out = x; return 0;
+    case 17: *out = ceil(x); return 0;
+    case 18: *out = floor(x); return 0;
+    default: return 1;
+  }
+}
+static int same_f(int op, float x, float *out) {
+  switch (op) {
+    case 0: *out = fabsf(x); return 0;
+    case 2: *out = 1.0f; return 0;
+    case 3: *out = -x; return 0;
+    case 4: *out = roundf(x); return 0;
+    case 5: *out = x * (1.0f - x); return 0;
+    case 6: *out = x * x * x; return 0;
+    case 7: *out = 1.0f - x; return 0;
+    case 11: *out = 1.0f / x; return 0;
+    case 12: *out = x * x; return 0;
+    case 15: case 21: *out = x; return 0;
+    case 17: *out = ceilf(x); return 0;
+    case 18: *out = floorf(x); return 0;
+    default: return 1;
+  }
+}
+int orc_transform_same(int opNum, const void *x, const int64_t *xsi, void *z, const int64_t *zsi) {
+  int xdt = orc_dtype(xsi), zdt = orc_dtype(zsi);
+  if (xdt != zdt || !dt_is_float(xdt)) return 2;
+  int64_t n = orc_length(xsi);
+  if (n != orc_length(zsi)) return 3;
+  double pd; if (same_d(opNum, 0.5, &pd)) return 1;
+  PAR_FOR
+  for (int64_t i = 0; i < n; i++) {
+    int64_t xo = orc_offset(xsi, i), zo = orc_offset(zsi, i);
+    if (xdt == ORC_DOUBLE) {
+      double r = 0; same_d(opNum, ((const double *)x)[xo], &r); ((double *)z)[zo] = r;
+    } else {
+      float r = 0; same_f(opNum, ldf(x, xdt, xo), &r); st(z, zdt, zo, r);
+    }
+  }
+  return 0;
+}
+
 /* ---------------------------------------------------------------------------------------------
  * execPairwiseTransform                       legacy/cpu/NativeOps.cpp:1238-1282
  *   -> NativeOpExecutioner_pairwise_floats.cpp:23-68 -> loops/cpu/pairwise.hpp:87-169
@@ -399,6 +528,105 @@ int orc_transform_float(int opNum, const void *x, const int64_t *xsi, void *z, c
  * The reference applies x->offset() twice for views (NativeOps.cpp:1245-1257 on top of buffer());
  * this restatement, like the product, applies it once.
  * ------------------------------------------------------------------------------------------- */
+/* Binary functors by name, shared by the three tables below (ops/ops.h lines beside each). */
+enum {
+  B_ADD, B_COPY, B_DIV, B_MUL, B_RSUB, B_SUB, B_MAX, B_MIN, B_RDIV, B_SQSUB, B_POW, B_REMAINDER, B_FMOD, B_ATAN2,
+  B_TRUNCDIV, B_FLOORDIV, B_FLOORMOD, B_REVMOD, B_SAFEDIV, B_MOD, B_LOR, B_LXOR, B_LNOT, B_LAND, B_AMAX, B_AMIN,
+  B_TRUNCMOD, B_REPLACENANS, B_ELU, B_ELU_D, B_LRELU, B_LRELU_D, B_LOGX, B_RELU, B_RELU6, B_RELU_D, B_STEP,
+  B_LSTMCLIP, B_SQRSUB, B_REVPOW, B_SXE, B_NONE
+};
+#define BINARY_BODY(T, M)                                                                                      \
+  switch (fn) {                                                                                                \
+    case B_ADD: return a + b;                              /* ops.h:56 */                                      \
+    case B_COPY: return b;                                 /* ops.h:312-317 */                                 \
+    case B_DIV: return a / b;                                                                                  \
+    case B_MUL: return a * b;                                                                                  \
+    case B_RSUB: return b - a;                             /* ops.h:63 */                                      \
+    case B_SUB: return a - b;                                                                                  \
+    case B_MAX: return a > b ? a : b;                      /* ops.h:103-108 */                                 \
+    case B_MIN: return a < b ? a : b;                                                                          \
+    case B_RDIV: return b / a;                             /* ops.h:64 */                                      \
+    case B_SQSUB: { T d = a - b; return d * d; }           /* ops.h:174 */                                     \
+    case B_POW: return M(pow)(a, b);                       /* ops.h:165 */                                     \
+    case B_REMAINDER: return M(remainder)(a, b);           /* ops.h:228 */                                     \
+    case B_FMOD: return M(fmod)(a, b);                     /* ops.h:229 */                                     \
+    case B_ATAN2: return M(atan2)(a, b);                   /* ops.h:79; templatemath.h:321-324 */              \
+    case B_TRUNCDIV: return (int)b == 0 ? (T)0 : (T)((int)a / (int)b);   /* ops.h:240-245; a zero divisor traps there */ \
+    case B_FLOORDIV: return (T)floor((double)a / (double)b);   /* op_macros_special.h:87-93 */                 \
+    case B_FLOORMOD: {                                     /* ops.h:260-267 */                                 \
+      T m = M(fmod)(a, b);                                                                                     \
+      return ((a < 0) == (b < 0)) ? m : M(fmod)(m + b, b);                                                     \
+    }                                                                                                          \
+    case B_REVMOD: return (int)a == 0 ? (T)0 : (T)((int)b % (int)a);     /* ops.h:1747-1752 */                 \
+    case B_SAFEDIV: return b == 0 ? (T)0 : a / b;          /* ops.h:232-233 */                                 \
+    case B_MOD: return a - M(floor)(a / b) * b;            /* ops.h:1708-1715 */                               \
+    case B_LOR: return (T)((int)a | (int)b);               /* ops.h:2423-2428 */                               \
+    case B_LXOR: return (T)(((int)a | (int)b) & ~((int)a & (int)b));                                           \
+    case B_LNOT: return (T)(!((int)a && (int)b));                                                              \
+    case B_LAND: return (T)((int)a & (int)b);                                                                  \
+    case B_AMAX: return M(fabs)(a) > M(fabs)(b) ? a : b;   /* ops.h:89-101 */                                  \
+    case B_AMIN: return M(fabs)(a) < M(fabs)(b) ? a : b;                                                       \
+    case B_TRUNCMOD: return (int)b == 0 ? (T)0 : (T)((int)a % (int)b);   /* ops.h:247-252 */                   \
+    case B_REPLACENANS: return isnan(a) ? b : a;           /* ops.h:582-587 */                                 \
+    case B_ELU: return a >= 0 ? a : b * (M(exp)(a) - (T)1);    /* templatemath.h:233-240 */                    \
+    case B_ELU_D: return a >= 0 ? (T)1 : b * M(exp)(a);        /* templatemath.h:255-262 */                    \
+    case B_LRELU: return a < 0 ? b * a : a;                /* ops.h:1127-1131 */                               \
+    case B_LRELU_D: return a >= 0 ? (T)1 : b;              /* ops.h:1133-1138 */                               \
+    case B_LOGX: return M(log)(a) / M(log)(b);             /* ops.h:144-149 */                                 \
+    case B_RELU: return a < b ? b : a;                     /* ops.h:1108-1112 */                               \
+    case B_RELU6: { T r = a < b ? b : a; return r < 6 ? r : (T)6; }                                            \
+    case B_RELU_D: return a > b ? (T)1 : (T)0;                                                                 \
+    case B_STEP: return a > b ? (T)1 : (T)0;               /* ops.h:347-350 */                                 \
+    case B_LSTMCLIP: return a > b ? b : a < -b ? -b : a;   /* ops.h:337-345 */                                 \
+    case B_SQRSUB: { T d = b - a; return d * d; }          /* op_macros_special.h:820-827 */                   \
+    case B_REVPOW: return M(pow)(b, a);                    /* ops.h:166 */                                     \
+    case B_SXE: return a * ((T)1 - b) + (T)0.5f * b;       /* ops.h:352-355 */                                 \
+    default: return a;                                                                                         \
+  }
+static float bin_f(int fn, float a, float b) { BINARY_BODY(float, MF) }
+static double bin_d(int fn, double a, double b) { BINARY_BODY(double, MD) }
+/* loops/legacy_ops.h:121-129 */
+static int pairwise_fn(int op) {
+  switch (op) {
+    case 0: return B_ADD; case 1: return B_COPY; case 2: return B_DIV; case 3: return B_MUL; case 4: return B_POW;
+    case 5: return B_RSUB; case 6: return B_SUB; case 7: return B_MAX; case 8: return B_MIN; case 9: return B_COPY;
+    case 11: return B_RDIV; case 14: return B_REMAINDER; case 15: return B_FMOD; case 16: return B_ATAN2;
+    case 17: return B_TRUNCDIV; case 18: return B_FLOORDIV; case 19: return B_FLOORMOD; case 20: return B_SQSUB;
+    case 21: return B_REVMOD; case 22: return B_SAFEDIV; case 23: return B_MOD; case 27: return B_LOR;
+    case 28: return B_LXOR; case 29: return B_LNOT; case 30: return B_LAND; case 34: return B_AMAX;
+    case 35: return B_AMIN; case 36: return B_TRUNCMOD; case 37: return B_REPLACENANS; case 38: return B_SAFEDIV;
+    default: return B_NONE;
+  }
+}
+/* loops/legacy_ops.h:78-86 */
+static int scalar_fn(int op) {
+  switch (op) {
+    case 0: return B_ADD; case 1: return B_SUB; case 2: return B_MUL; case 3: return B_DIV; case 4: return B_RDIV;
+    case 5: return B_RSUB; case 6: return B_MAX; case 7: return B_ELU; case 8: return B_ELU_D; case 13: return B_MIN;
+    case 14: return B_COPY; case 15: return B_MOD; case 16: return B_REVMOD; case 17: return B_REMAINDER;
+    case 18: return B_FMOD; case 19: return B_TRUNCDIV; case 20: return B_FLOORDIV; case 21: return B_FLOORMOD;
+    case 22: return B_SQSUB; case 23: return B_SAFEDIV; case 24: return B_AMAX; case 25: return B_AMIN;
+    case 26: return B_ATAN2; case 27: return B_LOR; case 28: return B_LXOR; case 29: return B_LNOT; case 30: return B_LAND;
+    case 31: return B_POW; case 34: return B_SXE; case 35: return B_LRELU; case 36: return B_LRELU_D;
+    case 37: return B_REPLACENANS; case 38: return B_LOGX; case 39: return B_RELU; case 40: return B_RELU6;
+    case 41: return B_STEP; case 42: return B_LSTMCLIP; case 43: return B_TRUNCMOD; case 44: return B_SQRSUB;
+    case 45: return B_REVPOW; case 46: return B_SAFEDIV; case 49: return B_RELU_D;
+    default: return B_NONE;
+  }
+}
+/* loops/legacy_ops.h:34-39 */
+static int broadcast_fn(int op) {
+  switch (op) {
+    case 0: return B_ADD; case 1: return B_SUB; case 2: return B_MUL; case 3: return B_DIV; case 4: return B_RDIV;
+    case 5: return B_RSUB; case 6: return B_COPY; case 7: return B_POW; case 13: return B_MIN; case 14: return B_MAX;
+    case 15: return B_AMIN; case 16: return B_AMAX; case 17: return B_SQSUB; case 18: return B_FLOORMOD;
+    case 19: return B_FLOORDIV; case 20: return B_REVMOD; case 21: return B_SAFEDIV; case 22: return B_MOD;
+    case 23: return B_TRUNCDIV; case 26: return B_ATAN2; case 27: return B_LOR; case 28: return B_LXOR;
+    case 29: return B_LNOT; case 30: return B_LAND; case 31: return B_SAFEDIV;
+    default: return B_NONE;
+  }
+}
+
 static inline int pw_d(int op, double a, double b, double *r) {
   switch (op) {
     case 0: *r = a + b; return 0;
@@ -411,7 +639,7 @@ static inline int pw_d(int op, double a, double b, double *r) {
     case 8: *r = a < b ? a : b; return 0;   /* MinPairwise */
     case 11: *r = b / a; return 0;          /* ReverseDivide */
     case 20: *r = (a - b) * (a - b); return 0; /* SquaredSubtract */
-    default: return 1;
+    default: { int fn = pairwise_fn(op); if (fn == B_NONE) return 1; *r = bin_d(fn, a, b); return 0; }
   }
 }
 static inline int pw_f(int op, float a, float b, float *r) {
@@ -426,7 +654,7 @@ static inline int pw_f(int op, float a, float b, float *r) {
     case 8: *r = a < b ? a : b; return 0;
     case 11: *r = b / a; return 0;
     case 20: { float d = a - b; *r = d * d; return 0; }
-    default: return 1;
+    default: { int fn = pairwise_fn(op); if (fn == B_NONE) return 1; *r = bin_f(fn, a, b); return 0; }
   }
 }
 int orc_pairwise(int opNum, const void *x, const int64_t *xsi, const void *y, const int64_t *ysi, void *z,
@@ -447,6 +675,60 @@ int orc_pairwise(int opNum, const void *x, const int64_t *xsi, const void *y, co
       float r = 0; pw_f(opNum, rnd(ldf(x, xdt, xo), zdt), rnd(ldf(y, ydt, yo), zdt), &r); st(z, zdt, zo, r);
     }
   }
+  return 0;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * execScalar                                   legacy/cpu/NativeOps.cpp (execScalar) -> loops/cpu/scalar.hpp
+ * z[i] = op(x[i], scalar, params) for every element, x and z through their own shapeInfo; the scalar is held
+ * in an array of x's type, so it is rounded to that type first.  opNums loops/legacy_ops.h:78-86.
+ * ------------------------------------------------------------------------------------------- */
+int orc_scalar(int opNum, const void *x, const int64_t *xsi, double scalar, void *z, const int64_t *zsi) {
+  int xdt = orc_dtype(xsi), zdt = orc_dtype(zsi);
+  if (xdt != zdt || !dt_is_float(xdt)) return 2;
+  int64_t n = orc_length(xsi);
+  if (n != orc_length(zsi)) return 3;
+  int fn = scalar_fn(opNum);
+  if (fn == B_NONE) return 1;
+  float sf = rnd((float)scalar, xdt);
+  PAR_FOR
+  for (int64_t i = 0; i < n; i++) {
+    int64_t xo = orc_offset(xsi, i), zo = orc_offset(zsi, i);
+    if (xdt == ORC_DOUBLE) ((double *)z)[zo] = bin_d(fn, ((const double *)x)[xo], scalar);
+    else st(z, zdt, zo, bin_f(fn, ldf(x, xdt, xo), sf));
+  }
+  return 0;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * execBroadcast                                loops/cpu/broadcasting.hpp (exec over TADs)
+ * x is cut into TADs along `dims`; y has the TAD's length; z_tad[i] = op(x_tad[i], y[i]) for every TAD.
+ * opNums loops/legacy_ops.h:34-39.  z must have x's shape; here z's TADs are taken with the same dims.
+ * ------------------------------------------------------------------------------------------- */
+int orc_broadcast(int opNum, const void *x, const int64_t *xsi, const void *y, const int64_t *ysi, void *z,
+                  const int64_t *zsi, const int64_t *dims, int ndims) {
+  int xdt = orc_dtype(xsi), ydt = orc_dtype(ysi), zdt = orc_dtype(zsi);
+  if (xdt != zdt || ydt != zdt || !dt_is_float(zdt)) return 2;
+  int fn = broadcast_fn(opNum);
+  if (fn == B_NONE) return 1;
+  int64_t n = orc_length(xsi);
+  if (n != orc_length(zsi)) return 3;
+  int64_t xtad[2 * ORC_MAX_RANK + 4], ztad[2 * ORC_MAX_RANK + 4];
+  int64_t ntads = orc_tad(xsi, dims, ndims, xtad, NULL);
+  if (ntads <= 0) return 3;
+  int64_t *xoff = (int64_t *)malloc(sizeof(int64_t) * (size_t)ntads), *zoff = (int64_t *)malloc(sizeof(int64_t) * (size_t)ntads);
+  orc_tad(xsi, dims, ndims, xtad, xoff);
+  orc_tad(zsi, dims, ndims, ztad, zoff);
+  int64_t tadLen = orc_length(xtad);
+  if (tadLen != orc_length(ysi)) { free(xoff); free(zoff); return 3; }
+  for (int64_t t = 0; t < ntads; t++) {
+    for (int64_t i = 0; i < tadLen; i++) {
+      int64_t xo = xoff[t] + orc_offset(xtad, i), zo = zoff[t] + orc_offset(ztad, i), yo = orc_offset(ysi, i);
+      if (zdt == ORC_DOUBLE) ((double *)z)[zo] = bin_d(fn, ((const double *)x)[xo], ((const double *)y)[yo]);
+      else st(z, zdt, zo, bin_f(fn, ldf(x, xdt, xo), ldf(y, ydt, yo)));
+    }
+  }
+  free(xoff); free(zoff);
   return 0;
 }
 
@@ -487,9 +769,10 @@ static inline int64_t walk(int rank, const int64_t *shape, const int64_t *stride
 }
 
 /* ReduceSame: 0 Sum 1 Max 2 Min 3 Prod 4 ASum 5 AMax 6 AMin   loops/legacy_ops.h:100-101; ops/ops.h:2363-2368,1170-1243
- * ReduceFloat: 0 Mean 1 AMean 2 Norm1 3 Norm2 4 NormMax 7 SquaredNorm   legacy_ops.h:103-105; ops.h:2370-2378,1217-1298
+ * ReduceFloat: 0 Mean 1 AMean 2 Norm1 3 Norm2 4 NormMax 7 SquaredNorm 8 Entropy 9 LogEntropy 10 ShannonEntropy
+ *   legacy_ops.h:103-105; ops.h:2370-2378,1217-1298,1956-1973,2147-2153
  * accumulator type = float for float/half/bf16 (InterType, ops/op_types.h:213-226), double for double. */
-#define RED_BODY(ACC_T, LOAD, ABS, SQRT, INF)                                                          \
+#define RED_BODY(ACC_T, LOAD, ABS, SQRT, INF, LOG, LOG2, RX, RZ)                                                        \
   ACC_T s;                                                                                              \
   switch (kind) {                                                                                       \
     case 1: s = -INF; break;                                                                            \
@@ -509,11 +792,17 @@ static inline int64_t walk(int rank, const int64_t *shape, const int64_t *stride
       case 5: case 14: s = ABS(v) > s ? ABS(v) : s; break;                                              \
       case 6: s = ABS(v) < s ? ABS(v) : s; break;                                                       \
       case 13: case 17: s = v * v + s; break;                                                           \
+      /* Entropy / LogEntropy: x * log(x), the log taken in x's own type (ops.h:1966-1973,2147-2153) */ \
+      case 18: case 19: s = v * RX(LOG(v)) + s; break;                                                  \
+      /* ShannonEntropy: p * log2(p), the product formed in z's type (ops.h:1956-1963) */              \
+      case 20: s = RZ(v * RX(LOG2(v))) + s; break;                                                      \
     }                                                                                                   \
   }                                                                                                     \
   switch (kind) {                                                                                       \
     case 10: case 11: s = s / (ACC_T)p.ilen; break;                                                     \
     case 13: s = SQRT(s); break;                                                                        \
+    case 18: case 20: s = -s; break;                                                                    \
+    case 19: s = LOG(-s); break;                                                                        \
   }
 
 static int reduce_impl(int kind, const void *x, const int64_t *xsi, void *z, const int64_t *zsi, const int64_t *dims,
@@ -532,11 +821,14 @@ static int reduce_impl(int kind, const void *x, const int64_t *xsi, void *z, con
     int64_t zo = walk(zr, zshape, zstride, o);
     if (xdt == ORC_DOUBLE) {
 #define LOADD(j) (((const double *)x)[base + walk(p.irank, p.ishape, p.istride, (j))])
-      RED_BODY(double, LOADD, fabs, sqrt, INFINITY)
+#define NOROUND(v) (v)
+      RED_BODY(double, LOADD, fabs, sqrt, INFINITY, log, log2, NOROUND, NOROUND)
       st(z, zdt, zo, s);
     } else {
 #define LOADF(j) (ldf(x, xdt, base + walk(p.irank, p.ishape, p.istride, (j))))
-      RED_BODY(float, LOADF, fabsf, sqrtf, INFINITY)
+#define RNDX(v) rnd((v), xdt)
+#define RNDZ(v) rnd((v), zdt)
+      RED_BODY(float, LOADF, fabsf, sqrtf, INFINITY, logf, log2f, RNDX, RNDZ)
       st(z, zdt, zo, s);
     }
   }
@@ -563,6 +855,9 @@ int orc_reduce_float(int opNum, const void *x, const int64_t *xsi, void *z, cons
     case 3: return reduce_impl(13, x, xsi, z, zsi, dims, ndims);
     case 4: return reduce_impl(14, x, xsi, z, zsi, dims, ndims);
     case 7: return reduce_impl(17, x, xsi, z, zsi, dims, ndims);
+    case 8: return reduce_impl(18, x, xsi, z, zsi, dims, ndims);   /* Entropy */
+    case 9: return reduce_impl(19, x, xsi, z, zsi, dims, ndims);   /* LogEntropy */
+    case 10: return reduce_impl(20, x, xsi, z, zsi, dims, ndims);  /* ShannonEntropy */
     default: return 1;
   }
 }

@@ -25,7 +25,15 @@
  *   pairwise .......................... NativeOpsTests.cpp:170-186, bit-exact vs numpy
  *   transform strict/float ............ NativeOpsTests.cpp:658-760, closed forms
  *                                       TestTransformOpValidation.java:1043-1054
- *   reduce same/float ................. NativeOpsTests.cpp:209-238, fp64 bounds
+ *   transform strict, rest of table ... library routines (numpy/scipy), identities, and central
+ *   (tests/test_oracle_tail_ops.py)     differences of the primal op for every *Derivative op;
+ *                                       PreciseGELUDerivative away from zero: parity unpinned (the
+ *                                       reference cubes the scaled argument; only f'(x)+f'(-x)=1 and the
+ *                                       values near zero are pinned)
+ *   transform same, pairwise/scalar/
+ *   broadcast tables, rest of tables .. numpy / math routines per function, table numbering per opNum,
+ *                                       broadcast vs numpy broadcasting over TADs
+ *   reduce same/float ................. NativeOpsTests.cpp:209-238, fp64 bounds; entropies vs scipy.stats
  *   index reduce / argmax ............. NativeOpsTests.cpp:84-117, LegacyOpsTests.cpp:279-310,
  *                                       DeclarableOpsTests1.cpp:2197-2300, brute force
  *   top_k ............................. DeclarableOpsTests5.cpp:1074-1245 (Test_TopK_0..5), brute force
@@ -74,6 +82,10 @@ int orc_pairwise(int opNum, const void *x, const int64_t *xsi, const void *y, co
                  const int64_t *zsi);
 int orc_transform_strict(int opNum, const void *x, const int64_t *xsi, void *z, const int64_t *zsi);
 int orc_transform_float(int opNum, const void *x, const int64_t *xsi, void *z, const int64_t *zsi);
+int orc_transform_same(int opNum, const void *x, const int64_t *xsi, void *z, const int64_t *zsi);
+int orc_scalar(int opNum, const void *x, const int64_t *xsi, double scalar, void *z, const int64_t *zsi);
+int orc_broadcast(int opNum, const void *x, const int64_t *xsi, const void *y, const int64_t *ysi, void *z,
+                  const int64_t *zsi, const int64_t *dims, int ndims);
 int orc_reduce_same(int opNum, const void *x, const int64_t *xsi, void *z, const int64_t *zsi, const int64_t *dims,
                     int ndims);
 int orc_reduce_float(int opNum, const void *x, const int64_t *xsi, void *z, const int64_t *zsi, const int64_t *dims,

@@ -55,6 +55,9 @@ def lib():
         L.orc_pairwise.argtypes = [i32, vp, i64p, vp, i64p, vp, i64p]
         L.orc_transform_strict.argtypes = [i32, vp, i64p, vp, i64p]
         L.orc_transform_float.argtypes = [i32, vp, i64p, vp, i64p]
+        L.orc_transform_same.argtypes = [i32, vp, i64p, vp, i64p]
+        L.orc_scalar.argtypes = [i32, vp, i64p, dbl, vp, i64p]
+        L.orc_broadcast.argtypes = [i32, vp, i64p, vp, i64p, vp, i64p, i64p, i32]
         for f in (L.orc_reduce_same, L.orc_reduce_float, L.orc_index_reduce):
             f.argtypes = [i32, vp, i64p, vp, i64p, i64p, i32]
         L.orc_softmax.argtypes = [vp, i64p, vp, i64p, i32, i32]
@@ -161,6 +164,25 @@ def transform_strict(op, x, z):
 def transform_float(op, x, z):
     x, z = _arr(x), _arr(z)
     _check(lib().orc_transform_float(op, _p(x.a), _s(x.si), _p(z.a), _s(z.si)), "transform_float")
+    return z.a
+
+
+def transform_same(op, x, z):
+    x, z = _arr(x), _arr(z)
+    _check(lib().orc_transform_same(op, _p(x.a), _s(x.si), _p(z.a), _s(z.si)), "transform_same")
+    return z.a
+
+
+def scalar(op, x, value, z):
+    x, z = _arr(x), _arr(z)
+    _check(lib().orc_scalar(op, _p(x.a), _s(x.si), float(value), _p(z.a), _s(z.si)), "scalar")
+    return z.a
+
+
+def broadcast(op, x, y, z, dims):
+    x, y, z = _arr(x), _arr(y), _arr(z)
+    d, n = _dims(dims)
+    _check(lib().orc_broadcast(op, _p(x.a), _s(x.si), _p(y.a), _s(y.si), _p(z.a), _s(z.si), _s(d), n), "broadcast")
     return z.a
 
 
