@@ -727,6 +727,349 @@ static std::vector<std::vector<LongType>> concatShapeFn(Context& c) {
   return {makeShapeInfo(first->dataType(), 'c', out)};
 }
 
+// ---- shape ops: every one of them is "z = a view of x, enumerated in some order" -------------------------------------------------
+// integer arguments that may come as IArgs or as an integer input array
+static std::vector<LongType> hostIndexVector(NDArray* a, const char* what) {
+  std::vector<LongType> out;
+  if (!a || a->isEmpty() || a->lengthOf() == 0) return out;
+  ND4J_REQUIRE(a->buf, std::string(what) + ": index array has no buffer");
+  a->buf->syncToPrimary();
+  out.resize(a->lengthOf());
+  for (LongType i = 0; i < (LongType)out.size(); i++) {
+    LongType off = 0, idx = i;
+    for (int d = a->rankOf() - 1; d >= 0; d--) { off += (idx % a->sizeAt(d)) * a->strideAt(d); idx /= a->sizeAt(d); }
+    if (a->dataType() == INT64) out[i] = a->hostAs<LongType>()[off];
+    else if (a->dataType() == INT32) out[i] = a->hostAs<int>()[off];
+    else ND4J_THROW(std::string(what) + ": index array must be INT32 or INT64");
+  }
+  return out;
+}
+static bool denseIn(const std::vector<LongType>& shape, const std::vector<LongType>& stride) {   // row-major without gaps
+  LongType expect = 1;
+  for (int d = (int)shape.size() - 1; d >= 0; d--) {
+    if (shape[d] != 1 && stride[d] != expect) return false;
+    expect *= shape[d];
+  }
+  return true;
+}
+// z[i-th element] = view[i-th element], both enumerated row-major over their own shapes (column-major for order 'f');
+// the view is (src + srcOffsetElems, shape, strides) over x's buffer
+static void assignEnumerated(NDArray* z, NDArray* x, LongType srcOffsetElems, std::vector<LongType> vshape, std::vector<LongType> vstride,
+                             char order, const char* name) {
+  ND4J_REQUIRE(z->dataType() == x->dataType(), std::string(name) + ": output must carry the input's data type");
+  LongType n = 1;
+  for (auto v : vshape) n *= v;
+  ND4J_REQUIRE(n == z->lengthOf(), std::string(name) + ": output length " + std::to_string(z->lengthOf()) + " does not match " + std::to_string(n));
+  if (n == 0) return;
+  std::vector<LongType> zshape = shapeOf(z), zstride(z->rankOf());
+  for (int d = 0; d < z->rankOf(); d++) zstride[d] = z->strideAt(d);
+  if (order == 'f') {
+    std::reverse(vshape.begin(), vshape.end()); std::reverse(vstride.begin(), vstride.end());
+    std::reverse(zshape.begin(), zshape.end()); std::reverse(zstride.begin(), zstride.end());
+  }
+  if (vshape.empty()) { vshape = {1}; vstride = {1}; }
+  if (zshape.empty()) { zshape = {1}; zstride = {1}; }
+  if (denseIn(vshape, vstride) && denseIn(zshape, zstride)) {   // both flat: one contiguous copy
+    vshape = zshape = {n};
+    vstride = zstride = {1};
+  }
+  auto vsi = makeShapeInfo(x->dataType(), 'c', vshape, vstride.data());
+  auto zsi = makeShapeInfo(z->dataType(), 'c', zshape, zstride.data());
+  EwPlan p = buildEwPlan({zsi.data(), vsi.data()});
+  prepareSpecialUse({z}, {x});
+  const char* src = (const char*)x->specialBuffer() + (size_t)srcOffsetElems * sizeOf(x->dataType());
+  launchUnary(stream(), U_IDENTITY, x->dataType(), z->dataType(), src, z->specialBuffer(), p);
+  registerSpecialUse({z}, {x});
+}
+static std::vector<LongType> stridesOf(const NDArray* a) {
+  std::vector<LongType> st(a->rankOf());
+  for (int d = 0; d < a->rankOf(); d++) st[d] = a->strideAt(d);
+  return st;
+}
+
+// permute (generic/shape/permute.cpp:35-63) and transpose (generic/shape/transpose.cpp:33-77): z = dense copy of the permuted view;
+// the permutation comes from the IArgs or a second input, none = reversed axes
+static std::vector<LongType> permutationOf(Context& c, const char* name) {
+  NDArray* x = c.input(0);
+  std::vector<LongType> perm = c.width() > 1 ? hostIndexVector(c.input(1), name) : c.iArgs;
+  const int r = x->rankOf();
+  if (perm.empty()) { perm.resize(r); for (int i = 0; i < r; i++) perm[i] = r - 1 - i; return perm; }
+  ND4J_REQUIRE((int)perm.size() == r, std::string(name) + ": number of permutations is less in size than input rank.");
+  std::vector<bool> seen(r, false);
+  for (auto& v : perm) {
+    if (v < 0) v += r;
+    ND4J_REQUIRE(v >= 0 && v < r && !seen[v], std::string(name) + ": not a permutation of the input's axes");
+    seen[v] = true;
+  }
+  return perm;
+}
+static void permuteExec(Context& c, const char* name) {
+  NDArray* x = c.input(0); NDArray* z = c.output(0);
+  if (x->isEmpty()) { ND4J_REQUIRE(z->isEmpty(), std::string(name) + ": when input is empty, output must also be empty"); return; }
+  auto perm = permutationOf(c, name);
+  std::vector<LongType> shp(perm.size()), st(perm.size());
+  for (size_t i = 0; i < perm.size(); i++) { shp[i] = x->sizeAt((int)perm[i]); st[i] = x->strideAt((int)perm[i]); }
+  ND4J_REQUIRE(shp == shapeOf(z), std::string(name) + ": output shape " + shapeStr(z) + " is not the permuted input shape");
+  assignEnumerated(z, x, 0, shp, st, 'c', name);
+}
+static std::vector<std::vector<LongType>> permuteShapeFn(Context& c, const char* name) {
+  NDArray* x = c.input(0);
+  if (x->rankOf() < 1) return {scalarShapeInfo(x->dataType())};
+  auto perm = permutationOf(c, name);
+  std::vector<LongType> shp(perm.size());
+  for (size_t i = 0; i < perm.size(); i++) shp[i] = x->sizeAt((int)perm[i]);
+  return {makeShapeInfo(x->dataType(), 'c', shp)};
+}
+
+// reshape (generic/shape/reshape.cpp:33-71,174-260): shape from the IArgs ({-order, dims...}, order -99 = 'c', -102 = 'f') or from a
+// second input; one -1 is inferred; the data keeps its sequence in the chosen order
+static std::vector<LongType> reshapeTarget(Context& c, char& order) {
+  NDArray* x = c.input(0);
+  std::vector<LongType> args = c.width() > 1 ? hostIndexVector(c.input(1), "Reshape") : c.iArgs;
+  order = 'c';
+  if (!args.empty() && args[0] < 0 && args[0] != -1) {
+    ND4J_REQUIRE(args[0] == -99 || args[0] == -102, "reshape:: Value passed in must be -99 or -102 for the ordering if an int array is present.");
+    order = (char)(-args[0]);
+    args.erase(args.begin());
+  }
+  if (c.width() > 1 && !c.iArgs.empty() && (c.iArgs[0] == 99 || c.iArgs[0] == 102 || c.iArgs[0] == -99 || c.iArgs[0] == -102))
+    order = (char)std::abs(c.iArgs[0]);
+  LongType known = 1; int pos = -1;
+  for (size_t i = 0; i < args.size(); i++) {
+    if (args[i] == -1) { ND4J_REQUIRE(pos == -1, "Reshape : Only one unknown dimension (-1) is allowed."); pos = (int)i; }
+    else { ND4J_REQUIRE(args[i] >= 0, "Reshape: negative dimension"); known *= args[i]; }
+  }
+  if (pos >= 0) {
+    if (x->lengthOf() == 1 && x->rankOf() <= 1) args[pos] = 1;
+    else { ND4J_REQUIRE(known > 0 && x->lengthOf() % known == 0, "Reshape: the unknown dimension cannot be resolved"); args[pos] = x->lengthOf() / known; }
+  }
+  return args;
+}
+static void reshapeExec(Context& c) {
+  NDArray* x = c.input(0); NDArray* z = c.output(0);
+  if (x->isEmpty()) { ND4J_REQUIRE(z->isEmpty(), "Reshape: when input is empty, output must also be empty"); return; }
+  ND4J_REQUIRE(x->lengthOf() == z->lengthOf(), "Reshape: lengths before and after reshape should match, but got " + std::to_string(x->lengthOf()) + " vs " + std::to_string(z->lengthOf()));
+  ND4J_REQUIRE(z->ordering() == 'c' || z->ordering() == 'f', "Reshape: new shape has unknown order");
+  assignEnumerated(z, x, 0, shapeOf(x), stridesOf(x), z->ordering(), "Reshape");
+}
+static std::vector<std::vector<LongType>> reshapeShapeFn(Context& c) {
+  char order;
+  auto shp = reshapeTarget(c, order);
+  NDArray* x = c.input(0);
+  if (shp.empty()) return {scalarShapeInfo(x->dataType())};
+  return {makeShapeInfo(x->dataType(), order, shp)};
+}
+
+// squeeze (generic/shape/squeeze.cpp:32-78) / expand_dims (generic/shape/expand_dims.cpp:32-50): same data in the input's order
+static std::vector<LongType> squeezedShape(Context& c) {
+  NDArray* x = c.input(0);
+  std::vector<LongType> axis = !c.iArgs.empty() ? c.iArgs : (c.width() > 1 ? hostIndexVector(c.input(1), "squeeze") : std::vector<LongType>{});
+  for (auto& a : axis) if (a < 0) a += x->rankOf();
+  std::vector<LongType> shp;
+  for (int d = 0; d < x->rankOf(); d++) {
+    if (x->sizeAt(d) == 1 && (axis.empty() || std::find(axis.begin(), axis.end(), (LongType)d) != axis.end())) continue;
+    shp.push_back(x->sizeAt(d));
+  }
+  return shp;
+}
+static void sameDataExec(Context& c, const char* name) {
+  NDArray* x = c.input(0); NDArray* z = c.output(0);
+  if (x->isEmpty()) return;
+  assignEnumerated(z, x, 0, shapeOf(x), stridesOf(x), x->ordering() == 'f' && z->ordering() == 'f' ? 'f' : 'c', name);
+}
+static std::vector<std::vector<LongType>> squeezeShapeFn(Context& c) {
+  NDArray* x = c.input(0);
+  if (x->rankOf() == 0 || (x->rankOf() == 1 && x->lengthOf() == 1)) return {scalarShapeInfo(x->dataType())};
+  return {makeShapeInfo(x->dataType(), x->ordering(), squeezedShape(c))};
+}
+static std::vector<std::vector<LongType>> expandDimsShapeFn(Context& c) {
+  NDArray* x = c.input(0);
+  if (x->lengthOf() == 1 && x->rankOf() <= 1 && !x->isEmpty())
+    return {makeShapeInfo(x->dataType(), 'c', x->rankOf() < 1 ? std::vector<LongType>{1} : std::vector<LongType>{1, 1})};
+  LongType axis = !c.iArgs.empty() ? c.iArgs[0] : hostIndexVector(c.input(1), "ExpandDims").at(0);
+  if (axis < 0) axis += x->rankOf() + 1;
+  ND4J_REQUIRE(axis >= 0 && axis <= x->rankOf(), "ExpandDims: axis should be in range of 0..." + std::to_string(x->rankOf() + 1) + " in this case, but got " + std::to_string(axis) + " instead");
+  std::vector<LongType> shp = shapeOf(x);
+  shp.insert(shp.begin() + axis, 1);
+  return {makeShapeInfo(x->dataType(), x->ordering(), shp)};
+}
+
+// split (generic/transforms/split.cpp:32-72): IArg0 equal parts along the axis (IArg1, or a scalar input before/after the array)
+static NDArray* splitInput(Context& c, LongType& axis) {
+  NDArray* x = c.input(0);
+  axis = 0;
+  if (c.width() > 1) {
+    NDArray* a = c.input(0); NDArray* b = c.input(1);
+    if (a->lengthOf() == 1 && a->rankOf() == 0) { axis = hostIndexVector(a, "Split").at(0); x = b; }
+    else if (b->lengthOf() == 1 && b->rankOf() == 0) { axis = hostIndexVector(b, "Split").at(0); x = a; }
+  }
+  if (c.iArgs.size() == 2) axis = c.iArgs[1];
+  if (axis < 0) axis += x->rankOf();
+  return x;
+}
+static void splitExec(Context& c) {
+  ND4J_REQUIRE(!c.iArgs.empty(), "Split: num_splits is required as the first integer argument");
+  const LongType parts = c.iArgs[0];
+  LongType axis;
+  NDArray* x = splitInput(c, axis);
+  if (x->isEmpty()) return;
+  ND4J_REQUIRE(axis >= 0 && axis < x->rankOf(), "Split: axis out of range");
+  ND4J_REQUIRE(parts > 0 && x->sizeAt((int)axis) % parts == 0, "Split: num_splits has wrong value, remainder of division should be 0, but it's " +
+                                                                    std::to_string(parts > 0 ? x->sizeAt((int)axis) % parts : -1));
+  ND4J_REQUIRE((LongType)c.outputs.size() >= parts, "Split: " + std::to_string(parts) + " output arrays are required");
+  std::vector<LongType> shp = shapeOf(x);
+  shp[axis] /= parts;
+  for (LongType i = 0; i < parts; i++) {
+    NDArray* z = c.output((int)i);
+    ND4J_REQUIRE(z && shapeOf(z) == shp, "Split: output " + std::to_string(i) + " has the wrong shape");
+    assignEnumerated(z, x, i * shp[axis] * x->strideAt((int)axis), shp, stridesOf(x), 'c', "Split");
+  }
+}
+static std::vector<std::vector<LongType>> splitShapeFn(Context& c) {
+  ND4J_REQUIRE(!c.iArgs.empty(), "Split: num_splits is required as the first integer argument");
+  const LongType parts = c.iArgs[0];
+  LongType axis;
+  NDArray* x = splitInput(c, axis);
+  ND4J_REQUIRE(axis >= 0 && axis < x->rankOf() && parts > 0, "Split: axis or num_splits out of range");
+  std::vector<LongType> shp = shapeOf(x);
+  shp[axis] /= parts;
+  std::vector<std::vector<LongType>> out;
+  for (LongType i = 0; i < parts; i++) out.push_back(makeShapeInfo(x->dataType(), x->ordering(), shp));
+  return out;
+}
+
+// strided_slice (generic/tensor/strided_slice.cpp:135-370,372-530): IArgs = begin_mask, ellipsis_mask, end_mask, new_axis_mask,
+// shrink_axis_mask [, begin.., end.., strides..]; or begin/end/strides as inputs 1..3.  The sparse specification (one entry per
+// written index) is spread over the input's axes, every axis gets a canonical [begin, end) and a step, and the output is the
+// strided view copied out, with new axes inserted and shrunk axes dropped.
+struct SliceGeometry {
+  std::vector<LongType> begin, count, step;   // per input axis
+  std::vector<LongType> outShape;
+  bool empty = false;
+};
+static SliceGeometry sliceGeometry(Context& c) {
+  NDArray* x = c.input(0);
+  ND4J_REQUIRE(c.iArgs.size() >= 5, "StridedSlice: five mask arguments are required");
+  const LongType beginMask = c.iArgs[0], ellipsisMaskIn = c.iArgs[1], endMask = c.iArgs[2], newAxisMask = c.iArgs[3], shrinkMask = c.iArgs[4];
+  std::vector<LongType> b, e, st;
+  if (c.iArgs.size() > 5) {
+    const size_t vals = c.iArgs.size() - 5;
+    ND4J_REQUIRE(vals % 3 == 0, "StridedSlice: Number of Integer arguments should be equal to input rank x 3 = " + std::to_string(x->rankOf() * 3) + ", but got " + std::to_string(vals) + " instead");
+    const size_t n = vals / 3;
+    b.assign(c.iArgs.begin() + 5, c.iArgs.begin() + 5 + n);
+    e.assign(c.iArgs.begin() + 5 + n, c.iArgs.begin() + 5 + 2 * n);
+    st.assign(c.iArgs.begin() + 5 + 2 * n, c.iArgs.end());
+  } else if (c.width() > 1) {
+    ND4J_REQUIRE(c.width() >= 3, "StridedSlice: begin and end inputs are required");
+    auto asLong = [](NDArray* a) {
+      std::vector<LongType> out;
+      if (!a || a->lengthOf() == 0) return out;
+      if (a->dataType() == INT32 || a->dataType() == INT64) return hostIndexVector(a, "StridedSlice");
+      a->buf->syncToPrimary();   // the reference's tests also pass these as float / double arrays
+      out.resize(a->lengthOf());
+      for (LongType i = 0; i < (LongType)out.size(); i++) {
+        const LongType off = a->rankOf() == 0 ? 0 : i * a->strideAt(a->rankOf() - 1);
+        if (a->dataType() == FLOAT32) out[i] = (LongType)a->hostAs<float>()[off];
+        else if (a->dataType() == DOUBLE) out[i] = (LongType)a->hostAs<double>()[off];
+        else ND4J_THROW("StridedSlice: begin/end/strides must be integer, float or double arrays");
+      }
+      return out;
+    };
+    b = asLong(c.input(1)); e = asLong(c.input(2));
+    ND4J_REQUIRE(b.size() == e.size(), "StridedSlice: Length of begin/end should match, but got " + std::to_string(b.size()) + " vs " + std::to_string(e.size()) + " instead");
+    for (size_t i = 0; i < e.size(); i++)   // negative ends count from the end of the axis with the same position (strided_slice.cpp:424-436)
+      if (e[i] < 0 && (int)i < x->rankOf()) e[i] = e[i] == -1 ? x->sizeAt((int)i) : e[i] + x->sizeAt((int)i);
+    if (c.width() > 3) {
+      st = asLong(c.input(3));
+      ND4J_REQUIRE(st.size() == b.size(), "StridedSlice: Length of begin/end/stride should match");
+    } else st.assign(b.size(), 1);
+  } else ND4J_THROW("StridedSlice: Can't find begin/end/stride information neither in IArguments or in input arrays");
+  const int n = (int)st.size(), rank = x->rankOf();
+  ND4J_REQUIRE(n > 0, "Strided_Slice: empty arguments");
+  if (rank == 0) return SliceGeometry{};   // a scalar stays a scalar (strided_slice.cpp:519-522)
+  for (auto v : st) ND4J_REQUIRE(v != 0, "StridedSlice: zero stride");
+
+  // spread the sparse specification over the input's axes
+  LongType ellipsisMask = ellipsisMaskIn;
+  int sparseDims = n, axesAfterEllipsis = 0;
+  bool seen = false;
+  for (int i = 0; i < n; i++) {
+    if (seen && (newAxisMask >> i & 1)) axesAfterEllipsis++;
+    if (ellipsisMask >> i & 1) seen = true;
+  }
+  if (!seen) { ellipsisMask |= 1LL << n; sparseDims++; }
+  std::vector<LongType> db(rank, 0), de(rank, 0), ds(rank, 1);
+  std::vector<bool> mb(rank, false), me(rank, false), shrink(rank, false);
+  std::vector<int> gather;   // per output axis: input axis, -1 shrunk away, -2 new axis
+  int full = 0;
+  for (int i = 0; i < sparseDims; i++) {
+    if (ellipsisMask >> i & 1) {
+      const int next = std::min(rank - (sparseDims - i) + 1 + axesAfterEllipsis, rank);
+      for (; full < next; full++) { mb[full] = me[full] = true; gather.push_back(full); }
+    } else if (newAxisMask >> i & 1) {
+      gather.push_back(-2);
+    } else {
+      ND4J_REQUIRE(full < rank, "StridedSlice: shape calculation failed");
+      db[full] = b[i]; de[full] = e[i]; ds[full] = st[i];
+      mb[full] = beginMask >> i & 1; me[full] = endMask >> i & 1;
+      if (shrinkMask >> i & 1) { shrink[full] = true; gather.push_back(-1); }
+      else gather.push_back(full);
+      full++;
+    }
+  }
+  SliceGeometry g;
+  g.begin.resize(rank); g.count.resize(rank); g.step = ds;
+  for (int d = 0; d < rank; d++) {
+    const LongType size = x->sizeAt(d), step = ds[d];
+    if (shrink[d]) {
+      const LongType at = db[d] < 0 ? db[d] + size : db[d];
+      ND4J_REQUIRE(at >= 0 && at < size, "StridedSlice: shape calculation failed");
+      g.begin[d] = at; g.count[d] = 1; g.step[d] = 1;
+      continue;
+    }
+    // canonical positions: masked = the far ends for this direction; otherwise wrapped once and clamped to what a walk can reach
+    const LongType lo = step > 0 ? 0 : -1, hi = step > 0 ? size : size - 1;
+    auto canon = [&](LongType v, bool masked, bool isEnd) {
+      if (masked) return step > 0 ? (isEnd ? hi : lo) : (isEnd ? lo : hi);
+      if (v < 0) v += size;
+      return std::max(lo, std::min(hi, v));
+    };
+    const LongType from = canon(db[d], mb[d], false), to = canon(de[d], me[d], true);
+    LongType span = to - from;
+    if ((step > 0 && span < 0) || (step < 0 && span > 0)) span = 0;
+    const LongType astep = step < 0 ? -step : step, aspan = span < 0 ? -span : span;
+    g.begin[d] = from; g.count[d] = (aspan + astep - 1) / astep;
+  }
+  for (int idx : gather) {
+    if (idx == -1) continue;
+    g.outShape.push_back(idx == -2 ? 1 : g.count[idx]);
+  }
+  for (int d = 0; d < rank; d++) if (g.count[d] == 0) g.empty = true;
+  return g;
+}
+static void stridedSliceExec(Context& c) {
+  NDArray* x = c.input(0); NDArray* z = c.output(0);
+  if (z->isEmpty() || z->lengthOf() == 0) return;
+  SliceGeometry g = sliceGeometry(c);
+  ND4J_REQUIRE(!g.empty && g.outShape == shapeOf(z), "StridedSlice: output shape " + shapeStr(z) + " does not match the slice");
+  LongType offset = 0;
+  std::vector<LongType> st(x->rankOf());
+  for (int d = 0; d < x->rankOf(); d++) { offset += g.begin[d] * x->strideAt(d); st[d] = g.step[d] * x->strideAt(d); }
+  assignEnumerated(z, x, offset, g.count, st, 'c', "StridedSlice");
+}
+static std::vector<std::vector<LongType>> stridedSliceShapeFn(Context& c) {
+  NDArray* x = c.input(0);
+  SliceGeometry g = sliceGeometry(c);
+  if (g.empty || x->isEmpty()) {
+    bool hasZero = false;
+    for (auto v : g.outShape) hasZero |= v == 0;
+    if (!hasZero) return {makeShapeInfo(x->dataType(), 'c', {}, nullptr, ARRAY_EMPTY)};
+    return {makeShapeInfo(x->dataType(), 'c', g.outShape, nullptr, ARRAY_EMPTY)};
+  }
+  if (g.outShape.empty()) return {scalarShapeInfo(x->dataType())};
+  return {makeShapeInfo(x->dataType(), 'c', g.outShape)};
+}
+
 // ---- registry ---------------------------------------------------------------------------------------------------------------
 static std::map<LongType, OpDescriptor>& byHash() {
   static std::map<LongType, OpDescriptor> m;
@@ -760,6 +1103,13 @@ static void ensureRegistered() {
     reg("subtract", 2, 1, true, 0, 0, [](Context& c) { broadcastableExec(c, P_SUB, "SUBTRACT OP"); }, broadcastableShapeFn);
     reg("multiply", 2, 1, true, 0, 0, [](Context& c) { broadcastableExec(c, P_MUL, "MULTIPLY OP"); }, broadcastableShapeFn);
     reg("divide", 2, 1, true, 0, 0, [](Context& c) { broadcastableExec(c, P_DIV, "DIVIDE OP"); }, broadcastableShapeFn);
+    reg("permute", 1, 1, true, 0, -2, [](Context& c) { permuteExec(c, "PERMUTE OP"); }, [](Context& c) { return permuteShapeFn(c, "PERMUTE OP"); });
+    reg("transpose", 1, 1, false, 0, 0, [](Context& c) { permuteExec(c, "TRANSPOSE OP"); }, [](Context& c) { return permuteShapeFn(c, "TRANSPOSE OP"); });
+    reg("reshape", 1, 1, false, 0, -2, reshapeExec, reshapeShapeFn);
+    reg("squeeze", 1, 1, false, 0, -2, [](Context& c) { sameDataExec(c, "squeeze"); }, squeezeShapeFn);
+    reg("expand_dims", 1, 1, false, 0, -2, [](Context& c) { sameDataExec(c, "ExpandDims"); }, expandDimsShapeFn);
+    reg("split", 1, -1, false, 0, 1, splitExec, splitShapeFn);
+    for (const char* alias : {"strided_slice", "stridedslice"}) reg(alias, 1, 1, false, 0, 5, stridedSliceExec, stridedSliceShapeFn);
   });
 }
 const OpDescriptor* findOp(LongType hash) {

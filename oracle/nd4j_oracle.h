@@ -38,6 +38,10 @@
  *                                       DeclarableOpsTests1.cpp:2197-2300, brute force
  *   top_k ............................. DeclarableOpsTests5.cpp:1074-1245 (Test_TopK_0..5), brute force
  *                                       on tie-free rows; behaviour on repeated values: source only
+ *   shape ops (oracle.py, numpy) ...... strided_slice: IndexingTests.cpp:34-330, DeclarableOpsTests4.cpp:1268-1336,
+ *                                       DeclarableOpsTests6.cpp:40-215 (tests/golden/strided_slice_vectors.json) and
+ *                                       brute force over python ranges; negative steps and reshape order 'f':
+ *                                       parity unpinned (numpy semantics only)
  *   xw_plus_b ......................... composition of matmul and the bias row (xw_plus_b.cpp:117-133)
  *   matmul ............................ DeclarableOpsTests14.cpp:601-1260, DeclarableOpsTests19.cpp:52-140
  *   softmax ........................... DeclarableOpsTests1.cpp:2523-2740; inf/nan clamp

@@ -256,3 +256,54 @@ def set_threads(n):
 
 def get_threads():
     return lib().orc_get_threads()
+
+
+# ---- shape ops: numpy restatements (index work, bit-exact) ------------------------------------------------------------
+def permute(x, perm=None):
+    """permute / transpose (generic/shape/permute.cpp:35-63, transpose.cpp:33-77): dense copy of the permuted view;
+    no permutation = reversed axes."""
+    return np.ascontiguousarray(np.transpose(x, perm if perm else None))
+
+
+def reshape(x, shape, order="c"):
+    """reshape (generic/shape/reshape.cpp:33-71): the element sequence in `order` is kept; one -1 is inferred."""
+    return np.reshape(x, shape, order=order.upper())
+
+
+def squeeze(x, axes=None):
+    """squeeze (generic/shape/squeeze.cpp:32-78): unit axes dropped -- all of them, or the listed ones that are unit."""
+    if x.ndim == 0 or (x.ndim == 1 and x.size == 1):
+        return x.reshape(())
+    axes = [a + x.ndim if a < 0 else a for a in (axes or [])]
+    keep = [s for d, s in enumerate(x.shape) if not (s == 1 and (not axes or d in axes))]
+    return x.reshape(keep)
+
+
+def expand_dims(x, axis):
+    """expand_dims (generic/shape/expand_dims.cpp:32-50,56-98)."""
+    if x.size == 1 and x.ndim <= 1:
+        return x.reshape((1,) if x.ndim < 1 else (1, 1))
+    return np.expand_dims(x, axis + x.ndim + 1 if axis < 0 else axis)
+
+
+def split(x, num_splits, axis=0):
+    """split (generic/transforms/split.cpp:32-72): equal parts along the axis."""
+    return [np.ascontiguousarray(p) for p in np.split(x, num_splits, axis=axis)]
+
+
+def strided_slice(x, begin, end, strides, begin_mask=0, ellipsis_mask=0, end_mask=0, new_axis_mask=0, shrink_axis_mask=0):
+    """strided_slice (generic/tensor/strided_slice.cpp:135-370): every written index becomes one numpy index term --
+    Ellipsis, a new axis, an integer (shrink) or a slice whose masked ends are left open -- and numpy's own slicing rules
+    (the ones the op's canonical/clamp arithmetic encodes) do the rest."""
+    idx = []
+    for i in range(len(strides)):
+        bit = 1 << i
+        if ellipsis_mask & bit:
+            idx.append(Ellipsis)
+        elif new_axis_mask & bit:
+            idx.append(np.newaxis)
+        elif shrink_axis_mask & bit:
+            idx.append(int(begin[i]))
+        else:
+            idx.append(slice(None if begin_mask & bit else int(begin[i]), None if end_mask & bit else int(end[i]), int(strides[i])))
+    return np.ascontiguousarray(np.asarray(x)[tuple(idx)])
