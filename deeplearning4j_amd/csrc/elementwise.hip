@@ -12,6 +12,7 @@
 //
 // Functor formulas follow the reference's simdOps (libnd4j/include/ops/ops.h) and sd::math
 // (libnd4j/include/math/templatemath.h); the citations sit on each functor.
+#include "anyio.h"
 #include "device.h"
 #include "kernels.h"
 #include "runtime.h"
@@ -226,6 +227,14 @@ __device__ __forceinline__ A unary_tail(int k, A x) {
     case U_TIMES_ONE_MINUS: return x * (one - x);                                              // ops.h:1165
     case U_CEIL: return M::ceil_(x);                                                           // ops.h:193
     case U_FLOOR: return M::floor_(x);                                                         // ops.h:196
+    // TransformBool (ops.h:1140-1163,1927-1933): 1 where the predicate holds
+    case U_IS_INF: return (x == x && (x - x) != (x - x)) ? one : (A)0;
+    case U_IS_NAN: return x != x ? one : (A)0;
+    case U_IS_FINITE: return (x - x) == (x - x) ? one : (A)0;
+    case U_IS_INF_OR_NAN: return (x - x) == (x - x) ? (A)0 : one;
+    case U_IS_POSITIVE: return x > (A)0 ? one : (A)0;
+    case U_IS_NEGATIVE: return x < (A)0 ? one : (A)0;
+    case U_NOT: return x == (A)0 ? one : (A)0;
     default: return x;
   }
 }
@@ -383,38 +392,6 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_nd(NdArgs a, const T* __restrict_
 template <int K> struct UnaryAs2 { template <typename A> static __device__ __forceinline__ A apply(A a, A) { return Unary<K>::template apply<A>(a); } };
 
 // ---- generic kernel (own shapes, run-time dtypes) ------------------------------------------------------
-__device__ __forceinline__ double load_any(const void* p, int dt, LongType off) {
-  switch (dt) {
-    case FLOAT32: return ((const float*)p)[off];
-    case DOUBLE: return ((const double*)p)[off];
-    case HALF: return to_float(((const f16_t*)p)[off]);
-    case BFLOAT16: return to_float(((const bf16_t*)p)[off]);
-    case INT32: return ((const int*)p)[off];
-    case INT64: return (double)((const LongType*)p)[off];
-    case BOOL: return ((const unsigned char*)p)[off];
-    default: return 0.0;
-  }
-}
-__device__ __forceinline__ void store_any(void* p, int dt, LongType off, double v) {
-  switch (dt) {
-    case FLOAT32: ((float*)p)[off] = (float)v; break;
-    case DOUBLE: ((double*)p)[off] = v; break;
-    case HALF: ((f16_t*)p)[off] = Conv<f16_t>::from((float)v); break;
-    case BFLOAT16: ((bf16_t*)p)[off] = Conv<bf16_t>::from((float)v); break;
-    case INT32: ((int*)p)[off] = (int)v; break;
-    case INT64: ((LongType*)p)[off] = (LongType)v; break;
-    case BOOL: ((unsigned char*)p)[off] = v != 0.0; break;
-    default: break;
-  }
-}
-// rounding through the output storage type, applied to operands before the arithmetic as the reference's
-// sd_add<X,Y,Z> family casts both operands to Z first
-__device__ __forceinline__ float round_as(float v, int dt) {
-  if (dt == HALF) return to_float(Conv<f16_t>::from(v));
-  if (dt == BFLOAT16) return to_float(Conv<bf16_t>::from(v));
-  return v;
-}
-
 template <typename F, int NIN>
 __global__ __launch_bounds__(EW_BLOCK) void ew_generic(DevShape sz, DevShape sx, DevShape sy, int zdt, int xdt, int ydt,
                                                        void* z, const void* x, const void* y, LongType n) {
@@ -462,7 +439,7 @@ __global__ __launch_bounds__(EW_BLOCK) void tail_generic(int k, DevShape sz, Dev
     LongType oz = walk<LongType>(sz, i), ox = walk<LongType>(sx, i);
     double a = load_any(x, xdt, ox), b = scalar;
     if (NIN > 1 && !hasScalar) b = load_any(y, ydt, walk<LongType>(sy, i));
-    if (zdt == DOUBLE) {
+    if (zdt == DOUBLE || xdt == DOUBLE) {   // predicates on doubles must not see them narrowed
       store_any(z, zdt, oz, NIN > 1 ? binary_tail<double>(k, a, b) : unary_tail<double>(k, a));
     } else {
       float fa = round_as((float)a, zdt), fb = round_as((float)b, zdt);

@@ -25,6 +25,8 @@ enum UnaryKind : int {
   U_ASINH, U_RINT, U_LOG_SIGMOID, U_ERFC, U_EXPM1, U_ATANH, U_GELU_D, U_PRECISE_GELU_D, U_MISH, U_MISH_D,
   // TransformSame
   U_ONES, U_ROUND, U_TIMES_ONE_MINUS, U_CEIL, U_FLOOR,
+  // TransformBool (output type BOOL)
+  U_IS_INF, U_IS_NAN, U_IS_FINITE, U_IS_INF_OR_NAN, U_IS_POSITIVE, U_NOT, U_IS_NEGATIVE,
   U_TAIL_END
 };
 enum PairwiseKind : int {
@@ -70,6 +72,9 @@ enum ReduceKind : int {
   R_COUNT
 };
 enum IndexKind : int { I_MAX, I_MIN, I_AMAX, I_AMIN, I_COUNT };
+// reductions whose accumulator or output type differs from the input's: summary statistics (double triple n, mean, M2),
+// counts (INT64 out), Any / All (BOOL out)
+enum MiscReduceKind : int { M_VARIANCE, M_STDDEV, M_COUNT_NONZERO, M_COUNT_ZERO, M_ANY, M_ALL };
 
 // outer = kept dims (one output element each), inner = reduced dims
 struct ReducePlan {
@@ -83,6 +88,9 @@ struct ReducePlan {
 
 void launchReduce(hipStream_t s, ReduceKind k, DataType xdt, DataType zdt, const void* x, void* z, const ReducePlan& p,
                   void* scratch, size_t scratchBytes);
+// zdt: the float type for variance / standard deviation, INT64 for counts, BOOL for Any / All
+void launchReduceMisc(hipStream_t s, MiscReduceKind k, DataType xdt, DataType zdt, const void* x, void* z, const ReducePlan& p,
+                      bool biasCorrected, void* scratch, size_t scratchBytes);
 void launchIndexReduce(hipStream_t s, IndexKind k, DataType xdt, DataType zdt, const void* x, void* z,
                        const ReducePlan& p, void* scratch, size_t scratchBytes);
 

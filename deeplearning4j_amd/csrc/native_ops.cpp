@@ -718,6 +718,101 @@ void execReduceFloat2(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueND
   GUARD_END_VOID
 }
 
+// reductions with their own accumulator / output types
+static void runReduceMisc(const char* fn, MiscReduceKind k, NDArray* x, NDArray* z, std::vector<LongType> d, bool biasCorrected) {
+  ND4J_REQUIRE(!x->isEmpty(), std::string(fn) + ": reductions of empty arrays are not implemented in nd4j-hip");
+  if (z->isEmpty()) return;
+  if (z->lengthOf() == 1 && x->lengthOf() != 1) {
+    bool keptAllUnit = true;
+    std::vector<bool> red(x->rankOf(), false);
+    for (auto v : d) red[v] = true;
+    for (int i = 0; i < x->rankOf(); i++) if (!red[i] && x->sizeAt(i) != 1) keptAllUnit = false;
+    if (!keptAllUnit) d.clear();
+  }
+  ReducePlan p = buildReducePlan(x->shapeInfo(), z->shapeInfo(), d, false);
+  auto lc = LaunchContext::defaultContext();
+  prepareSpecialUse({z}, {x});
+  launchReduceMisc(lc->execStream, k, x->dataType(), z->dataType(), x->specialBuffer(), z->specialBuffer(), p, biasCorrected,
+                   lc->reductionBuffer, LaunchContext::REDUCTION_BYTES);
+  registerSpecialUse({z}, {x});
+}
+static MiscReduceKind summaryKind(int opNum) {
+  switch (opNum) {  // loops/legacy_ops.h:69
+    case 0: return M_VARIANCE; case 1: return M_STDDEV;
+    default: ND4J_THROW("execSummaryStats: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
+  }
+}
+extern "C" {
+void execSummaryStatsScalar(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, bool biasCorrected) {
+  GUARD_BEGIN
+  NDArray* x = arr(xa, "execSummaryStatsScalar", "x"); NDArray* z = arr(za, "execSummaryStatsScalar", "z");
+  ND4J_REQUIRE(isFloatType(z->dataType()), "execSummaryStatsScalar: Z must have a floating point type");
+  runReduceMisc("execSummaryStatsScalar", summaryKind(opNum), x, z, {}, biasCorrected);
+  GUARD_END_VOID
+}
+void execSummaryStatsTad(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da, bool biasCorrected) {
+  GUARD_BEGIN
+  NDArray* x = arr(xa, "execSummaryStatsTad", "x"); NDArray* z = arr(za, "execSummaryStatsTad", "z");
+  ND4J_REQUIRE(isFloatType(z->dataType()), "execSummaryStatsTad: Z must have a floating point type");
+  runReduceMisc("execSummaryStatsTad", summaryKind(opNum), x, z, hostDims(da, x->rankOf(), "execSummaryStatsTad"), biasCorrected);
+  GUARD_END_VOID
+}
+static void reduceLong(const char* fn, int opNum, OpaqueNDArray xa, OpaqueNDArray za, OpaqueNDArray da) {
+  NDArray* x = arr(xa, fn, "x"); NDArray* z = arr(za, fn, "z");
+  ND4J_REQUIRE(z->dataType() == INT64, std::string("NativeOpExecutioner::execReduceLong wrong Z data type: Z must be INT64, got ") + dtypeName(z->dataType()));
+  MiscReduceKind k;
+  switch (opNum) {  // loops/legacy_ops.h:95
+    case 0: k = M_COUNT_NONZERO; break; case 1: k = M_COUNT_ZERO; break;
+    default: ND4J_THROW(std::string(fn) + ": opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");   // 2 MatchCondition reads extra parameters
+  }
+  runReduceMisc(fn, k, x, z, da ? hostDims(da, x->rankOf(), fn) : std::vector<LongType>{}, false);
+}
+void execReduceLong(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
+  GUARD_BEGIN
+  reduceLong("execReduceLong", opNum, xa, za, da);
+  GUARD_END_VOID
+}
+void execReduceLong2(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
+  GUARD_BEGIN
+  reduceLong("execReduceLong2", opNum, xa, za, da);
+  GUARD_END_VOID
+}
+static void reduceBool(const char* fn, int opNum, OpaqueNDArray xa, OpaqueNDArray za, OpaqueNDArray da) {
+  NDArray* x = arr(xa, fn, "x"); NDArray* z = arr(za, fn, "z");
+  ND4J_REQUIRE(z->dataType() == BOOL, std::string("NativeOpExecutioner::execReduceBool requires Z operand to have BOOL type, got ") + dtypeName(z->dataType()));
+  MiscReduceKind k;
+  switch (opNum) {  // loops/legacy_ops.h:97-98
+    case 0: k = M_ANY; break; case 1: k = M_ALL; break;
+    default: ND4J_THROW(std::string(fn) + ": opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
+  }
+  runReduceMisc(fn, k, x, z, da ? hostDims(da, x->rankOf(), fn) : std::vector<LongType>{}, false);
+}
+void execReduceBool(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
+  GUARD_BEGIN
+  reduceBool("execReduceBool", opNum, xa, za, da);
+  GUARD_END_VOID
+}
+void execReduceBool2(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
+  GUARD_BEGIN
+  reduceBool("execReduceBool2", opNum, xa, za, da);
+  GUARD_END_VOID
+}
+void execTransformBool(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
+  GUARD_BEGIN
+  NDArray* x = arr(xa, "execTransformBool", "x"); NDArray* z = arr(za, "execTransformBool", "z");
+  ND4J_REQUIRE(z->dataType() == BOOL, std::string("NativeOpExecutioner::execTransformBool requires Z to have same boolean type, got ") + dtypeName(z->dataType()));
+  ND4J_REQUIRE(isFloatType(x->dataType()), "execTransformBool: non-float inputs are not implemented in nd4j-hip");
+  UnaryKind k;
+  switch (opNum) {  // loops/legacy_ops.h:49-51
+    case 1: k = U_IS_INF; break; case 2: k = U_IS_NAN; break; case 3: k = U_IS_FINITE; break; case 4: k = U_IS_INF_OR_NAN; break;
+    case 6: k = U_IS_POSITIVE; break; case 7: k = U_NOT; break; case 8: k = U_IS_NEGATIVE; break;
+    default: ND4J_THROW("execTransformBool: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");   // 5 MatchConditionBool reads extra parameters
+  }
+  runUnary("execTransformBool", k, x, z);
+  GUARD_END_VOID
+}
+}  // extern "C"
+
 static IndexKind indexKind(int opNum) {
   switch (opNum) {  // loops/legacy_ops.h:131-132
     case 0: return I_MAX; case 1: return I_MIN; case 2: return I_AMAX; case 3: return I_AMIN;

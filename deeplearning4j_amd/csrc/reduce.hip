@@ -15,6 +15,7 @@
 // Index semantics (ops/op_macros_index_reduce.h:33-69): strict comparison from {start, 0}, so the first
 // extreme wins, NaN is never selected and an all -inf row gives 0.  Here: NaN is mapped to the start
 // value on load and ties resolve to the lowest index, which yields the same integer.
+#include "anyio.h"
 #include "device.h"
 #include "kernels.h"
 #include "runtime.h"
@@ -261,6 +262,120 @@ void launchReduce(hipStream_t st, ReduceKind k, DataType xdt, DataType zdt, cons
     case R_SHANNON_ENTROPY: reduceDtype<SumOp, PRE_XLOG2X>(st, xdt, x, z, p, POST_NEG, scratch, scratchBytes); break;
     default: ND4J_THROW("reduce: unknown op kind");
   }
+  HIP_CHECK(hipGetLastError());
+}
+
+// ---- summary statistics, counts, Any / All -------------------------------------------------------------------------
+// One block per (output, split): any storage type through load_any, accumulation in double as the reference's
+// SummaryStatsData does (loops/summarystatsreduce.h:52-56,89-100).  A block makes its segment's (n, mean, M2) in two
+// passes over the segment (the second comes out of the caches); segments merge with Chan's update
+// (summarystatsreduce.h:190-211), also what the finish kernel applies across splits.
+struct MiscArgs {
+  DevShape outer, inner, zOuter;
+  LongType outerLen, innerLen, segLen;
+  int splits, kind, bias, xdt, zdt;
+};
+__device__ __forceinline__ double block_sum(double v, double* lds) {
+  const int t = threadIdx.x;
+  lds[t] = v;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if (t < w) lds[t] += lds[t + w];
+    __syncthreads();
+  }
+  const double r = lds[0];
+  __syncthreads();
+  return r;
+}
+__device__ __forceinline__ double misc_result(const MiscArgs& a, double n, double mean, double m2, double cnt) {
+  switch (a.kind) {
+    case M_VARIANCE: case M_STDDEV: {
+      double var = n <= 1.0 ? 0.0 : m2 / n;                       // summarystatsreduce.h:89-92
+      if (a.bias) {                                               // ops.h:2157-2190: falls back when the corrected value is negative
+        const double corrected = n <= 1.0 ? 0.0 : m2 / (n - 1.0);
+        if (!(corrected < 0.0)) var = corrected;
+      }
+      return a.kind == M_STDDEV ? sqrt(var) : var;
+    }
+    case M_ANY: return cnt > 0.0 ? 1.0 : 0.0;                     // ops.h:1200-1206: the sum of the elements is positive
+    case M_ALL: return cnt > 0.0 ? 0.0 : 1.0;                     // here cnt counts the zero elements
+    default: return cnt;
+  }
+}
+__global__ __launch_bounds__(256) void misc_partial(MiscArgs a, const void* __restrict__ x, void* __restrict__ z,
+                                                    double* __restrict__ partials) {
+  __shared__ double lds[256];
+  const LongType unit = blockIdx.x, row = unit / a.splits;
+  const int split = (int)(unit - row * a.splits);
+  const LongType base = walk<LongType>(a.outer, row);
+  const LongType j0 = (LongType)split * a.segLen;
+  LongType j1 = j0 + a.segLen;
+  if (j1 > a.innerLen) j1 = a.innerLen;
+  const bool linear = a.inner.rank == 1;
+  const LongType st = linear ? a.inner.stride[0] : 0;
+  auto at = [&](LongType q) { return load_any(x, a.xdt, base + (linear ? q * st : walk<LongType>(a.inner, q))); };
+  double n = (double)(j1 - j0), mean = 0.0, m2 = 0.0, cnt = 0.0;
+  if (a.kind == M_VARIANCE || a.kind == M_STDDEV) {
+    double s = 0.0;
+    for (LongType q = j0 + threadIdx.x; q < j1; q += 256) s += at(q);
+    mean = n > 0 ? block_sum(s, lds) / n : 0.0;
+    double d2 = 0.0;
+    for (LongType q = j0 + threadIdx.x; q < j1; q += 256) { const double d = at(q) - mean; d2 += d * d; }
+    m2 = block_sum(d2, lds);
+  } else {
+    double c = 0.0;
+    for (LongType q = j0 + threadIdx.x; q < j1; q += 256) {
+      const double v = at(q);
+      if (a.kind == M_COUNT_NONZERO) c += v == 0.0 ? 0.0 : 1.0;         // ops.h:1180-1188
+      else if (a.kind == M_COUNT_ZERO || a.kind == M_ALL) c += v == 0.0 ? 1.0 : 0.0;   // ops.h:1190-1198,1208-1215
+      else c += v;                                                     // Any
+    }
+    cnt = block_sum(c, lds);
+  }
+  if (threadIdx.x != 0) return;
+  if (a.splits == 1) {
+    store_any(z, a.zdt, walk<LongType>(a.zOuter, row), misc_result(a, n, mean, m2, cnt));
+  } else {
+    double* p = partials + unit * 4;
+    p[0] = n; p[1] = mean; p[2] = m2; p[3] = cnt;
+  }
+}
+__global__ __launch_bounds__(256) void misc_finish(MiscArgs a, const double* __restrict__ partials, void* __restrict__ z) {
+  const LongType row = (LongType)blockIdx.x * 256 + threadIdx.x;
+  if (row >= a.outerLen) return;
+  double n = 0.0, mean = 0.0, m2 = 0.0, cnt = 0.0;
+  for (int s = 0; s < a.splits; s++) {
+    const double* p = partials + (row * a.splits + s) * 4;
+    const double nb = p[0];
+    if (nb > 0.0) {
+      const double delta = p[1] - mean, tot = n + nb;
+      m2 += p[2] + delta * delta * n * nb / tot;
+      mean += delta * nb / tot;
+      n = tot;
+    }
+    cnt += p[3];
+  }
+  store_any(z, a.zdt, walk<LongType>(a.zOuter, row), misc_result(a, n, mean, m2, cnt));
+}
+void launchReduceMisc(hipStream_t st, MiscReduceKind k, DataType xdt, DataType zdt, const void* x, void* z, const ReducePlan& p,
+                      bool biasCorrected, void* scratch, size_t scratchBytes) {
+  if (p.outerLen == 0) return;
+  MiscArgs a;
+  a.outer = p.outer; a.inner = p.inner; a.zOuter = p.zOuter;
+  a.outerLen = p.outerLen; a.innerLen = p.innerLen;
+  a.kind = (int)k; a.bias = biasCorrected ? 1 : 0; a.xdt = (int)xdt; a.zdt = (int)zdt;
+  // few outputs with long runs: split every run over several blocks (about 2048 blocks in flight)
+  LongType splits = 1;
+  if (p.outerLen < 1024 && p.innerLen > 16384) {
+    splits = std::min<LongType>((2048 + p.outerLen - 1) / p.outerLen, (p.innerLen + 8191) / 8192);
+    const LongType cap = (LongType)(scratchBytes / (4 * sizeof(double))) / p.outerLen;
+    splits = std::max<LongType>(1, std::min(splits, cap));
+  }
+  a.splits = (int)splits;
+  a.segLen = (p.innerLen + splits - 1) / splits;
+  ND4J_REQUIRE(p.outerLen * splits < (1LL << 31), "reduce: too many outputs");
+  hipLaunchKernelGGL(misc_partial, dim3((unsigned)(p.outerLen * splits)), dim3(256), 0, st, a, x, z, (double*)scratch);
+  if (splits > 1) hipLaunchKernelGGL(misc_finish, dim3((unsigned)((p.outerLen + 255) / 256)), dim3(256), 0, st, a, (const double*)scratch, z);
   HIP_CHECK(hipGetLastError());
 }
 

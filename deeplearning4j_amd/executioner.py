@@ -55,6 +55,22 @@ class IndexReduce:
     IndexMax, IndexMin, IndexAbsoluteMax, IndexAbsoluteMin = 0, 1, 2, 3
 
 
+class TransformBool:
+    IsInf, IsNan, IsFinite, IsInfOrNan, IsPositive, Not, IsNegative = 1, 2, 3, 4, 6, 7, 8
+
+
+class SummaryStats:
+    Variance, StandardDeviation = 0, 1
+
+
+class ReduceLong:
+    CountNonZero, CountZero = 0, 1
+
+
+class ReduceBool:
+    Any, All = 0, 1
+
+
 class Scalar:
     Add, Subtract, Multiply, Divide, ReverseDivide, ReverseSubtract, MaxPairwise, ELU, ELUDerivative = 0, 1, 2, 3, 4, 5, 6, 7, 8
     MinPairwise, CopyPws, Mod, ReverseMod, Remainder, FMod, TruncateDiv, FloorDiv, FloorMod, SquaredSubtract = 13, 14, 15, 16, 17, 18, 19, 20, 21, 22
@@ -216,6 +232,37 @@ class Executioner:
 
     def exec_index_reduce(self, op_num, x, dims=None, keep_dims=False, z=None):
         return self._reduce(self.L.execIndexReduceScalar, self.L.execIndexReduce, "execIndexReduce", op_num, x, dims, keep_dims, z, INT64)
+
+    def exec_transform_bool(self, op_num, x, z=None):
+        if z is None:
+            z = NDArray.empty(x.shape, BOOL)
+        self.L.execTransformBool(None, op_num, x.handle, None, z.handle)
+        N.check("execTransformBool")
+        return z
+
+    def exec_summary_stats(self, op_num, x, dims=None, bias_corrected=False, keep_dims=False, z=None):
+        if z is None:
+            z = NDArray.empty(_reduced_shape(x.shape, dims, keep_dims), x.dtype)
+        if dims is None or len(dims) == 0:
+            self.L.execSummaryStatsScalar(None, op_num, x.handle, None, z.handle, bool(bias_corrected))
+        else:
+            self.L.execSummaryStatsTad(None, op_num, x.handle, None, z.handle, _dims_array(dims).handle, bool(bias_corrected))
+        N.check("execSummaryStats")
+        return z
+
+    def _reduce_dims_only(self, fn, name, op_num, x, dims, keep_dims, z, zdtype):
+        if z is None:
+            z = NDArray.empty(_reduced_shape(x.shape, dims, keep_dims), zdtype)
+        d = _dims_array(dims if dims else list(range(len(x.shape))))
+        fn(None, op_num, x.handle, None, z.handle, d.handle)
+        N.check(name)
+        return z
+
+    def exec_reduce_long(self, op_num, x, dims=None, keep_dims=False, z=None):
+        return self._reduce_dims_only(self.L.execReduceLong, "execReduceLong", op_num, x, dims, keep_dims, z, INT64)
+
+    def exec_reduce_bool(self, op_num, x, dims=None, keep_dims=False, z=None):
+        return self._reduce_dims_only(self.L.execReduceBool, "execReduceBool", op_num, x, dims, keep_dims, z, BOOL)
 
     # ---- custom ops ----
     def op_hash(self, name):

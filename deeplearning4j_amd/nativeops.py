@@ -118,6 +118,13 @@ _SIGS = {
     "execReduceSame2": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
     "execIndexReduce": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
     "execIndexReduceScalar": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr]),
+    "execTransformBool": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr]),
+    "execSummaryStatsScalar": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, ctypes.c_bool]),
+    "execSummaryStatsTad": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr, ctypes.c_bool]),
+    "execReduceLong": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "execReduceLong2": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "execReduceBool": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "execReduceBool2": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
     "execScalar": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
     "execBroadcast": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
     "getAllCustomOps": (ctypes.c_char_p, []),

@@ -173,6 +173,13 @@ ND4JHIP_EXPORT void execReduceSame2(Nd4jPointer* extraPointers, int opNum, Opaqu
 ND4JHIP_EXPORT void execIndexReduce(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z, OpaqueNDArray dimension);  /* ref :214 */
 ND4JHIP_EXPORT void execIndexReduceScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z); /* ref :216 */
 ND4JHIP_EXPORT void execScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, OpaqueNDArray z, OpaqueNDArray scalar, void* extraParams); /* ref :204 */
+ND4JHIP_EXPORT void execTransformBool(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z);   /* ref :218 */
+ND4JHIP_EXPORT void execSummaryStatsScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z, bool biasCorrected); /* ref :197 */
+ND4JHIP_EXPORT void execSummaryStatsTad(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z, OpaqueNDArray dimension, bool biasCorrected); /* ref :198-199 */
+ND4JHIP_EXPORT void execReduceLong(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z, OpaqueNDArray dimension);  /* ref :211 */
+ND4JHIP_EXPORT void execReduceLong2(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z, OpaqueNDArray dimension); /* ref :349-351 */
+ND4JHIP_EXPORT void execReduceBool(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z, OpaqueNDArray dimension);  /* ref :213 */
+ND4JHIP_EXPORT void execReduceBool2(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z, OpaqueNDArray dimension); /* ref :212 */
 ND4JHIP_EXPORT void execBroadcast(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, OpaqueNDArray y, OpaqueNDArray z, void* extraParams, OpaqueNDArray dimension); /* ref :206 */
 
 /* ---- op context + declarable ops ---------------------------------------------------------------------------- */

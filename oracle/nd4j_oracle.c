@@ -863,6 +863,95 @@ int orc_reduce_float(int opNum, const void *x, const int64_t *xsi, void *z, cons
 }
 
 /* ---------------------------------------------------------------------------------------------
+ * execSummaryStatsScalar / execSummaryStatsTad   legacy/cpu/NativeOps.cpp:2167-2200 -> loops/cpu/summarystatsreduce.cpp
+ * per output: SummaryStatsData {n, mean, M2} in double, fed one element at a time (Welford's update, the form
+ * loops/summarystatsreduce.h:190-211 takes for a one-element right-hand side); variance = M2 / n (0 for n <= 1),
+ * bias-corrected M2 / (n - 1) unless that is negative (ops/ops.h:2157-2190); opNum 0 variance, 1 standard deviation.
+ * ------------------------------------------------------------------------------------------- */
+int orc_summary_stats(int opNum, const void *x, const int64_t *xsi, void *z, const int64_t *zsi, const int64_t *dims, int ndims,
+                      int biasCorrected) {
+  if (opNum != 0 && opNum != 1) return 1;
+  RedPlan p;
+  if (red_plan(xsi, dims, ndims, &p)) return 3;
+  int xdt = orc_dtype(xsi), zdt = orc_dtype(zsi);
+  if (!dt_is_float(zdt)) return 2;
+  if (orc_length(zsi) != p.olen) return 3;
+  int64_t zshape[ORC_MAX_RANK], zstride[ORC_MAX_RANK]; int zr = 0;
+  for (int i = 0; i < si_rank(zsi); i++)
+    if (si_shape(zsi)[i] != 1) { zshape[zr] = si_shape(zsi)[i]; zstride[zr++] = si_stride(zsi)[i]; }
+  for (int64_t o = 0; o < p.olen; o++) {
+    int64_t base = walk(p.orank, p.oshape, p.ostride, o);
+    double n = 0, mean = 0, m2 = 0;
+    for (int64_t j = 0; j < p.ilen; j++) {
+      double v = ld(x, xdt, base + walk(p.irank, p.ishape, p.istride, j));
+      n += 1.0;
+      double delta = v - mean;
+      mean += delta / n;
+      m2 += delta * (v - mean);
+    }
+    double var = n <= 1.0 ? 0.0 : m2 / n;
+    if (biasCorrected) { double c = n <= 1.0 ? 0.0 : m2 / (n - 1.0); if (!(c < 0.0)) var = c; }
+    st(z, zdt, walk(zr, zshape, zstride, o), opNum == 1 ? sqrt(var) : var);
+  }
+  return 0;
+}
+
+/* execReduceLong (0 CountNonZero, 1 CountZero: ops/ops.h:1180-1198) and execReduceBool (0 Any: the sum of the elements is
+ * positive, 1 All: no element is zero; ops/ops.h:1200-1215).  kind: 0/1 = long ops, 10/11 = bool ops. */
+int orc_reduce_count(int kind, const void *x, const int64_t *xsi, void *z, const int64_t *zsi, const int64_t *dims, int ndims) {
+  RedPlan p;
+  if (red_plan(xsi, dims, ndims, &p)) return 3;
+  int xdt = orc_dtype(xsi), zdt = orc_dtype(zsi);
+  if (orc_length(zsi) != p.olen) return 3;
+  if ((kind < 10 && zdt != ORC_INT64) || (kind >= 10 && zdt != ORC_BOOL)) return 2;
+  int64_t zshape[ORC_MAX_RANK], zstride[ORC_MAX_RANK]; int zr = 0;
+  for (int i = 0; i < si_rank(zsi); i++)
+    if (si_shape(zsi)[i] != 1) { zshape[zr] = si_shape(zsi)[i]; zstride[zr++] = si_stride(zsi)[i]; }
+  for (int64_t o = 0; o < p.olen; o++) {
+    int64_t base = walk(p.orank, p.oshape, p.ostride, o);
+    double sum = 0; int64_t zeros = 0;
+    for (int64_t j = 0; j < p.ilen; j++) {
+      double v = ld(x, xdt, base + walk(p.irank, p.ishape, p.istride, j));
+      sum += v;
+      zeros += v == 0.0;
+    }
+    int64_t zo = walk(zr, zshape, zstride, o);
+    switch (kind) {
+      case 0: ((int64_t *)z)[zo] = p.ilen - zeros; break;
+      case 1: ((int64_t *)z)[zo] = zeros; break;
+      case 10: ((unsigned char *)z)[zo] = sum > 0.0; break;
+      case 11: ((unsigned char *)z)[zo] = zeros == 0; break;
+      default: return 1;
+    }
+  }
+  return 0;
+}
+
+/* execTransformBool: loops/legacy_ops.h:49-51; predicates ops/ops.h:1140-1163,1927-1933; z is a BOOL array */
+int orc_transform_bool(int opNum, const void *x, const int64_t *xsi, void *z, const int64_t *zsi) {
+  int xdt = orc_dtype(xsi);
+  if (orc_dtype(zsi) != ORC_BOOL || !dt_is_float(xdt)) return 2;
+  int64_t n = orc_length(xsi);
+  if (n != orc_length(zsi)) return 3;
+  if (opNum < 1 || opNum > 8 || opNum == 5) return 1;
+  for (int64_t i = 0; i < n; i++) {
+    double v = ld(x, xdt, orc_offset(xsi, i));
+    int r = 0;
+    switch (opNum) {
+      case 1: r = isinf(v); break;
+      case 2: r = isnan(v); break;
+      case 3: r = isfinite(v); break;
+      case 4: r = !isfinite(v); break;
+      case 6: r = v > 0; break;
+      case 7: r = !(v != 0); break;     /* Not: !static_cast<bool>(d1) */
+      case 8: r = v < 0; break;
+    }
+    ((unsigned char *)z)[orc_offset(zsi, i)] = r != 0;
+  }
+  return 0;
+}
+
+/* ---------------------------------------------------------------------------------------------
  * execIndexReduce / execIndexReduceScalar     legacy/cpu/NativeOps.cpp:1110-1170
  *   -> NativeOpExecutioner_indexreduce.cpp:20-46 -> loops/cpu/indexreduce.hpp:55-140
  *   -> helpers/cpu/loops/IndexReductionLoops.hpp:40-243

@@ -34,6 +34,8 @@
  *   broadcast tables, rest of tables .. numpy / math routines per function, table numbering per opNum,
  *                                       broadcast vs numpy broadcasting over TADs
  *   reduce same/float ................. NativeOpsTests.cpp:209-238, fp64 bounds; entropies vs scipy.stats
+ *   summary stats, counts, Any/All,
+ *   transform bool .................... numpy var/std (ddof 0/1), count_nonzero, isnan/isinf/isfinite
  *   index reduce / argmax ............. NativeOpsTests.cpp:84-117, LegacyOpsTests.cpp:279-310,
  *                                       DeclarableOpsTests1.cpp:2197-2300, brute force
  *   top_k ............................. DeclarableOpsTests5.cpp:1074-1245 (Test_TopK_0..5), brute force
@@ -87,6 +89,10 @@ int orc_pairwise(int opNum, const void *x, const int64_t *xsi, const void *y, co
 int orc_transform_strict(int opNum, const void *x, const int64_t *xsi, void *z, const int64_t *zsi);
 int orc_transform_float(int opNum, const void *x, const int64_t *xsi, void *z, const int64_t *zsi);
 int orc_transform_same(int opNum, const void *x, const int64_t *xsi, void *z, const int64_t *zsi);
+int orc_transform_bool(int opNum, const void *x, const int64_t *xsi, void *z, const int64_t *zsi);
+int orc_summary_stats(int opNum, const void *x, const int64_t *xsi, void *z, const int64_t *zsi, const int64_t *dims, int ndims,
+                      int biasCorrected);
+int orc_reduce_count(int kind, const void *x, const int64_t *xsi, void *z, const int64_t *zsi, const int64_t *dims, int ndims);
 int orc_scalar(int opNum, const void *x, const int64_t *xsi, double scalar, void *z, const int64_t *zsi);
 int orc_broadcast(int opNum, const void *x, const int64_t *xsi, const void *y, const int64_t *ysi, void *z,
                   const int64_t *zsi, const int64_t *dims, int ndims);

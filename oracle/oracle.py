@@ -56,6 +56,9 @@ def lib():
         L.orc_transform_strict.argtypes = [i32, vp, i64p, vp, i64p]
         L.orc_transform_float.argtypes = [i32, vp, i64p, vp, i64p]
         L.orc_transform_same.argtypes = [i32, vp, i64p, vp, i64p]
+        L.orc_transform_bool.argtypes = [i32, vp, i64p, vp, i64p]
+        L.orc_summary_stats.argtypes = [i32, vp, i64p, vp, i64p, i64p, i32, i32]
+        L.orc_reduce_count.argtypes = [i32, vp, i64p, vp, i64p, i64p, i32]
         L.orc_scalar.argtypes = [i32, vp, i64p, dbl, vp, i64p]
         L.orc_broadcast.argtypes = [i32, vp, i64p, vp, i64p, vp, i64p, i64p, i32]
         for f in (L.orc_reduce_same, L.orc_reduce_float, L.orc_index_reduce):
@@ -183,6 +186,33 @@ def broadcast(op, x, y, z, dims):
     x, y, z = _arr(x), _arr(y), _arr(z)
     d, n = _dims(dims)
     _check(lib().orc_broadcast(op, _p(x.a), _s(x.si), _p(y.a), _s(y.si), _p(z.a), _s(z.si), _s(d), n), "broadcast")
+    return z.a
+
+
+def transform_bool(op, x, z):
+    x, z = _arr(x), _arr(z)
+    _check(lib().orc_transform_bool(op, _p(x.a), _s(x.si), _p(z.a), _s(z.si)), "transform_bool")
+    return z.a
+
+
+def summary_stats(op, x, z, dims=None, bias_corrected=False):
+    x, z = _arr(x), _arr(z)
+    d, n = _dims(dims)
+    _check(lib().orc_summary_stats(op, _p(x.a), _s(x.si), _p(z.a), _s(z.si), _s(d), n, int(bias_corrected)), "summary_stats")
+    return z.a
+
+
+def reduce_long(op, x, z, dims=None):
+    x, z = _arr(x), _arr(z)
+    d, n = _dims(dims)
+    _check(lib().orc_reduce_count(op, _p(x.a), _s(x.si), _p(z.a), _s(z.si), _s(d), n), "reduce_long")
+    return z.a
+
+
+def reduce_bool(op, x, z, dims=None):
+    x, z = _arr(x), _arr(z)
+    d, n = _dims(dims)
+    _check(lib().orc_reduce_count(10 + op, _p(x.a), _s(x.si), _p(z.a), _s(z.si), _s(d), n), "reduce_bool")
     return z.a
 
 

@@ -238,3 +238,59 @@ def test_entropy_reductions(ex, oracle, op, dtype, dims):
     got = ex.exec_reduce_float(op, dx, dims)
     rtol, atol = {FLOAT32: (2e-5, 1e-6), DOUBLE: (1e-12, 1e-13), HALF: (1e-2, 1e-2), BFLOAT16: (2e-2, 2e-2)}[dtype]
     assert_close(np.asarray(_got(got, dtype)).reshape(out_shape), np.asarray(_f(oz)).reshape(out_shape), rtol, atol, "entropy op %d dtype %d dims %s" % (op, dtype, dims))
+
+
+@pytest.mark.parametrize("dtype", [FLOAT32, DOUBLE, BFLOAT16])
+@pytest.mark.parametrize("dims", [[2], [0, 2], [1], None])
+def test_summary_stats(ex, oracle, dtype, dims):
+    from deeplearning4j_amd.executioner import SummaryStats
+    rng = np.random.default_rng(70)
+    x = rng.normal(100.0 if dtype != BFLOAT16 else 1.0, 2.0, (7, 9, 300))
+    ox, dx = _pair(oracle, x, dtype)
+    shape = () if dims is None else tuple(s for i, s in enumerate(x.shape) if i not in dims)
+    for op in (SummaryStats.Variance, SummaryStats.StandardDeviation):
+        for bias in (False, True):
+            oz = oracle.Arr(np.zeros(shape, ox.a.dtype), ox.dt)
+            oracle.summary_stats(op, ox, oz, dims, bias)
+            got = ex.exec_summary_stats(op, dx, dims, bias)
+            rtol = {FLOAT32: 2e-6, DOUBLE: 1e-11, BFLOAT16: 1e-2}[dtype]
+            assert_close(np.asarray(_got(got, dtype)).reshape(shape), np.asarray(_f(oz)).reshape(shape), rtol, 0, "summary stats op %d bias %s dims %s" % (op, bias, dims))
+
+
+def test_summary_stats_long_run_is_split_over_blocks(ex, oracle):
+    from deeplearning4j_amd.executioner import SummaryStats
+    rng = np.random.default_rng(71)
+    x = rng.normal(50.0, 3.0, (3, 400000)).astype(np.float32)
+    X = NDArray.from_numpy(x)
+    want = np.var(x.astype(np.float64), axis=1, ddof=1)
+    got = ex.exec_summary_stats(SummaryStats.Variance, X, [1], True).to_numpy()
+    assert_close(got, want, 2e-6, 0, "variance of long rows")
+    got = ex.exec_summary_stats(SummaryStats.StandardDeviation, X).to_numpy()
+    assert_close(np.asarray(got).reshape(()), np.std(x.astype(np.float64)), 2e-6, 0, "std of everything")
+
+
+def test_reduce_long_bool_and_transform_bool(ex, oracle):
+    from deeplearning4j_amd.executioner import ReduceBool, ReduceLong, TransformBool
+    from deeplearning4j_amd.ndarray import BOOL, INT64
+    rng = np.random.default_rng(72)
+    x = np.round(rng.normal(0, 1, (6, 50, 9))).astype(np.float32)          # many exact zeros
+    X = NDArray.from_numpy(x)
+    for dims in ([1], [0, 2], None):
+        shape = () if dims is None else tuple(s for i, s in enumerate(x.shape) if i not in dims)
+        for op in (ReduceLong.CountNonZero, ReduceLong.CountZero):
+            want = oracle.reduce_long(op, x, np.zeros(shape, np.int64), dims)
+            got = ex.exec_reduce_long(op, X, dims).to_numpy()
+            assert np.array_equal(np.asarray(got).reshape(shape), want), (op, dims)
+        for op in (ReduceBool.Any, ReduceBool.All):
+            want = oracle.reduce_bool(op, x, np.zeros(shape, np.bool_), dims)
+            got = ex.exec_reduce_bool(op, X, dims).to_numpy()
+            assert np.array_equal(np.asarray(got).reshape(shape), want), (op, dims)
+    v = np.array([0.0, -0.0, 1.0, -3.0, np.inf, -np.inf, np.nan, 1e300, 5e-324, 2.5], np.float64)
+    for dt in (np.float64, np.float32):
+        vv = v.astype(dt)
+        V = NDArray.from_numpy(vv)
+        for op in (TransformBool.IsInf, TransformBool.IsNan, TransformBool.IsFinite, TransformBool.IsInfOrNan, TransformBool.IsPositive,
+                   TransformBool.Not, TransformBool.IsNegative):
+            want = oracle.transform_bool(op, vv, np.zeros(vv.shape, np.bool_))
+            got = ex.exec_transform_bool(op, V).to_numpy()
+            assert np.array_equal(got, want), (op, dt)

@@ -264,3 +264,36 @@ def test_entropy_reductions_match_scipy():
     p32 = p.astype(np.float32)
     np.testing.assert_allclose(O.reduce_float(8, p32, np.zeros(5, np.float32), [1]), stats.entropy(p, axis=1), rtol=2e-6)
     np.testing.assert_allclose(O.reduce_float(10, p32.T.copy(), np.zeros(5, np.float32), [0]), stats.entropy(p, base=2, axis=1), rtol=2e-6)
+
+
+def test_summary_stats_match_numpy_var_std():
+    rng = np.random.default_rng(8)
+    x = rng.normal(1000.0, 2.0, (6, 5, 40))          # large mean: a sum-of-squares formula would lose every digit
+    for dims, axis in (([2], 2), ([0, 2], (0, 2)), (None, None)):
+        shape = () if dims is None else tuple(s for i, s in enumerate(x.shape) if i not in dims)
+        for bias in (False, True):
+            v = O.summary_stats(0, x, np.zeros(shape), dims, bias)
+            s = O.summary_stats(1, x, np.zeros(shape), dims, bias)
+            np.testing.assert_allclose(v, np.var(x, axis=axis, ddof=int(bias)), rtol=1e-12)
+            np.testing.assert_allclose(s, np.std(x, axis=axis, ddof=int(bias)), rtol=1e-12)
+    one = np.array([[3.0], [4.0]])
+    np.testing.assert_array_equal(O.summary_stats(0, one, np.zeros(2), [1], True), [0.0, 0.0])     # n <= 1 gives 0, not NaN
+    x32 = x.astype(np.float32)
+    np.testing.assert_allclose(O.summary_stats(0, x32, np.zeros((6, 5), np.float32), [2]), np.var(x32.astype(np.float64), axis=2), rtol=1e-6)
+
+
+def test_counts_any_all_and_predicates():
+    x = np.array([[0.0, 1.5, -2.0, 0.0], [0.0, 0.0, 0.0, 0.0], [1.0, 2.0, 3.0, -0.5], [-1.0, 1.0, 0.0, 0.0]])
+    np.testing.assert_array_equal(O.reduce_long(0, x, np.zeros(4, np.int64), [1]), np.count_nonzero(x, axis=1))
+    np.testing.assert_array_equal(O.reduce_long(1, x, np.zeros(4, np.int64), [1]), (x == 0).sum(1))
+    np.testing.assert_array_equal(O.reduce_long(0, x, np.zeros((), np.int64)), np.count_nonzero(x))
+    # Any is "the sum is positive" in the reference (ops.h:1200-1206): row 3 sums to 0 and row 0 to -0.5
+    np.testing.assert_array_equal(O.reduce_bool(0, x, np.zeros(4, np.bool_), [1]), [False, False, True, False])
+    np.testing.assert_array_equal(O.reduce_bool(1, x, np.zeros(4, np.bool_), [1]), [False, False, True, False])
+    b = np.array([[True, False], [False, False], [True, True]])
+    np.testing.assert_array_equal(O.reduce_bool(0, b, np.zeros(3, np.bool_), [1]), b.any(1))
+    np.testing.assert_array_equal(O.reduce_bool(1, b, np.zeros(3, np.bool_), [1]), b.all(1))
+    v = np.array([0.0, -0.0, 1.0, -3.0, np.inf, -np.inf, np.nan, 1e300])
+    for op, fn in ((1, np.isinf), (2, np.isnan), (3, np.isfinite), (4, lambda a: ~np.isfinite(a)), (6, lambda a: a > 0), (7, lambda a: a == 0),
+                   (8, lambda a: a < 0)):
+        np.testing.assert_array_equal(O.transform_bool(op, v, np.zeros(v.shape, np.bool_)), fn(v), err_msg="op %d" % op)
