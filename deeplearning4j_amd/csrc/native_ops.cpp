@@ -974,6 +974,61 @@ const Nd4jLong* getShape(OpaqueShapeList* list, Nd4jLong i) {
 void deleteShapeList(Nd4jPointer shapeList) { delete static_cast<Nd4jHipShapeList*>(shapeList); }
 
 void nd4jhipSetSyncAfterCustomOp(int enable) { Environment::get().syncAfterCustomOp = enable != 0; }
+
+// ---- stream capture: a launch-bound sequence of ops recorded once and replayed as one HIP graph -----------------------
+namespace {
+struct CapturedGraph { hipGraph_t graph = nullptr; hipGraphExec_t exec = nullptr; };
+bool g_capturing = false;
+bool g_syncBeforeCapture = true;
+}
+int nd4jhipGraphBeginCapture(void) {
+  GUARD_BEGIN
+  ND4J_REQUIRE(!g_capturing, "nd4jhipGraphBeginCapture: a capture is already in progress");
+  // every op call between begin and end records its kernels instead of running them: nothing may wait on the stream
+  g_syncBeforeCapture = Environment::get().syncAfterCustomOp;
+  Environment::get().syncAfterCustomOp = false;
+  HIP_CHECK(hipStreamSynchronize(execStream()));
+  HIP_CHECK(hipStreamBeginCapture(execStream(), hipStreamCaptureModeRelaxed));
+  g_capturing = true;
+  return 0;
+  GUARD_END(1)
+}
+Nd4jPointer nd4jhipGraphEndCapture(void) {
+  GUARD_BEGIN
+  ND4J_REQUIRE(g_capturing, "nd4jhipGraphEndCapture: no capture in progress");
+  g_capturing = false;
+  Environment::get().syncAfterCustomOp = g_syncBeforeCapture;
+  CapturedGraph* cg = new CapturedGraph();
+  hipError_t e = hipStreamEndCapture(execStream(), &cg->graph);
+  if (e != hipSuccess || cg->graph == nullptr) {
+    delete cg;
+    (void)hipGetLastError();
+    ND4J_THROW(std::string("nd4jhipGraphEndCapture: the capture was invalidated (an op waited on the stream or copied synchronously): ") + hipGetErrorString(e));
+  }
+  e = hipGraphInstantiate(&cg->exec, cg->graph, nullptr, nullptr, 0);
+  if (e != hipSuccess) {
+    (void)hipGraphDestroy(cg->graph);
+    delete cg;
+    ND4J_THROW(std::string("nd4jhipGraphEndCapture: hipGraphInstantiate failed: ") + hipGetErrorString(e));
+  }
+  return cg;
+  GUARD_END(nullptr)
+}
+int nd4jhipGraphLaunch(Nd4jPointer graph) {
+  GUARD_BEGIN
+  ND4J_REQUIRE(graph != nullptr, "nd4jhipGraphLaunch: graph is null");
+  ND4J_REQUIRE(!g_capturing, "nd4jhipGraphLaunch: a capture is in progress");
+  HIP_CHECK(hipGraphLaunch(static_cast<CapturedGraph*>(graph)->exec, execStream()));
+  return 0;
+  GUARD_END(1)
+}
+void nd4jhipGraphDestroy(Nd4jPointer graph) {
+  if (!graph) return;
+  CapturedGraph* cg = static_cast<CapturedGraph*>(graph);
+  if (cg->exec) (void)hipGraphExecDestroy(cg->exec);
+  if (cg->graph) (void)hipGraphDestroy(cg->graph);
+  delete cg;
+}
 const char* nd4jhipBuildInfo(void) { return "nd4j-hip gfx950 (hand-written HIP kernels; no CPU fallback)"; }
 
 }  // extern "C"

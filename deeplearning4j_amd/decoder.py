@@ -67,6 +67,8 @@ class Decoder:
         self.length = 0            # tokens in the cache
         self._programs = {}        # (T_new, past) -> list of bound op calls
         self._buffers = {}         # T_new -> activation arrays
+        self.use_graphs = False    # replay each single-token step as one captured HIP graph (one graph per cache length)
+        self._graphs = {}          # (past, source of the fed-back ids) -> captured graph handle
 
     @staticmethod
     def _resident(arr):
@@ -177,6 +179,11 @@ class Decoder:
             src = self._last_next
             if not hasattr(self, "_feed") or self._feed[0] is not src:
                 self._feed = (src, self._assign(src.view((self.B, 1), (1, 1)), a["ids"]))
+            if self.use_graphs and self.dtype in (BFLOAT16, HALF):   # fp32 attention goes through temporaries and a wait: not capturable
+                self._graph_step(prog)
+                self.length += 1
+                self._last_next = a["next"]
+                return a["next"]
             self._feed[1]()
         else:
             ids = np.asarray(ids, dtype=np.int64)
@@ -192,6 +199,34 @@ class Decoder:
         self._last_next = a["next"]
         return a["next"]
 
+    def _graph_step(self, prog):
+        """One decode step through a captured graph: the ops of the step (feedback copy of the last id included) are recorded
+        the first time this cache length is seen -- the kernels' arguments depend on it -- and replayed from then on.
+        Arrays, views and op contexts are built before the capture starts, so recording only launches kernels."""
+        L = self.L
+        key = (self.length, id(self._last_next))   # the recorded feedback copy reads the array the last ids were written to
+        g = self._graphs.get(key)
+        if g is None:
+            if L.nd4jhipGraphBeginCapture() != 0:
+                N.check("nd4jhipGraphBeginCapture")
+            try:
+                self._feed[1]()
+                for op in prog:
+                    op()
+            finally:
+                g = L.nd4jhipGraphEndCapture()
+            if not g:
+                N.check("nd4jhipGraphEndCapture")
+                raise N.NativeOpsError("nd4jhipGraphEndCapture returned no graph")
+            self._graphs[key] = g
+        if L.nd4jhipGraphLaunch(g) != 0:
+            N.check("nd4jhipGraphLaunch")
+
+    def close(self):
+        for g in self._graphs.values():
+            self.L.nd4jhipGraphDestroy(g)
+        self._graphs = {}
+
     def logits(self, T=None):
         """Logits [B, vocab] of the last forward call (as float32 on the host)."""
         T = T or max(k for k in self._buffers if self._buffers[k]["next"] is self._last_next)
@@ -200,18 +235,29 @@ class Decoder:
     def generate(self, prompt_ids, n_steps):
         """Prefill with `prompt_ids` [B, T0], then `n_steps - 1` further greedy steps; returns ids [B, n_steps]."""
         self.reset()
-        out = []
+        hist = self._history(n_steps)
         nxt = self.forward(prompt_ids)
-        held = [self._snapshot(nxt)]
-        for _ in range(n_steps - 1):
+        self._snapshot(nxt, hist, 0)
+        for i in range(1, n_steps):
             nxt = self.forward(None)
-            held.append(self._snapshot(nxt))
+            self._snapshot(nxt, hist, i)
         self.ex.synchronize()
-        return np.stack([h.to_numpy() for h in held], axis=1)
+        return np.ascontiguousarray(hist[0].to_numpy().T)
 
-    def _snapshot(self, arr):
-        """Device-side copy of a small array (the per-step ids), so that generate() reads back once at the end."""
-        z = NDArray.empty(arr.shape, arr.dtype)
-        self.L.execTransformAny(None, 0, arr.handle, None, z.handle)
+    def _history(self, n_steps):
+        """[n_steps, B] id buffer with one row view per step, kept between calls so that steady-state generation allocates nothing."""
+        h = getattr(self, "_hist", None)
+        if h is None or h[0].shape[0] < n_steps:
+            buf = NDArray.empty((n_steps, self.B), INT64)
+            h = (buf, [buf.view((self.B,), (1,), i * self.B) for i in range(n_steps)])
+            self._hist = h
+        if h[0].shape[0] != n_steps:
+            buf = NDArray.empty((n_steps, self.B), INT64)
+            h = (buf, [buf.view((self.B,), (1,), i * self.B) for i in range(n_steps)])
+            self._hist = h
+        return h
+
+    def _snapshot(self, arr, hist, i):
+        """Device-side copy of the step's ids into row i of the history, so that generate() reads back once at the end."""
+        self.L.execTransformAny(None, 0, arr.handle, None, hist[1][i].handle)
         N.check("execTransformAny")
-        return z

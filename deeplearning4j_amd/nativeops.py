@@ -164,6 +164,10 @@ _SIGS = {
     "nd4jhipCreateTimingEvent": (c_ptr, []),
     "nd4jhipEventElapsedMs": (ctypes.c_float, [c_ptr, c_ptr]),
     "nd4jhipSetSyncAfterCustomOp": (None, [ctypes.c_int]),
+    "nd4jhipGraphBeginCapture": (ctypes.c_int, []),
+    "nd4jhipGraphEndCapture": (c_ptr, []),
+    "nd4jhipGraphLaunch": (ctypes.c_int, [c_ptr]),
+    "nd4jhipGraphDestroy": (None, [c_ptr]),
     "nd4jhipBuildInfo": (ctypes.c_char_p, []),
 }
 

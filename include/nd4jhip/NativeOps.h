@@ -227,6 +227,14 @@ ND4JHIP_EXPORT float nd4jhipEventElapsedMs(Nd4jPointer startEvent, Nd4jPointer s
 /* 1: execCustomOp2 synchronises the stream before returning (default, reference behaviour); 0: the caller
  * synchronises itself (streamSynchronize / dbSyncToPrimary) -- used by tight decode loops. */
 ND4JHIP_EXPORT void nd4jhipSetSyncAfterCustomOp(int enable);
+/* Stream capture for launch-bound op sequences (a decode step is ~150 kernels of a few microseconds each): every op
+ * call between Begin and End is recorded on the execution stream instead of run; End returns a handle (null + error slot
+ * when an op waited on the stream, copied synchronously or allocated, which invalidates a capture); Launch replays the
+ * recorded kernels with the arguments they were recorded with.  Build arrays, views and OpContexts before Begin. */
+ND4JHIP_EXPORT int nd4jhipGraphBeginCapture(void);
+ND4JHIP_EXPORT Nd4jPointer nd4jhipGraphEndCapture(void);
+ND4JHIP_EXPORT int nd4jhipGraphLaunch(Nd4jPointer graph);
+ND4JHIP_EXPORT void nd4jhipGraphDestroy(Nd4jPointer graph);
 ND4JHIP_EXPORT const char* nd4jhipBuildInfo(void);
 
 #ifdef __cplusplus
