@@ -1081,12 +1081,129 @@ static bool mfmaEligible(const GemmDesc& d, const void* A, const void* B, size_t
   return true;
 }
 
+// ---- up to four rows of x against row-major W (a decode step's projections) --------------------------------------------------
+// One block of 16 waves per strip of CW output columns and all of K: a lane loads 8 neighbouring columns of one k-row
+// (16 bytes), a wave covers 64/(CW/8) k-rows per instruction, the waves interleave rows, and a lane issues up to eight
+// independent loads before it touches the first -- with so few strips (N/CW blocks) a CU has to keep about 100 KB in
+// flight to stream at its share of the bandwidth.  x sits in LDS.  Partial sums meet through lane shuffles (rows of a wave)
+// and LDS (waves), in a fixed order.  One launch, no partial tiles in global memory.
+template <typename T, int M, int CW>
+__global__ __launch_bounds__(1024) void gemv_strip(GemmArgs g, const T* __restrict__ x, const T* __restrict__ W, T* __restrict__ out) {
+  constexpr int NWAVE = 16, LPR = CW / 8, RPW = 64 / LPR, RB = NWAVE * RPW;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  float* red = reinterpret_cast<float*>(smem_raw);                      // [16 waves][M][CW]
+  T* xs = reinterpret_cast<T*>(red + NWAVE * M * CW);                    // [M][K]
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, cg = lane % LPR, rk = lane / LPR;
+  const LongType K = g.K;
+  const LongType c0 = (LongType)blockIdx.x * CW + cg * 8;
+  const T* wp = W + (LongType)(wave * RPW + rk) * g.bRow + c0;
+  const LongType step = (LongType)RB * g.bRow;
+  LongType k = wave * RPW + rk;
+  // the first batch of weight loads goes out before x is staged
+  u32x4 w[8];
+  const int first = (int)((K - k + RB - 1) / RB < 8 ? (K - k + RB - 1) / RB : 8);
+#pragma unroll
+  for (int i = 0; i < 8; i++)
+    if (i < first) w[i] = *reinterpret_cast<const u32x4*>(wp + i * step);
+  for (LongType i = t; i < (LongType)M * K; i += 1024) {
+    const LongType m = i / K, kk = i - m * K;
+    xs[i] = x[m * g.aRow + kk];
+  }
+  __syncthreads();
+  float acc[M][8];
+#pragma unroll
+  for (int m = 0; m < M; m++)
+#pragma unroll
+    for (int e = 0; e < 8; e++) acc[m][e] = 0.f;
+  auto fma8 = [&](const u32x4& wq, LongType kk) {
+    float wv[8];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      wv[2 * q] = to_float(__builtin_bit_cast(T, (unsigned short)(wq[q] & 0xffffu)));
+      wv[2 * q + 1] = to_float(__builtin_bit_cast(T, (unsigned short)(wq[q] >> 16)));
+    }
+#pragma unroll
+    for (int m = 0; m < M; m++) {
+      const float xv = to_float(xs[(LongType)m * K + kk]);
+#pragma unroll
+      for (int e = 0; e < 8; e++) acc[m][e] = fmaf(xv, wv[e], acc[m][e]);
+    }
+  };
+  int have = first;
+  while (have > 0) {
+    const LongType kNext = k + (LongType)have * RB;
+    const T* wpNext = wp + (LongType)have * step;
+    u32x4 nw[8];
+    const int more = (int)((K - kNext + RB - 1) / RB < 8 ? (kNext < K ? (K - kNext + RB - 1) / RB : 0) : 8);
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+      if (i < more) nw[i] = *reinterpret_cast<const u32x4*>(wpNext + i * step);
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+      if (i < have) fma8(w[i], k + (LongType)i * RB);
+#pragma unroll
+    for (int i = 0; i < 8; i++) w[i] = nw[i];
+    k = kNext; wp = wpNext; have = more;
+  }
+  // rows of the wave: lanes that share a column group
+#pragma unroll
+  for (int off = LPR; off < 64; off <<= 1)
+#pragma unroll
+    for (int m = 0; m < M; m++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) acc[m][e] += __shfl_xor(acc[m][e], off, 64);
+  if (rk == 0) {
+#pragma unroll
+    for (int m = 0; m < M; m++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) red[(wave * M + m) * CW + cg * 8 + e] = acc[m][e];
+  }
+  __syncthreads();
+  if (t < M * CW) {
+    const int m = t / CW, c = t % CW;
+    float v = 0.f;
+#pragma unroll
+    for (int q = 0; q < NWAVE; q++) v += red[(q * M + m) * CW + c];
+    const LongType col = (LongType)blockIdx.x * CW + c;
+    if (g.bias) v += to_float(static_cast<const T*>(g.bias)[col]);
+    out[(LongType)m * g.cRow + col] = Conv<T>::from(v);
+  }
+}
+template <typename T, int M>
+static void launchGemvStripM(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C) {
+  if (g.N >= 1536 && g.N % 64 == 0) {
+    const size_t lds = (size_t)16 * M * 64 * sizeof(float) + (size_t)M * g.K * sizeof(T);
+    hipLaunchKernelGGL((gemv_strip<T, M, 64>), dim3((unsigned)(g.N / 64)), dim3(1024), lds, s, g, (const T*)A, (const T*)B, (T*)C);
+  } else {
+    const size_t lds = (size_t)16 * M * 32 * sizeof(float) + (size_t)M * g.K * sizeof(T);
+    hipLaunchKernelGGL((gemv_strip<T, M, 32>), dim3((unsigned)(g.N / 32)), dim3(1024), lds, s, g, (const T*)A, (const T*)B, (T*)C);
+  }
+}
+// whether the strip kernel takes this product: a few dense rows, W row-major with aligned rows, plain C = A B (+ bias)
+template <typename T>
+static bool tryGemvStrip(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
+  if (d.M < 1 || d.M > 4 || d.batch != 1 || d.alpha != 1.f || d.beta != 0.f) return false;
+  if (d.aCol != 1 || d.bCol != 1 || d.cCol != 1 || d.bRow % 8 != 0) return false;
+  if (d.N % 32 != 0 || d.K % 256 != 0 || d.N < 256) return false;
+  if ((reinterpret_cast<uintptr_t>(B) & 15) != 0) return false;
+  if ((size_t)16 * d.M * 64 * sizeof(float) + (size_t)d.M * d.K * sizeof(T) > 60 * 1024) return false;
+  GemmArgs g = toArgs(d);
+  switch (d.M) {
+    case 1: launchGemvStripM<T, 1>(s, g, A, B, C); break;
+    case 2: launchGemvStripM<T, 2>(s, g, A, B, C); break;
+    case 3: launchGemvStripM<T, 3>(s, g, A, B, C); break;
+    default: launchGemvStripM<T, 4>(s, g, A, B, C); break;
+  }
+  return true;
+}
+
 template <typename T>
 static void dispatch16(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
   bool aKC = false, bKC = false;
   const bool eligible = (d.M * d.N >= 1024 || (d.M == 1 && d.N >= 64)) && d.K >= 32 && mfmaEligible(d, A, B, sizeof(T), aKC, bKC);
   // x[1, K] times row-major W[K, N]: the split-K tile kernel streams W with far more loads in flight than the
   // column-sum GEMV (the unused 31 rows of the MFMA tile cost nothing here)
+  if (tryGemvStrip<T>(s, d, A, B, C)) return;
   const bool rowTimesRowMajor = d.M == 1 && eligible && aKC && !bKC && d.batch == 1;
   if (!rowTimesRowMajor && tryGemv<T>(s, d, A, B, C)) return;
   if (eligible) {

@@ -208,6 +208,34 @@ def test_xw_plus_b_vs_oracle(ex, oracle, dtype, tol, M, K, N):
         assert_close(z3.to_float().reshape(M, N), _f(oz), tol, tol, "xw_plus_b, rank-3 x")
 
 
+@pytest.mark.parametrize("dtype", [BFLOAT16, HALF])
+@pytest.mark.parametrize("M", [1, 2, 3, 4])
+@pytest.mark.parametrize("K,N", [(768, 2304), (768, 768), (3072, 768), (768, 3072), (256, 288), (512, 1536), (320, 1536)])
+def test_few_rows_times_row_major_weights(ex, oracle, dtype, M, K, N):
+    """The decode-step shape: up to four rows of x against row-major weights (one strip kernel, no split-K partials),
+    with and without the bias row, against the fp32-accumulating oracle."""
+    rng = np.random.default_rng(M * 7 + K + N)
+    x = rng.normal(0, 1, (M, K))
+    w = rng.normal(0, 1 / math.sqrt(K), (K, N))
+    b = rng.normal(0, 1, (N,))
+    ox, dx = _pair(oracle, x, dtype)
+    ow, dw = _pair(oracle, w, dtype)
+    ob, db = _pair(oracle, b, dtype)
+    oz = _ozeros(oracle, (M, N), dtype)
+    oracle.matmul(ox, ow, oz, accumulate=1)
+    z = ex.exec_custom("matmul", [dx, dw])[0]
+    assert_close(z.to_float(), _f(oz), 1e-2, 1e-2, "few rows x row-major W")
+    oracle.add_row_vector(oz, ob, oz)
+    zb = ex.exec_custom("xw_plus_b", [dx, dw, db])[0]
+    assert_close(zb.to_float(), _f(oz), 1e-2, 1e-2, "few rows x row-major W + bias")
+    # the same rows as a strided view (row stride 2K) give the same bits
+    wide = np.zeros((M, 2 * K), np.asarray(ox.a).dtype)
+    wide[:, :K] = np.asarray(ox.a)
+    xv = NDArray.from_numpy(wide, dtype).view((M, K), (2 * K, 1), 0)
+    zv = ex.exec_custom("xw_plus_b", [xv, dw, db], outputs=[NDArray.empty((M, N), dtype)])[0]
+    assert np.array_equal(zv.to_numpy(), zb.to_numpy())
+
+
 def test_xw_plus_b_errors(ex):
     x = NDArray.from_numpy(np.ones((4, 8), np.float32))
     w = NDArray.from_numpy(np.ones((9, 5), np.float32))
