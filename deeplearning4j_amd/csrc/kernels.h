@@ -74,7 +74,11 @@ enum ReduceKind : int {
 enum IndexKind : int { I_MAX, I_MIN, I_AMAX, I_AMIN, I_COUNT };
 // reductions whose accumulator or output type differs from the input's: summary statistics (double triple n, mean, M2),
 // counts (INT64 out), Any / All (BOOL out)
-enum MiscReduceKind : int { M_VARIANCE, M_STDDEV, M_COUNT_NONZERO, M_COUNT_ZERO, M_ANY, M_ALL };
+enum MiscReduceKind : int {
+  M_VARIANCE, M_STDDEV, M_COUNT_NONZERO, M_COUNT_ZERO, M_ANY, M_ALL,
+  // two-operand reductions (reduce3), z in a float type
+  M3_MANHATTAN, M3_EUCLIDEAN, M3_COSINE_SIMILARITY, M3_DOT, M3_COSINE_DISTANCE, M3_JACCARD, M3_HAMMING
+};
 
 // outer = kept dims (one output element each), inner = reduced dims
 struct ReducePlan {
@@ -90,7 +94,8 @@ void launchReduce(hipStream_t s, ReduceKind k, DataType xdt, DataType zdt, const
                   void* scratch, size_t scratchBytes);
 // zdt: the float type for variance / standard deviation, INT64 for counts, BOOL for Any / All
 void launchReduceMisc(hipStream_t s, MiscReduceKind k, DataType xdt, DataType zdt, const void* x, void* z, const ReducePlan& p,
-                      bool biasCorrected, void* scratch, size_t scratchBytes);
+                      bool biasCorrected, void* scratch, size_t scratchBytes, const void* y = nullptr, DataType ydt = FLOAT32,
+                      const ReducePlan* yPlan = nullptr);
 void launchIndexReduce(hipStream_t s, IndexKind k, DataType xdt, DataType zdt, const void* x, void* z,
                        const ReducePlan& p, void* scratch, size_t scratchBytes);
 

@@ -736,6 +736,34 @@ static void runReduceMisc(const char* fn, MiscReduceKind k, NDArray* x, NDArray*
                    lc->reductionBuffer, LaunchContext::REDUCTION_BYTES);
   registerSpecialUse({z}, {x});
 }
+// reduce3: z[o] = f(x tad o, y tad o) with y shaped like x (loops/cpu/reduce3.hpp); opNums loops/legacy_ops.h:88-90
+static void runReduce3(const char* fn, int opNum, NDArray* x, NDArray* y, NDArray* z, std::vector<LongType> d) {
+  MiscReduceKind k;
+  switch (opNum) {
+    case 0: k = M3_MANHATTAN; break; case 1: k = M3_EUCLIDEAN; break; case 2: k = M3_COSINE_SIMILARITY; break; case 3: k = M3_DOT; break;
+    case 5: k = M3_COSINE_DISTANCE; break; case 6: k = M3_JACCARD; break; case 7: k = M3_HAMMING; break;
+    default: ND4J_THROW(std::string(fn) + ": opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");   // 4 EqualsWithEps reads extra parameters
+  }
+  ND4J_REQUIRE(isFloatType(z->dataType()), std::string(fn) + ": Z must have a floating point type");
+  ND4J_REQUIRE(x->rankOf() == y->rankOf() && x->lengthOf() == y->lengthOf(), std::string(fn) + ": x and y must have the same shape");
+  for (int i = 0; i < x->rankOf(); i++) ND4J_REQUIRE(x->sizeAt(i) == y->sizeAt(i), std::string(fn) + ": x and y must have the same shape");
+  ND4J_REQUIRE(!x->isEmpty(), std::string(fn) + ": reductions of empty arrays are not implemented in nd4j-hip");
+  if (z->isEmpty()) return;
+  if (z->lengthOf() == 1 && x->lengthOf() != 1) {
+    bool keptAllUnit = true;
+    std::vector<bool> red(x->rankOf(), false);
+    for (auto v : d) red[v] = true;
+    for (int i = 0; i < x->rankOf(); i++) if (!red[i] && x->sizeAt(i) != 1) keptAllUnit = false;
+    if (!keptAllUnit) d.clear();
+  }
+  ReducePlan p = buildReducePlan(x->shapeInfo(), z->shapeInfo(), d, false);
+  ReducePlan py = buildReducePlan(y->shapeInfo(), z->shapeInfo(), d, false);
+  auto lc = LaunchContext::defaultContext();
+  prepareSpecialUse({z}, {x, y});
+  launchReduceMisc(lc->execStream, k, x->dataType(), z->dataType(), x->specialBuffer(), z->specialBuffer(), p, false, lc->reductionBuffer,
+                   LaunchContext::REDUCTION_BYTES, y->specialBuffer(), y->dataType(), &py);
+  registerSpecialUse({z}, {x, y});
+}
 static MiscReduceKind summaryKind(int opNum) {
   switch (opNum) {  // loops/legacy_ops.h:69
     case 0: return M_VARIANCE; case 1: return M_STDDEV;
@@ -795,6 +823,22 @@ void execReduceBool(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDAr
 void execReduceBool2(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
   GUARD_BEGIN
   reduceBool("execReduceBool2", opNum, xa, za, da);
+  GUARD_END_VOID
+}
+void execReduce3(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray ya, OpaqueNDArray za) {
+  GUARD_BEGIN
+  runReduce3("execReduce3", opNum, arr(xa, "execReduce3", "x"), arr(ya, "execReduce3", "y"), arr(za, "execReduce3", "z"), {});
+  GUARD_END_VOID
+}
+void execReduce3Scalar(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray ya, OpaqueNDArray za) {
+  GUARD_BEGIN
+  runReduce3("execReduce3Scalar", opNum, arr(xa, "execReduce3Scalar", "x"), arr(ya, "execReduce3Scalar", "y"), arr(za, "execReduce3Scalar", "z"), {});
+  GUARD_END_VOID
+}
+void execReduce3Tad(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray ya, OpaqueNDArray za, OpaqueNDArray da) {
+  GUARD_BEGIN
+  NDArray* x = arr(xa, "execReduce3Tad", "x");
+  runReduce3("execReduce3Tad", opNum, x, arr(ya, "execReduce3Tad", "y"), arr(za, "execReduce3Tad", "z"), hostDims(da, x->rankOf(), "execReduce3Tad"));
   GUARD_END_VOID
 }
 void execTransformBool(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {

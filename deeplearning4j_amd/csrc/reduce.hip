@@ -272,8 +272,9 @@ void launchReduce(hipStream_t st, ReduceKind k, DataType xdt, DataType zdt, cons
 // (summarystatsreduce.h:190-211), also what the finish kernel applies across splits.
 struct MiscArgs {
   DevShape outer, inner, zOuter;
+  DevShape yOuter, yInner;          // second operand of the reduce3 kinds (same shapes, own strides)
   LongType outerLen, innerLen, segLen;
-  int splits, kind, bias, xdt, zdt;
+  int splits, kind, bias, xdt, zdt, ydt;
 };
 __device__ __forceinline__ double block_sum(double v, double* lds) {
   const int t = threadIdx.x;
@@ -299,10 +300,17 @@ __device__ __forceinline__ double misc_result(const MiscArgs& a, double n, doubl
     }
     case M_ANY: return cnt > 0.0 ? 1.0 : 0.0;                     // ops.h:1200-1206: the sum of the elements is positive
     case M_ALL: return cnt > 0.0 ? 0.0 : 1.0;                     // here cnt counts the zero elements
+    // reduce3 (ops.h:117-134,483-541): mean = first sum, m2 and cnt = the two auxiliary sums
+    case M3_MANHATTAN: case M3_DOT: return mean;
+    case M3_EUCLIDEAN: return sqrt(mean);
+    case M3_COSINE_SIMILARITY: return mean / (sqrt(m2) * sqrt(cnt));
+    case M3_COSINE_DISTANCE: return 1.0 - mean / (sqrt(m2) * sqrt(cnt));
+    case M3_JACCARD: return 1.0 - m2 / cnt;
+    case M3_HAMMING: return mean / n;
     default: return cnt;
   }
 }
-__global__ __launch_bounds__(256) void misc_partial(MiscArgs a, const void* __restrict__ x, void* __restrict__ z,
+__global__ __launch_bounds__(256) void misc_partial(MiscArgs a, const void* __restrict__ x, const void* __restrict__ y, void* __restrict__ z,
                                                     double* __restrict__ partials) {
   __shared__ double lds[256];
   const LongType unit = blockIdx.x, row = unit / a.splits;
@@ -315,7 +323,24 @@ __global__ __launch_bounds__(256) void misc_partial(MiscArgs a, const void* __re
   const LongType st = linear ? a.inner.stride[0] : 0;
   auto at = [&](LongType q) { return load_any(x, a.xdt, base + (linear ? q * st : walk<LongType>(a.inner, q))); };
   double n = (double)(j1 - j0), mean = 0.0, m2 = 0.0, cnt = 0.0;
-  if (a.kind == M_VARIANCE || a.kind == M_STDDEV) {
+  if (a.kind >= M3_MANHATTAN) {
+    const LongType ybase = walk<LongType>(a.yOuter, row);
+    const bool ylinear = a.yInner.rank == 1;
+    const LongType yst = ylinear ? a.yInner.stride[0] : 0;
+    double s0 = 0.0, s1 = 0.0, s2 = 0.0;
+    for (LongType q = j0 + threadIdx.x; q < j1; q += 256) {
+      const double u = at(q), v = load_any(y, a.ydt, ybase + (ylinear ? q * yst : walk<LongType>(a.yInner, q)));
+      switch (a.kind) {
+        case M3_MANHATTAN: s0 += fabs(u - v); break;
+        case M3_EUCLIDEAN: s0 += (u - v) * (u - v); break;
+        case M3_DOT: s0 += u * v; break;
+        case M3_COSINE_SIMILARITY: case M3_COSINE_DISTANCE: s0 += u * v; s1 += u * u; s2 += v * v; break;
+        case M3_JACCARD: s1 += u < v ? u : v; s2 += u > v ? u : v; break;
+        default: s0 += u == v ? 0.0 : 1.0; break;   // Hamming
+      }
+    }
+    mean = block_sum(s0, lds); m2 = block_sum(s1, lds); cnt = block_sum(s2, lds);
+  } else if (a.kind == M_VARIANCE || a.kind == M_STDDEV) {
     double s = 0.0;
     for (LongType q = j0 + threadIdx.x; q < j1; q += 256) s += at(q);
     mean = n > 0 ? block_sum(s, lds) / n : 0.0;
@@ -347,6 +372,7 @@ __global__ __launch_bounds__(256) void misc_finish(MiscArgs a, const double* __r
   for (int s = 0; s < a.splits; s++) {
     const double* p = partials + (row * a.splits + s) * 4;
     const double nb = p[0];
+    if (a.kind >= M3_MANHATTAN) { n += nb; mean += p[1]; m2 += p[2]; cnt += p[3]; continue; }
     if (nb > 0.0) {
       const double delta = p[1] - mean, tot = n + nb;
       m2 += p[2] + delta * delta * n * nb / tot;
@@ -358,10 +384,16 @@ __global__ __launch_bounds__(256) void misc_finish(MiscArgs a, const double* __r
   store_any(z, a.zdt, walk<LongType>(a.zOuter, row), misc_result(a, n, mean, m2, cnt));
 }
 void launchReduceMisc(hipStream_t st, MiscReduceKind k, DataType xdt, DataType zdt, const void* x, void* z, const ReducePlan& p,
-                      bool biasCorrected, void* scratch, size_t scratchBytes) {
+                      bool biasCorrected, void* scratch, size_t scratchBytes, const void* y, DataType ydt, const ReducePlan* yPlan) {
   if (p.outerLen == 0) return;
   MiscArgs a;
   a.outer = p.outer; a.inner = p.inner; a.zOuter = p.zOuter;
+  ND4J_REQUIRE((k >= M3_MANHATTAN) == (y != nullptr && yPlan != nullptr), "reduce: second operand mismatch");
+  if (yPlan) {
+    ND4J_REQUIRE(yPlan->outerLen == p.outerLen && yPlan->innerLen == p.innerLen, "reduce3: operands must have equal shapes");
+    a.yOuter = yPlan->outer; a.yInner = yPlan->inner;
+  } else { a.yOuter = p.outer; a.yInner = p.inner; }
+  a.ydt = (int)ydt;
   a.outerLen = p.outerLen; a.innerLen = p.innerLen;
   a.kind = (int)k; a.bias = biasCorrected ? 1 : 0; a.xdt = (int)xdt; a.zdt = (int)zdt;
   // few outputs with long runs: split every run over several blocks (about 2048 blocks in flight)
@@ -374,7 +406,7 @@ void launchReduceMisc(hipStream_t st, MiscReduceKind k, DataType xdt, DataType z
   a.splits = (int)splits;
   a.segLen = (p.innerLen + splits - 1) / splits;
   ND4J_REQUIRE(p.outerLen * splits < (1LL << 31), "reduce: too many outputs");
-  hipLaunchKernelGGL(misc_partial, dim3((unsigned)(p.outerLen * splits)), dim3(256), 0, st, a, x, z, (double*)scratch);
+  hipLaunchKernelGGL(misc_partial, dim3((unsigned)(p.outerLen * splits)), dim3(256), 0, st, a, x, y, z, (double*)scratch);
   if (splits > 1) hipLaunchKernelGGL(misc_finish, dim3((unsigned)((p.outerLen + 255) / 256)), dim3(256), 0, st, a, (const double*)scratch, z);
   HIP_CHECK(hipGetLastError());
 }

@@ -63,6 +63,10 @@ class SummaryStats:
     Variance, StandardDeviation = 0, 1
 
 
+class Reduce3:
+    ManhattanDistance, EuclideanDistance, CosineSimilarity, Dot, CosineDistance, JaccardDistance, SimpleHammingDistance = 0, 1, 2, 3, 5, 6, 7
+
+
 class ReduceLong:
     CountNonZero, CountZero = 0, 1
 
@@ -248,6 +252,16 @@ class Executioner:
         else:
             self.L.execSummaryStatsTad(None, op_num, x.handle, None, z.handle, _dims_array(dims).handle, bool(bias_corrected))
         N.check("execSummaryStats")
+        return z
+
+    def exec_reduce3(self, op_num, x, y, dims=None, keep_dims=False, z=None):
+        if z is None:
+            z = NDArray.empty(_reduced_shape(x.shape, dims, keep_dims), x.dtype)
+        if dims is None or len(dims) == 0:
+            self.L.execReduce3Scalar(None, op_num, x.handle, None, y.handle, z.handle)
+        else:
+            self.L.execReduce3Tad(None, op_num, x.handle, None, y.handle, z.handle, _dims_array(dims).handle)
+        N.check("execReduce3")
         return z
 
     def _reduce_dims_only(self, fn, name, op_num, x, dims, keep_dims, z, zdtype):

@@ -121,6 +121,9 @@ _SIGS = {
     "execTransformBool": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr]),
     "execSummaryStatsScalar": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, ctypes.c_bool]),
     "execSummaryStatsTad": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr, ctypes.c_bool]),
+    "execReduce3": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "execReduce3Scalar": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "execReduce3Tad": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
     "execReduceLong": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
     "execReduceLong2": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
     "execReduceBool": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),

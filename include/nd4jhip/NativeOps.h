@@ -176,6 +176,9 @@ ND4JHIP_EXPORT void execScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDAr
 ND4JHIP_EXPORT void execTransformBool(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z);   /* ref :218 */
 ND4JHIP_EXPORT void execSummaryStatsScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z, bool biasCorrected); /* ref :197 */
 ND4JHIP_EXPORT void execSummaryStatsTad(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z, OpaqueNDArray dimension, bool biasCorrected); /* ref :198-199 */
+ND4JHIP_EXPORT void execReduce3(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray y, OpaqueNDArray z);        /* ref :326 */
+ND4JHIP_EXPORT void execReduce3Scalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray y, OpaqueNDArray z);  /* ref :327 */
+ND4JHIP_EXPORT void execReduce3Tad(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray y, OpaqueNDArray z, OpaqueNDArray dimension); /* ref :328 */
 ND4JHIP_EXPORT void execReduceLong(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z, OpaqueNDArray dimension);  /* ref :211 */
 ND4JHIP_EXPORT void execReduceLong2(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z, OpaqueNDArray dimension); /* ref :349-351 */
 ND4JHIP_EXPORT void execReduceBool(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z, OpaqueNDArray dimension);  /* ref :213 */

@@ -927,6 +927,51 @@ int orc_reduce_count(int kind, const void *x, const int64_t *xsi, void *z, const
   return 0;
 }
 
+/* execReduce3 / execReduce3Scalar / execReduce3Tad   loops/cpu/reduce3.hpp; functors ops/ops.h:117-134,483-541
+ * 0 Manhattan sum|x-y|, 1 Euclidean sqrt(sum (x-y)^2), 2 CosineSimilarity xy / (|x| |y|), 3 Dot, 5 CosineDistance 1 - cos,
+ * 6 JaccardDistance 1 - sum min / sum max, 7 SimpleHamming (count x != y) / n.  Accumulated in double here.  The square root
+ * of the Euclidean distance is what the reference's tests expect (NDArrayTests.cpp:1455-1488); the functor macro of this
+ * snapshot leaves it out. */
+int orc_reduce3(int opNum, const void *x, const int64_t *xsi, const void *y, const int64_t *ysi, void *z, const int64_t *zsi,
+                const int64_t *dims, int ndims) {
+  RedPlan p, py;
+  if (red_plan(xsi, dims, ndims, &p) || red_plan(ysi, dims, ndims, &py)) return 3;
+  if (p.olen != py.olen || p.ilen != py.ilen) return 3;
+  int xdt = orc_dtype(xsi), ydt = orc_dtype(ysi), zdt = orc_dtype(zsi);
+  if (!dt_is_float(zdt)) return 2;
+  if (orc_length(zsi) != p.olen) return 3;
+  if (opNum < 0 || opNum > 7 || opNum == 4) return 1;
+  int64_t zshape[ORC_MAX_RANK], zstride[ORC_MAX_RANK]; int zr = 0;
+  for (int i = 0; i < si_rank(zsi); i++)
+    if (si_shape(zsi)[i] != 1) { zshape[zr] = si_shape(zsi)[i]; zstride[zr++] = si_stride(zsi)[i]; }
+  for (int64_t o = 0; o < p.olen; o++) {
+    int64_t xb = walk(p.orank, p.oshape, p.ostride, o), yb = walk(py.orank, py.oshape, py.ostride, o);
+    double s0 = 0, s1 = 0, s2 = 0;
+    for (int64_t j = 0; j < p.ilen; j++) {
+      double u = ld(x, xdt, xb + walk(p.irank, p.ishape, p.istride, j));
+      double v = ld(y, ydt, yb + walk(py.irank, py.ishape, py.istride, j));
+      switch (opNum) {
+        case 0: s0 += fabs(u - v); break;
+        case 1: s0 += (u - v) * (u - v); break;
+        case 2: case 5: s0 += u * v; s1 += u * u; s2 += v * v; break;
+        case 3: s0 += u * v; break;
+        case 6: s1 += u < v ? u : v; s2 += u > v ? u : v; break;
+        case 7: s0 += u != v; break;
+      }
+    }
+    double r = s0;
+    switch (opNum) {
+      case 1: r = sqrt(s0); break;
+      case 2: r = s0 / (sqrt(s1) * sqrt(s2)); break;
+      case 5: r = 1.0 - s0 / (sqrt(s1) * sqrt(s2)); break;
+      case 6: r = 1.0 - s1 / s2; break;
+      case 7: r = s0 / (double)p.ilen; break;
+    }
+    st(z, zdt, walk(zr, zshape, zstride, o), r);
+  }
+  return 0;
+}
+
 /* execTransformBool: loops/legacy_ops.h:49-51; predicates ops/ops.h:1140-1163,1927-1933; z is a BOOL array */
 int orc_transform_bool(int opNum, const void *x, const int64_t *xsi, void *z, const int64_t *zsi) {
   int xdt = orc_dtype(xsi);

@@ -34,6 +34,7 @@
  *   broadcast tables, rest of tables .. numpy / math routines per function, table numbering per opNum,
  *                                       broadcast vs numpy broadcasting over TADs
  *   reduce same/float ................. NativeOpsTests.cpp:209-238, fp64 bounds; entropies vs scipy.stats
+ *   reduce3 ........................... NDArrayTests.cpp:1455-1488, NDArrayTests2.cpp:1144-1152 (Euclidean), scipy.spatial
  *   summary stats, counts, Any/All,
  *   transform bool .................... numpy var/std (ddof 0/1), count_nonzero, isnan/isinf/isfinite
  *   index reduce / argmax ............. NativeOpsTests.cpp:84-117, LegacyOpsTests.cpp:279-310,
@@ -92,6 +93,8 @@ int orc_transform_same(int opNum, const void *x, const int64_t *xsi, void *z, co
 int orc_transform_bool(int opNum, const void *x, const int64_t *xsi, void *z, const int64_t *zsi);
 int orc_summary_stats(int opNum, const void *x, const int64_t *xsi, void *z, const int64_t *zsi, const int64_t *dims, int ndims,
                       int biasCorrected);
+int orc_reduce3(int opNum, const void *x, const int64_t *xsi, const void *y, const int64_t *ysi, void *z, const int64_t *zsi,
+                const int64_t *dims, int ndims);
 int orc_reduce_count(int kind, const void *x, const int64_t *xsi, void *z, const int64_t *zsi, const int64_t *dims, int ndims);
 int orc_scalar(int opNum, const void *x, const int64_t *xsi, double scalar, void *z, const int64_t *zsi);
 int orc_broadcast(int opNum, const void *x, const int64_t *xsi, const void *y, const int64_t *ysi, void *z,

@@ -59,6 +59,7 @@ def lib():
         L.orc_transform_bool.argtypes = [i32, vp, i64p, vp, i64p]
         L.orc_summary_stats.argtypes = [i32, vp, i64p, vp, i64p, i64p, i32, i32]
         L.orc_reduce_count.argtypes = [i32, vp, i64p, vp, i64p, i64p, i32]
+        L.orc_reduce3.argtypes = [i32, vp, i64p, vp, i64p, vp, i64p, i64p, i32]
         L.orc_scalar.argtypes = [i32, vp, i64p, dbl, vp, i64p]
         L.orc_broadcast.argtypes = [i32, vp, i64p, vp, i64p, vp, i64p, i64p, i32]
         for f in (L.orc_reduce_same, L.orc_reduce_float, L.orc_index_reduce):
@@ -199,6 +200,13 @@ def summary_stats(op, x, z, dims=None, bias_corrected=False):
     x, z = _arr(x), _arr(z)
     d, n = _dims(dims)
     _check(lib().orc_summary_stats(op, _p(x.a), _s(x.si), _p(z.a), _s(z.si), _s(d), n, int(bias_corrected)), "summary_stats")
+    return z.a
+
+
+def reduce3(op, x, y, z, dims=None):
+    x, y, z = _arr(x), _arr(y), _arr(z)
+    d, n = _dims(dims)
+    _check(lib().orc_reduce3(op, _p(x.a), _s(x.si), _p(y.a), _s(y.si), _p(z.a), _s(z.si), _s(d), n), "reduce3")
     return z.a
 
 

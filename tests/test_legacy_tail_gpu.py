@@ -294,3 +294,36 @@ def test_reduce_long_bool_and_transform_bool(ex, oracle):
             want = oracle.transform_bool(op, vv, np.zeros(vv.shape, np.bool_))
             got = ex.exec_transform_bool(op, V).to_numpy()
             assert np.array_equal(got, want), (op, dt)
+
+
+@pytest.mark.parametrize("dtype", [FLOAT32, DOUBLE, BFLOAT16])
+@pytest.mark.parametrize("dims", [[1], [0, 2], None])
+def test_reduce3(ex, oracle, dtype, dims):
+    from deeplearning4j_amd.executioner import Reduce3
+    rng = np.random.default_rng(80)
+    a = np.round(rng.uniform(0.25, 3, (6, 70, 5)) * 4) / 4
+    b = np.round(rng.uniform(0.25, 3, (6, 70, 5)) * 4) / 4
+    oa, da = _pair(oracle, a, dtype)
+    ob, db = _pair(oracle, b, dtype)
+    shape = () if dims is None else tuple(s for i, s in enumerate(a.shape) if i not in dims)
+    for op in (Reduce3.ManhattanDistance, Reduce3.EuclideanDistance, Reduce3.CosineSimilarity, Reduce3.Dot, Reduce3.CosineDistance,
+               Reduce3.JaccardDistance, Reduce3.SimpleHammingDistance):
+        oz = oracle.Arr(np.zeros(shape, oa.a.dtype), oa.dt)
+        oracle.reduce3(op, oa, ob, oz, dims)
+        got = ex.exec_reduce3(op, da, db, dims)
+        rtol, atol = {FLOAT32: (2e-6, 1e-6), DOUBLE: (1e-12, 1e-14), BFLOAT16: (1e-2, 1e-2)}[dtype]
+        assert_close(np.asarray(_got(got, dtype)).reshape(shape), np.asarray(_f(oz)).reshape(shape), rtol, atol, "reduce3 op %d dims %s" % (op, dims))
+
+
+def test_reduce3_reference_vectors_and_views(ex, oracle):
+    from deeplearning4j_amd.executioner import Reduce3
+    x = NDArray.from_numpy(np.array([[1, 2, 3], [4, 5, 6]], np.float32))
+    y = NDArray.from_numpy(np.full((2, 3), 2, np.float32))
+    got = ex.exec_reduce3(Reduce3.EuclideanDistance, x, y, [1]).to_numpy()        # NDArrayTests.cpp:1473-1488
+    assert_close(got, [1.414214, 5.385165], 1e-6, 0, "euclidean rows")
+    rng = np.random.default_rng(81)
+    a = rng.normal(size=(8, 12)).astype(np.float32)
+    b = rng.normal(size=(12, 8)).astype(np.float32)
+    want = oracle.reduce3(Reduce3.Dot, a, b.T, np.zeros(8, np.float32), [1])
+    got = ex.exec_reduce3(Reduce3.Dot, NDArray.from_numpy(a), NDArray.from_numpy(b).permute(1, 0), [1]).to_numpy()
+    assert_close(got, want, 2e-6, 1e-6, "dot against a transposed view")

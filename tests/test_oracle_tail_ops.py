@@ -297,3 +297,27 @@ def test_counts_any_all_and_predicates():
     for op, fn in ((1, np.isinf), (2, np.isnan), (3, np.isfinite), (4, lambda a: ~np.isfinite(a)), (6, lambda a: a > 0), (7, lambda a: a == 0),
                    (8, lambda a: a < 0)):
         np.testing.assert_array_equal(O.transform_bool(op, v, np.zeros(v.shape, np.bool_)), fn(v), err_msg="op %d" % op)
+
+
+def test_reduce3_reference_vectors_and_scipy():
+    import scipy.spatial.distance as D
+    # NDArrayTests.cpp:1473-1488 (applyReduce3EuclideanDistance is an all-pairs call; its diagonal is the pairwise result)
+    x = np.array([[1, 2, 3], [4, 5, 6]], np.float32)
+    y = np.full((2, 3), 2, np.float32)
+    np.testing.assert_allclose(O.reduce3(1, x, y, np.zeros(2, np.float32), [1]), [1.414214, 5.385165], rtol=1e-6)
+    # NDArrayTests2.cpp:1144-1152 reduce3_1
+    np.testing.assert_array_equal(O.reduce3(1, np.array([[1, 2, 3, 4.0]]), np.array([[2, 3, 4, 5.0]]), np.zeros(4), [0]), [1, 1, 1, 1])
+    rng = np.random.default_rng(9)
+    a, b = rng.uniform(0.1, 2, (5, 40)), rng.uniform(0.1, 2, (5, 40))
+    rows = lambda f: np.array([f(a[i], b[i]) for i in range(5)])
+    z = lambda: np.zeros(5)
+    np.testing.assert_allclose(O.reduce3(0, a, b, z(), [1]), rows(D.cityblock), rtol=1e-13)
+    np.testing.assert_allclose(O.reduce3(1, a, b, z(), [1]), rows(D.euclidean), rtol=1e-13)
+    np.testing.assert_allclose(O.reduce3(2, a, b, z(), [1]), 1 - rows(D.cosine), rtol=1e-12)
+    np.testing.assert_allclose(O.reduce3(3, a, b, z(), [1]), (a * b).sum(1), rtol=1e-13)
+    np.testing.assert_allclose(O.reduce3(5, a, b, z(), [1]), rows(D.cosine), rtol=1e-10, atol=1e-15)
+    np.testing.assert_allclose(O.reduce3(6, a, b, z(), [1]), 1 - np.minimum(a, b).sum(1) / np.maximum(a, b).sum(1), rtol=1e-13)
+    c = np.round(a)
+    d = np.round(b)
+    np.testing.assert_allclose(O.reduce3(7, c, d, z(), [1]), rows(lambda u, v: D.hamming(u, v)).astype(np.float64) * 0 + (c != d).mean(1), rtol=1e-15)
+    np.testing.assert_allclose(O.reduce3(3, a, b, np.zeros(())), (a * b).sum(), rtol=1e-13)
