@@ -1082,20 +1082,28 @@ static bool mfmaEligible(const GemmDesc& d, const void* A, const void* B, size_t
 }
 
 // ---- up to four rows of x against row-major W (a decode step's projections) --------------------------------------------------
-// One block of 16 waves per strip of CW output columns and all of K: a lane loads 8 neighbouring columns of one k-row
-// (16 bytes), a wave covers 64/(CW/8) k-rows per instruction, the waves interleave rows, and a lane issues up to eight
-// independent loads before it touches the first -- with so few strips (N/CW blocks) a CU has to keep about 100 KB in
-// flight to stream at its share of the bandwidth.  x sits in LDS.  Partial sums meet through lane shuffles (rows of a wave)
-// and LDS (waves), in a fixed order.  One launch, no partial tiles in global memory.
-template <typename T, int M, int CW>
-__global__ __launch_bounds__(1024) void gemv_strip(GemmArgs g, const T* __restrict__ x, const T* __restrict__ W, T* __restrict__ out) {
-  constexpr int NWAVE = 16, LPR = CW / 8, RPW = 64 / LPR, RB = NWAVE * RPW;
+// One block per strip of CW output columns and all of K: a lane loads 8 neighbouring columns of one k-row (16 bytes), a wave
+// covers 64/(CW/8) k-rows per instruction, the waves interleave rows, and a lane issues up to eight independent loads before
+// it touches the first.  Narrow strips (CW = 8: N/8 blocks) spread the weights over every CU -- one CU streams only at its
+// share of the bandwidth -- and the XCD-aware strip order lets the blocks that share a weight row's cache lines hit the same
+// L2.  x sits in LDS.  Partial sums meet through lane shuffles (rows of a wave) and LDS (waves), in a fixed order.  One
+// launch, no partial tiles in global memory.
+template <typename T, int M, int CW, int NWAVE>
+__global__ __launch_bounds__(NWAVE * 64) void gemv_strip(GemmArgs g, const T* __restrict__ x, const T* __restrict__ W, T* __restrict__ out) {
+  constexpr int LPR = CW / 8, RPW = 64 / LPR, RB = NWAVE * RPW;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   float* red = reinterpret_cast<float*>(smem_raw);                      // [16 waves][M][CW]
   T* xs = reinterpret_cast<T*>(red + NWAVE * M * CW);                    // [M][K]
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, cg = lane % LPR, rk = lane / LPR;
   const LongType K = g.K;
-  const LongType c0 = (LongType)blockIdx.x * CW + cg * 8;
+  // consecutive block ids sit on different XCDs: give every XCD a run of neighbouring strips, so that strips which share
+  // 128-byte lines of a weight row are served by one L2
+  unsigned strip;
+  {
+    const unsigned total = gridDim.x, xcd = blockIdx.x & 7u, idx = blockIdx.x >> 3, per = total >> 3, rem = total & 7u;
+    strip = xcd * per + (xcd < rem ? xcd : rem) + idx;
+  }
+  const LongType c0 = (LongType)strip * CW + cg * 8;
   const T* wp = W + (LongType)(wave * RPW + rk) * g.bRow + c0;
   const LongType step = (LongType)RB * g.bRow;
   LongType k = wave * RPW + rk;
@@ -1105,7 +1113,7 @@ __global__ __launch_bounds__(1024) void gemv_strip(GemmArgs g, const T* __restri
 #pragma unroll
   for (int i = 0; i < 8; i++)
     if (i < first) w[i] = *reinterpret_cast<const u32x4*>(wp + i * step);
-  for (LongType i = t; i < (LongType)M * K; i += 1024) {
+  for (LongType i = t; i < (LongType)M * K; i += NWAVE * 64) {
     const LongType m = i / K, kk = i - m * K;
     xs[i] = x[m * g.aRow + kk];
   }
@@ -1164,20 +1172,17 @@ __global__ __launch_bounds__(1024) void gemv_strip(GemmArgs g, const T* __restri
     float v = 0.f;
 #pragma unroll
     for (int q = 0; q < NWAVE; q++) v += red[(q * M + m) * CW + c];
-    const LongType col = (LongType)blockIdx.x * CW + c;
+    const LongType col = (LongType)strip * CW + c;
     if (g.bias) v += to_float(static_cast<const T*>(g.bias)[col]);
     out[(LongType)m * g.cRow + col] = Conv<T>::from(v);
   }
 }
 template <typename T, int M>
 static void launchGemvStripM(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C) {
-  if (g.N >= 1536 && g.N % 64 == 0) {
-    const size_t lds = (size_t)16 * M * 64 * sizeof(float) + (size_t)M * g.K * sizeof(T);
-    hipLaunchKernelGGL((gemv_strip<T, M, 64>), dim3((unsigned)(g.N / 64)), dim3(1024), lds, s, g, (const T*)A, (const T*)B, (T*)C);
-  } else {
-    const size_t lds = (size_t)16 * M * 32 * sizeof(float) + (size_t)M * g.K * sizeof(T);
-    hipLaunchKernelGGL((gemv_strip<T, M, 32>), dim3((unsigned)(g.N / 32)), dim3(1024), lds, s, g, (const T*)A, (const T*)B, (T*)C);
-  }
+  // strips of 8 columns (one 16-byte piece of every weight row): N/8 blocks keep every CU busy even for N = 768
+  constexpr int CW = 8, NWAVE = 4;
+  const size_t lds = (size_t)NWAVE * M * CW * sizeof(float) + (size_t)M * g.K * sizeof(T);
+  hipLaunchKernelGGL((gemv_strip<T, M, CW, NWAVE>), dim3((unsigned)(g.N / CW)), dim3(NWAVE * 64), lds, s, g, (const T*)A, (const T*)B, (T*)C);
 }
 // whether the strip kernel takes this product: a few dense rows, W row-major with aligned rows, plain C = A B (+ bias)
 template <typename T>
@@ -1186,7 +1191,7 @@ static bool tryGemvStrip(hipStream_t s, const GemmDesc& d, const void* A, const 
   if (d.aCol != 1 || d.bCol != 1 || d.cCol != 1 || d.bRow % 8 != 0) return false;
   if (d.N % 32 != 0 || d.K % 256 != 0 || d.N < 256) return false;
   if ((reinterpret_cast<uintptr_t>(B) & 15) != 0) return false;
-  if ((size_t)16 * d.M * 64 * sizeof(float) + (size_t)d.M * d.K * sizeof(T) > 60 * 1024) return false;
+  if ((size_t)4 * d.M * 8 * sizeof(float) + (size_t)d.M * d.K * sizeof(T) > 60 * 1024) return false;
   GemmArgs g = toArgs(d);
   switch (d.M) {
     case 1: launchGemvStripM<T, 1>(s, g, A, B, C); break;
