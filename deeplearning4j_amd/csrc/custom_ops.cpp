@@ -334,6 +334,24 @@ static std::vector<std::vector<LongType>> sameAsInputShapeFn(Context& c) {
   return {makeShapeInfo(x->dataType(), x->ordering(), shapeOf(x))};
 }
 
+// statistics groups of a standardisation over `axes`: the reduced dims form the inner walk, the others the outer one;
+// dimC (or -1) is the axis gain and bias run along
+static LnGenericPlan lnGenericPlan(const NDArray* x, const NDArray* z, const std::vector<LongType>& axes, int dimC) {
+  const int rank = x->rankOf();
+  LnGenericPlan p;
+  std::vector<bool> red(rank, false);
+  for (auto a : axes) red[a] = true;
+  std::vector<LongType> os, oxs, ozs, is, ixs, izs;
+  for (int d = 0; d < rank; d++) {
+    if (red[d]) { if (d == dimC) { p.channelInInner = 1; p.channelPos = (int)is.size(); } is.push_back(x->sizeAt(d)); ixs.push_back(x->strideAt(d)); izs.push_back(z->strideAt(d)); }
+    else { if (d == dimC) { p.channelInInner = 0; p.channelPos = (int)os.size(); } os.push_back(x->sizeAt(d)); oxs.push_back(x->strideAt(d)); ozs.push_back(z->strideAt(d)); }
+  }
+  p.outerLen = 1; for (auto s : os) p.outerLen *= s;
+  p.innerLen = 1; for (auto s : is) p.innerLen *= s;
+  p.outerX = toDevShape(os, oxs); p.outerZ = toDevShape(os, ozs);
+  p.innerX = toDevShape(is, ixs); p.innerZ = toDevShape(is, izs);
+  return p;
+}
 // ---- layer_norm ------------------------------------------------------------------------------------------------------
 // generic/nn/layer_norm.cpp:35-79: standardize over IArgs axes, then * gain (+ bias) along dim 1 (BArg0 true or
 // absent) or the last dim (BArg0 false); eps 1e-5 inside the sqrt (generic/transforms/standardize.cpp:34-78)
@@ -364,21 +382,9 @@ static void layerNormImpl(Context& c, NDArray* x, NDArray* gain, NDArray* bias, 
     RowPlan p = buildRowPlan(x->shapeInfo(), z->shapeInfo(), rank - 1);
     launchLayerNormRows(stream(), x->dataType(), x->specialBuffer(), gain->specialBuffer(), bias ? bias->specialBuffer() : nullptr, z->specialBuffer(), p, eps);
   } else {
-    ND4J_REQUIRE(gain != nullptr, "STANDARDIZE OP: the stand-alone op is reached through layer_norm in nd4j-hip");
-    ND4J_REQUIRE(gain->strideAt(0) == 1 && (!bias || bias->strideAt(0) == 1), "LAYER_NORM OP: gain/bias must be dense");
-    LnGenericPlan p;
-    std::vector<bool> red(rank, false);
-    for (auto a : axes) red[a] = true;
-    std::vector<LongType> os, oxs, ozs, is, ixs, izs;
-    for (int d = 0; d < rank; d++) {
-      if (red[d]) { if (d == dimC) { p.channelInInner = 1; p.channelPos = (int)is.size(); } is.push_back(x->sizeAt(d)); ixs.push_back(x->strideAt(d)); izs.push_back(z->strideAt(d)); }
-      else { if (d == dimC) { p.channelInInner = 0; p.channelPos = (int)os.size(); } os.push_back(x->sizeAt(d)); oxs.push_back(x->strideAt(d)); ozs.push_back(z->strideAt(d)); }
-    }
-    p.outerLen = 1; for (auto s : os) p.outerLen *= s;
-    p.innerLen = 1; for (auto s : is) p.innerLen *= s;
-    p.outerX = toDevShape(os, oxs); p.outerZ = toDevShape(os, ozs);
-    p.innerX = toDevShape(is, ixs); p.innerZ = toDevShape(is, izs);
-    launchLayerNormGeneric(stream(), x->dataType(), x->specialBuffer(), gain->specialBuffer(), bias ? bias->specialBuffer() : nullptr, z->specialBuffer(), p, eps);
+    ND4J_REQUIRE(!gain || (gain->strideAt(0) == 1 && (!bias || bias->strideAt(0) == 1)), "LAYER_NORM OP: gain/bias must be dense");
+    LnGenericPlan p = lnGenericPlan(x, z, axes, dimC);
+    launchLayerNormGeneric(stream(), x->dataType(), x->specialBuffer(), gain ? gain->specialBuffer() : nullptr, bias ? bias->specialBuffer() : nullptr, z->specialBuffer(), p, eps);
   }
   registerSpecialUse(std::vector<NDArray*>{z}, reads);
 }
@@ -1070,6 +1076,159 @@ static std::vector<std::vector<LongType>> stridedSliceShapeFn(Context& c) {
   return {makeShapeInfo(x->dataType(), 'c', g.outShape)};
 }
 
+// ---- gradient ops ---------------------------------------------------------------------------------------------------------
+// softmax_bp (generic/nn/softmax.cpp:53-95): inputs [input, gradO, softmaxedOut], IArg0 = dim (default last);
+// gradI = softmaxedOut * (gradO - sum_dim(softmaxedOut * gradO)).  The forward input only supplies the rank.
+static void softmaxBpExec(Context& c) {
+  ND4J_REQUIRE(c.width() >= 3, "SOFTMAX_BP OP: input, gradO and the softmax output are required");
+  NDArray* x = c.input(0);
+  NDArray* g = c.input(1);
+  NDArray* sm = c.input(2);
+  NDArray* z = c.output(0);
+  const int rank = x->rankOf();
+  int dim = (int)iArg(c, 0, rank - 1);
+  ND4J_REQUIRE(dim < rank || rank == 0, "SOFTMAX_BP OP: the value of input integer parameter (dimension) must be less than input array rank " + std::to_string(rank) + ", but got dimension = " + std::to_string(dim) + " instead !");
+  if (dim < 0) dim += rank;
+  ND4J_REQUIRE(rank == 0 || dim >= 0, "SOFTMAX_BP OP: dimension out of range");
+  const DataType dt = z->dataType();
+  ND4J_REQUIRE(isFloatType(dt) && g->dataType() == dt && sm->dataType() == dt, "SOFTMAX_BP OP: gradO, the softmax output and gradI must share a floating point type");
+  ND4J_REQUIRE(shapeOf(g) == shapeOf(x) && shapeOf(sm) == shapeOf(x) && shapeOf(z) == shapeOf(x), "SOFTMAX_BP OP: all arrays must have the input's shape");
+  if (x->isEmpty()) return;
+  prepareSpecialUse({z}, {g, sm});
+  if (rank == 0) {
+    fillValue(z, 0.0);   // a single probability of 1: s * (g - s * g) = 0
+  } else {
+    RowPlan pg = buildRowPlan(g->shapeInfo(), z->shapeInfo(), dim);
+    RowPlan ps = buildRowPlan(sm->shapeInfo(), z->shapeInfo(), dim);
+    launchSoftmaxBp(stream(), dt, g->specialBuffer(), sm->specialBuffer(), z->specialBuffer(), pg, ps);
+  }
+  registerSpecialUse({z}, {g, sm});
+}
+
+// standardize (generic/transforms/standardize.cpp:34-78): axes from IArgs or from a second input
+static std::vector<LongType> standardizeAxes(Context& c, int axesInput, const char* opName) {
+  std::vector<LongType> axes;
+  if (axesInput >= 0) axes = hostIndexVector(c.input(axesInput), opName);
+  else axes = c.iArgs;
+  ND4J_REQUIRE(!axes.empty(), "STANDARDIZE OP: axis has to be non-empty");
+  return axes;
+}
+static void standardizeExec(Context& c) {
+  layerNormImpl(c, c.input(0), nullptr, nullptr, c.output(0), standardizeAxes(c, c.width() > 1 ? 1 : -1, "STANDARDIZE OP"), false, "STANDARDIZE OP");
+}
+
+// standardize_bp (standardize.cpp:84-154): inputs [input, eps] or [input, axes, eps].  gain (layer_norm_bp only)
+// multiplies eps along dimC before the gradient is formed.
+static void standardizeBpImpl(NDArray* x, NDArray* eps, NDArray* gain, int dimC, NDArray* z, const std::vector<LongType>& axesIn, const char* opName) {
+  const int rank = x->rankOf();
+  auto axes = normalizeDims(rank, axesIn.data(), (LongType)axesIn.size(), opName);
+  const DataType dt = z->dataType();
+  ND4J_REQUIRE(isFloatType(dt) && x->dataType() == dt && eps->dataType() == dt, std::string(opName) + ": nd4j-hip requires input, eps and output to share a floating point type");
+  ND4J_REQUIRE(shapeOf(eps) == shapeOf(x) && shapeOf(z) == shapeOf(x), std::string(opName) + ": eps and the output must have the input's shape");
+  if (x->isEmpty()) return;
+  LnGenericPlan px = lnGenericPlan(x, z, axes, dimC);
+  LnGenericPlan pe = lnGenericPlan(eps, z, axes, dimC);
+  launchStandardizeBp(stream(), dt, x->specialBuffer(), eps->specialBuffer(), gain ? gain->specialBuffer() : nullptr, z->specialBuffer(), px, pe);
+}
+static void standardizeBpExec(Context& c) {
+  ND4J_REQUIRE(c.width() >= 2, "STANDARDIZE_BP OP: input and eps are required");
+  NDArray* x = c.input(0);
+  NDArray* eps = c.width() == 3 ? c.input(2) : c.input(1);
+  NDArray* z = c.output(0);
+  auto axes = standardizeAxes(c, c.width() == 3 ? 1 : -1, "STANDARDIZE_BP OP");
+  prepareSpecialUse({z}, {x, eps});
+  standardizeBpImpl(x, eps, nullptr, -1, z, axes, "STANDARDIZE_BP OP");
+  registerSpecialUse({z}, {x, eps});
+}
+
+// layer_norm_bp (generic/nn/layer_norm.cpp:85-157): inputs [input, gain, bias?, eps]; outputs [dLdx, dLdg, dLdb?];
+// IArgs = axes, BArg0 = channelsFirst (default true).
+//   dLdb = sum of eps over every dim but the channel one
+//   dLdg = sum of standardize(input) * eps over the same dims (a fused two-operand reduction of a temporary that holds
+//          the standardised input in the array type, as the reference's does)
+//   dLdx = standardize_bp(input, eps * gain)
+static void layerNormBpExec(Context& c) {
+  ND4J_REQUIRE(c.width() >= 3, "LAYER_NORM_BP OP: input, gain and eps arrays are required");
+  NDArray* x = c.input(0);
+  NDArray* gain = c.input(1);
+  NDArray* bias = c.width() == 4 ? c.input(2) : nullptr;
+  NDArray* eps = c.width() == 4 ? c.input(3) : c.input(2);
+  NDArray* dLdx = c.output(0);
+  NDArray* dLdg = c.output(1);
+  NDArray* dLdb = c.width() == 4 ? c.output(2) : nullptr;
+  const int rank = x->rankOf();
+  const bool channelsFirst = bArg(c, 0, true);
+  const int dimC = channelsFirst ? 1 : rank - 1;
+  ND4J_REQUIRE(dimC < rank, "LAYER_NORM_BP OP: input rank too small for the channel axis");
+  ND4J_REQUIRE(gain->rankOf() == 1 && gain->sizeAt(0) == x->sizeAt(dimC),
+               "LAYER_NORM_BP OP: wrong shape of gain array, expected is {" + std::to_string(x->sizeAt(dimC)) + "}, but got " + shapeStr(gain) + " instead !");
+  if (bias) ND4J_REQUIRE(bias->rankOf() == 1 && bias->sizeAt(0) == x->sizeAt(dimC),
+                         "LAYER_NORM_BP OP: wrong shape of bias array, expected is {" + std::to_string(x->sizeAt(dimC)) + "}, but got " + shapeStr(bias) + " instead !");
+  const DataType dt = x->dataType();
+  ND4J_REQUIRE(isFloatType(dt) && gain->dataType() == dt && eps->dataType() == dt && dLdx->dataType() == dt && dLdg->dataType() == dt && (!dLdb || dLdb->dataType() == dt),
+               "LAYER_NORM_BP OP: nd4j-hip requires all arrays to share one floating point type");
+  ND4J_REQUIRE(gain->strideAt(0) == 1, "LAYER_NORM_BP OP: gain must be dense");
+  ND4J_REQUIRE(dLdg->lengthOf() == gain->lengthOf() && (!dLdb || dLdb->lengthOf() == gain->lengthOf()), "LAYER_NORM_BP OP: wrong length of a parameter gradient");
+  ND4J_REQUIRE(!c.iArgs.empty(), "STANDARDIZE OP: axis has to be non-empty");
+  if (x->isEmpty()) return;
+  std::vector<NDArray*> writes = {dLdx, dLdg}, reads = {x, gain, eps};
+  if (dLdb) writes.push_back(dLdb);
+  prepareSpecialUse(writes, reads);
+  auto lc = LaunchContext::defaultContext();
+  std::vector<LongType> others;
+  for (int d = 0; d < rank; d++) if (d != dimC) others.push_back(d);
+  // a rank-1 descriptor of the parameter gradients lines up with the one kept dim
+  if (dLdb) {
+    ReducePlan p = buildReducePlan(eps->shapeInfo(), dLdb->shapeInfo(), others, false);
+    launchReduce(lc->execStream, R_SUM, dt, dt, eps->specialBuffer(), dLdb->specialBuffer(), p, lc->reductionBuffer, LaunchContext::REDUCTION_BYTES);
+  }
+  NDArray standardized;
+  standardized.si = makeShapeInfo(dt, 'c', shapeOf(x));
+  standardized.buf = std::make_shared<DataBuffer>((void*)nullptr, (void*)nullptr, (size_t)x->lengthOf() * sizeOf(dt), dt);
+  standardized.buf->allocateSpecial();
+  {
+    Context sub;
+    layerNormImpl(sub, x, nullptr, nullptr, &standardized, c.iArgs, false, "LAYER_NORM_BP OP");
+  }
+  {
+    ReducePlan p = buildReducePlan(standardized.shapeInfo(), dLdg->shapeInfo(), others, false);
+    ReducePlan pe = buildReducePlan(eps->shapeInfo(), dLdg->shapeInfo(), others, false);
+    launchReduceMisc(lc->execStream, M3_DOT, dt, dt, standardized.specialBuffer(), dLdg->specialBuffer(), p, false, lc->reductionBuffer,
+                     LaunchContext::REDUCTION_BYTES, eps->specialBuffer(), dt, &pe);
+  }
+  standardizeBpImpl(x, eps, gain, dimC, dLdx, c.iArgs, "LAYER_NORM_BP OP");
+  HIP_CHECK(hipStreamSynchronize(stream()));   // the temporary is released on return
+  registerSpecialUse(writes, reads);
+}
+static std::vector<std::vector<LongType>> layerNormBpShapeFn(Context& c) {
+  auto like = [](NDArray* a) { return makeShapeInfo(a->dataType(), a->ordering(), shapeOf(a)); };
+  if (c.width() > 3) return {like(c.input(0)), like(c.input(1)), like(c.input(2))};
+  return {like(c.input(0)), like(c.input(1))};
+}
+
+// matmul_bp (generic/blas/matmul.cpp:239-332): inputs [x, y, eps], outputs [dLdx, dLdy]; the two gradients are matmuls
+// of eps with the other operand under permuted transpose flags.  The scalar-eps branches of the reference (sums of
+// the operands times eps) are not implemented.
+static void matmulBpExec(Context& c) {
+  ND4J_REQUIRE(c.width() >= 3, "MATMUL_BP OP: x, y and eps are required");
+  ND4J_REQUIRE(c.outputs.size() >= 2 && c.outputs[1] != nullptr, "MATMUL_BP OP: two output arrays are required");
+  NDArray* x = c.input(0);
+  NDArray* y = c.input(1);
+  NDArray* eps = c.input(2);
+  ND4J_REQUIRE(eps->rankOf() != 0, "MATMUL_BP OP: a scalar eps is not implemented in nd4j-hip");
+  const LongType transX = iArg(c, 0, 0) ? 1 : 0, transY = iArg(c, 1, 0) ? 1 : 0, transZ = iArg(c, 2, 0) ? 1 : 0;
+  Context dx;
+  dx.inputs = {eps, y}; dx.outputs = {c.output(0)}; dx.tArgs = {tArg(c, 0, 1.0), tArg(c, 1, 0.0)}; dx.iArgs = {transZ, 1 - transY, transX};
+  matmulExec(dx);
+  Context dy;
+  dy.inputs = {x, eps}; dy.outputs = {c.output(1)}; dy.tArgs = dx.tArgs; dy.iArgs = {1 - transX, transZ, transY};
+  matmulExec(dy);
+}
+static std::vector<std::vector<LongType>> matmulBpShapeFn(Context& c) {
+  auto like = [](NDArray* a) { return makeShapeInfo(a->dataType(), a->ordering(), shapeOf(a)); };
+  return {like(c.input(0)), like(c.input(1))};
+}
+
 // ---- registry ---------------------------------------------------------------------------------------------------------------
 static std::map<LongType, OpDescriptor>& byHash() {
   static std::map<LongType, OpDescriptor> m;
@@ -1109,6 +1268,11 @@ static void ensureRegistered() {
     reg("squeeze", 1, 1, false, 0, -2, [](Context& c) { sameDataExec(c, "squeeze"); }, squeezeShapeFn);
     reg("expand_dims", 1, 1, false, 0, -2, [](Context& c) { sameDataExec(c, "ExpandDims"); }, expandDimsShapeFn);
     reg("split", 1, -1, false, 0, 1, splitExec, splitShapeFn);
+    reg("softmax_bp", 3, 1, true, 0, 0, softmaxBpExec, sameAsInputShapeFn);
+    reg("standardize", 1, 1, true, 0, -2, standardizeExec, sameAsInputShapeFn);
+    reg("standardize_bp", 2, 1, false, 0, -2, standardizeBpExec, sameAsInputShapeFn);
+    reg("layer_norm_bp", 3, -1, false, 0, -1, layerNormBpExec, layerNormBpShapeFn);
+    reg("matmul_bp", 3, 2, false, 0, -2, matmulBpExec, matmulBpShapeFn);
     for (const char* alias : {"strided_slice", "stridedslice"}) reg(alias, 1, 1, false, 0, 5, stridedSliceExec, stridedSliceShapeFn);
   });
 }

@@ -111,6 +111,9 @@ struct RowPlan {
 void launchSoftmax(hipStream_t s, DataType dt, const void* x, void* z, const RowPlan& p, bool clampMode);
 void launchLayerNormRows(hipStream_t s, DataType dt, const void* x, const void* gain, const void* bias, void* z,
                          const RowPlan& p, float eps);
+// gradI = softmaxed * (gradO - sum_row(softmaxed * gradO)); pg = row plan (gradO, gradI), ps = (softmaxed, gradI)
+void launchSoftmaxBp(hipStream_t s, DataType dt, const void* gradO, const void* softmaxed, void* gradI, const RowPlan& pg,
+                     const RowPlan& ps);
 // k largest elements of every row (last axis) with their positions; pv / pi are the row plans (x, values) and
 // (x, indices); sorted: descending values, else ascending positions
 void launchTopK(hipStream_t s, DataType xdt, DataType idt, const void* x, void* values, void* indices, const RowPlan& pv,
@@ -124,6 +127,10 @@ struct LnGenericPlan {
 };
 void launchLayerNormGeneric(hipStream_t s, DataType dt, const void* x, const void* gain, const void* bias, void* z,
                             const LnGenericPlan& p, float eps);
+// gradient of standardize over the plan's groups; gain (may be null) scales eps along the channel axis first.
+// px walks (x, z), pe walks eps in its outerX / innerX members.
+void launchStandardizeBp(hipStream_t s, DataType dt, const void* x, const void* eps, const void* gain, void* z,
+                         const LnGenericPlan& px, const LnGenericPlan& pe);
 
 // ---- GEMM ------------------------------------------------------------------------------------------
 struct GemmDesc {

@@ -481,7 +481,8 @@ __global__ __launch_bounds__(256) void layernorm_generic(LnArgs a, const T* __re
   const LongType cOuter = a.channelInInner ? 0 : coordAt(a.outerX, o, a.channelPos);
   for (LongType j = threadIdx.x; j < a.innerLen; j += 256) {
     const LongType c = a.channelInInner ? coordAt(a.innerX, j, a.channelPos) : cOuter;
-    A y = ((A)to_float(x[xb + walk<LongType>(a.innerX, j)]) - mean) / sd * (A)to_float(gain[c]);
+    A y = ((A)to_float(x[xb + walk<LongType>(a.innerX, j)]) - mean) / sd;
+    if (gain) y *= (A)to_float(gain[c]);   // no gain: the stand-alone standardize op
     if (bias) y += (A)to_float(bias[c]);
     z[zb + walk<LongType>(a.innerZ, j)] = Conv<T>::from(y);
   }

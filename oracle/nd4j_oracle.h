@@ -45,6 +45,9 @@
  *                                       DeclarableOpsTests6.cpp:40-215 (tests/golden/strided_slice_vectors.json) and
  *                                       brute force over python ranges; negative steps and reshape order 'f':
  *                                       parity unpinned (numpy semantics only)
+ *   gradient ops (oracle.py, numpy) ... softmax_bp, standardize_bp, layer_norm_bp, matmul_bp: central differences of the
+ *                                       pinned forward restatements (tests/test_oracle_bp_ops.py); the reference's own
+ *                                       tests hold shapes and all-zero cases only (DeclarableOpsTests15.cpp:72-90,397-408,484-512)
  *   xw_plus_b ......................... composition of matmul and the bias row (xw_plus_b.cpp:117-133)
  *   matmul ............................ DeclarableOpsTests14.cpp:601-1260, DeclarableOpsTests19.cpp:52-140
  *   softmax ........................... DeclarableOpsTests1.cpp:2523-2740; inf/nan clamp

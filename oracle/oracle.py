@@ -345,3 +345,66 @@ def strided_slice(x, begin, end, strides, begin_mask=0, ellipsis_mask=0, end_mas
         else:
             idx.append(slice(None if begin_mask & bit else int(begin[i]), None if end_mask & bit else int(end[i]), int(strides[i])))
     return np.ascontiguousarray(np.asarray(x)[tuple(idx)])
+
+
+# ---- gradient ops: numpy restatements of the reference's array-op compositions ------------------------------------------
+# Arrays are float32 or float64 numpy arrays; every intermediate keeps the array dtype, as the reference's
+# temporaries do.  16-bit inputs are widened by the caller and the result rounded once.
+def softmax_bp(grad_o, softmaxed, dim=-1):
+    """softmax_bp (generic/nn/softmax.cpp:53-95): gradI = s * (gradO - sum_dim(s * gradO))."""
+    s = softmaxed
+    summed = np.sum(s * grad_o, axis=dim, keepdims=True, dtype=s.dtype)
+    return s * (grad_o - summed)
+
+
+def standardize(x, axes):
+    """standardize (generic/transforms/standardize.cpp:34-78): (x - mean) / sqrt(population variance + 1e-5)."""
+    axes = tuple(int(a) for a in axes)
+    mean = np.mean(x, axis=axes, keepdims=True, dtype=x.dtype)
+    var = np.var(x.astype(np.float64), axis=axes, keepdims=True).astype(x.dtype)   # Welford in double, stored as T
+    return (x - mean) / np.sqrt(var + x.dtype.type(1e-5))
+
+
+def standardize_bp(x, eps, axes):
+    """standardize_bp (standardize.cpp:84-154) with reduce_mean_bp (gradO / N spread over the group) and
+    reduce_stdev_bp (generic/reduce/reduceStDev.cpp:109-177: gradO * divide_no_nan(x - mean, stdev * N)); the
+    standard deviation carries no epsilon here; NaN results become 0."""
+    axes = tuple(int(a) for a in axes)
+    n = 1
+    for a in axes:
+        n *= x.shape[a]
+    T = x.dtype.type
+    with np.errstate(all="ignore"):
+        mean = np.mean(x, axis=axes, keepdims=True, dtype=x.dtype)
+        stdev = np.std(x.astype(np.float64), axis=axes, keepdims=True).astype(x.dtype)
+        out = eps / stdev
+        dldu_sum = -np.sum(out, axis=axes, keepdims=True, dtype=x.dtype)
+        out = out + dldu_sum / T(n)
+        tmp = (mean - x) * eps / (stdev * stdev)
+        dlds_sum = np.sum(tmp, axis=axes, keepdims=True, dtype=x.dtype)
+        denom = np.broadcast_to(stdev * T(n), x.shape)
+        ratio = np.where(denom == 0, T(0), (x - mean) / np.where(denom == 0, T(1), denom))
+        out = out + ratio * dlds_sum
+    return np.where(np.isnan(out), T(0), out).astype(x.dtype)
+
+
+def layer_norm_bp(x, gain, eps, axes, channels_first=True, with_bias=True):
+    """layer_norm_bp (generic/nn/layer_norm.cpp:85-157): returns (dLdx, dLdg, dLdb or None)."""
+    dim_c = 1 if channels_first else x.ndim - 1
+    others = tuple(d for d in range(x.ndim) if d != dim_c)
+    dldb = np.sum(eps, axis=others, dtype=x.dtype) if with_bias else None
+    dldg = np.sum(standardize(x, axes) * eps, axis=others, dtype=x.dtype)
+    bshape = [1] * x.ndim
+    bshape[dim_c] = x.shape[dim_c]
+    dldx = standardize_bp(x, eps * gain.reshape(bshape), axes)
+    return dldx, dldg, dldb
+
+
+def matmul_bp(x, y, eps, trans_x=False, trans_y=False, trans_z=False, alpha=1.0, beta=0.0):
+    """matmul_bp (generic/blas/matmul.cpp:239-332), non-scalar eps: dLdx = matmul(eps, y; transZ, !transY, transX),
+    dLdy = matmul(x, eps; !transX, transZ, transY); each through the matmul restatement above."""
+    dldx = np.zeros_like(x)
+    dldy = np.zeros_like(y)
+    matmul(eps, y, dldx, bool(trans_z), not trans_y, bool(trans_x), alpha, beta)
+    matmul(x, eps, dldy, not trans_x, bool(trans_z), bool(trans_y), alpha, beta)
+    return dldx, dldy
