@@ -16,6 +16,8 @@
 //                path for small, odd-shaped or oddly strided problems.
 #include <cstdlib>
 
+#include <mutex>
+
 #include "device.h"
 #include <type_traits>
 
@@ -985,6 +987,80 @@ __global__ __launch_bounds__(256) void gemv_rowdot(const T* __restrict__ W, Long
     y[n * ys] = Conv<T>::from(v);
   }
 }
+// The same product for rows that fit a wave's registers (K <= NL * 64 * V): a wave owns OPW outputs and issues every
+// load of W and x before the first use, so one trip to memory covers the whole row; a decode step's projections
+// against k-contiguous weights run at the cost of a streaming read.
+template <typename T, int OPW, int NL, bool HAS_BIAS>
+__global__ __launch_bounds__(256) void gemv_rowdot_pre(const T* __restrict__ W, LongType ldw, const T* __restrict__ x, T* __restrict__ y, LongType ys,
+                                                       LongType N, LongType K, const T* __restrict__ bias) {
+  constexpr int V = 16 / sizeof(T);
+  using Raw = typename RawIO<T>::raw;
+  const int lane = threadIdx.x & 63;
+  const LongType n0 = ((LongType)blockIdx.x * 4 + (threadIdx.x >> 6)) * OPW;
+  if (n0 >= N) return;
+  const int kw = (int)(K / V);
+  // Every load is unconditional -- lanes past the end of the row re-read its last word and their x bits are masked
+  // to zero -- so that all of them are issued back to back rather than one predicated region (and one wait) per pass.
+  raw_u32x4 wr[OPW][NL], xr[NL];
+  const T* wrow[OPW];
+#pragma unroll
+  for (int o = 0; o < OPW; o++) wrow[o] = W + (n0 + o < N ? n0 + o : N - 1) * ldw;
+#pragma unroll
+  for (int i = 0; i < NL; i++) {
+    const int kk = lane + 64 * i, kc = kk < kw ? kk : kw - 1;
+#pragma unroll
+    for (int o = 0; o < OPW; o++) wr[o][i] = reinterpret_cast<const raw_u32x4*>(wrow[o])[kc];
+    xr[i] = reinterpret_cast<const raw_u32x4*>(x)[kc];
+  }
+  T bq[OPW];
+  if (HAS_BIAS) {
+#pragma unroll
+    for (int o = 0; o < OPW; o++) bq[o] = bias[n0 + o < N ? n0 + o : N - 1];
+  }
+  // the bias enters lane 0's partial sum ahead of the wave reduction: a use every lane depends on, so its load stays
+  // up here with the others instead of sinking into the one-lane store at the end
+  float acc[OPW];
+#pragma unroll
+  for (int o = 0; o < OPW; o++) acc[o] = HAS_BIAS && lane == 0 ? to_float(bq[o]) : 0.f;
+#pragma unroll
+  for (int i = 0; i < NL; i++) {
+    const unsigned keep = lane + 64 * i < kw ? 0xffffffffu : 0u;
+    const raw_u32x4 xm = xr[i] & keep;
+    float xf[V];
+    RawIO<T>::unpack(__builtin_bit_cast(Raw, xm), xf);
+#pragma unroll
+    for (int o = 0; o < OPW; o++) {
+      float wf[V];
+      RawIO<T>::unpack(__builtin_bit_cast(Raw, wr[o][i]), wf);
+#pragma unroll
+      for (int e = 0; e < V; e++) acc[o] = fmaf(wf[e], xf[e], acc[o]);
+    }
+  }
+#pragma unroll
+  for (int o = 0; o < OPW; o++) {
+    const float v = wave_allreduce<SumOp>(acc[o]);
+    if (lane == 0 && n0 + o < N) y[(n0 + o) * ys] = Conv<T>::from(v);
+  }
+}
+template <typename T>
+static bool tryGemvRowdotPre(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
+  constexpr int V = 16 / sizeof(T);
+  if (d.aCol != 1 || d.alpha != 1.f || d.beta != 0.f || d.K % V != 0 || d.bCol % V != 0) return false;
+  if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) return false;
+  const LongType passes = (d.K / V + 63) / 64;
+#define ROWDOT_B(OPW, NL, HB) hipLaunchKernelGGL((gemv_rowdot_pre<T, OPW, NL, HB>), dim3((unsigned)(((d.N + OPW - 1) / OPW + 3) / 4)), dim3(256), 0, s, \
+                                                 (const T*)B, d.bCol, (const T*)A, (T*)C, d.cCol, d.N, d.K, (const T*)d.bias)
+#define ROWDOT(OPW, NL) do { if (d.bias) ROWDOT_B(OPW, NL, true); else ROWDOT_B(OPW, NL, false); } while (0)
+  if (passes <= 2) ROWDOT(2, 2);
+  else if (passes <= 4) ROWDOT(2, 4);
+  else if (passes <= 6) ROWDOT(2, 6);
+  else if (passes <= 8) ROWDOT(2, 8);
+  else if (passes <= 12) ROWDOT(1, 12);
+  else return false;
+#undef ROWDOT
+#undef ROWDOT_B
+  return true;
+}
 // y[n] = alpha * sum_k x[k] * W[k][n]: W rows contiguous in n.  A thread owns V consecutive outputs of one k-slice;
 // slices are combined through LDS (block = 64 column groups x 4 k-slices).
 template <typename T>
@@ -1034,6 +1110,7 @@ static bool tryGemv(hipStream_t s, const GemmDesc& d, const void* A, const void*
   constexpr int V = 16 / sizeof(T);
   if (d.M == 1 && d.N > 1) {
     // y[n] = sum_k a[k] * op(B)[k][n]
+    if (d.bRow == 1 && tryGemvRowdotPre<T>(s, d, A, B, C)) return true;
     if (d.bRow == 1) { hipLaunchKernelGGL((gemv_rowdot<T>), dim3((unsigned)((d.N + 3) / 4)), dim3(256), 0, s, (const T*)B, d.bCol, (const T*)A, d.aCol, (T*)C, d.cCol, d.N, d.K, d.alpha, d.beta, (const T*)d.bias); return true; }
     if (d.bCol == 1) { hipLaunchKernelGGL((gemv_colsum<T>), dim3((unsigned)((d.N + 64 * V - 1) / (64 * V))), dim3(256), 0, s, (const T*)B, d.bRow, (const T*)A, d.aCol, (T*)C, d.cCol, d.N, d.K, d.alpha, d.beta, (const T*)d.bias); return true; }
   }
@@ -1202,6 +1279,91 @@ static bool tryGemvStrip(hipStream_t s, const GemmDesc& d, const void* A, const 
   return true;
 }
 
+// ---- up to 32 rows of x against k-contiguous weights (a batched decode step's projections) -----------------------------
+// C[m][n] = sum_k x[m][k] * Wt[n][k] (+ bias[n]).  A block owns 32 output columns and all of K, in chunks of up to 768 k:
+// every thread issues the chunk's loads at once (whole 128-byte lines: 8 lanes per row), parks them in LDS in the
+// [k-group][row] slot layout, and the four waves share the chunk's MFMA k-steps; the next chunk's loads are in flight
+// while the current one is multiplied.  The waves' 32x32 partial tiles are added up through LDS -- one launch, where the
+// split-K tile kernel needs a second one to add its partial tiles.
+// Accumulator layout: lane (m = lane % 32, h = lane / 32), register r holds column 8 * (r / 4) + 4 * h + r % 4.
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_skinny32(GemmArgs g, const T* __restrict__ X, const T* __restrict__ Wt, T* __restrict__ C) {
+  constexpr int CT = 12;                               // 64-k tiles per chunk
+  constexpr int GROUP = 33;                            // slots per k-group (32 rows + 1: conflict-free column reads)
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  u32x4* sW = reinterpret_cast<u32x4*>(smem_raw);      // [CT * 8 k-groups][GROUP]
+  u32x4* sX = sW + CT * 8 * GROUP;
+  float* red = reinterpret_cast<float*>(sX + CT * 8 * GROUP);   // [4 waves][16 registers][64 lanes]
+  const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int lrow = t >> 3, lkg = t & 7;                // this thread's (row, k-group) inside every 64-k tile
+  const LongType n0 = (LongType)blockIdx.x * 32;
+  const T* wp = Wt + (n0 + lrow) * g.bCol + lkg * 8;
+  const T* xp = X + (LongType)(lrow < g.M ? lrow : g.M - 1) * g.aRow + lkg * 8;
+  const int tiles = (int)(g.K / 64);
+  u32x4 wr[CT], xr[CT];
+  auto load = [&](int tile0) {
+    const int n = tiles - tile0 < CT ? tiles - tile0 : CT;
+#pragma unroll
+    for (int j = 0; j < CT; j++) {
+      const int jc = j < n ? j : n - 1;                // unconditional loads; a repeated tile is never multiplied
+      wr[j] = *reinterpret_cast<const u32x4*>(wp + (LongType)(tile0 + jc) * 64);
+      xr[j] = *reinterpret_cast<const u32x4*>(xp + (LongType)(tile0 + jc) * 64);
+    }
+  };
+  f32x16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[r] = 0.f;
+  const int mrow = lane & 31, h = lane >> 5;
+  load(0);
+  for (int tile0 = 0; tile0 < tiles; tile0 += CT) {
+    const int n = tiles - tile0 < CT ? tiles - tile0 : CT;
+#pragma unroll
+    for (int j = 0; j < CT; j++) {
+      sW[(j * 8 + lkg) * GROUP + lrow] = wr[j];
+      sX[(j * 8 + lkg) * GROUP + lrow] = xr[j];
+    }
+    __syncthreads();
+    if (tile0 + CT < tiles) load(tile0 + CT);
+    for (int s = wave; s < n * 4; s += 4)
+      acc = Mfma16<T>::mma(sW[(2 * s + h) * GROUP + mrow], sX[(2 * s + h) * GROUP + mrow], acc);
+    __syncthreads();
+  }
+#pragma unroll
+  for (int r = 0; r < 16; r++) red[(wave * 16 + r) * 64 + lane] = acc[r];
+  __syncthreads();
+  const int rq = wave;                                 // registers 4 * rq .. + 3: four consecutive columns
+  const LongType n = n0 + 8 * rq + 4 * h;
+  float v[4];
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; w++) sum += red[(w * 16 + 4 * rq + e) * 64 + lane];
+    if (g.bias) sum += to_float(reinterpret_cast<const T*>(g.bias)[n + e]);
+    v[e] = sum;
+  }
+  if (mrow < g.M) {
+    u32x2 o;
+    o[0] = (unsigned)Conv<T>::from(v[0]).bits | ((unsigned)Conv<T>::from(v[1]).bits << 16);
+    o[1] = (unsigned)Conv<T>::from(v[2]).bits | ((unsigned)Conv<T>::from(v[3]).bits << 16);
+    *reinterpret_cast<u32x2*>(C + (LongType)mrow * g.cRow + n) = o;
+  }
+}
+template <typename T>
+static bool tryGemmSkinny(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
+  if (d.M < 5 || d.M > 32 || d.batch != 1 || d.alpha != 1.f || d.beta != 0.f) return false;
+  if (d.aCol != 1 || d.bRow != 1 || d.cCol != 1) return false;                       // x and Wt k-contiguous, C row-major
+  // longer K runs chunk after chunk in one block and measured slower than split-K over many blocks (14 vs 10 us at K = 3072)
+  if (d.N % 32 != 0 || d.K % 64 != 0 || d.K > 1024 || d.aRow % 8 != 0 || d.bCol % 8 != 0 || d.cRow % 4 != 0) return false;
+  if (((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) != 0 || (reinterpret_cast<uintptr_t>(C) & 7) != 0) return false;
+  constexpr size_t LDS = (size_t)2 * 12 * 8 * 33 * 16 + (size_t)4 * 16 * 64 * sizeof(float);
+  static std::once_flag once;
+  std::call_once(once, [] { HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny32<T>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS)); });
+  GemmArgs g = toArgs(d);
+  hipLaunchKernelGGL((gemm_skinny32<T>), dim3((unsigned)(d.N / 32)), dim3(256), LDS, s, g, (const T*)A, (const T*)B, (T*)C);
+  return true;
+}
+
 template <typename T>
 static void dispatch16(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
   bool aKC = false, bKC = false;
@@ -1209,6 +1371,7 @@ static void dispatch16(hipStream_t s, const GemmDesc& d, const void* A, const vo
   // x[1, K] times row-major W[K, N]: the split-K tile kernel streams W with far more loads in flight than the
   // column-sum GEMV (the unused 31 rows of the MFMA tile cost nothing here)
   if (tryGemvStrip<T>(s, d, A, B, C)) return;
+  if (tryGemmSkinny<T>(s, d, A, B, C)) return;
   const bool rowTimesRowMajor = d.M == 1 && eligible && aKC && !bKC && d.batch == 1;
   if (!rowTimesRowMajor && tryGemv<T>(s, d, A, B, C)) return;
   if (eligible) {

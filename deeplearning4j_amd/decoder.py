@@ -6,7 +6,9 @@ one reference op executed through `execCustomOp2` or a legacy `exec*` entry poin
 embeddings), broadcastable `add`, `layer_norm`, `xw_plus_b` (the linear layers), transform-strict GELU (opNum 53),
 transform-any Assign (the write into the key/value cache), `dot_product_attention_v2`, pairwise Add (residuals),
 `matmul` (tied output embedding), `argmax`.  Nothing is fused on the Python side and no array leaves the device
-between ops.
+between ops.  The linear layers' weights are uploaded k-contiguous ([out, in]) and `xw_plus_b` is called with its
+weight-transpose flag (IArg 1, generic/nn/xw_plus_b.cpp:38,99-104): a single token's projection then reads whole
+weight rows, which streams several times faster than column strips of an [in, out] matrix.
 
 Memory layout (all activations token-major, so the head split needs no copy):
   x, attention output ... [B, T, d_model]
@@ -60,7 +62,8 @@ class Decoder:
         up = lambda a: self._resident(NDArray.from_numpy(a, dtype))
         self.wte, self.wpe = up(weights["wte"]), up(weights["wpe"])
         self.lnf_g, self.lnf_b = up(weights["lnf_g"]), up(weights["lnf_b"])
-        self.layers = [{k: up(v) for k, v in lw.items()} for lw in weights["layers"]]
+        linear = ("w_qkv", "w_o", "w_fc", "w_proj")   # stored [in, out] in `weights`, kept [out, in] on the device
+        self.layers = [{k: up(np.ascontiguousarray(v.T) if k in linear else v) for k, v in lw.items()} for lw in weights["layers"]]
         d = cfg.d_model
         self.kcache = [NDArray.empty((batch, cfg.max_len, d), dtype) for _ in range(cfg.n_layer)]
         self.vcache = [NDArray.empty((batch, cfg.max_len, d), dtype) for _ in range(cfg.n_layer)]
@@ -140,7 +143,7 @@ class Decoder:
         for li, w in enumerate(self.layers):
             kc, vc = self.kcache[li], self.vcache[li]
             ops.append(self._custom("layer_norm", [x2, w["ln1_g"], w["ln1_b"]], [ln2], i_args=[1], b_args=[False]))
-            ops.append(self._custom("xw_plus_b", [ln2, w["w_qkv"], w["b_qkv"]], [qkv2]))
+            ops.append(self._custom("xw_plus_b", [ln2, w["w_qkv"], w["b_qkv"]], [qkv2], i_args=[0, 1]))
             # append this chunk's keys / values to the cache
             ops.append(self._assign(knew, kc.view((B, T, d), (M * d, d, 1), past * d)))
             ops.append(self._assign(vnew, vc.view((B, T, d), (M * d, d, 1), past * d)))
@@ -148,12 +151,12 @@ class Decoder:
             v4 = vc.view((B, H, total, Dh), (M * d, Dh, d, 1), 0)
             # a chunk that starts at position 0 attends causally; a single new token sees the whole cache
             ops.append(self._custom("dot_product_attention_v2", [q4, v4, k4], [o4], t_args=[scale, 0.0], b_args=[past == 0 and T > 1, False]))
-            ops.append(self._custom("xw_plus_b", [att2, w["w_o"], w["b_o"]], [proj2]))
+            ops.append(self._custom("xw_plus_b", [att2, w["w_o"], w["b_o"]], [proj2], i_args=[0, 1]))
             ops.append(self._pairwise_add(x2, proj2, x2))
             ops.append(self._custom("layer_norm", [x2, w["ln2_g"], w["ln2_b"]], [ln2], i_args=[1], b_args=[False]))
-            ops.append(self._custom("xw_plus_b", [ln2, w["w_fc"], w["b_fc"]], [h2]))
+            ops.append(self._custom("xw_plus_b", [ln2, w["w_fc"], w["b_fc"]], [h2], i_args=[0, 1]))
             ops.append(self._gelu(h2, g2))
-            ops.append(self._custom("xw_plus_b", [g2, w["w_proj"], w["b_proj"]], [proj2]))
+            ops.append(self._custom("xw_plus_b", [g2, w["w_proj"], w["b_proj"]], [proj2], i_args=[0, 1]))
             ops.append(self._pairwise_add(x2, proj2, x2))
         # final layer norm on the last position only, tied output projection, greedy pick
         xlast = a["x"].view((B, d), (T * d, 1), (T - 1) * d)

@@ -1,7 +1,7 @@
 """CPU composition of the GPT-2-shaped decode step out of the oracle's ops -- test infrastructure only.
 
-Mirrors deeplearning4j_amd/decoder.py op for op (gather, add, layer_norm, xw_plus_b = mmul followed by the bias row
-as in generic/nn/xw_plus_b.cpp:117-133, GELU opNum 53, dot_product_attention_v2, argmax), each executed by the CPU
+Mirrors deeplearning4j_amd/decoder.py op for op (gather, add, layer_norm, xw_plus_b = mmul against the transposed
+[out, in] weights followed by the bias row as in generic/nn/xw_plus_b.cpp:99-133, GELU opNum 53, dot_product_attention_v2, argmax), each executed by the CPU
 restatement in nd4j_oracle.c, so that greedy token ids
 and logits of the HIP path can be compared on the same seeded weights.  Arrays are numpy: float32, or uint16 bit
 patterns for bf16.
@@ -18,7 +18,9 @@ class OracleDecoder:
         self.cfg, self.dt, self.B = cfg, dtype, batch
         conv = (lambda a: O.f32_to_bf16(a)) if dtype == O.BFLOAT16 else (lambda a: np.ascontiguousarray(a, dtype=np.float32))
         self.w = {k: conv(v) for k, v in weights.items() if k != "layers"}
-        self.layers = [{k: conv(v) for k, v in lw.items()} for lw in weights["layers"]]
+        # the linear layers' weights are kept [out, in] and multiplied with the transpose flag, as the device harness does
+        linear = ("w_qkv", "w_o", "w_fc", "w_proj")
+        self.layers = [{k: conv(np.ascontiguousarray(v.T) if k in linear else v) for k, v in lw.items()} for lw in weights["layers"]]
         self.np_dt = np.uint16 if dtype == O.BFLOAT16 else np.float32
         d = cfg.d_model
         self.kc = [np.zeros((batch, cfg.max_len, d), self.np_dt) for _ in range(cfg.n_layer)]
@@ -65,7 +67,7 @@ class OracleDecoder:
         scale = 1.0 / math.sqrt(Dh)
         for li, w in enumerate(self.layers):
             ln = self._ln(x, w["ln1_g"], w["ln1_b"])
-            qkv = self._bias(self._matmul(ln, w["w_qkv"]), w["b_qkv"]).reshape(B, T, 3, H, Dh)
+            qkv = self._bias(self._matmul(ln, w["w_qkv"], trans_y=True), w["b_qkv"]).reshape(B, T, 3, H, Dh)
             self.kc[li][:, past:total] = qkv[:, :, 1].reshape(B, T, d)
             self.vc[li][:, past:total] = qkv[:, :, 2].reshape(B, T, d)
             att = self._empty(B, T, H, Dh)
@@ -75,13 +77,13 @@ class OracleDecoder:
                 v3 = self.vc[li][b, :total].reshape(total, H, Dh).transpose(1, 0, 2)
                 o3 = att[b].transpose(1, 0, 2)
                 O.attention_v2(self._a(q3), self._a(v3), self._a(k3), self._a(o3), scale=scale, causal=(past == 0 and T > 1))
-            proj = self._bias(self._matmul(att.reshape(B * T, d), w["w_o"]), w["b_o"])
+            proj = self._bias(self._matmul(att.reshape(B * T, d), w["w_o"], trans_y=True), w["b_o"])
             x = self._add(x, proj)
             ln = self._ln(x, w["ln2_g"], w["ln2_b"])
-            h = self._bias(self._matmul(ln, w["w_fc"]), w["b_fc"])
+            h = self._bias(self._matmul(ln, w["w_fc"], trans_y=True), w["b_fc"])
             g = self._empty(*h.shape)
             O.transform_strict(53, self._a(h), self._a(g))
-            proj = self._bias(self._matmul(g, w["w_proj"]), w["b_proj"])
+            proj = self._bias(self._matmul(g, w["w_proj"], trans_y=True), w["b_proj"])
             x = self._add(x, proj)
         last = np.ascontiguousarray(x.reshape(B, T, d)[:, T - 1])
         last = self._ln(last, self.w["lnf_g"], self.w["lnf_b"])

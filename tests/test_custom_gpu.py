@@ -236,6 +236,55 @@ def test_few_rows_times_row_major_weights(ex, oracle, dtype, M, K, N):
     assert np.array_equal(zv.to_numpy(), zb.to_numpy())
 
 
+@pytest.mark.parametrize("dtype", [BFLOAT16, HALF, FLOAT32])
+@pytest.mark.parametrize("K,N", [(768, 2304), (768, 768), (3072, 768), (768, 3072), (768, 50257), (64, 5), (1024, 33), (8192, 7), (200, 64)])
+def test_row_times_k_contiguous_weights(ex, oracle, dtype, K, N):
+    """One row of x against [out, in] weights with the transpose flag (a decode step's projection and the tied output
+    embedding): rows up to 12 wave passes long are held in registers, longer ones take the looping kernel."""
+    rng = np.random.default_rng(K + N)
+    x = rng.normal(0, 1, (1, K))
+    wt = rng.normal(0, 1 / math.sqrt(K), (N, K))
+    b = rng.normal(0, 1, (N,))
+    ox, dx = _pair(oracle, x, dtype)
+    ow, dw = _pair(oracle, wt, dtype)
+    ob, db = _pair(oracle, b, dtype)
+    oz = _ozeros(oracle, (1, N), dtype)
+    oracle.matmul(ox, ow, oz, trans_y=True, accumulate=1)
+    tol = 1e-4 if dtype == FLOAT32 else 1e-2
+    z = ex.exec_custom("matmul", [dx, dw], i_args=[0, 1])[0]
+    assert_close(z.to_float(), _f(oz), tol, tol, "row x W^T")
+    oracle.add_row_vector(oz, ob, oz)
+    zb = ex.exec_custom("xw_plus_b", [dx, dw, db], i_args=[0, 1])[0]
+    assert_close(zb.to_float(), _f(oz), tol, tol, "row x W^T + bias")
+
+
+@pytest.mark.parametrize("dtype", [BFLOAT16, HALF])
+@pytest.mark.parametrize("M", [5, 16, 31, 32])
+@pytest.mark.parametrize("K,N", [(768, 2304), (768, 768), (3072, 768), (768, 3072), (256, 32), (1024, 64), (4096, 96), (8192, 64)])
+def test_up_to_32_rows_times_k_contiguous_weights(ex, oracle, dtype, M, K, N):
+    """The batched decode-step shape: 5..32 rows of x against [out, in] weights with the transpose flag run as one
+    launch (waves split K inside a block); with and without the bias row, and from a strided x view."""
+    rng = np.random.default_rng(M + K + N)
+    x = rng.normal(0, 1, (M, K))
+    wt = rng.normal(0, 1 / math.sqrt(K), (N, K))
+    b = rng.normal(0, 1, (N,))
+    ox, dx = _pair(oracle, x, dtype)
+    ow, dw = _pair(oracle, wt, dtype)
+    ob, db = _pair(oracle, b, dtype)
+    oz = _ozeros(oracle, (M, N), dtype)
+    oracle.matmul(ox, ow, oz, trans_y=True, accumulate=1)
+    z = ex.exec_custom("matmul", [dx, dw], i_args=[0, 1])[0]
+    assert_close(z.to_float(), _f(oz), 1e-2, 1e-2, "rows x W^T")
+    oracle.add_row_vector(oz, ob, oz)
+    zb = ex.exec_custom("xw_plus_b", [dx, dw, db], i_args=[0, 1])[0]
+    assert_close(zb.to_float(), _f(oz), 1e-2, 1e-2, "rows x W^T + bias")
+    wide = np.zeros((M, 2 * K), np.asarray(ox.a).dtype)
+    wide[:, :K] = np.asarray(ox.a)
+    xv = NDArray.from_numpy(wide, dtype).view((M, K), (2 * K, 1), 0)
+    zv = ex.exec_custom("xw_plus_b", [xv, dw, db], outputs=[NDArray.empty((M, N), dtype)], i_args=[0, 1])[0]
+    assert np.array_equal(zv.to_numpy(), zb.to_numpy())
+
+
 def test_xw_plus_b_errors(ex):
     x = NDArray.from_numpy(np.ones((4, 8), np.float32))
     w = NDArray.from_numpy(np.ones((9, 5), np.float32))
