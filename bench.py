@@ -31,7 +31,7 @@ MFMA_PEAK = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}   # dense TFLOP/s
 # `--pmc WRITE_SIZE` (separate runs of this script) and scaled by what the same counters read for the plain copy
 # kernel; the summary of those runs sits under profiles/.  Static figures: they are not re-measured here.
 TRAFFIC_MB = {
-    "mmul bf16 4096": 235.2, "mmul f16 4096": 235.2, "mmul f32 4096^3": 847.8, "mmul f32 4096^3 transposeB": 848.1,
+    "mmul bf16 4096": 235.2, "mmul f16 4096": 235.2, "mmul f32 4096^3": 847.8, "mmul f32 4096^3 transposeB": 851.7,
     "mmul f32 1024": 29.4, "mmul f16 1024": 14.8, "mmul bf16 1024": 14.8,
     "copy fp32": 268.4, "pairwise_add fp32": 402.6, "transform_tanh fp32": 268.4, "reduce_sum": 134.6, "argmax dim1": 134.6,
     "layer_norm fp32": 100.8, "gelu fp32": 100.7, "softmax fp32": 1610.6, "layer_norm bf16": 50.4, "gelu bf16": 50.4,
@@ -86,6 +86,8 @@ def main():
     ap.add_argument("--skip-ops", action="store_true", help="leave out the per-op lines of BASELINE configs 1-4")
     ap.add_argument("--skip-cpu", action="store_true", help="leave out the cpu_baseline leg")
     ap.add_argument("--skip-decode", action="store_true", help="leave out the GPT-2-shaped decode (tens of thousands of launches)")
+    ap.add_argument("--no-graphs", action="store_true",
+                    help="time the decode op by op only (for runs under rocprofv3: its kernel tracing aborts the queue on graph replays)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend is built and measured on one GPU; --gpus %d is not supported (no collectives are part of the op path)" % args.gpus)
@@ -120,6 +122,7 @@ def main():
 
     # ---- cpu baseline: the oracle's usualGemm restatement on a bounded sample ------------------------------------
     if not args.skip_cpu:
+        print("[bench] cpu baseline leg (about 15 s)", file=sys.stderr, flush=True)
         from oracle import oracle as O
         ab, bb = f32_to_bf16_bits(a), f32_to_bf16_bits(b)
         rows = 64
@@ -142,6 +145,7 @@ def main():
     # ---- the other BASELINE configs ------------------------------------------------------------------------------------
     ops = []
     if not args.skip_ops:
+        print("[bench] per-op leg", file=sys.stderr, flush=True)
         del A, B, Z
         # config 1: legacy chain, fp32 [8192, 4096]
         rng = np.random.default_rng(1001)
@@ -236,6 +240,7 @@ def main():
             del Q, K_, V, O_
         result["ops"] = ops
     if not args.skip_decode:
+        print("[bench] decode leg", file=sys.stderr, flush=True)
         ops = result.setdefault("ops", [])
         # config 5: GPT-2-small-shaped greedy decode, bf16, prefill 512 then 128 steps with a key/value cache
         from deeplearning4j_amd.decoder import Decoder, DecoderConfig, init_weights
@@ -244,6 +249,7 @@ def main():
         n_param_bytes = 2 * (cfg.n_layer * (cfg.d_model * 3 * cfg.d_model + cfg.d_model * cfg.d_model + 2 * cfg.d_model * cfg.d_ff) + cfg.vocab * cfg.d_model)
         prefill, n_new = 512, 128
         for batch in (1, 32):
+            print("[bench] decode batch %d" % batch, file=sys.stderr, flush=True)
             ids = np.random.default_rng(5005).integers(0, cfg.vocab, (batch, prefill))
             dec = Decoder(cfg, weights, BFLOAT16, batch=batch, executioner=ex)
             dec.generate(ids[:, :prefill], 4)      # builds and warms the prefill program and the first decode programs
@@ -262,8 +268,8 @@ def main():
             prefill_s = t1 - t0
             # the same steps replayed as captured HIP graphs (one per cache length): the first pass records them, the timed
             # passes replay; every kernel of the step still runs, only the per-op launch path on the host is gone
-            dec.use_graphs = True
-            for _ in range(3):
+            dec.use_graphs = not args.no_graphs
+            for _ in range(3 if dec.use_graphs else 0):
                 dec.reset()
                 dec.forward(ids)
                 L.streamSynchronize(None)
@@ -272,10 +278,11 @@ def main():
                     dec.forward(None)
                 L.streamSynchronize(None)
                 t2 = time.perf_counter()
-            step_ms = (t2 - t1) * 1e3 / (n_new - 1)
+            step_ms = (t2 - t1) * 1e3 / (n_new - 1)   # the op-by-op figure when graphs are off
             dec.close()
             kv_bytes = cfg.n_layer * 2 * (prefill + n_new / 2) * cfg.d_model * 2 * batch
-            ops.append({"op": "gpt2-small decode bf16 batch %d (prefill %d, %d greedy steps, KV cache, steps replayed as HIP graphs)" % (batch, prefill, n_new),
+            how = "steps replayed as HIP graphs" if dec.use_graphs else "op by op"
+            ops.append({"op": "gpt2-small decode bf16 batch %d (prefill %d, %d greedy steps, KV cache, %s)" % (batch, prefill, n_new, how),
                         "ms": round(step_ms, 4), "wall_ms": round(step_ms, 4), "tokens_per_s": round(batch * 1e3 / step_ms, 1),
                         "op_by_op_ms": round(eager_ms, 4), "op_by_op_tokens_per_s": round(batch * 1e3 / eager_ms, 1),
                         "prefill_ms": round(prefill_s * 1e3, 3), "prefill_tokens_per_s": round(batch * prefill / prefill_s, 1),
