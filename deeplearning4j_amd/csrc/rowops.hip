@@ -335,67 +335,86 @@ __global__ __launch_bounds__(256) void layernorm_rows(RowArgs a, const T* __rest
 // One wave per row for rows at a constant pitch (the usual case: a dense or row-strided matrix), vector path only.
 // No shape walk and no predicated loads: every lane issues its x / gain / bias vectors at once (lanes past the row's
 // end re-read the last vector and are masked out of the sums), so the three latencies overlap instead of queueing.
-template <typename T, int NV, bool HAS_BIAS>
+template <typename T, int NV, bool HAS_BIAS, int RPW>
 __global__ __launch_bounds__(256) void layernorm_linear(const T* __restrict__ x, const T* __restrict__ gain, const T* __restrict__ bias,
                                                         T* __restrict__ z, LongType rows, int L, LongType xPitch, LongType zPitch, float eps) {
   using A = typename Conv<T>::acc;
   using Raw = typename RawIO<T>::raw;
   constexpr int VEC = RawIO<T>::N;
   const int t = threadIdx.x & 63;
-  const LongType row = (LongType)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= rows) return;
-  const T* xr = x + row * xPitch;
+  // a wave owns RPW consecutive rows: gain and bias are fetched once for all of them
+  const LongType row0 = ((LongType)blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW;
+  if (row0 >= rows) return;
   int e0[NV];
   A keep[NV];
-  Raw xv[NV], gv[NV], bv[NV];
+  Raw xv[RPW][NV], gv[NV], bv[NV];
 #pragma unroll
   for (int i = 0; i < NV; i++) {
     const int e = (t + i * 64) * VEC;
     keep[i] = e < L ? (A)1 : (A)0;
     e0[i] = e < L ? e : L - VEC;
-    xv[i] = *reinterpret_cast<const Raw*>(xr + e0[i]);
+  }
+#pragma unroll
+  for (int r = 0; r < RPW; r++) {
+    const LongType row = row0 + r < rows ? row0 + r : rows - 1;
+#pragma unroll
+    for (int i = 0; i < NV; i++) xv[r][i] = *reinterpret_cast<const Raw*>(x + row * xPitch + e0[i]);
   }
 #pragma unroll
   for (int i = 0; i < NV; i++) {
     gv[i] = *reinterpret_cast<const Raw*>(gain + e0[i]);
     if (HAS_BIAS) bv[i] = *reinterpret_cast<const Raw*>(bias + e0[i]);
   }
-  A vals[NV * VEC];
-  A sum = (A)0;
+  A vals[RPW][NV * VEC];
+  A sum[RPW];
 #pragma unroll
-  for (int i = 0; i < NV; i++) {
-    RawIO<T>::unpack(xv[i], &vals[i * VEC]);
-    A part = (A)0;
+  for (int r = 0; r < RPW; r++) {
+    sum[r] = (A)0;
 #pragma unroll
-    for (int e = 0; e < VEC; e++) part += vals[i * VEC + e];
-    sum += part * keep[i];
-  }
-  sum = wave_allreduce<SumOp>(sum);
-  const A mean = sum / (A)L;
-  A sq = (A)0;
+    for (int i = 0; i < NV; i++) {
+      RawIO<T>::unpack(xv[r][i], &vals[r][i * VEC]);
+      A part = (A)0;
 #pragma unroll
-  for (int i = 0; i < NV; i++) {
-    A part = (A)0;
-#pragma unroll
-    for (int e = 0; e < VEC; e++) { const A d = vals[i * VEC + e] - mean; vals[i * VEC + e] = d; part += d * d; }
-    sq += part * keep[i];
-  }
-  sq = wave_allreduce<SumOp>(sq);
-  const A var = L > 1 ? sq / (A)L : (A)0;
-  const A rstd = (A)1 / r_sqrt<A>(var + (A)eps);
-  T* zr = z + row * zPitch;
-#pragma unroll
-  for (int i = 0; i < NV; i++) {
-    A g[VEC], b[VEC];
-    RawIO<T>::unpack(gv[i], g);
-    if (HAS_BIAS) RawIO<T>::unpack(bv[i], b);
-#pragma unroll
-    for (int e = 0; e < VEC; e++) {
-      A y = vals[i * VEC + e] * rstd * g[e];
-      if (HAS_BIAS) y += b[e];
-      vals[i * VEC + e] = y;
+      for (int e = 0; e < VEC; e++) part += vals[r][i * VEC + e];
+      sum[r] += part * keep[i];
     }
-    if (keep[i] != (A)0) *reinterpret_cast<Raw*>(zr + e0[i]) = RawIO<T>::pack(&vals[i * VEC]);
+  }
+#pragma unroll
+  for (int r = 0; r < RPW; r++) sum[r] = wave_allreduce<SumOp>(sum[r]);
+  A sq[RPW];
+#pragma unroll
+  for (int r = 0; r < RPW; r++) {
+    const A mean = sum[r] / (A)L;
+    sq[r] = (A)0;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      A part = (A)0;
+#pragma unroll
+      for (int e = 0; e < VEC; e++) { const A d = vals[r][i * VEC + e] - mean; vals[r][i * VEC + e] = d; part += d * d; }
+      sq[r] += part * keep[i];
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < RPW; r++) sq[r] = wave_allreduce<SumOp>(sq[r]);
+#pragma unroll
+  for (int r = 0; r < RPW; r++) {
+    if (row0 + r >= rows) break;
+    const A var = L > 1 ? sq[r] / (A)L : (A)0;
+    const A rstd = (A)1 / r_sqrt<A>(var + (A)eps);
+    T* zr = z + (row0 + r) * zPitch;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      A g[VEC], b[VEC];
+      RawIO<T>::unpack(gv[i], g);
+      if (HAS_BIAS) RawIO<T>::unpack(bv[i], b);
+#pragma unroll
+      for (int e = 0; e < VEC; e++) {
+        A y = vals[r][i * VEC + e] * rstd * g[e];
+        if (HAS_BIAS) y += b[e];
+        vals[r][i * VEC + e] = y;
+      }
+      if (keep[i] != (A)0) *reinterpret_cast<Raw*>(zr + e0[i]) = RawIO<T>::pack(&vals[r][i * VEC]);
+    }
   }
 }
 
@@ -414,10 +433,16 @@ static void layerNormTyped(hipStream_t s, const void* x, const void* gain, const
     const bool linear = p.outerX.rank <= 1 && p.outerZ.rank <= 1 && L < (1 << 30);
     if (linear && L <= 4 * perWave) {
       const LongType xp = p.outerX.rank ? p.outerX.stride[0] : 0, zp = p.outerZ.rank ? p.outerZ.stride[0] : 0;
-#define LNL(NV) do { if (bt) hipLaunchKernelGGL((layernorm_linear<T, NV, true>), dim3(gw), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); \
-                     else hipLaunchKernelGGL((layernorm_linear<T, NV, false>), dim3(gw), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); } while (0)
+      // many rows: two per wave (gain and bias fetched once for both); few rows: one per wave, so that every CU gets some
+      const bool pair = p.rows >= 4096;
+      const unsigned gp = (unsigned)((p.rows + 7) / 8);
+#define LNL(NV) do { if (pair) { if (bt) hipLaunchKernelGGL((layernorm_linear<T, NV, true, 2>), dim3(gp), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); \
+                                 else hipLaunchKernelGGL((layernorm_linear<T, NV, false, 2>), dim3(gp), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); } \
+                     else { if (bt) hipLaunchKernelGGL((layernorm_linear<T, NV, true, 1>), dim3(gw), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); \
+                            else hipLaunchKernelGGL((layernorm_linear<T, NV, false, 1>), dim3(gw), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); } } while (0)
       if (L <= perWave) { LNL(1); return; }
       if (L <= 2 * perWave) { LNL(2); return; }
+      if (L <= 3 * perWave) { LNL(3); return; }   // 768 floats: three full passes, no clamped re-reads
       LNL(4); return;
 #undef LNL
     }

@@ -299,6 +299,29 @@ def test_index_reduce_ties_nan_inf_and_scalar(ex, oracle):
     assert ex.exec_index_reduce(0, NDArray.from_numpy(big)).to_numpy() == 123456
 
 
+@pytest.mark.parametrize("rows,L,pitch", [(37, 1028, 1028), (5, 8192, 8192), (9, 5000, 5000), (33, 4096, 4352), (3, 1024, 2048)])
+def test_reductions_over_rows_at_a_constant_pitch(ex, oracle, rows, L, pitch):
+    """Rows of 1024..8192 elements at a constant pitch take the one-shot kernels (all loads up front, masked tail):
+    value reductions within the re-ordered-sum bound, index reductions bit-exact, also on a column slice of a wider
+    matrix."""
+    rng = np.random.default_rng(rows + L)
+    wide = rng.uniform(-1, 1, (rows, pitch)).astype(np.float32)
+    wide[:, L // 2] = 1.5
+    wide[: rows // 2, L - 1] = 1.5                      # a tie with the last element of the row
+    x = np.ascontiguousarray(wide[:, :L])
+    X = NDArray.from_numpy(wide).view((rows, L), (pitch, 1), 0)
+    atol = _sum_atol(x, 1)
+    assert_close(ex.exec_reduce_same(ReduceSame.Sum, X, [1]).to_numpy(), oracle.reduce_same(0, x, np.zeros(rows, np.float32), [1]), 1e-5, atol, "sum")
+    assert_close(ex.exec_reduce_float(ReduceFloat.Mean, X, [1]).to_numpy(), x.astype(np.float64).mean(1), 1e-5, atol / L, "mean")
+    assert_close(ex.exec_reduce_float(ReduceFloat.Norm2, X, [1]).to_numpy(), np.sqrt((x.astype(np.float64) ** 2).sum(1)), 1e-5, 0, "norm2")
+    assert np.array_equal(ex.exec_reduce_same(ReduceSame.Max, X, [1]).to_numpy(), x.max(1))
+    assert np.array_equal(ex.exec_reduce_same(ReduceSame.Min, X, [1]).to_numpy(), x.min(1))
+    for op in (0, 1, 2, 3):
+        want = oracle.index_reduce(op, x, np.zeros(rows, np.int64), [1])
+        assert np.array_equal(ex.exec_index_reduce(op, X, [1]).to_numpy(), want), op
+    assert list(ex.exec_index_reduce(0, X, [1]).to_numpy()) == [L // 2] * rows
+
+
 @pytest.mark.parametrize("dtype", [BFLOAT16, HALF])
 def test_index_reduce_half_types(ex, oracle, dtype):
     rng = np.random.default_rng(17)
