@@ -157,6 +157,90 @@ __global__ __launch_bounds__(256) void softmax_rows(RowArgs a, const T* __restri
   }
 }
 
+// Rows with unit inner stride that fit one wave's registers (softmax over the contiguous last axis of a dense array or of a
+// permuted view): every load unconditional (lanes past the row's end re-read its last vector and their bits are replaced
+// by the padding value) and pinned ahead of the first use, one wave per row.
+// Measured on fp32 [196608, 1024]: 253 us against 275 us for the general kernel (a plain copy of the same bytes: 242 us).
+template <typename T> struct PadBits;   // the 16-bit / 32-bit pattern of -max(T), repeated over a 32-bit word
+template <> struct PadBits<float> { static constexpr unsigned v = 0xff7fffffu; };
+template <> struct PadBits<bf16_t> { static constexpr unsigned v = 0xff7fff7fu; };
+template <> struct PadBits<f16_t> { static constexpr unsigned v = 0xfbfffbffu; };
+template <typename T, int NV, bool NT>
+__global__ __launch_bounds__(256) void softmax_linear(RowArgs a, const T* __restrict__ x, T* __restrict__ z, int clamp) {
+  using Raw = typename RawIO<T>::raw;
+  constexpr int VEC = RawIO<T>::N;
+  const int t = threadIdx.x & 63;
+  const LongType row = (LongType)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= a.rows) return;
+  const int L = (int)a.rowLen;
+  const T* xr = x + walk<LongType>(a.outerX, row);
+  raw_u32x4 bits[NV];
+  int e0[NV];
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const int e = (t + i * 64) * VEC;
+    e0[i] = e < L ? e : L - VEC;
+    const raw_u32x4* src = reinterpret_cast<const raw_u32x4*>(xr + e0[i]);
+    bits[i] = NT ? __builtin_nontemporal_load(src) : *src;
+  }
+  __builtin_amdgcn_sched_barrier(0);   // all loads are issued before the first use: one trip to memory per row
+  float vals[NV * VEC];
+  const float NEG = -r_tmax<float>();
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const unsigned keep = (t + i * 64) * VEC < L ? 0xffffffffu : 0u;
+    const raw_u32x4 b = (bits[i] & keep) | (raw_u32x4)(PadBits<T>::v & ~keep);
+    RawIO<T>::unpack(__builtin_bit_cast(Raw, b), &vals[i * VEC]);
+  }
+  // rows of finite numbers need neither the finite-only maximum nor the +-88 clamps (see softmax_rows); 0 * v is NaN
+  // exactly for v = +-inf or NaN; the padding (-max) is finite
+  float mx = NEG, probe = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV * VEC; i++) {
+    probe = __builtin_fmaf(vals[i], 0.f, probe);
+    mx = vals[i] > mx ? vals[i] : mx;
+  }
+  float sum = 0.f;
+  const float L2E = 1.44269502162933349609375f;
+  if (__builtin_amdgcn_ballot_w64(probe != probe) == 0) {
+    mx = wave_allreduce<MaxOp>(mx);
+#pragma unroll
+    for (int i = 0; i < NV * VEC; i++) {
+      const float r = __builtin_amdgcn_exp2f((vals[i] - mx) * L2E);
+      vals[i] = r;
+      sum += r;
+    }
+  } else {
+    mx = NEG;
+#pragma unroll
+    for (int i = 0; i < NV * VEC; i++) mx = softmax_maxstep<float>(mx, vals[i], clamp);
+    mx = wave_allreduce<MaxOp>(mx);
+    if (clamp && mx == NEG) mx = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++)
+#pragma unroll
+      for (int e = 0; e < VEC; e++) {
+        float r = 0.f;
+        if ((t + i * 64) * VEC < L) r = softmax_term(vals[i * VEC + e], mx, clamp);
+        vals[i * VEC + e] = r;
+        sum += r;
+      }
+  }
+  sum = wave_allreduce<SumOp>(sum);
+  if (clamp) sum = sum > 1e-6f ? sum : 1e-6f;
+  const float inv = 1.f / sum;
+  T* zr = z + walk<LongType>(a.outerZ, row);
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    if ((t + i * 64) * VEC >= L) continue;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) vals[i * VEC + e] *= inv;
+    Raw* dst = reinterpret_cast<Raw*>(zr + e0[i]);
+    if (NT) __builtin_nontemporal_store(RawIO<T>::pack(&vals[i * VEC]), dst);
+    else *dst = RawIO<T>::pack(&vals[i * VEC]);
+  }
+}
+
 // rows longer than the register budget: three passes over global memory, one block per row
 template <typename T>
 __global__ __launch_bounds__(256) void softmax_long(RowArgs a, const T* __restrict__ x, T* __restrict__ z, int clamp) {
@@ -215,6 +299,22 @@ static bool rowsVectorOk(const RowPlan& p, const void* x, const void* z, int V) 
 }
 
 template <typename T>
+static void softmaxLinear(hipStream_t s, const RowArgs& a, const T* x, T* z, int clamp, int nt) {
+  constexpr int V = 16 / sizeof(T);
+  const int passes = (int)((a.rowLen / V + 63) / 64);
+  const dim3 grid((unsigned)((a.rows + 3) / 4));
+#define SL(NV) do { if (nt) hipLaunchKernelGGL((softmax_linear<T, NV, true>), grid, dim3(256), 0, s, a, x, z, clamp); \
+                    else hipLaunchKernelGGL((softmax_linear<T, NV, false>), grid, dim3(256), 0, s, a, x, z, clamp); } while (0)
+  switch (passes) {
+    case 1: SL(1); break; case 2: SL(2); break; case 3: SL(3); break; case 4: SL(4); break;
+    case 5: SL(5); break; case 6: SL(6); break; case 7: SL(7); break; default: SL(8); break;
+  }
+#undef SL
+}
+template <>
+void softmaxLinear<double>(hipStream_t, const RowArgs&, const double*, double*, int, int) {}
+
+template <typename T>
 static void softmaxTyped(hipStream_t s, const void* x, void* z, const RowPlan& p, int clamp) {
   constexpr int V = 16 / sizeof(T);
   RowArgs a = rowArgs(p);
@@ -230,6 +330,10 @@ static void softmaxTyped(hipStream_t s, const void* x, void* z, const RowPlan& p
     const LongType perWave = 64 * V, perBlock = 256 * V;
     // rows streamed once and larger than the last-level cache: non-temporal accesses
     const int nt = (size_t)p.rows * (size_t)L * sizeof(T) * 2 > ((size_t)288 << 20) ? 1 : 0;
+    if (sizeof(T) <= 4 && L <= 8 * perWave) {
+      softmaxLinear<T>(s, a, xt, zt, clamp, nt);
+      return;
+    }
 #define SM(TPR, NV, GRID) hipLaunchKernelGGL((softmax_rows<T, TPR, NV, V>), dim3(GRID), dim3(256), 0, s, a, xt, zt, clamp, nt)
     if (L <= perWave) { SM(64, 1, gw); return; }
     if (L <= 2 * perWave) { SM(64, 2, gw); return; }
