@@ -469,6 +469,21 @@ __global__ __launch_bounds__(256) void layernorm_linear(const T* __restrict__ x,
     gv[i] = *reinterpret_cast<const Raw*>(gain + e0[i]);
     if (HAS_BIAS) bv[i] = *reinterpret_cast<const Raw*>(bias + e0[i]);
   }
+  // a lone row (a decode step) waits on gain and bias coming cold from HBM: one empty asm that "uses" every loaded
+  // vector makes the compiler issue all the loads ahead of it, instead of sinking gain and bias below the row's first
+  // reduction (a second trip to memory)
+  if (RPW == 1) {
+    if (!HAS_BIAS) {
+#pragma unroll
+      for (int i = 0; i < NV; i++) bv[i] = gv[i];
+    }
+    if (NV == 1) asm volatile("" : "+v"(xv[0][0]), "+v"(gv[0]), "+v"(bv[0]));
+    if (NV == 2) asm volatile("" : "+v"(xv[0][0]), "+v"(xv[0][NV > 1 ? 1 : 0]), "+v"(gv[0]), "+v"(gv[NV > 1 ? 1 : 0]), "+v"(bv[0]), "+v"(bv[NV > 1 ? 1 : 0]));
+    if (NV == 3) asm volatile("" : "+v"(xv[0][0]), "+v"(xv[0][NV > 1 ? 1 : 0]), "+v"(xv[0][NV > 2 ? 2 : 0]), "+v"(gv[0]), "+v"(gv[NV > 1 ? 1 : 0]), "+v"(gv[NV > 2 ? 2 : 0]),
+                                    "+v"(bv[0]), "+v"(bv[NV > 1 ? 1 : 0]), "+v"(bv[NV > 2 ? 2 : 0]));
+    if (NV == 4) asm volatile("" : "+v"(xv[0][0]), "+v"(xv[0][NV > 1 ? 1 : 0]), "+v"(xv[0][NV > 2 ? 2 : 0]), "+v"(xv[0][NV > 3 ? 3 : 0]), "+v"(gv[0]), "+v"(gv[NV > 1 ? 1 : 0]),
+                                    "+v"(gv[NV > 2 ? 2 : 0]), "+v"(gv[NV > 3 ? 3 : 0]), "+v"(bv[0]), "+v"(bv[NV > 1 ? 1 : 0]), "+v"(bv[NV > 2 ? 2 : 0]), "+v"(bv[NV > 3 ? 3 : 0]));
+  }
   A vals[RPW][NV * VEC];
   A sum[RPW];
 #pragma unroll
