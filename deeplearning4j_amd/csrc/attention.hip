@@ -304,16 +304,12 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
   }
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int g = lane / CH, c = lane % CH;
-  float q[8];
-  RawIO<T>::unpack(*reinterpret_cast<const typename RawIO<T>::raw*>(Q + qi * a.qT + c * 8), q);
-  const float L2E = 1.44269502162933349609375f;
-  float m = -1.0e30f, l = 0.f, o[8];
-#pragma unroll
-  for (int e = 0; e < 8; e++) o[e] = 0.f;
-
-  for (LongType k0 = (LongType)wave * (KPS * U); k0 < a.Tv; k0 += (LongType)NW * (KPS * U)) {
-    typename RawIO<T>::raw kr[U], vr[U];
-    bool valid[U];
+  // the query row was written by the kernel before this one and the first keys come cold from HBM: all of these loads
+  // are issued before the first value is touched, so the two latencies overlap
+  const typename RawIO<T>::raw qraw = *reinterpret_cast<const typename RawIO<T>::raw*>(Q + qi * a.qT + c * 8);
+  typename RawIO<T>::raw kr[U], vr[U];
+  bool valid[U];
+  auto issue = [&](LongType k0) {
 #pragma unroll
     for (int u = 0; u < U; u++) {
       LongType key = k0 + u * KPS + g;
@@ -322,6 +318,17 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
       kr[u] = *reinterpret_cast<const typename RawIO<T>::raw*>(K + key * a.kT + c * 8);
       vr[u] = *reinterpret_cast<const typename RawIO<T>::raw*>(V + key * a.vT + c * 8);
     }
+  };
+  LongType k0 = (LongType)wave * (KPS * U);
+  if (k0 < a.Tv) issue(k0);
+  float q[8];
+  RawIO<T>::unpack(qraw, q);
+  const float L2E = 1.44269502162933349609375f;
+  float m = -1.0e30f, l = 0.f, o[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) o[e] = 0.f;
+
+  while (k0 < a.Tv) {
     float sc[U], tmax = m;
 #pragma unroll
     for (int u = 0; u < U; u++) {
@@ -352,6 +359,8 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
 #pragma unroll
       for (int e = 0; e < 8; e++) o[e] = __builtin_fmaf(p, vf[e], o[e]);
     }
+    k0 += (LongType)NW * (KPS * U);
+    if (k0 < a.Tv) issue(k0);
   }
   // merge the lane groups of the wave (lanes with equal c): bring every state to the common maximum, then add
   float mAll = m;
