@@ -370,6 +370,123 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16p(GemmArgs g, const T
     }
 }
 
+// The same kernel with the global loads of PD K-tiles in flight (PD register sets, the K loop unrolled PD times so that
+// each set is a fixed group of registers): for launches that put one small tile on a CU, where a K-tile's MFMAs take
+// 130 cycles and the loop otherwise runs at one memory latency per K-tile.  Whole tiles only, K a multiple of PD K-tiles.
+template <typename T, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int PD>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16q(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
+                                                             unsigned tilesM, unsigned tilesN) {
+  constexpr int BK = 64, NT = WM * WN * 64;
+  constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
+  using LayA = TileLayout<BM, A_KC>;
+  using LayB = TileLayout<BN, B_KC>;
+  constexpr int SLOTS_A = LayA::SLOTS, SLOTS_B = LayB::SLOTS, STAGE = SLOTS_A + SLOTS_B;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  u32x4* smem = reinterpret_cast<u32x4*>(smem_raw);
+
+  unsigned tm, tn;
+  tileOf(blockIdx.x, gridDim.x, tilesM, tilesN, tm, tn);
+  const LongType m0 = (LongType)tm * BM, n0 = (LongType)tn * BN;
+  const LongType bz = blockIdx.z;
+  { LongType oa, ob, oc; batchOffsets(g, bz, oa, ob, oc); A += oa; B += ob; C += oc; }
+  const LongType lda = A_KC ? g.aRow : g.aCol, ldb = B_KC ? g.bCol : g.bRow;
+
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+  static_assert(PD % 2 == 0, "the LDS stage of a K-tile must be a compile-time constant inside the unrolled loop");
+  TileLoader<BM, NT, A_KC> la[PD];
+  TileLoader<BN, NT, B_KC> lb[PD];
+  const LongType KT = (g.K + BK - 1) / BK;
+
+  // K is a multiple of PD K-tiles (host), and nothing below is conditional: loads past the end re-read the last K-tile and
+  // the store after the last K-tile writes a stage nobody reads.  The K loop is then one basic block, which is what lets
+  // the compiler wait for exactly one register set while the younger loads stay in flight.
+#pragma unroll
+  for (int u = 0; u < PD; u++) {
+    la[u].loadFull(A, lda, m0, (LongType)u * BK, t);
+    lb[u].loadFull(B, ldb, n0, (LongType)u * BK, t);
+  }
+  la[0].store(smem, t);
+  lb[0].store(smem + SLOTS_A, t);
+  __syncthreads();
+
+  for (LongType kt0 = 0; kt0 < KT; kt0 += PD) {
+#pragma unroll
+  for (int u = 0; u < PD; u++) {
+    const LongType kt = kt0 + u;
+    const int cur = u & 1;
+    // K-tile kt sits in LDS: its register set takes K-tile kt + PD
+    {
+      const LongType nx = kt + PD < KT ? kt + PD : KT - 1;
+      la[u].loadFull(A, lda, m0, nx * BK, t);
+      lb[u].loadFull(B, ldb, n0, nx * BK, t);
+    }
+    const u32x4* sA = smem + cur * STAGE;
+    const u32x4* sB = sA + SLOTS_A;
+    // software pipeline over the four k-steps: fragments of step ks+1 are read while the MFMAs of step ks
+    // run; the next tile's registers are written to the other LDS stage in the shadow of step 2
+    u32x4 fa[2][TM], fb[2][TN];
+    auto readFrag = [&](int ks, int buf) {
+      const int kg = ks * 2 + (lane >> 5);
+#pragma unroll
+      for (int i = 0; i < TM; i++) fa[buf][i] = sA[LayA::slot(kg, wm * WTM + i * 32 + (lane & 31))];
+#pragma unroll
+      for (int j = 0; j < TN; j++) fb[buf][j] = sB[LayB::slot(kg, wn * WTN + j * 32 + (lane & 31))];
+    };
+    readFrag(0, 0);
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ks++) {
+      if (ks + 1 < BK / 16) readFrag(ks + 1, (ks + 1) & 1);
+      if (ks == 2) {
+        u32x4* dst = smem + (cur ^ 1) * STAGE;
+        la[(u + 1) % PD].store(dst, t);
+        lb[(u + 1) % PD].store(dst + SLOTS_A, t);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = Mfma16<T>::mma(fa[ks & 1][i], fb[ks & 1][j], acc[i][j]);
+      // interleave: one LDS read issued per pair of MFMAs
+#pragma unroll
+      for (int q = 0; q < (TM + TN); q++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, (TM * TN) / (TM + TN) > 0 ? (TM * TN) / (TM + TN) : 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+    }
+    __syncthreads();
+  }
+  }
+
+  // epilogue: lane owns column (lane % 32); register r of a 32x32 tile is row 8*(r/4) + 4*(lane/32) + r%4
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const LongType col = n0 + wn * WTN + j * 32 + (lane & 31);
+      if (col >= g.N) continue;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const LongType row = m0 + wm * WTM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r & 3);
+        if (row < g.M) {
+          const LongType off = row * g.cRow + col * g.cCol;
+          float v = g.alpha * acc[i][j][r];
+          if (g.beta != 0.f) v += g.beta * to_float(C[off]);
+          if (g.bias) v += to_float(static_cast<const T*>(g.bias)[col]);
+          C[off] = Conv<T>::from(v);
+        }
+      }
+    }
+}
+
 // Steady-state kernel for problems made of whole tiles (M % BM == 0, N % BN == 0, K % 64 == 0): no bounds handling,
 // so the K loop is one basic block and the instruction order below is the order the hardware sees.  A wave issues
 // in order, and an MFMA 32x32x16 keeps the matrix pipe busy for 32 cycles: every LDS / global instruction is placed
@@ -771,10 +888,15 @@ static void launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
   const bool usePipe = splits == 1;   // the split-K epilogue lives in the plain kernel
   // whole tiles only: the kernel without bounds handling (its K loop needs two K-tiles at least)
   const bool useFull = usePipe && BM * BN >= 128 * 128 && g.M % BM == 0 && g.N % BN == 0 && g.K % 64 == 0 && g.K >= 128;
+  // small tiles, at most a couple per CU and a long K: the loop is bound by one memory latency per K-tile unless several
+  // K-tiles are in flight
+  const unsigned nTiles = (unsigned)(((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN) * batch);
+  const bool useDeep = usePipe && !useFull && BM * BN <= 64 * 64 && nTiles <= 1024 && g.K >= 512 && g.M % BM == 0 && g.N % BN == 0 && g.K % 256 == 0;
   auto kern = useFull ? gemm_mfma16f<T, BM, BN, WM, WN, A_KC, B_KC>
-                      : usePipe ? gemm_mfma16p<T, BM, BN, WM, WN, A_KC, B_KC> : gemm_mfma16<T, BM, BN, WM, WN, A_KC, B_KC>;
-  const int which = useFull ? 2 : usePipe ? 1 : 0;
-  static bool attrSet[3] = {false, false, false};
+              : useDeep ? gemm_mfma16q<T, BM, BN, WM, WN, A_KC, B_KC, 4>
+              : usePipe ? gemm_mfma16p<T, BM, BN, WM, WN, A_KC, B_KC> : gemm_mfma16<T, BM, BN, WM, WN, A_KC, B_KC>;
+  const int which = useFull ? 2 : useDeep ? 3 : usePipe ? 1 : 0;
+  static bool attrSet[4] = {false, false, false, false};
   if (!attrSet[which]) {
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS));
     attrSet[which] = true;
