@@ -1063,9 +1063,126 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32(GemmArgs g, const fl
     }
 }
 
+// The fp32 kernel for launches of whole tiles that put one small tile on a CU: PD K-tiles of global loads in flight (PD
+// register sets, the K loop unrolled PD times and free of branches -- loads past the end re-read the last K-tile, the
+// store after the last K-tile fills a stage nobody reads), so the loop runs at the MFMA rate instead of one memory
+// latency per 16 k.  Host: M % BM == 0, N % BN == 0, K % (16 * PD) == 0.
+template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int PD>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32q(GemmArgs g, const float* __restrict__ A, const float* __restrict__ B,
+                                                              float* __restrict__ C, unsigned tilesM, unsigned tilesN) {
+  static_assert(PD % 2 == 0, "the LDS stage of a K-tile must be a compile-time constant inside the unrolled loop");
+  constexpr int BK = 16, NT = WM * WN * 64, PA = BM + 4, PB = BN + 4;
+  constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
+  constexpr int VA = BM * BK / 4 / NT, VB = BN * BK / 4 / NT;   // float4 per thread
+  __shared__ __attribute__((aligned(16))) float sA[2][BK * PA];
+  __shared__ __attribute__((aligned(16))) float sB[2][BK * PB];
+  unsigned tm, tn;
+  tileOf(blockIdx.x, gridDim.x, tilesM, tilesN, tm, tn);
+  const LongType m0 = (LongType)tm * BM, n0 = (LongType)tn * BN;
+  const LongType bz = blockIdx.z;
+  { LongType oa, ob, oc; batchOffsets(g, bz, oa, ob, oc); A += oa; B += ob; C += oc; }
+  const LongType lda = A_KC ? g.aRow : g.aCol, ldb = B_KC ? g.bCol : g.bRow;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wm = wave / WN, wn = wave % WN;
+  typedef __attribute__((ext_vector_type(4))) float f32x4;
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+  f32x4 ra[PD][VA], rb[PD][VB];
+  auto load = [&](int u, LongType k0) {
+#pragma unroll
+    for (int i = 0; i < VA; i++) {
+      const int v = t + i * NT;
+      if (A_KC) ra[u][i] = *reinterpret_cast<const f32x4*>(A + (m0 + (v >> 2)) * lda + k0 + (v & 3) * 4);
+      else ra[u][i] = *reinterpret_cast<const f32x4*>(A + (k0 + v / (BM / 4)) * lda + m0 + (v % (BM / 4)) * 4);
+    }
+#pragma unroll
+    for (int i = 0; i < VB; i++) {
+      const int v = t + i * NT;
+      if (B_KC) rb[u][i] = *reinterpret_cast<const f32x4*>(B + (n0 + (v >> 2)) * ldb + k0 + (v & 3) * 4);
+      else rb[u][i] = *reinterpret_cast<const f32x4*>(B + (k0 + v / (BN / 4)) * ldb + n0 + (v % (BN / 4)) * 4);
+    }
+  };
+  auto store = [&](int u, int stage) {
+#pragma unroll
+    for (int i = 0; i < VA; i++) {
+      const int v = t + i * NT;
+      if (A_KC) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) sA[stage][((v & 3) * 4 + q) * PA + (v >> 2)] = ra[u][i][q];
+      } else {
+        *reinterpret_cast<f32x4*>(&sA[stage][(v / (BM / 4)) * PA + (v % (BM / 4)) * 4]) = ra[u][i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < VB; i++) {
+      const int v = t + i * NT;
+      if (B_KC) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) sB[stage][((v & 3) * 4 + q) * PB + (v >> 2)] = rb[u][i][q];
+      } else {
+        *reinterpret_cast<f32x4*>(&sB[stage][(v / (BN / 4)) * PB + (v % (BN / 4)) * 4]) = rb[u][i];
+      }
+    }
+  };
+  const LongType KT = g.K / BK;
+#pragma unroll
+  for (int u = 0; u < PD; u++) load(u, (LongType)u * BK);
+  store(0, 0);
+  __syncthreads();
+  for (LongType kt0 = 0; kt0 < KT; kt0 += PD) {
+#pragma unroll
+    for (int u = 0; u < PD; u++) {
+      const LongType kt = kt0 + u;
+      const int cur = u & 1;
+      const LongType nx = kt + PD < KT ? kt + PD : KT - 1;
+      load(u, nx * BK);   // K-tile kt sits in LDS: its register set takes K-tile kt + PD
+#pragma unroll
+      for (int ks = 0; ks < BK / 2; ks++) {
+        const int k = ks * 2 + (lane >> 5);
+        float fa[TM], fb[TN];
+#pragma unroll
+        for (int i = 0; i < TM; i++) fa[i] = sA[cur][k * PA + wm * WTM + i * 32 + (lane & 31)];
+#pragma unroll
+        for (int j = 0; j < TN; j++) fb[j] = sB[cur][k * PB + wn * WTN + j * 32 + (lane & 31)];
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+          for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+      }
+      store((u + 1) % PD, cur ^ 1);
+      __syncthreads();
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const LongType col = n0 + wn * WTN + j * 32 + (lane & 31);
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const LongType row = m0 + wm * WTM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r & 3);
+        const LongType off = row * g.cRow + col * g.cCol;
+        float v = g.alpha * acc[i][j][r];
+        if (g.beta != 0.f) v += g.beta * C[off];
+        if (g.bias) v += static_cast<const float*>(g.bias)[col];
+        C[off] = v;
+      }
+    }
+}
+
 template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC>
 static void launchMfma32Cfg(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C, LongType batch) {
   const unsigned tilesM = (unsigned)((g.M + BM - 1) / BM), tilesN = (unsigned)((g.N + BN - 1) / BN);
+  if (g.K >= 256 && g.M % BM == 0 && g.N % BN == 0 && g.K % 128 == 0) {
+    constexpr int PD = BM * BN <= 64 * 64 ? 8 : 4;
+    hipLaunchKernelGGL((gemm_mfma32q<BM, BN, WM, WN, A_KC, B_KC, PD>), dim3(tilesM * tilesN, 1, (unsigned)batch), dim3(WM * WN * 64), 0, s, g,
+                       (const float*)A, (const float*)B, (float*)C, tilesM, tilesN);
+    return;
+  }
   hipLaunchKernelGGL((gemm_mfma32<BM, BN, WM, WN, A_KC, B_KC>), dim3(tilesM * tilesN, 1, (unsigned)batch), dim3(WM * WN * 64), 0, s, g,
                      (const float*)A, (const float*)B, (float*)C, tilesM, tilesN);
 }
