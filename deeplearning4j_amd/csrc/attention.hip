@@ -124,6 +124,7 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
   }
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, h = lane >> 5;
   const float L2E = 1.44269502162933349609375f;
+  const float sc = a.applyScale ? a.scale : 1.f;
   const bool paired = a.perBatch != a.qTiles;
   for (int pass = 0; pass < (paired ? 2 : 1); pass++) {
   const int qt = pass == 0 ? a.qTiles - 1 - slot : slot;
@@ -153,8 +154,8 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
   TileLoader<D, NT, false> lv;            // rows = dv (contiguous in memory), "k" = keys
   auto loadKV = [&](LongType kv0) {
 #pragma unroll
-    for (int part = 0; part < D / 64; part++) lk[part].load(K + part * 64, a.kT, kv0, a.Tv, 0, 64, t);
-    lv.load(V, a.vT, 0, D, kv0, a.Tv, t);
+    for (int part = 0; part < D / 64; part++) lk[part].loadClamped(K + part * 64, a.kT, kv0, a.Tv, 0, 64, t);
+    lv.loadClamped(V, a.vT, 0, D, kv0, a.Tv, t);   // keys past the end repeat the last one: their weights are exactly 0
   };
   auto storeKV = [&](u32x4* dst) {
 #pragma unroll
@@ -167,6 +168,11 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
     storeKV(smem);
   }
   __syncthreads();
+  // Make the Q fragments "used" here, on every path into the key loop: otherwise the path that skips the block above
+  // leaves their loads pending as far as the compiler can tell, and it waits for them -- and with them for the freshly
+  // issued loads of the next tile -- in front of the first MFMAs of every iteration.
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ks++) asm volatile("" : "+v"(qf[ks]));
 
   for (LongType it = 0; it < nTiles; it++) {
     const int cur = (int)(it & 1);
@@ -196,7 +202,7 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
         float v0 = s[kt][r], v1 = s[kt][r + 1];
-        if (a.applyScale) { v0 *= a.scale; v1 *= a.scale; }
+        v0 *= sc; v1 *= sc;   // sc = 1 when no scale applies: one multiply instead of a multiply and a select
         v0 = __builtin_amdgcn_fmed3f(v0, -1.0e4f, 1.0e4f);
         v1 = __builtin_amdgcn_fmed3f(v1, -1.0e4f, 1.0e4f);
         round_pair<T>(v0, v1);
@@ -204,7 +210,10 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
       }
     // only tiles that touch the diagonal or the end of the keys carry masked entries (wave-uniform test)
     const int qFirst = (int)q0 + wave * 32;
-    if ((a.causal && (int)kv0 + BKV - 1 > qFirst) || kv0 + BKV > a.Tv) {
+    // a real branch (scalar condition, a body the compiler cannot speculate): turned into selects, the mask costs 86
+    // vector instructions on every tile instead of on the few that need it
+    if (__builtin_amdgcn_readfirstlane((int)((a.causal && (int)kv0 + BKV - 1 > qFirst) || kv0 + BKV > a.Tv)) != 0) {
+      asm volatile("; tile with masked entries");
       const int lastKey = a.causal ? ((int)query < (int)a.Tv - 1 ? (int)query : (int)a.Tv - 1) : (int)a.Tv - 1;
 #pragma unroll
       for (int kt = 0; kt < 2; kt++)
@@ -238,6 +247,7 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
     l = l * alpha + psum;
     // the accumulator only needs rescaling when some query's maximum moved
     if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+      asm volatile("; accumulator rescale");   // keeps this a branch: most tiles leave every maximum where it was
 #pragma unroll
       for (int i = 0; i < DT; i++)
 #pragma unroll
@@ -257,6 +267,9 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
         o[i] = Mfma16<T>::mma(vf, pf[ks], o[i]);
       }
     }
+    // nothing that consumes the next tile's registers (the V transposes) may drift up into the MFMA sections: the wait for
+    // those loads belongs here, after a whole tile of work
+    __builtin_amdgcn_sched_barrier(0);
     if (more) storeKV(smem + (cur ^ 1) * (KSLOTS + VSLOTS));
     __syncthreads();
   }

@@ -84,6 +84,36 @@ struct TileLoader {
       }
     }
   }
+  // load() without predicates: rows and k positions past the end are clamped to the last valid one instead of being
+  // zero-filled (the caller never uses what they hold, but it must be finite data).  Every load is unconditional, so
+  // the compiler places its wait where the registers are consumed instead of at the join after each predicated load.
+  // Needs K - k0 to be a multiple of 8 for a k-contiguous operand (whole 16-byte k-groups).
+  template <typename T>
+  __device__ __forceinline__ void loadClamped(const T* __restrict__ base, LongType ld, LongType row0, LongType rowLimit, LongType k0, LongType K, int t) {
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      const int u = t + i * NT;
+      if (PER * NT != UNITS && u >= UNITS) break;
+      if (KC) {
+        const int kg = u & 7, row = u >> 3;
+        LongType r = row0 + row;
+        r = r < rowLimit ? r : rowLimit - 1;
+        LongType k = k0 + kg * 8;
+        k = k < K ? k : K - 8;
+        reg[i] = *reinterpret_cast<const u32x4*>(base + r * ld + k);
+      } else {
+        const int rb = (u >> 1) % (ROWS / 8), kq = (u / (ROWS / 4)) * 2 + (u & 1);
+        LongType r = row0 + rb * 8;
+        r = r + 8 <= rowLimit ? r : rowLimit - 8;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          LongType k = k0 + kq * 4 + q;
+          k = k < K ? k : K - 1;
+          reg[i * 4 + q] = *reinterpret_cast<const u32x4*>(base + k * ld + r);
+        }
+      }
+    }
+  }
   // same as load() for a tile that lies wholly inside the operand: no clamping, no predicates
   template <typename T>
   __device__ __forceinline__ void loadFull(const T* __restrict__ base, LongType ld, LongType row0, LongType k0, int t) {
