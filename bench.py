@@ -31,9 +31,9 @@ MFMA_PEAK = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}   # dense TFLOP/s
 # `--pmc WRITE_SIZE` (separate runs of this script) and scaled by what the same counters read for the plain copy
 # kernel; the summary of those runs sits under profiles/.  Static figures: they are not re-measured here.
 TRAFFIC_MB = {
-    "mmul bf16 4096": 235.2, "mmul f16 4096": 235.2, "mmul f32 4096^3": 847.8, "mmul f32 4096^3 transposeB": 851.7,
-    "mmul f32 1024": 29.4, "mmul f16 1024": 14.8, "mmul bf16 1024": 14.8,
-    "copy fp32": 268.4, "pairwise_add fp32": 402.6, "transform_tanh fp32": 268.4, "reduce_sum": 134.6, "argmax dim1": 134.6,
+    "mmul bf16 4096": 235.2, "mmul f16 4096": 235.2, "mmul f32 4096^3": 859.1, "mmul f32 4096^3 transposeB": 866.0,
+    "mmul f32 1024": 29.5, "mmul f16 1024": 14.8, "mmul bf16 1024": 14.8,
+    "copy fp32": 268.4, "pairwise_add fp32": 402.6, "transform_tanh fp32": 268.4, "reduce_sum": 134.5, "argmax dim1": 134.5,
     "layer_norm fp32": 100.8, "gelu fp32": 100.7, "softmax fp32": 1610.6, "layer_norm bf16": 50.4, "gelu bf16": 50.4,
     "softmax bf16": 805.3, "dot_product_attention_v2": 53.5,
 }
