@@ -1,0 +1,113 @@
+"""BASELINE configs 3 and 4 at their full sizes: size-independent properties over the whole result, and the oracle
+on a sample of rows / batch entries (the oracle would need minutes for the whole arrays).
+
+Config 3: x [16, 1024, 768] -> layer_norm over the last axis -> gelu; softmax over the last axis of logits
+[16, 12, 1024, 1024], dense and through the permuted [0, 2, 1, 3] view.  Config 4: causal attention on
+[96, 1024, 64] (8 x 12 heads folded into the batch)."""
+import numpy as np
+import pytest
+
+from conftest import assert_close
+from deeplearning4j_amd.executioner import TransformStrict
+from deeplearning4j_amd.ndarray import BFLOAT16, FLOAT32, HALF, NDArray, bf16_bits_to_f32, f32_to_bf16_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def _store(a, dt):
+    """fp32 draw -> (values as stored, device array)."""
+    if dt == BFLOAT16:
+        bits = f32_to_bf16_bits(a)
+        return bf16_bits_to_f32(bits), NDArray.from_numpy(bits, BFLOAT16)
+    if dt == HALF:
+        h = a.astype(np.float16)
+        return h.astype(np.float32), NDArray.from_numpy(h)
+    return a, NDArray.from_numpy(a)
+
+
+def _oracle_arr(oracle, vals, dt):
+    if dt == BFLOAT16:
+        return oracle.Arr(f32_to_bf16_bits(vals), oracle.BFLOAT16)
+    if dt == HALF:
+        return oracle.Arr(vals.astype(np.float16))
+    return oracle.Arr(vals.astype(np.float32))
+
+
+def _as_float(oa):
+    return bf16_bits_to_f32(oa.a) if oa.dt == 17 else oa.a.astype(np.float32)
+
+
+@pytest.mark.parametrize("dt,tol", [(FLOAT32, 1e-5), (BFLOAT16, 1e-2)])
+def test_config3_layer_norm_then_gelu(ex, oracle, dt, tol):
+    rng = np.random.default_rng(3003)
+    x, X = _store(rng.normal(0, 1, (16, 1024, 768)).astype(np.float32), dt)
+    g, G = _store(rng.normal(1, 0.02, 768).astype(np.float32), dt)
+    b, B = _store(rng.normal(0, 0.02, 768).astype(np.float32), dt)
+    y = ex.exec_custom("layer_norm", [X, G, B], i_args=[2], b_args=[False])[0]
+    z = ex.exec_transform_strict(TransformStrict.GELU, y)
+    yf, zf = y.to_float(), z.to_float()
+    # whole result: undoing gain and bias leaves rows of mean 0 and variance var / (var + 1e-5)
+    u = (yf.astype(np.float64) - b) / g
+    atol = 3e-2 if dt == BFLOAT16 else 1e-4
+    assert np.abs(u.mean(-1)).max() < atol
+    var = x.astype(np.float64).var(-1)
+    assert np.abs(u.var(-1) - var / (var + 1e-5)).max() < (5e-2 if dt == BFLOAT16 else 1e-3)
+    # gelu(y) = y * sigmoid(1.702 y) has the sign of y and never exceeds |y|
+    assert np.all(np.abs(zf) <= np.abs(yf) + 1e-6) and np.all((zf >= 0) | (yf < 0))
+    # sampled rows against the oracle, both ops
+    rows = [(0, 0), (3, 517), (15, 1023), (8, 64)]
+    xs = np.stack([x[i, j] for i, j in rows])
+    oy = _oracle_arr(oracle, np.zeros_like(xs), dt)
+    oracle.layer_norm(_oracle_arr(oracle, xs, dt), _oracle_arr(oracle, g, dt), _oracle_arr(oracle, b, dt), oy, [1], channels_first=False)
+    got_y = np.stack([yf[i, j] for i, j in rows])
+    assert_close(got_y, _as_float(oy), tol, tol, "layer_norm rows")
+    oz = _oracle_arr(oracle, np.zeros_like(xs), dt)
+    oracle.transform_strict(TransformStrict.GELU, _oracle_arr(oracle, got_y, dt), oz)
+    assert_close(np.stack([zf[i, j] for i, j in rows]), _as_float(oz), tol, tol, "gelu rows")
+
+
+@pytest.mark.parametrize("dt,tol", [(FLOAT32, 1e-5), (BFLOAT16, 1e-2)])
+def test_config3_softmax_dense_and_permuted_view(ex, oracle, dt, tol):
+    rng = np.random.default_rng(3003)
+    shape = (16, 12, 1024, 1024)
+    logits, L = _store(rng.normal(0, 2, shape).astype(np.float32), dt)
+    z = ex.exec_custom("softmax", [L])[0].to_float()
+    # whole result: rows sum to one, entries lie in [0, 1], the largest logit keeps the largest weight
+    sums = z.sum(-1, dtype=np.float64)
+    assert np.abs(sums - 1).max() < (2e-2 if dt == BFLOAT16 else 1e-5)
+    assert z.min() >= 0 and z.max() <= 1
+    am = logits.argmax(-1)
+    assert np.all(np.take_along_axis(z, am[..., None], -1)[..., 0] >= z.max(-1) - 1e-7)
+    # sampled rows against the oracle
+    idx = [(0, 0, 0), (7, 5, 333), (15, 11, 1023)]
+    xs = np.stack([logits[i] for i in idx])
+    oz = _oracle_arr(oracle, np.zeros_like(xs), dt)
+    oracle.softmax(_oracle_arr(oracle, xs, dt), oz, 1)
+    assert_close(np.stack([z[i] for i in idx]), _as_float(oz), tol, tol * 1e-2, "softmax rows")
+    # the same numbers laid out [16, 1024, 12, 1024] and seen through permute(0, 2, 1, 3): bit-identical result
+    if dt == FLOAT32:
+        P = NDArray.from_numpy(np.ascontiguousarray(logits.transpose(0, 2, 1, 3))).permute(0, 2, 1, 3)
+        zp = ex.exec_custom("softmax", [P], [NDArray.empty(shape, dt)])[0].to_float()
+        assert np.array_equal(zp, z)
+
+
+@pytest.mark.parametrize("dt", [HALF, BFLOAT16])
+def test_config4_causal_attention(ex, oracle, dt):
+    rng = np.random.default_rng(4004)
+    B, T, D = 96, 1024, 64
+    q, Q = _store(rng.normal(0, 1, (B, T, D)).astype(np.float32), dt)
+    k, K = _store(rng.normal(0, 1, (B, T, D)).astype(np.float32), dt)
+    v, V = _store(rng.normal(0, 1, (B, T, D)).astype(np.float32), dt)
+    out = ex.exec_custom("dot_product_attention_v2", [Q, V, K], [NDArray.empty((B, T, D), dt)], t_args=[0.125, 0.0], b_args=[True, False])[0].to_float()
+    assert np.isfinite(out).all()
+    # whole result: the first query sees one key, so its output is that value row; every output is a convex
+    # combination of the value rows it may see
+    assert_close(out[:, 0], v[:, 0], 1e-2, 1e-2, "query 0")
+    vmax, vmin = np.maximum.accumulate(v, axis=1), np.minimum.accumulate(v, axis=1)
+    assert np.all(out <= vmax + 2e-2) and np.all(out >= vmin - 2e-2)
+    # sampled batch entries against the oracle (the reference's unfused sequence on [1, T, D])
+    for bi in (0, 41, 95):
+        oo = _oracle_arr(oracle, np.zeros((1, T, D), np.float32), dt)
+        oracle.attention_v2(_oracle_arr(oracle, q[bi:bi + 1], dt), _oracle_arr(oracle, v[bi:bi + 1], dt), _oracle_arr(oracle, k[bi:bi + 1], dt), oo,
+                            scale=0.125, causal=True)
+        assert_close(out[bi:bi + 1], _as_float(oo), 1e-2, 1e-2, "batch entry %d" % bi)
