@@ -612,6 +612,47 @@ static std::vector<std::vector<LongType>> argShapeFn(Context& c) {
   return {makeShapeInfo(dt, 'c', out)};
 }
 
+static std::vector<LongType> hostIndexVector(NDArray* a, const char* what);
+// ---- reduce_* custom ops ----------------------------------------------------------------------------------------------------
+// generic/reduce/reduce_sum.cpp:33-61 and its siblings (reduce_max, reduce_min, reduce_prod, reduceMean.cpp, reduce_norm1,
+// reduce_norm2, reduce_norm_max, reduce_sqnorm, reduceVariance.cpp, reduceStDev.cpp): dims from IArgs or from a second
+// input, keepDims from BArg 0 (or TArg 0), no dims = reduce everything; variance / stdev take biasCorrected from BArg 1
+// (or TArg 1).  Thin wrappers over the kernels of the legacy reduce loops, as the reference's are over reduceAlongDimension.
+struct ReduceArgs { std::vector<LongType> dims; bool keepDims = false, biasCorrected = false; };
+static ReduceArgs reduceArgs(Context& c, const char* name) {
+  ReduceArgs r;
+  NDArray* x = c.input(0);
+  std::vector<LongType> raw = c.width() > 1 ? hostIndexVector(c.input(1), name) : c.iArgs;
+  ND4J_REQUIRE((int)raw.size() <= x->rankOf() || x->rankOf() == 0, std::string(name) + ": the number of dimensions to reduce along must be <= input array rank, but got " + std::to_string(raw.size()) + " instead");
+  for (auto d : raw)
+    ND4J_REQUIRE(d >= -x->rankOf() && d < x->rankOf(), std::string(name) + ": the input dimension to reduce along must be in range [-" + std::to_string(x->rankOf()) + ", " + std::to_string(x->rankOf()) + "), but got " + std::to_string(d) + " instead !");
+  r.dims = normalizeDims(x->rankOf(), raw.data(), (LongType)raw.size(), name);
+  if (!c.bArgs.empty()) { r.keepDims = c.bArgs[0]; if (c.bArgs.size() > 1) r.biasCorrected = c.bArgs[1]; }
+  else if (!c.tArgs.empty()) { r.keepDims = c.tArgs[0] != 0.0; if (c.tArgs.size() > 1) r.biasCorrected = c.tArgs[1] != 0.0; }
+  return r;
+}
+static void reduceCustomExec(Context& c, ReduceKind k, const char* name) {
+  ReduceArgs r = reduceArgs(c, name);
+  runReduce(name, k, c.input(0), c.output(0), r.dims);
+}
+static void reduceStatsExec(Context& c, MiscReduceKind k, const char* name) {
+  ReduceArgs r = reduceArgs(c, name);
+  ND4J_REQUIRE(c.output(0)->dataType() == c.input(0)->dataType() && isFloatType(c.input(0)->dataType()), std::string(name) + ": nd4j-hip requires a floating point input and an output of the same type");
+  runReduceMisc(name, k, c.input(0), c.output(0), r.dims, r.biasCorrected);
+}
+static std::vector<std::vector<LongType>> reduceCustomShapeFn(Context& c, const char* name) {
+  NDArray* x = c.input(0);
+  ReduceArgs r = reduceArgs(c, name);
+  std::vector<LongType> out;
+  for (int d = 0; d < x->rankOf(); d++) {
+    const bool red = r.dims.empty() || std::find(r.dims.begin(), r.dims.end(), (LongType)d) != r.dims.end();
+    if (!red) out.push_back(x->sizeAt(d));
+    else if (r.keepDims) out.push_back(1);
+  }
+  if (out.empty()) return {scalarShapeInfo(x->dataType())};
+  return {makeShapeInfo(x->dataType(), x->ordering(), out)};
+}
+
 // ---- glue ops for the decode step ----------------------------------------------------------------------------------------------
 // gather (generic/transforms/gather.cpp:34): rows of a dense 2-D table picked by an index array, axis 0
 static void gatherExec(Context& c) {
@@ -1268,6 +1309,18 @@ static void ensureRegistered() {
     reg("squeeze", 1, 1, false, 0, -2, [](Context& c) { sameDataExec(c, "squeeze"); }, squeezeShapeFn);
     reg("expand_dims", 1, 1, false, 0, -2, [](Context& c) { sameDataExec(c, "ExpandDims"); }, expandDimsShapeFn);
     reg("split", 1, -1, false, 0, 1, splitExec, splitShapeFn);
+    {
+      struct R { const char* name; ReduceKind k; const char* label; };
+      for (const R& r : {R{"reduce_sum", R_SUM, "REDUCE_SUM OP"}, R{"reduce_max", R_MAX, "REDUCE_MAX OP"}, R{"reduce_min", R_MIN, "REDUCE_MIN OP"},
+                         R{"reduce_prod", R_PROD, "REDUCE_PROD OP"}, R{"reduce_mean", R_MEAN, "REDUCE_MEAN OP"}, R{"reduce_norm1", R_NORM1, "REDUCE_NORM1 OP"},
+                         R{"reduce_norm2", R_NORM2, "REDUCE_NORM2 OP"}, R{"reduce_norm_max", R_NORMMAX, "REDUCE_NORM_MAX OP"},
+                         R{"reduce_sqnorm", R_SQNORM, "REDUCE_SQNORM OP"}}) {
+        const ReduceKind k = r.k; const char* label = r.label;
+        reg(r.name, -1, 1, false, 0, 0, [k, label](Context& c) { reduceCustomExec(c, k, label); }, [label](Context& c) { return reduceCustomShapeFn(c, label); });
+      }
+      reg("reduce_variance", -1, 1, false, 0, 0, [](Context& c) { reduceStatsExec(c, M_VARIANCE, "REDUCE_VARIANCE OP"); }, [](Context& c) { return reduceCustomShapeFn(c, "REDUCE_VARIANCE OP"); });
+      reg("reduce_stdev", -1, 1, false, 0, 0, [](Context& c) { reduceStatsExec(c, M_STDDEV, "REDUCE_STDEV OP"); }, [](Context& c) { return reduceCustomShapeFn(c, "REDUCE_STDEV OP"); });
+    }
     reg("softmax_bp", 3, 1, true, 0, 0, softmaxBpExec, sameAsInputShapeFn);
     reg("standardize", 1, 1, true, 0, -2, standardizeExec, sameAsInputShapeFn);
     reg("standardize_bp", 2, 1, false, 0, -2, standardizeBpExec, sameAsInputShapeFn);

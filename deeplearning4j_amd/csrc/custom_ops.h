@@ -4,6 +4,7 @@
 #include <string>
 #include <vector>
 
+#include "kernels.h"
 #include "runtime.h"
 
 namespace nd4jhip {
@@ -29,5 +30,8 @@ void executeOp(const OpDescriptor& op, Context& ctx);
 
 // shared with the legacy facade
 void runIndexReduce(const char* fn, int opNum, NDArray* x, NDArray* z, const std::vector<LongType>& dims);
+// value reductions and summary statistics behind both the legacy entry points and the reduce_* custom ops
+void runReduce(const char* fn, ReduceKind k, NDArray* x, NDArray* z, const std::vector<LongType>& dims);
+void runReduceMisc(const char* fn, MiscReduceKind k, NDArray* x, NDArray* z, std::vector<LongType> dims, bool biasCorrected);
 
 }  // namespace nd4jhip

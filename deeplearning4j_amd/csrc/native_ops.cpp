@@ -656,7 +656,9 @@ void execBroadcast(Nd4jPointer*, int opNum, OpaqueNDArray xa, OpaqueNDArray ya, 
   GUARD_END_VOID
 }
 
-static void runReduce(const char* fn, ReduceKind k, NDArray* x, NDArray* z, const std::vector<LongType>& dims) {
+}  // extern "C"
+namespace nd4jhip {
+void runReduce(const char* fn, ReduceKind k, NDArray* x, NDArray* z, const std::vector<LongType>& dims) {
   ND4J_REQUIRE(isFloatType(x->dataType()), std::string(fn) + ": non-float inputs are not implemented in nd4j-hip");
   ND4J_REQUIRE(x->dataType() == z->dataType(), std::string(fn) + ": nd4j-hip requires Z to have X's type, got " + dtypeName(x->dataType()) + " -> " + dtypeName(z->dataType()));
   ND4J_REQUIRE(!x->isEmpty(), std::string(fn) + ": reductions of empty arrays are not implemented in nd4j-hip");
@@ -676,6 +678,8 @@ static void runReduce(const char* fn, ReduceKind k, NDArray* x, NDArray* z, cons
   launchReduce(lc->execStream, k, x->dataType(), z->dataType(), x->specialBuffer(), z->specialBuffer(), p, lc->reductionBuffer, LaunchContext::REDUCTION_BYTES);
   registerSpecialUse({z}, {x});
 }
+}  // namespace nd4jhip
+extern "C" {
 static ReduceKind reduceSameKind(int opNum) {
   switch (opNum) {  // loops/legacy_ops.h:100-101
     case 0: return R_SUM; case 1: return R_MAX; case 2: return R_MIN; case 3: return R_PROD; case 4: return R_ASUM;
@@ -719,7 +723,9 @@ void execReduceFloat2(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueND
 }
 
 // reductions with their own accumulator / output types
-static void runReduceMisc(const char* fn, MiscReduceKind k, NDArray* x, NDArray* z, std::vector<LongType> d, bool biasCorrected) {
+}  // extern "C"
+namespace nd4jhip {
+void runReduceMisc(const char* fn, MiscReduceKind k, NDArray* x, NDArray* z, std::vector<LongType> d, bool biasCorrected) {
   ND4J_REQUIRE(!x->isEmpty(), std::string(fn) + ": reductions of empty arrays are not implemented in nd4j-hip");
   if (z->isEmpty()) return;
   if (z->lengthOf() == 1 && x->lengthOf() != 1) {
@@ -736,6 +742,8 @@ static void runReduceMisc(const char* fn, MiscReduceKind k, NDArray* x, NDArray*
                    lc->reductionBuffer, LaunchContext::REDUCTION_BYTES);
   registerSpecialUse({z}, {x});
 }
+}  // namespace nd4jhip
+extern "C" {
 // reduce3: z[o] = f(x tad o, y tad o) with y shaped like x (loops/cpu/reduce3.hpp); opNums loops/legacy_ops.h:88-90
 static void runReduce3(const char* fn, int opNum, NDArray* x, NDArray* y, NDArray* z, std::vector<LongType> d) {
   MiscReduceKind k;

@@ -567,3 +567,46 @@ def test_top_k_types_views_ties_and_errors(ex, oracle):
         ex.exec_custom("top_k", [NDArray.from_numpy(t)], [NDArray.empty((2, 6), FLOAT32), NDArray.empty((2, 6), INT64)], i_args=[6])
     with pytest.raises(NativeOpsError, match="k should be positive"):
         ex.exec_custom("top_k", [NDArray.from_numpy(t)], i_args=[0])
+
+# ---- reduce_* custom ops -----------------------------------------------------------------------------------------------------
+_REDUCE_OPS = [("reduce_sum", lambda x, ax, kd: x.sum(axis=ax, keepdims=kd)), ("reduce_max", lambda x, ax, kd: x.max(axis=ax, keepdims=kd)),
+               ("reduce_min", lambda x, ax, kd: x.min(axis=ax, keepdims=kd)), ("reduce_prod", lambda x, ax, kd: x.prod(axis=ax, keepdims=kd)),
+               ("reduce_mean", lambda x, ax, kd: x.mean(axis=ax, keepdims=kd)), ("reduce_norm1", lambda x, ax, kd: np.abs(x).sum(axis=ax, keepdims=kd)),
+               ("reduce_norm2", lambda x, ax, kd: np.sqrt((x * x).sum(axis=ax, keepdims=kd))),
+               ("reduce_norm_max", lambda x, ax, kd: np.abs(x).max(axis=ax, keepdims=kd)),
+               ("reduce_sqnorm", lambda x, ax, kd: (x * x).sum(axis=ax, keepdims=kd))]
+
+
+@pytest.mark.parametrize("name,ref", _REDUCE_OPS, ids=[n for n, _ in _REDUCE_OPS])
+@pytest.mark.parametrize("shape,dims,keep", [((6, 40), [1], False), ((6, 40), [0], True), ((3, 5, 7), [0, 2], False), ((3, 5, 7), [-1], True),
+                                             ((4, 9), [], False), ((33, 4096), [1], False)])
+def test_reduce_custom_ops(ex, oracle, name, ref, shape, dims, keep):
+    """generic/reduce/reduce_sum.cpp and siblings: dims from IArgs, keepDims from BArg 0, no dims = everything; the
+    same kernels as the legacy reduce loops (whose oracle is pinned), checked here against fp64 numpy."""
+    rng = np.random.default_rng(len(shape) + len(dims))
+    x = rng.uniform(0.8, 1.2, shape) * rng.choice([-1.0, 1.0], shape) if name == "reduce_prod" and np.prod(shape) < 300 else rng.uniform(-1, 1, shape)
+    if name == "reduce_prod":
+        x = np.where(np.abs(x) < 0.5, 1.0, x)      # keeps long products away from underflow
+    x = x.astype(np.float32)
+    ax = tuple(dims) if dims else None
+    want = ref(x.astype(np.float64), ax, keep)
+    out = ex.exec_custom(name, [NDArray.from_numpy(x)], i_args=dims, b_args=[keep])[0]
+    assert list(out.shape) == list(np.shape(want))
+    assert_close(out.to_numpy(), want, 1e-5, 1e-5 * max(1.0, float(np.abs(want).max())), name)
+    if dims:                                       # dims as a second input array give the same bits
+        axes = NDArray.from_numpy(np.array(dims, dtype=np.int32))
+        out2 = ex.exec_custom(name, [NDArray.from_numpy(x), axes], b_args=[keep])[0]
+        assert np.array_equal(out2.to_numpy(), out.to_numpy())
+
+
+@pytest.mark.parametrize("name,ddof_fn", [("reduce_variance", np.var), ("reduce_stdev", np.std)])
+def test_reduce_variance_and_stdev_custom_ops(ex, name, ddof_fn):
+    rng = np.random.default_rng(77)
+    x = rng.normal(3, 2, (5, 300)).astype(np.float32)
+    for keep, bias in ((False, False), (True, True)):
+        out = ex.exec_custom(name, [NDArray.from_numpy(x)], i_args=[1], b_args=[keep, bias])[0]
+        want = ddof_fn(x.astype(np.float64), axis=1, ddof=1 if bias else 0, keepdims=keep)
+        assert list(out.shape) == list(want.shape)
+        assert_close(out.to_numpy(), want, 1e-5, 1e-5, name)
+    with pytest.raises(NativeOpsError, match="must be in range"):
+        ex.exec_custom(name, [NDArray.from_numpy(x)], i_args=[2])
