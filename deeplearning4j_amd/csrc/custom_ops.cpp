@@ -653,6 +653,31 @@ static std::vector<std::vector<LongType>> reduceCustomShapeFn(Context& c, const 
   return {makeShapeInfo(x->dataType(), x->ordering(), out)};
 }
 
+// ---- activation custom ops -------------------------------------------------------------------------------------------------------
+// generic/nn/activations/{tanh,sigmoid,softplus,softsign,cube,hardsigmoid,hardtanh,rationaltanh,rectifiedtanh,selu,
+// identity}.cpp apply one legacy transform, {relu,relu6,lrelu,elu}.cpp one legacy scalar op whose scalar is TArg 0
+// (defaults: relu 0, lrelu 0.01, elu 1); the kernels are those of execTransformStrict / execTransformSame / execScalar.
+static void activationExec(Context& c, UnaryKind k, const char* name) {
+  NDArray* x = c.input(0); NDArray* z = c.output(0);
+  ND4J_REQUIRE(x->dataType() == z->dataType() && isFloatType(x->dataType()), std::string(name) + ": input and output must share a floating point type");
+  ND4J_REQUIRE(x->lengthOf() == z->lengthOf(), std::string(name) + ": input and output lengths differ");
+  if (x->isEmpty() || z->isEmpty()) return;
+  EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo()});
+  prepareSpecialUse({z}, {x});
+  launchUnary(stream(), k, x->dataType(), z->dataType(), x->specialBuffer(), z->specialBuffer(), p);
+  registerSpecialUse({z}, {x});
+}
+static void scalarActivationExec(Context& c, PairwiseKind k, double defaultScalar, const char* name) {
+  NDArray* x = c.input(0); NDArray* z = c.output(0);
+  ND4J_REQUIRE(x->dataType() == z->dataType() && isFloatType(x->dataType()), std::string(name) + ": input and output must share a floating point type");
+  if (x->isEmpty() || z->isEmpty()) return;
+  EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo()});
+  ND4J_REQUIRE(p.sameShape, std::string(name) + ": input and output must share a shape");
+  prepareSpecialUse({z}, {x});
+  launchScalarOp(stream(), k, x->dataType(), x->specialBuffer(), tArg(c, 0, defaultScalar), z->specialBuffer(), p);
+  registerSpecialUse({z}, {x});
+}
+
 // ---- glue ops for the decode step ----------------------------------------------------------------------------------------------
 // gather (generic/transforms/gather.cpp:34): rows of a dense 2-D table picked by an index array, axis 0
 static void gatherExec(Context& c) {
@@ -1320,6 +1345,19 @@ static void ensureRegistered() {
       }
       reg("reduce_variance", -1, 1, false, 0, 0, [](Context& c) { reduceStatsExec(c, M_VARIANCE, "REDUCE_VARIANCE OP"); }, [](Context& c) { return reduceCustomShapeFn(c, "REDUCE_VARIANCE OP"); });
       reg("reduce_stdev", -1, 1, false, 0, 0, [](Context& c) { reduceStatsExec(c, M_STDDEV, "REDUCE_STDEV OP"); }, [](Context& c) { return reduceCustomShapeFn(c, "REDUCE_STDEV OP"); });
+    }
+    {
+      struct U { const char* name; UnaryKind k; };
+      for (const U& u : {U{"tanh", U_TANH}, U{"sigmoid", U_SIGMOID}, U{"softplus", U_SOFTPLUS}, U{"softsign", U_SOFTSIGN}, U{"cube", U_CUBE},
+                         U{"hardsigmoid", U_HARD_SIGMOID}, U{"hardtanh", U_HARD_TANH}, U{"rationaltanh", U_RATIONAL_TANH},
+                         U{"rectifiedtanh", U_RECTIFIED_TANH}, U{"selu", U_SELU}, U{"identity", U_IDENTITY}}) {
+        const UnaryKind k = u.k; const char* name = u.name;
+        reg(u.name, 1, 1, true, 0, 0, [k, name](Context& c) { activationExec(c, k, name); }, sameAsInputShapeFn);
+      }
+      reg("relu", 1, 1, true, 1, 0, [](Context& c) { scalarActivationExec(c, P_RELU, 0.0, "relu"); }, sameAsInputShapeFn);
+      reg("relu6", 1, 1, true, 1, 0, [](Context& c) { scalarActivationExec(c, P_RELU6, 0.0, "relu6"); }, sameAsInputShapeFn);
+      reg("lrelu", 1, 1, true, -2, 0, [](Context& c) { scalarActivationExec(c, P_LEAKY_RELU, 0.01f, "lrelu"); }, sameAsInputShapeFn);
+      reg("elu", 1, 1, true, -2, 0, [](Context& c) { scalarActivationExec(c, P_ELU, 1.0, "elu"); }, sameAsInputShapeFn);
     }
     reg("softmax_bp", 3, 1, true, 0, 0, softmaxBpExec, sameAsInputShapeFn);
     reg("standardize", 1, 1, true, 0, -2, standardizeExec, sameAsInputShapeFn);

@@ -610,3 +610,36 @@ def test_reduce_variance_and_stdev_custom_ops(ex, name, ddof_fn):
         assert_close(out.to_numpy(), want, 1e-5, 1e-5, name)
     with pytest.raises(NativeOpsError, match="must be in range"):
         ex.exec_custom(name, [NDArray.from_numpy(x)], i_args=[2])
+
+# ---- activation custom ops ---------------------------------------------------------------------------------------------------
+def test_activation_custom_ops_match_their_legacy_ops(ex, oracle):
+    """generic/nn/activations/*.cpp are one legacy transform or scalar op each: the custom op must give the legacy op's
+    bits (same kernels), and the legacy ops are checked against the oracle elsewhere; tanh and relu also here."""
+    from deeplearning4j_amd.executioner import Scalar, TransformSame, TransformStrict
+    rng = np.random.default_rng(88)
+    x = rng.normal(0, 2, (37, 129)).astype(np.float32)
+    X = NDArray.from_numpy(x)
+    S, T = TransformStrict, TransformSame
+    for name, op in [("tanh", S.Tanh), ("sigmoid", S.Sigmoid), ("softplus", S.SoftPlus), ("softsign", S.SoftSign), ("hardsigmoid", S.HardSigmoid),
+                     ("hardtanh", S.HardTanh), ("rationaltanh", S.RationalTanh), ("rectifiedtanh", S.RectifiedTanh), ("selu", S.SELU)]:
+        got = ex.exec_custom(name, [X])[0].to_numpy()
+        assert np.array_equal(got, ex.exec_transform_strict(op, X).to_numpy()), name
+    assert np.array_equal(ex.exec_custom("cube", [X])[0].to_numpy(), ex.exec_transform_same(T.Cube, X).to_numpy())
+    assert np.array_equal(ex.exec_custom("identity", [X])[0].to_numpy(), x)
+    for name, op, targs, sc in [("relu", Scalar.RELU, [], 0.0), ("relu", Scalar.RELU, [0.5], 0.5), ("relu6", Scalar.RELU6, [0.0], 0.0),
+                                ("lrelu", Scalar.LeakyRELU, [], 0.01), ("lrelu", Scalar.LeakyRELU, [0.2], 0.2), ("elu", Scalar.ELU, [], 1.0),
+                                ("elu", Scalar.ELU, [0.7], 0.7)]:
+        got = ex.exec_custom(name, [X], t_args=targs)[0].to_numpy()
+        assert np.array_equal(got, ex.exec_scalar(op, X, np.float32(sc)).to_numpy()), (name, targs)
+    want = np.zeros_like(x)
+    oracle.transform_strict(S.Tanh, x, want)
+    assert_close(ex.exec_custom("tanh", [X])[0].to_numpy(), want, 1e-5, 1e-6, "tanh")
+    assert np.array_equal(ex.exec_custom("relu", [X])[0].to_numpy(), np.maximum(x, 0))
+    # in place, bf16, and a type error
+    B = NDArray.from_numpy(x, BFLOAT16)
+    ref = ex.exec_transform_strict(S.Sigmoid, B).to_numpy()
+    ex.exec_custom("sigmoid", [B], [B])
+    assert np.array_equal(B.to_numpy(), ref)
+    with pytest.raises(NativeOpsError, match="floating point type"):
+        ex.exec_custom("tanh", [X], [NDArray.empty(x.shape, BFLOAT16)])
+
