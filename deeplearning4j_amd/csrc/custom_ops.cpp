@@ -334,6 +334,30 @@ static std::vector<std::vector<LongType>> sameAsInputShapeFn(Context& c) {
   return {makeShapeInfo(x->dataType(), x->ordering(), shapeOf(x))};
 }
 
+// log_softmax (generic/nn/logSoftmax.cpp:34-49): IArg0 = dim (default last); a vector is normalised whole unless dim names
+// its unit axis, which gives zeros (helpers/cpu/activations.cpp:236-246)
+static void logSoftmaxExec(Context& c) {
+  NDArray* x = c.input(0);
+  NDArray* z = c.output(0);
+  const int rank = x->rankOf();
+  int dim = (int)iArg(c, 0, rank - 1);
+  ND4J_REQUIRE(dim < rank || rank == 0, "LOG_SOFTMAX OP: the value of input integer parameter (dimension) must be less than input array rank " + std::to_string(rank) + ", but got dimension = " + std::to_string(dim) + " instead !");
+  if (dim < 0) dim += rank;
+  ND4J_REQUIRE(rank == 0 || dim >= 0, "LOG_SOFTMAX OP: dimension out of range");
+  ND4J_REQUIRE(x->dataType() == z->dataType() && isFloatType(x->dataType()), "LOG_SOFTMAX OP: input and output must share a floating point type");
+  ND4J_REQUIRE(x->lengthOf() == z->lengthOf(), "LOG_SOFTMAX OP: input and output lengths differ");
+  if (x->isEmpty()) return;
+  prepareSpecialUse({z}, {x});
+  if (rank == 0 || (isVector(x) && rank != 1 && x->sizeAt(dim) == 1)) {
+    fillValue(z, 0.0);
+  } else {
+    if (isVector(x) && rank == 2) dim = x->sizeAt(0) == 1 ? 1 : 0;
+    RowPlan p = buildRowPlan(x->shapeInfo(), z->shapeInfo(), dim);
+    launchLogSoftmax(stream(), x->dataType(), x->specialBuffer(), z->specialBuffer(), p);
+  }
+  registerSpecialUse({z}, {x});
+}
+
 // statistics groups of a standardisation over `axes`: the reduced dims form the inner walk, the others the outer one;
 // dimC (or -1) is the axis gain and bias run along
 static LnGenericPlan lnGenericPlan(const NDArray* x, const NDArray* z, const std::vector<LongType>& axes, int dimC) {
@@ -1317,6 +1341,7 @@ static void ensureRegistered() {
     for (const char* alias : {"matmul", "mMul", "mmul", "gemm", "gemv", "dot"}) reg(alias, 2, 1, false, 0, -2, matmulExec, matmulShapeFn);
     reg("xw_plus_b", 3, 1, false, 0, 0, xwPlusBExec, xwPlusBShapeFn);
     reg("softmax", 1, 1, true, 0, 0, softmaxExec, sameAsInputShapeFn);
+    reg("log_softmax", 1, 1, true, 0, 0, logSoftmaxExec, sameAsInputShapeFn);
     reg("top_k", 1, 2, false, 0, -1, topKExec, topKShapeFn);
     reg("layer_norm", 2, 1, false, 0, -1, layerNormExec, sameAsInputShapeFn);
     reg("dot_product_attention_v2", -2, -1, false, -2, -2, attentionExec, attentionShapeFn);

@@ -109,6 +109,8 @@ struct RowPlan {
 };
 // clampMode: true = the reference's same-shape branch (finite max, +-88 clamp, sum floor 1e-6)
 void launchSoftmax(hipStream_t s, DataType dt, const void* x, void* z, const RowPlan& p, bool clampMode);
+// log(exp(x - max) / sum) along the plan's rows, evaluated in that order
+void launchLogSoftmax(hipStream_t s, DataType dt, const void* x, void* z, const RowPlan& p);
 void launchLayerNormRows(hipStream_t s, DataType dt, const void* x, const void* gain, const void* bias, void* z,
                          const RowPlan& p, float eps);
 // gradI = softmaxed * (gradO - sum_row(softmaxed * gradO)); pg = row plan (gradO, gradI), ps = (softmaxed, gradI)

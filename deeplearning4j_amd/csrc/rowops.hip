@@ -363,6 +363,43 @@ void launchSoftmax(hipStream_t s, DataType dt, const void* x, void* z, const Row
   HIP_CHECK(hipGetLastError());
 }
 
+// ---- log_softmax ---------------------------------------------------------------------------------------------------------------
+// generic/nn/logSoftmax.cpp:34-49 -> helpers/cpu/activations.cpp:100-145,236-256: max, exp(x - max), sum, divide, log, in
+// that order (a term whose exponential underflows comes out as -inf, as it does there).  One block per row, three passes;
+// rows and inner strides are arbitrary.  Not a tuned kernel.
+template <typename A> __device__ __forceinline__ A r_log(A x);
+template <> __device__ __forceinline__ float r_log<float>(float x) { return logf(x); }
+template <> __device__ __forceinline__ double r_log<double>(double x) { return log(x); }
+template <typename T>
+__global__ __launch_bounds__(256) void log_softmax_rows(RowArgs a, const T* __restrict__ x, T* __restrict__ z) {
+  using A = typename Conv<T>::acc;
+  __shared__ A lds[4];
+  const LongType row = blockIdx.x;
+  const LongType xb = walk<LongType>(a.outerX, row), zb = walk<LongType>(a.outerZ, row);
+  A mx = -r_tmax<A>();
+  for (LongType j = threadIdx.x; j < a.rowLen; j += 256) { const A v = (A)to_float(x[xb + j * a.xInner]); mx = v > mx ? v : mx; }
+  mx = block_allreduce<MaxOp, 4, A>(mx, lds);
+  A sum = (A)0;
+  for (LongType j = threadIdx.x; j < a.rowLen; j += 256) sum += r_exp<A>((A)to_float(x[xb + j * a.xInner]) - mx);
+  sum = block_allreduce<SumOp, 4, A>(sum, lds);
+  for (LongType j = threadIdx.x; j < a.rowLen; j += 256)
+    z[zb + j * a.zInner] = Conv<T>::from(r_log<A>(r_exp<A>((A)to_float(x[xb + j * a.xInner]) - mx) / sum));
+}
+void launchLogSoftmax(hipStream_t s, DataType dt, const void* x, void* z, const RowPlan& p) {
+  if (p.rows == 0 || p.rowLen == 0) return;
+  ND4J_REQUIRE(p.rows < (1LL << 31), "log_softmax: too many rows");
+  RowArgs a = rowArgs(p);
+  const dim3 g((unsigned)p.rows), b(256);
+  switch (dt) {
+    case FLOAT32: hipLaunchKernelGGL((log_softmax_rows<float>), g, b, 0, s, a, (const float*)x, (float*)z); break;
+    case DOUBLE: hipLaunchKernelGGL((log_softmax_rows<double>), g, b, 0, s, a, (const double*)x, (double*)z); break;
+    case HALF: hipLaunchKernelGGL((log_softmax_rows<f16_t>), g, b, 0, s, a, (const f16_t*)x, (f16_t*)z); break;
+    case BFLOAT16: hipLaunchKernelGGL((log_softmax_rows<bf16_t>), g, b, 0, s, a, (const bf16_t*)x, (bf16_t*)z); break;
+    default: ND4J_THROW("log_softmax: unsupported dtype");
+  }
+  HIP_CHECK(hipGetLastError());
+}
+
 // ---- layer_norm -------------------------------------------------------------------------------------------
 template <typename A> __device__ __forceinline__ A r_sqrt(A x);
 template <> __device__ __forceinline__ float r_sqrt<float>(float x) { return sqrtf(x); }

@@ -52,6 +52,7 @@
  *   matmul ............................ DeclarableOpsTests14.cpp:601-1260, DeclarableOpsTests19.cpp:52-140
  *   softmax ........................... DeclarableOpsTests1.cpp:2523-2740; inf/nan clamp
  *                                       semantics: parity unpinned (source only)
+ *   log_softmax (oracle.py, numpy) .... DeclarableOpsTests5.cpp:2199-2340 (tests/golden/log_softmax_vectors.json)
  *   layer_norm ........................ closed form (TestLayerOpValidation.java:1188-1333)
  *   dot_product_attention_v2 .......... parity unpinned: the reference has no enabled
  *                                       test; pinned only as matmul+softmax composition

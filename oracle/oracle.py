@@ -408,3 +408,23 @@ def matmul_bp(x, y, eps, trans_x=False, trans_y=False, trans_z=False, alpha=1.0,
     matmul(eps, y, dldx, bool(trans_z), not trans_y, bool(trans_x), alpha, beta)
     matmul(x, eps, dldy, not trans_x, bool(trans_z), bool(trans_y), alpha, beta)
     return dldx, dldy
+
+
+def log_softmax(x, dim=-1):
+    """log_softmax (generic/nn/logSoftmax.cpp:34-49 -> helpers/cpu/activations.cpp:100-145,236-256): max, exp(x - max), sum,
+    divide, log -- in that order, in the array type (so a term that underflows in exp comes out as -inf).  A vector
+    ([n], [1, n] or [n, 1]) is normalised whole unless `dim` names its unit axis, which gives zeros."""
+    x = np.asarray(x)
+    if dim < 0:
+        dim += max(x.ndim, 1)
+    is_vector = x.ndim == 1 or (x.ndim == 2 and 1 in x.shape)
+    with np.errstate(divide="ignore"):
+        if x.ndim == 0:
+            return np.zeros_like(x)
+        if is_vector:
+            if x.ndim == 1 or x.shape[dim] != 1:
+                e = np.exp(x - x.max())
+                return np.log(e / e.sum(dtype=x.dtype))
+            return np.zeros_like(x)
+        e = np.exp(x - x.max(axis=dim, keepdims=True))
+        return np.log(e / e.sum(axis=dim, keepdims=True, dtype=x.dtype))

@@ -643,3 +643,34 @@ def test_activation_custom_ops_match_their_legacy_ops(ex, oracle):
     with pytest.raises(NativeOpsError, match="floating point type"):
         ex.exec_custom("tanh", [X], [NDArray.empty(x.shape, BFLOAT16)])
 
+# ---- log_softmax -------------------------------------------------------------------------------------------------------------
+import json as _json
+import os as _os
+_LSM = _json.load(open(_os.path.join(_os.path.dirname(__file__), "golden", "log_softmax_vectors.json")))["cases"]
+
+
+@pytest.mark.parametrize("case", _LSM, ids=[c["name"].split()[-1] for c in _LSM])
+def test_log_softmax_reference_vectors(ex, case):
+    x = np.array(case["x"], np.float64).reshape(case["shape"])
+    z = ex.exec_custom("log_softmax", [NDArray.from_numpy(x)], i_args=case["iargs"])[0].to_numpy()
+    want = np.array(case["exp"], np.float64).reshape(case["shape"])
+    assert z.shape == want.shape and np.allclose(z, want, rtol=2e-5, atol=case.get("tol", 1e-5))
+
+
+@pytest.mark.parametrize("dtype,rtol,atol", [(FLOAT32, 1e-5, 1e-5), (DOUBLE, 1e-12, 1e-12), (BFLOAT16, 1e-2, 1e-2), (HALF, 1e-2, 1e-2)])
+@pytest.mark.parametrize("shape,dim", [((7, 300), 1), ((5, 6, 33), 1), ((4, 5000), -1), ((3000, 3), 0)])
+def test_log_softmax_vs_oracle(ex, oracle, dtype, rtol, atol, shape, dim):
+    rng = np.random.default_rng(shape[0] + shape[-1])
+    ox, dx = _pair(oracle, rng.normal(0, 2, shape), dtype)
+    wide = np.float64 if dtype == DOUBLE else np.float32
+    want = oracle.log_softmax(_f(ox).astype(wide), dim)
+    i_args = [] if dim == -1 else [dim]
+    z = ex.exec_custom("log_softmax", [dx], i_args=i_args)[0]
+    assert_close(z.to_float(), want, rtol, atol, "log_softmax %s dim %d" % (shape, dim))
+    # a term whose exponential underflows is -inf, as in the reference's exp / sum / log sequence
+    if dtype == FLOAT32 and dim != 0:
+        a = np.zeros(shape, np.float32)
+        a[..., 0] = -200.0
+        got = ex.exec_custom("log_softmax", [NDArray.from_numpy(a)])[0].to_numpy()
+        assert np.isneginf(got[..., 0]).all() and np.isfinite(got[..., 1:]).all()
+
