@@ -1353,6 +1353,17 @@ static void ensureRegistered() {
     reg("subtract", 2, 1, true, 0, 0, [](Context& c) { broadcastableExec(c, P_SUB, "SUBTRACT OP"); }, broadcastableShapeFn);
     reg("multiply", 2, 1, true, 0, 0, [](Context& c) { broadcastableExec(c, P_MUL, "MULTIPLY OP"); }, broadcastableShapeFn);
     reg("divide", 2, 1, true, 0, 0, [](Context& c) { broadcastableExec(c, P_DIV, "DIVIDE OP"); }, broadcastableShapeFn);
+    {
+      // the other members of generic/broadcastable/: each applies one legacy pairwise functor under broadcasting
+      struct B { const char* name; PairwiseKind k; };
+      for (const B& b : {B{"maximum", P_MAX}, B{"minimum", P_MIN}, B{"Pow", P_POW}, B{"realdiv", P_DIV}, B{"reversedivide", P_RDIV},
+                         B{"reversesubtract", P_RSUB}, B{"squaredsubtract", P_SQSUB}, B{"floordiv", P_FLOOR_DIV}, B{"floormod", P_FLOOR_MOD},
+                         B{"mod", P_MOD}, B{"reversemod", P_REVERSE_MOD}, B{"truncatediv", P_TRUNCATE_DIV}, B{"divide_no_nan", P_DIVIDE_NO_NAN},
+                         B{"tf_atan2", P_ATAN2}, B{"assign", P_COPY}}) {
+        const PairwiseKind k = b.k; const char* name = b.name;
+        reg(b.name, 2, 1, true, 0, 0, [k, name](Context& c) { broadcastableExec(c, k, name); }, broadcastableShapeFn);
+      }
+    }
     reg("permute", 1, 1, true, 0, -2, [](Context& c) { permuteExec(c, "PERMUTE OP"); }, [](Context& c) { return permuteShapeFn(c, "PERMUTE OP"); });
     reg("transpose", 1, 1, false, 0, 0, [](Context& c) { permuteExec(c, "TRANSPOSE OP"); }, [](Context& c) { return permuteShapeFn(c, "TRANSPOSE OP"); });
     reg("reshape", 1, 1, false, 0, -2, reshapeExec, reshapeShapeFn);

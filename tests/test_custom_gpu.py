@@ -674,3 +674,25 @@ def test_log_softmax_vs_oracle(ex, oracle, dtype, rtol, atol, shape, dim):
         got = ex.exec_custom("log_softmax", [NDArray.from_numpy(a)])[0].to_numpy()
         assert np.isneginf(got[..., 0]).all() and np.isfinite(got[..., 1:]).all()
 
+# ---- the rest of the broadcastable family --------------------------------------------------------------------------------------
+def test_broadcastable_custom_ops_match_their_legacy_pairwise_ops(ex):
+    """generic/broadcastable/*.cpp apply one legacy pairwise functor each under broadcasting: on equal shapes the custom op
+    must give the legacy op's bits; under broadcasting, what the same op gives on the materialised operand."""
+    from deeplearning4j_amd.executioner import Pairwise as P
+    rng = np.random.default_rng(99)
+    x = rng.uniform(0.5, 3, (6, 1, 33)).astype(np.float32) * rng.choice([-1, 1], (6, 1, 33)).astype(np.float32)
+    y = rng.uniform(0.5, 3, (5, 33)).astype(np.float32)
+    xb, yb = np.broadcast_to(x, (6, 5, 33)).copy(), np.broadcast_to(y, (6, 5, 33)).copy()
+    X, Y, XB, YB = (NDArray.from_numpy(a) for a in (x, y, xb, yb))
+    for name, op in [("maximum", P.MaxPairwise), ("minimum", P.MinPairwise), ("Pow", P.Pow), ("realdiv", P.Divide), ("reversedivide", P.ReverseDivide),
+                     ("reversesubtract", P.ReverseSubtract), ("squaredsubtract", P.SquaredSubtract), ("floordiv", P.FloorDiv),
+                     ("floormod", P.FloorMod), ("mod", P.Mod), ("reversemod", P.ReverseMod), ("truncatediv", P.TruncateDiv),
+                     ("divide_no_nan", P.DivideNoNan), ("tf_atan2", P.Atan2), ("assign", P.CopyPws)]:
+        want = ex.exec_pairwise(op, XB, YB).to_numpy()
+        got = ex.exec_custom(name, [X, Y])[0]
+        assert list(got.shape) == [6, 5, 33], name
+        assert np.array_equal(got.to_numpy(), want, equal_nan=True), name
+    assert np.array_equal(ex.exec_custom("maximum", [X, Y])[0].to_numpy(), np.maximum(xb, yb))
+    assert_close(ex.exec_custom("Pow", [NDArray.from_numpy(np.abs(x)), Y])[0].to_numpy(), np.abs(xb).astype(np.float64) ** yb, 1e-5, 1e-6, "Pow")
+    assert np.array_equal(ex.exec_custom("assign", [X, Y])[0].to_numpy(), yb)
+
