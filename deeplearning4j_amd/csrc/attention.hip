@@ -17,6 +17,7 @@
 //                   Bound: MFMA for the contractions, in practice the per-score VALU work (exp, max, convert).
 //   logits fix-up - in-place pass over dense [B, Tq, Tv] logits for the composition path that writes the
 //                   logits / weights outputs: optional scale, clip to +-1e4, causal penalty.
+#include <cmath>
 #include "device.h"
 #include "kernels.h"
 #include "mfma_tile.h"
@@ -69,13 +70,14 @@ template <typename T> __device__ __forceinline__ float round_storage(float v) { 
 // two floats -> one register of two storage values (first in the low half), with one packed conversion for bf16
 typedef __attribute__((ext_vector_type(2))) float f32x2a;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2a;
-template <typename T> __device__ __forceinline__ unsigned pack_pair(float a, float b);
-template <> __device__ __forceinline__ unsigned pack_pair<bf16_t>(float a, float b) {
+// (by reference: the caller goes on with the registers that pass through the asm, so no copies are made for it)
+template <typename T> __device__ __forceinline__ unsigned pack_pair(float& a, float& b);
+template <> __device__ __forceinline__ unsigned pack_pair<bf16_t>(float& a, float& b) {
   asm("" : "+v"(a), "+v"(b));   // keeps source modifiers out of the packed conversion (see Conv<bf16_t>::from)
   const f32x2a v = {a, b};
   return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2a));
 }
-template <> __device__ __forceinline__ unsigned pack_pair<f16_t>(float a, float b) {
+template <> __device__ __forceinline__ unsigned pack_pair<f16_t>(float& a, float& b) {
   return (unsigned)Conv<f16_t>::from(a).bits | ((unsigned)Conv<f16_t>::from(b).bits << 16);
 }
 // round two values through the storage type in place
@@ -90,7 +92,10 @@ template <typename T> __device__ __forceinline__ unsigned pack2(float a, float b
   return (unsigned)Conv<T>::from(a).bits | ((unsigned)Conv<T>::from(b).bits << 16);
 }
 
-template <typename T, int D>
+// FOLD: the scale is a power of two (or 1) and the scores are bf16, so scaling commutes exactly with the clip and with
+// the rounding through the storage type; the kernel then keeps unscaled scores and multiplies inside the exponent's
+// fused multiply-add (scale * log2(e) is exact too), which saves one multiply per score.
+template <typename T, int D, bool FOLD>
 __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
                                                   T* __restrict__ O) {
   constexpr int BQ = 128, BKV = 64, NT = 256;
@@ -123,8 +128,17 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
     Q += b * a.qB; K += b * a.kB; V += b * a.vB; O += b * a.oB;
   }
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, h = lane >> 5;
-  const float L2E = 1.44269502162933349609375f;
-  const float sc = a.applyScale ? a.scale : 1.f;
+  const float sc = a.scale;   // 1 when the op applies no scale
+  const float L2E = FOLD ? 1.44269502162933349609375f * sc : 1.44269502162933349609375f;
+  const float clip = FOLD ? 1.0e4f / sc : 1.0e4f;
+  // per-lane byte offsets of this thread's loads inside a key / value tile.  The tile's own address is the same for
+  // the whole wave, so a load is "scalar base + 32-bit lane offset" and costs no address arithmetic per tile.
+  const unsigned kTb = (unsigned)a.kT * 2u, vTb = (unsigned)a.vT * 2u;
+  const unsigned kRow = (unsigned)t >> 3, kCol = ((unsigned)t & 7u) * 16u;
+  const unsigned offK[2] = {kRow * kTb + kCol, (kRow + 32u) * kTb + kCol};
+  constexpr int VUNITS = D * 2;   // threads that carry a 4 x 8 block of the value tile
+  const unsigned vRb = ((unsigned)t >> 1) % (D / 8), vKey = (((unsigned)t / (D / 4)) * 2u + ((unsigned)t & 1u)) * 4u;
+  const unsigned offV = vKey * vTb + vRb * 16u;
   const bool paired = a.perBatch != a.qTiles;
   for (int pass = 0; pass < (paired ? 2 : 1); pass++) {
   const int qt = pass == 0 ? a.qTiles - 1 - slot : slot;
@@ -153,9 +167,35 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
   TileLoader<BKV, NT, true> lk[D / 64];   // rows = keys, contiguous along d
   TileLoader<D, NT, false> lv;            // rows = dv (contiguous in memory), "k" = keys
   auto loadKV = [&](LongType kv0) {
+    const char* kt = reinterpret_cast<const char*>(K + kv0 * a.kT);
+    const char* vt = reinterpret_cast<const char*>(V + kv0 * a.vT);
+    if (kv0 + BKV <= a.Tv) {
 #pragma unroll
-    for (int part = 0; part < D / 64; part++) lk[part].loadClamped(K + part * 64, a.kT, kv0, a.Tv, 0, 64, t);
-    lv.loadClamped(V, a.vT, 0, D, kv0, a.Tv, t);   // keys past the end repeat the last one: their weights are exactly 0
+      for (int part = 0; part < D / 64; part++)
+#pragma unroll
+        for (int i = 0; i < 2; i++) lk[part].reg[i] = *reinterpret_cast<const u32x4*>(kt + part * 128 + offK[i]);
+      if (t < VUNITS) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) lv.reg[q] = *reinterpret_cast<const u32x4*>(vt + (LongType)q * vTb + offV);
+      }
+    } else {
+      // the last, ragged tile: keys past the end repeat the last one (their weights are exactly 0)
+      const unsigned last = (unsigned)(a.Tv - 1 - kv0);
+#pragma unroll
+      for (int part = 0; part < D / 64; part++)
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+          const unsigned row = kRow + 32u * i < last ? kRow + 32u * i : last;
+          lk[part].reg[i] = *reinterpret_cast<const u32x4*>(kt + part * 128 + (row * kTb + kCol));
+        }
+      if (t < VUNITS) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const unsigned key = vKey + q < last ? vKey + q : last;
+          lv.reg[q] = *reinterpret_cast<const u32x4*>(vt + (key * vTb + vRb * 16u));
+        }
+      }
+    }
   };
   auto storeKV = [&](u32x4* dst) {
 #pragma unroll
@@ -202,9 +242,9 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
         float v0 = s[kt][r], v1 = s[kt][r + 1];
-        v0 *= sc; v1 *= sc;   // sc = 1 when no scale applies: one multiply instead of a multiply and a select
-        v0 = __builtin_amdgcn_fmed3f(v0, -1.0e4f, 1.0e4f);
-        v1 = __builtin_amdgcn_fmed3f(v1, -1.0e4f, 1.0e4f);
+        if (!FOLD) { v0 *= sc; v1 *= sc; }
+        v0 = __builtin_amdgcn_fmed3f(v0, -clip, clip);
+        v1 = __builtin_amdgcn_fmed3f(v1, -clip, clip);
         round_pair<T>(v0, v1);
         s[kt][r] = v0; s[kt][r + 1] = v1;
       }
@@ -239,10 +279,10 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
     for (int kt = 0; kt < 2; kt++)
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
-        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][r], L2E, -mL));
-        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][r + 1], L2E, -mL));
-        psum += p0 + p1;
+        float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][r], L2E, -mL));
+        float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][r + 1], L2E, -mL));
         pf[kt * 2 + r / 8][(r % 8) / 2] = pack_pair<T>(p0, p1);
+        psum += p0 + p1;
       }
     l = l * alpha + psum;
     // the accumulator only needs rescaling when some query's maximum moved
@@ -446,20 +486,22 @@ bool attentionFusedSupported(DataType dt, const AttnDesc& d) {
   // 16-byte aligned rows
   for (LongType st : {d.qB, d.qT, d.kB, d.kT, d.vB, d.vT, d.qB2, d.kB2, d.vB2}) if (st % 8 != 0) return false;
   if (d.oB % 4 != 0 || d.oT % 4 != 0 || d.oB2 % 4 != 0) return false;
+  // the tile loads address a key inside a tile with a 32-bit byte offset
+  if (d.kT < 0 || d.vT < 0 || d.kT >= (1 << 24) || d.vT >= (1 << 24)) return false;
   return true;
 }
 
-template <typename T, int D>
+template <typename T, int D, bool FOLD>
 static void launchFusedTyped(hipStream_t s, const void* q, const void* k, const void* v, void* out, const AttnDesc& d) {
   FusedArgs a;
   a.Tq = d.Tq; a.Tv = d.Tv;
   a.qB = d.qB; a.qT = d.qT; a.kB = d.kB; a.kT = d.kT; a.vB = d.vB; a.vT = d.vT; a.oB = d.oB; a.oT = d.oT;
   a.H = d.H; a.qB2 = d.qB2; a.kB2 = d.kB2; a.vB2 = d.vB2; a.oB2 = d.oB2;
-  a.scale = d.scale; a.applyScale = d.applyScale ? 1 : 0; a.causal = d.causal ? 1 : 0;
+  a.scale = d.applyScale ? (float)d.scale : 1.f; a.applyScale = d.applyScale ? 1 : 0; a.causal = d.causal ? 1 : 0;
   a.qTiles = (int)((d.Tq + 127) / 128);
   a.perBatch = d.causal ? (a.qTiles + 1) / 2 : a.qTiles;
   constexpr size_t LDS = (size_t)2 * ((D / 64) * TileLayout<64, true>::SLOTS + TileLayout<D, false>::SLOTS) * 16;
-  auto kern = attn_fused<T, D>;
+  auto kern = attn_fused<T, D, FOLD>;
   static bool attrSet = false;
   if (!attrSet) {
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS));
@@ -472,8 +514,16 @@ void launchAttentionFused(hipStream_t s, DataType dt, const void* q, const void*
   ND4J_REQUIRE(attentionFusedSupported(dt, d), "attention: fused kernel does not take this problem");
   ND4J_REQUIRE((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) == 0 && ((uintptr_t)out & 7) == 0, "attention: operands must be 16-byte aligned");
   ND4J_REQUIRE(((d.Tq + 127) / 128) * d.B < (1LL << 31), "attention: too many query tiles");
-  if (dt == HALF) { if (d.D == 64) launchFusedTyped<f16_t, 64>(s, q, k, v, out, d); else launchFusedTyped<f16_t, 128>(s, q, k, v, out, d); }
-  else { if (d.D == 64) launchFusedTyped<bf16_t, 64>(s, q, k, v, out, d); else launchFusedTyped<bf16_t, 128>(s, q, k, v, out, d); }
+  // scale folded into the exponent: no scale at all, or bf16 scores with a power-of-two scale of moderate size (the
+  // fp16 storage type has too narrow a range for rounding to commute with the scaling)
+  const float sc = d.applyScale ? (float)d.scale : 1.f;
+  int e = 0;
+  const bool pow2 = sc > 0.f && std::frexp(sc, &e) == 0.5f && e >= -19 && e <= 21;
+  const bool fold = sc == 1.f || (dt == BFLOAT16 && pow2);
+#define ND4J_FUSED(T, DD) (fold ? launchFusedTyped<T, DD, true>(s, q, k, v, out, d) : launchFusedTyped<T, DD, false>(s, q, k, v, out, d))
+  if (dt == HALF) { if (d.D == 64) ND4J_FUSED(f16_t, 64); else ND4J_FUSED(f16_t, 128); }
+  else { if (d.D == 64) ND4J_FUSED(bf16_t, 64); else ND4J_FUSED(bf16_t, 128); }
+#undef ND4J_FUSED
   HIP_CHECK(hipGetLastError());
 }
 
