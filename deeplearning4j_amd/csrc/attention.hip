@@ -17,6 +17,7 @@
 //                   Bound: MFMA for the contractions, in practice the per-score VALU work (exp, max, convert).
 //   logits fix-up - in-place pass over dense [B, Tq, Tv] logits for the composition path that writes the
 //                   logits / weights outputs: optional scale, clip to +-1e4, causal penalty.
+#include <algorithm>
 #include <cmath>
 #include "device.h"
 #include "kernels.h"
@@ -63,7 +64,7 @@ struct FusedArgs {
   LongType H, qB2, kB2, vB2, oB2;     // second batch level (H = 0: none)
   float scale;
   int applyScale, causal;
-  int qTiles, perBatch;
+  int qTiles, perBatch, nBatch, heavyFirst;   // fused kernel: work slots per batch entry, batch entries, block order
 };
 
 template <typename T> __device__ __forceinline__ float round_storage(float v) { return to_float(Conv<T>::from(v)); }
@@ -108,19 +109,27 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   u32x4* smem = reinterpret_cast<u32x4*>(smem_raw);   // two stages of (K tile, V tile)
 
-  // Consecutive block ids go to different XCDs (8 of them, round-robin).  Give every XCD a contiguous run of the
-  // (batch entry, query tile) sequence instead: the query tiles of one batch entry then share that XCD's L2 copy of
-  // K and V, and under the causal mask every XCD gets the same mix of heavy (late) and light (early) query tiles,
-  // heavy first.
-  unsigned item;
-  {
+  // Two block orders.
+  // Batch-major (a.heavyFirst == 0): consecutive block ids go to different XCDs (8 of them, round-robin), so every XCD
+  // gets a contiguous run of the (batch entry, work slot) sequence: the query tiles of one batch entry then share that
+  // XCD's L2 copy of K and V.  Under the causal mask a block takes a heavy (late) query tile and then its light mirror
+  // image, so that every block carries the same number of key tiles (a.perBatch = ceil(qTiles / 2) work slots per
+  // batch entry, else qTiles).  Equal blocks waste up to a whole round when they are few per CU.
+  // Heavy first (causal mask only; chosen by the host when it pays): block id = query tile (major, last tile first) x
+  // batch entry (minor), one query tile per block.  Blocks are handed out in id order as slots on the CUs free up, so
+  // the light tiles fill the gaps the heavy ones leave and the CUs finish close together.  With a multiple of 8 batch
+  // entries every query tile of an entry still lands on one XCD.
+  int slot;
+  LongType b;
+  if (a.heavyFirst) {
+    slot = (int)(blockIdx.x / (unsigned)a.nBatch);
+    b = blockIdx.x % (unsigned)a.nBatch;
+  } else {
     const unsigned total = gridDim.x, xcd = blockIdx.x & 7u, idx = blockIdx.x >> 3, per = total >> 3, rem = total & 7u;
-    item = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    const unsigned item = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    slot = (int)(item % a.perBatch);
+    b = item / a.perBatch;
   }
-  // under the causal mask a block takes a heavy query tile and then its light mirror image, so that every block
-  // carries the same number of key tiles (a.perBatch = ceil(qTiles / 2) work slots per batch entry, else qTiles)
-  const int slot = (int)(item % a.perBatch);
-  const LongType b = item / a.perBatch;
   if (a.H > 0) {
     const LongType hi = b / a.H, lo = b - hi * a.H;
     Q += hi * a.qB2 + lo * a.qB; K += hi * a.kB2 + lo * a.kB; V += hi * a.vB2 + lo * a.vB; O += hi * a.oB2 + lo * a.oB;
@@ -139,7 +148,7 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
   constexpr int VUNITS = D * 2;   // threads that carry a 4 x 8 block of the value tile
   const unsigned vRb = ((unsigned)t >> 1) % (D / 8), vKey = (((unsigned)t / (D / 4)) * 2u + ((unsigned)t & 1u)) * 4u;
   const unsigned offV = vKey * vTb + vRb * 16u;
-  const bool paired = a.perBatch != a.qTiles;
+  const bool paired = !a.heavyFirst && a.perBatch != a.qTiles;
   for (int pass = 0; pass < (paired ? 2 : 1); pass++) {
   const int qt = pass == 0 ? a.qTiles - 1 - slot : slot;
   if (pass == 1 && qt >= a.qTiles - 1 - slot) break;   // odd count: the middle tile has no mirror image
@@ -499,7 +508,20 @@ static void launchFusedTyped(hipStream_t s, const void* q, const void* k, const 
   a.H = d.H; a.qB2 = d.qB2; a.kB2 = d.kB2; a.vB2 = d.vB2; a.oB2 = d.oB2;
   a.scale = d.applyScale ? (float)d.scale : 1.f; a.applyScale = d.applyScale ? 1 : 0; a.causal = d.causal ? 1 : 0;
   a.qTiles = (int)((d.Tq + 127) / 128);
+  a.nBatch = (int)d.B;
   a.perBatch = d.causal ? (a.qTiles + 1) / 2 : a.qTiles;
+  a.heavyFirst = 0;
+  if (d.causal && a.qTiles > 1) {
+    // time in key tiles per slot (a CU holds two blocks at D = 64, one at D = 128): equal paired blocks run in whole
+    // rounds; single query tiles handed out heavy first finish within about a tenth of the mean, but not before the
+    // longest tile.  The batch-major order keeps K and V closer, so it stays unless the rounds waste more than 8 %.
+    const double slots = 256.0 * (D == 64 ? 2 : 1);
+    const double pairCost = 2.0 * (a.qTiles + 1), pairs = (double)d.B * a.perBatch;
+    const double pairedTime = std::ceil(pairs / slots) * pairCost;
+    const double total = (double)d.B * a.qTiles * (a.qTiles + 1);
+    const double heavyTime = std::max(1.1 * total / slots, 2.0 * a.qTiles);
+    a.heavyFirst = pairedTime > 1.08 * heavyTime ? 1 : 0;
+  }
   constexpr size_t LDS = (size_t)2 * ((D / 64) * TileLayout<64, true>::SLOTS + TileLayout<D, false>::SLOTS) * 16;
   auto kern = attn_fused<T, D, FOLD>;
   static bool attrSet = false;
@@ -507,7 +529,7 @@ static void launchFusedTyped(hipStream_t s, const void* q, const void* k, const 
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS));
     attrSet = true;
   }
-  hipLaunchKernelGGL(kern, dim3((unsigned)(a.perBatch * d.B)), dim3(256), LDS, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
+  hipLaunchKernelGGL(kern, dim3((unsigned)((LongType)(a.heavyFirst ? a.qTiles : a.perBatch) * d.B)), dim3(256), LDS, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
 }
 
 void launchAttentionFused(hipStream_t s, DataType dt, const void* q, const void* k, const void* v, void* out, const AttnDesc& d) {
