@@ -41,9 +41,18 @@ __device__ __forceinline__ double d_tanh(double x) {
   return (1.0 - p) / (1.0 + p);
 }
 
+// applyLow is what the contiguous kernel calls for 16-bit arrays: the same function where a cheaper evaluation only moves
+// the fp32 value by a few 1e-7 relative, far below half a unit of a bf16 / fp16 result (those launches are bound by
+// instruction issue, not by memory: twice the elements per byte).
 template <int K> struct Unary;
-#define UNARY(K, EXPR) \
-  template <> struct Unary<K> { template <typename A> static __device__ __forceinline__ A apply(A x) { return EXPR; } }
+#define UNARY_LOW(K, EXPR, LOWEXPR) \
+  template <> struct Unary<K> { \
+    template <typename A> static __device__ __forceinline__ A apply(A x) { return EXPR; } \
+    template <typename A> static __device__ __forceinline__ A applyLow(A x) { return LOWEXPR; } }
+#define UNARY(K, EXPR) UNARY_LOW(K, EXPR, EXPR)
+// 1 / (1 + e^-x) with the exponential as one v_exp_f32 of x * log2(e)
+__device__ __forceinline__ float d_sigmoid_low(float x) { return fast_rcp(1.f + __builtin_amdgcn_exp2f(x * -1.44269502162933349609375f)); }
+__device__ __forceinline__ double d_sigmoid_low(double x) { return 1.0 / (1.0 + exp(-x)); }
 __device__ __forceinline__ float d_cos(float x) { return cosf(x); }
 __device__ __forceinline__ double d_cos(double x) { return cos(x); }
 __device__ __forceinline__ float d_sin(float x) { return sinf(x); }
@@ -72,13 +81,13 @@ __device__ __forceinline__ double d_pgelu(double x) {
 UNARY(U_COS, d_cos(x));                                        // ops.h:194
 UNARY(U_EXP, d_exp<A>(x));                                     // ops.h:195
 UNARY(U_LOG, d_log(x));                                        // ops.h:197
-UNARY(U_SIGMOID, d_sigmoid<A>(x));                             // ops.h:200
+UNARY_LOW(U_SIGMOID, d_sigmoid<A>(x), d_sigmoid_low(x));       // ops.h:200
 UNARY(U_SIN, d_sin(x));                                        // ops.h:198
 UNARY(U_SOFTPLUS, d_log((A)1 + fast_exp(x)));                  // templatemath.h:272-274
 UNARY(U_TANH, d_tanh(x));                                      // ops.h:199
-UNARY(U_SWISH, x * d_sigmoid<A>(x));                           // ops.h:988-990
+UNARY_LOW(U_SWISH, x * d_sigmoid<A>(x), x * d_sigmoid_low(x)); // ops.h:988-990
 UNARY(U_ERF, d_erf(x));                                        // ops.h:361
-UNARY(U_GELU, x * d_sigmoid<A>((A)1.702f * x));                // ops.h:1010-1012
+UNARY_LOW(U_GELU, x * d_sigmoid<A>((A)1.702f * x), x * d_sigmoid_low((A)1.702f * x));   // ops.h:1010-1012
 UNARY(U_PRECISE_GELU, d_pgelu(x));
 UNARY(U_SQRT, d_sqrt(x));                                      // ops.h:2200
 UNARY(U_RSQRT, (A)1 / d_sqrt(x));                              // ops.h:2203-2205
@@ -310,7 +319,7 @@ __global__ __launch_bounds__(EW_BLOCK) void unary_contig(const T* __restrict__ x
     A vals[V];
     IO::unpack(r, vals);
 #pragma unroll
-    for (int e = 0; e < V; e++) vals[e] = F::template apply<A>(vals[e]);
+    for (int e = 0; e < V; e++) vals[e] = sizeof(T) == 2 ? F::template applyLow<A>(vals[e]) : F::template apply<A>(vals[e]);
     st_stream<NT>(reinterpret_cast<RT*>(z) + i, IO::pack(vals));
   }
   // scalar tail (fewer than V elements)
