@@ -702,6 +702,38 @@ static void scalarActivationExec(Context& c, PairwiseKind k, double defaultScala
   registerSpecialUse({z}, {x});
 }
 
+// clipbyvalue (generic/transforms/clip_by_value.cpp:33-83): bounds from TArgs, else from two scalar input arrays
+static void clipByValueExec(Context& c) {
+  NDArray* x = c.input(0); NDArray* z = c.output(0);
+  ND4J_REQUIRE(x->dataType() == z->dataType() && isFloatType(x->dataType()), "clip_by_value: input and output must share a floating point type");
+  double left, right;
+  if (!c.tArgs.empty()) {
+    ND4J_REQUIRE(c.tArgs.size() >= 2, "clip_by_value: two bounds are required");
+    left = c.tArgs[0]; right = c.tArgs[1];
+    char msg[160];
+    std::snprintf(msg, sizeof msg, "clip_by_value: left bound should be lesser than right. But %f >= %f given.", left, right);
+    ND4J_REQUIRE(left < right, msg);
+  } else {
+    ND4J_REQUIRE(c.width() >= 3, "clip_by_value: bounds come as two T arguments or as two scalar inputs");
+    NDArray* bounds[2] = {c.input(1), c.input(2)};
+    double v[2];
+    for (int i = 0; i < 2; i++) {
+      ND4J_REQUIRE(isFloatType(bounds[i]->dataType()) && bounds[i]->lengthOf() >= 1, "clip_by_value: a bound must be a floating point scalar");
+      bounds[i]->buf->syncToPrimary();
+      // the reference reads element 0 as the input's type
+      const double raw = hostValueAsDouble(bounds[i]->hostAs<unsigned char>(), bounds[i]->dataType());
+      v[i] = x->dataType() == DOUBLE ? raw : (double)(float)raw;
+    }
+    left = v[0]; right = v[1];
+  }
+  if (x->isEmpty() || z->isEmpty()) return;
+  EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo()});
+  ND4J_REQUIRE(p.sameShape, "clip_by_value: input and output must share a shape");
+  prepareSpecialUse({z}, {x});
+  launchScalar2Op(stream(), S2_CLIP_BY_VALUE, x->dataType(), z->dataType(), x->specialBuffer(), left, right, z->specialBuffer(), p);
+  registerSpecialUse({z}, {x});
+}
+
 // ---- glue ops for the decode step ----------------------------------------------------------------------------------------------
 // gather (generic/transforms/gather.cpp:34): rows of a dense 2-D table picked by an index array, axis 0
 static void gatherExec(Context& c) {
@@ -1395,6 +1427,7 @@ static void ensureRegistered() {
       reg("lrelu", 1, 1, true, -2, 0, [](Context& c) { scalarActivationExec(c, P_LEAKY_RELU, 0.01f, "lrelu"); }, sameAsInputShapeFn);
       reg("elu", 1, 1, true, -2, 0, [](Context& c) { scalarActivationExec(c, P_ELU, 1.0, "elu"); }, sameAsInputShapeFn);
     }
+    for (const char* alias : {"clipbyvalue", "ClipByValue"}) reg(alias, -2, 1, true, -2, 0, clipByValueExec, sameAsInputShapeFn);
     reg("softmax_bp", 3, 1, true, 0, 0, softmaxBpExec, sameAsInputShapeFn);
     reg("standardize", 1, 1, true, 0, -2, standardizeExec, sameAsInputShapeFn);
     reg("standardize_bp", 2, 1, false, 0, -2, standardizeBpExec, sameAsInputShapeFn);

@@ -457,6 +457,28 @@ __global__ __launch_bounds__(EW_BLOCK) void tail_generic(int k, DevShape sz, Dev
   }
 }
 
+// transforms with two parameters; any strides, any float dtypes.  The clip compares in double against the bounds as given
+// and stores the bound rounded to the output type (helpers/cpu/clip.cpp:211-219); the other two evaluate in the
+// accumulator type of the array (float for 16- and 32-bit arrays).
+__global__ __launch_bounds__(EW_BLOCK) void scalar2_generic(int k, DevShape sz, DevShape sx, int zdt, int xdt, void* z, const void* x,
+                                                            LongType n, double s1, double s2) {
+  const LongType step = (LongType)gridDim.x * EW_BLOCK;
+  for (LongType i = (LongType)blockIdx.x * EW_BLOCK + threadIdx.x; i < n; i += step) {
+    const LongType oz = walk<LongType>(sz, i), ox = walk<LongType>(sx, i);
+    const double a = load_any(x, xdt, ox);
+    double r;
+    if (k == S2_CLIP_BY_VALUE) {
+      r = a > s2 ? s2 : (a < s1 ? s1 : a);
+    } else if (xdt == DOUBLE) {
+      r = k == S2_AFFINE ? s1 * a + s2 : s1 * d_tanh(s2 * a);
+    } else {
+      const float fa = (float)a, f1 = (float)s1, f2 = (float)s2;
+      r = k == S2_AFFINE ? f1 * fa + f2 : f1 * d_tanh(f2 * fa);
+    }
+    store_any(z, zdt, oz, r);
+  }
+}
+
 // ---- launch helpers ------------------------------------------------------------------------------------
 static int gridFor(LongType work, int perBlock) {
   LongType blocks = (work + perBlock - 1) / perBlock;
@@ -725,6 +747,14 @@ void launchScalarOp(hipStream_t s, PairwiseKind k, DataType dt, const void* x, d
     case P_COPY: scalarKind<P_COPY>(s, dt, x, scalar, z, p); break;
     default: ND4J_THROW("scalar op: unsupported op");
   }
+  HIP_CHECK(hipGetLastError());
+}
+
+void launchScalar2Op(hipStream_t s, Scalar2Kind k, DataType xdt, DataType zdt, const void* x, double s1, double s2, void* z,
+                     const EwPlan& p) {
+  if (p.length == 0) return;
+  hipLaunchKernelGGL(scalar2_generic, dim3(gridFor(p.length, EW_BLOCK)), dim3(EW_BLOCK), 0, s, (int)k, p.own[0], p.own[1], (int)zdt,
+                     (int)xdt, z, x, p.length, s1, s2);
   HIP_CHECK(hipGetLastError());
 }
 

@@ -61,6 +61,14 @@ void launchPairwise(hipStream_t s, PairwiseKind k, DataType xdt, DataType ydt, D
 // z[outer.., c] = x[outer.., c] (op) v[c]: broadcast of a vector along the last axis of a dense array
 void launchRowBroadcast(hipStream_t s, PairwiseKind k, DataType dt, const void* x, const void* v, void* z,
                         LongType rows, LongType cols);
+// z = f(x; s1, s2): the transforms of the legacy tables that read two extra parameters
+enum Scalar2Kind : int {
+  S2_CLIP_BY_VALUE,   // x > s2 ? s2 : (x < s1 ? s1 : x)      ops.h:412-415, helpers/cpu/clip.cpp:211-219
+  S2_AFFINE,          // s1 * x + s2                          ops.h:453
+  S2_SCALED_TANH      // s1 * tanh(s2 * x)                    ops.h:1088-1090
+};
+void launchScalar2Op(hipStream_t s, Scalar2Kind k, DataType xdt, DataType zdt, const void* x, double s1, double s2, void* z,
+                     const EwPlan& p);
 // z = x (op) scalar
 void launchScalarOp(hipStream_t s, PairwiseKind k, DataType dt, const void* x, double scalar, void* z, const EwPlan& p);
 

@@ -448,12 +448,32 @@ static void runUnary(const char* fn, UnaryKind k, NDArray* x, NDArray* z) {
   registerSpecialUse({z}, {x});
 }
 
-void execTransformStrict(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
+// The transforms that read two extra parameters.  extraParams holds them in the array's own type (the executioner
+// converts its extraArgs to X before the call); it may be device or host memory, so they are fetched with a blocking copy.
+static void runUnaryWithParams(const char* fn, Scalar2Kind k, NDArray* x, NDArray* z, const void* extraParams) {
+  if (extraParams == nullptr) ND4J_THROW(std::string(fn) + ": this op needs two extra parameters");
+  if (x->isEmpty() || z->isEmpty()) return;
+  unsigned char raw[16];
+  const size_t w = sizeOf(x->dataType());
+  HIP_CHECK(hipStreamSynchronize(execStream()));
+  HIP_CHECK(hipMemcpy(raw, extraParams, 2 * w, hipMemcpyDefault));
+  const double s1 = hostValueAsDouble(raw, x->dataType()), s2 = hostValueAsDouble(raw + w, x->dataType());
+  EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo()});
+  prepareSpecialUse({z}, {x});
+  launchScalar2Op(execStream(), k, x->dataType(), z->dataType(), x->specialBuffer(), s1, s2, z->specialBuffer(), p);
+  registerSpecialUse({z}, {x});
+}
+
+void execTransformStrict(Nd4jPointer*, int opNum, OpaqueNDArray xa, void* extraParams, OpaqueNDArray za) {
   GUARD_BEGIN
   NDArray* x = arr(xa, "execTransformStrict", "x"); NDArray* z = arr(za, "execTransformStrict", "z");
   // X -> X over float types only (NativeOpExecutioner_transform.cpp:115-131)
   ND4J_REQUIRE(x->dataType() == z->dataType() && isFloatType(x->dataType()),
                std::string("NativeOpExecutioner::execTransformStrict requires X & Z to have same floating point type, got ") + dtypeName(x->dataType()) + " and " + dtypeName(z->dataType()));
+  if (opNum == 2 || opNum == 3) {   // ScaledTanh, Affine (loops/legacy_ops.h:54)
+    runUnaryWithParams("execTransformStrict", opNum == 2 ? S2_SCALED_TANH : S2_AFFINE, x, z, extraParams);
+    return;
+  }
   UnaryKind k;
   switch (opNum) {  // loops/legacy_ops.h:54-64
     case 22: k = U_COS; break; case 23: k = U_EXP; break; case 24: k = U_LOG; break; case 26: k = U_SIGMOID; break;
@@ -470,7 +490,7 @@ void execTransformStrict(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, Opaqu
     case 48: k = U_RINT; break; case 49: k = U_LOG_SIGMOID; break; case 50: k = U_ERFC; break; case 51: k = U_EXPM1; break;
     case 52: k = U_ATANH; break; case 54: k = U_GELU_D; break; case 56: k = U_PRECISE_GELU_D; break; case 57: k = U_MISH; break;
     case 58: k = U_MISH_D; break;
-    // 2 ScaledTanh, 3 Affine, 19 Stabilize, 25 SetRange read extra parameters; 5 HardTanhDerivative, 10 HardSigmoidDerivative and
+    // 19 Stabilize and 25 SetRange read extra parameters; 5 HardTanhDerivative, 10 HardSigmoidDerivative and
     // 20 StabilizeFP16 are not restated (their reference macros return the input unchanged / a platform constant)
     default: ND4J_THROW("execTransformStrict: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
@@ -490,18 +510,22 @@ void execTransformFloat(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, Opaque
   runUnary("execTransformFloat", k, x, z);
   GUARD_END_VOID
 }
-void execTransformSame(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
+void execTransformSame(Nd4jPointer*, int opNum, OpaqueNDArray xa, void* extraParams, OpaqueNDArray za) {
   GUARD_BEGIN
   NDArray* x = arr(xa, "execTransformSame", "x"); NDArray* z = arr(za, "execTransformSame", "z");
   ND4J_REQUIRE(x->dataType() == z->dataType(), "NativeOpExecutioner::execTransformSame requires X & Z to have same type");
   ND4J_REQUIRE(isFloatType(x->dataType()), "execTransformSame: non-float types are not implemented in nd4j-hip");
+  if (opNum == 19) {   // ClipByValue (loops/legacy_ops.h:43)
+    runUnaryWithParams("execTransformSame", S2_CLIP_BY_VALUE, x, z, extraParams);
+    return;
+  }
   UnaryKind k;
   switch (opNum) {  // loops/legacy_ops.h:40-44
     case 0: k = U_ABS; break; case 3: k = U_NEG; break; case 6: k = U_CUBE; break; case 7: k = U_ONE_MINUS; break;
     case 11: k = U_RECIPROCAL; break; case 12: k = U_SQUARE; break; case 15: case 21: k = U_IDENTITY; break;
     case 2: k = U_ONES; break; case 4: k = U_ROUND; break; case 5: k = U_TIMES_ONE_MINUS; break; case 17: k = U_CEIL; break;
     case 18: k = U_FLOOR; break;
-    // 13 CompareAndSetTransform and 19 ClipByValue read extra parameters; 1 Sign is not restated (the reference macro
+    // 13 CompareAndSetTransform reads extra parameters; 1 Sign is not restated (the reference macro
     // yields +1 for every non-zero input and -1 for zero)
     default: ND4J_THROW("execTransformSame: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }

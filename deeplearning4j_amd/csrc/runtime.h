@@ -4,6 +4,9 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <cmath>
+#include <cstdint>
+#include <cstring>
 #include <map>
 #include <memory>
 #include <mutex>
@@ -180,5 +183,21 @@ struct Environment {
   int maxThreads = 1;
   static Environment& get();
 };
+
+// one element of host memory, widened to double (float types only)
+inline double hostValueAsDouble(const void* p, DataType dt) {
+  switch (dt) {
+    case DOUBLE: return *static_cast<const double*>(p);
+    case FLOAT32: return *static_cast<const float*>(p);
+    case BFLOAT16: { const uint32_t b = (uint32_t)*static_cast<const uint16_t*>(p) << 16; float f; std::memcpy(&f, &b, 4); return f; }
+    case HALF: {
+      const uint16_t h = *static_cast<const uint16_t*>(p);
+      const int e = (h >> 10) & 31, m = h & 1023;
+      double v = e == 0 ? std::ldexp((double)m, -24) : e == 31 ? (m ? NAN : INFINITY) : std::ldexp((double)(m | 1024), e - 25);
+      return (h & 0x8000) ? -v : v;
+    }
+    default: ND4J_THROW("a floating point value is required here");
+  }
+}
 
 }  // namespace nd4jhip

@@ -174,9 +174,19 @@ class Executioner:
                 self._hashes[parts[0]] = int(parts[1])
 
     # ---- legacy ops ----
-    def exec_transform_strict(self, op_num, x, z=None):
+    def _extra_params(self, extra_args, dtype):
+        """extraArgs of a legacy op as the native side gets them: a buffer of the array's own type, device pointer
+        (the Java executioners convert with `op.extraArgsDataBuff(dtype)` and pass the allocator's pointer)."""
+        if extra_args is None:
+            return None, None
+        holder = NDArray.from_numpy(np.asarray(extra_args, np.float64 if dtype == DOUBLE else np.float32), dtype)
+        holder.sync_to_device()
+        return holder, self.L.dbSpecialBuffer(holder.buffer.ptr)
+
+    def exec_transform_strict(self, op_num, x, z=None, extra_args=None):
         z = z if z is not None else NDArray.empty(x.shape, x.dtype)
-        self.L.execTransformStrict(None, op_num, x.handle, None, z.handle)
+        holder, extra = self._extra_params(extra_args, x.dtype)
+        self.L.execTransformStrict(None, op_num, x.handle, extra, z.handle)
         N.check("execTransformStrict")
         return z
 
@@ -186,9 +196,10 @@ class Executioner:
         N.check("execTransformFloat")
         return z
 
-    def exec_transform_same(self, op_num, x, z=None):
+    def exec_transform_same(self, op_num, x, z=None, extra_args=None):
         z = z if z is not None else NDArray.empty(x.shape, x.dtype)
-        self.L.execTransformSame(None, op_num, x.handle, None, z.handle)
+        holder, extra = self._extra_params(extra_args, x.dtype)
+        self.L.execTransformSame(None, op_num, x.handle, extra, z.handle)
         N.check("execTransformSame")
         return z
 

@@ -410,6 +410,25 @@ def matmul_bp(x, y, eps, trans_x=False, trans_y=False, trans_z=False, alpha=1.0,
     return dldx, dldy
 
 
+def clip_by_value(x, left, right):
+    """clipbyvalue / legacy ClipByValue (helpers/cpu/clip.cpp:211-219, ops/ops.h:412-415): the upper bound is tested first,
+    comparisons against the bounds as given, NaN passes through."""
+    x = np.asarray(x)
+    return np.where(x > right, np.asarray(right, x.dtype), np.where(x < left, np.asarray(left, x.dtype), x)).astype(x.dtype)
+
+
+def affine(x, a, b):
+    """legacy Affine (ops/ops.h:453): a * x + b in the array type."""
+    x = np.asarray(x)
+    return (x.dtype.type(a) * x + x.dtype.type(b)).astype(x.dtype)
+
+
+def scaled_tanh(x, a, b):
+    """legacy ScaledTanh (ops/ops.h:1088-1090): a * tanh(b * x) in the array type."""
+    x = np.asarray(x)
+    return (x.dtype.type(a) * np.tanh(x.dtype.type(b) * x)).astype(x.dtype)
+
+
 def log_softmax(x, dim=-1):
     """log_softmax (generic/nn/logSoftmax.cpp:34-49 -> helpers/cpu/activations.cpp:100-145,236-256): max, exp(x - max), sum,
     divide, log -- in that order, in the array type (so a term that underflows in exp comes out as -inf).  A vector

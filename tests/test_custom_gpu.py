@@ -696,3 +696,50 @@ def test_broadcastable_custom_ops_match_their_legacy_pairwise_ops(ex):
     assert_close(ex.exec_custom("Pow", [NDArray.from_numpy(np.abs(x)), Y])[0].to_numpy(), np.abs(xb).astype(np.float64) ** yb, 1e-5, 1e-6, "Pow")
     assert np.array_equal(ex.exec_custom("assign", [X, Y])[0].to_numpy(), yb)
 
+
+
+# ---- two-parameter transforms ---------------------------------------------------------------------------------------------
+def test_clipbyvalue_reference_vector_and_bounds_as_inputs(ex):
+    """DeclarableOpsTests1.cpp:801-848: bounds as T arguments (ClipByValue1) and as two scalar inputs (ClipByValue2)."""
+    x = np.full((5, 5), 4.0, np.float32)
+    x.flat[0], x.flat[1] = -1.0, 2.0
+    exp = np.full((5, 5), 3.0, np.float32)
+    exp.flat[0], exp.flat[1] = 0.0, 2.0
+    z = ex.exec_custom("clipbyvalue", [NDArray.from_numpy(x)], t_args=[0.0, 3.0])[0]
+    assert np.array_equal(z.to_numpy(), exp)
+    lo, hi = NDArray.from_numpy(np.zeros((1, 1), np.float32)), NDArray.from_numpy(np.full((1, 1), 3.0, np.float32))
+    X = NDArray.from_numpy(x)
+    ex.exec_custom("ClipByValue", [X, lo, hi], [X])      # in place, through the alias
+    assert np.array_equal(X.to_numpy(), exp)
+    with pytest.raises(NativeOpsError, match="left bound should be lesser than right"):
+        ex.exec_custom("clipbyvalue", [NDArray.from_numpy(x)], t_args=[3.0, 0.0])
+
+
+@pytest.mark.parametrize("dtype", [FLOAT32, DOUBLE, HALF, BFLOAT16])
+def test_two_parameter_transforms_match_oracle(ex, oracle, dtype):
+    """clipbyvalue and the legacy ClipByValue / Affine / ScaledTanh (extra parameters in device memory, array type)."""
+    from oracle import oracle as onp
+    rng = np.random.default_rng(77)
+    x = rng.normal(0, 2, (6, 5, 33)).astype(np.float32)
+    x[0, 0, :3] = [np.nan, np.inf, -np.inf]
+    ox, dx = _pair(oracle, x, dtype)
+    xr = _f(ox).astype(np.float64 if dtype == DOUBLE else np.float32)   # the values the device holds
+    tol = {FLOAT32: 1e-5, DOUBLE: 1e-12, HALF: 1e-2, BFLOAT16: 1e-2}[dtype]
+    view = dx.permute(2, 0, 1)                                           # strided input, dense output
+    for lo, hi in [(-1.25, 0.5), (0.0, 3.0)]:
+        want = onp.clip_by_value(xr, lo, hi)
+        got = ex.exec_custom("clipbyvalue", [dx], t_args=[lo, hi])[0].to_float()
+        assert np.array_equal(got, want, equal_nan=True), "clipbyvalue is exact"
+        got = ex.exec_transform_same(19, dx, extra_args=[lo, hi]).to_float()
+        assert np.array_equal(got, want, equal_nan=True), "legacy ClipByValue is exact"
+        got = ex.exec_transform_same(19, view, extra_args=[lo, hi]).to_float()
+        assert np.array_equal(got, want.transpose(2, 0, 1), equal_nan=True), "legacy ClipByValue, permuted view"
+    fin = np.isfinite(xr)
+    got = ex.exec_transform_strict(3, dx, extra_args=[2.5, -0.75]).to_float()
+    assert_close(got[fin], onp.affine(xr.astype(np.float64), 2.5, -0.75)[fin], tol, tol, "Affine")
+    got = ex.exec_transform_strict(2, dx, extra_args=[1.7159, 0.6666]).to_float()
+    # the parameters reach the kernel rounded to the array type
+    a, b = (np.asarray(v, np.float64) for v in (1.7159, 0.6666))
+    assert_close(got[fin], onp.scaled_tanh(xr.astype(np.float64), a, b)[fin], tol * 4, tol * 4, "ScaledTanh")
+    with pytest.raises(NativeOpsError, match="needs two extra parameters"):
+        ex.exec_transform_same(19, dx)
