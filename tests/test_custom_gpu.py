@@ -743,3 +743,38 @@ def test_two_parameter_transforms_match_oracle(ex, oracle, dtype):
     assert_close(got[fin], onp.scaled_tanh(xr.astype(np.float64), a, b)[fin], tol * 4, tol * 4, "ScaledTanh")
     with pytest.raises(NativeOpsError, match="needs two extra parameters"):
         ex.exec_transform_same(19, dx)
+
+
+# ---- broadcastable ops: the reference's own vectors ------------------------------------------------------------------------
+_BC = _json.load(open(_os.path.join(_os.path.dirname(__file__), "golden", "broadcastable_vectors.json")))
+
+
+def _bc_array(shape, values, np_dt):
+    if isinstance(values, dict):
+        return np.full(shape, values["fill"], np_dt)
+    return np.array(values, np_dt).reshape(shape)
+
+
+@pytest.mark.parametrize("case", _BC["cases"], ids=[c["name"].split()[-1] for c in _BC["cases"]])
+def test_broadcastable_reference_vectors(ex, case):
+    """BroadcastableOpsTests.cpp: row / column / scalar / rank-extending broadcasts, empty operands, caller-supplied outputs."""
+    np_dt, dt = (np.float64, DOUBLE) if case["dtype"] == "double" else (np.float32, FLOAT32)
+    x = NDArray.from_numpy(_bc_array(case["x_shape"], case["x"], np_dt))
+    y = NDArray.from_numpy(_bc_array(case["y_shape"], case["y"], np_dt))
+    exp = _bc_array(case["exp_shape"], case["exp"], np_dt)
+    got = ex.exec_custom(case["op"], [x, y])[0]                       # output sized by the op's shape function
+    assert list(got.shape) == case["exp_shape"]
+    if exp.size:
+        assert np.array_equal(got.to_numpy(), exp)
+    z = NDArray.from_numpy(np.full(case["exp_shape"], 119, np_dt))     # output supplied by the caller
+    ex.exec_custom(case["op"], [x, y], [z])
+    if exp.size:
+        assert np.array_equal(z.to_numpy(), exp)
+
+
+@pytest.mark.parametrize("case", _BC["shape_cases"], ids=[c["name"].split()[-1] for c in _BC["shape_cases"]])
+def test_broadcastable_reference_shape_function(ex, case):
+    x, y = NDArray.empty(case["x_shape"], FLOAT32), NDArray.empty(case["y_shape"], FLOAT32)
+    shapes = ex.calculate_output_shapes(_BC["shape_op"], [x, y])
+    si = shapes[0]
+    assert [int(s) for s in si[1:1 + int(si[0])]] == case["exp_shape"]
