@@ -1066,6 +1066,105 @@ static std::vector<std::vector<LongType>> splitShapeFn(Context& c) {
   return out;
 }
 
+// unstack (generic/transforms/unstack.cpp:32-108): one output per index along IArg0, each the input with that axis removed
+// (a vector falls apart into scalars)
+static std::vector<LongType> unstackShape(NDArray* x, LongType dim) {
+  std::vector<LongType> shp;
+  for (int d = 0; d < x->rankOf(); d++) if (d != dim) shp.push_back(x->sizeAt(d));
+  return shp;
+}
+static LongType unstackDim(Context& c, NDArray* x) {
+  ND4J_REQUIRE(!c.iArgs.empty(), "Unstack: the dimension is required as the first integer argument");
+  LongType dim = c.iArgs[0];
+  if (dim < 0) dim += x->rankOf();
+  ND4J_REQUIRE(dim < x->rankOf(), "Unstack dimension should be lower then rank of input " + std::to_string(x->rankOf()) + ", but got dimension=" + std::to_string(dim) + " !");
+  ND4J_REQUIRE(dim >= 0, "Unstack dimension should be non-negative value, but got " + std::to_string(dim) + " !");
+  return dim;
+}
+static void unstackExec(Context& c) {
+  NDArray* x = c.input(0);
+  if (x->isEmpty()) return;
+  const LongType dim = unstackDim(c, x);
+  const LongType n = x->sizeAt((int)dim);
+  ND4J_REQUIRE((LongType)c.outputs.size() >= n, "Unstack: " + std::to_string(n) + " output arrays are required");
+  std::vector<LongType> shp, st;
+  for (int d = 0; d < x->rankOf(); d++) if (d != dim) { shp.push_back(x->sizeAt(d)); st.push_back(x->strideAt(d)); }
+  for (LongType i = 0; i < n; i++) assignEnumerated(c.output((int)i), x, i * x->strideAt((int)dim), shp, st, 'c', "Unstack");
+}
+static std::vector<std::vector<LongType>> unstackShapeFn(Context& c) {
+  NDArray* x = c.input(0);
+  const LongType dim = unstackDim(c, x);
+  const LongType n = c.iArgs.size() > 1 ? c.iArgs[1] : x->sizeAt((int)dim);
+  std::vector<LongType> shp = unstackShape(x, dim);
+  std::vector<std::vector<LongType>> out;
+  for (LongType i = 0; i < n; i++) out.push_back(shp.empty() ? scalarShapeInfo(x->dataType()) : makeShapeInfo(x->dataType(), x->ordering(), shp));
+  return out;
+}
+
+// stack (generic/transforms/stack.cpp:31-92; aliases pack, Pack): equal-shaped inputs side by side along a new axis IArg0
+static LongType stackDim(Context& c, NDArray* first) {
+  LongType dim = iArg(c, 0, 0);
+  if (dim < 0) dim += first->rankOf() + 1;
+  ND4J_REQUIRE(dim >= 0 && dim <= first->rankOf(), "STACK op: the input dimension parameter must be <= rank of input arrays shapes (rank=" +
+               std::to_string(first->rankOf()) + "), but got " + std::to_string(dim) + " instead !");
+  return dim;
+}
+static void stackExec(Context& c) {
+  NDArray* first = c.input(0); NDArray* z = c.output(0);
+  const LongType dim = stackDim(c, first);
+  if (z->isEmpty()) return;
+  const int n = c.width();
+  for (int i = 0; i + 1 < n; i++)
+    ND4J_REQUIRE(shapeOf(c.input(i)) == shapeOf(c.input(i + 1)), "STACK op: the shapes of all input arrays must be the same !");
+  if (first->isEmpty()) return;
+  ND4J_REQUIRE(z->rankOf() == first->rankOf() + 1 && z->sizeAt((int)dim) == n && z->dataType() == first->dataType(), "STACK op: wrong output array");
+  std::vector<LongType> shp = shapeOf(first), zst;
+  for (int d = 0; d < z->rankOf(); d++) if (d != dim) zst.push_back(z->strideAt(d));
+  std::vector<NDArray*> reads;
+  for (int i = 0; i < n; i++) reads.push_back(c.input(i));
+  prepareSpecialUse(std::vector<NDArray*>{z}, reads);
+  for (int i = 0; i < n; i++) {
+    NDArray* a = c.input(i);
+    std::vector<LongType> vshape = shp, vstride = zst;
+    if (vshape.empty()) { vshape = {1}; vstride = {1}; }
+    auto vsi = makeShapeInfo(z->dataType(), 'c', vshape, vstride.data());
+    std::vector<LongType> ashape = shapeOf(a), astride = stridesOf(a);
+    if (ashape.empty()) { ashape = {1}; astride = {1}; }
+    auto asi = makeShapeInfo(a->dataType(), 'c', ashape, astride.data());
+    EwPlan p = buildEwPlan({vsi.data(), asi.data()});
+    char* dst = (char*)z->specialBuffer() + (size_t)(i * z->strideAt((int)dim)) * sizeOf(z->dataType());
+    launchUnary(stream(), U_IDENTITY, a->dataType(), z->dataType(), a->specialBuffer(), dst, p);
+  }
+  registerSpecialUse(std::vector<NDArray*>{z}, reads);
+}
+static std::vector<std::vector<LongType>> stackShapeFn(Context& c) {
+  NDArray* first = c.input(0);
+  const LongType dim = stackDim(c, first);
+  std::vector<LongType> out = shapeOf(first);
+  out.insert(out.begin() + dim, (LongType)c.width());
+  return {makeShapeInfo(first->dataType(), first->ordering(), out)};
+}
+
+// cast (generic/datatypes/cast.cpp:30-86; alias Cast): assignment into an array of the type named by DArg0 or IArg0
+static void castExec(Context& c) {
+  NDArray* x = c.input(0); NDArray* z = c.output(0);
+  if (x->isEmpty()) { ND4J_REQUIRE(z->isEmpty(), "If input is empty, output array must also be empty"); return; }
+  if (z == x) return;
+  ND4J_REQUIRE(z->lengthOf() == x->lengthOf(), "cast: output must have the input's length");
+  EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo()});
+  prepareSpecialUse({z}, {x});
+  launchUnary(stream(), U_IDENTITY, x->dataType(), z->dataType(), x->specialBuffer(), z->specialBuffer(), p);
+  registerSpecialUse({z}, {x});
+}
+static std::vector<std::vector<LongType>> castShapeFn(Context& c) {
+  NDArray* x = c.input(0);
+  DataType dt;
+  if (!c.dArgs.empty()) dt = c.dArgs[0];
+  else { ND4J_REQUIRE(!c.iArgs.empty(), "cast: the new data type is required as a D or I argument"); dt = (DataType)c.iArgs[0]; }
+  ND4J_REQUIRE(sizeOf(dt) > 0, "cast: new data type " + std::to_string((int)dt) + " is not supported by nd4j-hip");
+  return {makeShapeInfo(dt, x->ordering(), shapeOf(x))};
+}
+
 // strided_slice (generic/tensor/strided_slice.cpp:135-370,372-530): IArgs = begin_mask, ellipsis_mask, end_mask, new_axis_mask,
 // shrink_axis_mask [, begin.., end.., strides..]; or begin/end/strides as inputs 1..3.  The sparse specification (one entry per
 // written index) is spread over the input's axes, every axis gets a canonical [begin, end) and a step, and the output is the
@@ -1433,6 +1532,9 @@ static void ensureRegistered() {
     reg("standardize_bp", 2, 1, false, 0, -2, standardizeBpExec, sameAsInputShapeFn);
     reg("layer_norm_bp", 3, -1, false, 0, -1, layerNormBpExec, layerNormBpShapeFn);
     reg("matmul_bp", 3, 2, false, 0, -2, matmulBpExec, matmulBpShapeFn);
+    for (const char* alias : {"cast", "Cast"}) reg(alias, 1, 1, false, 0, -2, castExec, castShapeFn);
+    for (const char* alias : {"stack", "pack", "Pack"}) reg(alias, -1, 1, false, 0, 0, stackExec, stackShapeFn);
+    for (const char* alias : {"unstack", "unpack"}) reg(alias, 1, -1, false, 0, 1, unstackExec, unstackShapeFn);
     for (const char* alias : {"strided_slice", "stridedslice"}) reg(alias, 1, 1, false, 0, 5, stridedSliceExec, stridedSliceShapeFn);
   });
 }

@@ -778,3 +778,75 @@ def test_broadcastable_reference_shape_function(ex, case):
     shapes = ex.calculate_output_shapes(_BC["shape_op"], [x, y])
     si = shapes[0]
     assert [int(s) for s in si[1:1 + int(si[0])]] == case["exp_shape"]
+
+
+# ---- cast, stack, unstack ----------------------------------------------------------------------------------------------------
+def test_cast_reference_cases(ex):
+    """DeclarableOpsTests1.cpp:1543-1556 (5x5 linspace float -> half via IArg 3), DeclarableOpsTests16.cpp:158-166 (empty bool ->
+    int64 via IArg 10); the D argument names the type as well."""
+    x = np.arange(1, 26, dtype=np.float32).reshape(5, 5)
+    z = ex.exec_custom("cast", [NDArray.from_numpy(x)], i_args=[3])[0]
+    assert z.dtype == HALF and np.array_equal(z.to_numpy(), x.astype(np.float16))
+    from deeplearning4j_amd.ndarray import BOOL
+    e = ex.exec_custom("cast", [NDArray.empty((1, 0, 2), BOOL)], i_args=[10])[0]
+    assert e.dtype == INT64 and list(e.shape) == [1, 0, 2]
+    rng = np.random.default_rng(3)
+    v = (rng.normal(0, 40, (7, 9)).astype(np.float32))
+    for dt, npdt in [(DOUBLE, np.float64), (INT32, np.int32), (INT64, np.int64), (HALF, np.float16)]:
+        got = ex.exec_custom("Cast", [NDArray.from_numpy(v)], d_args=[dt])[0]
+        assert got.dtype == dt and np.array_equal(got.to_numpy(), v.astype(npdt)), dt     # numpy truncates toward zero as C++ does
+    b = ex.exec_custom("cast", [NDArray.from_numpy(v)], d_args=[BFLOAT16])[0]
+    assert np.array_equal(b.to_numpy(), f32_to_bf16_bits(v))
+    back = ex.exec_custom("cast", [NDArray.from_numpy(v.astype(np.int32))], d_args=[FLOAT32])[0]
+    assert np.array_equal(back.to_numpy(), v.astype(np.int32).astype(np.float32))
+
+
+def test_stack_reference_vectors(ex):
+    """DeclarableOpsTests14.cpp:1728-1800 (Stack_1..3), :1935-1955 (Stack_11), :2113-2135 (Stack_21: stack == reshaped concat)."""
+    a = np.arange(1, 13, dtype=np.float32).reshape(3, 4)
+    b = np.array([13, 14, 16, 16, 17, 18, 19, 20, 21, 22, 23, 24], np.float32).reshape(3, 4)
+    A, B = NDArray.from_numpy(a), NDArray.from_numpy(b)
+    z = ex.exec_custom("stack", [A, B], i_args=[0])[0]
+    assert list(z.shape) == [2, 3, 4] and np.array_equal(z.to_numpy().ravel(), np.concatenate([a.ravel(), b.ravel()]))
+    z = ex.exec_custom("stack", [A, B], i_args=[1])[0]
+    exp = np.array([1, 2, 3, 4, 13, 14, 16, 16, 5, 6, 7, 8, 17, 18, 19, 20, 9, 10, 11, 12, 21, 22, 23, 24], np.float32).reshape(3, 2, 4)
+    assert list(z.shape) == [3, 2, 4] and np.array_equal(z.to_numpy(), exp)
+    z = ex.exec_custom("pack", [NDArray.from_numpy(a.reshape(1, 12)), NDArray.from_numpy(b.reshape(1, 12))], i_args=[0])[0]
+    assert list(z.shape) == [2, 1, 12] and np.array_equal(z.to_numpy().ravel(), np.concatenate([a.ravel(), b.ravel()]))
+    one = NDArray.from_numpy(np.array([1.0], np.float32))
+    z = ex.exec_custom("stack", [one, one, one])[0]
+    assert list(z.shape) == [3, 1] and np.array_equal(z.to_numpy().ravel(), [1, 1, 1])
+    z = ex.exec_custom("stack", [one, one, one], i_args=[1])[0]
+    assert list(z.shape) == [1, 3]
+    x1, x2 = np.arange(0, 6, dtype=np.float32).reshape(3, 2), np.arange(6, 12, dtype=np.float32).reshape(3, 2)
+    st = ex.exec_custom("stack", [NDArray.from_numpy(x1), NDArray.from_numpy(x2)], i_args=[0])[0]
+    cc = ex.exec_custom("concat", [NDArray.from_numpy(x1), NDArray.from_numpy(x2)], i_args=[0])[0]
+    assert np.array_equal(st.to_numpy(), cc.to_numpy().reshape(2, 3, 2))
+    # last axis, strided inputs, negative axis; numpy.stack is the same function
+    rng = np.random.default_rng(8)
+    big = rng.normal(0, 1, (5, 6, 7)).astype(np.float32)
+    BIG = NDArray.from_numpy(big)
+    views = [BIG.permute(2, 0, 1), BIG.permute(2, 0, 1)]
+    z = ex.exec_custom("stack", views, i_args=[-1])[0]
+    assert np.array_equal(z.to_numpy(), np.stack([big.transpose(2, 0, 1)] * 2, axis=-1))
+    with pytest.raises(NativeOpsError, match="shapes of all input arrays must be the same"):
+        ex.exec_custom("stack", [A, one])
+
+
+def test_unstack_reference_cases(ex):
+    """DeclarableOpsTests9.cpp:833-866: a 5x5 array gives 5 rows; a vector of 5 gives 5 scalars 1..5."""
+    x = np.arange(1, 26, dtype=np.float64).reshape(5, 5)
+    outs = ex.exec_custom("unstack", [NDArray.from_numpy(x)], i_args=[0])
+    assert len(outs) == 5 and all(list(o.shape) == [5] for o in outs)
+    assert all(np.array_equal(o.to_numpy(), x[i]) for i, o in enumerate(outs))
+    outs = ex.exec_custom("unstack", [NDArray.from_numpy(x)], i_args=[1])
+    assert all(np.array_equal(o.to_numpy(), x[:, i]) for i, o in enumerate(outs))
+    outs = ex.exec_custom("unstack", [NDArray.from_numpy(np.arange(1, 6, dtype=np.float64))], i_args=[0])
+    assert len(outs) == 5 and all(list(o.shape) == [] for o in outs)
+    assert [float(o.to_numpy()) for o in outs] == [1, 2, 3, 4, 5]
+    rng = np.random.default_rng(9)
+    v = rng.normal(0, 1, (3, 4, 5)).astype(np.float32)
+    outs = ex.exec_custom("unpack", [NDArray.from_numpy(v)], i_args=[-2])
+    assert len(outs) == 4 and all(np.array_equal(o.to_numpy(), v[:, i]) for i, o in enumerate(outs))
+    with pytest.raises(NativeOpsError, match="Unstack dimension should be lower then rank"):
+        ex.exec_custom("unstack", [NDArray.from_numpy(v)], i_args=[3])
