@@ -802,6 +802,31 @@ static std::vector<std::vector<LongType>> broadcastableShapeFn(Context& c) {
   return {makeShapeInfo(x->dataType(), x->ordering(), broadcastShape(x, y))};
 }
 
+// biasadd (generic/nn/bias_add.cpp:33-73, alias bias_add; helpers/cpu/addBias.cpp): a rank-1 bias added along the channel
+// axis -- the last one, or axis 1 when BArg0 (NCHW) is set; the output carries the bias's data type
+static void biasAddExec(Context& c) {
+  NDArray* x = c.input(0); NDArray* b = c.input(1); NDArray* z = c.output(0);
+  const bool nchw = bArg(c, 0, false);
+  const int ch = nchw ? 1 : x->rankOf() - 1;
+  ND4J_REQUIRE(b->rankOf() == 1, "BIASADD CUSTOM_OP: bias array should have rank = 1, but got " + std::to_string(b->rankOf()) + " instead !");
+  ND4J_REQUIRE(x->rankOf() >= 1 && ch < x->rankOf() && b->sizeAt(0) == x->sizeAt(ch),
+               "BIASADD CUSTOM_OP: shapes of bias " + shapeStr(b) + " and input " + shapeStr(x) + " arrays are not suitable for broadcast operation along channel dimension " + std::to_string(ch) + " !");
+  ND4J_REQUIRE(shapeOf(z) == shapeOf(x), "BIASADD CUSTOM_OP: wrong shape of output array, expected is " + shapeStr(x) + " but got " + shapeStr(z) + " instead !");
+  ND4J_REQUIRE(isFloatType(x->dataType()) && isFloatType(b->dataType()) && isFloatType(z->dataType()), "BIASADD CUSTOM_OP: nd4j-hip implements floating point arrays only");
+  if (x->isEmpty() || z->isEmpty()) return;
+  std::vector<LongType> bs(x->rankOf(), 0);
+  bs[ch] = b->strideAt(0);
+  auto bsi = makeShapeInfo(b->dataType(), 'c', shapeOf(x), bs.data());
+  EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo(), bsi.data()});
+  prepareSpecialUse({z}, {x, b});
+  launchPairwise(stream(), P_ADD, x->dataType(), b->dataType(), z->dataType(), x->specialBuffer(), b->specialBuffer(), z->specialBuffer(), p);
+  registerSpecialUse({z}, {x, b});
+}
+static std::vector<std::vector<LongType>> biasAddShapeFn(Context& c) {
+  NDArray* x = c.input(0); NDArray* b = c.input(1);
+  return {makeShapeInfo(b->dataType(), x->ordering(), shapeOf(x))};
+}
+
 // concat (generic/transforms/concat.cpp:34): inputs joined along IArg0 (or the last input when BArg0 is set)
 static void concatExec(Context& c) {
   int n = c.width();
@@ -1532,6 +1557,7 @@ static void ensureRegistered() {
     reg("standardize_bp", 2, 1, false, 0, -2, standardizeBpExec, sameAsInputShapeFn);
     reg("layer_norm_bp", 3, -1, false, 0, -1, layerNormBpExec, layerNormBpShapeFn);
     reg("matmul_bp", 3, 2, false, 0, -2, matmulBpExec, matmulBpShapeFn);
+    for (const char* alias : {"biasadd", "bias_add"}) reg(alias, 2, 1, true, 0, 0, biasAddExec, biasAddShapeFn);
     for (const char* alias : {"cast", "Cast"}) reg(alias, 1, 1, false, 0, -2, castExec, castShapeFn);
     for (const char* alias : {"stack", "pack", "Pack"}) reg(alias, -1, 1, false, 0, 0, stackExec, stackShapeFn);
     for (const char* alias : {"unstack", "unpack"}) reg(alias, 1, -1, false, 0, 1, unstackExec, unstackShapeFn);

@@ -850,3 +850,25 @@ def test_unstack_reference_cases(ex):
     assert len(outs) == 4 and all(np.array_equal(o.to_numpy(), v[:, i]) for i, o in enumerate(outs))
     with pytest.raises(NativeOpsError, match="Unstack dimension should be lower then rank"):
         ex.exec_custom("unstack", [NDArray.from_numpy(v)], i_args=[3])
+
+
+def test_biasadd_reference_vectors(ex):
+    """DeclarableOpsTests4.cpp:692-741 (biasadd_1..3: NHWC, NCHW, rank 2) and :795-808 (double input, float bias and output)."""
+    b2 = NDArray.from_numpy(np.array([1.0, 2.0]))
+    z = ex.exec_custom("biasadd", [NDArray.from_numpy(np.zeros((2, 3, 3, 2))), b2])[0]
+    assert np.array_equal(z.to_numpy(), np.tile([1.0, 2.0], 18).reshape(2, 3, 3, 2))
+    z = ex.exec_custom("biasadd", [NDArray.from_numpy(np.zeros((2, 2, 3, 3))), b2], b_args=[True])[0]
+    assert np.array_equal(z.to_numpy(), np.tile(np.repeat([1.0, 2.0], 9), 2).reshape(2, 2, 3, 3))
+    row = NDArray.from_numpy(np.array([1.0, 2.0, 3.0]))
+    z = ex.exec_custom("bias_add", [NDArray.from_numpy(np.zeros((2, 3))), row], b_args=[True])[0]
+    assert np.array_equal(z.to_numpy(), [[1, 2, 3], [1, 2, 3]])
+    zf = NDArray.empty((2, 3), FLOAT32)
+    ex.exec_custom("biasadd", [NDArray.from_numpy(np.zeros((2, 3))), NDArray.from_numpy(np.array([1, 2, 3], np.float32))], [zf], b_args=[True])
+    assert np.array_equal(zf.to_numpy(), np.array([[1, 2, 3], [1, 2, 3]], np.float32))
+    rng = np.random.default_rng(12)
+    x = rng.normal(0, 1, (3, 5, 4, 6)).astype(np.float32)
+    b = rng.normal(0, 1, 5).astype(np.float32)
+    z = ex.exec_custom("biasadd", [NDArray.from_numpy(x), NDArray.from_numpy(b)], b_args=[True])[0]
+    assert np.array_equal(z.to_numpy(), x + b[None, :, None, None])
+    with pytest.raises(NativeOpsError, match="not suitable for broadcast operation along channel dimension"):
+        ex.exec_custom("biasadd", [NDArray.from_numpy(x), NDArray.from_numpy(b)])
