@@ -827,6 +827,28 @@ static std::vector<std::vector<LongType>> biasAddShapeFn(Context& c) {
   return {makeShapeInfo(b->dataType(), x->ordering(), shapeOf(x))};
 }
 
+// equals, not_equals, greater, greater_equal, less, less_equal (generic/broadcastable/equals.cpp:29-58 and siblings):
+// the comparison of the bool tables under broadcasting, BOOL output
+static void comparisonExec(Context& c, PairwiseKind k, const char* name) {
+  ND4J_REQUIRE(c.width() >= 2, std::string(name) + ": two inputs are required");
+  NDArray* x = c.input(0); NDArray* y = c.input(1); NDArray* z = c.output(0);
+  ND4J_REQUIRE(z->dataType() == BOOL, std::string(name) + ": the output must be a BOOL array");
+  ND4J_REQUIRE(x->dataType() == y->dataType(), std::string(name) + ": nd4j-hip compares arrays of one data type");
+  if (x->isEmpty() || y->isEmpty() || z->isEmpty()) return;
+  auto out = broadcastShape(x, y);
+  ND4J_REQUIRE(out == shapeOf(z), std::string(name) + ": output shape " + shapeStr(z) + " does not match the broadcast shape");
+  auto xs = broadcastStrides(x, out), ys = broadcastStrides(y, out);
+  auto xsi = makeShapeInfo(x->dataType(), 'c', out, xs.data()), ysi = makeShapeInfo(y->dataType(), 'c', out, ys.data());
+  EwPlan p = buildEwPlan({z->shapeInfo(), xsi.data(), ysi.data()});
+  prepareSpecialUse({z}, {x, y});
+  launchPairwise(stream(), k, x->dataType(), y->dataType(), BOOL, x->specialBuffer(), y->specialBuffer(), z->specialBuffer(), p);
+  registerSpecialUse({z}, {x, y});
+}
+static std::vector<std::vector<LongType>> comparisonShapeFn(Context& c) {
+  NDArray* x = c.input(0); NDArray* y = c.input(1);
+  return {makeShapeInfo(BOOL, x->ordering(), broadcastShape(x, y))};
+}
+
 // concat (generic/transforms/concat.cpp:34): inputs joined along IArg0 (or the last input when BArg0 is set)
 static void concatExec(Context& c) {
   int n = c.width();
@@ -1557,6 +1579,14 @@ static void ensureRegistered() {
     reg("standardize_bp", 2, 1, false, 0, -2, standardizeBpExec, sameAsInputShapeFn);
     reg("layer_norm_bp", 3, -1, false, 0, -1, layerNormBpExec, layerNormBpShapeFn);
     reg("matmul_bp", 3, 2, false, 0, -2, matmulBpExec, matmulBpShapeFn);
+    {
+      struct { const char* name; PairwiseKind kind; } cmp[] = {{"equals", P_EQ}, {"equal", P_EQ}, {"not_equals", P_NE}, {"greater", P_GT},
+                                                               {"greater_equal", P_GE}, {"less", P_LT}, {"less_equal", P_LE}};
+      for (auto& e : cmp) {
+        const PairwiseKind kind = e.kind; const char* name = e.name;
+        reg(name, 2, 1, true, 0, 0, [kind, name](Context& c) { comparisonExec(c, kind, name); }, comparisonShapeFn);
+      }
+    }
     for (const char* alias : {"biasadd", "bias_add"}) reg(alias, 2, 1, true, 0, 0, biasAddExec, biasAddShapeFn);
     for (const char* alias : {"cast", "Cast"}) reg(alias, 1, 1, false, 0, -2, castExec, castShapeFn);
     for (const char* alias : {"stack", "pack", "Pack"}) reg(alias, -1, 1, false, 0, 0, stackExec, stackShapeFn);

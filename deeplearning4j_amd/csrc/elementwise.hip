@@ -287,6 +287,12 @@ __device__ __forceinline__ A binary_tail(int k, A a, A b) {
     case P_SQ_RSUB: { A d = b - a; return d * d; }                                             // op_macros_special.h:820-827
     case P_REVERSE_POW: return M::pow_(b, a);                                                  // ops.h:166
     case P_SXE_LOGITS_SMOOTHER: return a * ((A)1 - b) + (A)0.5f * b;                           // ops.h:352-355
+    case P_EQ: return (A)(a == b);                                                             // ops.h:181-186 (comparison ops)
+    case P_NE: return (A)(a != b);
+    case P_GT: return (A)(a > b);
+    case P_GE: return (A)(a >= b);
+    case P_LT: return (A)(a < b);
+    case P_LE: return (A)(a <= b);
     default: return a;
   }
 }
@@ -448,7 +454,7 @@ __global__ __launch_bounds__(EW_BLOCK) void tail_generic(int k, DevShape sz, Dev
     LongType oz = walk<LongType>(sz, i), ox = walk<LongType>(sx, i);
     double a = load_any(x, xdt, ox), b = scalar;
     if (NIN > 1 && !hasScalar) b = load_any(y, ydt, walk<LongType>(sy, i));
-    if (zdt == DOUBLE || xdt == DOUBLE) {   // predicates on doubles must not see them narrowed
+    if (zdt == DOUBLE || xdt == DOUBLE || xdt == INT32 || xdt == INT64) {   // predicates on doubles and integers must not see them narrowed
       store_any(z, zdt, oz, NIN > 1 ? binary_tail<double>(k, a, b) : unary_tail<double>(k, a));
     } else {
       float fa = round_as((float)a, zdt), fb = round_as((float)b, zdt);

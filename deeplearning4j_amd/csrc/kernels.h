@@ -39,6 +39,8 @@ enum PairwiseKind : int {
   // scalar table only
   P_ELU, P_ELU_D, P_LEAKY_RELU, P_LEAKY_RELU_D, P_LOG_X, P_RELU, P_RELU6, P_RELU_D, P_STEP, P_LSTM_CLIP,
   P_SQ_RSUB, P_REVERSE_POW, P_SXE_LOGITS_SMOOTHER,
+  // comparisons (the bool tables): 1 / 0, stored into a BOOL output
+  P_EQ, P_NE, P_GT, P_GE, P_LT, P_LE,
   P_TAIL_END
 };
 

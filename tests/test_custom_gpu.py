@@ -872,3 +872,36 @@ def test_biasadd_reference_vectors(ex):
     assert np.array_equal(z.to_numpy(), x + b[None, :, None, None])
     with pytest.raises(NativeOpsError, match="not suitable for broadcast operation along channel dimension"):
         ex.exec_custom("biasadd", [NDArray.from_numpy(x), NDArray.from_numpy(b)])
+
+
+def test_comparison_ops_reference_vectors(ex):
+    """BroadcastableOpsTests.cpp:505-517 (broadcast_equals_1), :646-700 (broadcast_bool_1..3), :629-644 (broadcast_bool_empty_2)."""
+    from deeplearning4j_amd.ndarray import BOOL
+    x = NDArray.from_numpy(np.array([[1, 2, 3, 4]], np.float64))
+    y = NDArray.from_numpy(np.array([[0, 0, 0, 0], [1, 2, 3, 4], [1, 2, 3, 4]], np.float64))
+    z = ex.exec_custom("equals", [x, y])[0]
+    assert z.dtype == BOOL and np.array_equal(z.to_numpy().astype(bool), [[False] * 4, [True] * 4, [True] * 4])
+    a, b = NDArray.from_numpy(np.full((3, 1, 2), 4, np.float32)), NDArray.from_numpy(np.full((2, 2), 2, np.float32))
+    z = ex.exec_custom("greater", [a, b])[0]
+    assert list(z.shape) == [3, 2, 2] and z.to_numpy().astype(bool).all()
+    z = ex.exec_custom("equals", [NDArray.from_numpy(np.full((3, 1, 2), 1, np.float32)), b])[0]
+    assert list(z.shape) == [3, 2, 2] and not z.to_numpy().astype(bool).any()
+    z = ex.exec_custom("less", [NDArray.from_numpy(np.array(0, np.int32)), NDArray.from_numpy(np.array([2, 1, 2], np.int32))])[0]
+    assert list(z.shape) == [3] and z.to_numpy().astype(bool).all()
+    e = ex.exec_custom("greater", [NDArray.empty((0, 4), DOUBLE), NDArray.from_numpy(np.array([[1, 2, 3, 4]], np.float64))])[0]
+    assert e.dtype == BOOL and list(e.shape) == [0, 4]
+    # every comparison against numpy, NaN included, integers beyond the float mantissa
+    rng = np.random.default_rng(21)
+    u = rng.integers(-3, 4, (5, 1, 17)).astype(np.float32)
+    v = rng.integers(-3, 4, (6, 17)).astype(np.float32)
+    u[0, 0, 0] = np.nan
+    for name, fn in [("equals", np.equal), ("equal", np.equal), ("not_equals", np.not_equal), ("greater", np.greater),
+                     ("greater_equal", np.greater_equal), ("less", np.less), ("less_equal", np.less_equal)]:
+        got = ex.exec_custom(name, [NDArray.from_numpy(u), NDArray.from_numpy(v)])[0].to_numpy().astype(bool)
+        assert np.array_equal(got, fn(u, v)), name
+        for dt in (HALF, BFLOAT16):
+            got = ex.exec_custom(name, [NDArray.from_numpy(u, dt), NDArray.from_numpy(v, dt)])[0].to_numpy().astype(bool)
+            assert np.array_equal(got, fn(u, v)), (name, dt)
+    big = np.array([16777217, 16777216, -16777217], np.int64)
+    got = ex.exec_custom("greater", [NDArray.from_numpy(big), NDArray.from_numpy(np.array(16777216, np.int64))])[0].to_numpy().astype(bool)
+    assert np.array_equal(got, [True, False, False])
