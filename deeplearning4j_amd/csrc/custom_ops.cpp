@@ -1212,6 +1212,105 @@ static std::vector<std::vector<LongType>> castShapeFn(Context& c) {
   return {makeShapeInfo(dt, x->ordering(), shapeOf(x))};
 }
 
+// integer arguments given as an input array of any numeric type (the reference reads them with asVectorT<LongType>)
+static std::vector<LongType> hostNumbersAsLong(NDArray* a, const char* what) {
+  if (a->dataType() == INT32 || a->dataType() == INT64) return hostIndexVector(a, what);
+  std::vector<LongType> out;
+  if (a->isEmpty() || a->lengthOf() == 0) return out;
+  ND4J_REQUIRE(isFloatType(a->dataType()), std::string(what) + ": a numeric array is required");
+  a->buf->syncToPrimary();
+  for (LongType i = 0; i < a->lengthOf(); i++) {
+    const LongType off = a->rankOf() == 0 ? 0 : i * a->strideAt(a->rankOf() - 1);
+    out.push_back((LongType)hostValueAsDouble(a->hostAs<unsigned char>() + off * sizeOf(a->dataType()), a->dataType()));
+  }
+  return out;
+}
+
+// tile (generic/transforms/tile.cpp:31-108): the input repeated reps[d] times along every axis d; reps from IArgs (one per
+// axis) or from a second input
+static std::vector<LongType> tileReps(Context& c) {
+  NDArray* x = c.input(0);
+  std::vector<LongType> reps;
+  if ((int)c.iArgs.size() == x->rankOf()) reps = c.iArgs;
+  else if (c.width() > 1) {
+    reps = hostNumbersAsLong(c.input(1), "TILE op");
+    ND4J_REQUIRE((int)reps.size() == x->rankOf(), "TILE op: repeats vector length should be equal to input rank, but got " + std::to_string(reps.size()) + " and " + std::to_string(x->rankOf()) + " correspondingly !");
+  } else ND4J_THROW("TILE op: this op requires repeats vector, either as IArgs or second array with length equal to rank of input array to be tiled !");
+  LongType prod = 1;
+  for (auto r : reps) prod *= r;
+  ND4J_REQUIRE(prod > 0, "TILE op: reps can't contain 0s");
+  return reps;
+}
+static void tileExec(Context& c) {
+  NDArray* x = c.input(0); NDArray* z = c.output(0);
+  auto reps = tileReps(c);
+  const int rank = x->rankOf();
+  ND4J_REQUIRE(z->rankOf() == rank && z->dataType() == x->dataType(), "TILE op: wrong output array");
+  // z seen as [reps0, n0, reps1, n1, ...] and x as the same shape with stride 0 along the repeat axes
+  std::vector<LongType> shp, zs, xs;
+  for (int d = 0; d < rank; d++) {
+    ND4J_REQUIRE(z->sizeAt(d) == x->sizeAt(d) * reps[d], "TILE op: wrong output shape");
+    shp.push_back(reps[d]); zs.push_back(x->sizeAt(d) * z->strideAt(d)); xs.push_back(0);
+    shp.push_back(x->sizeAt(d)); zs.push_back(z->strideAt(d)); xs.push_back(x->strideAt(d));
+  }
+  if (x->isEmpty() || z->isEmpty() || x->lengthOf() == 0) return;
+  if (shp.empty()) { shp = {1}; zs = {1}; xs = {1}; }
+  auto zsi = makeShapeInfo(z->dataType(), 'c', shp, zs.data()), xsi = makeShapeInfo(x->dataType(), 'c', shp, xs.data());
+  EwPlan p = buildEwPlan({zsi.data(), xsi.data()});
+  prepareSpecialUse({z}, {x});
+  launchUnary(stream(), U_IDENTITY, x->dataType(), z->dataType(), x->specialBuffer(), z->specialBuffer(), p);
+  registerSpecialUse({z}, {x});
+}
+static std::vector<std::vector<LongType>> tileShapeFn(Context& c) {
+  NDArray* x = c.input(0);
+  auto reps = tileReps(c);
+  std::vector<LongType> out = shapeOf(x);
+  for (int d = 0; d < x->rankOf(); d++) out[d] *= reps[d];
+  return {makeShapeInfo(x->dataType(), x->ordering(), out)};
+}
+
+// slice (generic/transforms/slice.cpp:31-120): begin and size per axis (size -1 = to the end), from IArgs
+// [begin.., size..] or from two input arrays
+struct SliceArgs { std::vector<LongType> begin, size; bool empty = false; };
+static SliceArgs sliceArgs(Context& c) {
+  NDArray* x = c.input(0);
+  const int rank = x->rankOf();
+  SliceArgs a;
+  if (c.width() == 3) { a.begin = hostNumbersAsLong(c.input(1), "Slice"); a.size = hostNumbersAsLong(c.input(2), "Slice"); }
+  else {
+    ND4J_REQUIRE((int)c.iArgs.size() >= 2 * rank, "Number of IArgs should be equal to [" + std::to_string(2 * rank) + "] but got [" + std::to_string(c.iArgs.size()) + "] instead");
+    a.begin.assign(c.iArgs.begin(), c.iArgs.begin() + rank);
+    a.size.assign(c.iArgs.begin() + rank, c.iArgs.begin() + 2 * rank);
+  }
+  ND4J_REQUIRE((int)a.begin.size() == rank, "begin array should have length of [" + std::to_string(rank) + "] but got [" + std::to_string(a.begin.size()) + "] instead");
+  ND4J_REQUIRE((int)a.size.size() == rank, "size array should have length of [" + std::to_string(rank) + "] but got [" + std::to_string(a.size.size()) + "] instead");
+  for (int d = 0; d < rank; d++) {
+    const LongType start = a.begin[d];
+    ND4J_REQUIRE(start >= 0, "Slice: start index should not be negative");
+    ND4J_REQUIRE(start <= x->sizeAt(d), "Index " + std::to_string(start) + " is invalid for dimension " + std::to_string(d) + " with size " + std::to_string(x->sizeAt(d)) + ".");
+    if (a.size[d] == -1) a.size[d] = x->sizeAt(d) - start;
+    ND4J_REQUIRE(a.size[d] >= 0, "Slice: interval for dimension " + std::to_string(d) + " is less then 1");
+    ND4J_REQUIRE(start + a.size[d] <= x->sizeAt(d), "Slice: interval [" + std::to_string(start) + ", " + std::to_string(start + a.size[d]) + "] is out of bounds for dimension " +
+                 std::to_string(d) + " with size " + std::to_string(x->sizeAt(d)));
+    if (start == x->sizeAt(d) || a.size[d] == 0) a.empty = true;
+  }
+  return a;
+}
+static void sliceExec(Context& c) {
+  NDArray* x = c.input(0); NDArray* z = c.output(0);
+  SliceArgs a = sliceArgs(c);
+  if (a.empty || x->isEmpty() || z->isEmpty()) return;
+  ND4J_REQUIRE(shapeOf(z) == a.size, "Slice: output shape " + shapeStr(z) + " does not match the requested sizes");
+  LongType off = 0;
+  for (int d = 0; d < x->rankOf(); d++) off += a.begin[d] * x->strideAt(d);
+  assignEnumerated(z, x, off, a.size, stridesOf(x), 'c', "Slice");
+}
+static std::vector<std::vector<LongType>> sliceShapeFn(Context& c) {
+  NDArray* x = c.input(0);
+  SliceArgs a = sliceArgs(c);
+  return {makeShapeInfo(x->dataType(), 'c', a.size)};
+}
+
 // strided_slice (generic/tensor/strided_slice.cpp:135-370,372-530): IArgs = begin_mask, ellipsis_mask, end_mask, new_axis_mask,
 // shrink_axis_mask [, begin.., end.., strides..]; or begin/end/strides as inputs 1..3.  The sparse specification (one entry per
 // written index) is spread over the input's axes, every axis gets a canonical [begin, end) and a step, and the output is the
@@ -1587,6 +1686,8 @@ static void ensureRegistered() {
         reg(name, 2, 1, true, 0, 0, [kind, name](Context& c) { comparisonExec(c, kind, name); }, comparisonShapeFn);
       }
     }
+    reg("tile", 1, 1, false, 0, -2, tileExec, tileShapeFn);
+    reg("slice", 1, 1, false, 0, -2, sliceExec, sliceShapeFn);
     for (const char* alias : {"biasadd", "bias_add"}) reg(alias, 2, 1, true, 0, 0, biasAddExec, biasAddShapeFn);
     for (const char* alias : {"cast", "Cast"}) reg(alias, 1, 1, false, 0, -2, castExec, castShapeFn);
     for (const char* alias : {"stack", "pack", "Pack"}) reg(alias, -1, 1, false, 0, 0, stackExec, stackShapeFn);

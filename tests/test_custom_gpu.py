@@ -905,3 +905,38 @@ def test_comparison_ops_reference_vectors(ex):
     big = np.array([16777217, 16777216, -16777217], np.int64)
     got = ex.exec_custom("greater", [NDArray.from_numpy(big), NDArray.from_numpy(np.array(16777216, np.int64))])[0].to_numpy().astype(bool)
     assert np.array_equal(got, [True, False, False])
+
+
+def test_tile_and_slice_reference_vectors(ex):
+    """DeclarableOpsTests3.cpp:36-60 (Test_Tile_1/2: a 2x3 array tiled 2x2), DeclarableOpsTests9.cpp:736-750 ({1,6} tiled {2,1}),
+    IndexingTests.cpp:90-160 (SimpleSlice_1..4)."""
+    x = np.array([[1, 2, 3], [4, 5, 6]], np.float32)
+    want = np.tile(x, (2, 2))
+    z = ex.exec_custom("tile", [NDArray.from_numpy(x), NDArray.from_numpy(np.array([[2, 2]], np.int32))])[0]
+    assert list(z.shape) == [4, 6] and np.array_equal(z.to_numpy(), want)
+    z = ex.exec_custom("tile", [NDArray.from_numpy(x)], i_args=[2, 2])[0]
+    assert np.array_equal(z.to_numpy(), want)
+    row = np.array([[1, 2, 3, 4, 5, 6]], np.float64)
+    z = ex.exec_custom("tile", [NDArray.from_numpy(row), NDArray.from_numpy(np.array([[2, 1]], np.int32))])[0]
+    assert list(z.shape) == [2, 6] and np.array_equal(z.to_numpy(), np.array([[1, 2, 3, 4, 5, 6]] * 2, np.float64))
+    rng = np.random.default_rng(14)
+    v = rng.normal(0, 1, (3, 4, 5)).astype(np.float32)
+    z = ex.exec_custom("tile", [NDArray.from_numpy(v).permute(1, 2, 0)], i_args=[2, 1, 3])[0]
+    assert np.array_equal(z.to_numpy(), np.tile(v.transpose(1, 2, 0), (2, 1, 3)))
+    with pytest.raises(NativeOpsError, match="reps can't contain 0s"):
+        ex.exec_custom("tile", [NDArray.from_numpy(x)], i_args=[2, 0])
+
+    inp = np.array([1, 1, 1, 2, 2, 2, 3, 3, 3, 4, 4, 4, 5, 5, 5, 6, 6, 6], np.float32).reshape(3, 2, 3)
+    z = ex.exec_custom("slice", [NDArray.from_numpy(inp)], i_args=[1, 0, 0, 1, 1, 3])[0]
+    assert list(z.shape) == [1, 1, 3] and np.array_equal(z.to_numpy().ravel(), [3, 3, 3])
+    z = ex.exec_custom("slice", [NDArray.from_numpy(inp)], i_args=[1, 0, 0, 1, 2, 3])[0]
+    assert list(z.shape) == [1, 2, 3] and np.array_equal(z.to_numpy().ravel(), [3, 3, 3, 4, 4, 4])
+    z = ex.exec_custom("slice", [NDArray.from_numpy(inp)], i_args=[1, 0, 0, 2, 1, 3])[0]
+    assert list(z.shape) == [2, 1, 3] and np.array_equal(z.to_numpy().ravel(), [3, 3, 3, 5, 5, 5])
+    start, size = NDArray.from_numpy(np.array([1.0, 0.0, 0.0])), NDArray.from_numpy(np.array([2.0, 1.0, 3.0]))
+    z = ex.exec_custom("slice", [NDArray.from_numpy(inp.astype(np.float64)), start, size])[0]
+    assert list(z.shape) == [2, 1, 3] and np.array_equal(z.to_numpy().ravel(), [3, 3, 3, 5, 5, 5])
+    z = ex.exec_custom("slice", [NDArray.from_numpy(v)], i_args=[1, 2, 0, -1, 1, -1])[0]
+    assert np.array_equal(z.to_numpy(), v[1:, 2:3, :])
+    with pytest.raises(NativeOpsError, match="out of bounds for dimension 1"):
+        ex.exec_custom("slice", [NDArray.from_numpy(v)], i_args=[0, 2, 0, 1, 3, 1])
