@@ -476,10 +476,19 @@ __global__ __launch_bounds__(EW_BLOCK) void scalar2_generic(int k, DevShape sz, 
     if (k == S2_CLIP_BY_VALUE) {
       r = a > s2 ? s2 : (a < s1 ? s1 : a);
     } else if (xdt == DOUBLE) {
-      r = k == S2_AFFINE ? s1 * a + s2 : s1 * d_tanh(s2 * a);
+      const double cut = (double)3.79297773665f;
+      if (k == S2_AFFINE) r = s1 * a + s2;
+      else if (k == S2_SCALED_TANH) r = s1 * d_tanh(s2 * a);
+      else if (k == S2_STABILIZE) r = a * s1 > cut ? cut / s1 : (a * s1 < -cut ? -cut / s1 : a);
+      else if (a >= s1 && a <= s2) r = a;
+      else r = floor((s1 == 0.0 && s2 == 1.0 ? 1.0 / (1.0 + exp(-a)) : a) * (s2 - s1)) + s1;
     } else {
-      const float fa = (float)a, f1 = (float)s1, f2 = (float)s2;
-      r = k == S2_AFFINE ? f1 * fa + f2 : f1 * d_tanh(f2 * fa);
+      const float fa = (float)a, f1 = (float)s1, f2 = (float)s2, cut = 3.79297773665f;
+      if (k == S2_AFFINE) r = f1 * fa + f2;
+      else if (k == S2_SCALED_TANH) r = f1 * d_tanh(f2 * fa);
+      else if (k == S2_STABILIZE) r = fa * f1 > cut ? cut / f1 : (fa * f1 < -cut ? -cut / f1 : fa);
+      else if (fa >= f1 && fa <= f2) r = fa;
+      else r = floorf((f1 == 0.f && f2 == 1.f ? 1.f / (1.f + expf(-fa)) : fa) * (f2 - f1)) + f1;
     }
     store_any(z, zdt, oz, r);
   }

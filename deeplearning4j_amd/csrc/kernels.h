@@ -67,7 +67,9 @@ void launchRowBroadcast(hipStream_t s, PairwiseKind k, DataType dt, const void* 
 enum Scalar2Kind : int {
   S2_CLIP_BY_VALUE,   // x > s2 ? s2 : (x < s1 ? s1 : x)      ops.h:412-415, helpers/cpu/clip.cpp:211-219
   S2_AFFINE,          // s1 * x + s2                          ops.h:453
-  S2_SCALED_TANH      // s1 * tanh(s2 * x)                    ops.h:1088-1090
+  S2_SCALED_TANH,     // s1 * tanh(s2 * x)                    ops.h:1088-1090
+  S2_STABILIZE,       // x * s1 beyond +-3.79297773665: that cutoff / s1, else x   ops.h:458-468 (one parameter)
+  S2_SET_RANGE        // x inside [s1, s2]: x; else floor(v * (s2 - s1)) + s1 with v = sigmoid(x) for the range [0, 1], else x   ops.h:427-438
 };
 void launchScalar2Op(hipStream_t s, Scalar2Kind k, DataType xdt, DataType zdt, const void* x, double s1, double s2, void* z,
                      const EwPlan& p);

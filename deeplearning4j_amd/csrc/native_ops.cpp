@@ -451,13 +451,14 @@ static void runUnary(const char* fn, UnaryKind k, NDArray* x, NDArray* z) {
 // The transforms that read two extra parameters.  extraParams holds them in the array's own type (the executioner
 // converts its extraArgs to X before the call); it may be device or host memory, so they are fetched with a blocking copy.
 static void runUnaryWithParams(const char* fn, Scalar2Kind k, NDArray* x, NDArray* z, const void* extraParams) {
-  if (extraParams == nullptr) ND4J_THROW(std::string(fn) + ": this op needs two extra parameters");
+  const int nParams = k == S2_STABILIZE ? 1 : 2;
+  if (extraParams == nullptr) ND4J_THROW(std::string(fn) + (nParams == 1 ? ": this op needs one extra parameter" : ": this op needs two extra parameters"));
   if (x->isEmpty() || z->isEmpty()) return;
   unsigned char raw[16];
   const size_t w = sizeOf(x->dataType());
   HIP_CHECK(hipStreamSynchronize(execStream()));
-  HIP_CHECK(hipMemcpy(raw, extraParams, 2 * w, hipMemcpyDefault));
-  const double s1 = hostValueAsDouble(raw, x->dataType()), s2 = hostValueAsDouble(raw + w, x->dataType());
+  HIP_CHECK(hipMemcpy(raw, extraParams, nParams * w, hipMemcpyDefault));
+  const double s1 = hostValueAsDouble(raw, x->dataType()), s2 = nParams > 1 ? hostValueAsDouble(raw + w, x->dataType()) : 0.0;
   EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo()});
   prepareSpecialUse({z}, {x});
   launchScalar2Op(execStream(), k, x->dataType(), z->dataType(), x->specialBuffer(), s1, s2, z->specialBuffer(), p);
@@ -470,8 +471,8 @@ void execTransformStrict(Nd4jPointer*, int opNum, OpaqueNDArray xa, void* extraP
   // X -> X over float types only (NativeOpExecutioner_transform.cpp:115-131)
   ND4J_REQUIRE(x->dataType() == z->dataType() && isFloatType(x->dataType()),
                std::string("NativeOpExecutioner::execTransformStrict requires X & Z to have same floating point type, got ") + dtypeName(x->dataType()) + " and " + dtypeName(z->dataType()));
-  if (opNum == 2 || opNum == 3) {   // ScaledTanh, Affine (loops/legacy_ops.h:54)
-    runUnaryWithParams("execTransformStrict", opNum == 2 ? S2_SCALED_TANH : S2_AFFINE, x, z, extraParams);
+  if (opNum == 2 || opNum == 3 || opNum == 19 || opNum == 25) {   // ScaledTanh, Affine, Stabilize, SetRange (loops/legacy_ops.h:54-60)
+    runUnaryWithParams("execTransformStrict", opNum == 2 ? S2_SCALED_TANH : opNum == 3 ? S2_AFFINE : opNum == 19 ? S2_STABILIZE : S2_SET_RANGE, x, z, extraParams);
     return;
   }
   UnaryKind k;
@@ -490,7 +491,7 @@ void execTransformStrict(Nd4jPointer*, int opNum, OpaqueNDArray xa, void* extraP
     case 48: k = U_RINT; break; case 49: k = U_LOG_SIGMOID; break; case 50: k = U_ERFC; break; case 51: k = U_EXPM1; break;
     case 52: k = U_ATANH; break; case 54: k = U_GELU_D; break; case 56: k = U_PRECISE_GELU_D; break; case 57: k = U_MISH; break;
     case 58: k = U_MISH_D; break;
-    // 19 Stabilize and 25 SetRange read extra parameters; 5 HardTanhDerivative, 10 HardSigmoidDerivative and
+    // 5 HardTanhDerivative, 10 HardSigmoidDerivative and
     // 20 StabilizeFP16 are not restated (their reference macros return the input unchanged / a platform constant)
     default: ND4J_THROW("execTransformStrict: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }

@@ -52,8 +52,10 @@
  *   matmul ............................ DeclarableOpsTests14.cpp:601-1260, DeclarableOpsTests19.cpp:52-140
  *   softmax ........................... DeclarableOpsTests1.cpp:2523-2740; inf/nan clamp
  *                                       semantics: parity unpinned (source only)
- *   clip_by_value, affine, scaled_tanh
- *   (oracle.py, numpy) ................ DeclarableOpsTests1.cpp:801-848 (ClipByValue1/2), numpy.clip, library tanh
+ *   clip_by_value, affine, scaled_tanh,
+ *   stabilize, set_range
+ *   (oracle.py, numpy) ................ DeclarableOpsTests1.cpp:801-848 (ClipByValue1/2), numpy.clip, library tanh; stabilize and
+ *                                       set_range: hand-computed cases and invariants only (the reference has no test of them)
  *   log_softmax (oracle.py, numpy) .... DeclarableOpsTests5.cpp:2199-2340 (tests/golden/log_softmax_vectors.json)
  *   layer_norm ........................ closed form (TestLayerOpValidation.java:1188-1333)
  *   dot_product_attention_v2 .......... parity unpinned: the reference has no enabled

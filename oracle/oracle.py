@@ -429,6 +429,27 @@ def scaled_tanh(x, a, b):
     return (x.dtype.type(a) * np.tanh(x.dtype.type(b) * x)).astype(x.dtype)
 
 
+def stabilize(x, k):
+    """legacy Stabilize (ops/ops.h:458-468, system/common.h:164-165): where x * k leaves +-3.79297773665 the value becomes
+    that cutoff divided by k."""
+    x = np.asarray(x)
+    t = x.dtype.type
+    cut = t(np.float32(3.79297773665))
+    with np.errstate(invalid="ignore"):
+        return np.where(x * t(k) > cut, cut / t(k), np.where(x * t(k) < -cut, -cut / t(k), x)).astype(x.dtype)
+
+
+def set_range(x, lo, hi):
+    """legacy SetRange (ops/ops.h:427-438): values inside [lo, hi] stay; others become floor(v * (hi - lo)) + lo, with
+    v = sigmoid(x) when the range is [0, 1] and v = x otherwise."""
+    x = np.asarray(x)
+    t = x.dtype.type
+    lo, hi = t(lo), t(hi)
+    with np.errstate(over="ignore", invalid="ignore"):
+        v = t(1) / (t(1) + np.exp(-x)) if (lo == 0 and hi == 1) else x
+        return np.where((x >= lo) & (x <= hi), x, np.floor(v * (hi - lo)) + lo).astype(x.dtype)
+
+
 def log_softmax(x, dim=-1):
     """log_softmax (generic/nn/logSoftmax.cpp:34-49 -> helpers/cpu/activations.cpp:100-145,236-256): max, exp(x - max), sum,
     divide, log -- in that order, in the array type (so a term that underflows in exp comes out as -inf).  A vector

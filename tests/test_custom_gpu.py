@@ -743,6 +743,13 @@ def test_two_parameter_transforms_match_oracle(ex, oracle, dtype):
     assert_close(got[fin], onp.scaled_tanh(xr.astype(np.float64), a, b)[fin], tol * 4, tol * 4, "ScaledTanh")
     with pytest.raises(NativeOpsError, match="needs two extra parameters"):
         ex.exec_transform_same(19, dx)
+    # Stabilize (one parameter) and SetRange; k and the ranges are exact in every type
+    got = ex.exec_transform_strict(19, dx, extra_args=[2.0]).to_float()
+    assert_close(got[fin], onp.stabilize(xr, 2.0).astype(np.float64)[fin], tol, tol, "Stabilize")
+    for lo, hi in [(0.0, 1.0), (2.0, 4.0)]:
+        got = ex.exec_transform_strict(25, dx, extra_args=[lo, hi]).to_float()
+        want = onp.set_range(xr, lo, hi).astype(np.float64)
+        assert_close(got[fin], want[fin], tol, tol, "SetRange")
 
 
 # ---- broadcastable ops: the reference's own vectors ------------------------------------------------------------------------

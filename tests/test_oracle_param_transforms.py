@@ -42,3 +42,21 @@ def test_affine_and_scaled_tanh_closed_forms():
     assert np.abs(o.scaled_tanh(50 * x, 1.7159, 0.6666)).max() <= 1.7159
     h = 1e-6
     assert abs(o.scaled_tanh(np.array([h]), 1.7159, 0.6666)[0] / h - 1.7159 * 0.6666) < 1e-6
+
+
+def test_stabilize_and_set_range_hand_cases():
+    cut = float(np.float32(3.79297773665))
+    x = np.array([0.5, 2.0, -2.0, 1.8, -1.9], np.float64)
+    # k = 2: x*k = 1, 4, -4, 3.6, -3.8 -> inside, above, below, inside, below
+    got = o.stabilize(x, 2.0)
+    assert np.allclose(got, [0.5, cut / 2, -cut / 2, 1.8, -cut / 2], rtol=0, atol=1e-15)
+    # the result times k never leaves the cutoff, and values inside are untouched
+    rng = np.random.default_rng(8)
+    y = rng.normal(0, 5, 1000)
+    assert (np.abs(o.stabilize(y, 0.7) * 0.7) <= cut * (1 + 1e-12)).all()
+    inside = np.abs(y * 0.7) <= cut
+    assert np.array_equal(o.stabilize(y, 0.7)[inside], y[inside])
+    # SetRange: inside stays; outside the unit range goes through a sigmoid and floors to 0; another range floors x * width + lo
+    z = np.array([0.25, 1.0, 3.0, -3.0], np.float64)
+    assert np.array_equal(o.set_range(z, 0.0, 1.0), [0.25, 1.0, 0.0, 0.0])
+    assert np.array_equal(o.set_range(np.array([2.5, 7.25, -1.5]), 2.0, 4.0), [2.5, np.floor(7.25 * 2) + 2, np.floor(-1.5 * 2) + 2])
