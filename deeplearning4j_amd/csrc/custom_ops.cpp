@@ -849,6 +849,22 @@ static std::vector<std::vector<LongType>> comparisonShapeFn(Context& c) {
   return {makeShapeInfo(BOOL, x->ordering(), broadcastShape(x, y))};
 }
 
+// zeros_as (aliases zeroslike, zeros_like) and ones_as (generic/tensor/zeros_as.cpp:30-60, ones_as.cpp): an array of the
+// input's shape, of the type named by DArg0 (default: the input's), filled with 0 / 1
+static void fillAsExec(Context& c, double v, const char* name) {
+  NDArray* z = c.output(0);
+  if (z->isEmpty()) return;
+  ND4J_REQUIRE(isFloatType(z->dataType()), std::string(name) + ": nd4j-hip fills floating point arrays only");
+  prepareSpecialUse({z}, {});
+  fillValue(z, v);
+  registerSpecialUse({z}, {});
+}
+static std::vector<std::vector<LongType>> fillAsShapeFn(Context& c) {
+  NDArray* x = c.input(0);
+  const DataType dt = c.dArgs.empty() ? x->dataType() : c.dArgs[0];
+  return {makeShapeInfo(dt, x->ordering(), shapeOf(x))};
+}
+
 // concat (generic/transforms/concat.cpp:34): inputs joined along IArg0 (or the last input when BArg0 is set)
 static void concatExec(Context& c) {
   int n = c.width();
@@ -1686,6 +1702,8 @@ static void ensureRegistered() {
         reg(name, 2, 1, true, 0, 0, [kind, name](Context& c) { comparisonExec(c, kind, name); }, comparisonShapeFn);
       }
     }
+    for (const char* alias : {"zeros_as", "zeroslike", "zeros_like"}) reg(alias, 1, 1, false, 0, 0, [](Context& c) { fillAsExec(c, 0.0, "zeros_as"); }, fillAsShapeFn);
+    reg("ones_as", 1, 1, false, 0, 0, [](Context& c) { fillAsExec(c, 1.0, "ones_as"); }, fillAsShapeFn);
     reg("tile", 1, 1, false, 0, -2, tileExec, tileShapeFn);
     reg("slice", 1, 1, false, 0, -2, sliceExec, sliceShapeFn);
     for (const char* alias : {"biasadd", "bias_add"}) reg(alias, 2, 1, true, 0, 0, biasAddExec, biasAddShapeFn);

@@ -947,3 +947,17 @@ def test_tile_and_slice_reference_vectors(ex):
     assert np.array_equal(z.to_numpy(), v[1:, 2:3, :])
     with pytest.raises(NativeOpsError, match="out of bounds for dimension 1"):
         ex.exec_custom("slice", [NDArray.from_numpy(v)], i_args=[0, 2, 0, 1, 3, 1])
+
+
+def test_zeros_as_and_ones_as(ex):
+    """generic/tensor/zeros_as.cpp:30-60, ones_as.cpp: the input's shape, the type of DArg 0 when given."""
+    x = NDArray.from_numpy(np.arange(12, dtype=np.float32).reshape(3, 4))
+    for name in ("zeros_as", "zeroslike", "zeros_like"):
+        z = ex.exec_custom(name, [x])[0]
+        assert z.dtype == FLOAT32 and list(z.shape) == [3, 4] and not z.to_numpy().any()
+    o = ex.exec_custom("ones_as", [x], d_args=[DOUBLE])[0]
+    assert o.dtype == DOUBLE and np.array_equal(o.to_numpy(), np.ones((3, 4)))
+    h = ex.exec_custom("ones_as", [x], d_args=[BFLOAT16])[0]
+    assert np.array_equal(h.to_float(), np.ones((3, 4), np.float32))
+    e = ex.exec_custom("zeros_as", [NDArray.empty((2, 0, 3), FLOAT32)])[0]
+    assert list(e.shape) == [2, 0, 3]
