@@ -19,6 +19,8 @@
 //                   logits / weights outputs: optional scale, clip to +-1e4, causal penalty.
 #include <algorithm>
 #include <cmath>
+#include <mutex>
+
 #include "device.h"
 #include "kernels.h"
 #include "mfma_tile.h"
@@ -524,11 +526,8 @@ static void launchFusedTyped(hipStream_t s, const void* q, const void* k, const 
   }
   constexpr size_t LDS = (size_t)2 * ((D / 64) * TileLayout<64, true>::SLOTS + TileLayout<D, false>::SLOTS) * 16;
   auto kern = attn_fused<T, D, FOLD>;
-  static bool attrSet = false;
-  if (!attrSet) {
-    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS));
-    attrSet = true;
-  }
+  static std::once_flag attrOnce;
+  std::call_once(attrOnce, [&] { HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS)); });
   hipLaunchKernelGGL(kern, dim3((unsigned)((LongType)(a.heavyFirst ? a.qTiles : a.perBatch) * d.B)), dim3(256), LDS, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
 }
 

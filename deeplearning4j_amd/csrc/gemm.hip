@@ -14,6 +14,8 @@
 //   gemv_*       M == 1 or N == 1: HBM-bound streaming of the matrix operand.
 //   gemm_simple  any float dtype, any strides (also fp64): 32x32 tile per block through LDS.  Correctness
 //                path for small, odd-shaped or oddly strided problems.
+#include <cstdarg>
+#include <cstdio>
 #include <cstdlib>
 
 #include <mutex>
@@ -42,6 +44,18 @@ struct GemmArgs {
   const void* bias;   // optional [N] row added to every output row (xw_plus_b), same type as C
 };
 typedef __attribute__((ext_vector_type(4))) float f32x4v;
+
+// Name of the kernel the calling thread's most recent matmul launched ("family<tile,flags>"), so that a test can assert
+// which instantiation its shape reached.
+static thread_local char g_lastGemmKernel[96] = "";
+__attribute__((format(printf, 1, 2))) static void noteKernel(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_lastGemmKernel, sizeof(g_lastGemmKernel), fmt, ap);
+  va_end(ap);
+}
+const char* lastGemmKernel() { return g_lastGemmKernel; }
+template <typename T> static const char* tname() { return std::is_same<T, bf16_t>::value ? "bf16" : std::is_same<T, f16_t>::value ? "f16" : std::is_same<T, float>::value ? "f32" : "f64"; }
 
 // operand offsets of batch entry bz (one or two batch levels)
 __device__ __forceinline__ void batchOffsets(const GemmArgs& g, LongType bz, LongType& oa, LongType& ob, LongType& oc) {
@@ -896,12 +910,11 @@ static void launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
               : useDeep ? gemm_mfma16q<T, BM, BN, WM, WN, A_KC, B_KC, 4>
               : usePipe ? gemm_mfma16p<T, BM, BN, WM, WN, A_KC, B_KC> : gemm_mfma16<T, BM, BN, WM, WN, A_KC, B_KC>;
   const int which = useFull ? 2 : useDeep ? 3 : usePipe ? 1 : 0;
-  static bool attrSet[4] = {false, false, false, false};
-  if (!attrSet[which]) {
-    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS));
-    attrSet[which] = true;
-  }
+  static std::once_flag attrOnce[4];
+  std::call_once(attrOnce[which], [&] { HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS)); });
   const unsigned tilesM = (unsigned)((g.M + BM - 1) / BM), tilesN = (unsigned)((g.N + BN - 1) / BN);
+  noteKernel("%s<%s,%dx%d,akc=%d,bkc=%d>%s", useFull ? "gemm_mfma16f" : useDeep ? "gemm_mfma16q" : usePipe ? "gemm_mfma16p" : "gemm_mfma16", tname<T>(), BM, BN,
+             (int)A_KC, (int)B_KC, splits > 1 ? "+splitk_finish" : "");
   hipLaunchKernelGGL(kern, dim3(tilesM * tilesN, (unsigned)splits, (unsigned)batch), dim3(NT), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tilesM, tilesN);
   if (splits > 1)
     hipLaunchKernelGGL((splitk_finish<T, BM, BN, WM, WN>), dim3(tilesM * tilesN, (BM / WM / 32) * (BN / WN / 32) * 4, (unsigned)batch), dim3(NT), 0, s, g, (T*)C, tilesM, tilesN);
@@ -918,12 +931,10 @@ static void launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const 
   if (direct && A_KC && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 64 == 0 && g.K >= 128) {
     constexpr size_t LDS = 2 * 2 * 256 * 8 * 16;
     auto kern = gemm_mfma16d<T, B_KC>;
-    static bool attrSet = false;
-    if (!attrSet) {
-      HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS));
-      attrSet = true;
-    }
+    static std::once_flag attrOnce;
+    std::call_once(attrOnce, [&] { HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS)); });
     const unsigned tM = (unsigned)(g.M / 256), tN = (unsigned)(g.N / 256);
+    noteKernel("gemm_mfma16d<%s,256x256,akc=1,bkc=%d>", tname<T>(), (int)B_KC);
     hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(512), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
     return;
   }
@@ -1179,10 +1190,12 @@ static void launchMfma32Cfg(hipStream_t s, const GemmArgs& g, const void* A, con
   const unsigned tilesM = (unsigned)((g.M + BM - 1) / BM), tilesN = (unsigned)((g.N + BN - 1) / BN);
   if (g.K >= 256 && g.M % BM == 0 && g.N % BN == 0 && g.K % 128 == 0) {
     constexpr int PD = BM * BN <= 64 * 64 ? 8 : 4;
+    noteKernel("gemm_mfma32q<f32,%dx%d,akc=%d,bkc=%d,pd=%d>", BM, BN, (int)A_KC, (int)B_KC, PD);
     hipLaunchKernelGGL((gemm_mfma32q<BM, BN, WM, WN, A_KC, B_KC, PD>), dim3(tilesM * tilesN, 1, (unsigned)batch), dim3(WM * WN * 64), 0, s, g,
                        (const float*)A, (const float*)B, (float*)C, tilesM, tilesN);
     return;
   }
+  noteKernel("gemm_mfma32<f32,%dx%d,akc=%d,bkc=%d>", BM, BN, (int)A_KC, (int)B_KC);
   hipLaunchKernelGGL((gemm_mfma32<BM, BN, WM, WN, A_KC, B_KC>), dim3(tilesM * tilesN, 1, (unsigned)batch), dim3(WM * WN * 64), 0, s, g,
                      (const float*)A, (const float*)B, (float*)C, tilesM, tilesN);
 }
@@ -1289,7 +1302,7 @@ static bool tryGemvRowdotPre(hipStream_t s, const GemmDesc& d, const void* A, co
   const LongType passes = (d.K / V + 63) / 64;
 #define ROWDOT_B(OPW, NL, HB) hipLaunchKernelGGL((gemv_rowdot_pre<T, OPW, NL, HB>), dim3((unsigned)(((d.N + OPW - 1) / OPW + 3) / 4)), dim3(256), 0, s, \
                                                  (const T*)B, d.bCol, (const T*)A, (T*)C, d.cCol, d.N, d.K, (const T*)d.bias)
-#define ROWDOT(OPW, NL) do { if (d.bias) ROWDOT_B(OPW, NL, true); else ROWDOT_B(OPW, NL, false); } while (0)
+#define ROWDOT(OPW, NL) do { noteKernel("gemv_rowdot_pre<%s,opw=%d,nl=%d>", tname<T>(), OPW, NL); if (d.bias) ROWDOT_B(OPW, NL, true); else ROWDOT_B(OPW, NL, false); } while (0)
   if (passes <= 2) ROWDOT(2, 2);
   else if (passes <= 4) ROWDOT(2, 4);
   else if (passes <= 6) ROWDOT(2, 6);
@@ -1350,13 +1363,13 @@ static bool tryGemv(hipStream_t s, const GemmDesc& d, const void* A, const void*
   if (d.M == 1 && d.N > 1) {
     // y[n] = sum_k a[k] * op(B)[k][n]
     if (d.bRow == 1 && tryGemvRowdotPre<T>(s, d, A, B, C)) return true;
-    if (d.bRow == 1) { hipLaunchKernelGGL((gemv_rowdot<T>), dim3((unsigned)((d.N + 3) / 4)), dim3(256), 0, s, (const T*)B, d.bCol, (const T*)A, d.aCol, (T*)C, d.cCol, d.N, d.K, d.alpha, d.beta, (const T*)d.bias); return true; }
-    if (d.bCol == 1) { hipLaunchKernelGGL((gemv_colsum<T>), dim3((unsigned)((d.N + 64 * V - 1) / (64 * V))), dim3(256), 0, s, (const T*)B, d.bRow, (const T*)A, d.aCol, (T*)C, d.cCol, d.N, d.K, d.alpha, d.beta, (const T*)d.bias); return true; }
+    if (d.bRow == 1) { noteKernel("gemv_rowdot<%s>", tname<T>()); hipLaunchKernelGGL((gemv_rowdot<T>), dim3((unsigned)((d.N + 3) / 4)), dim3(256), 0, s, (const T*)B, d.bCol, (const T*)A, d.aCol, (T*)C, d.cCol, d.N, d.K, d.alpha, d.beta, (const T*)d.bias); return true; }
+    if (d.bCol == 1) { noteKernel("gemv_colsum<%s>", tname<T>()); hipLaunchKernelGGL((gemv_colsum<T>), dim3((unsigned)((d.N + 64 * V - 1) / (64 * V))), dim3(256), 0, s, (const T*)B, d.bRow, (const T*)A, d.aCol, (T*)C, d.cCol, d.N, d.K, d.alpha, d.beta, (const T*)d.bias); return true; }
   }
   if (d.N == 1 && d.M > 1 && !d.bias) {
     // y[m] = sum_k op(A)[m][k] * b[k]
-    if (d.aCol == 1) { hipLaunchKernelGGL((gemv_rowdot<T>), dim3((unsigned)((d.M + 3) / 4)), dim3(256), 0, s, (const T*)A, d.aRow, (const T*)B, d.bRow, (T*)C, d.cRow, d.M, d.K, d.alpha, d.beta, (const T*)nullptr); return true; }
-    if (d.aRow == 1) { hipLaunchKernelGGL((gemv_colsum<T>), dim3((unsigned)((d.M + 64 * V - 1) / (64 * V))), dim3(256), 0, s, (const T*)A, d.aCol, (const T*)B, d.bRow, (T*)C, d.cRow, d.M, d.K, d.alpha, d.beta, (const T*)nullptr); return true; }
+    if (d.aCol == 1) { noteKernel("gemv_rowdot<%s>", tname<T>()); hipLaunchKernelGGL((gemv_rowdot<T>), dim3((unsigned)((d.M + 3) / 4)), dim3(256), 0, s, (const T*)A, d.aRow, (const T*)B, d.bRow, (T*)C, d.cRow, d.M, d.K, d.alpha, d.beta, (const T*)nullptr); return true; }
+    if (d.aRow == 1) { noteKernel("gemv_colsum<%s>", tname<T>()); hipLaunchKernelGGL((gemv_colsum<T>), dim3((unsigned)((d.M + 64 * V - 1) / (64 * V))), dim3(256), 0, s, (const T*)A, d.aCol, (const T*)B, d.bRow, (T*)C, d.cRow, d.M, d.K, d.alpha, d.beta, (const T*)nullptr); return true; }
   }
   return false;
 }
@@ -1377,6 +1390,7 @@ template <typename T>
 static void launchSimple(hipStream_t s, const void* A, const void* B, void* C, const GemmDesc& d) {
   GemmArgs g = toArgs(d);
   dim3 grid((unsigned)((d.N + 31) / 32), (unsigned)((d.M + 31) / 32), (unsigned)d.batch);
+  noteKernel("gemm_simple<%s>", tname<T>());
   hipLaunchKernelGGL((gemm_simple<T>), grid, dim3(256), 0, s, g, (const T*)A, (const T*)B, (T*)C);
 }
 
@@ -1498,6 +1512,7 @@ static void launchGemvStripM(hipStream_t s, const GemmArgs& g, const void* A, co
   // strips of 8 columns (one 16-byte piece of every weight row): N/8 blocks keep every CU busy even for N = 768
   constexpr int CW = 8, NWAVE = 4;
   const size_t lds = (size_t)NWAVE * M * CW * sizeof(float) + (size_t)M * g.K * sizeof(T);
+  noteKernel("gemv_strip<%s,m=%d>", tname<T>(), M);
   hipLaunchKernelGGL((gemv_strip<T, M, CW, NWAVE>), dim3((unsigned)(g.N / CW)), dim3(NWAVE * 64), lds, s, g, (const T*)A, (const T*)B, (T*)C);
 }
 // whether the strip kernel takes this product: a few dense rows, W row-major with aligned rows, plain C = A B (+ bias)
@@ -1519,7 +1534,9 @@ static bool tryGemvStrip(hipStream_t s, const GemmDesc& d, const void* A, const 
 }
 
 // ---- up to 32 rows of x against k-contiguous weights (a batched decode step's projections) -----------------------------
-// C[m][n] = sum_k x[m][k] * Wt[n][k] (+ bias[n]).  A block owns 32 output columns and all of K, in chunks of up to 768 k:
+// C[m][n] = sum_k x[m][k] * Wt[n][k] (+ bias[n]).  A block owns 32 output columns and all of K, in chunks of up to 384 k
+// (two chunks for d_model = 768; the LDS footprint stays under 64 KiB, which every launch path -- graph kernel nodes
+// included -- takes without a raised per-function limit):
 // every thread issues the chunk's loads at once (whole 128-byte lines: 8 lanes per row), parks them in LDS in the
 // [k-group][row] slot layout, and the four waves share the chunk's MFMA k-steps; the next chunk's loads are in flight
 // while the current one is multiplied.  The waves' 32x32 partial tiles are added up through LDS -- one launch, where the
@@ -1527,12 +1544,12 @@ static bool tryGemvStrip(hipStream_t s, const GemmDesc& d, const void* A, const 
 // Accumulator layout: lane (m = lane % 32, h = lane / 32), register r holds column 8 * (r / 4) + 4 * h + r % 4.
 template <typename T>
 __global__ __launch_bounds__(256) void gemm_skinny32(GemmArgs g, const T* __restrict__ X, const T* __restrict__ Wt, T* __restrict__ C) {
-  constexpr int CT = 12;                               // 64-k tiles per chunk
+  constexpr int CT = 6;                                // 64-k tiles per chunk
   constexpr int GROUP = 33;                            // slots per k-group (32 rows + 1: conflict-free column reads)
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   u32x4* sW = reinterpret_cast<u32x4*>(smem_raw);      // [CT * 8 k-groups][GROUP]
   u32x4* sX = sW + CT * 8 * GROUP;
-  float* red = reinterpret_cast<float*>(sX + CT * 8 * GROUP);   // [4 waves][16 registers][64 lanes]
+  float* red = reinterpret_cast<float*>(smem_raw);     // [4 waves][16 registers][64 lanes]; reuses sW once the K loop is over
   const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int lrow = t >> 3, lkg = t & 7;                // this thread's (row, k-group) inside every 64-k tile
   const LongType n0 = (LongType)blockIdx.x * 32;
@@ -1595,10 +1612,10 @@ static bool tryGemmSkinny(hipStream_t s, const GemmDesc& d, const void* A, const
   // longer K runs chunk after chunk in one block and measured slower than split-K over many blocks (14 vs 10 us at K = 3072)
   if (d.N % 32 != 0 || d.K % 64 != 0 || d.K > 1024 || d.aRow % 8 != 0 || d.bCol % 8 != 0 || d.cRow % 4 != 0) return false;
   if (((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) != 0 || (reinterpret_cast<uintptr_t>(C) & 7) != 0) return false;
-  constexpr size_t LDS = (size_t)2 * 12 * 8 * 33 * 16 + (size_t)4 * 16 * 64 * sizeof(float);
-  static std::once_flag once;
-  std::call_once(once, [] { HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny32<T>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS)); });
+  constexpr size_t LDS = (size_t)2 * 6 * 8 * 33 * 16;   // 50,688 B; the 16 KiB of partial tiles reuse it
+  static_assert(LDS <= 64 * 1024 && (size_t)4 * 16 * 64 * sizeof(float) <= LDS / 2, "gemm_skinny32 must fit the default dynamic LDS limit");
   GemmArgs g = toArgs(d);
+  noteKernel("gemm_skinny32<%s>", tname<T>());
   hipLaunchKernelGGL((gemm_skinny32<T>), dim3((unsigned)(d.N / 32)), dim3(256), LDS, s, g, (const T*)A, (const T*)B, (T*)C);
   return true;
 }

@@ -160,6 +160,8 @@ struct GemmDesc {
   const void* bias = nullptr;   // optional dense [N] row (type of C) added to every output row
 };
 void launchGemm(hipStream_t s, DataType dt, const void* A, const void* B, void* C, const GemmDesc& d);
+// name of the kernel the calling thread's most recent launchGemm chose
+const char* lastGemmKernel();
 
 // ---- attention -------------------------------------------------------------------------------------
 struct AttnDesc {

@@ -33,6 +33,38 @@ struct Nd4jHipLaunchContext : public LaunchContext {};
   }
 #define GUARD_END_VOID GUARD_END()
 
+// Every compute entry point runs under one process-wide lock: the library has one execution stream and one pair of
+// scratch buffers, and an op may be several launches that share scratch (split-K partial tiles and their finishing
+// kernel, cross-block reduction partials), so two caller threads must not interleave inside an op.
+static std::recursive_mutex& opMutex() {
+  static std::recursive_mutex m;
+  return m;
+}
+// The caller's stream, when it hands one in (extraPointers[1] of the legacy loops, setGraphContextCudaContext for
+// declarable ops; a device backend passes what lcExecutionStream returned, ref CudaExecutioner.java:641-649): work the
+// caller queued there is ordered before the op, and the op before whatever the caller queues next.  A null slot or the
+// library's own stream needs nothing.
+struct OpScope {
+  std::lock_guard<std::recursive_mutex> lock;
+  hipStream_t caller = nullptr;
+  explicit OpScope(void* streamPtr) : lock(opMutex()) {
+    if (streamPtr == nullptr || captureActive()) return;
+    hipStream_t cs = *reinterpret_cast<hipStream_t*>(streamPtr);
+    LaunchContext* lc = LaunchContext::defaultContext();
+    if (cs == nullptr || cs == lc->execStream) return;
+    caller = cs;
+    HIP_CHECK(hipEventRecord(lc->bridgeIn, caller));
+    HIP_CHECK(hipStreamWaitEvent(lc->execStream, lc->bridgeIn, 0));
+  }
+  ~OpScope() {
+    if (!caller) return;
+    LaunchContext* lc = LaunchContext::defaultContext();
+    if (hipEventRecord(lc->bridgeOut, lc->execStream) == hipSuccess) (void)hipStreamWaitEvent(caller, lc->bridgeOut, 0);
+  }
+};
+static void* callerStream(Nd4jPointer* extraPointers) { return extraPointers ? extraPointers[1] : nullptr; }
+#define OP_BEGIN(streamPtr) try { OpScope _opScope(streamPtr);
+
 static NDArray* arr(OpaqueNDArray a, const char* fn, const char* name) {
   if (a == nullptr) ND4J_THROW(std::string(fn) + ": " + name + " is null");
   return static_cast<NDArray*>(a);
@@ -465,8 +497,8 @@ static void runUnaryWithParams(const char* fn, Scalar2Kind k, NDArray* x, NDArra
   registerSpecialUse({z}, {x});
 }
 
-void execTransformStrict(Nd4jPointer*, int opNum, OpaqueNDArray xa, void* extraParams, OpaqueNDArray za) {
-  GUARD_BEGIN
+void execTransformStrict(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void* extraParams, OpaqueNDArray za) {
+  OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execTransformStrict", "x"); NDArray* z = arr(za, "execTransformStrict", "z");
   // X -> X over float types only (NativeOpExecutioner_transform.cpp:115-131)
   ND4J_REQUIRE(x->dataType() == z->dataType() && isFloatType(x->dataType()),
@@ -498,8 +530,8 @@ void execTransformStrict(Nd4jPointer*, int opNum, OpaqueNDArray xa, void* extraP
   runUnary("execTransformStrict", k, x, z);
   GUARD_END_VOID
 }
-void execTransformFloat(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
-  GUARD_BEGIN
+void execTransformFloat(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
+  OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execTransformFloat", "x"); NDArray* z = arr(za, "execTransformFloat", "z");
   ND4J_REQUIRE(isFloatType(z->dataType()), "NativeOpExecutioner::execTransformFloat requires Z to have floating point type");
   ND4J_REQUIRE(isFloatType(x->dataType()), "execTransformFloat: non-float inputs are not implemented in nd4j-hip");
@@ -511,8 +543,8 @@ void execTransformFloat(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, Opaque
   runUnary("execTransformFloat", k, x, z);
   GUARD_END_VOID
 }
-void execTransformSame(Nd4jPointer*, int opNum, OpaqueNDArray xa, void* extraParams, OpaqueNDArray za) {
-  GUARD_BEGIN
+void execTransformSame(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void* extraParams, OpaqueNDArray za) {
+  OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execTransformSame", "x"); NDArray* z = arr(za, "execTransformSame", "z");
   ND4J_REQUIRE(x->dataType() == z->dataType(), "NativeOpExecutioner::execTransformSame requires X & Z to have same type");
   ND4J_REQUIRE(isFloatType(x->dataType()), "execTransformSame: non-float types are not implemented in nd4j-hip");
@@ -533,8 +565,8 @@ void execTransformSame(Nd4jPointer*, int opNum, OpaqueNDArray xa, void* extraPar
   runUnary("execTransformSame", k, x, z);
   GUARD_END_VOID
 }
-void execTransformAny(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
-  GUARD_BEGIN
+void execTransformAny(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
+  OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execTransformAny", "x"); NDArray* z = arr(za, "execTransformAny", "z");
   ND4J_REQUIRE(opNum == 0, "execTransformAny: only Assign (opNum 0) exists (loops/legacy_ops.h:46)");
   runUnary("execTransformAny", U_IDENTITY, x, z);
@@ -555,8 +587,8 @@ static PairwiseKind pairwiseKind(int opNum) {
     default: ND4J_THROW("execPairwiseTransform: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
 }
-void execPairwiseTransform(Nd4jPointer*, int opNum, OpaqueNDArray xa, OpaqueNDArray ya, OpaqueNDArray za, void*) {
-  GUARD_BEGIN
+void execPairwiseTransform(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueNDArray ya, OpaqueNDArray za, void*) {
+  OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execPairwiseTransform", "x"); NDArray* y = arr(ya, "execPairwiseTransform", "y");
   NDArray* z = arr(za, "execPairwiseTransform", "z");
   // NativeOpExecutioner_pairwise_floats.cpp:34-57
@@ -592,8 +624,8 @@ static double hostScalar(NDArray* s) {
     default: ND4J_THROW("scalar operand has an unsupported data type");
   }
 }
-void execScalar(Nd4jPointer*, int opNum, OpaqueNDArray xa, OpaqueNDArray za, OpaqueNDArray sa, void*) {
-  GUARD_BEGIN
+void execScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueNDArray za, OpaqueNDArray sa, void*) {
+  OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execScalar", "x"); NDArray* z = arr(za, "execScalar", "z"); NDArray* s = arr(sa, "execScalar", "scalar");
   ND4J_REQUIRE(x->dataType() == z->dataType() && isFloatType(x->dataType()), "execScalar: nd4j-hip implements same-type float arrays only");
   PairwiseKind k;
@@ -640,8 +672,8 @@ static std::vector<LongType> hostDims(NDArray* dimension, int rank, const char* 
 
 // y is a smaller array whose dims line up with `dimension` of x (loops/cpu/broadcasting.hpp); realised as a
 // pairwise walk in which y's stride is 0 along every other dim
-void execBroadcast(Nd4jPointer*, int opNum, OpaqueNDArray xa, OpaqueNDArray ya, OpaqueNDArray za, void*, OpaqueNDArray da) {
-  GUARD_BEGIN
+void execBroadcast(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueNDArray ya, OpaqueNDArray za, void*, OpaqueNDArray da) {
+  OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execBroadcast", "x"); NDArray* y = arr(ya, "execBroadcast", "y"); NDArray* z = arr(za, "execBroadcast", "z");
   NDArray* dim = arr(da, "execBroadcast", "dimension");
   ND4J_REQUIRE(x->dataType() == z->dataType() && y->dataType() == z->dataType() && isFloatType(z->dataType()),
@@ -722,26 +754,26 @@ static ReduceKind reduceFloatKind(int opNum) {
     default: ND4J_THROW("execReduceFloat: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
 }
-void execReduceSame(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
-  GUARD_BEGIN
+void execReduceSame(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
+  OP_BEGIN(callerStream(extraPointers))
   if (xa == nullptr || za == nullptr) ND4J_THROW("execReduceSame: null pointer in input parameters");
   runReduce("execReduceSame", reduceSameKind(opNum), xa, za, {});
   GUARD_END_VOID
 }
-void execReduceSame2(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
-  GUARD_BEGIN
+void execReduceSame2(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
+  OP_BEGIN(callerStream(extraPointers))
   if (xa == nullptr || za == nullptr || da == nullptr) ND4J_THROW("execReduceSame2: null pointer in input parameters");
   runReduce("execReduceSame2", reduceSameKind(opNum), xa, za, hostDims(da, xa->rankOf(), "execReduceSame2"));
   GUARD_END_VOID
 }
-void execReduceFloat(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
-  GUARD_BEGIN
+void execReduceFloat(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
+  OP_BEGIN(callerStream(extraPointers))
   if (xa == nullptr || za == nullptr) ND4J_THROW("execReduceFloat: null pointer in input parameters");
   runReduce("execReduceFloat", reduceFloatKind(opNum), xa, za, {});
   GUARD_END_VOID
 }
-void execReduceFloat2(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
-  GUARD_BEGIN
+void execReduceFloat2(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
+  OP_BEGIN(callerStream(extraPointers))
   if (xa == nullptr || za == nullptr || da == nullptr) ND4J_THROW("execReduceFloat2: null pointer in input parameters");
   runReduce("execReduceFloat2", reduceFloatKind(opNum), xa, za, hostDims(da, xa->rankOf(), "execReduceFloat2"));
   GUARD_END_VOID
@@ -804,15 +836,15 @@ static MiscReduceKind summaryKind(int opNum) {
   }
 }
 extern "C" {
-void execSummaryStatsScalar(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, bool biasCorrected) {
-  GUARD_BEGIN
+void execSummaryStatsScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, bool biasCorrected) {
+  OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execSummaryStatsScalar", "x"); NDArray* z = arr(za, "execSummaryStatsScalar", "z");
   ND4J_REQUIRE(isFloatType(z->dataType()), "execSummaryStatsScalar: Z must have a floating point type");
   runReduceMisc("execSummaryStatsScalar", summaryKind(opNum), x, z, {}, biasCorrected);
   GUARD_END_VOID
 }
-void execSummaryStatsTad(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da, bool biasCorrected) {
-  GUARD_BEGIN
+void execSummaryStatsTad(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da, bool biasCorrected) {
+  OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execSummaryStatsTad", "x"); NDArray* z = arr(za, "execSummaryStatsTad", "z");
   ND4J_REQUIRE(isFloatType(z->dataType()), "execSummaryStatsTad: Z must have a floating point type");
   runReduceMisc("execSummaryStatsTad", summaryKind(opNum), x, z, hostDims(da, x->rankOf(), "execSummaryStatsTad"), biasCorrected);
@@ -828,13 +860,13 @@ static void reduceLong(const char* fn, int opNum, OpaqueNDArray xa, OpaqueNDArra
   }
   runReduceMisc(fn, k, x, z, da ? hostDims(da, x->rankOf(), fn) : std::vector<LongType>{}, false);
 }
-void execReduceLong(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
-  GUARD_BEGIN
+void execReduceLong(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
+  OP_BEGIN(callerStream(extraPointers))
   reduceLong("execReduceLong", opNum, xa, za, da);
   GUARD_END_VOID
 }
-void execReduceLong2(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
-  GUARD_BEGIN
+void execReduceLong2(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
+  OP_BEGIN(callerStream(extraPointers))
   reduceLong("execReduceLong2", opNum, xa, za, da);
   GUARD_END_VOID
 }
@@ -848,34 +880,34 @@ static void reduceBool(const char* fn, int opNum, OpaqueNDArray xa, OpaqueNDArra
   }
   runReduceMisc(fn, k, x, z, da ? hostDims(da, x->rankOf(), fn) : std::vector<LongType>{}, false);
 }
-void execReduceBool(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
-  GUARD_BEGIN
+void execReduceBool(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
+  OP_BEGIN(callerStream(extraPointers))
   reduceBool("execReduceBool", opNum, xa, za, da);
   GUARD_END_VOID
 }
-void execReduceBool2(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
-  GUARD_BEGIN
+void execReduceBool2(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
+  OP_BEGIN(callerStream(extraPointers))
   reduceBool("execReduceBool2", opNum, xa, za, da);
   GUARD_END_VOID
 }
-void execReduce3(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray ya, OpaqueNDArray za) {
-  GUARD_BEGIN
+void execReduce3(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray ya, OpaqueNDArray za) {
+  OP_BEGIN(callerStream(extraPointers))
   runReduce3("execReduce3", opNum, arr(xa, "execReduce3", "x"), arr(ya, "execReduce3", "y"), arr(za, "execReduce3", "z"), {});
   GUARD_END_VOID
 }
-void execReduce3Scalar(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray ya, OpaqueNDArray za) {
-  GUARD_BEGIN
+void execReduce3Scalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray ya, OpaqueNDArray za) {
+  OP_BEGIN(callerStream(extraPointers))
   runReduce3("execReduce3Scalar", opNum, arr(xa, "execReduce3Scalar", "x"), arr(ya, "execReduce3Scalar", "y"), arr(za, "execReduce3Scalar", "z"), {});
   GUARD_END_VOID
 }
-void execReduce3Tad(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray ya, OpaqueNDArray za, OpaqueNDArray da) {
-  GUARD_BEGIN
+void execReduce3Tad(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray ya, OpaqueNDArray za, OpaqueNDArray da) {
+  OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execReduce3Tad", "x");
   runReduce3("execReduce3Tad", opNum, x, arr(ya, "execReduce3Tad", "y"), arr(za, "execReduce3Tad", "z"), hostDims(da, x->rankOf(), "execReduce3Tad"));
   GUARD_END_VOID
 }
-void execTransformBool(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
-  GUARD_BEGIN
+void execTransformBool(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
+  OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execTransformBool", "x"); NDArray* z = arr(za, "execTransformBool", "z");
   ND4J_REQUIRE(z->dataType() == BOOL, std::string("NativeOpExecutioner::execTransformBool requires Z to have same boolean type, got ") + dtypeName(z->dataType()));
   ND4J_REQUIRE(isFloatType(x->dataType()), "execTransformBool: non-float inputs are not implemented in nd4j-hip");
@@ -923,14 +955,14 @@ void runIndexReduce(const char* fn, int opNum, NDArray* x, NDArray* z, const std
 }
 }  // namespace nd4jhip
 extern "C" {
-void execIndexReduce(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
-  GUARD_BEGIN
+void execIndexReduce(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
+  OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execIndexReduce", "x"); NDArray* z = arr(za, "execIndexReduce", "z"); NDArray* d = arr(da, "execIndexReduce", "dimension");
   runIndexReduce("execIndexReduce", opNum, x, z, hostDims(d, x->rankOf(), "execIndexReduce"));
   GUARD_END_VOID
 }
-void execIndexReduceScalar(Nd4jPointer*, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
-  GUARD_BEGIN
+void execIndexReduceScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
+  OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execIndexReduceScalar", "x"); NDArray* z = arr(za, "execIndexReduceScalar", "z");
   runIndexReduce("execIndexReduceScalar", opNum, x, z, {});
   GUARD_END_VOID
@@ -943,6 +975,10 @@ OpaqueContext* createGraphContext(int nodeId) {
   return c;
 }
 void deleteGraphContext(OpaqueContext* ptr) { delete ptr; }
+void setGraphContextCudaContext(OpaqueContext* ptr, void* stream, void* reductionPointer, void* allocationPointer) {
+  if (!ptr) return;
+  ptr->callerStream = stream; ptr->callerReduction = reductionPointer; ptr->callerAllocation = allocationPointer;
+}
 void markGraphContextInplace(OpaqueContext* ptr, bool v) { if (ptr) ptr->inplace = v; }
 static void setAt(std::vector<NDArray*>& v, int index, NDArray* a) {
   if (index < 0) ND4J_THROW("graph context: negative array index");
@@ -1021,8 +1057,8 @@ Nd4jLong dataTypeNativeAt(OpaqueContext* ptr, int idx) { return ptr && idx >= 0 
 const char* getAllCustomOps(void) { return ops::allCustomOps(); }
 Nd4jLong nd4jhipOpHash(const char* name) { return name ? ops::opHash(name) : 0; }
 
-Nd4jStatus execCustomOp2(Nd4jPointer*, Nd4jLong hash, OpaqueContext* ctx) {
-  GUARD_BEGIN
+Nd4jStatus execCustomOp2(Nd4jPointer* extraPointers, Nd4jLong hash, OpaqueContext* ctx) {
+  OP_BEGIN(ctx && ctx->callerStream ? ctx->callerStream : callerStream(extraPointers))
   ND4J_REQUIRE(ctx != nullptr, "execCustomOp2: context is null");
   const ops::OpDescriptor* op = ops::findOp(hash);
   if (!op) ND4J_THROW("execCustomOp2: unknown op hash " + std::to_string(hash) + " (op is not implemented in nd4j-hip)");
@@ -1054,28 +1090,34 @@ void nd4jhipSetSyncAfterCustomOp(int enable) { Environment::get().syncAfterCusto
 
 // ---- stream capture: a launch-bound sequence of ops recorded once and replayed as one HIP graph -----------------------
 namespace {
-struct CapturedGraph { hipGraph_t graph = nullptr; hipGraphExec_t exec = nullptr; };
-bool g_capturing = false;
+struct CapturedGraph {
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  CaptureRecord record;   // the buffers the recorded kernels read and write
+};
+CapturedGraph* g_openCapture = nullptr;
 bool g_syncBeforeCapture = true;
 }
 int nd4jhipGraphBeginCapture(void) {
-  GUARD_BEGIN
-  ND4J_REQUIRE(!g_capturing, "nd4jhipGraphBeginCapture: a capture is already in progress");
+  OP_BEGIN(nullptr)
+  ND4J_REQUIRE(!captureActive(), "nd4jhipGraphBeginCapture: a capture is already in progress");
   // every op call between begin and end records its kernels instead of running them: nothing may wait on the stream
   g_syncBeforeCapture = Environment::get().syncAfterCustomOp;
   Environment::get().syncAfterCustomOp = false;
   HIP_CHECK(hipStreamSynchronize(execStream()));
   HIP_CHECK(hipStreamBeginCapture(execStream(), hipStreamCaptureModeRelaxed));
-  g_capturing = true;
+  g_openCapture = new CapturedGraph();
+  setActiveCapture(&g_openCapture->record);
   return 0;
   GUARD_END(1)
 }
 Nd4jPointer nd4jhipGraphEndCapture(void) {
-  GUARD_BEGIN
-  ND4J_REQUIRE(g_capturing, "nd4jhipGraphEndCapture: no capture in progress");
-  g_capturing = false;
+  OP_BEGIN(nullptr)
+  ND4J_REQUIRE(captureActive() && g_openCapture, "nd4jhipGraphEndCapture: no capture in progress");
+  CapturedGraph* cg = g_openCapture;
+  g_openCapture = nullptr;
+  setActiveCapture(nullptr);
   Environment::get().syncAfterCustomOp = g_syncBeforeCapture;
-  CapturedGraph* cg = new CapturedGraph();
   hipError_t e = hipStreamEndCapture(execStream(), &cg->graph);
   if (e != hipSuccess || cg->graph == nullptr) {
     delete cg;
@@ -1092,10 +1134,24 @@ Nd4jPointer nd4jhipGraphEndCapture(void) {
   GUARD_END(nullptr)
 }
 int nd4jhipGraphLaunch(Nd4jPointer graph) {
-  GUARD_BEGIN
+  OP_BEGIN(nullptr)
   ND4J_REQUIRE(graph != nullptr, "nd4jhipGraphLaunch: graph is null");
-  ND4J_REQUIRE(!g_capturing, "nd4jhipGraphLaunch: a capture is in progress");
-  HIP_CHECK(hipGraphLaunch(static_cast<CapturedGraph*>(graph)->exec, execStream()));
+  ND4J_REQUIRE(!captureActive(), "nd4jhipGraphLaunch: a capture is in progress");
+  CapturedGraph* cg = static_cast<CapturedGraph*>(graph);
+  // what prepareSpecialUse does per op, for the whole recorded sequence: an input (or a partly written output) whose
+  // host copy is newer goes to the device first
+  for (auto& b : cg->record.reads) {
+    ND4J_REQUIRE(!b->closed, "nd4jhipGraphLaunch: a buffer the graph reads has been closed");
+    b->syncToSpecial();
+  }
+  for (auto& b : cg->record.writes) {
+    ND4J_REQUIRE(!b->closed && b->special, "nd4jhipGraphLaunch: a buffer the graph writes has been closed");
+    if (!b->isSpecialActual()) b->syncToSpecial();
+  }
+  HIP_CHECK(hipGraphLaunch(cg->exec, execStream()));
+  // ... and what registerSpecialUse does: outputs are now newest on the device
+  for (auto& b : cg->record.reads) b->tickReadSpecial();
+  for (auto& b : cg->record.writes) b->tickWriteSpecial();
   return 0;
   GUARD_END(1)
 }
@@ -1106,6 +1162,7 @@ void nd4jhipGraphDestroy(Nd4jPointer graph) {
   if (cg->graph) (void)hipGraphDestroy(cg->graph);
   delete cg;
 }
+const char* nd4jhipLastGemmKernel(void) { return lastGemmKernel(); }
 const char* nd4jhipBuildInfo(void) { return "nd4j-hip gfx950 (hand-written HIP kernels; no CPU fallback)"; }
 
 }  // extern "C"

@@ -23,13 +23,12 @@ ErrorReference& errorRef() {
 void throwError(const std::string& msg) { throw std::runtime_error(msg); }
 
 Environment& Environment::get() {
-  static Environment e;
-  static bool init = false;
-  if (!init) {
-    init = true;
-    if (const char* v = getenv("ND4JHIP_VERBOSE")) e.verbose = atoi(v) != 0;
-    if (const char* v = getenv("ND4JHIP_SYNC_CUSTOM_OPS")) e.syncAfterCustomOp = atoi(v) != 0;
-  }
+  static Environment e = [] {
+    Environment v;
+    if (const char* s = getenv("ND4JHIP_VERBOSE")) v.verbose = atoi(s) != 0;
+    if (const char* s = getenv("ND4JHIP_SYNC_CUSTOM_OPS")) v.syncAfterCustomOp = atoi(s) != 0;
+    return v;
+  }();
   return e;
 }
 
@@ -113,14 +112,13 @@ std::vector<LongType> scalarShapeInfo(DataType dt) { return makeShapeInfo(dt, 'c
 
 // ---- launch context -------------------------------------------------------------------------------
 bool deviceAvailable() {
-  static int state = -1;
-  if (state < 0) {
+  static const bool available = [] {
     int n = 0;
     hipError_t e = hipGetDeviceCount(&n);
     if (e != hipSuccess) { (void)hipGetLastError(); n = 0; }
-    state = n > 0 ? 1 : 0;
-  }
-  return state == 1;
+    return n > 0;
+  }();
+  return available;
 }
 
 void LaunchContext::init() {
@@ -133,6 +131,8 @@ void LaunchContext::init() {
   HIP_CHECK(hipMalloc(&reductionBuffer, REDUCTION_BYTES));
   HIP_CHECK(hipMalloc(&allocationBuffer, ALLOCATION_BYTES));
   HIP_CHECK(hipHostMalloc(&scalarBuffer, 256, hipHostMallocDefault));
+  HIP_CHECK(hipEventCreateWithFlags(&bridgeIn, hipEventDisableTiming));
+  HIP_CHECK(hipEventCreateWithFlags(&bridgeOut, hipEventDisableTiming));
   ready = true;
 }
 LaunchContext* LaunchContext::defaultContext() {
@@ -224,6 +224,18 @@ void DataBuffer::close() {
   primary = special = nullptr;
 }
 
+// ---- stream capture ---------------------------------------------------------------------------------
+static std::atomic<CaptureRecord*> g_capture{nullptr};
+bool captureActive() { return g_capture.load(std::memory_order_acquire) != nullptr; }
+CaptureRecord* activeCapture() { return g_capture.load(std::memory_order_acquire); }
+void setActiveCapture(CaptureRecord* rec) { g_capture.store(rec, std::memory_order_release); }
+static void noteUnique(std::vector<std::shared_ptr<DataBuffer>>& v, const std::shared_ptr<DataBuffer>& b) {
+  for (auto& e : v) if (e.get() == b.get()) return;
+  v.push_back(b);
+}
+void CaptureRecord::noteRead(const std::shared_ptr<DataBuffer>& b) { noteUnique(reads, b); }
+void CaptureRecord::noteWrite(const std::shared_ptr<DataBuffer>& b) { noteUnique(writes, b); }
+
 // ---- array handle -------------------------------------------------------------------------------
 void* NDArray::buffer() const {
   if (!buf || !buf->primary) return nullptr;
@@ -250,6 +262,10 @@ template <typename W, typename R>
 static void registerImpl(const W& writes, const R& reads) {
   for (NDArray* a : reads) if (a && a->buf) a->buf->tickReadSpecial();
   for (NDArray* a : writes) if (a && a->buf) a->buf->tickWriteSpecial();
+  if (CaptureRecord* rec = activeCapture()) {
+    for (NDArray* a : reads) if (a && a->buf) rec->noteRead(a->buf);
+    for (NDArray* a : writes) if (a && a->buf) rec->noteWrite(a->buf);
+  }
 }
 void prepareSpecialUse(std::initializer_list<NDArray*> w, std::initializer_list<NDArray*> r) { prepareImpl(w, r); }
 void registerSpecialUse(std::initializer_list<NDArray*> w, std::initializer_list<NDArray*> r) { registerImpl(w, r); }
@@ -258,6 +274,8 @@ void registerSpecialUse(const std::vector<NDArray*>& w, const std::vector<NDArra
 
 // ---- descriptor cache ---------------------------------------------------------------------------
 const LongType* ConstantShapeBuffer::special() {
+  static std::mutex m;
+  std::lock_guard<std::mutex> g(m);
   if (!device) {
     HIP_CHECK(hipMalloc((void**)&device, host.size() * sizeof(LongType)));
     HIP_CHECK(hipMemcpy(device, host.data(), host.size() * sizeof(LongType), hipMemcpyHostToDevice));
@@ -283,6 +301,8 @@ ConstantShapeBuffer* cachedShapeBuffer(const LongType* si) {
 
 // ---- TAD pack -------------------------------------------------------------------------------------
 const LongType* TadPack::specialOffsets() {
+  static std::mutex m;
+  std::lock_guard<std::mutex> g(m);
   if (!deviceOffsets && !offsets.empty()) {
     HIP_CHECK(hipMalloc((void**)&deviceOffsets, offsets.size() * sizeof(LongType)));
     HIP_CHECK(hipMemcpy(deviceOffsets, offsets.data(), offsets.size() * sizeof(LongType), hipMemcpyHostToDevice));

@@ -52,6 +52,7 @@ struct LaunchContext {
   void* reductionBuffer = nullptr;   // device, REDUCTION_BYTES
   void* allocationBuffer = nullptr;  // device, ALLOCATION_BYTES
   void* scalarBuffer = nullptr;      // pinned host, 256 B
+  hipEvent_t bridgeIn = nullptr, bridgeOut = nullptr;   // order a caller-owned stream against execStream
   int deviceId = 0;
   bool ready = false;
   static constexpr size_t REDUCTION_BYTES = 8u << 20;
@@ -124,6 +125,18 @@ struct NDArray {
   template <typename T> T* hostAs() const { return reinterpret_cast<T*>(buffer()); }
 };
 
+// ---- stream capture ---------------------------------------------------------------------------------
+// While a capture is open, ops record their kernels instead of running them, and prepare/registerSpecialUse note which
+// buffers the recorded kernels read and write, so that a replay can bring inputs up to date and stamp outputs.
+struct CaptureRecord {
+  std::vector<std::shared_ptr<DataBuffer>> reads, writes;
+  void noteRead(const std::shared_ptr<DataBuffer>& b);
+  void noteWrite(const std::shared_ptr<DataBuffer>& b);
+};
+bool captureActive();
+CaptureRecord* activeCapture();
+void setActiveCapture(CaptureRecord* rec);   // null: no capture open
+
 // prepareSpecialUse / registerSpecialUse (array/cuda/NDArray.cu:331-357)
 void prepareSpecialUse(std::initializer_list<NDArray*> writes, std::initializer_list<NDArray*> reads);
 void registerSpecialUse(std::initializer_list<NDArray*> writes, std::initializer_list<NDArray*> reads);
@@ -169,6 +182,10 @@ struct Context {
   bool shapeFunctionOverride = false;
   int execMode = 0;
   LongType rootSeed = 0, nodeSeed = 0;
+  // what setGraphContextCudaContext handed in (graph/Context.h setCudaContext): pointer to the caller's stream, its scratch
+  void* callerStream = nullptr;
+  void* callerReduction = nullptr;
+  void* callerAllocation = nullptr;
   int width() const { return (int)inputs.size(); }
   NDArray* input(int i) const;
   NDArray* output(int i) const;

@@ -172,6 +172,8 @@ _SIGS = {
     "nd4jhipGraphLaunch": (ctypes.c_int, [c_ptr]),
     "nd4jhipGraphDestroy": (None, [c_ptr]),
     "nd4jhipBuildInfo": (ctypes.c_char_p, []),
+    "nd4jhipLastGemmKernel": (ctypes.c_char_p, []),
+    "setGraphContextCudaContext": (None, [c_ptr, c_ptr, c_ptr, c_ptr]),
 }
 
 

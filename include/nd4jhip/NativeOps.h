@@ -197,6 +197,10 @@ ND4JHIP_EXPORT void setGraphContextOutputArraysArr(OpaqueContext* ptr, int numAr
 ND4JHIP_EXPORT void setGraphContextTArguments(OpaqueContext* ptr, double* arguments, int numberOfArguments);   /* ref :433 */
 ND4JHIP_EXPORT void setGraphContextIArguments(OpaqueContext* ptr, Nd4jLong* arguments, int numberOfArguments); /* ref :434 */
 ND4JHIP_EXPORT void setGraphContextBArguments(OpaqueContext* ptr, bool* arguments, int numberOfArguments);     /* ref :435 */
+/* The caller's stream (pointer to it, as lcExecutionStream returns) and scratch for this op (ref CudaOpContext.java:291).  Work queued
+ * on that stream is ordered before the op and the op before what the caller queues next; kernels run on the library's own
+ * execution stream and use its own scratch. */
+ND4JHIP_EXPORT void setGraphContextCudaContext(OpaqueContext* ptr, void* stream, void* reductionPointer, void* allocationPointer);  /* ref :80 */
 ND4JHIP_EXPORT void setGraphContextDArguments(OpaqueContext* ptr, int* arguments, int numberOfArguments);      /* ref :436 */
 ND4JHIP_EXPORT void ctxAllowHelpers(OpaqueContext* ptr, bool reallyAllow);             /* ref :464 */
 ND4JHIP_EXPORT void ctxShapeFunctionOverride(OpaqueContext* ptr, bool reallyOverride); /* ref :458 */
@@ -233,12 +237,19 @@ ND4JHIP_EXPORT void nd4jhipSetSyncAfterCustomOp(int enable);
 /* Stream capture for launch-bound op sequences (a decode step is ~150 kernels of a few microseconds each): every op
  * call between Begin and End is recorded on the execution stream instead of run; End returns a handle (null + error slot
  * when an op waited on the stream, copied synchronously or allocated, which invalidates a capture); Launch replays the
- * recorded kernels with the arguments they were recorded with.  Build arrays, views and OpContexts before Begin. */
+ * recorded kernels with the arguments they were recorded with.  Build arrays, views and OpContexts before Begin.
+ * Launch keeps the buffers' host/device stamps as the recorded op calls would: a buffer the graph reads whose host copy
+ * is newer is uploaded first, and every buffer the graph writes counts as device-written afterwards, so dbSyncToPrimary
+ * after a replay returns that replay's values.  A capture is process-wide: ops other threads issue between Begin and End
+ * are recorded too. */
 ND4JHIP_EXPORT int nd4jhipGraphBeginCapture(void);
 ND4JHIP_EXPORT Nd4jPointer nd4jhipGraphEndCapture(void);
 ND4JHIP_EXPORT int nd4jhipGraphLaunch(Nd4jPointer graph);
 ND4JHIP_EXPORT void nd4jhipGraphDestroy(Nd4jPointer graph);
 ND4JHIP_EXPORT const char* nd4jhipBuildInfo(void);
+/* Name ("family<type,tile,flags>") of the kernel the calling thread's most recent matmul / xw_plus_b launched; lets a
+ * test assert that its shape reached the instantiation it means to check. */
+ND4JHIP_EXPORT const char* nd4jhipLastGemmKernel(void);
 
 #ifdef __cplusplus
 }

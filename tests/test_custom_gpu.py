@@ -385,10 +385,9 @@ def test_layer_norm_channels_first_and_views(ex, oracle):
 # ---- attention -------------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype,tol", [(FLOAT32, 1e-4), (HALF, 1e-2), (BFLOAT16, 1e-2)])
 @pytest.mark.parametrize("causal", [False, True])
-@pytest.mark.parametrize("B,Tq,Tv,D", [(3, 64, 64, 64), (2, 100, 100, 64), (2, 128, 256, 64), (1, 37, 91, 32)])
+@pytest.mark.parametrize("B,Tq,Tv,D", [(3, 64, 64, 64), (2, 100, 100, 64), (2, 128, 256, 64), (1, 37, 91, 32), (2, 300, 72, 64), (1, 520, 200, 64)])
 def test_attention_vs_oracle(ex, oracle, dtype, tol, causal, B, Tq, Tv, D):
-    if causal and Tq != Tv:
-        pytest.skip("causal mask is exercised on square score matrices")
+    # causal with Tq != Tv: key j is visible to query i iff j <= i (the lower-triangular mask of AttentionHelper.cpp:70-79)
     rng = np.random.default_rng(B * Tq + D)
     oq, dq = _pair(oracle, rng.normal(0, 1, (B, Tq, D)), dtype)
     ok, dk = _pair(oracle, rng.normal(0, 1, (B, Tv, D)), dtype)

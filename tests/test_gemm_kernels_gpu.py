@@ -1,0 +1,144 @@
+"""Every matmul kernel instantiation the dispatcher can pick for BASELINE config 2 (and the sizes around it), checked at
+its real shape.
+
+Each case asserts which kernel ran (`nd4jhipLastGemmKernel`), so that a change of the dispatch rules cannot silently
+leave a kernel untested, then checks
+  * 16 whole rows and 16 whole columns of the result against an fp64 product of the (rounded) inputs -- every tile row
+    and every tile column of the launch grid is crossed;
+  * whole-result identities: transposeB == plain B, transposeA == plain A, and fp16 == bf16 within the 16-bit gate.
+Gates (north star): fp32 1e-4, fp16 / bf16 1e-2.  Flag combinations follow the reference's matmul tests
+(libnd4j/tests_cpu/layers_tests/DeclarableOpsTests14.cpp:601-1260: transX / transY, c order).
+"""
+import math
+
+import numpy as np
+import pytest
+
+from conftest import assert_close
+from deeplearning4j_amd.ndarray import BFLOAT16, FLOAT32, HALF, NDArray, bf16_bits_to_f32, f32_to_bf16_bits
+
+pytestmark = pytest.mark.gpu
+
+TOL = {FLOAT32: 1e-4, HALF: 1e-2, BFLOAT16: 1e-2}
+
+
+def _device(a, dtype):
+    """(device array, fp64 view of the values it holds)"""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    if dtype == BFLOAT16:
+        bits = f32_to_bf16_bits(a)
+        return NDArray.from_numpy(bits, BFLOAT16), bf16_bits_to_f32(bits).astype(np.float64)
+    if dtype == HALF:
+        h = a.astype(np.float16)
+        return NDArray.from_numpy(h), h.astype(np.float64)
+    return NDArray.from_numpy(a), a.astype(np.float64)
+
+
+def _last_kernel(ex):
+    return ex.L.nd4jhipLastGemmKernel().decode()
+
+
+def _run(ex, A, B, i_args, expect_kernel):
+    z = ex.exec_custom("matmul", [A, B], i_args=i_args)[0]
+    name = _last_kernel(ex)
+    assert name.startswith(expect_kernel), "shape reached %s, the test means to check %s" % (name, expect_kernel)
+    return z.to_float()
+
+
+def _check_rows_cols(z, a64, b64, tol, rng, what):
+    M, N = z.shape
+    rows = rng.choice(M, min(16, M), replace=False)
+    cols = rng.choice(N, min(16, N), replace=False)
+    assert_close(z[rows], a64[rows] @ b64, tol, tol, what + ": sampled rows")
+    assert_close(z[:, cols], a64 @ b64[:, cols], tol, tol, what + ": sampled columns")
+
+
+# (dtype, M, N, K, kernel for plain B, kernel for transposeB, kernel for transposeA or None)
+CASES = [
+    # BASELINE config 2 at 4096^3
+    (FLOAT32, 4096, 4096, 4096, "gemm_mfma32q<f32,128x128,akc=1,bkc=0,pd=4>", "gemm_mfma32q<f32,128x128,akc=1,bkc=1,pd=4>", "gemm_mfma32q<f32,128x128,akc=0,bkc=0,pd=4>"),
+    (HALF, 4096, 4096, 4096, "gemm_mfma16d<f16,256x256,akc=1,bkc=0>", "gemm_mfma16d<f16,256x256,akc=1,bkc=1>", "gemm_mfma16f<f16,256x256,akc=0,bkc=0>"),
+    (BFLOAT16, 4096, 4096, 4096, "gemm_mfma16d<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1>", "gemm_mfma16f<bf16,256x256,akc=0,bkc=0>"),
+    # BASELINE config 2 at 1024^3
+    (FLOAT32, 1024, 1024, 1024, "gemm_mfma32q<f32,64x64,akc=1,bkc=0,pd=8>", "gemm_mfma32q<f32,64x64,akc=1,bkc=1,pd=8>", "gemm_mfma32q<f32,64x64,akc=0,bkc=0,pd=8>"),
+    (HALF, 1024, 1024, 1024, "gemm_mfma16q<f16,64x64,akc=1,bkc=0>", "gemm_mfma16q<f16,64x64,akc=1,bkc=1>", "gemm_mfma16q<f16,64x64,akc=0,bkc=0>"),
+    (BFLOAT16, 1024, 1024, 1024, "gemm_mfma16q<bf16,64x64,akc=1,bkc=0>", "gemm_mfma16q<bf16,64x64,akc=1,bkc=1>", "gemm_mfma16q<bf16,64x64,akc=0,bkc=0>"),
+    # the 128 x 128 configuration (2048-class sizes), whole tiles
+    (BFLOAT16, 2048, 2048, 2048, "gemm_mfma16f<bf16,128x128,akc=1,bkc=0>", "gemm_mfma16f<bf16,128x128,akc=1,bkc=1>", "gemm_mfma16f<bf16,128x128,akc=0,bkc=0>"),
+    (HALF, 2048, 2048, 1024, "gemm_mfma16f<f16,128x128,akc=1,bkc=0>", "gemm_mfma16f<f16,128x128,akc=1,bkc=1>", None),
+    # ragged edges on the large tiles (bounds-handling kernel)
+    (BFLOAT16, 3600, 3704, 1000, "gemm_mfma16p<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16p<bf16,256x256,akc=1,bkc=1>", "gemm_mfma16p<bf16,256x256,akc=0,bkc=0>"),
+    (HALF, 1800, 1800, 520, "gemm_mfma16p<f16,128x128,akc=1,bkc=0>", "gemm_mfma16p<f16,128x128,akc=1,bkc=1>", None),
+    (BFLOAT16, 1104, 904, 1000, "gemm_mfma16p<bf16,64x64,akc=1,bkc=0>", "gemm_mfma16p<bf16,64x64,akc=1,bkc=1>", None),
+    # K a multiple of 256 but not of 512: the four-deep prefetch ends in the middle of its ring
+    (BFLOAT16, 1024, 1024, 768, "gemm_mfma16q<bf16,64x64,akc=1,bkc=0>", "gemm_mfma16q<bf16,64x64,akc=1,bkc=1>", None),
+    (FLOAT32, 1024, 1024, 384, "gemm_mfma32q<f32,64x64,akc=1,bkc=0,pd=8>", "gemm_mfma32q<f32,64x64,akc=1,bkc=1,pd=8>", None),
+    (FLOAT32, 2048, 2048, 640, "gemm_mfma32q<f32,128x128,akc=1,bkc=0,pd=4>", "gemm_mfma32q<f32,128x128,akc=1,bkc=1,pd=4>", None),
+    # fp32 ragged
+    (FLOAT32, 1100, 900, 1000, "gemm_mfma32<f32,64x64,akc=1,bkc=0>", "gemm_mfma32<f32,64x64,akc=1,bkc=1>", None),
+    (FLOAT32, 2100, 2052, 520, "gemm_mfma32<f32,128x128,akc=1,bkc=0>", "gemm_mfma32<f32,128x128,akc=1,bkc=1>", "gemm_mfma32<f32,128x128,akc=0,bkc=0>"),
+]
+
+
+@pytest.mark.parametrize("dtype,M,N,K,kern_plain,kern_tb,kern_ta", CASES,
+                         ids=["%s-%dx%dx%d" % ({FLOAT32: "f32", HALF: "f16", BFLOAT16: "bf16"}[c[0]], c[1], c[2], c[3]) for c in CASES])
+def test_matmul_kernel_at_real_shape(ex, dtype, M, N, K, kern_plain, kern_tb, kern_ta):
+    rng = np.random.default_rng(2002 + M + 3 * N + 7 * K + dtype)
+    tol = TOL[dtype]
+    a = rng.normal(0, 1 / math.sqrt(K), (M, K)).astype(np.float32)
+    b = rng.normal(0, 1 / math.sqrt(K), (K, N)).astype(np.float32)
+    A, a64 = _device(a, dtype)
+    B, b64 = _device(b, dtype)
+    z = _run(ex, A, B, [0, 0], kern_plain)
+    _check_rows_cols(z, a64, b64, tol, rng, "plain")
+    Bt, _ = _device(b.T, dtype)
+    zt = _run(ex, A, Bt, [0, 1], kern_tb)
+    _check_rows_cols(zt, a64, b64, tol, rng, "transposeB")
+    assert_close(zt, z, tol, tol, "transposeB agrees with plain B over the whole result")
+    if kern_ta:
+        At, _ = _device(a.T, dtype)
+        za = _run(ex, At, B, [1, 0], kern_ta)
+        _check_rows_cols(za, a64, b64, tol, rng, "transposeA")
+        assert_close(za, z, tol, tol, "transposeA agrees with plain A over the whole result")
+
+
+@pytest.mark.parametrize("n", [1024, 4096])
+def test_fp16_and_bf16_agree(ex, n):
+    """Inputs exactly representable in both 16-bit types (multiples of 1/8 in [-2, 2]): fp16 and bf16 kernels multiply
+    the same numbers, so their results differ only by the final rounding."""
+    rng = np.random.default_rng(n)
+    a = (rng.integers(-16, 17, (n, n)) / 8.0).astype(np.float32) / math.sqrt(n)
+    b = (rng.integers(-16, 17, (n, n)) / 8.0).astype(np.float32)
+    # a / sqrt(n) stays exact in both types for n a power of four
+    Ah, a64 = _device(a, HALF)
+    Bh, b64 = _device(b, HALF)
+    Ab, a64b = _device(a, BFLOAT16)
+    Bb, b64b = _device(b, BFLOAT16)
+    assert np.array_equal(a64, a64b) and np.array_equal(b64, b64b)
+    zh = ex.exec_custom("matmul", [Ah, Bh])[0].to_float()
+    kh = _last_kernel(ex)
+    zb = ex.exec_custom("matmul", [Ab, Bb])[0].to_float()
+    kb = _last_kernel(ex)
+    assert "<f16," in kh and "<bf16," in kb and kh.split("<")[0] == kb.split("<")[0]
+    assert_close(zh, zb, 1e-2, 1e-2, "fp16 result against bf16 result")
+    rows = rng.choice(n, 8, replace=False)
+    assert_close(zh[rows], a64[rows] @ b64, 1e-2, 1e-2, "fp16 sampled rows")
+
+
+def test_alpha_beta_on_the_direct_kernel(ex):
+    """C = alpha A B + beta C through the 256 x 256 direct-to-LDS kernel (its epilogue reads C)."""
+    rng = np.random.default_rng(19)
+    M, N, K = 512, 768, 512
+    # a 256-tile launch needs at least 192 tiles: batch the problem
+    batch = 32
+    a = rng.normal(0, 1 / math.sqrt(K), (batch, M, K)).astype(np.float32)
+    b = rng.normal(0, 1 / math.sqrt(K), (batch, K, N)).astype(np.float32)
+    c0 = rng.normal(0, 1, (batch, M, N)).astype(np.float32)
+    A, a64 = _device(a, BFLOAT16)
+    B, b64 = _device(b, BFLOAT16)
+    C, c64 = _device(c0, BFLOAT16)
+    ex.exec_custom("matmul", [A, B], [C], t_args=[0.5, 2.0])
+    assert _last_kernel(ex).startswith("gemm_mfma16d<bf16,256x256,akc=1,bkc=0>"), _last_kernel(ex)
+    got = C.to_float()
+    for bi in (0, 13, 31):
+        assert_close(got[bi], 0.5 * (a64[bi] @ b64[bi]) + 2.0 * c64[bi], 1e-2, 2e-2, "batch %d" % bi)
