@@ -104,6 +104,13 @@ struct ReducePlan {
 
 void launchReduce(hipStream_t s, ReduceKind k, DataType xdt, DataType zdt, const void* x, void* z, const ReducePlan& p,
                   void* scratch, size_t scratchBytes);
+// Full reduction of a dense vector x[n] into z[1] whose cross-block partials live in a fixed device array instead of
+// allocated scratch: no allocation on any path.  reduceNoAllocScratch() resolves that array's address on the current
+// device (once per device); same kernels and split rule as launchReduce, hence the same bits.
+constexpr size_t NOALLOC_SCRATCH_BYTES = 64 * 1024;
+constexpr LongType NOALLOC_MAX_ELEMENTS = (1LL << 31) - 1;
+void* reduceNoAllocScratch();
+void launchReduceScalarNoAlloc(hipStream_t s, ReduceKind k, DataType dt, const void* x, LongType n, void* z);
 // zdt: the float type for variance / standard deviation, INT64 for counts, BOOL for Any / All
 void launchReduceMisc(hipStream_t s, MiscReduceKind k, DataType xdt, DataType zdt, const void* x, void* z, const ReducePlan& p,
                       bool biasCorrected, void* scratch, size_t scratchBytes, const void* y = nullptr, DataType ydt = FLOAT32,

@@ -77,6 +77,7 @@ extern "C" {
 void initializeDevicesAndFunctions(void) {
   GUARD_BEGIN
   LaunchContext::defaultContext();
+  (void)reduceNoAllocScratch();   // address of the fixed partials array on this device, for nd4jhipReduceSameScalarNoAlloc
   GUARD_END_VOID
 }
 void initializeShapeCache(void) {}
@@ -1163,6 +1164,23 @@ void nd4jhipGraphDestroy(Nd4jPointer graph) {
   delete cg;
 }
 const char* nd4jhipLastGemmKernel(void) { return lastGemmKernel(); }
+
+// execReduceSame (full reduction of a dense array) for callers that cannot allocate: plain device pointers in, one
+// element out, partials in a fixed device array.  No hipMalloc / hipFree on any path, the error paths included.
+int nd4jhipReduceSameScalarNoAlloc(Nd4jPointer stream, int opNum, int dataType, const void* dX, Nd4jLong length, void* dZ) {
+  OP_BEGIN(nullptr)
+  LaunchContext* lc = LaunchContext::ifReady();
+  ND4J_REQUIRE(lc != nullptr, "nd4jhipReduceSameScalarNoAlloc: call initializeDevicesAndFunctions first (initialisation allocates, this call must not)");
+  ND4J_REQUIRE(!captureActive() || stream != nullptr, "nd4jhipReduceSameScalarNoAlloc: pass the capturing stream");
+  ND4J_REQUIRE(dX != nullptr && dZ != nullptr, "nd4jhipReduceSameScalarNoAlloc: null device pointer");
+  const DataType dt = (DataType)dataType;
+  ND4J_REQUIRE(isFloatType(dt), "nd4jhipReduceSameScalarNoAlloc: FLOAT, DOUBLE, HALF or BFLOAT16 arrays only");
+  ND4J_REQUIRE((reinterpret_cast<uintptr_t>(dX) % sizeOf(dt)) == 0 && (reinterpret_cast<uintptr_t>(dZ) % sizeOf(dt)) == 0, "nd4jhipReduceSameScalarNoAlloc: misaligned pointer");
+  hipStream_t st = stream ? *reinterpret_cast<hipStream_t*>(stream) : lc->execStream;
+  launchReduceScalarNoAlloc(st, reduceSameKind(opNum), dt, dX, length, dZ);
+  return 0;
+  GUARD_END(1)
+}
 const char* nd4jhipBuildInfo(void) { return "nd4j-hip gfx950 (hand-written HIP kernels; no CPU fallback)"; }
 
 }  // extern "C"

@@ -16,6 +16,10 @@
 // extreme wins, NaN is never selected and an all -inf row gives 0.  Here: NaN is mapped to the start
 // value on load and ties resolve to the lowest index, which yields the same integer.
 #include "anyio.h"
+#include <cstring>
+#include <mutex>
+#include <string>
+
 #include "device.h"
 #include "kernels.h"
 #include "runtime.h"
@@ -310,6 +314,43 @@ void launchReduce(hipStream_t st, ReduceKind k, DataType xdt, DataType zdt, cons
     default: ND4J_THROW("reduce: unknown op kind");
   }
   HIP_CHECK(hipGetLastError());
+}
+
+// ---- full reduction for callers that cannot allocate ---------------------------------------------------------------
+// The cross-block partials of a split full reduction normally go to the launch context's hipMalloc'ed reduction buffer.
+// This variant parks them in a fixed array in the code object's own global segment, so the call needs no allocation
+// at all.  Every device that loads the library holds its own copy of the array (until the process ends) at its own
+// address; the host-side name is only a handle for hipGetSymbolAddress, never a device address.  Calls that overlap
+// on one device share the array and race; nothing in it has to start at zero (every partial a launch reads was
+// written by that launch).
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int NOALLOC_MAX_DEVICES = 64;
+void* g_noAllocScratch[NOALLOC_MAX_DEVICES];   // device address of `scratch`, per device
+std::mutex g_noAllocMutex;
+}
+void* reduceNoAllocScratch() {
+  int dev = 0;
+  HIP_CHECK(hipGetDevice(&dev));
+  ND4J_REQUIRE(dev >= 0 && dev < NOALLOC_MAX_DEVICES, "no-alloc reduction: device ordinal out of range");
+  std::lock_guard<std::mutex> g(g_noAllocMutex);
+  if (g_noAllocScratch[dev] == nullptr) {
+    void* p = nullptr;
+    HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    ND4J_REQUIRE(p != nullptr, "no-alloc reduction: hipGetSymbolAddress returned no address");
+    g_noAllocScratch[dev] = p;
+  }
+  return g_noAllocScratch[dev];
+}
+void launchReduceScalarNoAlloc(hipStream_t st, ReduceKind k, DataType dt, const void* x, LongType n, void* z) {
+  ND4J_REQUIRE(n >= 1, "no-alloc reduction: length must be at least 1");
+  ND4J_REQUIRE(n <= NOALLOC_MAX_ELEMENTS, "no-alloc reduction: length " + std::to_string(n) + " exceeds the maximum of " + std::to_string(NOALLOC_MAX_ELEMENTS) + " elements");
+  ReducePlan p;                       // a dense vector reduced to one element
+  memset(&p.outer, 0, sizeof(DevShape)); memset(&p.zOuter, 0, sizeof(DevShape)); memset(&p.inner, 0, sizeof(DevShape));
+  p.inner.rank = 1; p.inner.shape[0] = n; p.inner.stride[0] = 1;
+  p.outerLen = 1; p.innerLen = n; p.index32 = true; p.zLinear = true;
+  launchReduce(st, k, dt, dt, x, z, p, reduceNoAllocScratch(), NOALLOC_SCRATCH_BYTES);
 }
 
 // ---- summary statistics, counts, Any / All -------------------------------------------------------------------------

@@ -135,12 +135,16 @@ void LaunchContext::init() {
   HIP_CHECK(hipEventCreateWithFlags(&bridgeOut, hipEventDisableTiming));
   ready = true;
 }
+static LaunchContext g_defaultContext;
+static std::mutex g_defaultContextMutex;
 LaunchContext* LaunchContext::defaultContext() {
-  static LaunchContext lc;
-  static std::mutex m;
-  std::lock_guard<std::mutex> g(m);
-  lc.init();
-  return &lc;
+  std::lock_guard<std::mutex> g(g_defaultContextMutex);
+  g_defaultContext.init();
+  return &g_defaultContext;
+}
+LaunchContext* LaunchContext::ifReady() {
+  std::lock_guard<std::mutex> g(g_defaultContextMutex);
+  return g_defaultContext.ready ? &g_defaultContext : nullptr;
 }
 
 // ---- data buffer ----------------------------------------------------------------------------------

@@ -59,6 +59,7 @@ struct LaunchContext {
   static constexpr size_t ALLOCATION_BYTES = 8u << 20;
   void init();
   static LaunchContext* defaultContext();
+  static LaunchContext* ifReady();   // the default context if it has been initialised, else null (never allocates)
 };
 bool deviceAvailable();
 

@@ -173,6 +173,7 @@ _SIGS = {
     "nd4jhipGraphDestroy": (None, [c_ptr]),
     "nd4jhipBuildInfo": (ctypes.c_char_p, []),
     "nd4jhipLastGemmKernel": (ctypes.c_char_p, []),
+    "nd4jhipReduceSameScalarNoAlloc": (ctypes.c_int, [c_ptr, ctypes.c_int, ctypes.c_int, c_ptr, c_long, c_ptr]),
     "setGraphContextCudaContext": (None, [c_ptr, c_ptr, c_ptr, c_ptr]),
 }
 

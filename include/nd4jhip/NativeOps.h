@@ -251,6 +251,17 @@ ND4JHIP_EXPORT const char* nd4jhipBuildInfo(void);
  * test assert that its shape reached the instantiation it means to check. */
 ND4JHIP_EXPORT const char* nd4jhipLastGemmKernel(void);
 
+/* execReduceSame's full reduction for callers that cannot allocate.  No counterpart in the reference: it is for code
+ * under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.  z[0] = reduce(x[0 .. length)) for
+ * a dense device array x of `dataType` (FLOAT, DOUBLE, HALF, BFLOAT16) and the opNums of execReduceSame (0 Sum, 1 Max,
+ * 2 Min, 3 Prod, 4 ASum, 5 AMax, 6 AMin); same kernels as execReduceSame, hence the same bits.  dX / dZ are device
+ * pointers; stream is a pointer to the caller's stream as lcExecutionStream returns it, or null for the library's own.
+ * The cross-block partials go to a fixed 64 KiB device array inside the library (one copy per device, held until the
+ * process ends) instead of allocated scratch, and the call allocates nothing, on the error paths either.  Limits:
+ * 1 <= length <= 2^31 - 1 (larger: error); initializeDevicesAndFunctions must have run (it allocates; this call
+ * refuses to); calls that overlap on one device share the array and race.  Returns 0, or 1 with the error slot set. */
+ND4JHIP_EXPORT int nd4jhipReduceSameScalarNoAlloc(Nd4jPointer stream, int opNum, int dataType, const void* dX, Nd4jLong length, void* dZ);
+
 #ifdef __cplusplus
 }
 #endif
