@@ -786,7 +786,7 @@ static std::vector<LongType> broadcastStrides(const NDArray* a, const std::vecto
 static void broadcastableExec(Context& c, PairwiseKind k, const char* name) {
   ND4J_REQUIRE(c.width() >= 2, std::string(name) + ": two inputs are required");
   NDArray* x = c.input(0); NDArray* y = c.input(1); NDArray* z = c.output(0);
-  ND4J_REQUIRE(x->dataType() == z->dataType() && y->dataType() == z->dataType() && isFloatType(z->dataType()), std::string(name) + ": nd4j-hip implements same-type float arrays only");
+  ND4J_REQUIRE(x->dataType() == z->dataType() && y->dataType() == z->dataType() && (isFloatType(z->dataType()) || isIntLike(z->dataType())), std::string(name) + ": nd4j-hip requires inputs and output of one type");
   if (x->isEmpty() || y->isEmpty() || z->isEmpty()) return;
   auto out = broadcastShape(x, y);
   ND4J_REQUIRE(out == shapeOf(z), std::string(name) + ": output shape " + shapeStr(z) + " does not match the broadcast shape");

@@ -579,6 +579,7 @@ static bool tailContig(hipStream_t s, int k, DataType dt, const void* x, const v
 
 void launchUnary(hipStream_t s, UnaryKind k, DataType xdt, DataType zdt, const void* x, void* z, const EwPlan& p) {
   if (p.length == 0) return;
+  if (isIntLike(xdt) && isIntLike(zdt)) return launchIntElementwise(s, k, false, xdt, xdt, zdt, x, nullptr, z, p, 0, false);
   if (k >= U_TAIL_FIRST && k < U_TAIL_END) {
     if (!(p.sameShape && xdt == zdt && p.contiguous && aligned16(x) && aligned16(z) && tailContig<1>(s, k, xdt, x, x, z, p.length)))
       hipLaunchKernelGGL((tail_generic<1>), dim3(gridFor(p.length, EW_BLOCK)), dim3(EW_BLOCK), 0, s, (int)k, p.own[0], p.own[1], p.own[1],
@@ -627,6 +628,7 @@ static void pairwiseKind(hipStream_t s, DataType xdt, DataType ydt, DataType zdt
 void launchPairwise(hipStream_t s, PairwiseKind k, DataType xdt, DataType ydt, DataType zdt, const void* x,
                     const void* y, void* z, const EwPlan& p) {
   if (p.length == 0) return;
+  if (isIntLike(xdt) && isIntLike(ydt) && isIntLike(zdt)) return launchIntElementwise(s, k, true, xdt, ydt, zdt, x, y, z, p, 0, false);
   if (k >= P_TAIL_FIRST && k < P_TAIL_END) {
     if (!(p.sameShape && xdt == zdt && ydt == zdt && p.contiguous && aligned16(x) && aligned16(y) && aligned16(z) &&
           tailContig<2>(s, k, zdt, x, y, z, p.length)))
@@ -743,6 +745,7 @@ static void scalarKind(hipStream_t s, DataType dt, const void* x, double sc, voi
 void launchScalarOp(hipStream_t s, PairwiseKind k, DataType dt, const void* x, double scalar, void* z, const EwPlan& p) {
   if (p.length == 0) return;
   ND4J_REQUIRE(p.sameShape && p.rank >= 1, "scalar op: operands must share a shape");
+  if (isIntLike(dt)) return launchIntElementwise(s, k, true, dt, dt, dt, x, nullptr, z, p, (LongType)scalar, true);
   if (k >= P_TAIL_FIRST && k < P_TAIL_END) {
     // the scalar takes the array's storage type first, as the reference holds it in an array of that type
     hipLaunchKernelGGL((tail_generic<2>), dim3(gridFor(p.length, EW_BLOCK)), dim3(EW_BLOCK), 0, s, (int)k,

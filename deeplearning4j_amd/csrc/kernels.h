@@ -76,6 +76,13 @@ void launchScalar2Op(hipStream_t s, Scalar2Kind k, DataType xdt, DataType zdt, c
 // z = x (op) scalar
 void launchScalarOp(hipStream_t s, PairwiseKind k, DataType dt, const void* x, double scalar, void* z, const EwPlan& p);
 
+// Integer / bool arrays (intops.hip).  launchUnary, launchPairwise, launchScalarOp, launchReduce and launchIndexReduce
+// route there by themselves when every operand is of an integer type; these are the direct entry points.
+bool isIntLike(DataType t);
+// k is a UnaryKind (binary false) or a PairwiseKind (binary true; y, or `scalar` when hasScalar)
+void launchIntElementwise(hipStream_t s, int k, bool binary, DataType xdt, DataType ydt, DataType zdt, const void* x, const void* y,
+                          void* z, const EwPlan& p, LongType scalar, bool hasScalar);
+
 // ---- reductions ----------------------------------------------------------------------------------
 enum ReduceKind : int {
   R_SUM, R_MAX, R_MIN, R_PROD, R_ASUM, R_AMAX, R_AMIN,        // ReduceSame 0..6
@@ -117,6 +124,10 @@ void launchReduceMisc(hipStream_t s, MiscReduceKind k, DataType xdt, DataType zd
                       const ReducePlan* yPlan = nullptr);
 void launchIndexReduce(hipStream_t s, IndexKind k, DataType xdt, DataType zdt, const void* x, void* z,
                        const ReducePlan& p, void* scratch, size_t scratchBytes);
+
+// kind: a ReduceKind of the ReduceSame table (isIndex false) or an IndexKind (isIndex true)
+void launchIntReduce(hipStream_t s, int kind, bool isIndex, DataType xdt, DataType zdt, const void* x, void* z, const ReducePlan& p,
+                     void* scratch, size_t scratchBytes);
 
 // ---- row ops ---------------------------------------------------------------------------------------
 struct RowPlan {

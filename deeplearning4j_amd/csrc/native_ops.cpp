@@ -548,8 +548,9 @@ void execTransformSame(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, 
   OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execTransformSame", "x"); NDArray* z = arr(za, "execTransformSame", "z");
   ND4J_REQUIRE(x->dataType() == z->dataType(), "NativeOpExecutioner::execTransformSame requires X & Z to have same type");
-  ND4J_REQUIRE(isFloatType(x->dataType()), "execTransformSame: non-float types are not implemented in nd4j-hip");
-  if (opNum == 19) {   // ClipByValue (loops/legacy_ops.h:43)
+  ND4J_REQUIRE(isFloatType(x->dataType()) || isIntLike(x->dataType()), "execTransformSame: this data type is not implemented in nd4j-hip");
+  if (opNum == 19) {
+    ND4J_REQUIRE(isFloatType(x->dataType()), "execTransformSame: ClipByValue on integer arrays is not implemented in nd4j-hip");   // ClipByValue (loops/legacy_ops.h:43)
     runUnaryWithParams("execTransformSame", S2_CLIP_BY_VALUE, x, z, extraParams);
     return;
   }
@@ -595,8 +596,13 @@ void execPairwiseTransform(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray 
   // NativeOpExecutioner_pairwise_floats.cpp:34-57
   ND4J_REQUIRE(x->dataType() == z->dataType() || y->dataType() == z->dataType(),
                std::string("NativeOpExecutioner::execPairwiseTransform requires X or Y to have the same type as Z, got ") + dtypeName(x->dataType()) + ", " + dtypeName(y->dataType()) + " -> " + dtypeName(z->dataType()));
-  ND4J_REQUIRE(isFloatType(z->dataType()) && isFloatType(x->dataType()) && isFloatType(y->dataType()),
-               "execPairwiseTransform: non-float types are not implemented in nd4j-hip");
+  {
+    // all floating point, all integer / bool, or a floating point result from INT32 / INT64 / BOOL operands
+    const bool allInt = isIntLike(x->dataType()) && isIntLike(y->dataType()) && isIntLike(z->dataType());
+    auto loadable = [](DataType t) { return isFloatType(t) || t == INT32 || t == INT64 || t == BOOL; };
+    ND4J_REQUIRE(allInt || (isFloatType(z->dataType()) && loadable(x->dataType()) && loadable(y->dataType())),
+                 std::string("execPairwiseTransform: the combination ") + dtypeName(x->dataType()) + ", " + dtypeName(y->dataType()) + " -> " + dtypeName(z->dataType()) + " is not implemented in nd4j-hip");
+  }
   PairwiseKind k = pairwiseKind(opNum);
   if (z->isEmpty()) return;
   EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo(), y->shapeInfo()});
@@ -608,6 +614,11 @@ void execPairwiseTransform(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray 
   GUARD_END_VOID
 }
 
+static LongType hostScalarInt64(NDArray* s) {
+  ND4J_REQUIRE(s->lengthOf() >= 1 && s->buf, "scalar operand is empty");
+  s->buf->syncToPrimary();
+  return *static_cast<const LongType*>(s->buffer());
+}
 static double hostScalar(NDArray* s) {
   ND4J_REQUIRE(s->lengthOf() >= 1 && s->buf, "scalar operand is empty");
   s->buf->syncToPrimary();
@@ -617,6 +628,12 @@ static double hostScalar(NDArray* s) {
     case DOUBLE: return *(const double*)p;
     case INT32: return *(const int*)p;
     case INT64: return (double)*(const LongType*)p;
+    case BOOL: case UINT8: return *(const unsigned char*)p;
+    case INT8: return *(const signed char*)p;
+    case INT16: return *(const short*)p;
+    case UINT16: return *(const unsigned short*)p;
+    case UINT32: return *(const unsigned*)p;
+    case UINT64: return (double)*(const unsigned long long*)p;
     case HALF: { unsigned short h = *(const unsigned short*)p; unsigned sign = (h & 0x8000u) << 16, e = (h >> 10) & 31, m = h & 1023; float f; unsigned u;
       if (e == 0) { f = (float)m / 16777216.0f; if (sign) f = -f; return f; }
       if (e == 31) u = sign | 0x7f800000u | (m << 13); else u = sign | ((e + 112) << 23) | (m << 13);
@@ -628,7 +645,7 @@ static double hostScalar(NDArray* s) {
 void execScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueNDArray za, OpaqueNDArray sa, void*) {
   OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execScalar", "x"); NDArray* z = arr(za, "execScalar", "z"); NDArray* s = arr(sa, "execScalar", "scalar");
-  ND4J_REQUIRE(x->dataType() == z->dataType() && isFloatType(x->dataType()), "execScalar: nd4j-hip implements same-type float arrays only");
+  ND4J_REQUIRE(x->dataType() == z->dataType() && (isFloatType(x->dataType()) || isIntLike(x->dataType())), "execScalar: nd4j-hip requires X and Z of one type");
   PairwiseKind k;
   switch (opNum) {  // loops/legacy_ops.h:78-86
     case 0: k = P_ADD; break; case 1: k = P_SUB; break; case 2: k = P_MUL; break; case 3: k = P_DIV; break;
@@ -647,9 +664,17 @@ void execScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueN
     default: ND4J_THROW("execScalar: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
   if (z->isEmpty()) return;
-  double sc = hostScalar(s);
   EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo()});
   ND4J_REQUIRE(p.sameShape, "execScalar: x and z must share a shape");
+  if (isIntLike(x->dataType())) {
+    // the scalar takes the array's type (the reference reads it as X); an INT64 scalar stays exact
+    const LongType isc = s->dataType() == INT64 ? hostScalarInt64(s) : (LongType)hostScalar(s);
+    prepareSpecialUse({z}, {x});
+    launchIntElementwise(execStream(), k, true, x->dataType(), x->dataType(), z->dataType(), x->specialBuffer(), nullptr, z->specialBuffer(), p, isc, true);
+    registerSpecialUse({z}, {x});
+    return;
+  }
+  double sc = hostScalar(s);
   prepareSpecialUse({z}, {x});
   launchScalarOp(execStream(), k, x->dataType(), x->specialBuffer(), sc, z->specialBuffer(), p);
   registerSpecialUse({z}, {x});
@@ -677,8 +702,8 @@ void execBroadcast(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, Opaq
   OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execBroadcast", "x"); NDArray* y = arr(ya, "execBroadcast", "y"); NDArray* z = arr(za, "execBroadcast", "z");
   NDArray* dim = arr(da, "execBroadcast", "dimension");
-  ND4J_REQUIRE(x->dataType() == z->dataType() && y->dataType() == z->dataType() && isFloatType(z->dataType()),
-               "execBroadcast: nd4j-hip implements same-type float arrays only");
+  ND4J_REQUIRE(x->dataType() == z->dataType() && y->dataType() == z->dataType() && (isFloatType(z->dataType()) || isIntLike(z->dataType())),
+               "execBroadcast: nd4j-hip requires X, Y and Z of one type");
   PairwiseKind k;
   switch (opNum) {  // loops/legacy_ops.h:34-39
     case 0: k = P_ADD; break; case 1: k = P_SUB; break; case 2: k = P_MUL; break; case 3: k = P_DIV; break;
@@ -717,7 +742,7 @@ void execBroadcast(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, Opaq
 }  // extern "C"
 namespace nd4jhip {
 void runReduce(const char* fn, ReduceKind k, NDArray* x, NDArray* z, const std::vector<LongType>& dims) {
-  ND4J_REQUIRE(isFloatType(x->dataType()), std::string(fn) + ": non-float inputs are not implemented in nd4j-hip");
+  ND4J_REQUIRE(isFloatType(x->dataType()) || (isIntLike(x->dataType()) && k <= R_AMIN), std::string(fn) + ": this input type is not implemented in nd4j-hip");
   ND4J_REQUIRE(x->dataType() == z->dataType(), std::string(fn) + ": nd4j-hip requires Z to have X's type, got " + dtypeName(x->dataType()) + " -> " + dtypeName(z->dataType()));
   ND4J_REQUIRE(!x->isEmpty(), std::string(fn) + ": reductions of empty arrays are not implemented in nd4j-hip");
   if (z->isEmpty()) return;
@@ -911,7 +936,7 @@ void execTransformBool(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, 
   OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execTransformBool", "x"); NDArray* z = arr(za, "execTransformBool", "z");
   ND4J_REQUIRE(z->dataType() == BOOL, std::string("NativeOpExecutioner::execTransformBool requires Z to have same boolean type, got ") + dtypeName(z->dataType()));
-  ND4J_REQUIRE(isFloatType(x->dataType()), "execTransformBool: non-float inputs are not implemented in nd4j-hip");
+  ND4J_REQUIRE(isFloatType(x->dataType()) || isIntLike(x->dataType()), "execTransformBool: this input type is not implemented in nd4j-hip");
   UnaryKind k;
   switch (opNum) {  // loops/legacy_ops.h:49-51
     case 1: k = U_IS_INF; break; case 2: k = U_IS_NAN; break; case 3: k = U_IS_FINITE; break; case 4: k = U_IS_INF_OR_NAN; break;
@@ -932,7 +957,7 @@ static IndexKind indexKind(int opNum) {
 }  // extern "C"
 namespace nd4jhip {
 void runIndexReduce(const char* fn, int opNum, NDArray* x, NDArray* z, const std::vector<LongType>& dims) {
-  ND4J_REQUIRE(isFloatType(x->dataType()), std::string(fn) + ": non-float inputs are not implemented in nd4j-hip");
+  ND4J_REQUIRE(isFloatType(x->dataType()) || isIntLike(x->dataType()), std::string(fn) + ": this input type is not implemented in nd4j-hip");
   ND4J_REQUIRE(z->dataType() == INT64 || z->dataType() == INT32,
                std::string("NativeOpExecutioner::") + fn + " requires Z operand to have INT32/INT64 type, got " + dtypeName(z->dataType()));
   ND4J_REQUIRE(!x->isEmpty(), std::string(fn) + ": index reductions of empty arrays are not implemented in nd4j-hip");

@@ -294,6 +294,7 @@ void launchReduce(hipStream_t st, ReduceKind k, DataType xdt, DataType zdt, cons
   ND4J_REQUIRE(xdt == zdt, "reduce: output dtype must equal input dtype on this backend");
   ND4J_REQUIRE(p.outerLen < (1LL << 31) * 4, "reduce: too many outputs");
   if (p.outerLen == 0) return;
+  if (isIntLike(xdt)) return launchIntReduce(st, (int)k, false, xdt, zdt, x, z, p, scratch, scratchBytes);
   switch (k) {
     case R_SUM: reduceDtype<SumOp, PRE_ID>(st, xdt, x, z, p, POST_ID, scratch, scratchBytes); break;
     case R_MAX: reduceDtype<MaxOp, PRE_ID>(st, xdt, x, z, p, POST_ID, scratch, scratchBytes); break;
@@ -741,6 +742,7 @@ void launchIndexReduce(hipStream_t st, IndexKind k, DataType xdt, DataType zdt, 
                        const ReducePlan& p, void* scratch, size_t scratchBytes) {
   ND4J_REQUIRE(p.innerLen < 0x7fffffffLL, "index reduce: sub-array longer than 2^31-1 elements");
   if (p.outerLen == 0) return;
+  if (isIntLike(xdt)) return launchIntReduce(st, (int)k, true, xdt, zdt, x, z, p, scratch, scratchBytes);
   switch (k) {
     case I_MAX: indexKind<I_MAX>(st, xdt, zdt, x, z, p, scratch, scratchBytes); break;
     case I_MIN: indexKind<I_MIN>(st, xdt, zdt, x, z, p, scratch, scratchBytes); break;
