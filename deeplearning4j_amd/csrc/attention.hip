@@ -30,7 +30,7 @@ namespace nd4jhip {
 
 template <typename T>
 __global__ __launch_bounds__(256) void logits_fixup(T* __restrict__ l, LongType total, LongType Tq, LongType Tv, float scale,
-                                                    int applyScale, int causal, float maskValue) {
+                                                    int applyScale, int causal, float maskValue, const unsigned char* __restrict__ vmask) {
   const LongType step = (LongType)gridDim.x * 256;
   for (LongType i = (LongType)blockIdx.x * 256 + threadIdx.x; i < total; i += step) {
     const LongType j = i % Tv, r = (i / Tv) % Tq;
@@ -39,7 +39,10 @@ __global__ __launch_bounds__(256) void logits_fixup(T* __restrict__ l, LongType 
     if (applyScale) v = to_float(Conv<T>::from(v * to_float(Conv<T>::from(scale))));
     v = v > 1e4f ? to_float(Conv<T>::from(1e4f)) : v;
     v = v < -1e4f ? to_float(Conv<T>::from(-1e4f)) : v;
-    if (causal && j > r) v = v - maskValue;
+    // one penalty where the merged mask (causal AND value mask) is false (AttentionHelper.cpp:175-187,199-221)
+    bool masked = causal && j > r;
+    if (vmask != nullptr && vmask[(i / (Tv * Tq)) * Tv + j] == 0) masked = true;
+    if (masked) v = v - maskValue;
     l[i] = Conv<T>::from(v);
   }
 }
@@ -51,9 +54,31 @@ void launchAttentionLogitsFixup(hipStream_t s, DataType dt, void* logits, const 
   if (blocks > 256 * 16) blocks = 256 * 16;
   dim3 g((unsigned)blocks), b(256);
   switch (dt) {
-    case FLOAT32: hipLaunchKernelGGL((logits_fixup<float>), g, b, 0, s, (float*)logits, total, d.Tq, d.Tv, d.scale, (int)d.applyScale, (int)d.causal, d.maskValue); break;
-    case HALF: hipLaunchKernelGGL((logits_fixup<f16_t>), g, b, 0, s, (f16_t*)logits, total, d.Tq, d.Tv, d.scale, (int)d.applyScale, (int)d.causal, d.maskValue); break;
-    case BFLOAT16: hipLaunchKernelGGL((logits_fixup<bf16_t>), g, b, 0, s, (bf16_t*)logits, total, d.Tq, d.Tv, d.scale, (int)d.applyScale, (int)d.causal, d.maskValue); break;
+    case FLOAT32: hipLaunchKernelGGL((logits_fixup<float>), g, b, 0, s, (float*)logits, total, d.Tq, d.Tv, d.scale, (int)d.applyScale, (int)d.causal, d.maskValue, d.vmask); break;
+    case HALF: hipLaunchKernelGGL((logits_fixup<f16_t>), g, b, 0, s, (f16_t*)logits, total, d.Tq, d.Tv, d.scale, (int)d.applyScale, (int)d.causal, d.maskValue, d.vmask); break;
+    case BFLOAT16: hipLaunchKernelGGL((logits_fixup<bf16_t>), g, b, 0, s, (bf16_t*)logits, total, d.Tq, d.Tv, d.scale, (int)d.applyScale, (int)d.causal, d.maskValue, d.vmask); break;
+    default: ND4J_THROW("attention: unsupported dtype");
+  }
+  HIP_CHECK(hipGetLastError());
+}
+
+// weights[b, i, :] *= qmask[b, i], the mask value taken in the weights' type (AttentionHelper.cpp:463-467)
+template <typename T>
+__global__ __launch_bounds__(256) void weights_query_mask(T* __restrict__ w, LongType total, LongType Tv, const T* __restrict__ qmask) {
+  const LongType step = (LongType)gridDim.x * 256;
+  for (LongType i = (LongType)blockIdx.x * 256 + threadIdx.x; i < total; i += step)
+    w[i] = Conv<T>::from(to_float(w[i]) * to_float(qmask[i / Tv]));
+}
+void launchAttentionQueryMask(hipStream_t s, DataType dt, void* weights, const void* qmask, const AttnDesc& d) {
+  const LongType total = d.B * d.Tq * d.Tv;
+  if (total == 0) return;
+  LongType blocks = (total + 255) / 256;
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  dim3 g((unsigned)blocks), b(256);
+  switch (dt) {
+    case FLOAT32: hipLaunchKernelGGL((weights_query_mask<float>), g, b, 0, s, (float*)weights, total, d.Tv, (const float*)qmask); break;
+    case HALF: hipLaunchKernelGGL((weights_query_mask<f16_t>), g, b, 0, s, (f16_t*)weights, total, d.Tv, (const f16_t*)qmask); break;
+    case BFLOAT16: hipLaunchKernelGGL((weights_query_mask<bf16_t>), g, b, 0, s, (bf16_t*)weights, total, d.Tv, (const bf16_t*)qmask); break;
     default: ND4J_THROW("attention: unsupported dtype");
   }
   HIP_CHECK(hipGetLastError());
@@ -67,6 +92,8 @@ struct FusedArgs {
   float scale;
   int applyScale, causal;
   int qTiles, perBatch, nBatch, heavyFirst;   // fused kernel: work slots per batch entry, batch entries, block order
+  const unsigned char* vmask;                 // VM kernels: dense [batch entries, Tv] bytes, 0 = padded key
+  float maskValue;                            // what a masked logit has subtracted
 };
 
 template <typename T> __device__ __forceinline__ float round_storage(float v) { return to_float(Conv<T>::from(v)); }
@@ -98,7 +125,11 @@ template <typename T> __device__ __forceinline__ unsigned pack2(float a, float b
 // FOLD: the scale is a power of two (or 1) and the scores are bf16, so scaling commutes exactly with the clip and with
 // the rounding through the storage type; the kernel then keeps unscaled scores and multiplies inside the exponent's
 // fused multiply-add (scale * log2(e) is exact too), which saves one multiply per score.
-template <typename T, int D, bool FOLD>
+// VM: a value (padding) mask is present.  Masked logits -- padded keys and, under the causal flag, keys after the query --
+// then get the reference's penalty subtracted and rounded through the storage type instead of being dropped, and no key
+// tile is skipped: a query whose visible keys are all padded spreads its weight over every key, as the reference's
+// softmax over equally penalised logits does.
+template <typename T, int D, bool FOLD, bool VM>
 __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
                                                   T* __restrict__ O) {
   constexpr int BQ = 128, BKV = 64, NT = 256;
@@ -138,6 +169,7 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
   } else {
     Q += b * a.qB; K += b * a.kB; V += b * a.vB; O += b * a.oB;
   }
+  const unsigned char* vm = VM ? a.vmask + b * a.Tv : nullptr;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, h = lane >> 5;
   const float sc = a.scale;   // 1 when the op applies no scale
   const float L2E = FOLD ? 1.44269502162933349609375f * sc : 1.44269502162933349609375f;
@@ -171,7 +203,7 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
   float m = -1.0e30f, l = 0.f;
 
   LongType kvEnd = a.Tv;
-  if (a.causal) { const LongType lim = q0 + BQ; kvEnd = lim < kvEnd ? lim : kvEnd; }
+  if (a.causal && !VM) { const LongType lim = q0 + BQ; kvEnd = lim < kvEnd ? lim : kvEnd; }
   const LongType nTiles = (kvEnd + BKV - 1) / BKV;
 
   // the loader moves 64 k-values per pass: the K tile (D values of d per key) takes D/64 of them
@@ -263,7 +295,22 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
     const int qFirst = (int)q0 + wave * 32;
     // a real branch (scalar condition, a body the compiler cannot speculate): turned into selects, the mask costs 86
     // vector instructions on every tile instead of on the few that need it
-    if (__builtin_amdgcn_readfirstlane((int)((a.causal && (int)kv0 + BKV - 1 > qFirst) || kv0 + BKV > a.Tv)) != 0) {
+    if (VM) {
+      const int lastVisible = a.causal ? (int)query : (int)a.Tv - 1;
+#pragma unroll
+      for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; r4++) {
+          const int key0 = (int)kv0 + kt * 32 + 8 * r4 + 4 * h;   // registers 4*r4 .. +3 hold four consecutive keys
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const int key = key0 + e;
+            const float sv = s[kt][4 * r4 + e];
+            if (key >= (int)a.Tv) s[kt][4 * r4 + e] = -1.0e30f;    // beyond the keys: contributes exactly nothing
+            else if (key > lastVisible || vm[key] == 0) s[kt][4 * r4 + e] = round_storage<T>(sv - a.maskValue);
+          }
+        }
+    } else if (__builtin_amdgcn_readfirstlane((int)((a.causal && (int)kv0 + BKV - 1 > qFirst) || kv0 + BKV > a.Tv)) != 0) {
       asm volatile("; tile with masked entries");
       const int lastKey = a.causal ? ((int)query < (int)a.Tv - 1 ? (int)query : (int)a.Tv - 1) : (int)a.Tv - 1;
 #pragma unroll
@@ -282,7 +329,10 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
     // every query has seen key 0 by now, so the running maximum is a real score and masked entries (-1e30)
     // underflow to exactly 0 in the exponential
     const float mL = tmax * L2E;
-    const float alpha = __builtin_amdgcn_exp2f(m * L2E - mL);
+    // With a value mask a query may have seen nothing but hidden keys so far (fp16: their logits are -inf), so m and
+    // tmax may both still be the -1e30 start value: the difference is taken first, which is exactly 0 then, where the
+    // fused form below would turn the rounding error of -1e30 * log2(e) into a factor of 0 or inf.
+    const float alpha = VM ? __builtin_amdgcn_exp2f((m - tmax) * L2E) : __builtin_amdgcn_exp2f(m * L2E - mL);
     m = tmax;
     float psum = 0.f;
     u32x4 pf[4];   // P^T operand of k-step ks: registers 8*(ks%2) .. +7 of tile ks/2
@@ -352,7 +402,7 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
 // exactly where the P V accumulation needs it.  Each lane group keeps its own running (max, sum, o[8]) state;
 // states are merged across groups (shuffles), across waves (LDS) and normalised once.  Logits go through the same
 // scale / clip / storage-type rounding as in the tile kernel above; probabilities stay in fp32.
-template <typename T, int D, int NW>
+template <typename T, int D, int NW, bool VM>
 __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
                                                        T* __restrict__ O) {
   constexpr int CH = D / 8;          // lanes per key row
@@ -366,6 +416,7 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
   } else {
     Q += b * a.qB; K += b * a.kB; V += b * a.vB; O += b * a.oB;
   }
+  const unsigned char* vm = VM ? a.vmask + b * a.Tv : nullptr;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int g = lane / CH, c = lane % CH;
   // the query row was written by the kernel before this one and the first keys come cold from HBM: all of these loads
@@ -406,6 +457,10 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
       if (a.applyScale) d *= a.scale;
       d = __builtin_fminf(__builtin_fmaxf(d, -1.0e4f), 1.0e4f);
       d = round_storage<T>(d);
+      if (VM) {   // a padded key keeps its logit, penalised and rounded as the reference stores it
+        const LongType key = k0 + u * KPS + g;
+        if (valid[u] && vm[key] == 0) d = round_storage<T>(d - a.maskValue);
+      }
       sc[u] = valid[u] ? d : -1.0e30f;
       tmax = __builtin_fmaxf(tmax, sc[u]);
     }
@@ -476,10 +531,15 @@ static void launchDecodeTyped(hipStream_t s, const void* q, const void* k, const
   a.qB = d.qB; a.qT = d.qT; a.kB = d.kB; a.kT = d.kT; a.vB = d.vB; a.vT = d.vT; a.oB = d.oB; a.oT = d.oT;
   a.H = d.H; a.qB2 = d.qB2; a.kB2 = d.kB2; a.vB2 = d.vB2; a.oB2 = d.oB2;
   a.scale = d.scale; a.applyScale = d.applyScale ? 1 : 0; a.causal = 0; a.qTiles = 1; a.perBatch = 1;
+  a.vmask = d.vmask; a.maskValue = d.maskValue;
   const dim3 grid((unsigned)d.B, (unsigned)d.Tq);
+  if (d.vmask) {
+    hipLaunchKernelGGL((attn_decode<T, D, 4, true>), grid, dim3(256), 0, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
+    return;
+  }
   // few (batch, head) rows: more waves per row, so that the history is still spread over many loads in flight
-  if (d.B * d.Tq < 128) hipLaunchKernelGGL((attn_decode<T, D, 16>), grid, dim3(1024), 0, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
-  else hipLaunchKernelGGL((attn_decode<T, D, 4>), grid, dim3(256), 0, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
+  if (d.B * d.Tq < 128) hipLaunchKernelGGL((attn_decode<T, D, 16, false>), grid, dim3(1024), 0, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
+  else hipLaunchKernelGGL((attn_decode<T, D, 4, false>), grid, dim3(256), 0, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
 }
 
 void launchAttentionDecode(hipStream_t s, DataType dt, const void* q, const void* k, const void* v, void* out, const AttnDesc& d) {
@@ -502,7 +562,7 @@ bool attentionFusedSupported(DataType dt, const AttnDesc& d) {
   return true;
 }
 
-template <typename T, int D, bool FOLD>
+template <typename T, int D, bool FOLD, bool VM>
 static void launchFusedTyped(hipStream_t s, const void* q, const void* k, const void* v, void* out, const AttnDesc& d) {
   FusedArgs a;
   a.Tq = d.Tq; a.Tv = d.Tv;
@@ -511,9 +571,10 @@ static void launchFusedTyped(hipStream_t s, const void* q, const void* k, const 
   a.scale = d.applyScale ? (float)d.scale : 1.f; a.applyScale = d.applyScale ? 1 : 0; a.causal = d.causal ? 1 : 0;
   a.qTiles = (int)((d.Tq + 127) / 128);
   a.nBatch = (int)d.B;
-  a.perBatch = d.causal ? (a.qTiles + 1) / 2 : a.qTiles;
+  a.vmask = d.vmask; a.maskValue = d.maskValue;
+  a.perBatch = d.causal && !VM ? (a.qTiles + 1) / 2 : a.qTiles;   // with a value mask no key tile is skipped: equal tiles
   a.heavyFirst = 0;
-  if (d.causal && a.qTiles > 1) {
+  if (d.causal && !VM && a.qTiles > 1) {
     // time in key tiles per slot (a CU holds two blocks at D = 64, one at D = 128): equal paired blocks run in whole
     // rounds; single query tiles handed out heavy first finish within about a tenth of the mean, but not before the
     // longest tile.  The batch-major order keeps K and V closer, so it stays unless the rounds waste more than 8 %.
@@ -525,7 +586,7 @@ static void launchFusedTyped(hipStream_t s, const void* q, const void* k, const 
     a.heavyFirst = pairedTime > 1.08 * heavyTime ? 1 : 0;
   }
   constexpr size_t LDS = (size_t)2 * ((D / 64) * TileLayout<64, true>::SLOTS + TileLayout<D, false>::SLOTS) * 16;
-  auto kern = attn_fused<T, D, FOLD>;
+  auto kern = attn_fused<T, D, FOLD, VM>;
   static std::once_flag attrOnce;
   std::call_once(attrOnce, [&] { HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS)); });
   hipLaunchKernelGGL(kern, dim3((unsigned)((LongType)(a.heavyFirst ? a.qTiles : a.perBatch) * d.B)), dim3(256), LDS, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
@@ -541,7 +602,9 @@ void launchAttentionFused(hipStream_t s, DataType dt, const void* q, const void*
   int e = 0;
   const bool pow2 = sc > 0.f && std::frexp(sc, &e) == 0.5f && e >= -19 && e <= 21;
   const bool fold = sc == 1.f || (dt == BFLOAT16 && pow2);
-#define ND4J_FUSED(T, DD) (fold ? launchFusedTyped<T, DD, true>(s, q, k, v, out, d) : launchFusedTyped<T, DD, false>(s, q, k, v, out, d))
+  // the penalty of a masked logit is subtracted from the scaled logit, so the value-mask kernels keep the explicit scale
+#define ND4J_FUSED(T, DD) (d.vmask ? launchFusedTyped<T, DD, false, true>(s, q, k, v, out, d) \
+                           : fold ? launchFusedTyped<T, DD, true, false>(s, q, k, v, out, d) : launchFusedTyped<T, DD, false, false>(s, q, k, v, out, d))
   if (dt == HALF) { if (d.D == 64) ND4J_FUSED(f16_t, 64); else ND4J_FUSED(f16_t, 128); }
   else { if (d.D == 64) ND4J_FUSED(bf16_t, 64); else ND4J_FUSED(bf16_t, 128); }
 #undef ND4J_FUSED

@@ -421,9 +421,12 @@ static void layerNormExec(Context& c) {
 // ---- dot_product_attention_v2 ---------------------------------------------------------------------------------------------
 // generic/nn/dot_product_attention_v2.cpp:35-125 -> helpers/impl/AttentionHelper.cpp:411-469.
 // Inputs (queries, values, keys?); TArgs [scale, dropout]; BArgs [useCausalMask, training];
+// Inputs 3 / 4: optional query mask [batch.., Tq] and value mask [batch.., Tv].
 // outputs [out, weights?, logits?].  logits = clip(scale * q k^T, +-1e4) (scale applied unless 0 or 1),
-// masked (j > i) logits get 65504 (bf16) / 1e9 (other types) subtracted, weights = softmax(logits),
-// out = weights v.  With only `out` supplied the fused kernel runs and nothing of size Tq x Tv is written.
+// logits where the causal mask (j > i) or the value mask (cast to BOOL, false = padded key) hides the key get
+// 65504 (bf16) / 1e9 (other types) subtracted once, weights = softmax(logits), out = weights v, and last the weights
+// output is multiplied by the query mask (out is not: the reference forms it before).
+// With only `out` supplied the fused kernel runs and nothing of size Tq x Tv is written.
 // An operand seen as [outer, H, T, D]: rank 2 has no batch, rank 3 one batch level (H = 0), rank >= 4 two levels
 // (the last leading dim is the inner level; the dims before it must fold into one).  The two-level form is what a
 // [batch, heads, T, D] view of a token-major [batch, T, heads * D] buffer needs: its batch dims do not nest.
@@ -457,8 +460,9 @@ static void attentionExec(Context& c) {
   NDArray* q0 = c.input(0); NDArray* v0 = c.input(1); NDArray* k0 = c.width() > 2 ? c.input(2) : v0;
   NDArray* o0 = c.output(0);
   ND4J_REQUIRE(q0->rankOf() == v0->rankOf(), "Queries and values must be same ranks!");
-  for (int i = 3; i < c.width(); i++)
-    ND4J_REQUIRE(c.inputs[i] == nullptr || c.inputs[i]->isEmpty(), "dot_product_attention_v2: query/value masks are not implemented in nd4j-hip");
+  // optional masks (dot_product_attention_v2.cpp:57-58): input 3 = query mask [batch.., Tq], input 4 = value mask [batch.., Tv]
+  NDArray* qMask = c.width() > 3 && c.inputs[3] != nullptr && !c.inputs[3]->isEmpty() ? c.inputs[3] : nullptr;
+  NDArray* vMask = c.width() > 4 && c.inputs[4] != nullptr && !c.inputs[4]->isEmpty() ? c.inputs[4] : nullptr;
   const double dropout = tArg(c, 1, 0.0);
   const double scale = tArg(c, 0, 1.0);
   const bool causal = bArg(c, 0, false), training = bArg(c, 1, false);
@@ -479,8 +483,38 @@ static void attentionExec(Context& c) {
   std::vector<NDArray*> writes = {o0};
   if (wantW) writes.push_back(c.outputs[1]);
   if (wantL) writes.push_back(c.outputs[2]);
+  // a mask carries the batch dims of the queries followed by the sequence length (the reference expands it at -2 / -1
+  // and lets it broadcast against [batch.., Tq, Tv], AttentionHelper.cpp:434-436,463-466)
+  auto maskFits = [&](NDArray* m, LongType T, const char* what) {
+    bool ok = m->rankOf() == std::max(q0->rankOf() - 1, 1) && m->lengthOf() == d.B * T && m->sizeAt(-1) == T;
+    for (int i = 0; ok && i < m->rankOf() - 1; i++) ok = m->sizeAt(i) == q0->sizeAt(i);
+    ND4J_REQUIRE(ok, std::string("dot_product_attention_v2: the ") + what + " mask must have shape [batch.., " + std::to_string(T) + "], got " + shapeStr(m));
+    ND4J_REQUIRE(isFloatType(m->dataType()) || m->dataType() == BOOL || m->dataType() == INT32 || m->dataType() == INT64,
+                 std::string("dot_product_attention_v2: unsupported data type of the ") + what + " mask");
+  };
+  if (vMask) { maskFits(vMask, d.Tv, "value"); reads.push_back(vMask); }
+  if (qMask) { maskFits(qMask, d.Tq, "query"); reads.push_back(qMask); }
   if (d.B * d.Tq == 0) return;
   prepareSpecialUse(writes, reads);
+  // dense device copies of the masks in the form the kernels read: the value mask as bytes (cast to BOOL: non-zero keeps
+  // the key), the query mask in the arrays' type.  A mask that already is dense and of that type is used in place.
+  std::shared_ptr<DataBuffer> tmpVm, tmpQm;
+  auto denseMask = [&](NDArray* m, DataType want, std::shared_ptr<DataBuffer>& hold) -> const void* {
+    auto dsi = makeShapeInfo(want, 'c', shapeOf(m));
+    if (m->dataType() == want) {
+      bool dense = true;
+      for (int i = 0; i < m->rankOf(); i++) if (m->sizeAt(i) != 1 && m->strideAt(i) != shape::strideOf(dsi.data())[i]) dense = false;
+      if (dense) return m->specialBuffer();
+    }
+    hold = std::make_shared<DataBuffer>((void*)nullptr, (void*)nullptr, (size_t)m->lengthOf() * sizeOf(want), want);
+    hold->allocateSpecial();
+    EwPlan p = buildEwPlan({dsi.data(), m->shapeInfo()});
+    launchUnary(stream(), U_IDENTITY, m->dataType(), want, m->specialBuffer(), hold->special, p);
+    return hold->special;
+  };
+  if (vMask) d.vmask = static_cast<const unsigned char*>(denseMask(vMask, BOOL, tmpVm));
+  // the query mask scales the weights output only: out = weights v has been formed before (AttentionHelper.cpp:455-467)
+  const void* qm = qMask && wantW ? denseMask(qMask, dt, tmpQm) : nullptr;
   d.qB = q.sB; d.qT = q.sT; d.kB = k.sB; d.kT = k.sT; d.vB = v.sB; d.vT = v.sT; d.oB = out.sB; d.oT = out.sT;
   d.qB2 = q.sB2; d.kB2 = k.sB2; d.vB2 = v.sB2; d.oB2 = out.sB2;
   const bool unitInner = q.sD == 1 && k.sD == 1 && v.sD == 1 && out.sD == 1;
@@ -521,8 +555,10 @@ static void attentionExec(Context& c) {
     g2.bRow = v.sT; g2.bCol = v.sD; g2.bBatch = v.sB; g2.bBatch2 = v.sB2;
     g2.cRow = out.sT; g2.cCol = out.sD; g2.cBatch = out.sB; g2.cBatch2 = out.sB2;
     launchGemm(stream(), dt, weights, v0->specialBuffer(), o0->specialBuffer(), g2);
+    if (qm) launchAttentionQueryMask(stream(), dt, weights, qm, d);
     if (tmpL || tmpW) HIP_CHECK(hipStreamSynchronize(stream()));  // temporaries are released on return
   }
+  if (tmpVm || tmpQm) HIP_CHECK(hipStreamSynchronize(stream()));
   registerSpecialUse(writes, reads);
 }
 static std::vector<std::vector<LongType>> attentionShapeFn(Context& c) {

@@ -192,6 +192,7 @@ struct AttnDesc {
   bool applyScale = false;
   bool causal = false;
   float maskValue = 1e9f;
+  const unsigned char* vmask = nullptr;   // optional value (padding) mask, dense [B, Tv] bytes: 0 = masked key
 };
 // fused path (no logits/weights written)
 bool attentionFusedSupported(DataType dt, const AttnDesc& d);
@@ -203,6 +204,8 @@ void launchAttentionDecode(hipStream_t s, DataType dt, const void* q, const void
                            const AttnDesc& d);
 // logits[b,i,j] = clip(scale * logits, +-1e4) - mask  (in place, row-major [B,Tq,Tv])
 void launchAttentionLogitsFixup(hipStream_t s, DataType dt, void* logits, const AttnDesc& d);
+// weights[b, i, :] *= qmask[b, i] (in place; qmask dense [B, Tq] of the weights' type)
+void launchAttentionQueryMask(hipStream_t s, DataType dt, void* weights, const void* qmask, const AttnDesc& d);
 
 // ---- misc ------------------------------------------------------------------------------------------
 // z[i, :] = table[idx[i], :]

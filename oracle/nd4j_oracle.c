@@ -1353,10 +1353,12 @@ int orc_matmul(const void *x, const int64_t *xsi, const void *y, const int64_t *
  * weights = softmax(logits, -1) with the clamp semantics above; out = weights * v.
  * logits/weights outputs are stored rounded to the array dtype; the softmax reads the stored logits and
  * the final product reads the stored weights, as the reference's op-by-op composition does.
+ * qmask [batch, Tq] / vmask [batch, Tv] (any numeric dtype, may be NULL): see the two comments in the body.
  * ------------------------------------------------------------------------------------------- */
 int orc_attention_v2(const void *q, const int64_t *qsi, const void *v, const int64_t *vsi, const void *k,
                      const int64_t *ksi, void *out, const int64_t *osi, void *weights, const int64_t *wsi,
-                     void *logits, const int64_t *lsi, double scale, int causal) {
+                     void *logits, const int64_t *lsi, double scale, int causal, const void *qmask,
+                     const int64_t *qmsi, const void *vmask, const int64_t *vmsi) {
   if (si_rank(qsi) != 3 || si_rank(vsi) != 3 || si_rank(ksi) != 3) return 3;
   int dt = orc_dtype(qsi);
   if (!dt_is_float(dt) || dt == ORC_DOUBLE) return 2;
@@ -1382,7 +1384,11 @@ int orc_attention_v2(const void *q, const int64_t *qsi, const void *v, const int
       float l = rnd(acc, dt);
       if (scale != 0.0 && scale != 1.0) l = rnd(l * rnd((float)scale, dt), dt);
       l = l > 1e4f ? rnd(1e4f, dt) : l; l = l < -1e4f ? rnd(-1e4f, dt) : l;
-      if (causal && j > i) l = rnd(l - (dt == ORC_BFLOAT16 ? 65504.0f : 1.0e9f), dt);
+      /* scoresMask = value mask (cast to BOOL, expanded at -2) AND lower-triangular mask (:175-187, :434-452);
+       * where it is false the logit has the penalty subtracted once (:199-221) */
+      int hidden = causal && j > i;
+      if (vmask && ldf(vmask, orc_dtype(vmsi), b * si_stride(vmsi)[0] + j * si_stride(vmsi)[1]) == 0.0f) hidden = 1;
+      if (hidden) l = rnd(l - (dt == ORC_BFLOAT16 ? 65504.0f : 1.0e9f), dt);
       L[j] = l;
       if (logits) st(logits, dt, b * si_stride(lsi)[0] + i * si_stride(lsi)[1] + j * si_stride(lsi)[2], l);
     }
@@ -1398,14 +1404,18 @@ int orc_attention_v2(const void *q, const int64_t *qsi, const void *v, const int
       L[j] = expf(d); sum += L[j];
     }
     sum = sum > 1e-6f ? sum : 1e-6f;
-    for (int64_t j = 0; j < Tv; j++) {
-      L[j] = rnd(L[j] / sum, dt);
-      if (weights) st(weights, dt, b * si_stride(wsi)[0] + i * si_stride(wsi)[1] + j * si_stride(wsi)[2], L[j]);
-    }
+    for (int64_t j = 0; j < Tv; j++) L[j] = rnd(L[j] / sum, dt);
     for (int64_t d = 0; d < Dv; d++) {
       float acc = 0;
       for (int64_t j = 0; j < Tv; j++) acc += L[j] * ldf(v, dt, b * vs[0] + j * vs[1] + d * vs[2]);
       st(out, dt, b * os[0] + i * os[1] + d * os[2], acc);
+    }
+    /* the query mask (cast to the arrays' type, expanded at -1) multiplies the scores array after the output has
+     * been formed from it (:455-467): it shows in the weights output only */
+    if (weights) {
+      float qm = qmask ? rnd(ldf(qmask, orc_dtype(qmsi), b * si_stride(qmsi)[0] + i * si_stride(qmsi)[1]), dt) : 1.0f;
+      for (int64_t j = 0; j < Tv; j++)
+        st(weights, dt, b * si_stride(wsi)[0] + i * si_stride(wsi)[1] + j * si_stride(wsi)[2], qmask ? L[j] * qm : L[j]);
     }
   }
   free(lg);

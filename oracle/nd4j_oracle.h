@@ -125,7 +125,8 @@ int orc_matmul(const void *x, const int64_t *xsi, const void *y, const int64_t *
                int transX, int transY, int transZ, double alpha, double beta, int accumulate);
 int orc_attention_v2(const void *q, const int64_t *qsi, const void *v, const int64_t *vsi, const void *k,
                      const int64_t *ksi, void *out, const int64_t *osi, void *weights, const int64_t *wsi,
-                     void *logits, const int64_t *lsi, double scale, int causal);
+                     void *logits, const int64_t *lsi, double scale, int causal, const void *qmask,
+                     const int64_t *qmsi, const void *vmask, const int64_t *vmsi);
 
 /* decoder glue (broadcast add of a row vector, gather of rows) used by the decode harness check */
 int orc_add_row_vector(const void *x, const int64_t *xsi, const void *row, const int64_t *rsi, void *z,

@@ -68,7 +68,7 @@ def lib():
         L.orc_top_k.argtypes = [vp, i64p, vp, i64p, vp, i64p, i64, i32]
         L.orc_layer_norm.argtypes = [vp, i64p, vp, i64p, vp, i64p, vp, i64p, i64p, i32, i32]
         L.orc_matmul.argtypes = [vp, i64p, vp, i64p, vp, i64p, i32, i32, i32, dbl, dbl, i32]
-        L.orc_attention_v2.argtypes = [vp, i64p, vp, i64p, vp, i64p, vp, i64p, vp, i64p, vp, i64p, dbl, i32]
+        L.orc_attention_v2.argtypes = [vp, i64p, vp, i64p, vp, i64p, vp, i64p, vp, i64p, vp, i64p, dbl, i32, vp, i64p, vp, i64p]
         L.orc_add_row_vector.argtypes = [vp, i64p, vp, i64p, vp, i64p]
         L.orc_set_threads.argtypes = [i32]
         L.orc_get_threads.restype = i32
@@ -272,13 +272,16 @@ def matmul(x, y, z, trans_x=False, trans_y=False, trans_z=False, alpha=1.0, beta
     return z.a
 
 
-def attention_v2(q, v, k, out, weights=None, logits=None, scale=1.0, causal=False):
+def attention_v2(q, v, k, out, weights=None, logits=None, scale=1.0, causal=False, q_mask=None, v_mask=None):
     q, v, k, out = _arr(q), _arr(v), _arr(k), _arr(out)
     w = _arr(weights) if weights is not None else None
     lg = _arr(logits) if logits is not None else None
+    qm = _arr(q_mask) if q_mask is not None else None
+    vm = _arr(v_mask) if v_mask is not None else None
     _check(lib().orc_attention_v2(_p(q.a), _s(q.si), _p(v.a), _s(v.si), _p(k.a), _s(k.si), _p(out.a), _s(out.si),
                                   _p(w.a) if w else None, _s(w.si) if w else None, _p(lg.a) if lg else None,
-                                  _s(lg.si) if lg else None, scale, int(causal)), "attention_v2")
+                                  _s(lg.si) if lg else None, scale, int(causal), _p(qm.a) if qm else None, _s(qm.si) if qm else None,
+                                  _p(vm.a) if vm else None, _s(vm.si) if vm else None), "attention_v2")
     return out.a
 
 

@@ -406,6 +406,70 @@ def test_attention_vs_oracle(ex, oracle, dtype, tol, causal, B, Tq, Tv, D):
     assert_close(out1.to_float(), _f(oo), tol, tol, "out-only call")
 
 
+@pytest.mark.parametrize("dtype,tol", [(FLOAT32, 1e-4), (HALF, 1e-2), (BFLOAT16, 1e-2)])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("B,Tq,Tv,D", [(3, 64, 64, 64), (2, 200, 200, 64), (2, 130, 300, 64), (2, 4, 150, 64), (1, 37, 91, 32)])
+def test_attention_masks_vs_oracle(ex, oracle, dtype, tol, causal, B, Tq, Tv, D):
+    """Query and value masks (inputs 3 and 4): all three outputs through the composition path, then the output-only call
+    (fused prefill kernel, or the streaming decode kernel for a handful of query rows)."""
+    rng = np.random.default_rng(B * Tq + D + Tv)
+    oq, dq = _pair(oracle, rng.normal(0, 1, (B, Tq, D)), dtype)
+    ok, dk = _pair(oracle, rng.normal(0, 1, (B, Tv, D)), dtype)
+    ov, dv = _pair(oracle, rng.normal(0, 1, (B, Tv, D)), dtype)
+    vm = (rng.random((B, Tv)) > 0.3).astype(np.float32)
+    vm[:, 0] = 1                                           # key 0 stays: every query keeps a visible key
+    vm[-1, Tv // 2:] = 0                                   # a padded tail
+    qm = (rng.random((B, Tq)) > 0.3).astype(np.float32)
+    ovm, dvm = _pair(oracle, vm, dtype)
+    oqm, dqm = _pair(oracle, qm, dtype)
+    oo, ow, ol = _ozeros(oracle, (B, Tq, D), dtype), _ozeros(oracle, (B, Tq, Tv), dtype), _ozeros(oracle, (B, Tq, Tv), dtype)
+    scale = 1 / math.sqrt(D)
+    oracle.attention_v2(oq, ov, ok, oo, ow, ol, scale=scale, causal=causal, q_mask=oqm, v_mask=ovm)
+    out, w, lg = ex.exec_custom("dot_product_attention_v2", [dq, dv, dk, dqm, dvm], t_args=[scale, 0.0], b_args=[causal, False])
+    assert_close(out.to_float(), _f(oo), tol, tol, "out")
+    assert_close(w.to_float(), _f(ow), tol, tol * 1e-2, "weights")
+    keep = (np.tril(np.ones((Tq, Tv), bool)) if causal else np.ones((Tq, Tv), bool))[None] & (vm != 0)[:, None, :]
+    assert_close(lg.to_float()[keep], _f(ol)[keep], tol, tol, "visible logits")
+    hidden = lg.to_float()[~keep]
+    assert hidden.size == 0 or hidden.max() < -6.0e4       # hidden logits carry the penalty
+    # output only, masks of other types: BOOL value mask, INT64 value mask as a strided view
+    bvm = NDArray.from_numpy(vm != 0)
+    out1 = ex.exec_custom("dot_product_attention_v2", [dq, dv, dk, dqm, bvm], [NDArray.empty((B, Tq, D), dtype)], t_args=[scale, 0.0], b_args=[causal, False])[0]
+    assert_close(out1.to_float(), _f(oo), tol, tol, "out-only call, BOOL mask")
+    ivm = NDArray.from_numpy(np.ascontiguousarray(vm.T).astype(np.int64)).permute(1, 0)
+    out2 = ex.exec_custom("dot_product_attention_v2", [dq, dv, dk, dqm, ivm], [NDArray.empty((B, Tq, D), dtype)], t_args=[scale, 0.0], b_args=[causal, False])[0]
+    assert np.array_equal(out2.to_numpy(), out1.to_numpy())
+
+
+@pytest.mark.parametrize("dtype,tol", [(FLOAT32, 1e-4), (HALF, 1e-2), (BFLOAT16, 1e-2)])
+def test_attention_padded_batch_identity_and_hidden_rows(ex, oracle, dtype, tol):
+    """Masked trailing keys == truncated keys; a batch entry whose keys are all padded follows the reference's arithmetic
+    (uniform-like weights over penalised logits for float / bfloat16, zero weights for half, whose penalty is -inf)."""
+    rng = np.random.default_rng(8)
+    B, Tq, Tv, D, cut = 3, 150, 256, 64, 170
+    q, k, v = rng.normal(0, 1, (B, Tq, D)), rng.normal(0, 1, (B, Tv, D)), rng.normal(0, 1, (B, Tv, D))
+    oq, dq = _pair(oracle, q, dtype)
+    ok, dk = _pair(oracle, k, dtype)
+    ov, dv = _pair(oracle, v, dtype)
+    vm = np.ones((B, Tv), np.float32)
+    vm[:, cut:] = 0
+    _, dvm = _pair(oracle, vm, dtype)
+    none = NDArray.empty((0,), dtype)                      # an absent query mask travels as an empty array
+    masked = ex.exec_custom("dot_product_attention_v2", [dq, dv, dk, none, dvm], [NDArray.empty((B, Tq, D), dtype)], t_args=[0.125, 0.0], b_args=[False, False])[0].to_float()
+    _, dk2 = _pair(oracle, k[:, :cut], dtype)
+    _, dv2 = _pair(oracle, v[:, :cut], dtype)
+    trunc = ex.exec_custom("dot_product_attention_v2", [dq, dv2, dk2], [NDArray.empty((B, Tq, D), dtype)], t_args=[0.125, 0.0], b_args=[False, False])[0].to_float()
+    assert_close(masked, trunc, tol, tol, "masked tail against truncated keys")
+    # batch entry 1 entirely padded, causal on top
+    vm2 = np.ones((B, Tv), np.float32)
+    vm2[1] = 0
+    ovm2, dvm2 = _pair(oracle, vm2, dtype)
+    oo = _ozeros(oracle, (B, Tq, D), dtype)
+    oracle.attention_v2(oq, ov, ok, oo, scale=0.125, causal=True, v_mask=ovm2)
+    got = ex.exec_custom("dot_product_attention_v2", [dq, dv, dk, none, dvm2], [NDArray.empty((B, Tq, D), dtype)], t_args=[0.125, 0.0], b_args=[True, False])[0].to_float()
+    assert_close(got, _f(oo), tol, tol, "entirely padded batch entry")
+
+
 def test_attention_rank4_and_default_keys(ex, oracle):
     rng = np.random.default_rng(41)
     B, H, T, D = 2, 3, 48, 64
