@@ -261,10 +261,12 @@ static XwGeometry xwGeometry(Context& c, bool needOutput) {
   }
   return g;
 }
-static void xwPlusBExec(Context& c) {
+// epi: extra outputs for the product's epilogue (already prepared for device use by the caller); returns whether the kernel
+// that ran wrote them
+static bool xwPlusBImpl(Context& c, const GemmEpilogue* epi) {
   ND4J_REQUIRE(c.width() >= 3, "xw_plus_b: x, weights and bias are required");
   NDArray* x = c.input(0); NDArray* w = c.input(1); NDArray* b = c.input(2); NDArray* z = c.output(0);
-  if (x->isEmpty() || w->isEmpty() || b->isEmpty()) return;
+  if (x->isEmpty() || w->isEmpty() || b->isEmpty()) return epi == nullptr;
   XwGeometry g = xwGeometry(c, true);
   const DataType dt = z->dataType();
   ND4J_REQUIRE(x->dataType() == dt && w->dataType() == dt && b->dataType() == dt && isFloatType(dt), "xw_plus_b: nd4j-hip requires one floating point type for x, weights, bias and output");
@@ -277,9 +279,12 @@ static void xwPlusBExec(Context& c) {
   d.aRow = g.aRow; d.aCol = g.aCol; d.bRow = g.bRow; d.bCol = g.bCol; d.cRow = g.cRow; d.cCol = g.cCol;
   prepareSpecialUse({z}, {x, w, b});
   d.bias = b->specialBuffer();
-  launchGemm(stream(), dt, x->specialBuffer(), w->specialBuffer(), z->specialBuffer(), d);
+  d.epi = epi;
+  const bool applied = launchGemm(stream(), dt, x->specialBuffer(), w->specialBuffer(), z->specialBuffer(), d);
   registerSpecialUse({z}, {x, w, b});
+  return applied;
 }
+static void xwPlusBExec(Context& c) { xwPlusBImpl(c, nullptr); }
 static std::vector<std::vector<LongType>> xwPlusBShapeFn(Context& c) {
   XwGeometry g = xwGeometry(c, false);
   return {makeShapeInfo(c.input(0)->dataType(), 'c', g.zShape)};
@@ -1781,5 +1786,162 @@ void executeOp(const OpDescriptor& op, Context& ctx) {
   op.exec(ctx);
 }
 
+
+// ---- merging of recorded op sequences -----------------------------------------------------------------------------------
+// the two handles name the same elements: same buffer, offset, shape, strides and type
+static bool sameView(const NDArray* a, const NDArray* b) {
+  if (a == b) return true;
+  if (!a || !b || a->buf.get() != b->buf.get() || a->bufOffsetBytes != b->bufOffsetBytes || a->offset != b->offset) return false;
+  if (a->rankOf() != b->rankOf() || a->dataType() != b->dataType()) return false;
+  for (int d = 0; d < a->rankOf(); d++) if (a->sizeAt(d) != b->sizeAt(d) || (a->sizeAt(d) != 1 && a->strideAt(d) != b->strideAt(d))) return false;
+  return true;
+}
+// a view seen as [rows, cols] with a unit column stride and one row stride: all dims but the last fold into the rows
+static bool asRows(const NDArray* a, LongType& rows, LongType& cols, LongType& rowStride) {
+  const int r = a->rankOf();
+  if (r < 1 || a->isEmpty()) return false;
+  cols = a->sizeAt(r - 1);
+  if (cols != 1 && a->strideAt(r - 1) != 1) return false;
+  rows = 1; rowStride = 0;
+  LongType expect = -1;
+  for (int d = r - 2; d >= 0; d--) {
+    const LongType n = a->sizeAt(d);
+    if (n == 1) continue;
+    if (expect < 0) rowStride = a->strideAt(d);
+    else if (a->strideAt(d) != expect) return false;
+    expect = a->strideAt(d) * n;
+    rows *= n;
+  }
+  if (rows == 1) rowStride = cols;
+  return true;
+}
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// layer_norm over the last axis with gain and bias, as the row kernel runs it
+static bool isRowLayerNorm(const RecordedOp& r) {
+  if (r.kind != RecordedOp::CUSTOM || r.op->name != "layer_norm" || r.ctx.inputs.size() != 3 || r.ctx.outputs.empty()) return false;
+  const NDArray* x = r.ctx.inputs[0];
+  if (!x || !r.ctx.inputs[1] || !r.ctx.inputs[2] || !r.ctx.outputs[0] || x->rankOf() < 1) return false;
+  if (bArg(r.ctx, 0, true)) return false;                            // gain / bias along the last axis
+  if (r.ctx.iArgs.size() != 1) return false;
+  const LongType ax = r.ctx.iArgs[0] < 0 ? r.ctx.iArgs[0] + x->rankOf() : r.ctx.iArgs[0];
+  return ax == x->rankOf() - 1;
+}
+
+static void runRecorded(RecordedOp* p) {
+  if (p->kind == RecordedOp::CUSTOM) executeOp(*p->op, p->ctx);
+  else p->run();
+}
+// z = x + y (pairwise Add, all of one float type), then ln = layer_norm(z): one kernel
+static bool tryAddLayerNorm(const RecordedOp& add, const RecordedOp& ln) {
+  NDArray *x = add.x, *y = add.y, *z = add.z;
+  NDArray *lx = ln.ctx.inputs[0], *g = ln.ctx.inputs[1], *b = ln.ctx.inputs[2], *lz = ln.ctx.outputs[0];
+  const DataType dt = z->dataType();
+  if (!isFloatType(dt) || dt == DOUBLE || x->dataType() != dt || y->dataType() != dt || lz->dataType() != dt || g->dataType() != dt || b->dataType() != dt) return false;
+  LongType rx, cx, sx, ry, cy, sy, rz, cz, sz, rl, cl, sl;
+  if (!asRows(x, rx, cx, sx) || !asRows(y, ry, cy, sy) || !asRows(z, rz, cz, sz) || !asRows(lz, rl, cl, sl)) return false;
+  if (rx != rz || ry != rz || rl != rz || cx != cz || cy != cz || cl != cz) return false;
+  if (g->lengthOf() != cz || b->lengthOf() != cz || (g->rankOf() == 1 && g->strideAt(0) != 1 && cz > 1) || (b->rankOf() == 1 && b->strideAt(0) != 1 && cz > 1)) return false;
+  // the normalised output must not overlap what the merged kernel still reads
+  if (lz->buf.get() == x->buf.get() || lz->buf.get() == y->buf.get() || lz->buf.get() == z->buf.get()) return false;
+  if (y->buf.get() == z->buf.get() && !sameView(y, z)) return false;
+  if (x->buf.get() == z->buf.get() && !sameView(x, z)) return false;
+  std::vector<NDArray*> writes = {z, lz}, reads = {x, y, g, b};
+  prepareSpecialUse(writes, reads);
+  const bool ok = launchAddLayerNormRows(stream(), dt, x->specialBuffer(), y->specialBuffer(), z->specialBuffer(), g->specialBuffer(), b->specialBuffer(),
+                                         lz->specialBuffer(), rz, cz, sx, sy, sz, sl, 1e-5f);
+  registerSpecialUse(writes, reads);
+  return ok;
+}
+
 }  // namespace ops
+
+std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& rec, int& nFused) {
+  using namespace ops;
+  std::vector<std::function<void()>> plan;
+  nFused = 0;
+  const size_t n = rec.size();
+  for (size_t i = 0; i < n;) {
+    RecordedOp& r = rec[i];
+    // pairwise Add whose result the next op layer-normalises
+    if (r.kind == RecordedOp::PAIRWISE && r.opNum == 0 && i + 1 < n && isRowLayerNorm(rec[i + 1]) && sameView(r.z, rec[i + 1].ctx.inputs[0])) {
+      RecordedOp* a = &r;
+      RecordedOp* l = &rec[i + 1];
+      plan.push_back([a, l] { if (!tryAddLayerNorm(*a, *l)) { runRecorded(a); runRecorded(l); } });
+      nFused += 1;
+      i += 2;
+      continue;
+    }
+    // xw_plus_b followed by ops on its result that the product's epilogue can write: the GELU transform of the whole
+    // result, and assigns of column slices of it (key / value rows going into their caches)
+    if (r.kind == RecordedOp::CUSTOM && r.op->name == "xw_plus_b" && r.ctx.outputs.size() >= 1 && r.ctx.outputs[0] && r.ctx.inputs.size() >= 3) {
+      NDArray* z = r.ctx.outputs[0];
+      LongType zr, zc, zs;
+      const DataType dt = z->dataType();
+      const bool zOk = (dt == HALF || dt == BFLOAT16) && asRows(z, zr, zc, zs) && iArg(r.ctx, 2, 0) != 1;
+      GemmEpilogue epi;
+      std::vector<RecordedOp*> absorbed;
+      size_t j = i + 1;
+      while (zOk && j < n) {
+        RecordedOp& f = rec[j];
+        bool inputsTouched = false;   // an absorbed op must not write what the product reads
+        for (NDArray* in : r.ctx.inputs) if (in && f.z && in->buf.get() == f.z->buf.get()) inputsTouched = true;
+        if (inputsTouched) break;
+        LongType fr, fc, fs;
+        if (f.kind == RecordedOp::TRANSFORM_STRICT && f.opNum == 53 && epi.act == 0 && sameView(f.x, z) && f.z->dataType() == dt && asRows(f.z, fr, fc, fs) &&
+            fr == zr && fc == zc && f.z->buf.get() != z->buf.get()) {
+          // which GELU form the separate transform would take: dense, aligned 16-bit arrays of a multiple of 8 elements run the
+          // one-instruction exponential on every element
+          const bool dense = zs == zc && fs == fc && (zr * zc) % 8 == 0;
+          if (!dense) break;
+          epi.act = 1; epi.actOut = f.z; epi.actRow = fs;   // handle now, device pointer when the step runs
+          absorbed.push_back(&f);
+          j++;
+          continue;
+        }
+        if (f.kind == RecordedOp::TRANSFORM_ANY && epi.nCopy < 2 && f.x->buf.get() == z->buf.get() && f.x->bufOffsetBytes == z->bufOffsetBytes && f.x->dataType() == dt &&
+            f.z->dataType() == dt && f.z->buf.get() != z->buf.get()) {
+          LongType sr, sc, ss, dr, dc, ds;
+          if (!asRows(f.x, sr, sc, ss) || !asRows(f.z, dr, dc, ds) || sr != zr || dr != zr || dc != sc) break;
+          if (zr > 1 && ss != zs) break;
+          const LongType c0 = f.x->offset - z->offset;
+          if (c0 < 0 || c0 + sc > zc) break;
+          epi.copy[epi.nCopy].dst = f.z; epi.copy[epi.nCopy].c0 = c0; epi.copy[epi.nCopy].c1 = c0 + sc; epi.copy[epi.nCopy].dstRow = ds;
+          epi.nCopy++;
+          absorbed.push_back(&f);
+          j++;
+          continue;
+        }
+        break;
+      }
+      if (!absorbed.empty()) {
+        RecordedOp* x = &r;
+        plan.push_back([x, epi, absorbed]() mutable {
+          // the extra outputs become device pointers now (their buffers are allocated by this point)
+          GemmEpilogue e = epi;
+          std::vector<NDArray*> writes;
+          x->ctx.outputs[0]->buf->allocateSpecial();
+          bool aligned = aligned16(x->ctx.outputs[0]->specialBuffer());
+          if (e.act) { NDArray* a = static_cast<NDArray*>(e.actOut); writes.push_back(a); }
+          for (int c = 0; c < e.nCopy; c++) writes.push_back(static_cast<NDArray*>(e.copy[c].dst));
+          prepareSpecialUse(writes, std::vector<NDArray*>{});
+          if (e.act) { e.actOut = static_cast<NDArray*>(epi.actOut)->specialBuffer(); aligned = aligned && aligned16(e.actOut); }
+          for (int c = 0; c < e.nCopy; c++) e.copy[c].dst = static_cast<NDArray*>(epi.copy[c].dst)->specialBuffer();
+          // (a misaligned GELU operand would send the separate transform down another evaluation path: keep the ops apart)
+          const bool applied = xwPlusBImpl(x->ctx, e.act && !aligned ? nullptr : &e) && !(e.act && !aligned);
+          if (applied) registerSpecialUse(writes, std::vector<NDArray*>{x->ctx.outputs[0]});
+          else for (RecordedOp* f : absorbed) runRecorded(f);
+        });
+        nFused += (int)absorbed.size();
+        i = j;
+        continue;
+      }
+    }
+    RecordedOp* p = &r;
+    plan.push_back([p] { runRecorded(p); });
+    i++;
+  }
+  return plan;
+}
+
 }  // namespace nd4jhip

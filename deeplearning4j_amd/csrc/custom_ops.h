@@ -28,6 +28,23 @@ void executeOp(const OpDescriptor& op, Context& ctx);
 
 }  // namespace ops
 
+// ---- recorded op sequences --------------------------------------------------------------------------------------------
+// While a stream capture is open the facade also notes every op call it recognises (what was called, on which arrays, with
+// which arguments, and a closure that runs it as the eager call does).  When every call of the capture was recognised,
+// the sequence is replayed through fuseRecordedOps before the graph is instantiated: neighbouring ops that one kernel can
+// serve are merged (a pairwise Add and the layer_norm of its result; xw_plus_b and the GELU transform / the column-slice
+// assigns that follow it), every merged kernel writing exactly what the separate ops would have written, bit for bit.
+struct RecordedOp {
+  enum Kind { CUSTOM, PAIRWISE, TRANSFORM_STRICT, TRANSFORM_ANY } kind = CUSTOM;
+  const ops::OpDescriptor* op = nullptr;   // CUSTOM
+  Context ctx;                             // CUSTOM: copy of the caller's argument bag (arrays borrowed)
+  int opNum = 0;                           // legacy loops
+  NDArray *x = nullptr, *y = nullptr, *z = nullptr;
+  std::function<void()> run;               // executes the op exactly as the eager call does
+};
+// The launch plan of the sequence; nFused counts the ops that were absorbed into a neighbour's kernel.
+std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& ops, int& nFused);
+
 // shared with the legacy facade
 void runIndexReduce(const char* fn, int opNum, NDArray* x, NDArray* z, const std::vector<LongType>& dims);
 // value reductions and summary statistics behind both the legacy entry points and the reduce_* custom ops

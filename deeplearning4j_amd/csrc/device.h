@@ -124,6 +124,12 @@ __device__ __forceinline__ float fast_exp(float x) {
 }
 __device__ __forceinline__ double fast_exp(double x) { return exp(x); }
 
+// GELU as the legacy transform evaluates it, x * sigmoid(1.702 x) (ops.h:1010-1012), in the two forms the elementwise kernels
+// use: the full-precision exponential, and for dense 16-bit arrays one v_exp_f32 of x * log2(e).  GEMM epilogues that apply
+// the activation call the same functions, so a fused step reproduces the separate transform bit for bit.
+__device__ __forceinline__ float gelu_full(float x) { const float u = 1.702f * x; return x * fast_rcp(1.f + fast_exp(-u)); }
+__device__ __forceinline__ float gelu_low(float x) { const float u = 1.702f * x; return x * fast_rcp(1.f + __builtin_amdgcn_exp2f(u * -1.44269502162933349609375f)); }
+
 // ---- wave reductions ---------------------------------------------------------------------------------
 // Butterfly over a row of 16 lanes with DPP (quad_perm 1,0,3,2 / 2,3,0,1 / row_half_mirror / row_mirror),
 // then lanes 16 and 32 apart through the cross-lane permute.  Valid for commutative, associative ops;

@@ -87,7 +87,9 @@ UNARY(U_SOFTPLUS, d_log((A)1 + fast_exp(x)));                  // templatemath.h
 UNARY(U_TANH, d_tanh(x));                                      // ops.h:199
 UNARY_LOW(U_SWISH, x * d_sigmoid<A>(x), x * d_sigmoid_low(x)); // ops.h:988-990
 UNARY(U_ERF, d_erf(x));                                        // ops.h:361
-UNARY_LOW(U_GELU, x * d_sigmoid<A>((A)1.702f * x), x * d_sigmoid_low((A)1.702f * x));   // ops.h:1010-1012
+__device__ __forceinline__ double gelu_full(double x) { return x * d_sigmoid<double>(1.702f * x); }
+__device__ __forceinline__ double gelu_low(double x) { return x * d_sigmoid_low(1.702f * x); }
+UNARY_LOW(U_GELU, gelu_full(x), gelu_low(x));   // ops.h:1010-1012; the float forms live in device.h, shared with the GEMM epilogue
 UNARY(U_PRECISE_GELU, d_pgelu(x));
 UNARY(U_SQRT, d_sqrt(x));                                      // ops.h:2200
 UNARY(U_RSQRT, (A)1 / d_sqrt(x));                              // ops.h:2203-2205

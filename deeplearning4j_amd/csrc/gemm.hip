@@ -42,6 +42,8 @@ struct GemmArgs {
   LongType ktPerSplit;
   float* partial;
   const void* bias;   // optional [N] row added to every output row (xw_plus_b), same type as C
+  int hasEpi;
+  GemmEpilogue epi;   // extra outputs derived from the stored C (kernels that call epilogueExtras)
 };
 typedef __attribute__((ext_vector_type(4))) float f32x4v;
 
@@ -66,6 +68,22 @@ __device__ __forceinline__ void batchOffsets(const GemmArgs& g, LongType bz, Lon
     oa = bz * g.aBatch; ob = bz * g.bBatch; oc = bz * g.cBatch;
   }
 }
+
+// the extra outputs of a fused step, from the value just stored to C[row][col]
+template <typename T>
+__device__ __forceinline__ void epilogueExtras(int hasEpi, const GemmEpilogue& epi, LongType row, LongType col, T yv) {
+  if (!hasEpi) return;
+  const float y = to_float(yv);
+  if (epi.act) static_cast<T*>(epi.actOut)[row * epi.actRow + col] = Conv<T>::from(epi.act == 1 ? gelu_low(y) : gelu_full(y));
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+    if (i < epi.nCopy && col >= epi.copy[i].c0 && col < epi.copy[i].c1)
+      static_cast<T*>(epi.copy[i].dst)[row * epi.copy[i].dstRow + col - epi.copy[i].c0] = yv;
+  if (epi.resOut)
+    static_cast<T*>(epi.resOut)[row * epi.resOutRow + col] = Conv<T>::from(to_float(static_cast<const T*>(epi.resIn)[row * epi.resInRow + col]) + y);
+}
+template <typename T>
+__device__ __forceinline__ void epilogueExtras(const GemmArgs& g, LongType row, LongType col, T yv) { epilogueExtras<T>(g.hasEpi, g.epi, row, col, yv); }
 
 // ---- fallback --------------------------------------------------------------------------------------------------
 template <typename T>
@@ -279,7 +297,9 @@ __global__ __launch_bounds__(WM * WN * 64) void splitk_finish(GemmArgs g, T* __r
     float v = g.alpha * tot[e];
     if (g.beta != 0.f) v += g.beta * to_float(C[off]);
     if (g.bias) v += to_float(static_cast<const T*>(g.bias)[col]);
-    C[off] = Conv<T>::from(v);
+    const T yv = Conv<T>::from(v);
+    C[off] = yv;
+    epilogueExtras<T>(g, row0 + e, col, yv);
   }
 }
 
@@ -886,7 +906,7 @@ static int chooseSplits(const GemmArgs& g, LongType batch, LongType& ktPerSplit)
 }
 
 template <typename T, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC>
-static void launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void* B, void* C, LongType batch, bool allowSplit = false) {
+static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void* B, void* C, LongType batch, bool allowSplit = false) {
   constexpr int NT = WM * WN * 64;
   constexpr size_t LDS = (size_t)2 * (TileLayout<BM, A_KC>::SLOTS + TileLayout<BN, B_KC>::SLOTS) * 16;
   int splits = 1;
@@ -899,6 +919,8 @@ static void launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
       g.partial = static_cast<float*>(lc->allocationBuffer);
     }
   }
+  // an epilogue request is served by splitk_finish only (one batch entry, unit column stride of C)
+  if (g.hasEpi && (splits == 1 || batch != 1 || g.cCol != 1)) return false;
   const bool usePipe = splits == 1;   // the split-K epilogue lives in the plain kernel
   // whole tiles only: the kernel without bounds handling (its K loop needs two K-tiles at least)
   const bool useFull = usePipe && BM * BN >= 128 * 128 && g.M % BM == 0 && g.N % BN == 0 && g.K % 64 == 0 && g.K >= 128;
@@ -918,15 +940,17 @@ static void launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
   hipLaunchKernelGGL(kern, dim3(tilesM * tilesN, (unsigned)splits, (unsigned)batch), dim3(NT), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tilesM, tilesN);
   if (splits > 1)
     hipLaunchKernelGGL((splitk_finish<T, BM, BN, WM, WN>), dim3(tilesM * tilesN, (BM / WM / 32) * (BN / WN / 32) * 4, (unsigned)batch), dim3(NT), 0, s, g, (T*)C, tilesM, tilesN);
+  return true;
 }
 
 template <typename T, bool A_KC, bool B_KC>
-static void launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C, LongType batch) {
+static bool launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C, LongType batch) {
   const LongType tiles256 = ((g.M + 255) / 256) * ((g.N + 255) / 256) * batch;
   const LongType tiles128 = ((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
   if (g.M <= 32) return launchMfma16Cfg<T, 32, 128, 1, 4, A_KC, B_KC>(s, g, A, B, C, batch, true);
   if (g.M <= 64 || g.N <= 64 || tiles128 < 192) return launchMfma16Cfg<T, 64, 64, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch, true);
   if (tiles256 < 192) return launchMfma16Cfg<T, 128, 128, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
+  if (g.hasEpi) return false;
   static const bool direct = getenv("ND4JHIP_GEMM_DIRECT") ? atoi(getenv("ND4JHIP_GEMM_DIRECT")) != 0 : true;
   if (direct && A_KC && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 64 == 0 && g.K >= 128) {
     constexpr size_t LDS = 2 * 2 * 256 * 8 * 16;
@@ -936,7 +960,7 @@ static void launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const 
     const unsigned tM = (unsigned)(g.M / 256), tN = (unsigned)(g.N / 256);
     noteKernel("gemm_mfma16d<%s,256x256,akc=1,bkc=%d>", tname<T>(), (int)B_KC);
     hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(512), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
-    return;
+    return true;
   }
   return launchMfma16Cfg<T, 256, 256, 2, 4, A_KC, B_KC>(s, g, A, B, C, batch);
 }
@@ -1244,7 +1268,7 @@ __global__ __launch_bounds__(256) void gemv_rowdot(const T* __restrict__ W, Long
 // against k-contiguous weights run at the cost of a streaming read.
 template <typename T, int OPW, int NL, bool HAS_BIAS>
 __global__ __launch_bounds__(256) void gemv_rowdot_pre(const T* __restrict__ W, LongType ldw, const T* __restrict__ x, T* __restrict__ y, LongType ys,
-                                                       LongType N, LongType K, const T* __restrict__ bias) {
+                                                       LongType N, LongType K, const T* __restrict__ bias, int hasEpi, GemmEpilogue epi) {
   constexpr int V = 16 / sizeof(T);
   using Raw = typename RawIO<T>::raw;
   const int lane = threadIdx.x & 63;
@@ -1291,7 +1315,11 @@ __global__ __launch_bounds__(256) void gemv_rowdot_pre(const T* __restrict__ W, 
 #pragma unroll
   for (int o = 0; o < OPW; o++) {
     const float v = wave_allreduce<SumOp>(acc[o]);
-    if (lane == 0 && n0 + o < N) y[(n0 + o) * ys] = Conv<T>::from(v);
+    if (lane == 0 && n0 + o < N) {
+      const T yv = Conv<T>::from(v);
+      y[(n0 + o) * ys] = yv;
+      epilogueExtras<T>(hasEpi, epi, 0, n0 + o, yv);
+    }
   }
 }
 template <typename T>
@@ -1301,7 +1329,7 @@ static bool tryGemvRowdotPre(hipStream_t s, const GemmDesc& d, const void* A, co
   if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) return false;
   const LongType passes = (d.K / V + 63) / 64;
 #define ROWDOT_B(OPW, NL, HB) hipLaunchKernelGGL((gemv_rowdot_pre<T, OPW, NL, HB>), dim3((unsigned)(((d.N + OPW - 1) / OPW + 3) / 4)), dim3(256), 0, s, \
-                                                 (const T*)B, d.bCol, (const T*)A, (T*)C, d.cCol, d.N, d.K, (const T*)d.bias)
+                                                 (const T*)B, d.bCol, (const T*)A, (T*)C, d.cCol, d.N, d.K, (const T*)d.bias, d.epi ? 1 : 0, d.epi ? *d.epi : GemmEpilogue())
 #define ROWDOT(OPW, NL) do { noteKernel("gemv_rowdot_pre<%s,opw=%d,nl=%d>", tname<T>(), OPW, NL); if (d.bias) ROWDOT_B(OPW, NL, true); else ROWDOT_B(OPW, NL, false); } while (0)
   if (passes <= 2) ROWDOT(2, 2);
   else if (passes <= 4) ROWDOT(2, 4);
@@ -1362,11 +1390,12 @@ static bool tryGemv(hipStream_t s, const GemmDesc& d, const void* A, const void*
   constexpr int V = 16 / sizeof(T);
   if (d.M == 1 && d.N > 1) {
     // y[n] = sum_k a[k] * op(B)[k][n]
-    if (d.bRow == 1 && tryGemvRowdotPre<T>(s, d, A, B, C)) return true;
+    if (d.bRow == 1 && (!d.epi || d.cCol == 1) && tryGemvRowdotPre<T>(s, d, A, B, C)) return true;
+    if (d.epi) return false;
     if (d.bRow == 1) { noteKernel("gemv_rowdot<%s>", tname<T>()); hipLaunchKernelGGL((gemv_rowdot<T>), dim3((unsigned)((d.N + 3) / 4)), dim3(256), 0, s, (const T*)B, d.bCol, (const T*)A, d.aCol, (T*)C, d.cCol, d.N, d.K, d.alpha, d.beta, (const T*)d.bias); return true; }
     if (d.bCol == 1) { noteKernel("gemv_colsum<%s>", tname<T>()); hipLaunchKernelGGL((gemv_colsum<T>), dim3((unsigned)((d.N + 64 * V - 1) / (64 * V))), dim3(256), 0, s, (const T*)B, d.bRow, (const T*)A, d.aCol, (T*)C, d.cCol, d.N, d.K, d.alpha, d.beta, (const T*)d.bias); return true; }
   }
-  if (d.N == 1 && d.M > 1 && !d.bias) {
+  if (d.N == 1 && d.M > 1 && !d.bias && !d.epi) {
     // y[m] = sum_k op(A)[m][k] * b[k]
     if (d.aCol == 1) { noteKernel("gemv_rowdot<%s>", tname<T>()); hipLaunchKernelGGL((gemv_rowdot<T>), dim3((unsigned)((d.M + 3) / 4)), dim3(256), 0, s, (const T*)A, d.aRow, (const T*)B, d.bRow, (T*)C, d.cRow, d.M, d.K, d.alpha, d.beta, (const T*)nullptr); return true; }
     if (d.aRow == 1) { noteKernel("gemv_colsum<%s>", tname<T>()); hipLaunchKernelGGL((gemv_colsum<T>), dim3((unsigned)((d.M + 64 * V - 1) / (64 * V))), dim3(256), 0, s, (const T*)A, d.aCol, (const T*)B, d.bRow, (T*)C, d.cRow, d.M, d.K, d.alpha, d.beta, (const T*)nullptr); return true; }
@@ -1383,6 +1412,8 @@ static GemmArgs toArgs(const GemmDesc& d) {
   g.batchInner = d.batchInner; g.aBatch2 = d.aBatch2; g.bBatch2 = d.bBatch2; g.cBatch2 = d.cBatch2;
   g.alpha = d.alpha; g.beta = d.beta;
   g.splits = 1; g.ktPerSplit = 0; g.partial = nullptr; g.bias = d.bias;
+  g.hasEpi = d.epi ? 1 : 0;
+  if (d.epi) g.epi = *d.epi;
   return g;
 }
 
@@ -1518,7 +1549,7 @@ static void launchGemvStripM(hipStream_t s, const GemmArgs& g, const void* A, co
 // whether the strip kernel takes this product: a few dense rows, W row-major with aligned rows, plain C = A B (+ bias)
 template <typename T>
 static bool tryGemvStrip(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
-  if (d.M < 1 || d.M > 4 || d.batch != 1 || d.alpha != 1.f || d.beta != 0.f) return false;
+  if (d.M < 1 || d.M > 4 || d.batch != 1 || d.alpha != 1.f || d.beta != 0.f || d.epi) return false;
   if (d.aCol != 1 || d.bCol != 1 || d.cCol != 1 || d.bRow % 8 != 0) return false;
   if (d.N % 32 != 0 || d.K % 256 != 0 || d.N < 256) return false;
   if ((reinterpret_cast<uintptr_t>(B) & 15) != 0) return false;
@@ -1603,6 +1634,10 @@ __global__ __launch_bounds__(256) void gemm_skinny32(GemmArgs g, const T* __rest
     o[0] = (unsigned)Conv<T>::from(v[0]).bits | ((unsigned)Conv<T>::from(v[1]).bits << 16);
     o[1] = (unsigned)Conv<T>::from(v[2]).bits | ((unsigned)Conv<T>::from(v[3]).bits << 16);
     *reinterpret_cast<u32x2*>(C + (LongType)mrow * g.cRow + n) = o;
+    if (g.hasEpi) {
+#pragma unroll
+      for (int e = 0; e < 4; e++) epilogueExtras<T>(g, mrow, n + e, Conv<T>::from(v[e]));
+    }
   }
 }
 template <typename T>
@@ -1621,15 +1656,15 @@ static bool tryGemmSkinny(hipStream_t s, const GemmDesc& d, const void* A, const
 }
 
 template <typename T>
-static void dispatch16(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
+static bool dispatch16(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
   bool aKC = false, bKC = false;
   const bool eligible = (d.M * d.N >= 1024 || (d.M == 1 && d.N >= 64)) && d.K >= 32 && mfmaEligible(d, A, B, sizeof(T), aKC, bKC);
   // x[1, K] times row-major W[K, N]: the split-K tile kernel streams W with far more loads in flight than the
   // column-sum GEMV (the unused 31 rows of the MFMA tile cost nothing here)
-  if (tryGemvStrip<T>(s, d, A, B, C)) return;
-  if (tryGemmSkinny<T>(s, d, A, B, C)) return;
+  if (tryGemvStrip<T>(s, d, A, B, C)) return true;
+  if (tryGemmSkinny<T>(s, d, A, B, C)) return true;
   const bool rowTimesRowMajor = d.M == 1 && eligible && aKC && !bKC && d.batch == 1;
-  if (!rowTimesRowMajor && tryGemv<T>(s, d, A, B, C)) return;
+  if (!rowTimesRowMajor && tryGemv<T>(s, d, A, B, C)) return true;
   if (eligible) {
     GemmArgs g = toArgs(d);
     if (aKC && bKC) return launchMfma16<T, true, true>(s, g, A, B, C, d.batch);
@@ -1637,7 +1672,9 @@ static void dispatch16(hipStream_t s, const GemmDesc& d, const void* A, const vo
     if (!aKC && bKC) return launchMfma16<T, false, true>(s, g, A, B, C, d.batch);
     return launchMfma16<T, false, false>(s, g, A, B, C, d.batch);
   }
+  if (d.epi) return false;
   launchSimple<T>(s, A, B, C, d);
+  return true;
 }
 static void dispatch32(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
   if (tryGemv<float>(s, d, A, B, C)) return;
@@ -1652,9 +1689,22 @@ static void dispatch32(hipStream_t s, const GemmDesc& d, const void* A, const vo
   launchSimple<float>(s, A, B, C, d);
 }
 
-void launchGemm(hipStream_t s, DataType dt, const void* A, const void* B, void* C, const GemmDesc& d) {
-  if (d.M == 0 || d.N == 0 || d.batch == 0) return;
+bool launchGemm(hipStream_t s, DataType dt, const void* A, const void* B, void* C, const GemmDesc& d) {
+  if (d.M == 0 || d.N == 0 || d.batch == 0) return true;
   ND4J_REQUIRE(d.batch < 65536 && (d.M + 31) / 32 < 65536 && (d.N + 31) / 32 < (1LL << 31), "matmul: problem too large for the launch grid");
+  bool withEpilogue = d.epi != nullptr;
+  if (withEpilogue) {
+    // only the 16-bit decode-step kernels carry epilogue outputs; when the dispatch lands elsewhere nothing has been
+    // launched yet and the product runs again without the request
+    bool done = false;
+    if (dt == HALF) done = dispatch16<f16_t>(s, d, A, B, C);
+    else if (dt == BFLOAT16) done = dispatch16<bf16_t>(s, d, A, B, C);
+    if (done) { HIP_CHECK(hipGetLastError()); return true; }
+    GemmDesc plain = d;
+    plain.epi = nullptr;
+    launchGemm(s, dt, A, B, C, plain);
+    return false;
+  }
   switch (dt) {
     case FLOAT32: dispatch32(s, d, A, B, C); break;
     case DOUBLE: launchSimple<double>(s, A, B, C, d); break;
@@ -1663,6 +1713,7 @@ void launchGemm(hipStream_t s, DataType dt, const void* A, const void* B, void* 
     default: ND4J_THROW("matmul: unsupported dtype");
   }
   HIP_CHECK(hipGetLastError());
+  return true;
 }
 
 }  // namespace nd4jhip

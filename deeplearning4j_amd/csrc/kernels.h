@@ -143,6 +143,10 @@ void launchSoftmax(hipStream_t s, DataType dt, const void* x, void* z, const Row
 void launchLogSoftmax(hipStream_t s, DataType dt, const void* x, void* z, const RowPlan& p);
 void launchLayerNormRows(hipStream_t s, DataType dt, const void* x, const void* gain, const void* bias, void* z,
                          const RowPlan& p, float eps);
+// sumOut = x + addend (pairwise Add in the array type), z = layer_norm(sumOut) over rows of length L at constant pitches, in
+// one kernel; false when the shape is not the one-wave-per-row vector case (nothing launched then)
+bool launchAddLayerNormRows(hipStream_t s, DataType dt, const void* x, const void* addend, void* sumOut, const void* gain, const void* bias,
+                            void* z, LongType rows, LongType L, LongType xPitch, LongType aPitch, LongType sPitch, LongType zPitch, float eps);
 // gradI = softmaxed * (gradO - sum_row(softmaxed * gradO)); pg = row plan (gradO, gradI), ps = (softmaxed, gradI)
 void launchSoftmaxBp(hipStream_t s, DataType dt, const void* gradO, const void* softmaxed, void* gradI, const RowPlan& pg,
                      const RowPlan& ps);
@@ -165,6 +169,23 @@ void launchStandardizeBp(hipStream_t s, DataType dt, const void* x, const void* 
                          const LnGenericPlan& px, const LnGenericPlan& pe);
 
 // ---- GEMM ------------------------------------------------------------------------------------------
+// Extra outputs a product can write from its epilogue, each what a separate op would have computed from the stored result
+// C (same rounding points), so that a recorded op sequence "product, then an elementwise op on it" can run as one kernel:
+//   act:   actOut[m][n] = GELU(C[m][n])                       (the legacy transform opNum 53 applied to C)
+//   copy:  dst[m * dstRow + n - c0] = C[m][n] for c0 <= n < c1   (an assign of a column slice of C, e.g. into a key / value cache)
+//   res:   resOut[m][n] = resIn[m][n] + C[m][n]               (a pairwise Add of C to another array of the same shape)
+// Rows have unit column stride everywhere.  Only some kernels carry these (the decode-step ones); launchGemm says whether
+// the one it chose did.
+struct GemmEpilogue {
+  int act = 0;              // 0 none, 1 GELU as the dense 16-bit transform evaluates it, 2 GELU in its full-precision form
+  void* actOut = nullptr;
+  LongType actRow = 0;
+  int nCopy = 0;
+  struct Copy { void* dst; LongType c0, c1, dstRow; } copy[2] = {{nullptr, 0, 0, 0}, {nullptr, 0, 0, 0}};
+  const void* resIn = nullptr;
+  void* resOut = nullptr;
+  LongType resInRow = 0, resOutRow = 0;
+};
 struct GemmDesc {
   LongType M = 0, N = 0, K = 0, batch = 1;
   LongType aRow = 0, aCol = 0;   // element strides of op(A)[m][k]
@@ -176,8 +197,11 @@ struct GemmDesc {
   LongType batchInner = 0, aBatch2 = 0, bBatch2 = 0, cBatch2 = 0;
   float alpha = 1.f, beta = 0.f;
   const void* bias = nullptr;   // optional dense [N] row (type of C) added to every output row
+  const GemmEpilogue* epi = nullptr;
 };
-void launchGemm(hipStream_t s, DataType dt, const void* A, const void* B, void* C, const GemmDesc& d);
+// Returns true when every requested epilogue output was written; false: C was computed by a kernel without them and the
+// caller runs the follow-up ops itself (always true without an epilogue request).
+bool launchGemm(hipStream_t s, DataType dt, const void* A, const void* B, void* C, const GemmDesc& d);
 // name of the kernel the calling thread's most recent launchGemm chose
 const char* lastGemmKernel();
 

@@ -44,10 +44,12 @@ static std::recursive_mutex& opMutex() {
 // declarable ops; a device backend passes what lcExecutionStream returned, ref CudaExecutioner.java:641-649): work the
 // caller queued there is ordered before the op, and the op before whatever the caller queues next.  A null slot or the
 // library's own stream needs nothing.
+static int* g_captureOpCalls = nullptr;   // while a capture is open: how many op entry points were called
 struct OpScope {
   std::lock_guard<std::recursive_mutex> lock;
   hipStream_t caller = nullptr;
-  explicit OpScope(void* streamPtr) : lock(opMutex()) {
+  explicit OpScope(void* streamPtr, bool isOp = true) : lock(opMutex()) {
+    if (isOp && g_captureOpCalls && captureActive()) ++*g_captureOpCalls;
     if (streamPtr == nullptr || captureActive()) return;
     hipStream_t cs = *reinterpret_cast<hipStream_t*>(streamPtr);
     LaunchContext* lc = LaunchContext::defaultContext();
@@ -64,6 +66,10 @@ struct OpScope {
 };
 static void* callerStream(Nd4jPointer* extraPointers) { return extraPointers ? extraPointers[1] : nullptr; }
 #define OP_BEGIN(streamPtr) try { OpScope _opScope(streamPtr);
+#define GRAPH_BEGIN try { OpScope _opScope(nullptr, false);
+static void recordOp(RecordedOp&& r);
+static void transformStrictImpl(int opNum, NDArray* x, void* extraParams, NDArray* z);
+static void pairwiseImpl(int opNum, NDArray* x, NDArray* y, NDArray* z);
 
 static NDArray* arr(OpaqueNDArray a, const char* fn, const char* name) {
   if (a == nullptr) ND4J_THROW(std::string(fn) + ": " + name + " is null");
@@ -501,6 +507,18 @@ static void runUnaryWithParams(const char* fn, Scalar2Kind k, NDArray* x, NDArra
 void execTransformStrict(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void* extraParams, OpaqueNDArray za) {
   OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execTransformStrict", "x"); NDArray* z = arr(za, "execTransformStrict", "z");
+  transformStrictImpl(opNum, x, extraParams, z);
+  if (captureActive() && !(opNum == 2 || opNum == 3 || opNum == 19 || opNum == 25)) {
+    RecordedOp r;
+    r.kind = RecordedOp::TRANSFORM_STRICT; r.opNum = opNum; r.x = x; r.z = z;
+    r.run = [opNum, x, z] { transformStrictImpl(opNum, x, nullptr, z); };
+    recordOp(std::move(r));
+  }
+  GUARD_END_VOID
+}
+}  // extern "C"
+static void transformStrictImpl(int opNum, NDArray* x, void* extraParams, NDArray* z) {
+  {
   // X -> X over float types only (NativeOpExecutioner_transform.cpp:115-131)
   ND4J_REQUIRE(x->dataType() == z->dataType() && isFloatType(x->dataType()),
                std::string("NativeOpExecutioner::execTransformStrict requires X & Z to have same floating point type, got ") + dtypeName(x->dataType()) + " and " + dtypeName(z->dataType()));
@@ -529,8 +547,9 @@ void execTransformStrict(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa
     default: ND4J_THROW("execTransformStrict: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
   runUnary("execTransformStrict", k, x, z);
-  GUARD_END_VOID
+  }
 }
+extern "C" {
 void execTransformFloat(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
   OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execTransformFloat", "x"); NDArray* z = arr(za, "execTransformFloat", "z");
@@ -572,6 +591,12 @@ void execTransformAny(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, v
   NDArray* x = arr(xa, "execTransformAny", "x"); NDArray* z = arr(za, "execTransformAny", "z");
   ND4J_REQUIRE(opNum == 0, "execTransformAny: only Assign (opNum 0) exists (loops/legacy_ops.h:46)");
   runUnary("execTransformAny", U_IDENTITY, x, z);
+  if (captureActive()) {
+    RecordedOp r;
+    r.kind = RecordedOp::TRANSFORM_ANY; r.opNum = 0; r.x = x; r.z = z;
+    r.run = [x, z] { runUnary("execTransformAny", U_IDENTITY, x, z); };
+    recordOp(std::move(r));
+  }
   GUARD_END_VOID
 }
 
@@ -593,6 +618,17 @@ void execPairwiseTransform(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray 
   OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execPairwiseTransform", "x"); NDArray* y = arr(ya, "execPairwiseTransform", "y");
   NDArray* z = arr(za, "execPairwiseTransform", "z");
+  pairwiseImpl(opNum, x, y, z);
+  if (captureActive()) {
+    RecordedOp r;
+    r.kind = RecordedOp::PAIRWISE; r.opNum = opNum; r.x = x; r.y = y; r.z = z;
+    r.run = [opNum, x, y, z] { pairwiseImpl(opNum, x, y, z); };
+    recordOp(std::move(r));
+  }
+  GUARD_END_VOID
+}
+}  // extern "C"
+static void pairwiseImpl(int opNum, NDArray* x, NDArray* y, NDArray* z) {
   // NativeOpExecutioner_pairwise_floats.cpp:34-57
   ND4J_REQUIRE(x->dataType() == z->dataType() || y->dataType() == z->dataType(),
                std::string("NativeOpExecutioner::execPairwiseTransform requires X or Y to have the same type as Z, got ") + dtypeName(x->dataType()) + ", " + dtypeName(y->dataType()) + " -> " + dtypeName(z->dataType()));
@@ -611,8 +647,8 @@ void execPairwiseTransform(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray 
   // a second time for views (legacy/cpu/NativeOps.cpp:1245-1257)
   launchPairwise(execStream(), k, x->dataType(), y->dataType(), z->dataType(), x->specialBuffer(), y->specialBuffer(), z->specialBuffer(), p);
   registerSpecialUse({z}, {x, y});
-  GUARD_END_VOID
 }
+extern "C" {
 
 static LongType hostScalarInt64(NDArray* s) {
   ND4J_REQUIRE(s->lengthOf() >= 1 && s->buf, "scalar operand is empty");
@@ -1089,6 +1125,11 @@ Nd4jStatus execCustomOp2(Nd4jPointer* extraPointers, Nd4jLong hash, OpaqueContex
   const ops::OpDescriptor* op = ops::findOp(hash);
   if (!op) ND4J_THROW("execCustomOp2: unknown op hash " + std::to_string(hash) + " (op is not implemented in nd4j-hip)");
   ops::executeOp(*op, *ctx);
+  if (captureActive()) {
+    RecordedOp rec;   // run stays empty: a custom op is replayed from this record's own copy of the context
+    rec.kind = RecordedOp::CUSTOM; rec.op = op; rec.ctx = *ctx;
+    recordOp(std::move(rec));
+  }
   if (Environment::get().syncAfterCustomOp) HIP_CHECK(hipStreamSynchronize(execStream()));
   return 0;
   GUARD_END(1)
@@ -1119,13 +1160,25 @@ namespace {
 struct CapturedGraph {
   hipGraph_t graph = nullptr;
   hipGraphExec_t exec = nullptr;
-  CaptureRecord record;   // the buffers the recorded kernels read and write
+  CaptureRecord record;           // the buffers the recorded kernels read and write
+  std::vector<RecordedOp> ops;    // the op calls the facade recognised, in call order
+  int opCalls = 0;                // every op entry point called during the capture
+  int fusedOps = 0;               // ops that ended up inside a neighbour's kernel
 };
 CapturedGraph* g_openCapture = nullptr;
 bool g_syncBeforeCapture = true;
+bool graphFusionEnabled() {
+  static const bool on = [] { const char* v = getenv("ND4JHIP_GRAPH_FUSION"); return v == nullptr || atoi(v) != 0; }();
+  return on;
 }
+}
+}  // extern "C"
+static void recordOp(RecordedOp&& r) {
+  if (g_openCapture) g_openCapture->ops.push_back(std::move(r));
+}
+extern "C" {
 int nd4jhipGraphBeginCapture(void) {
-  OP_BEGIN(nullptr)
+  GRAPH_BEGIN
   ND4J_REQUIRE(!captureActive(), "nd4jhipGraphBeginCapture: a capture is already in progress");
   // every op call between begin and end records its kernels instead of running them: nothing may wait on the stream
   g_syncBeforeCapture = Environment::get().syncAfterCustomOp;
@@ -1133,23 +1186,62 @@ int nd4jhipGraphBeginCapture(void) {
   HIP_CHECK(hipStreamSynchronize(execStream()));
   HIP_CHECK(hipStreamBeginCapture(execStream(), hipStreamCaptureModeRelaxed));
   g_openCapture = new CapturedGraph();
+  g_captureOpCalls = &g_openCapture->opCalls;
   setActiveCapture(&g_openCapture->record);
   return 0;
   GUARD_END(1)
 }
 Nd4jPointer nd4jhipGraphEndCapture(void) {
-  OP_BEGIN(nullptr)
+  GRAPH_BEGIN
   ND4J_REQUIRE(captureActive() && g_openCapture, "nd4jhipGraphEndCapture: no capture in progress");
   CapturedGraph* cg = g_openCapture;
-  g_openCapture = nullptr;
-  setActiveCapture(nullptr);
-  Environment::get().syncAfterCustomOp = g_syncBeforeCapture;
+  auto closeCapture = [&] {
+    g_openCapture = nullptr;
+    g_captureOpCalls = nullptr;
+    setActiveCapture(nullptr);
+    Environment::get().syncAfterCustomOp = g_syncBeforeCapture;
+  };
   hipError_t e = hipStreamEndCapture(execStream(), &cg->graph);
   if (e != hipSuccess || cg->graph == nullptr) {
+    closeCapture();
     delete cg;
     (void)hipGetLastError();
     ND4J_THROW(std::string("nd4jhipGraphEndCapture: the capture was invalidated (an op waited on the stream or copied synchronously): ") + hipGetErrorString(e));
   }
+  // Every call of the capture was one the facade keeps a record of: run the sequence again through the merging pass and
+  // keep that recording instead (nothing has executed so far -- a capture only notes launches)
+  if (graphFusionEnabled() && !cg->ops.empty() && (int)cg->ops.size() == cg->opCalls) {
+    int nFused = 0;
+    auto plan = fuseRecordedOps(cg->ops, nFused);
+    if (nFused > 0) {
+      g_captureOpCalls = nullptr;             // the replay re-enters nothing that counts
+      hipGraph_t merged = nullptr;
+      cg->record = CaptureRecord();
+      std::string failure;
+      e = hipStreamBeginCapture(execStream(), hipStreamCaptureModeRelaxed);
+      if (e == hipSuccess) {
+        std::vector<RecordedOp> keep;
+        keep.swap(cg->ops);                   // replayed ops must not be recorded a second time
+        try { for (auto& step : plan) step(); } catch (std::exception& ex) { failure = ex.what(); }
+        cg->ops.swap(keep);
+        e = hipStreamEndCapture(execStream(), &merged);
+      }
+      if (e == hipSuccess && merged != nullptr && failure.empty()) {
+        (void)hipGraphDestroy(cg->graph);
+        cg->graph = merged;
+        cg->fusedOps = nFused;
+      } else {
+        if (merged) (void)hipGraphDestroy(merged);
+        (void)hipGetLastError();
+        closeCapture();
+        (void)hipGraphDestroy(cg->graph);
+        delete cg;
+        ND4J_THROW("nd4jhipGraphEndCapture: replaying the recorded ops through the merging pass failed: " + (failure.empty() ? std::string(hipGetErrorString(e)) : failure));
+      }
+    }
+  }
+  closeCapture();
+  cg->ops.clear();
   e = hipGraphInstantiate(&cg->exec, cg->graph, nullptr, nullptr, 0);
   if (e != hipSuccess) {
     (void)hipGraphDestroy(cg->graph);
@@ -1160,7 +1252,7 @@ Nd4jPointer nd4jhipGraphEndCapture(void) {
   GUARD_END(nullptr)
 }
 int nd4jhipGraphLaunch(Nd4jPointer graph) {
-  OP_BEGIN(nullptr)
+  GRAPH_BEGIN
   ND4J_REQUIRE(graph != nullptr, "nd4jhipGraphLaunch: graph is null");
   ND4J_REQUIRE(!captureActive(), "nd4jhipGraphLaunch: a capture is in progress");
   CapturedGraph* cg = static_cast<CapturedGraph*>(graph);
@@ -1181,6 +1273,7 @@ int nd4jhipGraphLaunch(Nd4jPointer graph) {
   return 0;
   GUARD_END(1)
 }
+int nd4jhipGraphFusedOps(Nd4jPointer graph) { return graph ? static_cast<CapturedGraph*>(graph)->fusedOps : 0; }
 void nd4jhipGraphDestroy(Nd4jPointer graph) {
   if (!graph) return;
   CapturedGraph* cg = static_cast<CapturedGraph*>(graph);

@@ -476,9 +476,12 @@ __global__ __launch_bounds__(256) void layernorm_rows(RowArgs a, const T* __rest
 // One wave per row for rows at a constant pitch (the usual case: a dense or row-strided matrix), vector path only.
 // No shape walk and no predicated loads: every lane issues its x / gain / bias vectors at once (lanes past the row's
 // end re-read the last vector and are masked out of the sums), so the three latencies overlap instead of queueing.
-template <typename T, int NV, bool HAS_BIAS, int RPW>
+// ADD: the row normalised is x + addend, rounded through the storage type and also written to sumOut -- a pairwise Add
+// followed by layer_norm on its result, in one pass (sumOut may be x itself: a wave reads a row before it writes it).
+template <typename T, int NV, bool HAS_BIAS, int RPW, bool ADD = false>
 __global__ __launch_bounds__(256) void layernorm_linear(const T* __restrict__ x, const T* __restrict__ gain, const T* __restrict__ bias,
-                                                        T* __restrict__ z, LongType rows, int L, LongType xPitch, LongType zPitch, float eps) {
+                                                        T* __restrict__ z, LongType rows, int L, LongType xPitch, LongType zPitch, float eps,
+                                                        const T* addend = nullptr, LongType aPitch = 0, T* sumOut = nullptr, LongType sPitch = 0) {
   using A = typename Conv<T>::acc;
   using Raw = typename RawIO<T>::raw;
   constexpr int VEC = RawIO<T>::N;
@@ -488,7 +491,7 @@ __global__ __launch_bounds__(256) void layernorm_linear(const T* __restrict__ x,
   if (row0 >= rows) return;
   int e0[NV];
   A keep[NV];
-  Raw xv[RPW][NV], gv[NV], bv[NV];
+  Raw xv[RPW][NV], gv[NV], bv[NV], av[ADD ? RPW : 1][ADD ? NV : 1];
 #pragma unroll
   for (int i = 0; i < NV; i++) {
     const int e = (t + i * 64) * VEC;
@@ -499,7 +502,10 @@ __global__ __launch_bounds__(256) void layernorm_linear(const T* __restrict__ x,
   for (int r = 0; r < RPW; r++) {
     const LongType row = row0 + r < rows ? row0 + r : rows - 1;
 #pragma unroll
-    for (int i = 0; i < NV; i++) xv[r][i] = *reinterpret_cast<const Raw*>(x + row * xPitch + e0[i]);
+    for (int i = 0; i < NV; i++) {
+      xv[r][i] = *reinterpret_cast<const Raw*>(x + row * xPitch + e0[i]);
+      if (ADD) av[ADD ? r : 0][ADD ? i : 0] = *reinterpret_cast<const Raw*>(addend + row * aPitch + e0[i]);
+    }
   }
 #pragma unroll
   for (int i = 0; i < NV; i++) {
@@ -529,6 +535,15 @@ __global__ __launch_bounds__(256) void layernorm_linear(const T* __restrict__ x,
 #pragma unroll
     for (int i = 0; i < NV; i++) {
       RawIO<T>::unpack(xv[r][i], &vals[r][i * VEC]);
+      if (ADD) {
+        A add[VEC];
+        RawIO<T>::unpack(av[ADD ? r : 0][ADD ? i : 0], add);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) vals[r][i * VEC + e] += add[e];
+        const Raw packed = RawIO<T>::pack(&vals[r][i * VEC]);   // the sum as the separate Add would have stored it
+        if (keep[i] != (A)0 && row0 + r < rows) *reinterpret_cast<Raw*>(sumOut + (row0 + r) * sPitch + e0[i]) = packed;
+        RawIO<T>::unpack(packed, &vals[r][i * VEC]);
+      }
       A part = (A)0;
 #pragma unroll
       for (int e = 0; e < VEC; e++) part += vals[r][i * VEC + e];
@@ -613,6 +628,41 @@ static void layerNormTyped(hipStream_t s, const void* x, const void* gain, const
   if (L <= 64 * 16) { hipLaunchKernelGGL((layernorm_rows<T, 64, 16, 1>), dim3(gw), dim3(256), 0, s, a, xt, gt, bt, zt, eps); return; }
   if (L <= 256 * 32) { hipLaunchKernelGGL((layernorm_rows<T, 256, 32, 1>), dim3(gb), dim3(256), 0, s, a, xt, gt, bt, zt, eps); return; }
   ND4J_THROW("layer_norm: rows longer than 8192 elements take the generic path");
+}
+
+// x + addend -> sumOut, layer_norm(sumOut) -> z in one kernel; only the one-wave-per-row vector case (rows at a constant
+// pitch, 16-byte aligned), anything else returns false and the caller runs the two ops
+template <typename T>
+static bool addLayerNormTyped(hipStream_t s, const void* x, const void* addend, void* sumOut, const void* gain, const void* bias, void* z, LongType rows,
+                              LongType L, LongType xPitch, LongType aPitch, LongType sPitch, LongType zPitch, float eps) {
+  constexpr int V = 16 / sizeof(T);
+  auto al = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  if (L % V != 0 || L > 4 * 64 * V || L < V || !bias) return false;
+  if (!al(x) || !al(addend) || !al(sumOut) || !al(gain) || !al(bias) || !al(z)) return false;
+  if (xPitch % V || aPitch % V || sPitch % V || zPitch % V) return false;
+  const unsigned gw = (unsigned)((rows + 3) / 4);
+  const LongType perWave = 64 * V;
+#define ALN(NV) hipLaunchKernelGGL((layernorm_linear<T, NV, true, 1, true>), dim3(gw), dim3(256), 0, s, (const T*)x, (const T*)gain, (const T*)bias, (T*)z, rows, (int)L, \
+                                   xPitch, zPitch, eps, (const T*)addend, aPitch, (T*)sumOut, sPitch)
+  if (L <= perWave) ALN(1);
+  else if (L <= 2 * perWave) ALN(2);
+  else if (L <= 3 * perWave) ALN(3);
+  else ALN(4);
+#undef ALN
+  return true;
+}
+bool launchAddLayerNormRows(hipStream_t s, DataType dt, const void* x, const void* addend, void* sumOut, const void* gain, const void* bias, void* z,
+                            LongType rows, LongType L, LongType xPitch, LongType aPitch, LongType sPitch, LongType zPitch, float eps) {
+  if (rows == 0 || L == 0) return true;
+  bool ok = false;
+  switch (dt) {
+    case FLOAT32: ok = addLayerNormTyped<float>(s, x, addend, sumOut, gain, bias, z, rows, L, xPitch, aPitch, sPitch, zPitch, eps); break;
+    case HALF: ok = addLayerNormTyped<f16_t>(s, x, addend, sumOut, gain, bias, z, rows, L, xPitch, aPitch, sPitch, zPitch, eps); break;
+    case BFLOAT16: ok = addLayerNormTyped<bf16_t>(s, x, addend, sumOut, gain, bias, z, rows, L, xPitch, aPitch, sPitch, zPitch, eps); break;
+    default: ok = false;
+  }
+  if (ok) HIP_CHECK(hipGetLastError());
+  return ok;
 }
 
 void launchLayerNormRows(hipStream_t s, DataType dt, const void* x, const void* gain, const void* bias, void* z,

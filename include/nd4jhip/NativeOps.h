@@ -246,6 +246,13 @@ ND4JHIP_EXPORT int nd4jhipGraphBeginCapture(void);
 ND4JHIP_EXPORT Nd4jPointer nd4jhipGraphEndCapture(void);
 ND4JHIP_EXPORT int nd4jhipGraphLaunch(Nd4jPointer graph);
 ND4JHIP_EXPORT void nd4jhipGraphDestroy(Nd4jPointer graph);
+/* When every op call of a capture is one the library keeps a record of (execCustomOp2, execPairwiseTransform,
+ * execTransformStrict, execTransformAny), End replays the recorded calls through a merging pass before it builds the graph:
+ * a pairwise Add and the layer_norm of its result become one kernel, and so do xw_plus_b and the GELU transform / the
+ * column-slice assigns that follow it.  Every merged kernel writes what the separate ops would have written, bit for
+ * bit, into the same arrays.  This returns how many op calls were absorbed that way (0: the graph holds the calls as
+ * made).  ND4JHIP_GRAPH_FUSION=0 in the environment switches the pass off. */
+ND4JHIP_EXPORT int nd4jhipGraphFusedOps(Nd4jPointer graph);
 ND4JHIP_EXPORT const char* nd4jhipBuildInfo(void);
 /* Name ("family<type,tile,flags>") of the kernel the calling thread's most recent matmul / xw_plus_b launched; lets a
  * test assert that its shape reached the instantiation it means to check. */
