@@ -263,7 +263,8 @@ static XwGeometry xwGeometry(Context& c, bool needOutput) {
 }
 // epi: extra outputs for the product's epilogue (already prepared for device use by the caller); returns whether the kernel
 // that ran wrote them
-static bool xwPlusBImpl(Context& c, const GemmEpilogue* epi) {
+struct LnPrologue { NDArray *x, *gain, *bias, *out; };   // out = layer_norm(x; gain, bias) is the product's input
+static bool xwPlusBImpl(Context& c, const GemmEpilogue* epi, const LnPrologue* ln = nullptr) {
   ND4J_REQUIRE(c.width() >= 3, "xw_plus_b: x, weights and bias are required");
   NDArray* x = c.input(0); NDArray* w = c.input(1); NDArray* b = c.input(2); NDArray* z = c.output(0);
   if (x->isEmpty() || w->isEmpty() || b->isEmpty()) return epi == nullptr;
@@ -277,6 +278,17 @@ static bool xwPlusBImpl(Context& c, const GemmEpilogue* epi) {
   GemmDesc d;
   d.M = g.M; d.N = g.N; d.K = g.K;
   d.aRow = g.aRow; d.aCol = g.aCol; d.bRow = g.bRow; d.bCol = g.bCol; d.cRow = g.cRow; d.cCol = g.cCol;
+  if (ln) {
+    // the product reads the row before normalisation and writes the normalised row where the separate op would have
+    if (g.M != 1 || g.aCol != 1 || ln->x->lengthOf() != g.K || ln->x->dataType() != dt) return false;
+    prepareSpecialUse({z, ln->out}, {ln->x, ln->gain, ln->bias, w, b});
+    d.bias = b->specialBuffer();
+    d.epi = epi;
+    d.lnGain = ln->gain->specialBuffer(); d.lnBias = ln->bias->specialBuffer(); d.lnOut = ln->out->specialBuffer();
+    const bool done = launchGemm(stream(), dt, ln->x->specialBuffer(), w->specialBuffer(), z->specialBuffer(), d);
+    if (done) registerSpecialUse({z, ln->out}, {ln->x, ln->gain, ln->bias, w, b});
+    return done;
+  }
   prepareSpecialUse({z}, {x, w, b});
   d.bias = b->specialBuffer();
   d.epi = epi;
@@ -1872,69 +1884,103 @@ std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& rec,
       i += 2;
       continue;
     }
-    // xw_plus_b followed by ops on its result that the product's epilogue can write: the GELU transform of the whole
-    // result, and assigns of column slices of it (key / value rows going into their caches)
-    if (r.kind == RecordedOp::CUSTOM && r.op->name == "xw_plus_b" && r.ctx.outputs.size() >= 1 && r.ctx.outputs[0] && r.ctx.inputs.size() >= 3) {
-      NDArray* z = r.ctx.outputs[0];
-      LongType zr, zc, zs;
-      const DataType dt = z->dataType();
-      const bool zOk = (dt == HALF || dt == BFLOAT16) && asRows(z, zr, zc, zs) && iArg(r.ctx, 2, 0) != 1;
-      GemmEpilogue epi;
-      std::vector<RecordedOp*> absorbed;
-      size_t j = i + 1;
-      while (zOk && j < n) {
-        RecordedOp& f = rec[j];
-        bool inputsTouched = false;   // an absorbed op must not write what the product reads
-        for (NDArray* in : r.ctx.inputs) if (in && f.z && in->buf.get() == f.z->buf.get()) inputsTouched = true;
-        if (inputsTouched) break;
-        LongType fr, fc, fs;
-        if (f.kind == RecordedOp::TRANSFORM_STRICT && f.opNum == 53 && epi.act == 0 && sameView(f.x, z) && f.z->dataType() == dt && asRows(f.z, fr, fc, fs) &&
-            fr == zr && fc == zc && f.z->buf.get() != z->buf.get()) {
-          // which GELU form the separate transform would take: dense, aligned 16-bit arrays of a multiple of 8 elements run the
-          // one-instruction exponential on every element
-          const bool dense = zs == zc && fs == fc && (zr * zc) % 8 == 0;
-          if (!dense) break;
-          epi.act = 1; epi.actOut = f.z; epi.actRow = fs;   // handle now, device pointer when the step runs
-          absorbed.push_back(&f);
-          j++;
-          continue;
-        }
-        if (f.kind == RecordedOp::TRANSFORM_ANY && epi.nCopy < 2 && f.x->buf.get() == z->buf.get() && f.x->bufOffsetBytes == z->bufOffsetBytes && f.x->dataType() == dt &&
-            f.z->dataType() == dt && f.z->buf.get() != z->buf.get()) {
-          LongType sr, sc, ss, dr, dc, ds;
-          if (!asRows(f.x, sr, sc, ss) || !asRows(f.z, dr, dc, ds) || sr != zr || dr != zr || dc != sc) break;
-          if (zr > 1 && ss != zs) break;
-          const LongType c0 = f.x->offset - z->offset;
-          if (c0 < 0 || c0 + sc > zc) break;
-          epi.copy[epi.nCopy].dst = f.z; epi.copy[epi.nCopy].c0 = c0; epi.copy[epi.nCopy].c1 = c0 + sc; epi.copy[epi.nCopy].dstRow = ds;
-          epi.nCopy++;
-          absorbed.push_back(&f);
-          j++;
-          continue;
-        }
-        break;
+    // xw_plus_b, with the ops around it that its kernel can take in: in front a layer_norm whose output row is the
+    // product's input (one-row products normalise the row on the way in), behind it ops on the result that the epilogue can
+    // write -- the GELU transform of the whole result, assigns of column slices (key / value rows going into their
+    // caches), a pairwise Add of the result to another array (the residual connection)
+    {
+      RecordedOp* lnOp = nullptr;
+      size_t xi = i;
+      if (isRowLayerNorm(r) && i + 1 < n && rec[i + 1].kind == RecordedOp::CUSTOM && rec[i + 1].op->name == "xw_plus_b" && rec[i + 1].ctx.inputs.size() >= 3 &&
+          rec[i + 1].ctx.inputs[0] && sameView(rec[i + 1].ctx.inputs[0], r.ctx.outputs[0])) {
+        NDArray *lx = r.ctx.inputs[0], *lg = r.ctx.inputs[1], *lb = r.ctx.inputs[2], *lo = r.ctx.outputs[0];
+        LongType rr, cc, ss, r2, c2, s2;
+        const DataType dt = lx->dataType();
+        const bool ok = (dt == HALF || dt == BFLOAT16) && lg->dataType() == dt && lb->dataType() == dt && lo->dataType() == dt && asRows(lx, rr, cc, ss) && rr == 1 &&
+                        asRows(lo, r2, c2, s2) && r2 == 1 && c2 == cc && lg->lengthOf() == cc && lb->lengthOf() == cc && lo->buf.get() != lx->buf.get() &&
+                        iArg(rec[i + 1].ctx, 0, 0) != 1;
+        if (ok) { lnOp = &r; xi = i + 1; }
       }
-      if (!absorbed.empty()) {
-        RecordedOp* x = &r;
-        plan.push_back([x, epi, absorbed]() mutable {
-          // the extra outputs become device pointers now (their buffers are allocated by this point)
-          GemmEpilogue e = epi;
-          std::vector<NDArray*> writes;
-          x->ctx.outputs[0]->buf->allocateSpecial();
-          bool aligned = aligned16(x->ctx.outputs[0]->specialBuffer());
-          if (e.act) { NDArray* a = static_cast<NDArray*>(e.actOut); writes.push_back(a); }
-          for (int c = 0; c < e.nCopy; c++) writes.push_back(static_cast<NDArray*>(e.copy[c].dst));
-          prepareSpecialUse(writes, std::vector<NDArray*>{});
-          if (e.act) { e.actOut = static_cast<NDArray*>(epi.actOut)->specialBuffer(); aligned = aligned && aligned16(e.actOut); }
-          for (int c = 0; c < e.nCopy; c++) e.copy[c].dst = static_cast<NDArray*>(epi.copy[c].dst)->specialBuffer();
-          // (a misaligned GELU operand would send the separate transform down another evaluation path: keep the ops apart)
-          const bool applied = xwPlusBImpl(x->ctx, e.act && !aligned ? nullptr : &e) && !(e.act && !aligned);
-          if (applied) registerSpecialUse(writes, std::vector<NDArray*>{x->ctx.outputs[0]});
-          else for (RecordedOp* f : absorbed) runRecorded(f);
-        });
-        nFused += (int)absorbed.size();
-        i = j;
-        continue;
+      RecordedOp& xw = rec[xi];
+      if (xw.kind == RecordedOp::CUSTOM && xw.op->name == "xw_plus_b" && xw.ctx.outputs.size() >= 1 && xw.ctx.outputs[0] && xw.ctx.inputs.size() >= 3 &&
+          xw.ctx.inputs[0] && xw.ctx.inputs[1] && xw.ctx.inputs[2]) {
+        NDArray* z = xw.ctx.outputs[0];
+        LongType zr = 0, zc = 0, zs = 0;
+        const DataType dt = z->dataType();
+        const bool zOk = (dt == HALF || dt == BFLOAT16) && asRows(z, zr, zc, zs) && iArg(xw.ctx, 2, 0) != 1;
+        GemmEpilogue epi;          // array handles for now; device pointers when the step runs
+        std::vector<RecordedOp*> absorbed;
+        size_t j = xi + 1;
+        while (zOk && j < n) {
+          RecordedOp& f = rec[j];
+          if (f.kind == RecordedOp::CUSTOM || f.z == nullptr) break;
+          bool clash = f.z->buf.get() == z->buf.get();   // an absorbed op writes neither the product's operands nor its result
+          for (NDArray* in : xw.ctx.inputs) if (in && in->buf.get() == f.z->buf.get()) clash = true;
+          if (lnOp) for (NDArray* in : lnOp->ctx.inputs) if (in && in->buf.get() == f.z->buf.get()) clash = true;
+          if (clash || f.z->dataType() != dt) break;
+          LongType fr, fc, fs;
+          if (f.kind == RecordedOp::TRANSFORM_STRICT && f.opNum == 53 && epi.act == 0 && sameView(f.x, z) && asRows(f.z, fr, fc, fs) && fr == zr && fc == zc) {
+            // the form the separate transform takes on dense, aligned 16-bit arrays of a multiple of 8 elements
+            if (!(zs == zc && fs == fc && (zr * zc) % 8 == 0)) break;
+            epi.act = 1; epi.actOut = f.z; epi.actRow = fs;
+          } else if (f.kind == RecordedOp::TRANSFORM_ANY && epi.nCopy < 2 && f.x->buf.get() == z->buf.get() && f.x->bufOffsetBytes == z->bufOffsetBytes &&
+                     f.x->dataType() == dt) {
+            LongType sr, sc, ss, dr, dc, ds;
+            if (!asRows(f.x, sr, sc, ss) || !asRows(f.z, dr, dc, ds) || sr != zr || dr != zr || dc != sc || (zr > 1 && ss != zs)) break;
+            const LongType c0 = f.x->offset - z->offset;
+            if (c0 < 0 || c0 + sc > zc) break;
+            epi.copy[epi.nCopy].dst = f.z; epi.copy[epi.nCopy].c0 = c0; epi.copy[epi.nCopy].c1 = c0 + sc; epi.copy[epi.nCopy].dstRow = ds;
+            epi.nCopy++;
+          } else if (f.kind == RecordedOp::PAIRWISE && f.opNum == 0 && epi.resOut == nullptr && zr == 1 && (sameView(f.y, z) || sameView(f.x, z)) &&
+                     f.x->dataType() == dt && f.y->dataType() == dt) {
+            // (one-row products only: with more rows the Add merges with the layer_norm behind it instead, which measured faster
+            // than per-element residual traffic in the tile kernels' epilogues)
+            NDArray* other = sameView(f.y, z) ? f.x : f.y;   // the addition commutes bit for bit
+            LongType orr, oc, os;
+            if (other->buf.get() == z->buf.get() || !asRows(other, orr, oc, os) || !asRows(f.z, fr, fc, fs) || orr != zr || oc != zc || fr != zr || fc != zc) break;
+            if (other->buf.get() == f.z->buf.get() && !sameView(other, f.z)) break;
+            epi.resIn = other; epi.resInRow = os; epi.resOut = f.z; epi.resOutRow = fs;
+          } else {
+            break;
+          }
+          absorbed.push_back(&f);
+          j++;
+          // nothing may follow an absorbed Add inside this kernel: later ops read its result
+          if (f.kind == RecordedOp::PAIRWISE) break;
+        }
+        if (lnOp || !absorbed.empty()) {
+          RecordedOp* x = &xw;
+          plan.push_back([x, lnOp, epi, absorbed] {
+            GemmEpilogue e = epi;
+            NDArray* z = x->ctx.outputs[0];
+            std::vector<NDArray*> writes, reads;
+            NDArray* actArr = static_cast<NDArray*>(epi.actOut);
+            if (e.act) writes.push_back(actArr);
+            for (int c = 0; c < e.nCopy; c++) writes.push_back(static_cast<NDArray*>(epi.copy[c].dst));
+            if (e.resOut) { writes.push_back(static_cast<NDArray*>(epi.resOut)); reads.push_back(static_cast<NDArray*>(const_cast<void*>(epi.resIn))); }
+            z->buf->allocateSpecial();
+            prepareSpecialUse(writes, reads);
+            if (e.act) e.actOut = actArr->specialBuffer();
+            for (int c = 0; c < e.nCopy; c++) e.copy[c].dst = static_cast<NDArray*>(epi.copy[c].dst)->specialBuffer();
+            if (e.resOut) { e.resOut = static_cast<NDArray*>(epi.resOut)->specialBuffer(); e.resIn = static_cast<NDArray*>(const_cast<void*>(epi.resIn))->specialBuffer(); }
+            // a misaligned GELU operand would send the separate transform down another evaluation path: keep the ops apart then
+            const bool epiOk = !absorbed.empty() && !(e.act && (!aligned16(z->specialBuffer()) || !aligned16(e.actOut)));
+            const GemmEpilogue* ep = epiOk ? &e : nullptr;
+            bool applied = false, done = false;
+            if (lnOp) {
+              LnPrologue ln{lnOp->ctx.inputs[0], lnOp->ctx.inputs[1], lnOp->ctx.inputs[2], lnOp->ctx.outputs[0]};
+              done = xwPlusBImpl(x->ctx, ep, &ln);
+              applied = done && epiOk;
+              if (!done) runRecorded(lnOp);
+            }
+            if (!done) applied = xwPlusBImpl(x->ctx, ep) && epiOk;
+            if (applied) registerSpecialUse(writes, reads);
+            else for (RecordedOp* f : absorbed) runRecorded(f);
+          });
+          nFused += (int)absorbed.size() + (lnOp ? 1 : 0);
+          i = j;
+          continue;
+        }
       }
     }
     RecordedOp* p = &r;

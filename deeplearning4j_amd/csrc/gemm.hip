@@ -25,6 +25,7 @@
 
 #include "kernels.h"
 #include "mfma_tile.h"
+#include "rowmath.h"
 #include "runtime.h"
 
 namespace nd4jhip {
@@ -1266,9 +1267,14 @@ __global__ __launch_bounds__(256) void gemv_rowdot(const T* __restrict__ W, Long
 // The same product for rows that fit a wave's registers (K <= NL * 64 * V): a wave owns OPW outputs and issues every
 // load of W and x before the first use, so one trip to memory covers the whole row; a decode step's projections
 // against k-contiguous weights run at the cost of a streaming read.
-template <typename T, int OPW, int NL, bool HAS_BIAS>
+// PRO_LN: the row multiplied is layer_norm(x; lnGain, lnBias) over its K elements -- every wave normalises the row it has
+// loaded anyway (the routine the row kernel runs, so the same bits), and the first wave of the grid also stores it to lnOut,
+// where the separate layer_norm op would have put it.
+template <typename T, int OPW, int NL, bool HAS_BIAS, bool PRO_LN = false>
 __global__ __launch_bounds__(256) void gemv_rowdot_pre(const T* __restrict__ W, LongType ldw, const T* __restrict__ x, T* __restrict__ y, LongType ys,
-                                                       LongType N, LongType K, const T* __restrict__ bias, int hasEpi, GemmEpilogue epi) {
+                                                       LongType N, LongType K, const T* __restrict__ bias, int hasEpi, GemmEpilogue epi,
+                                                       const T* __restrict__ lnGain = nullptr, const T* __restrict__ lnBias = nullptr,
+                                                       T* __restrict__ lnOut = nullptr, float lnEps = 0.f) {
   constexpr int V = 16 / sizeof(T);
   using Raw = typename RawIO<T>::raw;
   const int lane = threadIdx.x & 63;
@@ -1292,6 +1298,26 @@ __global__ __launch_bounds__(256) void gemv_rowdot_pre(const T* __restrict__ W, 
   if (HAS_BIAS) {
 #pragma unroll
     for (int o = 0; o < OPW; o++) bq[o] = bias[n0 + o < N ? n0 + o : N - 1];
+  }
+  if (PRO_LN) {
+    Raw gv[NL], bv[NL];
+    float keepf[NL], vals[NL * V];
+#pragma unroll
+    for (int i = 0; i < NL; i++) {
+      const int kk = lane + 64 * i, kc = kk < kw ? kk : kw - 1;
+      gv[i] = reinterpret_cast<const Raw*>(lnGain)[kc];
+      bv[i] = reinterpret_cast<const Raw*>(lnBias)[kc];
+      keepf[i] = kk < kw ? 1.f : 0.f;
+      RawIO<T>::unpack(__builtin_bit_cast(Raw, xr[i]), &vals[i * V]);
+    }
+    ln_wave_row<T, NL, true>(vals, gv, bv, keepf, (int)K, lnEps);
+    const bool first = blockIdx.x == 0 && (threadIdx.x >> 6) == 0;
+#pragma unroll
+    for (int i = 0; i < NL; i++) {
+      const Raw packed = RawIO<T>::pack(&vals[i * V]);
+      xr[i] = __builtin_bit_cast(raw_u32x4, packed);
+      if (first && lane + 64 * i < kw) reinterpret_cast<Raw*>(lnOut)[lane + 64 * i] = packed;
+    }
   }
   // the bias enters lane 0's partial sum ahead of the wave reduction: a use every lane depends on, so its load stays
   // up here with the others instead of sinking into the one-lane store at the end
@@ -1330,7 +1356,16 @@ static bool tryGemvRowdotPre(hipStream_t s, const GemmDesc& d, const void* A, co
   const LongType passes = (d.K / V + 63) / 64;
 #define ROWDOT_B(OPW, NL, HB) hipLaunchKernelGGL((gemv_rowdot_pre<T, OPW, NL, HB>), dim3((unsigned)(((d.N + OPW - 1) / OPW + 3) / 4)), dim3(256), 0, s, \
                                                  (const T*)B, d.bCol, (const T*)A, (T*)C, d.cCol, d.N, d.K, (const T*)d.bias, d.epi ? 1 : 0, d.epi ? *d.epi : GemmEpilogue())
+#define ROWDOT_LN(OPW, NL) hipLaunchKernelGGL((gemv_rowdot_pre<T, OPW, NL, true, true>), dim3((unsigned)(((d.N + OPW - 1) / OPW + 3) / 4)), dim3(256), 0, s, \
+                                              (const T*)B, d.bCol, (const T*)A, (T*)C, d.cCol, d.N, d.K, (const T*)d.bias, d.epi ? 1 : 0, d.epi ? *d.epi : GemmEpilogue(), \
+                                              (const T*)d.lnGain, (const T*)d.lnBias, (T*)d.lnOut, d.lnEps)
 #define ROWDOT(OPW, NL) do { noteKernel("gemv_rowdot_pre<%s,opw=%d,nl=%d>", tname<T>(), OPW, NL); if (d.bias) ROWDOT_B(OPW, NL, true); else ROWDOT_B(OPW, NL, false); } while (0)
+  if (d.lnGain) {   // the row is normalised on the way in: short rows with a bias only
+    if (!d.bias || passes > 4 || ((reinterpret_cast<uintptr_t>(d.lnGain) | reinterpret_cast<uintptr_t>(d.lnBias) | reinterpret_cast<uintptr_t>(d.lnOut)) & 15)) return false;
+    noteKernel("gemv_rowdot_pre<%s,ln,nl=%d>", tname<T>(), passes <= 2 ? 2 : 4);
+    if (passes <= 2) ROWDOT_LN(2, 2); else ROWDOT_LN(2, 4);
+    return true;
+  }
   if (passes <= 2) ROWDOT(2, 2);
   else if (passes <= 4) ROWDOT(2, 4);
   else if (passes <= 6) ROWDOT(2, 6);
@@ -1339,6 +1374,7 @@ static bool tryGemvRowdotPre(hipStream_t s, const GemmDesc& d, const void* A, co
   else return false;
 #undef ROWDOT
 #undef ROWDOT_B
+#undef ROWDOT_LN
   return true;
 }
 // y[n] = alpha * sum_k x[k] * W[k][n]: W rows contiguous in n.  A thread owns V consecutive outputs of one k-slice;
@@ -1657,6 +1693,10 @@ static bool tryGemmSkinny(hipStream_t s, const GemmDesc& d, const void* A, const
 
 template <typename T>
 static bool dispatch16(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
+  if (d.lnGain) {   // only the one-row product against k-contiguous weights normalises its row on the way in
+    if (d.M == 1 && d.N > 1 && d.batch == 1 && d.bRow == 1 && d.cCol == 1) return tryGemvRowdotPre<T>(s, d, A, B, C);
+    return false;
+  }
   bool aKC = false, bKC = false;
   const bool eligible = (d.M * d.N >= 1024 || (d.M == 1 && d.N >= 64)) && d.K >= 32 && mfmaEligible(d, A, B, sizeof(T), aKC, bKC);
   // x[1, K] times row-major W[K, N]: the split-K tile kernel streams W with far more loads in flight than the
@@ -1692,7 +1732,7 @@ static void dispatch32(hipStream_t s, const GemmDesc& d, const void* A, const vo
 bool launchGemm(hipStream_t s, DataType dt, const void* A, const void* B, void* C, const GemmDesc& d) {
   if (d.M == 0 || d.N == 0 || d.batch == 0) return true;
   ND4J_REQUIRE(d.batch < 65536 && (d.M + 31) / 32 < 65536 && (d.N + 31) / 32 < (1LL << 31), "matmul: problem too large for the launch grid");
-  bool withEpilogue = d.epi != nullptr;
+  bool withEpilogue = d.epi != nullptr || d.lnGain != nullptr;
   if (withEpilogue) {
     // only the 16-bit decode-step kernels carry epilogue outputs; when the dispatch lands elsewhere nothing has been
     // launched yet and the product runs again without the request
@@ -1700,6 +1740,7 @@ bool launchGemm(hipStream_t s, DataType dt, const void* A, const void* B, void* 
     if (dt == HALF) done = dispatch16<f16_t>(s, d, A, B, C);
     else if (dt == BFLOAT16) done = dispatch16<bf16_t>(s, d, A, B, C);
     if (done) { HIP_CHECK(hipGetLastError()); return true; }
+    if (d.lnGain) return false;   // nothing launched: the caller normalises the row with the separate op and calls again
     GemmDesc plain = d;
     plain.epi = nullptr;
     launchGemm(s, dt, A, B, C, plain);

@@ -13,6 +13,7 @@
 //   standardize.cpp:34-78) * gain + bias): one fused pass instead of the reference's eight:
 //   mean, population variance, y = (x - mean) / sqrt(var + 1e-5) * gain + bias.
 #include "device.h"
+#include "rowmath.h"
 #include "kernels.h"
 #include "runtime.h"
 
@@ -528,6 +529,28 @@ __global__ __launch_bounds__(256) void layernorm_linear(const T* __restrict__ x,
                                     "+v"(gv[NV > 2 ? 2 : 0]), "+v"(gv[NV > 3 ? 3 : 0]), "+v"(bv[0]), "+v"(bv[NV > 1 ? 1 : 0]), "+v"(bv[NV > 2 ? 2 : 0]), "+v"(bv[NV > 3 ? 3 : 0]));
   }
   A vals[RPW][NV * VEC];
+  if (RPW == 1) {
+    // one row per wave: the shared row routine (also what a product that normalises its input row runs)
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      RawIO<T>::unpack(xv[0][i], &vals[0][i * VEC]);
+      if (ADD) {
+        A add[VEC];
+        RawIO<T>::unpack(av[0][ADD ? i : 0], add);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) vals[0][i * VEC + e] += add[e];
+        const Raw packed = RawIO<T>::pack(&vals[0][i * VEC]);   // the sum as the separate Add would have stored it
+        if (keep[i] != (A)0) *reinterpret_cast<Raw*>(sumOut + row0 * sPitch + e0[i]) = packed;
+        RawIO<T>::unpack(packed, &vals[0][i * VEC]);
+      }
+    }
+    ln_wave_row<T, NV, HAS_BIAS>(vals[0], gv, bv, keep, L, eps);
+    T* zr = z + row0 * zPitch;
+#pragma unroll
+    for (int i = 0; i < NV; i++)
+      if (keep[i] != (A)0) *reinterpret_cast<Raw*>(zr + e0[i]) = RawIO<T>::pack(&vals[0][i * VEC]);
+    return;
+  }
   A sum[RPW];
 #pragma unroll
   for (int r = 0; r < RPW; r++) {
@@ -535,15 +558,6 @@ __global__ __launch_bounds__(256) void layernorm_linear(const T* __restrict__ x,
 #pragma unroll
     for (int i = 0; i < NV; i++) {
       RawIO<T>::unpack(xv[r][i], &vals[r][i * VEC]);
-      if (ADD) {
-        A add[VEC];
-        RawIO<T>::unpack(av[ADD ? r : 0][ADD ? i : 0], add);
-#pragma unroll
-        for (int e = 0; e < VEC; e++) vals[r][i * VEC + e] += add[e];
-        const Raw packed = RawIO<T>::pack(&vals[r][i * VEC]);   // the sum as the separate Add would have stored it
-        if (keep[i] != (A)0 && row0 + r < rows) *reinterpret_cast<Raw*>(sumOut + (row0 + r) * sPitch + e0[i]) = packed;
-        RawIO<T>::unpack(packed, &vals[r][i * VEC]);
-      }
       A part = (A)0;
 #pragma unroll
       for (int e = 0; e < VEC; e++) part += vals[r][i * VEC + e];

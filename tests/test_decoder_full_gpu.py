@@ -100,10 +100,11 @@ def test_gpt2_small_graph_replay_matches_eager(ex, gpt2, batch):
     dec.use_graphs = True
     assert np.array_equal(dec.generate(prompt, 6), want)                     # records
     assert np.array_equal(dec.logits(1), want_logits)
-    # the recorded steps went through the merging pass: per layer two Add + layer_norm pairs, the GELU after the first
-    # feed-forward product and the two cache writes after the qkv product ride in a neighbour's kernel
+    # the recorded steps went through the merging pass: per layer the two residual Adds, the GELU after the first feed-forward
+    # product and the two cache writes after the qkv product ride in a product's epilogue, and at batch 1 the two layer
+    # norms are computed by the products that consume them
     fused = [ex.L.nd4jhipGraphFusedOps(g) for g in dec._graphs.values()]
-    assert fused and min(fused) == 5 * cfg.n_layer, fused
+    assert fused and min(fused) == (7 if batch == 1 else 5) * cfg.n_layer, fused
     stale = dec.logits(1)                                                   # host copy read: a later replay must refresh it
     prompt2 = rng.integers(0, cfg.vocab, (batch, 24))
     want2 = eager.generate(prompt2, 6)
