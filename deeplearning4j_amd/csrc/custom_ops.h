@@ -49,6 +49,6 @@ std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& ops,
 void runIndexReduce(const char* fn, int opNum, NDArray* x, NDArray* z, const std::vector<LongType>& dims);
 // value reductions and summary statistics behind both the legacy entry points and the reduce_* custom ops
 void runReduce(const char* fn, ReduceKind k, NDArray* x, NDArray* z, const std::vector<LongType>& dims);
-void runReduceMisc(const char* fn, MiscReduceKind k, NDArray* x, NDArray* z, std::vector<LongType> dims, bool biasCorrected);
+void runReduceMisc(const char* fn, MiscReduceKind k, NDArray* x, NDArray* z, std::vector<LongType> dims, bool biasCorrected, double param = 0.0);
 
 }  // namespace nd4jhip

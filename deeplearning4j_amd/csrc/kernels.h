@@ -83,6 +83,17 @@ bool isIntLike(DataType t);
 void launchIntElementwise(hipStream_t s, int k, bool binary, DataType xdt, DataType ydt, DataType zdt, const void* x, const void* y,
                           void* z, const EwPlan& p, LongType scalar, bool hasScalar);
 
+// Ops that test a "match condition" read from the extra parameters (condops.hip)
+enum CondKind : int { C_MATCH_BOOL, C_SET_TRANSFORM, C_SET, C_REPLACE };
+enum CondReduceKind : int { CR_COUNT, CR_FIRST, CR_LAST };
+struct CondParams {
+  int mode = 0;
+  double compare = 0, set = 0, eps = 0;   // as the array's type holds them
+  int xdt = FLOAT32;                      // the type the comparisons run in
+};
+void launchCondElementwise(hipStream_t s, CondKind kind, const CondParams& c, DataType ydt, DataType zdt, const void* x, const void* y,
+                           void* z, const EwPlan& p, double scalar, bool hasScalar);
+
 // ---- reductions ----------------------------------------------------------------------------------
 enum ReduceKind : int {
   R_SUM, R_MAX, R_MIN, R_PROD, R_ASUM, R_AMAX, R_AMIN,        // ReduceSame 0..6
@@ -96,7 +107,9 @@ enum IndexKind : int { I_MAX, I_MIN, I_AMAX, I_AMIN, I_COUNT };
 enum MiscReduceKind : int {
   M_VARIANCE, M_STDDEV, M_COUNT_NONZERO, M_COUNT_ZERO, M_ANY, M_ALL,
   // two-operand reductions (reduce3), z in a float type
-  M3_MANHATTAN, M3_EUCLIDEAN, M3_COSINE_SIMILARITY, M3_DOT, M3_COSINE_DISTANCE, M3_JACCARD, M3_HAMMING
+  M3_MANHATTAN, M3_EUCLIDEAN, M3_COSINE_SIMILARITY, M3_DOT, M3_COSINE_DISTANCE, M3_JACCARD, M3_HAMMING,
+  M3_EQUALS_EPS,   // 1 when |x - y| <= param everywhere, else 0 (Reduce3 EqualsWithEps)
+  M_NORMP          // (sum |x|^param)^(1 / param), z in a float type (ReduceFloat NormP); not a two-operand kind
 };
 
 // outer = kept dims (one output element each), inner = reduced dims
@@ -121,7 +134,11 @@ void launchReduceScalarNoAlloc(hipStream_t s, ReduceKind k, DataType dt, const v
 // zdt: the float type for variance / standard deviation, INT64 for counts, BOOL for Any / All
 void launchReduceMisc(hipStream_t s, MiscReduceKind k, DataType xdt, DataType zdt, const void* x, void* z, const ReducePlan& p,
                       bool biasCorrected, void* scratch, size_t scratchBytes, const void* y = nullptr, DataType ydt = FLOAT32,
-                      const ReducePlan* yPlan = nullptr);
+                      const ReducePlan* yPlan = nullptr, double param = 0.0);
+// count of elements that meet the condition / position of the first or last one (-1: none); z INT32 or INT64
+struct ReducePlan;
+void launchCondReduce(hipStream_t s, CondReduceKind kind, const CondParams& c, DataType zdt, const void* x, void* z, const ReducePlan& p,
+                      void* scratch, size_t scratchBytes);
 void launchIndexReduce(hipStream_t s, IndexKind k, DataType xdt, DataType zdt, const void* x, void* z,
                        const ReducePlan& p, void* scratch, size_t scratchBytes);
 

@@ -487,6 +487,41 @@ static void runUnary(const char* fn, UnaryKind k, NDArray* x, NDArray* z) {
   registerSpecialUse({z}, {x});
 }
 
+// n extra parameters, held in data type dt (the executioner converts an op's extraArgs to the array's type before the call);
+// the pointer may be device or host memory, so they are fetched with a blocking copy
+static std::vector<double> fetchParams(const char* fn, const void* extraParams, DataType dt, int n) {
+  if (extraParams == nullptr) ND4J_THROW(std::string(fn) + ": this op reads " + std::to_string(n) + " extra parameters, got none");
+  unsigned char raw[64];
+  const size_t w = sizeOf(dt);
+  ND4J_REQUIRE(w > 0 && w * n <= sizeof(raw), std::string(fn) + ": unsupported type of the extra parameters");
+  ND4J_REQUIRE(!captureActive(), std::string(fn) + ": ops that read extra parameters cannot be recorded into a graph (the parameters are fetched with a blocking copy)");
+  HIP_CHECK(hipStreamSynchronize(execStream()));
+  HIP_CHECK(hipMemcpy(raw, extraParams, n * w, hipMemcpyDefault));
+  std::vector<double> out(n);
+  for (int i = 0; i < n; i++) {
+    const void* p = raw + i * w;
+    switch (dt) {
+      case INT32: out[i] = *(const int*)p; break;
+      case INT64: out[i] = (double)*(const LongType*)p; break;
+      case BOOL: out[i] = *(const unsigned char*)p; break;
+      default: out[i] = hostValueAsDouble(p, dt);
+    }
+  }
+  return out;
+}
+// [compare, eps, mode] (MatchCondition family) or [compare, set, eps, mode] (the CompareAndSet family)
+static CondParams condParams(const char* fn, const void* extraParams, DataType dt, bool withSet) {
+  auto v = fetchParams(fn, extraParams, dt, withSet ? 4 : 3);
+  CondParams c;
+  c.compare = v[0];
+  c.set = withSet ? v[1] : 0.0;
+  c.eps = v[withSet ? 2 : 1];
+  c.mode = (int)v[withSet ? 3 : 2];
+  c.xdt = (int)dt;
+  ND4J_REQUIRE(c.mode >= 0 && c.mode <= 15, std::string(fn) + ": undefined match condition " + std::to_string(c.mode));
+  return c;
+}
+
 // The transforms that read two extra parameters.  extraParams holds them in the array's own type (the executioner
 // converts its extraArgs to X before the call); it may be device or host memory, so they are fetched with a blocking copy.
 static void runUnaryWithParams(const char* fn, Scalar2Kind k, NDArray* x, NDArray* z, const void* extraParams) {
@@ -573,14 +608,23 @@ void execTransformSame(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, 
     runUnaryWithParams("execTransformSame", S2_CLIP_BY_VALUE, x, z, extraParams);
     return;
   }
+  if (opNum == 13) {   // CompareAndSetTransform (loops/legacy_ops.h:42)
+    ND4J_REQUIRE(isFloatType(x->dataType()) || x->dataType() == INT32, "execTransformSame: CompareAndSetTransform takes float or INT32 arrays here");
+    if (x->isEmpty() || z->isEmpty()) return;
+    const CondParams c = condParams("execTransformSame", extraParams, x->dataType(), true);
+    EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo()});
+    prepareSpecialUse({z}, {x});
+    launchCondElementwise(execStream(), C_SET_TRANSFORM, c, x->dataType(), z->dataType(), x->specialBuffer(), nullptr, z->specialBuffer(), p, 0.0, false);
+    registerSpecialUse({z}, {x});
+    return;
+  }
   UnaryKind k;
   switch (opNum) {  // loops/legacy_ops.h:40-44
     case 0: k = U_ABS; break; case 3: k = U_NEG; break; case 6: k = U_CUBE; break; case 7: k = U_ONE_MINUS; break;
     case 11: k = U_RECIPROCAL; break; case 12: k = U_SQUARE; break; case 15: case 21: k = U_IDENTITY; break;
     case 2: k = U_ONES; break; case 4: k = U_ROUND; break; case 5: k = U_TIMES_ONE_MINUS; break; case 17: k = U_CEIL; break;
     case 18: k = U_FLOOR; break;
-    // 13 CompareAndSetTransform reads extra parameters; 1 Sign is not restated (the reference macro
-    // yields +1 for every non-zero input and -1 for zero)
+    // 1 Sign is not restated (the reference macro yields +1 for every non-zero input and -1 for zero)
     default: ND4J_THROW("execTransformSame: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
   runUnary("execTransformSame", k, x, z);
@@ -609,15 +653,26 @@ static PairwiseKind pairwiseKind(int opNum) {
     case 22: return P_SAFE_DIVIDE; case 23: return P_MOD; case 27: return P_LOGICAL_OR; case 28: return P_LOGICAL_XOR;
     case 29: return P_LOGICAL_NOT; case 30: return P_LOGICAL_AND; case 34: return P_AMAX; case 35: return P_AMIN;
     case 36: return P_TRUNCATE_MOD; case 37: return P_REPLACE_NANS; case 38: return P_DIVIDE_NO_NAN;
-    // 10 Axpy, 12/13 CompareAnd*, 24-26 relative errors, 31 PowDerivative read extra parameters; 32/33 LogPoissonLoss and
-    // 39/40 IGamma* are not implemented
+    // 12/13 CompareAndSet / CompareAndReplace are served before this table is consulted; 10 Axpy, 24-26 relative errors and
+    // 31 PowDerivative read extra parameters and 32/33 LogPoissonLoss, 39/40 IGamma* are not implemented
     default: ND4J_THROW("execPairwiseTransform: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
 }
-void execPairwiseTransform(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueNDArray ya, OpaqueNDArray za, void*) {
+void execPairwiseTransform(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueNDArray ya, OpaqueNDArray za, void* extraParams) {
   OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execPairwiseTransform", "x"); NDArray* y = arr(ya, "execPairwiseTransform", "y");
   NDArray* z = arr(za, "execPairwiseTransform", "z");
+  if (opNum == 12 || opNum == 13) {   // CompareAndSet, CompareAndReplace (loops/legacy_ops.h:123): parameters in Z's type
+    // values travel through a double on the way to Z, which INT64 does not survive beyond 2^53
+    ND4J_REQUIRE((isFloatType(z->dataType()) || z->dataType() == INT32) && x->dataType() == z->dataType() && y->dataType() == z->dataType(), "execPairwiseTransform: CompareAndSet / CompareAndReplace take float or INT32 arrays of one type here");
+    if (z->isEmpty()) return;
+    const CondParams c = condParams("execPairwiseTransform", extraParams, z->dataType(), true);
+    EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo(), y->shapeInfo()});
+    prepareSpecialUse({z}, {x, y});
+    launchCondElementwise(execStream(), opNum == 12 ? C_SET : C_REPLACE, c, y->dataType(), z->dataType(), x->specialBuffer(), y->specialBuffer(), z->specialBuffer(), p, 0.0, false);
+    registerSpecialUse({z}, {x, y});
+    return;
+  }
   pairwiseImpl(opNum, x, y, z);
   if (captureActive()) {
     RecordedOp r;
@@ -678,10 +733,21 @@ static double hostScalar(NDArray* s) {
     default: ND4J_THROW("scalar operand has an unsupported data type");
   }
 }
-void execScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueNDArray za, OpaqueNDArray sa, void*) {
+void execScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueNDArray za, OpaqueNDArray sa, void* extraParams) {
   OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execScalar", "x"); NDArray* z = arr(za, "execScalar", "z"); NDArray* s = arr(sa, "execScalar", "scalar");
   ND4J_REQUIRE(x->dataType() == z->dataType() && (isFloatType(x->dataType()) || isIntLike(x->dataType())), "execScalar: nd4j-hip requires X and Z of one type");
+  if (opNum == 33) {   // CompareAndSet with the scalar as second operand: z = cond(scalar) ? scalar : x (ops.h:719-840)
+    ND4J_REQUIRE(isFloatType(x->dataType()) || x->dataType() == INT32, "execScalar: CompareAndSet takes float or INT32 arrays here");
+    if (z->isEmpty()) return;
+    const CondParams c = condParams("execScalar", extraParams, z->dataType(), true);
+    const double sc = hostScalar(s);
+    EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo()});
+    prepareSpecialUse({z}, {x});
+    launchCondElementwise(execStream(), C_SET, c, x->dataType(), z->dataType(), x->specialBuffer(), nullptr, z->specialBuffer(), p, sc, true);
+    registerSpecialUse({z}, {x});
+    return;
+  }
   PairwiseKind k;
   switch (opNum) {  // loops/legacy_ops.h:78-86
     case 0: k = P_ADD; break; case 1: k = P_SUB; break; case 2: k = P_MUL; break; case 3: k = P_DIV; break;
@@ -696,7 +762,7 @@ void execScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueN
     case 38: k = P_LOG_X; break; case 39: k = P_RELU; break; case 40: k = P_RELU6; break; case 41: k = P_STEP; break;
     case 42: k = P_LSTM_CLIP; break; case 43: k = P_TRUNCATE_MOD; break; case 45: k = P_REVERSE_POW; break;
     case 46: k = P_DIVIDE_NO_NAN; break; case 49: k = P_RELU_D; break;
-    // 32 PowDerivative, 33 CompareAndSet read extra parameters; 47/48 IGamma* are not implemented
+    // 33 CompareAndSet is served above; 32 PowDerivative reads an extra parameter and 47/48 IGamma* are not implemented
     default: ND4J_THROW("execScalar: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
   if (z->isEmpty()) return;
@@ -812,7 +878,7 @@ static ReduceKind reduceFloatKind(int opNum) {
     case 5: return R_NORM2;  // NormFrobenius = sqrt(sum |x|^2)
     case 7: return R_SQNORM;
     case 8: return R_ENTROPY; case 9: return R_LOG_ENTROPY; case 10: return R_SHANNON_ENTROPY;
-    // 6 NormP reads its exponent from the extra parameters
+    // 6 NormP is served before this table is consulted (its exponent comes from the extra parameters)
     default: ND4J_THROW("execReduceFloat: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
 }
@@ -828,15 +894,23 @@ void execReduceSame2(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, vo
   runReduce("execReduceSame2", reduceSameKind(opNum), xa, za, hostDims(da, xa->rankOf(), "execReduceSame2"));
   GUARD_END_VOID
 }
-void execReduceFloat(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
+// NormP (ReduceFloat 6): (sum |x|^p)^(1/p) with p = extraParams[0] in Z's type (ops.h:1280-1286)
+static void runNormP(const char* fn, NDArray* x, NDArray* z, const void* extraParams, std::vector<LongType> dims) {
+  ND4J_REQUIRE(isFloatType(x->dataType()) && isFloatType(z->dataType()), std::string(fn) + ": NormP takes floating point arrays here");
+  const double pw = fetchParams(fn, extraParams, z->dataType(), 1)[0];
+  runReduceMisc(fn, M_NORMP, x, z, dims, false, pw);
+}
+void execReduceFloat(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void* extraParams, OpaqueNDArray za) {
   OP_BEGIN(callerStream(extraPointers))
   if (xa == nullptr || za == nullptr) ND4J_THROW("execReduceFloat: null pointer in input parameters");
+  if (opNum == 6) { runNormP("execReduceFloat", xa, za, extraParams, {}); return; }
   runReduce("execReduceFloat", reduceFloatKind(opNum), xa, za, {});
   GUARD_END_VOID
 }
-void execReduceFloat2(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
+void execReduceFloat2(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void* extraParams, OpaqueNDArray za, OpaqueNDArray da) {
   OP_BEGIN(callerStream(extraPointers))
   if (xa == nullptr || za == nullptr || da == nullptr) ND4J_THROW("execReduceFloat2: null pointer in input parameters");
+  if (opNum == 6) { runNormP("execReduceFloat2", xa, za, extraParams, hostDims(da, xa->rankOf(), "execReduceFloat2")); return; }
   runReduce("execReduceFloat2", reduceFloatKind(opNum), xa, za, hostDims(da, xa->rankOf(), "execReduceFloat2"));
   GUARD_END_VOID
 }
@@ -844,7 +918,7 @@ void execReduceFloat2(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, v
 // reductions with their own accumulator / output types
 }  // extern "C"
 namespace nd4jhip {
-void runReduceMisc(const char* fn, MiscReduceKind k, NDArray* x, NDArray* z, std::vector<LongType> d, bool biasCorrected) {
+void runReduceMisc(const char* fn, MiscReduceKind k, NDArray* x, NDArray* z, std::vector<LongType> d, bool biasCorrected, double param) {
   ND4J_REQUIRE(!x->isEmpty(), std::string(fn) + ": reductions of empty arrays are not implemented in nd4j-hip");
   if (z->isEmpty()) return;
   if (z->lengthOf() == 1 && x->lengthOf() != 1) {
@@ -858,19 +932,22 @@ void runReduceMisc(const char* fn, MiscReduceKind k, NDArray* x, NDArray* z, std
   auto lc = LaunchContext::defaultContext();
   prepareSpecialUse({z}, {x});
   launchReduceMisc(lc->execStream, k, x->dataType(), z->dataType(), x->specialBuffer(), z->specialBuffer(), p, biasCorrected,
-                   lc->reductionBuffer, LaunchContext::REDUCTION_BYTES);
+                   lc->reductionBuffer, LaunchContext::REDUCTION_BYTES, nullptr, FLOAT32, nullptr, param);
   registerSpecialUse({z}, {x});
 }
 }  // namespace nd4jhip
 extern "C" {
 // reduce3: z[o] = f(x tad o, y tad o) with y shaped like x (loops/cpu/reduce3.hpp); opNums loops/legacy_ops.h:88-90
-static void runReduce3(const char* fn, int opNum, NDArray* x, NDArray* y, NDArray* z, std::vector<LongType> d) {
+static void runReduce3(const char* fn, int opNum, NDArray* x, NDArray* y, NDArray* z, std::vector<LongType> d, const void* extraParams = nullptr) {
   MiscReduceKind k;
+  double param = 0.0;
   switch (opNum) {
     case 0: k = M3_MANHATTAN; break; case 1: k = M3_EUCLIDEAN; break; case 2: k = M3_COSINE_SIMILARITY; break; case 3: k = M3_DOT; break;
     case 5: k = M3_COSINE_DISTANCE; break; case 6: k = M3_JACCARD; break; case 7: k = M3_HAMMING; break;
-    default: ND4J_THROW(std::string(fn) + ": opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");   // 4 EqualsWithEps reads extra parameters
+    case 4: k = M3_EQUALS_EPS; break;   // the tolerance is the third extra parameter, in Z's type (op_macros_special.h:449-457)
+    default: ND4J_THROW(std::string(fn) + ": opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
+  if (opNum == 4 && isFloatType(z->dataType())) param = fetchParams(fn, extraParams, z->dataType(), 3)[2];
   ND4J_REQUIRE(isFloatType(z->dataType()), std::string(fn) + ": Z must have a floating point type");
   ND4J_REQUIRE(x->rankOf() == y->rankOf() && x->lengthOf() == y->lengthOf(), std::string(fn) + ": x and y must have the same shape");
   for (int i = 0; i < x->rankOf(); i++) ND4J_REQUIRE(x->sizeAt(i) == y->sizeAt(i), std::string(fn) + ": x and y must have the same shape");
@@ -888,7 +965,7 @@ static void runReduce3(const char* fn, int opNum, NDArray* x, NDArray* y, NDArra
   auto lc = LaunchContext::defaultContext();
   prepareSpecialUse({z}, {x, y});
   launchReduceMisc(lc->execStream, k, x->dataType(), z->dataType(), x->specialBuffer(), z->specialBuffer(), p, false, lc->reductionBuffer,
-                   LaunchContext::REDUCTION_BYTES, y->specialBuffer(), y->dataType(), &py);
+                   LaunchContext::REDUCTION_BYTES, y->specialBuffer(), y->dataType(), &py, param);
   registerSpecialUse({z}, {x, y});
 }
 static MiscReduceKind summaryKind(int opNum) {
@@ -912,24 +989,49 @@ void execSummaryStatsTad(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa
   runReduceMisc("execSummaryStatsTad", summaryKind(opNum), x, z, hostDims(da, x->rankOf(), "execSummaryStatsTad"), biasCorrected);
   GUARD_END_VOID
 }
-static void reduceLong(const char* fn, int opNum, OpaqueNDArray xa, OpaqueNDArray za, OpaqueNDArray da) {
+}  // extern "C"
+// MatchCondition (count), FirstIndex / LastIndex: [compare, eps, mode] in X's type
+static void runCondReduce(const char* fn, CondReduceKind kind, NDArray* x, NDArray* z, std::vector<LongType> d, const void* extraParams) {
+  ND4J_REQUIRE(isFloatType(x->dataType()) || x->dataType() == INT32 || x->dataType() == INT64, std::string(fn) + ": match conditions take float, INT32 or INT64 arrays here");
+  ND4J_REQUIRE(!x->isEmpty(), std::string(fn) + ": reductions of empty arrays are not implemented in nd4j-hip");
+  if (z->isEmpty()) return;
+  const CondParams c = condParams(fn, extraParams, x->dataType(), false);
+  if (z->lengthOf() == 1 && x->lengthOf() != 1) {
+    bool keptAllUnit = true;
+    std::vector<bool> red(x->rankOf(), false);
+    for (auto v : d) red[v] = true;
+    for (int i = 0; i < x->rankOf(); i++) if (!red[i] && x->sizeAt(i) != 1) keptAllUnit = false;
+    if (!keptAllUnit) d.clear();
+  }
+  ReducePlan p = buildReducePlan(x->shapeInfo(), z->shapeInfo(), d, false);
+  auto lc = LaunchContext::defaultContext();
+  prepareSpecialUse({z}, {x});
+  launchCondReduce(lc->execStream, kind, c, z->dataType(), x->specialBuffer(), z->specialBuffer(), p, lc->reductionBuffer, LaunchContext::REDUCTION_BYTES);
+  registerSpecialUse({z}, {x});
+}
+extern "C" {
+static void reduceLong(const char* fn, int opNum, OpaqueNDArray xa, OpaqueNDArray za, OpaqueNDArray da, const void* extraParams) {
   NDArray* x = arr(xa, fn, "x"); NDArray* z = arr(za, fn, "z");
   ND4J_REQUIRE(z->dataType() == INT64, std::string("NativeOpExecutioner::execReduceLong wrong Z data type: Z must be INT64, got ") + dtypeName(z->dataType()));
+  if (opNum == 2) {   // MatchCondition (loops/legacy_ops.h:95)
+    runCondReduce(fn, CR_COUNT, x, z, da ? hostDims(da, x->rankOf(), fn) : std::vector<LongType>{}, extraParams);
+    return;
+  }
   MiscReduceKind k;
   switch (opNum) {  // loops/legacy_ops.h:95
     case 0: k = M_COUNT_NONZERO; break; case 1: k = M_COUNT_ZERO; break;
-    default: ND4J_THROW(std::string(fn) + ": opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");   // 2 MatchCondition reads extra parameters
+    default: ND4J_THROW(std::string(fn) + ": opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
   runReduceMisc(fn, k, x, z, da ? hostDims(da, x->rankOf(), fn) : std::vector<LongType>{}, false);
 }
-void execReduceLong(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
+void execReduceLong(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void* extraParams, OpaqueNDArray za, OpaqueNDArray da) {
   OP_BEGIN(callerStream(extraPointers))
-  reduceLong("execReduceLong", opNum, xa, za, da);
+  reduceLong("execReduceLong", opNum, xa, za, da, extraParams);
   GUARD_END_VOID
 }
-void execReduceLong2(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
+void execReduceLong2(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void* extraParams, OpaqueNDArray za, OpaqueNDArray da) {
   OP_BEGIN(callerStream(extraPointers))
-  reduceLong("execReduceLong2", opNum, xa, za, da);
+  reduceLong("execReduceLong2", opNum, xa, za, da, extraParams);
   GUARD_END_VOID
 }
 static void reduceBool(const char* fn, int opNum, OpaqueNDArray xa, OpaqueNDArray za, OpaqueNDArray da) {
@@ -952,32 +1054,42 @@ void execReduceBool2(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, vo
   reduceBool("execReduceBool2", opNum, xa, za, da);
   GUARD_END_VOID
 }
-void execReduce3(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray ya, OpaqueNDArray za) {
+void execReduce3(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void* extraParams, OpaqueNDArray ya, OpaqueNDArray za) {
   OP_BEGIN(callerStream(extraPointers))
-  runReduce3("execReduce3", opNum, arr(xa, "execReduce3", "x"), arr(ya, "execReduce3", "y"), arr(za, "execReduce3", "z"), {});
+  runReduce3("execReduce3", opNum, arr(xa, "execReduce3", "x"), arr(ya, "execReduce3", "y"), arr(za, "execReduce3", "z"), {}, extraParams);
   GUARD_END_VOID
 }
-void execReduce3Scalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray ya, OpaqueNDArray za) {
+void execReduce3Scalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void* extraParams, OpaqueNDArray ya, OpaqueNDArray za) {
   OP_BEGIN(callerStream(extraPointers))
-  runReduce3("execReduce3Scalar", opNum, arr(xa, "execReduce3Scalar", "x"), arr(ya, "execReduce3Scalar", "y"), arr(za, "execReduce3Scalar", "z"), {});
+  runReduce3("execReduce3Scalar", opNum, arr(xa, "execReduce3Scalar", "x"), arr(ya, "execReduce3Scalar", "y"), arr(za, "execReduce3Scalar", "z"), {}, extraParams);
   GUARD_END_VOID
 }
-void execReduce3Tad(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray ya, OpaqueNDArray za, OpaqueNDArray da) {
+void execReduce3Tad(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void* extraParams, OpaqueNDArray ya, OpaqueNDArray za, OpaqueNDArray da) {
   OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execReduce3Tad", "x");
-  runReduce3("execReduce3Tad", opNum, x, arr(ya, "execReduce3Tad", "y"), arr(za, "execReduce3Tad", "z"), hostDims(da, x->rankOf(), "execReduce3Tad"));
+  runReduce3("execReduce3Tad", opNum, x, arr(ya, "execReduce3Tad", "y"), arr(za, "execReduce3Tad", "z"), hostDims(da, x->rankOf(), "execReduce3Tad"), extraParams);
   GUARD_END_VOID
 }
-void execTransformBool(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
+void execTransformBool(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void* extraParams, OpaqueNDArray za) {
   OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execTransformBool", "x"); NDArray* z = arr(za, "execTransformBool", "z");
   ND4J_REQUIRE(z->dataType() == BOOL, std::string("NativeOpExecutioner::execTransformBool requires Z to have same boolean type, got ") + dtypeName(z->dataType()));
   ND4J_REQUIRE(isFloatType(x->dataType()) || isIntLike(x->dataType()), "execTransformBool: this input type is not implemented in nd4j-hip");
+  if (opNum == 5) {   // MatchConditionBool (loops/legacy_ops.h:50)
+    ND4J_REQUIRE(isFloatType(x->dataType()) || x->dataType() == INT32 || x->dataType() == INT64, "execTransformBool: MatchConditionBool takes float, INT32 or INT64 arrays here");
+    if (x->isEmpty() || z->isEmpty()) return;
+    const CondParams c = condParams("execTransformBool", extraParams, x->dataType(), false);
+    EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo()});
+    prepareSpecialUse({z}, {x});
+    launchCondElementwise(execStream(), C_MATCH_BOOL, c, x->dataType(), BOOL, x->specialBuffer(), nullptr, z->specialBuffer(), p, 0.0, false);
+    registerSpecialUse({z}, {x});
+    return;
+  }
   UnaryKind k;
   switch (opNum) {  // loops/legacy_ops.h:49-51
     case 1: k = U_IS_INF; break; case 2: k = U_IS_NAN; break; case 3: k = U_IS_FINITE; break; case 4: k = U_IS_INF_OR_NAN; break;
     case 6: k = U_IS_POSITIVE; break; case 7: k = U_NOT; break; case 8: k = U_IS_NEGATIVE; break;
-    default: ND4J_THROW("execTransformBool: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");   // 5 MatchConditionBool reads extra parameters
+    default: ND4J_THROW("execTransformBool: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
   runUnary("execTransformBool", k, x, z);
   GUARD_END_VOID
@@ -1017,15 +1129,25 @@ void runIndexReduce(const char* fn, int opNum, NDArray* x, NDArray* z, const std
 }
 }  // namespace nd4jhip
 extern "C" {
-void execIndexReduce(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za, OpaqueNDArray da) {
+void execIndexReduce(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void* extraParams, OpaqueNDArray za, OpaqueNDArray da) {
   OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execIndexReduce", "x"); NDArray* z = arr(za, "execIndexReduce", "z"); NDArray* d = arr(da, "execIndexReduce", "dimension");
+  if (opNum == 4 || opNum == 5) {   // FirstIndex, LastIndex (loops/legacy_ops.h:132): -1 where nothing matches
+    ND4J_REQUIRE(z->dataType() == INT64 || z->dataType() == INT32, "NativeOpExecutioner::execIndexReduce requires Z operand to have INT32/INT64 type");
+    runCondReduce("execIndexReduce", opNum == 4 ? CR_FIRST : CR_LAST, x, z, hostDims(d, x->rankOf(), "execIndexReduce"), extraParams);
+    return;
+  }
   runIndexReduce("execIndexReduce", opNum, x, z, hostDims(d, x->rankOf(), "execIndexReduce"));
   GUARD_END_VOID
 }
-void execIndexReduceScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void*, OpaqueNDArray za) {
+void execIndexReduceScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void* extraParams, OpaqueNDArray za) {
   OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execIndexReduceScalar", "x"); NDArray* z = arr(za, "execIndexReduceScalar", "z");
+  if (opNum == 4 || opNum == 5) {
+    ND4J_REQUIRE(z->dataType() == INT64 || z->dataType() == INT32, "NativeOpExecutioner::execIndexReduceScalar requires Z operand to have INT32/INT64 type");
+    runCondReduce("execIndexReduceScalar", opNum == 4 ? CR_FIRST : CR_LAST, x, z, {}, extraParams);
+    return;
+  }
   runIndexReduce("execIndexReduceScalar", opNum, x, z, {});
   GUARD_END_VOID
 }

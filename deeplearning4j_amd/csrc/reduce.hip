@@ -364,6 +364,7 @@ struct MiscArgs {
   DevShape yOuter, yInner;          // second operand of the reduce3 kinds (same shapes, own strides)
   LongType outerLen, innerLen, segLen;
   int splits, kind, bias, xdt, zdt, ydt;
+  double param;                     // NormP: the exponent; EqualsWithEps: the tolerance
 };
 __device__ __forceinline__ double block_sum(double v, double* lds) {
   const int t = threadIdx.x;
@@ -396,6 +397,8 @@ __device__ __forceinline__ double misc_result(const MiscArgs& a, double n, doubl
     case M3_COSINE_DISTANCE: return 1.0 - mean / (sqrt(m2) * sqrt(cnt));
     case M3_JACCARD: return 1.0 - m2 / cnt;
     case M3_HAMMING: return mean / n;
+    case M3_EQUALS_EPS: return mean > 0.0 ? 0.0 : 1.0;            // mean counts the pairs further apart than the tolerance
+    case M_NORMP: return pow(cnt, 1.0 / a.param);                 // ops.h:1280-1286
     default: return cnt;
   }
 }
@@ -412,7 +415,7 @@ __global__ __launch_bounds__(256) void misc_partial(MiscArgs a, const void* __re
   const LongType st = linear ? a.inner.stride[0] : 0;
   auto at = [&](LongType q) { return load_any(x, a.xdt, base + (linear ? q * st : walk<LongType>(a.inner, q))); };
   double n = (double)(j1 - j0), mean = 0.0, m2 = 0.0, cnt = 0.0;
-  if (a.kind >= M3_MANHATTAN) {
+  if (a.kind >= M3_MANHATTAN && a.kind != M_NORMP) {
     const LongType ybase = walk<LongType>(a.yOuter, row);
     const bool ylinear = a.yInner.rank == 1;
     const LongType yst = ylinear ? a.yInner.stride[0] : 0;
@@ -425,6 +428,7 @@ __global__ __launch_bounds__(256) void misc_partial(MiscArgs a, const void* __re
         case M3_DOT: s0 += u * v; break;
         case M3_COSINE_SIMILARITY: case M3_COSINE_DISTANCE: s0 += u * v; s1 += u * u; s2 += v * v; break;
         case M3_JACCARD: s1 += u < v ? u : v; s2 += u > v ? u : v; break;
+        case M3_EQUALS_EPS: s0 += fabs(u - v) <= a.param ? 0.0 : 1.0; break;   // templatemath.h:115
         default: s0 += u == v ? 0.0 : 1.0; break;   // Hamming
       }
     }
@@ -440,7 +444,8 @@ __global__ __launch_bounds__(256) void misc_partial(MiscArgs a, const void* __re
     double c = 0.0;
     for (LongType q = j0 + threadIdx.x; q < j1; q += 256) {
       const double v = at(q);
-      if (a.kind == M_COUNT_NONZERO) c += v == 0.0 ? 0.0 : 1.0;         // ops.h:1180-1188
+      if (a.kind == M_NORMP) c += pow(fabs(v), a.param);
+      else if (a.kind == M_COUNT_NONZERO) c += v == 0.0 ? 0.0 : 1.0;         // ops.h:1180-1188
       else if (a.kind == M_COUNT_ZERO || a.kind == M_ALL) c += v == 0.0 ? 1.0 : 0.0;   // ops.h:1190-1198,1208-1215
       else c += v;                                                     // Any
     }
@@ -461,7 +466,7 @@ __global__ __launch_bounds__(256) void misc_finish(MiscArgs a, const double* __r
   for (int s = 0; s < a.splits; s++) {
     const double* p = partials + (row * a.splits + s) * 4;
     const double nb = p[0];
-    if (a.kind >= M3_MANHATTAN) { n += nb; mean += p[1]; m2 += p[2]; cnt += p[3]; continue; }
+    if (a.kind >= M3_MANHATTAN && a.kind != M_NORMP) { n += nb; mean += p[1]; m2 += p[2]; cnt += p[3]; continue; }
     if (nb > 0.0) {
       const double delta = p[1] - mean, tot = n + nb;
       m2 += p[2] + delta * delta * n * nb / tot;
@@ -473,11 +478,12 @@ __global__ __launch_bounds__(256) void misc_finish(MiscArgs a, const double* __r
   store_any(z, a.zdt, walk<LongType>(a.zOuter, row), misc_result(a, n, mean, m2, cnt));
 }
 void launchReduceMisc(hipStream_t st, MiscReduceKind k, DataType xdt, DataType zdt, const void* x, void* z, const ReducePlan& p,
-                      bool biasCorrected, void* scratch, size_t scratchBytes, const void* y, DataType ydt, const ReducePlan* yPlan) {
+                      bool biasCorrected, void* scratch, size_t scratchBytes, const void* y, DataType ydt, const ReducePlan* yPlan, double param) {
   if (p.outerLen == 0) return;
   MiscArgs a;
+  a.param = param;
   a.outer = p.outer; a.inner = p.inner; a.zOuter = p.zOuter;
-  ND4J_REQUIRE((k >= M3_MANHATTAN) == (y != nullptr && yPlan != nullptr), "reduce: second operand mismatch");
+  ND4J_REQUIRE((k >= M3_MANHATTAN && k != M_NORMP) == (y != nullptr && yPlan != nullptr), "reduce: second operand mismatch");
   if (yPlan) {
     ND4J_REQUIRE(yPlan->outerLen == p.outerLen && yPlan->innerLen == p.innerLen, "reduce3: operands must have equal shapes");
     a.yOuter = yPlan->outer; a.yInner = yPlan->inner;

@@ -24,6 +24,7 @@ class Pairwise:
     ReverseDivide, Remainder, FMod, Atan2, TruncateDiv, FloorDiv, FloorMod, SquaredSubtract = 11, 14, 15, 16, 17, 18, 19, 20
     ReverseMod, SafeDivide, Mod, LogicalOr, LogicalXor, LogicalNot, LogicalAnd = 21, 22, 23, 27, 28, 29, 30
     AMaxPairwise, AMinPairwise, TruncateMod, ReplaceNans, DivideNoNan = 34, 35, 36, 37, 38
+    CompareAndSet, CompareAndReplace = 12, 13   # extraArgs [compare, set, eps, mode]
 
 
 class TransformStrict:
@@ -41,6 +42,7 @@ class TransformFloat:
 
 class TransformSame:
     Abs, Ones, Neg, Round, TimesOneMinus, Cube, OneMinus, Reciprocal, Square, Identity, Ceiling, Floor, Copy = 0, 2, 3, 4, 5, 6, 7, 11, 12, 15, 17, 18, 21
+    CompareAndSetTransform = 13   # extraArgs [compare, set, eps, mode]
 
 
 class ReduceSame:
@@ -49,14 +51,17 @@ class ReduceSame:
 
 class ReduceFloat:
     Mean, AMean, Norm1, Norm2, NormMax, NormFrobenius, SquaredNorm, Entropy, LogEntropy, ShannonEntropy = 0, 1, 2, 3, 4, 5, 7, 8, 9, 10
+    NormP = 6   # extraArgs [p]
 
 
 class IndexReduce:
     IndexMax, IndexMin, IndexAbsoluteMax, IndexAbsoluteMin = 0, 1, 2, 3
+    FirstIndex, LastIndex = 4, 5   # extraArgs [compare, eps, mode]
 
 
 class TransformBool:
     IsInf, IsNan, IsFinite, IsInfOrNan, IsPositive, Not, IsNegative = 1, 2, 3, 4, 6, 7, 8
+    MatchConditionBool = 5   # extraArgs [compare, eps, mode]
 
 
 class SummaryStats:
@@ -65,10 +70,12 @@ class SummaryStats:
 
 class Reduce3:
     ManhattanDistance, EuclideanDistance, CosineSimilarity, Dot, CosineDistance, JaccardDistance, SimpleHammingDistance = 0, 1, 2, 3, 5, 6, 7
+    EqualsWithEps = 4   # extraArgs [-, -, eps]
 
 
 class ReduceLong:
     CountNonZero, CountZero = 0, 1
+    MatchCondition = 2   # extraArgs [compare, eps, mode]
 
 
 class ReduceBool:
@@ -81,6 +88,7 @@ class Scalar:
     SafeDivide, AMaxPairwise, AMinPairwise, Atan2, LogicalOr, LogicalXor, LogicalNot, LogicalAnd, Pow = 23, 24, 25, 26, 27, 28, 29, 30, 31
     SXELogitsSmoother, LeakyRELU, LeakyRELUDerivative, ReplaceNans, LogX, RELU, RELU6, Step, LstmClip = 34, 35, 36, 37, 38, 39, 40, 41, 42
     TruncateMod, SquaredReverseSubtract, ReversePow, DivideNoNan, RELUDerivative = 43, 44, 45, 46, 49
+    CompareAndSet = 33   # extraArgs [compare, set, eps, mode]
 
 
 class Broadcast:
@@ -208,16 +216,18 @@ class Executioner:
         N.check("execTransformAny")
         return z
 
-    def exec_pairwise(self, op_num, x, y, z=None):
+    def exec_pairwise(self, op_num, x, y, z=None, extra_args=None):
         z = z if z is not None else NDArray.empty(x.shape, x.dtype)
-        self.L.execPairwiseTransform(None, op_num, x.handle, y.handle, z.handle, None)
+        holder, extra = self._extra_params(extra_args, z.dtype)
+        self.L.execPairwiseTransform(None, op_num, x.handle, y.handle, z.handle, extra)
         N.check("execPairwiseTransform")
         return z
 
-    def exec_scalar(self, op_num, x, scalar, z=None):
+    def exec_scalar(self, op_num, x, scalar, z=None, extra_args=None):
         z = z if z is not None else NDArray.empty(x.shape, x.dtype)
         s = scalar if isinstance(scalar, NDArray) else NDArray.scalar(scalar, x.dtype)
-        self.L.execScalar(None, op_num, x.handle, z.handle, s.handle, None)
+        holder, extra = self._extra_params(extra_args, z.dtype)
+        self.L.execScalar(None, op_num, x.handle, z.handle, s.handle, extra)
         N.check("execScalar")
         return z
 
@@ -228,30 +238,34 @@ class Executioner:
         N.check("execBroadcast")
         return z
 
-    def _reduce(self, scalar_fn, dim_fn, name, op_num, x, dims, keep_dims, z, zdtype):
+    def _reduce(self, scalar_fn, dim_fn, name, op_num, x, dims, keep_dims, z, zdtype, extra_args=None, extra_dtype=None):
         if z is None:
             z = NDArray.empty(_reduced_shape(x.shape, dims, keep_dims), zdtype)
+        holder, extra = self._extra_params(extra_args, extra_dtype if extra_dtype is not None else x.dtype)
         if dims is None or len(dims) == 0:
-            scalar_fn(None, op_num, x.handle, None, z.handle)
+            scalar_fn(None, op_num, x.handle, extra, z.handle)
         else:
             d = _dims_array(dims)
-            dim_fn(None, op_num, x.handle, None, z.handle, d.handle)
+            dim_fn(None, op_num, x.handle, extra, z.handle, d.handle)
         N.check(name)
         return z
 
     def exec_reduce_same(self, op_num, x, dims=None, keep_dims=False, z=None):
         return self._reduce(self.L.execReduceSame, self.L.execReduceSame2, "execReduceSame", op_num, x, dims, keep_dims, z, x.dtype)
 
-    def exec_reduce_float(self, op_num, x, dims=None, keep_dims=False, z=None):
-        return self._reduce(self.L.execReduceFloat, self.L.execReduceFloat2, "execReduceFloat", op_num, x, dims, keep_dims, z, x.dtype)
+    def exec_reduce_float(self, op_num, x, dims=None, keep_dims=False, z=None, extra_args=None):
+        """extra_args reach the native side in Z's type (NormP's exponent)."""
+        zdt = z.dtype if z is not None else x.dtype
+        return self._reduce(self.L.execReduceFloat, self.L.execReduceFloat2, "execReduceFloat", op_num, x, dims, keep_dims, z, x.dtype, extra_args, zdt)
 
-    def exec_index_reduce(self, op_num, x, dims=None, keep_dims=False, z=None):
-        return self._reduce(self.L.execIndexReduceScalar, self.L.execIndexReduce, "execIndexReduce", op_num, x, dims, keep_dims, z, INT64)
+    def exec_index_reduce(self, op_num, x, dims=None, keep_dims=False, z=None, extra_args=None):
+        return self._reduce(self.L.execIndexReduceScalar, self.L.execIndexReduce, "execIndexReduce", op_num, x, dims, keep_dims, z, INT64, extra_args)
 
-    def exec_transform_bool(self, op_num, x, z=None):
+    def exec_transform_bool(self, op_num, x, z=None, extra_args=None):
         if z is None:
             z = NDArray.empty(x.shape, BOOL)
-        self.L.execTransformBool(None, op_num, x.handle, None, z.handle)
+        holder, extra = self._extra_params(extra_args, x.dtype)
+        self.L.execTransformBool(None, op_num, x.handle, extra, z.handle)
         N.check("execTransformBool")
         return z
 
@@ -265,26 +279,28 @@ class Executioner:
         N.check("execSummaryStats")
         return z
 
-    def exec_reduce3(self, op_num, x, y, dims=None, keep_dims=False, z=None):
+    def exec_reduce3(self, op_num, x, y, dims=None, keep_dims=False, z=None, extra_args=None):
         if z is None:
             z = NDArray.empty(_reduced_shape(x.shape, dims, keep_dims), x.dtype)
+        holder, extra = self._extra_params(extra_args, z.dtype)
         if dims is None or len(dims) == 0:
-            self.L.execReduce3Scalar(None, op_num, x.handle, None, y.handle, z.handle)
+            self.L.execReduce3Scalar(None, op_num, x.handle, extra, y.handle, z.handle)
         else:
-            self.L.execReduce3Tad(None, op_num, x.handle, None, y.handle, z.handle, _dims_array(dims).handle)
+            self.L.execReduce3Tad(None, op_num, x.handle, extra, y.handle, z.handle, _dims_array(dims).handle)
         N.check("execReduce3")
         return z
 
-    def _reduce_dims_only(self, fn, name, op_num, x, dims, keep_dims, z, zdtype):
+    def _reduce_dims_only(self, fn, name, op_num, x, dims, keep_dims, z, zdtype, extra_args=None):
         if z is None:
             z = NDArray.empty(_reduced_shape(x.shape, dims, keep_dims), zdtype)
         d = _dims_array(dims if dims else list(range(len(x.shape))))
-        fn(None, op_num, x.handle, None, z.handle, d.handle)
+        holder, extra = self._extra_params(extra_args, x.dtype)
+        fn(None, op_num, x.handle, extra, z.handle, d.handle)
         N.check(name)
         return z
 
-    def exec_reduce_long(self, op_num, x, dims=None, keep_dims=False, z=None):
-        return self._reduce_dims_only(self.L.execReduceLong, "execReduceLong", op_num, x, dims, keep_dims, z, INT64)
+    def exec_reduce_long(self, op_num, x, dims=None, keep_dims=False, z=None, extra_args=None):
+        return self._reduce_dims_only(self.L.execReduceLong, "execReduceLong", op_num, x, dims, keep_dims, z, INT64, extra_args)
 
     def exec_reduce_bool(self, op_num, x, dims=None, keep_dims=False, z=None):
         return self._reduce_dims_only(self.L.execReduceBool, "execReduceBool", op_num, x, dims, keep_dims, z, BOOL)

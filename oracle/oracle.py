@@ -471,3 +471,81 @@ def log_softmax(x, dim=-1):
             return np.zeros_like(x)
         e = np.exp(x - x.max(axis=dim, keepdims=True))
         return np.log(e / e.sum(axis=dim, keepdims=True, dtype=x.dtype))
+
+
+# ---- ops built on a match condition read from the extra parameters (numpy restatements) -----------------------------------
+def _in_type(a, like):
+    """Round a float64 value / array through the dtype of `like` (comparisons run in the array's own type)."""
+    return np.asarray(a).astype(like.dtype)
+
+
+def match_mask(x, compare, eps, mode):
+    """MatchConditionBool (ops/ops.h:1800-1845): the sixteen modes of Conditions.ConditionMode, evaluated in x's type."""
+    x = np.asarray(x)
+    c, e = _in_type(compare, x), _in_type(eps, x)
+    with np.errstate(invalid="ignore"):
+        diff = np.abs((x - c).astype(x.dtype))
+        inf, nan = np.isinf(x) if x.dtype.kind == "f" else np.zeros(x.shape, bool), np.isnan(x) if x.dtype.kind == "f" else np.zeros(x.shape, bool)
+        table = {0: lambda: diff <= e, 1: lambda: diff > e, 2: lambda: x < c, 3: lambda: x > c, 4: lambda: x <= c, 5: lambda: x >= c,
+                 6: lambda: np.abs(x) < c, 7: lambda: np.abs(x) > c, 8: lambda: inf, 9: lambda: nan, 10: lambda: x == c, 11: lambda: x != c,
+                 12: lambda: np.abs(x) >= c, 13: lambda: np.abs(x) <= c, 14: lambda: ~(inf | nan), 15: lambda: inf | nan}
+        return np.asarray(table[int(mode)](), dtype=bool)
+
+
+def compare_and_set_transform(x, compare, set_value, eps, mode):
+    """TransformSame 13 (ops.h:845-940): z = cond(x) ? set : x."""
+    x = np.asarray(x)
+    return np.where(match_mask(x, compare, eps, mode), _in_type(set_value, x), x)
+
+
+def compare_and_set(x, y, compare, eps, mode):
+    """Pairwise 12 / Scalar 33 (ops.h:719-840): the SECOND operand is tested and taken: z = cond(y) ? y : x."""
+    x = np.asarray(x)
+    y = np.broadcast_to(np.asarray(y, dtype=x.dtype), x.shape)
+    return np.where(match_mask(y, compare, eps, mode), y, x)
+
+
+def compare_and_replace(x, y, compare, eps, mode):
+    """Pairwise 13 (ops.h:593-715): z = cond(x) ? y : x."""
+    x = np.asarray(x)
+    return np.where(match_mask(x, compare, eps, mode), np.asarray(y, dtype=x.dtype), x)
+
+
+def _along(x, dims):
+    x = np.asarray(x)
+    if dims is None or len(dims) == 0:
+        return x.reshape(1, -1), ()
+    dims = sorted(d + x.ndim if d < 0 else d for d in dims)
+    keep = [d for d in range(x.ndim) if d not in dims]
+    t = np.transpose(x, keep + dims)
+    out_shape = tuple(x.shape[d] for d in keep)
+    return t.reshape(int(np.prod(out_shape)) if out_shape else 1, -1), out_shape
+
+
+def match_count(x, compare, eps, mode, dims=None):
+    """ReduceLong 2 MatchCondition (ops.h:2430-2500): how many elements of each sub-array meet the condition."""
+    rows, shape = _along(x, dims)
+    return match_mask(rows, compare, eps, mode).sum(1).astype(np.int64).reshape(shape)
+
+
+def first_last_index(x, compare, eps, mode, dims=None, last=False):
+    """IndexReduce 4 / 5 (ops.h:2061-2150): position (row-major inside the sub-array) of the first / last element that meets
+    the condition, -1 when none does."""
+    rows, shape = _along(x, dims)
+    m = match_mask(rows, compare, eps, mode)
+    n = m.shape[1]
+    idx = np.where(m.any(1), (n - 1 - m[:, ::-1].argmax(1)) if last else m.argmax(1), -1)
+    return idx.astype(np.int64).reshape(shape)
+
+
+def norm_p(x, p, dims=None):
+    """ReduceFloat 6 NormP (ops.h:1280-1286): (sum |x|^p)^(1/p)."""
+    rows, shape = _along(np.asarray(x, dtype=np.float64), dims)
+    return ((np.abs(rows) ** p).sum(1) ** (1.0 / p)).reshape(shape)
+
+
+def equals_with_eps(x, y, eps, dims=None):
+    """Reduce3 4 EqualsWithEps (op_macros_special.h:449-480, templatemath.h:115): 1 when |x - y| <= eps for every pair."""
+    rx, shape = _along(np.asarray(x, dtype=np.float64), dims)
+    ry, _ = _along(np.asarray(y, dtype=np.float64), dims)
+    return (np.abs(rx - ry) <= eps).all(1).astype(np.float64).reshape(shape)
