@@ -60,7 +60,14 @@
  *   layer_norm ........................ closed form (TestLayerOpValidation.java:1188-1333)
  *   dot_product_attention_v2 .......... parity unpinned: the reference has no enabled
  *                                       test; pinned only as matmul+softmax composition
- *                                       and a textbook causal mask
+ *                                       and a textbook causal mask; query / value masks: the padded-batch identity
+ *                                       (masked keys == truncated keys) and the manual composition of
+ *                                       TestReductionOpValidation.java:1291-1327 (tests/test_oracle_attention_masks.py)
+ *   match-condition ops, norm_p,
+ *   equals_with_eps (oracle.py, numpy)  NDArrayTests2.cpp:96-103 (FirstIndex), BooleanIndexingTest.java:208-335
+ *                                       (CompareAndSet / CompareAndReplace / MatchCondition cases), closed forms
+ *                                       (tests/test_oracle_cond_ops.py)
+ *   integer arrays .................... no restatement: the GPU tests compare with numpy's integer arithmetic directly
  */
 #ifndef ND4J_ORACLE_H
 #define ND4J_ORACLE_H
