@@ -148,6 +148,45 @@ __device__ __forceinline__ void tileOf(unsigned bid, unsigned nb, unsigned tiles
   tn = inGroup / gsz;
 }
 
+// Stores a wave's TM x TN accumulator tiles of 32 x 32: lane owns column (lane % 32); register r of a tile is row
+// 8*(r/4) + 4*(lane/32) + r%4.  Whether C is read back (beta) and whether a bias row is added is decided once, outside
+// the element loops: left inside, the compiler keeps two branches and a wait per element (5 us of a 4096^3 launch).
+template <typename T, int TM, int TN, bool BOUNDS, bool HAS_BETA, bool HAS_BIAS>
+__device__ __forceinline__ void storeAccTilesImpl(const GemmArgs& g, T* __restrict__ C, const f32x16 (&acc)[TM][TN], LongType rowBase, LongType colBase,
+                                                  int lane) {
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const LongType col = colBase + j * 32 + (lane & 31);
+      if (BOUNDS && col >= g.N) continue;
+      const float bj = HAS_BIAS ? to_float(static_cast<const T*>(g.bias)[col]) : 0.f;
+      const LongType row0 = rowBase + i * 32 + 4 * (lane >> 5);
+      T* p = C + row0 * g.cRow + col * g.cCol;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int dr = 8 * (r / 4) + (r & 3);
+        if (BOUNDS && row0 + dr >= g.M) continue;
+        T* q = p + (LongType)dr * g.cRow;
+        float v = g.alpha * acc[i][j][r];
+        if (HAS_BETA) v += g.beta * to_float(*q);
+        if (HAS_BIAS) v += bj;
+        *q = Conv<T>::from(v);
+      }
+    }
+}
+template <typename T, int TM, int TN, bool BOUNDS>
+__device__ __forceinline__ void storeAccTiles(const GemmArgs& g, T* __restrict__ C, const f32x16 (&acc)[TM][TN], LongType rowBase, LongType colBase, int lane) {
+  if (g.beta != 0.f) {
+    if (g.bias) storeAccTilesImpl<T, TM, TN, BOUNDS, true, true>(g, C, acc, rowBase, colBase, lane);
+    else storeAccTilesImpl<T, TM, TN, BOUNDS, true, false>(g, C, acc, rowBase, colBase, lane);
+  } else if (g.bias) {
+    storeAccTilesImpl<T, TM, TN, BOUNDS, false, true>(g, C, acc, rowBase, colBase, lane);
+  } else {
+    storeAccTilesImpl<T, TM, TN, BOUNDS, false, false>(g, C, acc, rowBase, colBase, lane);
+  }
+}
+
 // ---- 16-bit MFMA kernel ----------------------------------------------------------------------------------------------
 template <typename T, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
@@ -243,24 +282,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16(GemmArgs g, const T*
         }
     return;
   }
-#pragma unroll
-  for (int i = 0; i < TM; i++)
-#pragma unroll
-    for (int j = 0; j < TN; j++) {
-      const LongType col = n0 + wn * WTN + j * 32 + (lane & 31);
-      if (col >= g.N) continue;
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const LongType row = m0 + wm * WTM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r & 3);
-        if (row < g.M) {
-          const LongType off = row * g.cRow + col * g.cCol;
-          float v = g.alpha * acc[i][j][r];
-          if (g.beta != 0.f) v += g.beta * to_float(C[off]);
-          if (g.bias) v += to_float(static_cast<const T*>(g.bias)[col]);
-          C[off] = Conv<T>::from(v);
-        }
-      }
-    }
+  storeAccTiles<T, TM, TN, true>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
 }
 
 // Second half of a split-K product: one block per (output tile, q-group), same thread -> element mapping as
@@ -384,25 +406,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16p(GemmArgs g, const T
     __syncthreads();
   }
 
-  // epilogue: lane owns column (lane % 32); register r of a 32x32 tile is row 8*(r/4) + 4*(lane/32) + r%4
-#pragma unroll
-  for (int i = 0; i < TM; i++)
-#pragma unroll
-    for (int j = 0; j < TN; j++) {
-      const LongType col = n0 + wn * WTN + j * 32 + (lane & 31);
-      if (col >= g.N) continue;
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const LongType row = m0 + wm * WTM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r & 3);
-        if (row < g.M) {
-          const LongType off = row * g.cRow + col * g.cCol;
-          float v = g.alpha * acc[i][j][r];
-          if (g.beta != 0.f) v += g.beta * to_float(C[off]);
-          if (g.bias) v += to_float(static_cast<const T*>(g.bias)[col]);
-          C[off] = Conv<T>::from(v);
-        }
-      }
-    }
+  storeAccTiles<T, TM, TN, true>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
 }
 
 // The same kernel with the global loads of PD K-tiles in flight (PD register sets, the K loop unrolled PD times so that
@@ -501,25 +505,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16q(GemmArgs g, const T
   }
   }
 
-  // epilogue: lane owns column (lane % 32); register r of a 32x32 tile is row 8*(r/4) + 4*(lane/32) + r%4
-#pragma unroll
-  for (int i = 0; i < TM; i++)
-#pragma unroll
-    for (int j = 0; j < TN; j++) {
-      const LongType col = n0 + wn * WTN + j * 32 + (lane & 31);
-      if (col >= g.N) continue;
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const LongType row = m0 + wm * WTM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r & 3);
-        if (row < g.M) {
-          const LongType off = row * g.cRow + col * g.cCol;
-          float v = g.alpha * acc[i][j][r];
-          if (g.beta != 0.f) v += g.beta * to_float(C[off]);
-          if (g.bias) v += to_float(static_cast<const T*>(g.bias)[col]);
-          C[off] = Conv<T>::from(v);
-        }
-      }
-    }
+  storeAccTiles<T, TM, TN, true>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
 }
 
 // Steady-state kernel for problems made of whole tiles (M % BM == 0, N % BN == 0, K % 64 == 0): no bounds handling,
@@ -664,22 +650,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16f(GemmArgs g, const T
     }
   }
 
-  // epilogue: lane owns column (lane % 32); register r of a 32x32 tile is row 8*(r/4) + 4*(lane/32) + r%4
-#pragma unroll
-  for (int i = 0; i < TM; i++)
-#pragma unroll
-    for (int j = 0; j < TN; j++) {
-      const LongType col = n0 + wn * WTN + j * 32 + (lane & 31);
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const LongType row = m0 + wm * WTM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r & 3);
-        const LongType off = row * g.cRow + col * g.cCol;
-        float v = g.alpha * acc[i][j][r];
-        if (g.beta != 0.f) v += g.beta * to_float(C[off]);
-        if (g.bias) v += to_float(static_cast<const T*>(g.bias)[col]);
-        C[off] = Conv<T>::from(v);
-      }
-    }
+  storeAccTiles<T, TM, TN, false>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
 }
 
 // Whole-tile kernel whose global loads write LDS directly (global_load_lds_dwordx4): no staging registers, no LDS
@@ -735,14 +706,24 @@ __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restr
     }
   }
   const LongType aStep = BK, bStep = B_KC ? (LongType)BK : (LongType)BK * ldb;
+  // The loads are written as assembly on purpose.  Issued through the builtin, the compiler's wait-count pass knows of
+  // an outstanding write into LDS and, having no alias information for the transposing read, puts s_waitcnt vmcnt(0)
+  // in front of every ds_read_b64_tr_b16 that follows -- twice per K-tile the wave then sits out the whole latency of
+  // loads it has only just issued.  All waiting on these loads is explicit in this kernel (s_waitcnt vmcnt before the
+  // barrier), so the compiler need not know of them.  M0 carries the LDS address of the wave's chunk; nothing else in
+  // this kernel uses M0 (it is a reserved register and cannot be named as a clobber).
+  auto loadToLds = [&](const T* src, u32x4* dst) {
+    const unsigned ldsAddr = (unsigned)(size_t)(lds_ptr)dst;
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(ldsAddr) : "memory");
+  };
   auto issueLoads = [&](u32x4* stage, int from, int to) {
 #pragma unroll
     for (int i = from; i < to; i++) {
       if (i < 4) {
-        __builtin_amdgcn_global_load_lds((glb_ptr)aSrc[i], (lds_ptr)(stage + (wave * 4 + i) * 64), 16, 0, 0);
+        loadToLds(aSrc[i], stage + (wave * 4 + i) * 64);
         aSrc[i] += aStep;
       } else {
-        __builtin_amdgcn_global_load_lds((glb_ptr)bSrc[i - 4], (lds_ptr)(stage + SLOTS_OP + (wave * 4 + i - 4) * 64), 16, 0, 0);
+        loadToLds(bSrc[i - 4], stage + SLOTS_OP + (wave * 4 + i - 4) * 64);
         bSrc[i - 4] += bStep;
       }
     }
@@ -871,22 +852,196 @@ __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restr
     }
   }
 
-  // epilogue: lane owns column (lane % 32); register r of a 32x32 tile is row 8*(r/4) + 4*(lane/32) + r%4
+  storeAccTiles<T, TM, TN, false>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
+}
+
+// The same 256 x 256 tile for A k-contiguous and B row-major with the operands in two RINGS of LDS units instead of two
+// whole stages, so that a slot is refilled as soon as it is drained and the direct loads are issued at an even rate --
+// one A and one B load per wave and eight MFMAs -- with at least one step (sixteen MFMAs per wave) between a load's
+// issue and the barrier that hands its data to the readers.
+//   step = 32 k = two k-steps of eight MFMAs (phase 0, phase 1), one barrier per step, between the phases.
+//   A ring: 3 units of 256 rows x 64 k (whole 128-byte lines of every row, chunk layout of gemm_mfma16d), 32 KiB each;
+//           unit j serves steps 2j and 2j + 1.
+//   B ring: 4 units of 32 k-rows x 256 n, 16 KiB each; unit s serves step s.            3 * 32 + 4 * 16 = 160 KiB.
+// Phase 0 of step s reads the fragments of phase 1; phase 1 reads those of step s + 1, phase 0.  The barrier of step s
+// therefore certifies (a) that the units step s + 1 reads have landed and (b) that every wave is through with the units
+// of step s - 1.  What is issued when (j = s / 2; a wave owns chunks 0..3 of every A unit and chunks 0..1 of every B unit):
+//   even s: phase 0: A chunk 3 of unit j + 1, B chunk 1 of unit s + 2;   phase 1: A chunk 0 of unit j + 2, B chunk 0 of unit s + 3
+//   odd s:  phase 0: A chunk 1 of unit j + 2, B chunk 1 of unit s + 2;   phase 1: A chunk 2 of unit j + 2, B chunk 0 of unit s + 3
+// Every load goes into a slot whose unit was last read two barriers ago, and is at least four loads old (two phases)
+// when the barrier that certifies it is reached: s_waitcnt vmcnt(4) in front of every barrier (loads complete in
+// order).  The loop is branch-free: past the end of K the pointers stop advancing, so the surplus loads re-read the
+// last unit into slots nobody reads any more.  K must be a multiple of 128 (four steps per loop iteration).
+template <typename T>
+__global__ __launch_bounds__(512) void gemm_mfma16r(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
+                                                    unsigned tilesM, unsigned tilesN) {
+  constexpr int BM = 256, BN = 256, WN = 4, WTM = 128, WTN = 64, TM = 4, TN = 2, NM = TM * TN;
+  constexpr int A_UNIT = 256 * 8;     // 16-byte slots of one A unit
+  constexpr int B_UNIT = 32 * 32;     // 16-byte slots of one B unit
+  constexpr int B_BASE = 3 * A_UNIT;  // the B ring sits behind the A ring
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  u32x4* smem = reinterpret_cast<u32x4*>(smem_raw);
+
+  unsigned tm, tn;
+  tileOf(blockIdx.x, gridDim.x, tilesM, tilesN, tm, tn);
+  const LongType m0 = (LongType)tm * BM, n0 = (LongType)tn * BN;
+  { LongType oa, ob, oc; batchOffsets(g, blockIdx.z, oa, ob, oc); A += oa; B += ob; C += oc; }
+  const LongType lda = g.aRow, ldb = g.bRow;
+  const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6), h = lane >> 5;
+  const int wm = wave / WN, wn = wave % WN;
+
+  // ---- global side ---------------------------------------------------------------------------------------------------
+  const int lj = lane >> 3, lp = lane & 7;
+  const T* aSrc[4];
+  const T* bSrc[2];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int cw = wave * 4 + i;                          // 8 rows, all 8 k-groups of the unit
+    const int lkg = (lp - 4 * (cw & 1) - (lj >> 1)) & 7;
+    aSrc[i] = A + (m0 + cw * 8 + lj) * lda + lkg * 8;
+  }
+#pragma unroll
+  for (int c = 0; c < 2; c++) {
+    const int kr = 2 * (wave * 2 + c) + (lane >> 5), q = lane & 31;   // two k-rows of 256 n per chunk
+    bSrc[c] = B + (LongType)kr * ldb + n0 + 8 * (q ^ (4 * (kr & 3)));
+  }
+  const int S = (int)(g.K / 32), nA = (int)(g.K / 64);   // steps, A units
+  const LongType aStep = 64, bStep = 32 * ldb;
+  auto loadToLds = [&](const T* src, u32x4* dst) {
+    const unsigned ldsAddr = (unsigned)(size_t)(lds_ptr)dst;
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(ldsAddr) : "memory");
+  };
+  // chunk i of A unit `unit` into ring slot `slot`; the pointer moves on only while there is a next unit
+  auto issueA = [&](int i, int slot, int unit) {
+    loadToLds(aSrc[i], smem + slot * A_UNIT + (wave * 4 + i) * 64);
+    aSrc[i] += unit + 1 < nA ? aStep : 0;
+  };
+  auto issueB = [&](int c, int slot, int unit) {
+    loadToLds(bSrc[c], smem + B_BASE + slot * B_UNIT + (wave * 2 + c) * 64);
+    bSrc[c] += unit + 1 < S ? bStep : 0;
+  };
+
+  // ---- LDS side --------------------------------------------------------------------------------------------------------
+  int offA[TM][4];   // slot of (row, k-step ks of the unit) inside an A unit, as in gemm_mfma16d
+#pragma unroll
+  for (int i = 0; i < TM; i++) {
+    const int r = wm * WTM + i * 32 + (lane & 31);
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) offA[i][ks] = (r >> 3) * 64 + 8 * (r & 7) + ((2 * ks + h + 4 * ((r >> 3) & 1) + ((r & 7) >> 1)) & 7);
+  }
+  int trB[TN];       // byte offset of the transposing read inside a B unit (k-step 0, first half)
+#pragma unroll
+  for (int jt = 0; jt < TN; jt++) {
+    const int grp = lane >> 4, i16 = lane & 15;
+    const int n4 = wn * WTN + jt * 32 + 16 * (grp & 1) + 4 * (i16 & 3);
+    const int k = 8 * (grp >> 1) + (i16 >> 2);
+    const int phys = (n4 >> 3) ^ (4 * ((i16 >> 2) & 3));
+    trB[jt] = k * 512 + phys * 16 + ((n4 >> 2) & 1) * 8;
+  }
+  u32x4 fa[2][TM], fb[2][TN];
+  // fragments of k-step ksA (0..3) of the A unit in ring slot aSlot and k-step ksB (0..1) of the B unit in slot bSlot
+  auto readFragA = [&](int aSlot, int ksA, int buf) {
+    const u32x4* ua = smem + aSlot * A_UNIT;
+#pragma unroll
+    for (int i = 0; i < TM; i++) fa[buf][i] = ua[offA[i][ksA]];
+  };
+  auto readFragB = [&](int bSlot, int ksB, int buf) {
+    const __attribute__((address_space(3))) unsigned char* ub =
+        (const __attribute__((address_space(3))) unsigned char*)(lds_ptr)(smem + B_BASE + bSlot * B_UNIT) + ksB * 8192;
+#pragma unroll
+    for (int jt = 0; jt < TN; jt++) {
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(ub + trB[jt]));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(ub + trB[jt] + 2048));
+      const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+      fb[buf][jt] = u32x4{l2[0], l2[1], h2[0], h2[1]};
+    }
+  };
+
+  f32x16 acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
-    for (int j = 0; j < TN; j++) {
-      const LongType col = n0 + wn * WTN + j * 32 + (lane & 31);
+    for (int j = 0; j < TN; j++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const LongType row = m0 + wm * WTM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r & 3);
-        const LongType off = row * g.cRow + col * g.cCol;
-        float v = g.alpha * acc[i][j][r];
-        if (g.beta != 0.f) v += g.beta * to_float(C[off]);
-        if (g.bias) v += to_float(static_cast<const T*>(g.bias)[col]);
-        C[off] = Conv<T>::from(v);
-      }
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+  auto mfmas = [&](int buf, int from, int to) {
+#pragma unroll
+    for (int idx = from; idx < to; idx++) {
+      const int i = idx / TN, j = idx % TN;
+      acc[i][j] = Mfma16<T>::mma(fa[buf][i], fb[buf][j], acc[i][j]);
     }
+  };
+
+  // ---- prologue: A unit 0, B units 0 and 1, A unit 1 chunks 0..2, B unit 2 chunk 0 -----------------------------------------
+#pragma unroll
+  for (int i = 0; i < 4; i++) issueA(i, 0, 0);
+  issueB(0, 0, 0); issueB(1, 0, 0);
+  issueB(0, 1, 1); issueB(1, 1, 1);
+  issueA(0, 1, 1); issueA(1, 1, 1); issueA(2, 1, 1);
+  issueB(0, 2, 2);
+  asm volatile("s_waitcnt vmcnt(6)" ::: "memory");   // A unit 0 and B unit 0 (the first six loads) have landed
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+  readFragA(0, 0, 0);
+  readFragB(0, 0, 0);
+
+  int a0 = 0, a1 = 1, a2 = 2;   // ring slots of A units j, j + 1, j + 2
+  // one phase = four pairs of MFMAs; the four A reads go out with the first pair, the four B reads with the second; the
+  // A load is issued in front of pair PA, the B load in front of pair PB
+  auto phase = [&](auto pa, auto pb, int buf, int aSlot, int ksA, int bSlot, int ksB, int nbuf, auto&& loadA, auto&& loadB) {
+    constexpr int PA = decltype(pa)::value, PB = decltype(pb)::value;
+#pragma unroll
+    for (int pr = 0; pr < 4; pr++) {
+      if (pr == PA) loadA();
+      if (pr == PB) loadB();
+      if (pr == 0) readFragA(aSlot, ksA, nbuf);
+      if (pr == 1) readFragB(bSlot, ksB, nbuf);
+      mfmas(buf, 2 * pr, 2 * pr + 2);
+      if (pr < 2) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto sync = [&]() {
+    asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto mainLoop = [&](auto pa, auto pb) {
+    for (int s = 0; s < S; s += 4) {
+      const int j = s >> 1;
+      // step s (even), B slot 0
+      phase(pa, pb, 0, a0, 1, 0, 1, 1, [&] { issueA(3, a1, j + 1); }, [&] { issueB(1, 2, s + 2); });
+      sync();
+      phase(pa, pb, 1, a0, 2, 1, 0, 0, [&] { issueA(0, a2, j + 2); }, [&] { issueB(0, 3, s + 3); });
+      // step s + 1 (odd), B slot 1
+      phase(pa, pb, 0, a0, 3, 1, 1, 1, [&] { issueA(1, a2, j + 2); }, [&] { issueB(1, 3, s + 3); });
+      sync();
+      phase(pa, pb, 1, a1, 0, 2, 0, 0, [&] { issueA(2, a2, j + 2); }, [&] { issueB(0, 0, s + 4); });
+      // step s + 2 (even), B slot 2; the A units have moved on by one: (a0, a1, a2) -> (a1, a2, a0)
+      phase(pa, pb, 0, a1, 1, 2, 1, 1, [&] { issueA(3, a2, j + 2); }, [&] { issueB(1, 0, s + 4); });
+      sync();
+      phase(pa, pb, 1, a1, 2, 3, 0, 0, [&] { issueA(0, a0, j + 3); }, [&] { issueB(0, 1, s + 5); });
+      // step s + 3 (odd), B slot 3
+      phase(pa, pb, 0, a1, 3, 3, 1, 1, [&] { issueA(1, a0, j + 3); }, [&] { issueB(1, 1, s + 5); });
+      sync();
+      phase(pa, pb, 1, a2, 0, 0, 0, 0, [&] { issueA(2, a0, j + 3); }, [&] { issueB(0, 2, s + 6); });
+      const int o0 = a0, o1 = a1;
+      a0 = a2; a1 = o0; a2 = o1;   // two units on: (a0, a1, a2) -> (a2, a0, a1)
+    }
+  };
+  // the A load goes out in front of the first pair of MFMAs of a phase, the B load in front of the third (measured: 1163
+  // cycles per step against 1190 with both loads in the second half of the phase; 1024 are the MFMAs alone)
+  mainLoop(std::integral_constant<int, 0>{}, std::integral_constant<int, 2>{});
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the surplus loads of the last steps
+
+  storeAccTiles<T, TM, TN, false>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
 }
 
 // How many K-splits a launch of BM x BN tiles gets: enough to put about two blocks on every CU when the tiles alone
@@ -953,6 +1108,19 @@ static bool launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const 
   if (tiles256 < 192) return launchMfma16Cfg<T, 128, 128, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
   if (g.hasEpi) return false;
   static const bool direct = getenv("ND4JHIP_GEMM_DIRECT") ? atoi(getenv("ND4JHIP_GEMM_DIRECT")) != 0 : true;
+  static const bool ring = getenv("ND4JHIP_GEMM_RING") ? atoi(getenv("ND4JHIP_GEMM_RING")) != 0 : true;
+  if constexpr (A_KC && !B_KC) {
+    if (direct && ring && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 128 == 0) {
+      constexpr size_t LDS = (3 * 256 * 8 + 4 * 32 * 32) * 16;   // 160 KiB: the whole LDS of a CU
+      auto kern = gemm_mfma16r<T>;
+      static std::once_flag attrOnce;
+      std::call_once(attrOnce, [&] { HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS)); });
+      const unsigned tM = (unsigned)(g.M / 256), tN = (unsigned)(g.N / 256);
+      noteKernel("gemm_mfma16r<%s,256x256,akc=1,bkc=0>", tname<T>());
+      hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(512), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
+      return true;
+    }
+  }
   if (direct && A_KC && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 64 == 0 && g.K >= 128) {
     constexpr size_t LDS = 2 * 2 * 256 * 8 * 16;
     auto kern = gemm_mfma16d<T, B_KC>;
@@ -1079,24 +1247,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32(GemmArgs g, const fl
     if (kt + 1 < KT) { storeA(cur ^ 1); storeB(cur ^ 1); }
     __syncthreads();
   }
-#pragma unroll
-  for (int i = 0; i < TM; i++)
-#pragma unroll
-    for (int j = 0; j < TN; j++) {
-      const LongType col = n0 + wn * WTN + j * 32 + (lane & 31);
-      if (col >= g.N) continue;
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const LongType row = m0 + wm * WTM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r & 3);
-        if (row < g.M) {
-          const LongType off = row * g.cRow + col * g.cCol;
-          float v = g.alpha * acc[i][j][r];
-          if (g.beta != 0.f) v += g.beta * C[off];
-          if (g.bias) v += static_cast<const float*>(g.bias)[col];
-          C[off] = v;
-        }
-      }
-    }
+  storeAccTiles<float, TM, TN, true>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
 }
 
 // The fp32 kernel for launches of whole tiles that put one small tile on a CU: PD K-tiles of global loads in flight (PD
@@ -1193,21 +1344,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32q(GemmArgs g, const f
       __syncthreads();
     }
   }
-#pragma unroll
-  for (int i = 0; i < TM; i++)
-#pragma unroll
-    for (int j = 0; j < TN; j++) {
-      const LongType col = n0 + wn * WTN + j * 32 + (lane & 31);
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const LongType row = m0 + wm * WTM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r & 3);
-        const LongType off = row * g.cRow + col * g.cCol;
-        float v = g.alpha * acc[i][j][r];
-        if (g.beta != 0.f) v += g.beta * C[off];
-        if (g.bias) v += static_cast<const float*>(g.bias)[col];
-        C[off] = v;
-      }
-    }
+  storeAccTiles<float, TM, TN, false>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
 }
 
 template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC>

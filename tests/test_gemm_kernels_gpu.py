@@ -57,8 +57,14 @@ def _check_rows_cols(z, a64, b64, tol, rng, what):
 CASES = [
     # BASELINE config 2 at 4096^3
     (FLOAT32, 4096, 4096, 4096, "gemm_mfma32q<f32,128x128,akc=1,bkc=0,pd=4>", "gemm_mfma32q<f32,128x128,akc=1,bkc=1,pd=4>", "gemm_mfma32q<f32,128x128,akc=0,bkc=0,pd=4>"),
-    (HALF, 4096, 4096, 4096, "gemm_mfma16d<f16,256x256,akc=1,bkc=0>", "gemm_mfma16d<f16,256x256,akc=1,bkc=1>", "gemm_mfma16f<f16,256x256,akc=0,bkc=0>"),
-    (BFLOAT16, 4096, 4096, 4096, "gemm_mfma16d<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1>", "gemm_mfma16f<bf16,256x256,akc=0,bkc=0>"),
+    (HALF, 4096, 4096, 4096, "gemm_mfma16r<f16,256x256,akc=1,bkc=0>", "gemm_mfma16d<f16,256x256,akc=1,bkc=1>", "gemm_mfma16f<f16,256x256,akc=0,bkc=0>"),
+    (BFLOAT16, 4096, 4096, 4096, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1>", "gemm_mfma16f<bf16,256x256,akc=0,bkc=0>"),
+    # the ring kernel at its shortest K (the prologue alone fills the rings) and at a K that ends in the middle of both rings;
+    # a K that is a multiple of 64 only stays on the two-stage direct kernel
+    (BFLOAT16, 4096, 4096, 128, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1>", None),
+    (HALF, 4096, 4096, 640, "gemm_mfma16r<f16,256x256,akc=1,bkc=0>", "gemm_mfma16d<f16,256x256,akc=1,bkc=1>", None),
+    (BFLOAT16, 4096, 4096, 1152, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1>", None),
+    (BFLOAT16, 4096, 4096, 192, "gemm_mfma16d<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1>", None),
     # BASELINE config 2 at 1024^3
     (FLOAT32, 1024, 1024, 1024, "gemm_mfma32q<f32,64x64,akc=1,bkc=0,pd=8>", "gemm_mfma32q<f32,64x64,akc=1,bkc=1,pd=8>", "gemm_mfma32q<f32,64x64,akc=0,bkc=0,pd=8>"),
     (HALF, 1024, 1024, 1024, "gemm_mfma16q<f16,64x64,akc=1,bkc=0>", "gemm_mfma16q<f16,64x64,akc=1,bkc=1>", "gemm_mfma16q<f16,64x64,akc=0,bkc=0>"),
@@ -125,8 +131,8 @@ def test_fp16_and_bf16_agree(ex, n):
     assert_close(zh[rows], a64[rows] @ b64, 1e-2, 1e-2, "fp16 sampled rows")
 
 
-def test_alpha_beta_on_the_direct_kernel(ex):
-    """C = alpha A B + beta C through the 256 x 256 direct-to-LDS kernel (its epilogue reads C)."""
+def test_alpha_beta_on_the_ring_kernel(ex):
+    """C = alpha A B + beta C through the 256 x 256 ring kernel (its epilogue reads C), batched."""
     rng = np.random.default_rng(19)
     M, N, K = 512, 768, 512
     # a 256-tile launch needs at least 192 tiles: batch the problem
@@ -138,7 +144,33 @@ def test_alpha_beta_on_the_direct_kernel(ex):
     B, b64 = _device(b, BFLOAT16)
     C, c64 = _device(c0, BFLOAT16)
     ex.exec_custom("matmul", [A, B], [C], t_args=[0.5, 2.0])
-    assert _last_kernel(ex).startswith("gemm_mfma16d<bf16,256x256,akc=1,bkc=0>"), _last_kernel(ex)
+    assert _last_kernel(ex).startswith("gemm_mfma16r<bf16,256x256,akc=1,bkc=0>"), _last_kernel(ex)
     got = C.to_float()
     for bi in (0, 13, 31):
         assert_close(got[bi], 0.5 * (a64[bi] @ b64[bi]) + 2.0 * c64[bi], 1e-2, 2e-2, "batch %d" % bi)
+    # the same through the two-stage direct kernel (transposed B)
+    Bt, _ = _device(np.ascontiguousarray(np.swapaxes(b, 1, 2)), BFLOAT16)
+    C2, _ = _device(c0, BFLOAT16)
+    ex.exec_custom("matmul", [A, Bt], [C2], t_args=[0.5, 2.0], i_args=[0, 1])
+    assert _last_kernel(ex).startswith("gemm_mfma16d<bf16,256x256,akc=1,bkc=1>"), _last_kernel(ex)
+    assert np.array_equal(C2.to_float(), got), "transposed B gives the same bits (same products, same order)"
+
+
+def test_bias_row_on_the_large_kernels(ex):
+    """xw_plus_b at a shape that lands on the 256 x 256 kernels: the bias row is added in their epilogue."""
+    rng = np.random.default_rng(23)
+    M, K, N = 4096, 512, 4096
+    x = rng.normal(0, 1 / math.sqrt(K), (M, K)).astype(np.float32)
+    w = rng.normal(0, 1, (K, N)).astype(np.float32)
+    bias = rng.normal(0, 1, (N,)).astype(np.float32)
+    X, x64 = _device(x, BFLOAT16)
+    W, w64 = _device(w, BFLOAT16)
+    Bv, b64 = _device(bias, BFLOAT16)
+    z = ex.exec_custom("xw_plus_b", [X, W, Bv])[0].to_float()
+    assert _last_kernel(ex).startswith("gemm_mfma16r<bf16,256x256,akc=1,bkc=0>"), _last_kernel(ex)
+    rows = rng.choice(M, 16, replace=False)
+    assert_close(z[rows], x64[rows] @ w64 + b64, 1e-2, 1e-2, "sampled rows")
+    Wt, _ = _device(np.ascontiguousarray(w.T), BFLOAT16)
+    zt = ex.exec_custom("xw_plus_b", [X, Wt, Bv], i_args=[0, 1])[0].to_float()
+    assert _last_kernel(ex).startswith("gemm_mfma16d<bf16,256x256,akc=1,bkc=1>"), _last_kernel(ex)
+    assert np.array_equal(zt, z)
