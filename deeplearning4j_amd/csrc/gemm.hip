@@ -458,50 +458,51 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16q(GemmArgs g, const T
   lb[0].store(smem + SLOTS_A, t);
   __syncthreads();
 
+  // All four k-steps' fragments of a K-tile are held in registers, and those of K-tile kt + 1 are read right after the
+  // barrier that completes its stage, under the MFMAs of K-tile kt.  With one wave per SIMD and one accumulator per wave
+  // there is nothing else to cover an LDS round trip: reading the fragments one k-step ahead of their MFMA (32 cycles
+  // of cover for a latency several times that) made every k-step wait, 750 cycles per K-tile where the L2 stream of the
+  // tile takes about 410.
+  u32x4 fa[2][BK / 16][TM], fb[2][BK / 16][TN];
+  auto readTile = [&](int stage, int buf) {
+    const u32x4* sA = smem + stage * STAGE;
+    const u32x4* sB = sA + SLOTS_A;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ks++) {
+      const int kg = ks * 2 + (lane >> 5);
+#pragma unroll
+      for (int i = 0; i < TM; i++) fa[buf][ks][i] = sA[LayA::slot(kg, wm * WTM + i * 32 + (lane & 31))];
+#pragma unroll
+      for (int j = 0; j < TN; j++) fb[buf][ks][j] = sB[LayB::slot(kg, wn * WTN + j * 32 + (lane & 31))];
+    }
+  };
+  readTile(0, 0);
+
   for (LongType kt0 = 0; kt0 < KT; kt0 += PD) {
 #pragma unroll
   for (int u = 0; u < PD; u++) {
     const LongType kt = kt0 + u;
     const int cur = u & 1;
-    // K-tile kt sits in LDS: its register set takes K-tile kt + PD
+    // K-tile kt + 1 leaves its registers for the other stage (whose fragments every wave read before the last barrier)
+    {
+      u32x4* dst = smem + (cur ^ 1) * STAGE;
+      la[(u + 1) % PD].store(dst, t);
+      lb[(u + 1) % PD].store(dst + SLOTS_A, t);
+    }
+    // K-tile kt went to LDS one round ago: its register set takes K-tile kt + PD
     {
       const LongType nx = kt + PD < KT ? kt + PD : KT - 1;
       la[u].loadFull(A, lda, m0, nx * BK, t);
       lb[u].loadFull(B, ldb, n0, nx * BK, t);
     }
-    const u32x4* sA = smem + cur * STAGE;
-    const u32x4* sB = sA + SLOTS_A;
-    // software pipeline over the four k-steps: fragments of step ks+1 are read while the MFMAs of step ks
-    // run; the next tile's registers are written to the other LDS stage in the shadow of step 2
-    u32x4 fa[2][TM], fb[2][TN];
-    auto readFrag = [&](int ks, int buf) {
-      const int kg = ks * 2 + (lane >> 5);
+    __syncthreads();
+    readTile(cur ^ 1, cur ^ 1);
 #pragma unroll
-      for (int i = 0; i < TM; i++) fa[buf][i] = sA[LayA::slot(kg, wm * WTM + i * 32 + (lane & 31))];
-#pragma unroll
-      for (int j = 0; j < TN; j++) fb[buf][j] = sB[LayB::slot(kg, wn * WTN + j * 32 + (lane & 31))];
-    };
-    readFrag(0, 0);
-#pragma unroll
-    for (int ks = 0; ks < BK / 16; ks++) {
-      if (ks + 1 < BK / 16) readFrag(ks + 1, (ks + 1) & 1);
-      if (ks == 2) {
-        u32x4* dst = smem + (cur ^ 1) * STAGE;
-        la[(u + 1) % PD].store(dst, t);
-        lb[(u + 1) % PD].store(dst + SLOTS_A, t);
-      }
+    for (int ks = 0; ks < BK / 16; ks++)
 #pragma unroll
       for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < TN; j++) acc[i][j] = Mfma16<T>::mma(fa[ks & 1][i], fb[ks & 1][j], acc[i][j]);
-      // interleave: one LDS read issued per pair of MFMAs
-#pragma unroll
-      for (int q = 0; q < (TM + TN); q++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, (TM * TN) / (TM + TN) > 0 ? (TM * TN) / (TM + TN) : 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      }
-    }
-    __syncthreads();
+        for (int j = 0; j < TN; j++) acc[i][j] = Mfma16<T>::mma(fa[cur][ks][i], fb[cur][ks][j], acc[i][j]);
   }
   }
 
