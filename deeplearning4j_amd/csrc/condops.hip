@@ -4,6 +4,10 @@
 //   CompareAndSet (Pairwise 12 / Scalar 33, :719-840)     z = cond(y) ? y : x               params [compare, -, eps, mode]
 //   CompareAndReplace (Pairwise 13, :593-715)             z = cond(x) ? y : x               params [compare, -, eps, mode]
 //   MatchCondition (ReduceLong 2, :2430-2500)             count of cond(x) per sub-array    params [compare, eps, mode]
+// and, through the same elementwise kernel, the three pairwise ops whose extraParams hold plain numbers:
+//   Axpy (Pairwise 10, :328-333)                          z = p0 x + y (one fused multiply-add in the array's type)
+//   BinaryRelativeError (Pairwise 25, :2218-2270)         z = re(x, y) > p0 ? 1 : 0,  re = |x - y| / (|x| + |y|), 0 for two zeros
+//   BinaryMinimumAbsoluteRelativeError (26, :2274-2340)   z = re(x, y) > p0 && !(|x - y| < p1) ? 1 : 0
 //   FirstIndex / LastIndex (IndexReduce 4 / 5, :2061-2150) first / last position with cond(x), -1 when none
 // The sixteen modes: 0 |v - c| <= eps, 1 |v - c| > eps, 2 <, 3 >, 4 <=, 5 >=, 6 |v| < c, 7 |v| > c, 8 isinf, 9 isnan, 10 ==, 11 !=,
 // 12 |v| >= c, 13 |v| <= c, 14 finite, 15 inf or nan.  Comparisons run in the array's own type: the difference of mode 0 / 1
@@ -20,6 +24,13 @@ __device__ __forceinline__ double sub_in_type(double a, double b, int dt) {
   if (dt == DOUBLE || dt == INT32 || dt == INT64 || dt == BOOL) return a - b;
   const float d = (float)a - (float)b;
   return (dt == HALF || dt == BFLOAT16) ? (double)round_as(d, dt) : (double)d;
+}
+// |a - b| / (|a| + |b|) in the array's type, 0 for two zeros (math/templatemath.h:1144-1153)
+__device__ __forceinline__ double rel_err_in_type(double a, double b, int dt) {
+  if (a == 0.0 && b == 0.0) return 0.0;
+  if (dt == DOUBLE) return fabs(a - b) / (fabs(a) + fabs(b));
+  const float fa = (float)a, fb = (float)b;
+  return (double)round_as(fabsf(fa - fb) / (fabsf(fa) + fabsf(fb)), dt);
 }
 __device__ __forceinline__ bool cond_holds(const CondParams& c, double v) {
   const bool inf = (v - v) != (v - v) && v == v, nan = v != v;
@@ -50,12 +61,17 @@ __global__ __launch_bounds__(256) void cond_ew(int kind, CondParams c, DevShape 
   for (LongType i = (LongType)blockIdx.x * 256 + threadIdx.x; i < n; i += step) {
     const double a = load_any(x, c.xdt, walk<LongType>(sx, i));
     double b = scalar, r;
-    if ((kind == C_SET || kind == C_REPLACE) && !hasScalar) b = load_any(y, ydt, walk<LongType>(sy, i));
+    if (kind >= C_SET && !hasScalar) b = load_any(y, ydt, walk<LongType>(sy, i));
     switch (kind) {
       case C_MATCH_BOOL: r = cond_holds(c, a) ? 1.0 : 0.0; break;
       case C_SET_TRANSFORM: r = cond_holds(c, a) ? c.set : a; break;
       case C_SET: r = cond_holds(c, b) ? b : a; break;          // the second operand is the one tested
-      default: r = cond_holds(c, a) ? b : a; break;             // C_REPLACE
+      case C_REPLACE: r = cond_holds(c, a) ? b : a; break;
+      case C_AXPY: r = c.xdt == DOUBLE ? fma(c.compare, a, b) : (double)fmaf((float)c.compare, (float)a, (float)b); break;   // alpha x + y
+      case C_BIN_REL_ERR: r = rel_err_in_type(a, b, c.xdt) > c.compare ? 1.0 : 0.0; break;
+      default:                                                  // C_BIN_MIN_ABS_REL_ERR: relative AND absolute threshold exceeded
+        r = rel_err_in_type(a, b, c.xdt) > c.compare ? (fabs(sub_in_type(a, b, c.xdt)) < c.set ? 0.0 : 1.0) : 0.0;
+        break;
     }
     store_any(z, zdt, walk<LongType>(sz, i), r);
   }
@@ -66,7 +82,7 @@ void launchCondElementwise(hipStream_t s, CondKind kind, const CondParams& c, Da
   if (p.length == 0) return;
   LongType blocks = (p.length + 255) / 256;
   if (blocks > 4096) blocks = 4096;
-  const bool binary = kind == C_SET || kind == C_REPLACE;
+  const bool binary = kind >= C_SET;
   hipLaunchKernelGGL(cond_ew, dim3((unsigned)blocks), dim3(256), 0, s, (int)kind, c, p.own[0], p.own[1], binary && !hasScalar ? p.own[2] : p.own[1], (int)zdt,
                      (int)ydt, z, x, binary && !hasScalar ? y : x, p.length, scalar, hasScalar ? 1 : 0);
   HIP_CHECK(hipGetLastError());

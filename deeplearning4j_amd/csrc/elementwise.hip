@@ -140,6 +140,7 @@ template <> struct Tm<float> {
   static __device__ __forceinline__ float fmod_(float a, float b) { return fmodf(a, b); }
   static __device__ __forceinline__ float remainder_(float a, float b) { return remainderf(a, b); }
   static __device__ __forceinline__ float atan2_(float a, float b) { return atan2f(a, b); }
+  static __device__ __forceinline__ float gamma_(float x) { return tgammaf(x); }
 };
 template <> struct Tm<double> {
   static __device__ __forceinline__ double exp_(double x) { return exp(x); }
@@ -162,6 +163,7 @@ template <> struct Tm<double> {
   static __device__ __forceinline__ double fmod_(double a, double b) { return fmod(a, b); }
   static __device__ __forceinline__ double remainder_(double a, double b) { return remainder(a, b); }
   static __device__ __forceinline__ double atan2_(double a, double b) { return atan2(a, b); }
+  static __device__ __forceinline__ double gamma_(double x) { return tgamma(x); }
 };
 // 1 / (1 + e^-x) with the library exponential: derivatives subtract it from one, so it keeps full precision
 template <typename A> __device__ __forceinline__ A exact_sigmoid(A x) { return (A)1 / ((A)1 + Tm<A>::exp_(-x)); }
@@ -250,6 +252,23 @@ __device__ __forceinline__ A unary_tail(int k, A x) {
   }
 }
 
+// |a - b| / (|a| + |b|), 0 for two zeros (templatemath.h:1144-1153)
+template <typename A> __device__ __forceinline__ A rel_err(A a, A b) { return (a == (A)0 && b == (A)0) ? (A)0 : d_abs(a - b) / (d_abs(a) + d_abs(b)); }
+// Regularised lower incomplete gamma function as the reference sums it (templatemath.h:963-984): x^a e^-x / Gamma(a) times
+// the series sum x^i / (a (a+1) .. (a+i)), cut off when the running denominator passes 1e12 (whatever x is), 0 for a <= 1e-6
+template <typename A>
+__device__ __forceinline__ A igamma_(A a, A x) {
+  if (a <= (A)0.000001) return (A)0;
+  const A aim = Tm<A>::pow_(x, a) / (Tm<A>::exp_(x) * Tm<A>::gamma_(a));
+  A sum = (A)0, denom = (A)1, xi = (A)1;
+  for (int i = 0; (A)1 / denom > (A)1.0e-12 && i < 4096; i++) {
+    denom *= a + (A)i;
+    sum += xi / denom;
+    xi *= x;
+  }
+  return aim * sum;
+}
+
 // a = element of x, b = element of y or the scalar
 template <typename A>
 __device__ __forceinline__ A binary_tail(int k, A a, A b) {
@@ -289,6 +308,13 @@ __device__ __forceinline__ A binary_tail(int k, A a, A b) {
     case P_SQ_RSUB: { A d = b - a; return d * d; }                                             // op_macros_special.h:820-827
     case P_REVERSE_POW: return M::pow_(b, a);                                                  // ops.h:166
     case P_SXE_LOGITS_SMOOTHER: return a * ((A)1 - b) + (A)0.5f * b;                           // ops.h:352-355
+    case P_REL_ERR: return rel_err(a, b);                                                      // ops.h:2208-2213
+    case P_POW_DERIV: return b * M::pow_(a, b - (A)1);                                          // ops.h:82-87
+    case P_LOG_POISSON: return M::exp_(b) - a * b;                                              // ops.h:2389-2394
+    case P_LOG_POISSON_FULL:                                                                    // ops.h:1494-1502 (Stirling term)
+      return M::exp_(b) - a * b + (a * M::log_(a) - a + (A)0.5 * M::log_((A)(2.0 * 3.14159265358979323846) * a));
+    case P_IGAMMA: return igamma_(a, b);                                                        // ops.h:137, templatemath.h:963-984
+    case P_IGAMMAC: return (A)1 - igamma_(a, b);                                                // ops.h:140, templatemath.h:986-991
     case P_EQ: return (A)(a == b);                                                             // ops.h:181-186 (comparison ops)
     case P_NE: return (A)(a != b);
     case P_GT: return (A)(a > b);

@@ -39,6 +39,8 @@ enum PairwiseKind : int {
   // scalar table only
   P_ELU, P_ELU_D, P_LEAKY_RELU, P_LEAKY_RELU_D, P_LOG_X, P_RELU, P_RELU6, P_RELU_D, P_STEP, P_LSTM_CLIP,
   P_SQ_RSUB, P_REVERSE_POW, P_SXE_LOGITS_SMOOTHER,
+  // pairwise / scalar ops that need no parameter although the executioner may pass some
+  P_REL_ERR, P_POW_DERIV, P_LOG_POISSON, P_LOG_POISSON_FULL, P_IGAMMA, P_IGAMMAC,
   // comparisons (the bool tables): 1 / 0, stored into a BOOL output
   P_EQ, P_NE, P_GT, P_GE, P_LT, P_LE,
   P_TAIL_END
@@ -84,7 +86,7 @@ void launchIntElementwise(hipStream_t s, int k, bool binary, DataType xdt, DataT
                           void* z, const EwPlan& p, LongType scalar, bool hasScalar);
 
 // Ops that test a "match condition" read from the extra parameters (condops.hip)
-enum CondKind : int { C_MATCH_BOOL, C_SET_TRANSFORM, C_SET, C_REPLACE };
+enum CondKind : int { C_MATCH_BOOL, C_SET_TRANSFORM, C_SET, C_REPLACE, C_AXPY, C_BIN_REL_ERR, C_BIN_MIN_ABS_REL_ERR };
 enum CondReduceKind : int { CR_COUNT, CR_FIRST, CR_LAST };
 struct CondParams {
   int mode = 0;

@@ -653,8 +653,10 @@ static PairwiseKind pairwiseKind(int opNum) {
     case 22: return P_SAFE_DIVIDE; case 23: return P_MOD; case 27: return P_LOGICAL_OR; case 28: return P_LOGICAL_XOR;
     case 29: return P_LOGICAL_NOT; case 30: return P_LOGICAL_AND; case 34: return P_AMAX; case 35: return P_AMIN;
     case 36: return P_TRUNCATE_MOD; case 37: return P_REPLACE_NANS; case 38: return P_DIVIDE_NO_NAN;
-    // 12/13 CompareAndSet / CompareAndReplace are served before this table is consulted; 10 Axpy, 24-26 relative errors and
-    // 31 PowDerivative read extra parameters and 32/33 LogPoissonLoss, 39/40 IGamma* are not implemented
+    case 24: return P_REL_ERR; case 31: return P_POW_DERIV; case 32: return P_LOG_POISSON; case 33: return P_LOG_POISSON_FULL;
+    case 39: return P_IGAMMA; case 40: return P_IGAMMAC;
+    // 10 Axpy, 12/13 CompareAndSet / CompareAndReplace and 25/26 the thresholded relative errors read extraParams and are
+    // served before this table is consulted
     default: ND4J_THROW("execPairwiseTransform: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
 }
@@ -670,6 +672,19 @@ void execPairwiseTransform(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray 
     EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo(), y->shapeInfo()});
     prepareSpecialUse({z}, {x, y});
     launchCondElementwise(execStream(), opNum == 12 ? C_SET : C_REPLACE, c, y->dataType(), z->dataType(), x->specialBuffer(), y->specialBuffer(), z->specialBuffer(), p, 0.0, false);
+    registerSpecialUse({z}, {x, y});
+    return;
+  }
+  if (opNum == 10 || opNum == 25 || opNum == 26) {   // Axpy [alpha], BinaryRelativeError [threshold], BinaryMinimumAbsoluteRelativeError [rel, abs]
+    ND4J_REQUIRE(isFloatType(z->dataType()) && x->dataType() == z->dataType() && y->dataType() == z->dataType(), "execPairwiseTransform: Axpy and the thresholded relative errors take float arrays of one type here");
+    if (z->isEmpty()) return;
+    const auto v = fetchParams("execPairwiseTransform", extraParams, z->dataType(), opNum == 26 ? 2 : 1);
+    CondParams c;
+    c.compare = v[0]; c.set = opNum == 26 ? v[1] : 0.0; c.eps = 0.0; c.mode = 0; c.xdt = (int)z->dataType();
+    EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo(), y->shapeInfo()});
+    prepareSpecialUse({z}, {x, y});
+    launchCondElementwise(execStream(), opNum == 10 ? C_AXPY : opNum == 25 ? C_BIN_REL_ERR : C_BIN_MIN_ABS_REL_ERR, c, y->dataType(), z->dataType(), x->specialBuffer(),
+                          y->specialBuffer(), z->specialBuffer(), p, 0.0, false);
     registerSpecialUse({z}, {x, y});
     return;
   }
@@ -762,7 +777,7 @@ void execScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueN
     case 38: k = P_LOG_X; break; case 39: k = P_RELU; break; case 40: k = P_RELU6; break; case 41: k = P_STEP; break;
     case 42: k = P_LSTM_CLIP; break; case 43: k = P_TRUNCATE_MOD; break; case 45: k = P_REVERSE_POW; break;
     case 46: k = P_DIVIDE_NO_NAN; break; case 49: k = P_RELU_D; break;
-    // 33 CompareAndSet is served above; 32 PowDerivative reads an extra parameter and 47/48 IGamma* are not implemented
+    case 32: k = P_POW_DERIV; break; case 47: k = P_IGAMMA; break; case 48: k = P_IGAMMAC; break;   // 33 CompareAndSet is served above
     default: ND4J_THROW("execScalar: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
   if (z->isEmpty()) return;

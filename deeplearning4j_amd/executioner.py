@@ -25,6 +25,8 @@ class Pairwise:
     ReverseMod, SafeDivide, Mod, LogicalOr, LogicalXor, LogicalNot, LogicalAnd = 21, 22, 23, 27, 28, 29, 30
     AMaxPairwise, AMinPairwise, TruncateMod, ReplaceNans, DivideNoNan = 34, 35, 36, 37, 38
     CompareAndSet, CompareAndReplace = 12, 13   # extraArgs [compare, set, eps, mode]
+    Axpy, RelativeError, BinaryRelativeError, BinaryMinimumAbsoluteRelativeError = 10, 24, 25, 26   # extraArgs [alpha] / - / [threshold] / [relative, absolute]
+    PowDerivative, LogPoissonLoss, LogPoissonLossFull, IGamma, IGammac = 31, 32, 33, 39, 40
 
 
 class TransformStrict:
@@ -89,6 +91,7 @@ class Scalar:
     SXELogitsSmoother, LeakyRELU, LeakyRELUDerivative, ReplaceNans, LogX, RELU, RELU6, Step, LstmClip = 34, 35, 36, 37, 38, 39, 40, 41, 42
     TruncateMod, SquaredReverseSubtract, ReversePow, DivideNoNan, RELUDerivative = 43, 44, 45, 46, 49
     CompareAndSet = 33   # extraArgs [compare, set, eps, mode]
+    PowDerivative, IGamma, IGammac = 32, 47, 48
 
 
 class Broadcast:

@@ -67,6 +67,11 @@
  *   equals_with_eps (oracle.py, numpy)  NDArrayTests2.cpp:96-103 (FirstIndex), BooleanIndexingTest.java:208-335
  *                                       (CompareAndSet / CompareAndReplace / MatchCondition cases), closed forms
  *                                       (tests/test_oracle_cond_ops.py)
+ *   remaining pairwise / scalar ops
+ *   (oracle.py, numpy) ................ igamma / igammac: DeclarableOpsTests10.cpp:481-515 and scipy.special.gammainc (exact for
+ *                                       x < 1, within the truncation of the reference's series beyond); relative errors, axpy,
+ *                                       pow_derivative, log_poisson_loss: closed forms, central differences, Stirling's bound
+ *                                       (tests/test_oracle_pairwise_params.py)
  *   integer arrays .................... no restatement: the GPU tests compare with numpy's integer arithmetic directly
  */
 #ifndef ND4J_ORACLE_H

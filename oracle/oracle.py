@@ -549,3 +549,78 @@ def equals_with_eps(x, y, eps, dims=None):
     rx, shape = _along(np.asarray(x, dtype=np.float64), dims)
     ry, _ = _along(np.asarray(y, dtype=np.float64), dims)
     return (np.abs(rx - ry) <= eps).all(1).astype(np.float64).reshape(shape)
+
+
+# ---- the remaining pairwise / scalar ops (numpy restatements, arithmetic in the array's type) --------------------------------
+def relative_error(x, y):
+    """sd_re (math/templatemath.h:1144-1153): |x - y| / (|x| + |y|), 0 where both are 0.  Pairwise 24 RelativeError."""
+    x = np.asarray(x)
+    y = np.asarray(y, dtype=x.dtype)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        r = (np.abs(x - y) / (np.abs(x) + np.abs(y))).astype(x.dtype)
+    return np.where((x == 0) & (y == 0), x.dtype.type(0), r)
+
+
+def binary_relative_error(x, y, threshold):
+    """Pairwise 25 (ops/ops.h:2218-2270): 1 where the relative error exceeds the threshold."""
+    x = np.asarray(x)
+    return (relative_error(x, y) > _in_type(threshold, x)).astype(x.dtype)
+
+
+def binary_min_abs_relative_error(x, y, rel, absolute):
+    """Pairwise 26 (ops/ops.h:2274-2340): 1 where the relative error exceeds `rel` and |x - y| is not below `absolute`."""
+    x = np.asarray(x)
+    y = np.asarray(y, dtype=x.dtype)
+    return ((relative_error(x, y) > _in_type(rel, x)) & ~(np.abs(x - y) < _in_type(absolute, x))).astype(x.dtype)
+
+
+def axpy(x, y, alpha):
+    """Pairwise 10 (ops/ops.h:328-333): alpha * x + y."""
+    x = np.asarray(x)
+    return (_in_type(alpha, x) * x + np.asarray(y, dtype=x.dtype)).astype(x.dtype)
+
+
+def pow_derivative(x, y):
+    """Pairwise 31 / Scalar 32 (ops/ops.h:82-87): y * x^(y - 1)."""
+    x = np.asarray(x)
+    y = np.broadcast_to(np.asarray(y, dtype=x.dtype), x.shape)
+    with np.errstate(all="ignore"):
+        return (y * np.power(x, y - x.dtype.type(1))).astype(x.dtype)
+
+
+def log_poisson_loss(x, y, full=False):
+    """Pairwise 32 / 33 (ops/ops.h:2389-2394, 1494-1502): exp(y) - x y, `full` adds Stirling's x log x - x + log(2 pi x) / 2."""
+    x = np.asarray(x)
+    y = np.asarray(y, dtype=x.dtype)
+    with np.errstate(all="ignore"):
+        r = np.exp(y) - x * y
+        if full:
+            r = r + (x * np.log(x) - x + x.dtype.type(0.5) * np.log(x.dtype.type(2.0 * np.pi) * x))
+    return r.astype(x.dtype)
+
+
+def igamma(a, x, complement=False):
+    """sd_igamma / sd_igammac (math/templatemath.h:963-991): the regularised lower incomplete gamma function summed as
+    x^a e^-x / Gamma(a) * sum_i x^i / (a (a+1) .. (a+i)), the series cut off once the running denominator passes 1e12;
+    0 where a <= 1e-6.  Evaluated in the array's type (float for float32, double for float64)."""
+    import math
+    a = np.asarray(a)
+    dt = a.dtype.type
+    x = np.broadcast_to(np.asarray(x, dtype=a.dtype), a.shape)
+    out = np.zeros(a.shape, a.dtype)
+    for idx in np.ndindex(a.shape):
+        av, xv = dt(a[idx]), dt(x[idx])
+        if av <= dt(0.000001):
+            r = dt(0)
+        else:
+            with np.errstate(all="ignore"):
+                aim = dt(np.power(xv, av) / (np.exp(xv) * dt(math.gamma(float(av)))))
+                s, denom, xi, i = dt(0), dt(1), dt(1), 0
+                while dt(1) / denom > dt(1.0e-12) and i < 4096:
+                    denom = dt(denom * dt(av + dt(i)))
+                    s = dt(s + xi / denom)
+                    xi = dt(xi * xv)
+                    i += 1
+                r = dt(aim * s)
+        out[idx] = dt(1) - r if complement else r
+    return out
