@@ -111,7 +111,9 @@ enum MiscReduceKind : int {
   // two-operand reductions (reduce3), z in a float type
   M3_MANHATTAN, M3_EUCLIDEAN, M3_COSINE_SIMILARITY, M3_DOT, M3_COSINE_DISTANCE, M3_JACCARD, M3_HAMMING,
   M3_EQUALS_EPS,   // 1 when |x - y| <= param everywhere, else 0 (Reduce3 EqualsWithEps)
-  M_NORMP          // (sum |x|^param)^(1 / param), z in a float type (ReduceFloat NormP); not a two-operand kind
+  M_NORMP,         // (sum |x|^param)^(1 / param), z in a float type (ReduceFloat NormP); not a two-operand kind
+  // ReduceBool 2-7: 1 when any element is finite / inf or nan / nan / inf / positive / negative (sum of indicators, ops.h:1139-1163)
+  M_ANY_FINITE, M_ANY_INF_OR_NAN, M_ANY_NAN, M_ANY_INF, M_ANY_POSITIVE, M_ANY_NEGATIVE
 };
 
 // outer = kept dims (one output element each), inner = reduced dims

@@ -830,7 +830,7 @@ void execBroadcast(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, Opaq
     case 19: k = P_FLOOR_DIV; break; case 20: k = P_REVERSE_MOD; break; case 21: k = P_SAFE_DIVIDE; break; case 22: k = P_MOD; break;
     case 23: k = P_TRUNCATE_DIV; break; case 26: k = P_ATAN2; break; case 27: k = P_LOGICAL_OR; break; case 28: k = P_LOGICAL_XOR; break;
     case 29: k = P_LOGICAL_NOT; break; case 30: k = P_LOGICAL_AND; break; case 31: k = P_DIVIDE_NO_NAN; break;
-    // 32/33 IGamma* and 34 PowDerivative are not implemented
+    case 32: k = P_IGAMMA; break; case 33: k = P_IGAMMAC; break; case 34: k = P_POW_DERIV; break;
     default: ND4J_THROW("execBroadcast: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
   if (z->isEmpty()) return;
@@ -1054,7 +1054,8 @@ static void reduceBool(const char* fn, int opNum, OpaqueNDArray xa, OpaqueNDArra
   ND4J_REQUIRE(z->dataType() == BOOL, std::string("NativeOpExecutioner::execReduceBool requires Z operand to have BOOL type, got ") + dtypeName(z->dataType()));
   MiscReduceKind k;
   switch (opNum) {  // loops/legacy_ops.h:97-98
-    case 0: k = M_ANY; break; case 1: k = M_ALL; break;
+    case 0: k = M_ANY; break; case 1: k = M_ALL; break; case 2: k = M_ANY_FINITE; break; case 3: k = M_ANY_INF_OR_NAN; break;
+    case 4: k = M_ANY_NAN; break; case 5: k = M_ANY_INF; break; case 6: k = M_ANY_POSITIVE; break; case 7: k = M_ANY_NEGATIVE; break;
     default: ND4J_THROW(std::string(fn) + ": opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
   runReduceMisc(fn, k, x, z, da ? hostDims(da, x->rankOf(), fn) : std::vector<LongType>{}, false);

@@ -389,6 +389,7 @@ __device__ __forceinline__ double misc_result(const MiscArgs& a, double n, doubl
       return a.kind == M_STDDEV ? sqrt(var) : var;
     }
     case M_ANY: return cnt > 0.0 ? 1.0 : 0.0;                     // ops.h:1200-1206: the sum of the elements is positive
+    case M_ANY_FINITE: case M_ANY_INF_OR_NAN: case M_ANY_NAN: case M_ANY_INF: case M_ANY_POSITIVE: case M_ANY_NEGATIVE: return cnt > 0.0 ? 1.0 : 0.0;
     case M_ALL: return cnt > 0.0 ? 0.0 : 1.0;                     // here cnt counts the zero elements
     // reduce3 (ops.h:117-134,483-541): mean = first sum, m2 and cnt = the two auxiliary sums
     case M3_MANHATTAN: case M3_DOT: return mean;
@@ -415,7 +416,7 @@ __global__ __launch_bounds__(256) void misc_partial(MiscArgs a, const void* __re
   const LongType st = linear ? a.inner.stride[0] : 0;
   auto at = [&](LongType q) { return load_any(x, a.xdt, base + (linear ? q * st : walk<LongType>(a.inner, q))); };
   double n = (double)(j1 - j0), mean = 0.0, m2 = 0.0, cnt = 0.0;
-  if (a.kind >= M3_MANHATTAN && a.kind != M_NORMP) {
+  if (a.kind >= M3_MANHATTAN && a.kind < M_NORMP) {
     const LongType ybase = walk<LongType>(a.yOuter, row);
     const bool ylinear = a.yInner.rank == 1;
     const LongType yst = ylinear ? a.yInner.stride[0] : 0;
@@ -447,6 +448,12 @@ __global__ __launch_bounds__(256) void misc_partial(MiscArgs a, const void* __re
       if (a.kind == M_NORMP) c += pow(fabs(v), a.param);
       else if (a.kind == M_COUNT_NONZERO) c += v == 0.0 ? 0.0 : 1.0;         // ops.h:1180-1188
       else if (a.kind == M_COUNT_ZERO || a.kind == M_ALL) c += v == 0.0 ? 1.0 : 0.0;   // ops.h:1190-1198,1208-1215
+      else if (a.kind >= M_ANY_FINITE) {                               // ops.h:1139-1163, indicator of the element
+        const bool nan = v != v, inf = !nan && (v - v) != (v - v);
+        const bool hit = a.kind == M_ANY_FINITE ? !(nan || inf) : a.kind == M_ANY_INF_OR_NAN ? (nan || inf) : a.kind == M_ANY_NAN ? nan
+                         : a.kind == M_ANY_INF ? inf : a.kind == M_ANY_POSITIVE ? v > 0.0 : v < 0.0;
+        c += hit ? 1.0 : 0.0;
+      }
       else c += v;                                                     // Any
     }
     cnt = block_sum(c, lds);
@@ -466,7 +473,7 @@ __global__ __launch_bounds__(256) void misc_finish(MiscArgs a, const double* __r
   for (int s = 0; s < a.splits; s++) {
     const double* p = partials + (row * a.splits + s) * 4;
     const double nb = p[0];
-    if (a.kind >= M3_MANHATTAN && a.kind != M_NORMP) { n += nb; mean += p[1]; m2 += p[2]; cnt += p[3]; continue; }
+    if (a.kind >= M3_MANHATTAN && a.kind < M_NORMP) { n += nb; mean += p[1]; m2 += p[2]; cnt += p[3]; continue; }
     if (nb > 0.0) {
       const double delta = p[1] - mean, tot = n + nb;
       m2 += p[2] + delta * delta * n * nb / tot;
@@ -483,7 +490,7 @@ void launchReduceMisc(hipStream_t st, MiscReduceKind k, DataType xdt, DataType z
   MiscArgs a;
   a.param = param;
   a.outer = p.outer; a.inner = p.inner; a.zOuter = p.zOuter;
-  ND4J_REQUIRE((k >= M3_MANHATTAN && k != M_NORMP) == (y != nullptr && yPlan != nullptr), "reduce: second operand mismatch");
+  ND4J_REQUIRE((k >= M3_MANHATTAN && k < M_NORMP) == (y != nullptr && yPlan != nullptr), "reduce: second operand mismatch");
   if (yPlan) {
     ND4J_REQUIRE(yPlan->outerLen == p.outerLen && yPlan->innerLen == p.innerLen, "reduce3: operands must have equal shapes");
     a.yOuter = yPlan->outer; a.yInner = yPlan->inner;

@@ -81,7 +81,7 @@ class ReduceLong:
 
 
 class ReduceBool:
-    Any, All = 0, 1
+    Any, All, IsFinite, IsInfOrNan, IsNan, IsInf, IsPositive, IsNegative = 0, 1, 2, 3, 4, 5, 6, 7   # 2-7: true when any element is
 
 
 class Scalar:
@@ -98,6 +98,7 @@ class Broadcast:
     Add, Subtract, Multiply, Divide, ReverseDivide, ReverseSubtract, CopyPws, Pow = 0, 1, 2, 3, 4, 5, 6, 7
     MinPairwise, MaxPairwise, AMinPairwise, AMaxPairwise, SquaredSubtract, FloorMod, FloorDiv, ReverseMod = 13, 14, 15, 16, 17, 18, 19, 20
     SafeDivide, Mod, TruncateDiv, Atan2, LogicalOr, LogicalXor, LogicalNot, LogicalAnd, DivideNoNan = 21, 22, 23, 26, 27, 28, 29, 30, 31
+    IGamma, IGammac, PowDerivative = 32, 33, 34
 
 
 def _reduced_shape(shape, dims, keep_dims):

@@ -102,3 +102,36 @@ def test_igamma_against_the_restatement(ex, dt, tol):
     np.testing.assert_allclose(got.astype(np.float64), O.igamma(a, 1.5).astype(np.float64), rtol=tol, atol=tol * 1e-3)
     got = ex.exec_scalar(Scalar.IGammac, A, 1.5).to_numpy()
     np.testing.assert_allclose(got.astype(np.float64), O.igamma(a, 1.5, complement=True).astype(np.float64), rtol=tol, atol=tol)
+
+
+def test_broadcast_igamma_and_pow_derivative(ex):
+    """Broadcast 32-34: the same functors with a row of second operands (the reference's IGamma_Test1 shape)."""
+    from deeplearning4j_amd.executioner import Broadcast
+    a = np.array([1.1, 2.1, 3.1, 4.1, 5.1, 6.1, 7.1, 8.1, 9.1, 10.1, 11.1, 12.1]).reshape(3, 4)
+    x = np.array([1.2, 2.2, 3.2, 4.2])
+    want = np.array([0.659917, 0.61757898, 0.59726304, 0.58478117, 0.0066205109, 0.022211598, 0.040677428, 0.059117373,
+                     0.0000039433403, 0.000086064574, 0.000436067, 0.0012273735]).reshape(3, 4)
+    A, X = NDArray.from_numpy(a), NDArray.from_numpy(x)
+    np.testing.assert_allclose(ex.exec_broadcast(Broadcast.IGamma, A, X, [1]).to_numpy(), want, rtol=2e-5)
+    np.testing.assert_allclose(ex.exec_broadcast(Broadcast.IGammac, A, X, [1]).to_numpy(), 1 - O.igamma(a, np.broadcast_to(x, a.shape)), rtol=1e-10)
+    np.testing.assert_allclose(ex.exec_broadcast(Broadcast.PowDerivative, A, X, [1]).to_numpy(), x * a ** (x - 1), rtol=1e-12)
+
+
+@pytest.mark.parametrize("dt", [DOUBLE, FLOAT32, HALF])
+def test_reduce_bool_predicates(ex, dt):
+    """ReduceBool 2-7 (ops/ops.h:1139-1163): true where any element of the sub-array is finite / inf or nan / nan / inf /
+    positive / negative."""
+    from deeplearning4j_amd.executioner import ReduceBool
+    x = np.zeros((6, 40), NP[dt])
+    x[1, 3] = np.nan
+    x[2, 7] = -np.inf
+    x[3, :] = np.nan            # nothing finite
+    x[4, 11] = 2.0
+    x[5, 39] = -0.5
+    X = NDArray.from_numpy(x)
+    fin = np.isfinite(x)
+    want = {ReduceBool.IsFinite: fin.any(1), ReduceBool.IsInfOrNan: (~fin).any(1), ReduceBool.IsNan: np.isnan(x).any(1),
+            ReduceBool.IsInf: np.isinf(x).any(1), ReduceBool.IsPositive: (x > 0).any(1), ReduceBool.IsNegative: (x < 0).any(1)}
+    for op, w in want.items():
+        assert np.array_equal(ex.exec_reduce_bool(op, X, [1]).to_numpy(), w), op
+        assert bool(ex.exec_reduce_bool(op, X).to_numpy()) == bool(w.any()), op
