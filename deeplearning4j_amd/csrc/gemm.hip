@@ -1321,6 +1321,76 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32q(GemmArgs g, const f
   for (int u = 0; u < PD; u++) load(u, (LongType)u * BK);
   store(0, 0);
   __syncthreads();
+  // One small tile per CU (one wave per SIMD, one accumulator per wave): nothing covers an LDS round trip, so the
+  // fragments of K-tile kt + 1 are read right after the barrier that completes its stage, under the MFMAs of K-tile kt
+  // (the same arrangement as gemm_mfma16q).  The larger tile keeps the plain order, which is already MFMA-bound.
+  constexpr bool EARLY = TM * TN == 1;
+  if constexpr (EARLY) {
+    float fa[2][BK / 2][TM], fb[2][BK / 2][TN];
+    f32x16 acc2[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc2[i][j][r] = 0.f;
+    auto readTile = [&](int stage, int buf) {
+#pragma unroll
+      for (int ks = 0; ks < BK / 2; ks++) {
+        const int k = ks * 2 + (lane >> 5);
+#pragma unroll
+        for (int i = 0; i < TM; i++) fa[buf][ks][i] = sA[stage][k * PA + wm * WTM + i * 32 + (lane & 31)];
+#pragma unroll
+        for (int j = 0; j < TN; j++) fb[buf][ks][j] = sB[stage][k * PB + wn * WTN + j * 32 + (lane & 31)];
+      }
+    };
+    readTile(0, 0);
+    for (LongType kt0 = 0; kt0 < KT; kt0 += PD) {
+#pragma unroll
+      for (int u = 0; u < PD; u++) {
+        const LongType kt = kt0 + u;
+        const int cur = u & 1;
+        const LongType nx = kt + PD < KT ? kt + PD : KT - 1;
+        // even and odd k-steps go to two accumulators: with a single one every MFMA would wait for the previous one's result
+        auto mfmas = [&](int from, int to) {
+#pragma unroll
+          for (int ks = from; ks < to; ks++)
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+              for (int j = 0; j < TN; j++) {
+                if (ks & 1) acc2[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][ks][i], fb[cur][ks][j], acc2[i][j], 0, 0, 0);
+                else acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][ks][i], fb[cur][ks][j], acc[i][j], 0, 0, 0);
+              }
+        };
+        // the wave's own bookkeeping for K-tile kt + 1 is issued between the MFMAs of K-tile kt (64 cycles of matrix pipe
+        // each): left in front of them it ran while the pipe stood still, 200 cycles for every 512 of MFMA
+        mfmas(0, 1);
+        store((u + 1) % PD, cur ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfmas(1, 2);
+        load(u, nx * BK);
+        __builtin_amdgcn_sched_barrier(0);
+        mfmas(2, 4);
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        mfmas(4, 5);
+        readTile(cur ^ 1, cur ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfmas(5, BK / 2);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[i][j][r] += acc2[i][j][r];
+    storeAccTiles<float, TM, TN, false>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
+    return;
+  }
   for (LongType kt0 = 0; kt0 < KT; kt0 += PD) {
 #pragma unroll
     for (int u = 0; u < PD; u++) {
