@@ -1111,11 +1111,17 @@ static bool launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const 
   static const bool direct = getenv("ND4JHIP_GEMM_DIRECT") ? atoi(getenv("ND4JHIP_GEMM_DIRECT")) != 0 : true;
   static const bool ring = getenv("ND4JHIP_GEMM_RING") ? atoi(getenv("ND4JHIP_GEMM_RING")) != 0 : true;
   if constexpr (A_KC && !B_KC) {
-    if (direct && ring && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 128 == 0) {
-      constexpr size_t LDS = (3 * 256 * 8 + 4 * 32 * 32) * 16;   // 160 KiB: the whole LDS of a CU
-      auto kern = gemm_mfma16r<T>;
-      static std::once_flag attrOnce;
-      std::call_once(attrOnce, [&] { HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS)); });
+    constexpr size_t LDS = (3 * 256 * 8 + 4 * 32 * 32) * 16;   // 160 KiB: the whole LDS of a CU
+    auto kern = gemm_mfma16r<T>;
+    // a device or driver that does not grant a block the whole LDS keeps the two-stage kernel below
+    static std::once_flag attrOnce;
+    static bool ringGranted = false;
+    if (direct && ring && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 128 == 0)
+      std::call_once(attrOnce, [&] {
+        ringGranted = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS) == hipSuccess;
+        if (!ringGranted) (void)hipGetLastError();
+      });
+    if (direct && ring && ringGranted && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 128 == 0) {
       const unsigned tM = (unsigned)(g.M / 256), tN = (unsigned)(g.N / 256);
       noteKernel("gemm_mfma16r<%s,256x256,akc=1,bkc=0>", tname<T>());
       hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(512), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
