@@ -410,6 +410,8 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
   // U: load instructions in flight per operand and wave (8, which covers a 1024-key history in one trip to memory when 16
   // waves share it, measured slower than 4: 0.36 against 0.34 ms per decode step)
   __shared__ float sm[NW][D + 2];
+  __shared__ __attribute__((aligned(16))) float so[NW][64 / (D / 8)][D];   // per wave: one partial output row per lane group
+  typedef __attribute__((ext_vector_type(4))) float f32x4s;
   const LongType b = blockIdx.x, qi = blockIdx.y;
   if (a.H > 0) {
     const LongType hi = b / a.H, lo = b - hi * a.H;
@@ -423,20 +425,24 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
   // the query row was written by the kernel before this one and the first keys come cold from HBM: all of these loads
   // are issued before the first value is touched, so the two latencies overlap
   const typename RawIO<T>::raw qraw = *reinterpret_cast<const typename RawIO<T>::raw*>(Q + qi * a.qT + c * 8);
-  typename RawIO<T>::raw kr[U], vr[U];
-  bool valid[U];
-  auto issue = [&](LongType k0) {
+  using Raw = typename RawIO<T>::raw;
+  // (a second register set, so that the next trip's loads fly while the current one is consumed, changed nothing at
+  // batch 1 and cost 1 % at batch 32: a block's stream is bound by what one CU can pull, not by a trip's latency)
+  Raw krA[U], vrA[U];
+  bool validA[U];
+  auto issue = [&](LongType k0, Raw (&kr)[U], Raw (&vr)[U], bool (&valid)[U]) {
 #pragma unroll
     for (int u = 0; u < U; u++) {
       LongType key = k0 + u * KPS + g;
       valid[u] = key < a.Tv;
       key = valid[u] ? key : a.Tv - 1;
-      kr[u] = *reinterpret_cast<const typename RawIO<T>::raw*>(K + key * a.kT + c * 8);
-      vr[u] = *reinterpret_cast<const typename RawIO<T>::raw*>(V + key * a.vT + c * 8);
+      kr[u] = *reinterpret_cast<const Raw*>(K + key * a.kT + c * 8);
+      vr[u] = *reinterpret_cast<const Raw*>(V + key * a.vT + c * 8);
     }
   };
+  const LongType step = (LongType)NW * (KPS * U);
   LongType k0 = (LongType)wave * (KPS * U);
-  if (k0 < a.Tv) issue(k0);
+  if (k0 < a.Tv) issue(k0, krA, vrA, validA);
   float q[8];
   RawIO<T>::unpack(qraw, q);
   const float L2E = 1.44269502162933349609375f;
@@ -444,7 +450,7 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
 #pragma unroll
   for (int e = 0; e < 8; e++) o[e] = 0.f;
 
-  while (k0 < a.Tv) {
+  auto consume = [&](LongType k0, const Raw (&kr)[U], const Raw (&vr)[U], const bool (&valid)[U]) {
     float sc[U], tmax = m;
 #pragma unroll
     for (int u = 0; u < U; u++) {
@@ -453,8 +459,12 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
       float d = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; e++) d = __builtin_fmaf(q[e], kf[e], d);
-#pragma unroll
-      for (int sh = 1; sh < CH; sh <<= 1) d += __shfl_xor(d, sh, WAVE);
+      // butterfly over the CH lanes of the key row, one DPP add per level (the same pairs in the same order as an
+      // exchange with lane ^ 1, ^ 2, ^ 4, ^ 8: after two levels a quad holds one value, so a mirror is an exchange)
+      d += dpp_f<0xB1>(d);                 // quad_perm [1,0,3,2]
+      d += dpp_f<0x4E>(d);                 // quad_perm [2,3,0,1]
+      d += dpp_f<0x141>(d);                // row_half_mirror
+      if (CH > 8) d += dpp_f<0x140>(d);    // row_mirror
       if (a.applyScale) d *= a.scale;
       d = __builtin_fminf(__builtin_fmaxf(d, -1.0e4f), 1.0e4f);
       d = round_storage<T>(d);
@@ -479,28 +489,35 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
 #pragma unroll
       for (int e = 0; e < 8; e++) o[e] = __builtin_fmaf(p, vf[e], o[e]);
     }
-    k0 += (LongType)NW * (KPS * U);
-    if (k0 < a.Tv) issue(k0);
+  };
+  while (k0 < a.Tv) {
+    consume(k0, krA, vrA, validA);
+    k0 += step;
+    if (k0 < a.Tv) issue(k0, krA, vrA, validA);
   }
-  // merge the lane groups of the wave (lanes with equal c): bring every state to the common maximum, then add
-  float mAll = m;
-#pragma unroll
-  for (int sh = CH; sh < 64; sh <<= 1) mAll = __builtin_fmaxf(mAll, __shfl_xor(mAll, sh, WAVE));
+  // merge the lane groups of the wave (lanes with equal c): bring every state to the wave's maximum, then add.  Max and
+  // sum of l run on DPP; the eight-float partial rows go through the wave's own LDS region, where lane d sums element d
+  // of every group -- exchanging them lane to lane instead (nine values, three levels of cross-lane permutes per wave)
+  // kept the LDS crossbar of the one CU a sixteen-wave block runs on busy for 2 us, half the kernel.
+  constexpr int G = 64 / CH;   // lane groups per wave
+  const float mAll = wave_allreduce<MaxOp>(m);
   const float f = __builtin_amdgcn_exp2f((m - mAll) * L2E);
-  l *= f;
-#pragma unroll
-  for (int e = 0; e < 8; e++) o[e] *= f;
-#pragma unroll
-  for (int sh = CH; sh < 64; sh <<= 1) {
-    l += __shfl_xor(l, sh, WAVE);
-#pragma unroll
-    for (int e = 0; e < 8; e++) o[e] += __shfl_xor(o[e], sh, WAVE);
+  // the CH lanes of a group hold one l: the wave sum counts it CH times (a power of two, so the division is exact)
+  const float lAll = wave_allreduce<SumOp>(l * f) * (1.0f / CH);
+  {
+    float* mine = &so[wave][g][c * 8];
+    *reinterpret_cast<f32x4s*>(mine) = f32x4s{o[0] * f, o[1] * f, o[2] * f, o[3] * f};
+    *reinterpret_cast<f32x4s*>(mine + 4) = f32x4s{o[4] * f, o[5] * f, o[6] * f, o[7] * f};
   }
-  if (g == 0) {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave reads what its own lanes wrote: no barrier needed
 #pragma unroll
-    for (int e = 0; e < 8; e++) sm[wave][c * 8 + e] = o[e];
-    if (c == 0) { sm[wave][D] = mAll; sm[wave][D + 1] = l; }
+  for (int part = 0; part < D / 64; part++) {
+    float acc = 0.f;
+#pragma unroll
+    for (int gg = 0; gg < G; gg++) acc += so[wave][gg][part * 64 + lane];
+    sm[wave][part * 64 + lane] = acc;
   }
+  if (lane == 0) { sm[wave][D] = mAll; sm[wave][D + 1] = lAll; }
   __syncthreads();
   if (t < D) {
     float mm = -1.0e30f;
