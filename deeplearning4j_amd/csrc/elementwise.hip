@@ -340,7 +340,7 @@ __device__ __forceinline__ void st_stream(VT* p, const VT& v) {
   else *p = v;
 }
 
-template <typename F, typename T, bool NT>
+template <typename F, typename T, bool NT, bool NTS>
 __global__ __launch_bounds__(EW_BLOCK) void unary_contig(const T* __restrict__ x, T* __restrict__ z, LongType n) {
   constexpr int V = 16 / sizeof(T);
   using IO = RawIO<T>;
@@ -354,14 +354,14 @@ __global__ __launch_bounds__(EW_BLOCK) void unary_contig(const T* __restrict__ x
     IO::unpack(r, vals);
 #pragma unroll
     for (int e = 0; e < V; e++) vals[e] = sizeof(T) == 2 ? F::template applyLow<A>(vals[e]) : F::template apply<A>(vals[e]);
-    st_stream<NT>(reinterpret_cast<RT*>(z) + i, IO::pack(vals));
+    st_stream<NTS>(reinterpret_cast<RT*>(z) + i, IO::pack(vals));
   }
   // scalar tail (fewer than V elements)
   const LongType tail = nvec * V + i;
   if (tail < n) z[tail] = Conv<T>::from(F::template apply<A>((A)to_float(x[tail])));
 }
 
-template <typename F, typename T, bool NT>
+template <typename F, typename T, bool NT, bool NTS>
 __global__ __launch_bounds__(EW_BLOCK) void pairwise_contig(const T* __restrict__ x, const T* __restrict__ y,
                                                             T* __restrict__ z, LongType n) {
   constexpr int V = 16 / sizeof(T);
@@ -378,7 +378,7 @@ __global__ __launch_bounds__(EW_BLOCK) void pairwise_contig(const T* __restrict_
     IO::unpack(rb, b);
 #pragma unroll
     for (int e = 0; e < V; e++) a[e] = F::template apply<A>(a[e], b[e]);
-    st_stream<NT>(reinterpret_cast<RT*>(z) + i, IO::pack(a));
+    st_stream<NTS>(reinterpret_cast<RT*>(z) + i, IO::pack(a));
   }
   const LongType tail = nvec * V + i;
   if (tail < n) z[tail] = Conv<T>::from(F::template apply<A>((A)to_float(x[tail]), (A)to_float(y[tail])));
@@ -532,7 +532,12 @@ static int gridFor(LongType work, int perBlock) {
   return (int)blocks;
 }
 // does a kernel's total traffic exceed what the last-level cache (256 MB) can usefully hold
-static bool streamsPastCache(size_t bytes) { return bytes > (size_t)288 << 20; }
+// Which accesses of a dense streaming op are non-temporal, by the bytes it moves (measured cold, over rotating operand sets,
+// on 50 MB - 270 MB transforms): 0 = none below 8 MiB; 2 = stores only up to the size of the last-level cache -- written
+// with ordinary stores the output sits dirty in L2 until the kernel ends and is flushed then, which the next launch waits
+// for (gelu bf16 [16,1024,768]: 10.8 -> 8.5 us per launch; a consumer that reads the result right away loses 3 % to it);
+// 3 = loads and stores for what cannot stay in the cache anyway.
+static int streamPolicy(size_t bytes) { return bytes > ((size_t)288 << 20) ? 3 : bytes >= ((size_t)8 << 20) ? 2 : 0; }
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 template <typename F2, typename T, int NIN>
@@ -568,8 +573,10 @@ static void unaryTyped(hipStream_t s, const EwPlan& p, const void* x, void* z) {
   if (p.contiguous && aligned16(x) && aligned16(z)) {
     constexpr int V = 16 / sizeof(T);
     const unsigned grid = (unsigned)((p.length / V + EW_BLOCK) / EW_BLOCK);
-    if (streamsPastCache(2 * sizeof(T) * (size_t)p.length)) hipLaunchKernelGGL((unary_contig<Unary<K>, T, true>), dim3(grid), dim3(EW_BLOCK), 0, s, xt, zt, p.length);
-    else hipLaunchKernelGGL((unary_contig<Unary<K>, T, false>), dim3(grid), dim3(EW_BLOCK), 0, s, xt, zt, p.length);
+    const int nt = streamPolicy(2 * sizeof(T) * (size_t)p.length);
+    if (nt == 3) hipLaunchKernelGGL((unary_contig<Unary<K>, T, true, true>), dim3(grid), dim3(EW_BLOCK), 0, s, xt, zt, p.length);
+    else if (nt == 2) hipLaunchKernelGGL((unary_contig<Unary<K>, T, false, true>), dim3(grid), dim3(EW_BLOCK), 0, s, xt, zt, p.length);
+    else hipLaunchKernelGGL((unary_contig<Unary<K>, T, false, false>), dim3(grid), dim3(EW_BLOCK), 0, s, xt, zt, p.length);
   } else {
     launchNd<UnaryAs2<K>, T, 1>(s, p, xt, (const T*)nullptr, zt);
   }
@@ -632,8 +639,10 @@ static void pairwiseTyped(hipStream_t s, const EwPlan& p, const void* x, const v
   if (p.contiguous && aligned16(x) && aligned16(y) && aligned16(z)) {
     constexpr int V = 16 / sizeof(T);
     const unsigned grid = (unsigned)((p.length / V + EW_BLOCK) / EW_BLOCK);
-    if (streamsPastCache(3 * sizeof(T) * (size_t)p.length)) hipLaunchKernelGGL((pairwise_contig<Pairwise<K>, T, true>), dim3(grid), dim3(EW_BLOCK), 0, s, xt, yt, zt, p.length);
-    else hipLaunchKernelGGL((pairwise_contig<Pairwise<K>, T, false>), dim3(grid), dim3(EW_BLOCK), 0, s, xt, yt, zt, p.length);
+    const int nt = streamPolicy(3 * sizeof(T) * (size_t)p.length);
+    if (nt == 3) hipLaunchKernelGGL((pairwise_contig<Pairwise<K>, T, true, true>), dim3(grid), dim3(EW_BLOCK), 0, s, xt, yt, zt, p.length);
+    else if (nt == 2) hipLaunchKernelGGL((pairwise_contig<Pairwise<K>, T, false, true>), dim3(grid), dim3(EW_BLOCK), 0, s, xt, yt, zt, p.length);
+    else hipLaunchKernelGGL((pairwise_contig<Pairwise<K>, T, false, false>), dim3(grid), dim3(EW_BLOCK), 0, s, xt, yt, zt, p.length);
   } else {
     launchNd<Pairwise<K>, T, 2>(s, p, xt, yt, zt);
   }
