@@ -111,3 +111,24 @@ def test_config4_causal_attention(ex, oracle, dt):
         oracle.attention_v2(_oracle_arr(oracle, q[bi:bi + 1], dt), _oracle_arr(oracle, v[bi:bi + 1], dt), _oracle_arr(oracle, k[bi:bi + 1], dt), oo,
                             scale=0.125, causal=True)
         assert_close(out[bi:bi + 1], _as_float(oo), 1e-2, 1e-2, "batch entry %d" % bi)
+
+
+@pytest.mark.parametrize("dt,L,tol", [(BFLOAT16, 768, 1e-2), (HALF, 768, 2e-3), (FLOAT32, 384, 1e-5)])
+@pytest.mark.parametrize("rows,has_bias,pitched", [(4097, True, False), (4608, False, False), (4099, True, True)])
+def test_layer_norm_rows_of_one_and_a_half_passes(ex, oracle, dt, L, tol, rows, has_bias, pitched):
+    """Many rows (two per wave) whose length is one and a half 16-byte wave passes, so that the second pass is half
+    masked: an odd row count (the last wave has a lone row), no bias, and rows at a pitch (the left columns of a wider
+    matrix), every row against the oracle."""
+    rng = np.random.default_rng(rows + L + int(has_bias))
+    width = L + 64 if pitched else L
+    full, Full = _store(rng.normal(0.3, 2.0, (rows, width)).astype(np.float32), dt)
+    x = full[:, :L]
+    X = Full.slice(1, 0, L) if pitched else Full
+    g, G = _store(rng.normal(1, 0.1, L).astype(np.float32), dt)
+    b, B = _store(rng.normal(0, 0.1, L).astype(np.float32), dt)
+    ins = [X, G, B] if has_bias else [X, G]
+    y = ex.exec_custom("layer_norm", ins, i_args=[1], b_args=[False])[0].to_float()
+    oy = _oracle_arr(oracle, np.zeros_like(x), dt)
+    oins = [_oracle_arr(oracle, np.ascontiguousarray(x), dt), _oracle_arr(oracle, g, dt)] + ([_oracle_arr(oracle, b, dt)] if has_bias else [None])
+    oracle.layer_norm(oins[0], oins[1], oins[2], oy, [1], channels_first=False)
+    assert_close(y, _as_float(oy), tol, tol, "layer_norm, %d rows of %d" % (rows, L))
