@@ -113,6 +113,41 @@ def test_config4_causal_attention(ex, oracle, dt):
         assert_close(out[bi:bi + 1], _as_float(oo), 1e-2, 1e-2, "batch entry %d" % bi)
 
 
+@pytest.mark.parametrize("dt", [HALF, BFLOAT16])
+def test_config4_weights_and_logits_outputs(ex, oracle, dt):
+    """The same op with its second and third outputs requested (attention weights and clipped, masked logits) at the
+    config's sequence length: [12, 1024, 64] -> weights and logits [12, 1024, 1024].  Whole-result properties, then two
+    batch entries against the oracle."""
+    rng = np.random.default_rng(4004)
+    B, T, D = 12, 1024, 64
+    q, Q = _store(rng.normal(0, 1, (B, T, D)).astype(np.float32), dt)
+    k, K = _store(rng.normal(0, 1, (B, T, D)).astype(np.float32), dt)
+    v, V = _store(rng.normal(0, 1, (B, T, D)).astype(np.float32), dt)
+    outs = ex.exec_custom("dot_product_attention_v2", [Q, V, K], [NDArray.empty((B, T, D), dt), NDArray.empty((B, T, T), dt), NDArray.empty((B, T, T), dt)],
+                          t_args=[0.125, 0.0], b_args=[True, False])
+    out, w, lg = (o.to_float() for o in outs)
+    # weights: rows are distributions over the keys a query may see (the mask leaves exact zeros)
+    upper = np.triu(np.ones((T, T), bool), 1)
+    assert np.all(w[:, upper] == 0.0) and np.all(w >= 0.0)
+    assert np.abs(w.astype(np.float64).sum(-1) - 1.0).max() < (2e-2 if dt == BFLOAT16 else 3e-3)
+    # logits: the scaled products below the diagonal, the penalty above it
+    assert np.all(lg[:, upper] < -6.0e4)
+    i, j = 700, 123
+    assert_close(lg[:, i, j], 0.125 * (q[:, i].astype(np.float64) * k[:, j]).sum(-1), 1e-2, 2e-2, "one logit per batch entry")
+    # the output is the weights applied to the values
+    assert_close(out[5], w[5].astype(np.float64) @ v[5], 1e-2, 2e-2, "out = weights v")
+    for bi in (0, 11):
+        oo, ow, ol = (_oracle_arr(oracle, np.zeros(s_, np.float32), dt) for s_ in ((1, T, D), (1, T, T), (1, T, T)))
+        oracle.attention_v2(_oracle_arr(oracle, q[bi:bi + 1], dt), _oracle_arr(oracle, v[bi:bi + 1], dt), _oracle_arr(oracle, k[bi:bi + 1], dt), oo,
+                            weights=ow, logits=ol, scale=0.125, causal=True)
+        assert_close(out[bi:bi + 1], _as_float(oo), 1e-2, 1e-2, "out, batch entry %d" % bi)
+        assert_close(w[bi:bi + 1], _as_float(ow), 1e-2, 1e-2, "weights, batch entry %d" % bi)
+        lo, lgot = _as_float(ol), lg[bi:bi + 1]
+        keep = ~upper[None]
+        assert_close(lgot[keep], lo[keep], 1e-2, 2e-2, "logits below the diagonal, batch entry %d" % bi)
+        assert np.array_equal(lgot[~keep], lo[~keep]) or np.allclose(lgot[~keep], lo[~keep], rtol=1e-2)
+
+
 @pytest.mark.parametrize("dt,L,tol", [(BFLOAT16, 768, 1e-2), (HALF, 768, 2e-3), (FLOAT32, 384, 1e-5)])
 @pytest.mark.parametrize("rows,has_bias,pitched", [(4097, True, False), (4608, False, False), (4099, True, True)])
 def test_layer_norm_rows_of_one_and_a_half_passes(ex, oracle, dt, L, tol, rows, has_bias, pitched):
