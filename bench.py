@@ -252,8 +252,8 @@ def main():
             """make_call(i) -> zero-argument callable on operand set i.  Cold = rotating over the sets, warm = set 0 only."""
             k = n_sets(nbytes)
             calls = [make_call(i) for i in range(k)]
-            w, e = timed_rotating(ex, L, calls, max(steps, 2 * k), warmup)
             _, e_warm = timed(ex, L, calls[0], steps, warmup)
+            w, e = timed_rotating(ex, L, calls, max(steps, 2 * k), warmup)   # last, so that a trace ends on the cold steps
             line = {"op": name, "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": hbm_entry(nbytes, e, label, e_warm, k)}
             if cpu and cpu_fn is not None:
                 line["cpu_baseline"] = cpu_fn()
