@@ -1260,12 +1260,16 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32(GemmArgs g, const fl
 // The fp32 kernel for launches of whole tiles that put one small tile on a CU: PD K-tiles of global loads in flight (PD
 // register sets, the K loop unrolled PD times and free of branches -- loads past the end re-read the last K-tile, the
 // store after the last K-tile fills a stage nobody reads), so the loop runs at the MFMA rate instead of one memory
-// latency per 16 k.  Host: M % BM == 0, N % BN == 0, K % (16 * PD) == 0.
-template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int PD>
+// latency per K-tile.  BK = 32 halves the barriers per MFMA (the one-tile-per-CU launch, where nothing else covers
+// them).  Host: M % BM == 0, N % BN == 0, K % (BK * PD) == 0, K >= 2 * BK * PD.
+template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int PD, int BK>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32q(GemmArgs g, const float* __restrict__ A, const float* __restrict__ B,
                                                               float* __restrict__ C, unsigned tilesM, unsigned tilesN) {
   static_assert(PD % 2 == 0, "the LDS stage of a K-tile must be a compile-time constant inside the unrolled loop");
-  constexpr int BK = 16, NT = WM * WN * 64, PA = BM + 4, PB = BN + 4;
+  static_assert(BK == 16 || BK == 32, "K-tile");
+  // row pitch of a stage: k-contiguous operands are scattered into it (a thread's 4 k land 4 rows apart, KQ threads share a
+  // row of the operand): 4 * pitch mod 64 banks must be 64 / KQ apart; the others are stored 16 bytes at a time
+  constexpr int KQ = BK / 4, NT = WM * WN * 64, PA = BM + (A_KC && BK == 32 ? 2 : 4), PB = BN + (B_KC && BK == 32 ? 2 : 4);
   constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
   constexpr int VA = BM * BK / 4 / NT, VB = BN * BK / 4 / NT;   // float4 per thread
   __shared__ __attribute__((aligned(16))) float sA[2][BK * PA];
@@ -1286,45 +1290,61 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32q(GemmArgs g, const f
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
   f32x4 ra[PD][VA], rb[PD][VB];
-  auto load = [&](int u, LongType k0) {
+  // Every thread keeps one running pointer per load, advanced by the K-tile's byte step (the same for all lanes: a scalar
+  // operand, set to zero once the last K-tile is reached so that loads past the end re-read it): one 64-bit add per load
+  // and K-tile.  Computed from the element coordinates each time it cost a 64-bit multiply-add chain in front of an MFMA.
+  typedef const __attribute__((address_space(1))) char* GlobalBytes;
+  GlobalBytes curA[VA], curB[VB];
 #pragma unroll
-    for (int i = 0; i < VA; i++) {
-      const int v = t + i * NT;
-      if (A_KC) ra[u][i] = *reinterpret_cast<const f32x4*>(A + (m0 + (v >> 2)) * lda + k0 + (v & 3) * 4);
-      else ra[u][i] = *reinterpret_cast<const f32x4*>(A + (k0 + v / (BM / 4)) * lda + m0 + (v % (BM / 4)) * 4);
+  for (int i = 0; i < VA; i++) {
+    const int v = t + i * NT;
+    curA[i] = (GlobalBytes)(A_KC ? A + (m0 + v / KQ) * lda + (v % KQ) * 4 : A + (LongType)(v / (BM / 4)) * lda + m0 + (v % (BM / 4)) * 4);
+  }
+#pragma unroll
+  for (int i = 0; i < VB; i++) {
+    const int v = t + i * NT;
+    curB[i] = (GlobalBytes)(B_KC ? B + (n0 + v / KQ) * ldb + (v % KQ) * 4 : B + (LongType)(v / (BN / 4)) * ldb + n0 + (v % (BN / 4)) * 4);
+  }
+  const LongType KT = g.K / BK;
+  const LongType stepA = (A_KC ? BK : BK * lda) * 4, stepB = (B_KC ? BK : BK * ldb) * 4;   // bytes per K-tile
+  // more: the K-tile loaded is not the last one (a condition on the loop counters, so a scalar one)
+  auto loadNext = [&](int u, bool more) {
+#pragma unroll
+    for (int i = 0; i < VA; i++) ra[u][i] = *(const __attribute__((address_space(1))) f32x4*)curA[i];
+#pragma unroll
+    for (int i = 0; i < VB; i++) rb[u][i] = *(const __attribute__((address_space(1))) f32x4*)curB[i];
+    const LongType sa = more ? stepA : 0, sb = more ? stepB : 0;
+#pragma unroll
+    for (int i = 0; i < VA; i++) curA[i] += sa;
+#pragma unroll
+    for (int i = 0; i < VB; i++) curB[i] += sb;
+  };
+  auto storeA = [&](int u, int stage, int i) {
+    const int v = t + i * NT;
+    if (A_KC) {
+#pragma unroll
+      for (int q = 0; q < 4; q++) sA[stage][((v % KQ) * 4 + q) * PA + v / KQ] = ra[u][i][q];
+    } else {
+      *reinterpret_cast<f32x4*>(&sA[stage][(v / (BM / 4)) * PA + (v % (BM / 4)) * 4]) = ra[u][i];
     }
+  };
+  auto storeB = [&](int u, int stage, int i) {
+    const int v = t + i * NT;
+    if (B_KC) {
 #pragma unroll
-    for (int i = 0; i < VB; i++) {
-      const int v = t + i * NT;
-      if (B_KC) rb[u][i] = *reinterpret_cast<const f32x4*>(B + (n0 + (v >> 2)) * ldb + k0 + (v & 3) * 4);
-      else rb[u][i] = *reinterpret_cast<const f32x4*>(B + (k0 + v / (BN / 4)) * ldb + n0 + (v % (BN / 4)) * 4);
+      for (int q = 0; q < 4; q++) sB[stage][((v % KQ) * 4 + q) * PB + v / KQ] = rb[u][i][q];
+    } else {
+      *reinterpret_cast<f32x4*>(&sB[stage][(v / (BN / 4)) * PB + (v % (BN / 4)) * 4]) = rb[u][i];
     }
   };
   auto store = [&](int u, int stage) {
 #pragma unroll
-    for (int i = 0; i < VA; i++) {
-      const int v = t + i * NT;
-      if (A_KC) {
+    for (int i = 0; i < VA; i++) storeA(u, stage, i);
 #pragma unroll
-        for (int q = 0; q < 4; q++) sA[stage][((v & 3) * 4 + q) * PA + (v >> 2)] = ra[u][i][q];
-      } else {
-        *reinterpret_cast<f32x4*>(&sA[stage][(v / (BM / 4)) * PA + (v % (BM / 4)) * 4]) = ra[u][i];
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < VB; i++) {
-      const int v = t + i * NT;
-      if (B_KC) {
-#pragma unroll
-        for (int q = 0; q < 4; q++) sB[stage][((v & 3) * 4 + q) * PB + (v >> 2)] = rb[u][i][q];
-      } else {
-        *reinterpret_cast<f32x4*>(&sB[stage][(v / (BN / 4)) * PB + (v % (BN / 4)) * 4]) = rb[u][i];
-      }
-    }
+    for (int i = 0; i < VB; i++) storeB(u, stage, i);
   };
-  const LongType KT = g.K / BK;
 #pragma unroll
-  for (int u = 0; u < PD; u++) load(u, (LongType)u * BK);
+  for (int u = 0; u < PD; u++) loadNext(u, true);   // KT >= 2 * PD
   store(0, 0);
   __syncthreads();
   // One small tile per CU (one wave per SIMD, one accumulator per wave): nothing covers an LDS round trip, so the
@@ -1340,9 +1360,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32q(GemmArgs g, const f
       for (int j = 0; j < TN; j++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc2[i][j][r] = 0.f;
-    auto readTile = [&](int stage, int buf) {
+    auto readPart = [&](int stage, int buf, int from, int to) {
 #pragma unroll
-      for (int ks = 0; ks < BK / 2; ks++) {
+      for (int ks = from; ks < to; ks++) {
         const int k = ks * 2 + (lane >> 5);
 #pragma unroll
         for (int i = 0; i < TM; i++) fa[buf][ks][i] = sA[stage][k * PA + wm * WTM + i * 32 + (lane & 31)];
@@ -1350,42 +1370,36 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32q(GemmArgs g, const f
         for (int j = 0; j < TN; j++) fb[buf][ks][j] = sB[stage][k * PB + wn * WTN + j * 32 + (lane & 31)];
       }
     };
-    readTile(0, 0);
+    constexpr int NS = BK / 2;   // MFMAs (k-steps of 2) per K-tile and accumulator tile
+    static_assert(VA + VB + 1 <= NS / 2, "stores and loads go in front of the barrier, one per MFMA");
+    readPart(0, 0, 0, NS);
     for (LongType kt0 = 0; kt0 < KT; kt0 += PD) {
 #pragma unroll
       for (int u = 0; u < PD; u++) {
-        const LongType kt = kt0 + u;
         const int cur = u & 1;
-        const LongType nx = kt + PD < KT ? kt + PD : KT - 1;
-        // even and odd k-steps go to two accumulators: with a single one every MFMA would wait for the previous one's result
-        auto mfmas = [&](int from, int to) {
+        // The wave's own bookkeeping for K-tile kt + 1 is issued between the MFMAs of K-tile kt (64 cycles of matrix pipe
+        // each), one piece per MFMA: left in front of them it ran while the pipe stood still, 200 cycles for every 512 of
+        // MFMA, and bunched behind one MFMA it overran that MFMA's shadow.  Even and odd k-steps go to two accumulators:
+        // with a single one every MFMA would wait for the previous one's result.
 #pragma unroll
-          for (int ks = from; ks < to; ks++)
+        for (int ks = 0; ks < NS; ks++) {
 #pragma unroll
-            for (int i = 0; i < TM; i++)
+          for (int i = 0; i < TM; i++)
 #pragma unroll
-              for (int j = 0; j < TN; j++) {
-                if (ks & 1) acc2[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][ks][i], fb[cur][ks][j], acc2[i][j], 0, 0, 0);
-                else acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][ks][i], fb[cur][ks][j], acc[i][j], 0, 0, 0);
-              }
-        };
-        // the wave's own bookkeeping for K-tile kt + 1 is issued between the MFMAs of K-tile kt (64 cycles of matrix pipe
-        // each): left in front of them it ran while the pipe stood still, 200 cycles for every 512 of MFMA
-        mfmas(0, 1);
-        store((u + 1) % PD, cur ^ 1);
-        __builtin_amdgcn_sched_barrier(0);
-        mfmas(1, 2);
-        load(u, nx * BK);
-        __builtin_amdgcn_sched_barrier(0);
-        mfmas(2, 4);
-        __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();
-        __builtin_amdgcn_sched_barrier(0);
-        mfmas(4, 5);
-        readTile(cur ^ 1, cur ^ 1);
-        __builtin_amdgcn_sched_barrier(0);
-        mfmas(5, BK / 2);
-        __builtin_amdgcn_sched_barrier(0);
+            for (int j = 0; j < TN; j++) {
+              if (ks & 1) acc2[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][ks][i], fb[cur][ks][j], acc2[i][j], 0, 0, 0);
+              else acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][ks][i], fb[cur][ks][j], acc[i][j], 0, 0, 0);
+            }
+          if (ks < VA) storeA((u + 1) % PD, cur ^ 1, ks);
+          else if (ks < VA + VB) storeB((u + 1) % PD, cur ^ 1, ks - VA);
+          else if (ks == VA + VB) loadNext(u, kt0 + u + PD < KT - 1);   // K-tile min(kt0 + u + PD, KT - 1)
+          if (ks == NS / 2 - 1) {
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();
+          }
+          if (ks >= NS / 2 && (ks - NS / 2) * 4 < NS) readPart(cur ^ 1, cur ^ 1, (ks - NS / 2) * 4, (ks - NS / 2) * 4 + 4);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
     }
 #pragma unroll
@@ -1400,10 +1414,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32q(GemmArgs g, const f
   for (LongType kt0 = 0; kt0 < KT; kt0 += PD) {
 #pragma unroll
     for (int u = 0; u < PD; u++) {
-      const LongType kt = kt0 + u;
       const int cur = u & 1;
-      const LongType nx = kt + PD < KT ? kt + PD : KT - 1;
-      load(u, nx * BK);   // K-tile kt sits in LDS: its register set takes K-tile kt + PD
+      loadNext(u, kt0 + u + PD < KT - 1);   // K-tile kt0 + u sits in LDS: its register set takes K-tile min(kt0 + u + PD, KT - 1)
 #pragma unroll
       for (int ks = 0; ks < BK / 2; ks++) {
         const int k = ks * 2 + (lane >> 5);
@@ -1428,9 +1440,9 @@ template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC>
 static void launchMfma32Cfg(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C, LongType batch) {
   const unsigned tilesM = (unsigned)((g.M + BM - 1) / BM), tilesN = (unsigned)((g.N + BN - 1) / BN);
   if (g.K >= 256 && g.M % BM == 0 && g.N % BN == 0 && g.K % 128 == 0) {
-    constexpr int PD = BM * BN <= 64 * 64 ? 8 : 4;
-    noteKernel("gemm_mfma32q<f32,%dx%d,akc=%d,bkc=%d,pd=%d>", BM, BN, (int)A_KC, (int)B_KC, PD);
-    hipLaunchKernelGGL((gemm_mfma32q<BM, BN, WM, WN, A_KC, B_KC, PD>), dim3(tilesM * tilesN, 1, (unsigned)batch), dim3(WM * WN * 64), 0, s, g,
+    constexpr int PD = 4, BK = BM * BN <= 64 * 64 ? 32 : 16;
+    noteKernel("gemm_mfma32q<f32,%dx%d,akc=%d,bkc=%d,pd=%d,bk=%d>", BM, BN, (int)A_KC, (int)B_KC, PD, BK);
+    hipLaunchKernelGGL((gemm_mfma32q<BM, BN, WM, WN, A_KC, B_KC, PD, BK>), dim3(tilesM * tilesN, 1, (unsigned)batch), dim3(WM * WN * 64), 0, s, g,
                        (const float*)A, (const float*)B, (float*)C, tilesM, tilesN);
     return;
   }

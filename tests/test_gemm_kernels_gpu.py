@@ -56,7 +56,7 @@ def _check_rows_cols(z, a64, b64, tol, rng, what):
 # (dtype, M, N, K, kernel for plain B, kernel for transposeB, kernel for transposeA or None)
 CASES = [
     # BASELINE config 2 at 4096^3
-    (FLOAT32, 4096, 4096, 4096, "gemm_mfma32q<f32,128x128,akc=1,bkc=0,pd=4>", "gemm_mfma32q<f32,128x128,akc=1,bkc=1,pd=4>", "gemm_mfma32q<f32,128x128,akc=0,bkc=0,pd=4>"),
+    (FLOAT32, 4096, 4096, 4096, "gemm_mfma32q<f32,128x128,akc=1,bkc=0,pd=4,bk=16>", "gemm_mfma32q<f32,128x128,akc=1,bkc=1,pd=4,bk=16>", "gemm_mfma32q<f32,128x128,akc=0,bkc=0,pd=4,bk=16>"),
     (HALF, 4096, 4096, 4096, "gemm_mfma16r<f16,256x256,akc=1,bkc=0>", "gemm_mfma16d<f16,256x256,akc=1,bkc=1>", "gemm_mfma16f<f16,256x256,akc=0,bkc=0>"),
     (BFLOAT16, 4096, 4096, 4096, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1>", "gemm_mfma16f<bf16,256x256,akc=0,bkc=0>"),
     # the ring kernel at its shortest K (the prologue alone fills the rings) and at a K that ends in the middle of both rings;
@@ -66,7 +66,7 @@ CASES = [
     (BFLOAT16, 4096, 4096, 1152, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1>", None),
     (BFLOAT16, 4096, 4096, 192, "gemm_mfma16d<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1>", None),
     # BASELINE config 2 at 1024^3
-    (FLOAT32, 1024, 1024, 1024, "gemm_mfma32q<f32,64x64,akc=1,bkc=0,pd=8>", "gemm_mfma32q<f32,64x64,akc=1,bkc=1,pd=8>", "gemm_mfma32q<f32,64x64,akc=0,bkc=0,pd=8>"),
+    (FLOAT32, 1024, 1024, 1024, "gemm_mfma32q<f32,64x64,akc=1,bkc=0,pd=4,bk=32>", "gemm_mfma32q<f32,64x64,akc=1,bkc=1,pd=4,bk=32>", "gemm_mfma32q<f32,64x64,akc=0,bkc=0,pd=4,bk=32>"),
     (HALF, 1024, 1024, 1024, "gemm_mfma16q<f16,64x64,akc=1,bkc=0>", "gemm_mfma16q<f16,64x64,akc=1,bkc=1>", "gemm_mfma16q<f16,64x64,akc=0,bkc=0>"),
     (BFLOAT16, 1024, 1024, 1024, "gemm_mfma16q<bf16,64x64,akc=1,bkc=0>", "gemm_mfma16q<bf16,64x64,akc=1,bkc=1>", "gemm_mfma16q<bf16,64x64,akc=0,bkc=0>"),
     # the 128 x 128 configuration (2048-class sizes), whole tiles
@@ -78,8 +78,8 @@ CASES = [
     (BFLOAT16, 1104, 904, 1000, "gemm_mfma16p<bf16,64x64,akc=1,bkc=0>", "gemm_mfma16p<bf16,64x64,akc=1,bkc=1>", None),
     # K a multiple of 256 but not of 512: the four-deep prefetch ends in the middle of its ring
     (BFLOAT16, 1024, 1024, 768, "gemm_mfma16q<bf16,64x64,akc=1,bkc=0>", "gemm_mfma16q<bf16,64x64,akc=1,bkc=1>", None),
-    (FLOAT32, 1024, 1024, 384, "gemm_mfma32q<f32,64x64,akc=1,bkc=0,pd=8>", "gemm_mfma32q<f32,64x64,akc=1,bkc=1,pd=8>", None),
-    (FLOAT32, 2048, 2048, 640, "gemm_mfma32q<f32,128x128,akc=1,bkc=0,pd=4>", "gemm_mfma32q<f32,128x128,akc=1,bkc=1,pd=4>", None),
+    (FLOAT32, 1024, 1024, 384, "gemm_mfma32q<f32,64x64,akc=1,bkc=0,pd=4,bk=32>", "gemm_mfma32q<f32,64x64,akc=1,bkc=1,pd=4,bk=32>", None),
+    (FLOAT32, 2048, 2048, 640, "gemm_mfma32q<f32,128x128,akc=1,bkc=0,pd=4,bk=16>", "gemm_mfma32q<f32,128x128,akc=1,bkc=1,pd=4,bk=16>", None),
     # fp32 ragged
     (FLOAT32, 1100, 900, 1000, "gemm_mfma32<f32,64x64,akc=1,bkc=0>", "gemm_mfma32<f32,64x64,akc=1,bkc=1>", None),
     (FLOAT32, 2100, 2052, 520, "gemm_mfma32<f32,128x128,akc=1,bkc=0>", "gemm_mfma32<f32,128x128,akc=1,bkc=1>", "gemm_mfma32<f32,128x128,akc=0,bkc=0>"),
