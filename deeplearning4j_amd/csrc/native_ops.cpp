@@ -324,7 +324,7 @@ Nd4jLong dbBufferLength(OpaqueDataBuffer* b) { return b && b->db ? b->db->numEle
 void dbSetPrimaryBuffer(OpaqueDataBuffer* b, Nd4jPointer p, Nd4jLong numBytes) {
   GUARD_BEGIN
   ND4J_REQUIRE(b && b->db, "dbSetPrimaryBuffer: buffer is null");
-  if (b->db->ownsPrimary && b->db->primary) free(b->db->primary);
+  b->db->releasePrimary();
   b->db->primary = p; b->db->ownsPrimary = false; b->db->lenBytes = (size_t)numBytes;
   b->db->tickWritePrimary();
   GUARD_END_VOID

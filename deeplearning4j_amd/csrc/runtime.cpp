@@ -160,13 +160,39 @@ DataBuffer::DataBuffer(void* prim, void* spec, size_t bytes, DataType dt)
   if (spec && !prim) writeSpecial = ++counter;
 }
 DataBuffer::~DataBuffer() { close(); }
+// Host buffers of this size and more are page-locked when a device is present (as the device backend's own host
+// allocations are, legacy/cuda/NativeOps.cu:1158-1168 mallocHost): the copies of syncToSpecial / syncToPrimary then run as
+// one DMA transfer at the link's rate instead of being staged through the runtime's bounce buffers.  Smaller ones stay
+// pageable, a page-locked allocation costs more than their copy.  ND4JHIP_PINNED_MIN_BYTES overrides the size (0 = never).
+static size_t pinnedMinBytes() {
+  static const size_t v = [] {
+    const char* e = getenv("ND4JHIP_PINNED_MIN_BYTES");
+    if (!e || !*e) return (size_t)1 << 20;
+    const unsigned long long n = strtoull(e, nullptr, 10);
+    return n == 0 ? (size_t)-1 : (size_t)n;
+  }();
+  return v;
+}
 void DataBuffer::allocatePrimary() {
   if (primary || lenBytes == 0) return;
   void* p = nullptr;
-  if (posix_memalign(&p, 64, lenBytes) != 0) ND4J_THROW("DataBuffer: host allocation failed");
+  if (lenBytes >= pinnedMinBytes() && deviceAvailable()) {
+    LaunchContext::defaultContext();
+    if (hipHostMalloc(&p, lenBytes, hipHostMallocDefault) == hipSuccess) pinnedPrimary = true;
+    else { (void)hipGetLastError(); p = nullptr; }   // no page-locked memory left: a pageable buffer does the same job, slower
+  }
+  if (!p && posix_memalign(&p, 64, lenBytes) != 0) ND4J_THROW("DataBuffer: host allocation failed");
   memset(p, 0, lenBytes);
   primary = p;
   ownsPrimary = true;
+}
+void DataBuffer::releasePrimary() {
+  if (ownsPrimary && primary) {
+    if (pinnedPrimary) (void)hipHostFree(primary);
+    else free(primary);
+  }
+  primary = nullptr;
+  ownsPrimary = pinnedPrimary = false;
 }
 void DataBuffer::allocateSpecial() {
   if (special || lenBytes == 0) return;
@@ -182,7 +208,7 @@ void DataBuffer::syncToSpecial(bool force) {
   if (!special) allocateSpecial();
   auto lc = LaunchContext::defaultContext();
   HIP_CHECK(hipMemcpyAsync(special, primary, lenBytes, hipMemcpyHostToDevice, lc->execStream));
-  // pageable source: make sure the staging copy has consumed the host memory before the caller reuses it
+  // the caller may rewrite the host memory as soon as this returns (array/cuda/DataBuffer.cu:399-413 copies synchronously)
   HIP_CHECK(hipStreamSynchronize(lc->execStream));
   readSpecial = ++counter;  // device copy is current; the host copy stays current too
 }
@@ -199,13 +225,15 @@ void DataBuffer::syncToPrimary(bool force) {
 void DataBuffer::expand(size_t newBytes) {
   if (newBytes <= lenBytes) return;
   if (primary) {
-    void* p = nullptr;
-    if (posix_memalign(&p, 64, newBytes) != 0) ND4J_THROW("DataBuffer::expand: host allocation failed");
-    memset(p, 0, newBytes);
-    memcpy(p, primary, lenBytes);
-    if (ownsPrimary) free(primary);
-    primary = p;
-    ownsPrimary = true;
+    void* const old = primary;
+    const bool oldOwned = ownsPrimary, oldPinned = pinnedPrimary;
+    const size_t oldBytes = lenBytes;
+    primary = nullptr; ownsPrimary = pinnedPrimary = false;
+    lenBytes = newBytes;
+    allocatePrimary();   // zero-filled, page-locked from the same size on
+    lenBytes = oldBytes;
+    memcpy(primary, old, oldBytes);
+    if (oldOwned) { if (oldPinned) (void)hipHostFree(old); else free(old); }
   }
   if (special) {
     void* d = nullptr;
@@ -223,9 +251,9 @@ void DataBuffer::expand(size_t newBytes) {
 void DataBuffer::close() {
   if (closed) return;
   closed = true;
-  if (ownsPrimary && primary) free(primary);
+  releasePrimary();
   if (ownsSpecial && special) (void)hipFree(special);
-  primary = special = nullptr;
+  special = nullptr;
 }
 
 // ---- stream capture ---------------------------------------------------------------------------------

@@ -72,6 +72,7 @@ struct DataBuffer {
   size_t lenBytes = 0;
   DataType dtype = FLOAT32;
   bool ownsPrimary = false, ownsSpecial = false;
+  bool pinnedPrimary = false;   // primary came from hipHostMalloc (owned buffers of 1 MiB and more)
   bool closed = false;
   int deviceId = 0;
   std::atomic<LongType> counter{0};
@@ -82,6 +83,7 @@ struct DataBuffer {
   ~DataBuffer();
   LongType numElements() const { return sizeOf(dtype) ? (LongType)(lenBytes / sizeOf(dtype)) : 0; }
   void allocatePrimary();
+  void releasePrimary();
   void allocateSpecial();
   bool isPrimaryActual() const { return writePrimary > writeSpecial || readPrimary > writeSpecial; }
   bool isSpecialActual() const { return writeSpecial > writePrimary || readSpecial > writePrimary; }
