@@ -442,8 +442,11 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16q(GemmArgs g, const T
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
   static_assert(PD % 2 == 0, "the LDS stage of a K-tile must be a compile-time constant inside the unrolled loop");
+  // B with unit column stride stays in LDS as it lies in memory and is read with the transposing LDS read; transposed in
+  // registers on the way in (v_perm_b32, eight 8-byte stores per thread) it cost 1.7 us of a 1024^3 launch
+  using LoaderB = std::conditional_t<B_KC, TileLoader<BN, NT, true>, RowTileLoader<BN, NT>>;
   TileLoader<BM, NT, A_KC> la[PD];
-  TileLoader<BN, NT, B_KC> lb[PD];
+  LoaderB lb[PD];
   const LongType KT = (g.K + BK - 1) / BK;
 
   // K is a multiple of PD K-tiles (host), and nothing below is conditional: loads past the end re-read the last K-tile and
@@ -464,6 +467,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16q(GemmArgs g, const T
   // of cover for a latency several times that) made every k-step wait, 750 cycles per K-tile where the L2 stream of the
   // tile takes about 410.
   u32x4 fa[2][BK / 16][TM], fb[2][BK / 16][TN];
+  int trB[TN];
+#pragma unroll
+  for (int j = 0; j < TN; j++) trB[j] = B_KC ? 0 : RowTileLoader<BN, NT>::fragOffset(wn * WTN + j * 32, lane);
   auto readTile = [&](int stage, int buf) {
     const u32x4* sA = smem + stage * STAGE;
     const u32x4* sB = sA + SLOTS_A;
@@ -473,7 +479,10 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16q(GemmArgs g, const T
 #pragma unroll
       for (int i = 0; i < TM; i++) fa[buf][ks][i] = sA[LayA::slot(kg, wm * WTM + i * 32 + (lane & 31))];
 #pragma unroll
-      for (int j = 0; j < TN; j++) fb[buf][ks][j] = sB[LayB::slot(kg, wn * WTN + j * 32 + (lane & 31))];
+      for (int j = 0; j < TN; j++) {
+        if constexpr (B_KC) fb[buf][ks][j] = sB[LayB::slot(kg, wn * WTN + j * 32 + (lane & 31))];
+        else fb[buf][ks][j] = RowTileLoader<BN, NT>::readFrag(sB, trB[j], ks);
+      }
     }
   };
   readTile(0, 0);

@@ -154,4 +154,54 @@ struct TileLoader {
   }
 };
 
+// Loader for a 64 (k) x ROWS tile of an operand stored [k][row] with unit row stride, kept in LDS as it lies in memory
+// (no register transpose): the fragments are taken with the transposing LDS read (ds_read_b64_tr_b16), which hands a lane
+// the four k-values of one row out of a 4 (k) x 16 (rows) block read by its 16-lane group.  A k-row is ROWS / 8 slots of
+// 16 bytes; slot s of k-row k sits at k * (ROWS / 8) + (s ^ swz(k)).  The swizzle keeps the read free of bank
+// conflicts: 32 lanes fetch 4 k-rows x 64 bytes per pass, and k-rows whose starts fall on the same bank (every second
+// one for 128-byte rows, all of them from 256-byte rows on) are moved to different 64-byte quarters of the row.
+template <int ROWS, int NT>
+struct RowTileLoader {
+  static_assert(ROWS >= 64 && ROWS % 64 == 0, "a k-row holds whole 128-byte lines");
+  static constexpr int SPR = ROWS / 8;              // slots per k-row
+  static constexpr int UNITS = 64 * SPR, PER = (UNITS + NT - 1) / NT;
+  static_assert(UNITS % NT == 0, "every thread moves the same number of vectors");
+  u32x4 reg[PER];
+  static __device__ __forceinline__ int swz(int k) { return ROWS == 64 ? 4 * ((k >> 1) & 1) : 4 * (k & 3); }
+  template <typename T>
+  __device__ __forceinline__ void loadFull(const T* __restrict__ base, LongType ld, LongType row0, LongType k0, int t) {
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      const int u = t + i * NT;
+      reg[i] = *reinterpret_cast<const u32x4*>(base + (k0 + u / SPR) * ld + row0 + (u % SPR) * 8);
+    }
+  }
+  __device__ __forceinline__ void store(u32x4* __restrict__ lds, int t) {
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      const int u = t + i * NT, k = u / SPR;
+      lds[k * SPR + ((u % SPR) ^ swz(k))] = reg[i];
+    }
+  }
+  // Byte offset (inside the tile) of the lane's first transposing read for the 32 rows starting at row32 and k-step 0;
+  // k-step ks adds ks * 16 k-rows, the second read of a k-step (k-values 4..7 of the lane's eight) adds 4 k-rows.
+  static __device__ __forceinline__ int fragOffset(int row32, int lane) {
+    const int grp = lane >> 4, i16 = lane & 15;
+    const int r4 = row32 + 16 * (grp & 1) + 4 * (i16 & 3);
+    const int k = 8 * (grp >> 1) + (i16 >> 2);
+    return (k * SPR + ((r4 >> 3) ^ swz(k))) * 16 + ((r4 >> 2) & 1) * 8;
+  }
+  static constexpr int KSTEP_BYTES = 16 * SPR * 16, HALF_BYTES = 4 * SPR * 16;
+  static __device__ __forceinline__ u32x4 readFrag(const u32x4* tile, int fragOff, int ks) {
+    typedef __attribute__((address_space(3))) void* lds_ptr;
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    const __attribute__((address_space(3))) unsigned char* base =
+        (const __attribute__((address_space(3))) unsigned char*)(lds_ptr)tile + fragOff + ks * KSTEP_BYTES;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)base);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(base + HALF_BYTES));
+    const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+    return u32x4{l2[0], l2[1], h2[0], h2[1]};
+  }
+};
+
 }  // namespace nd4jhip
