@@ -171,6 +171,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-ops", action="store_true", help="leave out the per-op lines of BASELINE configs 1-4")
+    ap.add_argument("--configs", default="1,2,3,4", help="which BASELINE configs the per-op lines cover (comma-separated; for profiling one op class)")
     ap.add_argument("--skip-cpu", action="store_true", help="leave out the cpu_baseline leg")
     ap.add_argument("--skip-decode", action="store_true", help="leave out the GPT-2-shaped decode (tens of thousands of launches)")
     ap.add_argument("--settle", type=float, default=SETTLE_S,
@@ -240,6 +241,7 @@ def main():
 
     # ---- the other BASELINE configs ------------------------------------------------------------------------------------
     ops = []
+    cfgs = {int(c) for c in args.configs.split(",") if c.strip()}
     if not args.skip_ops:
         print("[bench] per-op leg", file=sys.stderr, flush=True)
         del A, B, Z
@@ -259,181 +261,185 @@ def main():
                 line["cpu_baseline"] = cpu_fn()
             ops.append(line)
 
-        # config 1: legacy chain, fp32 [8192, 4096]
-        rng = np.random.default_rng(1001)
-        shp = (8192, 4096)
-        ne = shp[0] * shp[1]
-        xh = rng.uniform(-1, 1, shp).astype(np.float32)
-        yh = rng.uniform(-1, 1, shp).astype(np.float32)
-        K1 = n_sets(4 * ne)        # the reductions read 128 MiB per call: they need the most sets
-        Xs = [NDArray.from_numpy(xh) for _ in range(K1)]
-        Ys = [NDArray.from_numpy(yh) for _ in range(3)]
-        Ss = [NDArray.empty(shp, FLOAT32) for _ in range(3)]
-        Rs = [NDArray.empty((shp[0],), FLOAT32) for _ in range(K1)]
-        AMs = [NDArray.empty((shp[0],), INT64) for _ in range(K1)]
-        for arr in Xs + Ys:
-            arr.sync_to_device()
-        rows_s = 1024                                     # CPU sample: the first 1024 rows (4 Mi elements)
-        xs_, ys_ = xh[:rows_s].copy(), yh[:rows_s].copy()
-        zs_ = np.zeros_like(xs_)
-        samp = "first %d of 8192 rows" % rows_s
-        GB = 1e9
-        hbm_line("copy fp32 [8192,4096] (transform_same Copy; calibrates HBM counters)", "copy fp32", 2 * 4 * ne,
-                 lambda i: (lambda: ex.exec_transform_same(TransformSame.Copy, Xs[i], Ss[i % 3])),
-                 lambda: cpu_entry(2 * 4 * xs_.size, GB, "GB/s", lambda: O.transform_same(15, xs_, zs_), lambda: np.copyto(zs_, xs_), samp, "numpy copyto"))
-        hbm_line("pairwise_add fp32 [8192,4096]", "pairwise_add fp32", 3 * 4 * ne,
-                 lambda i: (lambda: ex.exec_pairwise(Pairwise.Add, Xs[i], Ys[i % 3], Ss[i % 3])),
-                 lambda: cpu_entry(3 * 4 * xs_.size, GB, "GB/s", lambda: O.pairwise(0, xs_, ys_, zs_), lambda: np.add(xs_, ys_, out=zs_), samp, "numpy add"))
-        hbm_line("transform_tanh fp32 [8192,4096]", "transform_tanh fp32", 2 * 4 * ne,
-                 lambda i: (lambda: ex.exec_transform_strict(TransformStrict.Tanh, Xs[i], Ss[i % 3])),
-                 lambda: cpu_entry(2 * 4 * xs_.size, GB, "GB/s", lambda: O.transform_strict(29, xs_, zs_), lambda: np.tanh(xs_, out=zs_), samp, "numpy tanh"))
-        r_ = np.zeros(rows_s, np.float32)
-        i_ = np.zeros(rows_s, np.int64)
-        hbm_line("reduce_sum dim1 fp32 [8192,4096]", "reduce_sum", 4 * ne + 4 * shp[0],
-                 lambda i: (lambda: ex.exec_reduce_same(ReduceSame.Sum, Xs[i], [1], z=Rs[i])),
-                 lambda: cpu_entry(4 * xs_.size, GB, "GB/s", lambda: O.reduce_same(0, xs_, r_, [1]), lambda: np.sum(xs_, axis=1, out=r_), samp, "numpy sum"))
-        hbm_line("argmax dim1 fp32 [8192,4096]", "argmax dim1", 4 * ne + 8 * shp[0],
-                 lambda i: (lambda: ex.exec_index_reduce(IndexReduce.IndexMax, Xs[i], [1], z=AMs[i])),
-                 lambda: cpu_entry(4 * xs_.size, GB, "GB/s", lambda: O.index_reduce(0, xs_, i_, [1]), lambda: np.argmax(xs_, axis=1, out=i_), samp, "numpy argmax"))
-        del Xs, Ys, Ss, Rs, AMs, xh, yh
-        # config 3: row ops on [16, 1024, 768] and softmax on [16, 12, 1024, 1024]
-        rng = np.random.default_rng(3003)
-        for dt, dtn, es in [(FLOAT32, "fp32", 4), (BFLOAT16, "bf16", 2)]:
-            xs = (16, 1024, 768)
-            nx = 16 * 1024 * 768
-            xr = rng.normal(0, 1, xs).astype(np.float32)
-            gh, bh = rng.normal(1, 0.02, 768).astype(np.float32), rng.normal(0, 0.02, 768).astype(np.float32)
-            K3 = n_sets(2 * es * nx)
-            Xr = [NDArray.from_numpy(xr, dt) for _ in range(K3)]
-            Zr = [NDArray.empty(xs, dt) for _ in range(K3)]
-            G, Bv = NDArray.from_numpy(gh, dt), NDArray.from_numpy(bh, dt)
-            for arr in Xr + [G, Bv]:
+        if 1 in cfgs:
+            # config 1: legacy chain, fp32 [8192, 4096]
+            rng = np.random.default_rng(1001)
+            shp = (8192, 4096)
+            ne = shp[0] * shp[1]
+            xh = rng.uniform(-1, 1, shp).astype(np.float32)
+            yh = rng.uniform(-1, 1, shp).astype(np.float32)
+            K1 = n_sets(4 * ne)        # the reductions read 128 MiB per call: they need the most sets
+            Xs = [NDArray.from_numpy(xh) for _ in range(K1)]
+            Ys = [NDArray.from_numpy(yh) for _ in range(3)]
+            Ss = [NDArray.empty(shp, FLOAT32) for _ in range(3)]
+            Rs = [NDArray.empty((shp[0],), FLOAT32) for _ in range(K1)]
+            AMs = [NDArray.empty((shp[0],), INT64) for _ in range(K1)]
+            for arr in Xs + Ys:
                 arr.sync_to_device()
-            # CPU sample: the first 2 of 16 batch entries
-            conv = (lambda v: O.Arr(f32_to_bf16_bits(v), O.BFLOAT16)) if dt == BFLOAT16 else (lambda v: O.Arr(np.ascontiguousarray(v, np.float32)))
-            sx = xr[:2].reshape(-1, 768)
+            rows_s = 1024                                     # CPU sample: the first 1024 rows (4 Mi elements)
+            xs_, ys_ = xh[:rows_s].copy(), yh[:rows_s].copy()
+            zs_ = np.zeros_like(xs_)
+            samp = "first %d of 8192 rows" % rows_s
+            GB = 1e9
+            hbm_line("copy fp32 [8192,4096] (transform_same Copy; calibrates HBM counters)", "copy fp32", 2 * 4 * ne,
+                     lambda i: (lambda: ex.exec_transform_same(TransformSame.Copy, Xs[i], Ss[i % 3])),
+                     lambda: cpu_entry(2 * 4 * xs_.size, GB, "GB/s", lambda: O.transform_same(15, xs_, zs_), lambda: np.copyto(zs_, xs_), samp, "numpy copyto"))
+            hbm_line("pairwise_add fp32 [8192,4096]", "pairwise_add fp32", 3 * 4 * ne,
+                     lambda i: (lambda: ex.exec_pairwise(Pairwise.Add, Xs[i], Ys[i % 3], Ss[i % 3])),
+                     lambda: cpu_entry(3 * 4 * xs_.size, GB, "GB/s", lambda: O.pairwise(0, xs_, ys_, zs_), lambda: np.add(xs_, ys_, out=zs_), samp, "numpy add"))
+            hbm_line("transform_tanh fp32 [8192,4096]", "transform_tanh fp32", 2 * 4 * ne,
+                     lambda i: (lambda: ex.exec_transform_strict(TransformStrict.Tanh, Xs[i], Ss[i % 3])),
+                     lambda: cpu_entry(2 * 4 * xs_.size, GB, "GB/s", lambda: O.transform_strict(29, xs_, zs_), lambda: np.tanh(xs_, out=zs_), samp, "numpy tanh"))
+            r_ = np.zeros(rows_s, np.float32)
+            i_ = np.zeros(rows_s, np.int64)
+            hbm_line("reduce_sum dim1 fp32 [8192,4096]", "reduce_sum", 4 * ne + 4 * shp[0],
+                     lambda i: (lambda: ex.exec_reduce_same(ReduceSame.Sum, Xs[i], [1], z=Rs[i])),
+                     lambda: cpu_entry(4 * xs_.size, GB, "GB/s", lambda: O.reduce_same(0, xs_, r_, [1]), lambda: np.sum(xs_, axis=1, out=r_), samp, "numpy sum"))
+            hbm_line("argmax dim1 fp32 [8192,4096]", "argmax dim1", 4 * ne + 8 * shp[0],
+                     lambda i: (lambda: ex.exec_index_reduce(IndexReduce.IndexMax, Xs[i], [1], z=AMs[i])),
+                     lambda: cpu_entry(4 * xs_.size, GB, "GB/s", lambda: O.index_reduce(0, xs_, i_, [1]), lambda: np.argmax(xs_, axis=1, out=i_), samp, "numpy argmax"))
+            del Xs, Ys, Ss, Rs, AMs, xh, yh
+        if 3 in cfgs:
+            # config 3: row ops on [16, 1024, 768] and softmax on [16, 12, 1024, 1024]
+            rng = np.random.default_rng(3003)
+            for dt, dtn, es in [(FLOAT32, "fp32", 4), (BFLOAT16, "bf16", 2)]:
+                xs = (16, 1024, 768)
+                nx = 16 * 1024 * 768
+                xr = rng.normal(0, 1, xs).astype(np.float32)
+                gh, bh = rng.normal(1, 0.02, 768).astype(np.float32), rng.normal(0, 0.02, 768).astype(np.float32)
+                K3 = n_sets(2 * es * nx)
+                Xr = [NDArray.from_numpy(xr, dt) for _ in range(K3)]
+                Zr = [NDArray.empty(xs, dt) for _ in range(K3)]
+                G, Bv = NDArray.from_numpy(gh, dt), NDArray.from_numpy(bh, dt)
+                for arr in Xr + [G, Bv]:
+                    arr.sync_to_device()
+                # CPU sample: the first 2 of 16 batch entries
+                conv = (lambda v: O.Arr(f32_to_bf16_bits(v), O.BFLOAT16)) if dt == BFLOAT16 else (lambda v: O.Arr(np.ascontiguousarray(v, np.float32)))
+                sx = xr[:2].reshape(-1, 768)
 
-            def ln_cpu():
-                ox, og, ob, oz = conv(sx), conv(gh), conv(bh), conv(np.zeros_like(sx))
-                def fast():
-                    m = sx.mean(-1, keepdims=True); v = sx.var(-1, keepdims=True)
-                    return (sx - m) / np.sqrt(v + 1e-5) * gh + bh
-                return cpu_entry(2 * es * sx.size, GB, "GB/s", lambda: O.layer_norm(ox, og, ob, oz, [1], channels_first=False), fast,
-                                 "first 2 of 16 batch entries", "numpy mean/var/normalise in fp32")
+                def ln_cpu():
+                    ox, og, ob, oz = conv(sx), conv(gh), conv(bh), conv(np.zeros_like(sx))
+                    def fast():
+                        m = sx.mean(-1, keepdims=True); v = sx.var(-1, keepdims=True)
+                        return (sx - m) / np.sqrt(v + 1e-5) * gh + bh
+                    return cpu_entry(2 * es * sx.size, GB, "GB/s", lambda: O.layer_norm(ox, og, ob, oz, [1], channels_first=False), fast,
+                                     "first 2 of 16 batch entries", "numpy mean/var/normalise in fp32")
 
-            def gelu_cpu():
-                ox, oz = conv(sx), conv(np.zeros_like(sx))
-                return cpu_entry(2 * es * sx.size, GB, "GB/s", lambda: O.transform_strict(53, ox, oz), lambda: sx / (1.0 + np.exp(-1.702 * sx)),
-                                 "first 2 of 16 batch entries", "numpy x * sigmoid(1.702 x) in fp32")
+                def gelu_cpu():
+                    ox, oz = conv(sx), conv(np.zeros_like(sx))
+                    return cpu_entry(2 * es * sx.size, GB, "GB/s", lambda: O.transform_strict(53, ox, oz), lambda: sx / (1.0 + np.exp(-1.702 * sx)),
+                                     "first 2 of 16 batch entries", "numpy x * sigmoid(1.702 x) in fp32")
 
-            binds = [ex.bind_custom("layer_norm", [Xr[i], G, Bv], [Zr[i]], i_args=[2], b_args=[False]) for i in range(K3)]
-            hbm_line("layer_norm %s [16,1024,768]" % dtn, "layer_norm %s" % dtn, 2 * es * nx + 2 * es * 768, lambda i: binds[i], ln_cpu)
-            hbm_line("gelu %s [16,1024,768]" % dtn, "gelu %s" % dtn, 2 * es * nx,
-                     lambda i: (lambda: ex.exec_transform_strict(TransformStrict.GELU, Xr[i], Zr[i])), gelu_cpu)
-            del Xr, Zr, binds
-            ls = (16, 12, 1024, 1024)
-            nl = 16 * 12 * 1024 * 1024
-            # logits are generated in the permuted storage layout [16, 1024, 12, 1024]; the dense case uses the same numbers.
-            # One call moves 1.6 GB (0.8 GB in bf16), several times the last-level cache, so every call is cold by itself.
-            raw = rng.normal(0, 2, (16, 1024, 12, 1024)).astype(np.float32)
-            Lg = NDArray.from_numpy(raw, dt)
-            srow = raw[0, :64].reshape(-1, 1024).copy()        # CPU sample: 768 rows
-            del raw
-            Lg.sync_to_device()
-            Zs = NDArray.empty(ls, dt)
+                binds = [ex.bind_custom("layer_norm", [Xr[i], G, Bv], [Zr[i]], i_args=[2], b_args=[False]) for i in range(K3)]
+                hbm_line("layer_norm %s [16,1024,768]" % dtn, "layer_norm %s" % dtn, 2 * es * nx + 2 * es * 768, lambda i: binds[i], ln_cpu)
+                hbm_line("gelu %s [16,1024,768]" % dtn, "gelu %s" % dtn, 2 * es * nx,
+                         lambda i: (lambda: ex.exec_transform_strict(TransformStrict.GELU, Xr[i], Zr[i])), gelu_cpu)
+                del Xr, Zr, binds
+                ls = (16, 12, 1024, 1024)
+                nl = 16 * 12 * 1024 * 1024
+                # logits are generated in the permuted storage layout [16, 1024, 12, 1024]; the dense case uses the same numbers.
+                # One call moves 1.6 GB (0.8 GB in bf16), several times the last-level cache, so every call is cold by itself.
+                raw = rng.normal(0, 2, (16, 1024, 12, 1024)).astype(np.float32)
+                Lg = NDArray.from_numpy(raw, dt)
+                srow = raw[0, :64].reshape(-1, 1024).copy()        # CPU sample: 768 rows
+                del raw
+                Lg.sync_to_device()
+                Zs = NDArray.empty(ls, dt)
 
-            def sm_cpu():
-                ox, oz = conv(srow), conv(np.zeros_like(srow))
-                def fast():
-                    e = np.exp(srow - srow.max(-1, keepdims=True))
-                    return e / e.sum(-1, keepdims=True)
-                return cpu_entry(2 * es * srow.size, GB, "GB/s", lambda: O.softmax(ox, oz, 1), fast, "768 of 196,608 rows", "numpy max/exp/sum/divide in fp32")
+                def sm_cpu():
+                    ox, oz = conv(srow), conv(np.zeros_like(srow))
+                    def fast():
+                        e = np.exp(srow - srow.max(-1, keepdims=True))
+                        return e / e.sum(-1, keepdims=True)
+                    return cpu_entry(2 * es * srow.size, GB, "GB/s", lambda: O.softmax(ox, oz, 1), fast, "768 of 196,608 rows", "numpy max/exp/sum/divide in fp32")
 
-            dense = Lg.reshape(16, 12, 1024, 1024)
-            w, e = timed(ex, L, ex.bind_custom("softmax", [dense], [Zs], i_args=[3]), steps, warmup)
-            line = {"op": "softmax %s [16,12,1024,1024]" % dtn, "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": hbm_entry(2 * es * nl, e, "softmax %s" % dtn)}
-            if cpu:
-                line["cpu_baseline"] = sm_cpu()
-            ops.append(line)
-            view = Lg.permute(0, 2, 1, 3)
-            w, e = timed(ex, L, ex.bind_custom("softmax", [view], [Zs], i_args=[3]), steps, warmup)
-            line2 = {"op": "softmax %s permuted[0,2,1,3] view" % dtn, "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": hbm_entry(2 * es * nl, e, "softmax %s" % dtn)}
-            if cpu:
-                line2["cpu_baseline"] = dict(line["cpu_baseline"], sample=line["cpu_baseline"]["sample"] + " (dense rows; the view changes addresses only)")
-            ops.append(line2)
-            del Lg, Zs, dense, view
-        # config 2, the remaining sizes/dtypes
-        for dt, dtn, peak in [(FLOAT32, "f32", "f32"), (HALF, "f16", "f16"), (BFLOAT16, "bf16", "bf16")]:
-            for m in (1024, 4096):
-                for transb in (False, True):
-                    if dt == BFLOAT16 and m == 4096 and not transb:
-                        continue   # the headline
-                    rng = np.random.default_rng(2002)
-                    a = rng.normal(0, 1 / math.sqrt(m), (m, m)).astype(np.float32)
-                    b = rng.normal(0, 1 / math.sqrt(m), (m, m)).astype(np.float32)
-                    if dt == HALF:
-                        a, b = a.astype(np.float16), b.astype(np.float16)
-                    Am, Bm = NDArray.from_numpy(a, dt), NDArray.from_numpy(b, dt)
-                    Zm = NDArray.empty((m, m), dt)
-                    Am.sync_to_device(); Bm.sync_to_device()
-                    ia = [0, 1] if transb else []
-                    w, e = timed(ex, L, ex.bind_custom("matmul", [Am, Bm], [Zm], i_args=ia), steps, warmup)
-                    line = {"op": "mmul %s %d^3%s" % (dtn, m, " transposeB" if transb else ""), "ms": round(e, 4), "wall_ms": round(w, 4),
-                            "roofline": mfma_entry(2.0 * m * m * m, e, peak, "mmul %s %d^3%s" % (dtn, m, " transposeB" if transb else ""))}
-                    if cpu and not transb:
-                        # faithful: the reference's own loop for this type (fp32 goes to BLAS there, so the port of its plain loop is
-                        # the lower bound and OpenBLAS sgemm through numpy the figure to compare with); 16-bit: usualGemm in the type
-                        rows = 64 if dt == FLOAT32 else 32
-                        a32, b32 = np.asarray(a, np.float32), np.asarray(b, np.float32)
-                        if dt == BFLOAT16:
-                            oa, ob, oz = O.Arr(f32_to_bf16_bits(a32[:rows]), O.BFLOAT16), O.Arr(f32_to_bf16_bits(b32), O.BFLOAT16), O.Arr(np.zeros((rows, m), np.uint16), O.BFLOAT16)
-                        else:
-                            oa, ob, oz = O.Arr(np.ascontiguousarray(a[:rows])), O.Arr(np.ascontiguousarray(b)), O.Arr(np.zeros((rows, m), a.dtype))
-                        line["cpu_baseline"] = cpu_entry(2.0 * rows * m * m, 1e12, "TFLOP/s", lambda: O.matmul(oa, ob, oz, accumulate=0 if dt != FLOAT32 else 1),
-                                                         lambda: a32 @ b32, "first %d of %d rows of A against the full B (plain loop in the array type)" % (rows, m),
-                                                         "numpy fp32 sgemm (bundled OpenBLAS, all cores) on the whole %d^3 product%s" % (m, "" if dt == FLOAT32 else ", inputs widened to fp32"),
-                                                         fast_cores=os.cpu_count())
-                        # the fast figure is for the whole product, not the sample
-                        tq = best_time(lambda: a32 @ b32)
-                        line["cpu_baseline"]["fast"]["value"] = round(2.0 * m * m * m / tq / 1e12, 4)
-                    elif cpu:
-                        line["cpu_baseline"] = dict(ops[-1]["cpu_baseline"], sample=ops[-1]["cpu_baseline"]["sample"] + " (the plain-B measurement; the CPU loops do not depend on the layout flag)")
-                    ops.append(line)
-                    del Am, Bm, Zm
-        # config 4: attention prefill, causal
-        for dt, dtn in [(HALF, "f16"), (BFLOAT16, "bf16")]:
-            rng = np.random.default_rng(4004)
-            qs = (96, 1024, 64)
-            mk = lambda: rng.normal(0, 1, qs).astype(np.float32)
-            q, k, v = mk(), mk(), mk()
-            if dt == HALF:
-                q, k, v = q.astype(np.float16), k.astype(np.float16), v.astype(np.float16)
-            Q, K_, V = NDArray.from_numpy(q, dt), NDArray.from_numpy(k, dt), NDArray.from_numpy(v, dt)
-            O_ = NDArray.empty(qs, dt)
-            for arr in (Q, K_, V):
-                arr.sync_to_device()
-            w, e = timed(ex, L, ex.bind_custom("dot_product_attention_v2", [Q, V, K_], [O_], t_args=[0.125, 0.0], b_args=[True, False]),
-                         max(steps // 5, 3), max(warmup // 5, 1))
-            line = {"op": "dot_product_attention_v2 %s causal [96,1024,64] (output only)" % dtn, "ms": round(e, 4), "wall_ms": round(w, 4),
-                    "roofline": mfma_entry(4.0 * 96 * 1024 * 1024 * 64, e, dtn, "dot_product_attention_v2"),
-                    "note": "achieved counts the dense 4*B*T*T*D flops; the causal mask makes about half of them useful"}
-            if cpu:
-                nb = 2
-                cv = (lambda t: O.Arr(f32_to_bf16_bits(np.asarray(t, np.float32)), O.BFLOAT16)) if dt == BFLOAT16 else (lambda t: O.Arr(np.ascontiguousarray(t)))
-                oq, ok_, ov = cv(q[:nb]), cv(k[:nb]), cv(v[:nb])
-                oo = cv(np.zeros((nb, 1024, 64), np.float32 if dt == BFLOAT16 else np.float16))
-                q32, k32, v32 = (np.asarray(t[:nb], np.float32) for t in (q, k, v))
+                dense = Lg.reshape(16, 12, 1024, 1024)
+                w, e = timed(ex, L, ex.bind_custom("softmax", [dense], [Zs], i_args=[3]), steps, warmup)
+                line = {"op": "softmax %s [16,12,1024,1024]" % dtn, "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": hbm_entry(2 * es * nl, e, "softmax %s" % dtn)}
+                if cpu:
+                    line["cpu_baseline"] = sm_cpu()
+                ops.append(line)
+                view = Lg.permute(0, 2, 1, 3)
+                w, e = timed(ex, L, ex.bind_custom("softmax", [view], [Zs], i_args=[3]), steps, warmup)
+                line2 = {"op": "softmax %s permuted[0,2,1,3] view" % dtn, "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": hbm_entry(2 * es * nl, e, "softmax %s" % dtn)}
+                if cpu:
+                    line2["cpu_baseline"] = dict(line["cpu_baseline"], sample=line["cpu_baseline"]["sample"] + " (dense rows; the view changes addresses only)")
+                ops.append(line2)
+                del Lg, Zs, dense, view
+        if 2 in cfgs:
+            # config 2, the remaining sizes/dtypes
+            for dt, dtn, peak in [(FLOAT32, "f32", "f32"), (HALF, "f16", "f16"), (BFLOAT16, "bf16", "bf16")]:
+                for m in (1024, 4096):
+                    for transb in (False, True):
+                        if dt == BFLOAT16 and m == 4096 and not transb:
+                            continue   # the headline
+                        rng = np.random.default_rng(2002)
+                        a = rng.normal(0, 1 / math.sqrt(m), (m, m)).astype(np.float32)
+                        b = rng.normal(0, 1 / math.sqrt(m), (m, m)).astype(np.float32)
+                        if dt == HALF:
+                            a, b = a.astype(np.float16), b.astype(np.float16)
+                        Am, Bm = NDArray.from_numpy(a, dt), NDArray.from_numpy(b, dt)
+                        Zm = NDArray.empty((m, m), dt)
+                        Am.sync_to_device(); Bm.sync_to_device()
+                        ia = [0, 1] if transb else []
+                        w, e = timed(ex, L, ex.bind_custom("matmul", [Am, Bm], [Zm], i_args=ia), steps, warmup)
+                        line = {"op": "mmul %s %d^3%s" % (dtn, m, " transposeB" if transb else ""), "ms": round(e, 4), "wall_ms": round(w, 4),
+                                "roofline": mfma_entry(2.0 * m * m * m, e, peak, "mmul %s %d^3%s" % (dtn, m, " transposeB" if transb else ""))}
+                        if cpu and not transb:
+                            # faithful: the reference's own loop for this type (fp32 goes to BLAS there, so the port of its plain loop is
+                            # the lower bound and OpenBLAS sgemm through numpy the figure to compare with); 16-bit: usualGemm in the type
+                            rows = 64 if dt == FLOAT32 else 32
+                            a32, b32 = np.asarray(a, np.float32), np.asarray(b, np.float32)
+                            if dt == BFLOAT16:
+                                oa, ob, oz = O.Arr(f32_to_bf16_bits(a32[:rows]), O.BFLOAT16), O.Arr(f32_to_bf16_bits(b32), O.BFLOAT16), O.Arr(np.zeros((rows, m), np.uint16), O.BFLOAT16)
+                            else:
+                                oa, ob, oz = O.Arr(np.ascontiguousarray(a[:rows])), O.Arr(np.ascontiguousarray(b)), O.Arr(np.zeros((rows, m), a.dtype))
+                            line["cpu_baseline"] = cpu_entry(2.0 * rows * m * m, 1e12, "TFLOP/s", lambda: O.matmul(oa, ob, oz, accumulate=0 if dt != FLOAT32 else 1),
+                                                             lambda: a32 @ b32, "first %d of %d rows of A against the full B (plain loop in the array type)" % (rows, m),
+                                                             "numpy fp32 sgemm (bundled OpenBLAS, all cores) on the whole %d^3 product%s" % (m, "" if dt == FLOAT32 else ", inputs widened to fp32"),
+                                                             fast_cores=os.cpu_count())
+                            # the fast figure is for the whole product, not the sample
+                            tq = best_time(lambda: a32 @ b32)
+                            line["cpu_baseline"]["fast"]["value"] = round(2.0 * m * m * m / tq / 1e12, 4)
+                        elif cpu:
+                            line["cpu_baseline"] = dict(ops[-1]["cpu_baseline"], sample=ops[-1]["cpu_baseline"]["sample"] + " (the plain-B measurement; the CPU loops do not depend on the layout flag)")
+                        ops.append(line)
+                        del Am, Bm, Zm
+        if 4 in cfgs:
+            # config 4: attention prefill, causal
+            for dt, dtn in [(HALF, "f16"), (BFLOAT16, "bf16")]:
+                rng = np.random.default_rng(4004)
+                qs = (96, 1024, 64)
+                mk = lambda: rng.normal(0, 1, qs).astype(np.float32)
+                q, k, v = mk(), mk(), mk()
+                if dt == HALF:
+                    q, k, v = q.astype(np.float16), k.astype(np.float16), v.astype(np.float16)
+                Q, K_, V = NDArray.from_numpy(q, dt), NDArray.from_numpy(k, dt), NDArray.from_numpy(v, dt)
+                O_ = NDArray.empty(qs, dt)
+                for arr in (Q, K_, V):
+                    arr.sync_to_device()
+                w, e = timed(ex, L, ex.bind_custom("dot_product_attention_v2", [Q, V, K_], [O_], t_args=[0.125, 0.0], b_args=[True, False]),
+                             max(steps // 5, 3), max(warmup // 5, 1))
+                line = {"op": "dot_product_attention_v2 %s causal [96,1024,64] (output only)" % dtn, "ms": round(e, 4), "wall_ms": round(w, 4),
+                        "roofline": mfma_entry(4.0 * 96 * 1024 * 1024 * 64, e, dtn, "dot_product_attention_v2"),
+                        "note": "achieved counts the dense 4*B*T*T*D flops; the causal mask makes about half of them useful"}
+                if cpu:
+                    nb = 2
+                    cv = (lambda t: O.Arr(f32_to_bf16_bits(np.asarray(t, np.float32)), O.BFLOAT16)) if dt == BFLOAT16 else (lambda t: O.Arr(np.ascontiguousarray(t)))
+                    oq, ok_, ov = cv(q[:nb]), cv(k[:nb]), cv(v[:nb])
+                    oo = cv(np.zeros((nb, 1024, 64), np.float32 if dt == BFLOAT16 else np.float16))
+                    q32, k32, v32 = (np.asarray(t[:nb], np.float32) for t in (q, k, v))
 
-                def fast():
-                    lg = np.einsum("bid,bjd->bij", q32, k32) * 0.125
-                    lg = np.where(np.tril(np.ones((1024, 1024), bool)), lg, -1e9)
-                    ee = np.exp(lg - lg.max(-1, keepdims=True))
-                    return (ee / ee.sum(-1, keepdims=True)) @ v32
-                line["cpu_baseline"] = cpu_entry(4.0 * nb * 1024 * 1024 * 64, 1e12, "TFLOP/s", lambda: O.attention_v2(oq, ov, ok_, oo, scale=0.125, causal=True), fast,
-                                                 "first %d of 96 batch entries (dense flop count)" % nb, "numpy einsum / exp / matmul in fp32", fast_cores=os.cpu_count())
-            ops.append(line)
-            del Q, K_, V, O_
-        result["ops"] = ops
+                    def fast():
+                        lg = np.einsum("bid,bjd->bij", q32, k32) * 0.125
+                        lg = np.where(np.tril(np.ones((1024, 1024), bool)), lg, -1e9)
+                        ee = np.exp(lg - lg.max(-1, keepdims=True))
+                        return (ee / ee.sum(-1, keepdims=True)) @ v32
+                    line["cpu_baseline"] = cpu_entry(4.0 * nb * 1024 * 1024 * 64, 1e12, "TFLOP/s", lambda: O.attention_v2(oq, ov, ok_, oo, scale=0.125, causal=True), fast,
+                                                     "first %d of 96 batch entries (dense flop count)" % nb, "numpy einsum / exp / matmul in fp32", fast_cores=os.cpu_count())
+                ops.append(line)
+                del Q, K_, V, O_
+            result["ops"] = ops
     if not args.skip_decode:
         print("[bench] decode leg", file=sys.stderr, flush=True)
         ops = result.setdefault("ops", [])
