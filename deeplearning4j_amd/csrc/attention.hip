@@ -278,21 +278,53 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
       }
     }
     // scores of this lane's query: register r of tile kt is key kv0 + 32*kt + 8*(r/4) + 4*h + r%4.
-    // scale, clip to +-1e4, round through the storage type (two scores per conversion)
-    float tmax = m;
-#pragma unroll
-    for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-      for (int r = 0; r < 16; r += 2) {
-        float v0 = s[kt][r], v1 = s[kt][r + 1];
-        if (!FOLD) { v0 *= sc; v1 *= sc; }
-        v0 = __builtin_amdgcn_fmed3f(v0, -clip, clip);
-        v1 = __builtin_amdgcn_fmed3f(v1, -clip, clip);
-        round_pair<T>(v0, v1);
-        s[kt][r] = v0; s[kt][r + 1] = v1;
-      }
-    // only tiles that touch the diagonal or the end of the keys carry masked entries (wave-uniform test)
+    // scale, clip to +-1e4, round through the storage type (two scores per conversion).  The clip is one instruction per
+    // score that almost never changes anything, so tiles without masked entries first take the maximum of the raw scores:
+    // scaling by a positive factor, clipping and rounding are monotonic, so the tile's maximum after all three is the
+    // three applied to that one value, and when it does not exceed the clip no score does.  At the lower end a score below
+    // -clip and its clipped value both give an exponential of exactly 0 once the running maximum lies 160 / log2(e)
+    // above -clip.  Only when a wave fails one of the two tests (or the scale is not positive) does it clip every score.
     const int qFirst = (int)q0 + wave * 32;
+    const bool maskedTile = VM || __builtin_amdgcn_readfirstlane((int)((a.causal && (int)kv0 + BKV - 1 > qFirst) || kv0 + BKV > a.Tv)) != 0;
+    float tmax = m;
+    bool clipAll = true;
+    if (!maskedTile) {
+      float rmax = s[0][0];
+#pragma unroll
+      for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) rmax = __builtin_fmaxf(rmax, s[kt][r]);
+      const float smax = FOLD ? rmax : rmax * sc;
+      tmax = __builtin_fmaxf(m, round_storage<T>(__builtin_amdgcn_fmed3f(smax, -clip, clip)));
+      tmax = __builtin_fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+      const bool fast = sc > 0.f && smax <= clip && tmax >= 160.f / L2E - clip;
+      clipAll = __builtin_amdgcn_ballot_w64(!fast) != 0;
+    }
+    if (clipAll) {
+      asm volatile("; scores clipped one by one");
+#pragma unroll
+      for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          float v0 = s[kt][r], v1 = s[kt][r + 1];
+          if (!FOLD) { v0 *= sc; v1 *= sc; }
+          v0 = __builtin_amdgcn_fmed3f(v0, -clip, clip);
+          v1 = __builtin_amdgcn_fmed3f(v1, -clip, clip);
+          round_pair<T>(v0, v1);
+          s[kt][r] = v0; s[kt][r + 1] = v1;
+        }
+    } else {
+#pragma unroll
+      for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          float v0 = s[kt][r], v1 = s[kt][r + 1];
+          if (!FOLD) { v0 *= sc; v1 *= sc; }
+          round_pair<T>(v0, v1);
+          s[kt][r] = v0; s[kt][r + 1] = v1;
+        }
+    }
+    // only tiles that touch the diagonal or the end of the keys carry masked entries (wave-uniform test)
     // a real branch (scalar condition, a body the compiler cannot speculate): turned into selects, the mask costs 86
     // vector instructions on every tile instead of on the few that need it
     if (VM) {
@@ -310,7 +342,7 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
             else if (key > lastVisible || vm[key] == 0) s[kt][4 * r4 + e] = round_storage<T>(sv - a.maskValue);
           }
         }
-    } else if (__builtin_amdgcn_readfirstlane((int)((a.causal && (int)kv0 + BKV - 1 > qFirst) || kv0 + BKV > a.Tv)) != 0) {
+    } else if (maskedTile) {
       asm volatile("; tile with masked entries");
       const int lastKey = a.causal ? ((int)query < (int)a.Tv - 1 ? (int)query : (int)a.Tv - 1) : (int)a.Tv - 1;
 #pragma unroll
@@ -321,11 +353,13 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
           s[kt][r] = key > lastKey ? -1.0e30f : s[kt][r];
         }
     }
+    if (maskedTile) {   // the maximum of what is left after masking
 #pragma unroll
-    for (int kt = 0; kt < 2; kt++)
+      for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) tmax = __builtin_fmaxf(tmax, s[kt][r]);
-    tmax = __builtin_fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+        for (int r = 0; r < 16; r++) tmax = __builtin_fmaxf(tmax, s[kt][r]);
+      tmax = __builtin_fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+    }
     // every query has seen key 0 by now, so the running maximum is a real score and masked entries (-1e30)
     // underflow to exactly 0 in the exponential
     const float mL = tmax * L2E;

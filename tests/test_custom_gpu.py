@@ -406,6 +406,42 @@ def test_attention_vs_oracle(ex, oracle, dtype, tol, causal, B, Tq, Tv, D):
     assert_close(out1.to_float(), _f(oo), tol, tol, "out-only call")
 
 
+@pytest.mark.parametrize("dtype,tol", [(HALF, 1e-2), (BFLOAT16, 1e-2)])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("scale", [0.125, 0.11])
+def test_attention_scores_beyond_the_clip(ex, oracle, dtype, tol, causal, scale):
+    """Scaled scores on both sides of the +-1e4 clip (AttentionHelper.cpp:340-352) in some key tiles and not in others:
+    the fused kernel clips score by score only in tiles whose maximum calls for it, and must give what the oracle's
+    clip of every score gives.  Rows differ in which keys tie at the clip, so a missed clip moves the output."""
+    B, T, D = 2, 384, 64
+    rng = np.random.default_rng(77)
+    q = rng.normal(0, 1, (B, T, D))
+    k = rng.normal(0, 1, (B, T, D))
+    v = rng.normal(0, 1, (B, T, D))
+    # a few long query / key pairs along one direction d: |q.k| * scale reaches 4e4 .. 6e4 there, of both signs; everything
+    # else is orthogonal to d (a power of two in one coordinate, so exactly in every storage type) and keeps ordinary scores.
+    # Key tile 0 (keys 0-63) is visible to every query under the causal mask, later tiles only to later queries.
+    q[:, :, 0] = 0.0
+    k[:, :, 0] = 0.0
+    for b in range(B):
+        for qi in (5, 130, 131, 260, 383):
+            q[b, qi, 0] = 512.0
+        for kj, mag in ((3, 768.0), (40, 1024.0), (41, -1024.0), (100, 896.0), (200, -768.0), (300, 1024.0), (301, 640.0)):
+            k[b, kj, 0] = mag
+    oq, dq = _pair(oracle, q, dtype)
+    ok, dk = _pair(oracle, k, dtype)
+    ov, dv = _pair(oracle, v, dtype)
+    oo, ow, ol = _ozeros(oracle, (B, T, D), dtype), _ozeros(oracle, (B, T, T), dtype), _ozeros(oracle, (B, T, T), dtype)
+    oracle.attention_v2(oq, ov, ok, oo, ow, ol, scale=scale, causal=causal)
+    lg = _f(ol)
+    fin = lg[:, np.tril(np.ones((T, T), bool)) if causal else np.ones((T, T), bool)]   # the visible entries
+    assert (np.abs(fin) >= 9.9e3).sum() >= 20 and (np.abs(fin) < 2e3).mean() > 0.9, "the case must have clipped and ordinary scores"
+    out1 = ex.exec_custom("dot_product_attention_v2", [dq, dv, dk], [NDArray.empty((B, T, D), dtype)], t_args=[scale, 0.0], b_args=[causal, False])[0]
+    assert_close(out1.to_float(), _f(oo), tol, tol, "output-only call")
+    out3 = ex.exec_custom("dot_product_attention_v2", [dq, dv, dk], t_args=[scale, 0.0], b_args=[causal, False])[0]
+    assert_close(out3.to_float(), _f(oo), tol, tol, "three-output call")
+
+
 @pytest.mark.parametrize("dtype,tol", [(FLOAT32, 1e-4), (HALF, 1e-2), (BFLOAT16, 1e-2)])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("B,Tq,Tv,D", [(3, 64, 64, 64), (2, 200, 200, 64), (2, 130, 300, 64), (2, 4, 150, 64), (1, 37, 91, 32)])
