@@ -1,0 +1,210 @@
+"""Seeded random sweep of the legacy loops over arbitrary views: rank 1-5, axes in any memory order, gaps between
+elements, offsets, zero strides on inputs, every operand with a layout of its own.  The expectation is numpy on the
+logical values (one IEEE operation per element, or a selection: identical bits; sums within the re-ordering bound), so
+what is under test is the shape walk of the kernels behind execPairwiseTransform / execTransformSame / execScalar /
+execBroadcast / execReduceSame / execIndexReduce (reference: helpers/shape.h:588-740 INDEX2COORDS / COORDS2INDEX, which
+every loop in loops/cpu/*.hpp goes through)."""
+import numpy as np
+import pytest
+
+from deeplearning4j_amd.executioner import Broadcast, IndexReduce, Pairwise, ReduceSame, Scalar, TransformSame
+from deeplearning4j_amd.ndarray import (BFLOAT16, DOUBLE, DT_NP, FLOAT32, HALF, INT32, INT64, DataBuffer, NDArray, bf16_bits_to_f32,
+                                        f32_to_bf16_bits)
+from deeplearning4j_amd import nativeops as N
+
+pytestmark = pytest.mark.gpu
+
+FLOATS = [FLOAT32, HALF, BFLOAT16, DOUBLE]
+ALL = FLOATS + [INT32, INT64]
+
+
+def logical(a, dt):
+    """stored values -> the numbers they stand for (bf16 travels as bit patterns)"""
+    return bf16_bits_to_f32(a) if dt == BFLOAT16 else a
+
+
+def store(v, dt):
+    """numbers -> stored values, rounded to nearest even where the type is narrower"""
+    if dt == BFLOAT16:
+        return f32_to_bf16_bits(np.asarray(v, np.float32))
+    return np.asarray(v).astype(DT_NP[dt])
+
+
+def random_shape(rng, max_rank=5, max_len=4000):
+    while True:
+        rank = int(rng.integers(1, max_rank + 1))
+        shape = [int(rng.choice([1, 2, 3, 4, 5, 7, 8, 16, 17, 33, 64])) for _ in range(rank)]
+        if np.prod(shape) <= max_len:
+            return shape
+
+
+def random_view(rng, shape, dt, values=None, writable=False):
+    """A device array of `shape` laid out at random inside a larger buffer, filled with `values` (or random ones).
+    Returns (NDArray, logical numpy values)."""
+    rank = len(shape)
+    order = list(rng.permutation(rank))                     # memory order of the axes, innermost first
+    strides = [0] * rank
+    run = 1
+    for ax in order:
+        gap = int(rng.choice([1, 1, 1, 2, 3]))
+        if not writable and shape[ax] > 1 and rng.random() < 0.08:
+            strides[ax] = 0                                 # a broadcast view: every index of the axis is one element
+            continue
+        strides[ax] = run * gap
+        run = strides[ax] * shape[ax]
+    offset = int(rng.integers(0, 9))
+    extent = offset + sum((s - 1) * st for s, st in zip(shape, strides)) + 1
+    n = extent + int(rng.integers(0, 5))
+    buf = DataBuffer(n, dt)
+    host = buf.host_view()
+    if dt in (INT32, INT64):
+        fill = rng.integers(-50, 50, n)
+    else:
+        fill = rng.uniform(-2, 2, n)
+    host[:n] = store(fill, dt)
+    arr = NDArray(buf, shape, strides, dt, offset)
+    item = host.itemsize
+    v = np.lib.stride_tricks.as_strided(host[offset:], shape=shape, strides=[s * item for s in strides], writeable=True)
+    if values is not None:
+        assert writable or 0 not in [st for s, st in zip(shape, strides) if s > 1]
+        v[...] = store(values, dt).reshape(shape)
+    N.load().dbTickHostWrite(buf.ptr)
+    return arr, np.array(logical(np.array(v), dt)), (np.array(host[:n]), offset, strides)
+
+
+def untouched_outside(arr, before):
+    """the elements of the buffer that the view does not cover still hold what they held"""
+    host0, offset, strides = before
+    arr.to_numpy()                                          # device -> host
+    host = arr.buffer.host_view()[: host0.size]
+    mask = np.ones(host0.size, bool)
+    idx = np.zeros(arr.shape, np.int64) + offset
+    for ax, (s, st) in enumerate(zip(arr.shape, strides)):
+        sh = [1] * len(arr.shape); sh[ax] = s
+        idx = idx + (np.arange(s) * st).reshape(sh)
+    mask[idx.ravel()] = False
+    return np.array_equal(np.array(host)[mask], host0[mask])
+
+
+PW = {Pairwise.Add: np.add, Pairwise.Subtract: np.subtract, Pairwise.Multiply: np.multiply}
+
+
+def test_pairwise_on_random_views(ex):
+    rng = np.random.default_rng(20240)
+    for case in range(90):
+        dt = ALL[case % len(ALL)]
+        shape = random_shape(rng)
+        op = list(PW)[case % 3]
+        x, xv, _ = random_view(rng, shape, dt)
+        y, yv, _ = random_view(rng, shape, dt)
+        z, _, before = random_view(rng, shape, dt, writable=True)
+        ex.exec_pairwise(op, x, y, z)
+        acc = np.float64 if dt == DOUBLE else np.int64 if dt in (INT32, INT64) else np.float32
+        want = store(PW[op](xv.astype(acc), yv.astype(acc)), dt)
+        got = z.to_numpy()
+        assert np.array_equal(got, want), "case %d: op %d dtype %d shape %s x%s y%s z%s" % (case, op, dt, shape, x.strides, y.strides, z.strides)
+        assert untouched_outside(z, before), "case %d wrote outside its view" % case
+
+
+def test_transform_and_scalar_on_random_views(ex):
+    rng = np.random.default_rng(20241)
+    for case in range(90):
+        dt = ALL[case % len(ALL)]
+        shape = random_shape(rng)
+        x, xv, _ = random_view(rng, shape, dt)
+        z, _, before = random_view(rng, shape, dt, writable=True)
+        acc = np.float64 if dt == DOUBLE else np.int64 if dt in (INT32, INT64) else np.float32
+        kind = case % 3
+        if kind == 0:
+            ex.exec_transform_same(TransformSame.Abs, x, z)
+            want = store(np.abs(xv.astype(acc)), dt)
+        elif kind == 1:
+            ex.exec_transform_same(TransformSame.Neg, x, z)
+            want = store(-xv.astype(acc), dt)
+        else:
+            sc = 3 if dt in (INT32, INT64) else 0.75
+            ex.exec_scalar(Scalar.Add, x, NDArray.scalar(sc, dt), z)
+            want = store(xv.astype(acc) + acc(sc), dt)
+        assert np.array_equal(z.to_numpy(), want), "case %d: kind %d dtype %d shape %s x%s z%s" % (case, kind, dt, shape, x.strides, z.strides)
+        assert untouched_outside(z, before), "case %d wrote outside its view" % case
+
+
+def test_broadcast_on_random_views(ex):
+    rng = np.random.default_rng(20242)
+    for case in range(60):
+        dt = FLOATS[case % len(FLOATS)]
+        shape = random_shape(rng, max_rank=4)
+        rank = len(shape)
+        k = int(rng.integers(1, rank + 1))
+        dims = sorted(int(d) for d in rng.choice(rank, size=k, replace=False))
+        x, xv, _ = random_view(rng, shape, dt)
+        y, yv, _ = random_view(rng, [shape[d] for d in dims], dt)
+        z, _, before = random_view(rng, shape, dt, writable=True)
+        ex.exec_broadcast(Broadcast.Add, x, y, dims, z)
+        sh = [shape[d] if d in dims else 1 for d in range(rank)]
+        acc = np.float64 if dt == DOUBLE else np.float32
+        want = store(xv.astype(acc) + yv.astype(acc).reshape(sh), dt)
+        assert np.array_equal(z.to_numpy(), want), "case %d: dtype %d shape %s dims %s" % (case, dt, shape, dims)
+        assert untouched_outside(z, before), "case %d wrote outside its view" % case
+
+
+def test_reductions_on_random_views(ex):
+    rng = np.random.default_rng(20243)
+    for case in range(90):
+        dt = [FLOAT32, DOUBLE, INT32, INT64, HALF, BFLOAT16][case % 6]
+        shape = random_shape(rng, max_rank=4, max_len=20000)
+        rank = len(shape)
+        k = int(rng.integers(0, rank + 1))
+        dims = sorted(int(d) for d in rng.choice(rank, size=k, replace=False)) if k else None
+        x, xv, _ = random_view(rng, shape, dt)
+        zshape = [s for d, s in enumerate(shape) if dims is not None and d not in dims] if dims else []
+        op = [ReduceSame.Sum, ReduceSame.Max, ReduceSame.Min][case % 3]
+        if len(zshape):
+            z, _, before = random_view(rng, zshape, dt, writable=True)
+        else:
+            z, before = NDArray.empty(zshape, dt), None
+        ex.exec_reduce_same(op, x, dims, z=z)
+        axes = tuple(dims) if dims else None
+        got = np.asarray(logical(z.to_numpy(), dt)).reshape(np.shape(xv.sum(axis=axes)))
+        if op == ReduceSame.Sum:
+            if dt in (INT32, INT64):
+                want = xv.astype(np.int64).sum(axis=axes).astype(DT_NP[dt])
+                assert np.array_equal(got, want), "case %d: int sum shape %s dims %s" % (case, shape, dims)
+            else:
+                want = xv.astype(np.float64).sum(axis=axes)
+                mag = np.abs(xv.astype(np.float64)).sum(axis=axes)
+                eps = {FLOAT32: 2.0 ** -23, DOUBLE: 2.0 ** -52, HALF: 2.0 ** -10, BFLOAT16: 2.0 ** -7}[dt]
+                n = xv.size / max(np.size(want), 1)
+                assert np.all(np.abs(got - want) <= eps * (np.abs(want) + 1e-30) + (2.0 ** -23 if dt in (HALF, BFLOAT16) else eps) * n * mag), \
+                    "case %d: sum dtype %d shape %s dims %s strides %s" % (case, dt, shape, dims, x.strides)
+        else:
+            want = (np.max if op == ReduceSame.Max else np.min)(xv, axis=axes)
+            assert np.array_equal(got, want), "case %d: op %d dtype %d shape %s dims %s strides %s" % (case, op, dt, shape, dims, x.strides)
+        if before is not None:
+            assert untouched_outside(z, before), "case %d wrote outside its view" % case
+
+
+def test_index_reduce_on_random_views(ex):
+    rng = np.random.default_rng(20244)
+    for case in range(60):
+        dt = [FLOAT32, HALF, BFLOAT16, INT32, DOUBLE][case % 5]
+        shape = random_shape(rng, max_rank=4, max_len=2000)
+        rank = len(shape)
+        n = int(np.prod(shape))
+        # distinct values, exactly representable in every type (|v| < 2^8 in steps of 1/2 at most 2000 of them is too many for
+        # bf16, so values repeat there: ties go to the lowest index, as numpy's argmax does)
+        vals = rng.permutation(n).astype(np.float64) - n // 2
+        if dt in (HALF, BFLOAT16):
+            vals = np.round(vals / max(n / 200.0, 1.0))
+        x, xv, _ = random_view(rng, shape, dt, values=vals.reshape(shape), writable=True)
+        full = case % 4 == 0
+        op = IndexReduce.IndexMax if case % 2 == 0 else IndexReduce.IndexMin
+        if full:
+            z = ex.exec_index_reduce(op, x)
+            want = (np.argmax if op == IndexReduce.IndexMax else np.argmin)(xv.ravel())
+            assert int(z.to_numpy()) == int(want), "case %d: full shape %s strides %s" % (case, shape, x.strides)
+        else:
+            d = int(rng.integers(0, rank))
+            z = ex.exec_index_reduce(op, x, [d])
+            want = (np.argmax if op == IndexReduce.IndexMax else np.argmin)(xv, axis=d)
+            assert np.array_equal(z.to_numpy().reshape(want.shape), want), "case %d: dim %d shape %s strides %s" % (case, d, shape, x.strides)
