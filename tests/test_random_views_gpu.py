@@ -208,3 +208,46 @@ def test_index_reduce_on_random_views(ex):
             z = ex.exec_index_reduce(op, x, [d])
             want = (np.argmax if op == IndexReduce.IndexMax else np.argmin)(xv, axis=d)
             assert np.array_equal(z.to_numpy().reshape(want.shape), want), "case %d: dim %d shape %s strides %s" % (case, d, shape, x.strides)
+
+
+def test_matmul_on_random_shapes_layouts_and_flags(ex):
+    """matmul (ops/declarable/generic/blas/matmul.cpp:36-170: transpose flags as integer arguments, alpha and beta as
+    floating ones, leading batch dimensions) over random sizes from one row to a few hundred, every combination of flags,
+    operands dense or as pitched views, against numpy in fp64.  The sizes straddle every dispatch boundary of the GEMM
+    (GEMV, skinny, split-K, small and large tiles, ragged edges)."""
+    rng = np.random.default_rng(20245)
+    sizes = [1, 2, 3, 5, 8, 17, 31, 32, 33, 64, 65, 96, 127, 128, 129, 200, 256, 257, 384]
+    for case in range(72):
+        dt = [FLOAT32, BFLOAT16, HALF][case % 3]
+        M, N, K = (int(rng.choice(sizes)) for _ in range(3))
+        ta, tb = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        batch = [] if case % 4 else [int(rng.integers(1, 4))]
+        alpha, beta = (1.0, 0.0) if case % 5 else (0.5, 2.0)
+        pitched = case % 3 == 1
+
+        def operand(rows, cols):
+            shape = batch + [rows, cols]
+            vals = rng.uniform(-1, 1, shape) / np.sqrt(K)
+            if not pitched:
+                arr = NDArray.from_numpy(store(vals, dt), dt)
+                return arr, np.asarray(logical(arr.to_numpy(), dt), np.float64)
+            big = NDArray.from_numpy(store(rng.uniform(-1, 1, batch + [rows + 3, cols + 8]), dt), dt)
+            v = big.slice(len(batch), 1, rows + 1).slice(len(batch) + 1, 8, cols + 8)
+            v.assign_numpy(store(vals, dt))
+            return v, np.asarray(logical(v.to_numpy(), dt), np.float64)
+
+        a, av = operand(K, M) if ta else operand(M, K)
+        b, bv = operand(N, K) if tb else operand(K, N)
+        c0 = rng.uniform(-1, 1, batch + [M, N])
+        c = NDArray.from_numpy(store(c0, dt), dt)
+        cv = np.asarray(logical(c.to_numpy(), dt), np.float64)
+        A = np.swapaxes(av, -1, -2) if ta else av
+        B = np.swapaxes(bv, -1, -2) if tb else bv
+        want = alpha * (A @ B) + (beta * cv if beta else 0.0)
+        ex.exec_custom("matmul", [a, b], [c], t_args=[alpha, beta], i_args=[int(ta), int(tb)])
+        got = np.asarray(logical(c.to_numpy(), dt), np.float64)
+        tol = {FLOAT32: 2e-6, BFLOAT16: 6e-3, HALF: 8e-4}[dt]
+        bound = tol * (alpha * (np.abs(A) @ np.abs(B)) + abs(beta) * np.abs(cv) + np.abs(want)) + (6e-8 if dt == HALF else 1e-30)   # fp16: subnormal spacing
+        kern = ex.L.nd4jhipLastGemmKernel().decode()
+        assert np.all(np.abs(got - want) <= bound), "case %d: dtype %d M %d N %d K %d ta %d tb %d batch %s alpha %g beta %g pitched %d kernel %s: worst %g of bound" % (
+            case, dt, M, N, K, ta, tb, batch, alpha, beta, pitched, kern, float(np.max(np.abs(got - want) / bound)))
