@@ -251,3 +251,67 @@ def test_matmul_on_random_shapes_layouts_and_flags(ex):
         kern = ex.L.nd4jhipLastGemmKernel().decode()
         assert np.all(np.abs(got - want) <= bound), "case %d: dtype %d M %d N %d K %d ta %d tb %d batch %s alpha %g beta %g pitched %d kernel %s: worst %g of bound" % (
             case, dt, M, N, K, ta, tb, batch, alpha, beta, pitched, kern, float(np.max(np.abs(got - want) / bound)))
+
+
+def _opair(oracle, a, dt):
+    if dt == BFLOAT16:
+        bits = f32_to_bf16_bits(np.asarray(a, np.float32))
+        return oracle.Arr(bits, oracle.BFLOAT16), NDArray.from_numpy(bits, BFLOAT16)
+    h = np.asarray(a).astype(DT_NP[dt])
+    return oracle.Arr(h), NDArray.from_numpy(h)
+
+
+def _ozero(oracle, shape, dt):
+    return oracle.Arr(np.zeros(shape, np.uint16 if dt == BFLOAT16 else DT_NP[dt]), dt)
+
+
+def _ovals(oa):
+    return bf16_bits_to_f32(oa.a).astype(np.float64) if oa.dt == BFLOAT16 else oa.a.astype(np.float64)
+
+
+ROW_LENGTHS = [1, 2, 3, 7, 8, 31, 63, 64, 65, 127, 128, 255, 256, 257, 384, 512, 640, 767, 768, 769, 1000, 1023, 1024, 1025, 1536, 2048,
+               2049, 3072, 4096, 4100, 6000, 8192, 8200, 12000]
+
+
+def test_row_ops_over_row_lengths_and_row_counts(ex, oracle):
+    """softmax, layer_norm and gelu (helpers/cpu/softmax.cpp:260-347, generic/nn/layer_norm.cpp:35-79 over standardize.cpp:34-78,
+    ops/ops.h GELU) for every row length around the switch points of the row kernels (rows held in one wave's registers, in
+    one block, walked in pieces), few and many rows (the layer_norm for many rows is a kernel of its own), dense and pitched
+    rows, against the CPU oracle."""
+    rng = np.random.default_rng(20246)
+    case = 0
+    for C in ROW_LENGTHS:
+        for rows in ([3, 37] if C > 2048 else [1, 5, 37, 4097 if C <= 1024 else 130]):
+            dt = [FLOAT32, BFLOAT16, HALF][case % 3]
+            case += 1
+            rtol, atol = {FLOAT32: (2e-5, 2e-6), BFLOAT16: (1e-2, 1e-2), HALF: (2e-3, 2e-3)}[dt]
+            a = rng.normal(0, 1.5, (rows, C))
+            ox, dx = _opair(oracle, a, dt)
+            if case % 4 == 0 and C >= 8:               # pitched rows: a column slice of a wider array
+                wide = np.concatenate([rng.normal(0, 1, (rows, 8)), a, rng.normal(0, 1, (rows, 8))], axis=1)
+                _, dw = _opair(oracle, wide, dt)
+                dx = dw.slice(1, 8, 8 + C)
+            tag = "rows %d x %d dtype %d pitched %d" % (rows, C, dt, case % 4 == 0 and C >= 8)
+            # softmax along the rows
+            oz = _ozero(oracle, (rows, C), dt)
+            oracle.softmax(ox, oz, 1)
+            z = ex.exec_custom("softmax", [dx], [NDArray.empty((rows, C), dt)], i_args=[1])[0]
+            got, want = z.to_float().astype(np.float64), _ovals(oz)
+            assert np.all(np.abs(got - want) <= atol * 1e-2 + rtol * np.abs(want)), "softmax " + tag
+            # layer_norm with gain and bias
+            g, b = rng.normal(1, 0.2, C), rng.normal(0, 0.2, C)
+            og, dg = _opair(oracle, g, dt)
+            ob, db = _opair(oracle, b, dt)
+            oz = _ozero(oracle, (rows, C), dt)
+            oracle.layer_norm(ox, og, ob, oz, [1], channels_first=False)
+            if C > 1:                                   # one element: the reference divides 0 by a zero deviation
+                z = ex.exec_custom("layer_norm", [dx, dg, db], [NDArray.empty((rows, C), dt)], i_args=[1], b_args=[False])[0]
+                got, want = z.to_float().astype(np.float64), _ovals(oz)
+                assert np.all(np.abs(got - want) <= atol + rtol * np.abs(want)), "layer_norm " + tag
+            # gelu
+            from deeplearning4j_amd.executioner import TransformStrict
+            oz = _ozero(oracle, (rows, C), dt)
+            oracle.transform_strict(TransformStrict.GELU, ox, oz)
+            z = ex.exec_transform_strict(TransformStrict.GELU, dx, NDArray.empty((rows, C), dt))
+            got, want = z.to_float().astype(np.float64), _ovals(oz)
+            assert np.all(np.abs(got - want) <= atol * 1e-1 + rtol * np.abs(want)), "gelu " + tag
