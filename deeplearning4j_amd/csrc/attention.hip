@@ -9,7 +9,8 @@
 //                   reductions run over a lane's own registers plus one exchange with the other half-wave.
 //                   P^T feeds the second MFMA straight from the score accumulators (the MFMA k-slots are
 //                   assigned to keys in exactly the order the accumulator registers hold them, and V^T is read
-//                   from LDS in that same order), so the probabilities never leave registers.
+//                   from LDS in that same order), so the probabilities never leave registers.  The V tile sits in
+//                   LDS as it lies in memory ([key][dv]) and is transposed by the read (ds_read_b64_tr_b16).
 //                   Logits are rounded through the storage type before the softmax, as the reference's
 //                   op-by-op composition stores them in an array of that type.  Masked (key > query) and
 //                   out-of-range keys contribute exactly zero; the reference's clamped softmax gives them
@@ -135,9 +136,8 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
   constexpr int BQ = 128, BKV = 64, NT = 256;
   constexpr int DG = D / 8;                      // 16-byte groups along d
   using LayK = TileLayout<BKV, true>;            // K tile: [d/8][key][8 d], one 64-wide pass per 64 values of d
-  using LayV = TileLayout<D, false>;             // V tile: [key/8][dv (permuted)][8 keys]
   constexpr int KSLOTS = (D / 64) * LayK::SLOTS;
-  constexpr int VSLOTS = LayV::SLOTS;
+  constexpr int VSLOTS = 64 * (D / 8);           // V tile: [key][dv] as in memory, 16-byte slots swizzled inside a key row
   constexpr int DT = D / 32;                     // dv tiles of the output accumulator
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   u32x4* smem = reinterpret_cast<u32x4*>(smem_raw);   // two stages of (K tile, V tile)
@@ -179,9 +179,27 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
   const unsigned kTb = (unsigned)a.kT * 2u, vTb = (unsigned)a.vT * 2u;
   const unsigned kRow = (unsigned)t >> 3, kCol = ((unsigned)t & 7u) * 16u;
   const unsigned offK[2] = {kRow * kTb + kCol, (kRow + 32u) * kTb + kCol};
-  constexpr int VUNITS = D * 2;   // threads that carry a 4 x 8 block of the value tile
-  const unsigned vRb = ((unsigned)t >> 1) % (D / 8), vKey = (((unsigned)t / (D / 4)) * 2u + ((unsigned)t & 1u)) * 4u;
-  const unsigned offV = vKey * vTb + vRb * 16u;
+  // value tile kept as it lies in memory ([key][dv], 16-byte slots swizzled inside a key row) and read with the transposing
+  // LDS read: thread t moves the slots t, t + 256, ... of the tile's 64 * D / 8
+  using RowV = RowTileLoader<D, NT>;
+  unsigned offVr[RowV::PER], keyVr[RowV::PER];
+#pragma unroll
+  for (int i = 0; i < RowV::PER; i++) {
+    const unsigned u = (unsigned)t + (unsigned)i * NT;
+    keyVr[i] = u / RowV::SPR;
+    offVr[i] = keyVr[i] * vTb + (u % RowV::SPR) * 16u;
+  }
+  // this lane's transposing reads of the value tile, per dv tile of 32: the 16-lane group reads 4 keys x 16 dv; key slot e of
+  // k-step ks on half h must be key 16 ks + 8 (e / 4) + 4 h + e % 4 (the order of the score accumulator), so the first read
+  // of a k-step starts at key 4 h and the second 8 keys further on
+  int trV[D / 32];
+#pragma unroll
+  for (int i = 0; i < D / 32; i++) {
+    const int grp = lane >> 4, i16 = lane & 15;
+    const int r4 = i * 32 + 16 * (grp & 1) + 4 * (i16 & 3);
+    const int k = 4 * (grp >> 1) + (i16 >> 2);
+    trV[i] = (k * RowV::SPR + ((r4 >> 3) ^ RowV::swz(k))) * 16 + ((r4 >> 2) & 1) * 8;
+  }
   const bool paired = !a.heavyFirst && a.perBatch != a.qTiles;
   for (int pass = 0; pass < (paired ? 2 : 1); pass++) {
   const int qt = pass == 0 ? a.qTiles - 1 - slot : slot;
@@ -208,7 +226,7 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
 
   // the loader moves 64 k-values per pass: the K tile (D values of d per key) takes D/64 of them
   TileLoader<BKV, NT, true> lk[D / 64];   // rows = keys, contiguous along d
-  TileLoader<D, NT, false> lv;            // rows = dv (contiguous in memory), "k" = keys
+  RowV lvr;                               // the value tile's 16-byte pieces, stored as they are
   auto loadKV = [&](LongType kv0) {
     const char* kt = reinterpret_cast<const char*>(K + kv0 * a.kT);
     const char* vt = reinterpret_cast<const char*>(V + kv0 * a.vT);
@@ -217,10 +235,8 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
       for (int part = 0; part < D / 64; part++)
 #pragma unroll
         for (int i = 0; i < 2; i++) lk[part].reg[i] = *reinterpret_cast<const u32x4*>(kt + part * 128 + offK[i]);
-      if (t < VUNITS) {
 #pragma unroll
-        for (int q = 0; q < 4; q++) lv.reg[q] = *reinterpret_cast<const u32x4*>(vt + (LongType)q * vTb + offV);
-      }
+      for (int i = 0; i < RowV::PER; i++) lvr.reg[i] = *reinterpret_cast<const u32x4*>(vt + offVr[i]);
     } else {
       // the last, ragged tile: keys past the end repeat the last one (their weights are exactly 0)
       const unsigned last = (unsigned)(a.Tv - 1 - kv0);
@@ -231,19 +247,17 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
           const unsigned row = kRow + 32u * i < last ? kRow + 32u * i : last;
           lk[part].reg[i] = *reinterpret_cast<const u32x4*>(kt + part * 128 + (row * kTb + kCol));
         }
-      if (t < VUNITS) {
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-          const unsigned key = vKey + q < last ? vKey + q : last;
-          lv.reg[q] = *reinterpret_cast<const u32x4*>(vt + (key * vTb + vRb * 16u));
-        }
+      for (int i = 0; i < RowV::PER; i++) {
+        const unsigned key = keyVr[i] < last ? keyVr[i] : last;
+        lvr.reg[i] = *reinterpret_cast<const u32x4*>(vt + (key * vTb + (offVr[i] - keyVr[i] * vTb)));
       }
     }
   };
   auto storeKV = [&](u32x4* dst) {
 #pragma unroll
     for (int part = 0; part < D / 64; part++) lk[part].store(dst + part * LayK::SLOTS, t);
-    lv.store(dst + KSLOTS, t);
+    lvr.store(dst + KSLOTS, t);
   };
 
   if (nTiles > 0) {
@@ -399,16 +413,19 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
     for (int ks = 0; ks < 4; ks++) {
 #pragma unroll
       for (int i = 0; i < DT; i++) {
-        const int dv = i * 32 + (lane & 31);
-        const u32x2* g0 = reinterpret_cast<const u32x2*>(&sV[LayV::slot(2 * ks, dv)]);
-        const u32x2* g1 = reinterpret_cast<const u32x2*>(&sV[LayV::slot(2 * ks + 1, dv)]);
-        const u32x2 lo = g0[h], hi = g1[h];
-        const u32x4 vf = {lo[0], lo[1], hi[0], hi[1]};
+        typedef __attribute__((address_space(3))) void* lds_ptr;
+        typedef short s16x4 __attribute__((ext_vector_type(4)));
+        const __attribute__((address_space(3))) unsigned char* base =
+            (const __attribute__((address_space(3))) unsigned char*)(lds_ptr)sV + trV[i] + ks * (16 * RowV::SPR * 16);
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)base);
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(base + 8 * RowV::SPR * 16));
+        const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+        const u32x4 vf = {l2[0], l2[1], h2[0], h2[1]};
         o[i] = Mfma16<T>::mma(vf, pf[ks], o[i]);
       }
     }
-    // nothing that consumes the next tile's registers (the V transposes) may drift up into the MFMA sections: the wait for
-    // those loads belongs here, after a whole tile of work
+    // nothing that consumes the next tile's registers may drift up into the MFMA sections: the wait for those loads belongs
+    // here, after a whole tile of work
     __builtin_amdgcn_sched_barrier(0);
     if (more) storeKV(smem + (cur ^ 1) * (KSLOTS + VSLOTS));
     __syncthreads();
@@ -642,7 +659,7 @@ static void launchFusedTyped(hipStream_t s, const void* q, const void* k, const 
     const double heavyTime = std::max(1.1 * total / slots, 2.0 * a.qTiles);
     a.heavyFirst = pairedTime > 1.08 * heavyTime ? 1 : 0;
   }
-  constexpr size_t LDS = (size_t)2 * ((D / 64) * TileLayout<64, true>::SLOTS + TileLayout<D, false>::SLOTS) * 16;
+  constexpr size_t LDS = (size_t)2 * ((D / 64) * TileLayout<64, true>::SLOTS + 64 * (D / 8)) * 16;   // two stages of (K tile, V tile)
   auto kern = attn_fused<T, D, FOLD, VM>;
   static std::once_flag attrOnce;
   std::call_once(attrOnce, [&] { HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS)); });
