@@ -21,6 +21,7 @@
 #include <algorithm>
 #include <cmath>
 #include <mutex>
+#include <type_traits>
 
 #include "device.h"
 #include "kernels.h"
@@ -135,6 +136,7 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
                                                   T* __restrict__ O) {
   constexpr int BQ = 128, BKV = 64, NT = 256;
   constexpr int DG = D / 8;                      // 16-byte groups along d
+  constexpr bool OVF = sizeof(T) == 2 && !std::is_same<T, bf16_t>::value;   // fp16: products beyond the type's range
   using LayK = TileLayout<BKV, true>;            // K tile: [d/8][key][8 d], one 64-wide pass per 64 values of d
   constexpr int KSLOTS = (D / 64) * LayK::SLOTS;
   constexpr int VSLOTS = 64 * (D / 8);           // V tile: [key][dv] as in memory, 16-byte slots swizzled inside a key row
@@ -315,7 +317,11 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
       const float smax = FOLD ? rmax : rmax * sc;
       tmax = __builtin_fmaxf(m, round_storage<T>(__builtin_amdgcn_fmed3f(smax, -clip, clip)));
       tmax = __builtin_fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
-      const bool fast = sc > 0.f && smax <= clip && tmax >= 160.f / L2E - clip;
+      // fp16: the reference's logits array holds the raw product in fp16, +-inf beyond 65504 (65520 with rounding), which
+      // scaling leaves and the clip turns into +-1e4 -- a tile with such a product is clipped score by score, with the
+      // overflow restated; at the lower end the same zero-exponential argument holds from -65520 * scale on
+      const float lowest = OVF && 65520.f * sc < clip ? 65520.f * sc : clip;
+      const bool fast = sc > 0.f && smax <= clip && (!OVF || rmax < 65520.f) && tmax >= 160.f / L2E - lowest;
       clipAll = __builtin_amdgcn_ballot_w64(!fast) != 0;
     }
     if (clipAll) {
@@ -325,6 +331,10 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
 #pragma unroll
         for (int r = 0; r < 16; r += 2) {
           float v0 = s[kt][r], v1 = s[kt][r + 1];
+          if (OVF) {
+            v0 = __builtin_fabsf(v0) >= 65520.f ? __builtin_copysignf(__builtin_inff(), v0) : v0;
+            v1 = __builtin_fabsf(v1) >= 65520.f ? __builtin_copysignf(__builtin_inff(), v1) : v1;
+          }
           if (!FOLD) { v0 *= sc; v1 *= sc; }
           v0 = __builtin_amdgcn_fmed3f(v0, -clip, clip);
           v1 = __builtin_amdgcn_fmed3f(v1, -clip, clip);
@@ -521,6 +531,7 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
       d += dpp_f<0x4E>(d);                 // quad_perm [2,3,0,1]
       d += dpp_f<0x141>(d);                // row_half_mirror
       if (CH > 8) d += dpp_f<0x140>(d);    // row_mirror
+      d = round_storage<T>(d);             // the product as the reference's logits array stores it (fp16: +-inf beyond its range)
       if (a.applyScale) d *= a.scale;
       d = __builtin_fminf(__builtin_fmaxf(d, -1.0e4f), 1.0e4f);
       d = round_storage<T>(d);

@@ -426,7 +426,9 @@ def test_attention_scores_beyond_the_clip(ex, oracle, dtype, tol, causal, scale)
     for b in range(B):
         for qi in (5, 130, 131, 260, 383):
             q[b, qi, 0] = 512.0
-        for kj, mag in ((3, 768.0), (40, 1024.0), (41, -1024.0), (100, 896.0), (200, -768.0), (300, 1024.0), (301, 640.0)):
+        # 140 and -144: products of 71,680 and -73,728, beyond the fp16 range (the reference's fp16 logits array holds +-inf
+        # there, which scaling leaves and the clip turns into +-1e4) but inside the clip once scaled in fp32
+        for kj, mag in ((3, 768.0), (40, 1024.0), (41, -1024.0), (100, 896.0), (150, 140.0), (151, -144.0), (200, -768.0), (300, 1024.0), (301, 640.0)):
             k[b, kj, 0] = mag
     oq, dq = _pair(oracle, q, dtype)
     ok, dk = _pair(oracle, k, dtype)
@@ -440,6 +442,12 @@ def test_attention_scores_beyond_the_clip(ex, oracle, dtype, tol, causal, scale)
     assert_close(out1.to_float(), _f(oo), tol, tol, "output-only call")
     out3 = ex.exec_custom("dot_product_attention_v2", [dq, dv, dk], t_args=[scale, 0.0], b_args=[causal, False])[0]
     assert_close(out3.to_float(), _f(oo), tol, tol, "three-output call")
+    if not causal:   # four query rows against the whole history: the streaming kernel of the decode steps
+        oq4, dq4 = _pair(oracle, q[:, 4:8], dtype)
+        oo4, ow4, ol4 = _ozeros(oracle, (B, 4, D), dtype), _ozeros(oracle, (B, 4, T), dtype), _ozeros(oracle, (B, 4, T), dtype)
+        oracle.attention_v2(oq4, ov, ok, oo4, ow4, ol4, scale=scale, causal=False)
+        out4 = ex.exec_custom("dot_product_attention_v2", [dq4, dv, dk], [NDArray.empty((B, 4, D), dtype)], t_args=[scale, 0.0], b_args=[False, False])[0]
+        assert_close(out4.to_float(), _f(oo4), tol, tol, "four query rows")
 
 
 @pytest.mark.parametrize("dtype,tol", [(FLOAT32, 1e-4), (HALF, 1e-2), (BFLOAT16, 1e-2)])
