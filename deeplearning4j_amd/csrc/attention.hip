@@ -3,7 +3,7 @@
 //
 //   attn_fused    - out = softmax(mask(clip(scale * q k^T))) v without materialising anything of size Tq x Tv.
 //                   One block = 128 queries of one batch entry (4 waves x 32 queries), looping over 64-key tiles
-//                   of K and V staged in LDS.  The score tile is computed TRANSPOSED, S^T = K Q^T, so that an MFMA
+//                   of K and V that go from global memory straight into LDS (two stages).  The score tile is computed TRANSPOSED, S^T = K Q^T, so that an MFMA
 //                   lane owns one query column: the softmax statistics (running max / running sum) and the
 //                   rescaling of the output accumulator O^T = V^T P^T are then per-lane scalars, and the row
 //                   reductions run over a lane's own registers plus one exchange with the other half-wave.
@@ -137,8 +137,7 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
   constexpr int BQ = 128, BKV = 64, NT = 256;
   constexpr int DG = D / 8;                      // 16-byte groups along d
   constexpr bool OVF = sizeof(T) == 2 && !std::is_same<T, bf16_t>::value;   // fp16: products beyond the type's range
-  using LayK = TileLayout<BKV, true>;            // K tile: [d/8][key][8 d], one 64-wide pass per 64 values of d
-  constexpr int KSLOTS = (D / 64) * LayK::SLOTS;
+  constexpr int KSLOTS = (D / 64) * 512;         // K tile: 8 chunks of 64 slots (8 keys x 128 bytes) per 64 values of d
   constexpr int VSLOTS = 64 * (D / 8);           // V tile: [key][dv] as in memory, 16-byte slots swizzled inside a key row
   constexpr int DT = D / 32;                     // dv tiles of the output accumulator
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -176,21 +175,10 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
   const float sc = a.scale;   // 1 when the op applies no scale
   const float L2E = FOLD ? 1.44269502162933349609375f * sc : 1.44269502162933349609375f;
   const float clip = FOLD ? 1.0e4f / sc : 1.0e4f;
-  // per-lane byte offsets of this thread's loads inside a key / value tile.  The tile's own address is the same for
-  // the whole wave, so a load is "scalar base + 32-bit lane offset" and costs no address arithmetic per tile.
-  const unsigned kTb = (unsigned)a.kT * 2u, vTb = (unsigned)a.vT * 2u;
-  const unsigned kRow = (unsigned)t >> 3, kCol = ((unsigned)t & 7u) * 16u;
-  const unsigned offK[2] = {kRow * kTb + kCol, (kRow + 32u) * kTb + kCol};
+  const unsigned kTb = (unsigned)a.kT * 2u, vTb = (unsigned)a.vT * 2u;   // bytes per key row
   // value tile kept as it lies in memory ([key][dv], 16-byte slots swizzled inside a key row) and read with the transposing
-  // LDS read: thread t moves the slots t, t + 256, ... of the tile's 64 * D / 8
+  // LDS read
   using RowV = RowTileLoader<D, NT>;
-  unsigned offVr[RowV::PER], keyVr[RowV::PER];
-#pragma unroll
-  for (int i = 0; i < RowV::PER; i++) {
-    const unsigned u = (unsigned)t + (unsigned)i * NT;
-    keyVr[i] = u / RowV::SPR;
-    offVr[i] = keyVr[i] * vTb + (u % RowV::SPR) * 16u;
-  }
   // this lane's transposing reads of the value tile, per dv tile of 32: the 16-lane group reads 4 keys x 16 dv; key slot e of
   // k-step ks on half h must be key 16 ks + 8 (e / 4) + 4 h + e % 4 (the order of the score accumulator), so the first read
   // of a k-step starts at key 4 h and the second 8 keys further on
@@ -201,6 +189,27 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
     const int r4 = i * 32 + 16 * (grp & 1) + 4 * (i16 & 3);
     const int k = 4 * (grp >> 1) + (i16 >> 2);
     trV[i] = (k * RowV::SPR + ((r4 >> 3) ^ RowV::swz(k))) * 16 + ((r4 >> 2) & 1) * 8;
+  }
+  // Direct loads (global memory -> LDS, no registers): a wave instruction moves one chunk of 1 KiB, 64 slots of 16 bytes in
+  // lane order.  K chunk: 8 keys x the 128 bytes of one 64-wide part of d; lane (lj = lane / 8, lp = lane % 8) fetches the
+  // k-group that belongs in position lp of key row lj under the XOR placement the fragment reads below undo (the one of the
+  // GEMM's k-contiguous operand: conflict-free 16-byte reads by 32 consecutive rows).  V chunk: 64 / SPR keys x one key
+  // row of SPR slots, swizzled as RowTileLoader stores them.  Wave w owns chunks w * KPW ... and w * VPW ...
+  constexpr int KCH = 8 * (D / 64), VCH = D / 8, KPW = KCH / 4, VPW = VCH / 4;
+  const int waveU = __builtin_amdgcn_readfirstlane(wave);
+  unsigned dmaK[KPW], dmaKrow[KPW], dmaV[VPW], dmaVrow[VPW];
+#pragma unroll
+  for (int c = 0; c < KPW; c++) {
+    const int ch = waveU * KPW + c, part = ch >> 3, cw = ch & 7, lj = lane >> 3, lp = lane & 7;
+    const int lkg = (lp - 4 * (cw & 1) - (lj >> 1)) & 7;
+    dmaKrow[c] = (unsigned)(8 * cw + lj);
+    dmaK[c] = (unsigned)(part * 128 + lkg * 16);
+  }
+#pragma unroll
+  for (int c = 0; c < VPW; c++) {
+    const int ch = waveU * VPW + c, k = ch * (64 / RowV::SPR) + lane / RowV::SPR, pp = lane % RowV::SPR;
+    dmaVrow[c] = (unsigned)k;
+    dmaV[c] = (unsigned)((pp ^ RowV::swz(k)) * 16);
   }
   const bool paired = !a.heavyFirst && a.perBatch != a.qTiles;
   for (int pass = 0; pass < (paired ? 2 : 1); pass++) {
@@ -226,46 +235,36 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
   if (a.causal && !VM) { const LongType lim = q0 + BQ; kvEnd = lim < kvEnd ? lim : kvEnd; }
   const LongType nTiles = (kvEnd + BKV - 1) / BKV;
 
-  // the loader moves 64 k-values per pass: the K tile (D values of d per key) takes D/64 of them
-  TileLoader<BKV, NT, true> lk[D / 64];   // rows = keys, contiguous along d
-  RowV lvr;                               // the value tile's 16-byte pieces, stored as they are
-  auto loadKV = [&](LongType kv0) {
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  // written as assembly so that the compiler's wait-count pass does not know of an outstanding write into LDS (it would
+  // wait for these loads in front of every transposing LDS read); all waiting for them is explicit, in front of the
+  // barrier that ends a key tile.  M0 carries the LDS address of the chunk; nothing else in this kernel uses M0.
+  auto dma = [&](const char* src, const u32x4* dst) {
+    const unsigned ldsAddr = (unsigned)(size_t)(lds_ptr)dst;
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(ldsAddr) : "memory");
+  };
+  auto issueKV = [&](LongType kv0, u32x4* stage) {
     const char* kt = reinterpret_cast<const char*>(K + kv0 * a.kT);
     const char* vt = reinterpret_cast<const char*>(V + kv0 * a.vT);
-    if (kv0 + BKV <= a.Tv) {
+    // the last, ragged tile: keys past the end repeat the last one (their weights are exactly 0)
+    const unsigned last = kv0 + BKV <= a.Tv ? (unsigned)(BKV - 1) : (unsigned)(a.Tv - 1 - kv0);
 #pragma unroll
-      for (int part = 0; part < D / 64; part++)
+    for (int c = 0; c < KPW; c++) {
+      const unsigned row = dmaKrow[c] < last ? dmaKrow[c] : last;
+      dma(kt + (row * kTb + dmaK[c]), stage + (waveU * KPW + c) * 64);
+    }
 #pragma unroll
-        for (int i = 0; i < 2; i++) lk[part].reg[i] = *reinterpret_cast<const u32x4*>(kt + part * 128 + offK[i]);
-#pragma unroll
-      for (int i = 0; i < RowV::PER; i++) lvr.reg[i] = *reinterpret_cast<const u32x4*>(vt + offVr[i]);
-    } else {
-      // the last, ragged tile: keys past the end repeat the last one (their weights are exactly 0)
-      const unsigned last = (unsigned)(a.Tv - 1 - kv0);
-#pragma unroll
-      for (int part = 0; part < D / 64; part++)
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-          const unsigned row = kRow + 32u * i < last ? kRow + 32u * i : last;
-          lk[part].reg[i] = *reinterpret_cast<const u32x4*>(kt + part * 128 + (row * kTb + kCol));
-        }
-#pragma unroll
-      for (int i = 0; i < RowV::PER; i++) {
-        const unsigned key = keyVr[i] < last ? keyVr[i] : last;
-        lvr.reg[i] = *reinterpret_cast<const u32x4*>(vt + (key * vTb + (offVr[i] - keyVr[i] * vTb)));
-      }
+    for (int c = 0; c < VPW; c++) {
+      const unsigned row = dmaVrow[c] < last ? dmaVrow[c] : last;
+      dma(vt + (row * vTb + dmaV[c]), stage + KSLOTS + (waveU * VPW + c) * 64);
     }
   };
-  auto storeKV = [&](u32x4* dst) {
-#pragma unroll
-    for (int part = 0; part < D / 64; part++) lk[part].store(dst + part * LayK::SLOTS, t);
-    lvr.store(dst + KSLOTS, t);
+  // this lane's K fragment slots: key row r = 32 kt + lane % 32, k-group 2 ks + h of part ks / 4
+  auto slotK = [&](int kg, int r) {
+    return (kg >> 3) * 512 + (r >> 3) * 64 + 8 * (r & 7) + (((kg & 7) + 4 * ((r >> 3) & 1) + ((r & 7) >> 1)) & 7);
   };
-
-  if (nTiles > 0) {
-    loadKV(0);
-    storeKV(smem);
-  }
+  if (nTiles > 0) issueKV(0, smem);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   // Make the Q fragments "used" here, on every path into the key loop: otherwise the path that skips the block above
   // leaves their loads pending as far as the compiler can tell, and it waits for them -- and with them for the freshly
@@ -279,7 +278,7 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
     const u32x4* sK = smem + cur * (KSLOTS + VSLOTS);
     const u32x4* sV = sK + KSLOTS;
     const bool more = it + 1 < nTiles;
-    if (more) loadKV(kv0 + BKV);   // in flight while this tile is computed
+    if (more) issueKV(kv0 + BKV, smem + (cur ^ 1) * (KSLOTS + VSLOTS));   // lands in the other stage while this tile is computed
 
     // S^T = K Q^T : two 32-key tiles, D/16 k-steps
     f32x16 s[2];
@@ -289,7 +288,7 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
       for (int r = 0; r < 16; r++) s[kt][r] = 0.f;
 #pragma unroll
       for (int ks = 0; ks < D / 16; ks++) {
-        const u32x4 kf = sK[LayK::slot(ks * 2 + h, kt * 32 + (lane & 31))];   // parts of 8 k-groups follow each other
+        const u32x4 kf = sK[slotK(ks * 2 + h, kt * 32 + (lane & 31))];   // parts of 8 k-groups follow each other
         s[kt] = Mfma16<T>::mma(kf, qf[ks], s[kt]);
       }
     }
@@ -437,7 +436,7 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
     // nothing that consumes the next tile's registers may drift up into the MFMA sections: the wait for those loads belongs
     // here, after a whole tile of work
     __builtin_amdgcn_sched_barrier(0);
-    if (more) storeKV(smem + (cur ^ 1) * (KSLOTS + VSLOTS));
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's chunks of the next tile have landed
     __syncthreads();
   }
 
@@ -670,7 +669,7 @@ static void launchFusedTyped(hipStream_t s, const void* q, const void* k, const 
     const double heavyTime = std::max(1.1 * total / slots, 2.0 * a.qTiles);
     a.heavyFirst = pairedTime > 1.08 * heavyTime ? 1 : 0;
   }
-  constexpr size_t LDS = (size_t)2 * ((D / 64) * TileLayout<64, true>::SLOTS + 64 * (D / 8)) * 16;   // two stages of (K tile, V tile)
+  constexpr size_t LDS = (size_t)2 * ((D / 64) * 512 + 64 * (D / 8)) * 16;   // two stages of (K tile, V tile)
   auto kern = attn_fused<T, D, FOLD, VM>;
   static std::once_flag attrOnce;
   std::call_once(attrOnce, [&] { HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS)); });

@@ -385,7 +385,8 @@ def test_layer_norm_channels_first_and_views(ex, oracle):
 # ---- attention -------------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype,tol", [(FLOAT32, 1e-4), (HALF, 1e-2), (BFLOAT16, 1e-2)])
 @pytest.mark.parametrize("causal", [False, True])
-@pytest.mark.parametrize("B,Tq,Tv,D", [(3, 64, 64, 64), (2, 100, 100, 64), (2, 128, 256, 64), (1, 37, 91, 32), (2, 300, 72, 64), (1, 520, 200, 64)])
+@pytest.mark.parametrize("B,Tq,Tv,D", [(3, 64, 64, 64), (2, 100, 100, 64), (2, 128, 256, 64), (1, 37, 91, 32), (2, 300, 72, 64), (1, 520, 200, 64),
+                                      (2, 200, 200, 128), (1, 70, 330, 128), (2, 3, 200, 128)])
 def test_attention_vs_oracle(ex, oracle, dtype, tol, causal, B, Tq, Tv, D):
     # causal with Tq != Tv: key j is visible to query i iff j <= i (the lower-triangular mask of AttentionHelper.cpp:70-79)
     rng = np.random.default_rng(B * Tq + D)
@@ -401,9 +402,20 @@ def test_attention_vs_oracle(ex, oracle, dtype, tol, causal, B, Tq, Tv, D):
     assert_close(w.to_float(), _f(ow), tol, tol * 1e-2, "weights")
     keep = np.tril(np.ones((Tq, Tv), bool)) if causal else np.ones((Tq, Tv), bool)
     assert_close(lg.to_float()[:, keep], _f(ol)[:, keep], tol, tol, "logits")
-    # output only (fused path where available): same numbers
+    # output only (fused path where available): same numbers.  At D = 128 in bf16 the reference's own op-by-op composition
+    # (every intermediate rounded to bf16) is 0.014 away from the exact result and the fused kernel 0.009: the two are
+    # compared at 2.5 times the gate, and the kernel must not be further from the exact result than the composition is
+    wide = 2.5 if (D == 128 and dtype == BFLOAT16) else 1.0
     out1 = ex.exec_custom("dot_product_attention_v2", [dq, dv, dk], [NDArray.empty((B, Tq, D), dtype)], t_args=[scale, 0.0], b_args=[causal, False])[0]
-    assert_close(out1.to_float(), _f(oo), tol, tol, "out-only call")
+    assert_close(out1.to_float(), _f(oo), wide * tol, wide * tol, "out-only call")
+    if D == 128:
+        q64, k64, v64 = _f(oq), _f(ok), _f(ov)
+        sc64 = np.einsum("bqd,bkd->bqk", q64, k64) * scale
+        if causal:
+            sc64 = np.where(np.tril(np.ones((Tq, Tv), bool)), sc64, -np.inf)
+        p64 = np.exp(sc64 - sc64.max(-1, keepdims=True))
+        truth = np.einsum("bqk,bkd->bqd", p64 / p64.sum(-1, keepdims=True), v64)
+        assert np.abs(out1.to_float() - truth).max() <= 1.25 * np.abs(_f(oo) - truth).max() + 1e-3, "fused kernel against the exact result"
 
 
 @pytest.mark.parametrize("dtype,tol", [(HALF, 1e-2), (BFLOAT16, 1e-2)])
@@ -452,7 +464,8 @@ def test_attention_scores_beyond_the_clip(ex, oracle, dtype, tol, causal, scale)
 
 @pytest.mark.parametrize("dtype,tol", [(FLOAT32, 1e-4), (HALF, 1e-2), (BFLOAT16, 1e-2)])
 @pytest.mark.parametrize("causal", [False, True])
-@pytest.mark.parametrize("B,Tq,Tv,D", [(3, 64, 64, 64), (2, 200, 200, 64), (2, 130, 300, 64), (2, 4, 150, 64), (1, 37, 91, 32)])
+@pytest.mark.parametrize("B,Tq,Tv,D", [(3, 64, 64, 64), (2, 200, 200, 64), (2, 130, 300, 64), (2, 4, 150, 64), (1, 37, 91, 32), (2, 130, 300, 128),
+                                      (2, 4, 150, 128)])
 def test_attention_masks_vs_oracle(ex, oracle, dtype, tol, causal, B, Tq, Tv, D):
     """Query and value masks (inputs 3 and 4): all three outputs through the composition path, then the output-only call
     (fused prefill kernel, or the streaming decode kernel for a handful of query rows)."""
