@@ -323,34 +323,33 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
       const bool fast = sc > 0.f && smax <= clip && (!OVF || rmax < 65520.f) && tmax >= 160.f / L2E - lowest;
       clipAll = __builtin_amdgcn_ballot_w64(!fast) != 0;
     }
+    // (the clip works on the registers in place and the rounding below is common to both cases: written as two complete
+    // alternatives the compiler merged them with 32 register copies per tile)
     if (clipAll) {
       asm volatile("; scores clipped one by one");
 #pragma unroll
       for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-          float v0 = s[kt][r], v1 = s[kt][r + 1];
-          if (OVF) {
-            v0 = __builtin_fabsf(v0) >= 65520.f ? __builtin_copysignf(__builtin_inff(), v0) : v0;
-            v1 = __builtin_fabsf(v1) >= 65520.f ? __builtin_copysignf(__builtin_inff(), v1) : v1;
-          }
-          if (!FOLD) { v0 *= sc; v1 *= sc; }
-          v0 = __builtin_amdgcn_fmed3f(v0, -clip, clip);
-          v1 = __builtin_amdgcn_fmed3f(v1, -clip, clip);
-          round_pair<T>(v0, v1);
-          s[kt][r] = v0; s[kt][r + 1] = v1;
+        for (int r = 0; r < 16; r++) {
+          float v = s[kt][r];
+          if (OVF) v = __builtin_fabsf(v) >= 65520.f ? __builtin_copysignf(__builtin_inff(), v) : v;
+          if (!FOLD) v *= sc;
+          s[kt][r] = __builtin_amdgcn_fmed3f(v, -clip, clip);
         }
-    } else {
+    } else if (!FOLD) {
 #pragma unroll
       for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-          float v0 = s[kt][r], v1 = s[kt][r + 1];
-          if (!FOLD) { v0 *= sc; v1 *= sc; }
-          round_pair<T>(v0, v1);
-          s[kt][r] = v0; s[kt][r + 1] = v1;
-        }
+        for (int r = 0; r < 16; r++) s[kt][r] *= sc;
     }
+#pragma unroll
+    for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) {
+        float v0 = s[kt][r], v1 = s[kt][r + 1];
+        round_pair<T>(v0, v1);
+        s[kt][r] = v0; s[kt][r + 1] = v1;
+      }
     // only tiles that touch the diagonal or the end of the keys carry masked entries (wave-uniform test)
     // a real branch (scalar condition, a body the compiler cannot speculate): turned into selects, the mask costs 86
     // vector instructions on every tile instead of on the few that need it
