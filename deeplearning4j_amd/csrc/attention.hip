@@ -239,24 +239,37 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
   // written as assembly so that the compiler's wait-count pass does not know of an outstanding write into LDS (it would
   // wait for these loads in front of every transposing LDS read); all waiting for them is explicit, in front of the
   // barrier that ends a key tile.  M0 carries the LDS address of the chunk; nothing else in this kernel uses M0.
-  auto dma = [&](const char* src, const u32x4* dst) {
+  // address = scalar base (the tile's first key row, the same for every lane) + 32-bit lane offset: no vector arithmetic
+  auto dma = [&](const char* base, unsigned off, const u32x4* dst) {
     const unsigned ldsAddr = (unsigned)(size_t)(lds_ptr)dst;
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(ldsAddr) : "memory");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(ldsAddr) : "memory");
   };
+  unsigned fullK[KPW], fullV[VPW];   // lane offsets inside a whole tile
+#pragma unroll
+  for (int c = 0; c < KPW; c++) fullK[c] = dmaKrow[c] * kTb + dmaK[c];
+#pragma unroll
+  for (int c = 0; c < VPW; c++) fullV[c] = dmaVrow[c] * vTb + dmaV[c];
   auto issueKV = [&](LongType kv0, u32x4* stage) {
     const char* kt = reinterpret_cast<const char*>(K + kv0 * a.kT);
     const char* vt = reinterpret_cast<const char*>(V + kv0 * a.vT);
-    // the last, ragged tile: keys past the end repeat the last one (their weights are exactly 0)
-    const unsigned last = kv0 + BKV <= a.Tv ? (unsigned)(BKV - 1) : (unsigned)(a.Tv - 1 - kv0);
+    if (kv0 + BKV <= a.Tv) {
 #pragma unroll
-    for (int c = 0; c < KPW; c++) {
-      const unsigned row = dmaKrow[c] < last ? dmaKrow[c] : last;
-      dma(kt + (row * kTb + dmaK[c]), stage + (waveU * KPW + c) * 64);
-    }
+      for (int c = 0; c < KPW; c++) dma(kt, fullK[c], stage + (waveU * KPW + c) * 64);
 #pragma unroll
-    for (int c = 0; c < VPW; c++) {
-      const unsigned row = dmaVrow[c] < last ? dmaVrow[c] : last;
-      dma(vt + (row * vTb + dmaV[c]), stage + KSLOTS + (waveU * VPW + c) * 64);
+      for (int c = 0; c < VPW; c++) dma(vt, fullV[c], stage + KSLOTS + (waveU * VPW + c) * 64);
+    } else {
+      // the last, ragged tile: keys past the end repeat the last one (their weights are exactly 0)
+      const unsigned last = (unsigned)(a.Tv - 1 - kv0);
+#pragma unroll
+      for (int c = 0; c < KPW; c++) {
+        const unsigned row = dmaKrow[c] < last ? dmaKrow[c] : last;
+        dma(kt, row * kTb + dmaK[c], stage + (waveU * KPW + c) * 64);
+      }
+#pragma unroll
+      for (int c = 0; c < VPW; c++) {
+        const unsigned row = dmaVrow[c] < last ? dmaVrow[c] : last;
+        dma(vt, row * vTb + dmaV[c], stage + KSLOTS + (waveU * VPW + c) * 64);
+      }
     }
   };
   // this lane's K fragment slots: key row r = 32 kt + lane % 32, k-group 2 ks + h of part ks / 4
