@@ -109,8 +109,10 @@ template <> __device__ __forceinline__ unsigned pack_pair<bf16_t>(float& a, floa
   const f32x2a v = {a, b};
   return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2a));
 }
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2a;
 template <> __device__ __forceinline__ unsigned pack_pair<f16_t>(float& a, float& b) {
-  return (unsigned)Conv<f16_t>::from(a).bits | ((unsigned)Conv<f16_t>::from(b).bits << 16);
+  const f32x2a v = {a, b};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, f16x2a));   // one packed conversion, round to nearest even
 }
 // round two values through the storage type in place
 template <typename T> __device__ __forceinline__ void round_pair(float& a, float& b);
@@ -119,7 +121,11 @@ template <> __device__ __forceinline__ void round_pair<bf16_t>(float& a, float& 
   a = __uint_as_float(p << 16);
   b = __uint_as_float(p & 0xffff0000u);
 }
-template <> __device__ __forceinline__ void round_pair<f16_t>(float& a, float& b) { a = round_storage<f16_t>(a); b = round_storage<f16_t>(b); }
+template <> __device__ __forceinline__ void round_pair<f16_t>(float& a, float& b) {
+  const f32x2a v = {a, b};
+  const f32x2a r = __builtin_convertvector(__builtin_convertvector(v, f16x2a), f32x2a);
+  a = r[0]; b = r[1];
+}
 template <typename T> __device__ __forceinline__ unsigned pack2(float a, float b) {
   return (unsigned)Conv<T>::from(a).bits | ((unsigned)Conv<T>::from(b).bits << 16);
 }
