@@ -518,6 +518,111 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16q(GemmArgs g, const T
   storeAccTiles<T, TM, TN, true>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
 }
 
+// 64 x 64 tiles with the operands going from global memory straight into LDS (no registers, no LDS stores), NST stages in
+// a ring: for launches that put one or two small tiles on a CU (1024^3; the projections of a prefill), where the
+// register-staged kernel above spends more on parking the tiles in LDS than on multiplying them.  A k-contiguous, B either
+// way; whole tiles, K a multiple of NST K-tiles.  A wave instruction moves a chunk of 1 KiB (64 slots of 16 bytes in lane
+// order): 8 rows x 128 bytes of a k-contiguous operand, placed so that the fragment read of 32 consecutive rows is free of
+// bank conflicts (the placement of gemm_mfma16d), or 8 k-rows x 128 bytes of row-major B, swizzled as RowTileLoader keeps
+// them and read with the transposing LDS read.  Round kt: wait for tile kt + 1 (this wave's chunks), barrier (everybody's),
+// refill the stage tile kt - 1 left, read the fragments of tile kt + 1 while the four MFMAs of tile kt run.
+template <typename T, bool B_KC, int NST>
+__global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
+                                                    unsigned tilesM, unsigned tilesN) {
+  constexpr int BM = 64, BN = 64, BK = 64, STAGE = 1024;   // slots of 16 bytes: 512 of A, 512 of B
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  u32x4* smem = reinterpret_cast<u32x4*>(smem_raw);
+  unsigned tm, tn;
+  tileOf(blockIdx.x, gridDim.x, tilesM, tilesN, tm, tn);
+  const LongType m0 = (LongType)tm * BM, n0 = (LongType)tn * BN;
+  { LongType oa, ob, oc; batchOffsets(g, (LongType)blockIdx.z, oa, ob, oc); A += oa; B += ob; C += oc; }
+  const LongType lda = g.aRow, ldb = B_KC ? g.bCol : g.bRow;
+  const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6), h = lane >> 5;
+  const int wm = wave >> 1, wn = wave & 1;
+  using RowB = RowTileLoader<BN, 256>;
+
+  // ---- global side: two chunks of each operand per wave; a load is scalar base (the tile's first byte) + lane offset ----
+  unsigned offA[2], offB[2];
+#pragma unroll
+  for (int c = 0; c < 2; c++) {
+    const int cw = wave * 2 + c, lj = lane >> 3, lp = lane & 7;
+    const int lkg = (lp - 4 * (cw & 1) - (lj >> 1)) & 7;
+    offA[c] = (unsigned)(((LongType)(cw * 8 + lj) * lda + lkg * 8) * 2);
+    if (B_KC) {
+      offB[c] = (unsigned)(((LongType)(cw * 8 + lj) * ldb + lkg * 8) * 2);
+    } else {
+      const int k = cw * 8 + (lane >> 3), pp = lane & 7;
+      offB[c] = (unsigned)(((LongType)k * ldb + (pp ^ RowB::swz(k)) * 8) * 2);
+    }
+  }
+  const char* const baseA = reinterpret_cast<const char*>(A + m0 * lda);
+  const char* const baseB = reinterpret_cast<const char*>(B_KC ? B + n0 * ldb : B + n0);
+  const LongType stepA = BK * 2, stepB = (B_KC ? (LongType)BK : (LongType)BK * ldb) * 2;   // bytes per K-tile
+  const LongType KT = g.K / BK;
+  auto dma = [&](const char* base, unsigned off, const u32x4* dst) {
+    const unsigned ldsAddr = (unsigned)(size_t)(lds_ptr)dst;
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(ldsAddr) : "memory");
+  };
+  auto issue = [&](LongType tile, int stage) {   // tiles past the end re-read the last one into a stage nobody reads
+    const LongType kt = tile < KT ? tile : KT - 1;
+    u32x4* const st = smem + stage * STAGE;
+#pragma unroll
+    for (int c = 0; c < 2; c++) dma(baseA + kt * stepA, offA[c], st + (wave * 2 + c) * 64);
+#pragma unroll
+    for (int c = 0; c < 2; c++) dma(baseB + kt * stepB, offB[c], st + 512 + (wave * 2 + c) * 64);
+  };
+
+  // ---- LDS side ----
+  int fragA[4], fragB[4];
+  {
+    const int r = wm * 32 + (lane & 31);
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) fragA[ks] = (r >> 3) * 64 + 8 * (r & 7) + ((2 * ks + h + 4 * ((r >> 3) & 1) + ((r & 7) >> 1)) & 7);
+    const int rb = wn * 32 + (lane & 31);
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) fragB[ks] = 512 + (rb >> 3) * 64 + 8 * (rb & 7) + ((2 * ks + h + 4 * ((rb >> 3) & 1) + ((rb & 7) >> 1)) & 7);
+  }
+  const int trB = RowB::fragOffset(wn * 32, lane);
+  u32x4 fa[2][4], fb[2][4];
+  auto readTile = [&](int stage, int buf) {
+    const u32x4* st = smem + stage * STAGE;
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      fa[buf][ks] = st[fragA[ks]];
+      if (B_KC) fb[buf][ks] = st[fragB[ks]];
+      else fb[buf][ks] = RowB::readFrag(st + 512, trB, ks);
+    }
+  };
+  f32x16 acc[1][1];
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[0][0][r] = 0.f;
+
+  // tiles 0 .. NST - 2 on their way; tile 0 read before the loop
+#pragma unroll
+  for (int u = 0; u < NST - 1; u++) issue(u, u);
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 2) * 4) : "memory");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+  readTile(0, 0);
+  for (LongType kt0 = 0; kt0 < KT; kt0 += NST) {
+#pragma unroll
+    for (int u = 0; u < NST; u++) {
+      // tile kt0 + u + 1 has landed (the loads of the NST - 3 tiles after it may still be out) and is visible after the barrier
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 3) * 4) : "memory");
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      issue(kt0 + u + NST - 1, (u + NST - 1) % NST);   // the stage of tile kt0 + u - 1: everybody is past its fragments
+      readTile((u + 1) % NST, (u + 1) & 1);
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++) acc[0][0] = Mfma16<T>::mma(fa[u & 1][ks], fb[u & 1][ks], acc[0][0]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the surplus loads of the last rounds
+  storeAccTiles<T, 1, 1, false>(g, C, acc, m0 + wm * 32, n0 + wn * 32, lane);
+}
+
 // Steady-state kernel for problems made of whole tiles (M % BM == 0, N % BN == 0, K % 64 == 0): no bounds handling,
 // so the K loop is one basic block and the instruction order below is the order the hardware sees.  A wave issues
 // in order, and an MFMA 32x32x16 keeps the matrix pipe busy for 32 cycles: every LDS / global instruction is placed
@@ -1094,6 +1199,33 @@ static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
   // K-tiles are in flight
   const unsigned nTiles = (unsigned)(((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN) * batch);
   const bool useDeep = usePipe && !useFull && BM * BN <= 64 * 64 && nTiles <= 1024 && g.K >= 512 && g.M % BM == 0 && g.N % BN == 0 && g.K % 256 == 0;
+  // the direct-load ring takes the small-tile launches it can: 64 x 64 tiles, A k-contiguous, 16-byte aligned rows
+  if constexpr (BM == 64 && BN == 64 && A_KC) {
+    static const bool small = getenv("ND4JHIP_GEMM_SMALL_RING") ? atoi(getenv("ND4JHIP_GEMM_SMALL_RING")) != 0 : true;
+    const LongType ldaS = g.aRow, ldbS = B_KC ? g.bCol : g.bRow;
+    if (small && useDeep && ldaS % 8 == 0 && ldbS % 8 == 0 && ldaS < (1 << 24) && ldbS < (1 << 24) &&
+        ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 && g.aBatch % 8 == 0 && g.bBatch % 8 == 0 &&
+        g.aBatch2 % 8 == 0 && g.bBatch2 % 8 == 0) {
+      const unsigned tM = (unsigned)(g.M / 64), tN = (unsigned)(g.N / 64);
+      // one tile per CU and a K of whole eight-tile rounds: eight stages (128 KiB), else four (two blocks fit a CU)
+      static std::once_flag once8;
+      static bool granted8 = false;
+      const bool want8 = nTiles <= 256 && g.K % 512 == 0;
+      if (want8)
+        std::call_once(once8, [&] {
+          granted8 = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_mfma16s<T, B_KC, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, 8 * 16384) == hipSuccess;
+          if (!granted8) (void)hipGetLastError();
+        });
+      if (want8 && granted8) {
+        noteKernel("gemm_mfma16s<%s,64x64,akc=1,bkc=%d,stages=8>", tname<T>(), (int)B_KC);
+        hipLaunchKernelGGL((gemm_mfma16s<T, B_KC, 8>), dim3(tM * tN, 1, (unsigned)batch), dim3(256), 8 * 16384, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
+      } else {
+        noteKernel("gemm_mfma16s<%s,64x64,akc=1,bkc=%d,stages=4>", tname<T>(), (int)B_KC);
+        hipLaunchKernelGGL((gemm_mfma16s<T, B_KC, 4>), dim3(tM * tN, 1, (unsigned)batch), dim3(256), 4 * 16384, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
+      }
+      return true;
+    }
+  }
   auto kern = useFull ? gemm_mfma16f<T, BM, BN, WM, WN, A_KC, B_KC>
               : useDeep ? gemm_mfma16q<T, BM, BN, WM, WN, A_KC, B_KC, 4>
               : usePipe ? gemm_mfma16p<T, BM, BN, WM, WN, A_KC, B_KC> : gemm_mfma16<T, BM, BN, WM, WN, A_KC, B_KC>;

@@ -67,8 +67,8 @@ CASES = [
     (BFLOAT16, 4096, 4096, 192, "gemm_mfma16d<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1>", None),
     # BASELINE config 2 at 1024^3
     (FLOAT32, 1024, 1024, 1024, "gemm_mfma32q<f32,64x64,akc=1,bkc=0,pd=4,bk=32>", "gemm_mfma32q<f32,64x64,akc=1,bkc=1,pd=4,bk=32>", "gemm_mfma32q<f32,64x64,akc=0,bkc=0,pd=4,bk=32>"),
-    (HALF, 1024, 1024, 1024, "gemm_mfma16q<f16,64x64,akc=1,bkc=0>", "gemm_mfma16q<f16,64x64,akc=1,bkc=1>", "gemm_mfma16q<f16,64x64,akc=0,bkc=0>"),
-    (BFLOAT16, 1024, 1024, 1024, "gemm_mfma16q<bf16,64x64,akc=1,bkc=0>", "gemm_mfma16q<bf16,64x64,akc=1,bkc=1>", "gemm_mfma16q<bf16,64x64,akc=0,bkc=0>"),
+    (HALF, 1024, 1024, 1024, "gemm_mfma16s<f16,64x64,akc=1,bkc=0,stages=8>", "gemm_mfma16s<f16,64x64,akc=1,bkc=1,stages=8>", "gemm_mfma16q<f16,64x64,akc=0,bkc=0>"),
+    (BFLOAT16, 1024, 1024, 1024, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=8>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=8>", "gemm_mfma16q<bf16,64x64,akc=0,bkc=0>"),
     # the 128 x 128 configuration (2048-class sizes), whole tiles
     (BFLOAT16, 2048, 2048, 2048, "gemm_mfma16f<bf16,128x128,akc=1,bkc=0>", "gemm_mfma16f<bf16,128x128,akc=1,bkc=1>", "gemm_mfma16f<bf16,128x128,akc=0,bkc=0>"),
     (HALF, 2048, 2048, 1024, "gemm_mfma16f<f16,128x128,akc=1,bkc=0>", "gemm_mfma16f<f16,128x128,akc=1,bkc=1>", None),
@@ -76,8 +76,11 @@ CASES = [
     (BFLOAT16, 3600, 3704, 1000, "gemm_mfma16p<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16p<bf16,256x256,akc=1,bkc=1>", "gemm_mfma16p<bf16,256x256,akc=0,bkc=0>"),
     (HALF, 1800, 1800, 520, "gemm_mfma16p<f16,128x128,akc=1,bkc=0>", "gemm_mfma16p<f16,128x128,akc=1,bkc=1>", None),
     (BFLOAT16, 1104, 904, 1000, "gemm_mfma16p<bf16,64x64,akc=1,bkc=0>", "gemm_mfma16p<bf16,64x64,akc=1,bkc=1>", None),
-    # K a multiple of 256 but not of 512: the four-deep prefetch ends in the middle of its ring
-    (BFLOAT16, 1024, 1024, 768, "gemm_mfma16q<bf16,64x64,akc=1,bkc=0>", "gemm_mfma16q<bf16,64x64,akc=1,bkc=1>", None),
+    # K a multiple of 256 but not of 512: the four-stage ring; more tiles than CUs (two blocks on a CU): four stages as well;
+    # the shortest K the ring takes
+    (BFLOAT16, 1024, 1024, 768, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=4>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=4>", "gemm_mfma16q<bf16,64x64,akc=0,bkc=0>"),
+    (HALF, 512, 2304, 1024, "gemm_mfma16s<f16,64x64,akc=1,bkc=0,stages=4>", "gemm_mfma16s<f16,64x64,akc=1,bkc=1,stages=4>", None),
+    (BFLOAT16, 1024, 1024, 512, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=8>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=8>", None),
     (FLOAT32, 1024, 1024, 384, "gemm_mfma32q<f32,64x64,akc=1,bkc=0,pd=4,bk=32>", "gemm_mfma32q<f32,64x64,akc=1,bkc=1,pd=4,bk=32>", None),
     (FLOAT32, 2048, 2048, 640, "gemm_mfma32q<f32,128x128,akc=1,bkc=0,pd=4,bk=16>", "gemm_mfma32q<f32,128x128,akc=1,bkc=1,pd=4,bk=16>", None),
     # fp32 ragged
@@ -174,3 +177,43 @@ def test_bias_row_on_the_large_kernels(ex):
     zt = ex.exec_custom("xw_plus_b", [X, Wt, Bv], i_args=[0, 1])[0].to_float()
     assert _last_kernel(ex).startswith("gemm_mfma16d<bf16,256x256,akc=1,bkc=1>"), _last_kernel(ex)
     assert np.array_equal(zt, z)
+
+
+def test_small_tile_ring_and_register_staged_kernel_give_the_same_bits(tmp_path):
+    """The 64 x 64 direct-load ring (gemm_mfma16s) and the register-staged kernel it replaced by default (gemm_mfma16q, kept
+    for operands the ring does not take) add the same products in the same order: identical results, with a pitched A and
+    with alpha / beta / bias as well."""
+    import os, subprocess, sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    child = r"""
+import sys, math, numpy as np
+sys.path.insert(0, %r)
+from deeplearning4j_amd.executioner import Executioner
+from deeplearning4j_amd.ndarray import NDArray, BFLOAT16, HALF, f32_to_bf16_bits
+ex = Executioner()
+rng = np.random.default_rng(77)
+out, names = {}, []
+for n, (dt, M, N, K) in enumerate([(BFLOAT16, 1024, 1024, 1024), (HALF, 1024, 1024, 768), (BFLOAT16, 1024, 1024, 512)]):
+    conv = (lambda v: f32_to_bf16_bits(v.astype(np.float32))) if dt == BFLOAT16 else (lambda v: v.astype(np.float16))
+    a = rng.normal(0, 1 / math.sqrt(K), (M, K + 8)); b = rng.normal(0, 1, (K, N)); c = rng.normal(0, 1, (M, N))
+    A = NDArray.from_numpy(conv(a), dt).slice(1, 0, K)                  # pitched rows
+    B, Bt = NDArray.from_numpy(conv(b), dt), NDArray.from_numpy(conv(np.ascontiguousarray(b.T)), dt)
+    for tag, ops, ia in (("plain", [A, B], [0, 0]), ("tb", [A, Bt], [0, 1])):
+        Z = NDArray.from_numpy(conv(c), dt)
+        ex.exec_custom("matmul", ops, [Z], t_args=[0.5, 2.0], i_args=ia)
+        out["%%d_%%s" %% (n, tag)] = Z.to_numpy(); names.append(ex.L.nd4jhipLastGemmKernel().decode())
+np.savez(sys.argv[1], names=np.array(names), **out)
+"""
+    res = []
+    for ring in (1, 0):
+        path = str(tmp_path / ("ring%d.npz" % ring))
+        r = subprocess.run([sys.executable, "-c", child % root, path], env=dict(os.environ, ND4JHIP_GEMM_SMALL_RING=str(ring)),
+                           capture_output=True, text=True, timeout=300)
+        assert r.returncode == 0, r.stderr[-2000:]
+        res.append(np.load(path))
+    one, two = res
+    assert all("gemm_mfma16s" in str(s_) for s_ in one["names"]), list(one["names"])
+    assert all("gemm_mfma16q" in str(s_) for s_ in two["names"]), list(two["names"])
+    for key in one.files:
+        if key != "names":
+            assert np.array_equal(one[key], two[key]), key
