@@ -518,18 +518,21 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16q(GemmArgs g, const T
   storeAccTiles<T, TM, TN, true>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
 }
 
-// 64 x 64 tiles with the operands going from global memory straight into LDS (no registers, no LDS stores), NST stages in
-// a ring: for launches that put one or two small tiles on a CU (1024^3; the projections of a prefill), where the
-// register-staged kernel above spends more on parking the tiles in LDS than on multiplying them.  A k-contiguous, B either
-// way; whole tiles, K a multiple of NST K-tiles.  A wave instruction moves a chunk of 1 KiB (64 slots of 16 bytes in lane
-// order): 8 rows x 128 bytes of a k-contiguous operand, placed so that the fragment read of 32 consecutive rows is free of
-// bank conflicts (the placement of gemm_mfma16d), or 8 k-rows x 128 bytes of row-major B, swizzled as RowTileLoader keeps
-// them and read with the transposing LDS read.  Round kt: wait for tile kt + 1 (this wave's chunks), barrier (everybody's),
-// refill the stage tile kt - 1 left, read the fragments of tile kt + 1 while the four MFMAs of tile kt run.
-template <typename T, bool B_KC, int NST>
+// Small tiles (64 x 64 or 128 x 128, four waves of TW x TW accumulator tiles) with the operands going from global memory
+// straight into LDS (no registers, no LDS stores), NST stages in a ring: for launches that put one or two tiles on a CU
+// (1024^3, 2048^3; the projections of a prefill), where the register-staged kernels spend more on parking the tiles in LDS
+// than on multiplying them.  A k-contiguous, B either way; whole tiles, K a multiple of NST K-tiles.  A wave instruction moves
+// a chunk of 1 KiB (64 slots of 16 bytes in lane order): 8 rows x 128 bytes of a k-contiguous operand, placed so that the
+// fragment read of 32 consecutive rows is free of bank conflicts (the placement of gemm_mfma16d), or whole k-rows of
+// row-major B, swizzled as RowTileLoader keeps them and read with the transposing LDS read.  Round kt: wait for tile kt + 1
+// (this wave's chunks), barrier (everybody's), refill the stage tile kt - 1 left, read the fragments of tile kt + 1 while the
+// MFMAs of tile kt run.
+template <typename T, bool B_KC, int NST, int TW>
 __global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
                                                     unsigned tilesM, unsigned tilesN) {
-  constexpr int BM = 64, BN = 64, BK = 64, STAGE = 1024;   // slots of 16 bytes: 512 of A, 512 of B
+  constexpr int BM = 64 * TW, BN = 64 * TW, BK = 64;
+  constexpr int SLOTS_A = BM * 8, STAGE = (BM + BN) * 8;   // slots of 16 bytes
+  constexpr int CPW = BM / 32;                             // chunks per wave and operand
   typedef __attribute__((address_space(3))) void* lds_ptr;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   u32x4* smem = reinterpret_cast<u32x4*>(smem_raw);
@@ -542,17 +545,17 @@ __global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restr
   const int wm = wave >> 1, wn = wave & 1;
   using RowB = RowTileLoader<BN, 256>;
 
-  // ---- global side: two chunks of each operand per wave; a load is scalar base (the tile's first byte) + lane offset ----
-  unsigned offA[2], offB[2];
+  // ---- global side: CPW chunks of each operand per wave; a load is scalar base (the tile's first byte) + lane offset ----
+  unsigned offA[CPW], offB[CPW];
 #pragma unroll
-  for (int c = 0; c < 2; c++) {
-    const int cw = wave * 2 + c, lj = lane >> 3, lp = lane & 7;
+  for (int c = 0; c < CPW; c++) {
+    const int cw = wave * CPW + c, lj = lane >> 3, lp = lane & 7;
     const int lkg = (lp - 4 * (cw & 1) - (lj >> 1)) & 7;
     offA[c] = (unsigned)(((LongType)(cw * 8 + lj) * lda + lkg * 8) * 2);
     if (B_KC) {
       offB[c] = (unsigned)(((LongType)(cw * 8 + lj) * ldb + lkg * 8) * 2);
     } else {
-      const int k = cw * 8 + (lane >> 3), pp = lane & 7;
+      const int k = cw * (64 / RowB::SPR) + lane / RowB::SPR, pp = lane % RowB::SPR;
       offB[c] = (unsigned)(((LongType)k * ldb + (pp ^ RowB::swz(k)) * 8) * 2);
     }
   }
@@ -568,40 +571,48 @@ __global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restr
     const LongType kt = tile < KT ? tile : KT - 1;
     u32x4* const st = smem + stage * STAGE;
 #pragma unroll
-    for (int c = 0; c < 2; c++) dma(baseA + kt * stepA, offA[c], st + (wave * 2 + c) * 64);
+    for (int c = 0; c < CPW; c++) dma(baseA + kt * stepA, offA[c], st + (wave * CPW + c) * 64);
 #pragma unroll
-    for (int c = 0; c < 2; c++) dma(baseB + kt * stepB, offB[c], st + 512 + (wave * 2 + c) * 64);
+    for (int c = 0; c < CPW; c++) dma(baseB + kt * stepB, offB[c], st + SLOTS_A + (wave * CPW + c) * 64);
   };
 
   // ---- LDS side ----
-  int fragA[4], fragB[4];
-  {
-    const int r = wm * 32 + (lane & 31);
+  int fragA[TW][4], fragB[TW][4], trB[TW];
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) fragA[ks] = (r >> 3) * 64 + 8 * (r & 7) + ((2 * ks + h + 4 * ((r >> 3) & 1) + ((r & 7) >> 1)) & 7);
-    const int rb = wn * 32 + (lane & 31);
+  for (int i = 0; i < TW; i++) {
+    const int r = wm * 32 * TW + i * 32 + (lane & 31);
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) fragB[ks] = 512 + (rb >> 3) * 64 + 8 * (rb & 7) + ((2 * ks + h + 4 * ((rb >> 3) & 1) + ((rb & 7) >> 1)) & 7);
+    for (int ks = 0; ks < 4; ks++) fragA[i][ks] = (r >> 3) * 64 + 8 * (r & 7) + ((2 * ks + h + 4 * ((r >> 3) & 1) + ((r & 7) >> 1)) & 7);
+    const int rb = wn * 32 * TW + i * 32 + (lane & 31);
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++)
+      fragB[i][ks] = SLOTS_A + (rb >> 3) * 64 + 8 * (rb & 7) + ((2 * ks + h + 4 * ((rb >> 3) & 1) + ((rb & 7) >> 1)) & 7);
+    trB[i] = RowB::fragOffset(wn * 32 * TW + i * 32, lane);
   }
-  const int trB = RowB::fragOffset(wn * 32, lane);
-  u32x4 fa[2][4], fb[2][4];
+  u32x4 fa[2][4][TW], fb[2][4][TW];
   auto readTile = [&](int stage, int buf) {
     const u32x4* st = smem + stage * STAGE;
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) {
-      fa[buf][ks] = st[fragA[ks]];
-      if (B_KC) fb[buf][ks] = st[fragB[ks]];
-      else fb[buf][ks] = RowB::readFrag(st + 512, trB, ks);
-    }
-  };
-  f32x16 acc[1][1];
+    for (int ks = 0; ks < 4; ks++)
 #pragma unroll
-  for (int r = 0; r < 16; r++) acc[0][0][r] = 0.f;
+      for (int i = 0; i < TW; i++) {
+        fa[buf][ks][i] = st[fragA[i][ks]];
+        if (B_KC) fb[buf][ks][i] = st[fragB[i][ks]];
+        else fb[buf][ks][i] = RowB::readFrag(st + SLOTS_A, trB[i], ks);
+      }
+  };
+  f32x16 acc[TW][TW];
+#pragma unroll
+  for (int i = 0; i < TW; i++)
+#pragma unroll
+    for (int j = 0; j < TW; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
   // tiles 0 .. NST - 2 on their way; tile 0 read before the loop
 #pragma unroll
   for (int u = 0; u < NST - 1; u++) issue(u, u);
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 2) * 4) : "memory");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 2) * 2 * CPW) : "memory");
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_sched_barrier(0);
   readTile(0, 0);
@@ -609,18 +620,22 @@ __global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restr
 #pragma unroll
     for (int u = 0; u < NST; u++) {
       // tile kt0 + u + 1 has landed (the loads of the NST - 3 tiles after it may still be out) and is visible after the barrier
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 3) * 4) : "memory");
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 3) * 2 * CPW) : "memory");
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_sched_barrier(0);
       issue(kt0 + u + NST - 1, (u + NST - 1) % NST);   // the stage of tile kt0 + u - 1: everybody is past its fragments
       readTile((u + 1) % NST, (u + 1) & 1);
 #pragma unroll
-      for (int ks = 0; ks < 4; ks++) acc[0][0] = Mfma16<T>::mma(fa[u & 1][ks], fb[u & 1][ks], acc[0][0]);
+      for (int ks = 0; ks < 4; ks++)
+#pragma unroll
+        for (int i = 0; i < TW; i++)
+#pragma unroll
+          for (int j = 0; j < TW; j++) acc[i][j] = Mfma16<T>::mma(fa[u & 1][ks][i], fb[u & 1][ks][j], acc[i][j]);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the surplus loads of the last rounds
-  storeAccTiles<T, 1, 1, false>(g, C, acc, m0 + wm * 32, n0 + wn * 32, lane);
+  storeAccTiles<T, TW, TW, false>(g, C, acc, m0 + wm * 32 * TW, n0 + wn * 32 * TW, lane);
 }
 
 // Steady-state kernel for problems made of whole tiles (M % BM == 0, N % BN == 0, K % 64 == 0): no bounds handling,
@@ -1199,31 +1214,41 @@ static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
   // K-tiles are in flight
   const unsigned nTiles = (unsigned)(((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN) * batch);
   const bool useDeep = usePipe && !useFull && BM * BN <= 64 * 64 && nTiles <= 1024 && g.K >= 512 && g.M % BM == 0 && g.N % BN == 0 && g.K % 256 == 0;
-  // the direct-load ring takes the small-tile launches it can: 64 x 64 tiles, A k-contiguous, 16-byte aligned rows
-  if constexpr (BM == 64 && BN == 64 && A_KC) {
+  // the direct-load ring takes the small-tile launches it can: 64 x 64 or 128 x 128 tiles, A k-contiguous, 16-byte aligned rows
+  if constexpr ((BM == 64 && BN == 64 || BM == 128 && BN == 128) && WM == 2 && WN == 2 && A_KC) {
+    constexpr int TW = BM / 64;
+    constexpr int STAGE_BYTES = (BM + BN) * 8 * 16;
     static const bool small = getenv("ND4JHIP_GEMM_SMALL_RING") ? atoi(getenv("ND4JHIP_GEMM_SMALL_RING")) != 0 : true;
     const LongType ldaS = g.aRow, ldbS = B_KC ? g.bCol : g.bRow;
-    if (small && useDeep && ldaS % 8 == 0 && ldbS % 8 == 0 && ldaS < (1 << 24) && ldbS < (1 << 24) &&
+    const bool shape = TW == 1 ? useDeep : (useFull && nTiles <= 1024 && g.K >= 512 && g.K % 256 == 0);
+    if (small && shape && ldaS % 8 == 0 && ldbS % 8 == 0 && ldaS < (1 << 23) && ldbS < (1 << 23) &&
         ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 && g.aBatch % 8 == 0 && g.bBatch % 8 == 0 &&
         g.aBatch2 % 8 == 0 && g.bBatch2 % 8 == 0) {
-      const unsigned tM = (unsigned)(g.M / 64), tN = (unsigned)(g.N / 64);
-      // one tile per CU and a K of whole eight-tile rounds: eight stages (128 KiB), else four (two blocks fit a CU)
-      static std::once_flag once8;
-      static bool granted8 = false;
-      const bool want8 = nTiles <= 256 && g.K % 512 == 0;
-      if (want8)
-        std::call_once(once8, [&] {
-          granted8 = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_mfma16s<T, B_KC, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, 8 * 16384) == hipSuccess;
-          if (!granted8) (void)hipGetLastError();
+      const unsigned tM = (unsigned)(g.M / BM), tN = (unsigned)(g.N / BN);
+      // 64 x 64: one tile per CU and a K of whole eight-tile rounds take eight stages (128 KiB), else four (two blocks fit a
+      // CU); 128 x 128: four stages (128 KiB)
+      constexpr int DEEP = TW == 1 ? 8 : 4;
+      static std::once_flag onceDeep;
+      static bool grantedDeep = false;
+      const bool wantDeep = TW == 2 || (nTiles <= 256 && g.K % 512 == 0);
+      if (wantDeep)
+        std::call_once(onceDeep, [&] {
+          grantedDeep = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_mfma16s<T, B_KC, DEEP, TW>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                            DEEP * STAGE_BYTES) == hipSuccess;
+          if (!grantedDeep) (void)hipGetLastError();
         });
-      if (want8 && granted8) {
-        noteKernel("gemm_mfma16s<%s,64x64,akc=1,bkc=%d,stages=8>", tname<T>(), (int)B_KC);
-        hipLaunchKernelGGL((gemm_mfma16s<T, B_KC, 8>), dim3(tM * tN, 1, (unsigned)batch), dim3(256), 8 * 16384, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
-      } else {
-        noteKernel("gemm_mfma16s<%s,64x64,akc=1,bkc=%d,stages=4>", tname<T>(), (int)B_KC);
-        hipLaunchKernelGGL((gemm_mfma16s<T, B_KC, 4>), dim3(tM * tN, 1, (unsigned)batch), dim3(256), 4 * 16384, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
+      if (wantDeep && grantedDeep) {
+        noteKernel("gemm_mfma16s<%s,%dx%d,akc=1,bkc=%d,stages=%d>", tname<T>(), BM, BN, (int)B_KC, DEEP);
+        hipLaunchKernelGGL((gemm_mfma16s<T, B_KC, DEEP, TW>), dim3(tM * tN, 1, (unsigned)batch), dim3(256), DEEP * STAGE_BYTES, s, g, (const T*)A,
+                           (const T*)B, (T*)C, tM, tN);
+        return true;
       }
-      return true;
+      if constexpr (TW == 1) {
+        noteKernel("gemm_mfma16s<%s,64x64,akc=1,bkc=%d,stages=4>", tname<T>(), (int)B_KC);
+        hipLaunchKernelGGL((gemm_mfma16s<T, B_KC, 4, 1>), dim3(tM * tN, 1, (unsigned)batch), dim3(256), 4 * STAGE_BYTES, s, g, (const T*)A, (const T*)B,
+                           (T*)C, tM, tN);
+        return true;
+      }
     }
   }
   auto kern = useFull ? gemm_mfma16f<T, BM, BN, WM, WN, A_KC, B_KC>

@@ -70,8 +70,10 @@ CASES = [
     (HALF, 1024, 1024, 1024, "gemm_mfma16s<f16,64x64,akc=1,bkc=0,stages=8>", "gemm_mfma16s<f16,64x64,akc=1,bkc=1,stages=8>", "gemm_mfma16q<f16,64x64,akc=0,bkc=0>"),
     (BFLOAT16, 1024, 1024, 1024, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=8>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=8>", "gemm_mfma16q<bf16,64x64,akc=0,bkc=0>"),
     # the 128 x 128 configuration (2048-class sizes), whole tiles
-    (BFLOAT16, 2048, 2048, 2048, "gemm_mfma16f<bf16,128x128,akc=1,bkc=0>", "gemm_mfma16f<bf16,128x128,akc=1,bkc=1>", "gemm_mfma16f<bf16,128x128,akc=0,bkc=0>"),
-    (HALF, 2048, 2048, 1024, "gemm_mfma16f<f16,128x128,akc=1,bkc=0>", "gemm_mfma16f<f16,128x128,akc=1,bkc=1>", None),
+    (BFLOAT16, 2048, 2048, 2048, "gemm_mfma16s<bf16,128x128,akc=1,bkc=0,stages=4>", "gemm_mfma16s<bf16,128x128,akc=1,bkc=1,stages=4>", "gemm_mfma16f<bf16,128x128,akc=0,bkc=0>"),
+    (HALF, 2048, 2048, 1024, "gemm_mfma16s<f16,128x128,akc=1,bkc=0,stages=4>", "gemm_mfma16s<f16,128x128,akc=1,bkc=1,stages=4>", None),
+    # a K of whole K-tiles that is not a multiple of four of them stays on the register-staged kernel
+    (HALF, 2048, 2048, 320, "gemm_mfma16f<f16,128x128,akc=1,bkc=0>", "gemm_mfma16f<f16,128x128,akc=1,bkc=1>", None),
     # ragged edges on the large tiles (bounds-handling kernel)
     (BFLOAT16, 3600, 3704, 1000, "gemm_mfma16p<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16p<bf16,256x256,akc=1,bkc=1>", "gemm_mfma16p<bf16,256x256,akc=0,bkc=0>"),
     (HALF, 1800, 1800, 520, "gemm_mfma16p<f16,128x128,akc=1,bkc=0>", "gemm_mfma16p<f16,128x128,akc=1,bkc=1>", None),
