@@ -2015,33 +2015,40 @@ __global__ __launch_bounds__(256) void gemm_skinny32(GemmArgs g, const T* __rest
   const T* wp = Wt + (n0 + lrow) * g.bCol + lkg * 8;
   const T* xp = X + (LongType)(lrow < g.M ? lrow : g.M - 1) * g.aRow + lkg * 8;
   const int tiles = (int)(g.K / 64);
-  u32x4 wr[CT], xr[CT];
-  auto load = [&](int tile0) {
+  // two register sets: the loads of two chunks are on their way at any time, so that K = 768 (two chunks) costs one trip
+  // to memory, not two -- the second chunk's latency was a quarter of the kernel's time
+  u32x4 wr[2][CT], xr[2][CT];
+  auto load = [&](int set, int tile0) {
     const int n = tiles - tile0 < CT ? tiles - tile0 : CT;
 #pragma unroll
     for (int j = 0; j < CT; j++) {
       const int jc = j < n ? j : n - 1;                // unconditional loads; a repeated tile is never multiplied
-      wr[j] = *reinterpret_cast<const u32x4*>(wp + (LongType)(tile0 + jc) * 64);
-      xr[j] = *reinterpret_cast<const u32x4*>(xp + (LongType)(tile0 + jc) * 64);
+      wr[set][j] = *reinterpret_cast<const u32x4*>(wp + (LongType)(tile0 + jc) * 64);
+      xr[set][j] = *reinterpret_cast<const u32x4*>(xp + (LongType)(tile0 + jc) * 64);
     }
   };
   f32x16 acc;
 #pragma unroll
   for (int r = 0; r < 16; r++) acc[r] = 0.f;
   const int mrow = lane & 31, h = lane >> 5;
-  load(0);
-  for (int tile0 = 0; tile0 < tiles; tile0 += CT) {
+  load(0, 0);
+  if (CT < tiles) load(1, CT);
+  auto chunk = [&](int set, int tile0) {
     const int n = tiles - tile0 < CT ? tiles - tile0 : CT;
 #pragma unroll
     for (int j = 0; j < CT; j++) {
-      sW[(j * 8 + lkg) * GROUP + lrow] = wr[j];
-      sX[(j * 8 + lkg) * GROUP + lrow] = xr[j];
+      sW[(j * 8 + lkg) * GROUP + lrow] = wr[set][j];
+      sX[(j * 8 + lkg) * GROUP + lrow] = xr[set][j];
     }
     __syncthreads();
-    if (tile0 + CT < tiles) load(tile0 + CT);
+    if (tile0 + 2 * CT < tiles) load(set, tile0 + 2 * CT);
     for (int s = wave; s < n * 4; s += 4)
       acc = Mfma16<T>::mma(sW[(2 * s + h) * GROUP + mrow], sX[(2 * s + h) * GROUP + mrow], acc);
     __syncthreads();
+  };
+  for (int tile0 = 0; tile0 < tiles; tile0 += 2 * CT) {
+    chunk(0, tile0);
+    if (tile0 + CT < tiles) chunk(1, tile0 + CT);
   }
 #pragma unroll
   for (int r = 0; r < 16; r++) red[(wave * 16 + r) * 64 + lane] = acc[r];
