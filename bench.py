@@ -43,7 +43,7 @@ TRAFFIC_MB = {
     "mmul f32 1024": 29.5, "mmul f16 1024": 14.8, "mmul bf16 1024": 14.8,
     "copy fp32": 268.4, "pairwise_add fp32": 402.6, "transform_tanh fp32": 268.4, "reduce_sum": 134.5, "argmax dim1": 134.5,
     "layer_norm fp32": 100.8, "gelu fp32": 100.7, "softmax fp32": 1610.6, "layer_norm bf16": 50.4, "gelu bf16": 50.4,
-    "softmax bf16": 805.3, "dot_product_attention_v2": 53.5,
+    "softmax bf16": 805.3, "dot_product_attention_v2": 50.5,
 }
 
 
