@@ -315,3 +315,64 @@ def test_row_ops_over_row_lengths_and_row_counts(ex, oracle):
             z = ex.exec_transform_strict(TransformStrict.GELU, dx, NDArray.empty((rows, C), dt))
             got, want = z.to_float().astype(np.float64), _ovals(oz)
             assert np.all(np.abs(got - want) <= atol * 1e-1 + rtol * np.abs(want)), "gelu " + tag
+
+
+def test_attention_on_random_shapes_masks_and_layouts(ex, oracle):
+    """dot_product_attention_v2, output only (the fused tile kernel, the streaming kernel for a handful of query rows, or the
+    composition for head sizes the fused kernels do not take): random batch, lengths from one key to a few tiles with ragged
+    ends, head sizes 32 / 64 / 128, causal or not, with and without a value mask, operands dense or as token-major head
+    views [T, heads, D] -> [heads, T, D], against the oracle's literal composition (AttentionHelper.cpp:189-241, 340-352).
+    bf16 at head size 128 is held to 2.5 times the gate: the composition itself is that far from the exact result."""
+    import math
+    rng = np.random.default_rng(20247)
+    for case in range(48):
+        dt = [BFLOAT16, HALF][case % 2]
+        D = [64, 64, 128, 32][case % 4]
+        B = int(rng.integers(1, 4))
+        Tq = int(rng.choice([1, 2, 5, 8, 9, 31, 64, 65, 127, 128, 129, 200, 257, 300]))
+        Tv = int(rng.choice([1, 3, 63, 64, 65, 100, 128, 191, 192, 193, 320, 400]))
+        causal = bool(rng.integers(0, 2))
+        masked = case % 3 == 0
+        views = case % 5 == 1
+        scale = [1 / math.sqrt(D), 0.11, 1.0][case % 3]
+
+        def operand(T):
+            vals = rng.normal(0, 1, (B, T, D))
+            if not views:
+                return _opair(oracle, vals, dt) + (None,)
+            tok = np.ascontiguousarray(vals.transpose(1, 0, 2))          # [T, heads, D] in memory
+            o, d = _opair(oracle, tok, dt)
+            return oracle.Arr(np.ascontiguousarray(o.a.transpose(1, 0, 2)), o.dt), d.permute(1, 0, 2), d
+        oq, dq, _k1 = operand(Tq)
+        ok, dk, _k2 = operand(Tv)
+        ov, dv, _k3 = operand(Tv)
+        oo, ow, ol = _ozero(oracle, (B, Tq, D), dt), _ozero(oracle, (B, Tq, Tv), dt), _ozero(oracle, (B, Tq, Tv), dt)
+        ins = [dq, dv, dk]
+        kw = {}
+        if masked:
+            vm = (rng.random((B, Tv)) > 0.4).astype(np.float32)
+            vm[:, 0] = 1
+            ovm, dvm = _opair(oracle, vm, dt)
+            kw["v_mask"] = ovm
+            ins = [dq, dv, dk, NDArray.empty((0,), dt), dvm]
+        oracle.attention_v2(oq, ov, ok, oo, ow, ol, scale=scale, causal=causal, **kw)
+        out = ex.exec_custom("dot_product_attention_v2", ins, [NDArray.empty((B, Tq, D), dt)], t_args=[scale, 0.0], b_args=[causal, False])[0]
+        got, want = out.to_float().astype(np.float64), _ovals(oo)
+        tol = 1e-2 if dt == BFLOAT16 else 2e-3
+        tag = "case %d: dtype %d B %d Tq %d Tv %d D %d causal %d masked %d views %d scale %g" % (case, dt, B, Tq, Tv, D, causal, masked, views, scale)
+        # the composition rounds every intermediate to the storage type and is itself some way from the exact result (at bf16
+        # up to 0.02 on single elements): the kernel must stay within 2.5 times the gate of the composition and must not be
+        # further from the exact result than the composition is
+        assert np.all(np.abs(got - want) <= 2.5 * tol * (1 + np.abs(want))), tag + ": worst %g against the composition" % float(np.abs(got - want).max())
+        q64, k64, v64 = _ovals(oq), _ovals(ok), _ovals(ov)
+        sc64 = np.clip(np.einsum("bqd,bkd->bqk", q64, k64) * scale, -1e4, 1e4)
+        hide = np.zeros((B, Tq, Tv), bool)
+        if causal:
+            hide |= ~np.tril(np.ones((Tq, Tv), bool))[None]
+        if masked:
+            hide |= (vm == 0)[:, None, :]
+        sc64 = np.where(hide, -np.inf, sc64)
+        p64 = np.exp(sc64 - sc64.max(-1, keepdims=True))
+        truth = np.einsum("bqk,bkd->bqd", p64 / p64.sum(-1, keepdims=True), v64)
+        assert np.abs(got - truth).max() <= 1.25 * np.abs(want - truth).max() + tol / 4, tag + ": %g from the exact result, the composition %g" % (
+            float(np.abs(got - truth).max()), float(np.abs(want - truth).max()))
