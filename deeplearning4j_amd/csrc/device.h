@@ -107,6 +107,34 @@ template <> struct RawIO<f16_t> {
   }
 };
 
+// 12-byte vectors of a 16-bit type (six values, one global_load_dwordx3): a wave pass covers 384 values, so a row of 768
+// is two full passes where 16-byte vectors leave a quarter of the load slots idle.  Rows need 4-byte alignment only.
+struct alignas(4) raw_u32x3 {
+  unsigned v[3];
+  __device__ __forceinline__ unsigned& operator[](int i) { return v[i]; }
+  __device__ __forceinline__ unsigned operator[](int i) const { return v[i]; }
+};
+template <typename T> struct RawIO12 {
+  using raw = raw_u32x3;
+  static constexpr int N = 6;
+  static __device__ __forceinline__ void unpack(raw r, float* out) {
+#pragma unroll
+    for (int p = 0; p < 3; p++) {
+      T lo, hi;
+      lo.bits = (unsigned short)(r[p] & 0xffffu);
+      hi.bits = (unsigned short)(r[p] >> 16);
+      out[2 * p] = to_float(lo);
+      out[2 * p + 1] = to_float(hi);
+    }
+  }
+  static __device__ __forceinline__ raw pack(const float* in) {
+    raw r;
+#pragma unroll
+    for (int p = 0; p < 3; p++) r[p] = (unsigned)Conv<T>::from(in[2 * p]).bits | ((unsigned)Conv<T>::from(in[2 * p + 1]).bits << 16);
+    return r;
+  }
+};
+
 // ---- fast math for the fused row/activation kernels ---------------------------------------------------
 // 1/x from the hardware reciprocal (1 ulp) instead of the 11-instruction IEEE division sequence
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }

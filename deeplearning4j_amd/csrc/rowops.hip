@@ -607,12 +607,12 @@ __global__ __launch_bounds__(256) void layernorm_linear(const T* __restrict__ x,
 // the first use.  The grid normally gives every wave one pair; beyond 2^20 blocks a wave walks on to pair pr + W with
 // that pair's loads issued ahead.  (About ten vector instructions per element: a 16-bit row is as much arithmetic as an
 // fp32 row of the same length in half the bytes, which is why bf16 [16384, 768] takes 9.5 us where gelu takes 5.3.)
-template <typename T, int NV, bool HAS_BIAS>
+template <typename T, int NV, bool HAS_BIAS, typename IO = RawIO<T>>
 __global__ __launch_bounds__(256) void layernorm_stream(const T* __restrict__ x, const T* __restrict__ gain, const T* __restrict__ bias, T* __restrict__ z,
                                                         LongType rows, int L, LongType xPitch, LongType zPitch, float eps) {
   using A = typename Conv<T>::acc;
-  using Raw = typename RawIO<T>::raw;
-  constexpr int VEC = RawIO<T>::N;
+  using Raw = typename IO::raw;
+  constexpr int VEC = IO::N;
   const int t = threadIdx.x & 63;
   const LongType W = (LongType)gridDim.x * 4, pairs = (rows + 1) / 2;
   LongType pr = (LongType)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -649,7 +649,7 @@ __global__ __launch_bounds__(256) void layernorm_stream(const T* __restrict__ x,
       sum[r] = (A)0;
 #pragma unroll
       for (int i = 0; i < NV; i++) {
-        RawIO<T>::unpack(cur[r][i], &vals[r][i * VEC]);
+        IO::unpack(cur[r][i], &vals[r][i * VEC]);
         A part = (A)0;
 #pragma unroll
         for (int e = 0; e < VEC; e++) part += vals[r][i * VEC + e];
@@ -682,15 +682,15 @@ __global__ __launch_bounds__(256) void layernorm_stream(const T* __restrict__ x,
 #pragma unroll
       for (int i = 0; i < NV; i++) {
         A g[VEC], b[VEC];
-        RawIO<T>::unpack(gv[i], g);
-        if (HAS_BIAS) RawIO<T>::unpack(bv[i], b);
+        IO::unpack(gv[i], g);
+        if (HAS_BIAS) IO::unpack(bv[i], b);
 #pragma unroll
         for (int e = 0; e < VEC; e++) {
           A y = vals[r][i * VEC + e] * rstd * g[e];
           if (HAS_BIAS) y += b[e];
           vals[r][i * VEC + e] = y;
         }
-        if (keep[i] != (A)0) *reinterpret_cast<Raw*>(zr + e0[i]) = RawIO<T>::pack(&vals[r][i * VEC]);
+        if (keep[i] != (A)0) *reinterpret_cast<Raw*>(zr + e0[i]) = IO::pack(&vals[r][i * VEC]);
       }
     }
     if (more) {
@@ -727,6 +727,17 @@ static void layerNormTyped(hipStream_t s, const void* x, const void* gain, const
         const unsigned gs = (unsigned)std::min<LongType>((p.rows + 7) / 8, (LongType)1 << 20);
 #define LNS(NV) do { if (bt) hipLaunchKernelGGL((layernorm_stream<T, NV, true>), dim3(gs), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); \
                      else hipLaunchKernelGGL((layernorm_stream<T, NV, false>), dim3(gs), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); } while (0)
+        // 16-bit rows of a whole number of 384-value passes that are not a whole number of 512-value ones (768: one and a
+        // half): 12-byte vectors, every load slot used
+        if constexpr (sizeof(T) == 2) {
+          if (L % 384 == 0 && L % 512 != 0 && L <= 4 * 384) {
+#define LNS12(NV) do { if (bt) hipLaunchKernelGGL((layernorm_stream<T, NV, true, RawIO12<T>>), dim3(gs), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); \
+                       else hipLaunchKernelGGL((layernorm_stream<T, NV, false, RawIO12<T>>), dim3(gs), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); } while (0)
+            if (L == 384) LNS12(1); else if (L == 768) LNS12(2); else LNS12(3);
+#undef LNS12
+            return;
+          }
+        }
         if (L <= perWave) LNS(1); else if (L <= 2 * perWave) LNS(2); else if (L <= 3 * perWave) LNS(3); else LNS(4);
 #undef LNS
         return;

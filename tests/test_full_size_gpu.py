@@ -148,12 +148,14 @@ def test_config4_weights_and_logits_outputs(ex, oracle, dt):
         assert np.array_equal(lgot[~keep], lo[~keep]) or np.allclose(lgot[~keep], lo[~keep], rtol=1e-2)
 
 
-@pytest.mark.parametrize("dt,L,tol", [(BFLOAT16, 768, 1e-2), (HALF, 768, 2e-3), (FLOAT32, 384, 1e-5)])
+@pytest.mark.parametrize("dt,L,tol", [(BFLOAT16, 768, 1e-2), (HALF, 768, 2e-3), (FLOAT32, 384, 1e-5),
+                                      (BFLOAT16, 384, 1e-2), (HALF, 1152, 2e-3), (BFLOAT16, 1152, 1e-2), (HALF, 640, 2e-3)])
 @pytest.mark.parametrize("rows,has_bias,pitched", [(4097, True, False), (4608, False, False), (4099, True, True)])
 def test_layer_norm_rows_of_one_and_a_half_passes(ex, oracle, dt, L, tol, rows, has_bias, pitched):
-    """Many rows (two per wave) whose length is one and a half 16-byte wave passes, so that the second pass is half
-    masked: an odd row count (the last wave has a lone row), no bias, and rows at a pitch (the left columns of a wider
-    matrix), every row against the oracle."""
+    """Many rows (two per wave) whose length is not a whole number of 16-byte wave passes: 16-bit rows of 384, 768 and
+    1152 go in 12-byte vectors (one, two, three full passes), fp32 rows of 384 and 16-bit rows of 640 in 16-byte vectors
+    with the last pass partly masked.  An odd row count (the last wave has a lone row), no bias, and rows at a pitch (the
+    left columns of a wider matrix), every row against the oracle."""
     rng = np.random.default_rng(rows + L + int(has_bias))
     width = L + 64 if pitched else L
     full, Full = _store(rng.normal(0.3, 2.0, (rows, width)).astype(np.float32), dt)
