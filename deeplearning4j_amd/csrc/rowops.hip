@@ -607,8 +607,8 @@ __global__ __launch_bounds__(256) void layernorm_linear(const T* __restrict__ x,
 // the first use.  The grid normally gives every wave one pair; beyond 2^20 blocks a wave walks on to pair pr + W with
 // that pair's loads issued ahead.  (About ten vector instructions per element: a 16-bit row is as much arithmetic as an
 // fp32 row of the same length in half the bytes, which is why bf16 [16384, 768] takes 9.5 us where gelu takes 5.3.)
-template <typename T, int NV, bool HAS_BIAS, typename IO = RawIO<T>>
-__global__ __launch_bounds__(256) void layernorm_stream(const T* __restrict__ x, const T* __restrict__ gain, const T* __restrict__ bias, T* __restrict__ z,
+template <typename T, int NV, bool HAS_BIAS, typename IO = RawIO<T>, bool WALK = true>
+__global__ __launch_bounds__(256, WALK ? 1 : 8) void layernorm_stream(const T* __restrict__ x, const T* __restrict__ gain, const T* __restrict__ bias, T* __restrict__ z,
                                                         LongType rows, int L, LongType xPitch, LongType zPitch, float eps) {
   using A = typename Conv<T>::acc;
   using Raw = typename IO::raw;
@@ -635,13 +635,16 @@ __global__ __launch_bounds__(256) void layernorm_stream(const T* __restrict__ x,
     }
   };
   load(pr, cur);
+  auto loadGainBias = [&]() {
 #pragma unroll
-  for (int i = 0; i < NV; i++) {
-    gv[i] = *reinterpret_cast<const Raw*>(gain + e0[i]);
-    if (HAS_BIAS) bv[i] = *reinterpret_cast<const Raw*>(bias + e0[i]);
-  }
+    for (int i = 0; i < NV; i++) {
+      gv[i] = *reinterpret_cast<const Raw*>(gain + e0[i]);
+      if (HAS_BIAS) bv[i] = *reinterpret_cast<const Raw*>(bias + e0[i]);
+    }
+  };
+  loadGainBias();
   for (; pr < pairs; pr += W) {
-    const bool more = pr + W < pairs;
+    const bool more = WALK && pr + W < pairs;
     if (more) load(pr + W, nxt);
     A vals[2][NV * VEC], sum[2];
 #pragma unroll
@@ -693,6 +696,7 @@ __global__ __launch_bounds__(256) void layernorm_stream(const T* __restrict__ x,
         if (keep[i] != (A)0) *reinterpret_cast<Raw*>(zr + e0[i]) = IO::pack(&vals[r][i * VEC]);
       }
     }
+    if (!WALK) break;
     if (more) {
 #pragma unroll
       for (int r = 0; r < 2; r++)
@@ -725,16 +729,22 @@ static void layerNormTyped(hipStream_t s, const void* x, const void* gain, const
         // one pair per wave while the grid allows it (fewer, longer-running waves measured slower: bf16 [16384, 768] 12.7 us
         // per launch with one pair per wave, 13.5 with four, 14.1 with eight)
         const unsigned gs = (unsigned)std::min<LongType>((p.rows + 7) / 8, (LongType)1 << 20);
+        // every wave has one pair only (12-byte vectors, up to two passes): the variant without the next pair's registers,
+        // 59 instead of 93 of them, eight waves per SIMD.  bf16 [16384, 768] 12.7 -> 11.8 us; the same variant of the 16-byte
+        // kernels measured equal or slower (bf16 rows of 512 8.8 -> 9.1 us, fp32 rows of 384 12.0 -> 12.6) and is not built
+        const bool oneEach = (LongType)gs * 8 >= p.rows;
 #define LNS(NV) do { if (bt) hipLaunchKernelGGL((layernorm_stream<T, NV, true>), dim3(gs), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); \
                      else hipLaunchKernelGGL((layernorm_stream<T, NV, false>), dim3(gs), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); } while (0)
         // 16-bit rows of a whole number of 384-value passes that are not a whole number of 512-value ones (768: one and a
         // half): 12-byte vectors, every load slot used
         if constexpr (sizeof(T) == 2) {
           if (L % 384 == 0 && L % 512 != 0 && L <= 4 * 384) {
-#define LNS12(NV) do { if (bt) hipLaunchKernelGGL((layernorm_stream<T, NV, true, RawIO12<T>>), dim3(gs), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); \
-                       else hipLaunchKernelGGL((layernorm_stream<T, NV, false, RawIO12<T>>), dim3(gs), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); } while (0)
+#define LNS12W(NV, WALK) do { if (bt) hipLaunchKernelGGL((layernorm_stream<T, NV, true, RawIO12<T>, WALK>), dim3(gs), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); \
+                       else hipLaunchKernelGGL((layernorm_stream<T, NV, false, RawIO12<T>, WALK>), dim3(gs), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); } while (0)
+#define LNS12(NV) do { if (oneEach && NV <= 2) LNS12W(NV, (NV > 2)); else LNS12W(NV, true); } while (0)
             if (L == 384) LNS12(1); else if (L == 768) LNS12(2); else LNS12(3);
 #undef LNS12
+#undef LNS12W
             return;
           }
         }
