@@ -164,6 +164,7 @@ struct LaunchShape {
   LongType segLen;
   bool flat;
   int vectorOk;
+  int peelOk;   // unit-stride runs whose starts are not 16-byte aligned: vector loads after a scalar head (index kernels)
 };
 
 static LaunchShape shapeLaunch(const ReducePlan& p, size_t elemSize, const void* x, size_t partialSize, size_t scratchBytes) {
@@ -199,6 +200,7 @@ static LaunchShape shapeLaunch(const ReducePlan& p, size_t elemSize, const void*
   for (int d = 0; d < p.outer.rank && ok; d++) if (p.outer.shape[d] > 1 && p.outer.stride[d] % V != 0) ok = false;
   if (s.splits > 1 && s.segLen % V != 0) ok = false;
   s.vectorOk = ok ? 1 : 0;
+  s.peelOk = unitInner ? 1 : 0;
   return s;
 }
 
@@ -583,27 +585,35 @@ __global__ __launch_bounds__(256) void index_coop(CoopArgs a, const T* __restric
       LongType j = j0;
       if (vectorOk) {
         using VT = Vec<T, V>;
-        const LongType nv = (j1 - j0) / V;
-        const VT* pv = reinterpret_cast<const VT*>(p + j0);
+        // vectorOk 2: the run starts anywhere (rows of an odd length): the elements up to the first 16-byte boundary are
+        // read one by one, as the tail is.  Ties go to the lower index whatever the order of the visits.
+        LongType f0 = j0;
+        if (vectorOk == 2) {
+          f0 = j0 + (LongType)(((16 - (reinterpret_cast<uintptr_t>(p + j0) & 15)) & 15) / sizeof(T));
+          if (f0 > j1) f0 = j1;
+          for (LongType q = j0 + t; q < f0; q += TPR) { A c = idxPre<IK, A>((A)to_float(p[q])); if (idxBetter<IK, A>(bv, bi, c, (int)q)) { bv = c; bi = (int)q; } }
+        }
+        const LongType nv = (j1 - f0) / V;
+        const VT* pv = reinterpret_cast<const VT*>(p + f0);
         LongType i = t;
         for (; i + 3 * TPR < nv; i += 4 * TPR) {
           VT v0 = pv[i], v1 = pv[i + TPR], v2 = pv[i + 2 * TPR], v3 = pv[i + 3 * TPR];
           // ascending index order inside a thread: a strict comparison keeps the first extreme
 #pragma unroll
-          for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v0.v[e])); int ci = (int)(j0 + i * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
+          for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v0.v[e])); int ci = (int)(f0 + i * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
 #pragma unroll
-          for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v1.v[e])); int ci = (int)(j0 + (i + TPR) * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
+          for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v1.v[e])); int ci = (int)(f0 + (i + TPR) * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
 #pragma unroll
-          for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v2.v[e])); int ci = (int)(j0 + (i + 2 * TPR) * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
+          for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v2.v[e])); int ci = (int)(f0 + (i + 2 * TPR) * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
 #pragma unroll
-          for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v3.v[e])); int ci = (int)(j0 + (i + 3 * TPR) * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
+          for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v3.v[e])); int ci = (int)(f0 + (i + 3 * TPR) * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
         }
         for (; i < nv; i += TPR) {
           VT v0 = pv[i];
 #pragma unroll
-          for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v0.v[e])); int ci = (int)(j0 + i * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
+          for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v0.v[e])); int ci = (int)(f0 + i * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
         }
-        j = j0 + nv * V;
+        j = f0 + nv * V;
       }
       for (LongType q = j + t; q < j1; q += TPR) { A c = idxPre<IK, A>((A)to_float(p[q])); if (idxBetter<IK, A>(bv, bi, c, (int)q)) { bv = c; bi = (int)q; } }
     } else if (a.inner.rank == 1) {
@@ -723,15 +733,16 @@ static void indexTyped(hipStream_t st, const void* x, void* z, const ReducePlan&
   LaunchShape s = shapeLaunch(p, sizeof(T), x, sizeof(IdxVal<A>), scratchBytes);
   CoopArgs a = makeArgs(p, s, POST_ID);
   if (tryIndexRowsFast<IK, T, ZT>(st, x, z, p, s)) return;
+  const int vec = s.vectorOk ? 1 : (s.peelOk ? 2 : 0);
   if (s.flat) {
     hipLaunchKernelGGL((index_flat<IK, T, ZT>), dim3((unsigned)((p.outerLen + 255) / 256)), dim3(256), 0, st, a, (const T*)x, (ZT*)z);
     return;
   }
   const LongType units = p.outerLen * s.splits;
   if (s.tpr == 64)
-    hipLaunchKernelGGL((index_coop<IK, T, 64, ZT>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, st, a, (const T*)x, (ZT*)z, (IdxVal<A>*)scratch, s.vectorOk);
+    hipLaunchKernelGGL((index_coop<IK, T, 64, ZT>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, st, a, (const T*)x, (ZT*)z, (IdxVal<A>*)scratch, vec);
   else
-    hipLaunchKernelGGL((index_coop<IK, T, 256, ZT>), dim3((unsigned)units), dim3(256), 0, st, a, (const T*)x, (ZT*)z, (IdxVal<A>*)scratch, s.vectorOk);
+    hipLaunchKernelGGL((index_coop<IK, T, 256, ZT>), dim3((unsigned)units), dim3(256), 0, st, a, (const T*)x, (ZT*)z, (IdxVal<A>*)scratch, vec);
   if (s.splits > 1)
     hipLaunchKernelGGL((index_finish<IK, T, ZT>), dim3((unsigned)((p.outerLen + 255) / 256)), dim3(256), 0, st, a, (const IdxVal<A>*)scratch, (ZT*)z);
 }

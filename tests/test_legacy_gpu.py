@@ -303,6 +303,28 @@ def test_index_reduce_ties_nan_inf_and_scalar(ex, oracle):
     assert ex.exec_index_reduce(0, NDArray.from_numpy(big)).to_numpy() == 123456
 
 
+@pytest.mark.parametrize("dtype", [FLOAT32, BFLOAT16, HALF, DOUBLE])
+@pytest.mark.parametrize("rows,L,first", [(32, 50257, 0), (1, 50257, 3), (4, 200003, 1), (7, 3001, 5), (3, 17, 1), (2, 40001, 7)])
+def test_index_reduce_rows_that_start_off_a_16_byte_boundary(ex, oracle, dtype, rows, L, first):
+    """Rows of an odd length, and the columns first.. of a wider matrix: no row starts on a 16-byte boundary, so a run is
+    read as a scalar head, vectors and a scalar tail (cut into segments where the rows are few and long).  Heavy ties, and
+    rows whose only extreme sits in the head, in the last element, or on both sides of a segment boundary."""
+    rng = np.random.default_rng(rows * L + first)
+    full = rng.integers(-3, 4, (rows, L + first)).astype(np.float64)
+    x = full[:, first:]
+    x[0, :] = 1.0                                   # all equal: index 0
+    if rows > 1: x[1, :] = -3.0; x[1, 0] = 5.0; x[1, L - 1] = -5.0          # extremes in the head and in the last element
+    if rows > 2: x[2, :] = 0.0; x[2, L - 1] = 4.0; x[2, 1] = -4.0
+    if rows > 3 and L > 8448 + 2: x[3, :] = 0.0; x[3, [8447, 8448, 8449]] = 2.0    # a tie across a segment boundary
+    _, dfull = _oracle_arr(oracle, full, dtype)     # small integers: exact in every storage type
+    dx = dfull.slice(1, first, first + L) if first else dfull
+    xr = np.ascontiguousarray(x).astype(np.float64 if dtype == DOUBLE else np.float32)
+    for op in (0, 1, 2, 3):
+        want = oracle.index_reduce(op, xr, np.zeros(rows, np.int64), [1])
+        assert np.array_equal(ex.exec_index_reduce(op, dx, [1]).to_numpy(), want), (op, rows, L, first)
+    assert np.array_equal(ex.exec_index_reduce(0, dx, [1]).to_numpy(), xr.argmax(1))
+
+
 @pytest.mark.parametrize("rows,L,pitch", [(37, 1028, 1028), (5, 8192, 8192), (9, 5000, 5000), (33, 4096, 4352), (3, 1024, 2048)])
 def test_reductions_over_rows_at_a_constant_pitch(ex, oracle, rows, L, pitch):
     """Rows of 1024..8192 elements at a constant pitch take the one-shot kernels (all loads up front, masked tail):
