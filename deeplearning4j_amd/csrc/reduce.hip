@@ -560,14 +560,14 @@ __device__ __forceinline__ void wave_idx_allreduce(double& v, int& i) {
 template <typename ZT>
 __device__ __forceinline__ void storeIndex(ZT* z, LongType off, int idx) { z[off] = (ZT)idx; }
 
-template <int IK, typename T, int TPR, typename ZT>
-__global__ __launch_bounds__(256) void index_coop(CoopArgs a, const T* __restrict__ x, ZT* __restrict__ z,
-                                                  IdxVal<typename Conv<T>::acc>* __restrict__ partials, int vectorOk) {
+template <int IK, typename T, int TPR, typename ZT, int BLOCK = 256>
+__global__ __launch_bounds__(BLOCK) void index_coop(CoopArgs a, const T* __restrict__ x, ZT* __restrict__ z,
+                                                    IdxVal<typename Conv<T>::acc>* __restrict__ partials, int vectorOk) {
   using A = typename Conv<T>::acc;
   constexpr int V = 16 / sizeof(T);
-  constexpr int ROWS = 256 / TPR;
-  __shared__ A ldsV[4];
-  __shared__ int ldsI[4];
+  constexpr int ROWS = BLOCK / TPR;
+  __shared__ A ldsV[BLOCK / 64];
+  __shared__ int ldsI[BLOCK / 64];
   const int t = threadIdx.x % TPR;
   const LongType unit = (LongType)blockIdx.x * ROWS + threadIdx.x / TPR;
   const LongType row = unit / a.splits;
@@ -595,23 +595,21 @@ __global__ __launch_bounds__(256) void index_coop(CoopArgs a, const T* __restric
         }
         const LongType nv = (j1 - f0) / V;
         const VT* pv = reinterpret_cast<const VT*>(p + f0);
-        LongType i = t;
-        for (; i + 3 * TPR < nv; i += 4 * TPR) {
-          VT v0 = pv[i], v1 = pv[i + TPR], v2 = pv[i + 2 * TPR], v3 = pv[i + 3 * TPR];
-          // ascending index order inside a thread: a strict comparison keeps the first extreme
+        // eight vectors per thread and trip, all asked for before the first is looked at (past the end: the last vector
+        // again, not counted), so that a run of up to 8 * TPR vectors costs one trip to memory
+        constexpr int UNR = 8;
+        for (LongType i = t; i < nv; i += (LongType)UNR * TPR) {
+          VT v[UNR];
 #pragma unroll
-          for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v0.v[e])); int ci = (int)(f0 + i * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
+          for (int k = 0; k < UNR; k++) { const LongType ik = i + (LongType)k * TPR; v[k] = pv[ik < nv ? ik : nv - 1]; }
 #pragma unroll
-          for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v1.v[e])); int ci = (int)(f0 + (i + TPR) * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
+          for (int k = 0; k < UNR; k++) {
+            const LongType ik = i + (LongType)k * TPR;
+            if (ik < nv) {
 #pragma unroll
-          for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v2.v[e])); int ci = (int)(f0 + (i + 2 * TPR) * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
-#pragma unroll
-          for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v3.v[e])); int ci = (int)(f0 + (i + 3 * TPR) * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
-        }
-        for (; i < nv; i += TPR) {
-          VT v0 = pv[i];
-#pragma unroll
-          for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v0.v[e])); int ci = (int)(f0 + i * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
+              for (int e = 0; e < V; e++) { A c = idxPre<IK, A>((A)to_float(v[k].v[e])); int ci = (int)(f0 + ik * V + e); if (idxBetter<IK, A>(bv, bi, c, ci)) { bv = c; bi = ci; } }
+            }
+          }
         }
         j = f0 + nv * V;
       }
@@ -624,13 +622,14 @@ __global__ __launch_bounds__(256) void index_coop(CoopArgs a, const T* __restric
     }
   }
   wave_idx_allreduce<IK>(bv, bi);
-  if (TPR == 256) {
+  if (TPR > 64) {
+    static_assert(TPR <= 64 || TPR == BLOCK, "a row takes one wave or the whole block");
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     if (lane == 0) { ldsV[w] = bv; ldsI[w] = bi; }
     __syncthreads();
     bv = ldsV[0]; bi = ldsI[0];
 #pragma unroll
-    for (int q = 1; q < 4; q++) idxMerge<IK, A>(bv, bi, ldsV[q], ldsI[q]);
+    for (int q = 1; q < BLOCK / 64; q++) idxMerge<IK, A>(bv, bi, ldsV[q], ldsI[q]);
   }
   if (live && t == 0) {
     if (a.splits == 1) {
@@ -734,6 +733,16 @@ static void indexTyped(hipStream_t st, const void* x, void* z, const ReducePlan&
   CoopArgs a = makeArgs(p, s, POST_ID);
   if (tryIndexRowsFast<IK, T, ZT>(st, x, z, p, s)) return;
   const int vec = s.vectorOk ? 1 : (s.peelOk ? 2 : 0);
+  // a few long rows (the logits of a decode step): one block of 1024 threads per row instead of segments plus a finishing
+  // launch -- at this size the second launch costs more than the narrower read (kernel time for bf16 [32, 50257]:
+  // 9.6 + 2.6 us in two launches, 9.0 us in one; [1, 50257] 6.6 + 2.7 against 8.0; rows of 200003 are faster cut up)
+  if (s.splits > 1 && vec && p.outerLen <= 64 && p.innerLen <= (1 << 16)) {
+    LaunchShape one = s;
+    one.splits = 1; one.segLen = p.innerLen; one.tpr = 1024;
+    CoopArgs a1 = makeArgs(p, one, POST_ID);
+    hipLaunchKernelGGL((index_coop<IK, T, 1024, ZT, 1024>), dim3((unsigned)p.outerLen), dim3(1024), 0, st, a1, (const T*)x, (ZT*)z, (IdxVal<A>*)scratch, vec);
+    return;
+  }
   if (s.flat) {
     hipLaunchKernelGGL((index_flat<IK, T, ZT>), dim3((unsigned)((p.outerLen + 255) / 256)), dim3(256), 0, st, a, (const T*)x, (ZT*)z);
     return;
