@@ -178,6 +178,9 @@ def main():
                     help="seconds of untimed launches of an op before its warmup steps (0 for counter-collection runs under rocprofv3)")
     ap.add_argument("--no-graphs", action="store_true",
                     help="time the decode op by op only (for runs under rocprofv3: its kernel tracing aborts the queue on graph replays)")
+    ap.add_argument("--decode-batches", default="1,32", help="batch sizes of the decode leg (comma-separated)")
+    ap.add_argument("--replay-kernels", action="store_true",
+                    help="decode: time only the replay that launches each recorded, merged step kernel by kernel (no graph launch: for a kernel trace of the merged step)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend is built and measured on one GPU; --gpus %d is not supported (no collectives are part of the op path)" % args.gpus)
@@ -449,12 +452,12 @@ def main():
         weights = init_weights(cfg, 5005)
         n_param_bytes = 2 * (cfg.n_layer * (cfg.d_model * 3 * cfg.d_model + cfg.d_model * cfg.d_model + 2 * cfg.d_model * cfg.d_ff) + cfg.vocab * cfg.d_model)
         prefill, n_new = 512, 128
-        for batch in (1, 32):
+        for batch in [int(b) for b in args.decode_batches.split(",") if b.strip()]:
             print("[bench] decode batch %d" % batch, file=sys.stderr, flush=True)
             ids = np.random.default_rng(5005).integers(0, cfg.vocab, (batch, prefill))
             dec = Decoder(cfg, weights, BFLOAT16, batch=batch, executioner=ex)
             dec.generate(ids[:, :prefill], 4)      # builds and warms the prefill program and the first decode programs
-            for _ in range(2):                     # second pass replays fully built programs
+            for _ in range(1 if args.replay_kernels else 2):   # second pass replays fully built programs
                 dec.reset()
                 L.streamSynchronize(None)
                 t0 = time.perf_counter()
@@ -469,22 +472,35 @@ def main():
             prefill_s = t1 - t0
             # the same steps replayed as captured HIP graphs (one per cache length): the first pass records them, the timed
             # passes replay; every kernel of the step still runs, only the per-op launch path on the host is gone
+            # Two ways to replay a recorded step (nd4jhipSetGraphReplayMode): the instantiated graph, and the merged sequence
+            # launched kernel by kernel from inside the library.  Both are timed, alternating; the line reports the faster.
             dec.use_graphs = not args.no_graphs
-            for _ in range(3 if dec.use_graphs else 0):
-                dec.reset()
-                dec.forward(ids)
-                L.streamSynchronize(None)
-                t1 = time.perf_counter()
-                for _ in range(n_new - 1):
-                    dec.forward(None)
-                L.streamSynchronize(None)
-                t2 = time.perf_counter()
-            step_ms = (t2 - t1) * 1e3 / (n_new - 1)   # the op-by-op figure when graphs are off
+            replay_ms = {}
+            for rep in range(3 if dec.use_graphs else 0):
+                for mode, name in ((0, "graph"), (1, "kernels")):
+                    if args.replay_kernels and mode == 0:
+                        continue
+                    L.nd4jhipSetGraphReplayMode(mode)
+                    dec.reset()
+                    dec.forward(ids)
+                    L.streamSynchronize(None)
+                    t1 = time.perf_counter()
+                    for _ in range(n_new - 1):
+                        dec.forward(None)
+                    L.streamSynchronize(None)
+                    t2 = time.perf_counter()
+                    if rep > 0 or args.replay_kernels:   # the first pass records
+                        replay_ms[name] = min(replay_ms.get(name, 1e9), (t2 - t1) * 1e3 / (n_new - 1))
+            L.nd4jhipSetGraphReplayMode(0)
+            best = min(replay_ms, key=replay_ms.get) if replay_ms else None
+            step_ms = replay_ms[best] if best else eager_ms   # the op-by-op figure when graphs are off
             dec.close()
             kv_bytes = cfg.n_layer * 2 * (prefill + n_new / 2) * cfg.d_model * 2 * batch
-            how = "steps replayed as HIP graphs" if dec.use_graphs else "op by op"
+            how = {"graph": "recorded steps replayed as HIP graphs", "kernels": "recorded, merged steps launched kernel by kernel by the library",
+                   None: "op by op"}[best]
             ops.append({"op": "gpt2-small decode bf16 batch %d (prefill %d, %d greedy steps, KV cache, %s)" % (batch, prefill, n_new, how),
                         "ms": round(step_ms, 4), "wall_ms": round(step_ms, 4), "tokens_per_s": round(batch * 1e3 / step_ms, 1),
+                        "replay_ms": {k: round(v, 4) for k, v in replay_ms.items()},
                         "op_by_op_ms": round(eager_ms, 4), "op_by_op_tokens_per_s": round(batch * 1e3 / eager_ms, 1),
                         "prefill_ms": round(prefill_s * 1e3, 3), "prefill_tokens_per_s": round(batch * prefill / prefill_s, 1),
                         "roofline": hbm_entry(n_param_bytes + kv_bytes, step_ms)})

@@ -1842,7 +1842,7 @@ static bool isRowLayerNorm(const RecordedOp& r) {
 
 static void runRecorded(RecordedOp* p) {
   if (p->kind == RecordedOp::CUSTOM) executeOp(*p->op, p->ctx);
-  else p->run();
+  else p->run(*p);
 }
 // z = x + y (pairwise Add, all of one float type), then ln = layer_norm(z): one kernel
 static bool tryAddLayerNorm(const RecordedOp& add, const RecordedOp& ln) {
@@ -1867,6 +1867,20 @@ static bool tryAddLayerNorm(const RecordedOp& add, const RecordedOp& ln) {
 }
 
 }  // namespace ops
+
+void RecordedOp::adopt() {
+  std::vector<std::pair<NDArray*, NDArray*>> seen;   // one copy per handle: an op called in place keeps input == output
+  auto own = [&](NDArray*& a) {
+    if (!a) return;
+    for (auto& s : seen) if (s.first == a) { a = s.second; return; }
+    owned.push_back(std::make_shared<NDArray>(*a));
+    seen.emplace_back(a, owned.back().get());
+    a = owned.back().get();
+  };
+  own(x); own(y); own(z);
+  for (NDArray*& a : ctx.inputs) own(a);
+  for (NDArray*& a : ctx.outputs) own(a);
+}
 
 std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& rec, int& nFused) {
   using namespace ops;

@@ -40,7 +40,12 @@ struct RecordedOp {
   Context ctx;                             // CUSTOM: copy of the caller's argument bag (arrays borrowed)
   int opNum = 0;                           // legacy loops
   NDArray *x = nullptr, *y = nullptr, *z = nullptr;
-  std::function<void()> run;               // executes the op exactly as the eager call does
+  std::function<void(const RecordedOp&)> run;   // legacy loops: executes the op on this record's arrays exactly as the eager call does
+  // The arrays above are the caller's while the capture is open.  adopt() replaces every one of them by a copy of the view
+  // held here (same buffer, offset, shape and strides; the buffer is shared), so that a plan built from the record does
+  // not depend on how long the caller keeps its array handles.
+  std::vector<std::shared_ptr<NDArray>> owned;
+  void adopt();
 };
 // The launch plan of the sequence; nFused counts the ops that were absorbed into a neighbour's kernel.
 std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& ops, int& nFused);

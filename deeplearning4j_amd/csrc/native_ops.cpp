@@ -546,7 +546,7 @@ void execTransformStrict(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa
   if (captureActive() && !(opNum == 2 || opNum == 3 || opNum == 19 || opNum == 25)) {
     RecordedOp r;
     r.kind = RecordedOp::TRANSFORM_STRICT; r.opNum = opNum; r.x = x; r.z = z;
-    r.run = [opNum, x, z] { transformStrictImpl(opNum, x, nullptr, z); };
+    r.run = [](const RecordedOp& o) { transformStrictImpl(o.opNum, o.x, nullptr, o.z); };
     recordOp(std::move(r));
   }
   GUARD_END_VOID
@@ -638,7 +638,7 @@ void execTransformAny(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, v
   if (captureActive()) {
     RecordedOp r;
     r.kind = RecordedOp::TRANSFORM_ANY; r.opNum = 0; r.x = x; r.z = z;
-    r.run = [x, z] { runUnary("execTransformAny", U_IDENTITY, x, z); };
+    r.run = [](const RecordedOp& o) { runUnary("execTransformAny", U_IDENTITY, o.x, o.z); };
     recordOp(std::move(r));
   }
   GUARD_END_VOID
@@ -692,7 +692,7 @@ void execPairwiseTransform(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray 
   if (captureActive()) {
     RecordedOp r;
     r.kind = RecordedOp::PAIRWISE; r.opNum = opNum; r.x = x; r.y = y; r.z = z;
-    r.run = [opNum, x, y, z] { pairwiseImpl(opNum, x, y, z); };
+    r.run = [](const RecordedOp& o) { pairwiseImpl(o.opNum, o.x, o.y, o.z); };
     recordOp(std::move(r));
   }
   GUARD_END_VOID
@@ -1302,7 +1302,10 @@ struct CapturedGraph {
   std::vector<RecordedOp> ops;    // the op calls the facade recognised, in call order
   int opCalls = 0;                // every op entry point called during the capture
   int fusedOps = 0;               // ops that ended up inside a neighbour's kernel
+  std::vector<std::function<void()>> plan;   // the merged sequence as ordinary launches (empty: a call went unrecorded)
 };
+// how nd4jhipGraphLaunch replays: 0 the instantiated HIP graph, 1 the merged sequence launched kernel by kernel
+int g_graphReplayMode = [] { const char* v = getenv("ND4JHIP_GRAPH_REPLAY"); return v != nullptr && std::string(v) == "kernels" ? 1 : 0; }();
 CapturedGraph* g_openCapture = nullptr;
 bool g_syncBeforeCapture = true;
 bool graphFusionEnabled() {
@@ -1348,9 +1351,13 @@ Nd4jPointer nd4jhipGraphEndCapture(void) {
   }
   // Every call of the capture was one the facade keeps a record of: run the sequence again through the merging pass and
   // keep that recording instead (nothing has executed so far -- a capture only notes launches)
+  bool keepPlan = false;
   if (graphFusionEnabled() && !cg->ops.empty() && (int)cg->ops.size() == cg->opCalls) {
     int nFused = 0;
+    for (RecordedOp& r : cg->ops) r.adopt();   // from here on the record holds its own views of the arrays
     auto plan = fuseRecordedOps(cg->ops, nFused);
+    cg->plan = plan;
+    keepPlan = true;
     if (nFused > 0) {
       g_captureOpCalls = nullptr;             // the replay re-enters nothing that counts
       hipGraph_t merged = nullptr;
@@ -1379,7 +1386,7 @@ Nd4jPointer nd4jhipGraphEndCapture(void) {
     }
   }
   closeCapture();
-  cg->ops.clear();
+  if (!keepPlan) cg->ops.clear();   // (the plan's steps point into the list)
   e = hipGraphInstantiate(&cg->exec, cg->graph, nullptr, nullptr, 0);
   if (e != hipSuccess) {
     (void)hipGraphDestroy(cg->graph);
@@ -1394,6 +1401,16 @@ int nd4jhipGraphLaunch(Nd4jPointer graph) {
   ND4J_REQUIRE(graph != nullptr, "nd4jhipGraphLaunch: graph is null");
   ND4J_REQUIRE(!captureActive(), "nd4jhipGraphLaunch: a capture is in progress");
   CapturedGraph* cg = static_cast<CapturedGraph*>(graph);
+  if (g_graphReplayMode == 1 && !cg->plan.empty()) {
+    // the merged sequence as ordinary launches: every step prepares and registers its own arrays, as the eager call does
+    for (auto& b : cg->record.reads) ND4J_REQUIRE(!b->closed, "nd4jhipGraphLaunch: a buffer the graph reads has been closed");
+    for (auto& b : cg->record.writes) ND4J_REQUIRE(!b->closed, "nd4jhipGraphLaunch: a buffer the graph writes has been closed");
+    const bool syncWas = Environment::get().syncAfterCustomOp;
+    Environment::get().syncAfterCustomOp = false;   // as during the capture: nothing waits inside a step
+    try { for (auto& step : cg->plan) step(); } catch (...) { Environment::get().syncAfterCustomOp = syncWas; throw; }
+    Environment::get().syncAfterCustomOp = syncWas;
+    return 0;
+  }
   // what prepareSpecialUse does per op, for the whole recorded sequence: an input (or a partly written output) whose
   // host copy is newer goes to the device first
   for (auto& b : cg->record.reads) {
@@ -1412,6 +1429,8 @@ int nd4jhipGraphLaunch(Nd4jPointer graph) {
   GUARD_END(1)
 }
 int nd4jhipGraphFusedOps(Nd4jPointer graph) { return graph ? static_cast<CapturedGraph*>(graph)->fusedOps : 0; }
+void nd4jhipSetGraphReplayMode(int mode) { g_graphReplayMode = mode == 1 ? 1 : 0; }
+int nd4jhipGetGraphReplayMode(void) { return g_graphReplayMode; }
 void nd4jhipGraphDestroy(Nd4jPointer graph) {
   if (!graph) return;
   CapturedGraph* cg = static_cast<CapturedGraph*>(graph);

@@ -116,6 +116,10 @@ class Decoder:
             "h": NDArray.empty((B, T, ff), dt), "g": NDArray.empty((B, T, ff), dt),
             "last": NDArray.empty((B, d), dt), "logits": NDArray.empty((B, c.vocab), dt), "next": NDArray.empty((B,), INT64),
         }
+        if T == 1:
+            # single-token steps: argmax writes the next ids where the following step's gather reads them (one array seen
+            # as [B] and as [B, 1]), so consecutive steps need no feedback copy
+            a["next"] = a["ids"].view((B,), (1,), 0)
         self._buffers[T] = a
         return a
 
@@ -181,7 +185,13 @@ class Decoder:
             # previous `next` [B] -> ids [B, 1]
             src = self._last_next
             if not hasattr(self, "_feed") or self._feed[0] is not src:
-                self._feed = (src, self._assign(src.view((self.B, 1), (1, 1)), a["ids"]))
+                # (every feedback copy ever built stays alive: a recorded step may hold its views)
+                if not hasattr(self, "_feeds"):
+                    self._feeds = {}
+                if id(src) not in self._feeds:
+                    copy = (lambda: None) if src is a["next"] else self._assign(src.view((self.B, 1), (1, 1)), a["ids"])
+                    self._feeds[id(src)] = (src, copy)
+                self._feed = self._feeds[id(src)]
             if self.use_graphs and self.dtype in (BFLOAT16, HALF):   # fp32 attention goes through temporaries and a wait: not capturable
                 self._graph_step(prog)
                 self.length += 1

@@ -172,6 +172,8 @@ _SIGS = {
     "nd4jhipGraphLaunch": (ctypes.c_int, [c_ptr]),
     "nd4jhipGraphDestroy": (None, [c_ptr]),
     "nd4jhipGraphFusedOps": (ctypes.c_int, [c_ptr]),
+    "nd4jhipSetGraphReplayMode": (None, [ctypes.c_int]),
+    "nd4jhipGetGraphReplayMode": (ctypes.c_int, []),
     "nd4jhipBuildInfo": (ctypes.c_char_p, []),
     "nd4jhipLastGemmKernel": (ctypes.c_char_p, []),
     "nd4jhipReduceSameScalarNoAlloc": (ctypes.c_int, [c_ptr, ctypes.c_int, ctypes.c_int, c_ptr, c_long, c_ptr]),

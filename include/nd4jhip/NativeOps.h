@@ -253,6 +253,16 @@ ND4JHIP_EXPORT void nd4jhipGraphDestroy(Nd4jPointer graph);
  * bit, into the same arrays.  This returns how many op calls were absorbed that way (0: the graph holds the calls as
  * made).  ND4JHIP_GRAPH_FUSION=0 in the environment switches the pass off. */
 ND4JHIP_EXPORT int nd4jhipGraphFusedOps(Nd4jPointer graph);
+/* How nd4jhipGraphLaunch replays a recording (no counterpart in the reference, like the capture calls themselves).
+ * 0: the instantiated HIP graph, one launch.  1: the recorded, merged sequence launched kernel by kernel on the execution
+ * stream by the library itself -- the same kernels with the same arguments, without the caller's per-op calls; a kernel
+ * tracer then sees the merged step as ordinary dispatches, and on hosts where a graph launch costs more per node than a
+ * plain launch it is also the faster of the two.  A recording made while some call went unrecorded has no such sequence
+ * and is always launched as a graph.  The recording keeps its own views of the arrays (the buffers are shared), so the
+ * caller's array handles may go away in either mode; the buffers may not.  The setting is process-wide and read at
+ * every launch; it starts as 0, or 1 when ND4JHIP_GRAPH_REPLAY=kernels is in the environment. */
+ND4JHIP_EXPORT void nd4jhipSetGraphReplayMode(int mode);
+ND4JHIP_EXPORT int nd4jhipGetGraphReplayMode(void);
 ND4JHIP_EXPORT const char* nd4jhipBuildInfo(void);
 /* Name ("family<type,tile,flags>") of the kernel the calling thread's most recent matmul / xw_plus_b launched; lets a
  * test assert that its shape reached the instantiation it means to check. */

@@ -86,10 +86,19 @@ def test_gpt2_small_bf16_teacher_forced_logits(ex, oracle, gpt2, batch, prompt, 
         got = dec.forward(feed)
 
 
-@pytest.mark.parametrize("batch", [1, 8, 32])
-def test_gpt2_small_graph_replay_matches_eager(ex, gpt2, batch):
+@pytest.mark.parametrize("batch,replay_mode", [(1, 0), (8, 0), (32, 0), (1, 1), (32, 1)])
+def test_gpt2_small_graph_replay_matches_eager(ex, gpt2, batch, replay_mode):
     """Recorded steps against eager steps at the real shape: ids and the logits read back after a replay (the replay must
-    stamp the buffers it writes, or the host would keep serving the previous copy)."""
+    stamp the buffers it writes, or the host would keep serving the previous copy); replayed as graphs (0) and as the
+    merged sequence launched kernel by kernel (1)."""
+    ex.L.nd4jhipSetGraphReplayMode(replay_mode)
+    try:
+        _gpt2_small_graph_replay_matches_eager(ex, gpt2, batch)
+    finally:
+        ex.L.nd4jhipSetGraphReplayMode(0)
+
+
+def _gpt2_small_graph_replay_matches_eager(ex, gpt2, batch):
     cfg, w = gpt2
     rng = np.random.default_rng(batch)
     prompt = rng.integers(0, cfg.vocab, (batch, 24))

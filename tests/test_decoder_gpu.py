@@ -62,12 +62,23 @@ def test_decode_head_dim_64_uses_fused_attention(ex):
     assert (a == b).all()
 
 
-def test_graph_replay_matches_eager_steps(ex):
+@pytest.mark.parametrize("replay_mode", [0, 1])
+def test_graph_replay_matches_eager_steps(ex, replay_mode):
     """Decode steps recorded as HIP graphs: the first generation records one graph per cache length, the second replays
     them; eager op-by-op work and synchronisations sit between the replays, and every generation must reproduce the
-    eager ids bit for bit (a replayed kernel runs with exactly the recorded arguments)."""
+    eager ids bit for bit (a replayed kernel runs with exactly the recorded arguments).  Both ways of replaying: the
+    instantiated graph (0) and the merged sequence launched kernel by kernel by the library (1)."""
     from deeplearning4j_amd.decoder import Decoder, DecoderConfig, init_weights
     from deeplearning4j_amd.ndarray import BFLOAT16, HALF
+    ex.L.nd4jhipSetGraphReplayMode(replay_mode)
+    assert ex.L.nd4jhipGetGraphReplayMode() == replay_mode
+    try:
+        _graph_replay_matches_eager_steps(ex, Decoder, DecoderConfig, init_weights, BFLOAT16, HALF)
+    finally:
+        ex.L.nd4jhipSetGraphReplayMode(0)
+
+
+def _graph_replay_matches_eager_steps(ex, Decoder, DecoderConfig, init_weights, BFLOAT16, HALF):
     cfg = DecoderConfig(vocab=512, d_model=128, n_head=2, n_layer=2, max_len=96)
     w = init_weights(cfg, seed=5)
     rng = np.random.default_rng(6)

@@ -98,9 +98,52 @@ def test_caller_stream_is_ordered_before_the_op(ex):
     L.freeHost(host)
 
 
-def test_graph_replay_keeps_buffer_stamps(ex):
+@pytest.mark.parametrize("replay_mode", [0, 1])
+def test_graph_replay_keeps_buffer_stamps(ex, replay_mode):
     """A replayed graph must upload an input the host rewrote after the capture and must mark what it writes, so that a
-    host read after each replay returns that replay's values (not the copy fetched after the previous one)."""
+    host read after each replay returns that replay's values (not the copy fetched after the previous one).  Both ways
+    of replaying (the graph; the recorded sequence launched kernel by kernel)."""
+    ex.L.nd4jhipSetGraphReplayMode(replay_mode)
+    try:
+        _graph_replay_keeps_buffer_stamps(ex)
+    finally:
+        ex.L.nd4jhipSetGraphReplayMode(0)
+
+
+def test_recording_outlives_the_callers_array_handles(ex):
+    """A recording holds its own views of the arrays it was made on: the caller may drop its view handles (the buffers
+    stay), and both ways of replaying still write the right columns."""
+    import gc
+    L = ex.L
+    rng = np.random.default_rng(77)
+    a, b = rng.normal(0, 1, (64, 96)).astype(np.float32), rng.normal(0, 1, (64, 96)).astype(np.float32)
+    A, B, Z = NDArray.from_numpy(a), NDArray.from_numpy(b), NDArray.from_numpy(np.zeros((64, 96), np.float32))
+    for arr in (A, B, Z):
+        arr.sync_to_device()
+    va, vb, vz = A.slice(1, 8, 72), B.slice(1, 16, 80), Z.slice(1, 32, 96)
+    assert L.nd4jhipGraphBeginCapture() == 0, L.lastErrorMessage()
+    L.execPairwiseTransform(None, Pairwise.Add, va.handle, vb.handle, vz.handle, None)
+    g = L.nd4jhipGraphEndCapture()
+    N.check("nd4jhipGraphEndCapture")
+    assert g
+    del va, vb, vz
+    gc.collect()
+    junk = [NDArray.from_numpy(np.full((64, 96), 7.0, np.float32)).slice(1, 1, 5) for _ in range(32)]   # recycles freed handles
+    want = np.zeros((64, 96), np.float32)
+    want[:, 32:] = a[:, 8:72] + b[:, 16:80]
+    try:
+        for mode in (1, 0, 1):
+            L.nd4jhipSetGraphReplayMode(mode)
+            Z.assign_numpy(np.zeros((64, 96), np.float32))
+            assert L.nd4jhipGraphLaunch(g) == 0, L.lastErrorMessage()
+            assert np.array_equal(Z.to_numpy(), want), mode
+    finally:
+        L.nd4jhipSetGraphReplayMode(0)
+        L.nd4jhipGraphDestroy(g)
+    assert len(junk) == 32
+
+
+def _graph_replay_keeps_buffer_stamps(ex):
     L = ex.L
     x = np.arange(4096, dtype=np.float32)
     X, Y, Z = NDArray.from_numpy(x), NDArray.from_numpy(np.ones(4096, np.float32)), NDArray.empty((4096,), FLOAT32)
