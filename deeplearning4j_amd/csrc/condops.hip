@@ -9,6 +9,9 @@
 //   BinaryRelativeError (Pairwise 25, :2218-2270)         z = re(x, y) > p0 ? 1 : 0,  re = |x - y| / (|x| + |y|), 0 for two zeros
 //   BinaryMinimumAbsoluteRelativeError (26, :2274-2340)   z = re(x, y) > p0 && !(|x - y| < p1) ? 1 : 0
 //   FirstIndex / LastIndex (IndexReduce 4 / 5, :2061-2150) first / last position with cond(x), -1 when none
+// and the members of the bool tables (pairwise / scalar / broadcast, BOOL result) that are more than a comparison:
+//   Epsilon (3, :1755-1790)                               |x - y| <= p0 when parameters are given, else <= 1e-5 (as the type holds it)
+//   And / Or / Xor (7 / 8 / 9, :1051-1063, :1896-1925)    on "differs from p0" when parameters are given, else on "is not zero"
 // The sixteen modes: 0 |v - c| <= eps, 1 |v - c| > eps, 2 <, 3 >, 4 <=, 5 >=, 6 |v| < c, 7 |v| > c, 8 isinf, 9 isnan, 10 ==, 11 !=,
 // 12 |v| >= c, 13 |v| <= c, 14 finite, 15 inf or nan.  Comparisons run in the array's own type: the difference of mode 0 / 1
 // is rounded through a 16-bit storage type as the reference's half / bfloat16 operators round it.
@@ -69,8 +72,18 @@ __global__ __launch_bounds__(256) void cond_ew(int kind, CondParams c, DevShape 
       case C_REPLACE: r = cond_holds(c, a) ? b : a; break;
       case C_AXPY: r = c.xdt == DOUBLE ? fma(c.compare, a, b) : (double)fmaf((float)c.compare, (float)a, (float)b); break;   // alpha x + y
       case C_BIN_REL_ERR: r = rel_err_in_type(a, b, c.xdt) > c.compare ? 1.0 : 0.0; break;
-      default:                                                  // C_BIN_MIN_ABS_REL_ERR: relative AND absolute threshold exceeded
+      case C_BIN_MIN_ABS_REL_ERR:                               // relative AND absolute threshold exceeded
         r = rel_err_in_type(a, b, c.xdt) > c.compare ? (fabs(sub_in_type(a, b, c.xdt)) < c.set ? 0.0 : 1.0) : 0.0;
+        break;
+      case C_BOOL_EPSILON: {                                    // |a - b| <= params[0] if given, else <= 1e-5 -- both held in the array's type
+        const double ad = fabs(sub_in_type(a, b, c.xdt));
+        r = ((c.mode && ad <= c.compare) || ad <= c.eps) ? 1.0 : 0.0;
+        break;
+      }
+      case C_BOOL_AND: r = (c.mode ? (a != c.compare && b != c.compare) : (a != 0.0 && b != 0.0)) ? 1.0 : 0.0; break;
+      case C_BOOL_OR: r = (c.mode ? (a != c.compare || b != c.compare) : (a != 0.0 || b != 0.0)) ? 1.0 : 0.0; break;
+      default:                                                  // C_BOOL_XOR
+        r = (c.mode ? ((a == c.compare) != (b == c.compare)) : ((a != 0.0) != (b != 0.0))) ? 1.0 : 0.0;
         break;
     }
     store_any(z, zdt, walk<LongType>(sz, i), r);

@@ -86,7 +86,12 @@ void launchIntElementwise(hipStream_t s, int k, bool binary, DataType xdt, DataT
                           void* z, const EwPlan& p, LongType scalar, bool hasScalar);
 
 // Ops that test a "match condition" read from the extra parameters (condops.hip)
-enum CondKind : int { C_MATCH_BOOL, C_SET_TRANSFORM, C_SET, C_REPLACE, C_AXPY, C_BIN_REL_ERR, C_BIN_MIN_ABS_REL_ERR };
+enum CondKind : int {
+  C_MATCH_BOOL, C_SET_TRANSFORM, C_SET, C_REPLACE, C_AXPY, C_BIN_REL_ERR, C_BIN_MIN_ABS_REL_ERR,
+  // the members of the bool tables that are not plain comparisons (ops.h:1051-1063, 1755-1790, 1896-1925): compare holds the
+  // one extra parameter, mode whether the caller passed any
+  C_BOOL_EPSILON, C_BOOL_AND, C_BOOL_OR, C_BOOL_XOR
+};
 enum CondReduceKind : int { CR_COUNT, CR_FIRST, CR_LAST };
 struct CondParams {
   int mode = 0;

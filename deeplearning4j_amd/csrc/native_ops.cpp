@@ -748,21 +748,7 @@ static double hostScalar(NDArray* s) {
     default: ND4J_THROW("scalar operand has an unsupported data type");
   }
 }
-void execScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueNDArray za, OpaqueNDArray sa, void* extraParams) {
-  OP_BEGIN(callerStream(extraPointers))
-  NDArray* x = arr(xa, "execScalar", "x"); NDArray* z = arr(za, "execScalar", "z"); NDArray* s = arr(sa, "execScalar", "scalar");
-  ND4J_REQUIRE(x->dataType() == z->dataType() && (isFloatType(x->dataType()) || isIntLike(x->dataType())), "execScalar: nd4j-hip requires X and Z of one type");
-  if (opNum == 33) {   // CompareAndSet with the scalar as second operand: z = cond(scalar) ? scalar : x (ops.h:719-840)
-    ND4J_REQUIRE(isFloatType(x->dataType()) || x->dataType() == INT32, "execScalar: CompareAndSet takes float or INT32 arrays here");
-    if (z->isEmpty()) return;
-    const CondParams c = condParams("execScalar", extraParams, z->dataType(), true);
-    const double sc = hostScalar(s);
-    EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo()});
-    prepareSpecialUse({z}, {x});
-    launchCondElementwise(execStream(), C_SET, c, x->dataType(), z->dataType(), x->specialBuffer(), nullptr, z->specialBuffer(), p, sc, true);
-    registerSpecialUse({z}, {x});
-    return;
-  }
+static PairwiseKind scalarKind(const char* fn, int opNum) {
   PairwiseKind k;
   switch (opNum) {  // loops/legacy_ops.h:78-86
     case 0: k = P_ADD; break; case 1: k = P_SUB; break; case 2: k = P_MUL; break; case 3: k = P_DIV; break;
@@ -778,8 +764,26 @@ void execScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueN
     case 42: k = P_LSTM_CLIP; break; case 43: k = P_TRUNCATE_MOD; break; case 45: k = P_REVERSE_POW; break;
     case 46: k = P_DIVIDE_NO_NAN; break; case 49: k = P_RELU_D; break;
     case 32: k = P_POW_DERIV; break; case 47: k = P_IGAMMA; break; case 48: k = P_IGAMMAC; break;   // 33 CompareAndSet is served above
-    default: ND4J_THROW("execScalar: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
+    default: ND4J_THROW(std::string(fn) + ": opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
+  return k;
+}
+void execScalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueNDArray za, OpaqueNDArray sa, void* extraParams) {
+  OP_BEGIN(callerStream(extraPointers))
+  NDArray* x = arr(xa, "execScalar", "x"); NDArray* z = arr(za, "execScalar", "z"); NDArray* s = arr(sa, "execScalar", "scalar");
+  ND4J_REQUIRE(x->dataType() == z->dataType() && (isFloatType(x->dataType()) || isIntLike(x->dataType())), "execScalar: nd4j-hip requires X and Z of one type");
+  if (opNum == 33) {   // CompareAndSet with the scalar as second operand: z = cond(scalar) ? scalar : x (ops.h:719-840)
+    ND4J_REQUIRE(isFloatType(x->dataType()) || x->dataType() == INT32, "execScalar: CompareAndSet takes float or INT32 arrays here");
+    if (z->isEmpty()) return;
+    const CondParams c = condParams("execScalar", extraParams, z->dataType(), true);
+    const double sc = hostScalar(s);
+    EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo()});
+    prepareSpecialUse({z}, {x});
+    launchCondElementwise(execStream(), C_SET, c, x->dataType(), z->dataType(), x->specialBuffer(), nullptr, z->specialBuffer(), p, sc, true);
+    registerSpecialUse({z}, {x});
+    return;
+  }
+  const PairwiseKind k = scalarKind("execScalar", opNum);
   if (z->isEmpty()) return;
   EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo()});
   ND4J_REQUIRE(p.sameShape, "execScalar: x and z must share a shape");
@@ -813,6 +817,46 @@ static std::vector<LongType> hostDims(NDArray* dimension, int rank, const char* 
   return normalizeDims(rank, raw.data(), (LongType)raw.size(), fn);
 }
 
+// y seen with x's shape: its non-unit dims line up with `dims` of x, its stride is 0 along every other dim
+static std::vector<LongType> broadcastOperandShape(const char* fn, NDArray* x, NDArray* y, const std::vector<LongType>& dims) {
+  // squeeze y's unit dims, then its remaining dims must match x along `dims`
+  std::vector<LongType> yshape, ystride;
+  for (int d = 0; d < y->rankOf(); d++) if (y->sizeAt(d) != 1) { yshape.push_back(y->sizeAt(d)); ystride.push_back(y->strideAt(d)); }
+  std::vector<LongType> bstride(x->rankOf(), 0);
+  size_t q = 0;
+  for (auto d : dims) {
+    if (x->sizeAt((int)d) == 1) continue;
+    ND4J_REQUIRE(q < yshape.size() && yshape[q] == x->sizeAt((int)d), std::string(fn) + ": y's shape does not match x along the broadcast dimensions");
+    bstride[d] = ystride[q++];
+  }
+  ND4J_REQUIRE(q == yshape.size(), std::string(fn) + ": y has more non-unit dims than broadcast dimensions");
+  std::vector<LongType> xshape(x->rankOf());
+  for (int d = 0; d < x->rankOf(); d++) xshape[d] = x->sizeAt(d);
+  return makeShapeInfo(y->dataType(), 'c', xshape, bstride.data());
+}
+// one scalar per sub-array of x along `dims` (loops/cpu/scalar.hpp:37-80): the scalars, numbered in c order over x's other
+// dims, seen with x's shape -- stride 0 along `dims`
+static std::vector<LongType> scalarsPerTadShape(const char* fn, NDArray* x, NDArray* scalars, const std::vector<LongType>& dims) {
+  const int rank = x->rankOf();
+  std::vector<bool> inTad(rank, false);
+  for (auto d : dims) inTad[d] = true;
+  LongType tads = 1;
+  for (int d = 0; d < rank; d++) if (!inTad[d]) tads *= x->sizeAt(d);
+  ND4J_REQUIRE(scalars->lengthOf() == tads, std::string(fn) + ": " + std::to_string(scalars->lengthOf()) + " scalars for " + std::to_string(tads) + " sub-arrays");
+  LongType step = 1;   // element stride of the scalars seen as a vector
+  for (int d = 0; d < scalars->rankOf(); d++) if (scalars->sizeAt(d) != 1) {
+    ND4J_REQUIRE(scalars->lengthOf() == scalars->sizeAt(d), std::string(fn) + ": the scalars must form a vector");
+    step = scalars->strideAt(d);
+  }
+  std::vector<LongType> xshape(rank), st(rank, 0);
+  LongType run = step;
+  for (int d = rank - 1; d >= 0; d--) {
+    xshape[d] = x->sizeAt(d);
+    if (!inTad[d]) { st[d] = run; run *= x->sizeAt(d); }
+  }
+  return makeShapeInfo(scalars->dataType(), 'c', xshape, st.data());
+}
+
 // y is a smaller array whose dims line up with `dimension` of x (loops/cpu/broadcasting.hpp); realised as a
 // pairwise walk in which y's stride is 0 along every other dim
 void execBroadcast(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueNDArray ya, OpaqueNDArray za, void*, OpaqueNDArray da) {
@@ -834,25 +878,111 @@ void execBroadcast(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, Opaq
     default: ND4J_THROW("execBroadcast: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
   if (z->isEmpty()) return;
-  auto dims = hostDims(dim, x->rankOf(), "execBroadcast");
-  // squeeze y's unit dims, then its remaining dims must match x along `dims`
-  std::vector<LongType> yshape, ystride;
-  for (int d = 0; d < y->rankOf(); d++) if (y->sizeAt(d) != 1) { yshape.push_back(y->sizeAt(d)); ystride.push_back(y->strideAt(d)); }
-  std::vector<LongType> bstride(x->rankOf(), 0);
-  size_t q = 0;
-  for (auto d : dims) {
-    if (x->sizeAt((int)d) == 1) continue;
-    ND4J_REQUIRE(q < yshape.size() && yshape[q] == x->sizeAt((int)d), "execBroadcast: y's shape does not match x along the broadcast dimensions");
-    bstride[d] = ystride[q++];
-  }
-  ND4J_REQUIRE(q == yshape.size(), "execBroadcast: y has more non-unit dims than broadcast dimensions");
-  std::vector<LongType> xshape(x->rankOf());
-  for (int d = 0; d < x->rankOf(); d++) xshape[d] = x->sizeAt(d);
-  auto ysi = makeShapeInfo(y->dataType(), 'c', xshape, bstride.data());
+  auto ysi = broadcastOperandShape("execBroadcast", x, y, hostDims(dim, x->rankOf(), "execBroadcast"));
   EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo(), ysi.data()});
   prepareSpecialUse({z}, {x, y});
   launchPairwise(execStream(), k, x->dataType(), y->dataType(), z->dataType(), x->specialBuffer(), y->specialBuffer(), z->specialBuffer(), p);
   registerSpecialUse({z}, {x, y});
+  GUARD_END_VOID
+}
+
+// ---- the bool tables: z = op(x, y) with x and y of one type and a BOOL result (loops/legacy_ops.h:30-32, 74-76, 117-119;
+// loops/cpu/pairwise_bool.cpp:60-145, scalar_bool.cpp:60-140, broadcasting_bool.hpp:60-330 -- every loop calls the functor's
+// three-argument form, op(x, y, extraParams)).  `ysi` describes y with x's shape (its own, or strides of 0 where it repeats).
+static void boolTableImpl(const char* fn, int opNum, NDArray* x, NDArray* y, const LongType* ysi, void* extraParams, NDArray* z) {
+  ND4J_REQUIRE(z->dataType() == BOOL, std::string(fn) + ": Z must be a BOOL array, got " + dtypeName(z->dataType()));
+  ND4J_REQUIRE(x->dataType() == y->dataType(), std::string(fn) + ": X and Y must have one type, got " + dtypeName(x->dataType()) + ", " + dtypeName(y->dataType()));
+  const DataType dt = x->dataType();
+  ND4J_REQUIRE(isFloatType(dt) || dt == INT32 || dt == INT64 || dt == BOOL, std::string(fn) + ": " + dtypeName(dt) + " operands are not implemented in nd4j-hip");
+  if (z->isEmpty()) return;
+  EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo(), ysi});
+  PairwiseKind k = P_EQ;
+  CondKind ck = C_BOOL_AND;
+  bool comparison = true;
+  switch (opNum) {
+    case 0: k = P_EQ; break; case 1: k = P_GT; break; case 2: k = P_LT; break; case 4: k = P_GE; break; case 6: k = P_NE; break;
+    case 11: k = P_LE; break;
+    case 10: k = P_NE; break;   // Not: the three-argument form is x != y (ops.h:1927-1932)
+    case 3: ck = C_BOOL_EPSILON; comparison = false; break;
+    case 7: ck = C_BOOL_AND; comparison = false; break; case 8: ck = C_BOOL_OR; comparison = false; break; case 9: ck = C_BOOL_XOR; comparison = false; break;
+    default: ND4J_THROW(std::string(fn) + ": opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");   // 5 MatchCondition
+  }
+  if (comparison) {
+    prepareSpecialUse({z}, {x, y});
+    launchPairwise(execStream(), k, dt, dt, BOOL, x->specialBuffer(), y->specialBuffer(), z->specialBuffer(), p);
+    registerSpecialUse({z}, {x, y});
+    return;
+  }
+  ND4J_REQUIRE(ck != C_BOOL_EPSILON || dt != BOOL, std::string(fn) + ": Epsilon of BOOL arrays is not implemented in nd4j-hip");
+  CondParams c;
+  c.xdt = (int)dt;
+  c.mode = extraParams != nullptr ? 1 : 0;
+  if (extraParams) c.compare = fetchParams(fn, extraParams, dt, 1)[0];
+  // the default tolerance as the array's type holds it, static_cast<X>(1e-5): bfloat16 rounds it to 0x3728 and half to the
+  // subnormal 168 * 2^-24, which are the same number; the integer types hold 0
+  c.eps = dt == DOUBLE ? 1e-5 : dt == FLOAT32 ? (double)1e-5f : isFloatType(dt) ? 168.0 / 16777216.0 : 0.0;
+  prepareSpecialUse({z}, {x, y});
+  launchCondElementwise(execStream(), ck, c, dt, BOOL, x->specialBuffer(), y->specialBuffer(), z->specialBuffer(), p, 0.0, false);
+  registerSpecialUse({z}, {x, y});
+}
+// y with x's shape and stride 0 everywhere: the scalar operand
+static std::vector<LongType> repeatedScalarShape(NDArray* x, NDArray* s) {
+  std::vector<LongType> xshape(x->rankOf()), st(x->rankOf(), 0);
+  for (int d = 0; d < x->rankOf(); d++) xshape[d] = x->sizeAt(d);
+  return makeShapeInfo(s->dataType(), 'c', xshape, st.data());
+}
+void execPairwiseTransformBool(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueNDArray ya, void* extraParams, OpaqueNDArray za) {
+  OP_BEGIN(callerStream(extraPointers))
+  NDArray* x = arr(xa, "execPairwiseTransformBool", "x"); NDArray* y = arr(ya, "execPairwiseTransformBool", "y"); NDArray* z = arr(za, "execPairwiseTransformBool", "z");
+  // a one-element y stands for a scalar (pairwise_bool.cpp:66-86); otherwise the arrays are walked by linear index
+  if (y->lengthOf() == 1 && x->lengthOf() != 1) {
+    auto ysi = repeatedScalarShape(x, y);
+    boolTableImpl("execPairwiseTransformBool", opNum, x, y, ysi.data(), extraParams, z);
+  } else {
+    ND4J_REQUIRE(x->lengthOf() == y->lengthOf() && x->lengthOf() == z->lengthOf(), "execPairwiseTransformBool: x, y and z must have one length");
+    boolTableImpl("execPairwiseTransformBool", opNum, x, y, y->shapeInfo(), extraParams, z);
+  }
+  GUARD_END_VOID
+}
+void execScalarBool(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueNDArray za, OpaqueNDArray sa, void* extraParams) {
+  OP_BEGIN(callerStream(extraPointers))
+  NDArray* x = arr(xa, "execScalarBool", "x"); NDArray* z = arr(za, "execScalarBool", "z"); NDArray* s = arr(sa, "execScalarBool", "scalar");
+  ND4J_REQUIRE(s->lengthOf() >= 1 && s->buf, "execScalarBool: scalar operand is empty");
+  auto ysi = repeatedScalarShape(x, s);
+  boolTableImpl("execScalarBool", opNum, x, s, ysi.data(), extraParams, z);
+  GUARD_END_VOID
+}
+void execBroadcastBool(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueNDArray ya, OpaqueNDArray za, void* extraParams, OpaqueNDArray da) {
+  OP_BEGIN(callerStream(extraPointers))
+  NDArray* x = arr(xa, "execBroadcastBool", "x"); NDArray* y = arr(ya, "execBroadcastBool", "y"); NDArray* z = arr(za, "execBroadcastBool", "z");
+  NDArray* dim = arr(da, "execBroadcastBool", "dimension");
+  auto ysi = broadcastOperandShape("execBroadcastBool", x, y, hostDims(dim, x->rankOf(), "execBroadcastBool"));
+  boolTableImpl("execBroadcastBool", opNum, x, y, ysi.data(), extraParams, z);
+  GUARD_END_VOID
+}
+void execScalarBoolTad(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueNDArray za, OpaqueNDArray sa, void* extraParams, OpaqueNDArray da) {
+  OP_BEGIN(callerStream(extraPointers))
+  NDArray* x = arr(xa, "execScalarBoolTad", "x"); NDArray* z = arr(za, "execScalarBoolTad", "z"); NDArray* s = arr(sa, "execScalarBoolTad", "scalars");
+  NDArray* dim = arr(da, "execScalarBoolTad", "dimension");
+  auto ysi = scalarsPerTadShape("execScalarBoolTad", x, s, hostDims(dim, x->rankOf(), "execScalarBoolTad"));
+  boolTableImpl("execScalarBoolTad", opNum, x, s, ysi.data(), extraParams, z);
+  GUARD_END_VOID
+}
+// execScalar with one scalar per sub-array along `dimension` (legacy/NativeOps.h:205; loops/cpu/scalar.hpp:37-80)
+void execScalarTad(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueNDArray za, OpaqueNDArray sa, void*, OpaqueNDArray da) {
+  OP_BEGIN(callerStream(extraPointers))
+  NDArray* x = arr(xa, "execScalarTad", "x"); NDArray* z = arr(za, "execScalarTad", "z"); NDArray* s = arr(sa, "execScalarTad", "scalars");
+  NDArray* dim = arr(da, "execScalarTad", "dimension");
+  ND4J_REQUIRE(x->dataType() == z->dataType() && s->dataType() == z->dataType() && (isFloatType(x->dataType()) || isIntLike(x->dataType())),
+               "execScalarTad: nd4j-hip requires X, the scalars and Z of one type");
+  ND4J_REQUIRE(opNum != 33, "execScalarTad: CompareAndSet along a dimension is not implemented in nd4j-hip");
+  const PairwiseKind k = scalarKind("execScalarTad", opNum);
+  if (z->isEmpty()) return;
+  auto ysi = scalarsPerTadShape("execScalarTad", x, s, hostDims(dim, x->rankOf(), "execScalarTad"));
+  EwPlan p = buildEwPlan({z->shapeInfo(), x->shapeInfo(), ysi.data()});
+  prepareSpecialUse({z}, {x, s});
+  launchPairwise(execStream(), k, x->dataType(), s->dataType(), z->dataType(), x->specialBuffer(), s->specialBuffer(), z->specialBuffer(), p);
+  registerSpecialUse({z}, {x, s});
   GUARD_END_VOID
 }
 

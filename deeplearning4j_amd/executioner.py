@@ -84,6 +84,11 @@ class ReduceBool:
     Any, All, IsFinite, IsInfOrNan, IsNan, IsInf, IsPositive, IsNegative = 0, 1, 2, 3, 4, 5, 6, 7   # 2-7: true when any element is
 
 
+class BoolOp:
+    """The bool tables of the pairwise / scalar / broadcast families (loops/legacy_ops.h:30-32, 74-76, 117-119)."""
+    EqualTo, GreaterThan, LessThan, Epsilon, GreaterThanOrEqual, MatchCondition, NotEqualTo, And, Or, Xor, Not, LessThanOrEqual = range(12)
+
+
 class Scalar:
     Add, Subtract, Multiply, Divide, ReverseDivide, ReverseSubtract, MaxPairwise, ELU, ELUDerivative = 0, 1, 2, 3, 4, 5, 6, 7, 8
     MinPairwise, CopyPws, Mod, ReverseMod, Remainder, FMod, TruncateDiv, FloorDiv, FloorMod, SquaredSubtract = 13, 14, 15, 16, 17, 18, 19, 20, 21, 22
@@ -240,6 +245,47 @@ class Executioner:
         d = _dims_array(dims)
         self.L.execBroadcast(None, op_num, x.handle, y.handle, z.handle, None, d.handle)
         N.check("execBroadcast")
+        return z
+
+    # ---- the bool tables (loops/legacy_ops.h:30-32, 74-76, 117-119): operands of one type, BOOL result ----
+    def exec_pairwise_bool(self, op_num, x, y, z=None, extra_args=None):
+        z = z if z is not None else NDArray.empty(x.shape, BOOL)
+        holder, extra = self._extra_params(extra_args, x.dtype)
+        self.L.execPairwiseTransformBool(None, op_num, x.handle, y.handle, extra, z.handle)
+        N.check("execPairwiseTransformBool")
+        return z
+
+    def exec_scalar_bool(self, op_num, x, scalar, z=None, extra_args=None):
+        z = z if z is not None else NDArray.empty(x.shape, BOOL)
+        s = scalar if isinstance(scalar, NDArray) else NDArray.scalar(scalar, x.dtype)
+        holder, extra = self._extra_params(extra_args, x.dtype)
+        self.L.execScalarBool(None, op_num, x.handle, z.handle, s.handle, extra)
+        N.check("execScalarBool")
+        return z
+
+    def exec_broadcast_bool(self, op_num, x, y, dims, z=None, extra_args=None):
+        z = z if z is not None else NDArray.empty(x.shape, BOOL)
+        d = _dims_array(dims)
+        holder, extra = self._extra_params(extra_args, x.dtype)
+        self.L.execBroadcastBool(None, op_num, x.handle, y.handle, z.handle, extra, d.handle)
+        N.check("execBroadcastBool")
+        return z
+
+    def exec_scalar_bool_tad(self, op_num, x, scalars, dims, z=None, extra_args=None):
+        """One scalar per sub-array of x along `dims`."""
+        z = z if z is not None else NDArray.empty(x.shape, BOOL)
+        d = _dims_array(dims)
+        holder, extra = self._extra_params(extra_args, x.dtype)
+        self.L.execScalarBoolTad(None, op_num, x.handle, z.handle, scalars.handle, extra, d.handle)
+        N.check("execScalarBoolTad")
+        return z
+
+    def exec_scalar_tad(self, op_num, x, scalars, dims, z=None):
+        """execScalar with one scalar per sub-array of x along `dims`."""
+        z = z if z is not None else NDArray.empty(x.shape, x.dtype)
+        d = _dims_array(dims)
+        self.L.execScalarTad(None, op_num, x.handle, z.handle, scalars.handle, None, d.handle)
+        N.check("execScalarTad")
         return z
 
     def _reduce(self, scalar_fn, dim_fn, name, op_num, x, dims, keep_dims, z, zdtype, extra_args=None, extra_dtype=None):

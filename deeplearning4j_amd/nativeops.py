@@ -130,6 +130,11 @@ _SIGS = {
     "execReduceBool2": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
     "execScalar": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
     "execBroadcast": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "execPairwiseTransformBool": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "execBroadcastBool": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "execScalarBool": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "execScalarBoolTad": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "execScalarTad": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
     "getAllCustomOps": (ctypes.c_char_p, []),
     "createGraphContext": (c_ptr, [ctypes.c_int]),
     "deleteGraphContext": (None, [c_ptr]),

@@ -184,6 +184,15 @@ ND4JHIP_EXPORT void execReduceLong2(Nd4jPointer* extraPointers, int opNum, Opaqu
 ND4JHIP_EXPORT void execReduceBool(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z, OpaqueNDArray dimension);  /* ref :213 */
 ND4JHIP_EXPORT void execReduceBool2(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z, OpaqueNDArray dimension); /* ref :212 */
 ND4JHIP_EXPORT void execBroadcast(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, OpaqueNDArray y, OpaqueNDArray z, void* extraParams, OpaqueNDArray dimension); /* ref :206 */
+/* The bool tables (loops/legacy_ops.h:30-32, 74-76, 117-119): x and y (or the scalar) of one type, z BOOL.  EqualTo, GreaterThan,
+ * LessThan, Epsilon, GreaterThanOrEqual, NotEqualTo, And, Or, Xor, Not, LessThanOrEqual; 5 (MatchCondition) is refused.
+ * Epsilon / And / Or / Xor read one extra parameter when extraParams is not null (held in x's type, fetched with a blocking copy). */
+ND4JHIP_EXPORT void execPairwiseTransformBool(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, OpaqueNDArray y, void* extraParams, OpaqueNDArray z); /* ref :196 */
+ND4JHIP_EXPORT void execBroadcastBool(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, OpaqueNDArray y, OpaqueNDArray z, void* extraParams, OpaqueNDArray dimension); /* ref :200 */
+ND4JHIP_EXPORT void execScalarBool(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, OpaqueNDArray z, OpaqueNDArray scalar, void* extraParams); /* ref :201 */
+/* One scalar per sub-array of x along `dimension` (the scalars numbered in c order over x's other dims). */
+ND4JHIP_EXPORT void execScalarBoolTad(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, OpaqueNDArray z, OpaqueNDArray scalars, void* extraParams, OpaqueNDArray dimension); /* ref :203 */
+ND4JHIP_EXPORT void execScalarTad(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, OpaqueNDArray z, OpaqueNDArray scalars, void* extraParams, OpaqueNDArray dimension); /* ref :205 */
 
 /* ---- op context + declarable ops ---------------------------------------------------------------------------- */
 ND4JHIP_EXPORT const char* getAllCustomOps(void);                                      /* ref :76 */

@@ -624,3 +624,72 @@ def igamma(a, x, complement=False):
                 r = dt(aim * s)
         out[idx] = dt(1) - r if complement else r
     return out
+
+
+# ---- the bool tables: pairwise / scalar / broadcast ops with a BOOL result (numpy restatements) -------------------------------
+def bool_table(op, x, y, params=None, bf16=False):
+    """z = op(x, y, extraParams) for the members of BROADCAST_BOOL_OPS / SCALAR_BOOL_OPS / PAIRWISE_BOOL_OPS
+    (loops/legacy_ops.h:30-32, 74-76, 117-119); every loop of the three families calls the functor's three-argument form
+    (loops/cpu/pairwise_bool.cpp:73-143, scalar_bool.cpp:77-138, broadcasting_bool.hpp:91-325).  x and y are numpy arrays
+    of one dtype and one shape (see operand_along / scalars_along for the operand shapes of the other families); with
+    bf16=True they are float32 arrays holding bfloat16 values and differences are rounded to bfloat16.
+    0 EqualTo, 1 GreaterThan, 2 LessThan, 4 GreaterThanOrEqual, 6 NotEqualTo, 11 LessThanOrEqual: ops.h:181-186 (x OP y).
+    3 Epsilon (ops.h:1755-1790): |x - y| <= params[0] when parameters are given, else (also) |x - y| <= X(1e-5).
+    7 And / 8 Or / 9 Xor (ops.h:1051-1063, 1896-1925): with parameters on "differs from params[0]", without on bool(x), bool(y).
+    10 Not (ops.h:1927-1932): the three-argument form is x != y."""
+    x, y = np.asarray(x), np.asarray(y)
+    assert x.dtype == y.dtype and x.shape == y.shape
+    op = int(op)
+    with np.errstate(invalid="ignore", over="ignore"):
+        if op in (0, 1, 2, 4, 6, 10, 11):
+            return {0: x == y, 1: x > y, 2: x < y, 4: x >= y, 6: x != y, 10: x != y, 11: x <= y}[op]
+        if op == 3:
+            assert x.dtype != np.bool_
+            if bf16:
+                diff = bf16_to_f32(f32_to_bf16((x - y).astype(np.float32)))
+                tol = bf16_to_f32(f32_to_bf16(np.array([1e-5], np.float32)))[0]
+            else:
+                diff = (x - y).astype(x.dtype)
+                tol = np.array(1e-5).astype(x.dtype)          # static_cast<X>(1e-5): 0 for the integer types
+            ad = np.abs(diff)
+            hit = ad <= tol
+            if params is not None:
+                p0 = np.float32(params[0]) if bf16 else np.array(params[0]).astype(x.dtype)
+                hit = hit | (ad <= p0)
+            return hit
+        if params is not None:
+            c = np.float32(params[0]) if bf16 else np.array(params[0]).astype(x.dtype)
+            a, b = x != c, y != c
+            if op == 9:                                       # exactly one of the two equals the parameter
+                a, b = x == c, y == c
+                return a != b
+        else:
+            a, b = x != 0, y != 0                             # static_cast<bool>: NaN counts as true
+            if op == 9:
+                return a != b
+        return {7: a & b, 8: a | b}[op]
+
+
+def operand_along(y, x_shape, dims):
+    """The second operand of the broadcast loops seen with x's shape: y's non-unit dims line up with `dims` of x
+    (loops/cpu/broadcasting_bool.hpp:60-120: one sub-array of x along `dims` per pass, y walked alongside it)."""
+    y = np.asarray(y)
+    dims = sorted(d + len(x_shape) if d < 0 else d for d in dims)
+    yshape = [s for s in y.shape if s != 1]
+    full = [1] * len(x_shape)
+    it = iter(yshape)
+    for d in dims:
+        if x_shape[d] != 1:
+            full[d] = next(it)
+    return np.broadcast_to(y.reshape(full), x_shape)
+
+
+def scalars_along(s, x_shape, dims):
+    """One scalar per sub-array of x along `dims`, the sub-arrays numbered in c order over x's other dims
+    (loops/cpu/scalar.hpp:37-80, scalar_bool.cpp:37-80), seen with x's shape."""
+    s = np.asarray(s).reshape(-1)
+    dims = sorted(d + len(x_shape) if d < 0 else d for d in dims)
+    other = [d for d in range(len(x_shape)) if d not in dims]
+    full = [x_shape[d] if d in other else 1 for d in range(len(x_shape))]
+    assert s.size == int(np.prod([x_shape[d] for d in other])) if other else s.size == 1
+    return np.broadcast_to(s.reshape(full), x_shape)
