@@ -1216,6 +1216,51 @@ void execReduce3Tad(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, voi
   runReduce3("execReduce3Tad", opNum, x, arr(ya, "execReduce3Tad", "y"), arr(za, "execReduce3Tad", "z"), hostDims(da, x->rankOf(), "execReduce3Tad"), extraParams);
   GUARD_END_VOID
 }
+// every sub-array of x along `dimension` against every sub-array of y along it: z[i][j] = f(x tad i, y tad j), the
+// sub-arrays numbered in c order over the other dims (loops/cpu/reduce3.hpp execAll).  Realised as execReduce3Tad on two
+// views of rank |x's other dims| + |y's other dims| + |dimension|, x repeated (stride 0) along y's dims and y along x's.
+void execReduce3All(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, OpaqueNDArray ya, OpaqueNDArray za, OpaqueNDArray da, void* extraParams) {
+  OP_BEGIN(callerStream(extraPointers))
+  const char* fn = "execReduce3All";
+  NDArray* x = arr(xa, fn, "x"); NDArray* y = arr(ya, fn, "y"); NDArray* z = arr(za, fn, "z");
+  ND4J_REQUIRE(x->rankOf() == y->rankOf(), std::string(fn) + ": x and y must have one rank");
+  ND4J_REQUIRE(!x->isEmpty() && !y->isEmpty(), std::string(fn) + ": reductions of empty arrays are not implemented in nd4j-hip");
+  const int rank = x->rankOf();
+  auto dims = hostDims(da, rank, fn);
+  ND4J_REQUIRE(!dims.empty(), std::string(fn) + ": the dimensions of the sub-arrays are required");
+  std::vector<bool> inTad(rank, false);
+  for (auto d : dims) { inTad[d] = true; ND4J_REQUIRE(x->sizeAt((int)d) == y->sizeAt((int)d), std::string(fn) + ": the sub-arrays of x and y must have one shape"); }
+  std::vector<LongType> shape, xs, ys, zs;
+  LongType nx = 1, ny = 1;
+  for (int d = 0; d < rank; d++) if (!inTad[d]) { nx *= x->sizeAt(d); ny *= y->sizeAt(d); }
+  ND4J_REQUIRE(z->lengthOf() == nx * ny, std::string(fn) + ": z must hold " + std::to_string(nx) + " x " + std::to_string(ny) + " results");
+  if (z->isEmpty()) return;
+  // z as [nx, ny]: its own two dims when it has that shape, else a dense c-order array
+  LongType zRow = ny, zCol = 1;
+  if (z->rankOf() == 2 && z->sizeAt(0) == nx && z->sizeAt(1) == ny) { zRow = z->strideAt(0); zCol = z->strideAt(1); }
+  else {
+    bool dense = true;
+    LongType expect = 1;
+    for (int d = z->rankOf() - 1; d >= 0; d--) { if (z->sizeAt(d) != 1 && z->strideAt(d) != expect) dense = false; expect *= z->sizeAt(d); }
+    ND4J_REQUIRE(dense, std::string(fn) + ": z must have shape [sub-arrays of x, sub-arrays of y] or be dense in c order");
+  }
+  LongType run = zRow * nx;
+  for (int d = 0; d < rank; d++) if (!inTad[d]) { run /= x->sizeAt(d); shape.push_back(x->sizeAt(d)); xs.push_back(x->strideAt(d)); ys.push_back(0); zs.push_back(run); }
+  run = zCol * ny;
+  for (int d = 0; d < rank; d++) if (!inTad[d]) { run /= y->sizeAt(d); shape.push_back(y->sizeAt(d)); xs.push_back(0); ys.push_back(y->strideAt(d)); zs.push_back(run); }
+  std::vector<LongType> tadAxes;
+  const size_t outRank = shape.size();
+  std::vector<LongType> zshape(shape.begin(), shape.end());
+  for (auto d : dims) { tadAxes.push_back((LongType)shape.size()); shape.push_back(x->sizeAt((int)d)); xs.push_back(x->strideAt((int)d)); ys.push_back(y->strideAt((int)d)); }
+  ND4J_REQUIRE((int)shape.size() <= MAX_RANK, std::string(fn) + ": too many dims");
+  NDArray xv = *x, yv = *y, zv = *z;
+  xv.si = makeShapeInfo(x->dataType(), 'c', shape, xs.data());
+  yv.si = makeShapeInfo(y->dataType(), 'c', shape, ys.data());
+  if (outRank == 0) { zshape = {1}; zs = {1}; }
+  zv.si = makeShapeInfo(z->dataType(), 'c', zshape, zs.data());
+  runReduce3(fn, opNum, &xv, &yv, &zv, tadAxes, extraParams);
+  GUARD_END_VOID
+}
 void execTransformBool(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, void* extraParams, OpaqueNDArray za) {
   OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execTransformBool", "x"); NDArray* z = arr(za, "execTransformBool", "z");

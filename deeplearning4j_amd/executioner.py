@@ -340,6 +340,18 @@ class Executioner:
         N.check("execReduce3")
         return z
 
+    def exec_reduce3_all(self, op_num, x, y, dims, z=None, extra_args=None):
+        """Every sub-array of x along `dims` against every sub-array of y along them: z [sub-arrays of x, sub-arrays of y]."""
+        if z is None:
+            nd = [d + len(x.shape) if d < 0 else d for d in dims]
+            nx = int(np.prod([s for i, s in enumerate(x.shape) if i not in nd]))
+            ny = int(np.prod([s for i, s in enumerate(y.shape) if i not in nd]))
+            z = NDArray.empty((nx, ny), x.dtype)
+        holder, extra = self._extra_params(extra_args, z.dtype)
+        self.L.execReduce3All(None, op_num, x.handle, y.handle, z.handle, _dims_array(dims).handle, extra)
+        N.check("execReduce3All")
+        return z
+
     def _reduce_dims_only(self, fn, name, op_num, x, dims, keep_dims, z, zdtype, extra_args=None):
         if z is None:
             z = NDArray.empty(_reduced_shape(x.shape, dims, keep_dims), zdtype)

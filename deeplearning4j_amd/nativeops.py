@@ -124,6 +124,7 @@ _SIGS = {
     "execReduce3": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
     "execReduce3Scalar": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
     "execReduce3Tad": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "execReduce3All": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
     "execReduceLong": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
     "execReduceLong2": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
     "execReduceBool": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),

@@ -179,6 +179,8 @@ ND4JHIP_EXPORT void execSummaryStatsTad(Nd4jPointer* extraPointers, int opNum, O
 ND4JHIP_EXPORT void execReduce3(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray y, OpaqueNDArray z);        /* ref :326 */
 ND4JHIP_EXPORT void execReduce3Scalar(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray y, OpaqueNDArray z);  /* ref :327 */
 ND4JHIP_EXPORT void execReduce3Tad(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray y, OpaqueNDArray z, OpaqueNDArray dimension); /* ref :328 */
+/* every sub-array of x along `dimension` against every sub-array of y along it: z[i][j], shape [sub-arrays of x, sub-arrays of y] */
+ND4JHIP_EXPORT void execReduce3All(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, OpaqueNDArray y, OpaqueNDArray z, OpaqueNDArray dimension, void* extraParams); /* ref :208 */
 ND4JHIP_EXPORT void execReduceLong(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z, OpaqueNDArray dimension);  /* ref :211 */
 ND4JHIP_EXPORT void execReduceLong2(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z, OpaqueNDArray dimension); /* ref :349-351 */
 ND4JHIP_EXPORT void execReduceBool(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray x, void* extraParams, OpaqueNDArray z, OpaqueNDArray dimension);  /* ref :213 */

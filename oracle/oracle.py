@@ -693,3 +693,19 @@ def scalars_along(s, x_shape, dims):
     full = [x_shape[d] if d in other else 1 for d in range(len(x_shape))]
     assert s.size == int(np.prod([x_shape[d] for d in other])) if other else s.size == 1
     return np.broadcast_to(s.reshape(full), x_shape)
+
+
+def reduce3_all(op, x, y, dims):
+    """execReduce3All (loops/cpu/reduce3.hpp execAll; legacy/NativeOps.h:208): z[i][j] = reduce3(op, x's sub-array i, y's
+    sub-array j), the sub-arrays taken along `dims` and numbered in c order over the other dims.  The pairing is restated
+    here; each pair goes through the oracle's reduce3."""
+    x, y = np.asarray(x), np.asarray(y)
+    dims = sorted(d + x.ndim if d < 0 else d for d in dims)
+    other = [d for d in range(x.ndim) if d not in dims]
+    xt = np.transpose(x, other + dims).reshape((-1,) + tuple(x.shape[d] for d in dims))
+    yt = np.transpose(y, other + dims).reshape((-1,) + tuple(y.shape[d] for d in dims))
+    z = np.zeros((xt.shape[0], yt.shape[0]), x.dtype)
+    for i in range(xt.shape[0]):
+        for j in range(yt.shape[0]):
+            z[i, j] = reduce3(op, np.ascontiguousarray(xt[i]), np.ascontiguousarray(yt[j]), np.zeros((), x.dtype))
+    return z

@@ -175,3 +175,49 @@ def test_errors(ex):
     with pytest.raises(N.NativeOpsError, match="does not match"):
         ex.exec_broadcast_bool(BoolOp.EqualTo, x, NDArray.from_numpy(np.ones(3, np.float32)), [1])
     assert L.lastErrorCode() == 0
+
+
+# ---- execReduce3All: every sub-array of x against every sub-array of y ----------------------------------------------------
+def test_reduce3_all_reference_vectors(ex):
+    from deeplearning4j_amd.executioner import Reduce3
+    x, y = NDArray.from_numpy(np.array([[1, 2, 3], [4, 5, 6]], np.float32)), NDArray.from_numpy(np.full((2, 3), 2, np.float32))
+    got = ex.exec_reduce3_all(Reduce3.EuclideanDistance, x, y, [1]).to_numpy()                     # NDArrayTests.cpp:1455-1470
+    np.testing.assert_allclose(got, [[1.414214, 1.414214], [5.385165, 5.385165]], rtol=1e-6)
+    c = NDArray.from_numpy(np.array([[1, 2, 3], [2, 3, 4]], np.float64))
+    np.testing.assert_allclose(ex.exec_reduce3_all(Reduce3.EuclideanDistance, c, c, [1]).to_numpy(), [[0, 1.73205], [1.73205, 0]], rtol=1e-5)   # NDArrayTests2.cpp:199-209
+    x4, x3 = NDArray.from_numpy(np.array([[1, 2], [3, 4]], np.float64)), NDArray.from_numpy(np.full((2, 3), 1.5))
+    assert np.array_equal(ex.exec_reduce3_all(Reduce3.Dot, x4, x3, [0]).to_numpy(), [[6, 6, 6], [9, 9, 9]])        # MultiDataTypeTests.cpp:1629-1644
+
+
+@pytest.mark.parametrize("dt,tol", [(FLOAT32, 1e-5), (DOUBLE, 1e-12), (BFLOAT16, 1e-2), (HALF, 2e-3)])
+def test_reduce3_all_against_the_oracle(ex, oracle, dt, tol):
+    from conftest import assert_close
+    from deeplearning4j_amd.executioner import Reduce3
+    rng = np.random.default_rng(dt)
+
+    def held(a):
+        if dt == BFLOAT16:
+            return bf16_bits_to_f32(f32_to_bf16_bits(a.astype(np.float32))).astype(np.float64)
+        return a.astype(NP[dt]).astype(np.float64)
+
+    def out(z):
+        return bf16_bits_to_f32(z).astype(np.float64) if dt == BFLOAT16 else z.astype(np.float64)
+
+    for xs, ys, dims in (((5, 33), (7, 33), [1]), ((40, 6), (40, 3), [0]), ((2, 9, 3, 5), (3, 9, 2, 5), [1, 3]), ((4, 300), (4, 300), [1])):
+        x, y = held(rng.normal(0, 1, xs)), held(rng.normal(0, 1, ys))
+        X = NDArray.from_numpy(x.astype(np.float32), dt) if dt == BFLOAT16 else NDArray.from_numpy(x.astype(NP[dt]))
+        Y = NDArray.from_numpy(y.astype(np.float32), dt) if dt == BFLOAT16 else NDArray.from_numpy(y.astype(NP[dt]))
+        for op in (Reduce3.ManhattanDistance, Reduce3.EuclideanDistance, Reduce3.CosineSimilarity, Reduce3.Dot, Reduce3.CosineDistance):
+            want = oracle.reduce3_all(op, x, y, dims)                    # the oracle in float64 on the values the arrays hold
+            got = out(ex.exec_reduce3_all(op, X, Y, dims).to_numpy())
+            scale = max(1.0, float(np.abs(want).max()))
+            assert_close(got, want, tol, tol * scale, "reduce3 all-pairs op %d %s %s" % (op, xs, dims))
+    # the result may be a view: columns 2.. of a wider matrix
+    x, y = held(rng.normal(0, 1, (5, 16))), held(rng.normal(0, 1, (6, 16)))
+    X = NDArray.from_numpy(x.astype(np.float32), dt) if dt == BFLOAT16 else NDArray.from_numpy(x.astype(NP[dt]))
+    Y = NDArray.from_numpy(y.astype(np.float32), dt) if dt == BFLOAT16 else NDArray.from_numpy(y.astype(NP[dt]))
+    wide = NDArray.from_numpy(np.zeros((5, 10), np.float32), dt) if dt == BFLOAT16 else NDArray.from_numpy(np.zeros((5, 10), NP[dt]))
+    ex.exec_reduce3_all(Reduce3.Dot, X, Y, [1], z=wide.slice(1, 2, 8))
+    w = out(wide.to_numpy())
+    assert_close(w[:, 2:8], x @ y.T, tol, tol * 8, "into a view")
+    assert not w[:, :2].any() and not w[:, 8:].any()

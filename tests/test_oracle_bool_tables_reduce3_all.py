@@ -119,3 +119,29 @@ def test_epsilon_boundaries():
     yb = O.bf16_to_f32(O.f32_to_bf16(np.array([1.0, 1.0078125], np.float32)))
     assert O.bool_table(EPS, xb, yb, None, bf16=True).tolist() == [1, 0]
     assert O.bool_table(EPS, xb, yb, [0.0078125], bf16=True).tolist() == [1, 1]
+
+
+def test_reduce3_all_reference_vectors():
+    # NDArrayTests.cpp:1455-1470 (applyAllReduce3EuclideanDistance): rows of x against rows of y
+    x, y = np.array([[1, 2, 3], [4, 5, 6]], np.float32), np.full((2, 3), 2, np.float32)
+    np.testing.assert_allclose(O.reduce3_all(1, x, y, [1]), [[1.414214, 1.414214], [5.385165, 5.385165]], rtol=1e-6)
+    # NDArrayTests2.cpp:186-209 (Test_AllReduce3_1 / _2)
+    a, b = np.array([[1, 2, 3], [1, 2, 3]], np.float64), np.array([[2, 3, 4], [2, 3, 4]], np.float64)
+    np.testing.assert_allclose(O.reduce3_all(1, a, b, [1]), np.full((2, 2), 1.73205), rtol=1e-5)
+    c = np.array([[1, 2, 3], [2, 3, 4]], np.float64)
+    np.testing.assert_allclose(O.reduce3_all(1, c, c, [1]), [[0, 1.73205], [1.73205, 0]], rtol=1e-5)
+    # MultiDataTypeTests.cpp:1629-1644 (applyAllReduce3_test1): Dot over the columns (dimension 0), operands of different widths
+    x4, x3 = np.array([[1, 2], [3, 4]], np.float64), np.full((2, 3), 1.5)
+    assert np.array_equal(O.reduce3_all(3, x4, x3, [0]), [[6, 6, 6], [9, 9, 9]])
+    x1, x2 = np.array([[1, 2], [3, 4]], np.float64), np.array([[-1, 1, -1], [1, -1, 1]], np.float64)
+    assert np.array_equal(O.reduce3_all(3, x1, x2, [0]), [[2, -2, 2], [2, -2, 2]])
+
+
+def test_reduce3_all_dot_is_a_matrix_product():
+    rng = np.random.default_rng(9)
+    x, y = rng.integers(-4, 5, (5, 7)).astype(np.float64), rng.integers(-4, 5, (6, 7)).astype(np.float64)
+    assert np.array_equal(O.reduce3_all(3, x, y, [1]), x @ y.T)
+    # sub-arrays of rank 2, the other dims numbered in c order
+    x3, y3 = rng.integers(-4, 5, (2, 4, 3, 5)).astype(np.float64), rng.integers(-4, 5, (3, 4, 2, 5)).astype(np.float64)
+    want = np.einsum("aibk,cidk->abcd", x3, y3).reshape(6, 6)
+    assert np.array_equal(O.reduce3_all(3, x3, y3, [1, 3]), want)
