@@ -719,10 +719,10 @@ static void layerNormTyped(hipStream_t s, const void* x, const void* gain, const
 #define LN(TPR, NV, GRID) hipLaunchKernelGGL((layernorm_rows<T, TPR, NV, V>), dim3(GRID), dim3(256), 0, s, a, xt, gt, bt, zt, eps)
     // rows at a constant pitch that fit one wave
     const bool linear = p.outerX.rank <= 1 && p.outerZ.rank <= 1 && L < (1 << 30);
-    if (linear && L <= 4 * perWave) {
+    if (linear && L <= 8 * perWave) {
       const LongType xp = p.outerX.rank ? p.outerX.stride[0] : 0, zp = p.outerZ.rank ? p.outerZ.stride[0] : 0;
       // many rows: two per wave (layernorm_stream: gain and bias fetched once for both); few rows: one per wave, so that every CU gets some
-      const bool pair = p.rows >= 4096;
+      const bool pair = p.rows >= 4096 && L <= 4 * perWave;
 #define LNL(NV) do { if (bt) hipLaunchKernelGGL((layernorm_linear<T, NV, true, 1>), dim3(gw), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); \
                      else hipLaunchKernelGGL((layernorm_linear<T, NV, false, 1>), dim3(gw), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); } while (0)
       if (pair) {
@@ -755,7 +755,11 @@ static void layerNormTyped(hipStream_t s, const void* x, const void* gain, const
       if (L <= perWave) { LNL(1); return; }
       if (L <= 2 * perWave) { LNL(2); return; }
       if (L <= 3 * perWave) { LNL(3); return; }   // 768 floats: three full passes, no clamped re-reads
-      LNL(4); return;
+      if (L <= 4 * perWave) { LNL(4); return; }
+      // up to eight passes in registers (fp32 rows of up to 2048, 16-bit rows of up to 4096): the same kernel with more
+      // vectors per lane, every load of the row, the gain and the bias in flight at once
+      if (L <= 6 * perWave) { LNL(6); return; }
+      LNL(8); return;
 #undef LNL
     }
     if (L <= perWave) { LN(64, 1, gw); return; }

@@ -269,6 +269,30 @@ def _ovals(oa):
     return bf16_bits_to_f32(oa.a).astype(np.float64) if oa.dt == BFLOAT16 else oa.a.astype(np.float64)
 
 
+@pytest.mark.parametrize("dt,lengths", [(FLOAT32, (1028, 1280, 1536, 1540, 2048)), (DOUBLE, (516, 768, 1024)), (BFLOAT16, (2056, 2560, 3072, 3080, 4096)),
+                                        (HALF, (2056, 3072, 4096))])
+def test_layer_norm_rows_of_five_to_eight_wave_passes(ex, oracle, dt, lengths):
+    """Rows longer than four 16-byte wave passes and up to eight stay in one wave's registers (six or eight vectors per lane,
+    the last ones partly or wholly masked): few rows and many, with and without bias, dense and at a pitch, against the oracle."""
+    rng = np.random.default_rng(int(dt) * 7 + 1)
+    rtol, atol = {FLOAT32: (2e-5, 2e-6), DOUBLE: (1e-12, 1e-12), BFLOAT16: (1e-2, 1e-2), HALF: (2e-3, 2e-3)}[dt]
+    for C in lengths:
+        for rows, bias, pitched in ((3, True, False), (130, False, True), (4100, True, False) if C <= 2048 else (37, True, True)):
+            a = rng.normal(0.2, 1.5, (rows, C))
+            ox, dx = _opair(oracle, a, dt)
+            if pitched:
+                wide = np.concatenate([a, rng.normal(0, 1, (rows, 16))], axis=1)
+                _, dw = _opair(oracle, wide, dt)
+                dx = dw.slice(1, 0, C)
+            og, dg = _opair(oracle, rng.normal(1, 0.2, C), dt)
+            ob, db = _opair(oracle, rng.normal(0, 0.2, C), dt)
+            oz = _ozero(oracle, (rows, C), dt)
+            oracle.layer_norm(ox, og, ob if bias else None, oz, [1], channels_first=False)
+            z = ex.exec_custom("layer_norm", [dx, dg, db] if bias else [dx, dg], [NDArray.empty((rows, C), dt)], i_args=[1], b_args=[False])[0]
+            got, want = z.to_float().astype(np.float64), _ovals(oz)
+            assert np.all(np.abs(got - want) <= atol + rtol * np.abs(want)), "layer_norm rows %d x %d dtype %d bias %d pitched %d" % (rows, C, dt, bias, pitched)
+
+
 ROW_LENGTHS = [1, 2, 3, 7, 8, 31, 63, 64, 65, 127, 128, 255, 256, 257, 384, 512, 640, 767, 768, 769, 1000, 1023, 1024, 1025, 1536, 2048,
                2049, 3072, 4096, 4100, 6000, 8192, 8200, 12000]
 
