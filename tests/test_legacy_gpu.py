@@ -325,6 +325,35 @@ def test_index_reduce_rows_that_start_off_a_16_byte_boundary(ex, oracle, dtype, 
     assert np.array_equal(ex.exec_index_reduce(0, dx, [1]).to_numpy(), xr.argmax(1))
 
 
+@pytest.mark.parametrize("dtype", [FLOAT32, BFLOAT16, HALF, DOUBLE])
+@pytest.mark.parametrize("rows,cols,first,width", [(6144, 512, 0, 512), (1000, 4096, 0, 4096), (777, 1001, 0, 1001), (4100, 96, 3, 128), (300, 64, 0, 64),
+                                                   (9, 2048, 0, 2048), (40000, 17, 0, 17)])
+def test_reductions_down_the_columns(ex, oracle, dtype, rows, cols, first, width):
+    """Reductions over dim 0 of a row-major matrix (the outputs lie side by side, the reduced axis walks at the row pitch):
+    many rows cut over several blocks, few rows, an odd column count, columns first.. of a wider matrix (rows at a pitch, starts
+    off the 4-byte pairs of the 16-bit types).  Sums within the re-ordered-sum bound, extremes exact; also the leading two dims
+    of a rank-3 array."""
+    rng = np.random.default_rng(rows + cols + first)
+    full = rng.uniform(-1, 1, (rows, width))
+    _, dfull = _oracle_arr(oracle, full, dtype)
+    X = dfull.slice(1, first, first + cols) if width != cols else dfull
+    held = dfull.to_float().astype(np.float64)[:, first:first + cols]
+    tol = {FLOAT32: 1e-5, DOUBLE: 1e-12, BFLOAT16: 1e-2, HALF: 2e-3}[dtype]
+    atol = _sum_atol(held.astype(np.float32), 0) if dtype == FLOAT32 else tol * np.abs(held).sum(0).max()
+    got = ex.exec_reduce_same(ReduceSame.Sum, X, [0]).to_float().astype(np.float64)
+    assert_close(got, held.sum(0), tol, atol, "sum down the columns")
+    got = ex.exec_reduce_float(ReduceFloat.Mean, X, [0]).to_float().astype(np.float64)
+    assert_close(got, held.mean(0), tol, atol / rows + tol * 1e-3, "mean down the columns")
+    got = ex.exec_reduce_float(ReduceFloat.Norm2, X, [0]).to_float().astype(np.float64)
+    assert_close(got, np.sqrt((held ** 2).sum(0)), 2 * tol, 0, "norm2 down the columns")
+    assert np.array_equal(ex.exec_reduce_same(ReduceSame.Max, X, [0]).to_float().astype(np.float64), held.max(0))
+    assert np.array_equal(ex.exec_reduce_same(ReduceSame.Min, X, [0]).to_float().astype(np.float64), held.min(0))
+    if width == cols and rows % 4 == 0:
+        X3 = dfull.reshape(4, rows // 4, cols)
+        got = ex.exec_reduce_same(ReduceSame.Sum, X3, [0, 1]).to_float().astype(np.float64)
+        assert_close(got, held.sum(0), tol, atol, "sum over the two leading dims")
+
+
 @pytest.mark.parametrize("rows,L,pitch", [(37, 1028, 1028), (5, 8192, 8192), (9, 5000, 5000), (33, 4096, 4352), (3, 1024, 2048)])
 def test_reductions_over_rows_at_a_constant_pitch(ex, oracle, rows, L, pitch):
     """Rows of 1024..8192 elements at a constant pitch take the one-shot kernels (all loads up front, masked tail):
