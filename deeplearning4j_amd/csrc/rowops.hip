@@ -264,6 +264,76 @@ __global__ __launch_bounds__(256) void softmax_long(RowArgs a, const T* __restri
     z[zb + j * a.zInner] = Conv<T>::from(softmax_term((A)to_float(x[xb + j * a.xInner]), mx, clamp) / sum);
 }
 
+// The same for unit-stride rows (a vocabulary's worth of logits): one block of 1024 threads per row, 16-byte loads four at a
+// time per thread.  A row may start anywhere (rows of an odd length do): the elements up to the first 16-byte boundary and
+// after the last whole vector are read one by one; x and z must sit at the same offset from such a boundary.  The row is read
+// from memory once and twice more from the cache it fits in; the exponential is taken twice per element, as above.
+template <typename T>
+__global__ __launch_bounds__(1024) void softmax_long_vec(RowArgs a, const T* __restrict__ x, T* __restrict__ z, int clamp) {
+  using A = typename Conv<T>::acc;
+  using Raw = typename RawIO<T>::raw;
+  constexpr int VEC = RawIO<T>::N, NT = 1024, UNR = 4;
+  __shared__ A lds[NT / 64];
+  const LongType row = blockIdx.x;
+  const T* xr = x + walk<LongType>(a.outerX, row);
+  T* zr = z + walk<LongType>(a.outerZ, row);
+  const LongType L = a.rowLen;
+  const int t = threadIdx.x;
+  LongType head = (LongType)(((16 - (reinterpret_cast<uintptr_t>(xr) & 15)) & 15) / sizeof(T));
+  if (head > L) head = L;
+  const LongType nv = (L - head) / VEC, tail0 = head + nv * VEC;
+  const Raw* xv = reinterpret_cast<const Raw*>(xr + head);
+  // f(value, position) over the whole row: head and tail element by element, the body UNR vectors per thread and trip
+  auto sweep = [&](auto&& f) {
+    for (LongType j = t; j < head; j += NT) f((A)to_float(xr[j]), j);
+    for (LongType j = tail0 + t; j < L; j += NT) f((A)to_float(xr[j]), j);
+    for (LongType i = t; i < nv; i += (LongType)UNR * NT) {
+      Raw v[UNR];
+#pragma unroll
+      for (int u = 0; u < UNR; u++) { const LongType iu = i + (LongType)u * NT; v[u] = xv[iu < nv ? iu : nv - 1]; }
+#pragma unroll
+      for (int u = 0; u < UNR; u++) {
+        const LongType iu = i + (LongType)u * NT;
+        if (iu < nv) {
+          A vals[VEC];
+          RawIO<T>::unpack(v[u], vals);
+#pragma unroll
+          for (int e = 0; e < VEC; e++) f(vals[e], head + iu * VEC + e);
+        }
+      }
+    }
+  };
+  const A NEG = -r_tmax<A>();
+  A mx = NEG;
+  sweep([&](A v, LongType) { mx = softmax_maxstep<A>(mx, v, clamp); });
+  mx = block_allreduce<MaxOp, NT / 64, A>(mx, lds);
+  if (clamp && mx == NEG) mx = (A)0;
+  A sum = (A)0;
+  sweep([&](A v, LongType) { sum += softmax_term(v, mx, clamp); });
+  sum = block_allreduce<SumOp, NT / 64, A>(sum, lds);
+  if (clamp) sum = sum > (A)1e-6f ? sum : (A)1e-6f;
+  // the result: whole vectors where whole vectors were read
+  for (LongType j = t; j < head; j += NT) zr[j] = Conv<T>::from(softmax_term((A)to_float(xr[j]), mx, clamp) / sum);
+  for (LongType j = tail0 + t; j < L; j += NT) zr[j] = Conv<T>::from(softmax_term((A)to_float(xr[j]), mx, clamp) / sum);
+  Raw* zv = reinterpret_cast<Raw*>(zr + head);
+  for (LongType i = t; i < nv; i += (LongType)UNR * NT) {
+    Raw v[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; u++) { const LongType iu = i + (LongType)u * NT; v[u] = xv[iu < nv ? iu : nv - 1]; }
+#pragma unroll
+    for (int u = 0; u < UNR; u++) {
+      const LongType iu = i + (LongType)u * NT;
+      if (iu < nv) {
+        A vals[VEC];
+        RawIO<T>::unpack(v[u], vals);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) vals[e] = softmax_term(vals[e], mx, clamp) / sum;
+        zv[iu] = RawIO<T>::pack(vals);
+      }
+    }
+  }
+}
+
 // many short strided rows (softmax over a non-last axis): one thread per row, neighbouring threads
 // own neighbouring rows so that accesses coalesce across the wave
 template <typename T>
@@ -347,6 +417,17 @@ static void softmaxTyped(hipStream_t s, const void* x, void* z, const RowPlan& p
   } else {
     if (L <= 64 * 16) { hipLaunchKernelGGL((softmax_rows<T, 64, 16, 1>), dim3(gw), dim3(256), 0, s, a, xt, zt, clamp, 0); return; }
     if (L <= 256 * 32) { hipLaunchKernelGGL((softmax_rows<T, 256, 32, 1>), dim3(gb), dim3(256), 0, s, a, xt, zt, clamp, 0); return; }
+  }
+  // unit-stride rows whose x and z starts sit at the same offset from a 16-byte boundary in every row
+  if constexpr (sizeof(T) <= 4) {
+    constexpr LongType V = 16 / sizeof(T);
+    bool same = p.xInner == 1 && p.zInner == 1 && ((reinterpret_cast<uintptr_t>(x) ^ reinterpret_cast<uintptr_t>(z)) & 15) == 0 && p.outerX.rank == p.outerZ.rank;
+    for (int d = 0; same && d < p.outerX.rank; d++)
+      if (p.outerX.shape[d] > 1 && (p.outerX.stride[d] - p.outerZ.stride[d]) % V != 0) same = false;
+    if (same) {
+      hipLaunchKernelGGL((softmax_long_vec<T>), dim3(gb), dim3(1024), 0, s, a, xt, zt, clamp);
+      return;
+    }
   }
   hipLaunchKernelGGL((softmax_long<T>), dim3(gb), dim3(256), 0, s, a, xt, zt, clamp);
 }

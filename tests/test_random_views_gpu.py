@@ -293,6 +293,33 @@ def test_layer_norm_rows_of_five_to_eight_wave_passes(ex, oracle, dt, lengths):
             assert np.all(np.abs(got - want) <= atol + rtol * np.abs(want)), "layer_norm rows %d x %d dtype %d bias %d pitched %d" % (rows, C, dt, bias, pitched)
 
 
+@pytest.mark.parametrize("dt", [FLOAT32, BFLOAT16, HALF])
+def test_softmax_over_a_vocabulary(ex, oracle, dt):
+    """Rows too long for a block's registers (a vocabulary's worth of logits): an odd length, so that no row after the first
+    starts on a 16-byte boundary, lengths around the kernel's vector trips, a result written at a pitch of its own, and rows
+    whose x and z starts differ in alignment (the element-by-element kernel)."""
+    rng = np.random.default_rng(int(dt) + 50257)
+    rtol, atol = {FLOAT32: (2e-5, 1e-9), BFLOAT16: (1e-2, 1e-6), HALF: (2e-3, 1e-7)}[dt]
+    for rows, C in ((5, 50257), (3, 20000), (2, 131075), (4, 16385 if dt == FLOAT32 else 32770)):
+        a = rng.normal(0, 2.0, (rows, C))
+        a[0, C // 3] = 9.0                                   # one dominant entry
+        ox, dx = _opair(oracle, a, dt)
+        oz = _ozero(oracle, (rows, C), dt)
+        oracle.softmax(ox, oz, 1)
+        want = _ovals(oz)
+        z = ex.exec_custom("softmax", [dx], [NDArray.empty((rows, C), dt)], i_args=[1])[0]
+        got = z.to_float().astype(np.float64)
+        assert np.all(np.abs(got - want) <= atol + rtol * np.abs(want)), "softmax rows %d x %d dtype %d" % (rows, C, dt)
+        assert np.all(np.abs(got.sum(1) - 1.0) < (2e-2 if dt != FLOAT32 else 1e-4))
+        # the result into columns 8.. of a wider array (another pitch, the same alignment) and into columns 3.. (another alignment)
+        for first in (8, 3):
+            wide = NDArray.from_numpy(np.full((rows, C + 16), 7.0, np.float32), dt) if dt == BFLOAT16 else NDArray.from_numpy(np.full((rows, C + 16), 7.0, DT_NP[dt]))
+            ex.exec_custom("softmax", [dx], [wide.slice(1, first, first + C)], i_args=[1])
+            w = wide.to_float().astype(np.float64)
+            assert np.all(np.abs(w[:, first:first + C] - want) <= atol + rtol * np.abs(want)), "pitched result, first column %d" % first
+            assert np.all(w[:, :first] == 7.0) and np.all(w[:, first + C:] == 7.0)
+
+
 ROW_LENGTHS = [1, 2, 3, 7, 8, 31, 63, 64, 65, 127, 128, 255, 256, 257, 384, 512, 640, 767, 768, 769, 1000, 1023, 1024, 1025, 1536, 2048,
                2049, 3072, 4096, 4100, 6000, 8192, 8200, 12000]
 
