@@ -419,10 +419,12 @@ static void layerNormImpl(Context& c, NDArray* x, NDArray* gain, NDArray* bias, 
   prepareSpecialUse(std::vector<NDArray*>{z}, reads);
   const float eps = 1e-5f;
   const bool lastAxisOnly = axes.size() == 1 && axes[0] == rank - 1 && dimC == rank - 1 && gain && gain->strideAt(0) == 1 && (!bias || bias->strideAt(0) == 1);
-  if (lastAxisOnly && x->sizeAt(rank - 1) <= 8192) {
+  bool done = false;
+  if (lastAxisOnly && x->sizeAt(rank - 1) <= 16384) {   // the row kernels say themselves which lengths they take
     RowPlan p = buildRowPlan(x->shapeInfo(), z->shapeInfo(), rank - 1);
-    launchLayerNormRows(stream(), x->dataType(), x->specialBuffer(), gain->specialBuffer(), bias ? bias->specialBuffer() : nullptr, z->specialBuffer(), p, eps);
-  } else {
+    done = launchLayerNormRows(stream(), x->dataType(), x->specialBuffer(), gain->specialBuffer(), bias ? bias->specialBuffer() : nullptr, z->specialBuffer(), p, eps);
+  }
+  if (!done) {
     ND4J_REQUIRE(!gain || (gain->strideAt(0) == 1 && (!bias || bias->strideAt(0) == 1)), "LAYER_NORM OP: gain/bias must be dense");
     LnGenericPlan p = lnGenericPlan(x, z, axes, dimC);
     launchLayerNormGeneric(stream(), x->dataType(), x->specialBuffer(), gain ? gain->specialBuffer() : nullptr, bias ? bias->specialBuffer() : nullptr, z->specialBuffer(), p, eps);

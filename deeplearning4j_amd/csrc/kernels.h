@@ -167,7 +167,8 @@ struct RowPlan {
 void launchSoftmax(hipStream_t s, DataType dt, const void* x, void* z, const RowPlan& p, bool clampMode);
 // log(exp(x - max) / sum) along the plan's rows, evaluated in that order
 void launchLogSoftmax(hipStream_t s, DataType dt, const void* x, void* z, const RowPlan& p);
-void launchLayerNormRows(hipStream_t s, DataType dt, const void* x, const void* gain, const void* bias, void* z,
+// false: the rows are longer than the row kernels take (nothing launched; launchLayerNormGeneric serves them)
+bool launchLayerNormRows(hipStream_t s, DataType dt, const void* x, const void* gain, const void* bias, void* z,
                          const RowPlan& p, float eps);
 // sumOut = x + addend (pairwise Add in the array type), z = layer_norm(sumOut) over rows of length L at constant pitches, in
 // one kernel; false when the shape is not the one-wave-per-row vector case (nothing launched then)

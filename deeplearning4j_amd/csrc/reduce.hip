@@ -85,8 +85,16 @@ __global__ __launch_bounds__(256) void reduce_coop(CoopArgs a, const T* __restri
       LongType j = j0;
       if (vectorOk) {
         using VT = Vec<T, V>;
-        const LongType nv = (j1 - j0) / V;
-        const VT* pv = reinterpret_cast<const VT*>(p + j0);
+        // vectorOk 2: the run starts anywhere (rows of an odd length): the elements up to the first 16-byte boundary are
+        // read one by one, as the tail is
+        LongType f0 = j0;
+        if (vectorOk == 2) {
+          f0 = j0 + (LongType)(((16 - (reinterpret_cast<uintptr_t>(p + j0) & 15)) & 15) / sizeof(T));
+          if (f0 > j1) f0 = j1;
+          for (LongType q = j0 + t; q < f0; q += TPR) acc = Op::apply(acc, pre<PRE, A>((A)to_float(p[q])));
+        }
+        const LongType nv = (j1 - f0) / V;
+        const VT* pv = reinterpret_cast<const VT*>(p + f0);
         LongType i = t;
         for (; i + 3 * TPR < nv; i += 4 * TPR) {
           VT v0 = pv[i], v1 = pv[i + TPR], v2 = pv[i + 2 * TPR], v3 = pv[i + 3 * TPR];
@@ -103,7 +111,7 @@ __global__ __launch_bounds__(256) void reduce_coop(CoopArgs a, const T* __restri
 #pragma unroll
           for (int e = 0; e < V; e++) acc = Op::apply(acc, pre<PRE, A>((A)to_float(v0.v[e])));
         }
-        j = j0 + nv * V;
+        j = f0 + nv * V;
       }
       for (LongType q = j + t; q < j1; q += TPR) acc = Op::apply(acc, pre<PRE, A>((A)to_float(p[q])));
     } else if (a.inner.rank == 1) {
@@ -164,7 +172,7 @@ struct LaunchShape {
   LongType segLen;
   bool flat;
   int vectorOk;
-  int peelOk;   // unit-stride runs whose starts are not 16-byte aligned: vector loads after a scalar head (index kernels)
+  int peelOk;   // unit-stride runs whose starts are not 16-byte aligned: vector loads after a scalar head
 };
 
 static LaunchShape shapeLaunch(const ReducePlan& p, size_t elemSize, const void* x, size_t partialSize, size_t scratchBytes) {
@@ -364,10 +372,11 @@ static void reduceTyped(hipStream_t st, const void* x, void* z, const ReducePlan
     return;
   }
   const LongType units = p.outerLen * s.splits;
+  const int vec = s.vectorOk ? 1 : (s.peelOk ? 2 : 0);
   if (s.tpr == 64) {
-    hipLaunchKernelGGL((reduce_coop<Op, PRE, T, 64>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, st, a, (const T*)x, (T*)z, (A*)scratch, s.vectorOk);
+    hipLaunchKernelGGL((reduce_coop<Op, PRE, T, 64>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, st, a, (const T*)x, (T*)z, (A*)scratch, vec);
   } else {
-    hipLaunchKernelGGL((reduce_coop<Op, PRE, T, 256>), dim3((unsigned)units), dim3(256), 0, st, a, (const T*)x, (T*)z, (A*)scratch, s.vectorOk);
+    hipLaunchKernelGGL((reduce_coop<Op, PRE, T, 256>), dim3((unsigned)units), dim3(256), 0, st, a, (const T*)x, (T*)z, (A*)scratch, vec);
   }
   if (s.splits > 1)
     hipLaunchKernelGGL((reduce_finish<Op, T>), dim3((unsigned)((p.outerLen + 255) / 256)), dim3(256), 0, st, a, (const A*)scratch, (T*)z);

@@ -502,12 +502,22 @@ __global__ __launch_bounds__(256) void layernorm_rows(RowArgs a, const T* __rest
   const LongType L = a.rowLen;
   A vals[NV * VEC];
   A sum = (A)0;
+  // vector rows (L a multiple of VEC, so at least one whole vector): every load is issued unconditionally, past the row's end
+  // on its last vector, so that the row costs one trip to memory and not one per vector
+  typename RawIO<T>::raw xraw[VEC > 1 ? NV : 1];
+  if (VEC > 1) {
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      const LongType e0 = ((LongType)t + (LongType)i * TPR) * VEC;
+      xraw[VEC > 1 ? i : 0] = *reinterpret_cast<const typename RawIO<T>::raw*>(x + xb + (e0 < L ? e0 : L - VEC));
+    }
+  }
 #pragma unroll
   for (int i = 0; i < NV; i++) {
     const LongType e0 = ((LongType)t + (LongType)i * TPR) * VEC;
     if (VEC > 1) {
       if (e0 < L) {
-        RawIO<T>::unpack(*reinterpret_cast<const typename RawIO<T>::raw*>(x + xb + e0), &vals[i * VEC]);
+        RawIO<T>::unpack(xraw[VEC > 1 ? i : 0], &vals[i * VEC]);
 #pragma unroll
         for (int e = 0; e < VEC; e++) sum += vals[i * VEC + e];
       } else {
@@ -532,14 +542,24 @@ __global__ __launch_bounds__(256) void layernorm_rows(RowArgs a, const T* __rest
   const A var = L > 1 ? sq / (A)L : (A)0;
   const A rstd = (A)1 / r_sqrt<A>(var + (A)eps);   // one division per row
   if (!live) return;
+  typename RawIO<T>::raw graw[VEC > 1 ? NV : 1], braw[VEC > 1 ? NV : 1];
+  if (VEC > 1) {   // gain and bias the same way: all loads before the first use
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      const LongType e0 = ((LongType)t + (LongType)i * TPR) * VEC;
+      const LongType ec = e0 < L ? e0 : L - VEC;
+      graw[VEC > 1 ? i : 0] = *reinterpret_cast<const typename RawIO<T>::raw*>(gain + ec);
+      braw[VEC > 1 ? i : 0] = bias ? *reinterpret_cast<const typename RawIO<T>::raw*>(bias + ec) : graw[VEC > 1 ? i : 0];
+    }
+  }
 #pragma unroll
   for (int i = 0; i < NV; i++) {
     const LongType e0 = ((LongType)t + (LongType)i * TPR) * VEC;
     if (e0 >= L) continue;
     if (VEC > 1) {
       A g[VEC], b[VEC];
-      RawIO<T>::unpack(*reinterpret_cast<const typename RawIO<T>::raw*>(gain + e0), g);
-      if (bias) RawIO<T>::unpack(*reinterpret_cast<const typename RawIO<T>::raw*>(bias + e0), b);
+      RawIO<T>::unpack(graw[VEC > 1 ? i : 0], g);
+      if (bias) RawIO<T>::unpack(braw[VEC > 1 ? i : 0], b);
 #pragma unroll
       for (int e = 0; e < VEC; e++) {
         A y = (vals[i * VEC + e] - mean) * rstd * g[e];
@@ -788,7 +808,7 @@ __global__ __launch_bounds__(256, WALK ? 1 : 8) void layernorm_stream(const T* _
 }
 
 template <typename T>
-static void layerNormTyped(hipStream_t s, const void* x, const void* gain, const void* bias, void* z, const RowPlan& p, float eps) {
+static bool layerNormTyped(hipStream_t s, const void* x, const void* gain, const void* bias, void* z, const RowPlan& p, float eps) {
   constexpr int V = 16 / sizeof(T);
   RowArgs a = rowArgs(p);
   const T* xt = (const T*)x; const T* gt = (const T*)gain; const T* bt = (const T*)bias; T* zt = (T*)z;
@@ -826,34 +846,34 @@ static void layerNormTyped(hipStream_t s, const void* x, const void* gain, const
             if (L == 384) LNS12(1); else if (L == 768) LNS12(2); else LNS12(3);
 #undef LNS12
 #undef LNS12W
-            return;
+            return true;
           }
         }
         if (L <= perWave) LNS(1); else if (L <= 2 * perWave) LNS(2); else if (L <= 3 * perWave) LNS(3); else LNS(4);
 #undef LNS
-        return;
+        return true;
       }
-      if (L <= perWave) { LNL(1); return; }
-      if (L <= 2 * perWave) { LNL(2); return; }
-      if (L <= 3 * perWave) { LNL(3); return; }   // 768 floats: three full passes, no clamped re-reads
-      if (L <= 4 * perWave) { LNL(4); return; }
+      if (L <= perWave) { LNL(1); return true; }
+      if (L <= 2 * perWave) { LNL(2); return true; }
+      if (L <= 3 * perWave) { LNL(3); return true; }   // 768 floats: three full passes, no clamped re-reads
+      if (L <= 4 * perWave) { LNL(4); return true; }
       // up to eight passes in registers (fp32 rows of up to 2048, 16-bit rows of up to 4096): the same kernel with more
       // vectors per lane, every load of the row, the gain and the bias in flight at once
-      if (L <= 6 * perWave) { LNL(6); return; }
-      LNL(8); return;
+      if (L <= 6 * perWave) { LNL(6); return true; }
+      LNL(8); return true;
 #undef LNL
     }
-    if (L <= perWave) { LN(64, 1, gw); return; }
-    if (L <= 2 * perWave) { LN(64, 2, gw); return; }
-    if (L <= 4 * perWave) { LN(64, 4, gw); return; }
-    if (L <= 8 * perWave) { LN(64, 8, gw); return; }
-    if (L <= 4 * perBlock) { LN(256, 4, gb); return; }
-    if (L <= 8 * perBlock) { LN(256, 8, gb); return; }
+    if (L <= perWave) { LN(64, 1, gw); return true; }
+    if (L <= 2 * perWave) { LN(64, 2, gw); return true; }
+    if (L <= 4 * perWave) { LN(64, 4, gw); return true; }
+    if (L <= 8 * perWave) { LN(64, 8, gw); return true; }
+    if (L <= 4 * perBlock) { LN(256, 4, gb); return true; }
+    if (L <= 8 * perBlock) { LN(256, 8, gb); return true; }
 #undef LN
   }
-  if (L <= 64 * 16) { hipLaunchKernelGGL((layernorm_rows<T, 64, 16, 1>), dim3(gw), dim3(256), 0, s, a, xt, gt, bt, zt, eps); return; }
-  if (L <= 256 * 32) { hipLaunchKernelGGL((layernorm_rows<T, 256, 32, 1>), dim3(gb), dim3(256), 0, s, a, xt, gt, bt, zt, eps); return; }
-  ND4J_THROW("layer_norm: rows longer than 8192 elements take the generic path");
+  if (L <= 64 * 16) { hipLaunchKernelGGL((layernorm_rows<T, 64, 16, 1>), dim3(gw), dim3(256), 0, s, a, xt, gt, bt, zt, eps); return true; }
+  if (L <= 256 * 32) { hipLaunchKernelGGL((layernorm_rows<T, 256, 32, 1>), dim3(gb), dim3(256), 0, s, a, xt, gt, bt, zt, eps); return true; }
+  return false;   // longer rows: the caller takes the generic kernel
 }
 
 // x + addend -> sumOut, layer_norm(sumOut) -> z in one kernel; only the one-wave-per-row vector case (rows at a constant
@@ -891,17 +911,19 @@ bool launchAddLayerNormRows(hipStream_t s, DataType dt, const void* x, const voi
   return ok;
 }
 
-void launchLayerNormRows(hipStream_t s, DataType dt, const void* x, const void* gain, const void* bias, void* z,
+bool launchLayerNormRows(hipStream_t s, DataType dt, const void* x, const void* gain, const void* bias, void* z,
                          const RowPlan& p, float eps) {
-  if (p.rows == 0 || p.rowLen == 0) return;
+  if (p.rows == 0 || p.rowLen == 0) return true;
+  bool done = false;
   switch (dt) {
-    case FLOAT32: layerNormTyped<float>(s, x, gain, bias, z, p, eps); break;
-    case DOUBLE: layerNormTyped<double>(s, x, gain, bias, z, p, eps); break;
-    case HALF: layerNormTyped<f16_t>(s, x, gain, bias, z, p, eps); break;
-    case BFLOAT16: layerNormTyped<bf16_t>(s, x, gain, bias, z, p, eps); break;
+    case FLOAT32: done = layerNormTyped<float>(s, x, gain, bias, z, p, eps); break;
+    case DOUBLE: done = layerNormTyped<double>(s, x, gain, bias, z, p, eps); break;
+    case HALF: done = layerNormTyped<f16_t>(s, x, gain, bias, z, p, eps); break;
+    case BFLOAT16: done = layerNormTyped<bf16_t>(s, x, gain, bias, z, p, eps); break;
     default: ND4J_THROW("layer_norm: unsupported dtype");
   }
   HIP_CHECK(hipGetLastError());
+  return done;
 }
 
 // generic axes: one block per statistics group, elements reached through the inner walk; gain/bias are

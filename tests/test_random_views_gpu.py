@@ -269,11 +269,12 @@ def _ovals(oa):
     return bf16_bits_to_f32(oa.a).astype(np.float64) if oa.dt == BFLOAT16 else oa.a.astype(np.float64)
 
 
-@pytest.mark.parametrize("dt,lengths", [(FLOAT32, (1028, 1280, 1536, 1540, 2048)), (DOUBLE, (516, 768, 1024)), (BFLOAT16, (2056, 2560, 3072, 3080, 4096)),
-                                        (HALF, (2056, 3072, 4096))])
+@pytest.mark.parametrize("dt,lengths", [(FLOAT32, (1028, 1280, 1536, 1540, 2048, 6144, 8192, 12288)), (DOUBLE, (516, 768, 1024, 5000)),
+                                        (BFLOAT16, (2056, 2560, 3072, 3080, 4096, 12288, 16384, 16392)), (HALF, (2056, 3072, 4096, 12296))])
 def test_layer_norm_rows_of_five_to_eight_wave_passes(ex, oracle, dt, lengths):
     """Rows longer than four 16-byte wave passes and up to eight stay in one wave's registers (six or eight vectors per lane,
-    the last ones partly or wholly masked): few rows and many, with and without bias, dense and at a pitch, against the oracle."""
+    the last ones partly or wholly masked); longer ones take a block per row up to 8192 fp32 / 16384 16-bit elements and the
+    generic kernel beyond: few rows and many, with and without bias, dense and at a pitch, against the oracle."""
     rng = np.random.default_rng(int(dt) * 7 + 1)
     rtol, atol = {FLOAT32: (2e-5, 2e-6), DOUBLE: (1e-12, 1e-12), BFLOAT16: (1e-2, 1e-2), HALF: (2e-3, 2e-3)}[dt]
     for C in lengths:
