@@ -1196,7 +1196,19 @@ static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
   constexpr int NT = WM * WN * 64;
   constexpr size_t LDS = (size_t)2 * (TileLayout<BM, A_KC>::SLOTS + TileLayout<BN, B_KC>::SLOTS) * 16;
   int splits = 1;
-  if (allowSplit) {
+  // 64 x 64 tiles that the direct-load ring kernel below can take, K up to 2048: one block per tile and no split beats
+  // split-K plus its finishing launch even with a quarter of the CUs busy (bf16 512^3 4.5 against 11.2 us, 768^3 4.7 against
+  // 12.0, 512 x 512 x 2048 7.7 against 13.0; from K = 4096 on the split wins: 256 x 256 x 4096 10.4 against 11.9)
+  bool ringInstead = false;
+  if constexpr (BM == 64 && BN == 64 && WM == 2 && WN == 2 && A_KC) {
+    static const bool small = getenv("ND4JHIP_GEMM_SMALL_RING") ? atoi(getenv("ND4JHIP_GEMM_SMALL_RING")) != 0 : true;
+    const LongType ldaS = g.aRow, ldbS = B_KC ? g.bCol : g.bRow;
+    ringInstead = small && g.K >= 512 && g.K <= 2048 && g.K % 256 == 0 && g.M % BM == 0 && g.N % BN == 0 && (g.M / BM) * (g.N / BN) * batch <= 1024 &&
+                  ldaS % 8 == 0 && ldbS % 8 == 0 && ldaS < (1 << 23) && ldbS < (1 << 23) &&
+                  ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 && g.aBatch % 8 == 0 && g.bBatch % 8 == 0 &&
+                  g.aBatch2 % 8 == 0 && g.bBatch2 % 8 == 0 && !g.hasEpi;
+  }
+  if (allowSplit && !ringInstead) {
     LongType per = 0;
     splits = chooseSplits<BM, BN>(g, batch, per);
     if (splits > 1) {

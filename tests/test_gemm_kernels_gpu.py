@@ -85,6 +85,10 @@ CASES = [
     (BFLOAT16, 1024, 1024, 512, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=8>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=8>", None),
     (FLOAT32, 1024, 1024, 384, "gemm_mfma32q<f32,64x64,akc=1,bkc=0,pd=4,bk=32>", "gemm_mfma32q<f32,64x64,akc=1,bkc=1,pd=4,bk=32>", None),
     (FLOAT32, 2048, 2048, 640, "gemm_mfma32q<f32,128x128,akc=1,bkc=0,pd=4,bk=16>", "gemm_mfma32q<f32,128x128,akc=1,bkc=1,pd=4,bk=16>", None),
+    # few 64 x 64 tiles: up to K = 2048 one block per tile on the ring kernel, beyond that split-K with its finishing launch
+    (BFLOAT16, 512, 512, 512, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=8>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=8>", None),
+    (HALF, 512, 768, 2048, "gemm_mfma16s<f16,64x64,akc=1,bkc=0,stages=8>", "gemm_mfma16s<f16,64x64,akc=1,bkc=1,stages=8>", None),
+    (BFLOAT16, 256, 256, 4096, "gemm_mfma16<bf16,64x64,akc=1,bkc=0>+splitk_finish", "gemm_mfma16<bf16,64x64,akc=1,bkc=1>+splitk_finish", None),
     # fp32 ragged
     (FLOAT32, 1100, 900, 1000, "gemm_mfma32<f32,64x64,akc=1,bkc=0>", "gemm_mfma32<f32,64x64,akc=1,bkc=1>", None),
     (FLOAT32, 2100, 2052, 520, "gemm_mfma32<f32,128x128,akc=1,bkc=0>", "gemm_mfma32<f32,128x128,akc=1,bkc=1>", "gemm_mfma32<f32,128x128,akc=0,bkc=0>"),
