@@ -146,6 +146,21 @@ __global__ __launch_bounds__(256) void reduce_finish(CoopArgs a, const typename 
   z[zo] = Conv<T>::from(post<A>(acc, a.postKind, a.innerLen));
 }
 
+// few outputs, many partials each (a whole array reduced to one element: 1024 partials): a block per output, its threads
+// over the partials, so that the partials cost one trip to memory and not a chain of loads in a single thread
+template <typename Op, typename T>
+__global__ __launch_bounds__(256) void reduce_finish_wide(CoopArgs a, const typename Conv<T>::acc* __restrict__ partials, T* __restrict__ z) {
+  using A = typename Conv<T>::acc;
+  __shared__ A lds[4];
+  const LongType row = blockIdx.x;
+  A acc = Identity<Op, A>::v();
+  for (int s = threadIdx.x; s < a.splits; s += 256) acc = Op::apply(acc, partials[row * a.splits + s]);
+  acc = block_allreduce<Op, 4, A>(acc, lds);
+  if (threadIdx.x != 0) return;
+  const LongType zo = a.zLinear ? row : walk<LongType>(a.zOuter, row);
+  z[zo] = Conv<T>::from(post<A>(acc, a.postKind, a.innerLen));
+}
+
 // ---- value reduce, one thread per output -----------------------------------------------------------------
 template <typename Op, int PRE, typename T>
 __global__ __launch_bounds__(256) void reduce_flat(CoopArgs a, const T* __restrict__ x, T* __restrict__ z) {
@@ -354,8 +369,12 @@ static bool tryReduceCols(hipStream_t st, const void* x, void* z, const ReducePl
   if (cpl == 2) { if constexpr (sizeof(T) <= 2) RC(2); }
   else RC(1);
 #undef RC
-  if (splits > 1)
-    hipLaunchKernelGGL((reduce_finish<Op, T>), dim3((unsigned)((p.outerLen + 255) / 256)), dim3(256), 0, st, a, (const A*)scratch, (T*)z);
+  if (splits > 1) {
+    if (splits >= 32 && p.outerLen <= 4096)
+      hipLaunchKernelGGL((reduce_finish_wide<Op, T>), dim3((unsigned)p.outerLen), dim3(256), 0, st, a, (const A*)scratch, (T*)z);
+    else
+      hipLaunchKernelGGL((reduce_finish<Op, T>), dim3((unsigned)((p.outerLen + 255) / 256)), dim3(256), 0, st, a, (const A*)scratch, (T*)z);
+  }
   return true;
 }
 
@@ -378,8 +397,12 @@ static void reduceTyped(hipStream_t st, const void* x, void* z, const ReducePlan
   } else {
     hipLaunchKernelGGL((reduce_coop<Op, PRE, T, 256>), dim3((unsigned)units), dim3(256), 0, st, a, (const T*)x, (T*)z, (A*)scratch, vec);
   }
-  if (s.splits > 1)
-    hipLaunchKernelGGL((reduce_finish<Op, T>), dim3((unsigned)((p.outerLen + 255) / 256)), dim3(256), 0, st, a, (const A*)scratch, (T*)z);
+  if (s.splits > 1) {
+    if (s.splits >= 32 && p.outerLen <= 4096)
+      hipLaunchKernelGGL((reduce_finish_wide<Op, T>), dim3((unsigned)p.outerLen), dim3(256), 0, st, a, (const A*)scratch, (T*)z);
+    else
+      hipLaunchKernelGGL((reduce_finish<Op, T>), dim3((unsigned)((p.outerLen + 255) / 256)), dim3(256), 0, st, a, (const A*)scratch, (T*)z);
+  }
 }
 
 template <typename Op, int PRE>
