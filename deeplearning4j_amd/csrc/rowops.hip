@@ -264,11 +264,14 @@ __global__ __launch_bounds__(256) void softmax_long(RowArgs a, const T* __restri
     z[zb + j * a.zInner] = Conv<T>::from(softmax_term((A)to_float(x[xb + j * a.xInner]), mx, clamp) / sum);
 }
 
+template <typename A> __device__ __forceinline__ A r_log(A x);
+template <> __device__ __forceinline__ float r_log<float>(float x) { return logf(x); }
+template <> __device__ __forceinline__ double r_log<double>(double x) { return log(x); }
 // The same for unit-stride rows (a vocabulary's worth of logits): one block of 1024 threads per row, 16-byte loads four at a
 // time per thread.  A row may start anywhere (rows of an odd length do): the elements up to the first 16-byte boundary and
 // after the last whole vector are read one by one; x and z must sit at the same offset from such a boundary.  The row is read
 // from memory once and twice more from the cache it fits in; the exponential is taken twice per element, as above.
-template <typename T>
+template <typename T, bool LOG = false>
 __global__ __launch_bounds__(1024) void softmax_long_vec(RowArgs a, const T* __restrict__ x, T* __restrict__ z, int clamp) {
   using A = typename Conv<T>::acc;
   using Raw = typename RawIO<T>::raw;
@@ -305,16 +308,19 @@ __global__ __launch_bounds__(1024) void softmax_long_vec(RowArgs a, const T* __r
   };
   const A NEG = -r_tmax<A>();
   A mx = NEG;
-  sweep([&](A v, LongType) { mx = softmax_maxstep<A>(mx, v, clamp); });
+  sweep([&](A v, LongType) { mx = LOG ? (v > mx ? v : mx) : softmax_maxstep<A>(mx, v, clamp); });
   mx = block_allreduce<MaxOp, NT / 64, A>(mx, lds);
-  if (clamp && mx == NEG) mx = (A)0;
+  if (!LOG && clamp && mx == NEG) mx = (A)0;
   A sum = (A)0;
-  sweep([&](A v, LongType) { sum += softmax_term(v, mx, clamp); });
+  // LOG: log(exp(x - max) / sum) in that order, as log_softmax_rows evaluates it
+  auto term = [&](A v) -> A { if constexpr (LOG) return r_exp<A>(v - mx); else return softmax_term(v, mx, clamp); };
+  sweep([&](A v, LongType) { sum += term(v); });
   sum = block_allreduce<SumOp, NT / 64, A>(sum, lds);
-  if (clamp) sum = sum > (A)1e-6f ? sum : (A)1e-6f;
+  if (!LOG && clamp) sum = sum > (A)1e-6f ? sum : (A)1e-6f;
+  auto result = [&](A v) -> A { if constexpr (LOG) return r_log<A>(term(v) / sum); else return term(v) / sum; };
   // the result: whole vectors where whole vectors were read
-  for (LongType j = t; j < head; j += NT) zr[j] = Conv<T>::from(softmax_term((A)to_float(xr[j]), mx, clamp) / sum);
-  for (LongType j = tail0 + t; j < L; j += NT) zr[j] = Conv<T>::from(softmax_term((A)to_float(xr[j]), mx, clamp) / sum);
+  for (LongType j = t; j < head; j += NT) zr[j] = Conv<T>::from(result((A)to_float(xr[j])));
+  for (LongType j = tail0 + t; j < L; j += NT) zr[j] = Conv<T>::from(result((A)to_float(xr[j])));
   Raw* zv = reinterpret_cast<Raw*>(zr + head);
   for (LongType i = t; i < nv; i += (LongType)UNR * NT) {
     Raw v[UNR];
@@ -327,7 +333,7 @@ __global__ __launch_bounds__(1024) void softmax_long_vec(RowArgs a, const T* __r
         A vals[VEC];
         RawIO<T>::unpack(v[u], vals);
 #pragma unroll
-        for (int e = 0; e < VEC; e++) vals[e] = softmax_term(vals[e], mx, clamp) / sum;
+        for (int e = 0; e < VEC; e++) vals[e] = result(vals[e]);
         zv[iu] = RawIO<T>::pack(vals);
       }
     }
@@ -449,9 +455,6 @@ void launchSoftmax(hipStream_t s, DataType dt, const void* x, void* z, const Row
 // generic/nn/logSoftmax.cpp:34-49 -> helpers/cpu/activations.cpp:100-145,236-256: max, exp(x - max), sum, divide, log, in
 // that order (a term whose exponential underflows comes out as -inf, as it does there).  One block per row, three passes;
 // rows and inner strides are arbitrary.  Not a tuned kernel.
-template <typename A> __device__ __forceinline__ A r_log(A x);
-template <> __device__ __forceinline__ float r_log<float>(float x) { return logf(x); }
-template <> __device__ __forceinline__ double r_log<double>(double x) { return log(x); }
 template <typename T>
 __global__ __launch_bounds__(256) void log_softmax_rows(RowArgs a, const T* __restrict__ x, T* __restrict__ z) {
   using A = typename Conv<T>::acc;
@@ -472,6 +475,22 @@ void launchLogSoftmax(hipStream_t s, DataType dt, const void* x, void* z, const 
   ND4J_REQUIRE(p.rows < (1LL << 31), "log_softmax: too many rows");
   RowArgs a = rowArgs(p);
   const dim3 g((unsigned)p.rows), b(256);
+  // long unit-stride rows whose x and z starts sit at the same offset from a 16-byte boundary: the vector kernel of the
+  // long-row softmax with the logarithm on the way out
+  if ((dt == FLOAT32 || dt == HALF || dt == BFLOAT16) && p.rowLen >= 8192 && p.xInner == 1 && p.zInner == 1 &&
+      ((reinterpret_cast<uintptr_t>(x) ^ reinterpret_cast<uintptr_t>(z)) & 15) == 0 && p.outerX.rank == p.outerZ.rank) {
+    const LongType V = dt == FLOAT32 ? 4 : 8;
+    bool same = true;
+    for (int d = 0; same && d < p.outerX.rank; d++)
+      if (p.outerX.shape[d] > 1 && (p.outerX.stride[d] - p.outerZ.stride[d]) % V != 0) same = false;
+    if (same) {
+      if (dt == FLOAT32) hipLaunchKernelGGL((softmax_long_vec<float, true>), g, dim3(1024), 0, s, a, (const float*)x, (float*)z, 0);
+      else if (dt == HALF) hipLaunchKernelGGL((softmax_long_vec<f16_t, true>), g, dim3(1024), 0, s, a, (const f16_t*)x, (f16_t*)z, 0);
+      else hipLaunchKernelGGL((softmax_long_vec<bf16_t, true>), g, dim3(1024), 0, s, a, (const bf16_t*)x, (bf16_t*)z, 0);
+      HIP_CHECK(hipGetLastError());
+      return;
+    }
+  }
   switch (dt) {
     case FLOAT32: hipLaunchKernelGGL((log_softmax_rows<float>), g, b, 0, s, a, (const float*)x, (float*)z); break;
     case DOUBLE: hipLaunchKernelGGL((log_softmax_rows<double>), g, b, 0, s, a, (const double*)x, (double*)z); break;

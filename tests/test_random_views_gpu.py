@@ -321,6 +321,28 @@ def test_softmax_over_a_vocabulary(ex, oracle, dt):
             assert np.all(w[:, :first] == 7.0) and np.all(w[:, first + C:] == 7.0)
 
 
+@pytest.mark.parametrize("dt", [FLOAT32, BFLOAT16, HALF])
+def test_log_softmax_over_a_vocabulary(ex, oracle, dt):
+    """log_softmax (generic/nn/activations/log_softmax.cpp: log(exp(x - max) / sum)) over rows of a vocabulary's length -- an odd
+    length, so that the rows start off the 16-byte boundaries -- and of a length just past the switch to the long-row kernel,
+    against the oracle's restatement."""
+    rng = np.random.default_rng(int(dt) + 11)
+    rtol, atol = {FLOAT32: (2e-5, 2e-5), BFLOAT16: (1e-2, 2e-2), HALF: (2e-3, 4e-3)}[dt]
+    for rows, C in ((4, 50257), (3, 8200), (2, 8192)):
+        a = rng.normal(0, 2.0, (rows, C))
+        if dt == BFLOAT16:
+            held = bf16_bits_to_f32(f32_to_bf16_bits(a.astype(np.float32)))
+            dx = NDArray.from_numpy(held, BFLOAT16)
+        else:
+            held = a.astype(DT_NP[dt])
+            dx = NDArray.from_numpy(held)
+        want = oracle.log_softmax(held.astype(np.float32), 1).astype(np.float64)
+        z = ex.exec_custom("log_softmax", [dx], [NDArray.empty((rows, C), dt)], i_args=[1])[0]
+        got = z.to_float().astype(np.float64)
+        assert np.all(np.abs(got - want) <= atol + rtol * np.abs(want)), "log_softmax rows %d x %d dtype %d" % (rows, C, dt)
+        assert np.all(np.abs(np.exp(got).sum(1) - 1.0) < (5e-2 if dt != FLOAT32 else 1e-3))
+
+
 ROW_LENGTHS = [1, 2, 3, 7, 8, 31, 63, 64, 65, 127, 128, 255, 256, 257, 384, 512, 640, 767, 768, 769, 1000, 1023, 1024, 1025, 1536, 2048,
                2049, 3072, 4096, 4100, 6000, 8192, 8200, 12000]
 
