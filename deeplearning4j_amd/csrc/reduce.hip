@@ -852,9 +852,102 @@ static bool tryIndexRowsFast(hipStream_t st, const void* x, void* z, const Reduc
   return true;
 }
 
+// index reduce down the columns of a row-major matrix: the counterpart of reduce_cols (a wave reads 256 bytes of one row per
+// load, the four waves of a block take every fourth row of the block's share; a thread meets its rows in ascending order, so
+// the strict comparison keeps the first extreme, and waves, then blocks, merge with ties going to the lower row)
+template <int IK, typename T, int CPL, typename ZT>
+__global__ __launch_bounds__(256) void index_cols(CoopArgs a, const T* __restrict__ x, ZT* __restrict__ z, IdxVal<typename Conv<T>::acc>* __restrict__ partials,
+                                                  LongType pitch, LongType rowsPerSplit) {
+  using A = typename Conv<T>::acc;
+  using Raw = Vec<T, CPL>;
+  constexpr int UNR = 8;
+  __shared__ A ldsV[4][64 * CPL];
+  __shared__ int ldsI[4][64 * CPL];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const LongType col0 = ((LongType)blockIdx.x * 64 + lane) * CPL;
+  const bool live = col0 < a.outerLen;
+  const LongType r0 = (LongType)blockIdx.y * rowsPerSplit;
+  LongType r1 = r0 + rowsPerSplit;
+  if (r1 > a.innerLen) r1 = a.innerLen;
+  A bv[CPL];
+  int bi[CPL];
+#pragma unroll
+  for (int c = 0; c < CPL; c++) { bv[c] = idxStart<IK, A>(); bi[c] = 0x7fffffff; }
+  if (live) {
+    const T* p = x + col0;
+    auto take = [&](const Raw& v, LongType r) {
+#pragma unroll
+      for (int c = 0; c < CPL; c++) {
+        const A cv = idxPre<IK, A>((A)to_float(v.v[c]));
+        if (idxBetter<IK, A>(bv[c], bi[c], cv, (int)r)) { bv[c] = cv; bi[c] = (int)r; }
+      }
+    };
+    LongType r = r0 + wave;
+    for (; r + 4 * (UNR - 1) < r1; r += 4 * UNR) {
+      Raw v[UNR];
+#pragma unroll
+      for (int u = 0; u < UNR; u++) v[u] = *reinterpret_cast<const Raw*>(p + (r + 4 * u) * pitch);
+#pragma unroll
+      for (int u = 0; u < UNR; u++) take(v[u], r + 4 * u);
+    }
+    for (; r < r1; r += 4) take(*reinterpret_cast<const Raw*>(p + r * pitch), r);
+  }
+#pragma unroll
+  for (int c = 0; c < CPL; c++) { ldsV[wave][lane * CPL + c] = bv[c]; ldsI[wave][lane * CPL + c] = bi[c]; }
+  __syncthreads();
+  if (wave != 0 || !live) return;
+#pragma unroll
+  for (int c = 0; c < CPL; c++) {
+    A v = ldsV[0][lane * CPL + c];
+    int i = ldsI[0][lane * CPL + c];
+#pragma unroll
+    for (int w = 1; w < 4; w++) idxMerge<IK, A>(v, i, ldsV[w][lane * CPL + c], ldsI[w][lane * CPL + c]);
+    const LongType col = col0 + c;
+    if (a.splits == 1) {
+      const LongType zo = a.zLinear ? col : walk<LongType>(a.zOuter, col);
+      storeIndex<ZT>(z, zo, i == 0x7fffffff ? 0 : i);
+    } else {
+      partials[col * a.splits + blockIdx.y].v = v; partials[col * a.splits + blockIdx.y].i = i;
+    }
+  }
+}
+template <int IK, typename T, typename ZT>
+static bool tryIndexCols(hipStream_t st, const void* x, void* z, const ReducePlan& p, void* scratch, size_t scratchBytes) {
+  using A = typename Conv<T>::acc;
+  if (p.outer.rank != 1 || p.outer.stride[0] != 1 || p.inner.rank != 1 || p.innerLen < 8 || p.outerLen < 16 || p.innerLen >= (1LL << 31)) return false;
+  const LongType pitch = p.inner.stride[0], C = p.outerLen, R = p.innerLen;
+  if (pitch < C || C >= (1LL << 31)) return false;
+  int cpl = 1;
+  if (sizeof(T) == 2 && C % 2 == 0 && pitch % 2 == 0 && (reinterpret_cast<uintptr_t>(x) & 3) == 0) cpl = 2;
+  const LongType gx = (C + 64 * cpl - 1) / (64 * cpl);
+  LongType splits = gx >= 1024 ? 1 : (1024 + gx - 1) / gx;
+  if (splits > R / 32) splits = R / 32;
+  const LongType cap = (LongType)(scratchBytes / sizeof(IdxVal<A>)) / C;
+  if (splits > cap) splits = cap;
+  if (splits > 65535) splits = 65535;
+  if (splits < 1) splits = 1;
+  LongType rowsPerSplit = (R + splits - 1) / splits;
+  rowsPerSplit = (rowsPerSplit + 3) / 4 * 4;
+  splits = (R + rowsPerSplit - 1) / rowsPerSplit;
+  LaunchShape s{};
+  s.tpr = 256; s.splits = (int)splits; s.segLen = rowsPerSplit; s.flat = false; s.vectorOk = 0; s.peelOk = 0;
+  CoopArgs a = makeArgs(p, s, POST_ID);
+  const dim3 grid((unsigned)gx, (unsigned)splits);
+  if (cpl == 2) {
+    if constexpr (sizeof(T) == 2)
+      hipLaunchKernelGGL((index_cols<IK, T, 2, ZT>), grid, dim3(256), 0, st, a, (const T*)x, (ZT*)z, (IdxVal<A>*)scratch, pitch, rowsPerSplit);
+  } else {
+    hipLaunchKernelGGL((index_cols<IK, T, 1, ZT>), grid, dim3(256), 0, st, a, (const T*)x, (ZT*)z, (IdxVal<A>*)scratch, pitch, rowsPerSplit);
+  }
+  if (splits > 1)
+    hipLaunchKernelGGL((index_finish<IK, T, ZT>), dim3((unsigned)((p.outerLen + 255) / 256)), dim3(256), 0, st, a, (const IdxVal<A>*)scratch, (ZT*)z);
+  return true;
+}
+
 template <int IK, typename T, typename ZT>
 static void indexTyped(hipStream_t st, const void* x, void* z, const ReducePlan& p, void* scratch, size_t scratchBytes) {
   using A = typename Conv<T>::acc;
+  if (tryIndexCols<IK, T, ZT>(st, x, z, p, scratch, scratchBytes)) return;
   LaunchShape s = shapeLaunch(p, sizeof(T), x, sizeof(IdxVal<A>), scratchBytes);
   CoopArgs a = makeArgs(p, s, POST_ID);
   if (tryIndexRowsFast<IK, T, ZT>(st, x, z, p, s)) return;

@@ -354,6 +354,26 @@ def test_reductions_down_the_columns(ex, oracle, dtype, rows, cols, first, width
         assert_close(got, held.sum(0), tol, atol, "sum over the two leading dims")
 
 
+@pytest.mark.parametrize("dtype", [FLOAT32, BFLOAT16, HALF, DOUBLE])
+@pytest.mark.parametrize("rows,cols,first,width", [(6144, 512, 0, 512), (777, 1001, 0, 1001), (4100, 96, 3, 128), (9, 2048, 0, 2048), (40000, 17, 0, 17)])
+def test_index_reductions_down_the_columns(ex, oracle, dtype, rows, cols, first, width):
+    """IndexMax / IndexMin / IndexAbsoluteMax / IndexAbsoluteMin over dim 0 of a row-major matrix: heavy ties (the first row
+    with the extreme wins, whichever wave or block met it), an all-equal column, NaN never selected; dense, an odd column
+    count, and the columns first.. of a wider matrix."""
+    rng = np.random.default_rng(rows * 3 + cols + first)
+    full = rng.integers(-3, 4, (rows, width)).astype(np.float64)
+    full[:, first] = 1.0                                         # an all-equal column: row 0
+    full[rows - 1, first + 1] = 9.0                              # the extreme in the last row
+    if dtype != DOUBLE:
+        full[rows // 2, first + 2] = np.nan
+    _, dfull = _oracle_arr(oracle, full, dtype)
+    X = dfull.slice(1, first, first + cols) if width != cols else dfull
+    x = np.ascontiguousarray(full[:, first:first + cols]).astype(np.float64 if dtype == DOUBLE else np.float32)
+    for op in (0, 1, 2, 3):
+        want = oracle.index_reduce(op, x, np.zeros(cols, np.int64), [0])
+        assert np.array_equal(ex.exec_index_reduce(op, X, [0]).to_numpy(), want), (op, rows, cols)
+
+
 @pytest.mark.parametrize("rows,L,pitch", [(37, 1028, 1028), (5, 8192, 8192), (9, 5000, 5000), (33, 4096, 4352), (3, 1024, 2048)])
 def test_reductions_over_rows_at_a_constant_pitch(ex, oracle, rows, L, pitch):
     """Rows of 1024..8192 elements at a constant pitch take the one-shot kernels (all loads up front, masked tail):
