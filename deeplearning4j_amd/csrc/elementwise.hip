@@ -566,6 +566,58 @@ static void launchNd(hipStream_t s, const EwPlan& p, const T* x, const T* y, T* 
   }
 }
 
+// ---- copies that transpose: z runs along one axis, x along another ---------------------------------------------------------
+// A 64 x 64 tile goes through LDS: read along x's contiguous axis (axis A), written along z's (the last axis), both sides in
+// whole 64-element runs; the other axes are a batch walked per block.  Rows of 65 keep the transposed LDS reads conflict-free.
+struct TransposeArgs {
+  LongType nA, nB, xB, zA;          // extents of the two axes; x's stride along z's axis, z's stride along x's axis
+  int nOther;
+  LongType oShape[MAX_DEV_RANK], oX[MAX_DEV_RANK], oZ[MAX_DEV_RANK];
+  unsigned tilesA, tilesB;
+};
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_tiled(TransposeArgs a, const T* __restrict__ x, T* __restrict__ z) {
+  __shared__ T tile[64][65];
+  const unsigned tb = blockIdx.x % a.tilesB, ta = blockIdx.x / a.tilesB;
+  LongType rest = blockIdx.y, xo = 0, zo = 0;
+  for (int d = a.nOther - 1; d >= 0; d--) { const LongType q = rest / a.oShape[d], c = rest - q * a.oShape[d]; xo += c * a.oX[d]; zo += c * a.oZ[d]; rest = q; }
+  const LongType a0 = (LongType)ta * 64, b0 = (LongType)tb * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  if (a0 + tx < a.nA) {
+#pragma unroll 4
+    for (int j = ty; j < 64; j += 4)
+      if (b0 + j < a.nB) tile[j][tx] = x[xo + (a0 + tx) + (b0 + j) * a.xB];
+  }
+  __syncthreads();
+  if (b0 + tx < a.nB) {
+#pragma unroll 4
+    for (int j = ty; j < 64; j += 4)
+      if (a0 + j < a.nA) z[zo + (a0 + j) * a.zA + (b0 + tx)] = tile[tx][j];
+  }
+}
+// whether the copy described by p (operand 0: z, operand 1: x) is such a transpose; launches it if so
+template <typename T>
+static bool tryTransposeCopy(hipStream_t s, const EwPlan& p, const T* x, T* z) {
+  const int r = p.rank;
+  if (r < 2 || p.stride[0][r - 1] != 1 || p.stride[1][r - 1] == 1) return false;
+  int dA = -1;
+  for (int d = 0; d < r - 1; d++) if (p.stride[1][d] == 1 && p.shape[d] > 1) dA = d;
+  if (dA < 0 || p.shape[dA] < 16 || p.shape[r - 1] < 16) return false;
+  TransposeArgs a;
+  a.nA = p.shape[dA]; a.nB = p.shape[r - 1]; a.xB = p.stride[1][r - 1]; a.zA = p.stride[0][dA];
+  a.nOther = 0;
+  LongType batch = 1;
+  for (int d = 0; d < r - 1; d++) {
+    if (d == dA) continue;
+    a.oShape[a.nOther] = p.shape[d]; a.oX[a.nOther] = p.stride[1][d]; a.oZ[a.nOther] = p.stride[0][d]; a.nOther++;
+    batch *= p.shape[d];
+  }
+  a.tilesA = (unsigned)((a.nA + 63) / 64); a.tilesB = (unsigned)((a.nB + 63) / 64);
+  if (batch > 65535 || (LongType)a.tilesA * a.tilesB >= (1LL << 31)) return false;
+  hipLaunchKernelGGL((transpose_tiled<T>), dim3(a.tilesA * a.tilesB, (unsigned)batch), dim3(256), 0, s, a, x, z);
+  return true;
+}
+
 template <int K, typename T>
 static void unaryTyped(hipStream_t s, const EwPlan& p, const void* x, void* z) {
   const T* xt = (const T*)x;
@@ -578,6 +630,7 @@ static void unaryTyped(hipStream_t s, const EwPlan& p, const void* x, void* z) {
     else if (nt == 2) hipLaunchKernelGGL((unary_contig<Unary<K>, T, false, true>), dim3(grid), dim3(EW_BLOCK), 0, s, xt, zt, p.length);
     else hipLaunchKernelGGL((unary_contig<Unary<K>, T, false, false>), dim3(grid), dim3(EW_BLOCK), 0, s, xt, zt, p.length);
   } else {
+    if (K == U_IDENTITY && x != z && tryTransposeCopy<T>(s, p, xt, zt)) return;
     launchNd<UnaryAs2<K>, T, 1>(s, p, xt, (const T*)nullptr, zt);
   }
 }

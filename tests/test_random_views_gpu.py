@@ -294,6 +294,43 @@ def test_layer_norm_rows_of_five_to_eight_wave_passes(ex, oracle, dt, lengths):
             assert np.all(np.abs(got - want) <= atol + rtol * np.abs(want)), "layer_norm rows %d x %d dtype %d bias %d pitched %d" % (rows, C, dt, bias, pitched)
 
 
+@pytest.mark.parametrize("dt", [FLOAT32, DOUBLE, BFLOAT16, HALF, INT32])
+def test_transposing_copies(ex, dt):
+    """permute (generic/shape/permute.cpp: a strided view copied out) where the result runs along another axis than the input:
+    whole and ragged 64 x 64 tiles, batches in front of and between the two axes, an input that is itself a view, and a
+    result written into the middle of a larger array (nothing outside it may change).  Copies: exact."""
+    rng = np.random.default_rng(int(dt) + 99)
+
+    def make(shape):
+        v = rng.integers(-100, 100, shape)
+        if dt == BFLOAT16:
+            return v.astype(np.float32), NDArray.from_numpy(v.astype(np.float32), BFLOAT16)
+        a = v.astype(DT_NP[dt])
+        return a, NDArray.from_numpy(a)
+
+    def vals(arr):
+        return arr.to_float() if dt in (BFLOAT16, HALF) else arr.to_numpy()
+
+    for shape, perm in (((128, 192), (1, 0)), ((130, 67), (1, 0)), ((17, 1000), (1, 0)), ((3, 70, 5, 129), (0, 3, 2, 1)), ((4, 6, 100, 64), (0, 1, 3, 2)),
+                        ((2, 96, 3, 80), (2, 0, 3, 1)), ((500, 257), (1, 0))):
+        a, A = make(shape)
+        want = np.transpose(a, perm)
+        Z = NDArray.empty(want.shape, dt)
+        ex.exec_custom("permute", [A], [Z], i_args=list(perm))
+        assert np.array_equal(vals(Z), want.astype(vals(Z).dtype)), (shape, perm)
+    # the input a column range of a wider array, the result rows 2.. and columns 3.. of a larger one
+    a, A = make((150, 200))
+    src = A.slice(1, 8, 8 + 130)
+    want = a[:, 8:138].T
+    big_np, Big = make((140, 160))
+    dst = Big.slice(0, 2, 132).slice(1, 3, 153)
+    ex.exec_custom("permute", [src], [dst], i_args=[1, 0])
+    got = vals(Big)
+    expect = big_np.astype(got.dtype).copy()
+    expect[2:132, 3:153] = want.astype(got.dtype)
+    assert np.array_equal(got, expect)
+
+
 @pytest.mark.parametrize("dt", [FLOAT32, BFLOAT16, HALF])
 def test_softmax_over_a_vocabulary(ex, oracle, dt):
     """Rows too long for a block's registers (a vocabulary's worth of logits): an odd length, so that no row after the first
