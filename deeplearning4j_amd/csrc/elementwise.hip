@@ -415,8 +415,20 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_nd(NdArgs a, const T* __restrict_
       outer = q;
     }
     if (VEC > 1) {
-      VT vx = *reinterpret_cast<const VT*>(x + ox), vy, out;
-      if (NIN > 1) vy = *reinterpret_cast<const VT*>(y + oy);
+      // an input that repeats along the inner axis (stride 0: a value per row, a scalar) is read once and spread
+      VT vx, vy, out;
+      if (a.stride[1][a.rank - 1] == 0) {
+        const T sx = x[ox];
+#pragma unroll
+        for (int e = 0; e < VEC; e++) vx.v[e] = sx;
+      } else vx = *reinterpret_cast<const VT*>(x + ox);
+      if (NIN > 1) {
+        if (a.stride[2][a.rank - 1] == 0) {
+          const T sy = y[oy];
+#pragma unroll
+          for (int e = 0; e < VEC; e++) vy.v[e] = sy;
+        } else vy = *reinterpret_cast<const VT*>(y + oy);
+      }
 #pragma unroll
       for (int e = 0; e < VEC; e++) {
         if (NIN > 1) out.v[e] = Conv<T>::from(F::template apply<A>((A)to_float(vx.v[e]), (A)to_float(vy.v[e])));
@@ -550,9 +562,13 @@ static void launchNd(hipStream_t s, const EwPlan& p, const T* x, const T* y, T* 
     for (int o = 0; o < 3; o++) a.stride[o][d] = p.stride[o][d];
   }
   const LongType inner = p.shape[p.rank - 1];
-  bool vec = inner % V == 0 && aligned16(x) && aligned16(z) && (NIN < 2 || aligned16(y));
+  // vectors along the inner axis: the output and every input run along it with unit stride from aligned starts -- or an
+  // input repeats along it (stride 0), which needs no alignment
+  bool vec = inner % V == 0 && aligned16(z);
   for (int o = 0; o <= NIN && vec; o++) {
-    if (p.stride[o][p.rank - 1] != 1) vec = false;
+    const LongType is = p.stride[o][p.rank - 1];
+    if (o > 0 && is == 0) continue;
+    if (is != 1 || !aligned16(o == 0 ? (const void*)z : o == 1 ? (const void*)x : (const void*)y)) vec = false;
     for (int d = 0; d < p.rank - 1; d++) if (p.stride[o][d] % V != 0) vec = false;
   }
   if (vec) {
