@@ -184,6 +184,19 @@ __device__ __forceinline__ float wave_allreduce(float v) {
   v = Op::apply(v, __shfl_xor(v, 32, WAVE));
   return v;
 }
+// the same over aligned groups of G = 8, 16, 32 or 64 neighbouring lanes (several short rows per wave): the first levels of
+// the butterfly above, each of which stays inside such a group
+template <typename Op, int G>
+__device__ __forceinline__ float group_allreduce(float v) {
+  static_assert(G == 8 || G == 16 || G == 32 || G == 64, "group size");
+  v = Op::apply(v, dpp_f<0xB1>(v));
+  v = Op::apply(v, dpp_f<0x4E>(v));
+  v = Op::apply(v, dpp_f<0x141>(v));
+  if (G >= 16) v = Op::apply(v, dpp_f<0x140>(v));
+  if (G >= 32) v = Op::apply(v, __shfl_xor(v, 16, WAVE));
+  if (G >= 64) v = Op::apply(v, __shfl_xor(v, 32, WAVE));
+  return v;
+}
 template <typename Op>
 __device__ __forceinline__ double wave_allreduce(double v) {
 #pragma unroll

@@ -166,12 +166,13 @@ template <typename T> struct PadBits;   // the 16-bit / 32-bit pattern of -max(T
 template <> struct PadBits<float> { static constexpr unsigned v = 0xff7fffffu; };
 template <> struct PadBits<bf16_t> { static constexpr unsigned v = 0xff7fff7fu; };
 template <> struct PadBits<f16_t> { static constexpr unsigned v = 0xfbfffbffu; };
-template <typename T, int NV, bool NT>
+// G: lanes per row (64: a wave per row; 8, 16, 32: several short rows per wave, NV == 1)
+template <typename T, int NV, bool NT, int G = 64>
 __global__ __launch_bounds__(256) void softmax_linear(RowArgs a, const T* __restrict__ x, T* __restrict__ z, int clamp) {
   using Raw = typename RawIO<T>::raw;
   constexpr int VEC = RawIO<T>::N;
-  const int t = threadIdx.x & 63;
-  const LongType row = (LongType)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int t = threadIdx.x & (G - 1);
+  const LongType row = (LongType)blockIdx.x * (256 / G) + threadIdx.x / G;
   if (row >= a.rows) return;
   const int L = (int)a.rowLen;
   const T* xr = x + walk<LongType>(a.outerX, row);
@@ -179,7 +180,7 @@ __global__ __launch_bounds__(256) void softmax_linear(RowArgs a, const T* __rest
   int e0[NV];
 #pragma unroll
   for (int i = 0; i < NV; i++) {
-    const int e = (t + i * 64) * VEC;
+    const int e = (t + i * G) * VEC;
     e0[i] = e < L ? e : L - VEC;
     const raw_u32x4* src = reinterpret_cast<const raw_u32x4*>(xr + e0[i]);
     bits[i] = NT ? __builtin_nontemporal_load(src) : *src;
@@ -189,7 +190,7 @@ __global__ __launch_bounds__(256) void softmax_linear(RowArgs a, const T* __rest
   const float NEG = -r_tmax<float>();
 #pragma unroll
   for (int i = 0; i < NV; i++) {
-    const unsigned keep = (t + i * 64) * VEC < L ? 0xffffffffu : 0u;
+    const unsigned keep = (t + i * G) * VEC < L ? 0xffffffffu : 0u;
     const raw_u32x4 b = (bits[i] & keep) | (raw_u32x4)(PadBits<T>::v & ~keep);
     RawIO<T>::unpack(__builtin_bit_cast(Raw, b), &vals[i * VEC]);
   }
@@ -204,7 +205,7 @@ __global__ __launch_bounds__(256) void softmax_linear(RowArgs a, const T* __rest
   float sum = 0.f;
   const float L2E = 1.44269502162933349609375f;
   if (__builtin_amdgcn_ballot_w64(probe != probe) == 0) {
-    mx = wave_allreduce<MaxOp>(mx);
+    mx = group_allreduce<MaxOp, G>(mx);
 #pragma unroll
     for (int i = 0; i < NV * VEC; i++) {
       const float r = __builtin_amdgcn_exp2f((vals[i] - mx) * L2E);
@@ -215,25 +216,25 @@ __global__ __launch_bounds__(256) void softmax_linear(RowArgs a, const T* __rest
     mx = NEG;
 #pragma unroll
     for (int i = 0; i < NV * VEC; i++) mx = softmax_maxstep<float>(mx, vals[i], clamp);
-    mx = wave_allreduce<MaxOp>(mx);
+    mx = group_allreduce<MaxOp, G>(mx);
     if (clamp && mx == NEG) mx = 0.f;
 #pragma unroll
     for (int i = 0; i < NV; i++)
 #pragma unroll
       for (int e = 0; e < VEC; e++) {
         float r = 0.f;
-        if ((t + i * 64) * VEC < L) r = softmax_term(vals[i * VEC + e], mx, clamp);
+        if ((t + i * G) * VEC < L) r = softmax_term(vals[i * VEC + e], mx, clamp);
         vals[i * VEC + e] = r;
         sum += r;
       }
   }
-  sum = wave_allreduce<SumOp>(sum);
+  sum = group_allreduce<SumOp, G>(sum);
   if (clamp) sum = sum > 1e-6f ? sum : 1e-6f;
   const float inv = 1.f / sum;
   T* zr = z + walk<LongType>(a.outerZ, row);
 #pragma unroll
   for (int i = 0; i < NV; i++) {
-    if ((t + i * 64) * VEC >= L) continue;
+    if ((t + i * G) * VEC >= L) continue;
 #pragma unroll
     for (int e = 0; e < VEC; e++) vals[i * VEC + e] *= inv;
     Raw* dst = reinterpret_cast<Raw*>(zr + e0[i]);
@@ -379,6 +380,17 @@ template <typename T>
 static void softmaxLinear(hipStream_t s, const RowArgs& a, const T* x, T* z, int clamp, int nt) {
   constexpr int V = 16 / sizeof(T);
   const int passes = (int)((a.rowLen / V + 63) / 64);
+  // short rows: 8, 16 or 32 lanes per row, so that a wave's loads cover several rows instead of leaving most lanes idle
+  // (bf16 rows of 64: 8 of 64 lanes had a vector)
+  const LongType lanes = a.rowLen / V;
+  if (lanes <= 32) {
+#define SG(G) do { const dim3 gg((unsigned)((a.rows + 256 / G - 1) / (256 / G))); \
+                   if (nt) hipLaunchKernelGGL((softmax_linear<T, 1, true, G>), gg, dim3(256), 0, s, a, x, z, clamp); \
+                   else hipLaunchKernelGGL((softmax_linear<T, 1, false, G>), gg, dim3(256), 0, s, a, x, z, clamp); } while (0)
+    if (lanes <= 8) SG(8); else if (lanes <= 16) SG(16); else SG(32);
+#undef SG
+    return;
+  }
   const dim3 grid((unsigned)((a.rows + 3) / 4));
 #define SL(NV) do { if (nt) hipLaunchKernelGGL((softmax_linear<T, NV, true>), grid, dim3(256), 0, s, a, x, z, clamp); \
                     else hipLaunchKernelGGL((softmax_linear<T, NV, false>), grid, dim3(256), 0, s, a, x, z, clamp); } while (0)
