@@ -8,7 +8,7 @@ namespace nd4jhip {
 // vals: the row's elements, lane t holding elements (t + 64 i) * VEC .. + VEC - 1 of pass i; keep[i] = 0 for a pass whose
 // vector lies beyond the row (such lanes hold a re-read of the last vector).  On return vals holds
 // (x - mean) / sqrt(var + eps) * gain (+ bias), population variance.
-template <typename T, int NV, bool HAS_BIAS>
+template <typename T, int NV, bool HAS_BIAS, int G = 64>
 __device__ __forceinline__ void ln_wave_row(typename Conv<T>::acc (&vals)[NV * RawIO<T>::N], const typename RawIO<T>::raw (&gv)[NV],
                                             const typename RawIO<T>::raw (&bv)[NV], const typename Conv<T>::acc (&keep)[NV], int L, float eps) {
   using A = typename Conv<T>::acc;
@@ -21,7 +21,7 @@ __device__ __forceinline__ void ln_wave_row(typename Conv<T>::acc (&vals)[NV * R
     for (int e = 0; e < VEC; e++) part += vals[i * VEC + e];
     sum += part * keep[i];
   }
-  sum = wave_allreduce<SumOp>(sum);
+  if constexpr (G == 64) sum = wave_allreduce<SumOp>(sum); else sum = group_allreduce<SumOp, G>(sum);   // G < 64: a row per G lanes
   const A mean = sum / (A)L;
   A sq = (A)0;
 #pragma unroll
@@ -31,7 +31,7 @@ __device__ __forceinline__ void ln_wave_row(typename Conv<T>::acc (&vals)[NV * R
     for (int e = 0; e < VEC; e++) { const A d = vals[i * VEC + e] - mean; vals[i * VEC + e] = d; part += d * d; }
     sq += part * keep[i];
   }
-  sq = wave_allreduce<SumOp>(sq);
+  if constexpr (G == 64) sq = wave_allreduce<SumOp>(sq); else sq = group_allreduce<SumOp, G>(sq);
   const A var = L > 1 ? sq / (A)L : (A)0;
   const A rstd = (A)1 / (sizeof(A) == 8 ? (A)sqrt((double)(var + (A)eps)) : (A)sqrtf((float)(var + (A)eps)));
 #pragma unroll

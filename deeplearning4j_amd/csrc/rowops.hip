@@ -611,23 +611,24 @@ __global__ __launch_bounds__(256) void layernorm_rows(RowArgs a, const T* __rest
 // end re-read the last vector and are masked out of the sums), so the three latencies overlap instead of queueing.
 // ADD: the row normalised is x + addend, rounded through the storage type and also written to sumOut -- a pairwise Add
 // followed by layer_norm on its result, in one pass (sumOut may be x itself: a wave reads a row before it writes it).
-template <typename T, int NV, bool HAS_BIAS, int RPW, bool ADD = false>
+// G: lanes per row (64: a wave per row; 8, 16, 32 with NV == 1 and RPW == 1: several short rows per wave)
+template <typename T, int NV, bool HAS_BIAS, int RPW, bool ADD = false, int G = 64>
 __global__ __launch_bounds__(256) void layernorm_linear(const T* __restrict__ x, const T* __restrict__ gain, const T* __restrict__ bias,
                                                         T* __restrict__ z, LongType rows, int L, LongType xPitch, LongType zPitch, float eps,
                                                         const T* addend = nullptr, LongType aPitch = 0, T* sumOut = nullptr, LongType sPitch = 0) {
   using A = typename Conv<T>::acc;
   using Raw = typename RawIO<T>::raw;
   constexpr int VEC = RawIO<T>::N;
-  const int t = threadIdx.x & 63;
+  const int t = threadIdx.x & (G - 1);
   // a wave owns RPW consecutive rows: gain and bias are fetched once for all of them
-  const LongType row0 = ((LongType)blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW;
+  const LongType row0 = ((LongType)blockIdx.x * (256 / G) + threadIdx.x / G) * RPW;
   if (row0 >= rows) return;
   int e0[NV];
   A keep[NV];
   Raw xv[RPW][NV], gv[NV], bv[NV], av[ADD ? RPW : 1][ADD ? NV : 1];
 #pragma unroll
   for (int i = 0; i < NV; i++) {
-    const int e = (t + i * 64) * VEC;
+    const int e = (t + i * G) * VEC;
     keep[i] = e < L ? (A)1 : (A)0;
     e0[i] = e < L ? e : L - VEC;
   }
@@ -676,7 +677,7 @@ __global__ __launch_bounds__(256) void layernorm_linear(const T* __restrict__ x,
         RawIO<T>::unpack(packed, &vals[0][i * VEC]);
       }
     }
-    ln_wave_row<T, NV, HAS_BIAS>(vals[0], gv, bv, keep, L, eps);
+    ln_wave_row<T, NV, HAS_BIAS, G>(vals[0], gv, bv, keep, L, eps);
     T* zr = z + row0 * zPitch;
 #pragma unroll
     for (int i = 0; i < NV; i++)
@@ -857,6 +858,18 @@ static bool layerNormTyped(hipStream_t s, const void* x, const void* gain, const
       const bool pair = p.rows >= 4096 && L <= 4 * perWave;
 #define LNL(NV) do { if (bt) hipLaunchKernelGGL((layernorm_linear<T, NV, true, 1>), dim3(gw), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); \
                      else hipLaunchKernelGGL((layernorm_linear<T, NV, false, 1>), dim3(gw), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); } while (0)
+      // short rows: 8, 16 or 32 lanes per row
+      if constexpr (sizeof(T) <= 4) {
+        const LongType lanes = L / V;
+        if (lanes <= 32) {
+#define LNG(G) do { const unsigned gg = (unsigned)((p.rows + 256 / G - 1) / (256 / G)); \
+                    if (bt) hipLaunchKernelGGL((layernorm_linear<T, 1, true, 1, false, G>), dim3(gg), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); \
+                    else hipLaunchKernelGGL((layernorm_linear<T, 1, false, 1, false, G>), dim3(gg), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); } while (0)
+          if (lanes <= 8) LNG(8); else if (lanes <= 16) LNG(16); else LNG(32);
+#undef LNG
+          return true;
+        }
+      }
       if (pair) {
         // one pair per wave while the grid allows it (fewer, longer-running waves measured slower: bf16 [16384, 768] 12.7 us
         // per launch with one pair per wave, 13.5 with four, 14.1 with eight)
