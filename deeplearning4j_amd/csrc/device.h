@@ -197,6 +197,12 @@ __device__ __forceinline__ float group_allreduce(float v) {
   if (G >= 64) v = Op::apply(v, __shfl_xor(v, 32, WAVE));
   return v;
 }
+template <typename Op, int G>
+__device__ __forceinline__ double group_allreduce(double v) {
+#pragma unroll
+  for (int m = 1; m < G; m <<= 1) v = Op::apply(v, __shfl_xor(v, m, WAVE));
+  return v;
+}
 template <typename Op>
 __device__ __forceinline__ double wave_allreduce(double v) {
 #pragma unroll

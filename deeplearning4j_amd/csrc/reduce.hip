@@ -123,6 +123,7 @@ __global__ __launch_bounds__(256) void reduce_coop(CoopArgs a, const T* __restri
     }
   }
   if (TPR == 64) acc = wave_allreduce<Op>(acc);
+  else if (TPR < 64) acc = group_allreduce<Op, TPR < 64 ? TPR : 8>(acc);   // short rows: 8, 16 or 32 lanes each
   else acc = block_allreduce<Op, 4, A>(acc, lds);
   if (live && t == 0) {
     if (a.splits == 1) {
@@ -195,6 +196,11 @@ static LaunchShape shapeLaunch(const ReducePlan& p, size_t elemSize, const void*
   const bool unitInner = p.inner.rank == 1 && p.inner.stride[0] == 1;
   s.flat = !unitInner && p.outerLen >= 4096;
   s.tpr = p.innerLen >= 2048 ? 256 : 64;
+  // short unit-stride rows: 8, 16 or 32 lanes per row (one 16-byte vector per lane), several rows per wave
+  if (unitInner && p.innerLen * (LongType)elemSize <= 32 * 16) {
+    const LongType lanes = (p.innerLen * (LongType)elemSize + 15) / 16;
+    s.tpr = lanes <= 8 ? 8 : lanes <= 16 ? 16 : 32;
+  }
   s.splits = 1;
   s.segLen = p.innerLen;
   // few outputs and a long run: cut the run so that the whole chip participates
@@ -392,7 +398,11 @@ static void reduceTyped(hipStream_t st, const void* x, void* z, const ReducePlan
   }
   const LongType units = p.outerLen * s.splits;
   const int vec = s.vectorOk ? 1 : (s.peelOk ? 2 : 0);
-  if (s.tpr == 64) {
+  if (s.tpr < 64) {
+#define RS(G) hipLaunchKernelGGL((reduce_coop<Op, PRE, T, G>), dim3((unsigned)((units + 256 / G - 1) / (256 / G))), dim3(256), 0, st, a, (const T*)x, (T*)z, (A*)scratch, vec)
+    if (s.tpr == 8) RS(8); else if (s.tpr == 16) RS(16); else RS(32);
+#undef RS
+  } else if (s.tpr == 64) {
     hipLaunchKernelGGL((reduce_coop<Op, PRE, T, 64>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, st, a, (const T*)x, (T*)z, (A*)scratch, vec);
   } else {
     hipLaunchKernelGGL((reduce_coop<Op, PRE, T, 256>), dim3((unsigned)units), dim3(256), 0, st, a, (const T*)x, (T*)z, (A*)scratch, vec);
@@ -677,6 +687,19 @@ __device__ __forceinline__ void wave_idx_allreduce(float& v, int& i) {
   idxMerge<IK, float>(v, i, __shfl_xor(v, 16, WAVE), __shfl_xor(i, 16, WAVE));
   idxMerge<IK, float>(v, i, __shfl_xor(v, 32, WAVE), __shfl_xor(i, 32, WAVE));
 }
+template <int IK, int G>
+__device__ __forceinline__ void group_idx_allreduce(float& v, int& i) {   // aligned groups of G = 8, 16, 32 lanes
+  idxMerge<IK, float>(v, i, dpp_f<0xB1>(v), dpp_i<0xB1>(i));
+  idxMerge<IK, float>(v, i, dpp_f<0x4E>(v), dpp_i<0x4E>(i));
+  idxMerge<IK, float>(v, i, dpp_f<0x141>(v), dpp_i<0x141>(i));
+  if (G >= 16) idxMerge<IK, float>(v, i, dpp_f<0x140>(v), dpp_i<0x140>(i));
+  if (G >= 32) idxMerge<IK, float>(v, i, __shfl_xor(v, 16, WAVE), __shfl_xor(i, 16, WAVE));
+}
+template <int IK, int G>
+__device__ __forceinline__ void group_idx_allreduce(double& v, int& i) {
+#pragma unroll
+  for (int m = 1; m < G; m <<= 1) idxMerge<IK, double>(v, i, __shfl_xor(v, m, WAVE), __shfl_xor(i, m, WAVE));
+}
 template <int IK>
 __device__ __forceinline__ void wave_idx_allreduce(double& v, int& i) {
 #pragma unroll
@@ -747,7 +770,8 @@ __global__ __launch_bounds__(BLOCK) void index_coop(CoopArgs a, const T* __restr
       for (LongType q = j0 + t; q < j1; q += TPR) { A c = idxPre<IK, A>((A)to_float(x[base + walk<LongType>(a.inner, q)])); if (idxBetter<IK, A>(bv, bi, c, (int)q)) { bv = c; bi = (int)q; } }
     }
   }
-  wave_idx_allreduce<IK>(bv, bi);
+  if (TPR < 64) group_idx_allreduce<IK, TPR < 64 ? TPR : 8>(bv, bi);   // short rows: 8, 16 or 32 lanes each
+  else wave_idx_allreduce<IK>(bv, bi);
   if (TPR > 64) {
     static_assert(TPR <= 64 || TPR == BLOCK, "a row takes one wave or the whole block");
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -967,7 +991,11 @@ static void indexTyped(hipStream_t st, const void* x, void* z, const ReducePlan&
     return;
   }
   const LongType units = p.outerLen * s.splits;
-  if (s.tpr == 64)
+  if (s.tpr < 64) {
+#define IS(G) hipLaunchKernelGGL((index_coop<IK, T, G, ZT>), dim3((unsigned)((units + 256 / G - 1) / (256 / G))), dim3(256), 0, st, a, (const T*)x, (ZT*)z, (IdxVal<A>*)scratch, vec)
+    if (s.tpr == 8) IS(8); else if (s.tpr == 16) IS(16); else IS(32);
+#undef IS
+  } else if (s.tpr == 64)
     hipLaunchKernelGGL((index_coop<IK, T, 64, ZT>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, st, a, (const T*)x, (ZT*)z, (IdxVal<A>*)scratch, vec);
   else
     hipLaunchKernelGGL((index_coop<IK, T, 256, ZT>), dim3((unsigned)units), dim3(256), 0, st, a, (const T*)x, (ZT*)z, (IdxVal<A>*)scratch, vec);
