@@ -681,8 +681,45 @@ static bool tailContig(hipStream_t s, int k, DataType dt, const void* x, const v
   }
 }
 
+// ---- dense casts between fp32 and the 16-bit types (the assign loop between two types) -------------------------------------
+// eight elements per thread: the wider side moves as two 16-byte vectors, the narrower as one; the tail one by one
+template <typename TI, typename TO>
+__global__ __launch_bounds__(EW_BLOCK) void cast_contig(const TI* __restrict__ x, TO* __restrict__ z, LongType n) {
+  const LongType i = ((LongType)blockIdx.x * EW_BLOCK + threadIdx.x) * 8;
+  if (i + 8 <= n) {
+    Vec<TI, 8> v = *reinterpret_cast<const Vec<TI, 8>*>(x + i);
+    Vec<TO, 8> o;
+#pragma unroll
+    for (int e = 0; e < 8; e++) o.v[e] = Conv<TO>::from(to_float(v.v[e]));
+    *reinterpret_cast<Vec<TO, 8>*>(z + i) = o;
+  } else {
+    for (LongType j = i; j < n; j++) z[j] = Conv<TO>::from(to_float(x[j]));
+  }
+}
+template <typename TI>
+static bool castFrom(hipStream_t s, DataType zdt, const void* x, void* z, LongType n) {
+  const unsigned grid = (unsigned)((n / 8 + EW_BLOCK) / EW_BLOCK);
+  switch (zdt) {
+    case FLOAT32: if constexpr (!std::is_same<TI, float>::value) { hipLaunchKernelGGL((cast_contig<TI, float>), dim3(grid), dim3(EW_BLOCK), 0, s, (const TI*)x, (float*)z, n); return true; } break;
+    case HALF: if constexpr (!std::is_same<TI, f16_t>::value) { hipLaunchKernelGGL((cast_contig<TI, f16_t>), dim3(grid), dim3(EW_BLOCK), 0, s, (const TI*)x, (f16_t*)z, n); return true; } break;
+    case BFLOAT16: if constexpr (!std::is_same<TI, bf16_t>::value) { hipLaunchKernelGGL((cast_contig<TI, bf16_t>), dim3(grid), dim3(EW_BLOCK), 0, s, (const TI*)x, (bf16_t*)z, n); return true; } break;
+    default: break;
+  }
+  return false;
+}
+static bool tryCastContig(hipStream_t s, DataType xdt, DataType zdt, const void* x, void* z, const EwPlan& p) {
+  if (xdt == zdt || !p.sameShape || !p.contiguous || ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(z)) & 31) != 0 || p.length >= (1LL << 40)) return false;
+  switch (xdt) {
+    case FLOAT32: return castFrom<float>(s, zdt, x, z, p.length);
+    case HALF: return castFrom<f16_t>(s, zdt, x, z, p.length);
+    case BFLOAT16: return castFrom<bf16_t>(s, zdt, x, z, p.length);
+    default: return false;
+  }
+}
+
 void launchUnary(hipStream_t s, UnaryKind k, DataType xdt, DataType zdt, const void* x, void* z, const EwPlan& p) {
   if (p.length == 0) return;
+  if (k == U_IDENTITY && tryCastContig(s, xdt, zdt, x, z, p)) { HIP_CHECK(hipGetLastError()); return; }
   if (isIntLike(xdt) && isIntLike(zdt)) return launchIntElementwise(s, k, false, xdt, xdt, zdt, x, nullptr, z, p, 0, false);
   if (k >= U_TAIL_FIRST && k < U_TAIL_END) {
     if (!(p.sameShape && xdt == zdt && p.contiguous && aligned16(x) && aligned16(z) && tailContig<1>(s, k, xdt, x, x, z, p.length)))
@@ -829,6 +866,38 @@ __global__ __launch_bounds__(EW_BLOCK) void scalar_nd(NdArgs a, const T* __restr
     z[oz] = Conv<T>::from(F::template apply<A>((A)to_float(x[ox]), sc));
   }
 }
+// 16 bytes per thread along unit-stride inner runs; a dense array is one run whose last few elements go one by one
+template <typename F, typename T, typename I>
+__global__ __launch_bounds__(EW_BLOCK) void scalar_nd_vec(NdArgs a, const T* __restrict__ x, T* __restrict__ z,
+                                                          typename Conv<T>::acc sc, I chunksPerRow, I totalChunks, LongType n) {
+  using A = typename Conv<T>::acc;
+  constexpr int V = 16 / sizeof(T);
+  using VT = Vec<T, V>;
+  const I step = (I)gridDim.x * EW_BLOCK;
+  for (I c = (I)blockIdx.x * EW_BLOCK + threadIdx.x; c < totalChunks; c += step) {
+    I outer = c / chunksPerRow;
+    const LongType inner = (LongType)(c - outer * chunksPerRow) * V;
+    LongType oz = inner, ox = inner;
+#pragma unroll 1
+    for (int d = a.rank - 2; d >= 0; d--) {
+      const I dim = (I)a.shape[d];
+      const I q = outer / dim;
+      const LongType cd = (LongType)(outer - q * dim);
+      oz += cd * a.stride[0][d]; ox += cd * a.stride[1][d];
+      outer = q;
+    }
+    const VT vx = *reinterpret_cast<const VT*>(x + ox);
+    VT out;
+#pragma unroll
+    for (int e = 0; e < V; e++) out.v[e] = Conv<T>::from(F::template apply<A>((A)to_float(vx.v[e]), sc));
+    *reinterpret_cast<VT*>(z + oz) = out;
+  }
+  // rank 1 only: what is left after the last whole vector
+  if (blockIdx.x == 0) {
+    const LongType i = (LongType)totalChunks * V + threadIdx.x;
+    if (a.rank == 1 && i < n) z[i] = Conv<T>::from(F::template apply<A>((A)to_float(x[i]), sc));
+  }
+}
 template <int K, typename T>
 static void scalarTyped(hipStream_t s, const void* x, double sc, void* z, const EwPlan& p) {
   NdArgs a;
@@ -836,6 +905,17 @@ static void scalarTyped(hipStream_t s, const void* x, double sc, void* z, const 
   for (int d = 0; d < p.rank; d++) { a.shape[d] = p.shape[d]; for (int o = 0; o < 3; o++) a.stride[o][d] = p.stride[o][d]; }
   using A = typename Conv<T>::acc;
   A scv = (A)sc;
+  constexpr int V = 16 / sizeof(T);
+  const LongType inner = p.shape[p.rank - 1];
+  bool vec = aligned16(x) && aligned16(z) && p.stride[0][p.rank - 1] == 1 && p.stride[1][p.rank - 1] == 1 &&
+             (p.rank == 1 ? inner >= V : inner % V == 0);
+  for (int d = 0; d < p.rank - 1 && vec; d++) if (p.stride[0][d] % V != 0 || p.stride[1][d] % V != 0) vec = false;
+  if (vec) {
+    const LongType cpr = inner / V, total = p.rank == 1 ? cpr : p.length / V;
+    if (p.index32) hipLaunchKernelGGL((scalar_nd_vec<Pairwise<K>, T, unsigned>), dim3(gridFor(total, EW_BLOCK)), dim3(EW_BLOCK), 0, s, a, (const T*)x, (T*)z, scv, (unsigned)cpr, (unsigned)total, p.length);
+    else hipLaunchKernelGGL((scalar_nd_vec<Pairwise<K>, T, unsigned long long>), dim3(gridFor(total, EW_BLOCK)), dim3(EW_BLOCK), 0, s, a, (const T*)x, (T*)z, scv, (unsigned long long)cpr, (unsigned long long)total, p.length);
+    return;
+  }
   hipLaunchKernelGGL((scalar_nd<Pairwise<K>, T>), dim3(gridFor(p.length, EW_BLOCK)), dim3(EW_BLOCK), 0, s, a, (const T*)x, (T*)z, scv, p.length);
 }
 template <int K>
@@ -905,6 +985,17 @@ void launchGatherRows(hipStream_t s, DataType dt, DataType idxDt, const void* ta
 #define GATHER(T)                                                                                                         \
   if (idxDt == INT32) hipLaunchKernelGGL((gather_rows<T, int>), g, b, 0, s, (const T*)table, (const int*)idx, (T*)z, nIdx, rowLen, tableRows); \
   else hipLaunchKernelGGL((gather_rows<T, LongType>), g, b, 0, s, (const T*)table, (const LongType*)idx, (T*)z, nIdx, rowLen, tableRows);
+  // rows that are whole 16-byte units in aligned arrays move as such
+  using U16 = Vec<unsigned, 4>;
+  const LongType es = (LongType)sizeOf(dt);
+  if ((rowLen * es) % 16 == 0 && aligned16(table) && aligned16(z)) {
+    const LongType units = rowLen * es / 16;
+    g = dim3(gridFor(nIdx * units, EW_BLOCK));
+    rowLen = units;
+    GATHER(U16)
+    HIP_CHECK(hipGetLastError());
+    return;
+  }
   switch (sizeOf(dt)) {
     case 2: GATHER(unsigned short) break;
     case 4: GATHER(unsigned) break;

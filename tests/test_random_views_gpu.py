@@ -487,3 +487,77 @@ def test_attention_on_random_shapes_masks_and_layouts(ex, oracle):
         truth = np.einsum("bqk,bkd->bqd", p64 / p64.sum(-1, keepdims=True), v64)
         assert np.abs(got - truth).max() <= 1.25 * np.abs(want - truth).max() + tol / 4, tag + ": %g from the exact result, the composition %g" % (
             float(np.abs(got - truth).max()), float(np.abs(want - truth).max()))
+
+
+@pytest.mark.gpu
+def test_dense_casts_between_fp32_and_the_16_bit_types(ex):
+    """cast (generic/datatypes/cast.cpp -> NDArray::assign between two types, helpers/Loops.h: a static_cast per element, through
+    float for the 16-bit types): lengths that are whole vectors of eight, lengths with a rest, and fewer than eight; fp32 -> f16
+    and f16 <-> f16-representable values against numpy's round-to-nearest-even, fp32 -> bf16 against the bit-level rounding,
+    the widening casts exact."""
+    rng = np.random.default_rng(515)
+    for n in (1, 5, 8, 64, 1000, 4096 * 3 + 7, 1 << 18):
+        v = rng.normal(0, 30, n).astype(np.float32)
+        v[:: max(1, n // 7)] = 0.0
+        A = NDArray.from_numpy(v)
+        h = ex.exec_custom("cast", [A], d_args=[HALF])[0]
+        assert np.array_equal(h.to_numpy(), v.astype(np.float16)), n
+        b = ex.exec_custom("cast", [A], d_args=[BFLOAT16])[0]
+        assert np.array_equal(b.to_numpy(), f32_to_bf16_bits(v)), n
+        assert np.array_equal(ex.exec_custom("cast", [h], d_args=[FLOAT32])[0].to_numpy(), v.astype(np.float16).astype(np.float32)), n
+        assert np.array_equal(ex.exec_custom("cast", [b], d_args=[FLOAT32])[0].to_numpy(), bf16_bits_to_f32(f32_to_bf16_bits(v))), n
+        # 16-bit to 16-bit goes through float: the bf16 values are exact in fp32, then rounded to f16
+        hb = ex.exec_custom("cast", [b], d_args=[HALF])[0]
+        assert np.array_equal(hb.to_numpy(), bf16_bits_to_f32(f32_to_bf16_bits(v)).astype(np.float16)), n
+        bh = ex.exec_custom("cast", [h], d_args=[BFLOAT16])[0]
+        assert np.array_equal(bh.to_numpy(), f32_to_bf16_bits(v.astype(np.float16).astype(np.float32))), n
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [FLOAT32, HALF, BFLOAT16, DOUBLE])
+def test_scalar_ops_on_dense_arrays_and_on_column_ranges(ex, dt):
+    """execScalar (legacy_ops.h SCALAR_OPS, loops/cpu/scalar.hpp): the same values laid out three ways -- a dense array (16 bytes
+    per thread, the rest one by one), a column range of a wider array whose rows start on 16-byte boundaries, and a range that
+    starts one element off (element by element) -- must give the same bits; fp32 and double also equal numpy's.  Nothing
+    outside a range written to may change."""
+    rng = np.random.default_rng(616 + int(dt))
+    for rows, cols in ((1, 5), (1, 1003), (37, 64), (200, 136), (3, 8)):
+        vals = rng.normal(0, 3, (rows, cols)).astype(np.float32)
+        wide = rng.normal(0, 3, (rows, cols + 24)).astype(np.float32)
+        wide[:, 8:8 + cols] = vals
+        wide1 = rng.normal(0, 3, (rows, cols + 24)).astype(np.float32)
+        wide1[:, 9:9 + cols] = vals
+        for op, f in ((Scalar.Multiply, lambda a: a * a.dtype.type(1.5)), (Scalar.Add, lambda a: a + a.dtype.type(0.25)),
+                      (Scalar.ReverseSubtract, lambda a: a.dtype.type(2.0) - a)):
+            D = NDArray.from_numpy(vals, dt)
+            W = NDArray.from_numpy(wide, dt)
+            W1 = NDArray.from_numpy(wide1, dt)
+            zd = ex.exec_scalar(op, D, 1.5 if op == Scalar.Multiply else 0.25 if op == Scalar.Add else 2.0)
+            sc = 1.5 if op == Scalar.Multiply else 0.25 if op == Scalar.Add else 2.0
+            before, before1 = W.to_numpy().copy(), W1.to_numpy().copy()
+            ex.exec_scalar(op, W.slice(1, 8, 8 + cols), sc, z=W.slice(1, 8, 8 + cols))
+            ex.exec_scalar(op, W1.slice(1, 9, 9 + cols), sc, z=W1.slice(1, 9, 9 + cols))
+            got = zd.to_numpy()
+            after, after1 = W.to_numpy(), W1.to_numpy()
+            assert np.array_equal(after[:, 8:8 + cols], got), (rows, cols, op)
+            assert np.array_equal(after1[:, 9:9 + cols], got), (rows, cols, op)
+            before[:, 8:8 + cols] = got
+            before1[:, 9:9 + cols] = got
+            assert np.array_equal(after, before) and np.array_equal(after1, before1), (rows, cols, op)
+            if dt in (FLOAT32, DOUBLE):
+                assert np.array_equal(got, f(D.to_numpy())), (rows, cols, op)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [FLOAT32, BFLOAT16, DOUBLE])
+def test_gather_rows_of_whole_and_ragged_16_byte_units(ex, dt):
+    """gather along axis 0 (generic/transforms/gather.cpp, helpers/cpu/gather.cpp: row idx[i] of the table becomes row i): rows
+    that are whole 16-byte units move as such, others element by element; negative ids count from the end.  Copies: exact."""
+    rng = np.random.default_rng(717 + int(dt))
+    for rows, cols, n in ((50, 8, 33), (50, 12, 33), (1000, 768, 257), (7, 1, 20), (64, 100, 5)):
+        t = rng.integers(-100, 100, (rows, cols)).astype(np.float32)
+        T = NDArray.from_numpy(t, dt)
+        for idt in (np.int32, np.int64):
+            idx = rng.integers(-rows, rows, n).astype(idt)
+            g = ex.exec_custom("gather", [T, NDArray.from_numpy(idx)], i_args=[0])[0]
+            assert np.array_equal(g.to_numpy(), T.to_numpy()[idx]), (rows, cols, n, idt)
