@@ -164,6 +164,85 @@ def mfma_entry(flops, ev_ms, dtype, label=""):
             "traffic": traffic_of(label)}
 
 
+def clock_study(ex, L):
+    """The 4096^3 product under a sampled clock.  The published matrix peak assumes the top shader clock; under a sustained
+    matrix load the package power limit decides the clock, and the power depends on the operand VALUES (bits that toggle in the
+    multipliers), not only on the instruction stream.  Same kernel, same launch count per case; what changes is the data."""
+    import subprocess
+    import threading
+    from deeplearning4j_amd.ndarray import BFLOAT16, FLOAT32, HALF, NDArray
+    n = 4096
+    rng = np.random.default_rng(2002)
+    base_a = rng.normal(0, 1 / math.sqrt(n), (n, n)).astype(np.float32)
+    base_b = rng.normal(0, 1 / math.sqrt(n), (n, n)).astype(np.float32)
+    data = {"N(0,1/sqrt(K)) (the BASELINE operands)": (base_a, base_b), "all zeros": (np.zeros_like(base_a), np.zeros_like(base_b)),
+            "all ones / 64": (np.full_like(base_a, 1 / 64), np.full_like(base_b, 1 / 64))}
+    samples, stop = [], [False]
+
+    def sampler():
+        while not stop[0]:
+            try:
+                out = subprocess.run(["/opt/rocm/bin/rocm-smi", "--showpower", "--showclocks", "--json"], capture_output=True, text=True, timeout=10).stdout
+                samples.append((time.perf_counter(), out))
+            except Exception as exc:   # the tool is not there: the timings still stand
+                samples.append((time.perf_counter(), "ERR %r" % (exc,)))
+            time.sleep(0.25)
+
+    def digits(v):
+        m = "".join(ch for ch in str(v) if ch.isdigit() or ch == ".")
+        return float(m) if m else None
+
+    cases, first_sample = [], []
+    for dt, dtn, launches in ((BFLOAT16, "bf16", 12000), (HALF, "f16", 12000), (FLOAT32, "f32", 1500)):
+        for label, (a, b) in data.items():
+            if dt == HALF:
+                A, B = NDArray.from_numpy(a.astype(np.float16), dt), NDArray.from_numpy(b.astype(np.float16), dt)
+            else:
+                A, B = NDArray.from_numpy(a, dt), NDArray.from_numpy(b, dt)
+            Z = NDArray.empty((n, n), dt)
+            A.sync_to_device(); B.sync_to_device()
+            fn = ex.bind_custom("matmul", [A, B], [Z])
+            settle(L, fn, 0.3)
+            del samples[:]
+            stop[0] = False
+            th = threading.Thread(target=sampler)
+            th.start()
+            t_start = time.perf_counter()
+            per_launch = []
+            for _ in range(3):
+                _, e = timed(ex, L, fn, launches, 0, settled=False)
+                per_launch.append(e * 1e3)
+            t_end = time.perf_counter()
+            stop[0] = True
+            th.join()
+            sclk, power = [], []
+            for ts, out in samples:
+                if not (t_start + 0.3 <= ts <= t_end):
+                    continue
+                try:
+                    card = json.loads(out)
+                    card = card[sorted(card.keys())[0]]
+                    if not first_sample:
+                        first_sample.append(card)
+                    for k, v in card.items():
+                        kl = k.lower()
+                        if "sclk" in kl and "clock speed" in kl:
+                            sclk.append(digits(str(v).split("(")[-1]))
+                        elif "power" in kl and ("socket" in kl or "average" in kl or "package" in kl):
+                            power.append(digits(v))
+                except Exception:
+                    pass
+            us = sorted(per_launch)[1]
+            cases.append({"dtype": dtn, "operands": label, "kernel": L.nd4jhipLastGemmKernel().decode(), "us_per_launch": [round(v, 2) for v in per_launch],
+                          "tflops": round(2.0 * n ** 3 / (us * 1e-6) / 1e12, 1),
+                          "sclk_mhz": {"samples": len(sclk), "min": min(sclk) if sclk else None, "median": sorted(sclk)[len(sclk) // 2] if sclk else None, "max": max(sclk) if sclk else None},
+                          "power_w": {"samples": len(power), "median": sorted(power)[len(power) // 2] if power else None, "max": max(power) if power else None}})
+            print("[clock-study] %s" % json.dumps(cases[-1]), file=sys.stderr, flush=True)
+            del A, B, Z, fn
+    print(json.dumps({"clock_study": cases, "one_raw_sample": first_sample[:1], "launches_per_case": "3 x 12000 (16-bit) / 3 x 1500 (fp32), back to back; the middle figure is quoted",
+                      "sampling": "rocm-smi --showpower --showclocks --json every 0.25 s while the launches run (the first 0.3 s dropped)"}))
+
+
 def main():
     global SETTLE_S
     ap = argparse.ArgumentParser()
@@ -171,7 +250,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-ops", action="store_true", help="leave out the per-op lines of BASELINE configs 1-4")
-    ap.add_argument("--configs", default="1,2,3,4", help="which BASELINE configs the per-op lines cover (comma-separated; for profiling one op class)")
+    ap.add_argument("--configs", default="1,2,3,4,x", help="which BASELINE configs the per-op lines cover (comma-separated; for profiling one op class); "
+                                                           "x = the kernels for shapes outside the configs (column reductions, transposing copies, long softmax rows, casts)")
     ap.add_argument("--skip-cpu", action="store_true", help="leave out the cpu_baseline leg")
     ap.add_argument("--skip-decode", action="store_true", help="leave out the GPT-2-shaped decode (tens of thousands of launches)")
     ap.add_argument("--settle", type=float, default=SETTLE_S,
@@ -179,6 +259,9 @@ def main():
     ap.add_argument("--no-graphs", action="store_true",
                     help="time the decode op by op only (for runs under rocprofv3: its kernel tracing aborts the queue on graph replays)")
     ap.add_argument("--decode-batches", default="1,32", help="batch sizes of the decode leg (comma-separated)")
+    ap.add_argument("--clock-study", action="store_true",
+                    help="instead of the benchmark: run the 4096^3 product for a few seconds per case (bf16 / f16 / f32; the BASELINE data, all-zero "
+                         "operands, constant operands) while rocm-smi samples the shader clock and the package power; prints one JSON object")
     ap.add_argument("--replay-kernels", action="store_true",
                     help="decode: time only the replay that launches each recorded, merged step kernel by kernel (no graph launch: for a kernel trace of the merged step)")
     args = ap.parse_args()
@@ -193,6 +276,10 @@ def main():
     L.nd4jhipSetSyncAfterCustomOp(0)     # the timed loop synchronises once at its end
     steps, warmup = args.steps, args.warmup
     SETTLE_S = args.settle
+
+    if args.clock_study:
+        clock_study(ex, L)
+        return
 
     # ---- headline: mmul bf16 4096^3 ----------------------------------------------------------------------------
     n = 4096
@@ -244,7 +331,8 @@ def main():
 
     # ---- the other BASELINE configs ------------------------------------------------------------------------------------
     ops = []
-    cfgs = {int(c) for c in args.configs.split(",") if c.strip()}
+    cfgs = {int(c) for c in args.configs.split(",") if c.strip() and c.strip() != "x"}
+    extras = "x" in [c.strip() for c in args.configs.split(",")]
     if not args.skip_ops:
         print("[bench] per-op leg", file=sys.stderr, flush=True)
         del A, B, Z
@@ -262,7 +350,43 @@ def main():
             line = {"op": name, "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": hbm_entry(nbytes, e, label, e_warm, k)}
             if cpu and cpu_fn is not None:
                 line["cpu_baseline"] = cpu_fn()
-            ops.append(line)
+            ops.append(with_copy_fraction(line, nbytes))
+
+        # What a cold launch of a given size reaches at all on this chip: the plain copy kernel (transform_same Copy, fp32) at
+        # the total traffic of each memory-bound line below, timed the same way (cold over rotating sets, then warm).  Every
+        # memory-bound line then carries `frac_of_copy` = its rate over the rate of the copy of the nearest size.
+        copy_rate = {}      # total bytes per launch -> (cold GB/s, warm GB/s)
+        if cfgs & {1, 3}:
+            sizes = []
+            if 1 in cfgs:
+                sizes += [134217728, 268435456, 402653184]
+            if 3 in cfgs:
+                sizes += [50331648, 100663296, 805306368, 1610612736]
+            for total in sorted(sizes):
+                ne_c = total // 8
+                kc = 1 if total >= 600e6 else n_sets(total)
+                Cin = [NDArray.empty((ne_c,), FLOAT32) for _ in range(kc)]
+                Cout = [NDArray.empty((ne_c,), FLOAT32) for _ in range(min(kc, 3))]
+                for arr in Cin + Cout:
+                    L.dbAllocateSpecialBuffer(arr.buffer.ptr)
+                    L.dbTickDeviceWrite(arr.buffer.ptr)           # contents do not matter: no upload
+                calls = [(lambda i: (lambda: ex.exec_transform_same(TransformSame.Copy, Cin[i], Cout[i % len(Cout)])))(i) for i in range(kc)]
+                w_warm, e_warm = timed(ex, L, calls[0], steps, warmup)
+                if kc > 1:
+                    w, e = timed_rotating(ex, L, calls, max(steps, 2 * kc), warmup)
+                else:
+                    w, e = w_warm, e_warm     # one call streams past the cache by itself
+                copy_rate[total] = (total / (e * 1e-3) / 1e9, total / (e_warm * 1e-3) / 1e9)
+                ops.append({"op": "copy fp32, %.1f MB in + %.1f MB out (calibration: what a cold launch of this size reaches)" % (total / 2e6, total / 2e6),
+                            "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": hbm_entry(total, e, "", e_warm if kc > 1 else None, kc if kc > 1 else None)})
+                del Cin, Cout, calls
+
+        def with_copy_fraction(line, nbytes):
+            if copy_rate:
+                near = min(copy_rate, key=lambda t: abs(math.log(t / nbytes)))
+                line["roofline"]["frac_of_copy"] = round(line["roofline"]["achieved"] / copy_rate[near][0], 4)
+                line["roofline"]["copy_of_bytes"] = near
+            return line
 
         if 1 in cfgs:
             # config 1: legacy chain, fp32 [8192, 4096]
@@ -361,16 +485,50 @@ def main():
                 line = {"op": "softmax %s [16,12,1024,1024]" % dtn, "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": hbm_entry(2 * es * nl, e, "softmax %s" % dtn)}
                 if cpu:
                     line["cpu_baseline"] = sm_cpu()
-                ops.append(line)
+                ops.append(with_copy_fraction(line, 2 * es * nl))
                 view = Lg.permute(0, 2, 1, 3)
                 w, e = timed(ex, L, ex.bind_custom("softmax", [view], [Zs], i_args=[3]), steps, warmup)
                 line2 = {"op": "softmax %s permuted[0,2,1,3] view" % dtn, "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": hbm_entry(2 * es * nl, e, "softmax %s" % dtn)}
                 if cpu:
                     line2["cpu_baseline"] = dict(line["cpu_baseline"], sample=line["cpu_baseline"]["sample"] + " (dense rows; the view changes addresses only)")
-                ops.append(line2)
+                ops.append(with_copy_fraction(line2, 2 * es * nl))
                 del Lg, Zs, dense, view
+        if extras:
+            # kernels for shapes no BASELINE config uses, measured the same way (cold over rotating sets, then warm)
+            rng = np.random.default_rng(77)
+            GBx = 1e9
+            rc_shape = (6144, 4096)
+            xc = rng.normal(0, 1, rc_shape).astype(np.float32)
+            Kx = n_sets(4 * xc.size)
+            Xc = [NDArray.from_numpy(xc) for _ in range(Kx)]
+            for arr in Xc:
+                arr.sync_to_device()
+            Rc = [NDArray.empty((rc_shape[1],), FLOAT32) for _ in range(Kx)]
+            Ic = [NDArray.empty((rc_shape[1],), INT64) for _ in range(Kx)]
+            hbm_line("reduce_sum dim0 fp32 [6144,4096] (column sums: reduce_cols)", "", 4 * xc.size + 4 * rc_shape[1],
+                     lambda i: (lambda: ex.exec_reduce_same(ReduceSame.Sum, Xc[i], [0], z=Rc[i])))
+            hbm_line("argmax dim0 fp32 [6144,4096] (index_cols)", "", 4 * xc.size + 8 * rc_shape[1],
+                     lambda i: (lambda: ex.exec_index_reduce(IndexReduce.IndexMax, Xc[i], [0], z=Ic[i])))
+            Tc = [NDArray.empty((rc_shape[1], rc_shape[0]), FLOAT32) for _ in range(3)]
+            Xt = [x_.permute(1, 0) for x_ in Xc]
+            hbm_line("assign of a transposed view fp32 [6144,4096] -> [4096,6144] (transpose_tiled)", "", 2 * 4 * xc.size,
+                     lambda i: (lambda: ex.exec_assign(Xt[i], Tc[i % 3])))
+            Bc = [NDArray.empty(rc_shape, BFLOAT16) for _ in range(3)]
+            hbm_line("cast fp32 -> bf16 [6144,4096] (cast_contig)", "", 6 * xc.size,
+                     lambda i: (lambda: ex.exec_assign(Xc[i], Bc[i % 3])))
+            del Xc, Xt, Rc, Ic, Tc, Bc, xc
+            lv = rng.normal(0, 2, (500, 50257)).astype(np.float32)
+            Kl = n_sets(2 * 4 * lv.size)
+            Lv = [NDArray.from_numpy(lv) for _ in range(Kl)]
+            for arr in Lv:
+                arr.sync_to_device()
+            Zl = [NDArray.empty(lv.shape, FLOAT32) for _ in range(3)]
+            sm_binds = [ex.bind_custom("softmax", [Lv[i]], [Zl[i % 3]], i_args=[1]) for i in range(Kl)]
+            hbm_line("softmax fp32 [500,50257] (vocabulary-length rows: softmax_long_vec)", "", 2 * 4 * lv.size, lambda i: sm_binds[i])
+            del Lv, Zl, sm_binds, lv
         if 2 in cfgs:
             # config 2, the remaining sizes/dtypes
+            plain_cpu = {}     # (dtype, size) -> cpu_baseline of the plain-B product: the CPU loops do not depend on the layout flag
             for dt, dtn, peak in [(FLOAT32, "f32", "f32"), (HALF, "f16", "f16"), (BFLOAT16, "bf16", "bf16")]:
                 for m in (1024, 4096):
                     for transb in (False, True):
@@ -405,7 +563,10 @@ def main():
                             tq = best_time(lambda: a32 @ b32)
                             line["cpu_baseline"]["fast"]["value"] = round(2.0 * m * m * m / tq / 1e12, 4)
                         elif cpu:
-                            line["cpu_baseline"] = dict(ops[-1]["cpu_baseline"], sample=ops[-1]["cpu_baseline"]["sample"] + " (the plain-B measurement; the CPU loops do not depend on the layout flag)")
+                            src = plain_cpu.get((dtn, m)) or result.get("cpu_baseline")   # bf16 4096: the headline's own measurement
+                            line["cpu_baseline"] = dict(src, sample=src["sample"] + " (the plain-B measurement; the CPU loops do not depend on the layout flag)")
+                        if cpu and not transb:
+                            plain_cpu[(dtn, m)] = line["cpu_baseline"]
                         ops.append(line)
                         del Am, Bm, Zm
         if 4 in cfgs:
@@ -423,9 +584,19 @@ def main():
                     arr.sync_to_device()
                 w, e = timed(ex, L, ex.bind_custom("dot_product_attention_v2", [Q, V, K_], [O_], t_args=[0.125, 0.0], b_args=[True, False]),
                              max(steps // 5, 3), max(warmup // 5, 1))
+                dense_flops = 4.0 * 96 * 1024 * 1024 * 64
+                # what the kernel executes: a block owns 128 queries and walks the 64-key tiles up to its last query's diagonal
+                executed_flops = 96 * sum(4.0 * 64 * 128 * min(1024, 64 * math.ceil(128 * (blk + 1) / 64)) for blk in range(8))
+                useful_flops = 4.0 * 96 * 64 * (1024 * 1025 / 2)       # the scores on and below the diagonal
+                rf = mfma_entry(dense_flops, e, dtn, "dot_product_attention_v2")
+                rf["achieved_executed"] = round(executed_flops / (e * 1e-3) / 1e12, 2)
+                rf["frac_executed"] = round(rf["achieved_executed"] / MFMA_PEAK[dtn], 4)
+                rf["achieved_causal_useful"] = round(useful_flops / (e * 1e-3) / 1e12, 2)
                 line = {"op": "dot_product_attention_v2 %s causal [96,1024,64] (output only)" % dtn, "ms": round(e, 4), "wall_ms": round(w, 4),
-                        "roofline": mfma_entry(4.0 * 96 * 1024 * 1024 * 64, e, dtn, "dot_product_attention_v2"),
-                        "note": "achieved counts the dense 4*B*T*T*D flops; the causal mask makes about half of them useful"}
+                        "roofline": rf,
+                        "note": "achieved / frac count the dense 4*B*T*T*D flops (25.77 GFLOP); achieved_executed the flops of the key tiles the kernel "
+                                "multiplies (%.2f GFLOP: tiles wholly above the diagonal are skipped), achieved_causal_useful the scores on and below "
+                                "the diagonal (%.2f GFLOP)" % (executed_flops / 1e9, useful_flops / 1e9)}
                 if cpu:
                     nb = 2
                     cv = (lambda t: O.Arr(f32_to_bf16_bits(np.asarray(t, np.float32)), O.BFLOAT16)) if dt == BFLOAT16 else (lambda t: O.Arr(np.ascontiguousarray(t)))
@@ -506,27 +677,52 @@ def main():
                         "roofline": hbm_entry(n_param_bytes + kv_bytes, step_ms)})
             del dec
         if not args.skip_cpu:
-            # CPU side of config 5 (part of the cpu-baseline leg): the oracle's composition of the same ops, fp32, batch 1,
-            # on a bounded sample (prompt of 32 tokens, 8 greedy steps); its ids are also compared with the HIP fp32 run
+            # CPU side of config 5 (part of the cpu-baseline leg): the oracle's composition of the same ops, fp32, on a bounded
+            # sample per batch size (a short prompt, a few greedy steps); at batch 1 its ids are also compared with the HIP fp32 run
             from oracle import oracle as O
             from oracle.decoder_oracle import OracleDecoder
-            ids = np.random.default_rng(5005).integers(0, cfg.vocab, (1, 32))
-            cpu = OracleDecoder(cfg, weights, O.FLOAT32, batch=1)
-            nxt = cpu.forward(ids)
-            cpu_ids = [nxt]
-            t0 = time.perf_counter()
-            for _ in range(7):
-                nxt = cpu.forward(nxt.reshape(1, 1))
-                cpu_ids.append(nxt)
-            cpu_step = (time.perf_counter() - t0) / 7
-            dec = Decoder(cfg, weights, FLOAT32, batch=1, executioner=ex)
-            gpu_ids = dec.generate(ids, 8)
-            ops[-2]["cpu_tokens_per_s"] = round(1.0 / cpu_step, 2)
-            ops[-2]["cpu_sample"] = "oracle decoder fp32, batch 1, 7 decode steps after a 32-token prompt, %d threads" % O.get_threads()
-            ops[-2]["fp32_ids_match_cpu"] = bool((gpu_ids == np.stack(cpu_ids, 1)).all())
-            del dec, cpu
+            decode_lines = {int(l["op"].split("batch ")[1].split(" ")[0]): l for l in ops if l["op"].startswith("gpt2-small decode")}
+            for batch, n_steps, n_prompt in ((1, 7, 32), (32, 3, 8)):
+                if batch not in decode_lines:
+                    continue
+                ids = np.random.default_rng(5005).integers(0, cfg.vocab, (batch, n_prompt))
+                cpu = OracleDecoder(cfg, weights, O.FLOAT32, batch=batch)
+                nxt = cpu.forward(ids)
+                cpu_ids = [nxt]
+                t0 = time.perf_counter()
+                for _ in range(n_steps):
+                    nxt = cpu.forward(nxt.reshape(batch, 1))
+                    cpu_ids.append(nxt)
+                cpu_step = (time.perf_counter() - t0) / n_steps
+                line = decode_lines[batch]
+                line["cpu_baseline"] = {"value": round(batch / cpu_step, 2), "unit": "tokens/s", "cores": O.get_threads(), "kind": "port",
+                                        "sample": "oracle decoder (the same op composition on the CPU restatement), fp32, batch %d, %d greedy steps after a %d-token prompt, %.1f s"
+                                                  % (batch, n_steps, n_prompt, cpu_step * n_steps)}
+                if batch == 1:
+                    dec = Decoder(cfg, weights, FLOAT32, batch=1, executioner=ex)
+                    gpu_ids = dec.generate(ids, n_steps + 1)
+                    line["fp32_ids_match_cpu"] = bool((gpu_ids == np.stack(cpu_ids, 1)).all())
+                    del dec
+                del cpu
         result["ops"] = ops
     print(json.dumps(result))
+    sys.stdout.flush()
+    # One compact row per line of the record, last on stderr, so that a reader who only keeps the tail of the output still
+    # has every figure: time per call, fraction of the roofline cold (and warm / of the same-size copy where measured), CPU
+    # port and CPU fast in the roofline's unit (tokens/s for the decode).
+    def row(name, ms, rf, cb):
+        f = lambda v: "-" if v is None else ("%.3f" % v)
+        port = cb.get("value") if cb else None
+        fast = cb.get("fast", {}).get("value") if cb else None
+        g = lambda v: "-" if v is None else ("%.4g" % v)
+        return "%-34.34s|%8.4f|%5s|%5s|%5s|%8s|%8s" % (name, ms, f(rf.get("frac")), f(rf.get("frac_warm")), f(rf.get("frac_of_copy")), g(port), g(fast))
+    print("%-34s|%8s|%5s|%5s|%5s|%8s|%8s" % ("op", "ms", "frac", "warm", "/copy", "cpu port", "cpu fast"), file=sys.stderr)
+    print(row("mmul bf16 4096^3 (headline)", result["ms_per_step"], result["roofline"], result.get("cpu_baseline")), file=sys.stderr)
+    for l in result.get("ops", []):
+        short = l["op"].replace("dot_product_attention_v2", "attention").replace(" (transform_same Copy; calibrates HBM counters)", "").replace("[8192,4096]", "").replace("[16,1024,768]", "")
+        short = short.replace("gpt2-small decode bf16", "decode").replace("[16,12,1024,1024]", "").replace("  ", " ")
+        print(row(short, l["ms"], l["roofline"], l.get("cpu_baseline")), file=sys.stderr)
+    sys.stderr.flush()
 
 
 if __name__ == "__main__":

@@ -689,8 +689,7 @@ static void launchFusedTyped(hipStream_t s, const void* q, const void* k, const 
   }
   constexpr size_t LDS = (size_t)2 * ((D / 64) * 512 + 64 * (D / 8)) * 16;   // two stages of (K tile, V tile)
   auto kern = attn_fused<T, D, FOLD, VM>;
-  static std::once_flag attrOnce;
-  std::call_once(attrOnce, [&] { HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS)); });
+  ND4J_REQUIRE((DynLds<attn_fused<T, D, FOLD, VM>, (int)LDS>::granted()), "attention: the device does not grant the fused kernel its LDS");
   hipLaunchKernelGGL(kern, dim3((unsigned)((LongType)(a.heavyFirst ? a.qTiles : a.perBatch) * d.B)), dim3(256), LDS, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
 }
 

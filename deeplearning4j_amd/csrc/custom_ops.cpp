@@ -145,7 +145,7 @@ static void matmulExec(Context& c) {
   if (z->isEmpty()) return;
   DataType dt = z->dataType();
   ND4J_REQUIRE(g.x->dataType() == dt && g.y->dataType() == dt, "MATMUL OP: nd4j-hip requires x, y and z to share one data type");
-  ND4J_REQUIRE(isFloatType(dt), "MATMUL OP: integer types are not implemented in nd4j-hip");
+  ND4J_REQUIRE(isFloatType(dt) || dt == INT32 || dt == INT64, std::string("MATMUL OP: ") + dtypeName(dt) + " arrays are not implemented in nd4j-hip");
   GemmDesc d;
   d.M = g.M; d.N = g.N; d.K = g.K;
   d.aRow = g.aRow; d.aCol = g.aCol; d.bRow = g.bRow; d.bCol = g.bCol;

@@ -35,15 +35,15 @@ void executeOp(const OpDescriptor& op, Context& ctx);
 // serve are merged (a pairwise Add and the layer_norm of its result; xw_plus_b and the GELU transform / the column-slice
 // assigns that follow it), every merged kernel writing exactly what the separate ops would have written, bit for bit.
 struct RecordedOp {
-  enum Kind { CUSTOM, PAIRWISE, TRANSFORM_STRICT, TRANSFORM_ANY } kind = CUSTOM;
+  enum Kind { CUSTOM, PAIRWISE, TRANSFORM_STRICT, TRANSFORM_ANY, RAW } kind = CUSTOM;   // RAW: a copy or fill on plain device pointers (memcpyAsync / memsetAsync), never merged
   const ops::OpDescriptor* op = nullptr;   // CUSTOM
   Context ctx;                             // CUSTOM: copy of the caller's argument bag (arrays borrowed)
   int opNum = 0;                           // legacy loops
   NDArray *x = nullptr, *y = nullptr, *z = nullptr;
   std::function<void(const RecordedOp&)> run;   // legacy loops: executes the op on this record's arrays exactly as the eager call does
-  // The arrays above are the caller's while the capture is open.  adopt() replaces every one of them by a copy of the view
-  // held here (same buffer, offset, shape and strides; the buffer is shared), so that a plan built from the record does
-  // not depend on how long the caller keeps its array handles.
+  // adopt() replaces every array above by a copy of the view held here (same buffer, offset, shape and strides; the
+  // buffer is shared).  The facade calls it the moment the op is recorded, so neither the merging pass nor a replay
+  // depends on how long the caller keeps its array handles.
   std::vector<std::shared_ptr<NDArray>> owned;
   void adopt();
 };

@@ -240,6 +240,9 @@ __device__ __forceinline__ A unary_tail(int k, A x) {
     case U_TIMES_ONE_MINUS: return x * (one - x);                                              // ops.h:1165
     case U_CEIL: return M::ceil_(x);                                                           // ops.h:193
     case U_FLOOR: return M::floor_(x);                                                         // ops.h:196
+    // ops.h:217-219 through op_macros_unary.h:109-113: the sign expression is the CONDITION, so every non-zero number gives 1
+    case U_SIGN_REF: return ((x > (A)0) - (x < (A)0)) != 0 ? one : -one;
+    case U_STABILIZE_FP16: return x <= (A)0 ? (A)6.103515625e-05 : x;                          // ops.h:381-384 (HALF's smallest normal)
     // TransformBool (ops.h:1140-1163,1927-1933): 1 where the predicate holds
     case U_IS_INF: return (x == x && (x - x) != (x - x)) ? one : (A)0;
     case U_IS_NAN: return x != x ? one : (A)0;

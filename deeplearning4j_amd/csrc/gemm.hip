@@ -128,6 +128,27 @@ __global__ __launch_bounds__(256) void gemm_simple(GemmArgs g, const T* __restri
     }
 }
 
+// Integer arrays (INT32 / INT64): the reference's plain loop in the array's own type (helpers/cpu/MmulHelper.cpp:35-110:
+// val += A * B in T3, then alphaZ * val (+ betaZ * C) with alpha and beta cast to T3).  Sums and products in 64-bit
+// integers narrowed on the store are the same values (two's complement wrap-around).  One thread per element of C.
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_int(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C, LongType alphaZ, LongType betaZ,
+                                                int betaPresent) {
+  const LongType bz = blockIdx.z;
+  { LongType oa, ob, oc; batchOffsets(g, bz, oa, ob, oc); A += oa; B += ob; C += oc; }
+  const LongType idx = (LongType)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= g.M * g.N) return;
+  const LongType m = idx / g.N, n = idx - m * g.N;
+  const T* a = A + m * g.aRow;
+  const T* b = B + n * g.bCol;
+  unsigned long long acc = 0;
+  for (LongType k = 0; k < g.K; k++) acc += (unsigned long long)(LongType)a[k * g.aCol] * (unsigned long long)(LongType)b[k * g.bRow];
+  const LongType off = m * g.cRow + n * g.cCol;
+  unsigned long long v = (unsigned long long)alphaZ * acc;
+  if (betaPresent) v += (unsigned long long)betaZ * (unsigned long long)(LongType)C[off];
+  C[off] = (T)v;
+}
+
 // ---- tile scheduling ---------------------------------------------------------------------------------------------
 // Hardware hands consecutive workgroup ids to the 8 XCDs round-robin.  Give every XCD a contiguous range of
 // tiles instead, and walk that range in groups of GROUP_M tile-rows so that concurrently running workgroups
@@ -1240,15 +1261,8 @@ static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
       // 64 x 64: one tile per CU and a K of whole eight-tile rounds take eight stages (128 KiB), else four (two blocks fit a
       // CU); 128 x 128: four stages (128 KiB)
       constexpr int DEEP = TW == 1 ? 8 : 4;
-      static std::once_flag onceDeep;
-      static bool grantedDeep = false;
       const bool wantDeep = TW == 2 || (nTiles <= 256 && g.K % 512 == 0);
-      if (wantDeep)
-        std::call_once(onceDeep, [&] {
-          grantedDeep = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_mfma16s<T, B_KC, DEEP, TW>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                            DEEP * STAGE_BYTES) == hipSuccess;
-          if (!grantedDeep) (void)hipGetLastError();
-        });
+      const bool grantedDeep = DynLds<gemm_mfma16s<T, B_KC, DEEP, TW>, DEEP * STAGE_BYTES>::granted();
       if (wantDeep && grantedDeep) {
         noteKernel("gemm_mfma16s<%s,%dx%d,akc=1,bkc=%d,stages=%d>", tname<T>(), BM, BN, (int)B_KC, DEEP);
         hipLaunchKernelGGL((gemm_mfma16s<T, B_KC, DEEP, TW>), dim3(tM * tN, 1, (unsigned)batch), dim3(256), DEEP * STAGE_BYTES, s, g, (const T*)A,
@@ -1266,9 +1280,11 @@ static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
   auto kern = useFull ? gemm_mfma16f<T, BM, BN, WM, WN, A_KC, B_KC>
               : useDeep ? gemm_mfma16q<T, BM, BN, WM, WN, A_KC, B_KC, 4>
               : usePipe ? gemm_mfma16p<T, BM, BN, WM, WN, A_KC, B_KC> : gemm_mfma16<T, BM, BN, WM, WN, A_KC, B_KC>;
-  const int which = useFull ? 2 : useDeep ? 3 : usePipe ? 1 : 0;
-  static std::once_flag attrOnce[4];
-  std::call_once(attrOnce[which], [&] { HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS)); });
+  const bool ldsGranted = useFull ? DynLds<gemm_mfma16f<T, BM, BN, WM, WN, A_KC, B_KC>, (int)LDS>::granted()
+                          : useDeep ? DynLds<gemm_mfma16q<T, BM, BN, WM, WN, A_KC, B_KC, 4>, (int)LDS>::granted()
+                          : usePipe ? DynLds<gemm_mfma16p<T, BM, BN, WM, WN, A_KC, B_KC>, (int)LDS>::granted()
+                                    : DynLds<gemm_mfma16<T, BM, BN, WM, WN, A_KC, B_KC>, (int)LDS>::granted();
+  ND4J_REQUIRE(ldsGranted, "matmul: the device does not grant the tile kernel its LDS");
   const unsigned tilesM = (unsigned)((g.M + BM - 1) / BM), tilesN = (unsigned)((g.N + BN - 1) / BN);
   noteKernel("%s<%s,%dx%d,akc=%d,bkc=%d>%s", useFull ? "gemm_mfma16f" : useDeep ? "gemm_mfma16q" : usePipe ? "gemm_mfma16p" : "gemm_mfma16", tname<T>(), BM, BN,
              (int)A_KC, (int)B_KC, splits > 1 ? "+splitk_finish" : "");
@@ -1292,13 +1308,7 @@ static bool launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const 
     constexpr size_t LDS = (3 * 256 * 8 + 4 * 32 * 32) * 16;   // 160 KiB: the whole LDS of a CU
     auto kern = gemm_mfma16r<T>;
     // a device or driver that does not grant a block the whole LDS keeps the two-stage kernel below
-    static std::once_flag attrOnce;
-    static bool ringGranted = false;
-    if (direct && ring && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 128 == 0)
-      std::call_once(attrOnce, [&] {
-        ringGranted = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS) == hipSuccess;
-        if (!ringGranted) (void)hipGetLastError();
-      });
+    const bool ringGranted = DynLds<gemm_mfma16r<T>, (int)LDS>::granted();
     if (direct && ring && ringGranted && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 128 == 0) {
       const unsigned tM = (unsigned)(g.M / 256), tN = (unsigned)(g.N / 256);
       noteKernel("gemm_mfma16r<%s,256x256,akc=1,bkc=0>", tname<T>());
@@ -1309,8 +1319,7 @@ static bool launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const 
   if (direct && A_KC && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 64 == 0 && g.K >= 128) {
     constexpr size_t LDS = 2 * 2 * 256 * 8 * 16;
     auto kern = gemm_mfma16d<T, B_KC>;
-    static std::once_flag attrOnce;
-    std::call_once(attrOnce, [&] { HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS)); });
+    ND4J_REQUIRE((DynLds<gemm_mfma16d<T, B_KC>, (int)LDS>::granted()), "matmul: the device does not grant the two-stage kernel its LDS");
     const unsigned tM = (unsigned)(g.M / 256), tN = (unsigned)(g.N / 256);
     noteKernel("gemm_mfma16d<%s,256x256,akc=1,bkc=%d>", tname<T>(), (int)B_KC);
     hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(512), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
@@ -2162,6 +2171,16 @@ bool launchGemm(hipStream_t s, DataType dt, const void* A, const void* B, void* 
     case DOUBLE: launchSimple<double>(s, A, B, C, d); break;
     case HALF: dispatch16<f16_t>(s, d, A, B, C); break;
     case BFLOAT16: dispatch16<bf16_t>(s, d, A, B, C); break;
+    case INT32: case INT64: {
+      ND4J_REQUIRE(d.bias == nullptr, "matmul: a bias row with integer arrays is not implemented in nd4j-hip");
+      ND4J_REQUIRE(d.M * d.N < (1LL << 39), "matmul: problem too large for the launch grid");
+      GemmArgs g = toArgs(d);
+      const dim3 grid((unsigned)((d.M * d.N + 255) / 256), 1, (unsigned)d.batch);
+      const LongType alphaZ = (LongType)d.alpha, betaZ = (LongType)d.beta;
+      if (dt == INT32) { noteKernel("gemm_int<int32>"); hipLaunchKernelGGL((gemm_int<int>), grid, dim3(256), 0, s, g, (const int*)A, (const int*)B, (int*)C, alphaZ, betaZ, d.beta != 0.f ? 1 : 0); }
+      else { noteKernel("gemm_int<int64>"); hipLaunchKernelGGL((gemm_int<LongType>), grid, dim3(256), 0, s, g, (const LongType*)A, (const LongType*)B, (LongType*)C, alphaZ, betaZ, d.beta != 0.f ? 1 : 0); }
+      break;
+    }
     default: ND4J_THROW("matmul: unsupported dtype");
   }
   HIP_CHECK(hipGetLastError());

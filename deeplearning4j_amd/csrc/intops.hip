@@ -106,6 +106,7 @@ __device__ __forceinline__ LongType int_unary(int k, LongType x) {
     case U_RECIPROCAL: return x == 0 ? 0 : 1 / x;               // ops.h:207
     case U_ONES: return 1;                                      // ops.h:481
     case U_TIMES_ONE_MINUS: return x * (1 - x);                 // ops.h:1165
+    case U_SIGN_REF: return x != 0 ? 1 : -1;                    // ops.h:217-219: the macro tests the sign expression
     case U_IS_POSITIVE: return x > 0;                           // TransformBool, ops.h:1140-1163
     case U_IS_NEGATIVE: return x < 0;
     case U_NOT: return x == 0;
@@ -117,8 +118,26 @@ __device__ __forceinline__ LongType int_unary(int k, LongType x) {
 bool intUnarySupported(UnaryKind k) {
   switch (k) {
     case U_ABS: case U_NEG: case U_SQUARE: case U_CUBE: case U_ONE_MINUS: case U_RECIPROCAL: case U_ONES: case U_TIMES_ONE_MINUS:
-    case U_IDENTITY: case U_ROUND: case U_CEIL: case U_FLOOR: case U_RINT:
+    case U_IDENTITY: case U_ROUND: case U_CEIL: case U_FLOOR: case U_RINT: case U_SIGN_REF:
     case U_IS_POSITIVE: case U_IS_NEGATIVE: case U_NOT: case U_IS_FINITE: case U_IS_INF: case U_IS_NAN: case U_IS_INF_OR_NAN: return true;
+    default: return false;
+  }
+}
+
+// UINT64 travels through the signed 64-bit arithmetic above bit for bit, which is the right result only where wrap-around
+// arithmetic does not look at the sign: values of 2^63 and more would compare, divide and take remainders as negative
+// numbers.  Those ops are refused for UINT64 operands rather than computed wrongly.
+static bool signAgnosticBinary(PairwiseKind k) {
+  switch (k) {
+    case P_ADD: case P_SUB: case P_MUL: case P_RSUB: case P_COPY: case P_SQSUB: case P_SQ_RSUB: case P_LOGICAL_OR: case P_LOGICAL_XOR:
+    case P_LOGICAL_NOT: case P_LOGICAL_AND: case P_EQ: case P_NE: return true;
+    default: return false;
+  }
+}
+static bool signAgnosticUnary(UnaryKind k) {
+  switch (k) {
+    case U_NEG: case U_SQUARE: case U_CUBE: case U_ONE_MINUS: case U_ONES: case U_TIMES_ONE_MINUS: case U_IDENTITY: case U_ROUND: case U_CEIL:
+    case U_FLOOR: case U_RINT: case U_SIGN_REF: case U_NOT: case U_IS_FINITE: case U_IS_INF: case U_IS_NAN: case U_IS_INF_OR_NAN: return true;
     default: return false;
   }
 }
@@ -171,6 +190,11 @@ void launchIntElementwise(hipStream_t s, int k, bool binary, DataType xdt, DataT
   ND4J_REQUIRE(isIntLike(xdt) && isIntLike(zdt) && (!binary || hasScalar || isIntLike(ydt)), "integer elementwise op: integer or bool operands only");
   if (binary) ND4J_REQUIRE(intBinarySupported((PairwiseKind)k), "this pairwise / scalar / broadcast op is not implemented for integer arrays in nd4j-hip");
   else ND4J_REQUIRE(intUnarySupported((UnaryKind)k), "this transform is not implemented for integer arrays in nd4j-hip");
+  if (xdt == UINT64 || zdt == UINT64 || (binary && !hasScalar && ydt == UINT64)) {
+    ND4J_REQUIRE(!hasScalar, "scalar ops on UINT64 arrays are not implemented in nd4j-hip (the scalar travels as a signed 64-bit value)");
+    ND4J_REQUIRE(binary ? signAgnosticBinary((PairwiseKind)k) : signAgnosticUnary((UnaryKind)k),
+                 "this op orders, divides or takes remainders of its operands, which nd4j-hip computes in signed 64-bit arithmetic: not implemented for UINT64 arrays");
+  }
   const bool same = xdt == zdt && (!binary || hasScalar || ydt == zdt);
   if (same && p.sameShape && p.contiguous && (zdt == INT32 || zdt == INT64) && al16(x) && al16(z) && (!binary || hasScalar || al16(y))) {
     const LongType V = zdt == INT32 ? 4 : 2;
@@ -283,6 +307,9 @@ void launchIntReduce(hipStream_t st, int kind, bool isIndex, DataType xdt, DataT
                      size_t scratchBytes) {
   if (p.outerLen == 0) return;
   ND4J_REQUIRE(isIntLike(xdt) && isIntLike(zdt), "integer reduction: integer or bool arrays only");
+  // signed 64-bit accumulators: sums and products wrap around as UINT64's do, extremes and their positions would not be UINT64's
+  ND4J_REQUIRE(xdt != UINT64 || (!isIndex && ((ReduceKind)kind == R_SUM || (ReduceKind)kind == R_PROD)),
+               "extremes, absolute values and index reductions of UINT64 arrays are not implemented in nd4j-hip (signed 64-bit arithmetic)");
   IntReduceArgs a;
   a.outer = p.outer; a.inner = p.inner; a.zOuter = p.zOuter;
   a.outerLen = p.outerLen; a.innerLen = p.innerLen;

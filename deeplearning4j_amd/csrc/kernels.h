@@ -25,6 +25,8 @@ enum UnaryKind : int {
   U_ASINH, U_RINT, U_LOG_SIGMOID, U_ERFC, U_EXPM1, U_ATANH, U_GELU_D, U_PRECISE_GELU_D, U_MISH, U_MISH_D,
   // TransformSame
   U_ONES, U_ROUND, U_TIMES_ONE_MINUS, U_CEIL, U_FLOOR,
+  U_SIGN_REF,         // TransformSame Sign as the reference's macro evaluates it: 1 for every non-zero number, -1 for zero and NaN
+  U_STABILIZE_FP16,   // TransformStrict StabilizeFP16: 2^-14 (the smallest normal HALF) for x <= 0, else x
   // TransformBool (output type BOOL)
   U_IS_INF, U_IS_NAN, U_IS_FINITE, U_IS_INF_OR_NAN, U_IS_POSITIVE, U_NOT, U_IS_NEGATIVE,
   U_TAIL_END
@@ -118,7 +120,10 @@ enum MiscReduceKind : int {
   M3_EQUALS_EPS,   // 1 when |x - y| <= param everywhere, else 0 (Reduce3 EqualsWithEps)
   M_NORMP,         // (sum |x|^param)^(1 / param), z in a float type (ReduceFloat NormP); not a two-operand kind
   // ReduceBool 2-7: 1 when any element is finite / inf or nan / nan / inf / positive / negative (sum of indicators, ops.h:1139-1163)
-  M_ANY_FINITE, M_ANY_INF_OR_NAN, M_ANY_NAN, M_ANY_INF, M_ANY_POSITIVE, M_ANY_NEGATIVE
+  M_ANY_FINITE, M_ANY_INF_OR_NAN, M_ANY_NAN, M_ANY_INF, M_ANY_POSITIVE, M_ANY_NEGATIVE,
+  // the ReduceFloat table for an input type that differs from the output's (any numeric X into any float Z); the
+  // ReduceKind travels in `param`
+  M_REDUCE_FLOAT
 };
 
 // outer = kept dims (one output element each), inner = reduced dims

@@ -4,6 +4,7 @@
 #include "../../include/nd4jhip/NativeOps.h"
 
 #include <cstring>
+#include <link.h>
 
 #include "custom_ops.h"
 #include "kernels.h"
@@ -251,9 +252,25 @@ int memcpySync(Nd4jPointer dst, Nd4jPointer src, Nd4jLong size, int flags, Nd4jP
   return 1;
   GUARD_END(0)
 }
+// memcpyAsync / memsetAsync on the library's own stream while a capture is open are part of the recording: they run
+// under the op lock, count as op calls and leave a RAW record, so that a recording that holds them replays them in
+// both replay modes (as a graph node, and as a step of the kernel-by-kernel plan).  Only device-to-device copies can be
+// recorded; a copy that touches host memory inside a capture is an error.
+static bool rawOpInCapture(hipStream_t st) { return captureActive() && g_captureOpCalls != nullptr && st == execStream(); }
 int memcpyAsync(Nd4jPointer dst, Nd4jPointer src, Nd4jLong size, int flags, Nd4jPointer reserved) {
-  GUARD_BEGIN
-  HIP_CHECK(hipMemcpyAsync(dst, src, (size_t)size, kindOf(flags), streamOf(reserved)));
+  GRAPH_BEGIN
+  const hipStream_t st = streamOf(reserved);
+  const hipMemcpyKind kind = kindOf(flags);
+  const bool recorded = rawOpInCapture(st);
+  if (recorded) ND4J_REQUIRE(kind == hipMemcpyDeviceToDevice, "memcpyAsync: only device-to-device copies can be recorded into a graph");
+  HIP_CHECK(hipMemcpyAsync(dst, src, (size_t)size, kind, st));
+  if (recorded) {
+    ++*g_captureOpCalls;
+    RecordedOp r;
+    r.kind = RecordedOp::RAW;
+    r.run = [dst, src, size](const RecordedOp&) { HIP_CHECK(hipMemcpyAsync(dst, src, (size_t)size, hipMemcpyDeviceToDevice, execStream())); };
+    recordOp(std::move(r));
+  }
   return 1;
   GUARD_END(0)
 }
@@ -264,9 +281,18 @@ int memsetSync(Nd4jPointer dst, int value, Nd4jLong size, int, Nd4jPointer) {
   GUARD_END(0)
 }
 int memsetAsync(Nd4jPointer dst, int value, Nd4jLong size, int, Nd4jPointer reserved) {
-  GUARD_BEGIN
+  GRAPH_BEGIN
   // a fill kernel rather than a memset node, so that callers may capture this call into a graph
-  launchFill(streamOf(reserved), dst, value, (size_t)size);
+  const hipStream_t st = streamOf(reserved);
+  const bool recorded = rawOpInCapture(st);
+  launchFill(st, dst, value, (size_t)size);
+  if (recorded) {
+    ++*g_captureOpCalls;
+    RecordedOp r;
+    r.kind = RecordedOp::RAW;
+    r.run = [dst, value, size](const RecordedOp&) { launchFill(execStream(), dst, value, (size_t)size); };
+    recordOp(std::move(r));
+  }
   return 1;
   GUARD_END(0)
 }
@@ -282,6 +308,79 @@ Nd4jPointer lcAllocationPointer(OpaqueLaunchContext lc) { return lc ? lc->alloca
 Nd4jPointer lcExecutionStream(OpaqueLaunchContext lc) { return lc ? &lc->execStream : nullptr; }
 Nd4jPointer lcCopyStream(OpaqueLaunchContext lc) { return lc ? &lc->copyStream : nullptr; }
 Nd4jPointer lcBlasHandle(OpaqueLaunchContext) { return nullptr; }
+Nd4jPointer lcSolverHandle(OpaqueLaunchContext) { return nullptr; }
+Nd4jPointer lcScalarPointerPtr(OpaqueLaunchContext* lc) { return lc ? lcScalarPointer(*lc) : nullptr; }
+Nd4jPointer lcReductionPointerPtr(OpaqueLaunchContext* lc) { return lc ? lcReductionPointer(*lc) : nullptr; }
+Nd4jPointer lcAllocationPointerPtr(OpaqueLaunchContext* lc) { return lc ? lcAllocationPointer(*lc) : nullptr; }
+Nd4jPointer lcExecutionStreamPtr(OpaqueLaunchContext* lc) { return lc ? lcExecutionStream(*lc) : nullptr; }
+Nd4jPointer lcCopyStreamPtr(OpaqueLaunchContext* lc) { return lc ? lcCopyStream(*lc) : nullptr; }
+Nd4jPointer lcBlasHandlePtr(OpaqueLaunchContext*) { return nullptr; }
+
+// ---- start-up queries of a device backend ---------------------------------------------------------------------------
+// Peer access between devices (legacy/cuda/NativeOps.cu:1015-1095): supported when every device reaches every other,
+// and trivially with one device.
+static bool g_supportedP2P = false, g_allowedP2P = false;
+void checkP2P(void) {
+  int n = 0, cur = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) { (void)hipGetLastError(); n = 0; }
+  bool all = true;
+  if (n > 1) {
+    (void)hipGetDevice(&cur);
+    for (int a = 0; a < n && all; a++)
+      for (int b = 0; b < n; b++) {
+        if (a == b) continue;
+        int can = 0;
+        if (hipDeviceCanAccessPeer(&can, a, b) != hipSuccess) { (void)hipGetLastError(); can = 0; }
+        if (!can) { all = false; break; }
+      }
+  }
+  g_supportedP2P = all;
+}
+void enableP2P(bool enable) {
+  if (enable == g_allowedP2P) return;
+  int n = 0, cur = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) { (void)hipGetLastError(); n = 0; }
+  if (n > 1) {
+    (void)hipGetDevice(&cur);
+    for (int a = 0; a < n; a++)
+      for (int b = 0; b < n; b++) {
+        if (a == b) continue;
+        int can = 0;
+        (void)hipSetDevice(a);
+        if (hipDeviceCanAccessPeer(&can, a, b) != hipSuccess) can = 0;
+        if (can) { if (enable) (void)hipDeviceEnablePeerAccess(b, 0); else (void)hipDeviceDisablePeerAccess(b); }
+        (void)hipGetLastError();   // "already enabled" and the like are not failures of this call
+      }
+    (void)hipSetDevice(cur);
+  }
+  g_allowedP2P = enable;
+}
+bool isP2PAvailable(void) {
+  static std::once_flag once;
+  std::call_once(once, [] { checkP2P(); });   // the reference's initializeDevicesAndFunctions runs the check
+  return g_supportedP2P;
+}
+void initializeFunctions(Nd4jPointer*) {}     // the host BLAS function table of the CPU backend; nothing here calls a vendor BLAS
+bool isBlasVersionMatches(int, int, int) { return true; }
+int binaryLevel(void) { return 0; }           // legacy/cuda/NativeOps.cu:2769-2775
+int optimalLevel(void) { return 0; }
+bool isMinimalRequirementsMet(void) { return true; }
+bool isOptimalRequirementsMet(void) { return true; }
+bool isExperimentalEnabled(void) { return false; }
+void setOmpMinThreads(int) {}
+void setGridLimit(int) {}
+Nd4jPointer getConstantSpace(void) { return nullptr; }
+
+// ---- outside this backend's path --------------------------------------------------------------------------------------
+static void notImplemented(const char* fn) { errorRef().set(1, std::string(fn) + " is not implemented in nd4j-hip"); }
+void execRandom(Nd4jPointer*, int, Nd4jPointer, OpaqueNDArray, void*) { notImplemented("execRandom"); }
+void execRandom2(Nd4jPointer*, int, Nd4jPointer, OpaqueNDArray, OpaqueNDArray, void*) { notImplemented("execRandom2"); }
+void execRandom3(Nd4jPointer*, int, Nd4jPointer, OpaqueNDArray, OpaqueNDArray, OpaqueNDArray, void*) { notImplemented("execRandom3"); }
+void sort(Nd4jPointer*, OpaqueNDArray, bool) { notImplemented("sort"); }
+void sortTad(Nd4jPointer*, OpaqueNDArray, Nd4jLong*, Nd4jLong, Nd4jLong*, Nd4jLong*, bool) { notImplemented("sortTad"); }
+void shuffle(Nd4jPointer*, OpaqueNDArrayArr, OpaqueNDArrayArr, int, OpaqueNDArray, OpaqueNDArray) { notImplemented("shuffle"); }
+void pullRows(Nd4jPointer*, OpaqueNDArray, OpaqueNDArray, Nd4jLong, OpaqueNDArray, Nd4jLong) { notImplemented("pullRows"); }
+void convertTypes(Nd4jPointer*, int, Nd4jPointer, Nd4jLong, int, Nd4jPointer) { notImplemented("convertTypes"); }
 
 // ---- data buffers -----------------------------------------------------------------------------------
 OpaqueDataBuffer* allocateDataBuffer(Nd4jLong elements, int dataType, bool allocateBoth) {
@@ -577,8 +676,11 @@ static void transformStrictImpl(int opNum, NDArray* x, void* extraParams, NDArra
     case 48: k = U_RINT; break; case 49: k = U_LOG_SIGMOID; break; case 50: k = U_ERFC; break; case 51: k = U_EXPM1; break;
     case 52: k = U_ATANH; break; case 54: k = U_GELU_D; break; case 56: k = U_PRECISE_GELU_D; break; case 57: k = U_MISH; break;
     case 58: k = U_MISH_D; break;
-    // 5 HardTanhDerivative, 10 HardSigmoidDerivative and
-    // 20 StabilizeFP16 are not restated (their reference macros return the input unchanged / a platform constant)
+    // 5 HardTanhDerivative and 10 HardSigmoidDerivative: the reference declares them through a macro that takes the
+    // derivative's expression as its CONDITION and the input as both outcomes (ops/ops.h:222-226 through
+    // ops/op_macros_unary.h:109-113), so both return the input unchanged; restated as they compute
+    case 5: case 10: k = U_IDENTITY; break;
+    case 20: k = U_STABILIZE_FP16; break;   // ops/ops.h:381-384
     default: ND4J_THROW("execTransformStrict: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
   runUnary("execTransformStrict", k, x, z);
@@ -589,7 +691,10 @@ void execTransformFloat(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa,
   OP_BEGIN(callerStream(extraPointers))
   NDArray* x = arr(xa, "execTransformFloat", "x"); NDArray* z = arr(za, "execTransformFloat", "z");
   ND4J_REQUIRE(isFloatType(z->dataType()), "NativeOpExecutioner::execTransformFloat requires Z to have floating point type");
-  ND4J_REQUIRE(isFloatType(x->dataType()), "execTransformFloat: non-float inputs are not implemented in nd4j-hip");
+  // any common type into any float type (NativeOpExecutioner_transform.cpp:35-37: SD_COMMON_TYPES x SD_FLOAT_TYPES); an
+  // integer or bool element is converted to Z first and the op runs in Z's arithmetic
+  ND4J_REQUIRE(isFloatType(x->dataType()) || x->dataType() == INT32 || x->dataType() == INT64 || x->dataType() == BOOL,
+               std::string("execTransformFloat: input type ") + dtypeName(x->dataType()) + " is not implemented in nd4j-hip");
   UnaryKind k;
   switch (opNum) {  // loops/legacy_ops.h:67
     case 1: k = U_SQRT; break; case 3: k = U_RSQRT; break;
@@ -624,7 +729,7 @@ void execTransformSame(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, 
     case 11: k = U_RECIPROCAL; break; case 12: k = U_SQUARE; break; case 15: case 21: k = U_IDENTITY; break;
     case 2: k = U_ONES; break; case 4: k = U_ROUND; break; case 5: k = U_TIMES_ONE_MINUS; break; case 17: k = U_CEIL; break;
     case 18: k = U_FLOOR; break;
-    // 1 Sign is not restated (the reference macro yields +1 for every non-zero input and -1 for zero)
+    case 1: k = U_SIGN_REF; break;   // Sign as the reference computes it (ops/ops.h:217-219): 1 for every non-zero number, -1 for 0 and NaN
     default: ND4J_THROW("execTransformSame: opNum " + std::to_string(opNum) + " is not implemented in nd4j-hip");
   }
   runUnary("execTransformSame", k, x, z);
@@ -913,14 +1018,14 @@ static void boolTableImpl(const char* fn, int opNum, NDArray* x, NDArray* y, con
     registerSpecialUse({z}, {x, y});
     return;
   }
-  ND4J_REQUIRE(ck != C_BOOL_EPSILON || dt != BOOL, std::string(fn) + ": Epsilon of BOOL arrays is not implemented in nd4j-hip");
   CondParams c;
   c.xdt = (int)dt;
   c.mode = extraParams != nullptr ? 1 : 0;
   if (extraParams) c.compare = fetchParams(fn, extraParams, dt, 1)[0];
   // the default tolerance as the array's type holds it, static_cast<X>(1e-5): bfloat16 rounds it to 0x3728 and half to the
-  // subnormal 168 * 2^-24, which are the same number; the integer types hold 0
-  c.eps = dt == DOUBLE ? 1e-5 : dt == FLOAT32 ? (double)1e-5f : isFloatType(dt) ? 168.0 / 16777216.0 : 0.0;
+  // subnormal 168 * 2^-24, which are the same number; the integer types hold 0; BOOL holds true, so that every pair of
+  // BOOL elements is within the tolerance (their difference, held as a BOOL, is at most true)
+  c.eps = dt == DOUBLE ? 1e-5 : dt == FLOAT32 ? (double)1e-5f : isFloatType(dt) ? 168.0 / 16777216.0 : dt == BOOL ? 1.0 : 0.0;
   prepareSpecialUse({z}, {x, y});
   launchCondElementwise(execStream(), ck, c, dt, BOOL, x->specialBuffer(), y->specialBuffer(), z->specialBuffer(), p, 0.0, false);
   registerSpecialUse({z}, {x, y});
@@ -987,12 +1092,67 @@ void execScalarTad(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, Opaq
 }
 
 }  // extern "C"
+// ---- reductions of EMPTY arrays ------------------------------------------------------------------------------------
+// The reference's loops give every element of Z the op's starting value when X is EMPTY (loops/cpu/reduce/reduce_same.hpp:47,
+// 166-176, reduce_float.hpp:103-106,243-251, reduce_long.hpp:50-53,212-217, reduce_bool.hpp:45-48, indexreduce.hpp:106-113).
+static void fillWithStart(NDArray* z, double fv, LongType iv) {
+  if (z->isEmpty() || z->lengthOf() == 0) return;
+  EwPlan p = buildEwPlan({z->shapeInfo(), z->shapeInfo()});
+  prepareSpecialUse({z}, {});
+  const DataType zdt = z->dataType();
+  if (isIntLike(zdt)) launchIntElementwise(execStream(), P_COPY, true, zdt, zdt, zdt, z->specialBuffer(), nullptr, z->specialBuffer(), p, iv, true);
+  else launchScalarOp(execStream(), P_COPY, zdt, z->specialBuffer(), fv, z->specialBuffer(), p);
+  registerSpecialUse({z}, {});
+}
+// largest finite value of an integer type; DataTypeUtils::infOrMax is +inf for FLOAT and DOUBLE only and the type's largest
+// value for everything else, HALF (65504) and BFLOAT16 included (array/DataTypeUtils.h:588-617)
+static LongType intMax(DataType t) {
+  switch (t) {
+    case BOOL: return 1; case INT8: return 127; case UINT8: return 255; case INT16: return 32767; case UINT16: return 65535;
+    case INT32: return 2147483647LL; case UINT32: return 4294967295LL; default: return 0x7fffffffffffffffLL;
+  }
+}
+static void fillReduceStart(const char* fn, ReduceKind k, NDArray* x, NDArray* z) {
+  const DataType xdt = x->dataType(), zdt = z->dataType();
+  double fv = 0.0;
+  LongType iv = 0;
+  switch (k) {
+    case R_PROD: fv = 1.0; iv = 1; break;                                      // ops.h:2364
+    case R_MAX: case R_MIN: {                                                  // ops.h:2365-2368: -+ infOrMax<X>
+      const double big = xdt == HALF ? 65504.0 : xdt == BFLOAT16 ? 3.3895313892515355e38 : (double)INFINITY;
+      fv = k == R_MAX ? -big : big;
+      iv = k == R_MAX ? -intMax(xdt) : intMax(xdt);
+      break;
+    }
+    case R_AMAX: case R_AMIN:                                                  // ops.h:1225-1243: the starting value is input[0]
+      ND4J_THROW(std::string(fn) + ": AMax / AMin of an EMPTY array start from the array's first element in the reference, which does not exist");
+    case R_MEAN:                                                               // reduce_float.hpp:244-246: nanOrZero<Z>, NaN for FLOAT and DOUBLE only
+      fv = (zdt == FLOAT32 || zdt == DOUBLE) ? (double)NAN : 0.0;
+      break;
+    default: break;                                                            // every other op of the two tables starts from 0
+  }
+  fillWithStart(z, fv, iv);
+}
 namespace nd4jhip {
+// the ReduceFloat table when Z's type is not X's: any numeric X into any float Z (NativeOpExecutioner_reduce.cpp:34-37,104-106),
+// accumulated in double by the type-agnostic kernel (the reference accumulates in float for HALF / BFLOAT16 / FLOAT results
+// and in double for DOUBLE ones, ops/op_types.h:213-226)
+static void runReduceFloatMixed(const char* fn, ReduceKind k, NDArray* x, NDArray* z, const std::vector<LongType>& dims) {
+  runReduceMisc(fn, M_REDUCE_FLOAT, x, z, dims, false, (double)(int)k);
+}
 void runReduce(const char* fn, ReduceKind k, NDArray* x, NDArray* z, const std::vector<LongType>& dims) {
-  ND4J_REQUIRE(isFloatType(x->dataType()) || (isIntLike(x->dataType()) && k <= R_AMIN), std::string(fn) + ": this input type is not implemented in nd4j-hip");
-  ND4J_REQUIRE(x->dataType() == z->dataType(), std::string(fn) + ": nd4j-hip requires Z to have X's type, got " + dtypeName(x->dataType()) + " -> " + dtypeName(z->dataType()));
-  ND4J_REQUIRE(!x->isEmpty(), std::string(fn) + ": reductions of empty arrays are not implemented in nd4j-hip");
+  const bool floatTable = k >= R_MEAN;
+  if (floatTable) {
+    ND4J_REQUIRE(isFloatType(z->dataType()), std::string("NativeOpExecutioner::") + fn + " requires Z operand to have floating point data type, got " + dtypeName(z->dataType()));
+    ND4J_REQUIRE(isFloatType(x->dataType()) || x->dataType() == INT32 || x->dataType() == INT64 || x->dataType() == BOOL,
+                 std::string(fn) + ": input type " + dtypeName(x->dataType()) + " is not implemented in nd4j-hip");
+  } else {
+    ND4J_REQUIRE(isFloatType(x->dataType()) || isIntLike(x->dataType()), std::string(fn) + ": this input type is not implemented in nd4j-hip");
+    ND4J_REQUIRE(x->dataType() == z->dataType(), std::string("NativeOpExecutioner::") + fn + " requires both X & Z operands to have same type, got " + dtypeName(x->dataType()) + " -> " + dtypeName(z->dataType()));
+  }
   if (z->isEmpty()) return;
+  if (x->isEmpty()) { fillReduceStart(fn, k, x, z); return; }
+  if (floatTable && x->dataType() != z->dataType()) { runReduceFloatMixed(fn, k, x, z, dims); return; }
   std::vector<LongType> d = dims;
   if (z->lengthOf() == 1 && x->lengthOf() != 1) {
     // a single output means "reduce everything" unless the kept dims are all of extent 1
@@ -1041,7 +1201,9 @@ void execReduceSame2(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, vo
 }
 // NormP (ReduceFloat 6): (sum |x|^p)^(1/p) with p = extraParams[0] in Z's type (ops.h:1280-1286)
 static void runNormP(const char* fn, NDArray* x, NDArray* z, const void* extraParams, std::vector<LongType> dims) {
-  ND4J_REQUIRE(isFloatType(x->dataType()) && isFloatType(z->dataType()), std::string(fn) + ": NormP takes floating point arrays here");
+  ND4J_REQUIRE(isFloatType(z->dataType()), std::string("NativeOpExecutioner::") + fn + " requires Z operand to have floating point data type");
+  ND4J_REQUIRE(isFloatType(x->dataType()) || x->dataType() == INT32 || x->dataType() == INT64 || x->dataType() == BOOL, std::string(fn) + ": this input type is not implemented in nd4j-hip");
+  if (x->isEmpty()) { if (!z->isEmpty()) fillWithStart(z, 0.0, 0); return; }
   const double pw = fetchParams(fn, extraParams, z->dataType(), 1)[0];
   runReduceMisc(fn, M_NORMP, x, z, dims, false, pw);
 }
@@ -1064,8 +1226,14 @@ void execReduceFloat2(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, v
 }  // extern "C"
 namespace nd4jhip {
 void runReduceMisc(const char* fn, MiscReduceKind k, NDArray* x, NDArray* z, std::vector<LongType> d, bool biasCorrected, double param) {
-  ND4J_REQUIRE(!x->isEmpty(), std::string(fn) + ": reductions of empty arrays are not implemented in nd4j-hip");
   if (z->isEmpty()) return;
+  if (x->isEmpty()) {
+    // the starting values of the counting, Any / All and NormP ops (ops.h:1180-1215,1139-1163,1280-1286); the summary
+    // statistics initialise from x[0], which an EMPTY array does not have (loops/cpu/summarystatsreduce.cpp:106-113)
+    ND4J_REQUIRE(k != M_VARIANCE && k != M_STDDEV, std::string(fn) + ": the reference initialises the statistics of an EMPTY array from its first element, which does not exist");
+    fillWithStart(z, k == M_ALL ? 1.0 : 0.0, k == M_ALL ? 1 : 0);
+    return;
+  }
   if (z->lengthOf() == 1 && x->lengthOf() != 1) {
     bool keptAllUnit = true;
     std::vector<bool> red(x->rankOf(), false);
@@ -1096,8 +1264,8 @@ static void runReduce3(const char* fn, int opNum, NDArray* x, NDArray* y, NDArra
   ND4J_REQUIRE(isFloatType(z->dataType()), std::string(fn) + ": Z must have a floating point type");
   ND4J_REQUIRE(x->rankOf() == y->rankOf() && x->lengthOf() == y->lengthOf(), std::string(fn) + ": x and y must have the same shape");
   for (int i = 0; i < x->rankOf(); i++) ND4J_REQUIRE(x->sizeAt(i) == y->sizeAt(i), std::string(fn) + ": x and y must have the same shape");
-  ND4J_REQUIRE(!x->isEmpty(), std::string(fn) + ": reductions of empty arrays are not implemented in nd4j-hip");
-  if (z->isEmpty()) return;
+  // an EMPTY operand: the reference's loop over x's (zero) elements writes nothing (loops/cpu/reduce3.hpp:49-57)
+  if (z->isEmpty() || x->isEmpty() || y->isEmpty()) return;
   if (z->lengthOf() == 1 && x->lengthOf() != 1) {
     bool keptAllUnit = true;
     std::vector<bool> red(x->rankOf(), false);
@@ -1138,8 +1306,9 @@ void execSummaryStatsTad(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa
 // MatchCondition (count), FirstIndex / LastIndex: [compare, eps, mode] in X's type
 static void runCondReduce(const char* fn, CondReduceKind kind, NDArray* x, NDArray* z, std::vector<LongType> d, const void* extraParams) {
   ND4J_REQUIRE(isFloatType(x->dataType()) || x->dataType() == INT32 || x->dataType() == INT64, std::string(fn) + ": match conditions take float, INT32 or INT64 arrays here");
-  ND4J_REQUIRE(!x->isEmpty(), std::string(fn) + ": reductions of empty arrays are not implemented in nd4j-hip");
   if (z->isEmpty()) return;
+  // EMPTY x: a count of 0 (reduce_long.hpp:50-53,212-217), no index (-1, ops.h:2079-2085,2123-2129)
+  if (x->isEmpty()) { fillWithStart(z, kind == CR_COUNT ? 0.0 : -1.0, kind == CR_COUNT ? 0 : -1); return; }
   const CondParams c = condParams(fn, extraParams, x->dataType(), false);
   if (z->lengthOf() == 1 && x->lengthOf() != 1) {
     bool keptAllUnit = true;
@@ -1224,7 +1393,7 @@ void execReduce3All(Nd4jPointer* extraPointers, int opNum, OpaqueNDArray xa, Opa
   const char* fn = "execReduce3All";
   NDArray* x = arr(xa, fn, "x"); NDArray* y = arr(ya, fn, "y"); NDArray* z = arr(za, fn, "z");
   ND4J_REQUIRE(x->rankOf() == y->rankOf(), std::string(fn) + ": x and y must have one rank");
-  ND4J_REQUIRE(!x->isEmpty() && !y->isEmpty(), std::string(fn) + ": reductions of empty arrays are not implemented in nd4j-hip");
+  if (x->isEmpty() || y->isEmpty()) return;   // nothing is written (loops/cpu/reduce3.hpp:49-57)
   const int rank = x->rankOf();
   auto dims = hostDims(da, rank, fn);
   ND4J_REQUIRE(!dims.empty(), std::string(fn) + ": the dimensions of the sub-arrays are required");
@@ -1299,9 +1468,10 @@ void runIndexReduce(const char* fn, int opNum, NDArray* x, NDArray* z, const std
   ND4J_REQUIRE(isFloatType(x->dataType()) || isIntLike(x->dataType()), std::string(fn) + ": this input type is not implemented in nd4j-hip");
   ND4J_REQUIRE(z->dataType() == INT64 || z->dataType() == INT32,
                std::string("NativeOpExecutioner::") + fn + " requires Z operand to have INT32/INT64 type, got " + dtypeName(z->dataType()));
-  ND4J_REQUIRE(!x->isEmpty(), std::string(fn) + ": index reductions of empty arrays are not implemented in nd4j-hip");
   if (z->isEmpty()) return;
   IndexKind k = indexKind(opNum);
+  // EMPTY x: the starting pair's index, 0 (loops/cpu/indexreduce.hpp:106-113, ops/op_macros_index_reduce.h:46-51)
+  if (x->isEmpty()) { fillWithStart(z, 0.0, 0); return; }
   std::vector<LongType> d = dims;
   if (z->lengthOf() == 1 && (int)d.size() < x->rankOf()) {
     bool keptAllUnit = true;
@@ -1490,7 +1660,9 @@ bool graphFusionEnabled() {
 }
 }  // extern "C"
 static void recordOp(RecordedOp&& r) {
-  if (g_openCapture) g_openCapture->ops.push_back(std::move(r));
+  if (!g_openCapture) return;
+  r.adopt();   // the record keeps its own views of the arrays from here on: the caller may delete its handles before End
+  g_openCapture->ops.push_back(std::move(r));
 }
 extern "C" {
 int nd4jhipGraphBeginCapture(void) {
@@ -1510,17 +1682,23 @@ int nd4jhipGraphBeginCapture(void) {
 Nd4jPointer nd4jhipGraphEndCapture(void) {
   GRAPH_BEGIN
   ND4J_REQUIRE(captureActive() && g_openCapture, "nd4jhipGraphEndCapture: no capture in progress");
-  CapturedGraph* cg = g_openCapture;
-  auto closeCapture = [&] {
-    g_openCapture = nullptr;
-    g_captureOpCalls = nullptr;
-    setActiveCapture(nullptr);
-    Environment::get().syncAfterCustomOp = g_syncBeforeCapture;
-  };
+  // Whatever happens below, the capture is closed and, unless the graph is handed to the caller, freed.
+  struct Closer {
+    CapturedGraph* cg;
+    bool streamOpen = true;    // the stream is still in capture mode
+    ~Closer() {
+      if (streamOpen) { hipGraph_t dropped = nullptr; (void)hipStreamEndCapture(execStream(), &dropped); if (dropped) (void)hipGraphDestroy(dropped); (void)hipGetLastError(); }
+      g_openCapture = nullptr;
+      g_captureOpCalls = nullptr;
+      setActiveCapture(nullptr);
+      Environment::get().syncAfterCustomOp = g_syncBeforeCapture;
+      if (cg) { if (cg->exec) (void)hipGraphExecDestroy(cg->exec); if (cg->graph) (void)hipGraphDestroy(cg->graph); delete cg; }
+    }
+  } closer{g_openCapture};
+  CapturedGraph* cg = closer.cg;
   hipError_t e = hipStreamEndCapture(execStream(), &cg->graph);
+  closer.streamOpen = false;
   if (e != hipSuccess || cg->graph == nullptr) {
-    closeCapture();
-    delete cg;
     (void)hipGetLastError();
     ND4J_THROW(std::string("nd4jhipGraphEndCapture: the capture was invalidated (an op waited on the stream or copied synchronously): ") + hipGetErrorString(e));
   }
@@ -1529,9 +1707,7 @@ Nd4jPointer nd4jhipGraphEndCapture(void) {
   bool keepPlan = false;
   if (graphFusionEnabled() && !cg->ops.empty() && (int)cg->ops.size() == cg->opCalls) {
     int nFused = 0;
-    for (RecordedOp& r : cg->ops) r.adopt();   // from here on the record holds its own views of the arrays
-    auto plan = fuseRecordedOps(cg->ops, nFused);
-    cg->plan = plan;
+    cg->plan = fuseRecordedOps(cg->ops, nFused);
     keepPlan = true;
     if (nFused > 0) {
       g_captureOpCalls = nullptr;             // the replay re-enters nothing that counts
@@ -1540,11 +1716,13 @@ Nd4jPointer nd4jhipGraphEndCapture(void) {
       std::string failure;
       e = hipStreamBeginCapture(execStream(), hipStreamCaptureModeRelaxed);
       if (e == hipSuccess) {
+        closer.streamOpen = true;
         std::vector<RecordedOp> keep;
         keep.swap(cg->ops);                   // replayed ops must not be recorded a second time
-        try { for (auto& step : plan) step(); } catch (std::exception& ex) { failure = ex.what(); }
+        try { for (auto& step : cg->plan) step(); } catch (std::exception& ex) { failure = ex.what(); } catch (...) { failure = "unknown native error"; }
         cg->ops.swap(keep);
         e = hipStreamEndCapture(execStream(), &merged);
+        closer.streamOpen = false;
       }
       if (e == hipSuccess && merged != nullptr && failure.empty()) {
         (void)hipGraphDestroy(cg->graph);
@@ -1553,30 +1731,56 @@ Nd4jPointer nd4jhipGraphEndCapture(void) {
       } else {
         if (merged) (void)hipGraphDestroy(merged);
         (void)hipGetLastError();
-        closeCapture();
-        (void)hipGraphDestroy(cg->graph);
-        delete cg;
         ND4J_THROW("nd4jhipGraphEndCapture: replaying the recorded ops through the merging pass failed: " + (failure.empty() ? std::string(hipGetErrorString(e)) : failure));
       }
     }
   }
-  closeCapture();
   if (!keepPlan) cg->ops.clear();   // (the plan's steps point into the list)
   e = hipGraphInstantiate(&cg->exec, cg->graph, nullptr, nullptr, 0);
   if (e != hipSuccess) {
-    (void)hipGraphDestroy(cg->graph);
-    delete cg;
+    (void)hipGetLastError();
     ND4J_THROW(std::string("nd4jhipGraphEndCapture: hipGraphInstantiate failed: ") + hipGetErrorString(e));
   }
+  closer.cg = nullptr;   // handed to the caller
   return cg;
   GUARD_END(nullptr)
 }
+}  // extern "C"
+// Is a rocprofiler tool library attached to this process?  A graph launch under the kernel tracer once ended in a queue
+// abort ("AQL packet is malformed") whose cause was never established, so a traced process does not launch graphs:
+// nd4jhipGraphLaunch replays the recorded plan kernel by kernel instead (same kernels, same arguments).  The tool is
+// found by what loads it: ROCP_TOOL_LIBRARIES or LD_PRELOAD naming it, or the loaded object itself.
+static bool nameIsProfilerTool(const char* s) { return s != nullptr && (strstr(s, "rocprofiler-sdk-tool") != nullptr || strstr(s, "librocprofv3") != nullptr); }
+static bool profilerToolAttached() {
+  const char* tools = getenv("ROCP_TOOL_LIBRARIES");
+  if (tools != nullptr && *tools) return true;
+  if (nameIsProfilerTool(getenv("LD_PRELOAD"))) return true;
+  bool found = false;
+  dl_iterate_phdr([](struct dl_phdr_info* info, size_t, void* data) -> int {
+    if (nameIsProfilerTool(info->dlpi_name)) { *static_cast<bool*>(data) = true; return 1; }
+    return 0;
+  }, &found);
+  return found;
+}
+extern "C" {
+int nd4jhipProfilerAttached(void) { return profilerToolAttached() ? 1 : 0; }
 int nd4jhipGraphLaunch(Nd4jPointer graph) {
   GRAPH_BEGIN
   ND4J_REQUIRE(graph != nullptr, "nd4jhipGraphLaunch: graph is null");
   ND4J_REQUIRE(!captureActive(), "nd4jhipGraphLaunch: a capture is in progress");
   CapturedGraph* cg = static_cast<CapturedGraph*>(graph);
-  if (g_graphReplayMode == 1 && !cg->plan.empty()) {
+  bool asKernels = g_graphReplayMode == 1 && !cg->plan.empty();
+  if (!asKernels) {
+    static const bool traced = profilerToolAttached();   // a tool attaches before main(): asked once
+    if (traced) {
+      ND4J_REQUIRE(!cg->plan.empty(), "nd4jhipGraphLaunch: a rocprofiler tool is attached to this process and this recording has no kernel-by-kernel plan (an op "
+                                      "call went unrecorded during its capture); graphs are not launched under the tracer");
+      static std::once_flag said;
+      if (Environment::get().verbose) std::call_once(said, [] { fprintf(stderr, "nd4j-hip: a rocprofiler tool is attached; recorded graphs are replayed kernel by kernel\n"); });
+      asKernels = true;
+    }
+  }
+  if (asKernels) {
     // the merged sequence as ordinary launches: every step prepares and registers its own arrays, as the eager call does
     for (auto& b : cg->record.reads) ND4J_REQUIRE(!b->closed, "nd4jhipGraphLaunch: a buffer the graph reads has been closed");
     for (auto& b : cg->record.writes) ND4J_REQUIRE(!b->closed, "nd4jhipGraphLaunch: a buffer the graph writes has been closed");
@@ -1603,6 +1807,48 @@ int nd4jhipGraphLaunch(Nd4jPointer graph) {
   return 0;
   GUARD_END(1)
 }
+// Host-side audit of a recording: every kernel node's block size, dynamic LDS request and grid against what the runtime
+// reports for that function (hipFuncGetAttributes) and for the device.  Launches nothing.  Returns the number of nodes
+// that break a limit (their description goes to the error slot), 0 for a clean graph, -1 when the graph cannot be walked.
+int nd4jhipGraphAudit(Nd4jPointer graph) {
+  GRAPH_BEGIN
+  ND4J_REQUIRE(graph != nullptr, "nd4jhipGraphAudit: graph is null");
+  CapturedGraph* cg = static_cast<CapturedGraph*>(graph);
+  size_t n = 0;
+  HIP_CHECK(hipGraphGetNodes(cg->graph, nullptr, &n));
+  std::vector<hipGraphNode_t> nodes(n);
+  if (n) HIP_CHECK(hipGraphGetNodes(cg->graph, nodes.data(), &n));
+  int dev = 0;
+  HIP_CHECK(hipGetDevice(&dev));
+  hipDeviceProp_t prop;
+  HIP_CHECK(hipGetDeviceProperties(&prop, dev));
+  int bad = 0, kernels = 0;
+  std::string report;
+  for (size_t i = 0; i < n; i++) {
+    hipGraphNodeType type;
+    HIP_CHECK(hipGraphNodeGetType(nodes[i], &type));
+    if (type != hipGraphNodeTypeKernel) continue;
+    kernels++;
+    hipKernelNodeParams kp;
+    HIP_CHECK(hipGraphKernelNodeGetParams(nodes[i], &kp));
+    hipFuncAttributes fa;
+    std::string why;
+    if (hipFuncGetAttributes(&fa, kp.func) != hipSuccess) { (void)hipGetLastError(); why = "hipFuncGetAttributes failed"; }
+    else {
+      const long long threads = (long long)kp.blockDim.x * kp.blockDim.y * kp.blockDim.z;
+      if (threads <= 0 || threads > fa.maxThreadsPerBlock) why += " block of " + std::to_string(threads) + " threads (limit " + std::to_string(fa.maxThreadsPerBlock) + ")";
+      if ((long long)kp.sharedMemBytes > (long long)fa.maxDynamicSharedSizeBytes) why += " dynamic LDS " + std::to_string(kp.sharedMemBytes) + " B (granted " + std::to_string(fa.maxDynamicSharedSizeBytes) + ")";
+      if ((long long)kp.sharedMemBytes + (long long)fa.sharedSizeBytes > (long long)prop.sharedMemPerBlock && (long long)kp.sharedMemBytes + (long long)fa.sharedSizeBytes > (long long)prop.maxSharedMemoryPerMultiProcessor)
+        why += " LDS total " + std::to_string((long long)kp.sharedMemBytes + (long long)fa.sharedSizeBytes) + " B beyond the CU's";
+      if (kp.gridDim.x == 0 || kp.gridDim.y == 0 || kp.gridDim.z == 0 || kp.gridDim.y > 65535u || kp.gridDim.z > 65535u) why += " grid " + std::to_string(kp.gridDim.x) + "x" + std::to_string(kp.gridDim.y) + "x" + std::to_string(kp.gridDim.z);
+      if (kp.kernelParams == nullptr && kp.extra == nullptr) why += " no kernel arguments recorded";
+    }
+    if (!why.empty()) { bad++; report += "node " + std::to_string(i) + ":" + why + "; "; }
+  }
+  if (bad) errorRef().set(1, "nd4jhipGraphAudit: " + std::to_string(bad) + " of " + std::to_string(kernels) + " kernel nodes: " + report);
+  return bad;
+  GUARD_END(-1)
+}
 int nd4jhipGraphFusedOps(Nd4jPointer graph) { return graph ? static_cast<CapturedGraph*>(graph)->fusedOps : 0; }
 void nd4jhipSetGraphReplayMode(int mode) { g_graphReplayMode = mode == 1 ? 1 : 0; }
 int nd4jhipGetGraphReplayMode(void) { return g_graphReplayMode; }
@@ -1621,7 +1867,8 @@ int nd4jhipReduceSameScalarNoAlloc(Nd4jPointer stream, int opNum, int dataType, 
   OP_BEGIN(nullptr)
   LaunchContext* lc = LaunchContext::ifReady();
   ND4J_REQUIRE(lc != nullptr, "nd4jhipReduceSameScalarNoAlloc: call initializeDevicesAndFunctions first (initialisation allocates, this call must not)");
-  ND4J_REQUIRE(!captureActive() || stream != nullptr, "nd4jhipReduceSameScalarNoAlloc: pass the capturing stream");
+  // between nd4jhipGraphBeginCapture and End a null stream is the capturing stream itself: the launches become nodes of
+  // that graph (the call leaves no record for the kernel-by-kernel plan, so such a recording replays as a graph only)
   ND4J_REQUIRE(dX != nullptr && dZ != nullptr, "nd4jhipReduceSameScalarNoAlloc: null device pointer");
   const DataType dt = (DataType)dataType;
   ND4J_REQUIRE(isFloatType(dt), "nd4jhipReduceSameScalarNoAlloc: FLOAT, DOUBLE, HALF or BFLOAT16 arrays only");

@@ -516,6 +516,18 @@ __device__ __forceinline__ double block_sum(double v, double* lds) {
   __syncthreads();
   return r;
 }
+__device__ __forceinline__ double block_max(double v, double* lds) {
+  const int t = threadIdx.x;
+  lds[t] = v;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if (t < w) lds[t] = fmax(lds[t], lds[t + w]);
+    __syncthreads();
+  }
+  const double r = lds[0];
+  __syncthreads();
+  return r;
+}
 __device__ __forceinline__ double misc_result(const MiscArgs& a, double n, double mean, double m2, double cnt) {
   switch (a.kind) {
     case M_VARIANCE: case M_STDDEV: {
@@ -538,6 +550,14 @@ __device__ __forceinline__ double misc_result(const MiscArgs& a, double n, doubl
     case M3_HAMMING: return mean / n;
     case M3_EQUALS_EPS: return mean > 0.0 ? 0.0 : 1.0;            // mean counts the pairs further apart than the tolerance
     case M_NORMP: return pow(cnt, 1.0 / a.param);                 // ops.h:1280-1286
+    case M_REDUCE_FLOAT: {                                        // the post-processing steps of ops.h:1216-1297,1956-1975,2147-2155,2370-2377
+      const int rk = (int)a.param;
+      if (rk == R_MEAN || rk == R_AMEAN) return cnt / n;
+      if (rk == R_NORM2) return sqrt(cnt);
+      if (rk == R_ENTROPY || rk == R_SHANNON_ENTROPY) return -cnt;
+      if (rk == R_LOG_ENTROPY) return log(-cnt);
+      return cnt;                                                 // Norm1, NormMax, SquaredNorm
+    }
     default: return cnt;
   }
 }
@@ -579,6 +599,27 @@ __global__ __launch_bounds__(256) void misc_partial(MiscArgs a, const void* __re
     double d2 = 0.0;
     for (LongType q = j0 + threadIdx.x; q < j1; q += 256) { const double d = at(q) - mean; d2 += d * d; }
     m2 = block_sum(d2, lds);
+  } else if (a.kind == M_REDUCE_FLOAT) {
+    const int rk = (int)a.param;
+    double c = 0.0;
+    for (LongType q = j0 + threadIdx.x; q < j1; q += 256) {
+      const double v = at(q);
+      switch (rk) {
+        case R_AMEAN: case R_NORM1: c += fabs(v); break;
+        case R_NORMMAX: c = fmax(c, fabs(v)); break;
+        case R_NORM2: case R_SQNORM: c += v * v; break;
+        // the logarithm is taken in X's own type (sd_log<X, Z> casts p_log<X>'s result, templatemath.h:287-299); ShannonEntropy
+        // forms the product in Z (ops.h:1956-1963)
+        case R_ENTROPY: case R_LOG_ENTROPY: c += v * (a.xdt == DOUBLE ? log(v) : (double)round_as(logf((float)v), a.xdt)); break;
+        case R_SHANNON_ENTROPY: {
+          const double pr = v * (a.xdt == DOUBLE ? log2(v) : (double)round_as(log2f((float)v), a.xdt));
+          c += a.zdt == DOUBLE ? pr : (double)round_as((float)pr, a.zdt);
+          break;
+        }
+        default: c += v; break;   // Mean
+      }
+    }
+    cnt = rk == R_NORMMAX ? block_max(c, lds) : block_sum(c, lds);
   } else {
     double c = 0.0;
     for (LongType q = j0 + threadIdx.x; q < j1; q += 256) {
@@ -618,7 +659,8 @@ __global__ __launch_bounds__(256) void misc_finish(MiscArgs a, const double* __r
       mean += delta * nb / tot;
       n = tot;
     }
-    cnt += p[3];
+    if (a.kind == M_REDUCE_FLOAT && (int)a.param == R_NORMMAX) cnt = fmax(cnt, p[3]);
+    else cnt += p[3];
   }
   store_any(z, a.zdt, walk<LongType>(a.zOuter, row), misc_result(a, n, mean, m2, cnt));
 }

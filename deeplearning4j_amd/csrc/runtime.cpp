@@ -121,6 +121,25 @@ bool deviceAvailable() {
   return available;
 }
 
+namespace {
+struct AttrRegistry {
+  std::mutex m;
+  std::vector<void (*)()> setters;
+  size_t applied = 0;
+};
+AttrRegistry& attrRegistry() { static AttrRegistry* r = new AttrRegistry(); return *r; }   // outlives every static that registers
+}
+void registerKernelAttribute(void (*apply)()) {
+  AttrRegistry& r = attrRegistry();
+  std::lock_guard<std::mutex> g(r.m);
+  r.setters.push_back(apply);
+}
+void applyKernelAttributes() {
+  AttrRegistry& r = attrRegistry();
+  std::lock_guard<std::mutex> g(r.m);
+  while (r.applied < r.setters.size()) r.setters[r.applied++]();
+}
+
 void LaunchContext::init() {
   if (ready) return;
   if (!deviceAvailable())
@@ -133,6 +152,7 @@ void LaunchContext::init() {
   HIP_CHECK(hipHostMalloc(&scalarBuffer, 256, hipHostMallocDefault));
   HIP_CHECK(hipEventCreateWithFlags(&bridgeIn, hipEventDisableTiming));
   HIP_CHECK(hipEventCreateWithFlags(&bridgeOut, hipEventDisableTiming));
+  applyKernelAttributes();
   ready = true;
 }
 static LaunchContext g_defaultContext;

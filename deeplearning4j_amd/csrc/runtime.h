@@ -128,6 +128,30 @@ struct NDArray {
   template <typename T> T* hostAs() const { return reinterpret_cast<T*>(buffer()); }
 };
 
+// ---- kernels that ask for more dynamic LDS than the default limit -----------------------------------------------------
+// Such a kernel needs one hipFuncSetAttribute call before its first launch.  Every instantiation the dispatchers can pick
+// registers its setter when the library is loaded (DynLds below), and the launch context runs all of them when it is
+// created, so that no attribute call can fire for the first time between the Begin and End of a stream capture.
+void registerKernelAttribute(void (*apply)());
+void applyKernelAttributes();   // runs the setters registered so far that have not run yet (the device must be current)
+template <auto Kern, int BYTES>
+struct DynLds {
+  static bool granted_;
+  static const bool registered_;
+  static void apply() {
+    granted_ = hipFuncSetAttribute(reinterpret_cast<const void*>(Kern), hipFuncAttributeMaxDynamicSharedMemorySize, BYTES) == hipSuccess;
+    if (!granted_) (void)hipGetLastError();
+  }
+  // did the device grant this kernel BYTES of dynamic LDS
+  static bool granted() {
+    (void)registered_;          // forces the registration of this instantiation at load time
+    applyKernelAttributes();    // a no-op once the launch context exists
+    return granted_;
+  }
+};
+template <auto Kern, int BYTES> bool DynLds<Kern, BYTES>::granted_ = false;
+template <auto Kern, int BYTES> const bool DynLds<Kern, BYTES>::registered_ = (registerKernelAttribute(&DynLds<Kern, BYTES>::apply), true);
+
 // ---- stream capture ---------------------------------------------------------------------------------
 // While a capture is open, ops record their kernels instead of running them, and prepare/registerSpecialUse note which
 // buffers the recorded kernels read and write, so that a replay can bring inputs up to date and stamp outputs.

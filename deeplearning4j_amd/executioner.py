@@ -34,6 +34,7 @@ class TransformStrict:
     TanhDerivative, SigmoidDerivative, SoftSignDerivative, TanDerivative, SELUDerivative = 4, 6, 7, 8, 9
     RationalTanhDerivative, RectifiedTanhDerivative, SwishDerivative, ACoshDerivative, ASinhDerivative = 11, 12, 13, 14, 15
     SinhDerivative, LogSigmoidDerivative, SpecialDerivative, CubeDerivative = 16, 17, 18, 21
+    HardTanhDerivative, HardSigmoidDerivative, StabilizeFP16 = 5, 10, 20   # the first two return their input (ops/ops.h:222-226)
     ACos, ASin, ATan, HardTanh, SoftSign, HardSigmoid, RationalTanh, RectifiedTanh, Sinh, Cosh, Tan, SELU = 30, 31, 32, 33, 34, 36, 37, 38, 39, 40, 41, 42
     Log1p, ACosh, ASinh, Rint, LogSigmoid, Erfc, Expm1, ATanh, GELUDerivative, PreciseGELUDerivative, Mish, MishDerivative = 44, 46, 47, 48, 49, 50, 51, 52, 54, 56, 57, 58
 
@@ -45,6 +46,7 @@ class TransformFloat:
 class TransformSame:
     Abs, Ones, Neg, Round, TimesOneMinus, Cube, OneMinus, Reciprocal, Square, Identity, Ceiling, Floor, Copy = 0, 2, 3, 4, 5, 6, 7, 11, 12, 15, 17, 18, 21
     CompareAndSetTransform = 13   # extraArgs [compare, set, eps, mode]
+    Sign = 1   # as the reference computes it: 1 for every non-zero number, -1 for 0 and NaN (ops/ops.h:217-219)
 
 
 class ReduceSame:
@@ -104,6 +106,9 @@ class Broadcast:
     MinPairwise, MaxPairwise, AMinPairwise, AMaxPairwise, SquaredSubtract, FloorMod, FloorDiv, ReverseMod = 13, 14, 15, 16, 17, 18, 19, 20
     SafeDivide, Mod, TruncateDiv, Atan2, LogicalOr, LogicalXor, LogicalNot, LogicalAnd, DivideNoNan = 21, 22, 23, 26, 27, 28, 29, 30, 31
     IGamma, IGammac, PowDerivative = 32, 33, 34
+
+
+_FLOAT_TYPES = (HALF, FLOAT32, DOUBLE, BFLOAT16)
 
 
 def _reduced_shape(shape, dims, keep_dims):
@@ -208,7 +213,9 @@ class Executioner:
         return z
 
     def exec_transform_float(self, op_num, x, z=None):
-        z = z if z is not None else NDArray.empty(x.shape, x.dtype)
+        # the result of a float transform or reduction of an integer / bool array takes the default floating point type, as
+        # Op.resultType() gives it on the Java side
+        z = z if z is not None else NDArray.empty(x.shape, x.dtype if x.dtype in _FLOAT_TYPES else FLOAT32)
         self.L.execTransformFloat(None, op_num, x.handle, None, z.handle)
         N.check("execTransformFloat")
         return z
@@ -305,8 +312,8 @@ class Executioner:
 
     def exec_reduce_float(self, op_num, x, dims=None, keep_dims=False, z=None, extra_args=None):
         """extra_args reach the native side in Z's type (NormP's exponent)."""
-        zdt = z.dtype if z is not None else x.dtype
-        return self._reduce(self.L.execReduceFloat, self.L.execReduceFloat2, "execReduceFloat", op_num, x, dims, keep_dims, z, x.dtype, extra_args, zdt)
+        zdt = z.dtype if z is not None else (x.dtype if x.dtype in _FLOAT_TYPES else FLOAT32)
+        return self._reduce(self.L.execReduceFloat, self.L.execReduceFloat2, "execReduceFloat", op_num, x, dims, keep_dims, z, zdt, extra_args, zdt)
 
     def exec_index_reduce(self, op_num, x, dims=None, keep_dims=False, z=None, extra_args=None):
         return self._reduce(self.L.execIndexReduceScalar, self.L.execIndexReduce, "execIndexReduce", op_num, x, dims, keep_dims, z, INT64, extra_args)

@@ -184,6 +184,36 @@ _SIGS = {
     "nd4jhipLastGemmKernel": (ctypes.c_char_p, []),
     "nd4jhipReduceSameScalarNoAlloc": (ctypes.c_int, [c_ptr, ctypes.c_int, ctypes.c_int, c_ptr, c_long, c_ptr]),
     "setGraphContextCudaContext": (None, [c_ptr, c_ptr, c_ptr, c_ptr]),
+    "nd4jhipProfilerAttached": (ctypes.c_int, []),
+    "nd4jhipGraphAudit": (ctypes.c_int, [c_ptr]),
+    "lcSolverHandle": (c_ptr, [c_ptr]),
+    "lcScalarPointerPtr": (c_ptr, [ctypes.POINTER(c_ptr)]),
+    "lcReductionPointerPtr": (c_ptr, [ctypes.POINTER(c_ptr)]),
+    "lcAllocationPointerPtr": (c_ptr, [ctypes.POINTER(c_ptr)]),
+    "lcExecutionStreamPtr": (c_ptr, [ctypes.POINTER(c_ptr)]),
+    "lcCopyStreamPtr": (c_ptr, [ctypes.POINTER(c_ptr)]),
+    "lcBlasHandlePtr": (c_ptr, [ctypes.POINTER(c_ptr)]),
+    "checkP2P": (None, []),
+    "enableP2P": (None, [ctypes.c_bool]),
+    "isP2PAvailable": (ctypes.c_bool, []),
+    "initializeFunctions": (None, [ctypes.POINTER(c_ptr)]),
+    "isBlasVersionMatches": (ctypes.c_bool, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "binaryLevel": (ctypes.c_int, []),
+    "optimalLevel": (ctypes.c_int, []),
+    "isMinimalRequirementsMet": (ctypes.c_bool, []),
+    "isOptimalRequirementsMet": (ctypes.c_bool, []),
+    "isExperimentalEnabled": (ctypes.c_bool, []),
+    "setOmpMinThreads": (None, [ctypes.c_int]),
+    "setGridLimit": (None, [ctypes.c_int]),
+    "getConstantSpace": (c_ptr, []),
+    "execRandom": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr]),
+    "execRandom2": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "execRandom3": (None, [c_ptr, ctypes.c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "sort": (None, [c_ptr, c_ptr, ctypes.c_bool]),
+    "sortTad": (None, [c_ptr, c_ptr, LongPtr, c_long, LongPtr, LongPtr, ctypes.c_bool]),
+    "shuffle": (None, [c_ptr, c_ptr, c_ptr, ctypes.c_int, c_ptr, c_ptr]),
+    "pullRows": (None, [c_ptr, c_ptr, c_ptr, c_long, c_ptr, c_long]),
+    "convertTypes": (None, [c_ptr, ctypes.c_int, c_ptr, c_long, ctypes.c_int, c_ptr]),
 }
 
 

@@ -7,8 +7,8 @@
  * with opaque handle types so that any FFI (JavaCPP, JNI, ctypes) can bind them.  Two consequences:
  *   - the reference's C++ overload getShapeInfoLength(OpaqueNDArray) gets the distinct name
  *     getOpaqueNDArrayShapeInfoLength, and of the two lc* overload sets (by value :451-457, by pointer
- *     :500-512) only the by-value one is exported; everything else keeps its name, argument order and
- *     meaning;
+ *     :500-512) the by-value one keeps the names while the by-pointer one carries the suffix "Ptr"
+ *     (lcScalarPointerPtr ...); everything else keeps its name, argument order and meaning;
  *   - handles are plain pointers: OpaqueNDArray = array handle created by createOpaqueNDArray,
  *     OpaqueDataBuffer = host+device buffer pair, OpaqueContext = per-op argument bag.
  *
@@ -104,6 +104,40 @@ ND4JHIP_EXPORT Nd4jPointer lcAllocationPointer(OpaqueLaunchContext lc);         
 ND4JHIP_EXPORT Nd4jPointer lcExecutionStream(OpaqueLaunchContext lc);                  /* ref :454 */
 ND4JHIP_EXPORT Nd4jPointer lcCopyStream(OpaqueLaunchContext lc);                       /* ref :455 */
 ND4JHIP_EXPORT Nd4jPointer lcBlasHandle(OpaqueLaunchContext lc);                       /* ref :456 (no vendor BLAS is used: returns NULL) */
+ND4JHIP_EXPORT Nd4jPointer lcSolverHandle(OpaqueLaunchContext lc);                     /* ref :457 (no vendor solver is used: returns NULL) */
+/* the reference's second overload set takes a pointer to the handle (what defaultLaunchContext's Java wrapper holds) */
+ND4JHIP_EXPORT Nd4jPointer lcScalarPointerPtr(OpaqueLaunchContext* lc);                /* ref :502 */
+ND4JHIP_EXPORT Nd4jPointer lcReductionPointerPtr(OpaqueLaunchContext* lc);             /* ref :504 */
+ND4JHIP_EXPORT Nd4jPointer lcAllocationPointerPtr(OpaqueLaunchContext* lc);            /* ref :506 */
+ND4JHIP_EXPORT Nd4jPointer lcExecutionStreamPtr(OpaqueLaunchContext* lc);              /* ref :508 */
+ND4JHIP_EXPORT Nd4jPointer lcCopyStreamPtr(OpaqueLaunchContext* lc);                   /* ref :510 */
+ND4JHIP_EXPORT Nd4jPointer lcBlasHandlePtr(OpaqueLaunchContext* lc);                   /* ref :512 */
+
+/* what a device backend asks at start-up (AtomicAllocator.java:140, CudaAffinityManager.java:353,
+ * CudaExecutioner's static initialiser) */
+ND4JHIP_EXPORT void checkP2P(void);                                                    /* ref :222 */
+ND4JHIP_EXPORT void enableP2P(bool enable);                                            /* ref :223 */
+ND4JHIP_EXPORT bool isP2PAvailable(void);                                              /* ref :224 (one device counts as available, ref legacy/cuda/NativeOps.cu:1046-1049) */
+ND4JHIP_EXPORT void initializeFunctions(Nd4jPointer* functions);                       /* ref :226 (host BLAS pointers; unused here) */
+ND4JHIP_EXPORT bool isBlasVersionMatches(int major, int minor, int build);             /* ref :398 (no vendor BLAS to mismatch: true) */
+ND4JHIP_EXPORT int binaryLevel(void);                                                  /* ref :460 */
+ND4JHIP_EXPORT int optimalLevel(void);                                                 /* ref :461 */
+ND4JHIP_EXPORT bool isMinimalRequirementsMet(void);                                    /* ref :462 */
+ND4JHIP_EXPORT bool isOptimalRequirementsMet(void);                                    /* ref :463 */
+ND4JHIP_EXPORT bool isExperimentalEnabled(void);                                       /* ref :316 */
+ND4JHIP_EXPORT void setOmpMinThreads(int threads);                                     /* ref :317 (no-op) */
+ND4JHIP_EXPORT void setGridLimit(int gridSize);                                        /* ref :275 (no-op: grids follow the problem) */
+ND4JHIP_EXPORT Nd4jPointer getConstantSpace(void);                                     /* ref :315 (no constant-memory staging area: NULL) */
+/* entry points of the reference that lie outside this backend's path: exported so that a binding resolves them; each
+ * sets the error slot to "... is not implemented in nd4j-hip" and does nothing else */
+ND4JHIP_EXPORT void execRandom(Nd4jPointer* extraPointers, int opNum, Nd4jPointer stateHost, OpaqueNDArray z, void* extraArguments);                  /* ref :166 */
+ND4JHIP_EXPORT void execRandom2(Nd4jPointer* extraPointers, int opNum, Nd4jPointer stateHost, OpaqueNDArray x, OpaqueNDArray z, void* extraArguments); /* ref :168 */
+ND4JHIP_EXPORT void execRandom3(Nd4jPointer* extraPointers, int opNum, Nd4jPointer stateHost, OpaqueNDArray x, OpaqueNDArray y, OpaqueNDArray z, void* extraArguments); /* ref :170 */
+ND4JHIP_EXPORT void sort(Nd4jPointer* extraPointers, OpaqueNDArray x, bool descending);                                                               /* ref :343 */
+ND4JHIP_EXPORT void sortTad(Nd4jPointer* extraPointers, OpaqueNDArray x, Nd4jLong* dimension, Nd4jLong dimensionLength, Nd4jLong* tadShapeInfo, Nd4jLong* tadOffsets, bool descending); /* ref :344 */
+ND4JHIP_EXPORT void shuffle(Nd4jPointer* extras, OpaqueNDArrayArr x, OpaqueNDArrayArr z, int N, OpaqueNDArray dimension, OpaqueNDArray shuffleMap);   /* ref :84 */
+ND4JHIP_EXPORT void pullRows(Nd4jPointer* extraPointers, OpaqueNDArray x, OpaqueNDArray z, Nd4jLong n, OpaqueNDArray indexes, Nd4jLong dimension);    /* ref :95 */
+ND4JHIP_EXPORT void convertTypes(Nd4jPointer* extras, int srcType, Nd4jPointer dX, Nd4jLong N, int dstType, Nd4jPointer dZ);                         /* ref :390 */
 
 /* ---- data buffers (ref :466-488) ------------------------------------------------------------------- */
 ND4JHIP_EXPORT OpaqueDataBuffer* dbAllocateDataBuffer(Nd4jLong elements, int dataType, bool allocateBoth);        /* ref :487 */
@@ -249,6 +283,11 @@ ND4JHIP_EXPORT void nd4jhipSetSyncAfterCustomOp(int enable);
  * call between Begin and End is recorded on the execution stream instead of run; End returns a handle (null + error slot
  * when an op waited on the stream, copied synchronously or allocated, which invalidates a capture); Launch replays the
  * recorded kernels with the arguments they were recorded with.  Build arrays, views and OpContexts before Begin.
+ * Handle lifetime: every recorded call copies its array views (shape, strides, offset; the DataBuffers are shared) the
+ * moment it is recorded, so array handles and OpContexts may be deleted right after the op call that used them, before
+ * End; the DataBuffers must outlive the graph.  memcpyAsync (device to device) and memsetAsync on the library's stream
+ * (a null `reserved`, or what lcExecutionStream returned) between Begin and End are recorded too and replay in both
+ * replay modes; a copy that touches host memory there is an error.
  * Launch keeps the buffers' host/device stamps as the recorded op calls would: a buffer the graph reads whose host copy
  * is newer is uploaded first, and every buffer the graph writes counts as device-written afterwards, so dbSyncToPrimary
  * after a replay returns that replay's values.  A capture is process-wide: ops other threads issue between Begin and End
@@ -271,9 +310,18 @@ ND4JHIP_EXPORT int nd4jhipGraphFusedOps(Nd4jPointer graph);
  * plain launch it is also the faster of the two.  A recording made while some call went unrecorded has no such sequence
  * and is always launched as a graph.  The recording keeps its own views of the arrays (the buffers are shared), so the
  * caller's array handles may go away in either mode; the buffers may not.  The setting is process-wide and read at
- * every launch; it starts as 0, or 1 when ND4JHIP_GRAPH_REPLAY=kernels is in the environment. */
+ * every launch; it starts as 0, or 1 when ND4JHIP_GRAPH_REPLAY=kernels is in the environment.
+ * One exception to mode 0: when a rocprofiler tool library is attached to the process (ROCP_TOOL_LIBRARIES or LD_PRELOAD
+ * names it, or it is among the loaded objects -- nd4jhipProfilerAttached() returns 1), nd4jhipGraphLaunch replays the
+ * recorded plan as in mode 1 whatever the setting, and fails for a recording that has no plan: a graph launch under the
+ * kernel tracer once aborted the queue, the cause was never established, and the library keeps callers off that path. */
 ND4JHIP_EXPORT void nd4jhipSetGraphReplayMode(int mode);
 ND4JHIP_EXPORT int nd4jhipGetGraphReplayMode(void);
+ND4JHIP_EXPORT int nd4jhipProfilerAttached(void);
+/* Host-side audit of a recording: walks the graph's kernel nodes and checks each one's block size, dynamic LDS request and
+ * grid against what the runtime reports for the function and the device.  Launches nothing.  Returns the number of nodes
+ * that break a limit (described in the error slot), 0 for a clean graph, -1 when the graph cannot be walked. */
+ND4JHIP_EXPORT int nd4jhipGraphAudit(Nd4jPointer graph);
 ND4JHIP_EXPORT const char* nd4jhipBuildInfo(void);
 /* Name ("family<type,tile,flags>") of the kernel the calling thread's most recent matmul / xw_plus_b launched; lets a
  * test assert that its shape reached the instantiation it means to check. */
@@ -287,7 +335,10 @@ ND4JHIP_EXPORT const char* nd4jhipLastGemmKernel(void);
  * The cross-block partials go to a fixed 64 KiB device array inside the library (one copy per device, held until the
  * process ends) instead of allocated scratch, and the call allocates nothing, on the error paths either.  Limits:
  * 1 <= length <= 2^31 - 1 (larger: error); initializeDevicesAndFunctions must have run (it allocates; this call
- * refuses to); calls that overlap on one device share the array and race.  Returns 0, or 1 with the error slot set. */
+ * refuses to); calls that overlap on one device share the array and race.  Under a caller's own stream capture pass
+ * that stream; between nd4jhipGraphBeginCapture and End a null stream is the capturing stream, and the launches become
+ * nodes of that recording (which then replays as a graph only: the call leaves no step in the kernel-by-kernel plan).
+ * Returns 0, or 1 with the error slot set. */
 ND4JHIP_EXPORT int nd4jhipReduceSameScalarNoAlloc(Nd4jPointer stream, int opNum, int dataType, const void* dX, Nd4jLong length, void* dZ);
 
 #ifdef __cplusplus

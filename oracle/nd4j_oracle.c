@@ -302,11 +302,16 @@ static inline double ref_sigmoidd(double x) { return 1.0 / (1.0 + exp(-x)); }
 /* The rest of the TransformStrict table (loops/legacy_ops.h:54-64), restated from ops/ops.h and
  * math/templatemath.h (lines beside each case).  One body, expanded for float (libm *f functions, as the
  * reference's float path uses) and for double.  Not restated: 2 ScaledTanh, 3 Affine, 19 Stabilize, 25 SetRange
- * (extra parameters), 5 HardTanhDerivative, 10 HardSigmoidDerivative (their macros return the input), 20. */
+ * (extra parameters).  5 HardTanhDerivative and 10 HardSigmoidDerivative are declared through DECLARE_UNARY_CONDITIONAL_OP
+ * (ops/op_macros_unary.h:109-113: (CONDITION) ? (TRUE_VAL) : (FALSE_VAL)) with the derivative's expression as the
+ * CONDITION and d1 as both values (ops.h:222-226), so both return their input; 20 StabilizeFP16 (ops.h:381-384) returns
+ * float16's smallest normal number, 2^-14 (DataTypeUtils::min<float16>, array/DataTypeUtils.h:463-465), for x <= 0. */
 #define SELU_A 1.6732632423543772848170429916717
 #define SELU_L 1.0507009873554804934193349852946
 #define STRICT_TAIL(T, M, TANH, SIGM)                                                                         \
   switch (op) {                                                                                               \
+    case 5: case 10: *out = x; return 0;                                      /* ops.h:222-226 */            \
+    case 20: *out = x <= (T)0 ? (T)6.103515625e-05 : x; return 0;             /* ops.h:381-384 */            \
     case 4: { T t = TANH(x); *out = (T)1 - t * t; return 0; }                 /* templatemath.h:335-339 */   \
     case 6: { T g = SIGM(x); *out = g * ((T)1 - g); return 0; }               /* templatemath.h:343-347 */   \
     case 7: { T y = (T)1 + M(fabs)(x); *out = (T)1 / (y * y); return 0; }     /* templatemath.h:351-355 */   \
@@ -466,11 +471,14 @@ int orc_transform_float(int opNum, const void *x, const int64_t *xsi, void *z, c
   return 0;
 }
 
-/* TransformSame: loops/legacy_ops.h:40-44; functors ops/ops.h:192-207,359,481,1165.  Not restated: 1 Sign (its
- * macro yields +1 for every non-zero input), 13 CompareAndSetTransform and 19 ClipByValue (extra parameters). */
+/* TransformSame: loops/legacy_ops.h:40-44; functors ops/ops.h:192-207,359,481,1165.  1 Sign is declared through
+ * DECLARE_UNARY_CONDITIONAL_OP with the sign expression (d1 > 0) - (d1 < 0) as the CONDITION and 1 / -1 as the values
+ * (ops.h:217-219): 1 for every non-zero number, -1 for zero and NaN.  Not restated here: 13 CompareAndSetTransform and
+ * 19 ClipByValue (extra parameters; oracle.py holds them). */
 static int same_d(int op, double x, double *out) {
   switch (op) {
     case 0: *out = fabs(x); return 0;
+    case 1: *out = ((x > 0.0) - (x < 0.0)) ? 1.0 : -1.0; return 0;
     case 2: *out = 1.0; return 0;
     case 3: *out = -x; return 0;
     case 4: *out = round(x); return 0;           /* p_round = round(): halves away from zero */
@@ -488,6 +496,7 @@ static int same_d(int op, double x, double *out) {
 static int same_f(int op, float x, float *out) {
   switch (op) {
     case 0: *out = fabsf(x); return 0;
+    case 1: *out = ((x > 0.0f) - (x < 0.0f)) ? 1.0f : -1.0f; return 0;
     case 2: *out = 1.0f; return 0;
     case 3: *out = -x; return 0;
     case 4: *out = roundf(x); return 0;
@@ -771,7 +780,9 @@ static inline int64_t walk(int rank, const int64_t *shape, const int64_t *stride
 /* ReduceSame: 0 Sum 1 Max 2 Min 3 Prod 4 ASum 5 AMax 6 AMin   loops/legacy_ops.h:100-101; ops/ops.h:2363-2368,1170-1243
  * ReduceFloat: 0 Mean 1 AMean 2 Norm1 3 Norm2 4 NormMax 7 SquaredNorm 8 Entropy 9 LogEntropy 10 ShannonEntropy
  *   legacy_ops.h:103-105; ops.h:2370-2378,1217-1298,1956-1973,2147-2153
- * accumulator type = float for float/half/bf16 (InterType, ops/op_types.h:213-226), double for double. */
+ * accumulator type = float for float/half/bf16 (InterType, ops/op_types.h:213-226), double for double; the ReduceFloat
+ * ops take it from Z (op_macros_reduce.h:778-782), and X may be any numeric type there
+ * (NativeOpExecutioner_reduce.cpp:34-37,104-106: SD_NUMERIC_TYPES x SD_FLOAT_TYPES). */
 #define RED_BODY(ACC_T, LOAD, ABS, SQRT, INF, LOG, LOG2, RX, RZ)                                                        \
   ACC_T s;                                                                                              \
   switch (kind) {                                                                                       \
@@ -802,7 +813,8 @@ static inline int64_t walk(int rank, const int64_t *shape, const int64_t *stride
     case 10: case 11: s = s / (ACC_T)p.ilen; break;                                                     \
     case 13: s = SQRT(s); break;                                                                        \
     case 18: case 20: s = -s; break;                                                                    \
-    case 19: s = LOG(-s); break;                                                                        \
+    /* sd_log<InterType, Z>(-reduction): this logarithm is the accumulator type's (ops.h:1966-1973) */  \
+    case 19: s = sizeof(ACC_T) == 8 ? (ACC_T)log((double)-s) : (ACC_T)logf((float)-s); break;           \
   }
 
 static int reduce_impl(int kind, const void *x, const int64_t *xsi, void *z, const int64_t *zsi, const int64_t *dims,
@@ -819,10 +831,13 @@ static int reduce_impl(int kind, const void *x, const int64_t *xsi, void *z, con
   for (int64_t o = 0; o < p.olen; o++) {
     int64_t base = walk(p.orank, p.oshape, p.ostride, o);
     int64_t zo = walk(zr, zshape, zstride, o);
-    if (xdt == ORC_DOUBLE) {
-#define LOADD(j) (((const double *)x)[base + walk(p.irank, p.ishape, p.istride, (j))])
+    if (kind >= 10 ? zdt == ORC_DOUBLE : xdt == ORC_DOUBLE) {
+#define LOADD(j) (ld(x, xdt, base + walk(p.irank, p.ishape, p.istride, (j))))
 #define NOROUND(v) (v)
-      RED_BODY(double, LOADD, fabs, sqrt, INFINITY, log, log2, NOROUND, NOROUND)
+/* the logarithm is taken in X's own type whatever the accumulator is (sd_log<X, Z> casts p_log<X>'s result, templatemath.h:287-299) */
+#define LOGX(v) (xdt == ORC_DOUBLE ? log(v) : (double)rnd(logf((float)(v)), xdt))
+#define LOG2X(v) (xdt == ORC_DOUBLE ? log2(v) : (double)rnd(log2f((float)(v)), xdt))
+      RED_BODY(double, LOADD, fabs, sqrt, INFINITY, LOGX, LOG2X, NOROUND, NOROUND)
       st(z, zdt, zo, s);
     } else {
 #define LOADF(j) (ldf(x, xdt, base + walk(p.irank, p.ishape, p.istride, (j))))
@@ -847,7 +862,7 @@ int orc_reduce_same(int opNum, const void *x, const int64_t *xsi, void *z, const
  *   -> NativeOpExecutioner_reduce.cpp:98-120 -> loops/cpu/reduce/reduce_float.hpp:79-175,220-289 */
 int orc_reduce_float(int opNum, const void *x, const int64_t *xsi, void *z, const int64_t *zsi, const int64_t *dims,
                      int ndims) {
-  if (!dt_is_float(orc_dtype(zsi)) || !dt_is_float(orc_dtype(xsi))) return 2;
+  if (!dt_is_float(orc_dtype(zsi)) || dt_size(orc_dtype(xsi)) == 0) return 2;
   switch (opNum) {
     case 0: return reduce_impl(10, x, xsi, z, zsi, dims, ndims);
     case 1: return reduce_impl(11, x, xsi, z, zsi, dims, ndims);

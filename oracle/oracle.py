@@ -239,6 +239,67 @@ def reduce_float(op, x, z, dims=None):
     return _reduce(lib().orc_reduce_float, "reduce_float", op, x, z, dims)
 
 
+def reduce_of_empty(table, op, x_dtype, z_dtype):
+    """What every element of Z holds after a reduction of an EMPTY X: the op's starting value
+    (loops/cpu/reduce/reduce_same.hpp:47,166-176; reduce_float.hpp:103-106,243-251; reduce_long.hpp:50-53,212-217;
+    reduce_bool.hpp:45-48; indexreduce.hpp:106-113 with ops/op_macros_index_reduce.h:46-51 and ops.h:2079-2085,2123-2129).
+    table: "same", "float", "long", "bool", "index".  Starting values: Sum / ASum 0, Prod 1 (ops.h:2363-2364,1170), Max / Min
+    -+infOrMax<X> (ops.h:2365-2368) where infOrMax is infinity for float and double only and the largest finite value for
+    every other type, float16 (65504) and bfloat16 included (array/DataTypeUtils.h:588-617); Mean nanOrZero<Z>, NaN for float
+    and double only (reduce_float.hpp:244-246, DataTypeUtils.h:619-636); every other ReduceFloat op 0; counts 0; Any 0, All 1
+    (ops.h:1200-1215), the other ReduceBool ops 0; IndexMax / IndexMin ... index 0, FirstIndex / LastIndex -1.
+    AMax / AMin (ops.h:1225-1243) and the summary statistics start from x[0], which does not exist: None.
+    x_dtype / z_dtype: numpy dtypes, or the strings "bfloat16" / "float16"."""
+    xk, zk = str(x_dtype), str(z_dtype)
+
+    def largest(kind):
+        if kind in ("float32", "float64"):
+            return np.inf
+        if kind == "float16":
+            return 65504.0
+        if kind == "bfloat16":
+            return float(bf16_to_f32(np.array([0x7F7F], np.uint16))[0])
+        if kind == "bool":
+            return 1
+        return np.iinfo(np.dtype(kind)).max
+
+    if table == "same":
+        if op in (0, 4):
+            return 0
+        if op == 3:
+            return 1
+        if op == 1:
+            return -largest(xk)
+        if op == 2:
+            return largest(xk)
+        return None
+    if table == "float":
+        if op == 0:
+            return np.nan if zk in ("float32", "float64") else 0.0
+        return 0.0
+    if table == "long":
+        return 0
+    if table == "bool":
+        return 1 if op == 1 else 0
+    if table == "index":
+        return -1 if op in (4, 5) else 0
+    raise ValueError(table)
+
+
+def matmul_int(x, y, z=None, alpha=1.0, beta=0.0):
+    """matmul of integer arrays: the reference's plain loop in the arrays' own type (helpers/cpu/MmulHelper.cpp:35-110:
+    val += A * B in T3, then alphaZ * val (+ betaZ * C) with alpha and beta cast to T3).  numpy's integer matmul wraps
+    around the same way; 32-bit arrays are widened first and narrowed at the end, which gives the same residues."""
+    x, y = np.asarray(x), np.asarray(y)
+    assert x.dtype == y.dtype and x.dtype in (np.int32, np.int64)
+    with np.errstate(over="ignore"):
+        v = np.matmul(x.astype(np.int64), y.astype(np.int64))
+        out = np.int64(int(alpha)) * v
+        if beta:
+            out = out + np.int64(int(beta)) * np.asarray(z).astype(np.int64)
+    return out.astype(x.dtype)
+
+
 def index_reduce(op, x, z, dims=None):
     return _reduce(lib().orc_index_reduce, "index_reduce", op, x, z, dims)
 
@@ -634,7 +695,7 @@ def bool_table(op, x, y, params=None, bf16=False):
     of one dtype and one shape (see operand_along / scalars_along for the operand shapes of the other families); with
     bf16=True they are float32 arrays holding bfloat16 values and differences are rounded to bfloat16.
     0 EqualTo, 1 GreaterThan, 2 LessThan, 4 GreaterThanOrEqual, 6 NotEqualTo, 11 LessThanOrEqual: ops.h:181-186 (x OP y).
-    3 Epsilon (ops.h:1755-1790): |x - y| <= params[0] when parameters are given, else (also) |x - y| <= X(1e-5).
+    3 Epsilon (ops.h:1755-1790): |x - y| <= params[0] when parameters are given, else (also) |x - y| <= X(1e-5); all true for BOOL.
     7 And / 8 Or / 9 Xor (ops.h:1051-1063, 1896-1925): with parameters on "differs from params[0]", without on bool(x), bool(y).
     10 Not (ops.h:1927-1932): the three-argument form is x != y."""
     x, y = np.asarray(x), np.asarray(y)
@@ -644,7 +705,10 @@ def bool_table(op, x, y, params=None, bf16=False):
         if op in (0, 1, 2, 4, 6, 10, 11):
             return {0: x == y, 1: x > y, 2: x < y, 4: x >= y, 6: x != y, 10: x != y, 11: x <= y}[op]
         if op == 3:
-            assert x.dtype != np.bool_
+            if x.dtype == np.bool_:
+                # X = bool: the difference and both tolerances are held as bool, static_cast<bool>(1e-5) is true, and
+                # "absDiff <= true" holds for either value of absDiff: every pair matches
+                return np.ones(x.shape, np.bool_)
             if bf16:
                 diff = bf16_to_f32(f32_to_bf16((x - y).astype(np.float32)))
                 tol = bf16_to_f32(f32_to_bf16(np.array([1e-5], np.float32)))[0]

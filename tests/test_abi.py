@@ -2,11 +2,14 @@
 (op hash, registry listing, descriptor cache, TAD packs, error slot) behaves like the reference's.
 No compute entry point is called here."""
 import ctypes
+import os
 
 import numpy as np
 import pytest
 
 from deeplearning4j_amd import nativeops as N
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def test_library_exports_every_declared_symbol():
@@ -131,3 +134,47 @@ def test_compute_without_gpu_fails_loudly():
     L.initializeDevicesAndFunctions()
     assert L.lastErrorCode() != 0
     assert b"no CPU fallback" in L.lastErrorMessage()
+
+
+def test_start_up_queries_and_out_of_scope_entry_points():
+    # what a device backend asks while it starts (AtomicAllocator.java:140 enableP2P, CudaAffinityManager.java:353
+    # isP2PAvailable, the executioner's version and capability checks): answered without a device
+    L = N.load()
+    L.lastErrorMessage()
+    assert L.isBlasVersionMatches(12, 3, 0) is True        # no vendor BLAS underneath, nothing to mismatch
+    assert (L.binaryLevel(), L.optimalLevel()) == (0, 0)   # legacy/cuda/NativeOps.cu:2769-2775
+    assert L.isMinimalRequirementsMet() and L.isOptimalRequirementsMet() and not L.isExperimentalEnabled()
+    L.initializeFunctions(None); L.setOmpMinThreads(4); L.setGridLimit(128)
+    assert L.getConstantSpace() is None and L.lcSolverHandle(None) is None and L.lcBlasHandlePtr(None) is None
+    L.checkP2P()
+    # fewer than two devices: the reference reports peer access as available (legacy/cuda/NativeOps.cu:1046-1049)
+    if L.getAvailableDevices() < 2:
+        assert L.isP2PAvailable() is True
+    L.enableP2P(True); L.enableP2P(False)
+    assert L.lastErrorCode() == 0
+    # the by-pointer overloads read the handle through the pointer
+    null_handle = ctypes.c_void_p(None)
+    assert L.lcExecutionStreamPtr(ctypes.byref(null_handle)) is None and L.lcScalarPointerPtr(None) is None
+    # entry points outside this backend's path resolve, do nothing and say so in the error slot
+    for name, args in (("execRandom", (None, 0, None, None, None)), ("execRandom2", (None, 0, None, None, None, None)),
+                       ("execRandom3", (None, 0, None, None, None, None, None)), ("sort", (None, None, False)),
+                       ("sortTad", (None, None, None, 0, None, None, False)), ("shuffle", (None, None, None, 0, None, None)),
+                       ("pullRows", (None, None, None, 0, None, 0)), ("convertTypes", (None, 5, None, 0, 6, None))):
+        getattr(L, name)(*args)
+        assert L.lastErrorCode() == 1
+        assert (name + " is not implemented in nd4j-hip").encode() in L.lastErrorMessage()
+
+
+def test_profiler_detection_keeps_graph_launches_off_the_tracer():
+    # nd4jhipGraphLaunch replays kernel by kernel when a rocprofiler tool library is attached; the detection reads the
+    # environment the tool is started with and the list of loaded objects.  Each case in a fresh process.
+    import subprocess
+    import sys
+    code = ("import sys; sys.path.insert(0, %r); from deeplearning4j_amd import nativeops as N; "
+            "print(N.load().nd4jhipProfilerAttached())" % ROOT)
+    def run(extra):
+        env = {k: v for k, v in os.environ.items() if k not in ("ROCP_TOOL_LIBRARIES",)}
+        env.update(extra)
+        return subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=120).stdout.strip().splitlines()[-1]
+    assert run({}) == "0"
+    assert run({"ROCP_TOOL_LIBRARIES": "/opt/rocm/lib/rocprofiler-sdk/librocprofiler-sdk-tool.so"}) == "1"

@@ -77,8 +77,6 @@ def test_reference_vectors(ex, oracle):
 @pytest.mark.parametrize("dt", [FLOAT32, DOUBLE, HALF, BFLOAT16, INT32, INT64, BOOL])
 @pytest.mark.parametrize("op", OPS)
 def test_pairwise_and_scalar_against_the_oracle(ex, oracle, dt, op):
-    if op == BoolOp.Epsilon and dt == BOOL:
-        pytest.skip("Epsilon of BOOL arrays is refused")
     rng = np.random.default_rng(100 * op + dt)
     shape = (37, 53)
     x, X = _values(rng, shape, dt)
@@ -100,8 +98,6 @@ def test_pairwise_and_scalar_against_the_oracle(ex, oracle, dt, op):
     # the ops that read a parameter
     if op in (BoolOp.Epsilon, BoolOp.And, BoolOp.Or, BoolOp.Xor):
         for p0 in ((0.5, 1.0) if op == BoolOp.Epsilon else (1.0, 0.0)):
-            if dt == BOOL and op == BoolOp.Epsilon:
-                continue
             got = ex.exec_pairwise_bool(op, X, Y, extra_args=[p0]).to_numpy()
             assert np.array_equal(got, _want(oracle, op, x, y, dt, [p0])), ("parameter", p0)
 
@@ -109,8 +105,6 @@ def test_pairwise_and_scalar_against_the_oracle(ex, oracle, dt, op):
 @pytest.mark.parametrize("dt", [FLOAT32, BFLOAT16, INT32, BOOL])
 @pytest.mark.parametrize("op", [BoolOp.EqualTo, BoolOp.LessThan, BoolOp.Epsilon, BoolOp.And, BoolOp.Xor, BoolOp.Not, BoolOp.GreaterThanOrEqual])
 def test_broadcast_and_per_sub_array_scalars_against_the_oracle(ex, oracle, dt, op):
-    if op == BoolOp.Epsilon and dt == BOOL:
-        pytest.skip("Epsilon of BOOL arrays is refused")
     rng = np.random.default_rng(7 * op + dt)
     shape = (3, 5, 4, 6)
     x, X = _values(rng, shape, dt)

@@ -114,6 +114,9 @@ def _gpt2_small_graph_replay_matches_eager(ex, gpt2, batch):
     # norms are computed by the products that consume them
     fused = [ex.L.nd4jhipGraphFusedOps(g) for g in dec._graphs.values()]
     assert fused and min(fused) == (7 if batch == 1 else 5) * cfg.n_layer, fused
+    # every kernel node of every recorded step within the limits the runtime reports for its function (host-side walk)
+    for g in dec._graphs.values():
+        assert ex.L.nd4jhipGraphAudit(g) == 0, ex.L.lastErrorMessage()
     stale = dec.logits(1)                                                   # host copy read: a later replay must refresh it
     prompt2 = rng.integers(0, cfg.vocab, (batch, 24))
     want2 = eager.generate(prompt2, 6)

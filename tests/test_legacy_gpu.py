@@ -172,7 +172,7 @@ def test_transform_strict_rejects_type_change(ex):
     with pytest.raises(NativeOpsError, match="same floating point type"):
         ex.exec_transform_strict(TransformStrict.Tanh, NDArray.from_numpy(np.zeros(4, np.float32)), NDArray.empty((4,), DOUBLE))
     with pytest.raises(NativeOpsError, match="not implemented"):
-        ex.exec_transform_strict(20, NDArray.from_numpy(np.zeros(4, np.float32)))      # StabilizeFP16
+        ex.exec_transform_strict(35, NDArray.from_numpy(np.zeros(4, np.float32)))      # no such opNum in the table
     with pytest.raises(NativeOpsError, match="needs one extra parameter"):
         ex.exec_transform_strict(19, NDArray.from_numpy(np.zeros(4, np.float32)))      # Stabilize without its extraArgs
     with pytest.raises(NativeOpsError, match="needs two extra parameters"):

@@ -101,10 +101,10 @@ def test_transform_same_tail(ex, oracle, dtype):
             assert np.array_equal(_got(got, dtype), _f(oz)), "same op %d dtype %d" % (op, dtype)
 
 
-def test_transform_same_rejects_sign(ex):
+def test_transform_same_rejects_unknown_op_numbers(ex):
     from deeplearning4j_amd.nativeops import NativeOpsError
     with pytest.raises(NativeOpsError, match="not implemented"):
-        ex.exec_transform_same(1, NDArray.from_numpy(np.ones(4, np.float32)))
+        ex.exec_transform_same(9, NDArray.from_numpy(np.ones(4, np.float32)))
 
 
 P = Pairwise

@@ -128,8 +128,92 @@ def test_transform_same_ops():
     np.testing.assert_array_equal(same(18), np.floor(x))
     np.testing.assert_array_equal(same(0), np.abs(x))
     np.testing.assert_array_equal(same(6), x ** 3)
-    with pytest.raises(Exception):
-        same(1)        # Sign is deliberately not restated
+    # Sign: the reference's macro takes the sign expression as its CONDITION (ops.h:217-219 through
+    # op_macros_unary.h:109-113), i.e. ((d1 > 0) - (d1 < 0)) ? 1 : -1.  Evaluated by hand: -3 -> (0 - 1) = -1, non-zero -> 1;
+    # 0 -> 0 -> -1; 2 -> 1 -> 1; NaN -> (0 - 0) = 0 -> -1
+    np.testing.assert_array_equal(O.transform_same(1, np.array([-3.0, 0.0, 2.0, np.nan, -0.0]), np.zeros(5)), [1.0, -1.0, 1.0, -1.0, -1.0])
+    np.testing.assert_array_equal(O.transform_same(1, np.array([-3.0, 0.0, 2.0], np.float32), np.zeros(3, np.float32)), [1.0, -1.0, 1.0])
+
+
+def test_strict_ops_whose_macros_return_the_input():
+    # HardTanhDerivative (5) and HardSigmoidDerivative (10): (CONDITION) ? d1 : d1 -- the input whatever the condition says;
+    # StabilizeFP16 (20): x <= 0 ? 2^-14 : x (ops.h:381-384; 2^-14 = 6.103515625e-05 is float16's smallest normal number,
+    # which is what static_cast<float16>(6.1035e-05) rounds to: the neighbouring subnormal 1023 * 2^-24 is 5.96e-8 further away)
+    x = np.array([-3.0, -1.0, -0.5, 0.0, 0.5, 1.0, 2.5, 2.6, 7.0])
+    for dt in (np.float32, np.float64):
+        xt = x.astype(dt)
+        np.testing.assert_array_equal(O.transform_strict(5, xt, np.zeros_like(xt)), xt)
+        np.testing.assert_array_equal(O.transform_strict(10, xt, np.zeros_like(xt)), xt)
+        np.testing.assert_array_equal(O.transform_strict(20, xt, np.zeros_like(xt)), np.where(x <= 0, 2.0 ** -14, x).astype(dt))
+    assert np.float16(6.1035e-05) == np.float16(2.0 ** -14)
+
+
+def test_transform_float_takes_integer_and_bool_inputs():
+    # NativeOpExecutioner_transform.cpp:35-37: any common type into any float type; sd_sqrt<X, Z> converts to Z first
+    for xdt in (np.int32, np.int64):
+        x = np.array([0, 1, 4, 9, 16, 2, 1000003], xdt)
+        np.testing.assert_array_equal(O.transform_float(1, x, np.zeros(x.shape, np.float32)), np.sqrt(x.astype(np.float32)))
+        np.testing.assert_array_equal(O.transform_float(1, x, np.zeros(x.shape, np.float64)), np.sqrt(x.astype(np.float64)))
+    b = np.array([True, False, True])
+    np.testing.assert_array_equal(O.transform_float(1, b, np.zeros(3, np.float32)), [1.0, 0.0, 1.0])
+    h = O.transform_float(3, np.array([4, 16], np.int32), np.zeros(2, np.float16))
+    np.testing.assert_array_equal(h, np.array([0.5, 0.25], np.float16))
+
+
+def test_reduce_float_of_other_input_types():
+    # MultiDataTypeTests.cpp:246-256 (ndarray_reduceAlongDimension_test2): Mean of INT32 {0, 1, 2, 3} into FLOAT32
+    x = np.array([[0, 1], [2, 3]], np.int32)
+    assert O.reduce_float(0, x, np.zeros((), np.float32)) == np.float32(1.5)
+    np.testing.assert_array_equal(O.reduce_float(0, x, np.zeros(2, np.float32), [1]), np.array([0.5, 2.5], np.float32))
+    # the accumulator follows Z (op_macros_reduce.h:778-782): fp32 values whose fp32 running sum loses the small terms
+    # are summed exactly when Z is DOUBLE
+    v = np.array([1e8, 1.0, 1.0, 1.0, 1.0, -1e8], np.float32)
+    assert O.reduce_float(0, v, np.zeros((), np.float64)) == 4.0 / 6.0
+    assert O.reduce_float(0, v, np.zeros((), np.float32)) == np.float32(0.0)      # 1e8 + 1 == 1e8 in fp32
+    rng = np.random.default_rng(5)
+    for xdt in (np.int64, np.float16, np.float64, np.bool_):
+        a = rng.integers(0, 2, (5, 7)).astype(xdt) if xdt == np.bool_ else (rng.uniform(-4, 4, (5, 7)) * 3).astype(xdt)
+        a64 = a.astype(np.float64)
+        for op, want in ((0, a64.mean(1)), (1, np.abs(a64).mean(1)), (2, np.abs(a64).sum(1)), (3, np.sqrt((a64 ** 2).sum(1))),
+                         (4, np.abs(a64).max(1)), (7, (a64 ** 2).sum(1))):
+            np.testing.assert_allclose(O.reduce_float(op, a, np.zeros(5, np.float32), [1]), want, rtol=2e-6, atol=1e-6)
+            np.testing.assert_allclose(O.reduce_float(op, a, np.zeros(5, np.float64), [1]), want, rtol=1e-12, atol=1e-12)
+
+
+def test_reductions_of_empty_arrays():
+    # LegacyOpsTests.cpp:616-658 (test_legacy_reduce_empty_1/2/3): Sum of [2, 0, 3] along 1 -> zeros, Min -> +inf, Max -> -inf;
+    # DeclarableOpsTests14.cpp:230-265: reduce_min of a float [1, 0] -> infOrMax<float>, reduce_sum -> 0, reduce_mean -> NaN
+    f32 = np.dtype(np.float32)
+    assert O.reduce_of_empty("same", 0, f32, f32) == 0
+    assert O.reduce_of_empty("same", 2, f32, f32) == np.inf and O.reduce_of_empty("same", 1, f32, f32) == -np.inf
+    assert np.isnan(O.reduce_of_empty("float", 0, f32, f32))
+    # DeclarableOpsTests14.cpp:306-317 argmax of an empty array gives an empty result; the loop's own fill is index 0
+    assert O.reduce_of_empty("index", 0, f32, np.dtype(np.int64)) == 0 and O.reduce_of_empty("index", 4, f32, np.dtype(np.int64)) == -1
+    # infOrMax / nanOrZero are specialised for float and double only (array/DataTypeUtils.h:600-636)
+    assert O.reduce_of_empty("same", 1, "float16", "float16") == -65504.0
+    assert O.reduce_of_empty("same", 2, "bfloat16", "bfloat16") == float(np.float32(2.0 ** 127 * (2 - 2.0 ** -7)))
+    assert O.reduce_of_empty("same", 1, np.dtype(np.int32), np.dtype(np.int32)) == -(2 ** 31 - 1)
+    assert O.reduce_of_empty("float", 0, np.dtype(np.int32), "float16") == 0.0
+    assert O.reduce_of_empty("same", 3, f32, f32) == 1 and O.reduce_of_empty("bool", 1, f32, np.dtype(bool)) == 1
+    assert O.reduce_of_empty("same", 5, f32, f32) is None
+
+
+def test_matmul_of_integer_arrays():
+    # the reference's loop in the arrays' own type (MmulHelper.cpp:35-110) against Python's exact integers reduced modulo 2^bits
+    rng = np.random.default_rng(11)
+    for dt, bits in ((np.int32, 32), (np.int64, 64)):
+        a = rng.integers(-2 ** (bits - 2), 2 ** (bits - 2), (3, 5)).astype(dt)
+        b = rng.integers(-2 ** (bits - 2), 2 ** (bits - 2), (5, 4)).astype(dt)
+        c = rng.integers(-100, 100, (3, 4)).astype(dt)
+        def wrap(v):
+            v %= 2 ** bits
+            return v - 2 ** bits if v >= 2 ** (bits - 1) else v
+        for alpha, beta in ((1.0, 0.0), (3.0, 2.0), (2.9, 0.0)):
+            want = np.array([[wrap(int(alpha) * sum(int(a[i, k]) * int(b[k, j]) for k in range(5)) + (int(beta) * int(c[i, j]) if beta else 0))
+                              for j in range(4)] for i in range(3)], dtype=dt)
+            np.testing.assert_array_equal(O.matmul_int(a, b, c, alpha, beta), want)
+    # DeclarableOpsTests-style small case: exact products
+    np.testing.assert_array_equal(O.matmul_int(np.array([[1, 2], [3, 4]], np.int32), np.array([[5, 6], [7, 8]], np.int32)), [[19, 22], [43, 50]])
 
 
 def _c_int_div(a, b):

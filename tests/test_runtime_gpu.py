@@ -161,3 +161,85 @@ def _graph_replay_keeps_buffer_stamps(ex):
         assert L.nd4jhipGraphLaunch(g) == 0, L.lastErrorMessage()
         assert np.array_equal(Z.to_numpy(), x * k + 1)
     L.nd4jhipGraphDestroy(g)
+
+
+def test_recorded_copies_and_fills_replay_in_both_modes(ex, oracle):
+    """memsetAsync and a device-to-device memcpyAsync issued on the library's stream between Begin and End belong to the
+    recording: both replay modes must run them, also when the ops around them were merged (Add + layer_norm become one
+    kernel, so the kept graph is the re-recorded plan).  Array handles and the OpContext are dropped before End."""
+    import gc
+    L = ex.L
+    rng = np.random.default_rng(77)
+    rows, cols = 8, 768
+    gain, bias = rng.normal(1, 0.02, cols).astype(np.float32), rng.normal(0, 0.02, cols).astype(np.float32)
+    X, Y = NDArray.empty((rows, cols), FLOAT32), NDArray.empty((rows, cols), FLOAT32)
+    S, Ln, T, U = (NDArray.empty((rows, cols), FLOAT32) for _ in range(4))
+    G, B = NDArray.from_numpy(gain), NDArray.from_numpy(bias)
+    for a in (X, Y, S, Ln, T, U, G, B):
+        a.sync_to_device()
+    nbytes = rows * cols * 4
+    dT, dU, dLn = (L.dbSpecialBuffer(a.buffer.ptr) for a in (T, U, Ln))
+
+    def sequence(keep):
+        # fill, add, normalise, copy the normalised rows out -- the handles used by the op calls die right after them
+        assert L.memsetAsync(dU, 0, nbytes, 0, None) == 1
+        x, y, s, ln = X.view(X.shape, X.strides), Y.view(Y.shape, Y.strides), S.view(S.shape, S.strides), Ln.view(Ln.shape, Ln.strides)
+        L.execPairwiseTransform(None, Pairwise.Add, x.handle, y.handle, s.handle, None)
+        N.check("execPairwiseTransform")
+        call = ex.bind_custom("layer_norm", [s, G, B], [ln], i_args=[1], b_args=[False])
+        call()
+        assert L.memcpyAsync(dT, dLn, nbytes, 3, None) == 1
+        if not keep:
+            del call, x, y, s, ln
+            gc.collect()
+
+    def fresh(seed):
+        r = np.random.default_rng(seed)
+        x, y = r.normal(0, 1, (rows, cols)).astype(np.float32), r.normal(0, 1, (rows, cols)).astype(np.float32)
+        X.assign_numpy(x); Y.assign_numpy(y)
+        T.assign_numpy(np.full((rows, cols), -5.0, np.float32)); U.assign_numpy(np.ones((rows, cols), np.float32))
+        for a in (T, U):
+            a.sync_to_device()
+        return x, y
+
+    def read(a):
+        L.dbTickDeviceWrite(a.buffer.ptr)     # the raw copy / fill wrote device memory behind the buffer's stamps
+        return a.to_numpy()
+
+    # eager
+    x, y = fresh(1)
+    sequence(keep=True)
+    ex.synchronize()
+    eager_ln = Ln.to_numpy()
+    assert np.array_equal(read(T), eager_ln) and not read(U).any()
+    assert_close(eager_ln, oracle.layer_norm(x + y, gain, bias, np.zeros_like(x), [1], channels_first=False), 1e-5, 1e-5, "eager")
+    # recorded
+    assert L.nd4jhipGraphBeginCapture() == 0, L.lastErrorMessage()
+    sequence(keep=False)
+    g = L.nd4jhipGraphEndCapture()
+    N.check("nd4jhipGraphEndCapture")
+    assert g and L.nd4jhipGraphFusedOps(g) == 1
+    try:
+        for i, mode in enumerate((0, 1, 0, 1)):
+            L.nd4jhipSetGraphReplayMode(mode)
+            x, y = fresh(10 + i)
+            assert L.nd4jhipGraphLaunch(g) == 0, L.lastErrorMessage()
+            ex.synchronize()
+            want = oracle.layer_norm(x + y, gain, bias, np.zeros_like(x), [1], channels_first=False)
+            got = Ln.to_numpy()
+            assert_close(got, want, 1e-5, 1e-5, "replay %d" % i)
+            assert np.array_equal(read(T), got), ("the recorded copy did not run", mode)
+            assert not read(U).any(), ("the recorded fill did not run", mode)
+    finally:
+        L.nd4jhipSetGraphReplayMode(0)
+        L.nd4jhipGraphDestroy(g)
+    # a copy that touches host memory cannot be part of a recording
+    host = L.mallocHost(64, 0)
+    assert L.nd4jhipGraphBeginCapture() == 0
+    assert L.memcpyAsync(host, dT, 64, 2, None) == 0
+    assert b"device-to-device" in L.lastErrorMessage()
+    g2 = L.nd4jhipGraphEndCapture()
+    L.lastErrorMessage()
+    if g2:
+        L.nd4jhipGraphDestroy(g2)
+    L.freeHost(host)

@@ -45,6 +45,32 @@ def test_no_alloc_reduce_matches_exec_reduce_same(ex, dt, op):
         assert got.tobytes() == want.tobytes(), (n, got, want)
 
 
+@pytest.mark.parametrize("dt", [FLOAT32, DOUBLE, HALF, BFLOAT16])
+def test_no_alloc_reduce_of_short_arrays_allocates_nothing(ex, dt):
+    """One element, and the lengths whose bytes select the 8-, 16- and 32-lanes-per-row launches; the device's free memory
+    is the same before and after the calls."""
+    L = ex.L
+    L.initializeDevicesAndFunctions()
+    rng = np.random.default_rng(dt)
+    cases = []
+    for n in (1, 7, 64, 200, 3000):
+        X = _device(rng.normal(0, 1, n), dt)
+        X.sync_to_device()
+        Z = NDArray.empty((), dt)
+        L.dbAllocateSpecialBuffer(Z.buffer.ptr)
+        cases.append((n, X, Z, [ex.exec_reduce_same(op, X, None).to_numpy() for op in (ReduceSame.Sum, ReduceSame.Max, ReduceSame.AMin)]))
+    ex.synchronize()
+    free_before = L.getDeviceFreeMemory(L.getDevice())
+    for n, X, Z, want in cases:
+        for op, w in zip((ReduceSame.Sum, ReduceSame.Max, ReduceSame.AMin), want):
+            assert L.nd4jhipReduceSameScalarNoAlloc(None, op, dt, L.dbSpecialBuffer(X.buffer.ptr), n, L.dbSpecialBuffer(Z.buffer.ptr)) == 0, L.lastErrorMessage()
+            L.streamSynchronize(None)
+            assert L.getDeviceFreeMemory(L.getDevice()) == free_before, ("the call changed the device's free memory", n, op)
+            L.dbTickDeviceWrite(Z.buffer.ptr)
+            got = Z.to_numpy()
+            assert got.tobytes() == w.tobytes(), (n, op, got, w)
+
+
 def test_no_alloc_reduce_on_a_caller_stream_and_limits(ex):
     L = ex.L
     L.initializeDevicesAndFunctions()
