@@ -485,6 +485,25 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
 // exactly where the P V accumulation needs it.  Each lane group keeps its own running (max, sum, o[8]) state;
 // states are merged across groups (shuffles), across waves (LDS) and normalised once.  Logits go through the same
 // scale / clip / storage-type rounding as in the tile kernel above; probabilities stay in fp32.
+// eight consecutive values of d as a lane holds them: one 16-byte load for the 16-bit types, two for fp32
+template <typename T> struct Row8 {
+  using raw = typename RawIO<T>::raw;
+  static __device__ __forceinline__ raw load(const T* p) { return *reinterpret_cast<const raw*>(p); }
+  static __device__ __forceinline__ void unpack(const raw& r, float* out) { RawIO<T>::unpack(r, out); }
+};
+template <> struct Row8<float> {
+  struct raw { raw_f32x4 lo, hi; };
+  static __device__ __forceinline__ raw load(const float* p) {
+    raw r;
+    r.lo = *reinterpret_cast<const raw_f32x4*>(p);
+    r.hi = *reinterpret_cast<const raw_f32x4*>(p + 4);
+    return r;
+  }
+  static __device__ __forceinline__ void unpack(const raw& r, float* out) {
+#pragma unroll
+    for (int e = 0; e < 4; e++) { out[e] = r.lo[e]; out[4 + e] = r.hi[e]; }
+  }
+};
 template <typename T, int D, int NW, bool VM, int U = 4>
 __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
                                                        T* __restrict__ O) {
@@ -507,8 +526,8 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
   const int g = lane / CH, c = lane % CH;
   // the query row was written by the kernel before this one and the first keys come cold from HBM: all of these loads
   // are issued before the first value is touched, so the two latencies overlap
-  const typename RawIO<T>::raw qraw = *reinterpret_cast<const typename RawIO<T>::raw*>(Q + qi * a.qT + c * 8);
-  using Raw = typename RawIO<T>::raw;
+  using Raw = typename Row8<T>::raw;
+  const Raw qraw = Row8<T>::load(Q + qi * a.qT + c * 8);
   // (a second register set, so that the next trip's loads fly while the current one is consumed, changed nothing at
   // batch 1 and cost 1 % at batch 32: a block's stream is bound by what one CU can pull, not by a trip's latency)
   Raw krA[U], vrA[U];
@@ -519,15 +538,15 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
       LongType key = k0 + u * KPS + g;
       valid[u] = key < a.Tv;
       key = valid[u] ? key : a.Tv - 1;
-      kr[u] = *reinterpret_cast<const Raw*>(K + key * a.kT + c * 8);
-      vr[u] = *reinterpret_cast<const Raw*>(V + key * a.vT + c * 8);
+      kr[u] = Row8<T>::load(K + key * a.kT + c * 8);
+      vr[u] = Row8<T>::load(V + key * a.vT + c * 8);
     }
   };
   const LongType step = (LongType)NW * (KPS * U);
   LongType k0 = (LongType)wave * (KPS * U);
   if (k0 < a.Tv) issue(k0, krA, vrA, validA);
   float q[8];
-  RawIO<T>::unpack(qraw, q);
+  Row8<T>::unpack(qraw, q);
   const float L2E = 1.44269502162933349609375f;
   float m = -1.0e30f, l = 0.f, o[8];
 #pragma unroll
@@ -538,7 +557,7 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
 #pragma unroll
     for (int u = 0; u < U; u++) {
       float kf[8];
-      RawIO<T>::unpack(kr[u], kf);
+      Row8<T>::unpack(kr[u], kf);
       float d = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; e++) d = __builtin_fmaf(q[e], kf[e], d);
@@ -568,7 +587,7 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
     for (int u = 0; u < U; u++) {
       const float p = valid[u] ? __builtin_amdgcn_exp2f((sc[u] - m) * L2E) : 0.f;
       float vf[8];
-      RawIO<T>::unpack(vr[u], vf);
+      Row8<T>::unpack(vr[u], vf);
       l += p;
 #pragma unroll
       for (int e = 0; e < 8; e++) o[e] = __builtin_fmaf(p, vf[e], o[e]);
@@ -619,10 +638,11 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
 }
 
 bool attentionDecodeSupported(DataType dt, const AttnDesc& d) {
-  if (dt != HALF && dt != BFLOAT16) return false;
+  if (dt != HALF && dt != BFLOAT16 && dt != FLOAT32) return false;
   if (d.D != d.Dv || (d.D != 64 && d.D != 128)) return false;
   if (d.causal || d.Tq < 1 || d.Tq > 8 || d.Tv < 1) return false;
-  for (LongType st : {d.qB, d.qT, d.kB, d.kT, d.vB, d.vT, d.qB2, d.kB2, d.vB2}) if (st % 8 != 0) return false;
+  const LongType perVector = dt == FLOAT32 ? 4 : 8;   // rows start on 16-byte boundaries
+  for (LongType st : {d.qB, d.qT, d.kB, d.kT, d.vB, d.vT, d.qB2, d.kB2, d.vB2}) if (st % perVector != 0) return false;
   return d.B < (1LL << 31);
 }
 
@@ -648,6 +668,7 @@ void launchAttentionDecode(hipStream_t s, DataType dt, const void* q, const void
   ND4J_REQUIRE(attentionDecodeSupported(dt, d), "attention: decode kernel does not take this problem");
   ND4J_REQUIRE((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) == 0, "attention: operands must be 16-byte aligned");
   if (dt == HALF) { if (d.D == 64) launchDecodeTyped<f16_t, 64>(s, q, k, v, out, d); else launchDecodeTyped<f16_t, 128>(s, q, k, v, out, d); }
+  else if (dt == FLOAT32) { if (d.D == 64) launchDecodeTyped<float, 64>(s, q, k, v, out, d); else launchDecodeTyped<float, 128>(s, q, k, v, out, d); }
   else { if (d.D == 64) launchDecodeTyped<bf16_t, 64>(s, q, k, v, out, d); else launchDecodeTyped<bf16_t, 128>(s, q, k, v, out, d); }
   HIP_CHECK(hipGetLastError());
 }

@@ -515,49 +515,52 @@ static void attentionExec(Context& c) {
   if (qMask) { maskFits(qMask, d.Tq, "query"); reads.push_back(qMask); }
   if (d.B * d.Tq == 0) return;
   prepareSpecialUse(writes, reads);
+  d.qB = q.sB; d.qT = q.sT; d.kB = k.sB; d.kT = k.sT; d.vB = v.sB; d.vT = v.sT; d.oB = out.sB; d.oT = out.sT;
+  d.qB2 = q.sB2; d.kB2 = k.sB2; d.vB2 = v.sB2; d.oB2 = out.sB2;
+  const bool unitInner = q.sD == 1 && k.sD == 1 && v.sD == 1 && out.sD == 1;
+  const bool useDecode = !wantW && !wantL && unitInner && attentionDecodeSupported(dt, d);
+  const bool useFused = !useDecode && !wantW && !wantL && unitInner && attentionFusedSupported(dt, d);
+  // Temporaries (dense copies of the masks; logits and weights of the composition when they are not outputs) are carved out
+  // of the launch context's grow-only scratch: no allocation and no wait per call once it has grown to the problem's size.
+  const LongType lw = d.Tq * d.Tv;
+  auto round256 = [](size_t b) { return (b + 255) & ~(size_t)255; };
+  size_t need = 0;
+  if (vMask) need += round256((size_t)vMask->lengthOf());
+  if (qMask && wantW) need += round256((size_t)qMask->lengthOf() * sizeOf(dt));
+  if (!useDecode && !useFused) need += (wantL ? 0 : round256((size_t)(d.B * lw) * sizeOf(dt))) + (wantW ? 0 : round256((size_t)(d.B * lw) * sizeOf(dt)));
+  char* ws = need ? static_cast<char*>(LaunchContext::defaultContext()->workspace(need)) : nullptr;
+  auto carve = [&](size_t bytes) { char* p = ws; ws += round256(bytes); return static_cast<void*>(p); };
   // dense device copies of the masks in the form the kernels read: the value mask as bytes (cast to BOOL: non-zero keeps
   // the key), the query mask in the arrays' type.  A mask that already is dense and of that type is used in place.
-  std::shared_ptr<DataBuffer> tmpVm, tmpQm;
-  auto denseMask = [&](NDArray* m, DataType want, std::shared_ptr<DataBuffer>& hold) -> const void* {
+  auto denseMask = [&](NDArray* m, DataType want) -> const void* {
     auto dsi = makeShapeInfo(want, 'c', shapeOf(m));
+    void* copy = carve((size_t)m->lengthOf() * sizeOf(want));   // (carved either way: the sum above counted it)
     if (m->dataType() == want) {
       bool dense = true;
       for (int i = 0; i < m->rankOf(); i++) if (m->sizeAt(i) != 1 && m->strideAt(i) != shape::strideOf(dsi.data())[i]) dense = false;
       if (dense) return m->specialBuffer();
     }
-    hold = std::make_shared<DataBuffer>((void*)nullptr, (void*)nullptr, (size_t)m->lengthOf() * sizeOf(want), want);
-    hold->allocateSpecial();
     EwPlan p = buildEwPlan({dsi.data(), m->shapeInfo()});
-    launchUnary(stream(), U_IDENTITY, m->dataType(), want, m->specialBuffer(), hold->special, p);
-    return hold->special;
+    launchUnary(stream(), U_IDENTITY, m->dataType(), want, m->specialBuffer(), copy, p);
+    return copy;
   };
-  if (vMask) d.vmask = static_cast<const unsigned char*>(denseMask(vMask, BOOL, tmpVm));
+  if (vMask) d.vmask = static_cast<const unsigned char*>(denseMask(vMask, BOOL));
   // the query mask scales the weights output only: out = weights v has been formed before (AttentionHelper.cpp:455-467)
-  const void* qm = qMask && wantW ? denseMask(qMask, dt, tmpQm) : nullptr;
-  d.qB = q.sB; d.qT = q.sT; d.kB = k.sB; d.kT = k.sT; d.vB = v.sB; d.vT = v.sT; d.oB = out.sB; d.oT = out.sT;
-  d.qB2 = q.sB2; d.kB2 = k.sB2; d.vB2 = v.sB2; d.oB2 = out.sB2;
-  const bool unitInner = q.sD == 1 && k.sD == 1 && v.sD == 1 && out.sD == 1;
-  if (!wantW && !wantL && unitInner && attentionDecodeSupported(dt, d)) {
+  const void* qm = qMask && wantW ? denseMask(qMask, dt) : nullptr;
+  if (useDecode) {
     launchAttentionDecode(stream(), dt, q0->specialBuffer(), k0->specialBuffer(), v0->specialBuffer(), o0->specialBuffer(), d);
-  } else if (!wantW && !wantL && unitInner && attentionFusedSupported(dt, d)) {
+  } else if (useFused) {
     launchAttentionFused(stream(), dt, q0->specialBuffer(), k0->specialBuffer(), v0->specialBuffer(), o0->specialBuffer(), d);
   } else {
     // composition: logits = q k^T -> fix-up (scale, clip, mask) -> softmax -> out = weights v
-    const LongType lw = d.Tq * d.Tv;
-    std::shared_ptr<DataBuffer> tmpL, tmpW;
-    auto scratch = [&](std::shared_ptr<DataBuffer>& hold) {
-      hold = std::make_shared<DataBuffer>((void*)nullptr, (void*)nullptr, (size_t)(d.B * lw) * sizeOf(dt), dt);
-      hold->allocateSpecial();
-      return hold->special;
-    };
     auto denseOutput = [&](NDArray* a, const char* what) {
       const BatchedView b = batchedView(a, what);
       ND4J_REQUIRE(b.B == d.B && b.T == d.Tq && b.D == d.Tv && a->dataType() == dt && denseRows(b),
                    std::string("dot_product_attention_v2: ") + what + " output must be a dense row-major [batch, Tq, Tv] array");
       return a->specialBuffer();
     };
-    void* logits = wantL ? denseOutput(c.outputs[2], "logits") : scratch(tmpL);
-    void* weights = wantW ? denseOutput(c.outputs[1], "weights") : scratch(tmpW);
+    void* logits = wantL ? denseOutput(c.outputs[2], "logits") : carve((size_t)(d.B * lw) * sizeOf(dt));
+    void* weights = wantW ? denseOutput(c.outputs[1], "weights") : carve((size_t)(d.B * lw) * sizeOf(dt));
     GemmDesc g1;
     g1.M = d.Tq; g1.N = d.Tv; g1.K = d.D; g1.batch = d.B; g1.batchInner = d.H;
     g1.aRow = q.sT; g1.aCol = q.sD; g1.aBatch = q.sB; g1.aBatch2 = q.sB2;
@@ -575,9 +578,7 @@ static void attentionExec(Context& c) {
     g2.cRow = out.sT; g2.cCol = out.sD; g2.cBatch = out.sB; g2.cBatch2 = out.sB2;
     launchGemm(stream(), dt, weights, v0->specialBuffer(), o0->specialBuffer(), g2);
     if (qm) launchAttentionQueryMask(stream(), dt, weights, qm, d);
-    if (tmpL || tmpW) HIP_CHECK(hipStreamSynchronize(stream()));  // temporaries are released on return
   }
-  if (tmpVm || tmpQm) HIP_CHECK(hipStreamSynchronize(stream()));
   registerSpecialUse(writes, reads);
 }
 static std::vector<std::vector<LongType>> attentionShapeFn(Context& c) {

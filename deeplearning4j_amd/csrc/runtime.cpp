@@ -155,6 +155,18 @@ void LaunchContext::init() {
   applyKernelAttributes();
   ready = true;
 }
+void* LaunchContext::workspace(size_t bytes) {
+  if (bytes <= workspaceBytes) return workspaceBuffer;
+  ND4J_REQUIRE(!captureActive(), "this op needs " + std::to_string(bytes) + " bytes of device scratch and " + std::to_string(workspaceBytes) +
+                                     " are allocated: run it once outside the capture (allocating would invalidate the recording)");
+  HIP_CHECK(hipStreamSynchronize(execStream));   // kernels of earlier ops may still read the old block
+  if (workspaceBuffer) (void)hipFree(workspaceBuffer);
+  workspaceBuffer = nullptr; workspaceBytes = 0;
+  const size_t want = ((bytes + bytes / 4) + 0xfffffu) & ~(size_t)0xfffffu;   // a quarter of headroom, whole MiB
+  HIP_CHECK(hipMalloc(&workspaceBuffer, want));
+  workspaceBytes = want;
+  return workspaceBuffer;
+}
 static LaunchContext g_defaultContext;
 static std::mutex g_defaultContextMutex;
 LaunchContext* LaunchContext::defaultContext() {

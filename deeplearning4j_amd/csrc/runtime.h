@@ -57,6 +57,13 @@ struct LaunchContext {
   bool ready = false;
   static constexpr size_t REDUCTION_BYTES = 8u << 20;
   static constexpr size_t ALLOCATION_BYTES = 8u << 20;
+  // Grow-only device scratch for ops whose temporaries are as large as their operands (the attention composition's logits
+  // and weights, dense copies of masks).  It only ever grows, and only outside a stream capture: an op that fits what is
+  // there neither allocates nor waits, and whatever the previous op left in it is no longer read once this op's first
+  // kernel starts (one stream, one op at a time).  Call with the sum of what the op will carve out of it.
+  void* workspace(size_t bytes);
+  void* workspaceBuffer = nullptr;
+  size_t workspaceBytes = 0;
   void init();
   static LaunchContext* defaultContext();
   static LaunchContext* ifReady();   // the default context if it has been initialised, else null (never allocates)

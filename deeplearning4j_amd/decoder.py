@@ -192,7 +192,7 @@ class Decoder:
                     copy = (lambda: None) if src is a["next"] else self._assign(src.view((self.B, 1), (1, 1)), a["ids"])
                     self._feeds[id(src)] = (src, copy)
                 self._feed = self._feeds[id(src)]
-            if self.use_graphs and self.dtype in (BFLOAT16, HALF):   # fp32 attention goes through temporaries and a wait: not capturable
+            if self.use_graphs:
                 self._graph_step(prog)
                 self.length += 1
                 self._last_next = a["next"]

@@ -69,20 +69,20 @@ def test_graph_replay_matches_eager_steps(ex, replay_mode):
     eager ids bit for bit (a replayed kernel runs with exactly the recorded arguments).  Both ways of replaying: the
     instantiated graph (0) and the merged sequence launched kernel by kernel by the library (1)."""
     from deeplearning4j_amd.decoder import Decoder, DecoderConfig, init_weights
-    from deeplearning4j_amd.ndarray import BFLOAT16, HALF
+    from deeplearning4j_amd.ndarray import BFLOAT16, FLOAT32, HALF
     ex.L.nd4jhipSetGraphReplayMode(replay_mode)
     assert ex.L.nd4jhipGetGraphReplayMode() == replay_mode
     try:
-        _graph_replay_matches_eager_steps(ex, Decoder, DecoderConfig, init_weights, BFLOAT16, HALF)
+        _graph_replay_matches_eager_steps(ex, Decoder, DecoderConfig, init_weights, BFLOAT16, HALF, FLOAT32)
     finally:
         ex.L.nd4jhipSetGraphReplayMode(0)
 
 
-def _graph_replay_matches_eager_steps(ex, Decoder, DecoderConfig, init_weights, BFLOAT16, HALF):
+def _graph_replay_matches_eager_steps(ex, Decoder, DecoderConfig, init_weights, BFLOAT16, HALF, FLOAT32):
     cfg = DecoderConfig(vocab=512, d_model=128, n_head=2, n_layer=2, max_len=96)
     w = init_weights(cfg, seed=5)
     rng = np.random.default_rng(6)
-    for dtype in (HALF, BFLOAT16):
+    for dtype in (HALF, BFLOAT16, FLOAT32):    # fp32: the streaming attention kernel takes the single-token steps, nothing allocates
         for batch in (1, 3):
             prompt = rng.integers(0, cfg.vocab, (batch, 17))
             eager = Decoder(cfg, w, dtype, batch=batch, executioner=ex)
