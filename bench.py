@@ -571,7 +571,7 @@ def main():
                         del Am, Bm, Zm
         if 4 in cfgs:
             # config 4: attention prefill, causal
-            for dt, dtn in [(HALF, "f16"), (BFLOAT16, "bf16")]:
+            for dt, dtn in [(HALF, "f16"), (BFLOAT16, "bf16")] + ([(FLOAT32, "f32")] if extras else []):
                 rng = np.random.default_rng(4004)
                 qs = (96, 1024, 64)
                 mk = lambda: rng.normal(0, 1, qs).astype(np.float32)
@@ -601,7 +601,7 @@ def main():
                     nb = 2
                     cv = (lambda t: O.Arr(f32_to_bf16_bits(np.asarray(t, np.float32)), O.BFLOAT16)) if dt == BFLOAT16 else (lambda t: O.Arr(np.ascontiguousarray(t)))
                     oq, ok_, ov = cv(q[:nb]), cv(k[:nb]), cv(v[:nb])
-                    oo = cv(np.zeros((nb, 1024, 64), np.float32 if dt == BFLOAT16 else np.float16))
+                    oo = cv(np.zeros((nb, 1024, 64), np.float16 if dt == HALF else np.float32))
                     q32, k32, v32 = (np.asarray(t[:nb], np.float32) for t in (q, k, v))
 
                     def fast():

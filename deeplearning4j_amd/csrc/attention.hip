@@ -673,7 +673,195 @@ void launchAttentionDecode(hipStream_t s, DataType dt, const void* q, const void
   HIP_CHECK(hipGetLastError());
 }
 
+
+// ---- fused kernel, fp32 ------------------------------------------------------------------------------------------------
+// The same formulation on the fp32 matrix instruction (v_mfma_f32_32x32x2_f32: a 32 x 32 tile, two k per issue, 64 cycles):
+// one block = 128 queries of one batch entry (4 waves x 32 queries), 32-key tiles of K and V staged through LDS in two
+// stages (global -> registers -> LDS: at 64 cycles per MFMA the matrix pipe, not the staging, sets the pace).
+// S^T = K Q^T: the k index of an MFMA step may be any permutation as long as both operands agree, so the half-wave h takes
+// d = h * D/2 + step; a lane then reads its key row's d-range as 16-byte vectors and keeps its query's d-range in registers.
+// Lane (query = lane % 32, h) ends up with the scores of keys 8 (r / 4) + 4 h + r % 4, r = 0..15, of its own query: the
+// running maximum and sum are per-lane scalars shared with the other half-wave by one exchange, and the probabilities feed
+// O^T = V^T P^T straight from those registers (step r of the second product pairs register r of both half-waves).
+// Scores are scale * q.k clipped to +-1e4 (AttentionHelper.cpp:340-352); masked and out-of-range keys weigh exactly 0
+// (the reference's clamped softmax gives them e^-88 / sum).  No value mask here: such calls take the composition.
+template <int D>
+__global__ __launch_bounds__(256, D == 64 ? 3 : 1) void attn_fused_f32(FusedArgs a, const float* __restrict__ Q, const float* __restrict__ K, const float* __restrict__ V,
+                                                      float* __restrict__ O) {
+  constexpr int BQ = 128, BKV = 32, HD = D / 2, PITCH = D + 4;   // row pitch in floats: 16 consecutive rows start in different banks
+  constexpr int DT = D / 32;                                     // dv tiles of the output accumulator
+  constexpr int VPT = BKV * D / 4 / 256;                         // 16-byte vectors of a K (or V) tile per thread
+  typedef __attribute__((ext_vector_type(4))) float f32x4s;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  float* smem = reinterpret_cast<float*>(smem_raw);              // [2 stages][K tile, V tile][BKV][PITCH]
+  // Work items = (query tile, batch entry), the late (heavy, under the causal mask) query tiles first.  Several blocks
+  // share a CU and the hardware deals consecutive block ids out CU after CU, so rounds of 256 block ids walk the item
+  // list alternately forwards and backwards: the CU that got the heaviest item of one round gets the lightest of the next.
+  unsigned item = blockIdx.x;
+  {
+    const unsigned round = blockIdx.x >> 8, first = round << 8;
+    const unsigned last = first + 255u < gridDim.x ? first + 255u : gridDim.x - 1u;
+    if (round & 1u) item = last - (blockIdx.x - first);
+  }
+  const int qt = a.qTiles - 1 - (int)(item / (unsigned)a.nBatch);
+  const LongType b = item % (unsigned)a.nBatch;
+  if (a.H > 0) {
+    const LongType hi = b / a.H, lo = b - hi * a.H;
+    Q += hi * a.qB2 + lo * a.qB; K += hi * a.kB2 + lo * a.kB; V += hi * a.vB2 + lo * a.vB; O += hi * a.oB2 + lo * a.oB;
+  } else {
+    Q += b * a.qB; K += b * a.kB; V += b * a.vB; O += b * a.oB;
+  }
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, h = lane >> 5;
+  const LongType q0 = (LongType)qt * BQ;
+  const LongType query = q0 + wave * 32 + (lane & 31);
+  const LongType qrow = query < a.Tq ? query : a.Tq - 1;
+  const float L2E = 1.44269502162933349609375f;
+  const float sc = a.applyScale ? a.scale : 1.f;
+
+  float qf[HD];
+#pragma unroll
+  for (int i = 0; i < HD / 4; i++) {
+    const f32x4s v = *reinterpret_cast<const f32x4s*>(Q + qrow * a.qT + h * HD + 4 * i);
+    qf[4 * i] = v[0]; qf[4 * i + 1] = v[1]; qf[4 * i + 2] = v[2]; qf[4 * i + 3] = v[3];
+  }
+  f32x16 o[DT];
+#pragma unroll
+  for (int i = 0; i < DT; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) o[i][r] = 0.f;
+  float m = -1.0e30f, l = 0.f;
+
+  LongType kvEnd = a.Tv;
+  if (a.causal) { const LongType lim = q0 + BQ; kvEnd = lim < kvEnd ? lim : kvEnd; }
+  const LongType nTiles = (kvEnd + BKV - 1) / BKV;
+
+  // staging: vector i of this thread is (row, 16-byte column) = ((t + 256 i) / (D / 4), (t + 256 i) % (D / 4)) of the tile
+  f32x4s kreg[VPT], vreg[VPT];
+  auto fetch = [&](LongType kv0) {
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+      const int idx = t + 256 * i, row = idx / (D / 4), col = idx % (D / 4);
+      LongType key = kv0 + row;
+      key = key < a.Tv ? key : a.Tv - 1;              // keys past the end repeat the last one (their weights are exactly 0)
+      kreg[i] = *reinterpret_cast<const f32x4s*>(K + key * a.kT + 4 * col);
+      vreg[i] = *reinterpret_cast<const f32x4s*>(V + key * a.vT + 4 * col);
+    }
+  };
+  auto park = [&](int stage) {
+    float* sk = smem + stage * (2 * BKV * PITCH);
+    float* sv = sk + BKV * PITCH;
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+      const int idx = t + 256 * i, row = idx / (D / 4), col = idx % (D / 4);
+      *reinterpret_cast<f32x4s*>(sk + row * PITCH + 4 * col) = kreg[i];
+      *reinterpret_cast<f32x4s*>(sv + row * PITCH + 4 * col) = vreg[i];
+    }
+  };
+  if (nTiles > 0) { fetch(0); park(0); }
+  __syncthreads();
+
+  for (LongType it = 0; it < nTiles; it++) {
+    const int cur = (int)(it & 1);
+    const LongType kv0 = it * BKV;
+    const float* sK = smem + cur * (2 * BKV * PITCH);
+    const float* sV = sK + BKV * PITCH;
+    const bool more = it + 1 < nTiles;
+    if (more) fetch(kv0 + BKV);                       // in flight while this tile is multiplied
+
+    // under the causal mask a wave sits out the tiles that lie wholly after its 32 queries (it still parks its share of
+    // the next tile and meets the barrier)
+    const bool idleWave = a.causal && kv0 > q0 + wave * 32 + 31;
+    if (!idleWave) {
+    // S^T = K Q^T for the 32 keys of the tile; two accumulators, so that consecutive MFMAs do not wait for each other
+    f32x16 s, s2;
+#pragma unroll
+    for (int r = 0; r < 16; r++) { s[r] = 0.f; s2[r] = 0.f; }
+    const float* krow = sK + (lane & 31) * PITCH + h * HD;
+#pragma unroll
+    for (int i = 0; i < HD / 4; i++) {
+      const f32x4s kv = *reinterpret_cast<const f32x4s*>(krow + 4 * i);
+      s = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[0], qf[4 * i], s, 0, 0, 0);
+      s2 = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[1], qf[4 * i + 1], s2, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[2], qf[4 * i + 2], s, 0, 0, 0);
+      s2 = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[3], qf[4 * i + 3], s2, 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++) s[r] += s2[r];
+    // register r: key kv0 + 8 (r / 4) + 4 h + r % 4 against this lane's query
+    const bool edge = (a.causal && kv0 + BKV - 1 > q0 + wave * 32) || kv0 + BKV > a.Tv;
+    float tmax = m;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      float v = s[r] * sc;
+      v = __builtin_fminf(__builtin_fmaxf(v, -1.0e4f), 1.0e4f);
+      if (edge) {
+        const LongType key = kv0 + 8 * (r >> 2) + 4 * h + (r & 3);
+        if (key >= a.Tv || (a.causal && key > query)) v = -1.0e30f;
+      }
+      s[r] = v;
+      tmax = __builtin_fmaxf(tmax, v);
+    }
+    tmax = __builtin_fmaxf(tmax, __shfl_xor(tmax, 32));
+    const float alpha = __builtin_amdgcn_exp2f((m - tmax) * L2E);
+    m = tmax;
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      // a masked score (-1e30) sits 1e30 below the maximum whenever the row has seen a visible key; before that (m = -1e30
+      // too) the difference is 0 and the weight must still be 0
+      const float p = s[r] <= -1.0e30f ? 0.f : __builtin_amdgcn_exp2f((s[r] - m) * L2E);
+      s[r] = p;
+      psum += p;
+    }
+    psum += __shfl_xor(psum, 32);
+    l = l * alpha + psum;
+#pragma unroll
+    for (int i = 0; i < DT; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) o[i][r] *= alpha;
+    // O^T += V^T P^T: step r pairs key 8 (r / 4) + 4 h + r % 4 of both half-waves
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const float* vrow = sV + (8 * (r >> 2) + 4 * h + (r & 3)) * PITCH + (lane & 31);
+#pragma unroll
+      for (int i = 0; i < DT; i++) o[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[32 * i], s[r], o[i], 0, 0, 0);
+    }
+    }   // !idleWave
+    if (more) park(cur ^ 1);                          // the other stage was last read before the barrier that ended the previous tile
+    __syncthreads();
+  }
+  if (query < a.Tq) {
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    float* orow = O + query * a.oT;
+#pragma unroll
+    for (int i = 0; i < DT; i++)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; g4++) {
+        const f32x4s w = {o[i][4 * g4] * inv, o[i][4 * g4 + 1] * inv, o[i][4 * g4 + 2] * inv, o[i][4 * g4 + 3] * inv};
+        *reinterpret_cast<f32x4s*>(orow + 32 * i + 8 * g4 + 4 * h) = w;
+      }
+  }
+}
+template <int D>
+static void launchFusedF32(hipStream_t s, const void* q, const void* k, const void* v, void* out, const AttnDesc& d) {
+  FusedArgs a;
+  a.Tq = d.Tq; a.Tv = d.Tv;
+  a.qB = d.qB; a.qT = d.qT; a.kB = d.kB; a.kT = d.kT; a.vB = d.vB; a.vT = d.vT; a.oB = d.oB; a.oT = d.oT;
+  a.H = d.H; a.qB2 = d.qB2; a.kB2 = d.kB2; a.vB2 = d.vB2; a.oB2 = d.oB2;
+  a.scale = d.scale; a.applyScale = d.applyScale ? 1 : 0; a.causal = d.causal ? 1 : 0;
+  a.qTiles = (int)((d.Tq + 127) / 128); a.perBatch = a.qTiles; a.nBatch = (int)d.B; a.heavyFirst = 1;
+  a.vmask = nullptr; a.maskValue = d.maskValue;
+  constexpr int LDS = 2 * 2 * 32 * (D + 4) * 4;
+  ND4J_REQUIRE((DynLds<attn_fused_f32<D>, LDS>::granted()), "attention: the device does not grant the fp32 fused kernel its LDS");
+  hipLaunchKernelGGL((attn_fused_f32<D>), dim3((unsigned)((LongType)a.qTiles * d.B)), dim3(256), LDS, s, a, (const float*)q, (const float*)k, (const float*)v, (float*)out);
+}
+
 bool attentionFusedSupported(DataType dt, const AttnDesc& d) {
+  if (dt == FLOAT32) {
+    if (d.vmask != nullptr || d.D != d.Dv || (d.D != 64 && d.D != 128) || d.Tq < 1 || d.Tv < 1) return false;
+    for (LongType st : {d.qB, d.qT, d.kB, d.kT, d.vB, d.vT, d.oB, d.oT, d.qB2, d.kB2, d.vB2, d.oB2}) if (st % 4 != 0) return false;   // 16-byte aligned rows
+    return ((d.Tq + 127) / 128) * d.B < (1LL << 31);
+  }
   if (dt != HALF && dt != BFLOAT16) return false;
   if (d.D != d.Dv || (d.D != 64 && d.D != 128)) return false;
   if (d.Tq < 1 || d.Tv < 1) return false;
@@ -717,6 +905,12 @@ static void launchFusedTyped(hipStream_t s, const void* q, const void* k, const 
 void launchAttentionFused(hipStream_t s, DataType dt, const void* q, const void* k, const void* v, void* out, const AttnDesc& d) {
   ND4J_REQUIRE(attentionFusedSupported(dt, d), "attention: fused kernel does not take this problem");
   ND4J_REQUIRE((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) == 0 && ((uintptr_t)out & 7) == 0, "attention: operands must be 16-byte aligned");
+  if (dt == FLOAT32) {
+    ND4J_REQUIRE(((uintptr_t)out & 15) == 0, "attention: operands must be 16-byte aligned");
+    if (d.D == 64) launchFusedF32<64>(s, q, k, v, out, d); else launchFusedF32<128>(s, q, k, v, out, d);
+    HIP_CHECK(hipGetLastError());
+    return;
+  }
   ND4J_REQUIRE(((d.Tq + 127) / 128) * d.B < (1LL << 31), "attention: too many query tiles");
   // scale folded into the exponent: no scale at all, or bf16 scores with a power-of-two scale of moderate size (the
   // fp16 storage type has too narrow a range for rounding to commute with the scaling)

@@ -519,7 +519,8 @@ static void attentionExec(Context& c) {
   d.qB2 = q.sB2; d.kB2 = k.sB2; d.vB2 = v.sB2; d.oB2 = out.sB2;
   const bool unitInner = q.sD == 1 && k.sD == 1 && v.sD == 1 && out.sD == 1;
   const bool useDecode = !wantW && !wantL && unitInner && attentionDecodeSupported(dt, d);
-  const bool useFused = !useDecode && !wantW && !wantL && unitInner && attentionFusedSupported(dt, d);
+  // (the fp32 tile kernel takes no value mask; d.vmask is only filled in below)
+  const bool useFused = !useDecode && !wantW && !wantL && unitInner && !(dt == FLOAT32 && vMask) && attentionFusedSupported(dt, d);
   // Temporaries (dense copies of the masks; logits and weights of the composition when they are not outputs) are carved out
   // of the launch context's grow-only scratch: no allocation and no wait per call once it has grown to the problem's size.
   const LongType lw = d.Tq * d.Tv;
