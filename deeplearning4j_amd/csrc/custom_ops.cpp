@@ -263,7 +263,8 @@ static XwGeometry xwGeometry(Context& c, bool needOutput) {
 }
 // epi: extra outputs for the product's epilogue (already prepared for device use by the caller); returns whether the kernel
 // that ran wrote them
-struct LnPrologue { NDArray *x, *gain, *bias, *out; };   // out = layer_norm(x; gain, bias) is the product's input
+// out = layer_norm(x; gain, bias) is the product's input: `rows` rows of unit element stride, xPitch / outPitch elements apart
+struct LnPrologue { NDArray *x, *gain, *bias, *out; LongType rows, xPitch, outPitch; };
 static bool xwPlusBImpl(Context& c, const GemmEpilogue* epi, const LnPrologue* ln = nullptr) {
   ND4J_REQUIRE(c.width() >= 3, "xw_plus_b: x, weights and bias are required");
   NDArray* x = c.input(0); NDArray* w = c.input(1); NDArray* b = c.input(2); NDArray* z = c.output(0);
@@ -280,11 +281,12 @@ static bool xwPlusBImpl(Context& c, const GemmEpilogue* epi, const LnPrologue* l
   d.aRow = g.aRow; d.aCol = g.aCol; d.bRow = g.bRow; d.bCol = g.bCol; d.cRow = g.cRow; d.cCol = g.cCol;
   if (ln) {
     // the product reads the row before normalisation and writes the normalised row where the separate op would have
-    if (g.M != 1 || g.aCol != 1 || ln->x->lengthOf() != g.K || ln->x->dataType() != dt) return false;
+    if (g.M != ln->rows || g.aCol != 1 || ln->x->lengthOf() != g.M * g.K || ln->x->dataType() != dt) return false;
     prepareSpecialUse({z, ln->out}, {ln->x, ln->gain, ln->bias, w, b});
     d.bias = b->specialBuffer();
     d.epi = epi;
-    d.lnGain = ln->gain->specialBuffer(); d.lnBias = ln->bias->specialBuffer(); d.lnOut = ln->out->specialBuffer();
+    d.aRow = ln->xPitch;
+    d.lnGain = ln->gain->specialBuffer(); d.lnBias = ln->bias->specialBuffer(); d.lnOut = ln->out->specialBuffer(); d.lnOutRow = ln->outPitch;
     const bool done = launchGemm(stream(), dt, ln->x->specialBuffer(), w->specialBuffer(), z->specialBuffer(), d);
     if (done) registerSpecialUse({z, ln->out}, {ln->x, ln->gain, ln->bias, w, b});
     return done;
@@ -1891,6 +1893,24 @@ std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& rec,
   std::vector<std::function<void()>> plan;
   nFused = 0;
   const size_t n = rec.size();
+  // is rec[li] a layer_norm that the xw_plus_b behind it can run as its prologue (products of one row, and of 5 to 32 rows
+  // of 320 to 768 values, the lengths the few-row product kernel normalises)?
+  auto lnPrologueAt = [&](size_t li, LnPrologue& out) {
+    if (li + 1 >= n) return false;
+    RecordedOp& r = rec[li];
+    RecordedOp& x = rec[li + 1];
+    if (!isRowLayerNorm(r) || x.kind != RecordedOp::CUSTOM || x.op->name != "xw_plus_b" || x.ctx.inputs.size() < 3 || !x.ctx.inputs[0] ||
+        !sameView(x.ctx.inputs[0], r.ctx.outputs[0])) return false;
+    NDArray *lx = r.ctx.inputs[0], *lg = r.ctx.inputs[1], *lb = r.ctx.inputs[2], *lo = r.ctx.outputs[0];
+    LongType rr, cc, ss, r2, c2, s2;
+    const DataType dt = lx->dataType();
+    const bool ok = (dt == HALF || dt == BFLOAT16) && lg->dataType() == dt && lb->dataType() == dt && lo->dataType() == dt && asRows(lx, rr, cc, ss) &&
+                    (rr == 1 || (rr >= 5 && rr <= 32 && cc >= 320 && cc <= 768 && cc % 64 == 0)) && asRows(lo, r2, c2, s2) && r2 == rr && c2 == cc && lg->lengthOf() == cc && lb->lengthOf() == cc &&
+                    lo->buf.get() != lx->buf.get() && iArg(x.ctx, 0, 0) != 1;
+    if (!ok) return false;
+    out = LnPrologue{lx, lg, lb, lo, rr, ss, s2};
+    return true;
+  };
   for (size_t i = 0; i < n;) {
     RecordedOp& r = rec[i];
     // pairwise Add whose result the next op layer-normalises
@@ -1908,17 +1928,9 @@ std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& rec,
     // caches), a pairwise Add of the result to another array (the residual connection)
     {
       RecordedOp* lnOp = nullptr;
+      LnPrologue lnPro{};
       size_t xi = i;
-      if (isRowLayerNorm(r) && i + 1 < n && rec[i + 1].kind == RecordedOp::CUSTOM && rec[i + 1].op->name == "xw_plus_b" && rec[i + 1].ctx.inputs.size() >= 3 &&
-          rec[i + 1].ctx.inputs[0] && sameView(rec[i + 1].ctx.inputs[0], r.ctx.outputs[0])) {
-        NDArray *lx = r.ctx.inputs[0], *lg = r.ctx.inputs[1], *lb = r.ctx.inputs[2], *lo = r.ctx.outputs[0];
-        LongType rr, cc, ss, r2, c2, s2;
-        const DataType dt = lx->dataType();
-        const bool ok = (dt == HALF || dt == BFLOAT16) && lg->dataType() == dt && lb->dataType() == dt && lo->dataType() == dt && asRows(lx, rr, cc, ss) && rr == 1 &&
-                        asRows(lo, r2, c2, s2) && r2 == 1 && c2 == cc && lg->lengthOf() == cc && lb->lengthOf() == cc && lo->buf.get() != lx->buf.get() &&
-                        iArg(rec[i + 1].ctx, 0, 0) != 1;
-        if (ok) { lnOp = &r; xi = i + 1; }
-      }
+      if (lnPrologueAt(i, lnPro)) { lnOp = &r; xi = i + 1; }
       RecordedOp& xw = rec[xi];
       if (xw.kind == RecordedOp::CUSTOM && xw.op->name == "xw_plus_b" && xw.ctx.outputs.size() >= 1 && xw.ctx.outputs[0] && xw.ctx.inputs.size() >= 3 &&
           xw.ctx.inputs[0] && xw.ctx.inputs[1] && xw.ctx.inputs[2]) {
@@ -1928,6 +1940,7 @@ std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& rec,
         const bool zOk = (dt == HALF || dt == BFLOAT16) && asRows(z, zr, zc, zs) && iArg(xw.ctx, 2, 0) != 1;
         GemmEpilogue epi;          // array handles for now; device pointers when the step runs
         std::vector<RecordedOp*> absorbed;
+        LnPrologue lnAhead{};
         size_t j = xi + 1;
         while (zOk && j < n) {
           RecordedOp& f = rec[j];
@@ -1949,10 +1962,12 @@ std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& rec,
             if (c0 < 0 || c0 + sc > zc) break;
             epi.copy[epi.nCopy].dst = f.z; epi.copy[epi.nCopy].c0 = c0; epi.copy[epi.nCopy].c1 = c0 + sc; epi.copy[epi.nCopy].dstRow = ds;
             epi.nCopy++;
-          } else if (f.kind == RecordedOp::PAIRWISE && f.opNum == 0 && epi.resOut == nullptr && zr == 1 && (sameView(f.y, z) || sameView(f.x, z)) &&
-                     f.x->dataType() == dt && f.y->dataType() == dt) {
-            // (one-row products only: with more rows the Add merges with the layer_norm behind it instead, which measured faster
-            // than per-element residual traffic in the tile kernels' epilogues)
+          } else if (f.kind == RecordedOp::PAIRWISE && f.opNum == 0 && epi.resOut == nullptr && (sameView(f.y, z) || sameView(f.x, z)) &&
+                     f.x->dataType() == dt && f.y->dataType() == dt &&
+                     (zr == 1 || (zr >= 5 && zr <= 32 && j + 1 < n && isRowLayerNorm(rec[j + 1]) && sameView(f.z, rec[j + 1].ctx.inputs[0]) && lnPrologueAt(j + 1, lnAhead)))) {
+            // (one-row products, and the few-row ones whose sum goes into a layer_norm that the next product normalises on its
+            // way in; otherwise the Add merges with the layer_norm behind it, which measured faster than per-element residual
+            // traffic in the tile kernels' epilogues)
             NDArray* other = sameView(f.y, z) ? f.x : f.y;   // the addition commutes bit for bit
             LongType orr, oc, os;
             if (other->buf.get() == z->buf.get() || !asRows(other, orr, oc, os) || !asRows(f.z, fr, fc, fs) || orr != zr || oc != zc || fr != zr || fc != zc) break;
@@ -1968,7 +1983,7 @@ std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& rec,
         }
         if (lnOp || !absorbed.empty()) {
           RecordedOp* x = &xw;
-          plan.push_back([x, lnOp, epi, absorbed] {
+          plan.push_back([x, lnOp, lnPro, epi, absorbed] {
             GemmEpilogue e = epi;
             NDArray* z = x->ctx.outputs[0];
             std::vector<NDArray*> writes, reads;
@@ -1986,8 +2001,7 @@ std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& rec,
             const GemmEpilogue* ep = epiOk ? &e : nullptr;
             bool applied = false, done = false;
             if (lnOp) {
-              LnPrologue ln{lnOp->ctx.inputs[0], lnOp->ctx.inputs[1], lnOp->ctx.inputs[2], lnOp->ctx.outputs[0]};
-              done = xwPlusBImpl(x->ctx, ep, &ln);
+              done = xwPlusBImpl(x->ctx, ep, &lnPro);
               applied = done && epiOk;
               if (!done) runRecorded(lnOp);
             }

@@ -45,6 +45,12 @@ struct GemmArgs {
   const void* bias;   // optional [N] row added to every output row (xw_plus_b), same type as C
   int hasEpi;
   GemmEpilogue epi;   // extra outputs derived from the stored C (kernels that call epilogueExtras)
+  // layer-norm prologue over the rows of A (gemm_skinny32 with its LN flag only)
+  const void* lnGain;
+  const void* lnBias;
+  void* lnOut;
+  LongType lnOutRow;
+  float lnEps;
 };
 typedef __attribute__((ext_vector_type(4))) float f32x4v;
 
@@ -1863,6 +1869,7 @@ static GemmArgs toArgs(const GemmDesc& d) {
   g.splits = 1; g.ktPerSplit = 0; g.partial = nullptr; g.bias = d.bias;
   g.hasEpi = d.epi ? 1 : 0;
   if (d.epi) g.epi = *d.epi;
+  g.lnGain = d.lnGain; g.lnBias = d.lnBias; g.lnOut = d.lnOut; g.lnOutRow = d.lnOutRow; g.lnEps = d.lnEps;
   return g;
 }
 
@@ -2022,7 +2029,14 @@ static bool tryGemvStrip(hipStream_t s, const GemmDesc& d, const void* A, const 
 // while the current one is multiplied.  The waves' 32x32 partial tiles are added up through LDS -- one launch, where the
 // split-K tile kernel needs a second one to add its partial tiles.
 // Accumulator layout: lane (m = lane % 32, h = lane / 32), register r holds column 8 * (r / 4) + 4 * h + r % 4.
-template <typename T>
+// LN_NV > 0: the rows of X are layer-normalised over K on the way in (and block 0 writes the normalised rows to g.lnOut),
+// with the bits of the separate layer_norm kernel, which gives a wave to a row: lane l of that wave sums the 8-value
+// vectors l and l + 64 of the row (LN_NV = 2 passes; one pass for K <= 512), then the wave adds its lanes up as a balanced
+// tree over the lane numbers.  Here the 8 threads of a row hold vector 8 * tile + lkg of every tile, so thread lkg stands in
+// for that wave's lanes 8 * jj + lkg, jj = 0..7: the first three levels of the tree run across the 8 threads (the same lane
+// exchanges), the last three inside a thread over jj.  Everything else of the normalisation is per element.  Needs the
+// whole row in registers: K <= 768.
+template <typename T, int LN_NV = 0>
 __global__ __launch_bounds__(256) void gemm_skinny32(GemmArgs g, const T* __restrict__ X, const T* __restrict__ Wt, T* __restrict__ C) {
   constexpr int CT = 6;                                // 64-k tiles per chunk
   constexpr int GROUP = 33;                            // slots per k-group (32 rows + 1: conflict-free column reads)
@@ -2052,8 +2066,100 @@ __global__ __launch_bounds__(256) void gemm_skinny32(GemmArgs g, const T* __rest
 #pragma unroll
   for (int r = 0; r < 16; r++) acc[r] = 0.f;
   const int mrow = lane & 31, h = lane >> 5;
-  load(0, 0);
-  if (CT < tiles) load(1, CT);
+  if constexpr (LN_NV == 0) {
+    load(0, 0);
+    if (CT < tiles) load(1, CT);
+  }
+  if constexpr (LN_NV > 0) {
+    using IO = RawIO<T>;
+    using Raw = typename IO::raw;
+    const T* gp = reinterpret_cast<const T*>(g.lnGain) + lkg * 8;
+    const T* bp = reinterpret_cast<const T*>(g.lnBias) + lkg * 8;
+    u32x4 gr[2 * CT], br[2 * CT];
+    // loads come back in the order they were issued: the rows (written by the kernel before this one, so close by), gain
+    // and bias go first and the weights, which come from far away, last -- the normalisation then runs while they travel
+#pragma unroll
+    for (int j = 0; j < 2 * CT; j++) {
+      const int jc = j < tiles ? j : tiles - 1;
+      xr[j / CT][j % CT] = *reinterpret_cast<const u32x4*>(xp + (LongType)jc * 64);
+    }
+#pragma unroll
+    for (int j = 0; j < 2 * CT; j++) {
+      const int jc = j < tiles ? j : tiles - 1;
+      gr[j] = *reinterpret_cast<const u32x4*>(gp + jc * 64);
+      br[j] = *reinterpret_cast<const u32x4*>(bp + jc * 64);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 2 * CT; j++) {
+      const int jc = j < tiles ? j : tiles - 1;
+      wr[j / CT][j % CT] = *reinterpret_cast<const u32x4*>(wp + (LongType)jc * 64);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // the row's total of f(vector), f evaluated per tile into part[]: per stand-in lane the passes in order (a lane past
+    // the row's end adds the row's last vector times zero, as the separate kernel's lanes do), then the tree
+    auto rowTotal = [&](const float (&part)[2 * CT]) {
+      float last = 0.f;
+#pragma unroll
+      for (int j = 0; j < 2 * CT; j++) if (j == tiles - 1) last = part[j];
+      last = __shfl(last, lane | 7, 64);                  // the row's last vector sits with lkg = 7
+      float o[8];
+#pragma unroll
+      for (int jj = 0; jj < 8; jj++) {
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < LN_NV; i++) {
+          const int tile = jj + 8 * i;
+          const bool in = tile < tiles;
+          const float p = tile < 2 * CT && in ? part[tile < 2 * CT ? tile : 0] : last;
+          s += p * (in ? 1.f : 0.f);
+        }
+        o[jj] = group_allreduce<SumOp, 8>(s);
+      }
+      return ((o[0] + o[1]) + (o[2] + o[3])) + ((o[4] + o[5]) + (o[6] + o[7]));
+    };
+    float part[2 * CT];
+#pragma unroll
+    for (int j = 0; j < 2 * CT; j++) {
+      float v[8];
+      IO::unpack(__builtin_bit_cast(Raw, xr[j / CT][j % CT]), v);
+      float p = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e++) p += v[e];
+      part[j] = p;
+    }
+    const float mean = rowTotal(part) / (float)(int)g.K;
+#pragma unroll
+    for (int j = 0; j < 2 * CT; j++) {
+      float v[8];
+      IO::unpack(__builtin_bit_cast(Raw, xr[j / CT][j % CT]), v);
+      float p = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e++) { const float d = v[e] - mean; p += d * d; }
+      part[j] = p;
+    }
+    const float var = rowTotal(part) / (float)(int)g.K;
+    const float rstd = 1.f / sqrtf(var + g.lnEps);
+    const bool writer = blockIdx.x == 0 && lrow < g.M;
+    T* lo = reinterpret_cast<T*>(g.lnOut) + (LongType)lrow * g.lnOutRow + lkg * 8;
+#pragma unroll
+    for (int j = 0; j < 2 * CT; j++) {
+      float v[8], gn[8], bs[8];
+      IO::unpack(__builtin_bit_cast(Raw, xr[j / CT][j % CT]), v);
+      IO::unpack(__builtin_bit_cast(Raw, gr[j]), gn);
+      IO::unpack(__builtin_bit_cast(Raw, br[j]), bs);
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        const float d = v[e] - mean;
+        float y = d * rstd * gn[e];
+        y += bs[e];
+        v[e] = y;
+      }
+      const Raw packed = IO::pack(v);
+      xr[j / CT][j % CT] = __builtin_bit_cast(u32x4, packed);
+      if (writer && j < tiles) *reinterpret_cast<Raw*>(lo + j * 64) = packed;
+    }
+  }
   auto chunk = [&](int set, int tile0) {
     const int n = tiles - tile0 < CT ? tiles - tile0 : CT;
 #pragma unroll
@@ -2106,6 +2212,16 @@ static bool tryGemmSkinny(hipStream_t s, const GemmDesc& d, const void* A, const
   constexpr size_t LDS = (size_t)2 * 6 * 8 * 33 * 16;   // 50,688 B; the 16 KiB of partial tiles reuse it
   static_assert(LDS <= 64 * 1024 && (size_t)4 * 16 * 64 * sizeof(float) <= LDS / 2, "gemm_skinny32 must fit the default dynamic LDS limit");
   GemmArgs g = toArgs(d);
+  if (d.lnGain) {
+    // what the separate layer_norm runs as one wave per row with one or two 512-value passes: rows of 320 to 768 values
+    // with a bias, every vector 16-byte aligned
+    if (!d.lnBias || !d.lnOut || d.K < 320 || d.K > 768 || d.lnOutRow % 8 != 0) return false;
+    if ((reinterpret_cast<uintptr_t>(d.lnGain) | reinterpret_cast<uintptr_t>(d.lnBias) | reinterpret_cast<uintptr_t>(d.lnOut)) & 15) return false;
+    noteKernel("gemm_skinny32<%s,ln>", tname<T>());
+    if (d.K <= 512) hipLaunchKernelGGL((gemm_skinny32<T, 1>), dim3((unsigned)(d.N / 32)), dim3(256), LDS, s, g, (const T*)A, (const T*)B, (T*)C);
+    else hipLaunchKernelGGL((gemm_skinny32<T, 2>), dim3((unsigned)(d.N / 32)), dim3(256), LDS, s, g, (const T*)A, (const T*)B, (T*)C);
+    return true;
+  }
   noteKernel("gemm_skinny32<%s>", tname<T>());
   hipLaunchKernelGGL((gemm_skinny32<T>), dim3((unsigned)(d.N / 32)), dim3(256), LDS, s, g, (const T*)A, (const T*)B, (T*)C);
   return true;
@@ -2113,8 +2229,9 @@ static bool tryGemmSkinny(hipStream_t s, const GemmDesc& d, const void* A, const
 
 template <typename T>
 static bool dispatch16(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
-  if (d.lnGain) {   // only the one-row product against k-contiguous weights normalises its row on the way in
+  if (d.lnGain) {   // only the products of 1 and of 5 to 32 rows against k-contiguous weights normalise their rows on the way in
     if (d.M == 1 && d.N > 1 && d.batch == 1 && d.bRow == 1 && d.cCol == 1) return tryGemvRowdotPre<T>(s, d, A, B, C);
+    if (d.M >= 5 && d.M <= 32) return tryGemmSkinny<T>(s, d, A, B, C);
     return false;
   }
   bool aKC = false, bKC = false;

@@ -230,12 +230,13 @@ struct GemmDesc {
   float alpha = 1.f, beta = 0.f;
   const void* bias = nullptr;   // optional dense [N] row (type of C) added to every output row
   const GemmEpilogue* epi = nullptr;
-  // optional prologue: op(A) is one row (M = 1) and what is multiplied is layer_norm(row; lnGain, lnBias, lnEps) over its K
-  // elements, which also goes to lnOut [K].  Counts as an epilogue request for the return value of launchGemm: kernels
-  // that cannot do it launch nothing.
+  // optional prologue: op(A) is one row (M = 1) or 5 to 32 rows, and what is multiplied is layer_norm(row; lnGain, lnBias,
+  // lnEps) over each row's K elements, which also goes to lnOut (rows lnOutRow elements apart).  Counts as an epilogue
+  // request for the return value of launchGemm: kernels that cannot do it launch nothing.
   const void* lnGain = nullptr;
   const void* lnBias = nullptr;
   void* lnOut = nullptr;
+  LongType lnOutRow = 0;
   float lnEps = 1e-5f;
 };
 // Returns true when every requested epilogue output was written; false: C was computed by a kernel without them and the
