@@ -422,7 +422,7 @@ static void layerNormImpl(Context& c, NDArray* x, NDArray* gain, NDArray* bias, 
   const float eps = 1e-5f;
   const bool lastAxisOnly = axes.size() == 1 && axes[0] == rank - 1 && dimC == rank - 1 && gain && gain->strideAt(0) == 1 && (!bias || bias->strideAt(0) == 1);
   bool done = false;
-  if (lastAxisOnly && x->sizeAt(rank - 1) <= 16384) {   // the row kernels say themselves which lengths they take
+  if (lastAxisOnly) {   // the row kernels say themselves which rows they take
     RowPlan p = buildRowPlan(x->shapeInfo(), z->shapeInfo(), rank - 1);
     done = launchLayerNormRows(stream(), x->dataType(), x->specialBuffer(), gain->specialBuffer(), bias ? bias->specialBuffer() : nullptr, z->specialBuffer(), p, eps);
   }
@@ -1888,6 +1888,8 @@ void RecordedOp::adopt() {
   for (NDArray*& a : ctx.outputs) own(a);
 }
 
+int& fusedAppliedCounter() { static int n = 0; return n; }
+
 std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& rec, int& nFused) {
   using namespace ops;
   std::vector<std::function<void()>> plan;
@@ -1917,7 +1919,7 @@ std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& rec,
     if (r.kind == RecordedOp::PAIRWISE && r.opNum == 0 && i + 1 < n && isRowLayerNorm(rec[i + 1]) && sameView(r.z, rec[i + 1].ctx.inputs[0])) {
       RecordedOp* a = &r;
       RecordedOp* l = &rec[i + 1];
-      plan.push_back([a, l] { if (!tryAddLayerNorm(*a, *l)) { runRecorded(a); runRecorded(l); } });
+      plan.push_back([a, l] { if (tryAddLayerNorm(*a, *l)) fusedAppliedCounter() += 1; else { runRecorded(a); runRecorded(l); } });
       nFused += 1;
       i += 2;
       continue;
@@ -2003,9 +2005,10 @@ std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& rec,
             if (lnOp) {
               done = xwPlusBImpl(x->ctx, ep, &lnPro);
               applied = done && epiOk;
-              if (!done) runRecorded(lnOp);
+              if (done) fusedAppliedCounter() += 1; else runRecorded(lnOp);
             }
             if (!done) applied = xwPlusBImpl(x->ctx, ep) && epiOk;
+            if (applied) fusedAppliedCounter() += (int)absorbed.size();
             if (applied) registerSpecialUse(writes, reads);
             else for (RecordedOp* f : absorbed) runRecorded(f);
           });

@@ -47,8 +47,11 @@ struct RecordedOp {
   std::vector<std::shared_ptr<NDArray>> owned;
   void adopt();
 };
-// The launch plan of the sequence; nFused counts the ops that were absorbed into a neighbour's kernel.
+// The launch plan of the sequence; nFused counts the ops that the plan gives to a neighbour's kernel.  A step may still
+// run its ops separately when the kernel declines the operands it meets at run time: fusedAppliedCounter() is raised by
+// every op whose work did run inside a neighbour's kernel (the caller zeroes it before running a plan).
 std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& ops, int& nFused);
+int& fusedAppliedCounter();
 
 // shared with the legacy facade
 void runIndexReduce(const char* fn, int opNum, NDArray* x, NDArray* z, const std::vector<LongType>& dims);

@@ -509,31 +509,59 @@ __global__ __launch_bounds__(EW_BLOCK) void tail_generic(int k, DevShape sz, Dev
 // transforms with two parameters; any strides, any float dtypes.  The clip compares in double against the bounds as given
 // and stores the bound rounded to the output type (helpers/cpu/clip.cpp:211-219); the other two evaluate in the
 // accumulator type of the array (float for 16- and 32-bit arrays).
+__device__ __forceinline__ double scalar2_eval(int k, double a, bool inDouble, double s1, double s2) {
+  double r;
+  if (k == S2_CLIP_BY_VALUE) {
+    r = a > s2 ? s2 : (a < s1 ? s1 : a);
+  } else if (inDouble) {
+    const double cut = (double)3.79297773665f;
+    if (k == S2_AFFINE) r = s1 * a + s2;
+    else if (k == S2_SCALED_TANH) r = s1 * d_tanh(s2 * a);
+    else if (k == S2_STABILIZE) r = a * s1 > cut ? cut / s1 : (a * s1 < -cut ? -cut / s1 : a);
+    else if (a >= s1 && a <= s2) r = a;
+    else r = floor((s1 == 0.0 && s2 == 1.0 ? 1.0 / (1.0 + exp(-a)) : a) * (s2 - s1)) + s1;
+  } else {
+    const float fa = (float)a, f1 = (float)s1, f2 = (float)s2, cut = 3.79297773665f;
+    if (k == S2_AFFINE) r = f1 * fa + f2;
+    else if (k == S2_SCALED_TANH) r = f1 * d_tanh(f2 * fa);
+    else if (k == S2_STABILIZE) r = fa * f1 > cut ? cut / f1 : (fa * f1 < -cut ? -cut / f1 : fa);
+    else if (fa >= f1 && fa <= f2) r = fa;
+    else r = floorf((f1 == 0.f && f2 == 1.f ? 1.f / (1.f + expf(-fa)) : fa) * (f2 - f1)) + f1;
+  }
+  return r;
+}
 __global__ __launch_bounds__(EW_BLOCK) void scalar2_generic(int k, DevShape sz, DevShape sx, int zdt, int xdt, void* z, const void* x,
                                                             LongType n, double s1, double s2) {
   const LongType step = (LongType)gridDim.x * EW_BLOCK;
   for (LongType i = (LongType)blockIdx.x * EW_BLOCK + threadIdx.x; i < n; i += step) {
     const LongType oz = walk<LongType>(sz, i), ox = walk<LongType>(sx, i);
-    const double a = load_any(x, xdt, ox);
-    double r;
-    if (k == S2_CLIP_BY_VALUE) {
-      r = a > s2 ? s2 : (a < s1 ? s1 : a);
-    } else if (xdt == DOUBLE) {
-      const double cut = (double)3.79297773665f;
-      if (k == S2_AFFINE) r = s1 * a + s2;
-      else if (k == S2_SCALED_TANH) r = s1 * d_tanh(s2 * a);
-      else if (k == S2_STABILIZE) r = a * s1 > cut ? cut / s1 : (a * s1 < -cut ? -cut / s1 : a);
-      else if (a >= s1 && a <= s2) r = a;
-      else r = floor((s1 == 0.0 && s2 == 1.0 ? 1.0 / (1.0 + exp(-a)) : a) * (s2 - s1)) + s1;
-    } else {
-      const float fa = (float)a, f1 = (float)s1, f2 = (float)s2, cut = 3.79297773665f;
-      if (k == S2_AFFINE) r = f1 * fa + f2;
-      else if (k == S2_SCALED_TANH) r = f1 * d_tanh(f2 * fa);
-      else if (k == S2_STABILIZE) r = fa * f1 > cut ? cut / f1 : (fa * f1 < -cut ? -cut / f1 : fa);
-      else if (fa >= f1 && fa <= f2) r = fa;
-      else r = floorf((f1 == 0.f && f2 == 1.f ? 1.f / (1.f + expf(-fa)) : fa) * (f2 - f1)) + f1;
+    store_any(z, zdt, oz, scalar2_eval(k, load_any(x, xdt, ox), xdt == DOUBLE, s1, s2));
+  }
+}
+// the same on dense arrays of one float type: 16-byte vectors, one per thread, and a scalar tail
+template <typename T>
+__global__ __launch_bounds__(EW_BLOCK) void scalar2_contig(int k, const T* __restrict__ x, T* __restrict__ z, LongType n, double s1, double s2) {
+  constexpr int V = 16 / sizeof(T);
+  using IO = RawIO<T>;
+  using RT = typename IO::raw;
+  using A = typename Conv<T>::acc;
+  constexpr bool DBL = sizeof(T) == 8;
+  const LongType nvec = n / V;
+  const LongType i = (LongType)blockIdx.x * EW_BLOCK + threadIdx.x;
+  if (i < nvec) {
+    A a[V];
+    IO::unpack(*(reinterpret_cast<const RT*>(x) + i), a);
+#pragma unroll
+    for (int e = 0; e < V; e++) {
+      const double r = scalar2_eval(k, (double)a[e], DBL, s1, s2);
+      a[e] = DBL ? (A)r : (A)(float)r;
     }
-    store_any(z, zdt, oz, r);
+    *(reinterpret_cast<RT*>(z) + i) = IO::pack(a);
+  }
+  const LongType tail = nvec * V + i;
+  if (tail < n) {
+    const double r = scalar2_eval(k, (double)to_float(x[tail]), DBL, s1, s2);
+    z[tail] = Conv<T>::from(DBL ? (A)r : (A)(float)r);
   }
 }
 
@@ -960,6 +988,19 @@ void launchScalarOp(hipStream_t s, PairwiseKind k, DataType dt, const void* x, d
 void launchScalar2Op(hipStream_t s, Scalar2Kind k, DataType xdt, DataType zdt, const void* x, double s1, double s2, void* z,
                      const EwPlan& p) {
   if (p.length == 0) return;
+  if (p.sameShape && p.contiguous && xdt == zdt && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(z)) & 15) == 0 &&
+      (xdt == FLOAT32 || xdt == DOUBLE || xdt == HALF || xdt == BFLOAT16)) {
+    const LongType V = 16 / (LongType)sizeOf(xdt);
+    const dim3 grid((unsigned)((p.length / V + EW_BLOCK) / EW_BLOCK));   // one vector per thread; the block after the last whole one holds the tail
+    switch (xdt) {
+      case FLOAT32: hipLaunchKernelGGL((scalar2_contig<float>), grid, dim3(EW_BLOCK), 0, s, (int)k, (const float*)x, (float*)z, p.length, s1, s2); break;
+      case DOUBLE: hipLaunchKernelGGL((scalar2_contig<double>), grid, dim3(EW_BLOCK), 0, s, (int)k, (const double*)x, (double*)z, p.length, s1, s2); break;
+      case HALF: hipLaunchKernelGGL((scalar2_contig<f16_t>), grid, dim3(EW_BLOCK), 0, s, (int)k, (const f16_t*)x, (f16_t*)z, p.length, s1, s2); break;
+      default: hipLaunchKernelGGL((scalar2_contig<bf16_t>), grid, dim3(EW_BLOCK), 0, s, (int)k, (const bf16_t*)x, (bf16_t*)z, p.length, s1, s2); break;
+    }
+    HIP_CHECK(hipGetLastError());
+    return;
+  }
   hipLaunchKernelGGL(scalar2_generic, dim3(gridFor(p.length, EW_BLOCK)), dim3(EW_BLOCK), 0, s, (int)k, p.own[0], p.own[1], (int)zdt,
                      (int)xdt, z, x, p.length, s1, s2);
   HIP_CHECK(hipGetLastError());

@@ -1201,6 +1201,110 @@ __global__ __launch_bounds__(512) void gemm_mfma16r(GemmArgs g, const T* __restr
   storeAccTiles<T, TM, TN, false>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
 }
 
+// ---- 16-bit MFMA kernel for operands the vector loaders cannot take ---------------------------------------------------------
+// Rows that do not start on 16-byte boundaries (a row-major [K, 50257] matrix), a contiguous extent that is not a multiple
+// of 8, two non-unit strides, negative strides: the tiles are gathered element by element (2-byte loads, zero beyond the
+// edges) into the k-contiguous LDS layout, and from there on it is the two-stage tile kernel.  RF ("row fast"): neighbouring
+// lanes take neighbouring rows of one k -- for an operand whose unit (or smaller) stride runs along its rows; otherwise
+// neighbouring lanes take neighbouring k-groups of one row.
+template <int ROWS, int NT, bool RF>
+struct ElementTileLoader {
+  using Layout = TileLayout<ROWS, true>;
+  static constexpr int UNITS = ROWS * 8, PER = UNITS / NT;
+  static_assert(UNITS % NT == 0, "every thread gathers the same number of k-groups");
+  u32x4 reg[PER];
+  static __device__ __forceinline__ void unitOf(int u, int& kg, int& row) {
+    if (RF) { row = u % ROWS; kg = u / ROWS; } else { kg = u & 7; row = u >> 3; }
+  }
+  template <typename T>
+  __device__ __forceinline__ void load(const T* __restrict__ base, LongType rs, LongType ks, LongType row0, LongType rowLimit, LongType k0, LongType K, int t) {
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      int kg, row;
+      unitOf(t + i * NT, kg, row);
+      // every load is unconditional (positions past an edge re-read the last valid one and are zeroed afterwards): a
+      // predicated load would put a wait at every join, one memory latency per element
+      const LongType r = row0 + row, kb = k0 + kg * 8;
+      const T* p = base + (r < rowLimit ? r : rowLimit - 1) * rs;
+      unsigned e[8];
+#pragma unroll
+      for (int j = 0; j < 8; j++) e[j] = (unsigned)p[(kb + j < K ? kb + j : K - 1) * ks].bits;
+#pragma unroll
+      for (int j = 0; j < 8; j++) e[j] = (r < rowLimit && kb + j < K) ? e[j] : 0u;
+      reg[i] = u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
+    }
+  }
+  __device__ __forceinline__ void store(u32x4* __restrict__ lds, int t) {
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      int kg, row;
+      unitOf(t + i * NT, kg, row);
+      lds[Layout::slot(kg, row)] = reg[i];
+    }
+  }
+};
+template <typename T, int BM, int BN, int WM, int WN, bool A_RF, bool B_RF>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16u(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
+                                                              unsigned tilesM, unsigned tilesN) {
+  constexpr int BK = 64, NT = WM * WN * 64;
+  constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
+  using LayA = TileLayout<BM, true>;
+  using LayB = TileLayout<BN, true>;
+  constexpr int SLOTS_A = LayA::SLOTS, SLOTS_B = LayB::SLOTS, STAGE = SLOTS_A + SLOTS_B;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  u32x4* smem = reinterpret_cast<u32x4*>(smem_raw);
+  unsigned tm, tn;
+  tileOf(blockIdx.x, gridDim.x, tilesM, tilesN, tm, tn);
+  const LongType m0 = (LongType)tm * BM, n0 = (LongType)tn * BN;
+  { LongType oa, ob, oc; batchOffsets(g, blockIdx.z, oa, ob, oc); A += oa; B += ob; C += oc; }
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+  ElementTileLoader<BM, NT, A_RF> la;
+  ElementTileLoader<BN, NT, B_RF> lb;
+  const LongType KT = (g.K + BK - 1) / BK;
+  la.load(A, g.aRow, g.aCol, m0, g.M, 0, g.K, t);
+  lb.load(B, g.bCol, g.bRow, n0, g.N, 0, g.K, t);
+  la.store(smem, t);
+  lb.store(smem + SLOTS_A, t);
+  __syncthreads();
+  for (LongType kt = 0; kt < KT; kt++) {
+    const int cur = (int)(kt & 1);
+    if (kt + 1 < KT) {
+      la.load(A, g.aRow, g.aCol, m0, g.M, (kt + 1) * BK, g.K, t);
+      lb.load(B, g.bCol, g.bRow, n0, g.N, (kt + 1) * BK, g.K, t);
+    }
+    const u32x4* sA = smem + cur * STAGE;
+    const u32x4* sB = sA + SLOTS_A;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ks++) {
+      const int kg = ks * 2 + (lane >> 5);
+      u32x4 fa[TM], fb[TN];
+#pragma unroll
+      for (int i = 0; i < TM; i++) fa[i] = sA[LayA::slot(kg, wm * WTM + i * 32 + (lane & 31))];
+#pragma unroll
+      for (int j = 0; j < TN; j++) fb[j] = sB[LayB::slot(kg, wn * WTN + j * 32 + (lane & 31))];
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = Mfma16<T>::mma(fa[i], fb[j], acc[i][j]);
+    }
+    if (kt + 1 < KT) {
+      u32x4* dst = smem + (cur ^ 1) * STAGE;
+      la.store(dst, t);
+      lb.store(dst + SLOTS_A, t);
+    }
+    __syncthreads();
+  }
+  storeAccTiles<T, TM, TN, true>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
+}
+
 // How many K-splits a launch of BM x BN tiles gets: enough to put about two blocks on every CU when the tiles alone
 // cannot, bounded by the K-tiles there are and the partial-tile scratch.
 template <int BM, int BN>
@@ -2227,6 +2331,31 @@ static bool tryGemmSkinny(hipStream_t s, const GemmDesc& d, const void* A, const
   return true;
 }
 
+// the element-gathering tile kernel: any strides, any alignment (no epilogue outputs, no split-K)
+template <typename T, int BM, int BN, int WM, int WN>
+static bool launchMfma16uCfg(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
+  constexpr size_t LDS = (size_t)2 * (TileLayout<BM, true>::SLOTS + TileLayout<BN, true>::SLOTS) * 16;
+  const GemmArgs g = toArgs(d);
+  auto absl = [](LongType v) { return v < 0 ? -v : v; };
+  const bool aRF = absl(d.aRow) < absl(d.aCol), bRF = absl(d.bCol) < absl(d.bRow);   // the smaller stride runs along the rows
+  const unsigned tilesM = (unsigned)((d.M + BM - 1) / BM), tilesN = (unsigned)((d.N + BN - 1) / BN);
+  const dim3 grid(tilesM * tilesN, 1, (unsigned)d.batch), block(WM * WN * 64);
+  noteKernel("gemm_mfma16u<%s,%dx%d,arf=%d,brf=%d>", tname<T>(), BM, BN, (int)aRF, (int)bRF);
+#define LAUNCH_U(ARF, BRF) do { \
+    if (!DynLds<gemm_mfma16u<T, BM, BN, WM, WN, ARF, BRF>, (int)LDS>::granted()) return false; \
+    hipLaunchKernelGGL((gemm_mfma16u<T, BM, BN, WM, WN, ARF, BRF>), grid, block, LDS, s, g, (const T*)A, (const T*)B, (T*)C, tilesM, tilesN); } while (0)
+  if (aRF && bRF) LAUNCH_U(true, true); else if (aRF) LAUNCH_U(true, false); else if (bRF) LAUNCH_U(false, true); else LAUNCH_U(false, false);
+#undef LAUNCH_U
+  return true;
+}
+template <typename T>
+static bool launchMfma16u(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
+  if (d.M * d.N < 4096 || d.K < 32 || (d.M + 127) / 128 * ((d.N + 127) / 128) >= (1LL << 31)) return false;
+  if (d.M <= 32) return launchMfma16uCfg<T, 32, 128, 1, 4>(s, d, A, B, C);
+  // (256 x 256 tiles, twice the products per gathered element, measured no faster: 4095^3 720 against 744 us, 2047^3 377 against 202)
+  return launchMfma16uCfg<T, 128, 128, 2, 2>(s, d, A, B, C);
+}
+
 template <typename T>
 static bool dispatch16(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
   if (d.lnGain) {   // only the products of 1 and of 5 to 32 rows against k-contiguous weights normalise their rows on the way in
@@ -2250,6 +2379,7 @@ static bool dispatch16(hipStream_t s, const GemmDesc& d, const void* A, const vo
     return launchMfma16<T, false, false>(s, g, A, B, C, d.batch);
   }
   if (d.epi) return false;
+  if (launchMfma16u<T>(s, d, A, B, C)) return true;
   launchSimple<T>(s, A, B, C, d);
   return true;
 }

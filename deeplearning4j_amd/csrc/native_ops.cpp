@@ -1646,7 +1646,8 @@ struct CapturedGraph {
   CaptureRecord record;           // the buffers the recorded kernels read and write
   std::vector<RecordedOp> ops;    // the op calls the facade recognised, in call order
   int opCalls = 0;                // every op entry point called during the capture
-  int fusedOps = 0;               // ops that ended up inside a neighbour's kernel
+  int fusedOps = 0;               // ops that the merged plan gives to a neighbour's kernel
+  int fusedApplied = 0;           // ... and how many of them ran there the last time the plan was executed
   std::vector<std::function<void()>> plan;   // the merged sequence as ordinary launches (empty: a call went unrecorded)
 };
 // how nd4jhipGraphLaunch replays: 0 the instantiated HIP graph, 1 the merged sequence launched kernel by kernel
@@ -1719,7 +1720,9 @@ Nd4jPointer nd4jhipGraphEndCapture(void) {
         closer.streamOpen = true;
         std::vector<RecordedOp> keep;
         keep.swap(cg->ops);                   // replayed ops must not be recorded a second time
+        fusedAppliedCounter() = 0;
         try { for (auto& step : cg->plan) step(); } catch (std::exception& ex) { failure = ex.what(); } catch (...) { failure = "unknown native error"; }
+        cg->fusedApplied = fusedAppliedCounter();
         cg->ops.swap(keep);
         e = hipStreamEndCapture(execStream(), &merged);
         closer.streamOpen = false;
@@ -1786,7 +1789,9 @@ int nd4jhipGraphLaunch(Nd4jPointer graph) {
     for (auto& b : cg->record.writes) ND4J_REQUIRE(!b->closed, "nd4jhipGraphLaunch: a buffer the graph writes has been closed");
     const bool syncWas = Environment::get().syncAfterCustomOp;
     Environment::get().syncAfterCustomOp = false;   // as during the capture: nothing waits inside a step
+    fusedAppliedCounter() = 0;
     try { for (auto& step : cg->plan) step(); } catch (...) { Environment::get().syncAfterCustomOp = syncWas; throw; }
+    cg->fusedApplied = fusedAppliedCounter();
     Environment::get().syncAfterCustomOp = syncWas;
     return 0;
   }
@@ -1850,6 +1855,7 @@ int nd4jhipGraphAudit(Nd4jPointer graph) {
   GUARD_END(-1)
 }
 int nd4jhipGraphFusedOps(Nd4jPointer graph) { return graph ? static_cast<CapturedGraph*>(graph)->fusedOps : 0; }
+int nd4jhipGraphFusedApplied(Nd4jPointer graph) { return graph ? static_cast<CapturedGraph*>(graph)->fusedApplied : 0; }
 void nd4jhipSetGraphReplayMode(int mode) { g_graphReplayMode = mode == 1 ? 1 : 0; }
 int nd4jhipGetGraphReplayMode(void) { return g_graphReplayMode; }
 void nd4jhipGraphDestroy(Nd4jPointer graph) {

@@ -839,6 +839,81 @@ __global__ __launch_bounds__(256, WALK ? 1 : 8) void layernorm_stream(const T* _
   }
 }
 
+// Rows too long for a block's registers (beyond 8 vectors per thread): one block of 16 waves per row and three passes over
+// it with 16-byte vectors -- total, squared distances, output; the second and third find the row in the L2.
+template <typename T, bool HAS_BIAS>
+__global__ __launch_bounds__(1024) void layernorm_long(const T* __restrict__ x, const T* __restrict__ gain, const T* __restrict__ bias, T* __restrict__ z,
+                                                       LongType L, LongType xPitch, LongType zPitch, float eps) {
+  using A = typename Conv<T>::acc;
+  using IO = RawIO<T>;
+  using Raw = typename IO::raw;
+  constexpr int VEC = IO::N;
+  __shared__ A lds[16];
+  const T* xr = x + (LongType)blockIdx.x * xPitch;
+  T* zr = z + (LongType)blockIdx.x * zPitch;
+  const LongType nv = L / VEC;
+  constexpr int U = 4;   // vectors a thread has in flight (positions past the row's end re-read its last vector and are left out)
+  A sum = (A)0;
+  for (LongType v0 = threadIdx.x; v0 < nv; v0 += U * 1024) {
+    Raw r[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) { const LongType v = v0 + u * 1024; r[u] = *reinterpret_cast<const Raw*>(xr + (v < nv ? v : nv - 1) * VEC); }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      A vals[VEC];
+      IO::unpack(r[u], vals);
+      A part = (A)0;
+#pragma unroll
+      for (int e = 0; e < VEC; e++) part += vals[e];
+      if (v0 + u * 1024 < nv) sum += part;
+    }
+  }
+  sum = block_allreduce<SumOp, 16, A>(sum, lds);
+  const A mean = sum / (A)L;
+  A sq = (A)0;
+  for (LongType v0 = threadIdx.x; v0 < nv; v0 += U * 1024) {
+    Raw r[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) { const LongType v = v0 + u * 1024; r[u] = *reinterpret_cast<const Raw*>(xr + (v < nv ? v : nv - 1) * VEC); }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      A vals[VEC];
+      IO::unpack(r[u], vals);
+      A part = (A)0;
+#pragma unroll
+      for (int e = 0; e < VEC; e++) { const A d = vals[e] - mean; part += d * d; }
+      if (v0 + u * 1024 < nv) sq += part;
+    }
+  }
+  sq = block_allreduce<SumOp, 16, A>(sq, lds);
+  const A var = L > 1 ? sq / (A)L : (A)0;
+  const A rstd = (A)1 / r_sqrt<A>(var + (A)eps);
+  for (LongType v0 = threadIdx.x; v0 < nv; v0 += 2 * 1024) {
+    Raw r[2], gr[2], br[2];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const LongType v = v0 + u * 1024, vc = v < nv ? v : nv - 1;
+      r[u] = *reinterpret_cast<const Raw*>(xr + vc * VEC);
+      gr[u] = *reinterpret_cast<const Raw*>(gain + vc * VEC);
+      if (HAS_BIAS) br[u] = *reinterpret_cast<const Raw*>(bias + vc * VEC);
+    }
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      A vals[VEC], g[VEC], b[VEC];
+      IO::unpack(r[u], vals);
+      IO::unpack(gr[u], g);
+      if (HAS_BIAS) IO::unpack(br[u], b);
+#pragma unroll
+      for (int e = 0; e < VEC; e++) {
+        A y = (vals[e] - mean) * rstd * g[e];
+        if (HAS_BIAS) y += b[e];
+        vals[e] = y;
+      }
+      if (v0 + u * 1024 < nv) *reinterpret_cast<Raw*>(zr + (v0 + u * 1024) * VEC) = IO::pack(vals);
+    }
+  }
+}
+
 template <typename T>
 static bool layerNormTyped(hipStream_t s, const void* x, const void* gain, const void* bias, void* z, const RowPlan& p, float eps) {
   constexpr int V = 16 / sizeof(T);
@@ -914,6 +989,12 @@ static bool layerNormTyped(hipStream_t s, const void* x, const void* gain, const
     if (L <= 4 * perBlock) { LN(256, 4, gb); return true; }
     if (L <= 8 * perBlock) { LN(256, 8, gb); return true; }
 #undef LN
+    if (p.outerX.rank <= 1 && p.outerZ.rank <= 1 && L % V == 0 && p.rows < (1LL << 31)) {
+      const LongType xp = p.outerX.rank ? p.outerX.stride[0] : 0, zp = p.outerZ.rank ? p.outerZ.stride[0] : 0;
+      if (bt) hipLaunchKernelGGL((layernorm_long<T, true>), dim3((unsigned)p.rows), dim3(1024), 0, s, xt, gt, bt, zt, L, xp, zp, eps);
+      else hipLaunchKernelGGL((layernorm_long<T, false>), dim3((unsigned)p.rows), dim3(1024), 0, s, xt, gt, bt, zt, L, xp, zp, eps);
+      return true;
+    }
   }
   if (L <= 64 * 16) { hipLaunchKernelGGL((layernorm_rows<T, 64, 16, 1>), dim3(gw), dim3(256), 0, s, a, xt, gt, bt, zt, eps); return true; }
   if (L <= 256 * 32) { hipLaunchKernelGGL((layernorm_rows<T, 256, 32, 1>), dim3(gb), dim3(256), 0, s, a, xt, gt, bt, zt, eps); return true; }

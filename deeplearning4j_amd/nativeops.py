@@ -178,6 +178,7 @@ _SIGS = {
     "nd4jhipGraphLaunch": (ctypes.c_int, [c_ptr]),
     "nd4jhipGraphDestroy": (None, [c_ptr]),
     "nd4jhipGraphFusedOps": (ctypes.c_int, [c_ptr]),
+    "nd4jhipGraphFusedApplied": (ctypes.c_int, [c_ptr]),
     "nd4jhipSetGraphReplayMode": (None, [ctypes.c_int]),
     "nd4jhipGetGraphReplayMode": (ctypes.c_int, []),
     "nd4jhipBuildInfo": (ctypes.c_char_p, []),

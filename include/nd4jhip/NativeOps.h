@@ -303,6 +303,11 @@ ND4JHIP_EXPORT void nd4jhipGraphDestroy(Nd4jPointer graph);
  * bit, into the same arrays.  This returns how many op calls were absorbed that way (0: the graph holds the calls as
  * made).  ND4JHIP_GRAPH_FUSION=0 in the environment switches the pass off. */
 ND4JHIP_EXPORT int nd4jhipGraphFusedOps(Nd4jPointer graph);
+/* The count above is taken when the merged plan is laid out.  A merged step still asks its kernel at run time whether it
+ * takes the operands it meets (alignment, strides) and runs the ops apart when it does not.  This returns how many op
+ * calls did run inside a neighbour's kernel the last time the plan was executed: while End re-recorded it, or on the
+ * latest kernel-by-kernel replay.  Equal to nd4jhipGraphFusedOps when every merged kernel ran. */
+ND4JHIP_EXPORT int nd4jhipGraphFusedApplied(Nd4jPointer graph);
 /* How nd4jhipGraphLaunch replays a recording (no counterpart in the reference, like the capture calls themselves).
  * 0: the instantiated HIP graph, one launch.  1: the recorded, merged sequence launched kernel by kernel on the execution
  * stream by the library itself -- the same kernels with the same arguments, without the caller's per-op calls; a kernel

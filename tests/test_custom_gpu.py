@@ -342,7 +342,7 @@ def test_softmax_edge_semantics(ex, oracle):
 
 # ---- layer_norm ------------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype,rtol,atol", [(FLOAT32, 1e-5, 1e-5), (BFLOAT16, 1e-2, 1e-2), (HALF, 1e-2, 1e-2)])
-@pytest.mark.parametrize("shape", [(4, 64, 768), (3, 5, 100), (7, 2048), (2, 3, 5000), (4099, 768), (4097, 40), (41, 101, 256)])
+@pytest.mark.parametrize("shape", [(4, 64, 768), (3, 5, 100), (7, 2048), (2, 3, 5000), (4099, 768), (4097, 40), (41, 101, 256), (3, 40000), (2, 20004)])
 def test_layer_norm_last_axis(ex, oracle, dtype, rtol, atol, shape):
     rng = np.random.default_rng(shape[-1])
     C = shape[-1]
@@ -857,6 +857,11 @@ def test_two_parameter_transforms_match_oracle(ex, oracle, dtype):
     fin = np.isfinite(xr)
     got = ex.exec_transform_strict(3, dx, extra_args=[2.5, -0.75]).to_float()
     assert_close(got[fin], onp.affine(xr.astype(np.float64), 2.5, -0.75)[fin], tol, tol, "Affine")
+    # the dense array goes through the vector kernel, the permuted view through the element-wise one: same bits
+    for op_num, extra in ((3, [2.5, -0.75]), (2, [1.7159, 0.6666]), (19, [2.0]), (25, [0.0, 1.0]), (25, [2.0, 4.0])):
+        dense = ex.exec_transform_strict(op_num, dx, extra_args=extra).to_numpy()
+        strided = ex.exec_transform_strict(op_num, view, extra_args=extra).to_numpy()
+        assert np.array_equal(strided.view(np.uint8), dense.transpose(2, 0, 1).copy().view(np.uint8)), (op_num, extra)
     got = ex.exec_transform_strict(2, dx, extra_args=[1.7159, 0.6666]).to_float()
     # the parameters reach the kernel rounded to the array type
     a, b = (np.asarray(v, np.float64) for v in (1.7159, 0.6666))

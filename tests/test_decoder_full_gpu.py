@@ -114,6 +114,8 @@ def _gpt2_small_graph_replay_matches_eager(ex, gpt2, batch):
     # computed by the products that consume them
     fused = [ex.L.nd4jhipGraphFusedOps(g) for g in dec._graphs.values()]
     assert fused and min(fused) == 7 * cfg.n_layer, fused
+    # ... and every one of them did run inside its neighbour's kernel (no merged step fell back to separate launches)
+    assert [ex.L.nd4jhipGraphFusedApplied(g) for g in dec._graphs.values()] == fused
     # every kernel node of every recorded step within the limits the runtime reports for its function (host-side walk)
     for g in dec._graphs.values():
         assert ex.L.nd4jhipGraphAudit(g) == 0, ex.L.lastErrorMessage()

@@ -57,6 +57,7 @@ def test_add_layer_norm_product_chain_on_few_rows(ex, dt, rows, k, n1, n2):
             N.check("nd4jhipGraphEndCapture")
             assert g
             fused = L.nd4jhipGraphFusedOps(g)
+            assert L.nd4jhipGraphFusedApplied(g) == fused      # no merged step fell back to separate launches
             assert L.nd4jhipGraphAudit(g) == 0, L.lastErrorMessage()
             outs = []
             try:

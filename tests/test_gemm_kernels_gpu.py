@@ -89,6 +89,10 @@ CASES = [
     (BFLOAT16, 512, 512, 512, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=8>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=8>", None),
     (HALF, 512, 768, 2048, "gemm_mfma16s<f16,64x64,akc=1,bkc=0,stages=8>", "gemm_mfma16s<f16,64x64,akc=1,bkc=1,stages=8>", None),
     (BFLOAT16, 256, 256, 4096, "gemm_mfma16<bf16,64x64,akc=1,bkc=0>+splitk_finish", "gemm_mfma16<bf16,64x64,akc=1,bkc=1>+splitk_finish", None),
+    # operands the vector loaders cannot take (row lengths that are not multiples of 8): the element-gathering tile kernel --
+    # a batched decode step's logits against the row-major [768, 50257] embedding, and a product with nothing aligned
+    (BFLOAT16, 32, 50257, 768, "gemm_mfma16u<bf16,32x128,arf=0,brf=1>", "gemm_mfma16p<bf16,32x128,akc=1,bkc=1>", None),
+    (HALF, 1000, 1003, 515, "gemm_mfma16u<f16,128x128,arf=0,brf=1>", "gemm_mfma16u<f16,128x128,arf=0,brf=0>", "gemm_mfma16u<f16,128x128,arf=1,brf=1>"),
     # fp32 ragged
     (FLOAT32, 1100, 900, 1000, "gemm_mfma32<f32,64x64,akc=1,bkc=0>", "gemm_mfma32<f32,64x64,akc=1,bkc=1>", None),
     (FLOAT32, 2100, 2052, 520, "gemm_mfma32<f32,128x128,akc=1,bkc=0>", "gemm_mfma32<f32,128x128,akc=1,bkc=1>", "gemm_mfma32<f32,128x128,akc=0,bkc=0>"),
