@@ -618,7 +618,7 @@ def main():
                                                      "first %d of 96 batch entries (dense flop count)" % nb, "numpy einsum / exp / matmul in fp32", fast_cores=os.cpu_count())
                 ops.append(line)
                 del Q, K_, V, O_
-            result["ops"] = ops
+        result["ops"] = ops
     if not args.skip_decode:
         print("[bench] decode leg", file=sys.stderr, flush=True)
         ops = result.setdefault("ops", [])

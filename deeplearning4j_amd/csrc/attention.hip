@@ -99,21 +99,6 @@ struct FusedArgs {
 };
 
 template <typename T> __device__ __forceinline__ float round_storage(float v) { return to_float(Conv<T>::from(v)); }
-// two floats -> one register of two storage values (first in the low half), with one packed conversion for bf16
-typedef __attribute__((ext_vector_type(2))) float f32x2a;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2a;
-// (by reference: the caller goes on with the registers that pass through the asm, so no copies are made for it)
-template <typename T> __device__ __forceinline__ unsigned pack_pair(float& a, float& b);
-template <> __device__ __forceinline__ unsigned pack_pair<bf16_t>(float& a, float& b) {
-  asm("" : "+v"(a), "+v"(b));   // keeps source modifiers out of the packed conversion (see Conv<bf16_t>::from)
-  const f32x2a v = {a, b};
-  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2a));
-}
-typedef __attribute__((ext_vector_type(2))) _Float16 f16x2a;
-template <> __device__ __forceinline__ unsigned pack_pair<f16_t>(float& a, float& b) {
-  const f32x2a v = {a, b};
-  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, f16x2a));   // one packed conversion, round to nearest even
-}
 // round two values through the storage type in place
 template <typename T> __device__ __forceinline__ void round_pair(float& a, float& b);
 template <> __device__ __forceinline__ void round_pair<bf16_t>(float& a, float& b) {

@@ -42,6 +42,22 @@ template <> struct Conv<f16_t> {
   static __device__ __forceinline__ f16_t from(float f) { f16_t r; r.bits = __half_as_ushort(__float2half_rn(f)); return r; }
 };
 
+// two floats -> one register of two storage values (first in the low half), with one packed conversion for bf16
+typedef __attribute__((ext_vector_type(2))) float f32x2a;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2a;
+// (by reference: the caller goes on with the registers that pass through the asm, so no copies are made for it)
+template <typename T> __device__ __forceinline__ unsigned pack_pair(float& a, float& b);
+template <> __device__ __forceinline__ unsigned pack_pair<bf16_t>(float& a, float& b) {
+  asm("" : "+v"(a), "+v"(b));   // keeps source modifiers out of the packed conversion (see Conv<bf16_t>::from)
+  const f32x2a v = {a, b};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2a));
+}
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2a;
+template <> __device__ __forceinline__ unsigned pack_pair<f16_t>(float& a, float& b) {
+  const f32x2a v = {a, b};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, f16x2a));   // one packed conversion, round to nearest even
+}
+
 // 16-byte (or narrower) vector of storage elements
 template <typename T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };
 
@@ -80,8 +96,8 @@ template <> struct RawIO<bf16_t> {
     raw r;
 #pragma unroll
     for (int p = 0; p < 4; p++) {
-      const unsigned lo = Conv<bf16_t>::from(in[2 * p]).bits, hi = Conv<bf16_t>::from(in[2 * p + 1]).bits;
-      r[p] = lo | (hi << 16);
+      float lo = in[2 * p], hi = in[2 * p + 1];
+      r[p] = pack_pair<bf16_t>(lo, hi);
     }
     return r;
   }
@@ -99,6 +115,7 @@ template <> struct RawIO<f16_t> {
   static __device__ __forceinline__ raw pack(const float* in) {
     raw r;
 #pragma unroll
+    // (one conversion per value: the packed fp16 conversion does not give the same bits for every input)
     for (int p = 0; p < 4; p++) {
       const unsigned lo = Conv<f16_t>::from(in[2 * p]).bits, hi = Conv<f16_t>::from(in[2 * p + 1]).bits;
       r[p] = lo | (hi << 16);
@@ -130,7 +147,11 @@ template <typename T> struct RawIO12 {
   static __device__ __forceinline__ raw pack(const float* in) {
     raw r;
 #pragma unroll
-    for (int p = 0; p < 3; p++) r[p] = (unsigned)Conv<T>::from(in[2 * p]).bits | ((unsigned)Conv<T>::from(in[2 * p + 1]).bits << 16);
+    for (int p = 0; p < 3; p++) {
+      float lo = in[2 * p], hi = in[2 * p + 1];
+      if constexpr (sizeof(typename Conv<T>::acc) == 4 && __is_same(T, bf16_t)) r[p] = pack_pair<bf16_t>(lo, hi);
+      else r[p] = (unsigned)Conv<T>::from(lo).bits | ((unsigned)Conv<T>::from(hi).bits << 16);
+    }
     return r;
   }
 };
