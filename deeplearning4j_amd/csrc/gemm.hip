@@ -2177,9 +2177,9 @@ __global__ __launch_bounds__(256) void gemm_skinny32(GemmArgs g, const T* __rest
   if constexpr (LN_NV > 0) {
     using IO = RawIO<T>;
     using Raw = typename IO::raw;
-    const T* gp = reinterpret_cast<const T*>(g.lnGain) + lkg * 8;
-    const T* bp = reinterpret_cast<const T*>(g.lnBias) + lkg * 8;
-    u32x4 gr[2 * CT], br[2 * CT];
+    // gain and bias go through LDS (a stage of their own behind the chunk stages): 2 x K / 8 vector loads per block instead
+    // of 24 per thread, and no registers held for them while the row is normalised
+    u32x4* sGB = sW + 2 * CT * 8 * GROUP;                  // [2][128] vectors: gain, then bias
     // loads come back in the order they were issued: the rows (written by the kernel before this one, so close by), gain
     // and bias go first and the weights, which come from far away, last -- the normalisation then runs while they travel
 #pragma unroll
@@ -2187,11 +2187,10 @@ __global__ __launch_bounds__(256) void gemm_skinny32(GemmArgs g, const T* __rest
       const int jc = j < tiles ? j : tiles - 1;
       xr[j / CT][j % CT] = *reinterpret_cast<const u32x4*>(xp + (LongType)jc * 64);
     }
-#pragma unroll
-    for (int j = 0; j < 2 * CT; j++) {
-      const int jc = j < tiles ? j : tiles - 1;
-      gr[j] = *reinterpret_cast<const u32x4*>(gp + jc * 64);
-      br[j] = *reinterpret_cast<const u32x4*>(bp + jc * 64);
+    {
+      const int v = t & 127, vc = v < tiles * 8 ? v : tiles * 8 - 1;
+      const T* src = reinterpret_cast<const T*>(t < 128 ? g.lnGain : g.lnBias) + vc * 8;
+      sGB[t] = *reinterpret_cast<const u32x4*>(src);
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -2222,44 +2221,42 @@ __global__ __launch_bounds__(256) void gemm_skinny32(GemmArgs g, const T* __rest
       }
       return ((o[0] + o[1]) + (o[2] + o[3])) + ((o[4] + o[5]) + (o[6] + o[7]));
     };
-    float part[2 * CT];
+    // the row in fp32, kept in registers through the three passes
+    float part[2 * CT], vals[2 * CT][8];
 #pragma unroll
     for (int j = 0; j < 2 * CT; j++) {
-      float v[8];
-      IO::unpack(__builtin_bit_cast(Raw, xr[j / CT][j % CT]), v);
+      IO::unpack(__builtin_bit_cast(Raw, xr[j / CT][j % CT]), vals[j]);
       float p = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; e++) p += v[e];
+      for (int e = 0; e < 8; e++) p += vals[j][e];
       part[j] = p;
     }
     const float mean = rowTotal(part) / (float)(int)g.K;
 #pragma unroll
     for (int j = 0; j < 2 * CT; j++) {
-      float v[8];
-      IO::unpack(__builtin_bit_cast(Raw, xr[j / CT][j % CT]), v);
       float p = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; e++) { const float d = v[e] - mean; p += d * d; }
+      for (int e = 0; e < 8; e++) { const float d = vals[j][e] - mean; vals[j][e] = d; p += d * d; }
       part[j] = p;
     }
     const float var = rowTotal(part) / (float)(int)g.K;
     const float rstd = 1.f / sqrtf(var + g.lnEps);
     const bool writer = blockIdx.x == 0 && lrow < g.M;
     T* lo = reinterpret_cast<T*>(g.lnOut) + (LongType)lrow * g.lnOutRow + lkg * 8;
+    __syncthreads();                                       // gain and bias are in LDS
 #pragma unroll
     for (int j = 0; j < 2 * CT; j++) {
-      float v[8], gn[8], bs[8];
-      IO::unpack(__builtin_bit_cast(Raw, xr[j / CT][j % CT]), v);
-      IO::unpack(__builtin_bit_cast(Raw, gr[j]), gn);
-      IO::unpack(__builtin_bit_cast(Raw, br[j]), bs);
+      float gn[8], bs[8];
+      const int vj = j < tiles ? j * 8 + lkg : 0;
+      IO::unpack(__builtin_bit_cast(Raw, sGB[vj]), gn);
+      IO::unpack(__builtin_bit_cast(Raw, sGB[128 + vj]), bs);
 #pragma unroll
       for (int e = 0; e < 8; e++) {
-        const float d = v[e] - mean;
-        float y = d * rstd * gn[e];
+        float y = vals[j][e] * rstd * gn[e];
         y += bs[e];
-        v[e] = y;
+        vals[j][e] = y;
       }
-      const Raw packed = IO::pack(v);
+      const Raw packed = IO::pack(vals[j]);
       xr[j / CT][j % CT] = __builtin_bit_cast(u32x4, packed);
       if (writer && j < tiles) *reinterpret_cast<Raw*>(lo + j * 64) = packed;
     }
@@ -2322,8 +2319,10 @@ static bool tryGemmSkinny(hipStream_t s, const GemmDesc& d, const void* A, const
     if (!d.lnBias || !d.lnOut || d.K < 320 || d.K > 768 || d.lnOutRow % 8 != 0) return false;
     if ((reinterpret_cast<uintptr_t>(d.lnGain) | reinterpret_cast<uintptr_t>(d.lnBias) | reinterpret_cast<uintptr_t>(d.lnOut)) & 15) return false;
     noteKernel("gemm_skinny32<%s,ln>", tname<T>());
-    if (d.K <= 512) hipLaunchKernelGGL((gemm_skinny32<T, 1>), dim3((unsigned)(d.N / 32)), dim3(256), LDS, s, g, (const T*)A, (const T*)B, (T*)C);
-    else hipLaunchKernelGGL((gemm_skinny32<T, 2>), dim3((unsigned)(d.N / 32)), dim3(256), LDS, s, g, (const T*)A, (const T*)B, (T*)C);
+    constexpr size_t LDS_LN = LDS + 2 * 128 * 16;          // + gain and bias
+    static_assert(LDS_LN <= 64 * 1024, "gemm_skinny32 must fit the default dynamic LDS limit");
+    if (d.K <= 512) hipLaunchKernelGGL((gemm_skinny32<T, 1>), dim3((unsigned)(d.N / 32)), dim3(256), LDS_LN, s, g, (const T*)A, (const T*)B, (T*)C);
+    else hipLaunchKernelGGL((gemm_skinny32<T, 2>), dim3((unsigned)(d.N / 32)), dim3(256), LDS_LN, s, g, (const T*)A, (const T*)B, (T*)C);
     return true;
   }
   noteKernel("gemm_skinny32<%s>", tname<T>());
