@@ -1323,7 +1323,7 @@ static int chooseSplits(const GemmArgs& g, LongType batch, LongType& ktPerSplit)
 }
 
 template <typename T, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC>
-static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void* B, void* C, LongType batch, bool allowSplit = false) {
+static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void* B, void* C, LongType batch, bool allowSplit, bool aligned) {
   constexpr int NT = WM * WN * 64;
   constexpr size_t LDS = (size_t)2 * (TileLayout<BM, A_KC>::SLOTS + TileLayout<BN, B_KC>::SLOTS) * 16;
   int splits = 1;
@@ -1352,11 +1352,11 @@ static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
   if (g.hasEpi && (splits == 1 || batch != 1 || g.cCol != 1)) return false;
   const bool usePipe = splits == 1;   // the split-K epilogue lives in the plain kernel
   // whole tiles only: the kernel without bounds handling (its K loop needs two K-tiles at least)
-  const bool useFull = usePipe && BM * BN >= 128 * 128 && g.M % BM == 0 && g.N % BN == 0 && g.K % 64 == 0 && g.K >= 128;
+  const bool useFull = aligned && usePipe && BM * BN >= 128 * 128 && g.M % BM == 0 && g.N % BN == 0 && g.K % 64 == 0 && g.K >= 128;
   // small tiles, at most a couple per CU and a long K: the loop is bound by one memory latency per K-tile unless several
   // K-tiles are in flight
   const unsigned nTiles = (unsigned)(((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN) * batch);
-  const bool useDeep = usePipe && !useFull && BM * BN <= 64 * 64 && nTiles <= 1024 && g.K >= 512 && g.M % BM == 0 && g.N % BN == 0 && g.K % 256 == 0;
+  const bool useDeep = aligned && usePipe && !useFull && BM * BN <= 64 * 64 && nTiles <= 1024 && g.K >= 512 && g.M % BM == 0 && g.N % BN == 0 && g.K % 256 == 0;
   // the direct-load ring takes the small-tile launches it can: 64 x 64 or 128 x 128 tiles, A k-contiguous, 16-byte aligned rows
   if constexpr ((BM == 64 && BN == 64 || BM == 128 && BN == 128) && WM == 2 && WN == 2 && A_KC) {
     constexpr int TW = BM / 64;
@@ -1405,13 +1405,14 @@ static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
 }
 
 template <typename T, bool A_KC, bool B_KC>
-static bool launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C, LongType batch) {
+static bool launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C, LongType batch, bool aligned) {
   const LongType tiles256 = ((g.M + 255) / 256) * ((g.N + 255) / 256) * batch;
   const LongType tiles128 = ((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
-  if (g.M <= 32) return launchMfma16Cfg<T, 32, 128, 1, 4, A_KC, B_KC>(s, g, A, B, C, batch, true);
-  if (g.M <= 64 || g.N <= 64 || tiles128 < 192) return launchMfma16Cfg<T, 64, 64, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch, true);
-  if (tiles256 < 192) return launchMfma16Cfg<T, 128, 128, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
+  if (g.M <= 32) return launchMfma16Cfg<T, 32, 128, 1, 4, A_KC, B_KC>(s, g, A, B, C, batch, true, aligned);
+  if (g.M <= 64 || g.N <= 64 || tiles128 < 192) return launchMfma16Cfg<T, 64, 64, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch, true, aligned);
+  if (tiles256 < 192) return launchMfma16Cfg<T, 128, 128, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch, false, aligned);
   if (g.hasEpi) return false;
+  if (!aligned) return launchMfma16Cfg<T, 256, 256, 2, 4, A_KC, B_KC>(s, g, A, B, C, batch, false, false);
   static const bool direct = getenv("ND4JHIP_GEMM_DIRECT") ? atoi(getenv("ND4JHIP_GEMM_DIRECT")) != 0 : true;
   static const bool ring = getenv("ND4JHIP_GEMM_RING") ? atoi(getenv("ND4JHIP_GEMM_RING")) != 0 : true;
   if constexpr (A_KC && !B_KC) {
@@ -1435,7 +1436,7 @@ static bool launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const 
     hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(512), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
     return true;
   }
-  return launchMfma16Cfg<T, 256, 256, 2, 4, A_KC, B_KC>(s, g, A, B, C, batch);
+  return launchMfma16Cfg<T, 256, 256, 2, 4, A_KC, B_KC>(s, g, A, B, C, batch, false, true);
 }
 
 // ---- fp32 MFMA kernel ------------------------------------------------------------------------------------------------
@@ -1986,20 +1987,25 @@ static void launchSimple(hipStream_t s, const void* A, const void* B, void* C, c
 }
 
 // can the MFMA kernels take this problem: 16-byte aligned vectors along each operand's contiguous axis
-static bool mfmaEligible(const GemmDesc& d, const void* A, const void* B, size_t es, bool& aKC, bool& bKC) {
+// `aligned`: every operand vector the loaders fetch starts on a 16-byte boundary and the contiguous extents are whole vectors --
+// what the direct-to-LDS kernels and the kernels without bounds handling need.  Without it only the 16-bit kernels whose loader
+// takes element-aligned rows and ragged extents (gemm_mfma16p, gemm_mfma16) may run.
+static bool mfmaEligible(const GemmDesc& d, const void* A, const void* B, size_t es, bool& aKC, bool& bKC, bool& aligned) {
   const LongType V = 16 / (LongType)es;
-  if (d.M < 1 || d.N < 1 || d.K < 1) return false;
-  if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) return false;
-  if (d.batch > 1 && (d.aBatch % V || d.bBatch % V)) return false;
-  if (d.batchInner > 0 && (d.aBatch2 % V || d.bBatch2 % V)) return false;
-  if (d.aCol == 1 && d.K % V == 0 && d.aRow % V == 0) aKC = true;
-  else if (d.aRow == 1 && d.M % V == 0 && d.M >= V && d.aCol % V == 0) aKC = false;
-  else return false;
-  if (d.bRow == 1 && d.K % V == 0 && d.bCol % V == 0) bKC = true;
-  else if (d.bCol == 1 && d.N % V == 0 && d.N >= V && d.bRow % V == 0) bKC = false;
-  else return false;
+  if (d.M < 1 || d.N < 1 || d.K < V) return false;
   if (d.aRow < 0 || d.aCol < 0 || d.bRow < 0 || d.bCol < 0) return false;
-  return true;
+  if (d.aCol == 1) aKC = true;
+  else if (d.aRow == 1 && d.M >= V) aKC = false;
+  else return false;
+  if (d.bRow == 1) bKC = true;
+  else if (d.bCol == 1 && d.N >= V) bKC = false;
+  else return false;
+  aligned = ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0;
+  if (d.batch > 1 && (d.aBatch % V || d.bBatch % V)) aligned = false;
+  if (d.batchInner > 0 && (d.aBatch2 % V || d.bBatch2 % V)) aligned = false;
+  if (aKC ? (d.K % V != 0 || d.aRow % V != 0) : (d.M % V != 0 || d.aCol % V != 0)) aligned = false;
+  if (bKC ? (d.K % V != 0 || d.bCol % V != 0) : (d.N % V != 0 || d.bRow % V != 0)) aligned = false;
+  return aligned || es == 2;
 }
 
 // ---- up to four rows of x against row-major W (a decode step's projections) --------------------------------------------------
@@ -2362,8 +2368,8 @@ static bool dispatch16(hipStream_t s, const GemmDesc& d, const void* A, const vo
     if (d.M >= 5 && d.M <= 32) return tryGemmSkinny<T>(s, d, A, B, C);
     return false;
   }
-  bool aKC = false, bKC = false;
-  const bool eligible = (d.M * d.N >= 1024 || (d.M == 1 && d.N >= 64)) && d.K >= 32 && mfmaEligible(d, A, B, sizeof(T), aKC, bKC);
+  bool aKC = false, bKC = false, aligned = false;
+  const bool eligible = (d.M * d.N >= 1024 || (d.M == 1 && d.N >= 64)) && d.K >= 32 && mfmaEligible(d, A, B, sizeof(T), aKC, bKC, aligned);
   // x[1, K] times row-major W[K, N]: the split-K tile kernel streams W with far more loads in flight than the
   // column-sum GEMV (the unused 31 rows of the MFMA tile cost nothing here)
   if (tryGemvStrip<T>(s, d, A, B, C)) return true;
@@ -2372,10 +2378,10 @@ static bool dispatch16(hipStream_t s, const GemmDesc& d, const void* A, const vo
   if (!rowTimesRowMajor && tryGemv<T>(s, d, A, B, C)) return true;
   if (eligible) {
     GemmArgs g = toArgs(d);
-    if (aKC && bKC) return launchMfma16<T, true, true>(s, g, A, B, C, d.batch);
-    if (aKC && !bKC) return launchMfma16<T, true, false>(s, g, A, B, C, d.batch);
-    if (!aKC && bKC) return launchMfma16<T, false, true>(s, g, A, B, C, d.batch);
-    return launchMfma16<T, false, false>(s, g, A, B, C, d.batch);
+    if (aKC && bKC) return launchMfma16<T, true, true>(s, g, A, B, C, d.batch, aligned);
+    if (aKC && !bKC) return launchMfma16<T, true, false>(s, g, A, B, C, d.batch, aligned);
+    if (!aKC && bKC) return launchMfma16<T, false, true>(s, g, A, B, C, d.batch, aligned);
+    return launchMfma16<T, false, false>(s, g, A, B, C, d.batch, aligned);
   }
   if (d.epi) return false;
   if (launchMfma16u<T>(s, d, A, B, C)) return true;
@@ -2384,8 +2390,8 @@ static bool dispatch16(hipStream_t s, const GemmDesc& d, const void* A, const vo
 }
 static void dispatch32(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
   if (tryGemv<float>(s, d, A, B, C)) return;
-  bool aKC = false, bKC = false;
-  if (d.M * d.N >= 1024 && d.K >= 16 && mfmaEligible(d, A, B, 4, aKC, bKC)) {
+  bool aKC = false, bKC = false, aligned = false;
+  if (d.M * d.N >= 1024 && d.K >= 16 && mfmaEligible(d, A, B, 4, aKC, bKC, aligned)) {
     GemmArgs g = toArgs(d);
     if (aKC && bKC) return launchMfma32<true, true>(s, g, A, B, C, d.batch);
     if (aKC && !bKC) return launchMfma32<true, false>(s, g, A, B, C, d.batch);

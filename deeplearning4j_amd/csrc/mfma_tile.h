@@ -51,6 +51,28 @@ struct TileLayout {
   }
 };
 
+// 16 bytes from an address that is only element-aligned (one global_load_dwordx4: the platform runs global memory in
+// unaligned access mode and the compiler emits the wide load itself for such a copy)
+__device__ __forceinline__ u32x4 load16u(const void* p) {
+  u32x4 v;
+  __builtin_memcpy(&v, p, 16);
+  return v;
+}
+// the eight 16-bit elements of v moved down by sh places: element j + sh lands in place j, zeros come in from the top
+// (sh >= 8: all zeros).  Selects only, no indexed register access.
+__device__ __forceinline__ u32x4 shiftDownElems(u32x4 v, int sh) {
+  const int ds = sh >> 1;
+  const bool odd = (sh & 1) != 0;
+  auto pick = [&](int idx) -> unsigned { return idx == 0 ? v[0] : idx == 1 ? v[1] : idx == 2 ? v[2] : idx == 3 ? v[3] : 0u; };
+  u32x4 o;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const unsigned lo = pick(ds + i), hi = pick(ds + i + 1);
+    o[i] = odd ? (lo >> 16) | (hi << 16) : lo;
+  }
+  return o;
+}
+
 template <int ROWS, int NT, bool KC>
 struct TileLoader {
   using Layout = TileLayout<ROWS, KC>;
@@ -59,6 +81,12 @@ struct TileLoader {
   static constexpr int NREG = KC ? PER : PER * 4;
   u32x4 reg[NREG];
 
+  // The loader of the kernels that handle ragged shapes.  Rows need element alignment only (any row pitch, any start), and the
+  // contiguous extent need not be a multiple of 8: every load is an unconditional 16-byte read from a position inside the
+  // operand -- a group that would run over the end of its row (k-contiguous operand: k + 8 > K; row-contiguous operand: the
+  // last rows) is read 8 elements back from the end instead and moved down in registers, zeros coming in for what lies
+  // beyond; k positions past K give zeros (they meet the other operand's tail); rows past the limit of a k-contiguous
+  // operand repeat the last row (their products are never stored).  Needs K >= 8 (k-contiguous) or rowLimit >= 8.
   template <typename T>
   __device__ __forceinline__ void load(const T* __restrict__ base, LongType ld, LongType row0, LongType rowLimit, LongType k0, LongType K, int t) {
     const u32x4 zero = {0u, 0u, 0u, 0u};
@@ -71,15 +99,23 @@ struct TileLoader {
         LongType r = row0 + row;
         r = r < rowLimit ? r : rowLimit - 1;
         const LongType k = k0 + kg * 8;
-        reg[i] = k < K ? *reinterpret_cast<const u32x4*>(base + r * ld + k) : zero;
+        const LongType kk = k + 8 <= K ? k : K - 8;
+        reg[i] = load16u(base + r * ld + kk);
+        if (k != kk) reg[i] = shiftDownElems(reg[i], (int)(k - kk < 8 ? k - kk : 8));
       } else {
         const int rb = (u >> 1) % (ROWS / 8), kq = (u / (ROWS / 4)) * 2 + (u & 1);   // 8-row block, 4-k quad (16 per tile)
-        LongType r = row0 + rb * 8;
-        r = r + 8 <= rowLimit ? r : rowLimit - 8;
+        const LongType r = row0 + rb * 8;
+        const LongType rr = r + 8 <= rowLimit ? r : rowLimit - 8;
+        const int sh = (int)(r - rr < 8 ? r - rr : 8);
 #pragma unroll
         for (int q = 0; q < 4; q++) {
           const LongType k = k0 + kq * 4 + q;
-          reg[i * 4 + q] = k < K ? *reinterpret_cast<const u32x4*>(base + k * ld + r) : zero;
+          reg[i * 4 + q] = load16u(base + (k < K ? k : K - 1) * ld + rr);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          if (k0 + kq * 4 + q >= K) reg[i * 4 + q] = zero;
+          else if (sh) reg[i * 4 + q] = shiftDownElems(reg[i * 4 + q], sh);
         }
       }
     }

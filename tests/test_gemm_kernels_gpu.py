@@ -89,10 +89,14 @@ CASES = [
     (BFLOAT16, 512, 512, 512, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=8>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=8>", None),
     (HALF, 512, 768, 2048, "gemm_mfma16s<f16,64x64,akc=1,bkc=0,stages=8>", "gemm_mfma16s<f16,64x64,akc=1,bkc=1,stages=8>", None),
     (BFLOAT16, 256, 256, 4096, "gemm_mfma16<bf16,64x64,akc=1,bkc=0>+splitk_finish", "gemm_mfma16<bf16,64x64,akc=1,bkc=1>+splitk_finish", None),
-    # operands the vector loaders cannot take (row lengths that are not multiples of 8): the element-gathering tile kernel --
-    # a batched decode step's logits against the row-major [768, 50257] embedding, and a product with nothing aligned
-    (BFLOAT16, 32, 50257, 768, "gemm_mfma16u<bf16,32x128,arf=0,brf=1>", "gemm_mfma16p<bf16,32x128,akc=1,bkc=1>", None),
-    (HALF, 1000, 1003, 515, "gemm_mfma16u<f16,128x128,arf=0,brf=1>", "gemm_mfma16u<f16,128x128,arf=0,brf=0>", "gemm_mfma16u<f16,128x128,arf=1,brf=1>"),
+    # row lengths that are not multiples of 8 (rows start off 16-byte boundaries, the last vector of a row is partial): the
+    # bounds-handling kernels read element-aligned vectors -- a batched decode step's logits against the row-major
+    # [768, 50257] embedding, a prefill's, and a product with nothing aligned in any layout
+    (BFLOAT16, 32, 50257, 768, "gemm_mfma16p<bf16,32x128,akc=1,bkc=0>", "gemm_mfma16p<bf16,32x128,akc=1,bkc=1>", None),
+    (BFLOAT16, 1024, 50257, 768, "gemm_mfma16p<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16p<bf16,256x256,akc=1,bkc=1>", None),
+    (HALF, 1000, 1003, 515, "gemm_mfma16p<f16,64x64,akc=1,bkc=0>", "gemm_mfma16p<f16,64x64,akc=1,bkc=1>", "gemm_mfma16p<f16,64x64,akc=0,bkc=0>"),
+    (BFLOAT16, 2001, 1999, 1003, "gemm_mfma16p<bf16,128x128,akc=1,bkc=0>", "gemm_mfma16p<bf16,128x128,akc=1,bkc=1>", "gemm_mfma16p<bf16,128x128,akc=0,bkc=0>"),
+    (HALF, 20, 4097, 2051, "gemm_mfma16<f16,32x128,akc=1,bkc=0>+splitk_finish", "gemm_mfma16<f16,32x128,akc=1,bkc=1>+splitk_finish", None),
     # fp32 ragged
     (FLOAT32, 1100, 900, 1000, "gemm_mfma32<f32,64x64,akc=1,bkc=0>", "gemm_mfma32<f32,64x64,akc=1,bkc=1>", None),
     (FLOAT32, 2100, 2052, 520, "gemm_mfma32<f32,128x128,akc=1,bkc=0>", "gemm_mfma32<f32,128x128,akc=1,bkc=1>", "gemm_mfma32<f32,128x128,akc=0,bkc=0>"),
@@ -227,3 +231,25 @@ np.savez(sys.argv[1], names=np.array(names), **out)
     for key in one.files:
         if key != "names":
             assert np.array_equal(one[key], two[key]), key
+
+
+@pytest.mark.parametrize("dtype", [HALF, BFLOAT16])
+def test_matmul_on_views_without_a_unit_stride(ex, dtype):
+    """Operands whose elements are two apart along both axes (every second row and column of a larger array) and a
+    result written into such a view: no vector loader takes them, the element-gathering tile kernel does."""
+    rng = np.random.default_rng(99 + dtype)
+    M, N, K = 300, 260, 200
+    a = rng.normal(0, 1 / math.sqrt(K), (2 * M, 2 * K)).astype(np.float32)
+    b = rng.normal(0, 1 / math.sqrt(K), (2 * K, 2 * N)).astype(np.float32)
+    A, a64 = _device(a, dtype)
+    B, b64 = _device(b, dtype)
+    Av = A.view((M, K), (4 * K, 2))
+    Bv = B.view((K, N), (4 * N, 2))
+    z = ex.exec_custom("matmul", [Av, Bv])[0]
+    assert _last_kernel(ex).startswith("gemm_mfma16u<%s,128x128,arf=0,brf=1>" % ("f16" if dtype == HALF else "bf16")), _last_kernel(ex)
+    assert_close(z.to_float(), a64[::2, ::2] @ b64[::2, ::2], TOL[dtype], TOL[dtype], "every second row and column")
+    # transposed views of the same operands: the smaller stride now runs along the rows of A and along k of B
+    At, Bt = Av.permute(1, 0), Bv.permute(1, 0)
+    zt = ex.exec_custom("matmul", [At, Bt], i_args=[1, 1])[0]
+    assert _last_kernel(ex).startswith("gemm_mfma16u<"), _last_kernel(ex)
+    assert_close(zt.to_float(), a64[::2, ::2] @ b64[::2, ::2], TOL[dtype], TOL[dtype], "transposed views, both flags")
