@@ -1467,39 +1467,47 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32(GemmArgs g, const fl
   f32x4 ra[VA], rb[VB];
   const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
 
-  auto loadA = [&](LongType k0) {
+  // Rows need element alignment only and the contiguous extent need not be a multiple of 4: every load is an unconditional
+  // 16-byte read from a position inside the operand (a group that would run over the end of its row is read 4 elements back
+  // from the end and moved down in registers, zeros coming in; k positions past K give zeros; rows past the limit of a
+  // k-contiguous operand repeat the last row).  Needs K >= 4 (k-contiguous) or 4 rows (row-contiguous).
+  auto vec4 = [&](const float* p) { f32x4 v; __builtin_memcpy(&v, p, 16); return v; };
+  auto down = [&](f32x4 v, int sh) {
+    f32x4 o;
 #pragma unroll
-    for (int i = 0; i < VA; i++) {
+    for (int j = 0; j < 4; j++) {
+      const int i = j + sh;
+      o[j] = i == 0 ? v[0] : i == 1 ? v[1] : i == 2 ? v[2] : i == 3 ? v[3] : 0.f;
+    }
+    return o;
+  };
+  auto loadTile = [&](auto& reg, auto nv, auto kc, auto rows, const float* base, LongType ld, LongType row0, LongType limit, LongType k0) {
+    constexpr int NV = decltype(nv)::value, ROWS = decltype(rows)::value;
+    constexpr bool KC = decltype(kc)::value;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
       const int v = t + i * NT;
-      if (A_KC) {
+      if (KC) {
         const int kq = v & 3, row = v >> 2;
-        LongType r = m0 + row; r = r < g.M ? r : g.M - 1;
-        const LongType k = k0 + kq * 4;
-        ra[i] = k < g.K ? *reinterpret_cast<const f32x4*>(A + r * lda + k) : zero;
+        LongType r = row0 + row; r = r < limit ? r : limit - 1;
+        const LongType k = k0 + kq * 4, kk = k + 4 <= g.K ? k : g.K - 4;
+        reg[i] = vec4(base + r * ld + kk);
+        if (k != kk) reg[i] = down(reg[i], (int)(k - kk < 4 ? k - kk : 4));
       } else {
-        const int rq = v % (BM / 4), kk = v / (BM / 4);
-        LongType r = m0 + rq * 4; r = r + 4 <= g.M ? r : g.M - 4;
+        const int rq = v % (ROWS / 4), kk = v / (ROWS / 4);
+        const LongType r = row0 + rq * 4, rr = r + 4 <= limit ? r : limit - 4;
         const LongType k = k0 + kk;
-        ra[i] = k < g.K ? *reinterpret_cast<const f32x4*>(A + k * lda + r) : zero;
+        reg[i] = vec4(base + (k < g.K ? k : g.K - 1) * ld + rr);
+        if (k >= g.K) reg[i] = zero;
+        else if (r != rr) reg[i] = down(reg[i], (int)(r - rr < 4 ? r - rr : 4));
       }
     }
   };
+  auto loadA = [&](LongType k0) {
+    loadTile(ra, std::integral_constant<int, VA>(), std::integral_constant<bool, A_KC>(), std::integral_constant<int, BM>(), A, lda, m0, g.M, k0);
+  };
   auto loadB = [&](LongType k0) {
-#pragma unroll
-    for (int i = 0; i < VB; i++) {
-      const int v = t + i * NT;
-      if (B_KC) {
-        const int kq = v & 3, row = v >> 2;
-        LongType r = n0 + row; r = r < g.N ? r : g.N - 1;
-        const LongType k = k0 + kq * 4;
-        rb[i] = k < g.K ? *reinterpret_cast<const f32x4*>(B + r * ldb + k) : zero;
-      } else {
-        const int rq = v % (BN / 4), kk = v / (BN / 4);
-        LongType r = n0 + rq * 4; r = r + 4 <= g.N ? r : g.N - 4;
-        const LongType k = k0 + kk;
-        rb[i] = k < g.K ? *reinterpret_cast<const f32x4*>(B + k * ldb + r) : zero;
-      }
-    }
+    loadTile(rb, std::integral_constant<int, VB>(), std::integral_constant<bool, B_KC>(), std::integral_constant<int, BN>(), B, ldb, n0, g.N, k0);
   };
   auto storeA = [&](int stage) {
 #pragma unroll
@@ -1735,9 +1743,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32q(GemmArgs g, const f
 }
 
 template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC>
-static void launchMfma32Cfg(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C, LongType batch) {
+static void launchMfma32Cfg(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C, LongType batch, bool aligned) {
   const unsigned tilesM = (unsigned)((g.M + BM - 1) / BM), tilesN = (unsigned)((g.N + BN - 1) / BN);
-  if (g.K >= 256 && g.M % BM == 0 && g.N % BN == 0 && g.K % 128 == 0) {
+  if (aligned && g.K >= 256 && g.M % BM == 0 && g.N % BN == 0 && g.K % 128 == 0) {
     constexpr int PD = 4, BK = BM * BN <= 64 * 64 ? 32 : 16;
     noteKernel("gemm_mfma32q<f32,%dx%d,akc=%d,bkc=%d,pd=%d,bk=%d>", BM, BN, (int)A_KC, (int)B_KC, PD, BK);
     hipLaunchKernelGGL((gemm_mfma32q<BM, BN, WM, WN, A_KC, B_KC, PD, BK>), dim3(tilesM * tilesN, 1, (unsigned)batch), dim3(WM * WN * 64), 0, s, g,
@@ -1749,10 +1757,10 @@ static void launchMfma32Cfg(hipStream_t s, const GemmArgs& g, const void* A, con
                      (const float*)A, (const float*)B, (float*)C, tilesM, tilesN);
 }
 template <bool A_KC, bool B_KC>
-static void launchMfma32(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C, LongType batch) {
+static void launchMfma32(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C, LongType batch, bool aligned) {
   const LongType tiles128 = ((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
-  if (g.M <= 64 || g.N <= 64 || tiles128 < 192) return launchMfma32Cfg<64, 64, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
-  return launchMfma32Cfg<128, 128, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch);
+  if (g.M <= 64 || g.N <= 64 || tiles128 < 192) return launchMfma32Cfg<64, 64, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch, aligned);
+  return launchMfma32Cfg<128, 128, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch, aligned);
 }
 
 // ---- GEMV: one skinny operand, the matrix is streamed once ----------------------------------------------------------
@@ -1988,8 +1996,8 @@ static void launchSimple(hipStream_t s, const void* A, const void* B, void* C, c
 
 // can the MFMA kernels take this problem: 16-byte aligned vectors along each operand's contiguous axis
 // `aligned`: every operand vector the loaders fetch starts on a 16-byte boundary and the contiguous extents are whole vectors --
-// what the direct-to-LDS kernels and the kernels without bounds handling need.  Without it only the 16-bit kernels whose loader
-// takes element-aligned rows and ragged extents (gemm_mfma16p, gemm_mfma16) may run.
+// what the direct-to-LDS kernels and the kernels without bounds handling need.  Without it only the kernels whose loader
+// takes element-aligned rows and ragged extents (gemm_mfma16p, gemm_mfma16, gemm_mfma32) may run.
 static bool mfmaEligible(const GemmDesc& d, const void* A, const void* B, size_t es, bool& aKC, bool& bKC, bool& aligned) {
   const LongType V = 16 / (LongType)es;
   if (d.M < 1 || d.N < 1 || d.K < V) return false;
@@ -2005,7 +2013,7 @@ static bool mfmaEligible(const GemmDesc& d, const void* A, const void* B, size_t
   if (d.batchInner > 0 && (d.aBatch2 % V || d.bBatch2 % V)) aligned = false;
   if (aKC ? (d.K % V != 0 || d.aRow % V != 0) : (d.M % V != 0 || d.aCol % V != 0)) aligned = false;
   if (bKC ? (d.K % V != 0 || d.bCol % V != 0) : (d.N % V != 0 || d.bRow % V != 0)) aligned = false;
-  return aligned || es == 2;
+  return true;
 }
 
 // ---- up to four rows of x against row-major W (a decode step's projections) --------------------------------------------------
@@ -2393,10 +2401,10 @@ static void dispatch32(hipStream_t s, const GemmDesc& d, const void* A, const vo
   bool aKC = false, bKC = false, aligned = false;
   if (d.M * d.N >= 1024 && d.K >= 16 && mfmaEligible(d, A, B, 4, aKC, bKC, aligned)) {
     GemmArgs g = toArgs(d);
-    if (aKC && bKC) return launchMfma32<true, true>(s, g, A, B, C, d.batch);
-    if (aKC && !bKC) return launchMfma32<true, false>(s, g, A, B, C, d.batch);
-    if (!aKC && bKC) return launchMfma32<false, true>(s, g, A, B, C, d.batch);
-    return launchMfma32<false, false>(s, g, A, B, C, d.batch);
+    if (aKC && bKC) return launchMfma32<true, true>(s, g, A, B, C, d.batch, aligned);
+    if (aKC && !bKC) return launchMfma32<true, false>(s, g, A, B, C, d.batch, aligned);
+    if (!aKC && bKC) return launchMfma32<false, true>(s, g, A, B, C, d.batch, aligned);
+    return launchMfma32<false, false>(s, g, A, B, C, d.batch, aligned);
   }
   launchSimple<float>(s, A, B, C, d);
 }

@@ -97,6 +97,9 @@ CASES = [
     (HALF, 1000, 1003, 515, "gemm_mfma16p<f16,64x64,akc=1,bkc=0>", "gemm_mfma16p<f16,64x64,akc=1,bkc=1>", "gemm_mfma16p<f16,64x64,akc=0,bkc=0>"),
     (BFLOAT16, 2001, 1999, 1003, "gemm_mfma16p<bf16,128x128,akc=1,bkc=0>", "gemm_mfma16p<bf16,128x128,akc=1,bkc=1>", "gemm_mfma16p<bf16,128x128,akc=0,bkc=0>"),
     (HALF, 20, 4097, 2051, "gemm_mfma16<f16,32x128,akc=1,bkc=0>+splitk_finish", "gemm_mfma16<f16,32x128,akc=1,bkc=1>+splitk_finish", None),
+    # the same for fp32 (row lengths that are not multiples of 4)
+    (FLOAT32, 1000, 1003, 515, "gemm_mfma32<f32,64x64,akc=1,bkc=0>", "gemm_mfma32<f32,64x64,akc=1,bkc=1>", "gemm_mfma32<f32,64x64,akc=0,bkc=0>"),
+    (FLOAT32, 257, 50257, 770, "gemm_mfma32<f32,128x128,akc=1,bkc=0>", "gemm_mfma32<f32,128x128,akc=1,bkc=1>", None),
     # fp32 ragged
     (FLOAT32, 1100, 900, 1000, "gemm_mfma32<f32,64x64,akc=1,bkc=0>", "gemm_mfma32<f32,64x64,akc=1,bkc=1>", None),
     (FLOAT32, 2100, 2052, 520, "gemm_mfma32<f32,128x128,akc=1,bkc=0>", "gemm_mfma32<f32,128x128,akc=1,bkc=1>", "gemm_mfma32<f32,128x128,akc=0,bkc=0>"),
