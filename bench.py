@@ -526,6 +526,16 @@ def main():
             sm_binds = [ex.bind_custom("softmax", [Lv[i]], [Zl[i % 3]], i_args=[1]) for i in range(Kl)]
             hbm_line("softmax fp32 [500,50257] (vocabulary-length rows: softmax_long_vec)", "", 2 * 4 * lv.size, lambda i: sm_binds[i])
             del Lv, Zl, sm_binds, lv
+            # a product against a row-major matrix whose rows do not start on 16-byte boundaries (the [768, 50257] embedding
+            # without the transpose flag): element-aligned vector loads in the bounds-handling tile kernel
+            ue = rng.normal(0, 768 ** -0.5, (768, 50257)).astype(np.float32)
+            ua = rng.normal(0, 1, (4096, 768)).astype(np.float32)
+            Ua, Ue, Uz = NDArray.from_numpy(ua, BFLOAT16), NDArray.from_numpy(ue, BFLOAT16), NDArray.empty((4096, 50257), BFLOAT16)
+            Ua.sync_to_device(); Ue.sync_to_device()
+            w, e = timed(ex, L, ex.bind_custom("matmul", [Ua, Ue], [Uz]), max(steps // 5, 3), max(warmup // 5, 1))
+            ops.append({"op": "mmul bf16 [4096,768] x [768,50257] (row length not a multiple of 8: %s)" % L.nd4jhipLastGemmKernel().decode(),
+                        "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": mfma_entry(2.0 * 4096 * 50257 * 768, e, "bf16", "")})
+            del Ua, Ue, Uz, ua, ue
         if 2 in cfgs:
             # config 2, the remaining sizes/dtypes
             plain_cpu = {}     # (dtype, size) -> cpu_baseline of the plain-B product: the CPU loops do not depend on the layout flag

@@ -341,6 +341,86 @@ __global__ __launch_bounds__(1024) void softmax_long_vec(RowArgs a, const T* __r
   }
 }
 
+// Unit-stride rows of up to NV x 512 vectors (fp32 up to 65,536 values, 16-bit up to 131,072: a vocabulary's logits): one
+// block of 512 threads (two waves per SIMD: 256 registers each) holds the whole row in registers, so it comes from memory once and the three passes (maximum, sum of
+// exponentials, result) run on registers.  Rows may start anywhere: the 16-byte loads and stores are element-aligned (global
+// memory runs in unaligned access mode), the values after the last whole vector go one per thread.
+template <typename T, int NV, bool LOG>
+__global__ __launch_bounds__(512) void softmax_block_regs(RowArgs a, const T* __restrict__ x, T* __restrict__ z, int clamp) {
+  using A = typename Conv<T>::acc;
+  using Raw = typename RawIO<T>::raw;
+  constexpr int VEC = RawIO<T>::N, NT = 512;
+  __shared__ A lds[NT / 64];
+  const LongType row = blockIdx.x;
+  const T* xr = x + walk<LongType>(a.outerX, row);
+  T* zr = z + walk<LongType>(a.outerZ, row);
+  const LongType L = a.rowLen, nv = L / VEC, tail0 = nv * VEC;
+  const int t = threadIdx.x;
+  Raw v[NV];
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const LongType iv = (LongType)i * NT + t;
+    __builtin_memcpy(&v[i], xr + (iv < nv ? iv : nv - 1) * VEC, sizeof(Raw));
+  }
+  const bool hasTail = tail0 + t < L;
+  const A tailv = hasTail ? (A)to_float(xr[tail0 + t]) : (A)0;
+  auto sweep = [&](auto&& f) {
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      if ((LongType)i * NT + t < nv) {
+        A vals[VEC];
+        // (16-bit rows: the opaque pass keeps the compiler from holding the unpacked row, twice or four times the registers)
+        if constexpr (sizeof(T) == 2 && NV > 16) asm volatile("" : "+v"(v[i]));
+        RawIO<T>::unpack(v[i], vals);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) f(vals[e]);
+      }
+      __builtin_amdgcn_sched_barrier(0);   // one vector's arithmetic at a time: the row itself fills most of the registers
+    }
+    if (hasTail) f(tailv);
+  };
+  const A NEG = -r_tmax<A>();
+  A mx = NEG;
+  sweep([&](A val) { mx = LOG ? (val > mx ? val : mx) : softmax_maxstep<A>(mx, val, clamp); });
+  mx = block_allreduce<MaxOp, NT / 64, A>(mx, lds);
+  if (!LOG && clamp && mx == NEG) mx = (A)0;
+  A sum = (A)0;
+  auto term = [&](A val) -> A { if constexpr (LOG) return r_exp<A>(val - mx); else return softmax_term(val, mx, clamp); };
+  sweep([&](A val) { sum += term(val); });
+  sum = block_allreduce<SumOp, NT / 64, A>(sum, lds);
+  if (!LOG && clamp) sum = sum > (A)1e-6f ? sum : (A)1e-6f;
+  // long rows: the maximum passes through an opaque copy, so that the exponentials of the sum pass are taken again here
+  // instead of being kept in (spilled) registers
+  if constexpr (NV > 16 && sizeof(A) == 4) asm volatile("" : "+v"(mx));
+  auto result = [&](A val) -> A { if constexpr (LOG) return r_log<A>(term(val) / sum); else return term(val) / sum; };
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const LongType iv = (LongType)i * NT + t;
+    if (iv < nv) {
+      A vals[VEC];
+      if constexpr (sizeof(T) == 2 && NV > 16) asm volatile("" : "+v"(v[i]));
+      RawIO<T>::unpack(v[i], vals);
+#pragma unroll
+      for (int e = 0; e < VEC; e++) vals[e] = result(vals[e]);
+      const Raw o = RawIO<T>::pack(vals);
+      __builtin_memcpy(zr + iv * VEC, &o, sizeof(Raw));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if (hasTail) zr[tail0 + t] = Conv<T>::from(result(tailv));
+}
+template <typename T, bool LOG>
+static bool softmaxBlockRegs(hipStream_t s, const RowArgs& a, const T* x, T* z, int clamp, const RowPlan& p) {
+  constexpr LongType V = 16 / sizeof(T);
+  if (p.xInner != 1 || p.zInner != 1 || p.rowLen < V || p.rowLen / V > 32 * 512) return false;
+  const dim3 grid((unsigned)p.rows), block(512);
+  const LongType per = (p.rowLen / V + 511) / 512;
+  if (per <= 16) hipLaunchKernelGGL((softmax_block_regs<T, 16, LOG>), grid, block, 0, s, a, x, z, clamp);
+  else if (per <= 26) hipLaunchKernelGGL((softmax_block_regs<T, 26, LOG>), grid, block, 0, s, a, x, z, clamp);
+  else hipLaunchKernelGGL((softmax_block_regs<T, 32, LOG>), grid, block, 0, s, a, x, z, clamp);
+  return true;
+}
+
 // many short strided rows (softmax over a non-last axis): one thread per row, neighbouring threads
 // own neighbouring rows so that accesses coalesce across the wave
 template <typename T>
@@ -436,6 +516,9 @@ static void softmaxTyped(hipStream_t s, const void* x, void* z, const RowPlan& p
     if (L <= 64 * 16) { hipLaunchKernelGGL((softmax_rows<T, 64, 16, 1>), dim3(gw), dim3(256), 0, s, a, xt, zt, clamp, 0); return; }
     if (L <= 256 * 32) { hipLaunchKernelGGL((softmax_rows<T, 256, 32, 1>), dim3(gb), dim3(256), 0, s, a, xt, zt, clamp, 0); return; }
   }
+  if constexpr (sizeof(T) <= 4) {
+    if (softmaxBlockRegs<T, false>(s, a, xt, zt, clamp, p)) return;
+  }
   // unit-stride rows whose x and z starts sit at the same offset from a 16-byte boundary in every row
   if constexpr (sizeof(T) <= 4) {
     constexpr LongType V = 16 / sizeof(T);
@@ -489,6 +572,13 @@ void launchLogSoftmax(hipStream_t s, DataType dt, const void* x, void* z, const 
   const dim3 g((unsigned)p.rows), b(256);
   // long unit-stride rows whose x and z starts sit at the same offset from a 16-byte boundary: the vector kernel of the
   // long-row softmax with the logarithm on the way out
+  if (p.rowLen >= 8192) {
+    bool done = false;
+    if (dt == FLOAT32) done = softmaxBlockRegs<float, true>(s, a, (const float*)x, (float*)z, 0, p);
+    else if (dt == HALF) done = softmaxBlockRegs<f16_t, true>(s, a, (const f16_t*)x, (f16_t*)z, 0, p);
+    else if (dt == BFLOAT16) done = softmaxBlockRegs<bf16_t, true>(s, a, (const bf16_t*)x, (bf16_t*)z, 0, p);
+    if (done) { HIP_CHECK(hipGetLastError()); return; }
+  }
   if ((dt == FLOAT32 || dt == HALF || dt == BFLOAT16) && p.rowLen >= 8192 && p.xInner == 1 && p.zInner == 1 &&
       ((reinterpret_cast<uintptr_t>(x) ^ reinterpret_cast<uintptr_t>(z)) & 15) == 0 && p.outerX.rank == p.outerZ.rank) {
     const LongType V = dt == FLOAT32 ? 4 : 8;
