@@ -629,6 +629,38 @@ __global__ __launch_bounds__(256) void transpose_tiled(TransposeArgs a, const T*
   LongType rest = blockIdx.y, xo = 0, zo = 0;
   for (int d = a.nOther - 1; d >= 0; d--) { const LongType q = rest / a.oShape[d], c = rest - q * a.oShape[d]; xo += c * a.oX[d]; zo += c * a.oZ[d]; rest = q; }
   const LongType a0 = (LongType)ta * 64, b0 = (LongType)tb * 64;
+  if constexpr (sizeof(T) <= 4) {
+    // whole tiles: 16 bytes per lane on both sides of the copy (element-aligned vectors: any row pitch, any start), the
+    // transposition itself in LDS element by element -- with rows of 65 a wave's writes (4 or 8 tile rows, every V-th
+    // column) and its transposed reads both fall on every bank equally often
+    if (a0 + 64 <= a.nA && b0 + 64 <= a.nB) {
+      constexpr int V = 16 / sizeof(T), CPR = 64 / V, PER = 64 * CPR / 256;   // vectors per tile row, per thread
+      struct alignas(sizeof(T)) Pack { T e[V]; };
+      const int c = threadIdx.x % CPR, r = threadIdx.x / CPR;
+      Pack in[PER];
+#pragma unroll
+      for (int u = 0; u < PER; u++) {
+        const int j = r + u * (256 / CPR);
+        __builtin_memcpy(&in[u], x + xo + (a0 + c * V) + (b0 + j) * a.xB, sizeof(Pack));
+      }
+#pragma unroll
+      for (int u = 0; u < PER; u++) {
+        const int j = r + u * (256 / CPR);
+#pragma unroll
+        for (int e = 0; e < V; e++) tile[j][c * V + e] = in[u].e[e];
+      }
+      __syncthreads();
+#pragma unroll
+      for (int u = 0; u < PER; u++) {
+        const int i = r + u * (256 / CPR);
+        Pack out;
+#pragma unroll
+        for (int e = 0; e < V; e++) out.e[e] = tile[c * V + e][i];
+        __builtin_memcpy(z + zo + (a0 + i) * a.zA + (b0 + c * V), &out, sizeof(Pack));
+      }
+      return;
+    }
+  }
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   if (a0 + tx < a.nA) {
 #pragma unroll 4
