@@ -106,6 +106,26 @@ def test_permute_transpose_reshape(ex, oracle, dtype):
     assert np.array_equal(got, oracle.reshape(x.transpose(2, 1, 0), [10, -1]))
 
 
+@pytest.mark.parametrize("np_dt,dtype", [(np.float32, FLOAT32), (np.float64, DOUBLE), (np.float16, None), (np.uint16, BFLOAT16)])
+@pytest.mark.parametrize("shape,perm,lo", [((130, 200), (1, 0), 0), ((128, 192), (1, 0), 0), ((3, 128, 256), (0, 2, 1), 0), ((2, 70, 129), (2, 0, 1), 0),
+                                           ((131, 203), (1, 0), 3), ((64, 64), (1, 0), 1)])
+def test_transposing_copies_whole_and_ragged_tiles(ex, np_dt, dtype, shape, perm, lo):
+    """permute writes a dense copy of a view whose unit stride runs along another axis than the result's: whole 64 x 64 tiles
+    move as 16-byte vectors on both sides, ragged edges element by element; `lo` cuts rows and columns off the input so that
+    its rows start off 16-byte boundaries.  Bit patterns are compared (bf16 arrays are carried as their uint16 patterns)."""
+    rng = np.random.default_rng(sum(shape) + lo)
+    full = rng.integers(0, 60000, size=shape).astype(np.uint16)
+    host = full if np_dt == np.uint16 else (full.view(np.float16) if np_dt == np.float16 else (full % 1000).astype(np_dt))
+    X = NDArray.from_numpy(host, dtype) if dtype == BFLOAT16 else NDArray.from_numpy(host)
+    view, want = X, host
+    if lo:
+        view = X.slice(len(shape) - 1, lo, shape[-1]).slice(len(shape) - 2, lo, shape[-2])
+        want = host[..., lo:, lo:]
+    got = _run(ex, "permute", [view], i_args=list(perm))[0].to_numpy()
+    assert got.shape == tuple(want.shape[p] for p in perm)
+    assert np.array_equal(got.view(np.uint8), np.ascontiguousarray(want.transpose(perm)).view(np.uint8))
+
+
 def test_reshape_errors(ex):
     X = NDArray.from_numpy(np.zeros((3, 4), np.float32))
     with pytest.raises(NativeOpsError, match="Only one unknown dimension"):
