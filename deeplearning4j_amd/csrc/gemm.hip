@@ -91,6 +91,61 @@ __device__ __forceinline__ void epilogueExtras(int hasEpi, const GemmEpilogue& e
 }
 template <typename T>
 __device__ __forceinline__ void epilogueExtras(const GemmArgs& g, LongType row, LongType col, T yv) { epilogueExtras<T>(g.hasEpi, g.epi, row, col, yv); }
+// The same for four consecutive columns of one row held by one lane (col a multiple of 4, 16-bit T): 8-byte loads and
+// stores wherever the target's rows and column range allow them, the element path otherwise.  Same values either way.
+template <typename T>
+__device__ __forceinline__ void epilogueExtras4(const GemmArgs& g, LongType row, LongType col, const float (&v)[4]) {
+  if (!g.hasEpi) return;
+  const GemmEpilogue& epi = g.epi;
+  T yv[4];
+#pragma unroll
+  for (int e = 0; e < 4; e++) yv[e] = Conv<T>::from(v[e]);
+  auto pack4 = [](const T (&q)[4]) { u32x2 o; o[0] = (unsigned)q[0].bits | ((unsigned)q[1].bits << 16); o[1] = (unsigned)q[2].bits | ((unsigned)q[3].bits << 16); return o; };
+  auto ok8 = [](const void* p, LongType pitch) { return (reinterpret_cast<uintptr_t>(p) & 7) == 0 && pitch % 4 == 0; };
+  if (epi.act) {
+    T a[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) { const float y = to_float(yv[e]); a[e] = Conv<T>::from(epi.act == 1 ? gelu_low(y) : gelu_full(y)); }
+    T* dst = static_cast<T*>(epi.actOut) + row * epi.actRow + col;
+    if (ok8(epi.actOut, epi.actRow)) *reinterpret_cast<u32x2*>(dst) = pack4(a);
+    else {
+#pragma unroll
+      for (int e = 0; e < 4; e++) dst[e] = a[e];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    if (i >= epi.nCopy) break;
+    const auto& c = epi.copy[i];
+    if (col + 4 <= c.c0 || col >= c.c1) continue;
+    T* dst = static_cast<T*>(c.dst) + row * c.dstRow + (col - c.c0);
+    if (col >= c.c0 && col + 4 <= c.c1 && ok8(c.dst, c.dstRow) && c.c0 % 4 == 0) *reinterpret_cast<u32x2*>(dst) = pack4(yv);
+    else {
+#pragma unroll
+      for (int e = 0; e < 4; e++) if (col + e >= c.c0 && col + e < c.c1) dst[e] = yv[e];
+    }
+  }
+  if (epi.resOut) {
+    const T* in = static_cast<const T*>(epi.resIn) + row * epi.resInRow + col;
+    T* out = static_cast<T*>(epi.resOut) + row * epi.resOutRow + col;
+    T r[4];
+    if (ok8(epi.resIn, epi.resInRow)) {
+      const u32x2 w = *reinterpret_cast<const u32x2*>(in);
+      r[0].bits = (unsigned short)(w[0] & 0xffffu); r[1].bits = (unsigned short)(w[0] >> 16);
+      r[2].bits = (unsigned short)(w[1] & 0xffffu); r[3].bits = (unsigned short)(w[1] >> 16);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; e++) r[e] = in[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 4; e++) r[e] = Conv<T>::from(to_float(r[e]) + to_float(yv[e]));
+    if (ok8(epi.resOut, epi.resOutRow)) *reinterpret_cast<u32x2*>(out) = pack4(r);
+    else {
+#pragma unroll
+      for (int e = 0; e < 4; e++) out[e] = r[e];
+    }
+  }
+}
 
 // ---- fallback --------------------------------------------------------------------------------------------------
 template <typename T>
@@ -2311,10 +2366,7 @@ __global__ __launch_bounds__(256) void gemm_skinny32(GemmArgs g, const T* __rest
     o[0] = (unsigned)Conv<T>::from(v[0]).bits | ((unsigned)Conv<T>::from(v[1]).bits << 16);
     o[1] = (unsigned)Conv<T>::from(v[2]).bits | ((unsigned)Conv<T>::from(v[3]).bits << 16);
     *reinterpret_cast<u32x2*>(C + (LongType)mrow * g.cRow + n) = o;
-    if (g.hasEpi) {
-#pragma unroll
-      for (int e = 0; e < 4; e++) epilogueExtras<T>(g, mrow, n + e, Conv<T>::from(v[e]));
-    }
+    epilogueExtras4<T>(g, mrow, n, v);
   }
 }
 template <typename T>
