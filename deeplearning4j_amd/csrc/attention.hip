@@ -26,6 +26,7 @@
 #include "device.h"
 #include "kernels.h"
 #include "mfma_tile.h"
+#include "rowmath.h"
 #include "runtime.h"
 
 namespace nd4jhip {
@@ -96,6 +97,8 @@ struct FusedArgs {
   int qTiles, perBatch, nBatch, heavyFirst;   // fused kernel: work slots per batch entry, batch entries, block order
   const unsigned char* vmask;                 // VM kernels: dense [batch entries, Tv] bytes, 0 = padded key
   float maskValue;                            // what a masked logit has subtracted
+  int splits = 1;                             // decode kernel: key ranges per (batch entry, query), blockIdx.z picks one
+  float* partial = nullptr;                   // ... and where a range's partial result goes (null: the block writes the output)
 };
 
 template <typename T> __device__ __forceinline__ float round_storage(float v) { return to_float(Conv<T>::from(v)); }
@@ -513,6 +516,14 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
   // are issued before the first value is touched, so the two latencies overlap
   using Raw = typename Row8<T>::raw;
   const Raw qraw = Row8<T>::load(Q + qi * a.qT + c * 8);
+  // this block's key range (the whole history unless it is cut up)
+  LongType kBeg = 0, kEnd = a.Tv;
+  if (a.splits > 1) {
+    const LongType per = (a.Tv + a.splits - 1) / a.splits;
+    kBeg = (LongType)blockIdx.z * per;
+    kEnd = kBeg + per < a.Tv ? kBeg + per : a.Tv;
+    if (kBeg > kEnd) kBeg = kEnd;
+  }
   // (a second register set, so that the next trip's loads fly while the current one is consumed, changed nothing at
   // batch 1 and cost 1 % at batch 32: a block's stream is bound by what one CU can pull, not by a trip's latency)
   Raw krA[U], vrA[U];
@@ -521,15 +532,15 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
 #pragma unroll
     for (int u = 0; u < U; u++) {
       LongType key = k0 + u * KPS + g;
-      valid[u] = key < a.Tv;
+      valid[u] = key < kEnd;
       key = valid[u] ? key : a.Tv - 1;
       kr[u] = Row8<T>::load(K + key * a.kT + c * 8);
       vr[u] = Row8<T>::load(V + key * a.vT + c * 8);
     }
   };
   const LongType step = (LongType)NW * (KPS * U);
-  LongType k0 = (LongType)wave * (KPS * U);
-  if (k0 < a.Tv) issue(k0, krA, vrA, validA);
+  LongType k0 = kBeg + (LongType)wave * (KPS * U);
+  if (k0 < kEnd) issue(k0, krA, vrA, validA);
   float q[8];
   Row8<T>::unpack(qraw, q);
   const float L2E = 1.44269502162933349609375f;
@@ -578,10 +589,10 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
       for (int e = 0; e < 8; e++) o[e] = __builtin_fmaf(p, vf[e], o[e]);
     }
   };
-  while (k0 < a.Tv) {
+  while (k0 < kEnd) {
     consume(k0, krA, vrA, validA);
     k0 += step;
-    if (k0 < a.Tv) issue(k0, krA, vrA, validA);
+    if (k0 < kEnd) issue(k0, krA, vrA, validA);
   }
   // merge the lane groups of the wave (lanes with equal c): bring every state to the wave's maximum, then add.  Max and
   // sum of l run on DPP; the eight-float partial rows go through the wave's own LDS region, where lane d sums element d
@@ -618,8 +629,42 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
       lt = __builtin_fmaf(sm[w][D + 1], fw, lt);
       ot = __builtin_fmaf(sm[w][t], fw, ot);
     }
-    O[qi * a.oT + t] = Conv<T>::from(lt > 0.f ? ot / lt : 0.f);
+    if (a.partial) {
+      // one key range of several: the sums stay relative to this range's maximum; whoever merges the ranges normalises
+      float* P = a.partial + ((b * a.Tq + qi) * a.splits + blockIdx.z) * ATTN_PART_PITCH(D);
+      P[t] = ot;
+      if (t == 0) { P[D] = mm; P[D + 1] = lt; }
+    } else {
+      O[qi * a.oT + t] = Conv<T>::from(lt > 0.f ? ot / lt : 0.f);
+    }
   }
+}
+// the output rows from the partial results of the key ranges: one block per (batch entry, query), a thread per element
+template <typename T, int D>
+__global__ __launch_bounds__(D) void attn_merge(FusedArgs a, T* __restrict__ O) {
+  const LongType b = blockIdx.x, qi = blockIdx.y;
+  if (a.H > 0) {
+    const LongType hi = b / a.H, lo = b - hi * a.H;
+    O += hi * a.oB2 + lo * a.oB;
+  } else {
+    O += b * a.oB;
+  }
+  float v[1];
+  attn_merge_vec<1>(a.partial + (b * a.Tq + qi) * a.splits * ATTN_PART_PITCH(D), a.splits, D, (int)threadIdx.x, v);
+  O[qi * a.oT + threadIdx.x] = Conv<T>::from(v[0]);
+}
+
+// One query token against a long history (a decode step at batch 1: one block per head, whose keys and values all come
+// through one CU): cut the history into ranges of at least 128 keys so that about 48 blocks share the read.  Only where the
+// heads of that one token are the whole problem: the merge of the ranges is then a step the one-row product that consumes
+// the output can take in (a recorded sequence does that); with more rows it would stay a launch of its own, which costs more
+// than the cut saves.
+int attentionDecodeSplits(const AttnDesc& d) {
+  const bool oneToken = d.Tq == 1 && (d.H > 0 ? d.B == d.H : d.B == 1);
+  if (!oneToken || d.vmask != nullptr || d.B > 24 || d.Tv < 256) return 1;
+  LongType s = 48 / (d.B * d.Tq);
+  if (s > d.Tv / 128) s = d.Tv / 128;
+  return s >= 8 ? 8 : s >= 4 ? 4 : s >= 2 ? 2 : 1;   // (the merge routines are built for 2, 4 and 8 parts)
 }
 
 bool attentionDecodeSupported(DataType dt, const AttnDesc& d) {
@@ -639,6 +684,17 @@ static void launchDecodeTyped(hipStream_t s, const void* q, const void* k, const
   a.H = d.H; a.qB2 = d.qB2; a.kB2 = d.kB2; a.vB2 = d.vB2; a.oB2 = d.oB2;
   a.scale = d.scale; a.applyScale = d.applyScale ? 1 : 0; a.causal = 0; a.qTiles = 1; a.perBatch = 1;
   a.vmask = d.vmask; a.maskValue = d.maskValue;
+  a.splits = 1; a.partial = nullptr;
+  if (d.splits > 1) {
+    // a range per block (8 waves: a range of a few hundred keys is one trip to memory), then the merge unless the caller
+    // leaves it to its next kernel
+    ND4J_REQUIRE(d.partial != nullptr && d.vmask == nullptr, "attention: the cut-up decode kernel needs a partial buffer and takes no value mask");
+    a.splits = d.splits; a.partial = d.partial;
+    hipLaunchKernelGGL((attn_decode<T, D, 8, false>), dim3((unsigned)d.B, (unsigned)d.Tq, (unsigned)d.splits), dim3(512), 0, s, a, (const T*)q, (const T*)k,
+                       (const T*)v, (T*)out);
+    if (!d.mergeLater) hipLaunchKernelGGL((attn_merge<T, D>), dim3((unsigned)d.B, (unsigned)d.Tq), dim3(D), 0, s, a, (T*)out);
+    return;
+  }
   const dim3 grid((unsigned)d.B, (unsigned)d.Tq);
   if (d.vmask) {
     hipLaunchKernelGGL((attn_decode<T, D, 4, true>), grid, dim3(256), 0, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
@@ -649,6 +705,20 @@ static void launchDecodeTyped(hipStream_t s, const void* q, const void* k, const
   else hipLaunchKernelGGL((attn_decode<T, D, 4, false>), grid, dim3(256), 0, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
 }
 
+template <typename T, int D>
+static void launchMergeTyped(hipStream_t s, void* out, const AttnDesc& d) {
+  FusedArgs a;
+  a.Tq = d.Tq; a.Tv = d.Tv; a.oB = d.oB; a.oT = d.oT; a.H = d.H; a.oB2 = d.oB2;
+  a.splits = d.splits; a.partial = d.partial;
+  hipLaunchKernelGGL((attn_merge<T, D>), dim3((unsigned)d.B, (unsigned)d.Tq), dim3(D), 0, s, a, (T*)out);
+}
+void launchAttentionDecodeMerge(hipStream_t s, DataType dt, void* out, const AttnDesc& d) {
+  ND4J_REQUIRE(d.splits > 1 && d.partial != nullptr && (d.D == 64 || d.D == 128), "attention: nothing to merge");
+  if (dt == HALF) { if (d.D == 64) launchMergeTyped<f16_t, 64>(s, out, d); else launchMergeTyped<f16_t, 128>(s, out, d); }
+  else if (dt == BFLOAT16) { if (d.D == 64) launchMergeTyped<bf16_t, 64>(s, out, d); else launchMergeTyped<bf16_t, 128>(s, out, d); }
+  else { if (d.D == 64) launchMergeTyped<float, 64>(s, out, d); else launchMergeTyped<float, 128>(s, out, d); }
+  HIP_CHECK(hipGetLastError());
+}
 void launchAttentionDecode(hipStream_t s, DataType dt, const void* q, const void* k, const void* v, void* out, const AttnDesc& d) {
   ND4J_REQUIRE(attentionDecodeSupported(dt, d), "attention: decode kernel does not take this problem");
   ND4J_REQUIRE((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) == 0, "attention: operands must be 16-byte aligned");

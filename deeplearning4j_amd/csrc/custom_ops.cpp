@@ -265,7 +265,10 @@ static XwGeometry xwGeometry(Context& c, bool needOutput) {
 // that ran wrote them
 // out = layer_norm(x; gain, bias) is the product's input: `rows` rows of unit element stride, xPitch / outPitch elements apart
 struct LnPrologue { NDArray *x, *gain, *bias, *out; LongType rows, xPitch, outPitch; };
-static bool xwPlusBImpl(Context& c, const GemmEpilogue* epi, const LnPrologue* ln = nullptr) {
+// the product's input row is the output of an attention that left the records of its key ranges in `partial` (device memory):
+// the product merges them on its way in and writes the row to `out` as well
+struct AttnMergePrologue { const float* partial; int splits, D; NDArray* out; };
+static bool xwPlusBImpl(Context& c, const GemmEpilogue* epi, const LnPrologue* ln = nullptr, const AttnMergePrologue* am = nullptr) {
   ND4J_REQUIRE(c.width() >= 3, "xw_plus_b: x, weights and bias are required");
   NDArray* x = c.input(0); NDArray* w = c.input(1); NDArray* b = c.input(2); NDArray* z = c.output(0);
   if (x->isEmpty() || w->isEmpty() || b->isEmpty()) return epi == nullptr;
@@ -289,6 +292,16 @@ static bool xwPlusBImpl(Context& c, const GemmEpilogue* epi, const LnPrologue* l
     d.lnGain = ln->gain->specialBuffer(); d.lnBias = ln->bias->specialBuffer(); d.lnOut = ln->out->specialBuffer(); d.lnOutRow = ln->outPitch;
     const bool done = launchGemm(stream(), dt, ln->x->specialBuffer(), w->specialBuffer(), z->specialBuffer(), d);
     if (done) registerSpecialUse({z, ln->out}, {ln->x, ln->gain, ln->bias, w, b});
+    return done;
+  }
+  if (am) {
+    if (g.M != 1 || g.aCol != 1 || am->out->lengthOf() != g.K || am->out->dataType() != dt) return false;
+    prepareSpecialUse({z, am->out}, {w, b});
+    d.bias = b->specialBuffer();
+    d.epi = epi;
+    d.attnPartial = am->partial; d.attnSplits = am->splits; d.attnD = am->D; d.attnOut = am->out->specialBuffer();
+    const bool done = launchGemm(stream(), dt, am->out->specialBuffer(), w->specialBuffer(), z->specialBuffer(), d);
+    if (done) registerSpecialUse({z, am->out}, {w, b});
     return done;
   }
   prepareSpecialUse({z}, {x, w, b});
@@ -476,6 +489,10 @@ static bool denseRows(const BatchedView& v) {   // row-major [B, T, D] without g
   if (v.H > 0) return v.sB == v.T * v.D && v.sB2 == v.H * v.T * v.D;
   return v.B == 1 || v.sB == v.T * v.D;
 }
+// Set by a merged step of a recording around its call of the attention op: when the decode kernel cuts the key range up, it
+// leaves the merge of the parts to the caller's next kernel and says here where the parts are.
+struct AttnMergeRequest { bool deferred = false; AttnDesc desc; DataType dt = FLOAT32; };
+static AttnMergeRequest* g_attnMergeRequest = nullptr;
 static void attentionExec(Context& c) {
   ND4J_REQUIRE(c.width() >= 2, "dot_product_attention_v2: queries and values are required");
   NDArray* q0 = c.input(0); NDArray* v0 = c.input(1); NDArray* k0 = c.width() > 2 ? c.input(2) : v0;
@@ -551,6 +568,13 @@ static void attentionExec(Context& c) {
   // the query mask scales the weights output only: out = weights v has been formed before (AttentionHelper.cpp:455-467)
   const void* qm = qMask && wantW ? denseMask(qMask, dt) : nullptr;
   if (useDecode) {
+    const int cut = attentionDecodeSplits(d);
+    if (cut > 1 && (size_t)(d.B * d.Tq * cut) * (size_t)(d.D + 4) * sizeof(float) <= LaunchContext::ALLOCATION_BYTES) {
+      // the parts' records go to the scratch the split-K products use: written and read back by kernels that follow each other
+      d.splits = cut;
+      d.partial = static_cast<float*>(LaunchContext::defaultContext()->allocationBuffer);
+      if (g_attnMergeRequest != nullptr) { d.mergeLater = true; g_attnMergeRequest->deferred = true; g_attnMergeRequest->desc = d; g_attnMergeRequest->dt = dt; }
+    }
     launchAttentionDecode(stream(), dt, q0->specialBuffer(), k0->specialBuffer(), v0->specialBuffer(), o0->specialBuffer(), d);
   } else if (useFused) {
     launchAttentionFused(stream(), dt, q0->specialBuffer(), k0->specialBuffer(), v0->specialBuffer(), o0->specialBuffer(), d);
@@ -1913,6 +1937,31 @@ std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& rec,
     out = LnPrologue{lx, lg, lb, lo, rr, ss, s2};
     return true;
   };
+  // is rec[li] an attention (output only) whose output row -- one query, the heads side by side -- is the input row of the
+  // xw_plus_b behind it?  Then, when the attention cuts its key range up, that product merges the parts on its way in.
+  auto attnMergeAt = [&](size_t li) {
+    if (li + 1 >= n) return false;
+    RecordedOp& r = rec[li];
+    RecordedOp& x = rec[li + 1];
+    if (r.kind != RecordedOp::CUSTOM || r.op->name != "dot_product_attention_v2" || r.ctx.outputs.empty() || !r.ctx.outputs[0]) return false;
+    for (size_t o = 1; o < r.ctx.outputs.size(); o++) if (r.ctx.outputs[o]) return false;
+    if (x.kind != RecordedOp::CUSTOM || x.op->name != "xw_plus_b" || x.ctx.inputs.size() < 3 || !x.ctx.inputs[0] || iArg(x.ctx, 0, 0) == 1) return false;
+    NDArray *o = r.ctx.outputs[0], *in = x.ctx.inputs[0];
+    if (o->buf.get() != in->buf.get() || o->offset != in->offset || o->dataType() != in->dataType() || o->lengthOf() != in->lengthOf()) return false;
+    LongType rr, cc, ss;
+    if (!asRows(in, rr, cc, ss) || rr != 1 || o->rankOf() < 2) return false;
+    // the output's elements in (head, value) order must be the row's elements in order: one query, unit value stride, heads D apart
+    const int rank = o->rankOf();
+    const LongType D = o->sizeAt(rank - 1);
+    if (o->sizeAt(rank - 2) != 1 || (D > 1 && o->strideAt(rank - 1) != 1)) return false;
+    LongType heads = 1;
+    for (int d = 0; d < rank - 2; d++) {
+      if (o->sizeAt(d) == 1) continue;
+      if (d != rank - 3 || o->strideAt(d) != D) return false;
+      heads = o->sizeAt(d);
+    }
+    return heads * D == cc;
+  };
   for (size_t i = 0; i < n;) {
     RecordedOp& r = rec[i];
     // pairwise Add whose result the next op layer-normalises
@@ -1930,9 +1979,11 @@ std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& rec,
     // caches), a pairwise Add of the result to another array (the residual connection)
     {
       RecordedOp* lnOp = nullptr;
+      RecordedOp* attnOp = nullptr;
       LnPrologue lnPro{};
       size_t xi = i;
       if (lnPrologueAt(i, lnPro)) { lnOp = &r; xi = i + 1; }
+      else if (attnMergeAt(i)) { attnOp = &r; xi = i + 1; }
       RecordedOp& xw = rec[xi];
       if (xw.kind == RecordedOp::CUSTOM && xw.op->name == "xw_plus_b" && xw.ctx.outputs.size() >= 1 && xw.ctx.outputs[0] && xw.ctx.inputs.size() >= 3 &&
           xw.ctx.inputs[0] && xw.ctx.inputs[1] && xw.ctx.inputs[2]) {
@@ -1950,6 +2001,7 @@ std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& rec,
           bool clash = f.z->buf.get() == z->buf.get();   // an absorbed op writes neither the product's operands nor its result
           for (NDArray* in : xw.ctx.inputs) if (in && in->buf.get() == f.z->buf.get()) clash = true;
           if (lnOp) for (NDArray* in : lnOp->ctx.inputs) if (in && in->buf.get() == f.z->buf.get()) clash = true;
+          if (attnOp) for (NDArray* in : attnOp->ctx.inputs) if (in && in->buf.get() == f.z->buf.get()) clash = true;
           if (clash || f.z->dataType() != dt) break;
           LongType fr, fc, fs;
           if (f.kind == RecordedOp::TRANSFORM_STRICT && f.opNum == 53 && epi.act == 0 && sameView(f.x, z) && asRows(f.z, fr, fc, fs) && fr == zr && fc == zc) {
@@ -1983,9 +2035,9 @@ std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& rec,
           // nothing may follow an absorbed Add inside this kernel: later ops read its result
           if (f.kind == RecordedOp::PAIRWISE) break;
         }
-        if (lnOp || !absorbed.empty()) {
+        if (lnOp || attnOp || !absorbed.empty()) {
           RecordedOp* x = &xw;
-          plan.push_back([x, lnOp, lnPro, epi, absorbed] {
+          plan.push_back([x, lnOp, attnOp, lnPro, epi, absorbed] {
             GemmEpilogue e = epi;
             NDArray* z = x->ctx.outputs[0];
             std::vector<NDArray*> writes, reads;
@@ -2006,6 +2058,20 @@ std::vector<std::function<void()>> fuseRecordedOps(std::vector<RecordedOp>& rec,
               done = xwPlusBImpl(x->ctx, ep, &lnPro);
               applied = done && epiOk;
               if (done) fusedAppliedCounter() += 1; else runRecorded(lnOp);
+            }
+            if (attnOp) {
+              // the attention runs as recorded; where it cuts its key range up it leaves the merge to this product
+              AttnMergeRequest req;
+              g_attnMergeRequest = &req;
+              try { runRecorded(attnOp); } catch (...) { g_attnMergeRequest = nullptr; throw; }
+              g_attnMergeRequest = nullptr;
+              if (req.deferred) {
+                NDArray* ao = attnOp->ctx.outputs[0];
+                AttnMergePrologue am{req.desc.partial, req.desc.splits, (int)req.desc.D, ao};
+                done = xwPlusBImpl(x->ctx, ep, nullptr, &am);
+                applied = done && epiOk;
+                if (!done) launchAttentionDecodeMerge(stream(), req.dt, ao->specialBuffer(), req.desc);   // the product declined: merge, then multiply
+              }
             }
             if (!done) applied = xwPlusBImpl(x->ctx, ep) && epiOk;
             if (applied) fusedAppliedCounter() += (int)absorbed.size();

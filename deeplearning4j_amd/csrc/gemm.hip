@@ -1857,11 +1857,16 @@ __global__ __launch_bounds__(256) void gemv_rowdot(const T* __restrict__ W, Long
 // PRO_LN: the row multiplied is layer_norm(x; lnGain, lnBias) over its K elements -- every wave normalises the row it has
 // loaded anyway (the routine the row kernel runs, so the same bits), and the first wave of the grid also stores it to lnOut,
 // where the separate layer_norm op would have put it.
-template <typename T, int OPW, int NL, bool HAS_BIAS, bool PRO_LN = false>
+// PRO == 2: the row multiplied is the output of an attention whose key range was cut up -- every wave merges the parts'
+// records into the piece of the row it needs (the routine the attention's own merge kernel runs, so the same bits), and the
+// first wave of the grid also stores the row where that kernel would have put it (x is then only written, as am.out).
+struct AttnMergeArgs { const float* partial = nullptr; int D = 0, logD = 0; void* out = nullptr; };
+template <typename T, int OPW, int NL, bool HAS_BIAS, int PRO = 0>
 __global__ __launch_bounds__(256) void gemv_rowdot_pre(const T* __restrict__ W, LongType ldw, const T* __restrict__ x, T* __restrict__ y, LongType ys,
                                                        LongType N, LongType K, const T* __restrict__ bias, int hasEpi, GemmEpilogue epi,
                                                        const T* __restrict__ lnGain = nullptr, const T* __restrict__ lnBias = nullptr,
-                                                       T* __restrict__ lnOut = nullptr, float lnEps = 0.f) {
+                                                       T* __restrict__ lnOut = nullptr, float lnEps = 0.f, AttnMergeArgs am = AttnMergeArgs()) {
+  constexpr bool PRO_LN = PRO == 1;
   constexpr int V = 16 / sizeof(T);
   using Raw = typename RawIO<T>::raw;
   const int lane = threadIdx.x & 63;
@@ -1879,7 +1884,21 @@ __global__ __launch_bounds__(256) void gemv_rowdot_pre(const T* __restrict__ W, 
     const int kk = lane + 64 * i, kc = kk < kw ? kk : kw - 1;
 #pragma unroll
     for (int o = 0; o < OPW; o++) wr[o][i] = reinterpret_cast<const raw_u32x4*>(wrow[o])[kc];
-    xr[i] = reinterpret_cast<const raw_u32x4*>(x)[kc];
+    if constexpr (PRO != 2) xr[i] = reinterpret_cast<const raw_u32x4*>(x)[kc];
+  }
+  if constexpr (PRO == 2) {
+    const bool first = blockIdx.x == 0 && (threadIdx.x >> 6) == 0;
+#pragma unroll
+    for (int i = 0; i < NL; i++) {
+      const int kk = lane + 64 * i, kc = kk < kw ? kk : kw - 1;
+      // (four parts and a head size that is a power of two -- the host checks both -- keep this prologue one short code path)
+      const int k = kc * V, head = k >> am.logD, t0 = k - (head << am.logD);
+      float vals[V];
+      attn_merge_parts<V, 4>(am.partial + (LongType)head * 4 * ATTN_PART_PITCH(am.D), am.D, t0, vals);
+      const Raw packed = RawIO<T>::pack(vals);
+      xr[i] = __builtin_bit_cast(raw_u32x4, packed);
+      if (first && kk < kw) reinterpret_cast<Raw*>(am.out)[kk] = packed;
+    }
   }
   T bq[OPW];
   if (HAS_BIAS) {
@@ -1946,7 +1965,18 @@ static bool tryGemvRowdotPre(hipStream_t s, const GemmDesc& d, const void* A, co
 #define ROWDOT_LN(OPW, NL) hipLaunchKernelGGL((gemv_rowdot_pre<T, OPW, NL, true, true>), dim3((unsigned)(((d.N + OPW - 1) / OPW + 3) / 4)), dim3(256), 0, s, \
                                               (const T*)B, d.bCol, (const T*)A, (T*)C, d.cCol, d.N, d.K, (const T*)d.bias, d.epi ? 1 : 0, d.epi ? *d.epi : GemmEpilogue(), \
                                               (const T*)d.lnGain, (const T*)d.lnBias, (T*)d.lnOut, d.lnEps)
+#define ROWDOT_AM(OPW, NL) hipLaunchKernelGGL((gemv_rowdot_pre<T, OPW, NL, true, 2>), dim3((unsigned)(((d.N + OPW - 1) / OPW + 3) / 4)), dim3(256), 0, s, \
+                                              (const T*)B, d.bCol, (const T*)A, (T*)C, d.cCol, d.N, d.K, (const T*)d.bias, d.epi ? 1 : 0, d.epi ? *d.epi : GemmEpilogue(), \
+                                              (const T*)nullptr, (const T*)nullptr, (T*)nullptr, 0.f, am)
 #define ROWDOT(OPW, NL) do { noteKernel("gemv_rowdot_pre<%s,opw=%d,nl=%d>", tname<T>(), OPW, NL); if (d.bias) ROWDOT_B(OPW, NL, true); else ROWDOT_B(OPW, NL, false); } while (0)
+  if (d.attnPartial) {   // the row is merged from the records of a cut-up attention on the way in: short rows with a bias only
+    if (!d.bias || passes > 2 || d.attnSplits != 4 || (d.attnD != 64 && d.attnD != 128) || d.K % d.attnD != 0 || (reinterpret_cast<uintptr_t>(d.attnOut) & 15)) return false;
+    AttnMergeArgs am;
+    am.partial = d.attnPartial; am.D = d.attnD; am.logD = d.attnD == 64 ? 6 : 7; am.out = d.attnOut;
+    noteKernel("gemv_rowdot_pre<%s,attn-merge,nl=2>", tname<T>());
+    ROWDOT_AM(2, 2);
+    return true;
+  }
   if (d.lnGain) {   // the row is normalised on the way in: short rows with a bias only
     if (!d.bias || passes > 4 || ((reinterpret_cast<uintptr_t>(d.lnGain) | reinterpret_cast<uintptr_t>(d.lnBias) | reinterpret_cast<uintptr_t>(d.lnOut)) & 15)) return false;
     noteKernel("gemv_rowdot_pre<%s,ln,nl=%d>", tname<T>(), passes <= 2 ? 2 : 4);
@@ -1962,6 +1992,7 @@ static bool tryGemvRowdotPre(hipStream_t s, const GemmDesc& d, const void* A, co
 #undef ROWDOT
 #undef ROWDOT_B
 #undef ROWDOT_LN
+#undef ROWDOT_AM
   return true;
 }
 // y[n] = alpha * sum_k x[k] * W[k][n]: W rows contiguous in n.  A thread owns V consecutive outputs of one k-slice;
@@ -2423,6 +2454,10 @@ static bool launchMfma16u(hipStream_t s, const GemmDesc& d, const void* A, const
 
 template <typename T>
 static bool dispatch16(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
+  if (d.attnPartial) {   // only the one-row product against k-contiguous weights merges an attention's parts on the way in
+    if (d.M == 1 && d.N > 1 && d.batch == 1 && d.bRow == 1 && d.cCol == 1 && !d.lnGain) return tryGemvRowdotPre<T>(s, d, A, B, C);
+    return false;
+  }
   if (d.lnGain) {   // only the products of 1 and of 5 to 32 rows against k-contiguous weights normalise their rows on the way in
     if (d.M == 1 && d.N > 1 && d.batch == 1 && d.bRow == 1 && d.cCol == 1) return tryGemvRowdotPre<T>(s, d, A, B, C);
     if (d.M >= 5 && d.M <= 32) return tryGemmSkinny<T>(s, d, A, B, C);
@@ -2464,7 +2499,7 @@ static void dispatch32(hipStream_t s, const GemmDesc& d, const void* A, const vo
 bool launchGemm(hipStream_t s, DataType dt, const void* A, const void* B, void* C, const GemmDesc& d) {
   if (d.M == 0 || d.N == 0 || d.batch == 0) return true;
   ND4J_REQUIRE(d.batch < 65536 && (d.M + 31) / 32 < 65536 && (d.N + 31) / 32 < (1LL << 31), "matmul: problem too large for the launch grid");
-  bool withEpilogue = d.epi != nullptr || d.lnGain != nullptr;
+  bool withEpilogue = d.epi != nullptr || d.lnGain != nullptr || d.attnPartial != nullptr;
   if (withEpilogue) {
     // only the 16-bit decode-step kernels carry epilogue outputs; when the dispatch lands elsewhere nothing has been
     // launched yet and the product runs again without the request
@@ -2472,7 +2507,7 @@ bool launchGemm(hipStream_t s, DataType dt, const void* A, const void* B, void* 
     if (dt == HALF) done = dispatch16<f16_t>(s, d, A, B, C);
     else if (dt == BFLOAT16) done = dispatch16<bf16_t>(s, d, A, B, C);
     if (done) { HIP_CHECK(hipGetLastError()); return true; }
-    if (d.lnGain) return false;   // nothing launched: the caller normalises the row with the separate op and calls again
+    if (d.lnGain || d.attnPartial) return false;   // nothing launched: the caller runs the separate op (layer_norm, merge) and calls again
     GemmDesc plain = d;
     plain.epi = nullptr;
     launchGemm(s, dt, A, B, C, plain);

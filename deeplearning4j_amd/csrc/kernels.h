@@ -238,6 +238,12 @@ struct GemmDesc {
   void* lnOut = nullptr;
   LongType lnOutRow = 0;
   float lnEps = 1e-5f;
+  // other optional prologue (one row, M = 1): op(A) is the output row of an attention whose key range was cut into attnSplits
+  // parts -- the row is merged from the parts' records in attnPartial (heads of attnD values side by side along K) on the way in
+  // and also written to attnOut, where the attention's own merge kernel would have put it.  Counts like the one above.
+  const float* attnPartial = nullptr;
+  int attnSplits = 0, attnD = 0;
+  void* attnOut = nullptr;
 };
 // Returns true when every requested epilogue output was written; false: C was computed by a kernel without them and the
 // caller runs the follow-up ops itself (always true without an epilogue request).
@@ -257,13 +263,23 @@ struct AttnDesc {
   bool causal = false;
   float maskValue = 1e9f;
   const unsigned char* vmask = nullptr;   // optional value (padding) mask, dense [B, Tv] bytes: 0 = masked key
+  // decode kernel only: the keys of every (batch entry, query) cut into `splits` ranges, one block each, which leave
+  // partial results in `partial` ([B * Tq][splits][ATTN_PART_PITCH(D)] floats); a merge kernel then writes `out` unless
+  // mergeLater is set (the caller's next kernel merges on its way in)
+  int splits = 1;
+  float* partial = nullptr;
+  bool mergeLater = false;
 };
+// how many key ranges the decode kernel should cut a problem into (1: do not cut)
+int attentionDecodeSplits(const AttnDesc& d);
 // fused path (no logits/weights written)
 bool attentionFusedSupported(DataType dt, const AttnDesc& d);
 void launchAttentionFused(hipStream_t s, DataType dt, const void* q, const void* k, const void* v, void* out,
                           const AttnDesc& d);
 // a few query rows against a long history, no causal mask (decode steps with a key/value cache)
 bool attentionDecodeSupported(DataType dt, const AttnDesc& d);
+// the merge step of a cut-up decode attention on its own (d.splits, d.partial as given to launchAttentionDecode with mergeLater)
+void launchAttentionDecodeMerge(hipStream_t s, DataType dt, void* out, const AttnDesc& d);
 void launchAttentionDecode(hipStream_t s, DataType dt, const void* q, const void* k, const void* v, void* out,
                            const AttnDesc& d);
 // logits[b,i,j] = clip(scale * logits, +-1e4) - mask  (in place, row-major [B,Tq,Tv])

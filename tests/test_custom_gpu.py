@@ -387,7 +387,9 @@ def test_layer_norm_channels_first_and_views(ex, oracle):
 @pytest.mark.parametrize("dtype,tol", [(FLOAT32, 1e-4), (HALF, 1e-2), (BFLOAT16, 1e-2)])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("B,Tq,Tv,D", [(3, 64, 64, 64), (2, 100, 100, 64), (2, 128, 256, 64), (1, 37, 91, 32), (2, 300, 72, 64), (1, 520, 200, 64),
-                                      (2, 200, 200, 128), (1, 70, 330, 128), (2, 3, 200, 128)])
+                                      (2, 200, 200, 128), (1, 70, 330, 128), (2, 3, 200, 128),
+                                      # a few queries against a long history: the streaming kernel cuts the key range into parts and merges them
+                                      (12, 1, 640, 64), (1, 1, 1000, 128), (2, 1, 300, 64), (5, 4, 513, 64)])
 def test_attention_vs_oracle(ex, oracle, dtype, tol, causal, B, Tq, Tv, D):
     # causal with Tq != Tv: key j is visible to query i iff j <= i (the lower-triangular mask of AttentionHelper.cpp:70-79)
     rng = np.random.default_rng(B * Tq + D)
@@ -417,6 +419,25 @@ def test_attention_vs_oracle(ex, oracle, dtype, tol, causal, B, Tq, Tv, D):
         p64 = np.exp(sc64 - sc64.max(-1, keepdims=True))
         truth = np.einsum("bqk,bkd->bqd", p64 / p64.sum(-1, keepdims=True), v64)
         assert np.abs(out1.to_float() - truth).max() <= 1.25 * np.abs(_f(oo) - truth).max() + 1e-3, "fused kernel against the exact result"
+
+
+@pytest.mark.parametrize("dtype,tol", [(FLOAT32, 1e-4), (HALF, 1e-2), (BFLOAT16, 1e-2)])
+@pytest.mark.parametrize("H,Tv,D", [(12, 640, 64), (12, 257, 64), (3, 2000, 128), (24, 513, 64), (1, 1100, 64)])
+def test_attention_of_one_token_over_a_cut_up_history(ex, oracle, dtype, tol, H, Tv, D):
+    """One query token, its heads as the inner batch level ([1, H, 1, D] against [1, H, Tv, D]): the streaming kernel cuts the
+    key range into 2, 4 or 8 parts, a block each, and a second kernel merges the parts' records."""
+    rng = np.random.default_rng(H * Tv + D)
+    q, k, v = rng.normal(0, 1, (H, 1, D)), rng.normal(0, 1, (H, Tv, D)), rng.normal(0, 1, (H, Tv, D))
+    oq, dq = _pair(oracle, q, dtype)
+    ok, dk = _pair(oracle, k, dtype)
+    ov, dv = _pair(oracle, v, dtype)
+    oo = _ozeros(oracle, (H, 1, D), dtype)
+    scale = 1 / math.sqrt(D)
+    oracle.attention_v2(oq, ov, ok, oo, None, None, scale=scale, causal=False)
+    q4, k4, v4 = dq.reshape(1, H, 1, D), dk.reshape(1, H, Tv, D), dv.reshape(1, H, Tv, D)
+    out = ex.exec_custom("dot_product_attention_v2", [q4, v4, k4], [NDArray.empty((1, H, 1, D), dtype)], t_args=[scale, 0.0], b_args=[False, False])[0]
+    wide = 2.5 if (D == 128 and dtype == BFLOAT16) else 1.0
+    assert_close(out.to_float().reshape(H, 1, D), _f(oo), wide * tol, wide * tol, "one token, %d heads, %d keys" % (H, Tv))
 
 
 @pytest.mark.parametrize("dtype,tol", [(HALF, 1e-2), (BFLOAT16, 1e-2)])

@@ -85,3 +85,61 @@ def test_add_layer_norm_product_chain_on_few_rows(ex, dt, rows, k, n1, n2):
     ln = want[2]
     lnf = bf16_bits_to_f32(ln) if dt == BFLOAT16 else ln.view(np.float16).astype(np.float32)
     assert np.isfinite(lnf).all() and 0.5 < lnf.std() < 2.0
+
+
+@pytest.mark.parametrize("dt", [BFLOAT16, HALF])
+@pytest.mark.parametrize("heads,dh,tv", [(12, 64, 640), (6, 128, 900)])
+def test_one_token_attention_merges_inside_the_projection(ex, dt, heads, dh, tv):
+    """att = attention(q [1, H, 1, D]; cache [1, H, Tv, D]);  p = att W' + b;  h += p.  The attention cuts its key range into
+    four parts; recorded, the projection merges the parts on its way in (no merge launch) and still writes `att`."""
+    L = ex.L
+    rng = np.random.default_rng(heads * tv)
+    d = heads * dh
+    q, k, v = rng.normal(0, 1, (1, heads, 1, dh)), rng.normal(0, 1, (1, heads, tv, dh)), rng.normal(0, 1, (1, heads, tv, dh))
+    w, b, h = rng.normal(0, d ** -0.5, (d, d)), rng.normal(0, 0.1, d), rng.normal(0, 1, (1, d))
+    Q, K, V, W, B = (_arr(a, dt) for a in (q, k, v, w, b))
+    scale = dh ** -0.5
+
+    def run(record):
+        H = _arr(h, dt)
+        Att, P = NDArray.empty((1, d), dt), NDArray.empty((1, d), dt)
+        for arr in (Q, K, V, W, B, H):
+            arr.sync_to_device()
+        for arr in (Att, P):
+            L.dbAllocateSpecialBuffer(arr.buffer.ptr)
+        att4 = Att.view((1, heads, 1, dh), (d, dh, dh, 1))
+        calls = [ex.bind_custom("dot_product_attention_v2", [Q, V, K], [att4], t_args=[scale, 0.0], b_args=[False, False]),
+                 ex.bind_custom("xw_plus_b", [Att, W, B], [P], i_args=[0, 1]),
+                 lambda: (L.execPairwiseTransform(None, Pairwise.Add, H.handle, P.handle, H.handle, None), N.check("execPairwiseTransform"))]
+        if not record:
+            for c in calls:
+                c()
+            return [[_bits(x).copy() for x in (Att, P, H)]], ""
+        assert L.nd4jhipGraphBeginCapture() == 0, L.lastErrorMessage()
+        for c in calls:
+            c()
+        g = L.nd4jhipGraphEndCapture()
+        N.check("nd4jhipGraphEndCapture")
+        assert g and L.nd4jhipGraphFusedOps(g) == 1 and L.nd4jhipGraphFusedApplied(g) == 1     # the Add rides in the projection
+        assert L.nd4jhipGraphAudit(g) == 0, L.lastErrorMessage()
+        outs, kern = [], ""
+        try:
+            for mode in (1, 0):
+                L.nd4jhipSetGraphReplayMode(mode)
+                H.assign_numpy(_arr(h, dt).to_numpy())
+                Att.assign_numpy(np.zeros((1, d), np.uint16 if dt == BFLOAT16 else np.float16))
+                assert L.nd4jhipGraphLaunch(g) == 0, L.lastErrorMessage()
+                if mode == 1:
+                    kern = L.nd4jhipLastGemmKernel().decode()
+                outs.append([_bits(x).copy() for x in (Att, P, H)])
+        finally:
+            L.nd4jhipSetGraphReplayMode(0)
+            L.nd4jhipGraphDestroy(g)
+        return outs, kern
+
+    (want,), _ = run(False)
+    got, kern = run(True)
+    assert "attn-merge" in kern, kern
+    for outs in got:
+        for name, g_, w_ in zip(("att", "p", "h"), outs, want):
+            assert np.array_equal(g_, w_), (name, int((g_ != w_).sum()))
