@@ -43,7 +43,9 @@ TRAFFIC_MB = {
     "mmul f32 1024": 29.5, "mmul f16 1024": 14.8, "mmul bf16 1024": 14.8,
     "copy fp32": 268.4, "pairwise_add fp32": 402.6, "transform_tanh fp32": 268.4, "reduce_sum": 134.5, "argmax dim1": 134.5,
     "layer_norm fp32": 100.8, "gelu fp32": 100.7, "softmax fp32": 1610.6, "layer_norm bf16": 50.4, "gelu bf16": 50.4,
-    "softmax bf16": 805.3, "dot_product_attention_v2": 50.5,
+    "softmax bf16": 805.3, "dot_product_attention_v2": 50.5, "dot_product_attention_v2 f32": 140.5,
+    "reduce_cols": 101.0, "index_cols": 101.2, "transpose_tiled": 201.2, "cast_contig": 150.9, "softmax_block_regs": 203.3,
+    "mmul unaligned": 1223.4,
 }
 
 
@@ -505,16 +507,16 @@ def main():
                 arr.sync_to_device()
             Rc = [NDArray.empty((rc_shape[1],), FLOAT32) for _ in range(Kx)]
             Ic = [NDArray.empty((rc_shape[1],), INT64) for _ in range(Kx)]
-            hbm_line("reduce_sum dim0 fp32 [6144,4096] (column sums: reduce_cols)", "", 4 * xc.size + 4 * rc_shape[1],
+            hbm_line("reduce_sum dim0 fp32 [6144,4096] (column sums: reduce_cols)", "reduce_cols", 4 * xc.size + 4 * rc_shape[1],
                      lambda i: (lambda: ex.exec_reduce_same(ReduceSame.Sum, Xc[i], [0], z=Rc[i])))
-            hbm_line("argmax dim0 fp32 [6144,4096] (index_cols)", "", 4 * xc.size + 8 * rc_shape[1],
+            hbm_line("argmax dim0 fp32 [6144,4096] (index_cols)", "index_cols", 4 * xc.size + 8 * rc_shape[1],
                      lambda i: (lambda: ex.exec_index_reduce(IndexReduce.IndexMax, Xc[i], [0], z=Ic[i])))
             Tc = [NDArray.empty((rc_shape[1], rc_shape[0]), FLOAT32) for _ in range(3)]
             Xt = [x_.permute(1, 0) for x_ in Xc]
-            hbm_line("assign of a transposed view fp32 [6144,4096] -> [4096,6144] (transpose_tiled)", "", 2 * 4 * xc.size,
+            hbm_line("assign of a transposed view fp32 [6144,4096] -> [4096,6144] (transpose_tiled)", "transpose_tiled", 2 * 4 * xc.size,
                      lambda i: (lambda: ex.exec_assign(Xt[i], Tc[i % 3])))
             Bc = [NDArray.empty(rc_shape, BFLOAT16) for _ in range(3)]
-            hbm_line("cast fp32 -> bf16 [6144,4096] (cast_contig)", "", 6 * xc.size,
+            hbm_line("cast fp32 -> bf16 [6144,4096] (cast_contig)", "cast_contig", 6 * xc.size,
                      lambda i: (lambda: ex.exec_assign(Xc[i], Bc[i % 3])))
             del Xc, Xt, Rc, Ic, Tc, Bc, xc
             lv = rng.normal(0, 2, (500, 50257)).astype(np.float32)
@@ -524,7 +526,7 @@ def main():
                 arr.sync_to_device()
             Zl = [NDArray.empty(lv.shape, FLOAT32) for _ in range(3)]
             sm_binds = [ex.bind_custom("softmax", [Lv[i]], [Zl[i % 3]], i_args=[1]) for i in range(Kl)]
-            hbm_line("softmax fp32 [500,50257] (vocabulary-length rows: softmax_long_vec)", "", 2 * 4 * lv.size, lambda i: sm_binds[i])
+            hbm_line("softmax fp32 [500,50257] (vocabulary-length rows: softmax_block_regs)", "softmax_block_regs", 2 * 4 * lv.size, lambda i: sm_binds[i])
             del Lv, Zl, sm_binds, lv
             # a product against a row-major matrix whose rows do not start on 16-byte boundaries (the [768, 50257] embedding
             # without the transpose flag): element-aligned vector loads in the bounds-handling tile kernel
@@ -534,7 +536,7 @@ def main():
             Ua.sync_to_device(); Ue.sync_to_device()
             w, e = timed(ex, L, ex.bind_custom("matmul", [Ua, Ue], [Uz]), max(steps // 5, 3), max(warmup // 5, 1))
             ops.append({"op": "mmul bf16 [4096,768] x [768,50257] (row length not a multiple of 8: %s)" % L.nd4jhipLastGemmKernel().decode(),
-                        "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": mfma_entry(2.0 * 4096 * 50257 * 768, e, "bf16", "")})
+                        "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": mfma_entry(2.0 * 4096 * 50257 * 768, e, "bf16", "mmul unaligned")})
             del Ua, Ue, Uz, ua, ue
         if 2 in cfgs:
             # config 2, the remaining sizes/dtypes
@@ -598,7 +600,7 @@ def main():
                 # what the kernel executes: a block owns 128 queries and walks the 64-key tiles up to its last query's diagonal
                 executed_flops = 96 * sum(4.0 * 64 * 128 * min(1024, 64 * math.ceil(128 * (blk + 1) / 64)) for blk in range(8))
                 useful_flops = 4.0 * 96 * 64 * (1024 * 1025 / 2)       # the scores on and below the diagonal
-                rf = mfma_entry(dense_flops, e, dtn, "dot_product_attention_v2")
+                rf = mfma_entry(dense_flops, e, dtn, "dot_product_attention_v2 f32" if dt == FLOAT32 else "dot_product_attention_v2")
                 rf["achieved_executed"] = round(executed_flops / (e * 1e-3) / 1e12, 2)
                 rf["frac_executed"] = round(rf["achieved_executed"] / MFMA_PEAK[dtn], 4)
                 rf["achieved_causal_useful"] = round(useful_flops / (e * 1e-3) / 1e12, 2)
