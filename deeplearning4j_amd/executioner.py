@@ -401,7 +401,7 @@ class Executioner:
     def exec_custom(self, name, inputs, outputs=None, t_args=(), i_args=(), b_args=(), d_args=(), n_outputs=None):
         """Returns the list of output arrays.  `outputs=None` sizes them with calculateOutputShapes2;
         `n_outputs` limits how many of the reported outputs are materialised."""
-        from .ndarray import DT_FLAG
+        from .ndarray import dtype_of_extra
         if outputs is None:
             shapes = self.calculate_output_shapes(name, inputs, t_args, i_args, b_args, d_args)
             if n_outputs is not None:
@@ -410,7 +410,7 @@ class Executioner:
             for si in shapes:
                 rank = int(si[0])
                 extra = int(si[3] if rank == 0 else si[2 * rank + 1])
-                dt = [k for k, v in DT_FLAG.items() if extra & v][0]
+                dt = dtype_of_extra(extra)
                 order = chr(int(si[-1]))
                 outputs.append(NDArray.empty([int(s) for s in si[1:1 + rank]], dt, order))
         ctx = OpContext()

@@ -12,12 +12,30 @@ import numpy as np
 from . import nativeops as N
 
 BOOL, HALF, FLOAT32, DOUBLE, INT32, INT64, BFLOAT16 = 1, 3, 5, 6, 9, 10, 17
-DT_SIZE = {BOOL: 1, HALF: 2, FLOAT32: 4, DOUBLE: 8, INT32: 4, INT64: 8, BFLOAT16: 2}
-DT_FLAG = {HALF: 4096, BFLOAT16: 2048, FLOAT32: 8192, DOUBLE: 16384, INT32: 131072, INT64: 262144, BOOL: 524288}
+INT8, INT16, UINT8, UINT16, UINT32, UINT64 = 7, 8, 11, 12, 13, 14          # array/DataType.h:27-50
+DT_SIZE = {BOOL: 1, HALF: 2, FLOAT32: 4, DOUBLE: 8, INT32: 4, INT64: 8, BFLOAT16: 2, INT8: 1, INT16: 2, UINT8: 1, UINT16: 2, UINT32: 4, UINT64: 8}
+_UNSIGNED = 8388608                                                            # array/ArrayOptions.h: ARRAY_UNSIGNED
+DT_FLAG = {HALF: 4096, BFLOAT16: 2048, FLOAT32: 8192, DOUBLE: 16384, INT32: 131072, INT64: 262144, BOOL: 524288, INT8: 32768, INT16: 65536,
+           UINT8: 32768 | _UNSIGNED, UINT16: 65536 | _UNSIGNED, UINT32: 131072 | _UNSIGNED, UINT64: 262144 | _UNSIGNED}
 DT_NP = {BOOL: np.bool_, HALF: np.float16, FLOAT32: np.float32, DOUBLE: np.float64, INT32: np.int32, INT64: np.int64,
-         BFLOAT16: np.uint16}
+         BFLOAT16: np.uint16, INT8: np.int8, INT16: np.int16, UINT8: np.uint8, UINT16: np.uint16, UINT32: np.uint32, UINT64: np.uint64}
+# (a numpy uint16 array is taken as bf16 bit patterns only when BFLOAT16 is asked for; by itself it is UINT16)
 NP_DT = {np.dtype(np.bool_): BOOL, np.dtype(np.float16): HALF, np.dtype(np.float32): FLOAT32,
-         np.dtype(np.float64): DOUBLE, np.dtype(np.int32): INT32, np.dtype(np.int64): INT64}
+         np.dtype(np.float64): DOUBLE, np.dtype(np.int32): INT32, np.dtype(np.int64): INT64, np.dtype(np.int8): INT8,
+         np.dtype(np.int16): INT16, np.dtype(np.uint8): UINT8, np.dtype(np.uint16): UINT16, np.dtype(np.uint32): UINT32,
+         np.dtype(np.uint64): UINT64}
+
+
+def dtype_of_extra(extra):
+    """The data type a shape descriptor's extra word names (array/ArrayOptions.hXX, dataType(): the sign bit picks the
+    unsigned twin of an integer type)."""
+    type_bits = 0
+    for v in DT_FLAG.values():
+        type_bits |= v
+    for k, v in DT_FLAG.items():
+        if extra & type_bits == v:
+            return k
+    raise ValueError("shape descriptor names no data type: extra = %d" % extra)
 
 
 def f32_to_bf16_bits(a):

@@ -8,7 +8,7 @@ import pytest
 
 from deeplearning4j_amd.executioner import Broadcast, IndexReduce, Pairwise, ReduceSame, Scalar, TransformBool, TransformSame
 from deeplearning4j_amd.nativeops import NativeOpsError
-from deeplearning4j_amd.ndarray import BOOL, FLOAT32, INT32, INT64, NDArray
+from deeplearning4j_amd.ndarray import BOOL, FLOAT32, INT8, INT16, INT32, INT64, UINT8, UINT16, UINT32, UINT64, NDArray
 
 pytestmark = pytest.mark.gpu
 
@@ -135,6 +135,114 @@ def test_index_reduce_int_first_extreme_wins(ex, dt):
     assert ex.exec_index_reduce(IndexReduce.IndexMin, Bg, None).to_numpy() == big.argmin()
     z32 = ex.exec_index_reduce(IndexReduce.IndexMax, A, [1], z=NDArray.empty((64,), INT32)).to_numpy()
     assert z32.dtype == np.int32 and np.array_equal(z32, a.argmax(1))
+
+
+def _u64(rng, shape):
+    """Half of the values at 2^63 and above, where a signed reading of the same bits is negative."""
+    a = rng.integers(0, 1 << 63, shape, dtype=np.uint64)
+    a[rng.random(shape) < 0.5] |= np.uint64(1 << 63)
+    a.flat[:4] = [np.uint64(1 << 63), np.uint64((1 << 64) - 1), np.uint64((1 << 63) + 1), np.uint64(0)]
+    return a
+
+
+def test_uint64_wraps_where_the_sign_does_not_matter(ex):
+    """UINT64 operands travel through 64-bit two's-complement arithmetic: sums, differences, products and bit ops are the
+    unsigned results modulo 2^64, also for values of 2^63 and above."""
+    rng = np.random.default_rng(64)
+    a, b = _u64(rng, (129, 257)), _u64(rng, (129, 257))
+    A, B = NDArray.from_numpy(a), NDArray.from_numpy(b)
+    assert A.dtype == UINT64
+    with np.errstate(over="ignore"):
+        for op, fn in ((Pairwise.Add, lambda u, v: u + v), (Pairwise.Subtract, lambda u, v: u - v), (Pairwise.Multiply, lambda u, v: u * v),
+                       (Pairwise.ReverseSubtract, lambda u, v: v - u), (Pairwise.SquaredSubtract, lambda u, v: (u - v) * (u - v)),
+                       (Pairwise.CopyPws, lambda u, v: v), (Pairwise.LogicalAnd, lambda u, v: u & v), (Pairwise.LogicalOr, lambda u, v: u | v),
+                       (Pairwise.LogicalXor, lambda u, v: u ^ v)):
+            z = ex.exec_pairwise(op, A, B).to_numpy()
+            assert z.dtype == np.uint64 and np.array_equal(z, fn(a, b)), op
+        # strided operands and a narrower unsigned y, which is read without sign extension
+        At = NDArray.from_numpy(np.ascontiguousarray(a.T)).permute(1, 0)
+        y32 = rng.integers(1 << 31, 1 << 32, a.shape, dtype=np.uint32)
+        z = ex.exec_pairwise(Pairwise.Add, At, NDArray.from_numpy(y32), NDArray.empty(a.shape, UINT64)).to_numpy()
+        assert np.array_equal(z, a + y32.astype(np.uint64))
+        for op, fn in ((TransformSame.Neg, lambda u: np.uint64(0) - u), (TransformSame.Square, lambda u: u * u), (TransformSame.Cube, lambda u: u * u * u),
+                       (TransformSame.OneMinus, lambda u: np.uint64(1) - u), (TransformSame.Identity, lambda u: u), (TransformSame.Ones, np.ones_like)):
+            assert np.array_equal(ex.exec_transform_same(op, A).to_numpy(), fn(a)), op
+        assert np.array_equal(ex.exec_transform_bool(TransformBool.Not, A).to_numpy(), a == 0)
+        for dims in ([1], [0], None):
+            ax = None if dims is None else tuple(dims)
+            assert np.array_equal(ex.exec_reduce_same(ReduceSame.Sum, A, dims).to_numpy(), a.sum(ax, dtype=np.uint64))
+            assert np.array_equal(ex.exec_reduce_same(ReduceSame.Prod, A, dims).to_numpy(), a.prod(ax, dtype=np.uint64))
+        big = _u64(rng, (3_000_017,))        # split over many blocks
+        assert ex.exec_reduce_same(ReduceSame.Sum, NDArray.from_numpy(big), None).to_numpy() == big.sum(dtype=np.uint64)
+    Z = NDArray.empty((257, 129), UINT64)
+    ex.exec_assign(A, Z.permute(1, 0))
+    assert np.array_equal(Z.to_numpy(), a.T)
+
+
+def test_uint64_is_refused_where_a_signed_reading_would_be_wrong(ex):
+    """Ordering, division, remainders, absolute values and scalar operands would treat 2^63 and above as negative numbers: the
+    library raises instead, and leaves z as it was."""
+    rng = np.random.default_rng(65)
+    a, b = _u64(rng, (40, 33)), _u64(rng, (40, 33))
+    b[b == 0] = 3
+    A, B = NDArray.from_numpy(a), NDArray.from_numpy(b)
+    for op in (Pairwise.Divide, Pairwise.FloorDiv, Pairwise.FloorMod, Pairwise.Mod, Pairwise.MaxPairwise, Pairwise.MinPairwise, Pairwise.TruncateDiv,
+               Pairwise.AMaxPairwise, Pairwise.ReverseDivide):
+        Z = NDArray.from_numpy(np.full(a.shape, 7, np.uint64))
+        with pytest.raises(NativeOpsError):
+            ex.exec_pairwise(op, A, B, Z)
+        assert np.array_equal(Z.to_numpy(), np.full(a.shape, 7, np.uint64)), op
+    for op in (Scalar.Add, Scalar.Multiply, Scalar.MaxPairwise, Scalar.Divide):
+        with pytest.raises(NativeOpsError):
+            ex.exec_scalar(op, A, NDArray.from_numpy(np.array(1 << 63, np.uint64)))
+    for op in (TransformSame.Abs, TransformSame.Reciprocal):
+        with pytest.raises(NativeOpsError):
+            ex.exec_transform_same(op, A)
+    for op in (TransformBool.IsPositive, TransformBool.IsNegative):
+        with pytest.raises(NativeOpsError):
+            ex.exec_transform_bool(op, A)
+    for op in (ReduceSame.Max, ReduceSame.Min, ReduceSame.ASum, ReduceSame.AMax, ReduceSame.AMin):
+        with pytest.raises(NativeOpsError):
+            ex.exec_reduce_same(op, A, [1])
+        with pytest.raises(NativeOpsError):
+            ex.exec_reduce_same(op, A, None)
+    for op in (IndexReduce.IndexMax, IndexReduce.IndexMin, IndexReduce.IndexAbsoluteMax):
+        with pytest.raises(NativeOpsError):
+            ex.exec_index_reduce(op, A, [1])
+    # the library still works afterwards
+    with np.errstate(over="ignore"):
+        assert np.array_equal(ex.exec_pairwise(Pairwise.Add, A, B).to_numpy(), a + b)
+
+
+@pytest.mark.parametrize("dt,npdt", [(INT8, np.int8), (UINT8, np.uint8), (INT16, np.int16), (UINT16, np.uint16), (UINT32, np.uint32)])
+def test_narrow_and_unsigned_integer_types(ex, dt, npdt):
+    """The narrow types are widened to 64 bits on the way in (with or without sign, as the type says) and cut back on the way
+    out, so that every op, ordering and division included, sees the values the type holds."""
+    rng = np.random.default_rng(70 + dt)
+    info = np.iinfo(npdt)
+    a = rng.integers(info.min, info.max, (130, 67), dtype=npdt, endpoint=True)
+    b = rng.integers(info.min, info.max, (130, 67), dtype=npdt, endpoint=True)
+    a.flat[:2] = [info.max, info.min]
+    b.flat[:2] = [info.max, info.max]
+    bd = b.copy()
+    bd[bd == 0] = 5
+    A, B, Bd = NDArray.from_numpy(a), NDArray.from_numpy(b), NDArray.from_numpy(bd)
+    assert A.dtype == dt
+    wide = lambda v: v.astype(np.int64)
+    with np.errstate(over="ignore"):
+        for op, want in ((Pairwise.Add, (wide(a) + wide(b)).astype(npdt)), (Pairwise.Multiply, (wide(a) * wide(b)).astype(npdt)),
+                         (Pairwise.Subtract, (wide(a) - wide(b)).astype(npdt)), (Pairwise.MaxPairwise, np.maximum(a, b)),
+                         (Pairwise.MinPairwise, np.minimum(a, b))):
+            z = ex.exec_pairwise(op, A, B).to_numpy()
+            assert z.dtype == npdt and np.array_equal(z, want), op
+        assert np.array_equal(ex.exec_pairwise(Pairwise.Divide, A, Bd).to_numpy(), _trunc_div(wide(a), wide(bd)).astype(npdt))
+        assert np.array_equal(ex.exec_pairwise(Pairwise.FloorMod, A, Bd).to_numpy(), np.mod(wide(a), wide(bd)).astype(npdt))
+        assert np.array_equal(ex.exec_reduce_same(ReduceSame.Sum, A, [1]).to_numpy(), wide(a).sum(1).astype(npdt))
+        assert np.array_equal(ex.exec_reduce_same(ReduceSame.Max, A, [0]).to_numpy(), a.max(0))
+        assert np.array_equal(ex.exec_reduce_same(ReduceSame.Min, A, None).to_numpy(), a.min())
+    assert np.array_equal(ex.exec_index_reduce(IndexReduce.IndexMax, A, [1]).to_numpy(), a.argmax(1))
+    assert np.array_equal(ex.exec_index_reduce(IndexReduce.IndexMin, A, [0]).to_numpy(), a.argmin(0))
+    assert np.array_equal(ex.exec_scalar(Scalar.Add, A, 3).to_numpy(), (wide(a) + 3).astype(npdt))
 
 
 def test_custom_ops_on_integer_arrays(ex):
