@@ -19,7 +19,10 @@
 //   logits fix-up - in-place pass over dense [B, Tq, Tv] logits for the composition path that writes the
 //                   logits / weights outputs: optional scale, clip to +-1e4, causal penalty.
 #include <algorithm>
+#include <array>
 #include <cmath>
+#include <map>
+#include <memory>
 #include <mutex>
 #include <type_traits>
 
@@ -100,6 +103,12 @@ struct FusedArgs {
   int splits = 1;                             // decode kernel: key ranges per (batch entry, query), blockIdx.z picks one
   float* partial = nullptr;                   // ... and where a range's partial result goes (null: the block writes the output)
 };
+// Fused kernels, block order 2: block id -> work item (query tile x batch entry, heavy tiles first), a table made on the
+// host and passed by value.  Used when every block of the launch is on the chip at once: block ids i, i + 256, i + 512
+// then share a CU (the hardware deals consecutive ids out CU after CU and comes round again), and the table gives every
+// CU about the same number of key tiles.
+constexpr int BLOCK_ORDER_MAX = 768;
+struct BlockOrder { unsigned short item[BLOCK_ORDER_MAX]; };
 
 template <typename T> __device__ __forceinline__ float round_storage(float v) { return to_float(Conv<T>::from(v)); }
 // round two values through the storage type in place
@@ -126,7 +135,7 @@ template <typename T> __device__ __forceinline__ unsigned pack2(float a, float b
 // tile is skipped: a query whose visible keys are all padded spreads its weight over every key, as the reference's
 // softmax over equally penalised logits does.
 template <typename T, int D, bool FOLD, bool VM>
-__global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
+__global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, BlockOrder ord, const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
                                                   T* __restrict__ O) {
   constexpr int BQ = 128, BKV = 64, NT = 256;
   constexpr int DG = D / 8;                      // 16-byte groups along d
@@ -150,8 +159,9 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
   int slot;
   LongType b;
   if (a.heavyFirst) {
-    slot = (int)(blockIdx.x / (unsigned)a.nBatch);
-    b = blockIdx.x % (unsigned)a.nBatch;
+    const unsigned item = a.heavyFirst == 2 ? ord.item[blockIdx.x] : blockIdx.x;   // 2: the host's table (see BlockOrder)
+    slot = (int)(item / (unsigned)a.nBatch);
+    b = item % (unsigned)a.nBatch;
   } else {
     const unsigned total = gridDim.x, xcd = blockIdx.x & 7u, idx = blockIdx.x >> 3, per = total >> 3, rem = total & 7u;
     const unsigned item = xcd * per + (xcd < rem ? xcd : rem) + idx;
@@ -741,7 +751,7 @@ void launchAttentionDecode(hipStream_t s, DataType dt, const void* q, const void
 // Scores are scale * q.k clipped to +-1e4 (AttentionHelper.cpp:340-352); masked and out-of-range keys weigh exactly 0
 // (the reference's clamped softmax gives them e^-88 / sum).  No value mask here: such calls take the composition.
 template <int D>
-__global__ __launch_bounds__(256, D == 64 ? 3 : 1) void attn_fused_f32(FusedArgs a, const float* __restrict__ Q, const float* __restrict__ K, const float* __restrict__ V,
+__global__ __launch_bounds__(256, D == 64 ? 3 : 1) void attn_fused_f32(FusedArgs a, BlockOrder ord, const float* __restrict__ Q, const float* __restrict__ K, const float* __restrict__ V,
                                                       float* __restrict__ O) {
   constexpr int BQ = 128, BKV = 32, HD = D / 2, PITCH = D + 4;   // row pitch in floats: 16 consecutive rows start in different banks
   constexpr int DT = D / 32;                                     // dv tiles of the output accumulator
@@ -753,7 +763,8 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 1) void attn_fused_f32(FusedArgs
   // share a CU and the hardware deals consecutive block ids out CU after CU, so rounds of 256 block ids walk the item
   // list alternately forwards and backwards: the CU that got the heaviest item of one round gets the lightest of the next.
   unsigned item = blockIdx.x;
-  {
+  if (a.heavyFirst == 2) item = ord.item[blockIdx.x];   // the host's table (see BlockOrder)
+  else {
     const unsigned round = blockIdx.x >> 8, first = round << 8;
     const unsigned last = first + 255u < gridDim.x ? first + 255u : gridDim.x - 1u;
     if (round & 1u) item = last - (blockIdx.x - first);
@@ -897,6 +908,49 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 1) void attn_fused_f32(FusedArgs
       }
   }
 }
+// The table of block order 2 for `nBatch` batch entries x `qTiles` query tiles under the causal mask, or null when the
+// launch does not fit on the chip at once (`resident` blocks per CU) or in the table.  Items (heaviest query tile first)
+// go one by one to the CU with the fewest key tiles so far that still has a block id left; with a multiple of 8 batch
+// entries a batch entry stays on one XCD (block id mod 8), whose L2 then holds its K and V once.
+static const BlockOrder* balancedBlockOrder(int nBatch, int qTiles, int keyTilesPerQueryTile, int resident) {
+  const long total = (long)nBatch * qTiles;
+  if (total > BLOCK_ORDER_MAX || total > 256L * resident || total <= 256 || qTiles < 2) return nullptr;
+  static std::mutex mu;
+  static std::map<std::array<int, 3>, std::unique_ptr<BlockOrder>> cache;
+  std::lock_guard<std::mutex> lock(mu);
+  auto& entry = cache[{nBatch, qTiles, keyTilesPerQueryTile}];
+  if (entry) return entry.get();
+  for (int attempt = 0; attempt < 2; attempt++) {
+    const bool byXcd = attempt == 0 && nBatch % 8 == 0;
+    if (attempt == 0 && !byXcd) continue;
+    auto t = std::make_unique<BlockOrder>();
+    int cap[256], cnt[256] = {0};
+    long load[256] = {0};
+    for (int c = 0; c < 256; c++) cap[c] = c < total ? (int)((total - c + 255) / 256) : 0;
+    bool ok = true;
+    for (long p = 0; p < total && ok; p++) {
+      const int slot = (int)(p / nBatch), b = (int)(p % nBatch);
+      const long w = (long)keyTilesPerQueryTile * (qTiles - slot) + 1;   // key tiles of the query tile + the block's start-up
+      int best = -1;
+      for (int c = 0; c < 256; c++)
+        if (cnt[c] < cap[c] && (!byXcd || (c & 7) == (b & 7)) && (best < 0 || load[c] < load[best])) best = c;
+      if (best < 0) { ok = false; break; }
+      t->item[cnt[best] * 256 + best] = (unsigned short)p;
+      cnt[best]++; load[best] += w;
+    }
+    if (ok) { entry = std::move(t); return entry.get(); }
+  }
+  return nullptr;
+}
+static const BlockOrder& noBlockOrder() { static const BlockOrder z{}; return z; }
+// blocks of `kern` a CU holds at once
+template <typename K>
+static int residentBlocks(K kern, int ldsBytes) {
+  int n = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, 256, (size_t)ldsBytes) != hipSuccess) { (void)hipGetLastError(); return 0; }
+  return n;
+}
+
 template <int D>
 static void launchFusedF32(hipStream_t s, const void* q, const void* k, const void* v, void* out, const AttnDesc& d) {
   FusedArgs a;
@@ -908,7 +962,11 @@ static void launchFusedF32(hipStream_t s, const void* q, const void* k, const vo
   a.vmask = nullptr; a.maskValue = d.maskValue;
   constexpr int LDS = 2 * 2 * 32 * (D + 4) * 4;
   ND4J_REQUIRE((DynLds<attn_fused_f32<D>, LDS>::granted()), "attention: the device does not grant the fp32 fused kernel its LDS");
-  hipLaunchKernelGGL((attn_fused_f32<D>), dim3((unsigned)((LongType)a.qTiles * d.B)), dim3(256), LDS, s, a, (const float*)q, (const float*)k, (const float*)v, (float*)out);
+  static const int resident = residentBlocks(attn_fused_f32<D>, LDS);
+  const BlockOrder* ord = d.causal && d.B * a.qTiles <= BLOCK_ORDER_MAX ? balancedBlockOrder((int)d.B, a.qTiles, 4, resident) : nullptr;
+  if (ord) a.heavyFirst = 2;
+  hipLaunchKernelGGL((attn_fused_f32<D>), dim3((unsigned)((LongType)a.qTiles * d.B)), dim3(256), LDS, s, a, ord ? *ord : noBlockOrder(), (const float*)q, (const float*)k,
+                     (const float*)v, (float*)out);
 }
 
 bool attentionFusedSupported(DataType dt, const AttnDesc& d) {
@@ -954,7 +1012,14 @@ static void launchFusedTyped(hipStream_t s, const void* q, const void* k, const 
   constexpr size_t LDS = (size_t)2 * ((D / 64) * 512 + 64 * (D / 8)) * 16;   // two stages of (K tile, V tile)
   auto kern = attn_fused<T, D, FOLD, VM>;
   ND4J_REQUIRE((DynLds<attn_fused<T, D, FOLD, VM>, (int)LDS>::granted()), "attention: the device does not grant the fused kernel its LDS");
-  hipLaunchKernelGGL(kern, dim3((unsigned)((LongType)(a.heavyFirst ? a.qTiles : a.perBatch) * d.B)), dim3(256), LDS, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
+  const BlockOrder* ord = nullptr;
+  if (d.causal && !VM && a.qTiles > 1 && d.B * a.qTiles <= BLOCK_ORDER_MAX) {
+    static const int resident = residentBlocks(kern, (int)LDS);
+    ord = balancedBlockOrder((int)d.B, a.qTiles, 2, resident);
+    if (ord) a.heavyFirst = 2;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)((LongType)(a.heavyFirst ? a.qTiles : a.perBatch) * d.B)), dim3(256), LDS, s, a, ord ? *ord : noBlockOrder(), (const T*)q, (const T*)k,
+                     (const T*)v, (T*)out);
 }
 
 void launchAttentionFused(hipStream_t s, DataType dt, const void* q, const void* k, const void* v, void* out, const AttnDesc& d) {

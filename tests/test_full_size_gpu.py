@@ -114,6 +114,31 @@ def test_config4_causal_attention(ex, oracle, dt):
         assert_close(out[bi:bi + 1], _as_float(oo), tol, tol, "batch entry %d" % bi)
 
 
+@pytest.mark.parametrize("dt", [BFLOAT16, FLOAT32])
+@pytest.mark.parametrize("B,T", [(40, 1024), (50, 768), (37, 1280), (72, 512), (264, 384)])
+def test_causal_attention_in_every_block_order(ex, oracle, dt, B, T):
+    """Launches whose blocks all fit on the chip at once take their query tiles in an order the host lays out (with a
+    multiple of 8 batch entries, and without), larger ones heavy tiles first, small ones in mirrored pairs: the same
+    results whichever applies.  Sampled batch entries against the oracle, and every row inside the hull of the value rows
+    it may see."""
+    tol = 1e-4 if dt == FLOAT32 else 1e-2
+    rng = np.random.default_rng(B * 10000 + T)
+    D = 64
+    q, Q = _store(rng.normal(0, 1, (B, T, D)).astype(np.float32), dt)
+    k, K = _store(rng.normal(0, 1, (B, T, D)).astype(np.float32), dt)
+    v, V = _store(rng.normal(0, 1, (B, T, D)).astype(np.float32), dt)
+    out = ex.exec_custom("dot_product_attention_v2", [Q, V, K], [NDArray.empty((B, T, D), dt)], t_args=[0.125, 0.0], b_args=[True, False])[0].to_float()
+    assert np.isfinite(out).all()
+    assert_close(out[:, 0], v[:, 0], tol, tol, "query 0")
+    vmax, vmin = np.maximum.accumulate(v, axis=1), np.minimum.accumulate(v, axis=1)
+    assert np.all(out <= vmax + 2 * tol) and np.all(out >= vmin - 2 * tol)
+    for bi in (0, B // 2 + 1, B - 1):
+        oo = _oracle_arr(oracle, np.zeros((1, T, D), np.float32), dt)
+        oracle.attention_v2(_oracle_arr(oracle, q[bi:bi + 1], dt), _oracle_arr(oracle, v[bi:bi + 1], dt), _oracle_arr(oracle, k[bi:bi + 1], dt), oo,
+                            scale=0.125, causal=True)
+        assert_close(out[bi:bi + 1], _as_float(oo), tol, tol, "batch entry %d" % bi)
+
+
 @pytest.mark.parametrize("dt", [HALF, BFLOAT16])
 def test_config4_weights_and_logits_outputs(ex, oracle, dt):
     """The same op with its second and third outputs requested (attention weights and clipped, masked logits) at the
