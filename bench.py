@@ -39,13 +39,13 @@ MFMA_PEAK = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}   # dense TFLOP/s
 # `--pmc WRITE_SIZE` (separate runs of this script) and scaled by what the same counters read for the plain copy
 # kernel; the summary of those runs sits under profiles/.  Static figures: they are not re-measured here.
 TRAFFIC_MB = {
-    "mmul bf16 4096": 235.2, "mmul f16 4096": 235.2, "mmul f32 4096^3": 859.1, "mmul f32 4096^3 transposeB": 866.0,
+    "mmul bf16 4096": 235.2, "mmul f16 4096": 235.2, "mmul f32 4096^3": 862.9, "mmul f32 4096^3 transposeB": 861.4,
     "mmul f32 1024": 29.5, "mmul f16 1024": 14.8, "mmul bf16 1024": 14.8,
     "copy fp32": 268.4, "pairwise_add fp32": 402.6, "transform_tanh fp32": 268.4, "reduce_sum": 134.5, "argmax dim1": 134.5,
     "layer_norm fp32": 100.8, "gelu fp32": 100.7, "softmax fp32": 1610.6, "layer_norm bf16": 50.4, "gelu bf16": 50.4,
-    "softmax bf16": 805.3, "dot_product_attention_v2": 50.5, "dot_product_attention_v2 f32": 140.5,
+    "softmax bf16": 805.3, "dot_product_attention_v2": 50.5, "dot_product_attention_v2 f32": 105.8,
     "reduce_cols": 101.0, "index_cols": 101.2, "transpose_tiled": 201.2, "cast_contig": 150.9, "softmax_block_regs": 203.3,
-    "mmul unaligned": 1223.4,
+    "mmul unaligned": 1223.8,
 }
 
 

@@ -916,9 +916,9 @@ static const BlockOrder* balancedBlockOrder(int nBatch, int qTiles, int keyTiles
   const long total = (long)nBatch * qTiles;
   if (total > BLOCK_ORDER_MAX || total > 256L * resident || total <= 256 || qTiles < 2) return nullptr;
   static std::mutex mu;
-  static std::map<std::array<int, 3>, std::unique_ptr<BlockOrder>> cache;
+  static std::map<std::array<int, 4>, std::unique_ptr<BlockOrder>> cache;
   std::lock_guard<std::mutex> lock(mu);
-  auto& entry = cache[{nBatch, qTiles, keyTilesPerQueryTile}];
+  auto& entry = cache[{nBatch, qTiles, keyTilesPerQueryTile, resident}];
   if (entry) return entry.get();
   for (int attempt = 0; attempt < 2; attempt++) {
     const bool byXcd = attempt == 0 && nBatch % 8 == 0;
@@ -943,6 +943,13 @@ static const BlockOrder* balancedBlockOrder(int nBatch, int qTiles, int keyTiles
   return nullptr;
 }
 static const BlockOrder& noBlockOrder() { static const BlockOrder z{}; return z; }
+int attentionBlockOrder(int nBatch, int qTiles, int keyTilesPerQueryTile, int resident, unsigned short* items) {
+  if (nBatch < 1 || qTiles < 1 || keyTilesPerQueryTile < 1 || resident < 1 || (long)nBatch * qTiles > BLOCK_ORDER_MAX) return 0;
+  const BlockOrder* t = balancedBlockOrder(nBatch, qTiles, keyTilesPerQueryTile, resident);
+  if (!t) return 0;
+  for (int i = 0; i < nBatch * qTiles; i++) items[i] = t->item[i];
+  return nBatch * qTiles;
+}
 // blocks of `kern` a CU holds at once
 template <typename K>
 static int residentBlocks(K kern, int ldsBytes) {

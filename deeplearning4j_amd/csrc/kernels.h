@@ -274,6 +274,8 @@ struct AttnDesc {
 int attentionDecodeSplits(const AttnDesc& d);
 // fused path (no logits/weights written)
 bool attentionFusedSupported(DataType dt, const AttnDesc& d);
+// the host-made block order of the fused attention kernels (see BlockOrder in attention.hip): fills items, returns their number or 0
+int attentionBlockOrder(int nBatch, int qTiles, int keyTilesPerQueryTile, int resident, unsigned short* items);
 void launchAttentionFused(hipStream_t s, DataType dt, const void* q, const void* k, const void* v, void* out,
                           const AttnDesc& d);
 // a few query rows against a long history, no causal mask (decode steps with a key/value cache)

@@ -1866,6 +1866,10 @@ void nd4jhipGraphDestroy(Nd4jPointer graph) {
   delete cg;
 }
 const char* nd4jhipLastGemmKernel(void) { return lastGemmKernel(); }
+int nd4jhipAttentionBlockOrder(int batchEntries, int queryTiles, int keyTilesPerQueryTile, int residentBlocksPerCu, unsigned short* items) {
+  if (items == nullptr) return 0;
+  return attentionBlockOrder(batchEntries, queryTiles, keyTilesPerQueryTile, residentBlocksPerCu, items);
+}
 
 // execReduceSame (full reduction of a dense array) for callers that cannot allocate: plain device pointers in, one
 // element out, partials in a fixed device array.  No hipMalloc / hipFree on any path, the error paths included.

@@ -183,6 +183,7 @@ _SIGS = {
     "nd4jhipGetGraphReplayMode": (ctypes.c_int, []),
     "nd4jhipBuildInfo": (ctypes.c_char_p, []),
     "nd4jhipLastGemmKernel": (ctypes.c_char_p, []),
+    "nd4jhipAttentionBlockOrder": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_ushort)]),
     "nd4jhipReduceSameScalarNoAlloc": (ctypes.c_int, [c_ptr, ctypes.c_int, ctypes.c_int, c_ptr, c_long, c_ptr]),
     "setGraphContextCudaContext": (None, [c_ptr, c_ptr, c_ptr, c_ptr]),
     "nd4jhipProfilerAttached": (ctypes.c_int, []),

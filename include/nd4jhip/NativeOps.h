@@ -331,6 +331,15 @@ ND4JHIP_EXPORT const char* nd4jhipBuildInfo(void);
 /* Name ("family<type,tile,flags>") of the kernel the calling thread's most recent matmul / xw_plus_b launched; lets a
  * test assert that its shape reached the instantiation it means to check. */
 ND4JHIP_EXPORT const char* nd4jhipLastGemmKernel(void);
+/* The order in which the fused attention kernels take the query tiles of a causal launch when all of its blocks are on
+ * the chip at once: items[blockId] = queryTileFromTheEnd * batchEntries + batchEntry, laid out on the host so that the
+ * block ids that share a CU (id mod 256) carry about the same number of key tiles and, with a multiple of 8 batch
+ * entries, a batch entry stays on one XCD (id mod 8).  Fills `items` (room for batchEntries * queryTiles values) and
+ * returns their number, or 0 when such a launch takes the plain heavy-first order instead (more blocks than
+ * 256 * residentBlocksPerCu or than the table holds, or at most one block per CU).  Pure host arithmetic: launches
+ * nothing and needs no device; lets a test check the layout the kernels are handed. */
+ND4JHIP_EXPORT int nd4jhipAttentionBlockOrder(int batchEntries, int queryTiles, int keyTilesPerQueryTile, int residentBlocksPerCu,
+                                              unsigned short* items);
 
 /* execReduceSame's full reduction for callers that cannot allocate.  No counterpart in the reference: it is for code
  * under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.  z[0] = reduce(x[0 .. length)) for

@@ -178,3 +178,35 @@ def test_profiler_detection_keeps_graph_launches_off_the_tracer():
         return subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=120).stdout.strip().splitlines()[-1]
     assert run({}) == "0"
     assert run({"ROCP_TOOL_LIBRARIES": "/opt/rocm/lib/rocprofiler-sdk/librocprofiler-sdk-tool.so"}) == "1"
+
+
+def test_attention_block_order_is_a_balanced_permutation():
+    """The host-side table that deals the query tiles of a causal attention launch out over the block ids: every item
+    once, the block ids that share a CU (id mod 256) within a few key tiles of each other, and with a multiple of 8 batch
+    entries every batch entry on one XCD (id mod 8)."""
+    import ctypes
+    L = N.load()
+    def order(nb, qt, per, resident):
+        buf = (ctypes.c_ushort * max(nb * qt, 1))()
+        n = L.nd4jhipAttentionBlockOrder(nb, qt, per, resident, buf)
+        return list(buf[:n])
+    for nb, qt, per, resident, by_xcd in ((96, 8, 2, 3, True), (96, 8, 4, 3, True), (40, 8, 2, 3, True), (50, 6, 2, 3, False), (37, 10, 2, 3, False),
+                                          (64, 8, 2, 2, True)):
+        items = order(nb, qt, per, resident)
+        total = nb * qt
+        assert sorted(items) == list(range(total)), (nb, qt)
+        load = [0] * 256
+        for block, item in enumerate(items):
+            slot, b = divmod(item, nb)
+            load[block % 256] += per * (qt - slot) + 1
+            if by_xcd:
+                assert block % 8 == b % 8, (nb, qt, block, item)
+        used = [v for v in load if v]
+        mean = sum(load) / 256.0
+        heaviest = per * qt + 1
+        # no CU more than one light tile above an even share (or above the heaviest single tile, when that is more)
+        assert max(load) <= max(mean, heaviest) + 2 * per + 2, (nb, qt, max(load), mean)
+        assert len(used) == min(total, 256)
+    # launches that are not on the chip at once, or have at most a block per CU, keep the plain order
+    assert order(96, 8, 2, 2) == [] and order(2, 8, 2, 3) == [] and order(200, 8, 2, 3) == [] and order(96, 1, 2, 3) == []
+
