@@ -124,6 +124,16 @@ template <> struct RawIO<f16_t> {
   }
 };
 
+// a 16-byte pack of elements of T on its way out through a non-temporal store, to an address that is only element-aligned
+typedef unsigned u32x4_align2 __attribute__((ext_vector_type(4), aligned(2)));
+typedef unsigned u32x4_align4 __attribute__((ext_vector_type(4), aligned(4)));
+template <typename T, typename P>
+__device__ __forceinline__ void nt_store16_elem_aligned(T* dst, const P& pack) {
+  static_assert(sizeof(P) == 16 && (sizeof(T) == 2 || sizeof(T) == 4), "16-byte packs of 2- or 4-byte elements");
+  if constexpr (sizeof(T) == 2) __builtin_nontemporal_store(__builtin_bit_cast(u32x4_align2, pack), reinterpret_cast<u32x4_align2*>(dst));
+  else __builtin_nontemporal_store(__builtin_bit_cast(u32x4_align4, pack), reinterpret_cast<u32x4_align4*>(dst));
+}
+
 // 12-byte vectors of a 16-bit type (six values, one global_load_dwordx3): a wave pass covers 384 values, so a row of 768
 // is two full passes where 16-byte vectors leave a quarter of the load slots idle.  Rows need 4-byte alignment only.
 struct alignas(4) raw_u32x3 {

@@ -622,7 +622,8 @@ struct TransposeArgs {
   LongType oShape[MAX_DEV_RANK], oX[MAX_DEV_RANK], oZ[MAX_DEV_RANK];
   unsigned tilesA, tilesB;
 };
-template <typename T>
+// NTS: the result leaves through non-temporal stores (the host asks for them from 8 MiB on, see streamPolicy)
+template <typename T, bool NTS>
 __global__ __launch_bounds__(256) void transpose_tiled(TransposeArgs a, const T* __restrict__ x, T* __restrict__ z) {
   __shared__ T tile[64][65];
   const unsigned tb = blockIdx.x % a.tilesB, ta = blockIdx.x / a.tilesB;
@@ -656,7 +657,12 @@ __global__ __launch_bounds__(256) void transpose_tiled(TransposeArgs a, const T*
         Pack out;
 #pragma unroll
         for (int e = 0; e < V; e++) out.e[e] = tile[c * V + e][i];
-        __builtin_memcpy(z + zo + (a0 + i) * a.zA + (b0 + c * V), &out, sizeof(Pack));
+        T* dst = z + zo + (a0 + i) * a.zA + (b0 + c * V);
+        if constexpr (NTS) {
+          nt_store16_elem_aligned(dst, out);
+        } else {
+          __builtin_memcpy(dst, &out, sizeof(Pack));
+        }
       }
       return;
     }
@@ -693,7 +699,8 @@ static bool tryTransposeCopy(hipStream_t s, const EwPlan& p, const T* x, T* z) {
   }
   a.tilesA = (unsigned)((a.nA + 63) / 64); a.tilesB = (unsigned)((a.nB + 63) / 64);
   if (batch > 65535 || (LongType)a.tilesA * a.tilesB >= (1LL << 31)) return false;
-  hipLaunchKernelGGL((transpose_tiled<T>), dim3(a.tilesA * a.tilesB, (unsigned)batch), dim3(256), 0, s, a, x, z);
+  if (streamPolicy(sizeof(T) * (size_t)p.length) >= 2) hipLaunchKernelGGL((transpose_tiled<T, true>), dim3(a.tilesA * a.tilesB, (unsigned)batch), dim3(256), 0, s, a, x, z);
+  else hipLaunchKernelGGL((transpose_tiled<T, false>), dim3(a.tilesA * a.tilesB, (unsigned)batch), dim3(256), 0, s, a, x, z);
   return true;
 }
 
@@ -746,7 +753,7 @@ static bool tailContig(hipStream_t s, int k, DataType dt, const void* x, const v
 
 // ---- dense casts between fp32 and the 16-bit types (the assign loop between two types) -------------------------------------
 // eight elements per thread: the wider side moves as two 16-byte vectors, the narrower as one; the tail one by one
-template <typename TI, typename TO>
+template <typename TI, typename TO, bool NTS>
 __global__ __launch_bounds__(EW_BLOCK) void cast_contig(const TI* __restrict__ x, TO* __restrict__ z, LongType n) {
   const LongType i = ((LongType)blockIdx.x * EW_BLOCK + threadIdx.x) * 8;
   if (i + 8 <= n) {
@@ -754,7 +761,14 @@ __global__ __launch_bounds__(EW_BLOCK) void cast_contig(const TI* __restrict__ x
     Vec<TO, 8> o;
 #pragma unroll
     for (int e = 0; e < 8; e++) o.v[e] = Conv<TO>::from(to_float(v.v[e]));
-    *reinterpret_cast<Vec<TO, 8>*>(z + i) = o;
+    if constexpr (NTS) {
+      struct Quads { raw_u32x4 q[sizeof(TO) * 8 / 16]; };
+      const Quads qs = __builtin_bit_cast(Quads, o);
+#pragma unroll
+      for (int k = 0; k < (int)(sizeof(TO) * 8 / 16); k++) __builtin_nontemporal_store(qs.q[k], reinterpret_cast<raw_u32x4*>(z + i) + k);
+    } else {
+      *reinterpret_cast<Vec<TO, 8>*>(z + i) = o;
+    }
   } else {
     for (LongType j = i; j < n; j++) z[j] = Conv<TO>::from(to_float(x[j]));
   }
@@ -762,12 +776,15 @@ __global__ __launch_bounds__(EW_BLOCK) void cast_contig(const TI* __restrict__ x
 template <typename TI>
 static bool castFrom(hipStream_t s, DataType zdt, const void* x, void* z, LongType n) {
   const unsigned grid = (unsigned)((n / 8 + EW_BLOCK) / EW_BLOCK);
+#define ND4J_CAST(TO) do { if (streamPolicy(sizeof(TO) * (size_t)n) >= 2) hipLaunchKernelGGL((cast_contig<TI, TO, true>), dim3(grid), dim3(EW_BLOCK), 0, s, (const TI*)x, (TO*)z, n); \
+                           else hipLaunchKernelGGL((cast_contig<TI, TO, false>), dim3(grid), dim3(EW_BLOCK), 0, s, (const TI*)x, (TO*)z, n); } while (0)
   switch (zdt) {
-    case FLOAT32: if constexpr (!std::is_same<TI, float>::value) { hipLaunchKernelGGL((cast_contig<TI, float>), dim3(grid), dim3(EW_BLOCK), 0, s, (const TI*)x, (float*)z, n); return true; } break;
-    case HALF: if constexpr (!std::is_same<TI, f16_t>::value) { hipLaunchKernelGGL((cast_contig<TI, f16_t>), dim3(grid), dim3(EW_BLOCK), 0, s, (const TI*)x, (f16_t*)z, n); return true; } break;
-    case BFLOAT16: if constexpr (!std::is_same<TI, bf16_t>::value) { hipLaunchKernelGGL((cast_contig<TI, bf16_t>), dim3(grid), dim3(EW_BLOCK), 0, s, (const TI*)x, (bf16_t*)z, n); return true; } break;
+    case FLOAT32: if constexpr (!std::is_same<TI, float>::value) { ND4J_CAST(float); return true; } break;
+    case HALF: if constexpr (!std::is_same<TI, f16_t>::value) { ND4J_CAST(f16_t); return true; } break;
+    case BFLOAT16: if constexpr (!std::is_same<TI, bf16_t>::value) { ND4J_CAST(bf16_t); return true; } break;
     default: break;
   }
+#undef ND4J_CAST
   return false;
 }
 static bool tryCastContig(hipStream_t s, DataType xdt, DataType zdt, const void* x, void* z, const EwPlan& p) {

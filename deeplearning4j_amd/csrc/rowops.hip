@@ -88,7 +88,7 @@ __global__ __launch_bounds__(256) void softmax_rows(RowArgs a, const T* __restri
     if (VEC > 1) {
       if (e0 < L) {
         const typename RawIO<T>::raw* src = reinterpret_cast<const typename RawIO<T>::raw*>(x + xb + e0);
-        RawIO<T>::unpack(nt ? __builtin_nontemporal_load(src) : *src, &vals[i * VEC]);
+        RawIO<T>::unpack(nt == 1 ? __builtin_nontemporal_load(src) : *src, &vals[i * VEC]);
       } else {
 #pragma unroll
         for (int e = 0; e < VEC; e++) vals[i * VEC + e] = NEG;
@@ -167,7 +167,8 @@ template <> struct PadBits<float> { static constexpr unsigned v = 0xff7fffffu; }
 template <> struct PadBits<bf16_t> { static constexpr unsigned v = 0xff7fff7fu; };
 template <> struct PadBits<f16_t> { static constexpr unsigned v = 0xfbfffbffu; };
 // G: lanes per row (64: a wave per row; 8, 16, 32: several short rows per wave, NV == 1)
-template <typename T, int NV, bool NT, int G = 64>
+// NT: 1 = non-temporal loads and stores (arrays beyond the last-level cache), 2 = stores only (results of 8 MiB and more)
+template <typename T, int NV, int NT, int G = 64>
 __global__ __launch_bounds__(256) void softmax_linear(RowArgs a, const T* __restrict__ x, T* __restrict__ z, int clamp) {
   using Raw = typename RawIO<T>::raw;
   constexpr int VEC = RawIO<T>::N;
@@ -183,7 +184,7 @@ __global__ __launch_bounds__(256) void softmax_linear(RowArgs a, const T* __rest
     const int e = (t + i * G) * VEC;
     e0[i] = e < L ? e : L - VEC;
     const raw_u32x4* src = reinterpret_cast<const raw_u32x4*>(xr + e0[i]);
-    bits[i] = NT ? __builtin_nontemporal_load(src) : *src;
+    bits[i] = NT == 1 ? __builtin_nontemporal_load(src) : *src;
   }
   __builtin_amdgcn_sched_barrier(0);   // all loads are issued before the first use: one trip to memory per row
   float vals[NV * VEC];
@@ -345,7 +346,7 @@ __global__ __launch_bounds__(1024) void softmax_long_vec(RowArgs a, const T* __r
 // block of 512 threads (two waves per SIMD: 256 registers each) holds the whole row in registers, so it comes from memory once and the three passes (maximum, sum of
 // exponentials, result) run on registers.  Rows may start anywhere: the 16-byte loads and stores are element-aligned (global
 // memory runs in unaligned access mode), the values after the last whole vector go one per thread.
-template <typename T, int NV, bool LOG>
+template <typename T, int NV, bool LOG, bool NTS = false>
 __global__ __launch_bounds__(512) void softmax_block_regs(RowArgs a, const T* __restrict__ x, T* __restrict__ z, int clamp) {
   using A = typename Conv<T>::acc;
   using Raw = typename RawIO<T>::raw;
@@ -403,7 +404,11 @@ __global__ __launch_bounds__(512) void softmax_block_regs(RowArgs a, const T* __
 #pragma unroll
       for (int e = 0; e < VEC; e++) vals[e] = result(vals[e]);
       const Raw o = RawIO<T>::pack(vals);
-      __builtin_memcpy(zr + iv * VEC, &o, sizeof(Raw));
+      if constexpr (NTS) {   // results of 8 MiB and more: non-temporal, element-aligned 16-byte stores
+        nt_store16_elem_aligned(zr + iv * VEC, o);
+      } else {
+        __builtin_memcpy(zr + iv * VEC, &o, sizeof(Raw));
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
   }
@@ -415,9 +420,11 @@ static bool softmaxBlockRegs(hipStream_t s, const RowArgs& a, const T* x, T* z, 
   if (p.xInner != 1 || p.zInner != 1 || p.rowLen < V || p.rowLen / V > 32 * 512) return false;
   const dim3 grid((unsigned)p.rows), block(512);
   const LongType per = (p.rowLen / V + 511) / 512;
-  if (per <= 16) hipLaunchKernelGGL((softmax_block_regs<T, 16, LOG>), grid, block, 0, s, a, x, z, clamp);
-  else if (per <= 26) hipLaunchKernelGGL((softmax_block_regs<T, 26, LOG>), grid, block, 0, s, a, x, z, clamp);
-  else hipLaunchKernelGGL((softmax_block_regs<T, 32, LOG>), grid, block, 0, s, a, x, z, clamp);
+  const bool nts = (size_t)p.rows * (size_t)p.rowLen * sizeof(T) >= ((size_t)8 << 20);
+#define SBR(NV) do { if (nts) hipLaunchKernelGGL((softmax_block_regs<T, NV, LOG, true>), grid, block, 0, s, a, x, z, clamp); \
+                     else hipLaunchKernelGGL((softmax_block_regs<T, NV, LOG, false>), grid, block, 0, s, a, x, z, clamp); } while (0)
+  if (per <= 16) SBR(16); else if (per <= 26) SBR(26); else SBR(32);
+#undef SBR
   return true;
 }
 
@@ -465,15 +472,17 @@ static void softmaxLinear(hipStream_t s, const RowArgs& a, const T* x, T* z, int
   const LongType lanes = a.rowLen / V;
   if (lanes <= 32) {
 #define SG(G) do { const dim3 gg((unsigned)((a.rows + 256 / G - 1) / (256 / G))); \
-                   if (nt) hipLaunchKernelGGL((softmax_linear<T, 1, true, G>), gg, dim3(256), 0, s, a, x, z, clamp); \
-                   else hipLaunchKernelGGL((softmax_linear<T, 1, false, G>), gg, dim3(256), 0, s, a, x, z, clamp); } while (0)
+                   if (nt == 1) hipLaunchKernelGGL((softmax_linear<T, 1, 1, G>), gg, dim3(256), 0, s, a, x, z, clamp); \
+                   else if (nt == 2) hipLaunchKernelGGL((softmax_linear<T, 1, 2, G>), gg, dim3(256), 0, s, a, x, z, clamp); \
+                   else hipLaunchKernelGGL((softmax_linear<T, 1, 0, G>), gg, dim3(256), 0, s, a, x, z, clamp); } while (0)
     if (lanes <= 8) SG(8); else if (lanes <= 16) SG(16); else SG(32);
 #undef SG
     return;
   }
   const dim3 grid((unsigned)((a.rows + 3) / 4));
-#define SL(NV) do { if (nt) hipLaunchKernelGGL((softmax_linear<T, NV, true>), grid, dim3(256), 0, s, a, x, z, clamp); \
-                    else hipLaunchKernelGGL((softmax_linear<T, NV, false>), grid, dim3(256), 0, s, a, x, z, clamp); } while (0)
+#define SL(NV) do { if (nt == 1) hipLaunchKernelGGL((softmax_linear<T, NV, 1>), grid, dim3(256), 0, s, a, x, z, clamp); \
+                    else if (nt == 2) hipLaunchKernelGGL((softmax_linear<T, NV, 2>), grid, dim3(256), 0, s, a, x, z, clamp); \
+                    else hipLaunchKernelGGL((softmax_linear<T, NV, 0>), grid, dim3(256), 0, s, a, x, z, clamp); } while (0)
   switch (passes) {
     case 1: SL(1); break; case 2: SL(2); break; case 3: SL(3); break; case 4: SL(4); break;
     case 5: SL(5); break; case 6: SL(6); break; case 7: SL(7); break; default: SL(8); break;
@@ -498,7 +507,10 @@ static void softmaxTyped(hipStream_t s, const void* x, void* z, const RowPlan& p
   if (rowsVectorOk(p, x, z, V)) {
     const LongType perWave = 64 * V, perBlock = 256 * V;
     // rows streamed once and larger than the last-level cache: non-temporal accesses
-    const int nt = (size_t)p.rows * (size_t)L * sizeof(T) * 2 > ((size_t)288 << 20) ? 1 : 0;
+    // ... and results of 8 MiB and more through non-temporal stores only (with ordinary stores they sit dirty in the L2
+    // until the kernel ends and are flushed then, which the next launch waits for)
+    const size_t outBytes = (size_t)p.rows * (size_t)L * sizeof(T);
+    const int nt = outBytes * 2 > ((size_t)288 << 20) ? 1 : outBytes >= ((size_t)8 << 20) ? 2 : 0;
     if (sizeof(T) <= 4 && L <= 8 * perWave) {
       softmaxLinear<T>(s, a, xt, zt, clamp, nt);
       return;
@@ -826,11 +838,27 @@ __global__ __launch_bounds__(256) void layernorm_linear(const T* __restrict__ x,
   }
 }
 
+// a result vector on its way out: through a non-temporal store when the host asks for it (results of 8 MiB and more:
+// written with ordinary stores they sit dirty in the L2 until the kernel ends and are flushed then, which the next launch
+// waits for), else an ordinary one
+template <bool NTS, typename Raw>
+__device__ __forceinline__ void store_row_vec(Raw* p, const Raw& v) {
+  if constexpr (!NTS) {
+    *p = v;
+  } else if constexpr (sizeof(Raw) == 12) {
+    typedef unsigned u32x3a __attribute__((ext_vector_type(3), aligned(4)));
+    const u32x3a t = {v[0], v[1], v[2]};
+    __builtin_nontemporal_store(t, reinterpret_cast<u32x3a*>(p));
+  } else {
+    __builtin_nontemporal_store(v, p);
+  }
+}
+
 // Many rows: two consecutive rows per wave, gain and bias fetched once for both, every load of the pair issued before
 // the first use.  The grid normally gives every wave one pair; beyond 2^20 blocks a wave walks on to pair pr + W with
 // that pair's loads issued ahead.  (About ten vector instructions per element: a 16-bit row is as much arithmetic as an
 // fp32 row of the same length in half the bytes, which is why bf16 [16384, 768] takes 9.5 us where gelu takes 5.3.)
-template <typename T, int NV, bool HAS_BIAS, typename IO = RawIO<T>, bool WALK = true>
+template <typename T, int NV, bool HAS_BIAS, typename IO = RawIO<T>, bool WALK = true, bool NTS = false>
 __global__ __launch_bounds__(256, WALK ? 1 : 8) void layernorm_stream(const T* __restrict__ x, const T* __restrict__ gain, const T* __restrict__ bias, T* __restrict__ z,
                                                         LongType rows, int L, LongType xPitch, LongType zPitch, float eps) {
   using A = typename Conv<T>::acc;
@@ -916,7 +944,7 @@ __global__ __launch_bounds__(256, WALK ? 1 : 8) void layernorm_stream(const T* _
           if (HAS_BIAS) y += b[e];
           vals[r][i * VEC + e] = y;
         }
-        if (keep[i] != (A)0) *reinterpret_cast<Raw*>(zr + e0[i]) = IO::pack(&vals[r][i * VEC]);
+        if (keep[i] != (A)0) store_row_vec<NTS>(reinterpret_cast<Raw*>(zr + e0[i]), IO::pack(&vals[r][i * VEC]));
       }
     }
     if (!WALK) break;
@@ -1043,23 +1071,29 @@ static bool layerNormTyped(hipStream_t s, const void* x, const void* gain, const
         // 59 instead of 93 of them, eight waves per SIMD.  bf16 [16384, 768] 12.7 -> 11.8 us; the same variant of the 16-byte
         // kernels measured equal or slower (bf16 rows of 512 8.8 -> 9.1 us, fp32 rows of 384 12.0 -> 12.6) and is not built
         const bool oneEach = (LongType)gs * 8 >= p.rows;
-#define LNS(NV) do { if (bt) hipLaunchKernelGGL((layernorm_stream<T, NV, true>), dim3(gs), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); \
-                     else hipLaunchKernelGGL((layernorm_stream<T, NV, false>), dim3(gs), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); } while (0)
+        // results of 8 MiB and more leave through non-temporal stores (see store_row_vec)
+        const bool nts = (size_t)p.rows * (size_t)L * sizeof(T) >= ((size_t)8 << 20);
+#define LNS_(NV, B, NTS) hipLaunchKernelGGL((layernorm_stream<T, NV, B, RawIO<T>, true, NTS>), dim3(gs), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps)
+#define LNS(NV) do { if (bt) { if (nts) LNS_(NV, true, true); else LNS_(NV, true, false); } \
+                     else { if (nts) LNS_(NV, false, true); else LNS_(NV, false, false); } } while (0)
         // 16-bit rows of a whole number of 384-value passes that are not a whole number of 512-value ones (768: one and a
         // half): 12-byte vectors, every load slot used
         if constexpr (sizeof(T) == 2) {
           if (L % 384 == 0 && L % 512 != 0 && L <= 4 * 384) {
-#define LNS12W(NV, WALK) do { if (bt) hipLaunchKernelGGL((layernorm_stream<T, NV, true, RawIO12<T>, WALK>), dim3(gs), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); \
-                       else hipLaunchKernelGGL((layernorm_stream<T, NV, false, RawIO12<T>, WALK>), dim3(gs), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); } while (0)
+#define LNS12_(NV, B, WALK, NTS) hipLaunchKernelGGL((layernorm_stream<T, NV, B, RawIO12<T>, WALK, NTS>), dim3(gs), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps)
+#define LNS12W(NV, WALK) do { if (bt) { if (nts) LNS12_(NV, true, WALK, true); else LNS12_(NV, true, WALK, false); } \
+                              else { if (nts) LNS12_(NV, false, WALK, true); else LNS12_(NV, false, WALK, false); } } while (0)
 #define LNS12(NV) do { if (oneEach && NV <= 2) LNS12W(NV, (NV > 2)); else LNS12W(NV, true); } while (0)
             if (L == 384) LNS12(1); else if (L == 768) LNS12(2); else LNS12(3);
 #undef LNS12
 #undef LNS12W
+#undef LNS12_
             return true;
           }
         }
         if (L <= perWave) LNS(1); else if (L <= 2 * perWave) LNS(2); else if (L <= 3 * perWave) LNS(3); else LNS(4);
 #undef LNS
+#undef LNS_
         return true;
       }
       if (L <= perWave) { LNL(1); return true; }
