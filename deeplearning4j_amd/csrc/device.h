@@ -124,6 +124,21 @@ template <> struct RawIO<f16_t> {
   }
 };
 
+// a naturally aligned vector of 4, 8 or 16 bytes on its way out: through a non-temporal store when `nts` says so (the hosts ask
+// for it for results of 8 MiB and more), else an ordinary one; other sizes always take the ordinary store
+template <typename VT>
+__device__ __forceinline__ void store_vec(VT* p, const VT& v, bool nts) {
+  if constexpr (sizeof(VT) == 16) {
+    if (nts) { __builtin_nontemporal_store(__builtin_bit_cast(raw_u32x4, v), reinterpret_cast<raw_u32x4*>(p)); return; }
+  } else if constexpr (sizeof(VT) == 8) {
+    typedef unsigned raw_u32x2 __attribute__((ext_vector_type(2)));
+    if (nts) { __builtin_nontemporal_store(__builtin_bit_cast(raw_u32x2, v), reinterpret_cast<raw_u32x2*>(p)); return; }
+  } else if constexpr (sizeof(VT) == 4) {
+    if (nts) { __builtin_nontemporal_store(__builtin_bit_cast(unsigned, v), reinterpret_cast<unsigned*>(p)); return; }
+  }
+  *p = v;
+}
+
 // a 16-byte pack of elements of T on its way out through a non-temporal store, to an address that is only element-aligned
 typedef unsigned u32x4_align2 __attribute__((ext_vector_type(4), aligned(2)));
 typedef unsigned u32x4_align4 __attribute__((ext_vector_type(4), aligned(4)));

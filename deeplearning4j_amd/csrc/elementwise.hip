@@ -391,6 +391,7 @@ struct NdArgs {
   int rank;                        // >= 1; dim rank-1 is the inner run
   LongType shape[MAX_DEV_RANK];
   LongType stride[3][MAX_DEV_RANK];
+  int nts = 0;                     // the vector kernels: the result leaves through non-temporal stores (8 MiB and more)
 };
 
 // One thread per chunk of VEC consecutive inner elements.  VEC > 1 requires unit inner strides, an inner
@@ -437,7 +438,7 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_nd(NdArgs a, const T* __restrict_
         if (NIN > 1) out.v[e] = Conv<T>::from(F::template apply<A>((A)to_float(vx.v[e]), (A)to_float(vy.v[e])));
         else out.v[e] = Conv<T>::from(F::template apply<A>((A)to_float(vx.v[e]), (A)to_float(vx.v[e])));
       }
-      *reinterpret_cast<VT*>(z + oz) = out;
+      store_vec(reinterpret_cast<VT*>(z + oz), out, a.nts != 0);
     } else {
       A vx = (A)to_float(x[ox]);
       A vy = NIN > 1 ? (A)to_float(y[oy]) : vx;
@@ -592,6 +593,7 @@ static void launchNd(hipStream_t s, const EwPlan& p, const T* x, const T* y, T* 
     a.shape[d] = p.shape[d];
     for (int o = 0; o < 3; o++) a.stride[o][d] = p.stride[o][d];
   }
+  a.nts = streamPolicy(sizeof(T) * (size_t)p.length) >= 2 ? 1 : 0;
   const LongType inner = p.shape[p.rank - 1];
   // vectors along the inner axis: the output and every input run along it with unit stride from aligned starts -- or an
   // input repeats along it (stride 0), which needs no alignment
@@ -884,7 +886,7 @@ __global__ __launch_bounds__(EW_BLOCK) void row_broadcast(const T* __restrict__ 
 }
 template <typename F, typename T>
 __global__ __launch_bounds__(EW_BLOCK) void row_broadcast_vec(const T* __restrict__ x, const T* __restrict__ v,
-                                                              T* __restrict__ z, LongType rows, LongType colVecs) {
+                                                              T* __restrict__ z, LongType rows, LongType colVecs, int nts) {
   constexpr int V = 16 / sizeof(T);
   using VT = Vec<T, V>;
   using A = typename Conv<T>::acc;
@@ -897,14 +899,15 @@ __global__ __launch_bounds__(EW_BLOCK) void row_broadcast_vec(const T* __restric
     VT a = xv[i], b = vv[i % colVecs], out;
 #pragma unroll
     for (int e = 0; e < V; e++) out.v[e] = Conv<T>::from(F::template apply<A>((A)to_float(a.v[e]), (A)to_float(b.v[e])));
-    zv[i] = out;
+    store_vec(zv + i, out, nts != 0);
   }
 }
 template <int K, typename T>
 static void rowBroadcastTyped(hipStream_t s, const void* x, const void* v, void* z, LongType rows, LongType cols) {
   constexpr int V = 16 / sizeof(T);
   if (cols % V == 0 && aligned16(x) && aligned16(v) && aligned16(z))
-    hipLaunchKernelGGL((row_broadcast_vec<Pairwise<K>, T>), dim3(gridFor(rows * cols / V, EW_BLOCK)), dim3(EW_BLOCK), 0, s, (const T*)x, (const T*)v, (T*)z, rows, cols / V);
+    hipLaunchKernelGGL((row_broadcast_vec<Pairwise<K>, T>), dim3(gridFor(rows * cols / V, EW_BLOCK)), dim3(EW_BLOCK), 0, s, (const T*)x, (const T*)v, (T*)z, rows, cols / V,
+                       streamPolicy(sizeof(T) * (size_t)(rows * cols)) >= 2 ? 1 : 0);
   else
     hipLaunchKernelGGL((row_broadcast<Pairwise<K>, T>), dim3(gridFor(rows * cols, EW_BLOCK)), dim3(EW_BLOCK), 0, s, (const T*)x, (const T*)v, (T*)z, rows, cols);
 }
@@ -970,7 +973,7 @@ __global__ __launch_bounds__(EW_BLOCK) void scalar_nd_vec(NdArgs a, const T* __r
     VT out;
 #pragma unroll
     for (int e = 0; e < V; e++) out.v[e] = Conv<T>::from(F::template apply<A>((A)to_float(vx.v[e]), sc));
-    *reinterpret_cast<VT*>(z + oz) = out;
+    store_vec(reinterpret_cast<VT*>(z + oz), out, a.nts != 0);
   }
   // rank 1 only: what is left after the last whole vector
   if (blockIdx.x == 0) {
@@ -983,6 +986,7 @@ static void scalarTyped(hipStream_t s, const void* x, double sc, void* z, const 
   NdArgs a;
   a.rank = p.rank;
   for (int d = 0; d < p.rank; d++) { a.shape[d] = p.shape[d]; for (int o = 0; o < 3; o++) a.stride[o][d] = p.stride[o][d]; }
+  a.nts = streamPolicy(sizeof(T) * (size_t)p.length) >= 2 ? 1 : 0;
   using A = typename Conv<T>::acc;
   A scv = (A)sc;
   constexpr int V = 16 / sizeof(T);
@@ -1058,7 +1062,7 @@ void launchScalar2Op(hipStream_t s, Scalar2Kind k, DataType xdt, DataType zdt, c
 // ---- gather rows / fill ------------------------------------------------------------------------------------
 template <typename T, typename IT>
 __global__ __launch_bounds__(EW_BLOCK) void gather_rows(const T* __restrict__ table, const IT* __restrict__ idx,
-                                                        T* __restrict__ z, LongType nIdx, LongType rowLen, LongType tableRows) {
+                                                        T* __restrict__ z, LongType nIdx, LongType rowLen, LongType tableRows, int nts) {
   const LongType n = nIdx * rowLen;
   const LongType step = (LongType)gridDim.x * EW_BLOCK;
   for (LongType i = (LongType)blockIdx.x * EW_BLOCK + threadIdx.x; i < n; i += step) {
@@ -1067,7 +1071,7 @@ __global__ __launch_bounds__(EW_BLOCK) void gather_rows(const T* __restrict__ ta
     if (src < 0) src += tableRows;
     // out-of-range ids are clamped so that a bad id cannot fault the device; the host validates ids it can see
     src = src < 0 ? 0 : (src >= tableRows ? tableRows - 1 : src);
-    z[i] = table[src * rowLen + c];
+    store_vec(z + i, table[src * rowLen + c], nts != 0);
   }
 }
 void launchGatherRows(hipStream_t s, DataType dt, DataType idxDt, const void* table, const void* idx, void* z,
@@ -1075,9 +1079,10 @@ void launchGatherRows(hipStream_t s, DataType dt, DataType idxDt, const void* ta
   if (nIdx * rowLen == 0) return;
   ND4J_REQUIRE(idxDt == INT32 || idxDt == INT64, "gather: indices must be INT32 or INT64");
   dim3 g(gridFor(nIdx * rowLen, EW_BLOCK)), b(EW_BLOCK);
+  const int nts = streamPolicy((size_t)(nIdx * rowLen) * sizeOf(dt)) >= 2 ? 1 : 0;   // only the 16-byte rows take it
 #define GATHER(T)                                                                                                         \
-  if (idxDt == INT32) hipLaunchKernelGGL((gather_rows<T, int>), g, b, 0, s, (const T*)table, (const int*)idx, (T*)z, nIdx, rowLen, tableRows); \
-  else hipLaunchKernelGGL((gather_rows<T, LongType>), g, b, 0, s, (const T*)table, (const LongType*)idx, (T*)z, nIdx, rowLen, tableRows);
+  if (idxDt == INT32) hipLaunchKernelGGL((gather_rows<T, int>), g, b, 0, s, (const T*)table, (const int*)idx, (T*)z, nIdx, rowLen, tableRows, nts); \
+  else hipLaunchKernelGGL((gather_rows<T, LongType>), g, b, 0, s, (const T*)table, (const LongType*)idx, (T*)z, nIdx, rowLen, tableRows, nts);
   // rows that are whole 16-byte units in aligned arrays move as such
   using U16 = Vec<unsigned, 4>;
   const LongType es = (LongType)sizeOf(dt);
