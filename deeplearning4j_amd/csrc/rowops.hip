@@ -717,7 +717,8 @@ __global__ __launch_bounds__(256) void layernorm_rows(RowArgs a, const T* __rest
 template <typename T, int NV, bool HAS_BIAS, int RPW, bool ADD = false, int G = 64>
 __global__ __launch_bounds__(256) void layernorm_linear(const T* __restrict__ x, const T* __restrict__ gain, const T* __restrict__ bias,
                                                         T* __restrict__ z, LongType rows, int L, LongType xPitch, LongType zPitch, float eps,
-                                                        const T* addend = nullptr, LongType aPitch = 0, T* sumOut = nullptr, LongType sPitch = 0) {
+                                                        const T* addend = nullptr, LongType aPitch = 0, T* sumOut = nullptr, LongType sPitch = 0,
+                                                        int nts = 0) {   // nts: the result through non-temporal stores (8 MiB and more)
   using A = typename Conv<T>::acc;
   using Raw = typename RawIO<T>::raw;
   constexpr int VEC = RawIO<T>::N;
@@ -783,7 +784,7 @@ __global__ __launch_bounds__(256) void layernorm_linear(const T* __restrict__ x,
     T* zr = z + row0 * zPitch;
 #pragma unroll
     for (int i = 0; i < NV; i++)
-      if (keep[i] != (A)0) *reinterpret_cast<Raw*>(zr + e0[i]) = RawIO<T>::pack(&vals[0][i * VEC]);
+      if (keep[i] != (A)0) store_vec(reinterpret_cast<Raw*>(zr + e0[i]), RawIO<T>::pack(&vals[0][i * VEC]), nts != 0);
     return;
   }
   A sum[RPW];
@@ -833,7 +834,7 @@ __global__ __launch_bounds__(256) void layernorm_linear(const T* __restrict__ x,
         if (HAS_BIAS) y += b[e];
         vals[r][i * VEC + e] = y;
       }
-      if (keep[i] != (A)0) *reinterpret_cast<Raw*>(zr + e0[i]) = RawIO<T>::pack(&vals[r][i * VEC]);
+      if (keep[i] != (A)0) store_vec(reinterpret_cast<Raw*>(zr + e0[i]), RawIO<T>::pack(&vals[r][i * VEC]), nts != 0);
     }
   }
 }
@@ -1049,8 +1050,9 @@ static bool layerNormTyped(hipStream_t s, const void* x, const void* gain, const
       const LongType xp = p.outerX.rank ? p.outerX.stride[0] : 0, zp = p.outerZ.rank ? p.outerZ.stride[0] : 0;
       // many rows: two per wave (layernorm_stream: gain and bias fetched once for both); few rows: one per wave, so that every CU gets some
       const bool pair = p.rows >= 4096 && L <= 4 * perWave;
-#define LNL(NV) do { if (bt) hipLaunchKernelGGL((layernorm_linear<T, NV, true, 1>), dim3(gw), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); \
-                     else hipLaunchKernelGGL((layernorm_linear<T, NV, false, 1>), dim3(gw), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps); } while (0)
+      const int ntsL = (size_t)p.rows * (size_t)L * sizeof(T) >= ((size_t)8 << 20) ? 1 : 0;   // see store_row_vec
+#define LNL(NV) do { if (bt) hipLaunchKernelGGL((layernorm_linear<T, NV, true, 1>), dim3(gw), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps, (const T*)nullptr, (LongType)0, (T*)nullptr, (LongType)0, ntsL); \
+                     else hipLaunchKernelGGL((layernorm_linear<T, NV, false, 1>), dim3(gw), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps, (const T*)nullptr, (LongType)0, (T*)nullptr, (LongType)0, ntsL); } while (0)
       // short rows: 8, 16 or 32 lanes per row
       if constexpr (sizeof(T) <= 4) {
         const LongType lanes = L / V;
