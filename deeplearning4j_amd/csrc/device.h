@@ -126,15 +126,16 @@ template <> struct RawIO<f16_t> {
 
 // a naturally aligned vector of 4, 8 or 16 bytes on its way out: through a non-temporal store when `nts` says so (the hosts ask
 // for it for results of 8 MiB and more), else an ordinary one; other sizes always take the ordinary store
+// (the 16-byte case is written as assembly: given both stores in one branch the compiler sinks them into a single ordinary
+// store and the non-temporal hint is gone)
 template <typename VT>
 __device__ __forceinline__ void store_vec(VT* p, const VT& v, bool nts) {
   if constexpr (sizeof(VT) == 16) {
-    if (nts) { __builtin_nontemporal_store(__builtin_bit_cast(raw_u32x4, v), reinterpret_cast<raw_u32x4*>(p)); return; }
-  } else if constexpr (sizeof(VT) == 8) {
-    typedef unsigned raw_u32x2 __attribute__((ext_vector_type(2)));
-    if (nts) { __builtin_nontemporal_store(__builtin_bit_cast(raw_u32x2, v), reinterpret_cast<raw_u32x2*>(p)); return; }
-  } else if constexpr (sizeof(VT) == 4) {
-    if (nts) { __builtin_nontemporal_store(__builtin_bit_cast(unsigned, v), reinterpret_cast<unsigned*>(p)); return; }
+    if (nts) {
+      const raw_u32x4 q = __builtin_bit_cast(raw_u32x4, v);
+      asm volatile("global_store_dwordx4 %0, %1, off nt" ::"v"(p), "v"(q) : "memory");
+      return;
+    }
   }
   *p = v;
 }

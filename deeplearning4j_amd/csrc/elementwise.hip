@@ -895,8 +895,20 @@ __global__ __launch_bounds__(EW_BLOCK) void row_broadcast_vec(const T* __restric
   const VT* xv = reinterpret_cast<const VT*>(x);
   const VT* vv = reinterpret_cast<const VT*>(v);
   VT* zv = reinterpret_cast<VT*>(z);
-  for (LongType i = (LongType)blockIdx.x * EW_BLOCK + threadIdx.x; i < n; i += step) {
-    VT a = xv[i], b = vv[i % colVecs], out;
+  // the column of a thread's vector: the block's first column comes from one scalar remainder, the thread's own from at most
+  // a few subtractions (a 64-bit remainder per vector cost more than the memory traffic of the 16-bit types)
+  for (LongType base = (LongType)blockIdx.x * EW_BLOCK; base < n; base += step) {
+    const LongType i = base + threadIdx.x;
+    if (i >= n) break;
+    LongType col;
+    if (colVecs < (1 << 30)) {
+      col = (LongType)__builtin_amdgcn_readfirstlane((int)(base % colVecs)) + threadIdx.x;
+      if (colVecs >= EW_BLOCK) { if (col >= colVecs) col -= colVecs; }
+      else col %= colVecs;
+    } else {
+      col = i % colVecs;
+    }
+    VT a = xv[i], b = vv[col], out;
 #pragma unroll
     for (int e = 0; e < V; e++) out.v[e] = Conv<T>::from(F::template apply<A>((A)to_float(a.v[e]), (A)to_float(b.v[e])));
     store_vec(zv + i, out, nts != 0);
@@ -958,16 +970,21 @@ __global__ __launch_bounds__(EW_BLOCK) void scalar_nd_vec(NdArgs a, const T* __r
   using VT = Vec<T, V>;
   const I step = (I)gridDim.x * EW_BLOCK;
   for (I c = (I)blockIdx.x * EW_BLOCK + threadIdx.x; c < totalChunks; c += step) {
-    I outer = c / chunksPerRow;
-    const LongType inner = (LongType)(c - outer * chunksPerRow) * V;
-    LongType oz = inner, ox = inner;
+    LongType oz, ox;
+    if (a.rank == 1) {   // a dense array: one run, no division
+      oz = ox = (LongType)c * V;
+    } else {
+      I outer = c / chunksPerRow;
+      const LongType inner = (LongType)(c - outer * chunksPerRow) * V;
+      oz = inner; ox = inner;
 #pragma unroll 1
-    for (int d = a.rank - 2; d >= 0; d--) {
-      const I dim = (I)a.shape[d];
-      const I q = outer / dim;
-      const LongType cd = (LongType)(outer - q * dim);
-      oz += cd * a.stride[0][d]; ox += cd * a.stride[1][d];
-      outer = q;
+      for (int d = a.rank - 2; d >= 0; d--) {
+        const I dim = (I)a.shape[d];
+        const I q = outer / dim;
+        const LongType cd = (LongType)(outer - q * dim);
+        oz += cd * a.stride[0][d]; ox += cd * a.stride[1][d];
+        outer = q;
+      }
     }
     const VT vx = *reinterpret_cast<const VT*>(x + ox);
     VT out;

@@ -150,8 +150,7 @@ __global__ __launch_bounds__(256) void softmax_rows(RowArgs a, const T* __restri
 #pragma unroll
       for (int e = 0; e < VEC; e++) vals[i * VEC + e] *= inv;
       typename RawIO<T>::raw* dst = reinterpret_cast<typename RawIO<T>::raw*>(z + zb + e0);
-      if (nt) __builtin_nontemporal_store(RawIO<T>::pack(&vals[i * VEC]), dst);
-      else *dst = RawIO<T>::pack(&vals[i * VEC]);
+      store_vec(dst, RawIO<T>::pack(&vals[i * VEC]), nt != 0);
     } else {
       z[zb + e0 * a.zInner] = Conv<T>::from(vals[i] * inv);
     }
