@@ -486,15 +486,25 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_fused(FusedArgs a, 
 // eight consecutive values of d as a lane holds them: one 16-byte load for the 16-bit types, two for fp32
 template <typename T> struct Row8 {
   using raw = typename RawIO<T>::raw;
-  static __device__ __forceinline__ raw load(const T* p) { return *reinterpret_cast<const raw*>(p); }
+  template <bool NT = false>
+  static __device__ __forceinline__ raw load(const T* p) {
+    if constexpr (NT) return __builtin_nontemporal_load(reinterpret_cast<const raw*>(p));
+    else return *reinterpret_cast<const raw*>(p);
+  }
   static __device__ __forceinline__ void unpack(const raw& r, float* out) { RawIO<T>::unpack(r, out); }
 };
 template <> struct Row8<float> {
   struct raw { raw_f32x4 lo, hi; };
+  template <bool NT = false>
   static __device__ __forceinline__ raw load(const float* p) {
     raw r;
-    r.lo = *reinterpret_cast<const raw_f32x4*>(p);
-    r.hi = *reinterpret_cast<const raw_f32x4*>(p + 4);
+    if constexpr (NT) {
+      r.lo = __builtin_nontemporal_load(reinterpret_cast<const raw_f32x4*>(p));
+      r.hi = __builtin_nontemporal_load(reinterpret_cast<const raw_f32x4*>(p + 4));
+    } else {
+      r.lo = *reinterpret_cast<const raw_f32x4*>(p);
+      r.hi = *reinterpret_cast<const raw_f32x4*>(p + 4);
+    }
     return r;
   }
   static __device__ __forceinline__ void unpack(const raw& r, float* out) {
@@ -502,7 +512,9 @@ template <> struct Row8<float> {
     for (int e = 0; e < 4; e++) { out[e] = r.lo[e]; out[4 + e] = r.hi[e]; }
   }
 };
-template <typename T, int D, int NW, bool VM, int U = 4>
+// STREAM: keys and values come through non-temporal loads -- a history that is large against the last-level cache (a
+// decode step at batch 32 reads 57 MB of it per layer, 680 MB per step) then does not push the weights out of it
+template <typename T, int D, int NW, bool VM, int U = 4, bool STREAM = false>
 __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
                                                        T* __restrict__ O) {
   constexpr int CH = D / 8;          // lanes per key row
@@ -544,8 +556,8 @@ __global__ __launch_bounds__(NW * 64) void attn_decode(FusedArgs a, const T* __r
       LongType key = k0 + u * KPS + g;
       valid[u] = key < kEnd;
       key = valid[u] ? key : a.Tv - 1;
-      kr[u] = Row8<T>::load(K + key * a.kT + c * 8);
-      vr[u] = Row8<T>::load(V + key * a.vT + c * 8);
+      kr[u] = Row8<T>::template load<STREAM>(K + key * a.kT + c * 8);
+      vr[u] = Row8<T>::template load<STREAM>(V + key * a.vT + c * 8);
     }
   };
   const LongType step = (LongType)NW * (KPS * U);
@@ -712,6 +724,8 @@ static void launchDecodeTyped(hipStream_t s, const void* q, const void* k, const
   }
   // few (batch, head) rows: more waves per row, so that the history is still spread over many loads in flight
   if (d.B * d.Tq < 128) hipLaunchKernelGGL((attn_decode<T, D, 16, false>), grid, dim3(1024), 0, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
+  else if ((double)d.B * (double)d.Tv * 2.0 * D * sizeof(T) >= (double)(32 << 20))
+    hipLaunchKernelGGL((attn_decode<T, D, 4, false, 4, true>), grid, dim3(256), 0, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
   else hipLaunchKernelGGL((attn_decode<T, D, 4, false>), grid, dim3(256), 0, s, a, (const T*)q, (const T*)k, (const T*)v, (T*)out);
 }
 

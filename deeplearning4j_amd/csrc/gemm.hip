@@ -408,7 +408,9 @@ __global__ __launch_bounds__(WM * WN * 64) void splitk_finish(GemmArgs g, T* __r
   }
 }
 
-template <typename T, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC>
+// STREAM_B: B comes through non-temporal loads (the host asks for it when the product has one row of tiles, so that every
+// element of B is read exactly once, and B is large against the last-level cache)
+template <typename T, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, bool STREAM_B = false>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16p(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
                                                              unsigned tilesM, unsigned tilesN) {
   constexpr int BK = 64, NT = WM * WN * 64;
@@ -442,7 +444,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16p(GemmArgs g, const T
   const LongType KT = (g.K + BK - 1) / BK;
 
   la.load(A, lda, m0, g.M, 0, g.K, t);
-  lb.load(B, ldb, n0, g.N, 0, g.K, t);
+  lb.template load<T, STREAM_B>(B, ldb, n0, g.N, 0, g.K, t);
   la.store(smem, t);
   lb.store(smem + SLOTS_A, t);
   __syncthreads();
@@ -451,7 +453,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16p(GemmArgs g, const T
     const int cur = (int)(kt & 1);
     if (kt + 1 < KT) {
       la.load(A, lda, m0, g.M, (kt + 1) * BK, g.K, t);
-      lb.load(B, ldb, n0, g.N, (kt + 1) * BK, g.K, t);
+      lb.template load<T, STREAM_B>(B, ldb, n0, g.N, (kt + 1) * BK, g.K, t);
     }
     const u32x4* sA = smem + cur * STAGE;
     const u32x4* sB = sA + SLOTS_A;
@@ -1451,6 +1453,15 @@ static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
                                     : DynLds<gemm_mfma16<T, BM, BN, WM, WN, A_KC, B_KC>, (int)LDS>::granted();
   ND4J_REQUIRE(ldsGranted, "matmul: the device does not grant the tile kernel its LDS");
   const unsigned tilesM = (unsigned)((g.M + BM - 1) / BM), tilesN = (unsigned)((g.N + BN - 1) / BN);
+  if constexpr (BM == 32) {
+    // a few rows against a matrix that is large against the last-level cache (the logits of a decode step against the
+    // embedding: 77 MB): every element of B is read once, through non-temporal loads, and what the step reads again -- the
+    // layers' weights -- stays in the cache (batch-32 step 0.616 -> see the bench line)
+    if (usePipe && !useFull && !useDeep && tilesM == 1 && batch == 1 &&
+        (double)g.N * (double)g.K * sizeof(T) >= (double)(32 << 20) &&
+        DynLds<gemm_mfma16p<T, BM, BN, WM, WN, A_KC, B_KC, true>, (int)LDS>::granted())
+      kern = gemm_mfma16p<T, BM, BN, WM, WN, A_KC, B_KC, true>;
+  }
   noteKernel("%s<%s,%dx%d,akc=%d,bkc=%d>%s", useFull ? "gemm_mfma16f" : useDeep ? "gemm_mfma16q" : usePipe ? "gemm_mfma16p" : "gemm_mfma16", tname<T>(), BM, BN,
              (int)A_KC, (int)B_KC, splits > 1 ? "+splitk_finish" : "");
   hipLaunchKernelGGL(kern, dim3(tilesM * tilesN, (unsigned)splits, (unsigned)batch), dim3(NT), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tilesM, tilesN);
@@ -1883,7 +1894,10 @@ __global__ __launch_bounds__(256) void gemv_rowdot_pre(const T* __restrict__ W, 
   for (int i = 0; i < NL; i++) {
     const int kk = lane + 64 * i, kc = kk < kw ? kk : kw - 1;
 #pragma unroll
-    for (int o = 0; o < OPW; o++) wr[o][i] = reinterpret_cast<const raw_u32x4*>(wrow[o])[kc];
+    for (int o = 0; o < OPW; o++) {
+      if constexpr (!HAS_BIAS && PRO == 0) wr[o][i] = __builtin_nontemporal_load(reinterpret_cast<const raw_u32x4*>(wrow[o]) + kc);
+      else wr[o][i] = reinterpret_cast<const raw_u32x4*>(wrow[o])[kc];
+    }
     if constexpr (PRO != 2) xr[i] = reinterpret_cast<const raw_u32x4*>(x)[kc];
   }
   if constexpr (PRO == 2) {

@@ -58,6 +58,17 @@ __device__ __forceinline__ u32x4 load16u(const void* p) {
   __builtin_memcpy(&v, p, 16);
   return v;
 }
+// the same through a non-temporal load: for operands that are read once and are large against the last-level cache
+// (a vocabulary's embedding under a few rows of activations), so that they do not push out what is read again
+template <bool NT>
+__device__ __forceinline__ u32x4 load16u_stream(const void* p) {
+  if constexpr (NT) {
+    typedef unsigned u32x4_elem __attribute__((ext_vector_type(4), aligned(2)));
+    return __builtin_bit_cast(u32x4, __builtin_nontemporal_load(reinterpret_cast<const u32x4_elem*>(p)));
+  } else {
+    return load16u(p);
+  }
+}
 // the eight 16-bit elements of v moved down by sh places: element j + sh lands in place j, zeros come in from the top
 // (sh >= 8: all zeros).  Selects only, no indexed register access.
 __device__ __forceinline__ u32x4 shiftDownElems(u32x4 v, int sh) {
@@ -87,7 +98,7 @@ struct TileLoader {
   // last rows) is read 8 elements back from the end instead and moved down in registers, zeros coming in for what lies
   // beyond; k positions past K give zeros (they meet the other operand's tail); rows past the limit of a k-contiguous
   // operand repeat the last row (their products are never stored).  Needs K >= 8 (k-contiguous) or rowLimit >= 8.
-  template <typename T>
+  template <typename T, bool STREAM = false>
   __device__ __forceinline__ void load(const T* __restrict__ base, LongType ld, LongType row0, LongType rowLimit, LongType k0, LongType K, int t) {
     const u32x4 zero = {0u, 0u, 0u, 0u};
 #pragma unroll
@@ -100,7 +111,7 @@ struct TileLoader {
         r = r < rowLimit ? r : rowLimit - 1;
         const LongType k = k0 + kg * 8;
         const LongType kk = k + 8 <= K ? k : K - 8;
-        reg[i] = load16u(base + r * ld + kk);
+        reg[i] = load16u_stream<STREAM>(base + r * ld + kk);
         if (k != kk) reg[i] = shiftDownElems(reg[i], (int)(k - kk < 8 ? k - kk : 8));
       } else {
         const int rb = (u >> 1) % (ROWS / 8), kq = (u / (ROWS / 4)) * 2 + (u & 1);   // 8-row block, 4-k quad (16 per tile)
@@ -110,7 +121,7 @@ struct TileLoader {
 #pragma unroll
         for (int q = 0; q < 4; q++) {
           const LongType k = k0 + kq * 4 + q;
-          reg[i * 4 + q] = load16u(base + (k < K ? k : K - 1) * ld + rr);
+          reg[i * 4 + q] = load16u_stream<STREAM>(base + (k < K ? k : K - 1) * ld + rr);
         }
 #pragma unroll
         for (int q = 0; q < 4; q++) {
