@@ -139,6 +139,31 @@ def test_causal_attention_in_every_block_order(ex, oracle, dt, B, T):
         assert_close(out[bi:bi + 1], _as_float(oo), tol, tol, "batch entry %d" % bi)
 
 
+@pytest.mark.parametrize("dt", [BFLOAT16, FLOAT32])
+def test_causal_prefill_over_token_major_heads_equals_the_dense_layout(ex, dt):
+    """A decoder's prefill: [batch, heads, T, 64] views of a token-major qkv buffer (batch and head strides that do not
+    nest), 5 x 12 heads x 8 query tiles -- a launch that is on the chip at once and takes the host-made block order with a
+    number of batch entries that is no multiple of 8.  The same numbers laid out densely [60, T, 64] give the same bits."""
+    rng = np.random.default_rng(77)
+    B, H, T, D = 5, 12, 1024, 64
+    d = H * D
+    qkv = rng.normal(0, 1, (B, T, 3 * d)).astype(np.float32)
+    _, Q = _store(qkv, dt)
+    qkv_r = Q.to_float().reshape(B, T, 3, H, D)
+    att = NDArray.empty((B, T, d), dt)
+    views = [Q.view((B, H, T, D), (T * 3 * d, D, 3 * d, 1), which * d) for which in range(3)]
+    o4 = att.view((B, H, T, D), (T * d, D, d, 1), 0)
+    ex.exec_custom("dot_product_attention_v2", [views[0], views[2], views[1]], [o4], t_args=[0.125, 0.0], b_args=[True, False])
+    got = att.to_float().reshape(B, T, H, D).transpose(0, 2, 1, 3).reshape(B * H, T, D)
+    dense = [NDArray.from_numpy(np.ascontiguousarray(qkv_r[:, :, which].transpose(0, 2, 1, 3).reshape(B * H, T, D)), dt) for which in range(3)]
+    want = ex.exec_custom("dot_product_attention_v2", [dense[0], dense[2], dense[1]], [NDArray.empty((B * H, T, D), dt)], t_args=[0.125, 0.0],
+                          b_args=[True, False])[0].to_float()
+    assert np.isfinite(got).all() and np.array_equal(got, want)
+    v = qkv_r[:, :, 2].transpose(0, 2, 1, 3).reshape(B * H, T, D)
+    tol = 1e-4 if dt == FLOAT32 else 1e-2
+    assert_close(got[:, 0], v[:, 0], tol, tol, "query 0")
+
+
 @pytest.mark.parametrize("dt", [HALF, BFLOAT16])
 def test_config4_weights_and_logits_outputs(ex, oracle, dt):
     """The same op with its second and third outputs requested (attention weights and clipped, masked logits) at the
