@@ -881,7 +881,10 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16f(GemmArgs g, const T
 // Two LDS stages of 64 KiB.  Per K-tile: k-steps 0..2 prefetch the next step's fragments; k-step 3 runs half of its
 // MFMAs, waits for the direct loads of tile kt+1, meets the barrier, then reads the first fragments of tile kt+1 and
 // issues the direct loads of tile kt+2 into the stage that was just drained.
-template <typename T, bool B_KC>
+// EDGE: M and N need not be whole tiles.  The direct loads of the last tile row / column take their rows (their 16-byte
+// column groups of a row-major B) from clamped positions inside the operand -- what they bring in only ever reaches
+// elements of C beyond the edge, which the bounds-checked store leaves out.
+template <typename T, bool B_KC, bool EDGE = false>
 __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
                                                     unsigned tilesM, unsigned tilesN) {
   constexpr int BM = 256, BN = 256, BK = 64, WN = 4, WTM = 128, WTN = 64, TM = 4, TN = 2, NM = TM * TN;
@@ -911,12 +914,18 @@ __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restr
   for (int i = 0; i < 4; i++) {
     const int cw = wave * 4 + i;
     const int lkg = (lp - 4 * (cw & 1) - (lj >> 1)) & 7;
-    aSrc[i] = A + (m0 + cw * 8 + lj) * lda + lkg * 8;
+    LongType ar = m0 + cw * 8 + lj;
+    if (EDGE) ar = ar < g.M ? ar : g.M - 1;
+    aSrc[i] = A + ar * lda + lkg * 8;
     if (B_KC) {
-      bSrc[i] = B + (n0 + cw * 8 + lj) * ldb + lkg * 8;
+      LongType br = n0 + cw * 8 + lj;
+      if (EDGE) br = br < g.N ? br : g.N - 1;
+      bSrc[i] = B + br * ldb + lkg * 8;
     } else {
       const int kr = 2 * cw + (lane >> 5), q = lane & 31, c = q ^ (4 * (kr & 3));
-      bSrc[i] = B + (LongType)kr * ldb + n0 + 8 * c;
+      LongType bc = n0 + 8 * c;
+      if (EDGE) bc = bc + 8 <= g.N ? bc : g.N - 8;
+      bSrc[i] = B + (LongType)kr * ldb + bc;
     }
   }
   const LongType aStep = BK, bStep = B_KC ? (LongType)BK : (LongType)BK * ldb;
@@ -1066,7 +1075,8 @@ __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restr
     }
   }
 
-  storeAccTiles<T, TM, TN, false>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
+  if (EDGE && (m0 + BM > g.M || n0 + BN > g.N)) storeAccTiles<T, TM, TN, true>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
+  else storeAccTiles<T, TM, TN, false>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);   // a whole tile, also of a ragged product
 }
 
 // The same 256 x 256 tile for A k-contiguous and B row-major with the operands in two RINGS of LDS units instead of two
@@ -1086,7 +1096,8 @@ __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restr
 // when the barrier that certifies it is reached: s_waitcnt vmcnt(4) in front of every barrier (loads complete in
 // order).  The loop is branch-free: past the end of K the pointers stop advancing, so the surplus loads re-read the
 // last unit into slots nobody reads any more.  K must be a multiple of 128 (four steps per loop iteration).
-template <typename T>
+// EDGE as in gemm_mfma16d: clamped loads and a bounds-checked store for an M or N that is not a whole number of tiles.
+template <typename T, bool EDGE = false>
 __global__ __launch_bounds__(512) void gemm_mfma16r(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
                                                     unsigned tilesM, unsigned tilesN) {
   constexpr int BM = 256, BN = 256, WN = 4, WTM = 128, WTN = 64, TM = 4, TN = 2, NM = TM * TN;
@@ -1114,12 +1125,16 @@ __global__ __launch_bounds__(512) void gemm_mfma16r(GemmArgs g, const T* __restr
   for (int i = 0; i < 4; i++) {
     const int cw = wave * 4 + i;                          // 8 rows, all 8 k-groups of the unit
     const int lkg = (lp - 4 * (cw & 1) - (lj >> 1)) & 7;
-    aSrc[i] = A + (m0 + cw * 8 + lj) * lda + lkg * 8;
+    LongType ar = m0 + cw * 8 + lj;
+    if (EDGE) ar = ar < g.M ? ar : g.M - 1;
+    aSrc[i] = A + ar * lda + lkg * 8;
   }
 #pragma unroll
   for (int c = 0; c < 2; c++) {
     const int kr = 2 * (wave * 2 + c) + (lane >> 5), q = lane & 31;   // two k-rows of 256 n per chunk
-    bSrc[c] = B + (LongType)kr * ldb + n0 + 8 * (q ^ (4 * (kr & 3)));
+    LongType bc = n0 + 8 * (q ^ (4 * (kr & 3)));
+    if (EDGE) bc = bc + 8 <= g.N ? bc : g.N - 8;
+    bSrc[c] = B + (LongType)kr * ldb + bc;
   }
   const int S = (int)(g.K / 32), nA = (int)(g.K / 64);   // steps, A units
   const LongType aStep = 64, bStep = 32 * ldb;
@@ -1255,7 +1270,8 @@ __global__ __launch_bounds__(512) void gemm_mfma16r(GemmArgs g, const T* __restr
   mainLoop(std::integral_constant<int, 0>{}, std::integral_constant<int, 2>{});
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the surplus loads of the last steps
 
-  storeAccTiles<T, TM, TN, false>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
+  if (EDGE && (m0 + BM > g.M || n0 + BN > g.N)) storeAccTiles<T, TM, TN, true>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
+  else storeAccTiles<T, TM, TN, false>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);   // a whole tile, also of a ragged product
 }
 
 // ---- 16-bit MFMA kernel for operands the vector loaders cannot take ---------------------------------------------------------
@@ -1478,27 +1494,57 @@ static bool launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const 
   if (g.M <= 64 || g.N <= 64 || tiles128 < 192) return launchMfma16Cfg<T, 64, 64, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch, true, aligned);
   if (tiles256 < 192) return launchMfma16Cfg<T, 128, 128, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch, false, aligned);
   if (g.hasEpi) return false;
+  if constexpr (A_KC && !B_KC) {
+    // A row-major B whose rows start off 16-byte boundaries (a [768, 50257] matrix) with everything else in place for the
+    // ring kernel: its loads into LDS take element-aligned addresses like any other global load, and every column group
+    // of 8 is whole up to the last multiple of 8 -- the edge instantiation over those columns, then the up to 7 columns
+    // that are left through the bounds-handling kernel (bf16 4096 x 50257 x 768: 0.71 -> 0.40 ms)
+    static const bool ub = getenv("ND4JHIP_GEMM_UNALIGNED_RING") ? atoi(getenv("ND4JHIP_GEMM_UNALIGNED_RING")) != 0 : true;
+    constexpr size_t LDS = (3 * 256 * 8 + 4 * 32 * 32) * 16;
+    if (!aligned && ub && batch == 1 && (reinterpret_cast<uintptr_t>(A) & 15) == 0 && g.aRow % 8 == 0 && g.K % 128 == 0 && g.N >= 264 &&
+        DynLds<gemm_mfma16r<T, true>, (int)LDS>::granted()) {
+      GemmArgs g1 = g;
+      g1.N = g.N & ~(LongType)7;
+      const unsigned tM = (unsigned)((g.M + 255) / 256), tN = (unsigned)((g1.N + 255) / 256);
+      auto kern = gemm_mfma16r<T, true>;
+      hipLaunchKernelGGL(kern, dim3(tM * tN, 1, 1), dim3(512), LDS, s, g1, (const T*)A, (const T*)B, (T*)C, tM, tN);
+      const LongType rem = g.N & 7;
+      if (rem) {
+        GemmArgs g2 = g;
+        g2.N = rem;
+        if (g.bias) g2.bias = static_cast<const T*>(g.bias) + g1.N;
+        if (!launchMfma16Cfg<T, 64, 64, 2, 2, A_KC, B_KC>(s, g2, A, (const T*)B + g1.N, (T*)C + g1.N * g.cCol, 1, false, false)) return false;
+      }
+      noteKernel("gemm_mfma16r<%s,256x256,akc=1,bkc=0,edge,unaligned>", tname<T>());
+      return true;
+    }
+  }
   if (!aligned) return launchMfma16Cfg<T, 256, 256, 2, 4, A_KC, B_KC>(s, g, A, B, C, batch, false, false);
   static const bool direct = getenv("ND4JHIP_GEMM_DIRECT") ? atoi(getenv("ND4JHIP_GEMM_DIRECT")) != 0 : true;
   static const bool ring = getenv("ND4JHIP_GEMM_RING") ? atoi(getenv("ND4JHIP_GEMM_RING")) != 0 : true;
+  // the direct-load kernels take an M or N that is not a whole number of tiles through their edge instantiations (a
+  // row-major B in whole 16-byte column groups only)
+  static const bool edge = getenv("ND4JHIP_GEMM_EDGE") ? atoi(getenv("ND4JHIP_GEMM_EDGE")) != 0 : true;
+  const bool whole = g.M % 256 == 0 && g.N % 256 == 0;
+  const bool edgeOk = whole || (edge && (B_KC || g.N % 8 == 0));
+  const unsigned tM = (unsigned)((g.M + 255) / 256), tN = (unsigned)((g.N + 255) / 256);
   if constexpr (A_KC && !B_KC) {
     constexpr size_t LDS = (3 * 256 * 8 + 4 * 32 * 32) * 16;   // 160 KiB: the whole LDS of a CU
-    auto kern = gemm_mfma16r<T>;
     // a device or driver that does not grant a block the whole LDS keeps the two-stage kernel below
-    const bool ringGranted = DynLds<gemm_mfma16r<T>, (int)LDS>::granted();
-    if (direct && ring && ringGranted && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 128 == 0) {
-      const unsigned tM = (unsigned)(g.M / 256), tN = (unsigned)(g.N / 256);
-      noteKernel("gemm_mfma16r<%s,256x256,akc=1,bkc=0>", tname<T>());
+    const bool ringGranted = whole ? DynLds<gemm_mfma16r<T>, (int)LDS>::granted() : DynLds<gemm_mfma16r<T, true>, (int)LDS>::granted();
+    if (direct && ring && ringGranted && edgeOk && g.K % 128 == 0) {
+      noteKernel("gemm_mfma16r<%s,256x256,akc=1,bkc=0%s>", tname<T>(), whole ? "" : ",edge");
+      auto kern = whole ? gemm_mfma16r<T, false> : gemm_mfma16r<T, true>;
       hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(512), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
       return true;
     }
   }
-  if (direct && A_KC && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 64 == 0 && g.K >= 128) {
+  if (direct && A_KC && edgeOk && g.K % 64 == 0 && g.K >= 128) {
     constexpr size_t LDS = 2 * 2 * 256 * 8 * 16;
-    auto kern = gemm_mfma16d<T, B_KC>;
-    ND4J_REQUIRE((DynLds<gemm_mfma16d<T, B_KC>, (int)LDS>::granted()), "matmul: the device does not grant the two-stage kernel its LDS");
-    const unsigned tM = (unsigned)(g.M / 256), tN = (unsigned)(g.N / 256);
-    noteKernel("gemm_mfma16d<%s,256x256,akc=1,bkc=%d>", tname<T>(), (int)B_KC);
+    const bool granted = whole ? DynLds<gemm_mfma16d<T, B_KC>, (int)LDS>::granted() : DynLds<gemm_mfma16d<T, B_KC, true>, (int)LDS>::granted();
+    ND4J_REQUIRE(granted, "matmul: the device does not grant the two-stage kernel its LDS");
+    noteKernel("gemm_mfma16d<%s,256x256,akc=1,bkc=%d%s>", tname<T>(), (int)B_KC, whole ? "" : ",edge");
+    auto kern = whole ? gemm_mfma16d<T, B_KC, false> : gemm_mfma16d<T, B_KC, true>;
     hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(512), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
     return true;
   }

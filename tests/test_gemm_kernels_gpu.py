@@ -76,6 +76,11 @@ CASES = [
     (HALF, 2048, 2048, 320, "gemm_mfma16f<f16,128x128,akc=1,bkc=0>", "gemm_mfma16f<f16,128x128,akc=1,bkc=1>", None),
     # ragged edges on the large tiles (bounds-handling kernel)
     (BFLOAT16, 3600, 3704, 1000, "gemm_mfma16p<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16p<bf16,256x256,akc=1,bkc=1>", "gemm_mfma16p<bf16,256x256,akc=0,bkc=0>"),
+    # ragged edges with aligned rows and a K of whole K-tiles: the direct-load kernels' edge instantiations (clamped loads,
+    # bounds-checked store) -- a last tile row of 16 rows and a last tile column of 120, of 8 (one column group) and of 1
+    (BFLOAT16, 3600, 3704, 1024, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0,edge>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1,edge>", "gemm_mfma16p<bf16,256x256,akc=0,bkc=0>"),
+    (HALF, 3599, 3592, 192, "gemm_mfma16d<f16,256x256,akc=1,bkc=0,edge>", "gemm_mfma16d<f16,256x256,akc=1,bkc=1,edge>", None),
+    (BFLOAT16, 3601, 3585, 256, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0,edge,unaligned>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1,edge>", None),
     (HALF, 1800, 1800, 520, "gemm_mfma16p<f16,128x128,akc=1,bkc=0>", "gemm_mfma16p<f16,128x128,akc=1,bkc=1>", None),
     (BFLOAT16, 1104, 904, 1000, "gemm_mfma16p<bf16,64x64,akc=1,bkc=0>", "gemm_mfma16p<bf16,64x64,akc=1,bkc=1>", None),
     # K a multiple of 256 but not of 512: the four-stage ring; more tiles than CUs (two blocks on a CU): four stages as well;
@@ -93,7 +98,7 @@ CASES = [
     # bounds-handling kernels read element-aligned vectors -- a batched decode step's logits against the row-major
     # [768, 50257] embedding, a prefill's, and a product with nothing aligned in any layout
     (BFLOAT16, 32, 50257, 768, "gemm_mfma16p<bf16,32x128,akc=1,bkc=0>", "gemm_mfma16p<bf16,32x128,akc=1,bkc=1>", None),
-    (BFLOAT16, 1024, 50257, 768, "gemm_mfma16p<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16p<bf16,256x256,akc=1,bkc=1>", None),
+    (BFLOAT16, 1024, 50257, 768, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0,edge,unaligned>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1,edge>", None),
     (HALF, 1000, 1003, 515, "gemm_mfma16p<f16,64x64,akc=1,bkc=0>", "gemm_mfma16p<f16,64x64,akc=1,bkc=1>", "gemm_mfma16p<f16,64x64,akc=0,bkc=0>"),
     (BFLOAT16, 2001, 1999, 1003, "gemm_mfma16p<bf16,128x128,akc=1,bkc=0>", "gemm_mfma16p<bf16,128x128,akc=1,bkc=1>", "gemm_mfma16p<bf16,128x128,akc=0,bkc=0>"),
     (HALF, 20, 4097, 2051, "gemm_mfma16<f16,32x128,akc=1,bkc=0>+splitk_finish", "gemm_mfma16<f16,32x128,akc=1,bkc=1>+splitk_finish", None),
@@ -126,6 +131,24 @@ def test_matmul_kernel_at_real_shape(ex, dtype, M, N, K, kern_plain, kern_tb, ke
         za = _run(ex, At, B, [1, 0], kern_ta)
         _check_rows_cols(za, a64, b64, tol, rng, "transposeA")
         assert_close(za, z, tol, tol, "transposeA agrees with plain A over the whole result")
+
+
+@pytest.mark.parametrize("dtype,M,N,K", [(BFLOAT16, 3600, 3705, 256), (HALF, 3599, 3591, 128), (BFLOAT16, 3585, 3704, 384)],
+                         ids=["bf16-rows-off-by-one", "f16-seven-columns-left", "bf16-aligned-ragged"])
+def test_ragged_product_on_the_direct_load_kernels_whole_result(ex, dtype, M, N, K):
+    """The edge instantiations of the direct-load kernels, every element of the result: a row-major B with rows of 3705
+    (every row starts 2 bytes further off a 16-byte boundary; one column is left for the bounds-handling kernel), of 3591
+    (seven columns left), and an aligned B with a ragged last tile row and column."""
+    rng = np.random.default_rng(M + N + K)
+    a = rng.normal(0, 1 / math.sqrt(K), (M, K)).astype(np.float32)
+    b = rng.normal(0, 1 / math.sqrt(K), (K, N)).astype(np.float32)
+    A, a64 = _device(a, dtype)
+    B, b64 = _device(b, dtype)
+    z = ex.exec_custom("matmul", [A, B])[0].to_float()
+    name = _last_kernel(ex)
+    assert ",edge" in name, name
+    assert ("unaligned" in name) == (N % 8 != 0), name
+    assert_close(z, a64 @ b64, TOL[dtype], TOL[dtype], "whole result")
 
 
 @pytest.mark.parametrize("n", [1024, 4096])
