@@ -611,7 +611,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16q(GemmArgs g, const T
 // row-major B, swizzled as RowTileLoader keeps them and read with the transposing LDS read.  Round kt: wait for tile kt + 1
 // (this wave's chunks), barrier (everybody's), refill the stage tile kt - 1 left, read the fragments of tile kt + 1 while the
 // MFMAs of tile kt run.
-template <typename T, bool B_KC, int NST, int TW>
+// EDGE: M and N need not be whole tiles -- rows (16-byte column groups of a row-major B) beyond the edge are read from
+// clamped positions inside the operand and only reach elements of C that the bounds-checked store leaves out.
+template <typename T, bool B_KC, int NST, int TW, bool EDGE = false>
 __global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
                                                     unsigned tilesM, unsigned tilesN) {
   constexpr int BM = 64 * TW, BN = 64 * TW, BK = 64;
@@ -635,12 +637,18 @@ __global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restr
   for (int c = 0; c < CPW; c++) {
     const int cw = wave * CPW + c, lj = lane >> 3, lp = lane & 7;
     const int lkg = (lp - 4 * (cw & 1) - (lj >> 1)) & 7;
-    offA[c] = (unsigned)(((LongType)(cw * 8 + lj) * lda + lkg * 8) * 2);
+    LongType ar = cw * 8 + lj;
+    if (EDGE) ar = m0 + ar < g.M ? ar : g.M - 1 - m0;
+    offA[c] = (unsigned)((ar * lda + lkg * 8) * 2);
     if (B_KC) {
-      offB[c] = (unsigned)(((LongType)(cw * 8 + lj) * ldb + lkg * 8) * 2);
+      LongType br = cw * 8 + lj;
+      if (EDGE) br = n0 + br < g.N ? br : g.N - 1 - n0;
+      offB[c] = (unsigned)((br * ldb + lkg * 8) * 2);
     } else {
       const int k = cw * (64 / RowB::SPR) + lane / RowB::SPR, pp = lane % RowB::SPR;
-      offB[c] = (unsigned)(((LongType)k * ldb + (pp ^ RowB::swz(k)) * 8) * 2);
+      LongType bc = (pp ^ RowB::swz(k)) * 8;
+      if (EDGE) bc = n0 + bc + 8 <= g.N ? bc : g.N - 8 - n0;
+      offB[c] = (unsigned)(((LongType)k * ldb + bc) * 2);
     }
   }
   const char* const baseA = reinterpret_cast<const char*>(A + m0 * lda);
@@ -719,7 +727,8 @@ __global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restr
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the surplus loads of the last rounds
-  storeAccTiles<T, TW, TW, false>(g, C, acc, m0 + wm * 32 * TW, n0 + wn * 32 * TW, lane);
+  if (EDGE && (m0 + BM > g.M || n0 + BN > g.N)) storeAccTiles<T, TW, TW, true>(g, C, acc, m0 + wm * 32 * TW, n0 + wn * 32 * TW, lane);
+  else storeAccTiles<T, TW, TW, false>(g, C, acc, m0 + wm * 32 * TW, n0 + wn * 32 * TW, lane);
 }
 
 // Steady-state kernel for problems made of whole tiles (M % BM == 0, N % BN == 0, K % 64 == 0): no bounds handling,
@@ -1404,10 +1413,16 @@ static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
   // split-K plus its finishing launch even with a quarter of the CUs busy (bf16 512^3 4.5 against 11.2 us, 768^3 4.7 against
   // 12.0, 512 x 512 x 2048 7.7 against 13.0; from K = 4096 on the split wins: 256 x 256 x 4096 10.4 against 11.9)
   bool ringInstead = false;
+  // the ring kernel's edge instantiation takes an M or N that is not a whole number of tiles (a row-major B in whole
+  // 16-byte column groups)
+  static const bool edge = getenv("ND4JHIP_GEMM_EDGE") ? atoi(getenv("ND4JHIP_GEMM_EDGE")) != 0 : true;
+  const bool whole = g.M % BM == 0 && g.N % BN == 0;
+  const bool edgeOk = whole || (edge && (B_KC || g.N % 8 == 0));
   if constexpr (BM == 64 && BN == 64 && WM == 2 && WN == 2 && A_KC) {
     static const bool small = getenv("ND4JHIP_GEMM_SMALL_RING") ? atoi(getenv("ND4JHIP_GEMM_SMALL_RING")) != 0 : true;
     const LongType ldaS = g.aRow, ldbS = B_KC ? g.bCol : g.bRow;
-    ringInstead = small && g.K >= 512 && g.K <= 2048 && g.K % 256 == 0 && g.M % BM == 0 && g.N % BN == 0 && (g.M / BM) * (g.N / BN) * batch <= 1024 &&
+    ringInstead = small && g.K >= 512 && g.K <= 2048 && g.K % 256 == 0 && edgeOk && (whole || aligned) &&
+                  ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN) * batch <= 1024 &&
                   ldaS % 8 == 0 && ldbS % 8 == 0 && ldaS < (1 << 23) && ldbS < (1 << 23) &&
                   ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 && g.aBatch % 8 == 0 && g.bBatch % 8 == 0 &&
                   g.aBatch2 % 8 == 0 && g.bBatch2 % 8 == 0 && !g.hasEpi;
@@ -1436,26 +1451,28 @@ static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
     constexpr int STAGE_BYTES = (BM + BN) * 8 * 16;
     static const bool small = getenv("ND4JHIP_GEMM_SMALL_RING") ? atoi(getenv("ND4JHIP_GEMM_SMALL_RING")) != 0 : true;
     const LongType ldaS = g.aRow, ldbS = B_KC ? g.bCol : g.bRow;
-    const bool shape = TW == 1 ? useDeep : (useFull && nTiles <= 1024 && g.K >= 512 && g.K % 256 == 0);
+    const bool edgeShape = !whole && edgeOk && aligned && usePipe && nTiles <= 1024 && g.K >= 512 && g.K % 256 == 0;
+    const bool shape = edgeShape || (TW == 1 ? useDeep : (useFull && nTiles <= 1024 && g.K >= 512 && g.K % 256 == 0));
     if (small && shape && ldaS % 8 == 0 && ldbS % 8 == 0 && ldaS < (1 << 23) && ldbS < (1 << 23) &&
         ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 && g.aBatch % 8 == 0 && g.bBatch % 8 == 0 &&
         g.aBatch2 % 8 == 0 && g.bBatch2 % 8 == 0) {
-      const unsigned tM = (unsigned)(g.M / BM), tN = (unsigned)(g.N / BN);
+      const unsigned tM = (unsigned)((g.M + BM - 1) / BM), tN = (unsigned)((g.N + BN - 1) / BN);
       // 64 x 64: one tile per CU and a K of whole eight-tile rounds take eight stages (128 KiB), else four (two blocks fit a
       // CU); 128 x 128: four stages (128 KiB)
       constexpr int DEEP = TW == 1 ? 8 : 4;
       const bool wantDeep = TW == 2 || (nTiles <= 256 && g.K % 512 == 0);
-      const bool grantedDeep = DynLds<gemm_mfma16s<T, B_KC, DEEP, TW>, DEEP * STAGE_BYTES>::granted();
+      const bool grantedDeep = whole ? DynLds<gemm_mfma16s<T, B_KC, DEEP, TW>, DEEP * STAGE_BYTES>::granted()
+                                     : DynLds<gemm_mfma16s<T, B_KC, DEEP, TW, true>, DEEP * STAGE_BYTES>::granted();
       if (wantDeep && grantedDeep) {
-        noteKernel("gemm_mfma16s<%s,%dx%d,akc=1,bkc=%d,stages=%d>", tname<T>(), BM, BN, (int)B_KC, DEEP);
-        hipLaunchKernelGGL((gemm_mfma16s<T, B_KC, DEEP, TW>), dim3(tM * tN, 1, (unsigned)batch), dim3(256), DEEP * STAGE_BYTES, s, g, (const T*)A,
-                           (const T*)B, (T*)C, tM, tN);
+        noteKernel("gemm_mfma16s<%s,%dx%d,akc=1,bkc=%d,stages=%d%s>", tname<T>(), BM, BN, (int)B_KC, DEEP, whole ? "" : ",edge");
+        auto kern = whole ? gemm_mfma16s<T, B_KC, DEEP, TW, false> : gemm_mfma16s<T, B_KC, DEEP, TW, true>;
+        hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(256), DEEP * STAGE_BYTES, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
         return true;
       }
       if constexpr (TW == 1) {
-        noteKernel("gemm_mfma16s<%s,64x64,akc=1,bkc=%d,stages=4>", tname<T>(), (int)B_KC);
-        hipLaunchKernelGGL((gemm_mfma16s<T, B_KC, 4, 1>), dim3(tM * tN, 1, (unsigned)batch), dim3(256), 4 * STAGE_BYTES, s, g, (const T*)A, (const T*)B,
-                           (T*)C, tM, tN);
+        noteKernel("gemm_mfma16s<%s,64x64,akc=1,bkc=%d,stages=4%s>", tname<T>(), (int)B_KC, whole ? "" : ",edge");
+        auto kern = whole ? gemm_mfma16s<T, B_KC, 4, 1, false> : gemm_mfma16s<T, B_KC, 4, 1, true>;
+        hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(256), 4 * STAGE_BYTES, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
         return true;
       }
     }

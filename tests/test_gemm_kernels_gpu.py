@@ -81,6 +81,9 @@ CASES = [
     (BFLOAT16, 3600, 3704, 1024, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0,edge>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1,edge>", "gemm_mfma16p<bf16,256x256,akc=0,bkc=0>"),
     (HALF, 3599, 3592, 192, "gemm_mfma16d<f16,256x256,akc=1,bkc=0,edge>", "gemm_mfma16d<f16,256x256,akc=1,bkc=1,edge>", None),
     (BFLOAT16, 3601, 3585, 256, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0,edge,unaligned>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1,edge>", None),
+    (BFLOAT16, 2000, 2000, 2048, "gemm_mfma16s<bf16,128x128,akc=1,bkc=0,stages=4,edge>", "gemm_mfma16s<bf16,128x128,akc=1,bkc=1,stages=4,edge>", None),
+    (HALF, 1000, 1000, 1024, "gemm_mfma16s<f16,64x64,akc=1,bkc=0,stages=8,edge>", "gemm_mfma16s<f16,64x64,akc=1,bkc=1,stages=8,edge>", None),
+    (BFLOAT16, 500, 2304, 768, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=4,edge>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=4,edge>", None),
     (HALF, 1800, 1800, 520, "gemm_mfma16p<f16,128x128,akc=1,bkc=0>", "gemm_mfma16p<f16,128x128,akc=1,bkc=1>", None),
     (BFLOAT16, 1104, 904, 1000, "gemm_mfma16p<bf16,64x64,akc=1,bkc=0>", "gemm_mfma16p<bf16,64x64,akc=1,bkc=1>", None),
     # K a multiple of 256 but not of 512: the four-stage ring; more tiles than CUs (two blocks on a CU): four stages as well;
@@ -133,8 +136,9 @@ def test_matmul_kernel_at_real_shape(ex, dtype, M, N, K, kern_plain, kern_tb, ke
         assert_close(za, z, tol, tol, "transposeA agrees with plain A over the whole result")
 
 
-@pytest.mark.parametrize("dtype,M,N,K", [(BFLOAT16, 3600, 3705, 256), (HALF, 3599, 3591, 128), (BFLOAT16, 3585, 3704, 384)],
-                         ids=["bf16-rows-off-by-one", "f16-seven-columns-left", "bf16-aligned-ragged"])
+@pytest.mark.parametrize("dtype,M,N,K", [(BFLOAT16, 3600, 3705, 256), (HALF, 3599, 3591, 128), (BFLOAT16, 3585, 3704, 384),
+                                         (BFLOAT16, 499, 2312, 768), (HALF, 1921, 1928, 512)],
+                         ids=["bf16-rows-off-by-one", "f16-seven-columns-left", "bf16-aligned-ragged", "bf16-64x64-tiles", "f16-128x128-tiles"])
 def test_ragged_product_on_the_direct_load_kernels_whole_result(ex, dtype, M, N, K):
     """The edge instantiations of the direct-load kernels, every element of the result: a row-major B with rows of 3705
     (every row starts 2 bytes further off a 16-byte boundary; one column is left for the bounds-handling kernel), of 3591
