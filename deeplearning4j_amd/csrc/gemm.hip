@@ -1696,8 +1696,10 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32(GemmArgs g, const fl
 // register sets, the K loop unrolled PD times and free of branches -- loads past the end re-read the last K-tile, the
 // store after the last K-tile fills a stage nobody reads), so the loop runs at the MFMA rate instead of one memory
 // latency per K-tile.  BK = 32 halves the barriers per MFMA (the one-tile-per-CU launch, where nothing else covers
-// them).  Host: M % BM == 0, N % BN == 0, K % (BK * PD) == 0, K >= 2 * BK * PD.
-template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int PD, int BK>
+// them).  Host: K % (BK * PD) == 0, K >= 2 * BK * PD; M % BM == 0 and N % BN == 0 unless EDGE: then the rows (the 16-byte
+// groups along M or N of an operand that is contiguous that way) beyond the edge are read from clamped positions inside the
+// operand and only reach elements of C that the bounds-checked store leaves out.
+template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int PD, int BK, bool EDGE = false>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32q(GemmArgs g, const float* __restrict__ A, const float* __restrict__ B,
                                                               float* __restrict__ C, unsigned tilesM, unsigned tilesN) {
   static_assert(PD % 2 == 0, "the LDS stage of a K-tile must be a compile-time constant inside the unrolled loop");
@@ -1733,12 +1735,16 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32q(GemmArgs g, const f
 #pragma unroll
   for (int i = 0; i < VA; i++) {
     const int v = t + i * NT;
-    curA[i] = (GlobalBytes)(A_KC ? A + (m0 + v / KQ) * lda + (v % KQ) * 4 : A + (LongType)(v / (BM / 4)) * lda + m0 + (v % (BM / 4)) * 4);
+    LongType am = A_KC ? m0 + v / KQ : m0 + (v % (BM / 4)) * 4;
+    if (EDGE) am = A_KC ? (am < g.M ? am : g.M - 1) : (am + 4 <= g.M ? am : g.M - 4);
+    curA[i] = (GlobalBytes)(A_KC ? A + am * lda + (v % KQ) * 4 : A + (LongType)(v / (BM / 4)) * lda + am);
   }
 #pragma unroll
   for (int i = 0; i < VB; i++) {
     const int v = t + i * NT;
-    curB[i] = (GlobalBytes)(B_KC ? B + (n0 + v / KQ) * ldb + (v % KQ) * 4 : B + (LongType)(v / (BN / 4)) * ldb + n0 + (v % (BN / 4)) * 4);
+    LongType bn = B_KC ? n0 + v / KQ : n0 + (v % (BN / 4)) * 4;
+    if (EDGE) bn = B_KC ? (bn < g.N ? bn : g.N - 1) : (bn + 4 <= g.N ? bn : g.N - 4);
+    curB[i] = (GlobalBytes)(B_KC ? B + bn * ldb + (v % KQ) * 4 : B + (LongType)(v / (BN / 4)) * ldb + bn);
   }
   const LongType KT = g.K / BK;
   const LongType stepA = (A_KC ? BK : BK * lda) * 4, stepB = (B_KC ? BK : BK * ldb) * 4;   // bytes per K-tile
@@ -1843,7 +1849,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32q(GemmArgs g, const f
       for (int j = 0; j < TN; j++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[i][j][r] += acc2[i][j][r];
-    storeAccTiles<float, TM, TN, false>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
+    if (EDGE && (m0 + BM > g.M || n0 + BN > g.N)) storeAccTiles<float, TM, TN, true>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
+    else storeAccTiles<float, TM, TN, false>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
     return;
   }
   for (LongType kt0 = 0; kt0 < KT; kt0 += PD) {
@@ -1868,17 +1875,22 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32q(GemmArgs g, const f
       __syncthreads();
     }
   }
-  storeAccTiles<float, TM, TN, false>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
+  if (EDGE && (m0 + BM > g.M || n0 + BN > g.N)) storeAccTiles<float, TM, TN, true>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
+  else storeAccTiles<float, TM, TN, false>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
 }
 
 template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC>
 static void launchMfma32Cfg(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C, LongType batch, bool aligned) {
   const unsigned tilesM = (unsigned)((g.M + BM - 1) / BM), tilesN = (unsigned)((g.N + BN - 1) / BN);
-  if (aligned && g.K >= 256 && g.M % BM == 0 && g.N % BN == 0 && g.K % 128 == 0) {
+  static const bool edge = getenv("ND4JHIP_GEMM_EDGE") ? atoi(getenv("ND4JHIP_GEMM_EDGE")) != 0 : true;
+  const bool whole = g.M % BM == 0 && g.N % BN == 0;
+  // `aligned` says that an operand which is contiguous along M or N has an extent of whole 16-byte groups
+  if (aligned && g.K >= 256 && (whole || (edge && g.M >= 4 && g.N >= 4)) && g.K % 128 == 0) {
     constexpr int PD = 4, BK = BM * BN <= 64 * 64 ? 32 : 16;
-    noteKernel("gemm_mfma32q<f32,%dx%d,akc=%d,bkc=%d,pd=%d,bk=%d>", BM, BN, (int)A_KC, (int)B_KC, PD, BK);
-    hipLaunchKernelGGL((gemm_mfma32q<BM, BN, WM, WN, A_KC, B_KC, PD, BK>), dim3(tilesM * tilesN, 1, (unsigned)batch), dim3(WM * WN * 64), 0, s, g,
-                       (const float*)A, (const float*)B, (float*)C, tilesM, tilesN);
+    noteKernel("gemm_mfma32q<f32,%dx%d,akc=%d,bkc=%d,pd=%d,bk=%d%s>", BM, BN, (int)A_KC, (int)B_KC, PD, BK, whole ? "" : ",edge");
+    auto kern = whole ? gemm_mfma32q<BM, BN, WM, WN, A_KC, B_KC, PD, BK, false> : gemm_mfma32q<BM, BN, WM, WN, A_KC, B_KC, PD, BK, true>;
+    hipLaunchKernelGGL(kern, dim3(tilesM * tilesN, 1, (unsigned)batch), dim3(WM * WN * 64), 0, s, g, (const float*)A, (const float*)B, (float*)C,
+                       tilesM, tilesN);
     return;
   }
   noteKernel("gemm_mfma32<f32,%dx%d,akc=%d,bkc=%d>", BM, BN, (int)A_KC, (int)B_KC);

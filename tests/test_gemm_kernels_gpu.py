@@ -108,6 +108,9 @@ CASES = [
     # the same for fp32 (row lengths that are not multiples of 4)
     (FLOAT32, 1000, 1003, 515, "gemm_mfma32<f32,64x64,akc=1,bkc=0>", "gemm_mfma32<f32,64x64,akc=1,bkc=1>", "gemm_mfma32<f32,64x64,akc=0,bkc=0>"),
     (FLOAT32, 257, 50257, 770, "gemm_mfma32<f32,128x128,akc=1,bkc=0>", "gemm_mfma32<f32,128x128,akc=1,bkc=1>", None),
+    # fp32 ragged with aligned rows and a K of whole rounds: the edge instantiation of the deep-pipeline kernel
+    (FLOAT32, 1000, 1000, 1024, "gemm_mfma32q<f32,64x64,akc=1,bkc=0,pd=4,bk=32,edge>", "gemm_mfma32q<f32,64x64,akc=1,bkc=1,pd=4,bk=32,edge>", "gemm_mfma32q<f32,64x64,akc=0,bkc=0,pd=4,bk=32,edge>"),
+    (FLOAT32, 2004, 2000, 512, "gemm_mfma32q<f32,128x128,akc=1,bkc=0,pd=4,bk=16,edge>", "gemm_mfma32q<f32,128x128,akc=1,bkc=1,pd=4,bk=16,edge>", "gemm_mfma32q<f32,128x128,akc=0,bkc=0,pd=4,bk=16,edge>"),
     # fp32 ragged
     (FLOAT32, 1100, 900, 1000, "gemm_mfma32<f32,64x64,akc=1,bkc=0>", "gemm_mfma32<f32,64x64,akc=1,bkc=1>", None),
     (FLOAT32, 2100, 2052, 520, "gemm_mfma32<f32,128x128,akc=1,bkc=0>", "gemm_mfma32<f32,128x128,akc=1,bkc=1>", "gemm_mfma32<f32,128x128,akc=0,bkc=0>"),
@@ -137,8 +140,9 @@ def test_matmul_kernel_at_real_shape(ex, dtype, M, N, K, kern_plain, kern_tb, ke
 
 
 @pytest.mark.parametrize("dtype,M,N,K", [(BFLOAT16, 3600, 3705, 256), (HALF, 3599, 3591, 128), (BFLOAT16, 3585, 3704, 384),
-                                         (BFLOAT16, 499, 2312, 768), (HALF, 1921, 1928, 512)],
-                         ids=["bf16-rows-off-by-one", "f16-seven-columns-left", "bf16-aligned-ragged", "bf16-64x64-tiles", "f16-128x128-tiles"])
+                                         (BFLOAT16, 499, 2312, 768), (HALF, 1921, 1928, 512), (FLOAT32, 999, 1004, 256), (FLOAT32, 1925, 1924, 384)],
+                         ids=["bf16-rows-off-by-one", "f16-seven-columns-left", "bf16-aligned-ragged", "bf16-64x64-tiles", "f16-128x128-tiles",
+                              "f32-64x64-tiles", "f32-128x128-tiles"])
 def test_ragged_product_on_the_direct_load_kernels_whole_result(ex, dtype, M, N, K):
     """The edge instantiations of the direct-load kernels, every element of the result: a row-major B with rows of 3705
     (every row starts 2 bytes further off a 16-byte boundary; one column is left for the bounds-handling kernel), of 3591
@@ -151,7 +155,7 @@ def test_ragged_product_on_the_direct_load_kernels_whole_result(ex, dtype, M, N,
     z = ex.exec_custom("matmul", [A, B])[0].to_float()
     name = _last_kernel(ex)
     assert ",edge" in name, name
-    assert ("unaligned" in name) == (N % 8 != 0), name
+    assert ("unaligned" in name) == (dtype != FLOAT32 and N % 8 != 0), name
     assert_close(z, a64 @ b64, TOL[dtype], TOL[dtype], "whole result")
 
 
