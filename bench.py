@@ -537,7 +537,27 @@ def main():
             w, e = timed(ex, L, ex.bind_custom("matmul", [Ua, Ue], [Uz]), max(steps // 5, 3), max(warmup // 5, 1))
             ops.append({"op": "mmul bf16 [4096,768] x [768,50257] (row length not a multiple of 8: %s)" % L.nd4jhipLastGemmKernel().decode(),
                         "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": mfma_entry(2.0 * 4096 * 50257 * 768, e, "bf16", "mmul unaligned")})
-            del Ua, Ue, Uz, ua, ue
+            # the same product against the k-contiguous [50257, 768] matrix (a tied embedding, transposeB): rows aligned, N not a
+            # whole number of tiles -- the edge instantiation of the two-stage direct-load kernel
+            Uet = NDArray.from_numpy(np.ascontiguousarray(ue.T), BFLOAT16)
+            Uet.sync_to_device()
+            w, e = timed(ex, L, ex.bind_custom("matmul", [Ua, Uet], [Uz], i_args=[0, 1, 0]), max(steps // 5, 3), max(warmup // 5, 1))
+            ops.append({"op": "mmul bf16 [4096,768] x [50257,768]^T (transposeB, N not a whole number of tiles: %s)" % L.nd4jhipLastGemmKernel().decode(),
+                        "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": mfma_entry(2.0 * 4096 * 50257 * 768, e, "bf16", "mmul ragged tb")})
+            del Ua, Ue, Uet, Uz, ua, ue
+            # ragged products of a few hundred to a few thousand rows and columns (a 500-token prompt's projections): the
+            # direct-load kernels' edge instantiations
+            for dt, nm, (rm, rn, rk) in ((BFLOAT16, "bf16", (500, 2304, 768)), (BFLOAT16, "bf16", (2000, 2000, 2048)), (FLOAT32, "f32", (2000, 2000, 2048))):
+                ra = rng.normal(0, 1, (rm, rk)).astype(np.float32)
+                rb = rng.normal(0, rk ** -0.5, (rk, rn)).astype(np.float32)
+                Ra = NDArray.from_numpy(ra, dt) if dt != FLOAT32 else NDArray.from_numpy(ra)
+                Rb = NDArray.from_numpy(rb, dt) if dt != FLOAT32 else NDArray.from_numpy(rb)
+                Rz = NDArray.empty((rm, rn), dt)
+                Ra.sync_to_device(); Rb.sync_to_device()
+                w, e = timed(ex, L, ex.bind_custom("matmul", [Ra, Rb], [Rz]), steps, warmup)
+                ops.append({"op": "mmul %s %d x %d x %d (ragged: %s)" % (nm, rm, rn, rk, L.nd4jhipLastGemmKernel().decode()),
+                            "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": mfma_entry(2.0 * rm * rn * rk, e, nm, "mmul ragged")})
+                del Ra, Rb, Rz, ra, rb
         if 2 in cfgs:
             # config 2, the remaining sizes/dtypes
             plain_cpu = {}     # (dtype, size) -> cpu_baseline of the plain-B product: the CPU loops do not depend on the layout flag
