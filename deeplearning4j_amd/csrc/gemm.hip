@@ -602,6 +602,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16q(GemmArgs g, const T
   storeAccTiles<T, TM, TN, true>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
 }
 
+// What a lane of a direct-load kernel reads for the part of an operand that lies beyond K (their KTAIL instantiations).
+__device__ __attribute__((aligned(256))) unsigned char gemmZeroPage[256];
+
 // Small tiles (64 x 64 or 128 x 128, four waves of TW x TW accumulator tiles) with the operands going from global memory
 // straight into LDS (no registers, no LDS stores), NST stages in a ring: for launches that put one or two tiles on a CU
 // (1024^3, 2048^3; the projections of a prefill), where the register-staged kernels spend more on parking the tiles in LDS
@@ -613,7 +616,11 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16q(GemmArgs g, const T
 // MFMAs of tile kt run.
 // EDGE: M and N need not be whole tiles -- rows (16-byte column groups of a row-major B) beyond the edge are read from
 // clamped positions inside the operand and only reach elements of C that the bounds-checked store leaves out.
-template <typename T, bool B_KC, int NST, int TW, bool EDGE = false>
+// KTAIL: K need not be a whole number of K-tiles (a multiple of 8 where an operand is k-contiguous).  Along K the products
+// beyond the edge must be zero: a lane whose 16 bytes start at k >= K reads them from a page of zeros instead (same
+// instruction, another address), so the loop and the LDS layouts do not change; the rounds past the last K-tile of an
+// NST-round multiply zeros.
+template <typename T, bool B_KC, int NST, int TW, bool EDGE = false, bool KTAIL = false>
 __global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
                                                     unsigned tilesM, unsigned tilesN) {
   constexpr int BM = 64 * TW, BN = 64 * TW, BK = 64;
@@ -633,10 +640,13 @@ __global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restr
 
   // ---- global side: CPW chunks of each operand per wave; a load is scalar base (the tile's first byte) + lane offset ----
   unsigned offA[CPW], offB[CPW];
+  int kA[CPW], kB[CPW];   // KTAIL: the k (inside a K-tile) this lane's 16 bytes start at
 #pragma unroll
   for (int c = 0; c < CPW; c++) {
     const int cw = wave * CPW + c, lj = lane >> 3, lp = lane & 7;
     const int lkg = (lp - 4 * (cw & 1) - (lj >> 1)) & 7;
+    kA[c] = lkg * 8;
+    kB[c] = B_KC ? lkg * 8 : cw * (64 / RowB::SPR) + lane / RowB::SPR;
     LongType ar = cw * 8 + lj;
     if (EDGE) ar = m0 + ar < g.M ? ar : g.M - 1 - m0;
     offA[c] = (unsigned)((ar * lda + lkg * 8) * 2);
@@ -654,14 +664,28 @@ __global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restr
   const char* const baseA = reinterpret_cast<const char*>(A + m0 * lda);
   const char* const baseB = reinterpret_cast<const char*>(B_KC ? B + n0 * ldb : B + n0);
   const LongType stepA = BK * 2, stepB = (B_KC ? (LongType)BK : (LongType)BK * ldb) * 2;   // bytes per K-tile
-  const LongType KT = g.K / BK;
+  const LongType KT = KTAIL ? (g.K + BK - 1) / BK : g.K / BK;
   auto dma = [&](const char* base, unsigned off, const u32x4* dst) {
     const unsigned ldsAddr = (unsigned)(size_t)(lds_ptr)dst;
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(ldsAddr) : "memory");
   };
+  auto dmaAt = [&](const char* src, const u32x4* dst) {   // a full address per lane
+    const unsigned ldsAddr = (unsigned)(size_t)(lds_ptr)dst;
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(ldsAddr) : "memory");
+  };
   auto issue = [&](LongType tile, int stage) {   // tiles past the end re-read the last one into a stage nobody reads
-    const LongType kt = tile < KT ? tile : KT - 1;
     u32x4* const st = smem + stage * STAGE;
+    if constexpr (KTAIL) {
+      // any tile, also past the end: zeros for everything from K on
+      const char* const zero = reinterpret_cast<const char*>(gemmZeroPage);
+      const int k0 = (int)(tile * BK);
+#pragma unroll
+      for (int c = 0; c < CPW; c++) dmaAt(k0 + kA[c] < (int)g.K ? baseA + tile * stepA + offA[c] : zero, st + (wave * CPW + c) * 64);
+#pragma unroll
+      for (int c = 0; c < CPW; c++) dmaAt(k0 + kB[c] < (int)g.K ? baseB + tile * stepB + offB[c] : zero, st + SLOTS_A + (wave * CPW + c) * 64);
+      return;
+    }
+    const LongType kt = tile < KT ? tile : KT - 1;
 #pragma unroll
     for (int c = 0; c < CPW; c++) dma(baseA + kt * stepA, offA[c], st + (wave * CPW + c) * 64);
 #pragma unroll
@@ -1421,7 +1445,7 @@ static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
   if constexpr (BM == 64 && BN == 64 && WM == 2 && WN == 2 && A_KC) {
     static const bool small = getenv("ND4JHIP_GEMM_SMALL_RING") ? atoi(getenv("ND4JHIP_GEMM_SMALL_RING")) != 0 : true;
     const LongType ldaS = g.aRow, ldbS = B_KC ? g.bCol : g.bRow;
-    ringInstead = small && g.K >= 512 && g.K <= 2048 && g.K % 256 == 0 && edgeOk && (whole || aligned) &&
+    ringInstead = small && g.K >= 512 && g.K <= 2048 && (g.K % 256 == 0 || (edge && aligned)) && edgeOk && (whole || aligned) &&
                   ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN) * batch <= 1024 &&
                   ldaS % 8 == 0 && ldbS % 8 == 0 && ldaS < (1 << 23) && ldbS < (1 << 23) &&
                   ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 && g.aBatch % 8 == 0 && g.bBatch % 8 == 0 &&
@@ -1451,7 +1475,10 @@ static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
     constexpr int STAGE_BYTES = (BM + BN) * 8 * 16;
     static const bool small = getenv("ND4JHIP_GEMM_SMALL_RING") ? atoi(getenv("ND4JHIP_GEMM_SMALL_RING")) != 0 : true;
     const LongType ldaS = g.aRow, ldbS = B_KC ? g.bCol : g.bRow;
-    const bool edgeShape = !whole && edgeOk && aligned && usePipe && nTiles <= 1024 && g.K >= 512 && g.K % 256 == 0;
+    // ragged M / N, or a K that is not a whole number of K-tiles: the edge instantiation, with the zero page for the end of
+    // K where K is not a multiple of 256 (whole tiles and a K of whole K-tiles keep the kernels they had)
+    const bool ktail = g.K % 256 != 0;
+    const bool edgeShape = (!whole || g.K % 64 != 0) && edge && edgeOk && aligned && usePipe && nTiles <= 1024 && g.K >= 512;
     const bool shape = edgeShape || (TW == 1 ? useDeep : (useFull && nTiles <= 1024 && g.K >= 512 && g.K % 256 == 0));
     if (small && shape && ldaS % 8 == 0 && ldbS % 8 == 0 && ldaS < (1 << 23) && ldbS < (1 << 23) &&
         ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 && g.aBatch % 8 == 0 && g.bBatch % 8 == 0 &&
@@ -1460,18 +1487,26 @@ static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
       // 64 x 64: one tile per CU and a K of whole eight-tile rounds take eight stages (128 KiB), else four (two blocks fit a
       // CU); 128 x 128: four stages (128 KiB)
       constexpr int DEEP = TW == 1 ? 8 : 4;
-      const bool wantDeep = TW == 2 || (nTiles <= 256 && g.K % 512 == 0);
-      const bool grantedDeep = whole ? DynLds<gemm_mfma16s<T, B_KC, DEEP, TW>, DEEP * STAGE_BYTES>::granted()
-                                     : DynLds<gemm_mfma16s<T, B_KC, DEEP, TW, true>, DEEP * STAGE_BYTES>::granted();
+      // a K that ends inside a round of eight K-tiles multiplies zeros for the rest of it: eight stages only if that is at
+      // most one K-tile
+      const LongType kTiles = (g.K + 63) / 64;
+      const bool wantDeep = TW == 2 || (nTiles <= 256 && (ktail ? (kTiles + 7) / 8 * 8 - kTiles <= 1 : g.K % 512 == 0));
+      const bool plain = !edgeShape;
+      const bool grantedDeep = plain   ? DynLds<gemm_mfma16s<T, B_KC, DEEP, TW>, DEEP * STAGE_BYTES>::granted()
+                               : ktail ? DynLds<gemm_mfma16s<T, B_KC, DEEP, TW, true, true>, DEEP * STAGE_BYTES>::granted()
+                                       : DynLds<gemm_mfma16s<T, B_KC, DEEP, TW, true>, DEEP * STAGE_BYTES>::granted();
+      const char* const flavour = plain ? "" : ktail ? ",edge,ktail" : ",edge";
       if (wantDeep && grantedDeep) {
-        noteKernel("gemm_mfma16s<%s,%dx%d,akc=1,bkc=%d,stages=%d%s>", tname<T>(), BM, BN, (int)B_KC, DEEP, whole ? "" : ",edge");
-        auto kern = whole ? gemm_mfma16s<T, B_KC, DEEP, TW, false> : gemm_mfma16s<T, B_KC, DEEP, TW, true>;
+        noteKernel("gemm_mfma16s<%s,%dx%d,akc=1,bkc=%d,stages=%d%s>", tname<T>(), BM, BN, (int)B_KC, DEEP, flavour);
+        auto kern = plain   ? gemm_mfma16s<T, B_KC, DEEP, TW, false, false>
+                    : ktail ? gemm_mfma16s<T, B_KC, DEEP, TW, true, true> : gemm_mfma16s<T, B_KC, DEEP, TW, true, false>;
         hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(256), DEEP * STAGE_BYTES, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
         return true;
       }
       if constexpr (TW == 1) {
-        noteKernel("gemm_mfma16s<%s,64x64,akc=1,bkc=%d,stages=4%s>", tname<T>(), (int)B_KC, whole ? "" : ",edge");
-        auto kern = whole ? gemm_mfma16s<T, B_KC, 4, 1, false> : gemm_mfma16s<T, B_KC, 4, 1, true>;
+        noteKernel("gemm_mfma16s<%s,64x64,akc=1,bkc=%d,stages=4%s>", tname<T>(), (int)B_KC, flavour);
+        auto kern = plain   ? gemm_mfma16s<T, B_KC, 4, 1, false, false>
+                    : ktail ? gemm_mfma16s<T, B_KC, 4, 1, true, true> : gemm_mfma16s<T, B_KC, 4, 1, true, false>;
         hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(256), 4 * STAGE_BYTES, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
         return true;
       }

@@ -84,8 +84,12 @@ CASES = [
     (BFLOAT16, 2000, 2000, 2048, "gemm_mfma16s<bf16,128x128,akc=1,bkc=0,stages=4,edge>", "gemm_mfma16s<bf16,128x128,akc=1,bkc=1,stages=4,edge>", None),
     (HALF, 1000, 1000, 1024, "gemm_mfma16s<f16,64x64,akc=1,bkc=0,stages=8,edge>", "gemm_mfma16s<f16,64x64,akc=1,bkc=1,stages=8,edge>", None),
     (BFLOAT16, 500, 2304, 768, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=4,edge>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=4,edge>", None),
-    (HALF, 1800, 1800, 520, "gemm_mfma16p<f16,128x128,akc=1,bkc=0>", "gemm_mfma16p<f16,128x128,akc=1,bkc=1>", None),
-    (BFLOAT16, 1104, 904, 1000, "gemm_mfma16p<bf16,64x64,akc=1,bkc=0>", "gemm_mfma16p<bf16,64x64,akc=1,bkc=1>", None),
+    # ... and with a K that is not a whole number of K-tiles (from 512 on: the ring kernel with the page of zeros; below: the
+    # bounds-handling kernel)
+    (HALF, 1800, 1800, 520, "gemm_mfma16s<f16,128x128,akc=1,bkc=0,stages=4,edge,ktail>", "gemm_mfma16s<f16,128x128,akc=1,bkc=1,stages=4,edge,ktail>", None),
+    (BFLOAT16, 1104, 904, 1000, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=4,edge,ktail>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=4,edge,ktail>", None),
+    (HALF, 1800, 1800, 328, "gemm_mfma16p<f16,128x128,akc=1,bkc=0>", "gemm_mfma16p<f16,128x128,akc=1,bkc=1>", None),
+    (BFLOAT16, 1104, 904, 200, "gemm_mfma16p<bf16,64x64,akc=1,bkc=0>", "gemm_mfma16p<bf16,64x64,akc=1,bkc=1>", None),
     # K a multiple of 256 but not of 512: the four-stage ring; more tiles than CUs (two blocks on a CU): four stages as well;
     # the shortest K the ring takes
     (BFLOAT16, 1024, 1024, 768, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=4>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=4>", "gemm_mfma16q<bf16,64x64,akc=0,bkc=0>"),
@@ -144,6 +148,20 @@ def test_matmul_kernel_at_real_shape(ex, dtype, M, N, K, kern_plain, kern_tb, ke
                          ids=["bf16-rows-off-by-one", "f16-seven-columns-left", "bf16-aligned-ragged", "bf16-64x64-tiles", "f16-128x128-tiles",
                               "f32-64x64-tiles", "f32-128x128-tiles"])
 def test_ragged_product_on_the_direct_load_kernels_whole_result(ex, dtype, M, N, K):
+    _whole_result(ex, dtype, M, N, K, False)
+
+
+@pytest.mark.parametrize("tb", [False, True], ids=["plain", "transposeB"])
+@pytest.mark.parametrize("dtype,M,N,K", [(BFLOAT16, 1000, 1000, 1000), (HALF, 1024, 1024, 520), (BFLOAT16, 2000, 2000, 1000), (HALF, 512, 512, 1992),
+                                         (BFLOAT16, 1920, 2048, 968)],
+                         ids=["bf16-1000", "f16-whole-tiles-k520", "bf16-128x128-tiles", "f16-few-tiles", "bf16-k968"])
+def test_k_tail_on_the_direct_load_kernels_whole_result(ex, dtype, M, N, K, tb):
+    """A K that is not a whole number of K-tiles on the ring kernel: the lanes beyond K read a page of zeros.  Every element of
+    the result, with operands whose neighbours in memory (the next row, which a load past K would bring in) are large."""
+    _whole_result(ex, dtype, M, N, K, tb, expect=",ktail")
+
+
+def _whole_result(ex, dtype, M, N, K, tb, expect=",edge"):
     """The edge instantiations of the direct-load kernels, every element of the result: a row-major B with rows of 3705
     (every row starts 2 bytes further off a 16-byte boundary; one column is left for the bounds-handling kernel), of 3591
     (seven columns left), and an aligned B with a ragged last tile row and column."""
@@ -152,10 +170,12 @@ def test_ragged_product_on_the_direct_load_kernels_whole_result(ex, dtype, M, N,
     b = rng.normal(0, 1 / math.sqrt(K), (K, N)).astype(np.float32)
     A, a64 = _device(a, dtype)
     B, b64 = _device(b, dtype)
-    z = ex.exec_custom("matmul", [A, B])[0].to_float()
+    if tb:
+        B, _ = _device(b.T, dtype)
+    z = ex.exec_custom("matmul", [A, B], i_args=[0, 1 if tb else 0])[0].to_float()
     name = _last_kernel(ex)
-    assert ",edge" in name, name
-    assert ("unaligned" in name) == (dtype != FLOAT32 and N % 8 != 0), name
+    assert expect in name, name
+    assert ("unaligned" in name) == (dtype != FLOAT32 and N % 8 != 0 and not tb), name
     assert_close(z, a64 @ b64, TOL[dtype], TOL[dtype], "whole result")
 
 
