@@ -917,7 +917,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16f(GemmArgs g, const T
 // EDGE: M and N need not be whole tiles.  The direct loads of the last tile row / column take their rows (their 16-byte
 // column groups of a row-major B) from clamped positions inside the operand -- what they bring in only ever reaches
 // elements of C beyond the edge, which the bounds-checked store leaves out.
-template <typename T, bool B_KC, bool EDGE = false>
+// KTAIL: K need not be a whole number of K-tiles -- lanes whose 16 bytes start at k >= K read a page of zeros (see
+// gemm_mfma16s).
+template <typename T, bool B_KC, bool EDGE = false, bool KTAIL = false>
 __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
                                                     unsigned tilesM, unsigned tilesN) {
   constexpr int BM = 256, BN = 256, BK = 64, WN = 4, WTM = 128, WTN = 64, TM = 4, TN = 2, NM = TM * TN;
@@ -943,10 +945,13 @@ __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restr
   const int lj = lane >> 3, lp = lane & 7;
   const T* aSrc[4];
   const T* bSrc[4];
+  int akg[4], bkg[4];   // KTAIL: the k (inside a K-tile) this lane's 16 bytes start at
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     const int cw = wave * 4 + i;
     const int lkg = (lp - 4 * (cw & 1) - (lj >> 1)) & 7;
+    akg[i] = lkg * 8;
+    bkg[i] = B_KC ? lkg * 8 : 2 * cw + (lane >> 5);
     LongType ar = m0 + cw * 8 + lj;
     if (EDGE) ar = ar < g.M ? ar : g.M - 1;
     aSrc[i] = A + ar * lda + lkg * 8;
@@ -972,15 +977,19 @@ __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restr
     const unsigned ldsAddr = (unsigned)(size_t)(lds_ptr)dst;
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(ldsAddr) : "memory");
   };
+  int ldA = 0, ldB = 0;   // KTAIL: first k of the K-tile the next A / B loads belong to
+  const T* const zero = reinterpret_cast<const T*>(gemmZeroPage);
   auto issueLoads = [&](u32x4* stage, int from, int to) {
 #pragma unroll
     for (int i = from; i < to; i++) {
       if (i < 4) {
-        loadToLds(aSrc[i], stage + (wave * 4 + i) * 64);
+        loadToLds(!KTAIL || ldA + akg[i] < (int)g.K ? aSrc[i] : zero, stage + (wave * 4 + i) * 64);
         aSrc[i] += aStep;
+        if (KTAIL && i == 3) ldA += BK;
       } else {
-        loadToLds(bSrc[i - 4], stage + SLOTS_OP + (wave * 4 + i - 4) * 64);
+        loadToLds(!KTAIL || ldB + bkg[i - 4] < (int)g.K ? bSrc[i - 4] : zero, stage + SLOTS_OP + (wave * 4 + i - 4) * 64);
         bSrc[i - 4] += bStep;
+        if (KTAIL && i == 7) ldB += BK;
       }
     }
   };
@@ -1046,7 +1055,7 @@ __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restr
     }
   };
 
-  const LongType KT = g.K / BK;
+  const LongType KT = KTAIL ? (g.K + BK - 1) / BK : g.K / BK;
   issueLoads(smem, 0, 8);            // tile 0 -> stage 0
   issueLoads(smem + STAGE, 0, 8);    // tile 1 -> stage 1 (K >= 2 tiles)
   asm volatile("s_waitcnt vmcnt(8)" ::: "memory");   // tile 0 has landed (loads complete in order)
@@ -1130,7 +1139,9 @@ __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restr
 // order).  The loop is branch-free: past the end of K the pointers stop advancing, so the surplus loads re-read the
 // last unit into slots nobody reads any more.  K must be a multiple of 128 (four steps per loop iteration).
 // EDGE as in gemm_mfma16d: clamped loads and a bounds-checked store for an M or N that is not a whole number of tiles.
-template <typename T, bool EDGE = false>
+// KTAIL: K need not be a multiple of 128 -- the loop runs over K rounded up, and lanes whose 16 bytes start at k >= K read a
+// page of zeros (see gemm_mfma16s).
+template <typename T, bool EDGE = false, bool KTAIL = false>
 __global__ __launch_bounds__(512) void gemm_mfma16r(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
                                                     unsigned tilesM, unsigned tilesN) {
   constexpr int BM = 256, BN = 256, WN = 4, WTM = 128, WTN = 64, TM = 4, TN = 2, NM = TM * TN;
@@ -1154,10 +1165,12 @@ __global__ __launch_bounds__(512) void gemm_mfma16r(GemmArgs g, const T* __restr
   const int lj = lane >> 3, lp = lane & 7;
   const T* aSrc[4];
   const T* bSrc[2];
+  int aK[4], bK[2];   // KTAIL: the k this lane's next 16 bytes of the chunk start at
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     const int cw = wave * 4 + i;                          // 8 rows, all 8 k-groups of the unit
     const int lkg = (lp - 4 * (cw & 1) - (lj >> 1)) & 7;
+    aK[i] = lkg * 8;
     LongType ar = m0 + cw * 8 + lj;
     if (EDGE) ar = ar < g.M ? ar : g.M - 1;
     aSrc[i] = A + ar * lda + lkg * 8;
@@ -1165,24 +1178,29 @@ __global__ __launch_bounds__(512) void gemm_mfma16r(GemmArgs g, const T* __restr
 #pragma unroll
   for (int c = 0; c < 2; c++) {
     const int kr = 2 * (wave * 2 + c) + (lane >> 5), q = lane & 31;   // two k-rows of 256 n per chunk
+    bK[c] = kr;
     LongType bc = n0 + 8 * (q ^ (4 * (kr & 3)));
     if (EDGE) bc = bc + 8 <= g.N ? bc : g.N - 8;
     bSrc[c] = B + (LongType)kr * ldb + bc;
   }
-  const int S = (int)(g.K / 32), nA = (int)(g.K / 64);   // steps, A units
+  const int Kr = KTAIL ? (int)((g.K + 127) / 128 * 128) : (int)g.K;
+  const int S = Kr / 32, nA = Kr / 64;   // steps, A units
   const LongType aStep = 64, bStep = 32 * ldb;
+  const T* const zero = reinterpret_cast<const T*>(gemmZeroPage);
   auto loadToLds = [&](const T* src, u32x4* dst) {
     const unsigned ldsAddr = (unsigned)(size_t)(lds_ptr)dst;
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(ldsAddr) : "memory");
   };
   // chunk i of A unit `unit` into ring slot `slot`; the pointer moves on only while there is a next unit
   auto issueA = [&](int i, int slot, int unit) {
-    loadToLds(aSrc[i], smem + slot * A_UNIT + (wave * 4 + i) * 64);
+    loadToLds(!KTAIL || aK[i] < (int)g.K ? aSrc[i] : zero, smem + slot * A_UNIT + (wave * 4 + i) * 64);
     aSrc[i] += unit + 1 < nA ? aStep : 0;
+    if (KTAIL) aK[i] += unit + 1 < nA ? 64 : 0;
   };
   auto issueB = [&](int c, int slot, int unit) {
-    loadToLds(bSrc[c], smem + B_BASE + slot * B_UNIT + (wave * 2 + c) * 64);
+    loadToLds(!KTAIL || bK[c] < (int)g.K ? bSrc[c] : zero, smem + B_BASE + slot * B_UNIT + (wave * 2 + c) * 64);
     bSrc[c] += unit + 1 < S ? bStep : 0;
+    if (KTAIL) bK[c] += unit + 1 < S ? 32 : 0;
   };
 
   // ---- LDS side --------------------------------------------------------------------------------------------------------
@@ -1553,12 +1571,12 @@ static bool launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const 
     // that are left through the bounds-handling kernel (bf16 4096 x 50257 x 768: 0.71 -> 0.40 ms)
     static const bool ub = getenv("ND4JHIP_GEMM_UNALIGNED_RING") ? atoi(getenv("ND4JHIP_GEMM_UNALIGNED_RING")) != 0 : true;
     constexpr size_t LDS = (3 * 256 * 8 + 4 * 32 * 32) * 16;
-    if (!aligned && ub && batch == 1 && (reinterpret_cast<uintptr_t>(A) & 15) == 0 && g.aRow % 8 == 0 && g.K % 128 == 0 && g.N >= 264 &&
-        DynLds<gemm_mfma16r<T, true>, (int)LDS>::granted()) {
+    if (!aligned && ub && batch == 1 && (reinterpret_cast<uintptr_t>(A) & 15) == 0 && g.aRow % 8 == 0 && g.K % 8 == 0 && g.K >= 128 && g.N >= 264 &&
+        DynLds<gemm_mfma16r<T, true>, (int)LDS>::granted() && DynLds<gemm_mfma16r<T, true, true>, (int)LDS>::granted()) {
       GemmArgs g1 = g;
       g1.N = g.N & ~(LongType)7;
       const unsigned tM = (unsigned)((g.M + 255) / 256), tN = (unsigned)((g1.N + 255) / 256);
-      auto kern = gemm_mfma16r<T, true>;
+      auto kern = g.K % 128 == 0 ? gemm_mfma16r<T, true, false> : gemm_mfma16r<T, true, true>;
       hipLaunchKernelGGL(kern, dim3(tM * tN, 1, 1), dim3(512), LDS, s, g1, (const T*)A, (const T*)B, (T*)C, tM, tN);
       const LongType rem = g.N & 7;
       if (rem) {
@@ -1567,7 +1585,7 @@ static bool launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const 
         if (g.bias) g2.bias = static_cast<const T*>(g.bias) + g1.N;
         if (!launchMfma16Cfg<T, 64, 64, 2, 2, A_KC, B_KC>(s, g2, A, (const T*)B + g1.N, (T*)C + g1.N * g.cCol, 1, false, false)) return false;
       }
-      noteKernel("gemm_mfma16r<%s,256x256,akc=1,bkc=0,edge,unaligned>", tname<T>());
+      noteKernel("gemm_mfma16r<%s,256x256,akc=1,bkc=0,edge%s,unaligned>", tname<T>(), g.K % 128 == 0 ? "" : ",ktail");
       return true;
     }
   }
@@ -1590,6 +1608,14 @@ static bool launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const 
       hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(512), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
       return true;
     }
+    // a K that is not a whole number of K-tiles: the ring over K rounded up, zeros from K on (a K of whole 64-k tiles keeps
+    // the two-stage kernel below)
+    if (direct && ring && edge && edgeOk && g.K % 64 != 0 && g.K >= 128 && DynLds<gemm_mfma16r<T, true, true>, (int)LDS>::granted()) {
+      noteKernel("gemm_mfma16r<%s,256x256,akc=1,bkc=0,edge,ktail>", tname<T>());
+      auto kern = gemm_mfma16r<T, true, true>;
+      hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(512), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
+      return true;
+    }
   }
   if (direct && A_KC && edgeOk && g.K % 64 == 0 && g.K >= 128) {
     constexpr size_t LDS = 2 * 2 * 256 * 8 * 16;
@@ -1599,6 +1625,15 @@ static bool launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const 
     auto kern = whole ? gemm_mfma16d<T, B_KC, false> : gemm_mfma16d<T, B_KC, true>;
     hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(512), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
     return true;
+  }
+  if constexpr (A_KC && B_KC) {
+    constexpr size_t LDS = 2 * 2 * 256 * 8 * 16;
+    if (direct && edge && edgeOk && g.K % 64 != 0 && g.K >= 128 && DynLds<gemm_mfma16d<T, true, true, true>, (int)LDS>::granted()) {
+      noteKernel("gemm_mfma16d<%s,256x256,akc=1,bkc=1,edge,ktail>", tname<T>());
+      auto kern = gemm_mfma16d<T, true, true, true>;
+      hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(512), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
+      return true;
+    }
   }
   return launchMfma16Cfg<T, 256, 256, 2, 4, A_KC, B_KC>(s, g, A, B, C, batch, false, true);
 }

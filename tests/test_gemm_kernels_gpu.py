@@ -75,7 +75,9 @@ CASES = [
     # a K of whole K-tiles that is not a multiple of four of them stays on the register-staged kernel
     (HALF, 2048, 2048, 320, "gemm_mfma16f<f16,128x128,akc=1,bkc=0>", "gemm_mfma16f<f16,128x128,akc=1,bkc=1>", None),
     # ragged edges on the large tiles (bounds-handling kernel)
-    (BFLOAT16, 3600, 3704, 1000, "gemm_mfma16p<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16p<bf16,256x256,akc=1,bkc=1>", "gemm_mfma16p<bf16,256x256,akc=0,bkc=0>"),
+    (BFLOAT16, 3600, 3704, 72, "gemm_mfma16p<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16p<bf16,256x256,akc=1,bkc=1>", "gemm_mfma16p<bf16,256x256,akc=0,bkc=0>"),
+    # ... from K = 128 on the direct-load kernels take them, also with a K that ends inside a K-tile
+    (BFLOAT16, 3600, 3704, 1000, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0,edge,ktail>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1,edge,ktail>", "gemm_mfma16p<bf16,256x256,akc=0,bkc=0>"),
     # ragged edges with aligned rows and a K of whole K-tiles: the direct-load kernels' edge instantiations (clamped loads,
     # bounds-checked store) -- a last tile row of 16 rows and a last tile column of 120, of 8 (one column group) and of 1
     (BFLOAT16, 3600, 3704, 1024, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0,edge>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1,edge>", "gemm_mfma16p<bf16,256x256,akc=0,bkc=0>"),
@@ -144,17 +146,18 @@ def test_matmul_kernel_at_real_shape(ex, dtype, M, N, K, kern_plain, kern_tb, ke
 
 
 @pytest.mark.parametrize("dtype,M,N,K", [(BFLOAT16, 3600, 3705, 256), (HALF, 3599, 3591, 128), (BFLOAT16, 3585, 3704, 384),
-                                         (BFLOAT16, 499, 2312, 768), (HALF, 1921, 1928, 512), (FLOAT32, 999, 1004, 256), (FLOAT32, 1925, 1924, 384)],
+                                         (BFLOAT16, 499, 2312, 768), (HALF, 1921, 1928, 512), (FLOAT32, 999, 1004, 256), (FLOAT32, 1925, 1924, 384),
+                                         (BFLOAT16, 3600, 3705, 200)],
                          ids=["bf16-rows-off-by-one", "f16-seven-columns-left", "bf16-aligned-ragged", "bf16-64x64-tiles", "f16-128x128-tiles",
-                              "f32-64x64-tiles", "f32-128x128-tiles"])
+                              "f32-64x64-tiles", "f32-128x128-tiles", "bf16-rows-off-by-one-k200"])
 def test_ragged_product_on_the_direct_load_kernels_whole_result(ex, dtype, M, N, K):
     _whole_result(ex, dtype, M, N, K, False)
 
 
 @pytest.mark.parametrize("tb", [False, True], ids=["plain", "transposeB"])
 @pytest.mark.parametrize("dtype,M,N,K", [(BFLOAT16, 1000, 1000, 1000), (HALF, 1024, 1024, 520), (BFLOAT16, 2000, 2000, 1000), (HALF, 512, 512, 1992),
-                                         (BFLOAT16, 1920, 2048, 968)],
-                         ids=["bf16-1000", "f16-whole-tiles-k520", "bf16-128x128-tiles", "f16-few-tiles", "bf16-k968"])
+                                         (BFLOAT16, 1920, 2048, 968), (BFLOAT16, 3700, 3704, 1000), (HALF, 4096, 3840, 136)],
+                         ids=["bf16-1000", "f16-whole-tiles-k520", "bf16-128x128-tiles", "f16-few-tiles", "bf16-k968", "bf16-256x256-tiles", "f16-256x256-k136"])
 def test_k_tail_on_the_direct_load_kernels_whole_result(ex, dtype, M, N, K, tb):
     """A K that is not a whole number of K-tiles on the ring kernel: the lanes beyond K read a page of zeros.  Every element of
     the result, with operands whose neighbours in memory (the next row, which a load past K would bring in) are large."""
