@@ -1769,7 +1769,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32(GemmArgs g, const fl
 // them).  Host: K % (BK * PD) == 0, K >= 2 * BK * PD; M % BM == 0 and N % BN == 0 unless EDGE: then the rows (the 16-byte
 // groups along M or N of an operand that is contiguous that way) beyond the edge are read from clamped positions inside the
 // operand and only reach elements of C that the bounds-checked store leaves out.
-template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int PD, int BK, bool EDGE = false>
+// KTAIL: K need not be a whole number of rounds (a multiple of 4 where an operand is k-contiguous) -- the loop runs over K
+// rounded up to PD K-tiles and a lane whose 16 bytes start at k >= K reads a page of zeros.
+template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int PD, int BK, bool EDGE = false, bool KTAIL = false>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32q(GemmArgs g, const float* __restrict__ A, const float* __restrict__ B,
                                                               float* __restrict__ C, unsigned tilesM, unsigned tilesN) {
   static_assert(PD % 2 == 0, "the LDS stage of a K-tile must be a compile-time constant inside the unrolled loop");
@@ -1802,6 +1804,11 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32q(GemmArgs g, const f
   // and K-tile.  Computed from the element coordinates each time it cost a 64-bit multiply-add chain in front of an MFMA.
   typedef const __attribute__((address_space(1))) char* GlobalBytes;
   GlobalBytes curA[VA], curB[VB];
+  int kOffA[VA], kOffB[VB];   // KTAIL: the k (inside a K-tile) this lane's 16 bytes start at
+#pragma unroll
+  for (int i = 0; i < VA; i++) kOffA[i] = A_KC ? ((t + i * NT) % KQ) * 4 : (t + i * NT) / (BM / 4);
+#pragma unroll
+  for (int i = 0; i < VB; i++) kOffB[i] = B_KC ? ((t + i * NT) % KQ) * 4 : (t + i * NT) / (BN / 4);
 #pragma unroll
   for (int i = 0; i < VA; i++) {
     const int v = t + i * NT;
@@ -1816,14 +1823,17 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma32q(GemmArgs g, const f
     if (EDGE) bn = B_KC ? (bn < g.N ? bn : g.N - 1) : (bn + 4 <= g.N ? bn : g.N - 4);
     curB[i] = (GlobalBytes)(B_KC ? B + bn * ldb + (v % KQ) * 4 : B + (LongType)(v / (BN / 4)) * ldb + bn);
   }
-  const LongType KT = g.K / BK;
+  const LongType KT = KTAIL ? (g.K + BK * PD - 1) / (BK * PD) * PD : g.K / BK;
   const LongType stepA = (A_KC ? BK : BK * lda) * 4, stepB = (B_KC ? BK : BK * ldb) * 4;   // bytes per K-tile
+  int kNext = 0;   // KTAIL: first k of the K-tile the pointers stand at (they move on with every load there)
+  const GlobalBytes zero = (GlobalBytes)gemmZeroPage;
   // more: the K-tile loaded is not the last one (a condition on the loop counters, so a scalar one)
   auto loadNext = [&](int u, bool more) {
 #pragma unroll
-    for (int i = 0; i < VA; i++) ra[u][i] = *(const __attribute__((address_space(1))) f32x4*)curA[i];
+    for (int i = 0; i < VA; i++) ra[u][i] = *(const __attribute__((address_space(1))) f32x4*)(!KTAIL || kNext + kOffA[i] < (int)g.K ? curA[i] : zero);
 #pragma unroll
-    for (int i = 0; i < VB; i++) rb[u][i] = *(const __attribute__((address_space(1))) f32x4*)curB[i];
+    for (int i = 0; i < VB; i++) rb[u][i] = *(const __attribute__((address_space(1))) f32x4*)(!KTAIL || kNext + kOffB[i] < (int)g.K ? curB[i] : zero);
+    if (KTAIL) { more = true; kNext += BK; }
     const LongType sa = more ? stepA : 0, sb = more ? stepB : 0;
 #pragma unroll
     for (int i = 0; i < VA; i++) curA[i] += sa;
@@ -1955,10 +1965,12 @@ static void launchMfma32Cfg(hipStream_t s, const GemmArgs& g, const void* A, con
   static const bool edge = getenv("ND4JHIP_GEMM_EDGE") ? atoi(getenv("ND4JHIP_GEMM_EDGE")) != 0 : true;
   const bool whole = g.M % BM == 0 && g.N % BN == 0;
   // `aligned` says that an operand which is contiguous along M or N has an extent of whole 16-byte groups
-  if (aligned && g.K >= 256 && (whole || (edge && g.M >= 4 && g.N >= 4)) && g.K % 128 == 0) {
+  const bool ktail = g.K % 128 != 0;
+  if (aligned && g.K >= 256 && (whole || (edge && g.M >= 4 && g.N >= 4)) && (!ktail || edge)) {
     constexpr int PD = 4, BK = BM * BN <= 64 * 64 ? 32 : 16;
-    noteKernel("gemm_mfma32q<f32,%dx%d,akc=%d,bkc=%d,pd=%d,bk=%d%s>", BM, BN, (int)A_KC, (int)B_KC, PD, BK, whole ? "" : ",edge");
-    auto kern = whole ? gemm_mfma32q<BM, BN, WM, WN, A_KC, B_KC, PD, BK, false> : gemm_mfma32q<BM, BN, WM, WN, A_KC, B_KC, PD, BK, true>;
+    noteKernel("gemm_mfma32q<f32,%dx%d,akc=%d,bkc=%d,pd=%d,bk=%d%s>", BM, BN, (int)A_KC, (int)B_KC, PD, BK, ktail ? ",edge,ktail" : whole ? "" : ",edge");
+    auto kern = ktail   ? gemm_mfma32q<BM, BN, WM, WN, A_KC, B_KC, PD, BK, true, true>
+                : whole ? gemm_mfma32q<BM, BN, WM, WN, A_KC, B_KC, PD, BK, false, false> : gemm_mfma32q<BM, BN, WM, WN, A_KC, B_KC, PD, BK, true, false>;
     hipLaunchKernelGGL(kern, dim3(tilesM * tilesN, 1, (unsigned)batch), dim3(WM * WN * 64), 0, s, g, (const float*)A, (const float*)B, (float*)C,
                        tilesM, tilesN);
     return;

@@ -118,8 +118,10 @@ CASES = [
     (FLOAT32, 1000, 1000, 1024, "gemm_mfma32q<f32,64x64,akc=1,bkc=0,pd=4,bk=32,edge>", "gemm_mfma32q<f32,64x64,akc=1,bkc=1,pd=4,bk=32,edge>", "gemm_mfma32q<f32,64x64,akc=0,bkc=0,pd=4,bk=32,edge>"),
     (FLOAT32, 2004, 2000, 512, "gemm_mfma32q<f32,128x128,akc=1,bkc=0,pd=4,bk=16,edge>", "gemm_mfma32q<f32,128x128,akc=1,bkc=1,pd=4,bk=16,edge>", "gemm_mfma32q<f32,128x128,akc=0,bkc=0,pd=4,bk=16,edge>"),
     # fp32 ragged
-    (FLOAT32, 1100, 900, 1000, "gemm_mfma32<f32,64x64,akc=1,bkc=0>", "gemm_mfma32<f32,64x64,akc=1,bkc=1>", None),
-    (FLOAT32, 2100, 2052, 520, "gemm_mfma32<f32,128x128,akc=1,bkc=0>", "gemm_mfma32<f32,128x128,akc=1,bkc=1>", "gemm_mfma32<f32,128x128,akc=0,bkc=0>"),
+    (FLOAT32, 1100, 900, 1000, "gemm_mfma32q<f32,64x64,akc=1,bkc=0,pd=4,bk=32,edge,ktail>", "gemm_mfma32q<f32,64x64,akc=1,bkc=1,pd=4,bk=32,edge,ktail>", None),
+    (FLOAT32, 2100, 2052, 520, "gemm_mfma32q<f32,128x128,akc=1,bkc=0,pd=4,bk=16,edge,ktail>", "gemm_mfma32q<f32,128x128,akc=1,bkc=1,pd=4,bk=16,edge,ktail>", "gemm_mfma32q<f32,128x128,akc=0,bkc=0,pd=4,bk=16,edge,ktail>"),
+    (FLOAT32, 1100, 900, 200, "gemm_mfma32<f32,64x64,akc=1,bkc=0>", "gemm_mfma32<f32,64x64,akc=1,bkc=1>", None),
+    (FLOAT32, 2100, 2052, 136, "gemm_mfma32<f32,128x128,akc=1,bkc=0>", "gemm_mfma32<f32,128x128,akc=1,bkc=1>", "gemm_mfma32<f32,128x128,akc=0,bkc=0>"),
 ]
 
 
@@ -156,8 +158,10 @@ def test_ragged_product_on_the_direct_load_kernels_whole_result(ex, dtype, M, N,
 
 @pytest.mark.parametrize("tb", [False, True], ids=["plain", "transposeB"])
 @pytest.mark.parametrize("dtype,M,N,K", [(BFLOAT16, 1000, 1000, 1000), (HALF, 1024, 1024, 520), (BFLOAT16, 2000, 2000, 1000), (HALF, 512, 512, 1992),
-                                         (BFLOAT16, 1920, 2048, 968), (BFLOAT16, 3700, 3704, 1000), (HALF, 4096, 3840, 136)],
-                         ids=["bf16-1000", "f16-whole-tiles-k520", "bf16-128x128-tiles", "f16-few-tiles", "bf16-k968", "bf16-256x256-tiles", "f16-256x256-k136"])
+                                         (BFLOAT16, 1920, 2048, 968), (BFLOAT16, 3700, 3704, 1000), (HALF, 4096, 3840, 136),
+                                         (FLOAT32, 1000, 1000, 1000), (FLOAT32, 1920, 2048, 268)],
+                         ids=["bf16-1000", "f16-whole-tiles-k520", "bf16-128x128-tiles", "f16-few-tiles", "bf16-k968", "bf16-256x256-tiles", "f16-256x256-k136",
+                              "f32-1000", "f32-128x128-k268"])
 def test_k_tail_on_the_direct_load_kernels_whole_result(ex, dtype, M, N, K, tb):
     """A K that is not a whole number of K-tiles on the ring kernel: the lanes beyond K read a page of zeros.  Every element of
     the result, with operands whose neighbours in memory (the next row, which a load past K would bring in) are large."""
