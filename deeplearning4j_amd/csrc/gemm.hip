@@ -620,7 +620,9 @@ __device__ __attribute__((aligned(256))) unsigned char gemmZeroPage[256];
 // beyond the edge must be zero: a lane whose 16 bytes start at k >= K reads them from a page of zeros instead (same
 // instruction, another address), so the loop and the LDS layouts do not change; the rounds past the last K-tile of an
 // NST-round multiply zeros.
-template <typename T, bool B_KC, int NST, int TW, bool EDGE = false, bool KTAIL = false>
+// A_KC = false: A lies [k][m] with unit m stride (a transposed A) and is handled like a row-major B: whole k-rows in LDS,
+// fragments through the transposing read.
+template <typename T, bool B_KC, int NST, int TW, bool EDGE = false, bool KTAIL = false, bool A_KC = true>
 __global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
                                                     unsigned tilesM, unsigned tilesN) {
   constexpr int BM = 64 * TW, BN = 64 * TW, BK = 64;
@@ -633,10 +635,11 @@ __global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restr
   tileOf(blockIdx.x, gridDim.x, tilesM, tilesN, tm, tn);
   const LongType m0 = (LongType)tm * BM, n0 = (LongType)tn * BN;
   { LongType oa, ob, oc; batchOffsets(g, (LongType)blockIdx.z, oa, ob, oc); A += oa; B += ob; C += oc; }
-  const LongType lda = g.aRow, ldb = B_KC ? g.bCol : g.bRow;
+  const LongType lda = A_KC ? g.aRow : g.aCol, ldb = B_KC ? g.bCol : g.bRow;
   const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6), h = lane >> 5;
   const int wm = wave >> 1, wn = wave & 1;
   using RowB = RowTileLoader<BN, 256>;
+  using RowA = RowTileLoader<BM, 256>;
 
   // ---- global side: CPW chunks of each operand per wave; a load is scalar base (the tile's first byte) + lane offset ----
   unsigned offA[CPW], offB[CPW];
@@ -645,11 +648,18 @@ __global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restr
   for (int c = 0; c < CPW; c++) {
     const int cw = wave * CPW + c, lj = lane >> 3, lp = lane & 7;
     const int lkg = (lp - 4 * (cw & 1) - (lj >> 1)) & 7;
-    kA[c] = lkg * 8;
+    kA[c] = A_KC ? lkg * 8 : cw * (64 / RowA::SPR) + lane / RowA::SPR;
     kB[c] = B_KC ? lkg * 8 : cw * (64 / RowB::SPR) + lane / RowB::SPR;
-    LongType ar = cw * 8 + lj;
-    if (EDGE) ar = m0 + ar < g.M ? ar : g.M - 1 - m0;
-    offA[c] = (unsigned)((ar * lda + lkg * 8) * 2);
+    if (A_KC) {
+      LongType ar = cw * 8 + lj;
+      if (EDGE) ar = m0 + ar < g.M ? ar : g.M - 1 - m0;
+      offA[c] = (unsigned)((ar * lda + lkg * 8) * 2);
+    } else {
+      const int k = cw * (64 / RowA::SPR) + lane / RowA::SPR, pp = lane % RowA::SPR;
+      LongType ac = (pp ^ RowA::swz(k)) * 8;
+      if (EDGE) ac = m0 + ac + 8 <= g.M ? ac : g.M - 8 - m0;
+      offA[c] = (unsigned)(((LongType)k * lda + ac) * 2);
+    }
     if (B_KC) {
       LongType br = cw * 8 + lj;
       if (EDGE) br = n0 + br < g.N ? br : g.N - 1 - n0;
@@ -661,9 +671,9 @@ __global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restr
       offB[c] = (unsigned)(((LongType)k * ldb + bc) * 2);
     }
   }
-  const char* const baseA = reinterpret_cast<const char*>(A + m0 * lda);
+  const char* const baseA = reinterpret_cast<const char*>(A_KC ? A + m0 * lda : A + m0);
   const char* const baseB = reinterpret_cast<const char*>(B_KC ? B + n0 * ldb : B + n0);
-  const LongType stepA = BK * 2, stepB = (B_KC ? (LongType)BK : (LongType)BK * ldb) * 2;   // bytes per K-tile
+  const LongType stepA = (A_KC ? (LongType)BK : (LongType)BK * lda) * 2, stepB = (B_KC ? (LongType)BK : (LongType)BK * ldb) * 2;   // bytes per K-tile
   const LongType KT = KTAIL ? (g.K + BK - 1) / BK : g.K / BK;
   auto dma = [&](const char* base, unsigned off, const u32x4* dst) {
     const unsigned ldsAddr = (unsigned)(size_t)(lds_ptr)dst;
@@ -693,9 +703,10 @@ __global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restr
   };
 
   // ---- LDS side ----
-  int fragA[TW][4], fragB[TW][4], trB[TW];
+  int fragA[TW][4], fragB[TW][4], trB[TW], trA[TW];
 #pragma unroll
   for (int i = 0; i < TW; i++) {
+    trA[i] = RowA::fragOffset(wm * 32 * TW + i * 32, lane);
     const int r = wm * 32 * TW + i * 32 + (lane & 31);
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) fragA[i][ks] = (r >> 3) * 64 + 8 * (r & 7) + ((2 * ks + h + 4 * ((r >> 3) & 1) + ((r & 7) >> 1)) & 7);
@@ -712,7 +723,8 @@ __global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restr
     for (int ks = 0; ks < 4; ks++)
 #pragma unroll
       for (int i = 0; i < TW; i++) {
-        fa[buf][ks][i] = st[fragA[i][ks]];
+        if (A_KC) fa[buf][ks][i] = st[fragA[i][ks]];
+        else fa[buf][ks][i] = RowA::readFrag(st, trA[i], ks);
         if (B_KC) fb[buf][ks][i] = st[fragB[i][ks]];
         else fb[buf][ks][i] = RowB::readFrag(st + SLOTS_A, trB[i], ks);
       }
@@ -1459,10 +1471,10 @@ static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
   // 16-byte column groups)
   static const bool edge = getenv("ND4JHIP_GEMM_EDGE") ? atoi(getenv("ND4JHIP_GEMM_EDGE")) != 0 : true;
   const bool whole = g.M % BM == 0 && g.N % BN == 0;
-  const bool edgeOk = whole || (edge && (B_KC || g.N % 8 == 0));
-  if constexpr (BM == 64 && BN == 64 && WM == 2 && WN == 2 && A_KC) {
+  const bool edgeOk = whole || (edge && (B_KC || g.N % 8 == 0) && (A_KC || g.M % 8 == 0));
+  if constexpr (BM == 64 && BN == 64 && WM == 2 && WN == 2) {
     static const bool small = getenv("ND4JHIP_GEMM_SMALL_RING") ? atoi(getenv("ND4JHIP_GEMM_SMALL_RING")) != 0 : true;
-    const LongType ldaS = g.aRow, ldbS = B_KC ? g.bCol : g.bRow;
+    const LongType ldaS = A_KC ? g.aRow : g.aCol, ldbS = B_KC ? g.bCol : g.bRow;
     ringInstead = small && g.K >= 512 && g.K <= 2048 && (g.K % 256 == 0 || (edge && aligned)) && edgeOk && (whole || aligned) &&
                   ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN) * batch <= 1024 &&
                   ldaS % 8 == 0 && ldbS % 8 == 0 && ldaS < (1 << 23) && ldbS < (1 << 23) &&
@@ -1488,11 +1500,11 @@ static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
   const unsigned nTiles = (unsigned)(((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN) * batch);
   const bool useDeep = aligned && usePipe && !useFull && BM * BN <= 64 * 64 && nTiles <= 1024 && g.K >= 512 && g.M % BM == 0 && g.N % BN == 0 && g.K % 256 == 0;
   // the direct-load ring takes the small-tile launches it can: 64 x 64 or 128 x 128 tiles, A k-contiguous, 16-byte aligned rows
-  if constexpr ((BM == 64 && BN == 64 || BM == 128 && BN == 128) && WM == 2 && WN == 2 && A_KC) {
+  if constexpr ((BM == 64 && BN == 64 || BM == 128 && BN == 128) && WM == 2 && WN == 2) {
     constexpr int TW = BM / 64;
     constexpr int STAGE_BYTES = (BM + BN) * 8 * 16;
     static const bool small = getenv("ND4JHIP_GEMM_SMALL_RING") ? atoi(getenv("ND4JHIP_GEMM_SMALL_RING")) != 0 : true;
-    const LongType ldaS = g.aRow, ldbS = B_KC ? g.bCol : g.bRow;
+    const LongType ldaS = A_KC ? g.aRow : g.aCol, ldbS = B_KC ? g.bCol : g.bRow;
     // ragged M / N, or a K that is not a whole number of K-tiles: the edge instantiation, with the zero page for the end of
     // K where K is not a multiple of 256 (whole tiles and a K of whole K-tiles keep the kernels they had)
     const bool ktail = g.K % 256 != 0;
@@ -1510,21 +1522,21 @@ static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
       const LongType kTiles = (g.K + 63) / 64;
       const bool wantDeep = TW == 2 || (nTiles <= 256 && (ktail ? (kTiles + 7) / 8 * 8 - kTiles <= 1 : g.K % 512 == 0));
       const bool plain = !edgeShape;
-      const bool grantedDeep = plain   ? DynLds<gemm_mfma16s<T, B_KC, DEEP, TW>, DEEP * STAGE_BYTES>::granted()
-                               : ktail ? DynLds<gemm_mfma16s<T, B_KC, DEEP, TW, true, true>, DEEP * STAGE_BYTES>::granted()
-                                       : DynLds<gemm_mfma16s<T, B_KC, DEEP, TW, true>, DEEP * STAGE_BYTES>::granted();
+      const bool grantedDeep = plain   ? DynLds<gemm_mfma16s<T, B_KC, DEEP, TW, false, false, A_KC>, DEEP * STAGE_BYTES>::granted()
+                               : ktail ? DynLds<gemm_mfma16s<T, B_KC, DEEP, TW, true, true, A_KC>, DEEP * STAGE_BYTES>::granted()
+                                       : DynLds<gemm_mfma16s<T, B_KC, DEEP, TW, true, false, A_KC>, DEEP * STAGE_BYTES>::granted();
       const char* const flavour = plain ? "" : ktail ? ",edge,ktail" : ",edge";
       if (wantDeep && grantedDeep) {
-        noteKernel("gemm_mfma16s<%s,%dx%d,akc=1,bkc=%d,stages=%d%s>", tname<T>(), BM, BN, (int)B_KC, DEEP, flavour);
-        auto kern = plain   ? gemm_mfma16s<T, B_KC, DEEP, TW, false, false>
-                    : ktail ? gemm_mfma16s<T, B_KC, DEEP, TW, true, true> : gemm_mfma16s<T, B_KC, DEEP, TW, true, false>;
+        noteKernel("gemm_mfma16s<%s,%dx%d,akc=%d,bkc=%d,stages=%d%s>", tname<T>(), BM, BN, (int)A_KC, (int)B_KC, DEEP, flavour);
+        auto kern = plain   ? gemm_mfma16s<T, B_KC, DEEP, TW, false, false, A_KC>
+                    : ktail ? gemm_mfma16s<T, B_KC, DEEP, TW, true, true, A_KC> : gemm_mfma16s<T, B_KC, DEEP, TW, true, false, A_KC>;
         hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(256), DEEP * STAGE_BYTES, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
         return true;
       }
       if constexpr (TW == 1) {
-        noteKernel("gemm_mfma16s<%s,64x64,akc=1,bkc=%d,stages=4%s>", tname<T>(), (int)B_KC, flavour);
-        auto kern = plain   ? gemm_mfma16s<T, B_KC, 4, 1, false, false>
-                    : ktail ? gemm_mfma16s<T, B_KC, 4, 1, true, true> : gemm_mfma16s<T, B_KC, 4, 1, true, false>;
+        noteKernel("gemm_mfma16s<%s,64x64,akc=%d,bkc=%d,stages=4%s>", tname<T>(), (int)A_KC, (int)B_KC, flavour);
+        auto kern = plain   ? gemm_mfma16s<T, B_KC, 4, 1, false, false, A_KC>
+                    : ktail ? gemm_mfma16s<T, B_KC, 4, 1, true, true, A_KC> : gemm_mfma16s<T, B_KC, 4, 1, true, false, A_KC>;
         hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(256), 4 * STAGE_BYTES, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
         return true;
       }

@@ -67,13 +67,13 @@ CASES = [
     (BFLOAT16, 4096, 4096, 192, "gemm_mfma16d<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1>", None),
     # BASELINE config 2 at 1024^3
     (FLOAT32, 1024, 1024, 1024, "gemm_mfma32q<f32,64x64,akc=1,bkc=0,pd=4,bk=32>", "gemm_mfma32q<f32,64x64,akc=1,bkc=1,pd=4,bk=32>", "gemm_mfma32q<f32,64x64,akc=0,bkc=0,pd=4,bk=32>"),
-    (HALF, 1024, 1024, 1024, "gemm_mfma16s<f16,64x64,akc=1,bkc=0,stages=8>", "gemm_mfma16s<f16,64x64,akc=1,bkc=1,stages=8>", "gemm_mfma16q<f16,64x64,akc=0,bkc=0>"),
-    (BFLOAT16, 1024, 1024, 1024, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=8>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=8>", "gemm_mfma16q<bf16,64x64,akc=0,bkc=0>"),
+    (HALF, 1024, 1024, 1024, "gemm_mfma16s<f16,64x64,akc=1,bkc=0,stages=8>", "gemm_mfma16s<f16,64x64,akc=1,bkc=1,stages=8>", "gemm_mfma16s<f16,64x64,akc=0,bkc=0,stages=8>"),
+    (BFLOAT16, 1024, 1024, 1024, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=8>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=8>", "gemm_mfma16s<bf16,64x64,akc=0,bkc=0,stages=8>"),
     # the 128 x 128 configuration (2048-class sizes), whole tiles
-    (BFLOAT16, 2048, 2048, 2048, "gemm_mfma16s<bf16,128x128,akc=1,bkc=0,stages=4>", "gemm_mfma16s<bf16,128x128,akc=1,bkc=1,stages=4>", "gemm_mfma16f<bf16,128x128,akc=0,bkc=0>"),
+    (BFLOAT16, 2048, 2048, 2048, "gemm_mfma16s<bf16,128x128,akc=1,bkc=0,stages=4>", "gemm_mfma16s<bf16,128x128,akc=1,bkc=1,stages=4>", "gemm_mfma16s<bf16,128x128,akc=0,bkc=0,stages=4>"),
     (HALF, 2048, 2048, 1024, "gemm_mfma16s<f16,128x128,akc=1,bkc=0,stages=4>", "gemm_mfma16s<f16,128x128,akc=1,bkc=1,stages=4>", None),
     # a K of whole K-tiles that is not a multiple of four of them stays on the register-staged kernel
-    (HALF, 2048, 2048, 320, "gemm_mfma16f<f16,128x128,akc=1,bkc=0>", "gemm_mfma16f<f16,128x128,akc=1,bkc=1>", None),
+    (HALF, 2048, 2048, 320, "gemm_mfma16f<f16,128x128,akc=1,bkc=0>", "gemm_mfma16f<f16,128x128,akc=1,bkc=1>", "gemm_mfma16f<f16,128x128,akc=0,bkc=0>"),
     # ragged edges on the large tiles (bounds-handling kernel)
     (BFLOAT16, 3600, 3704, 72, "gemm_mfma16p<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16p<bf16,256x256,akc=1,bkc=1>", "gemm_mfma16p<bf16,256x256,akc=0,bkc=0>"),
     # ... from K = 128 on the direct-load kernels take them, also with a K that ends inside a K-tile
@@ -83,18 +83,18 @@ CASES = [
     (BFLOAT16, 3600, 3704, 1024, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0,edge>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1,edge>", "gemm_mfma16p<bf16,256x256,akc=0,bkc=0>"),
     (HALF, 3599, 3592, 192, "gemm_mfma16d<f16,256x256,akc=1,bkc=0,edge>", "gemm_mfma16d<f16,256x256,akc=1,bkc=1,edge>", None),
     (BFLOAT16, 3601, 3585, 256, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0,edge,unaligned>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1,edge>", None),
-    (BFLOAT16, 2000, 2000, 2048, "gemm_mfma16s<bf16,128x128,akc=1,bkc=0,stages=4,edge>", "gemm_mfma16s<bf16,128x128,akc=1,bkc=1,stages=4,edge>", None),
-    (HALF, 1000, 1000, 1024, "gemm_mfma16s<f16,64x64,akc=1,bkc=0,stages=8,edge>", "gemm_mfma16s<f16,64x64,akc=1,bkc=1,stages=8,edge>", None),
+    (BFLOAT16, 2000, 2000, 2048, "gemm_mfma16s<bf16,128x128,akc=1,bkc=0,stages=4,edge>", "gemm_mfma16s<bf16,128x128,akc=1,bkc=1,stages=4,edge>", "gemm_mfma16s<bf16,128x128,akc=0,bkc=0,stages=4,edge>"),
+    (HALF, 1000, 1000, 1024, "gemm_mfma16s<f16,64x64,akc=1,bkc=0,stages=8,edge>", "gemm_mfma16s<f16,64x64,akc=1,bkc=1,stages=8,edge>", "gemm_mfma16s<f16,64x64,akc=0,bkc=0,stages=8,edge>"),
     (BFLOAT16, 500, 2304, 768, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=4,edge>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=4,edge>", None),
     # ... and with a K that is not a whole number of K-tiles (from 512 on: the ring kernel with the page of zeros; below: the
     # bounds-handling kernel)
     (HALF, 1800, 1800, 520, "gemm_mfma16s<f16,128x128,akc=1,bkc=0,stages=4,edge,ktail>", "gemm_mfma16s<f16,128x128,akc=1,bkc=1,stages=4,edge,ktail>", None),
-    (BFLOAT16, 1104, 904, 1000, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=4,edge,ktail>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=4,edge,ktail>", None),
+    (BFLOAT16, 1104, 904, 1000, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=4,edge,ktail>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=4,edge,ktail>", "gemm_mfma16s<bf16,64x64,akc=0,bkc=0,stages=4,edge,ktail>"),
     (HALF, 1800, 1800, 328, "gemm_mfma16p<f16,128x128,akc=1,bkc=0>", "gemm_mfma16p<f16,128x128,akc=1,bkc=1>", None),
     (BFLOAT16, 1104, 904, 200, "gemm_mfma16p<bf16,64x64,akc=1,bkc=0>", "gemm_mfma16p<bf16,64x64,akc=1,bkc=1>", None),
     # K a multiple of 256 but not of 512: the four-stage ring; more tiles than CUs (two blocks on a CU): four stages as well;
     # the shortest K the ring takes
-    (BFLOAT16, 1024, 1024, 768, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=4>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=4>", "gemm_mfma16q<bf16,64x64,akc=0,bkc=0>"),
+    (BFLOAT16, 1024, 1024, 768, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=4>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=4>", "gemm_mfma16s<bf16,64x64,akc=0,bkc=0,stages=4>"),
     (HALF, 512, 2304, 1024, "gemm_mfma16s<f16,64x64,akc=1,bkc=0,stages=4>", "gemm_mfma16s<f16,64x64,akc=1,bkc=1,stages=4>", None),
     (BFLOAT16, 1024, 1024, 512, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=8>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=8>", None),
     (FLOAT32, 1024, 1024, 384, "gemm_mfma32q<f32,64x64,akc=1,bkc=0,pd=4,bk=32>", "gemm_mfma32q<f32,64x64,akc=1,bkc=1,pd=4,bk=32>", None),
