@@ -931,7 +931,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16f(GemmArgs g, const T
 // elements of C beyond the edge, which the bounds-checked store leaves out.
 // KTAIL: K need not be a whole number of K-tiles -- lanes whose 16 bytes start at k >= K read a page of zeros (see
 // gemm_mfma16s).
-template <typename T, bool B_KC, bool EDGE = false, bool KTAIL = false>
+// A_KC = false: A lies [k][m] with unit m stride (a transposed A) and takes the row-major path of B on its side.
+template <typename T, bool B_KC, bool EDGE = false, bool KTAIL = false, bool A_KC = true>
 __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
                                                     unsigned tilesM, unsigned tilesN) {
   constexpr int BM = 256, BN = 256, BK = 64, WN = 4, WTM = 128, WTN = 64, TM = 4, TN = 2, NM = TM * TN;
@@ -948,7 +949,7 @@ __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restr
   const LongType m0 = (LongType)tm * BM, n0 = (LongType)tn * BN;
   const LongType bz = blockIdx.z;
   { LongType oa, ob, oc; batchOffsets(g, bz, oa, ob, oc); A += oa; B += ob; C += oc; }
-  const LongType lda = g.aRow, ldb = B_KC ? g.bCol : g.bRow;
+  const LongType lda = A_KC ? g.aRow : g.aCol, ldb = B_KC ? g.bCol : g.bRow;
   const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6), h = lane >> 5;
   const int wm = wave / WN, wn = wave % WN;
 
@@ -962,11 +963,18 @@ __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restr
   for (int i = 0; i < 4; i++) {
     const int cw = wave * 4 + i;
     const int lkg = (lp - 4 * (cw & 1) - (lj >> 1)) & 7;
-    akg[i] = lkg * 8;
+    akg[i] = A_KC ? lkg * 8 : 2 * cw + (lane >> 5);
     bkg[i] = B_KC ? lkg * 8 : 2 * cw + (lane >> 5);
-    LongType ar = m0 + cw * 8 + lj;
-    if (EDGE) ar = ar < g.M ? ar : g.M - 1;
-    aSrc[i] = A + ar * lda + lkg * 8;
+    if (A_KC) {
+      LongType ar = m0 + cw * 8 + lj;
+      if (EDGE) ar = ar < g.M ? ar : g.M - 1;
+      aSrc[i] = A + ar * lda + lkg * 8;
+    } else {
+      const int kr = 2 * cw + (lane >> 5), q = lane & 31, c = q ^ (4 * (kr & 3));
+      LongType ac = m0 + 8 * c;
+      if (EDGE) ac = ac + 8 <= g.M ? ac : g.M - 8;
+      aSrc[i] = A + (LongType)kr * lda + ac;
+    }
     if (B_KC) {
       LongType br = n0 + cw * 8 + lj;
       if (EDGE) br = br < g.N ? br : g.N - 1;
@@ -978,7 +986,7 @@ __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restr
       bSrc[i] = B + (LongType)kr * ldb + bc;
     }
   }
-  const LongType aStep = BK, bStep = B_KC ? (LongType)BK : (LongType)BK * ldb;
+  const LongType aStep = A_KC ? (LongType)BK : (LongType)BK * lda, bStep = B_KC ? (LongType)BK : (LongType)BK * ldb;
   // The loads are written as assembly on purpose.  Issued through the builtin, the compiler's wait-count pass knows of
   // an outstanding write into LDS and, having no alias information for the transposing read, puts s_waitcnt vmcnt(0)
   // in front of every ds_read_b64_tr_b16 that follows -- twice per K-tile the wave then sits out the whole latency of
@@ -1015,6 +1023,15 @@ __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restr
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) offA[i][ks] = (r >> 3) * 64 + 8 * (r & 7) + ((2 * ks + h + 4 * ((r >> 3) & 1) + ((r & 7) >> 1)) & 7);
   }
+  int trA[TM];   // byte offsets of the transposing reads (row-major A)
+#pragma unroll
+  for (int i = 0; i < TM; i++) {
+    const int grp = lane >> 4, i16 = lane & 15;
+    const int n4 = wm * WTM + i * 32 + 16 * (grp & 1) + 4 * (i16 & 3);
+    const int k = 8 * (grp >> 1) + (i16 >> 2);
+    const int phys = (n4 >> 3) ^ (4 * ((i16 >> 2) & 3));
+    trA[i] = k * 512 + phys * 16 + ((n4 >> 2) & 1) * 8;
+  }
   int trB[TN];   // byte offsets of the transposing reads (row-major B)
 #pragma unroll
   for (int jt = 0; jt < TN; jt++) {
@@ -1036,7 +1053,18 @@ __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restr
   u32x4 fa[2][TM], fb[2][TN];
   auto readFrag = [&](const u32x4* stage, int ks, int buf) {
 #pragma unroll
-    for (int i = 0; i < TM; i++) fa[buf][i] = stage[offA[i][ks]];
+    for (int i = 0; i < TM; i++) {
+      if (A_KC) {
+        fa[buf][i] = stage[offA[i][ks]];
+      } else {
+        const __attribute__((address_space(3))) unsigned char* base =
+            (const __attribute__((address_space(3))) unsigned char*)(lds_ptr)stage + trA[i] + ks * 8192;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)base);
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(base + 2048));
+        const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+        fa[buf][i] = u32x4{l2[0], l2[1], h2[0], h2[1]};
+      }
+    }
 #pragma unroll
     for (int jt = 0; jt < TN; jt++) {
       if (B_KC) {
@@ -1576,6 +1604,28 @@ static bool launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const 
   if (g.M <= 64 || g.N <= 64 || tiles128 < 192) return launchMfma16Cfg<T, 64, 64, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch, true, aligned);
   if (tiles256 < 192) return launchMfma16Cfg<T, 128, 128, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch, false, aligned);
   if (g.hasEpi) return false;
+  if constexpr (!A_KC && !B_KC) {
+    // the same for a transposed A (the two-stage kernel with both operands' k-rows in LDS as they lie in memory)
+    static const bool ub = getenv("ND4JHIP_GEMM_UNALIGNED_RING") ? atoi(getenv("ND4JHIP_GEMM_UNALIGNED_RING")) != 0 : true;
+    constexpr size_t LDS = 2 * 2 * 256 * 8 * 16;
+    if (!aligned && ub && batch == 1 && (reinterpret_cast<uintptr_t>(A) & 15) == 0 && g.aCol % 8 == 0 && g.M % 8 == 0 && g.K >= 128 && g.N >= 264 &&
+        DynLds<gemm_mfma16d<T, false, true, false, false>, (int)LDS>::granted() && DynLds<gemm_mfma16d<T, false, true, true, false>, (int)LDS>::granted()) {
+      GemmArgs g1 = g;
+      g1.N = g.N & ~(LongType)7;
+      const unsigned tM = (unsigned)((g.M + 255) / 256), tN = (unsigned)((g1.N + 255) / 256);
+      auto kern = g.K % 64 == 0 ? gemm_mfma16d<T, false, true, false, false> : gemm_mfma16d<T, false, true, true, false>;
+      hipLaunchKernelGGL(kern, dim3(tM * tN, 1, 1), dim3(512), LDS, s, g1, (const T*)A, (const T*)B, (T*)C, tM, tN);
+      const LongType rem = g.N & 7;
+      if (rem) {
+        GemmArgs g2 = g;
+        g2.N = rem;
+        if (g.bias) g2.bias = static_cast<const T*>(g.bias) + g1.N;
+        if (!launchMfma16Cfg<T, 64, 64, 2, 2, A_KC, B_KC>(s, g2, A, (const T*)B + g1.N, (T*)C + g1.N * g.cCol, 1, false, false)) return false;
+      }
+      noteKernel("gemm_mfma16d<%s,256x256,akc=0,bkc=0,edge%s,unaligned>", tname<T>(), g.K % 64 == 0 ? "" : ",ktail");
+      return true;
+    }
+  }
   if constexpr (A_KC && !B_KC) {
     // A row-major B whose rows start off 16-byte boundaries (a [768, 50257] matrix) with everything else in place for the
     // ring kernel: its loads into LDS take element-aligned addresses like any other global load, and every column group
@@ -1608,7 +1658,7 @@ static bool launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const 
   // row-major B in whole 16-byte column groups only)
   static const bool edge = getenv("ND4JHIP_GEMM_EDGE") ? atoi(getenv("ND4JHIP_GEMM_EDGE")) != 0 : true;
   const bool whole = g.M % 256 == 0 && g.N % 256 == 0;
-  const bool edgeOk = whole || (edge && (B_KC || g.N % 8 == 0));
+  const bool edgeOk = whole || (edge && (B_KC || g.N % 8 == 0) && (A_KC || g.M % 8 == 0));
   const unsigned tM = (unsigned)((g.M + 255) / 256), tN = (unsigned)((g.N + 255) / 256);
   if constexpr (A_KC && !B_KC) {
     constexpr size_t LDS = (3 * 256 * 8 + 4 * 32 * 32) * 16;   // 160 KiB: the whole LDS of a CU
@@ -1645,6 +1695,24 @@ static bool launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const 
       auto kern = gemm_mfma16d<T, true, true, true>;
       hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(512), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
       return true;
+    }
+  }
+  if constexpr (!A_KC) {
+    // a transposed A: the two-stage direct-load kernel with A's k-rows in LDS as they lie in memory
+    static const bool taDirect = getenv("ND4JHIP_GEMM_TA_DIRECT") ? atoi(getenv("ND4JHIP_GEMM_TA_DIRECT")) != 0 : true;
+    constexpr size_t LDS = 2 * 2 * 256 * 8 * 16;
+    const bool ktail = g.K % 64 != 0;
+    if (direct && taDirect && edgeOk && g.K >= 128 && (edge || (whole && !ktail))) {
+      auto kern = ktail   ? gemm_mfma16d<T, B_KC, true, true, false>
+                  : whole ? gemm_mfma16d<T, B_KC, false, false, false> : gemm_mfma16d<T, B_KC, true, false, false>;
+      const bool granted = ktail   ? DynLds<gemm_mfma16d<T, B_KC, true, true, false>, (int)LDS>::granted()
+                           : whole ? DynLds<gemm_mfma16d<T, B_KC, false, false, false>, (int)LDS>::granted()
+                                   : DynLds<gemm_mfma16d<T, B_KC, true, false, false>, (int)LDS>::granted();
+      if (granted) {
+        noteKernel("gemm_mfma16d<%s,256x256,akc=0,bkc=%d%s>", tname<T>(), (int)B_KC, ktail ? ",edge,ktail" : whole ? "" : ",edge");
+        hipLaunchKernelGGL(kern, dim3(tM * tN, 1, (unsigned)batch), dim3(512), LDS, s, g, (const T*)A, (const T*)B, (T*)C, tM, tN);
+        return true;
+      }
     }
   }
   return launchMfma16Cfg<T, 256, 256, 2, 4, A_KC, B_KC>(s, g, A, B, C, batch, false, true);

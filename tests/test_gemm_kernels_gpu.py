@@ -57,8 +57,8 @@ def _check_rows_cols(z, a64, b64, tol, rng, what):
 CASES = [
     # BASELINE config 2 at 4096^3
     (FLOAT32, 4096, 4096, 4096, "gemm_mfma32q<f32,128x128,akc=1,bkc=0,pd=4,bk=16>", "gemm_mfma32q<f32,128x128,akc=1,bkc=1,pd=4,bk=16>", "gemm_mfma32q<f32,128x128,akc=0,bkc=0,pd=4,bk=16>"),
-    (HALF, 4096, 4096, 4096, "gemm_mfma16r<f16,256x256,akc=1,bkc=0>", "gemm_mfma16d<f16,256x256,akc=1,bkc=1>", "gemm_mfma16f<f16,256x256,akc=0,bkc=0>"),
-    (BFLOAT16, 4096, 4096, 4096, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1>", "gemm_mfma16f<bf16,256x256,akc=0,bkc=0>"),
+    (HALF, 4096, 4096, 4096, "gemm_mfma16r<f16,256x256,akc=1,bkc=0>", "gemm_mfma16d<f16,256x256,akc=1,bkc=1>", "gemm_mfma16d<f16,256x256,akc=0,bkc=0>"),
+    (BFLOAT16, 4096, 4096, 4096, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1>", "gemm_mfma16d<bf16,256x256,akc=0,bkc=0>"),
     # the ring kernel at its shortest K (the prologue alone fills the rings) and at a K that ends in the middle of both rings;
     # a K that is a multiple of 64 only stays on the two-stage direct kernel
     (BFLOAT16, 4096, 4096, 128, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1>", None),
@@ -77,10 +77,10 @@ CASES = [
     # ragged edges on the large tiles (bounds-handling kernel)
     (BFLOAT16, 3600, 3704, 72, "gemm_mfma16p<bf16,256x256,akc=1,bkc=0>", "gemm_mfma16p<bf16,256x256,akc=1,bkc=1>", "gemm_mfma16p<bf16,256x256,akc=0,bkc=0>"),
     # ... from K = 128 on the direct-load kernels take them, also with a K that ends inside a K-tile
-    (BFLOAT16, 3600, 3704, 1000, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0,edge,ktail>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1,edge,ktail>", "gemm_mfma16p<bf16,256x256,akc=0,bkc=0>"),
+    (BFLOAT16, 3600, 3704, 1000, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0,edge,ktail>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1,edge,ktail>", "gemm_mfma16d<bf16,256x256,akc=0,bkc=0,edge,ktail>"),
     # ragged edges with aligned rows and a K of whole K-tiles: the direct-load kernels' edge instantiations (clamped loads,
     # bounds-checked store) -- a last tile row of 16 rows and a last tile column of 120, of 8 (one column group) and of 1
-    (BFLOAT16, 3600, 3704, 1024, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0,edge>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1,edge>", "gemm_mfma16p<bf16,256x256,akc=0,bkc=0>"),
+    (BFLOAT16, 3600, 3704, 1024, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0,edge>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1,edge>", "gemm_mfma16d<bf16,256x256,akc=0,bkc=0,edge>"),
     (HALF, 3599, 3592, 192, "gemm_mfma16d<f16,256x256,akc=1,bkc=0,edge>", "gemm_mfma16d<f16,256x256,akc=1,bkc=1,edge>", None),
     (BFLOAT16, 3601, 3585, 256, "gemm_mfma16r<bf16,256x256,akc=1,bkc=0,edge,unaligned>", "gemm_mfma16d<bf16,256x256,akc=1,bkc=1,edge>", None),
     (BFLOAT16, 2000, 2000, 2048, "gemm_mfma16s<bf16,128x128,akc=1,bkc=0,stages=4,edge>", "gemm_mfma16s<bf16,128x128,akc=1,bkc=1,stages=4,edge>", "gemm_mfma16s<bf16,128x128,akc=0,bkc=0,stages=4,edge>"),
@@ -184,6 +184,13 @@ def _whole_result(ex, dtype, M, N, K, tb, expect=",edge"):
     assert expect in name, name
     assert ("unaligned" in name) == (dtype != FLOAT32 and N % 8 != 0 and not tb), name
     assert_close(z, a64 @ b64, TOL[dtype], TOL[dtype], "whole result")
+    if dtype != FLOAT32 and M % 8 == 0:
+        # the same product with A handed over transposed ([K, M], the transposeA flag): the kernels that keep A's k-rows in LDS
+        At, _ = _device(a.T, dtype)
+        zt = ex.exec_custom("matmul", [At, B], i_args=[1, 1 if tb else 0])[0].to_float()
+        name = _last_kernel(ex)
+        assert expect in name and "akc=0" in name, name
+        assert_close(zt, a64 @ b64, TOL[dtype], TOL[dtype], "whole result, transposed A")
 
 
 @pytest.mark.parametrize("n", [1024, 4096])
