@@ -45,7 +45,7 @@ TRAFFIC_MB = {
     "layer_norm fp32": 100.8, "gelu fp32": 100.7, "softmax fp32": 1610.6, "layer_norm bf16": 50.4, "gelu bf16": 50.4,
     "softmax bf16": 805.3, "dot_product_attention_v2": 50.5, "dot_product_attention_v2 f32": 110.9,
     "reduce_cols": 101.0, "index_cols": 101.2, "transpose_tiled": 201.2, "cast_contig": 150.9, "softmax_block_regs": 205.8,
-    "mmul unaligned": 1223.8,
+    "mmul unaligned": 913.8, "mmul ragged tb": 903.1, "mmul ragged bf16 500": 12.6, "mmul ragged bf16 2000": 58.9, "mmul ragged f32 2000": 115.5,
 }
 
 
@@ -556,7 +556,7 @@ def main():
                 Ra.sync_to_device(); Rb.sync_to_device()
                 w, e = timed(ex, L, ex.bind_custom("matmul", [Ra, Rb], [Rz]), steps, warmup)
                 ops.append({"op": "mmul %s %d x %d x %d (ragged: %s)" % (nm, rm, rn, rk, L.nd4jhipLastGemmKernel().decode()),
-                            "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": mfma_entry(2.0 * rm * rn * rk, e, nm, "mmul ragged")})
+                            "ms": round(e, 4), "wall_ms": round(w, 4), "roofline": mfma_entry(2.0 * rm * rn * rk, e, nm, "mmul ragged %s %d" % (nm, rm))})
                 del Ra, Rb, Rz, ra, rb
         if 2 in cfgs:
             # config 2, the remaining sizes/dtypes

@@ -1536,7 +1536,8 @@ static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
     // ragged M / N, or a K that is not a whole number of K-tiles: the edge instantiation, with the zero page for the end of
     // K where K is not a multiple of 256 (whole tiles and a K of whole K-tiles keep the kernels they had)
     const bool ktail = g.K % 256 != 0;
-    const bool edgeShape = (!whole || g.K % 64 != 0) && edge && edgeOk && aligned && usePipe && nTiles <= 1024 && g.K >= 512;
+    static const LongType edgeMinK = getenv("ND4JHIP_GEMM_EDGE_MIN_K") ? atoi(getenv("ND4JHIP_GEMM_EDGE_MIN_K")) : 512;
+    const bool edgeShape = (!whole || g.K % 64 != 0) && edge && edgeOk && aligned && usePipe && nTiles <= 1024 && g.K >= edgeMinK;
     const bool shape = edgeShape || (TW == 1 ? useDeep : (useFull && nTiles <= 1024 && g.K >= 512 && g.K % 256 == 0));
     if (small && shape && ldaS % 8 == 0 && ldbS % 8 == 0 && ldaS < (1 << 23) && ldbS < (1 << 23) &&
         ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 && g.aBatch % 8 == 0 && g.bBatch % 8 == 0 &&
