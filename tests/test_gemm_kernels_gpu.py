@@ -86,12 +86,12 @@ CASES = [
     (BFLOAT16, 2000, 2000, 2048, "gemm_mfma16s<bf16,128x128,akc=1,bkc=0,stages=4,edge>", "gemm_mfma16s<bf16,128x128,akc=1,bkc=1,stages=4,edge>", "gemm_mfma16s<bf16,128x128,akc=0,bkc=0,stages=4,edge>"),
     (HALF, 1000, 1000, 1024, "gemm_mfma16s<f16,64x64,akc=1,bkc=0,stages=8,edge>", "gemm_mfma16s<f16,64x64,akc=1,bkc=1,stages=8,edge>", "gemm_mfma16s<f16,64x64,akc=0,bkc=0,stages=8,edge>"),
     (BFLOAT16, 500, 2304, 768, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=4,edge>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=4,edge>", None),
-    # ... and with a K that is not a whole number of K-tiles (from 512 on: the ring kernel with the page of zeros; below: the
+    # ... and with a K that is not a whole number of K-tiles (from 128 on: the ring kernel with the page of zeros; below: the
     # bounds-handling kernel)
     (HALF, 1800, 1800, 520, "gemm_mfma16s<f16,128x128,akc=1,bkc=0,stages=4,edge,ktail>", "gemm_mfma16s<f16,128x128,akc=1,bkc=1,stages=4,edge,ktail>", None),
     (BFLOAT16, 1104, 904, 1000, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=4,edge,ktail>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=4,edge,ktail>", "gemm_mfma16s<bf16,64x64,akc=0,bkc=0,stages=4,edge,ktail>"),
-    (HALF, 1800, 1800, 328, "gemm_mfma16p<f16,128x128,akc=1,bkc=0>", "gemm_mfma16p<f16,128x128,akc=1,bkc=1>", None),
-    (BFLOAT16, 1104, 904, 200, "gemm_mfma16p<bf16,64x64,akc=1,bkc=0>", "gemm_mfma16p<bf16,64x64,akc=1,bkc=1>", None),
+    (HALF, 1800, 1800, 72, "gemm_mfma16p<f16,128x128,akc=1,bkc=0>", "gemm_mfma16p<f16,128x128,akc=1,bkc=1>", None),
+    (BFLOAT16, 1104, 904, 104, "gemm_mfma16p<bf16,64x64,akc=1,bkc=0>", "gemm_mfma16p<bf16,64x64,akc=1,bkc=1>", None),
     # K a multiple of 256 but not of 512: the four-stage ring; more tiles than CUs (two blocks on a CU): four stages as well;
     # the shortest K the ring takes
     (BFLOAT16, 1024, 1024, 768, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=4>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=4>", "gemm_mfma16s<bf16,64x64,akc=0,bkc=0,stages=4>"),
@@ -159,9 +159,10 @@ def test_ragged_product_on_the_direct_load_kernels_whole_result(ex, dtype, M, N,
 @pytest.mark.parametrize("tb", [False, True], ids=["plain", "transposeB"])
 @pytest.mark.parametrize("dtype,M,N,K", [(BFLOAT16, 1000, 1000, 1000), (HALF, 1024, 1024, 520), (BFLOAT16, 2000, 2000, 1000), (HALF, 512, 512, 1992),
                                          (BFLOAT16, 1920, 2048, 968), (BFLOAT16, 3700, 3704, 1000), (HALF, 4096, 3840, 136),
-                                         (FLOAT32, 1000, 1000, 1000), (FLOAT32, 1920, 2048, 268)],
+                                         (FLOAT32, 1000, 1000, 1000), (FLOAT32, 1920, 2048, 268), (BFLOAT16, 1000, 1000, 136), (HALF, 2000, 1800, 328),
+                                         (BFLOAT16, 504, 504, 200)],
                          ids=["bf16-1000", "f16-whole-tiles-k520", "bf16-128x128-tiles", "f16-few-tiles", "bf16-k968", "bf16-256x256-tiles", "f16-256x256-k136",
-                              "f32-1000", "f32-128x128-k268"])
+                              "f32-1000", "f32-128x128-k268", "bf16-k136", "f16-128x128-k328", "bf16-few-tiles-k200"])
 def test_k_tail_on_the_direct_load_kernels_whole_result(ex, dtype, M, N, K, tb):
     """A K that is not a whole number of K-tiles on the ring kernel: the lanes beyond K read a page of zeros.  Every element of
     the result, with operands whose neighbours in memory (the next row, which a load past K would bring in) are large."""
