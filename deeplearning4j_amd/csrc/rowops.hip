@@ -386,13 +386,35 @@ __global__ __launch_bounds__(512) void softmax_block_regs(RowArgs a, const T* __
   if (!LOG && clamp && mx == NEG) mx = (A)0;
   A sum = (A)0;
   auto term = [&](A val) -> A { if constexpr (LOG) return r_exp<A>(val - mx); else return softmax_term(val, mx, clamp); };
-  sweep([&](A val) { sum += term(val); });
+  // fp32 rows: the exponentials take the place of the row in its registers (the same values in the same order of summation);
+  // a 16-bit row stays packed and its exponentials are taken again on the way out
+  constexpr bool KEEP = sizeof(T) == 4 && sizeof(A) == 4;
+  A tailE = tailv;
+  if constexpr (KEEP) {
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      if ((LongType)i * NT + t < nv) {
+        A vals[VEC];
+        RawIO<T>::unpack(v[i], vals);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) { vals[e] = term(vals[e]); sum += vals[e]; }
+        v[i] = RawIO<T>::pack(vals);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (hasTail) { tailE = term(tailv); sum += tailE; }
+  } else {
+    sweep([&](A val) { sum += term(val); });
+  }
   sum = block_allreduce<SumOp, NT / 64, A>(sum, lds);
   if (!LOG && clamp) sum = sum > (A)1e-6f ? sum : (A)1e-6f;
-  // long rows: the maximum passes through an opaque copy, so that the exponentials of the sum pass are taken again here
+  // long 16-bit rows: the maximum passes through an opaque copy, so that the exponentials of the sum pass are taken again here
   // instead of being kept in (spilled) registers
-  if constexpr (NV > 16 && sizeof(A) == 4) asm volatile("" : "+v"(mx));
-  auto result = [&](A val) -> A { if constexpr (LOG) return r_log<A>(term(val) / sum); else return term(val) / sum; };
+  if constexpr (NV > 16 && sizeof(A) == 4 && !KEEP) asm volatile("" : "+v"(mx));
+  auto result = [&](A val) -> A {
+    const A e = KEEP ? val : term(val);
+    if constexpr (LOG) return r_log<A>(e / sum); else return e / sum;
+  };
 #pragma unroll
   for (int i = 0; i < NV; i++) {
     const LongType iv = (LongType)i * NT + t;
@@ -411,7 +433,7 @@ __global__ __launch_bounds__(512) void softmax_block_regs(RowArgs a, const T* __
     }
     __builtin_amdgcn_sched_barrier(0);
   }
-  if (hasTail) zr[tail0 + t] = Conv<T>::from(result(tailv));
+  if (hasTail) zr[tail0 + t] = Conv<T>::from(result(tailE));
 }
 template <typename T, bool LOG>
 static bool softmaxBlockRegs(hipStream_t s, const RowArgs& a, const T* x, T* z, int clamp, const RowPlan& p) {
