@@ -269,6 +269,28 @@ __device__ __forceinline__ void storeAccTiles(const GemmArgs& g, T* __restrict__
   }
 }
 
+// split-K: park a block's partial tile (split blockIdx.y) for splitk_finish.  Layout of one partial tile:
+// [q-group (i, j, r / 4)][thread][4 floats] -- 16-byte accesses, coalesced over the block.  A q-group holds 4 consecutive
+// rows of one column; groups whose rows all lie beyond M are skipped.  rowBase / colBase: the wave's corner of the tile.
+template <int TM, int TN, int NT>
+__device__ __forceinline__ void storePartialTile(const GemmArgs& g, const f32x16 (&acc)[TM][TN], LongType tileLinear, LongType rowBase, LongType colBase,
+                                                 int t, int lane) {
+  constexpr int Q = TM * TN * 4;
+  f32x4v* const mine = reinterpret_cast<f32x4v*>(g.partial) + (tileLinear * g.splits + blockIdx.y) * (LongType)(Q * NT);
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const int idx = (i * TN + j) * 4 + q;
+        if (rowBase + i * 32 + 8 * q + 4 * (lane >> 5) < g.M && colBase + j * 32 + (lane & 31) < g.N) {
+          const f32x4v v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+          mine[idx * NT + t] = v;
+        }
+      }
+}
+
 // ---- 16-bit MFMA kernel ----------------------------------------------------------------------------------------------
 template <typename T, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
@@ -344,24 +366,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma16(GemmArgs g, const T*
 
   // lane owns column (lane % 32); register r of a 32x32 tile is row 8*(r/4) + 4*(lane/32) + r%4
   if (g.splits > 1) {
-    // split-K: park this block's partial tile for splitk_finish.  Layout of one partial tile:
-    // [q-group (i, j, r / 4)][thread][4 floats] -- 16-byte accesses, coalesced over the block.  A q-group holds 4
-    // consecutive rows of one column; groups whose rows all lie beyond M are skipped.
-    constexpr int Q = TM * TN * 4;
-    const LongType tileLinear = (bz * tilesM + tm) * tilesN + tn;
-    f32x4v* const mine = reinterpret_cast<f32x4v*>(g.partial) + (tileLinear * g.splits + blockIdx.y) * (LongType)(Q * NT);
-#pragma unroll
-    for (int i = 0; i < TM; i++)
-#pragma unroll
-      for (int j = 0; j < TN; j++)
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-          const int idx = (i * TN + j) * 4 + q;
-          if (m0 + wm * WTM + i * 32 + 8 * q + 4 * (lane >> 5) < g.M && n0 + wn * WTN + j * 32 + (lane & 31) < g.N) {
-            const f32x4v v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-            mine[idx * NT + t] = v;
-          }
-        }
+    storePartialTile<TM, TN, NT>(g, acc, (bz * tilesM + tm) * tilesN + tn, m0 + wm * WTM, n0 + wn * WTN, t, lane);
     return;
   }
   storeAccTiles<T, TM, TN, true>(g, C, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
@@ -622,7 +627,9 @@ __device__ __attribute__((aligned(256))) unsigned char gemmZeroPage[256];
 // NST-round multiply zeros.
 // A_KC = false: A lies [k][m] with unit m stride (a transposed A) and is handled like a row-major B: whole k-rows in LDS,
 // fragments through the transposing read.
-template <typename T, bool B_KC, int NST, int TW, bool EDGE = false, bool KTAIL = false, bool A_KC = true>
+// SPLIT (with EDGE and KTAIL): blockIdx.y owns g.ktPerSplit K-tiles and parks its tile for splitk_finish; what lies beyond its
+// range of K comes from the page of zeros like what lies beyond K.
+template <typename T, bool B_KC, int NST, int TW, bool EDGE = false, bool KTAIL = false, bool A_KC = true, bool SPLIT = false>
 __global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
                                                     unsigned tilesM, unsigned tilesN) {
   constexpr int BM = 64 * TW, BN = 64 * TW, BK = 64;
@@ -674,7 +681,10 @@ __global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restr
   const char* const baseA = reinterpret_cast<const char*>(A_KC ? A + m0 * lda : A + m0);
   const char* const baseB = reinterpret_cast<const char*>(B_KC ? B + n0 * ldb : B + n0);
   const LongType stepA = (A_KC ? (LongType)BK : (LongType)BK * lda) * 2, stepB = (B_KC ? (LongType)BK : (LongType)BK * ldb) * 2;   // bytes per K-tile
-  const LongType KT = KTAIL ? (g.K + BK - 1) / BK : g.K / BK;
+  static_assert(!SPLIT || (EDGE && KTAIL && TW == 1), "the split-K instantiation handles every edge");
+  const LongType ktBase = SPLIT ? (LongType)blockIdx.y * g.ktPerSplit : 0;   // first K-tile of this block
+  const LongType KT = SPLIT ? g.ktPerSplit : KTAIL ? (g.K + BK - 1) / BK : g.K / BK;
+  const int kEnd = SPLIT ? (int)((ktBase + g.ktPerSplit) * BK < g.K ? (ktBase + g.ktPerSplit) * BK : g.K) : (int)g.K;
   auto dma = [&](const char* base, unsigned off, const u32x4* dst) {
     const unsigned ldsAddr = (unsigned)(size_t)(lds_ptr)dst;
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(ldsAddr) : "memory");
@@ -688,11 +698,12 @@ __global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restr
     if constexpr (KTAIL) {
       // any tile, also past the end: zeros for everything from K on
       const char* const zero = reinterpret_cast<const char*>(gemmZeroPage);
-      const int k0 = (int)(tile * BK);
+      const LongType gt = tile + ktBase;
+      const int k0 = (int)(gt * BK);
 #pragma unroll
-      for (int c = 0; c < CPW; c++) dmaAt(k0 + kA[c] < (int)g.K ? baseA + tile * stepA + offA[c] : zero, st + (wave * CPW + c) * 64);
+      for (int c = 0; c < CPW; c++) dmaAt(k0 + kA[c] < kEnd ? baseA + gt * stepA + offA[c] : zero, st + (wave * CPW + c) * 64);
 #pragma unroll
-      for (int c = 0; c < CPW; c++) dmaAt(k0 + kB[c] < (int)g.K ? baseB + tile * stepB + offB[c] : zero, st + SLOTS_A + (wave * CPW + c) * 64);
+      for (int c = 0; c < CPW; c++) dmaAt(k0 + kB[c] < kEnd ? baseB + gt * stepB + offB[c] : zero, st + SLOTS_A + (wave * CPW + c) * 64);
       return;
     }
     const LongType kt = tile < KT ? tile : KT - 1;
@@ -763,6 +774,10 @@ __global__ __launch_bounds__(256) void gemm_mfma16s(GemmArgs g, const T* __restr
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the surplus loads of the last rounds
+  if constexpr (SPLIT) {
+    storePartialTile<TW, TW, 256>(g, acc, ((LongType)blockIdx.z * tilesM + tm) * tilesN + tn, m0 + wm * 32 * TW, n0 + wn * 32 * TW, t, lane);
+    return;
+  }
   if (EDGE && (m0 + BM > g.M || n0 + BN > g.N)) storeAccTiles<T, TW, TW, true>(g, C, acc, m0 + wm * 32 * TW, n0 + wn * 32 * TW, lane);
   else storeAccTiles<T, TW, TW, false>(g, C, acc, m0 + wm * 32 * TW, n0 + wn * 32 * TW, lane);
 }
@@ -1521,6 +1536,42 @@ static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
   }
   // an epilogue request is served by splitk_finish only (one batch entry, unit column stride of C)
   if (g.hasEpi && (splits == 1 || batch != 1 || g.cCol != 1)) return false;
+  // split-K on the direct-load ring: few 64 x 64 tiles and a long K.  Every block keeps a whole round of K-tiles in flight,
+  // where the register-staged split kernel pays one memory latency per K-tile; fewer, deeper splits (about one block per
+  // CU, four K-tiles at least) leave less for the finishing launch to add up.
+  if constexpr (BM == 64 && BN == 64 && WM == 2 && WN == 2) {
+    static const bool small = getenv("ND4JHIP_GEMM_SMALL_RING") ? atoi(getenv("ND4JHIP_GEMM_SMALL_RING")) != 0 : true;
+    static const bool splitRing = getenv("ND4JHIP_GEMM_SPLIT_RING") ? atoi(getenv("ND4JHIP_GEMM_SPLIT_RING")) != 0 : true;
+    const LongType ldaS = A_KC ? g.aRow : g.aCol, ldbS = B_KC ? g.bCol : g.bRow;
+    if (splits > 1 && small && splitRing && edge && aligned && (B_KC || g.N % 8 == 0) && (A_KC || g.M % 8 == 0) && ldaS % 8 == 0 && ldbS % 8 == 0 &&
+        ldaS < (1 << 23) && ldbS < (1 << 23) && ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 && g.aBatch % 8 == 0 &&
+        g.bBatch % 8 == 0 && g.aBatch2 % 8 == 0 && g.bBatch2 % 8 == 0) {
+      const unsigned tM = (unsigned)((g.M + BM - 1) / BM), tN = (unsigned)((g.N + BN - 1) / BN);
+      const LongType tiles = (LongType)tM * tN * batch, KT = (g.K + 63) / 64;
+      LongType want = 256 / tiles;             // one round of blocks: a block holds half the LDS of its CU or all of it
+      want = want < KT / 4 ? want : KT / 4;
+      want = want < splits ? want : splits;   // the partial-tile scratch bounds chooseSplits' figure
+      if (want >= 2) {
+        const LongType per = (KT + want - 1) / want;
+        g.ktPerSplit = per;
+        g.splits = (int)((KT + per - 1) / per);
+        constexpr int STAGE_BYTES = (BM + BN) * 8 * 16;
+        const bool deep = per > 4 && DynLds<gemm_mfma16s<T, B_KC, 8, 1, true, true, A_KC, true>, 8 * STAGE_BYTES>::granted();
+        if (deep || DynLds<gemm_mfma16s<T, B_KC, 4, 1, true, true, A_KC, true>, 4 * STAGE_BYTES>::granted()) {
+          noteKernel("gemm_mfma16s<%s,64x64,akc=%d,bkc=%d,stages=%d,split>+splitk_finish", tname<T>(), (int)A_KC, (int)B_KC, deep ? 8 : 4);
+          auto kern = deep ? gemm_mfma16s<T, B_KC, 8, 1, true, true, A_KC, true> : gemm_mfma16s<T, B_KC, 4, 1, true, true, A_KC, true>;
+          hipLaunchKernelGGL(kern, dim3(tM * tN, (unsigned)g.splits, (unsigned)batch), dim3(256), (deep ? 8 : 4) * STAGE_BYTES, s, g, (const T*)A, (const T*)B,
+                             (T*)C, tM, tN);
+          hipLaunchKernelGGL((splitk_finish<T, BM, BN, WM, WN>), dim3(tM * tN, (BM / WM / 32) * (BN / WN / 32) * 4, (unsigned)batch), dim3(NT), 0, s, g, (T*)C, tM, tN);
+          return true;
+        }
+        g.splits = splits;   // back to the register-staged split
+        LongType per0 = 0;
+        chooseSplits<BM, BN>(g, batch, per0);
+        g.ktPerSplit = per0;
+      }
+    }
+  }
   const bool usePipe = splits == 1;   // the split-K epilogue lives in the plain kernel
   // whole tiles only: the kernel without bounds handling (its K loop needs two K-tiles at least)
   const bool useFull = aligned && usePipe && BM * BN >= 128 * 128 && g.M % BM == 0 && g.N % BN == 0 && g.K % 64 == 0 && g.K >= 128;
@@ -1603,6 +1654,10 @@ template <typename T, bool A_KC, bool B_KC>
 static bool launchMfma16(hipStream_t s, const GemmArgs& g, const void* A, const void* B, void* C, LongType batch, bool aligned) {
   const LongType tiles256 = ((g.M + 255) / 256) * ((g.N + 255) / 256) * batch;
   const LongType tiles128 = ((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
+  // up to 32 rows against a long K (a batched decode step's second MLP product, K = 3072): the 64 x 64 configuration, whose
+  // split-K runs on the direct-load ring (7.6 against 8.7 us with the 32 x 128 tiles of the register-staged split)
+  static const bool skinnyRing = getenv("ND4JHIP_GEMM_SKINNY_RING") ? atoi(getenv("ND4JHIP_GEMM_SKINNY_RING")) != 0 : true;
+  if (g.M <= 32 && skinnyRing && aligned && g.K >= 2048 && launchMfma16Cfg<T, 64, 64, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch, true, aligned)) return true;
   if (g.M <= 32) return launchMfma16Cfg<T, 32, 128, 1, 4, A_KC, B_KC>(s, g, A, B, C, batch, true, aligned);
   if (g.M <= 64 || g.N <= 64 || tiles128 < 192) return launchMfma16Cfg<T, 64, 64, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch, true, aligned);
   if (tiles256 < 192) return launchMfma16Cfg<T, 128, 128, 2, 2, A_KC, B_KC>(s, g, A, B, C, batch, false, aligned);

@@ -102,7 +102,8 @@ CASES = [
     # few 64 x 64 tiles: up to K = 2048 one block per tile on the ring kernel, beyond that split-K with its finishing launch
     (BFLOAT16, 512, 512, 512, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=8>", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=8>", None),
     (HALF, 512, 768, 2048, "gemm_mfma16s<f16,64x64,akc=1,bkc=0,stages=8>", "gemm_mfma16s<f16,64x64,akc=1,bkc=1,stages=8>", None),
-    (BFLOAT16, 256, 256, 4096, "gemm_mfma16<bf16,64x64,akc=1,bkc=0>+splitk_finish", "gemm_mfma16<bf16,64x64,akc=1,bkc=1>+splitk_finish", None),
+    (BFLOAT16, 256, 256, 4096, "gemm_mfma16s<bf16,64x64,akc=1,bkc=0,stages=4,split>+splitk_finish", "gemm_mfma16s<bf16,64x64,akc=1,bkc=1,stages=4,split>+splitk_finish", "gemm_mfma16s<bf16,64x64,akc=0,bkc=0,stages=4,split>+splitk_finish"),
+    (HALF, 250, 250, 4104, "gemm_mfma16<f16,64x64,akc=1,bkc=0>+splitk_finish", "gemm_mfma16s<f16,64x64,akc=1,bkc=1,stages=", None),
     # row lengths that are not multiples of 8 (rows start off 16-byte boundaries, the last vector of a row is partial): the
     # bounds-handling kernels read element-aligned vectors -- a batched decode step's logits against the row-major
     # [768, 50257] embedding, a prefill's, and a product with nothing aligned in any layout
@@ -167,6 +168,15 @@ def test_k_tail_on_the_direct_load_kernels_whole_result(ex, dtype, M, N, K, tb):
     """A K that is not a whole number of K-tiles on the ring kernel: the lanes beyond K read a page of zeros.  Every element of
     the result, with operands whose neighbours in memory (the next row, which a load past K would bring in) are large."""
     _whole_result(ex, dtype, M, N, K, tb, expect=",ktail")
+
+
+@pytest.mark.parametrize("tb", [False, True], ids=["plain", "transposeB"])
+@pytest.mark.parametrize("dtype,M,N,K", [(BFLOAT16, 512, 768, 3072), (HALF, 504, 496, 4008), (BFLOAT16, 72, 768, 3072), (HALF, 256, 320, 2200)],
+                         ids=["bf16-mlp-down", "f16-ragged", "bf16-72-rows", "f16-k2200"])
+def test_split_k_on_the_direct_load_ring_whole_result(ex, dtype, M, N, K, tb):
+    """Few 64 x 64 tiles and a long K: split-K on the ring kernel (every block a range of K-tiles, zeros beyond its range and
+    beyond K), partial tiles added up by the finishing launch.  Every element of the result."""
+    _whole_result(ex, dtype, M, N, K, tb, expect=",split>+splitk_finish")
 
 
 def _whole_result(ex, dtype, M, N, K, tb, expect=",edge"):
