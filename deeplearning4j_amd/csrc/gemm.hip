@@ -1549,7 +1549,8 @@ static bool launchMfma16Cfg(hipStream_t s, GemmArgs g, const void* A, const void
       const unsigned tM = (unsigned)((g.M + BM - 1) / BM), tN = (unsigned)((g.N + BN - 1) / BN);
       const LongType tiles = (LongType)tM * tN * batch, KT = (g.K + 63) / 64;
       LongType want = 256 / tiles;             // one round of blocks: a block holds half the LDS of its CU or all of it
-      want = want < KT / 4 ? want : KT / 4;
+      constexpr LongType minPer = 4;   // K-tiles per split at least (the batch-32 decode step: 3 -> 0.556, 4 -> 0.552, 6 -> 0.558, 8 -> 0.555 ms)
+      want = want < KT / minPer ? want : KT / minPer;
       want = want < splits ? want : splits;   // the partial-tile scratch bounds chooseSplits' figure
       if (want >= 2) {
         const LongType per = (KT + want - 1) / want;
