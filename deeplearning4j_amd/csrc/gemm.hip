@@ -2716,6 +2716,154 @@ __global__ __launch_bounds__(256) void gemm_skinny32(GemmArgs g, const T* __rest
     epilogueExtras4<T>(g, mrow, n, v);
   }
 }
+// The layer-normalising few-row product with the rows cut in two: a block owns 32 output columns and 16 rows (grid: N / 32 x
+// ceil(M / 16)).  Every block of gemm_skinny32 normalises all 32 rows before it can multiply -- 96 values per thread, vector
+// ALU work at one wave per SIMD, 3.4 us of the kernel's 8.4 and the same in every block.  With 16 rows a thread holds 48
+// values, and twice as many CUs share the step's work; the weights are read by two blocks instead of one (from the cache).
+// 16 threads hold a row: thread lk16 of them holds vector 16 * t2 + lk16, t2 = 0..5, and stands in for lane
+// 16 * (t2 % 4) + lk16 of the separate layer_norm kernel's wave in its pass t2 / 4 -- the first four levels of that wave's
+// balanced tree run across the 16 threads, the last two inside a thread, so the statistics carry the same bits.
+// Rows 16..31 of the matrix instruction's X operand are whatever LDS holds: a row of the product depends on its own row of
+// X only, and those rows are not stored.
+template <typename T, int LN_NV>
+__global__ __launch_bounds__(256) void gemm_skinny16ln(GemmArgs g, const T* __restrict__ X, const T* __restrict__ Wt, T* __restrict__ C) {
+  constexpr int CT = 6, GROUP = 33, XV = 6;
+  using IO = RawIO<T>;
+  using Raw = typename IO::raw;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  u32x4* sW = reinterpret_cast<u32x4*>(smem_raw);      // [CT * 8 k-groups][GROUP]
+  u32x4* sX = sW + CT * 8 * GROUP;
+  u32x4* sGB = sW + 2 * CT * 8 * GROUP;                // [2][128] vectors: gain, then bias
+  float* red = reinterpret_cast<float*>(smem_raw);     // [4 waves][16 registers][64 lanes]; reuses sW once the K loop is over
+  const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int lrow = t >> 3, lkg = t & 7;                // W: this thread's (column, k-group) inside every 64-k tile
+  const int xr16 = t >> 4, lk16 = t & 15;              // X: this thread's row of the block's 16 and its vector index mod 16
+  const LongType n0 = (LongType)blockIdx.x * 32, m0 = (LongType)blockIdx.y * 16;
+  const T* wp = Wt + (n0 + lrow) * g.bCol + lkg * 8;
+  const T* xp = X + (m0 + xr16 < g.M ? m0 + xr16 : g.M - 1) * g.aRow;
+  const int tiles = (int)(g.K / 64), nv = tiles * 8;
+  u32x4 wr[2][CT], xv[XV];
+#pragma unroll
+  for (int t2 = 0; t2 < XV; t2++) {
+    const int v = 16 * t2 + lk16;
+    xv[t2] = *reinterpret_cast<const u32x4*>(xp + (LongType)(v < nv ? v : nv - 1) * 8);
+  }
+  {
+    const int v = t & 127, vc = v < nv ? v : nv - 1;
+    const T* src = reinterpret_cast<const T*>(t < 128 ? g.lnGain : g.lnBias) + vc * 8;
+    sGB[t] = *reinterpret_cast<const u32x4*>(src);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int j = 0; j < 2 * CT; j++) {
+    const int jc = j < tiles ? j : tiles - 1;
+    wr[j / CT][j % CT] = *reinterpret_cast<const u32x4*>(wp + (LongType)jc * 64);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  const int lastV = nv - 1, lastT2 = lastV >> 4, lastLk = lastV & 15;
+  auto rowTotal = [&](const float (&part)[XV]) {
+    float last = 0.f;
+#pragma unroll
+    for (int t2 = 0; t2 < XV; t2++) if (t2 == lastT2) last = part[t2];
+    last = __shfl(last, (lane & ~15) | lastLk, 64);
+    float o[4];
+#pragma unroll
+    for (int jj = 0; jj < 4; jj++) {
+      float s = 0.f;
+#pragma unroll
+      for (int i = 0; i < LN_NV; i++) {
+        const int t2 = jj + 4 * i;
+        const bool in = 16 * t2 + lk16 < nv;
+        const float p = t2 < XV && in ? part[t2 < XV ? t2 : 0] : last;
+        s += p * (in ? 1.f : 0.f);
+      }
+      o[jj] = group_allreduce<SumOp, 16>(s);
+    }
+    return (o[0] + o[1]) + (o[2] + o[3]);
+  };
+  float part[XV], vals[XV][8];
+#pragma unroll
+  for (int t2 = 0; t2 < XV; t2++) {
+    IO::unpack(__builtin_bit_cast(Raw, xv[t2]), vals[t2]);
+    float p = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; e++) p += vals[t2][e];
+    part[t2] = p;
+  }
+  const float mean = rowTotal(part) / (float)(int)g.K;
+#pragma unroll
+  for (int t2 = 0; t2 < XV; t2++) {
+    float p = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; e++) { const float d = vals[t2][e] - mean; vals[t2][e] = d; p += d * d; }
+    part[t2] = p;
+  }
+  const float var = rowTotal(part) / (float)(int)g.K;
+  const float rstd = 1.f / sqrtf(var + g.lnEps);
+  const bool writer = blockIdx.x == 0 && m0 + xr16 < g.M;
+  T* lo = reinterpret_cast<T*>(g.lnOut) + (m0 + xr16) * g.lnOutRow;
+  __syncthreads();                                       // gain and bias are in LDS
+#pragma unroll
+  for (int t2 = 0; t2 < XV; t2++) {
+    float gn[8], bs[8];
+    const int v = 16 * t2 + lk16, vj = v < nv ? v : 0;
+    IO::unpack(__builtin_bit_cast(Raw, sGB[vj]), gn);
+    IO::unpack(__builtin_bit_cast(Raw, sGB[128 + vj]), bs);
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      float y = vals[t2][e] * rstd * gn[e];
+      y += bs[e];
+      vals[t2][e] = y;
+    }
+    const Raw packed = IO::pack(vals[t2]);
+    xv[t2] = __builtin_bit_cast(u32x4, packed);
+    if (writer && v < nv) *reinterpret_cast<Raw*>(lo + (LongType)v * 8) = packed;
+  }
+  f32x16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[r] = 0.f;
+  const int mrow = lane & 31, h = lane >> 5;
+  // chunk `set`: K-tiles set * CT .. + CT - 1 -- the W registers of that set and this thread's X vectors 3 * set .. + 2
+  // (vector 16 * t2 + lk16 is k-group lk16 % 8 of K-tile 2 * t2 + lk16 / 8)
+  auto chunk = [&](auto setc) {
+    constexpr int set = decltype(setc)::value;
+    const int n = tiles - set * CT < CT ? tiles - set * CT : CT;
+#pragma unroll
+    for (int j = 0; j < CT; j++) sW[(j * 8 + lkg) * GROUP + lrow] = wr[set][j];
+#pragma unroll
+    for (int q = 0; q < 3; q++) {
+      const int t2 = 3 * set + q, tile = 2 * q + (lk16 >> 3);
+      sX[(tile * 8 + (lk16 & 7)) * GROUP + xr16] = xv[t2];
+    }
+    __syncthreads();
+    for (int s = wave; s < n * 4; s += 4)
+      acc = Mfma16<T>::mma(sW[(2 * s + h) * GROUP + mrow], sX[(2 * s + h) * GROUP + mrow], acc);
+    __syncthreads();
+  };
+  chunk(std::integral_constant<int, 0>{});
+  if (CT < tiles) chunk(std::integral_constant<int, 1>{});
+#pragma unroll
+  for (int r = 0; r < 16; r++) red[(wave * 16 + r) * 64 + lane] = acc[r];
+  __syncthreads();
+  const int rq = wave;                                 // registers 4 * rq .. + 3: four consecutive columns
+  const LongType n = n0 + 8 * rq + 4 * h;
+  float v[4];
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; w++) sum += red[(w * 16 + 4 * rq + e) * 64 + lane];
+    if (g.bias) sum += to_float(reinterpret_cast<const T*>(g.bias)[n + e]);
+    v[e] = sum;
+  }
+  if (mrow < 16 && m0 + mrow < g.M) {
+    u32x2 o;
+    o[0] = (unsigned)Conv<T>::from(v[0]).bits | ((unsigned)Conv<T>::from(v[1]).bits << 16);
+    o[1] = (unsigned)Conv<T>::from(v[2]).bits | ((unsigned)Conv<T>::from(v[3]).bits << 16);
+    *reinterpret_cast<u32x2*>(C + (m0 + mrow) * g.cRow + n) = o;
+    epilogueExtras4<T>(g, m0 + mrow, n, v);
+  }
+}
 template <typename T>
 static bool tryGemmSkinny(hipStream_t s, const GemmDesc& d, const void* A, const void* B, void* C) {
   if (d.M < 5 || d.M > 32 || d.batch != 1 || d.alpha != 1.f || d.beta != 0.f) return false;
@@ -2734,6 +2882,13 @@ static bool tryGemmSkinny(hipStream_t s, const GemmDesc& d, const void* A, const
     noteKernel("gemm_skinny32<%s,ln>", tname<T>());
     constexpr size_t LDS_LN = LDS + 2 * 128 * 16;          // + gain and bias
     static_assert(LDS_LN <= 64 * 1024, "gemm_skinny32 must fit the default dynamic LDS limit");
+    static const bool rows16 = getenv("ND4JHIP_GEMM_SKINNY_ROWS16") ? atoi(getenv("ND4JHIP_GEMM_SKINNY_ROWS16")) != 0 : true;
+    if (rows16) {
+      const dim3 grid((unsigned)(d.N / 32), (unsigned)((d.M + 15) / 16));
+      if (d.K <= 512) hipLaunchKernelGGL((gemm_skinny16ln<T, 1>), grid, dim3(256), LDS_LN, s, g, (const T*)A, (const T*)B, (T*)C);
+      else hipLaunchKernelGGL((gemm_skinny16ln<T, 2>), grid, dim3(256), LDS_LN, s, g, (const T*)A, (const T*)B, (T*)C);
+      return true;
+    }
     if (d.K <= 512) hipLaunchKernelGGL((gemm_skinny32<T, 1>), dim3((unsigned)(d.N / 32)), dim3(256), LDS_LN, s, g, (const T*)A, (const T*)B, (T*)C);
     else hipLaunchKernelGGL((gemm_skinny32<T, 2>), dim3((unsigned)(d.N / 32)), dim3(256), LDS_LN, s, g, (const T*)A, (const T*)B, (T*)C);
     return true;
