@@ -2725,9 +2725,11 @@ __global__ __launch_bounds__(256) void gemm_skinny32(GemmArgs g, const T* __rest
 // balanced tree run across the 16 threads, the last two inside a thread, so the statistics carry the same bits.
 // Rows 16..31 of the matrix instruction's X operand are whatever LDS holds: a row of the product depends on its own row of
 // X only, and those rows are not stored.
-template <typename T, int LN_NV>
+template <typename T, int LN_NV, int ROWS = 16>
 __global__ __launch_bounds__(256) void gemm_skinny16ln(GemmArgs g, const T* __restrict__ X, const T* __restrict__ Wt, T* __restrict__ C) {
-  constexpr int CT = 6, GROUP = 33, XV = 6;
+  static_assert(ROWS == 16 || ROWS == 8, "rows per block");
+  constexpr int CT = 6, GROUP = 33;
+  constexpr int TPR = 256 / ROWS, XV = 96 / TPR, JJ = 64 / TPR;   // threads per row, vectors per thread, stand-in lanes per thread
   using IO = RawIO<T>;
   using Raw = typename IO::raw;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -2737,15 +2739,15 @@ __global__ __launch_bounds__(256) void gemm_skinny16ln(GemmArgs g, const T* __re
   float* red = reinterpret_cast<float*>(smem_raw);     // [4 waves][16 registers][64 lanes]; reuses sW once the K loop is over
   const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int lrow = t >> 3, lkg = t & 7;                // W: this thread's (column, k-group) inside every 64-k tile
-  const int xr16 = t >> 4, lk16 = t & 15;              // X: this thread's row of the block's 16 and its vector index mod 16
-  const LongType n0 = (LongType)blockIdx.x * 32, m0 = (LongType)blockIdx.y * 16;
+  const int xr16 = t / TPR, lk16 = t % TPR;            // X: this thread's row of the block's ROWS and its vector index mod TPR
+  const LongType n0 = (LongType)blockIdx.x * 32, m0 = (LongType)blockIdx.y * ROWS;
   const T* wp = Wt + (n0 + lrow) * g.bCol + lkg * 8;
   const T* xp = X + (m0 + xr16 < g.M ? m0 + xr16 : g.M - 1) * g.aRow;
   const int tiles = (int)(g.K / 64), nv = tiles * 8;
   u32x4 wr[2][CT], xv[XV];
 #pragma unroll
   for (int t2 = 0; t2 < XV; t2++) {
-    const int v = 16 * t2 + lk16;
+    const int v = TPR * t2 + lk16;
     xv[t2] = *reinterpret_cast<const u32x4*>(xp + (LongType)(v < nv ? v : nv - 1) * 8);
   }
   {
@@ -2760,26 +2762,27 @@ __global__ __launch_bounds__(256) void gemm_skinny16ln(GemmArgs g, const T* __re
     wr[j / CT][j % CT] = *reinterpret_cast<const u32x4*>(wp + (LongType)jc * 64);
   }
   __builtin_amdgcn_sched_barrier(0);
-  const int lastV = nv - 1, lastT2 = lastV >> 4, lastLk = lastV & 15;
+  const int lastV = nv - 1, lastT2 = lastV / TPR, lastLk = lastV % TPR;
   auto rowTotal = [&](const float (&part)[XV]) {
     float last = 0.f;
 #pragma unroll
     for (int t2 = 0; t2 < XV; t2++) if (t2 == lastT2) last = part[t2];
-    last = __shfl(last, (lane & ~15) | lastLk, 64);
-    float o[4];
+    last = __shfl(last, (lane & ~(TPR - 1)) | lastLk, 64);
+    float o[JJ];
 #pragma unroll
-    for (int jj = 0; jj < 4; jj++) {
+    for (int jj = 0; jj < JJ; jj++) {
       float s = 0.f;
 #pragma unroll
       for (int i = 0; i < LN_NV; i++) {
-        const int t2 = jj + 4 * i;
-        const bool in = 16 * t2 + lk16 < nv;
+        const int t2 = jj + JJ * i;
+        const bool in = TPR * t2 + lk16 < nv;
         const float p = t2 < XV && in ? part[t2 < XV ? t2 : 0] : last;
         s += p * (in ? 1.f : 0.f);
       }
-      o[jj] = group_allreduce<SumOp, 16>(s);
+      o[jj] = group_allreduce<SumOp, TPR>(s);
     }
-    return (o[0] + o[1]) + (o[2] + o[3]);
+    if constexpr (JJ == 4) return (o[0] + o[1]) + (o[2] + o[3]);
+    else return o[0] + o[1];
   };
   float part[XV], vals[XV][8];
 #pragma unroll
@@ -2806,7 +2809,7 @@ __global__ __launch_bounds__(256) void gemm_skinny16ln(GemmArgs g, const T* __re
 #pragma unroll
   for (int t2 = 0; t2 < XV; t2++) {
     float gn[8], bs[8];
-    const int v = 16 * t2 + lk16, vj = v < nv ? v : 0;
+    const int v = TPR * t2 + lk16, vj = v < nv ? v : 0;
     IO::unpack(__builtin_bit_cast(Raw, sGB[vj]), gn);
     IO::unpack(__builtin_bit_cast(Raw, sGB[128 + vj]), bs);
 #pragma unroll
@@ -2831,9 +2834,9 @@ __global__ __launch_bounds__(256) void gemm_skinny16ln(GemmArgs g, const T* __re
 #pragma unroll
     for (int j = 0; j < CT; j++) sW[(j * 8 + lkg) * GROUP + lrow] = wr[set][j];
 #pragma unroll
-    for (int q = 0; q < 3; q++) {
-      const int t2 = 3 * set + q, tile = 2 * q + (lk16 >> 3);
-      sX[(tile * 8 + (lk16 & 7)) * GROUP + xr16] = xv[t2];
+    for (int t2 = 0; t2 < XV; t2++) {
+      const int tile = (TPR * t2 + lk16) >> 3;   // the K-tile of this vector; k-group lk16 % 8
+      if (tile / CT == set) sX[((tile - set * CT) * 8 + (lk16 & 7)) * GROUP + xr16] = xv[t2];
     }
     __syncthreads();
     for (int s = wave; s < n * 4; s += 4)
@@ -2856,7 +2859,7 @@ __global__ __launch_bounds__(256) void gemm_skinny16ln(GemmArgs g, const T* __re
     if (g.bias) sum += to_float(reinterpret_cast<const T*>(g.bias)[n + e]);
     v[e] = sum;
   }
-  if (mrow < 16 && m0 + mrow < g.M) {
+  if (mrow < ROWS && m0 + mrow < g.M) {
     u32x2 o;
     o[0] = (unsigned)Conv<T>::from(v[0]).bits | ((unsigned)Conv<T>::from(v[1]).bits << 16);
     o[1] = (unsigned)Conv<T>::from(v[2]).bits | ((unsigned)Conv<T>::from(v[3]).bits << 16);
@@ -2883,6 +2886,7 @@ static bool tryGemmSkinny(hipStream_t s, const GemmDesc& d, const void* A, const
     constexpr size_t LDS_LN = LDS + 2 * 128 * 16;          // + gain and bias
     static_assert(LDS_LN <= 64 * 1024, "gemm_skinny32 must fit the default dynamic LDS limit");
     static const bool rows16 = getenv("ND4JHIP_GEMM_SKINNY_ROWS16") ? atoi(getenv("ND4JHIP_GEMM_SKINNY_ROWS16")) != 0 : true;
+    // (8 rows per block, 32 threads to a row, measured slower: the batch-32 decode step 0.5215 against 0.5155 ms)
     if (rows16) {
       const dim3 grid((unsigned)(d.N / 32), (unsigned)((d.M + 15) / 16));
       if (d.K <= 512) hipLaunchKernelGGL((gemm_skinny16ln<T, 1>), grid, dim3(256), LDS_LN, s, g, (const T*)A, (const T*)B, (T*)C);
