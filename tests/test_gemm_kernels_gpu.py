@@ -252,6 +252,35 @@ def test_alpha_beta_on_the_ring_kernel(ex):
     assert np.array_equal(C2.to_float(), got), "transposed B gives the same bits (same products, same order)"
 
 
+@pytest.mark.parametrize("dtype", [BFLOAT16, FLOAT32], ids=["bf16", "f32"])
+def test_alpha_beta_batched_ragged_on_the_edge_kernels(ex, dtype):
+    """C = alpha A B + beta C, batched, with M, N and K all off the tile sizes: the edge instantiations read C back in their
+    bounds-checked epilogue, and every batch entry clamps against its own operand.  Then the same product with A and B as
+    pitched views (rows longer than the extent that is multiplied)."""
+    rng = np.random.default_rng(29)
+    batch, M, N, K = 5, 1000, 1096, 1000
+    tol = TOL[dtype]
+    a = rng.normal(0, 1 / math.sqrt(K), (batch, M, K)).astype(np.float32)
+    b = rng.normal(0, 1 / math.sqrt(K), (batch, K, N)).astype(np.float32)
+    c0 = rng.normal(0, 1, (batch, M, N)).astype(np.float32)
+    A, a64 = _device(a, dtype)
+    B, b64 = _device(b, dtype)
+    C, c64 = _device(c0, dtype)
+    ex.exec_custom("matmul", [A, B], [C], t_args=[0.5, 2.0])
+    assert ",edge,ktail" in _last_kernel(ex), _last_kernel(ex)
+    got = C.to_float()
+    for bi in range(batch):
+        assert_close(got[bi], 0.5 * (a64[bi] @ b64[bi]) + 2.0 * c64[bi], tol, 2 * tol, "batch %d" % bi)
+    # pitched views: A inside a [M, K + 24] array, B inside a [K, N + 40] array, one batch entry
+    wideA = rng.normal(0, 1 / math.sqrt(K), (M, K + 24)).astype(np.float32)
+    wideB = rng.normal(0, 1 / math.sqrt(K), (K, N + 40)).astype(np.float32)
+    WA, wa64 = _device(wideA, dtype)
+    WB, wb64 = _device(wideB, dtype)
+    z = ex.exec_custom("matmul", [WA.slice(1, 8, 8 + K), WB.slice(1, 16, 16 + N)])[0].to_float()
+    assert ",edge,ktail" in _last_kernel(ex), _last_kernel(ex)
+    assert_close(z, wa64[:, 8:8 + K] @ wb64[:, 16:16 + N], tol, tol, "pitched views")
+
+
 def test_bias_row_on_the_large_kernels(ex):
     """xw_plus_b at a shape that lands on the 256 x 256 kernels: the bias row is added in their epilogue."""
     rng = np.random.default_rng(23)
