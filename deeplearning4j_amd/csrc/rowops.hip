@@ -310,7 +310,7 @@ __global__ __launch_bounds__(1024) void softmax_long_vec(RowArgs a, const T* __r
   const A NEG = -r_tmax<A>();
   A mx = NEG;
   sweep([&](A v, LongType) { mx = LOG ? (v > mx ? v : mx) : softmax_maxstep<A>(mx, v, clamp); });
-  mx = block_allreduce<MaxOp, NT / 64, A>(mx, lds);
+  if constexpr (NT == 64) mx = wave_allreduce<MaxOp>(mx); else mx = block_allreduce<MaxOp, NT / 64, A>(mx, lds);
   if (!LOG && clamp && mx == NEG) mx = (A)0;
   A sum = (A)0;
   // LOG: log(exp(x - max) / sum) in that order, as log_softmax_rows evaluates it
@@ -345,17 +345,21 @@ __global__ __launch_bounds__(1024) void softmax_long_vec(RowArgs a, const T* __r
 // block of 512 threads (two waves per SIMD: 256 registers each) holds the whole row in registers, so it comes from memory once and the three passes (maximum, sum of
 // exponentials, result) run on registers.  Rows may start anywhere: the 16-byte loads and stores are element-aligned (global
 // memory runs in unaligned access mode), the values after the last whole vector go one per thread.
-template <typename T, int NV, bool LOG, bool NTS = false>
-__global__ __launch_bounds__(512) void softmax_block_regs(RowArgs a, const T* __restrict__ x, T* __restrict__ z, int clamp) {
+// NT = 64: a wave per row, four rows to a block of 256 threads -- rows of up to NV x 64 vectors whose starts or length keep
+// them off the aligned vector kernels (attention scores of a 1001-token prompt: bf16 [192, 1001, 1001] 2.4 -> see the launcher).
+template <typename T, int NV, bool LOG, bool NTS = false, int NT = 512>
+__global__ __launch_bounds__(NT == 64 ? 256 : NT) void softmax_block_regs(RowArgs a, const T* __restrict__ x, T* __restrict__ z, int clamp) {
   using A = typename Conv<T>::acc;
   using Raw = typename RawIO<T>::raw;
-  constexpr int VEC = RawIO<T>::N, NT = 512;
-  __shared__ A lds[NT / 64];
-  const LongType row = blockIdx.x;
+  constexpr int VEC = RawIO<T>::N;
+  static_assert(NT == 512 || NT == 64, "a block of 512 threads or a wave per row");
+  __shared__ A lds[NT == 64 ? 1 : NT / 64];
+  const LongType row = NT == 64 ? (LongType)blockIdx.x * 4 + threadIdx.x / 64 : (LongType)blockIdx.x;
+  if (NT == 64 && row >= a.rows) return;
   const T* xr = x + walk<LongType>(a.outerX, row);
   T* zr = z + walk<LongType>(a.outerZ, row);
   const LongType L = a.rowLen, nv = L / VEC, tail0 = nv * VEC;
-  const int t = threadIdx.x;
+  const int t = NT == 64 ? (int)(threadIdx.x & 63) : (int)threadIdx.x;
   Raw v[NV];
 #pragma unroll
   for (int i = 0; i < NV; i++) {
@@ -406,7 +410,7 @@ __global__ __launch_bounds__(512) void softmax_block_regs(RowArgs a, const T* __
   } else {
     sweep([&](A val) { sum += term(val); });
   }
-  sum = block_allreduce<SumOp, NT / 64, A>(sum, lds);
+  if constexpr (NT == 64) sum = wave_allreduce<SumOp>(sum); else sum = block_allreduce<SumOp, NT / 64, A>(sum, lds);
   if (!LOG && clamp) sum = sum > (A)1e-6f ? sum : (A)1e-6f;
   // long 16-bit rows: the maximum passes through an opaque copy, so that the exponentials of the sum pass are taken again here
   // instead of being kept in (spilled) registers
@@ -546,6 +550,19 @@ static void softmaxTyped(hipStream_t s, const void* x, void* z, const RowPlan& p
     if (L <= 8 * perBlock) { SM(256, 8, gb); return; }
 #undef SM
   } else {
+    // unit-stride rows that start anywhere or have any length: a wave per row, the row in registers through element-aligned
+    // 16-byte loads, the last L % V values one per lane (warm bf16 [192, 1001, 1001]: 2.4 TB/s with one element per load)
+    if constexpr (sizeof(T) == 2) {   // (fp32 rows are as fast with one 4-byte element per load: [192, 1023, 1023] 0.293 against 0.307 ms)
+      if (p.xInner == 1 && p.zInner == 1 && L >= 2 * V && L / V <= 64 * 16) {
+        const LongType per = (L / V + 63) / 64;
+        const bool nts = (size_t)p.rows * (size_t)L * sizeof(T) >= ((size_t)8 << 20);
+#define SWR(NV) do { if (nts) hipLaunchKernelGGL((softmax_block_regs<T, NV, false, true, 64>), dim3(gw), dim3(256), 0, s, a, xt, zt, clamp); \
+                     else hipLaunchKernelGGL((softmax_block_regs<T, NV, false, false, 64>), dim3(gw), dim3(256), 0, s, a, xt, zt, clamp); } while (0)
+        if (per <= 2) SWR(2); else if (per <= 4) SWR(4); else if (per <= 8) SWR(8); else SWR(16);
+#undef SWR
+        return;
+      }
+    }
     if (L <= 64 * 16) { hipLaunchKernelGGL((softmax_rows<T, 64, 16, 1>), dim3(gw), dim3(256), 0, s, a, xt, zt, clamp, 0); return; }
     if (L <= 256 * 32) { hipLaunchKernelGGL((softmax_rows<T, 256, 32, 1>), dim3(gb), dim3(256), 0, s, a, xt, zt, clamp, 0); return; }
   }
