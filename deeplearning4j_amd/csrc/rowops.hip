@@ -1071,6 +1071,84 @@ __global__ __launch_bounds__(1024) void layernorm_long(const T* __restrict__ x, 
   }
 }
 
+// One wave per row for unit-stride rows at a constant pitch that the aligned vector kernels cannot take -- a row length that is
+// not a whole number of 16-byte vectors (770), rows, gain or bias that start off 16-byte boundaries: element-aligned 16-byte
+// loads (global memory runs in unaligned access mode), the last L % VEC values one per lane, the row in registers.  Same
+// arithmetic as ln_wave_row.  (These rows used to go one element per load: warm bf16 [16000, 770] 2.0 TB/s.)
+template <typename T, int NV, bool HAS_BIAS, bool NTS>
+__global__ __launch_bounds__(256) void layernorm_wave_regs(const T* __restrict__ x, const T* __restrict__ gain, const T* __restrict__ bias,
+                                                           T* __restrict__ z, LongType rows, int L, LongType xPitch, LongType zPitch, float eps) {
+  using A = typename Conv<T>::acc;
+  using Raw = typename RawIO<T>::raw;
+  constexpr int VEC = RawIO<T>::N;
+  const int lane = threadIdx.x & 63;
+  const LongType row = (LongType)blockIdx.x * 4 + threadIdx.x / 64;
+  if (row >= rows) return;
+  const T* xr = x + row * xPitch;
+  T* zr = z + row * zPitch;
+  const int nv = L / VEC, tail0 = nv * VEC;
+  Raw xv[NV], gv[NV], bv[NV];
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const int iv = i * 64 + lane, c = (iv < nv ? iv : nv - 1) * VEC;
+    __builtin_memcpy(&xv[i], xr + c, sizeof(Raw));
+    __builtin_memcpy(&gv[i], gain + c, sizeof(Raw));
+    if (HAS_BIAS) __builtin_memcpy(&bv[i], bias + c, sizeof(Raw));
+  }
+  const bool hasTail = tail0 + lane < L;
+  const int te = hasTail ? tail0 + lane : 0;
+  A tx = hasTail ? (A)to_float(xr[te]) : (A)0;
+  const A tg = (A)to_float(gain[te]), tb = HAS_BIAS ? (A)to_float(bias[te]) : (A)0;
+  A vals[NV][VEC];
+  A sum = (A)0;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    RawIO<T>::unpack(xv[i], vals[i]);
+    A part = (A)0;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) part += vals[i][e];
+    sum += i * 64 + lane < nv ? part : (A)0;
+  }
+  sum += tx;
+  sum = wave_allreduce<SumOp>(sum);
+  const A mean = sum / (A)L;
+  A sq = (A)0;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    A part = (A)0;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) { const A d = vals[i][e] - mean; vals[i][e] = d; part += d * d; }
+    sq += i * 64 + lane < nv ? part : (A)0;
+  }
+  tx -= mean;
+  sq += hasTail ? tx * tx : (A)0;
+  sq = wave_allreduce<SumOp>(sq);
+  const A var = L > 1 ? sq / (A)L : (A)0;
+  const A rstd = (A)1 / (A)sqrtf((float)(var + (A)eps));
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const int iv = i * 64 + lane;
+    if (iv < nv) {
+      A g[VEC], b[VEC];
+      RawIO<T>::unpack(gv[i], g);
+      if (HAS_BIAS) RawIO<T>::unpack(bv[i], b);
+#pragma unroll
+      for (int e = 0; e < VEC; e++) {
+        A y = vals[i][e] * rstd * g[e];
+        if (HAS_BIAS) y += b[e];
+        vals[i][e] = y;
+      }
+      const Raw o = RawIO<T>::pack(vals[i]);
+      if constexpr (NTS) nt_store16_elem_aligned(zr + iv * VEC, o);
+      else __builtin_memcpy(zr + iv * VEC, &o, sizeof(Raw));
+    }
+  }
+  if (hasTail) {
+    A y = tx * rstd * tg;
+    if (HAS_BIAS) y += tb;
+    zr[te] = Conv<T>::from(y);
+  }
+}
 template <typename T>
 static bool layerNormTyped(hipStream_t s, const void* x, const void* gain, const void* bias, void* z, const RowPlan& p, float eps) {
   constexpr int V = 16 / sizeof(T);
@@ -1157,6 +1235,19 @@ static bool layerNormTyped(hipStream_t s, const void* x, const void* gain, const
       const LongType xp = p.outerX.rank ? p.outerX.stride[0] : 0, zp = p.outerZ.rank ? p.outerZ.stride[0] : 0;
       if (bt) hipLaunchKernelGGL((layernorm_long<T, true>), dim3((unsigned)p.rows), dim3(1024), 0, s, xt, gt, bt, zt, L, xp, zp, eps);
       else hipLaunchKernelGGL((layernorm_long<T, false>), dim3((unsigned)p.rows), dim3(1024), 0, s, xt, gt, bt, zt, L, xp, zp, eps);
+      return true;
+    }
+  }
+  if constexpr (sizeof(T) <= 4) {
+    if (!vec && p.xInner == 1 && p.zInner == 1 && p.outerX.rank <= 1 && p.outerZ.rank <= 1 && L >= V && L / V <= 64 * 8 && L < (1 << 30)) {
+      const LongType xp = p.outerX.rank ? p.outerX.stride[0] : 0, zp = p.outerZ.rank ? p.outerZ.stride[0] : 0;
+      const LongType per = (L / V + 63) / 64;
+      const bool nts = (size_t)p.rows * (size_t)L * sizeof(T) >= ((size_t)8 << 20);
+#define LWR_(NV, B, NTS) hipLaunchKernelGGL((layernorm_wave_regs<T, NV, B, NTS>), dim3(gw), dim3(256), 0, s, xt, gt, bt, zt, p.rows, (int)L, xp, zp, eps)
+#define LWR(NV) do { if (bt) { if (nts) LWR_(NV, true, true); else LWR_(NV, true, false); } else { if (nts) LWR_(NV, false, true); else LWR_(NV, false, false); } } while (0)
+      if (per <= 1) LWR(1); else if (per <= 2) LWR(2); else if (per <= 4) LWR(4); else LWR(8);
+#undef LWR
+#undef LWR_
       return true;
     }
   }

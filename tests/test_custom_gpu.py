@@ -345,7 +345,9 @@ def test_softmax_edge_semantics(ex, oracle):
 
 # ---- layer_norm ------------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype,rtol,atol", [(FLOAT32, 1e-5, 1e-5), (BFLOAT16, 1e-2, 1e-2), (HALF, 1e-2, 1e-2)])
-@pytest.mark.parametrize("shape", [(4, 64, 768), (3, 5, 100), (7, 2048), (2, 3, 5000), (4099, 768), (4097, 40), (41, 101, 256), (3, 40000), (2, 20004)])
+@pytest.mark.parametrize("shape", [(4, 64, 768), (3, 5, 100), (7, 2048), (2, 3, 5000), (4099, 768), (4097, 40), (41, 101, 256), (3, 40000), (2, 20004),
+                                   # row lengths that are not whole 16-byte vectors: a wave per row, element-aligned loads, the row in registers
+                                   (37, 770), (5, 769), (9, 13), (3, 7, 1001), (6, 2047), (2, 4093)])
 def test_layer_norm_last_axis(ex, oracle, dtype, rtol, atol, shape):
     rng = np.random.default_rng(shape[-1])
     C = shape[-1]
