@@ -584,6 +584,41 @@ static int gridFor(LongType work, int perBlock) {
 static int streamPolicy(size_t bytes) { return bytes > ((size_t)288 << 20) ? 3 : bytes >= ((size_t)8 << 20) ? 2 : 0; }
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+// A row vector against a dense [rows, cols] array whose row length is not a whole number of 16-byte vectors (or whose operands
+// start off 16-byte boundaries), which keeps it off the vector path of ew_nd: the dense array as one run of element-aligned
+// 16-byte vectors, one remainder per vector for the column of its first element, its stretch
+// of the row vector another such load (element by element where the vector runs over the end of a row).  bf16 [16000, 770] + [770]: 23.9 us with one element per thread.
+template <typename F, typename T>
+__global__ __launch_bounds__(EW_BLOCK) void row_broadcast_flat(const T* __restrict__ x, const T* __restrict__ v, T* __restrict__ z, LongType n, LongType cols,
+                                                               int nts) {
+  constexpr int V = 16 / sizeof(T);
+  using VT = Vec<T, V>;
+  using A = typename Conv<T>::acc;
+  const LongType nvec = n / V;
+  const LongType step = (LongType)gridDim.x * EW_BLOCK;
+  const bool small = n < ((LongType)1 << 32);
+  for (LongType i = (LongType)blockIdx.x * EW_BLOCK + threadIdx.x; i < nvec; i += step) {
+    VT a, out;
+    __builtin_memcpy(&a, x + i * V, sizeof(VT));
+    LongType c = small ? (LongType)((unsigned)(i * V) % (unsigned)cols) : (i * V) % cols;
+    if (c + V <= cols) {   // the usual case: the vector lies inside one row, its stretch of the row vector is one load too
+      VT b;
+      __builtin_memcpy(&b, v + c, sizeof(VT));
+#pragma unroll
+      for (int e = 0; e < V; e++) out.v[e] = Conv<T>::from(F::template apply<A>((A)to_float(a.v[e]), (A)to_float(b.v[e])));
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; e++) {
+        out.v[e] = Conv<T>::from(F::template apply<A>((A)to_float(a.v[e]), (A)to_float(v[c])));
+        c = c + 1 == cols ? 0 : c + 1;
+      }
+    }
+    if (nts) nt_store16_elem_aligned(z + i * V, out);
+    else __builtin_memcpy(z + i * V, &out, sizeof(VT));
+  }
+  const LongType j = nvec * V + (LongType)blockIdx.x * EW_BLOCK + threadIdx.x;   // the up to V - 1 elements that are left
+  if (j < n) z[j] = Conv<T>::from(F::template apply<A>((A)to_float(x[j]), (A)to_float(v[j % cols])));
+}
 template <typename F2, typename T, int NIN>
 static void launchNd(hipStream_t s, const EwPlan& p, const T* x, const T* y, T* z) {
   constexpr int V = 16 / sizeof(T);
@@ -609,6 +644,14 @@ static void launchNd(hipStream_t s, const EwPlan& p, const T* x, const T* y, T* 
     if (p.index32) hipLaunchKernelGGL((ew_nd<F2, T, NIN, V, unsigned>), dim3(gridFor(total, EW_BLOCK)), dim3(EW_BLOCK), 0, s, a, x, y, z, (unsigned)cpr, (unsigned)total);
     else hipLaunchKernelGGL((ew_nd<F2, T, NIN, V, unsigned long long>), dim3(gridFor(total, EW_BLOCK)), dim3(EW_BLOCK), 0, s, a, x, y, z, (unsigned long long)cpr, (unsigned long long)total);
   } else {
+    if constexpr (NIN == 2 && sizeof(T) <= 4) {
+      // x and z dense [rows, cols], y a row vector of cols elements
+      if (p.rank == 2 && p.stride[0][1] == 1 && p.stride[0][0] == inner && p.stride[1][1] == 1 && p.stride[1][0] == inner && p.stride[2][1] == 1 &&
+          p.stride[2][0] == 0 && p.length >= V && inner < ((LongType)1 << 31)) {
+        hipLaunchKernelGGL((row_broadcast_flat<F2, T>), dim3(gridFor(p.length / V, EW_BLOCK)), dim3(EW_BLOCK), 0, s, x, y, z, p.length, inner, a.nts);
+        return;
+      }
+    }
     LongType cpr = inner, total = p.length;
     if (p.index32) hipLaunchKernelGGL((ew_nd<F2, T, NIN, 1, unsigned>), dim3(gridFor(total, EW_BLOCK)), dim3(EW_BLOCK), 0, s, a, x, y, z, (unsigned)cpr, (unsigned)total);
     else hipLaunchKernelGGL((ew_nd<F2, T, NIN, 1, unsigned long long>), dim3(gridFor(total, EW_BLOCK)), dim3(EW_BLOCK), 0, s, a, x, y, z, (unsigned long long)cpr, (unsigned long long)total);
@@ -872,79 +915,7 @@ void launchPairwise(hipStream_t s, PairwiseKind k, DataType xdt, DataType ydt, D
   HIP_CHECK(hipGetLastError());
 }
 
-// ---- broadcast of a vector along the last axis / scalar ops ----------------------------------------------
-template <typename F, typename T>
-__global__ __launch_bounds__(EW_BLOCK) void row_broadcast(const T* __restrict__ x, const T* __restrict__ v,
-                                                          T* __restrict__ z, LongType rows, LongType cols) {
-  using A = typename Conv<T>::acc;
-  const LongType n = rows * cols;
-  const LongType step = (LongType)gridDim.x * EW_BLOCK;
-  for (LongType i = (LongType)blockIdx.x * EW_BLOCK + threadIdx.x; i < n; i += step) {
-    LongType c = i % cols;
-    z[i] = Conv<T>::from(F::template apply<A>((A)to_float(x[i]), (A)to_float(v[c])));
-  }
-}
-template <typename F, typename T>
-__global__ __launch_bounds__(EW_BLOCK) void row_broadcast_vec(const T* __restrict__ x, const T* __restrict__ v,
-                                                              T* __restrict__ z, LongType rows, LongType colVecs, int nts) {
-  constexpr int V = 16 / sizeof(T);
-  using VT = Vec<T, V>;
-  using A = typename Conv<T>::acc;
-  const LongType n = rows * colVecs;
-  const LongType step = (LongType)gridDim.x * EW_BLOCK;
-  const VT* xv = reinterpret_cast<const VT*>(x);
-  const VT* vv = reinterpret_cast<const VT*>(v);
-  VT* zv = reinterpret_cast<VT*>(z);
-  // the column of a thread's vector: the block's first column comes from one scalar remainder, the thread's own from at most
-  // a few subtractions (a 64-bit remainder per vector cost more than the memory traffic of the 16-bit types)
-  for (LongType base = (LongType)blockIdx.x * EW_BLOCK; base < n; base += step) {
-    const LongType i = base + threadIdx.x;
-    if (i >= n) break;
-    LongType col;
-    if (colVecs < (1 << 30)) {
-      col = (LongType)__builtin_amdgcn_readfirstlane((int)(base % colVecs)) + threadIdx.x;
-      if (colVecs >= EW_BLOCK) { if (col >= colVecs) col -= colVecs; }
-      else col %= colVecs;
-    } else {
-      col = i % colVecs;
-    }
-    VT a = xv[i], b = vv[col], out;
-#pragma unroll
-    for (int e = 0; e < V; e++) out.v[e] = Conv<T>::from(F::template apply<A>((A)to_float(a.v[e]), (A)to_float(b.v[e])));
-    store_vec(zv + i, out, nts != 0);
-  }
-}
-template <int K, typename T>
-static void rowBroadcastTyped(hipStream_t s, const void* x, const void* v, void* z, LongType rows, LongType cols) {
-  constexpr int V = 16 / sizeof(T);
-  if (cols % V == 0 && aligned16(x) && aligned16(v) && aligned16(z))
-    hipLaunchKernelGGL((row_broadcast_vec<Pairwise<K>, T>), dim3(gridFor(rows * cols / V, EW_BLOCK)), dim3(EW_BLOCK), 0, s, (const T*)x, (const T*)v, (T*)z, rows, cols / V,
-                       streamPolicy(sizeof(T) * (size_t)(rows * cols)) >= 2 ? 1 : 0);
-  else
-    hipLaunchKernelGGL((row_broadcast<Pairwise<K>, T>), dim3(gridFor(rows * cols, EW_BLOCK)), dim3(EW_BLOCK), 0, s, (const T*)x, (const T*)v, (T*)z, rows, cols);
-}
-template <int K>
-static void rowBroadcastKind(hipStream_t s, DataType dt, const void* x, const void* v, void* z, LongType rows, LongType cols) {
-  switch (dt) {
-    case FLOAT32: return rowBroadcastTyped<K, float>(s, x, v, z, rows, cols);
-    case DOUBLE: return rowBroadcastTyped<K, double>(s, x, v, z, rows, cols);
-    case HALF: return rowBroadcastTyped<K, f16_t>(s, x, v, z, rows, cols);
-    case BFLOAT16: return rowBroadcastTyped<K, bf16_t>(s, x, v, z, rows, cols);
-    default: ND4J_THROW("row broadcast: unsupported dtype");
-  }
-}
-void launchRowBroadcast(hipStream_t s, PairwiseKind k, DataType dt, const void* x, const void* v, void* z,
-                        LongType rows, LongType cols) {
-  if (rows * cols == 0) return;
-  switch (k) {
-    case P_ADD: rowBroadcastKind<P_ADD>(s, dt, x, v, z, rows, cols); break;
-    case P_SUB: rowBroadcastKind<P_SUB>(s, dt, x, v, z, rows, cols); break;
-    case P_MUL: rowBroadcastKind<P_MUL>(s, dt, x, v, z, rows, cols); break;
-    case P_DIV: rowBroadcastKind<P_DIV>(s, dt, x, v, z, rows, cols); break;
-    default: ND4J_THROW("row broadcast: unsupported op");
-  }
-  HIP_CHECK(hipGetLastError());
-}
+// ---- scalar ops ----------------------------------------------------------------------------------------------
 
 template <typename F, typename T>
 __global__ __launch_bounds__(EW_BLOCK) void scalar_nd(NdArgs a, const T* __restrict__ x, T* __restrict__ z,

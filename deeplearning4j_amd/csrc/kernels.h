@@ -64,9 +64,6 @@ struct EwPlan {
 void launchUnary(hipStream_t s, UnaryKind k, DataType xdt, DataType zdt, const void* x, void* z, const EwPlan& p);
 void launchPairwise(hipStream_t s, PairwiseKind k, DataType xdt, DataType ydt, DataType zdt, const void* x,
                     const void* y, void* z, const EwPlan& p);
-// z[outer.., c] = x[outer.., c] (op) v[c]: broadcast of a vector along the last axis of a dense array
-void launchRowBroadcast(hipStream_t s, PairwiseKind k, DataType dt, const void* x, const void* v, void* z,
-                        LongType rows, LongType cols);
 // z = f(x; s1, s2): the transforms of the legacy tables that read two extra parameters
 enum Scalar2Kind : int {
   S2_CLIP_BY_VALUE,   // x > s2 ? s2 : (x < s1 ? s1 : x)      ops.h:412-415, helpers/cpu/clip.cpp:211-219

@@ -193,6 +193,25 @@ def test_scalar_and_broadcast(ex, oracle):
     assert np.array_equal(ex.exec_broadcast(Broadcast.Add, A, NDArray.from_numpy(row), [1]).to_numpy(), oracle.add_row_vector(a, row, np.zeros_like(a)))
 
 
+@pytest.mark.parametrize("rows,cols", [(37, 770), (5, 769), (3, 5), (1, 3), (2, 1001), (1000, 7), (65, 4099)])
+def test_row_vector_against_rows_of_an_odd_length(ex, rows, cols):
+    """A row vector against a dense array whose rows are not whole 16-byte vectors: the array goes as one run of
+    element-aligned vectors (the row vector's stretch likewise, element by element across a row's end).  fp32 exactly,
+    bf16 as the rounded fp32 result."""
+    from deeplearning4j_amd.executioner import Broadcast
+    from deeplearning4j_amd.ndarray import BFLOAT16, bf16_bits_to_f32, f32_to_bf16_bits
+    rng = np.random.default_rng(rows * 7919 + cols)
+    a = rng.uniform(-1, 1, (rows, cols)).astype(np.float32)
+    row = rng.uniform(-1, 1, cols).astype(np.float32)
+    for op, f in ((Broadcast.Add, np.add), (Broadcast.Multiply, np.multiply), (Broadcast.Subtract, np.subtract)):
+        got = ex.exec_broadcast(op, NDArray.from_numpy(a), NDArray.from_numpy(row), [1]).to_numpy()
+        assert np.array_equal(got, f(a, row)), (op, rows, cols)
+    ab, rb = f32_to_bf16_bits(a), f32_to_bf16_bits(row)
+    got = ex.exec_broadcast(Broadcast.Add, NDArray.from_numpy(ab, BFLOAT16), NDArray.from_numpy(rb, BFLOAT16), [1])
+    want = f32_to_bf16_bits(bf16_bits_to_f32(ab) + bf16_bits_to_f32(rb))
+    assert np.array_equal(f32_to_bf16_bits(got.to_float()), want), (rows, cols)
+
+
 # ---- reductions ----------------------------------------------------------------------------------------------------------
 def _sum_atol(x, axis):
     # |tree sum - sequential sum| <= ~n eps sum|x| in the worst case; sqrt(n)-like in practice
