@@ -1117,7 +1117,7 @@ __global__ __launch_bounds__(512) void gemm_mfma16d(GemmArgs g, const T* __restr
   __syncthreads();
   readFrag(smem, 0, 0);
 
-  // one K-tile round; LOADS: the direct loads of tile kt + 2 are issued in this round (second half of k-step 3) and
+  // one K-tile round; LOADS: the direct loads of tile kt + 2 are issued here (second half of k-step 3) and
   // the first half of them in the NEXT round's k-step 0 -- spread out, each between two MFMAs
   auto round = [&](LongType kt, auto loadsNow, auto loadsLate) {
     u32x4* cur = smem + (kt & 1) * STAGE;
