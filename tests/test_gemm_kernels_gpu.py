@@ -179,6 +179,24 @@ def test_split_k_on_the_direct_load_ring_whole_result(ex, dtype, M, N, K, tb):
     _whole_result(ex, dtype, M, N, K, tb, expect=",split>+splitk_finish")
 
 
+def test_split_k_on_the_ring_batched_with_alpha_beta(ex):
+    """Three batch entries of few tiles and a long K: every entry's splits park their tiles under the entry's own index, and the
+    finishing launch applies alpha and beta."""
+    rng = np.random.default_rng(31)
+    batch, M, N, K = 3, 136, 128, 4104
+    a = rng.normal(0, 1 / math.sqrt(K), (batch, M, K)).astype(np.float32)
+    b = rng.normal(0, 1 / math.sqrt(K), (batch, K, N)).astype(np.float32)
+    c0 = rng.normal(0, 1, (batch, M, N)).astype(np.float32)
+    A, a64 = _device(a, BFLOAT16)
+    B, b64 = _device(b, BFLOAT16)
+    C, c64 = _device(c0, BFLOAT16)
+    ex.exec_custom("matmul", [A, B], [C], t_args=[0.5, 2.0])
+    assert ",split>+splitk_finish" in _last_kernel(ex), _last_kernel(ex)
+    got = C.to_float()
+    for bi in range(batch):
+        assert_close(got[bi], 0.5 * (a64[bi] @ b64[bi]) + 2.0 * c64[bi], 1e-2, 2e-2, "batch %d" % bi)
+
+
 def _whole_result(ex, dtype, M, N, K, tb, expect=",edge"):
     """The edge instantiations of the direct-load kernels, every element of the result: a row-major B with rows of 3705
     (every row starts 2 bytes further off a 16-byte boundary; one column is left for the bounds-handling kernel), of 3591
